@@ -1,0 +1,241 @@
+"""Write golden trajectories from the reference's *naive* optimizer classes.
+
+Run in the build container only (it needs /root/reference, which never travels):
+
+    python tests/golden/make_golden.py
+
+The reference package cannot be imported normally (``pylo/__init__.py`` pulls in
+``mup``, which is not installed), so the handful of modules needed are loaded by
+path under bare namespace packages.  The outputs are data only -- inputs, meta-net
+weights and the parameters / optimizer states after every step -- stored as
+``tests/golden/*.npz`` (numeric arrays, loaded with ``allow_pickle=False``).
+
+What each fixture pins: whole-``step()`` trajectories of ELO_CELO2_naive,
+VeLO_naive and AdafacLO_naive (op order, the var_rms quirk, tie rules, RNG order
+of the seeded meta-net initialisers), which no closed form fixes.
+"""
+
+import json
+import os
+import sys
+import tempfile
+import types
+
+import numpy as np
+import torch
+
+REF = os.environ.get("PYLO_REFERENCE", "/root/reference")
+OUT = os.path.dirname(os.path.abspath(__file__))
+
+
+def _load_reference():
+    for name in ("pylo", "pylo.optim", "pylo.models"):
+        mod = types.ModuleType(name)
+        mod.__path__ = [os.path.join(REF, *name.split("."))]
+        sys.modules[name] = mod
+    import importlib
+    m = importlib.import_module
+    return dict(
+        CELO2MLP=m("pylo.models.CELO2_MLP").CELO2MLP,
+        MetaMLP=m("pylo.models.Meta_MLP").MetaMLP,
+        VeLOMLP=m("pylo.models.VeLO_MLP").VeLOMLP,
+        VeLORNN=m("pylo.models.VeLO_RNN").VeLORNN,
+        ELO_CELO2_naive=m("pylo.optim.ELO_CELO2_naive").ELO_CELO2_naive,
+        VeLO_naive=m("pylo.optim.Velo_naive").VeLO_naive,
+        AdafacLO_naive=m("pylo.optim.AdafacLO_naive").AdafacLO_naive,
+    )
+
+
+def _np(t):
+    return t.detach().cpu().numpy().copy()
+
+
+def _to_leading(t, p_dim):
+    """naive state has the decay axis last; fixtures store it first (the CUDA classes' layout)."""
+    return t.movedim(-1, 0) if t.dim() == p_dim + 1 else t
+
+
+def _save(name, arrays, meta):
+    arrays["meta_json"] = np.frombuffer(json.dumps(meta).encode(), dtype=np.uint8)
+    path = os.path.join(OUT, name + ".npz")
+    np.savez_compressed(path, **arrays)
+    print(f"{name}: {len(arrays)} arrays, {os.path.getsize(path) / 1024:.1f} KiB")
+
+
+def _sd_arrays(prefix, module, arrays):
+    for k, v in module.state_dict().items():
+        arrays[f"{prefix}/{k}"] = _np(v)
+
+
+# ------------------------------------------------------------------ ELO-CELO2
+def celo2_case(R, name, shapes, n_steps, grad_scale, seed, cfg, net_seed=1, full=True, sample=4099,
+               init_std=1.0):
+    torch.manual_seed(net_seed)
+    net = R["CELO2MLP"]()
+    gen = torch.Generator().manual_seed(seed)
+    init = [torch.randn(s, generator=gen) * init_std for s in shapes]
+    params = [torch.nn.Parameter(v.clone()) for v in init]
+    opt = R["ELO_CELO2_naive"](params, network=net, hf_key=None, **cfg)
+    arrays = {}
+    _sd_arrays("net", net, arrays)
+    meta = dict(kind="elo_celo2", shapes=[list(s) for s in shapes], n_steps=n_steps, cfg=cfg,
+                grad_scale=grad_scale, seed=seed, net_seed=net_seed, full=full, sample=sample,
+                init_std=init_std)
+    if full:
+        for i, v in enumerate(init):
+            arrays[f"init/{i}"] = _np(v)
+    for t in range(n_steps):
+        grads = [torch.randn(s, generator=gen) * grad_scale for s in shapes]
+        for p, g in zip(params, grads):
+            p.grad = g.clone()
+        opt.step()
+        for i, p in enumerate(params):
+            st = opt.state[p]
+            rec = {"param": p.detach(), "mom": _to_leading(st["mom"], p.dim()),
+                   "rms": st["rms"][..., 0]}
+            if p.dim() >= 2:
+                # naive fac_vec_row (mean over dr, decay last) -> (3,*s with dr->1)
+                sorted_dims = np.argsort(p.shape)
+                dc, dr = int(sorted_dims[-2]), int(sorted_dims[-1])
+                rec["fac_r"] = st["fac_vec_row"].movedim(-1, 0).unsqueeze(dr + 1)
+                rec["fac_c"] = st["fac_vec_col"].movedim(-1, 0).unsqueeze(dc + 1)
+            for k, v in rec.items():
+                if full:
+                    arrays[f"step{t}/{k}/{i}"] = _np(v)
+                    if k == "param":
+                        arrays[f"grad{t}/{i}"] = _np(grads[i])
+                else:
+                    flat = v.reshape(-1)
+                    arrays[f"step{t}/{k}/{i}/sample"] = _np(flat[::sample])
+                    arrays[f"step{t}/{k}/{i}/norm"] = np.array(
+                        [float(torch.linalg.norm(flat.double()))], dtype=np.float64)
+    _save(name, arrays, meta)
+
+
+# ---------------------------------------------------------------------- VeLO
+def velo_case(R, name, shapes, n_steps, grad_scale, seed, num_steps, weight_decay, lr,
+              lstm_hidden=64, param_inits=32):
+    # A reduced LSTM width / bank size keeps the fixture small; both classes read the sizes
+    # from the saved config.json, and the arithmetic does not depend on them.
+    torch.manual_seed(11)
+    rnn = R["VeLORNN"](lstm_hidden_size=lstm_hidden, param_inits=param_inits)
+    with torch.no_grad():                       # non-trivial initial LSTM state and lr head
+        rnn.lstm_init_state[0].normal_(0, 0.1)
+        rnn.lstm_init_state[1].normal_(0, 0.1)
+    torch.manual_seed(12)
+    mlp = R["VeLOMLP"](param_inits=param_inits)
+    with torch.no_grad():                       # non-zero biases in the bank
+        for n_, p_ in mlp.named_parameters():
+            if "bias_" in n_:
+                p_.normal_(0, 0.5)
+    tmp = tempfile.mkdtemp()
+    rnn.save_pretrained(os.path.join(tmp, "rnn"))
+    mlp.save_pretrained(os.path.join(tmp, "mlp"))
+    gen = torch.Generator().manual_seed(seed)
+    init = [torch.randn(s, generator=gen) * 0.5 for s in shapes]
+    params = [torch.nn.Parameter(v.clone()) for v in init]
+    opt = R["VeLO_naive"](params, lr=lr, num_steps=num_steps, weight_decay=weight_decay,
+                          hf_key_rnn=os.path.join(tmp, "rnn"), hf_key_mlp=os.path.join(tmp, "mlp"))
+    arrays = {}
+    _sd_arrays("rnn", rnn, arrays)
+    _sd_arrays("mlp", mlp, arrays)
+    meta = dict(kind="velo", shapes=[list(s) for s in shapes], n_steps=n_steps, seed=seed,
+                num_steps=num_steps, weight_decay=weight_decay, lr=lr, grad_scale=grad_scale,
+                lstm_hidden=lstm_hidden, param_inits=param_inits)
+    for i, v in enumerate(init):
+        arrays[f"init/{i}"] = _np(v)
+    for t in range(n_steps):
+        grads = [torch.randn(s, generator=gen) * grad_scale for s in shapes]
+        loss = torch.tensor(2.0 * np.exp(-t / 5.0) + 0.1 + 0.05 * ((t * 7) % 3), dtype=torch.float32)
+        for p, g in zip(params, grads):
+            p.grad = g.clone()
+        opt.step(loss)
+        arrays[f"loss{t}"] = _np(loss)
+        arrays[f"step{t}/lstm_h"] = _np(opt.lstm_hidden_state[0])
+        arrays[f"step{t}/lstm_c"] = _np(opt.lstm_hidden_state[1])
+        for i, p in enumerate(params):
+            st = opt.state[p]
+            arrays[f"grad{t}/{i}"] = _np(grads[i])
+            arrays[f"step{t}/param/{i}"] = _np(p)
+            arrays[f"step{t}/mom/{i}"] = _np(st["mom"].movedim(-1, 0))
+            arrays[f"step{t}/rms/{i}"] = _np(st["rms"].movedim(-1, 0))
+            if st["fac_vec_v"].numel():
+                arrays[f"step{t}/fac_vec_v/{i}"] = _np(st["fac_vec_v"].movedim(-1, 0))
+            else:
+                arrays[f"step{t}/fac_vec_row_trailing/{i}"] = _np(st["fac_vec_row"])
+                arrays[f"step{t}/fac_vec_col_trailing/{i}"] = _np(st["fac_vec_col"])
+    _save(name, arrays, meta)
+
+
+# ------------------------------------------------------------------- AdafacLO
+def adafac_case(R, name, shapes, n_steps, grad_scale, seed, weight_decay, lr):
+    torch.manual_seed(21)
+    net = R["MetaMLP"](39, 32, 1)
+    tmp = tempfile.mkdtemp()
+    net.save_pretrained(os.path.join(tmp, "mlp"))
+    gen = torch.Generator().manual_seed(seed)
+    init = [torch.randn(s, generator=gen) * 0.5 for s in shapes]
+    params = [torch.nn.Parameter(v.clone()) for v in init]
+    opt = R["AdafacLO_naive"](params, lr=lr, weight_decay=weight_decay, hf_key=os.path.join(tmp, "mlp"))
+    arrays = {}
+    _sd_arrays("net", net, arrays)
+    meta = dict(kind="adafac", shapes=[list(s) for s in shapes], n_steps=n_steps, seed=seed,
+                weight_decay=weight_decay, lr=lr, grad_scale=grad_scale)
+    for i, v in enumerate(init):
+        arrays[f"init/{i}"] = _np(v)
+    for t in range(n_steps):
+        grads = [torch.randn(s, generator=gen) * grad_scale for s in shapes]
+        for p, g in zip(params, grads):
+            p.grad = g.clone()
+        opt.step()
+        for i, p in enumerate(params):
+            st = opt.state[p]
+            arrays[f"grad{t}/{i}"] = _np(grads[i])
+            arrays[f"step{t}/param/{i}"] = _np(p)
+            arrays[f"step{t}/exp_avg/{i}"] = _np(st["mom"].movedim(-1, 0))
+            arrays[f"step{t}/exp_avg_sq/{i}"] = _np(st["rms"][..., 0])
+            if st["fac_vec_v"].numel():
+                arrays[f"step{t}/fac_vec_v/{i}"] = _np(st["fac_vec_v"].movedim(-1, 0))
+            else:
+                arrays[f"step{t}/fac_vec_row_trailing/{i}"] = _np(st["fac_vec_row"])
+                arrays[f"step{t}/fac_vec_col_trailing/{i}"] = _np(st["fac_vec_col"])
+    _save(name, arrays, meta)
+
+
+def ctor_checksums(R):
+    """Sum and sum of squares (fp64) of every freshly constructed meta-net parameter under a fixed
+    seed: pins the order in which the constructors draw from the RNG."""
+    arrays = {}
+    for cls, args in (("CELO2MLP", ()), ("MetaMLP", (39, 32, 1)), ("VeLOMLP", ()), ("VeLORNN", ())):
+        torch.manual_seed(1234)
+        mod = R[cls](*args)
+        for k, v in mod.state_dict().items():
+            d = v.double()
+            arrays[f"{cls}/{k}"] = np.array([float(d.sum()), float((d * d).sum()), v.numel()])
+    _save("ctor_checksums", arrays, dict(kind="ctor", seed=1234))
+
+
+def main():
+    R = _load_reference()
+    torch.set_num_threads(8)
+    ctor_checksums(R)
+    # shapes of the reference's own CUDA-vs-naive test (tests/test_celo2_cuda.py:38,116)
+    celo2_case(R, "elo_celo2_small_clip", [(64, 32), (32, 64), (32,), (48, 24)], 10, 3.0, 2,
+               dict(lr=1e-2, adam_lr_mult=20.0))
+    celo2_case(R, "elo_celo2_small_noclip_exp", [(64, 32), (32, 64), (32,), (24, 24)], 10, 1e-3, 3,
+               dict(lr=1e-3, adam_lr_mult=20.0, exp_mult=0.01, weight_decay=0.05, rmsmult=0.7))
+    celo2_case(R, "elo_celo2_small_noortho", [(40, 56), (7,)], 8, 0.5, 4,
+               dict(lr=1e-2, orthogonalize=False, clip_grad=False, adam_lr_mult=1.0))
+    # BASELINE config 1: 1024x1024 weight + 1024 bias, N(0, 0.02) init, N(0, 1e-3) grads, 10 steps
+    celo2_case(R, "elo_celo2_cfg1", [(1024, 1024), (1024,)], 10, 1e-3, 0,
+               dict(lr=3.16e-4, weight_decay=0.1, adam_lr_mult=20.0), full=False, init_std=0.02)
+    velo_case(R, "velo_small", [(20, 10), (20,), (5, 20), (5,), (6, 3, 4, 4), (16, 16), (1, 1, 12)],
+              6, 0.3, 5, num_steps=40, weight_decay=0.0, lr=1e-2)
+    velo_case(R, "velo_small_wd", [(33, 17), (17,)], 5, 2.0, 6, num_steps=10, weight_decay=0.01, lr=1e-3)
+    adafac_case(R, "adafac_small", [(20, 10), (20,), (5, 20), (6, 3, 4, 4), (16, 16)], 6, 0.3, 7,
+                weight_decay=0.0, lr=1.0)
+    adafac_case(R, "adafac_small_wd", [(33, 17), (17,)], 5, 1e-3, 8, weight_decay=0.01, lr=0.5)
+
+
+if __name__ == "__main__":
+    main()

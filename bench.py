@@ -1,0 +1,179 @@
+"""Benchmark of the fused learned-optimizer step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gpt2s|cfg1] [--fused-only]
+
+Workload (default): BASELINE config 2 -- ELO-CELO2 on a GPT-2-small-shaped fp32 parameter set
+(98 tensors, 124 355 328 parameters), synthetic per-tensor Gaussian gradients with log-uniform
+scale in [1e-5, 1e-2], random-init CELO2MLP, everything resident in HBM before timing starts.
+
+A *step* of the metric is one pass of the fused hot path: the single C-ABI call
+``pylo_mi355_celo2_step`` (7 launches: gradient statistics, accumulator updates, features, MLP,
+raw step for the 2-D tensors, AdamW for the 1-D tensors).  Its duration is measured with HIP
+events recorded by the library on the launch stream, inside full ``optimizer.step()`` calls; the
+whole ``step()`` (which adds library-GEMM Newton-Schulz, normalisation and the parameter update)
+is reported next to it as ``whole_step_ms``.
+
+Prints ONE JSON line.
+"""
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+B_P0, B_STATS, B_APPLY = 4, 24, 44   # algorithmic bytes per element of a >=2-D tensor, per pass
+B_ADAM = 44                    # 1-D AdamW branch: read g,p,m0..2,rms; write m0..2,rms,p
+
+
+def gpt2_small_shapes():
+    shapes = [(50257, 768), (1024, 768)]
+    for _ in range(12):
+        shapes += [(768,), (768,), (768, 2304), (768, 768), (768,), (768,), (768, 3072), (3072, 768)]
+    return shapes
+
+
+def cfg1_shapes():
+    return [(1024, 1024), (1024,)]
+
+
+def layer_sample_shapes():
+    return [(768,), (768,), (768, 2304), (768, 768), (768,), (768,), (768, 3072), (3072, 768)]
+
+
+def make_inputs(shapes, device, seed=0):
+    import torch
+
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    scales = [10 ** (-5 + 3 * float(torch.rand((), generator=gen))) for _ in shapes]
+    ggen = torch.Generator(device=device).manual_seed(seed + 1)
+    params, grads = [], []
+    for s, sc in zip(shapes, scales):
+        params.append(torch.nn.Parameter(torch.randn(s, generator=ggen, device=device) * 0.02))
+        grads.append(torch.randn(s, generator=ggen, device=device) * sc)
+    return params, grads
+
+
+def cpu_baseline(steps=6):
+    """The oracle (CPU restatement of the reference's naive PyTorch path) on one transformer
+    layer of the same workload, host cores of this box."""
+    import torch
+
+    from oracle import pylo_oracle as O
+    from pylo_amd.models import CELO2MLP
+
+    shapes = layer_sample_shapes()
+    torch.manual_seed(1)
+    net = CELO2MLP()
+    params, grads = make_inputs(shapes, "cpu", seed=3)
+    params = [p.detach().clone() for p in params]
+    orc = O.EloCelo2Oracle(params, net.state_dict(), lr=3.16e-4, adam_lr_mult=20.0)
+    n = sum(p.numel() for p in params)
+    t_fused = t_all = 0.0
+    for it in range(steps + 1):
+        orc.finish_seconds = 0.0
+        t0 = time.perf_counter()
+        orc.step(grads)
+        dt = time.perf_counter() - t0
+        if it > 0:
+            t_all += dt
+            t_fused += dt - orc.finish_seconds
+    return {
+        "value": n * steps / t_fused, "unit": "params/s", "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"oracle (torch-CPU restatement of ELO_CELO2_naive) on one GPT-2-small layer "
+                  f"({n} params, {steps} steps after 1 warm-up): accumulators+features+MLP+AdamW only; "
+                  f"with Newton-Schulz/normalise/apply {n * steps / t_all:.3e} params/s",
+        "os_cpu_count": os.cpu_count(),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="gpt2s", choices=["gpt2s", "cfg1"])
+    ap.add_argument("--fused-only", action="store_true",
+                    help="loop the C-ABI call alone (no Newton-Schulz / apply), e.g. under rocprofv3")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
+
+    import torch
+
+    from pylo_amd import ELO_CELO2_CUDA
+    from pylo_amd.models import CELO2MLP
+
+    dev = torch.device("cuda:0")
+    shapes = gpt2_small_shapes() if a.workload == "gpt2s" else cfg1_shapes()
+    torch.manual_seed(1)
+    net = CELO2MLP()
+    params, grads = make_inputs(shapes, dev)
+    for p, g in zip(params, grads):
+        p.grad = g
+    opt = ELO_CELO2_CUDA(params, lr=3.16e-4, weight_decay=0.1, adam_lr_mult=20.0, network=net, hf_key=None)
+    n_params = sum(p.numel() for p in params)
+    n2d = sum(p.numel() for p in params if p.dim() >= 2)
+    n1d = n_params - n2d
+
+    def one_step():
+        if a.fused_only:
+            opt.fused_step()
+        else:
+            opt.step()
+
+    for _ in range(a.warmup):
+        one_step()
+    torch.cuda.synchronize()
+    plan = opt._plan
+    plan.timing_begin(a.steps)
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        one_step()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    per = plan.timing_end()                       # (steps, launches) ms
+    names = plan.launch_names()
+    mean = per.mean(axis=0)
+    fused_ms = float(per.sum(axis=1).mean())
+    bytes_fused = n2d * (B_P0 + B_STATS + B_APPLY) + n1d * B_ADAM
+    k_apply = names.index("k_celo2_apply")
+    apply_ms = float(mean[k_apply])
+    apply_gbs = n2d * B_APPLY / (apply_ms * 1e-3) / 1e9
+    out = {
+        "metric": "params_updated_per_sec (fused ELO-CELO2 step, C-ABI call)",
+        "value": n_params / (fused_ms * 1e-3),
+        "unit": "params/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": fused_ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": ("ELO_CELO2 fused step, GPT-2-small fp32 parameter set (98 tensors)"
+                                if a.workload == "gpt2s" else "ELO_CELO2 fused step, 1024x1024 + 1024"),
+                   "params": n_params, "tensors": len(shapes), "launches_per_step": len(names),
+                   "timed": "HIP events on the launch stream, first launch to last launch of the C-ABI call"},
+        "hbm_algorithmic_GB_per_step": bytes_fused / 1e9,
+        "hbm_GBps_fused_path": bytes_fused / (fused_ms * 1e-3) / 1e9,
+        "hbm_roofline_frac_fused_path": bytes_fused / (fused_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "whole_step_ms": None if a.fused_only else wall_ms,
+        "whole_step_note": "optimizer.step(): fused path + torch Newton-Schulz (fp32 GEMMs), normalise, apply",
+        "launch_ms": {nm: float(v) for nm, v in zip(names, mean)},
+        "roofline": {"bound": "hbm", "kernel": "k_celo2_apply", "achieved": apply_gbs, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": apply_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": n2d * B_APPLY, "avg_launch_ms": apply_ms},
+    }
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -23,6 +23,7 @@ Every function cites the reference lines it restates.
 from __future__ import annotations
 
 import math
+import time
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -214,6 +215,7 @@ class EloCelo2Oracle:
         self.ns = (tuple(float(c) for c in ns_coeffs), ns_iters, ns_eps)
         self.is_embedding = list(is_embedding) or [False] * len(params)
         self.t = 0
+        self.finish_seconds = 0.0     # time spent in finish_step (NS / normalise / apply), for bench.py
         self.state: List[Dict[str, torch.Tensor]] = []
         for p in params:
             s = tuple(p.shape)
@@ -301,7 +303,9 @@ class EloCelo2Oracle:
                 raw = self.raw_step(i, p, g)
                 if keep_raw is not None:
                     keep_raw[i] = raw.clone()
+                t0 = time.perf_counter()
                 self.finish_step(p, raw)
+                self.finish_seconds += time.perf_counter() - t0
 
 
 # ----------------------------------------------------------------------------

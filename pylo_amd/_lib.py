@@ -1,0 +1,161 @@
+"""ctypes binding of ``libpylo_mi355.so`` (the C ABI declared in include/pylo_mi355.h).
+
+There is no fallback: if the library is missing or a call fails, a RuntimeError is raised.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import List, Sequence
+
+import numpy as np
+import torch
+
+from .build import LIB_PATH
+
+MAX_DIMS = 8
+KIND_CELO2, KIND_VELO, KIND_ADAFAC = 0, 1, 2
+F_ADAM = 1
+
+
+class TensorShape(C.Structure):
+    _fields_ = [("ndim", C.c_int32), ("flags", C.c_int32), ("shape", C.c_int64 * MAX_DIMS)]
+
+
+class Decays(C.Structure):
+    _fields_ = [("beta_m", C.c_float * 3), ("beta_rms", C.c_float), ("beta_fac", C.c_float * 3)]
+
+
+# numpy mirror of PyloTensorArgs (8 pointers, 8 floats, no padding)
+ARGS_DTYPE = np.dtype([
+    ("grad", np.uint64), ("param", np.uint64), ("mom", np.uint64), ("rms", np.uint64),
+    ("fac_r", np.uint64), ("fac_c", np.uint64), ("fac_v", np.uint64), ("step_out", np.uint64),
+    ("lr", np.float32), ("weight_decay", np.float32), ("clip_norm", np.float32),
+    ("clip_val", np.float32), ("exp_mult", np.float32), ("step_mult", np.float32),
+    ("bc1", np.float32), ("bc2", np.float32),
+])
+assert ARGS_DTYPE.itemsize == 96
+
+_lib = None
+
+
+def load():
+    """Loads the shared library once; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m pylo_amd.build` "
+            "(there is no non-HIP fallback for the fused optimizer step)")
+    lib = C.CDLL(LIB_PATH)
+    lib.pylo_mi355_abi_version.restype = C.c_int
+    lib.pylo_mi355_last_error.restype = C.c_char_p
+    lib.pylo_mi355_plan_workspace_bytes.argtypes = [C.c_int, C.POINTER(TensorShape), C.c_int,
+                                                    C.POINTER(C.c_size_t)]
+    lib.pylo_mi355_plan_create.argtypes = [C.c_int, C.POINTER(TensorShape), C.c_int, C.c_void_p,
+                                           C.c_size_t, C.c_void_p, C.POINTER(C.c_void_p)]
+    lib.pylo_mi355_plan_destroy.argtypes = [C.c_void_p]
+    lib.pylo_mi355_plan_num_launches.argtypes = [C.c_void_p]
+    lib.pylo_mi355_plan_factored_dims.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int),
+                                                  C.POINTER(C.c_int)]
+    lib.pylo_mi355_plan_timing_begin.argtypes = [C.c_void_p, C.c_int]
+    lib.pylo_mi355_plan_timing_end.argtypes = [C.c_void_p, C.POINTER(C.c_float), C.c_int, C.POINTER(C.c_int)]
+    lib.pylo_mi355_plan_launch_name.argtypes = [C.c_void_p, C.c_int]
+    lib.pylo_mi355_plan_launch_name.restype = C.c_char_p
+    lib.pylo_mi355_celo2_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.c_void_p,
+                                          C.c_void_p]
+    if lib.pylo_mi355_abi_version() != 1:
+        raise RuntimeError("libpylo_mi355.so: ABI version mismatch, rebuild it")
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise RuntimeError(f"{what}: {load().pylo_mi355_last_error().decode()}")
+
+
+def make_shapes(shapes: Sequence[Sequence[int]], flags: Sequence[int]):
+    arr = (TensorShape * len(shapes))()
+    for i, (s, f) in enumerate(zip(shapes, flags)):
+        if len(s) > MAX_DIMS:
+            raise ValueError(f"tensors with more than {MAX_DIMS} dims are not supported")
+        arr[i].ndim = len(s)
+        arr[i].flags = int(f)
+        for j, v in enumerate(s):
+            arr[i].shape[j] = int(v)
+    return arr
+
+
+def make_decays(beta_m, beta_rms, beta_fac) -> Decays:
+    d = Decays()
+    for k in range(3):
+        d.beta_m[k] = float(beta_m[k])
+        d.beta_fac[k] = float(beta_fac[k])
+    d.beta_rms = float(beta_rms)
+    return d
+
+
+class Plan:
+    """A launch plan over a fixed list of tensor shapes; owns its device workspace."""
+
+    def __init__(self, kind: int, shapes: Sequence[Sequence[int]], flags: Sequence[int],
+                 device: torch.device):
+        lib = load()
+        self.kind = kind
+        self.n = len(shapes)
+        self._shapes = make_shapes(shapes, flags)
+        nbytes = C.c_size_t(0)
+        check(lib.pylo_mi355_plan_workspace_bytes(kind, self._shapes, self.n, C.byref(nbytes)),
+              "plan_workspace_bytes")
+        self.workspace = torch.empty(max(int(nbytes.value), 256), dtype=torch.uint8, device=device)
+        handle = C.c_void_p()
+        with torch.cuda.device(device):
+            stream = torch.cuda.current_stream(device).cuda_stream
+            check(lib.pylo_mi355_plan_create(kind, self._shapes, self.n, self.workspace.data_ptr(),
+                                             self.workspace.numel(), stream, C.byref(handle)),
+                  "plan_create")
+        self._h = handle
+        self.args = np.zeros(self.n, dtype=ARGS_DTYPE)
+
+    def factored_dims(self, i: int):
+        dc, dr = C.c_int(), C.c_int()
+        check(load().pylo_mi355_plan_factored_dims(self._h, i, C.byref(dc), C.byref(dr)), "factored_dims")
+        return (dc.value, dr.value) if dc.value >= 0 else None
+
+    @property
+    def num_launches(self) -> int:
+        return load().pylo_mi355_plan_num_launches(self._h)
+
+    def launch_names(self) -> List[str]:
+        lib = load()
+        return [lib.pylo_mi355_plan_launch_name(self._h, i).decode() for i in range(self.num_launches)]
+
+    def timing_begin(self, max_steps: int) -> None:
+        check(load().pylo_mi355_plan_timing_begin(self._h, max_steps), "timing_begin")
+        self._timing_cap = max_steps * self.num_launches
+
+    def timing_end(self) -> np.ndarray:
+        """(steps, num_launches) array of launch durations in ms, measured with HIP events."""
+        buf = (C.c_float * self._timing_cap)()
+        steps = C.c_int(0)
+        check(load().pylo_mi355_plan_timing_end(self._h, buf, self._timing_cap, C.byref(steps)), "timing_end")
+        nl = self.num_launches
+        return np.array(buf[:steps.value * nl], dtype=np.float64).reshape(steps.value, nl)
+
+    def celo2_step(self, decays: Decays, mlp: torch.Tensor, stream: int) -> None:
+        check(load().pylo_mi355_celo2_step(self._h, self.args.ctypes.data, C.byref(decays),
+                                           mlp.data_ptr(), stream), "celo2_step")
+
+    def close(self):
+        if getattr(self, "_h", None):
+            load().pylo_mi355_plan_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

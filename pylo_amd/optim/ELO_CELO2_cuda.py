@@ -1,0 +1,252 @@
+"""ELO_CELO2_CUDA on MI355X: the reference's ELO-CELO2 optimizer with its per-tensor Python
+loop and CUDA extension replaced by one multi-tensor HIP step.
+
+Drop-in for pylo/optim/ELO_CELO2_cuda.py:39-298: same constructor, ``step()``,
+``param_groups`` keys and per-parameter state (``mom (3,*s)``, ``rms (*s)``, ``fac_r``,
+``fac_c``).  What differs is *where* the work happens: gradient clipping, every
+accumulator update, the 1-D AdamW branch and the feature/MLP pass of all tensors run in
+seven launches of ``libpylo_mi355.so``; only Newton-Schulz (library GEMMs), the final RMS
+normalisation and the parameter update remain in PyTorch.  Arithmetic follows the
+reference's naive class (pylo/optim/ELO_CELO2_naive.py:126-306).
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch.optim import Optimizer
+
+from .. import _lib
+from ..models import CELO2MLP, pack_celo2
+
+_IN, _HID = 30, 8
+
+
+def newton_schulz(x: torch.Tensor, coeffs, iters: int, eps: float) -> torch.Tensor:
+    """Quintic Newton-Schulz over the last two dims (pylo/optim/CELO2_naive.py:59-73)."""
+    tall = x.shape[-2] > x.shape[-1]
+    if tall:
+        x = x.transpose(-2, -1)
+    x = x / (torch.linalg.norm(x, dim=(-2, -1), keepdim=True) + eps)
+    c0, c1, c2 = coeffs
+    for _ in range(iters):
+        a = x @ x.transpose(-2, -1)
+        x = c0 * x + (c1 * a + c2 * (a @ a)) @ x
+    return x.transpose(-2, -1) if tall else x
+
+
+def rms_normalize(x: torch.Tensor, dims, eps: float = 1e-9) -> torch.Tensor:
+    """x * rsqrt(eps + mean(x^2) over dims) (pylo/optim/CELO2_naive.py:54-56)."""
+    return x * torch.rsqrt(eps + torch.mean(x * x, dim=dims, keepdim=True))
+
+
+class ELO_CELO2_CUDA(Optimizer):
+    """Inference-time ELO-CELO2: CELO2 MLP steps for >=2-D tensors, shared-accumulator AdamW for
+    1-D tensors and ``is_embedding`` groups."""
+
+    def __init__(
+        self,
+        params,
+        lr=1e-3,
+        weight_decay=0.1,
+        clip_grad=True,
+        clip_norm=1.0,
+        adam_lr_mult=20.0,
+        adam_weight_decay=None,
+        use_adamw_for_1d=True,
+        orthogonalize=True,
+        ff_hidden_size=8,
+        ff_hidden_layers=2,
+        initial_momentum_decays=(0.9, 0.99, 0.999),
+        initial_rms_decays=(0.95,),
+        initial_adafactor_decays=(0.9, 0.99, 0.999),
+        exp_mult=0.0,
+        rmsmult=1.0,
+        param_scale_mult=False,
+        ns_coeffs=(3.4445, -4.7750, 2.0315),
+        ns_iters=5,
+        ns_eps=1e-8,
+        grad_clip_val=1000.0,
+        hf_key: Optional[str] = "DiamondXL/elo-celo2",
+        checkpoint_path: Optional[str] = None,
+        network: Optional[CELO2MLP] = None,
+    ):
+        if not torch.cuda.is_available():
+            raise RuntimeError("ELO_CELO2_CUDA requires a GPU (torch.cuda.is_available() is False).")
+        _lib.load()
+        defaults = dict(
+            lr=lr, weight_decay=weight_decay, adam_lr_mult=adam_lr_mult,
+            adam_weight_decay=weight_decay if adam_weight_decay is None else adam_weight_decay,
+            use_adamw_for_1d=use_adamw_for_1d, orthogonalize=orthogonalize, clip_grad=clip_grad,
+            clip_norm=clip_norm, exp_mult=exp_mult, rmsmult=rmsmult,
+            param_scale_mult=param_scale_mult, grad_clip_val=grad_clip_val, is_embedding=False)
+        super().__init__(params, defaults)
+        first = next(p for g in self.param_groups for p in g["params"])
+        self.device = first.device if first.is_cuda else torch.device("cuda", torch.cuda.current_device())
+
+        def decays(v):
+            return torch.clamp(torch.tensor(v, dtype=torch.float32, device=self.device), 0.0, 1.0)
+
+        self.beta_m, self.beta_rms, self.beta_fac = (decays(initial_momentum_decays),
+                                                      decays(initial_rms_decays),
+                                                      decays(initial_adafactor_decays))
+        self.n_mom, self.n_rms, self.n_fac = (self.beta_m.numel(), self.beta_rms.numel(),
+                                              self.beta_fac.numel())
+        if (self.n_mom, self.n_fac) != (3, 3) or self.n_rms < 1:
+            raise ValueError("the fused step supports 3 momentum decays, 3 adafactor decays and >=1 rms decay")
+        self.ns_coeffs = tuple(float(c) for c in ns_coeffs)
+        self.ns_iters, self.ns_eps = ns_iters, ns_eps
+
+        if network is None:
+            if checkpoint_path is not None:
+                network = CELO2MLP(hidden_size=ff_hidden_size, hidden_layers=ff_hidden_layers)
+                network.load_state_dict(torch.load(checkpoint_path, map_location="cpu"))
+            elif hf_key is not None:
+                network = CELO2MLP.from_pretrained(hf_key)
+            else:
+                network = CELO2MLP(hidden_size=ff_hidden_size, hidden_layers=ff_hidden_layers)
+        self.network = network.to(self.device)
+        if sum(self.network.feature_dims) != _IN:
+            raise ValueError(f"ELO_CELO2_CUDA kernel expects feature_dims summing to {_IN}, "
+                             f"got {sum(self.network.feature_dims)}.")
+        if self.network.hidden_size != _HID or len(self.network.dense_w) != 2:
+            raise ValueError("ELO_CELO2_CUDA kernel only supports ff_hidden_size=8, ff_hidden_layers=2.")
+        if self.network.activation != "relu" or self.network.output_size != 3:
+            raise ValueError("ELO_CELO2_CUDA kernel only supports relu activation and output_size=3.")
+        self._mlp = pack_celo2(self.network).to(self.device)
+        bm, bf = self.beta_m.tolist(), self.beta_fac.tolist()
+        self._decays = _lib.make_decays(bm, float(self.beta_rms[-1]), bf)
+        self._plan = None
+        self._plan_key = None
+
+    # ------------------------------------------------------------------ plan
+    def _tensors(self):
+        out = []
+        for group in self.param_groups:
+            for p in group["params"]:
+                adam = p.dim() <= 1 or group["is_embedding"]
+                if adam and not group["use_adamw_for_1d"]:
+                    raise NotImplementedError(
+                        "use_adamw_for_1d=False (CELO2 MLP on 1-D / embedding tensors) is not supported "
+                        "by the fused step")
+                out.append((group, p, adam))
+        return out
+
+    def _ensure_plan(self, tensors):
+        key = tuple((tuple(p.shape), adam) for _, p, adam in tensors)
+        if key == self._plan_key:
+            return
+        for _, p, _a in tensors:
+            if not p.is_cuda or p.device != self.device:
+                raise RuntimeError("ELO_CELO2_CUDA: every parameter must live on the optimizer's GPU")
+            if p.dtype != torch.float32 or not p.is_contiguous():
+                raise TypeError("ELO_CELO2_CUDA: parameters must be contiguous float32 tensors")
+        if self._plan is not None:
+            self._plan.close()
+        shapes = [tuple(p.shape) for _, p, _a in tensors]
+        flags = [_lib.F_ADAM if adam else 0 for _, _p, adam in tensors]
+        self._plan = _lib.Plan(_lib.KIND_CELO2, shapes, flags, self.device)
+        self._plan_key = key
+        # one flat buffer for the raw steps of all MLP tensors, 256-byte aligned slices
+        offs, total = [], 0
+        for _, p, adam in tensors:
+            offs.append(total)
+            if not adam:
+                total += (p.numel() + 63) // 64 * 64
+        flat = torch.empty(max(total, 1), dtype=torch.float32, device=self.device)
+        self._raw = [None if adam else flat[o:o + p.numel()].view(p.shape)
+                     for o, (_, p, adam) in zip(offs, tensors)]
+        self._raw_flat = flat
+
+    def _init_state(self, state, p):
+        shape = tuple(p.shape)
+        state["mom"] = torch.zeros((self.n_mom,) + shape, device=self.device)
+        state["rms"] = torch.zeros(shape, device=self.device)
+        if p.dim() >= 2:
+            dc, dr = _factored_dims_host(shape)
+            r_shape, c_shape = list(shape), list(shape)
+            r_shape[dr] = 1
+            c_shape[dc] = 1
+            state["fac_r"] = torch.zeros([self.n_fac] + r_shape, device=self.device)
+            state["fac_c"] = torch.zeros([self.n_fac] + c_shape, device=self.device)
+
+    # ------------------------------------------------------------------ step
+    @torch.no_grad()
+    def step(self, loss=None):
+        tensors = self.fused_step()
+        self.finish_step(tensors)
+        return loss
+
+    @torch.no_grad()
+    def fused_step(self):
+        """Everything up to the raw per-element step: one call into the HIP library."""
+        tensors = self._tensors()
+        self._ensure_plan(tensors)
+        plan = self._plan
+        for group in self.param_groups:
+            group["step"] = group.get("step", 0) + 1
+        beta1 = float(self.beta_m[0])
+        beta2 = float(self.beta_rms[-1])
+        n = len(tensors)
+        cols = {k: [0] * n for k in ("grad", "param", "mom", "rms", "fac_r", "fac_c", "step_out")}
+        fl = {k: [0.0] * n for k in ("lr", "weight_decay", "clip_norm", "clip_val", "exp_mult", "bc1", "bc2")}
+        keep = []   # contiguous copies of non-contiguous grads must outlive the launch
+        for i, (group, p, adam) in enumerate(tensors):
+            g = p.grad
+            if g is None:
+                continue
+            if g.is_sparse:
+                raise RuntimeError("ELO_CELO2_CUDA does not support sparse gradients")
+            if g.dtype != torch.float32:
+                raise TypeError("ELO_CELO2_CUDA: gradients must be float32")
+            if not g.is_contiguous():
+                g = g.contiguous()
+                keep.append(g)
+            state = self.state[p]
+            if len(state) == 0:
+                self._init_state(state, p)
+            t = group["step"]
+            cols["grad"][i], cols["param"][i] = g.data_ptr(), p.data_ptr()
+            cols["mom"][i], cols["rms"][i] = state["mom"].data_ptr(), state["rms"].data_ptr()
+            fl["clip_norm"][i] = group["clip_norm"] if group["clip_grad"] else 0.0
+            fl["clip_val"][i] = group["grad_clip_val"]
+            fl["exp_mult"][i] = group["exp_mult"]
+            if adam:
+                fl["lr"][i] = group["adam_lr_mult"] * group["lr"]
+                fl["weight_decay"][i] = group["adam_weight_decay"]
+                fl["bc1"][i] = 1.0 - beta1 ** t
+                fl["bc2"][i] = 1.0 - beta2 ** t
+            else:
+                cols["fac_r"][i], cols["fac_c"][i] = state["fac_r"].data_ptr(), state["fac_c"].data_ptr()
+                cols["step_out"][i] = self._raw[i].data_ptr()
+        args = plan.args
+        for k, v in cols.items():
+            args[k] = v
+        for k, v in fl.items():
+            args[k] = v
+        with torch.cuda.device(self.device):
+            plan.celo2_step(self._decays, self._mlp, torch.cuda.current_stream(self.device).cuda_stream)
+        del keep
+        return tensors
+
+    @torch.no_grad()
+    def finish_step(self, tensors):
+        """Newton-Schulz, RMS normalisation and the parameter update of the MLP tensors
+        (pylo/optim/ELO_CELO2_cuda.py:288-296)."""
+        for i, (group, p, adam) in enumerate(tensors):
+            if adam or p.grad is None:
+                continue
+            step = self._raw[i]
+            if group["param_scale_mult"]:
+                step = step * torch.sqrt(torch.mean(p * p) + 1e-9)
+            if group["orthogonalize"]:
+                step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
+            step = rms_normalize(step, list(range(p.dim()))[-2:]) * group["rmsmult"]
+            p.add_(step + group["weight_decay"] * p, alpha=-group["lr"])
+
+
+def _factored_dims_host(shape):
+    """(dc, dr) as pylo/optim/CELO2_naive.py:42-47: 2nd-largest and largest dim, ties by index."""
+    order = sorted(range(len(shape)), key=lambda i: (shape[i], i))
+    return order[-2], order[-1]

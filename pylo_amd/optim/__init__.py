@@ -1,0 +1,7 @@
+"""Fused learned-optimizer classes (same public names as ``pylo.optim``)."""
+
+from .ELO_CELO2_cuda import ELO_CELO2_CUDA
+
+ELO_CELO2 = ELO_CELO2_CUDA
+
+__all__ = ["ELO_CELO2_CUDA", "ELO_CELO2"]

@@ -1,0 +1,346 @@
+// ELO-CELO2 / CELO2 element kernels: statistics pass, weight folding, apply pass.
+#pragma once
+
+#include "pylo_common.h"
+
+namespace pylo {
+
+struct EmaConsts {
+  float bm[3], obm[3];  // momentum decays and 1-decay
+  float br, obr;        // rms
+};
+
+__device__ __forceinline__ EmaConsts make_ema(const PyloDecays& dec) {
+  EmaConsts e;
+#pragma unroll
+  for (int k = 0; k < 3; ++k) { e.bm[k] = dec.beta_m[k]; e.obm[k] = 1.0f - dec.beta_m[k]; }
+  e.br = dec.beta_rms;
+  e.obr = 1.0f - dec.beta_rms;
+  return e;
+}
+
+// acc <- beta*acc + (1-beta)*new, each product and the sum rounded (ELO_CELO2_naive.py:145,149)
+__device__ __forceinline__ void ema_update(const EmaConsts& e, float g, float (&m)[3], float& rms) {
+#pragma unroll
+  for (int k = 0; k < 3; ++k) m[k] = m[k] * e.bm[k] + e.obm[k] * g;
+  rms = rms * e.br + e.obr * (g * g);
+}
+
+// The 18 per-element channels (ELO_CELO2_naive.py:180-215); rs = rsqrt(rms + eps_rs), rfcf_k =
+// row_factor_k * col_factor_k of the element's row and column.
+__device__ __forceinline__ void lo_features(float g, float p, const float (&m)[3], float rms,
+                                            const float (&rfcf)[3], float eps_rs, float (&f)[kNStat]) {
+  const float rs = rsq(rms + eps_rs);
+  f[0] = g;
+  f[1] = fminf(fmaxf(g, -0.1f), 0.1f);
+  f[2] = p;
+  f[3] = m[0]; f[4] = m[1]; f[5] = m[2];
+  f[6] = rms;
+  f[7] = m[0] * rs; f[8] = m[1] * rs; f[9] = m[2] * rs;
+  f[10] = rs;
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    f[11 + k] = g * rfcf[k];
+    f[15 + k] = m[k] * rfcf[k];
+  }
+  f[14] = g * rs;
+}
+
+// AdamW over the shared mom[0] / rms accumulators (ELO_CELO2_naive.py:296-302).
+template <int V>
+__device__ __forceinline__ void celo2_adam_chunk(const TDesc& d, const PyloTensorArgs& a, int chunk,
+                                                 float scale, const EmaConsts& e) {
+  const long long base = (long long)chunk * (kThreads * V * kElemIters);
+  const long long n = d.n;
+#pragma unroll 2
+  for (int it = 0; it < kElemIters; ++it) {
+    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
+    if (idx >= n) break;
+    float g[V], p[V], m0[V], m1[V], m2[V], r[V];
+    load_vec<V>(a.grad + idx, g);
+    load_vec<V>(a.param + idx, p);
+    load_vec<V>(a.mom + idx, m0);
+    load_vec<V>(a.mom + n + idx, m1);
+    load_vec<V>(a.mom + 2 * n + idx, m2);
+    load_vec<V>(a.rms + idx, r);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      const float gg = clampf(g[v] * scale, a.clip_val);
+      float m[3] = {m0[v], m1[v], m2[v]};
+      ema_update(e, gg, m, r[v]);
+      m0[v] = m[0]; m1[v] = m[1]; m2[v] = m[2];
+      const float mh = m[0] / a.bc1;
+      const float vh = r[v] / a.bc2;
+      const float upd = mh / (sqrtf(vh) + 1e-8f);
+      p[v] = fmaf(upd + a.weight_decay * p[v], -a.lr, p[v]);
+    }
+    store_vec<V>(a.mom + idx, m0);
+    store_vec<V>(a.mom + n + idx, m1);
+    store_vec<V>(a.mom + 2 * n + idx, m2);
+    store_vec<V>(a.rms + idx, r);
+    store_vec<V>(a.param + idx, p);
+  }
+}
+
+// One vector of V consecutive elements (same dim-0 index i0, dim-1 indices i1..i1+V-1).
+template <int V>
+struct ElemIn {
+  float g[V], p[V], m[V][3], rms[V];
+  float rfcf[V][3];
+  int i0, i1;
+};
+
+template <int V>
+__device__ __forceinline__ void load_elems(const TDesc& d, const PyloTensorArgs& a, long long idx,
+                                           float scale, const float* f0, const float* f1, ElemIn<V>& x) {
+  const long long n = d.n;
+  float m0[V], m1[V], m2[V];
+  load_vec<V>(a.grad + idx, x.g);
+  load_vec<V>(a.param + idx, x.p);
+  load_vec<V>(a.mom + idx, m0);
+  load_vec<V>(a.mom + n + idx, m1);
+  load_vec<V>(a.mom + 2 * n + idx, m2);
+  load_vec<V>(a.rms + idx, x.rms);
+  const unsigned u = (unsigned)idx;  // n < 2^31
+  x.i0 = (int)(u / (unsigned)d.C0);
+  x.i1 = (int)(u - (unsigned)x.i0 * (unsigned)d.C0);
+  const float4 fa = load_f4(f0 + (size_t)x.i0 * 4);
+  float fb[3][V];
+#pragma unroll
+  for (int k = 0; k < 3; ++k) load_vec<V>(f1 + (size_t)k * d.C0r + x.i1, fb[k]);
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    x.g[v] = clampf(x.g[v] * scale, a.clip_val);
+    x.m[v][0] = m0[v]; x.m[v][1] = m1[v]; x.m[v][2] = m2[v];
+    x.rfcf[v][0] = fa.x * fb[0][v];
+    x.rfcf[v][1] = fa.y * fb[1][v];
+    x.rfcf[v][2] = fa.z * fb[2][v];
+  }
+}
+
+template <int V>
+__device__ __forceinline__ void celo2_stats_chunk(const TDesc& d, const PyloTensorArgs& a, int chunk,
+                                                  float scale, const EmaConsts& e, const float* f0,
+                                                  const float* f1, float (&acc)[kNStat]) {
+  const long long base = (long long)chunk * (kThreads * V * kElemIters);
+#pragma unroll 2
+  for (int it = 0; it < kElemIters; ++it) {
+    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
+    if (idx >= d.n) break;
+    ElemIn<V> x;
+    load_elems<V>(d, a, idx, scale, f0, f1, x);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      ema_update(e, x.g[v], x.m[v], x.rms[v]);
+      float f[kNStat];
+      lo_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.rfcf[v], 1e-8f, f);
+#pragma unroll
+      for (int c = 0; c < kNStat; ++c) acc[c] = fmaf(f[c], f[c], acc[c]);
+    }
+  }
+}
+
+// Statistics pass: sum of squares of the 18 per-element channels of every MLP tensor, with the
+// accumulators advanced in registers only (nothing is written back).  AdamW tensors are updated
+// completely here.
+__global__ __launch_bounds__(kThreads) void k_celo2_stats(const TDesc* __restrict__ descs,
+                                                          const PyloTensorArgs* __restrict__ dyn,
+                                                          const Item* __restrict__ items,
+                                                          const float* __restrict__ fac0,
+                                                          const float* __restrict__ fac1,
+                                                          const Globals* __restrict__ gl, PyloDecays dec,
+                                                          double* __restrict__ stats_part) {
+  __shared__ float red[kWaves][kNStat];
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  const float scale = clip_scale(gl->gnorm, a.clip_norm);
+  const EmaConsts e = make_ema(dec);
+  if (d.mode == kModeFlat) {
+    if (d.vec == 4) celo2_adam_chunk<4>(d, a, it.a, scale, e);
+    else celo2_adam_chunk<1>(d, a, it.a, scale, e);
+    return;
+  }
+  float acc[kNStat];
+#pragma unroll
+  for (int c = 0; c < kNStat; ++c) acc[c] = 0.0f;
+  const float* f0 = fac0 + d.fac0_off;
+  const float* f1 = fac1 + d.fac1_off;
+  if (d.vec == 4) celo2_stats_chunk<4>(d, a, it.a, scale, e, f0, f1, acc);
+  else celo2_stats_chunk<1>(d, a, it.a, scale, e, f0, f1, acc);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int c = 0; c < kNStat; ++c) {
+    const float s = wave_sum(acc[c]);
+    if (lane == 0) red[wave][c] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x < kNStat) {
+    const int c = threadIdx.x;
+    stats_part[(size_t)blockIdx.x * kNStat + c] =
+        ((double)red[0][c] + (double)red[1][c]) + ((double)red[2][c] + (double)red[3][c]);
+  }
+}
+
+// Per factored tensor: s_c = rsqrt(1e-9 + mean f_c^2) folded into the first-layer rows of the 18
+// per-element channels; the remaining layers are copied behind them so the apply kernel reads one
+// contiguous block per tensor.
+__global__ __launch_bounds__(kFoldThreads) void k_celo2_fold(const TDesc* __restrict__ descs,
+                                                             const PyloTensorArgs* __restrict__ dyn,
+                                                             const int* __restrict__ fac_list,
+                                                             const double* __restrict__ stats_part,
+                                                             const float* __restrict__ mlp,
+                                                             float* __restrict__ wfold, float* __restrict__ chan_ms) {
+  constexpr int G = kFoldThreads / kNStat;  // 56 groups x 18 channels
+  __shared__ double part[G][kNStat];
+  __shared__ float scale_c[kNStat];
+  const int t = fac_list[blockIdx.x];
+  const TDesc d = descs[t];
+  if (dyn[t].grad == nullptr) return;
+  const int c = threadIdx.x % kNStat, gI = threadIdx.x / kNStat;
+  if (gI < G) {
+    double s = 0.0;
+#pragma unroll 4
+    for (int b = gI; b < d.nblk; b += G) s += stats_part[(size_t)(d.blk0 + b) * kNStat + c];
+    part[gI][c] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x < kNStat) {
+    double s = 0.0;
+    for (int g2 = 0; g2 < G; ++g2) s += part[g2][threadIdx.x];
+    const float ms = (float)(s / (double)d.n);
+    chan_ms[(size_t)d.fac_slot * kNStat + threadIdx.x] = ms;
+    scale_c[threadIdx.x] = rsq(1e-9f + ms);
+  }
+  __syncthreads();
+  float* w = wfold + (size_t)d.fac_slot * kC2Fold;
+  const float* w_in = mlp;                  // (30,8)
+  const float* w_h = mlp + 240 + 8;         // (8,8)
+  const float* b_h = w_h + 64;              // 8
+  const float* w_out = b_h + 8;             // (8,3)
+  const float* b_out = w_out + 24;          // 3
+  for (int i = threadIdx.x; i < kNStat * 8; i += kFoldThreads) {
+    const int cc = i / 8, j = i % 8;
+    w[kC2W1 + i] = w_in[stat_channel(cc) * 8 + j] * scale_c[cc];
+  }
+  for (int i = threadIdx.x; i < 64; i += kFoldThreads) w[kC2WH + i] = w_h[i];
+  for (int i = threadIdx.x; i < 8; i += kFoldThreads) w[kC2BH + i] = b_h[i];
+  for (int i = threadIdx.x; i < 16; i += kFoldThreads) w[kC2WO + i] = w_out[(i / 2) * 3 + (i % 2)];
+  for (int i = threadIdx.x; i < 2; i += kFoldThreads) w[kC2BO + i] = b_out[i];
+}
+
+template <int V>
+__device__ __forceinline__ void celo2_apply_chunk(const TDesc& d, const PyloTensorArgs& a, int chunk,
+                                                  float scale, const EmaConsts& e, const float* f0,
+                                                  const float* f1, const float* t0, const float* t1,
+                                                  const float* wbase) {
+  const long long base = (long long)chunk * (kThreads * V * kElemIters);
+  const long long n = d.n;
+  const bool use_exp = a.exp_mult != 0.0f;
+  for (int it = 0; it < kElemIters; ++it) {
+    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
+    if (idx >= n) break;
+    ElemIn<V> x;
+    load_elems<V>(d, a, idx, scale, f0, f1, x);
+    float f[V][kNStat], h[V][8];
+    float m0[V], m1[V], m2[V];
+    {
+      const float4 a0 = load_f4(t0 + (size_t)x.i0 * 8), a1 = load_f4(t0 + (size_t)x.i0 * 8 + 4);
+      const float ta[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float tb[V];
+        load_vec<V>(t1 + (size_t)j * d.C0r + x.i1, tb);
+#pragma unroll
+        for (int v = 0; v < V; ++v) h[v][j] = ta[j] + tb[v];
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      ema_update(e, x.g[v], x.m[v], x.rms[v]);
+      m0[v] = x.m[v][0]; m1[v] = x.m[v][1]; m2[v] = x.m[v][2];
+      lo_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.rfcf[v], 1e-8f, f[v]);
+    }
+    store_vec<V>(a.mom + idx, m0);
+    store_vec<V>(a.mom + n + idx, m1);
+    store_vec<V>(a.mom + 2 * n + idx, m2);
+    store_vec<V>(a.rms + idx, x.rms);
+    // The weights are wave-uniform: they are fetched through the scalar cache into SGPRs one input
+    // row at a time and shared by the P elements processed together (channel-outer loop order).
+    constexpr int P = V >= 2 ? 2 : 1;
+    float out[V];
+#pragma unroll
+    for (int v0 = 0; v0 < V; v0 += P) {
+      const cfloat* w = launder(wbase);
+#pragma unroll
+      for (int c = 0; c < kNStat; ++c) {
+        float wc[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) wc[j] = w[kC2W1 + c * 8 + j];
+#pragma unroll
+        for (int v = v0; v < v0 + P; ++v) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) h[v][j] = fmaf(f[v][c], wc[j], h[v][j]);
+        }
+      }
+      float h1[P][8];
+#pragma unroll
+      for (int q = 0; q < P; ++q) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { h[v0 + q][j] = fmaxf(h[v0 + q][j], 0.0f); h1[q][j] = w[kC2BH + j]; }
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        float wk[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) wk[j] = w[kC2WH + k * 8 + j];
+#pragma unroll
+        for (int q = 0; q < P; ++q) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) h1[q][j] = fmaf(h[v0 + q][k], wk[j], h1[q][j]);
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < P; ++q) {
+        float o0 = w[kC2BO + 0], o1 = w[kC2BO + 1];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const float hk = fmaxf(h1[q][k], 0.0f);
+          o0 = fmaf(hk, w[kC2WO + k * 2 + 0], o0);
+          if (use_exp) o1 = fmaf(hk, w[kC2WO + k * 2 + 1], o1);
+        }
+        out[v0 + q] = use_exp ? o0 * expf(o1 * a.exp_mult) : o0;
+      }
+    }
+    store_vec<V>(a.step_out + idx, out);
+  }
+}
+
+// Apply pass: accumulators advanced and written, features, MLP, raw step.
+__global__ __launch_bounds__(kThreads) void k_celo2_apply(const TDesc* __restrict__ descs,
+                                                          const PyloTensorArgs* __restrict__ dyn,
+                                                          const Item* __restrict__ items,
+                                                          const float* __restrict__ fac0,
+                                                          const float* __restrict__ fac1,
+                                                          const float* __restrict__ term0,
+                                                          const float* __restrict__ term1,
+                                                          const Globals* __restrict__ gl, PyloDecays dec,
+                                                          const float* __restrict__ wfold) {
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  if (d.mode == kModeFlat) return;
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  const float scale = clip_scale(gl->gnorm, a.clip_norm);
+  const EmaConsts e = make_ema(dec);
+  const float* w = wfold + (size_t)d.fac_slot * kC2Fold;
+  if (d.vec == 4)
+    celo2_apply_chunk<4>(d, a, it.a, scale, e, fac0 + d.fac0_off, fac1 + d.fac1_off, term0 + d.term0_off,
+                         term1 + d.term1_off, w);
+  else
+    celo2_apply_chunk<1>(d, a, it.a, scale, e, fac0 + d.fac0_off, fac1 + d.fac1_off, term0 + d.term0_off,
+                         term1 + d.term1_off, w);
+}
+
+}  // namespace pylo

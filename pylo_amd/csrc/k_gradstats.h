@@ -1,0 +1,303 @@
+// Gradient statistics shared by the three optimizers: row / column sums of g^2 (P0), the global
+// gradient norm, and the Adafactor row / column vectors with everything derived from them (V0).
+#pragma once
+
+#include "pylo_common.h"
+
+namespace pylo {
+
+// =============================================================================================
+// P0: row / column sums of g^2 for 2-D factored tensors; sum g^2 and clamp flag for everything
+// =============================================================================================
+template <int V>
+__device__ __forceinline__ void p0_factored(const TDesc& d, const float* g, int strip, int cb, bool exact,
+                                            float scale, float clipv, float* __restrict__ rowpart,
+                                            float* __restrict__ colpart, float* lds_col, float* lds_row,
+                                            float& gsq, int& flag) {
+  constexpr int TC = 64 * V;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int C0 = d.C0, R0 = d.R0;
+  const int r0 = strip * kP0Rows;
+  const int r1 = min(R0, r0 + kP0Rows);
+  const int c = cb * TC + lane * V;
+  const bool in = c < C0;  // V == 4 implies C0 % 4 == 0, so the whole vector is in or out
+  float col[V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) col[v] = 0.0f;
+  for (int r = r0 + wave; r < r1; r += kWaves) {
+    float x[V];
+    if (in) {
+      load_vec<V>(g + (size_t)r * C0 + c, x);
+    } else {
+#pragma unroll
+      for (int v = 0; v < V; ++v) x[v] = 0.0f;
+    }
+    float rs = 0.0f;
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      const float raw = x[v];
+      gsq = fmaf(raw, raw, gsq);
+      if (!exact) flag |= (fabsf(raw) > clipv && clipv > 0.0f) ? 1 : 0;
+      const float y = exact ? clampf(raw * scale, clipv) : raw;
+      const float sq = y * y;
+      col[v] += sq;
+      rs += sq;
+    }
+    rs = wave_sum(rs);
+    if (lane == 0) lds_row[r - r0] = rs;
+  }
+#pragma unroll
+  for (int v = 0; v < V; ++v) lds_col[wave * TC + lane * V + v] = col[v];
+  __syncthreads();
+  for (int j = threadIdx.x; j < TC; j += kThreads) {
+    const float s = ((lds_col[j] + lds_col[TC + j]) + lds_col[2 * TC + j]) + lds_col[3 * TC + j];
+    const int cc = cb * TC + j;
+    if (cc < C0) colpart[(size_t)strip * C0 + cc] = s;
+  }
+  for (int j = threadIdx.x; j < r1 - r0; j += kThreads) rowpart[(size_t)cb * R0 + r0 + j] = lds_row[j];
+}
+
+template <int V>
+__device__ __forceinline__ void p0_flat(const TDesc& d, const float* g, int chunk, float clipv,
+                                        float& gsq, int& flag) {
+  const long long base = (long long)chunk * (kThreads * V * kElemIters);
+#pragma unroll
+  for (int it = 0; it < kElemIters; ++it) {
+    const long long e = base + (long long)(it * kThreads + threadIdx.x) * V;
+    if (e < d.n) {
+      float x[V];
+      load_vec<V>(g + e, x);
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        gsq = fmaf(x[v], x[v], gsq);
+        flag |= (fabsf(x[v]) > clipv && clipv > 0.0f) ? 1 : 0;
+      }
+    }
+  }
+}
+
+// pass 0: tensors with clip_norm > 0 are summed raw (the scale factors out of g^2) and flag
+//         elements beyond the clamp; tensors without global-norm clipping are clamped directly.
+// pass 1: only if the flag was raised: redo clip_norm > 0 tensors with scale and clamp applied.
+__global__ __launch_bounds__(kThreads) void k_p0(const TDesc* __restrict__ descs,
+                                                 const PyloTensorArgs* __restrict__ dyn,
+                                                 const Item* __restrict__ items,
+                                                 float* __restrict__ rowpart, float* __restrict__ colpart,
+                                                 double* __restrict__ gsq_part, int* __restrict__ flag_part,
+                                                 const Globals* __restrict__ gl, int pass) {
+  __shared__ float lds_col[kWaves * 256];
+  __shared__ float lds_row[kP0Rows];
+  __shared__ float lds_red[kWaves];
+  __shared__ int lds_flag[kWaves];
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  const bool clip_on = a.clip_norm > 0.0f;
+  if (pass == 1 && (!clip_on || d.mode == kModeFlat || gl->flag == 0)) return;
+  float gsq = 0.0f;
+  int flag = 0;
+  if (a.grad != nullptr) {
+    if (d.mode == kModeFac2D) {
+      const bool exact = (pass == 1) || !clip_on;
+      const float scale = (pass == 1) ? clip_scale(gl->gnorm, a.clip_norm) : 1.0f;
+      if (d.vec == 4)
+        p0_factored<4>(d, a.grad, it.a, it.b, exact, scale, a.clip_val, rowpart + d.rowpart_off,
+                       colpart + d.colpart_off, lds_col, lds_row, gsq, flag);
+      else
+        p0_factored<1>(d, a.grad, it.a, it.b, exact, scale, a.clip_val, rowpart + d.rowpart_off,
+                       colpart + d.colpart_off, lds_col, lds_row, gsq, flag);
+    } else {
+      if (d.vec == 4) p0_flat<4>(d, a.grad, it.a, a.clip_val, gsq, flag);
+      else p0_flat<1>(d, a.grad, it.a, a.clip_val, gsq, flag);
+    }
+  }
+  if (pass == 1) return;
+  gsq = wave_sum(gsq);
+  flag = __any(flag) ? 1 : 0;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) { lds_red[wave] = gsq; lds_flag[wave] = flag; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    gsq_part[blockIdx.x] = ((double)lds_red[0] + (double)lds_red[1]) + ((double)lds_red[2] + (double)lds_red[3]);
+    flag_part[blockIdx.x] = (clip_on && (lds_flag[0] | lds_flag[1] | lds_flag[2] | lds_flag[3])) ? 1 : 0;
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void k_gnorm(const double* __restrict__ gsq_part,
+                                                    const int* __restrict__ flag_part, int nblk,
+                                                    Globals* __restrict__ gl) {
+  __shared__ double red[kWaves];
+  __shared__ int fred[kWaves];
+  double s = 0.0;
+  int f = 0;
+  for (int i = threadIdx.x; i < nblk; i += kThreads) { s += gsq_part[i]; f |= flag_part[i]; }
+  s = wave_sum(s);
+  f = __any(f) ? 1 : 0;
+  if ((threadIdx.x & 63) == 0) { red[threadIdx.x >> 6] = s; fred[threadIdx.x >> 6] = f; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    gl->gnorm = (float)sqrt((red[0] + red[1]) + (red[2] + red[3]));
+    gl->flag = fred[0] | fred[1] | fred[2] | fred[3];
+  }
+}
+
+// =============================================================================================
+// V0a: one block per 64 entries of a row / column vector.  Finishes the sums of g^2 over the
+// partials, advances the three Adafactor accumulators (ELO_CELO2_naive.py:152-160) and leaves
+// per-block partial sums of  f, f^2, rsqrt(f+1e-8)^2  per decay.
+// =============================================================================================
+__global__ __launch_bounds__(kThreads) void k_v0a(const TDesc* __restrict__ descs,
+                                                  const PyloTensorArgs* __restrict__ dyn,
+                                                  const Item* __restrict__ items,
+                                                  const float* __restrict__ rowpart,
+                                                  const float* __restrict__ colpart,
+                                                  const Globals* __restrict__ gl, PyloDecays dec,
+                                                  double* __restrict__ v0part) {
+  __shared__ double lds[kWaves][kV0aEnt];
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  const int which = it.b;
+  const int len = which ? d.C0 : d.R0;       // entries of this vector
+  const int other = which ? d.R0 : d.C0;     // the dim that was summed over
+  const int npart = which ? d.n_strips : d.n_colblk;
+  const float* part = which ? colpart + d.colpart_off : rowpart + d.rowpart_off;
+  const int e = threadIdx.x & 63, grp = threadIdx.x >> 6;
+  const int i = it.a * kV0aEnt + e;
+  {
+    double s = 0.0;
+    if (i < len)
+      for (int q = grp; q < npart; q += kWaves) s += (double)part[(size_t)q * len + i];
+    lds[grp][e] = s;
+  }
+  __syncthreads();
+  const int k = grp;  // waves 0..2 take one decay each
+  if (k >= 3) return;
+  double s2 = 1.0;
+  if (a.clip_norm > 0.0f && gl->flag == 0) {
+    const float sc = clip_scale(gl->gnorm, a.clip_norm);
+    s2 = (double)sc * (double)sc;
+  }
+  const bool is_r = (which == 0) == (d.r_is_dim0 != 0);
+  float* fac = is_r ? a.fac_r : a.fac_c;
+  double s_f = 0.0, s_ff = 0.0, s_rr = 0.0;
+  if (i < len) {
+    const double S = ((lds[0][e] + lds[1][e]) + lds[2][e]) + lds[3][e];
+    const float q = (float)(s2 * S / (double)other) + 1e-30f;
+    const float beta = dec.beta_fac[k];
+    const float f = beta * fac[(size_t)k * len + i] + (1.0f - beta) * q;
+    fac[(size_t)k * len + i] = f;
+    const float rq = rsq(f + 1e-8f);
+    s_f = (double)f;
+    s_ff = (double)f * (double)f;
+    s_rr = (double)rq * (double)rq;
+  }
+  s_f = wave_sum(s_f);
+  s_ff = wave_sum(s_ff);
+  s_rr = wave_sum(s_rr);
+  if (e == 0) {
+    double* o = v0part + (size_t)blockIdx.x * kNV0 + k * 3;
+    o[0] = s_f; o[1] = s_ff; o[2] = s_rr;
+  }
+}
+
+// =============================================================================================
+// V0b: one block per 1024 entries of a row / column vector.  Reduces the V0a partials of its
+// tensor, then writes the factor tables (row_factor / col_factor, ELO_CELO2_naive.py:161-164)
+// and, when first-layer weights are given, the per-row / per-column MLP terms: the 12 feature
+// channels that depend on the row or on the column only (fac_r_k, fac_c_k and their rsqrt) are
+// normalised and pushed through the first layer once per row / column instead of once per element.
+//   w1: (30, H) row-major, (in, out); b1: (H).  Bias goes into the dim-0 terms.
+// =============================================================================================
+template <int H>
+__global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ descs,
+                                                  const PyloTensorArgs* __restrict__ dyn,
+                                                  const Item* __restrict__ items,
+                                                  const double* __restrict__ v0part, float norm_eps,
+                                                  const float* __restrict__ w1, const float* __restrict__ b1,
+                                                  float* __restrict__ fac0, float* __restrict__ fac1,
+                                                  float* __restrict__ term0, float* __restrict__ term1,
+                                                  BScale* __restrict__ bscale) {
+  constexpr int G = 14;  // 14 groups x 18 (vector, slot) pairs = 252 threads
+  __shared__ double red[G][2 * kNV0];
+  __shared__ double tot[2 * kNV0];
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  {
+    const int pair = threadIdx.x % (2 * kNV0), gI = threadIdx.x / (2 * kNV0);
+    if (gI < G) {
+      const int vecI = pair / kNV0, slot = pair % kNV0;
+      double s = 0.0;
+      for (int b = gI; b < d.v0a_n[vecI]; b += G) s += v0part[(size_t)(d.v0a_first[vecI] + b) * kNV0 + slot];
+      red[gI][pair] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x < 2 * kNV0) {
+      double s = 0.0;
+      for (int g2 = 0; g2 < G; ++g2) s += red[g2][threadIdx.x];
+      tot[threadIdx.x] = s;
+    }
+    __syncthreads();
+  }
+  // sums of the r-role vector and of the c-role vector
+  const double* tr = tot + (d.r_is_dim0 ? 0 : kNV0);
+  const double* tc = tot + (d.r_is_dim0 ? kNV0 : 0);
+  float rcm[3], s_fr[3], s_rr[3], s_fc[3], s_rc[3];
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    rcm[k] = (float)(tr[k * 3 + 0] / (double)d.len_r);
+    s_fr[k] = rsq(norm_eps + (float)(tr[k * 3 + 1] / (double)d.len_r));
+    s_rr[k] = rsq(norm_eps + (float)(tr[k * 3 + 2] / (double)d.len_r));
+    s_fc[k] = rsq(norm_eps + (float)(tc[k * 3 + 1] / (double)d.len_c));
+    s_rc[k] = rsq(norm_eps + (float)(tc[k * 3 + 2] / (double)d.len_c));
+  }
+  const int which = it.b;
+  const bool is_r = (which == 0) == (d.r_is_dim0 != 0);
+  if (which == 0 && it.a == 0 && threadIdx.x == 0) {
+    BScale bs;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      bs.s[k] = s_fr[k]; bs.s[3 + k] = s_fc[k]; bs.s[6 + k] = s_rr[k]; bs.s[9 + k] = s_rc[k];
+      bs.rcm[k] = rcm[k];
+    }
+    bs.pad_ = 0.0f;
+    bscale[d.fac_slot] = bs;
+  }
+  const int len = which ? d.C0 : d.R0;
+  const float* fac = is_r ? a.fac_r : a.fac_c;
+  // channel rows of the first layer this vector feeds: accumulator value, rsqrt(value + 1e-8)
+  const int ch_f = is_r ? 15 : 18, ch_q = is_r ? 21 : 24;
+  for (int i = it.a * kV0bEnt + threadIdx.x; i < min(len, (it.a + 1) * kV0bEnt); i += kThreads) {
+    float fct[3], x0[3], x1[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      const float f = fac[(size_t)k * len + i];
+      fct[k] = is_r ? rsq(fmaxf(f / (rcm[k] + 1e-9f), 1e-9f)) : rsq(fmaxf(f, 1e-9f));
+      x0[k] = f * (is_r ? s_fr[k] : s_fc[k]);
+      x1[k] = rsq(f + 1e-8f) * (is_r ? s_rr[k] : s_rc[k]);
+    }
+    if (which == 0) store_f4(fac0 + d.fac0_off + (size_t)i * 4, fct[0], fct[1], fct[2], 0.0f);
+    else {
+#pragma unroll
+      for (int k = 0; k < 3; ++k) fac1[d.fac1_off + (size_t)k * d.C0r + i] = fct[k];
+    }
+    if (w1 != nullptr) {
+#pragma unroll
+      for (int j = 0; j < H; ++j) {
+        float t = (which == 0) ? b1[j] : 0.0f;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+          t = fmaf(x0[k], w1[(ch_f + k) * H + j], t);
+          t = fmaf(x1[k], w1[(ch_q + k) * H + j], t);
+        }
+        if (which == 0) term0[d.term0_off + (size_t)i * H + j] = t;
+        else term1[d.term1_off + (size_t)j * d.C0r + i] = t;
+      }
+    }
+  }
+}
+
+}  // namespace pylo

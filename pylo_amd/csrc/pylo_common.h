@@ -17,9 +17,10 @@ constexpr int kP0Rows = 128;    // rows of one row/column-sum tile; tile columns
 constexpr int kElemIters = 8;   // an element chunk is kThreads * vec * kElemIters elements
 constexpr int kNStat = 18;      // feature channels that vary per element (the other 12 are
                                 // functions of the row or of the column only)
-constexpr int kTabW = 12;       // floats per row/column table entry: 3 factors, pad, 8 MLP terms
-constexpr int kV0Threads = 1024;
-constexpr int kNV0Sums = 15;
+constexpr int kV0aEnt = 64;     // vector entries per k_v0a block
+constexpr int kV0bEnt = 1024;   // vector entries per k_v0b block
+constexpr int kNV0 = 9;         // partial sums per k_v0a block
+constexpr int kFoldThreads = 1024;
 
 // Per-element channels, as indices into the reference's 30-channel order
 // (pylo/csrc/celo2_kernel.cu:86-124): g, clip(g), p, m0..2, rms, m_k*rs, rs, g*rf_k*cf_k, g*rs,
@@ -37,26 +38,36 @@ struct TDesc {
   int mode;        // kModeFlat: no factored statistics (CELO2 AdamW tensors); kModeFac2D: 2-D factored
   int vec;         // 4: 128-bit loads (row length % 4 == 0); 1: dword loads
   int R0, C0;      // sizes of dim 0 / dim 1
+  int C0r;         // C0 rounded up to a multiple of 4 (row pitch of the dim-1 tables)
   int r_is_dim0;   // fac_r / row_factor are indexed by the dim-0 coordinate (largest dim is dim 1)
   int len_r, len_c;
   int n_strips, n_colblk;
-  long long rowpart_off, colpart_off;  // floats
-  long long rtab_off, ctab_off;        // table entries
   int blk0, nblk;  // range of element-chunk blocks (rows of the statistics partials)
   int fac_slot;    // index among factored tensors
-  int pad_;
+  long long rowpart_off, colpart_off;  // floats
+  long long fac0_off, fac1_off;        // floats: dim-0 factors [R0][4], dim-1 factors [3][C0r]
+  long long term0_off, term1_off;      // floats: dim-0 terms [R0][H], dim-1 terms [H][C0r]
+  int v0a_first[2], v0a_n[2];          // k_v0a blocks of the dim-0 / dim-1 vector
 };
 
 struct Item {
   int tensor;
-  int a;  // P0: strip (or flat chunk); element kernels: chunk
-  int b;  // P0: column block
+  int a;  // P0: strip (or flat chunk); element kernels: chunk; V0: chunk
+  int b;  // P0: column block; V0: 0 = dim-0 vector, 1 = dim-1 vector
   int pad_;
 };
 
 struct Globals {
   float gnorm;  // ||all grads||_2
   int flag;     // some |g| exceeded clip_val on a tensor whose sums were taken un-clamped
+};
+
+// Per factored tensor, written by k_v0b: normalisation scales of the 12 broadcast channels in the
+// reference's channel order 15..26 (fac_r_k, fac_c_k, rsqrt(fac_r_k+1e-8), rsqrt(fac_c_k+1e-8)).
+struct BScale {
+  float s[12];
+  float rcm[3];
+  float pad_;
 };
 
 // ---- device helpers ---------------------------------------------------------------------------
@@ -84,34 +95,54 @@ __device__ __forceinline__ float clip_scale(float gnorm, float clip_norm) {
   return denom > 0.0f ? clip_norm / denom : 1.0f;
 }
 
-template <int V>
-struct VecT;
-template <>
-struct VecT<4> {
-  using type = float4;
-};
-template <>
-struct VecT<1> {
-  using type = float;
-};
+// 1/sqrt(x) for x in the normal range (callers add an epsilon >= 1e-9 first): v_rsq_f32, 1 ulp.
+__device__ __forceinline__ float rsq(float x) { return __builtin_amdgcn_rsqf(x); }
+
+// Tensor pointers come out of a table in memory, so the compiler cannot infer their address
+// space; these casts say "global" and turn flat_load/flat_store into global_load/global_store.
+typedef __attribute__((address_space(1))) float gfloat;
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) v4f gv4f;
 
 template <int V>
-__device__ __forceinline__ void load_vec(const float* __restrict__ p, float (&x)[V]) {
+__device__ __forceinline__ void load_vec(const float* p, float (&x)[V]) {
   if constexpr (V == 4) {
-    float4 t = *reinterpret_cast<const float4*>(p);
+    const v4f t = *(const gv4f*)(p);
     x[0] = t.x; x[1] = t.y; x[2] = t.z; x[3] = t.w;
   } else {
-    x[0] = *p;
+    x[0] = *(const gfloat*)(p);
   }
 }
 
 template <int V>
-__device__ __forceinline__ void store_vec(float* __restrict__ p, const float (&x)[V]) {
+__device__ __forceinline__ void store_vec(float* p, const float (&x)[V]) {
   if constexpr (V == 4) {
-    *reinterpret_cast<float4*>(p) = make_float4(x[0], x[1], x[2], x[3]);
+    v4f t;
+    t.x = x[0]; t.y = x[1]; t.z = x[2]; t.w = x[3];
+    *(gv4f*)(p) = t;
   } else {
-    *p = x[0];
+    *(gfloat*)(p) = x[0];
   }
+}
+
+__device__ __forceinline__ float4 load_f4(const float* p) {
+  const v4f t = *(const gv4f*)(p);
+  return make_float4(t.x, t.y, t.z, t.w);
+}
+
+__device__ __forceinline__ void store_f4(float* p, float a, float b, float c, float d) {
+  v4f t;
+  t.x = a; t.y = b; t.z = c; t.w = d;
+  *(gv4f*)(p) = t;
+}
+
+// Makes the compiler forget what it knows about a (wave-uniform) pointer, so loads through it
+// are re-issued where they are written instead of being hoisted out of the enclosing loop; the
+// result points to memory that is read-only for the life of the kernel (scalar loads).
+typedef __attribute__((address_space(4))) float cfloat;
+__device__ __forceinline__ const cfloat* launder(const float* p) {
+  asm volatile("" : "+s"(p));
+  return (const cfloat*)p;
 }
 
 }  // namespace pylo

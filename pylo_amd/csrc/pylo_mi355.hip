@@ -1,11 +1,12 @@
-// Fused learned-optimizer step for MI355X (gfx950): kernels and the C ABI of include/pylo_mi355.h.
+// Fused learned-optimizer step for MI355X (gfx950): the C ABI of include/pylo_mi355.h.
 //
-// Pipeline of one ELO-CELO2 step over all tensors of a plan (7 launches, no host sync):
+// Pipeline of one ELO-CELO2 step over all tensors of a plan (8 launches, no host sync):
 //   k_p0 (pass 0)   row / column sums of g^2 per tile, sum g^2 and clamp flag per block     4 B/elem
 //   k_gnorm         global gradient norm, clamp flag
 //   k_p0 (pass 1)   exits at once unless some |g| exceeded the clamp: redoes the sums exactly
-//   k_v0            per factored tensor: fac_r/fac_c EMAs, row/col factors, the 12 row-only /
-//                   column-only feature channels folded into 8-float MLP terms per row / column
+//   k_v0a           fac_r / fac_c EMAs per 64 vector entries, partial sums of their statistics
+//   k_v0b           row / column factor tables; the 12 row-only / column-only feature channels
+//                   normalised and folded into 8-float first-layer terms per row / column
 //   k_celo2_stats   sum of squares of the 18 per-element channels (accumulators advanced in
 //                   registers, nothing written); AdamW tensors are fully updated here      24 B/elem
 //   k_celo2_fold    per tensor: normalisation scales folded into the first-layer weights
@@ -15,618 +16,9 @@
 #include <cstring>
 #include <vector>
 
+#include "k_celo2.h"
+#include "k_gradstats.h"
 #include "pylo_common.h"
-
-namespace pylo {
-
-// =============================================================================================
-// P0: row / column sums of g^2 for 2-D factored tensors; sum g^2 and clamp flag for everything
-// =============================================================================================
-template <int V>
-__device__ __forceinline__ void p0_factored(const TDesc& d, const float* __restrict__ g, int strip,
-                                            int cb, bool exact, float scale, float clipv,
-                                            float* __restrict__ rowpart, float* __restrict__ colpart,
-                                            float* lds_col, float* lds_row, float& gsq, int& flag) {
-  constexpr int TC = 64 * V;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int C0 = d.C0, R0 = d.R0;
-  const int r0 = strip * kP0Rows;
-  const int r1 = min(R0, r0 + kP0Rows);
-  const int c = cb * TC + lane * V;
-  const bool in = c < C0;  // V == 4 implies C0 % 4 == 0, so the whole vector is in or out
-  float col[V];
-#pragma unroll
-  for (int v = 0; v < V; ++v) col[v] = 0.0f;
-  for (int r = r0 + wave; r < r1; r += kWaves) {
-    float x[V];
-    if (in) {
-      load_vec<V>(g + (size_t)r * C0 + c, x);
-    } else {
-#pragma unroll
-      for (int v = 0; v < V; ++v) x[v] = 0.0f;
-    }
-    float rs = 0.0f;
-#pragma unroll
-    for (int v = 0; v < V; ++v) {
-      const float raw = x[v];
-      gsq += raw * raw;
-      if (!exact) flag |= (fabsf(raw) > clipv && clipv > 0.0f) ? 1 : 0;
-      const float y = exact ? clampf(raw * scale, clipv) : raw;
-      const float sq = y * y;
-      col[v] += sq;
-      rs += sq;
-    }
-    rs = wave_sum(rs);
-    if (lane == 0) lds_row[r - r0] = rs;
-  }
-#pragma unroll
-  for (int v = 0; v < V; ++v) lds_col[wave * TC + lane * V + v] = col[v];
-  __syncthreads();
-  for (int j = threadIdx.x; j < TC; j += kThreads) {
-    const float s = ((lds_col[j] + lds_col[TC + j]) + lds_col[2 * TC + j]) + lds_col[3 * TC + j];
-    const int cc = cb * TC + j;
-    if (cc < C0) colpart[(size_t)strip * C0 + cc] = s;
-  }
-  for (int j = threadIdx.x; j < r1 - r0; j += kThreads) rowpart[(size_t)cb * R0 + r0 + j] = lds_row[j];
-}
-
-template <int V>
-__device__ __forceinline__ void p0_flat(const TDesc& d, const float* __restrict__ g, int chunk,
-                                        float clipv, float& gsq, int& flag) {
-  const long long base = (long long)chunk * (kThreads * V * kElemIters);
-#pragma unroll
-  for (int it = 0; it < kElemIters; ++it) {
-    const long long e = base + (long long)(it * kThreads + threadIdx.x) * V;
-    if (e < d.n) {
-      float x[V];
-      load_vec<V>(g + e, x);
-#pragma unroll
-      for (int v = 0; v < V; ++v) {
-        gsq += x[v] * x[v];
-        flag |= (fabsf(x[v]) > clipv && clipv > 0.0f) ? 1 : 0;
-      }
-    }
-  }
-}
-
-// pass 0: tensors with clip_norm > 0 are summed raw (the scale factors out of g^2) and flag
-//         elements beyond the clamp; tensors without global-norm clipping are clamped directly.
-// pass 1: only if the flag was raised: redo clip_norm > 0 tensors with scale and clamp applied.
-__global__ __launch_bounds__(kThreads) void k_p0(const TDesc* __restrict__ descs,
-                                                 const PyloTensorArgs* __restrict__ dyn,
-                                                 const Item* __restrict__ items,
-                                                 float* __restrict__ rowpart, float* __restrict__ colpart,
-                                                 double* __restrict__ gsq_part, int* __restrict__ flag_part,
-                                                 const Globals* __restrict__ gl, int pass) {
-  __shared__ float lds_col[kWaves * 256];
-  __shared__ float lds_row[kP0Rows];
-  __shared__ float lds_red[kWaves];
-  __shared__ int lds_flag[kWaves];
-  const Item it = items[blockIdx.x];
-  const TDesc d = descs[it.tensor];
-  const PyloTensorArgs a = dyn[it.tensor];
-  const bool clip_on = a.clip_norm > 0.0f;
-  if (pass == 1 && (!clip_on || d.mode == kModeFlat || gl->flag == 0)) return;
-  float gsq = 0.0f;
-  int flag = 0;
-  if (a.grad != nullptr) {
-    if (d.mode == kModeFac2D) {
-      const bool exact = (pass == 1) || !clip_on;
-      const float scale = (pass == 1) ? clip_scale(gl->gnorm, a.clip_norm) : 1.0f;
-      if (d.vec == 4)
-        p0_factored<4>(d, a.grad, it.a, it.b, exact, scale, a.clip_val, rowpart + d.rowpart_off,
-                       colpart + d.colpart_off, lds_col, lds_row, gsq, flag);
-      else
-        p0_factored<1>(d, a.grad, it.a, it.b, exact, scale, a.clip_val, rowpart + d.rowpart_off,
-                       colpart + d.colpart_off, lds_col, lds_row, gsq, flag);
-    } else {
-      if (d.vec == 4) p0_flat<4>(d, a.grad, it.a, a.clip_val, gsq, flag);
-      else p0_flat<1>(d, a.grad, it.a, a.clip_val, gsq, flag);
-    }
-  }
-  if (pass == 1) return;
-  gsq = wave_sum(gsq);
-  flag = __any(flag) ? 1 : 0;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (lane == 0) { lds_red[wave] = gsq; lds_flag[wave] = flag; }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    gsq_part[blockIdx.x] = ((double)lds_red[0] + (double)lds_red[1]) + ((double)lds_red[2] + (double)lds_red[3]);
-    flag_part[blockIdx.x] = (clip_on && (lds_flag[0] | lds_flag[1] | lds_flag[2] | lds_flag[3])) ? 1 : 0;
-  }
-}
-
-__global__ __launch_bounds__(kThreads) void k_gnorm(const double* __restrict__ gsq_part,
-                                                    const int* __restrict__ flag_part, int nblk,
-                                                    Globals* __restrict__ gl) {
-  __shared__ double red[kWaves];
-  __shared__ int fred[kWaves];
-  double s = 0.0;
-  int f = 0;
-  for (int i = threadIdx.x; i < nblk; i += kThreads) { s += gsq_part[i]; f |= flag_part[i]; }
-  s = wave_sum(s);
-  f = __any(f) ? 1 : 0;
-  if ((threadIdx.x & 63) == 0) { red[threadIdx.x >> 6] = s; fred[threadIdx.x >> 6] = f; }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    gl->gnorm = (float)sqrt((red[0] + red[1]) + (red[2] + red[3]));
-    gl->flag = fred[0] | fred[1] | fred[2] | fred[3];
-  }
-}
-
-// =============================================================================================
-// V0: per factored tensor, everything that lives on a row vector or a column vector
-// =============================================================================================
-struct V0Consts {  // reference epsilons per optimizer kind
-  float norm_eps;  // second-moment normaliser: 1e-9 CELO2 (CELO2_naive.py:54), 1e-5 VeLO / AdafacLO
-};
-
-__device__ __forceinline__ void block_sum_doubles(double (&acc)[kNV0Sums], double* lds /*[16][kNV0Sums]*/,
-                                                  double* out /*[kNV0Sums]*/) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-  for (int i = 0; i < kNV0Sums; ++i) {
-    const double s = wave_sum(acc[i]);
-    if (lane == 0) lds[wave * kNV0Sums + i] = s;
-  }
-  __syncthreads();
-  if (threadIdx.x < kNV0Sums) {
-    double s = 0.0;
-    for (int w = 0; w < kV0Threads / 64; ++w) s += lds[w * kNV0Sums + threadIdx.x];
-    out[threadIdx.x] = s;
-  }
-  __syncthreads();
-}
-
-// Sum indices: 0-2 sum fac_r_k, 3-5 sum fac_r_k^2, 6-8 sum rsqrt(fac_r_k+1e-8)^2,
-//              9-11 sum fac_c_k^2, 12-14 sum rsqrt(fac_c_k+1e-8)^2.
-//
-// in_w: first-layer weights (in, out) with `ld` outputs per input row; channels 15..26 of the
-// 30-channel order are the row-only / column-only ones.  For each row-vector entry the table holds
-// {rf_0..2, 0, A_0..7} with A_j = sum_k w[15+k][j] * fac_r_k * s + w[21+k][j] * rsqrt(fac_r_k+1e-8) * s',
-// and for each column-vector entry {cf_0..2, 0, B_0..7} with B_j = bias_j + the fac_c terms.
-__global__ __launch_bounds__(kV0Threads) void k_v0(const TDesc* __restrict__ descs,
-                                                   const PyloTensorArgs* __restrict__ dyn,
-                                                   const int* __restrict__ fac_list,
-                                                   const float* __restrict__ rowpart,
-                                                   const float* __restrict__ colpart,
-                                                   const Globals* __restrict__ gl, PyloDecays dec,
-                                                   const float* __restrict__ w_in /*(30,8)*/,
-                                                   const float* __restrict__ b_in /*8*/, float norm_eps,
-                                                   float* __restrict__ rtab, float* __restrict__ ctab) {
-  __shared__ double lds[(kV0Threads / 64) * kNV0Sums];
-  __shared__ double sums[kNV0Sums];
-  const int t = fac_list[blockIdx.x];
-  const TDesc d = descs[t];
-  const PyloTensorArgs a = dyn[t];
-  if (a.grad == nullptr) return;
-  double s2 = 1.0;
-  if (a.clip_norm > 0.0f && gl->flag == 0) {
-    const float sc = clip_scale(gl->gnorm, a.clip_norm);
-    s2 = (double)sc * (double)sc;
-  }
-  float beta[3], omb[3];
-#pragma unroll
-  for (int k = 0; k < 3; ++k) { beta[k] = dec.beta_fac[k]; omb[k] = 1.0f - dec.beta_fac[k]; }
-
-  double acc[kNV0Sums];
-#pragma unroll
-  for (int i = 0; i < kNV0Sums; ++i) acc[i] = 0.0;
-
-  // ---- phase 1: advance the accumulators (ELO_CELO2_naive.py:152-160)
-  // dim-0 vector: mean over dim 1 of g^2, from the row partials of every column block
-  {
-    float* fac = d.r_is_dim0 ? a.fac_r : a.fac_c;
-    const float* rp = rowpart + d.rowpart_off;
-    for (int i = threadIdx.x; i < d.R0; i += kV0Threads) {
-      double s = 0.0;
-      for (int cb = 0; cb < d.n_colblk; ++cb) s += (double)rp[(size_t)cb * d.R0 + i];
-      const float q = (float)(s2 * s / (double)d.C0) + 1e-30f;
-#pragma unroll
-      for (int k = 0; k < 3; ++k) {
-        const float f = beta[k] * fac[(size_t)k * d.R0 + i] + omb[k] * q;
-        fac[(size_t)k * d.R0 + i] = f;
-        const float rq = rsqrtf(f + 1e-8f);
-        if (d.r_is_dim0) {
-          acc[k] += (double)f; acc[3 + k] += (double)f * f; acc[6 + k] += (double)rq * rq;
-        } else {
-          acc[9 + k] += (double)f * f; acc[12 + k] += (double)rq * rq;
-        }
-      }
-    }
-  }
-  // dim-1 vector: mean over dim 0, from the column partials of every strip
-  {
-    float* fac = d.r_is_dim0 ? a.fac_c : a.fac_r;
-    const float* cp = colpart + d.colpart_off;
-    for (int i = threadIdx.x; i < d.C0; i += kV0Threads) {
-      double s = 0.0;
-      for (int st = 0; st < d.n_strips; ++st) s += (double)cp[(size_t)st * d.C0 + i];
-      const float q = (float)(s2 * s / (double)d.R0) + 1e-30f;
-#pragma unroll
-      for (int k = 0; k < 3; ++k) {
-        const float f = beta[k] * fac[(size_t)k * d.C0 + i] + omb[k] * q;
-        fac[(size_t)k * d.C0 + i] = f;
-        const float rq = rsqrtf(f + 1e-8f);
-        if (!d.r_is_dim0) {
-          acc[k] += (double)f; acc[3 + k] += (double)f * f; acc[6 + k] += (double)rq * rq;
-        } else {
-          acc[9 + k] += (double)f * f; acc[12 + k] += (double)rq * rq;
-        }
-      }
-    }
-  }
-  block_sum_doubles(acc, lds, sums);
-
-  // ---- phase 2: scales of the 12 broadcast channels, row_col_mean
-  float rcm[3], s_fr[3], s_rr[3], s_fc[3], s_rc[3];
-#pragma unroll
-  for (int k = 0; k < 3; ++k) {
-    rcm[k] = (float)(sums[k] / (double)d.len_r);
-    s_fr[k] = rsqrtf(norm_eps + (float)(sums[3 + k] / (double)d.len_r));
-    s_rr[k] = rsqrtf(norm_eps + (float)(sums[6 + k] / (double)d.len_r));
-    s_fc[k] = rsqrtf(norm_eps + (float)(sums[9 + k] / (double)d.len_c));
-    s_rc[k] = rsqrtf(norm_eps + (float)(sums[12 + k] / (double)d.len_c));
-  }
-
-  // ---- phase 3: tables.  The accumulators written in phase 1 by this block are re-read here
-  // (same threads wrote the same entries: thread i handles entries i, i + blockDim, ...).
-  {
-    const float* fr = a.fac_r;
-    float* tab = rtab + (size_t)d.rtab_off * kTabW;
-    for (int i = threadIdx.x; i < d.len_r; i += kV0Threads) {
-      float A[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) A[j] = 0.0f;
-      float rf[3];
-#pragma unroll
-      for (int k = 0; k < 3; ++k) {
-        const float f = fr[(size_t)k * d.len_r + i];
-        rf[k] = rsqrtf(fmaxf(f / (rcm[k] + 1e-9f), 1e-9f));
-        const float x0 = f * s_fr[k];
-        const float x1 = rsqrtf(f + 1e-8f) * s_rr[k];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          A[j] = fmaf(x0, w_in[(15 + k) * 8 + j], A[j]);
-          A[j] = fmaf(x1, w_in[(21 + k) * 8 + j], A[j]);
-        }
-      }
-      float4* o = reinterpret_cast<float4*>(tab + (size_t)i * kTabW);
-      o[0] = make_float4(rf[0], rf[1], rf[2], 0.0f);
-      o[1] = make_float4(A[0], A[1], A[2], A[3]);
-      o[2] = make_float4(A[4], A[5], A[6], A[7]);
-    }
-  }
-  {
-    const float* fc = a.fac_c;
-    float* tab = ctab + (size_t)d.ctab_off * kTabW;
-    for (int i = threadIdx.x; i < d.len_c; i += kV0Threads) {
-      float B[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) B[j] = b_in[j];
-      float cf[3];
-#pragma unroll
-      for (int k = 0; k < 3; ++k) {
-        const float f = fc[(size_t)k * d.len_c + i];
-        cf[k] = rsqrtf(fmaxf(f, 1e-9f));
-        const float x0 = f * s_fc[k];
-        const float x1 = rsqrtf(f + 1e-8f) * s_rc[k];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          B[j] = fmaf(x0, w_in[(18 + k) * 8 + j], B[j]);
-          B[j] = fmaf(x1, w_in[(24 + k) * 8 + j], B[j]);
-        }
-      }
-      float4* o = reinterpret_cast<float4*>(tab + (size_t)i * kTabW);
-      o[0] = make_float4(cf[0], cf[1], cf[2], 0.0f);
-      o[1] = make_float4(B[0], B[1], B[2], B[3]);
-      o[2] = make_float4(B[4], B[5], B[6], B[7]);
-    }
-  }
-}
-
-// =============================================================================================
-// CELO2 element kernels
-// =============================================================================================
-struct EmaConsts {
-  float bm[3], obm[3];  // momentum decays and 1-decay
-  float br, obr;        // rms
-};
-
-__device__ __forceinline__ EmaConsts make_ema(const PyloDecays& dec) {
-  EmaConsts e;
-#pragma unroll
-  for (int k = 0; k < 3; ++k) { e.bm[k] = dec.beta_m[k]; e.obm[k] = 1.0f - dec.beta_m[k]; }
-  e.br = dec.beta_rms;
-  e.obr = 1.0f - dec.beta_rms;
-  return e;
-}
-
-// acc <- beta*acc + (1-beta)*new, each product and the sum rounded (ELO_CELO2_naive.py:145,149)
-__device__ __forceinline__ void ema_update(const EmaConsts& e, float g, float (&m)[3], float& rms) {
-#pragma unroll
-  for (int k = 0; k < 3; ++k) m[k] = m[k] * e.bm[k] + e.obm[k] * g;
-  rms = rms * e.br + e.obr * (g * g);
-}
-
-// The 18 per-element CELO2 channels (ELO_CELO2_naive.py:180-215), rs = rsqrt(rms + eps_rs).
-__device__ __forceinline__ void celo2_features(float g, float p, const float (&m)[3], float rms,
-                                               const float (&rf)[3], const float (&cf)[3], float eps_rs,
-                                               float (&f)[kNStat]) {
-  const float rs = rsqrtf(rms + eps_rs);
-  f[0] = g;
-  f[1] = g < -0.1f ? -0.1f : (g > 0.1f ? 0.1f : g);
-  f[2] = p;
-  f[3] = m[0]; f[4] = m[1]; f[5] = m[2];
-  f[6] = rms;
-  f[7] = m[0] * rs; f[8] = m[1] * rs; f[9] = m[2] * rs;
-  f[10] = rs;
-#pragma unroll
-  for (int k = 0; k < 3; ++k) {
-    f[11 + k] = (g * rf[k]) * cf[k];
-    f[15 + k] = (m[k] * rf[k]) * cf[k];
-  }
-  f[14] = g * rs;
-}
-
-// AdamW over the shared mom[0] / rms accumulators (ELO_CELO2_naive.py:296-302).
-template <int V>
-__device__ __forceinline__ void celo2_adam_chunk(const TDesc& d, const PyloTensorArgs& a, int chunk,
-                                                 float scale, const EmaConsts& e) {
-  const long long base = (long long)chunk * (kThreads * V * kElemIters);
-  const long long n = d.n;
-#pragma unroll 2
-  for (int it = 0; it < kElemIters; ++it) {
-    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
-    if (idx >= n) break;
-    float g[V], p[V], m0[V], m1[V], m2[V], r[V];
-    load_vec<V>(a.grad + idx, g);
-    load_vec<V>(a.param + idx, p);
-    load_vec<V>(a.mom + idx, m0);
-    load_vec<V>(a.mom + n + idx, m1);
-    load_vec<V>(a.mom + 2 * n + idx, m2);
-    load_vec<V>(a.rms + idx, r);
-#pragma unroll
-    for (int v = 0; v < V; ++v) {
-      const float gg = clampf(g[v] * scale, a.clip_val);
-      float m[3] = {m0[v], m1[v], m2[v]};
-      ema_update(e, gg, m, r[v]);
-      m0[v] = m[0]; m1[v] = m[1]; m2[v] = m[2];
-      const float mh = m[0] / a.bc1;
-      const float vh = r[v] / a.bc2;
-      const float upd = mh / (sqrtf(vh) + 1e-8f);
-      p[v] = fmaf(upd + a.weight_decay * p[v], -a.lr, p[v]);
-    }
-    store_vec<V>(a.mom + idx, m0);
-    store_vec<V>(a.mom + n + idx, m1);
-    store_vec<V>(a.mom + 2 * n + idx, m2);
-    store_vec<V>(a.rms + idx, r);
-    store_vec<V>(a.param + idx, p);
-  }
-}
-
-// Loads one vector of V consecutive elements (same dim-0 index) and the factors of its row / columns.
-template <int V>
-struct ElemIn {
-  float g[V], p[V], m[V][3], rms[V];
-  float rf[V][3], cf[V][3];
-  int ir[V], ic[V];
-};
-
-template <int V>
-__device__ __forceinline__ void load_elems(const TDesc& d, const PyloTensorArgs& a, long long idx,
-                                           float scale, const float* __restrict__ rt,
-                                           const float* __restrict__ ct, ElemIn<V>& x) {
-  const long long n = d.n;
-  float m0[V], m1[V], m2[V];
-  load_vec<V>(a.grad + idx, x.g);
-  load_vec<V>(a.param + idx, x.p);
-  load_vec<V>(a.mom + idx, m0);
-  load_vec<V>(a.mom + n + idx, m1);
-  load_vec<V>(a.mom + 2 * n + idx, m2);
-  load_vec<V>(a.rms + idx, x.rms);
-  const unsigned u = (unsigned)idx;  // n < 2^31
-  const int i0 = (int)(u / (unsigned)d.C0);
-  const int i1 = (int)(u - (unsigned)i0 * (unsigned)d.C0);
-#pragma unroll
-  for (int v = 0; v < V; ++v) {
-    x.g[v] = clampf(x.g[v] * scale, a.clip_val);
-    x.m[v][0] = m0[v]; x.m[v][1] = m1[v]; x.m[v][2] = m2[v];
-    x.ir[v] = d.r_is_dim0 ? i0 : i1 + v;
-    x.ic[v] = d.r_is_dim0 ? i1 + v : i0;
-    const float4 r4 = *reinterpret_cast<const float4*>(rt + (size_t)x.ir[v] * kTabW);
-    const float4 c4 = *reinterpret_cast<const float4*>(ct + (size_t)x.ic[v] * kTabW);
-    x.rf[v][0] = r4.x; x.rf[v][1] = r4.y; x.rf[v][2] = r4.z;
-    x.cf[v][0] = c4.x; x.cf[v][1] = c4.y; x.cf[v][2] = c4.z;
-  }
-}
-
-template <int V>
-__device__ __forceinline__ void celo2_stats_chunk(const TDesc& d, const PyloTensorArgs& a, int chunk,
-                                                  float scale, const EmaConsts& e,
-                                                  const float* __restrict__ rt, const float* __restrict__ ct,
-                                                  float (&acc)[kNStat]) {
-  const long long base = (long long)chunk * (kThreads * V * kElemIters);
-#pragma unroll 2
-  for (int it = 0; it < kElemIters; ++it) {
-    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
-    if (idx >= d.n) break;
-    ElemIn<V> x;
-    load_elems<V>(d, a, idx, scale, rt, ct, x);
-#pragma unroll
-    for (int v = 0; v < V; ++v) {
-      ema_update(e, x.g[v], x.m[v], x.rms[v]);
-      float f[kNStat];
-      celo2_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.rf[v], x.cf[v], 1e-8f, f);
-#pragma unroll
-      for (int c = 0; c < kNStat; ++c) acc[c] += f[c] * f[c];
-    }
-  }
-}
-
-__global__ __launch_bounds__(kThreads) void k_celo2_stats(const TDesc* __restrict__ descs,
-                                                          const PyloTensorArgs* __restrict__ dyn,
-                                                          const Item* __restrict__ items,
-                                                          const float* __restrict__ rtab,
-                                                          const float* __restrict__ ctab,
-                                                          const Globals* __restrict__ gl, PyloDecays dec,
-                                                          double* __restrict__ stats_part) {
-  __shared__ float red[kWaves][kNStat];
-  const Item it = items[blockIdx.x];
-  const TDesc d = descs[it.tensor];
-  const PyloTensorArgs a = dyn[it.tensor];
-  if (a.grad == nullptr) return;
-  const float scale = clip_scale(gl->gnorm, a.clip_norm);
-  const EmaConsts e = make_ema(dec);
-  if (d.mode == kModeFlat) {
-    if (d.vec == 4) celo2_adam_chunk<4>(d, a, it.a, scale, e);
-    else celo2_adam_chunk<1>(d, a, it.a, scale, e);
-    return;
-  }
-  float acc[kNStat];
-#pragma unroll
-  for (int c = 0; c < kNStat; ++c) acc[c] = 0.0f;
-  const float* rt = rtab + (size_t)d.rtab_off * kTabW;
-  const float* ct = ctab + (size_t)d.ctab_off * kTabW;
-  if (d.vec == 4) celo2_stats_chunk<4>(d, a, it.a, scale, e, rt, ct, acc);
-  else celo2_stats_chunk<1>(d, a, it.a, scale, e, rt, ct, acc);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-  for (int c = 0; c < kNStat; ++c) {
-    const float s = wave_sum(acc[c]);
-    if (lane == 0) red[wave][c] = s;
-  }
-  __syncthreads();
-  if (threadIdx.x < kNStat) {
-    const int c = threadIdx.x;
-    stats_part[(size_t)blockIdx.x * kNStat + c] =
-        ((double)red[0][c] + (double)red[1][c]) + ((double)red[2][c] + (double)red[3][c]);
-  }
-}
-
-// Per factored tensor: s_c = rsqrt(1e-9 + mean f_c^2) folded into the first-layer rows of the 18
-// per-element channels; the remaining layers are copied behind them so the apply kernel reads one
-// contiguous block per tensor.
-__global__ __launch_bounds__(kThreads) void k_celo2_fold(const TDesc* __restrict__ descs,
-                                                         const PyloTensorArgs* __restrict__ dyn,
-                                                         const int* __restrict__ fac_list,
-                                                         const double* __restrict__ stats_part,
-                                                         const float* __restrict__ mlp,
-                                                         float* __restrict__ wfold, float* __restrict__ chan_ms) {
-  constexpr int G = 14;  // 14 groups x 18 channels = 252 threads
-  __shared__ double part[G][kNStat];
-  __shared__ float scale_c[kNStat];
-  const int t = fac_list[blockIdx.x];
-  const TDesc d = descs[t];
-  if (dyn[t].grad == nullptr) return;
-  const int c = threadIdx.x % kNStat, gI = threadIdx.x / kNStat;
-  if (gI < G) {
-    double s = 0.0;
-    for (int b = gI; b < d.nblk; b += G) s += stats_part[(size_t)(d.blk0 + b) * kNStat + c];
-    part[gI][c] = s;
-  }
-  __syncthreads();
-  if (threadIdx.x < kNStat) {
-    double s = 0.0;
-    for (int g2 = 0; g2 < G; ++g2) s += part[g2][threadIdx.x];
-    const float ms = (float)(s / (double)d.n);
-    chan_ms[(size_t)d.fac_slot * kNStat + threadIdx.x] = ms;
-    scale_c[threadIdx.x] = rsqrtf(1e-9f + ms);
-  }
-  __syncthreads();
-  float* w = wfold + (size_t)d.fac_slot * kC2Fold;
-  const float* w_in = mlp;                  // (30,8)
-  const float* w_h = mlp + 240 + 8;         // (8,8)
-  const float* b_h = w_h + 64;              // 8
-  const float* w_out = b_h + 8;             // (8,3)
-  const float* b_out = w_out + 24;          // 3
-  for (int i = threadIdx.x; i < kNStat * 8; i += kThreads) {
-    const int cc = i / 8, j = i % 8;
-    w[kC2W1 + i] = w_in[stat_channel(cc) * 8 + j] * scale_c[cc];
-  }
-  for (int i = threadIdx.x; i < 64; i += kThreads) w[kC2WH + i] = w_h[i];
-  for (int i = threadIdx.x; i < 8; i += kThreads) w[kC2BH + i] = b_h[i];
-  for (int i = threadIdx.x; i < 16; i += kThreads) w[kC2WO + i] = w_out[(i / 2) * 3 + (i % 2)];
-  for (int i = threadIdx.x; i < 2; i += kThreads) w[kC2BO + i] = b_out[i];
-}
-
-template <int V>
-__device__ __forceinline__ void celo2_apply_chunk(const TDesc& d, const PyloTensorArgs& a, int chunk,
-                                                  float scale, const EmaConsts& e,
-                                                  const float* __restrict__ rt, const float* __restrict__ ct,
-                                                  const float* __restrict__ w) {
-  const long long base = (long long)chunk * (kThreads * V * kElemIters);
-  const long long n = d.n;
-  const bool use_exp = a.exp_mult != 0.0f;
-  for (int it = 0; it < kElemIters; ++it) {
-    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
-    if (idx >= n) break;
-    ElemIn<V> x;
-    load_elems<V>(d, a, idx, scale, rt, ct, x);
-    float out[V], m0[V], m1[V], m2[V];
-#pragma unroll
-    for (int v = 0; v < V; ++v) {
-      ema_update(e, x.g[v], x.m[v], x.rms[v]);
-      m0[v] = x.m[v][0]; m1[v] = x.m[v][1]; m2[v] = x.m[v][2];
-      float f[kNStat];
-      celo2_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.rf[v], x.cf[v], 1e-8f, f);
-      const float4* ra = reinterpret_cast<const float4*>(rt + (size_t)x.ir[v] * kTabW);
-      const float4* ca = reinterpret_cast<const float4*>(ct + (size_t)x.ic[v] * kTabW);
-      const float4 a0 = ra[1], a1 = ra[2], b0 = ca[1], b1 = ca[2];
-      float h[8] = {a0.x + b0.x, a0.y + b0.y, a0.z + b0.z, a0.w + b0.w,
-                    a1.x + b1.x, a1.y + b1.y, a1.z + b1.z, a1.w + b1.w};
-#pragma unroll
-      for (int c = 0; c < kNStat; ++c) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) h[j] = fmaf(f[c], w[kC2W1 + c * 8 + j], h[j]);
-      }
-      float h1[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) { h[j] = fmaxf(h[j], 0.0f); h1[j] = w[kC2BH + j]; }
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) h1[j] = fmaf(h[k], w[kC2WH + k * 8 + j], h1[j]);
-      }
-      float o0 = w[kC2BO + 0], o1 = w[kC2BO + 1];
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const float hk = fmaxf(h1[k], 0.0f);
-        o0 = fmaf(hk, w[kC2WO + k * 2 + 0], o0);
-        if (use_exp) o1 = fmaf(hk, w[kC2WO + k * 2 + 1], o1);
-      }
-      out[v] = use_exp ? o0 * expf(o1 * a.exp_mult) : o0;
-    }
-    store_vec<V>(a.mom + idx, m0);
-    store_vec<V>(a.mom + n + idx, m1);
-    store_vec<V>(a.mom + 2 * n + idx, m2);
-    store_vec<V>(a.rms + idx, x.rms);
-    store_vec<V>(a.step_out + idx, out);
-  }
-}
-
-__global__ __launch_bounds__(kThreads) void k_celo2_apply(const TDesc* __restrict__ descs,
-                                                          const PyloTensorArgs* __restrict__ dyn,
-                                                          const Item* __restrict__ items,
-                                                          const float* __restrict__ rtab,
-                                                          const float* __restrict__ ctab,
-                                                          const Globals* __restrict__ gl, PyloDecays dec,
-                                                          const float* __restrict__ wfold) {
-  const Item it = items[blockIdx.x];
-  const TDesc d = descs[it.tensor];
-  if (d.mode == kModeFlat) return;
-  const PyloTensorArgs a = dyn[it.tensor];
-  if (a.grad == nullptr) return;
-  const float scale = clip_scale(gl->gnorm, a.clip_norm);
-  const EmaConsts e = make_ema(dec);
-  const float* rt = rtab + (size_t)d.rtab_off * kTabW;
-  const float* ct = ctab + (size_t)d.ctab_off * kTabW;
-  const float* w = wfold + (size_t)d.fac_slot * kC2Fold;
-  if (d.vec == 4) celo2_apply_chunk<4>(d, a, it.a, scale, e, rt, ct, w);
-  else celo2_apply_chunk<1>(d, a, it.a, scale, e, rt, ct, w);
-}
-
-}  // namespace pylo
 
 // =============================================================================================
 // Host side: plan construction and the C ABI
@@ -667,11 +59,13 @@ bool factored_dims(int kind, const PyloTensorShape& s, int* dc, int* dr) {
 
 struct Layout {
   std::vector<TDesc> descs;
-  std::vector<Item> p0_items, el_items;
+  std::vector<Item> p0_items, el_items, v0a_items, v0b_items;
   std::vector<int> fac_list;
   std::vector<int> dc, dr;
-  size_t off_descs, off_dyn, off_p0_items, off_el_items, off_fac_list, off_rowpart, off_colpart, off_gsq,
-      off_flag, off_globals, off_rtab, off_ctab, off_stats, off_wfold, off_chan_ms, total;
+  int H = 8;  // width of the first MLP layer (terms per row / column)
+  size_t off_descs, off_dyn, off_p0_items, off_el_items, off_v0a_items, off_v0b_items, off_fac_list,
+      off_rowpart, off_colpart, off_gsq, off_flag, off_globals, off_fac0, off_fac1, off_term0, off_term1,
+      off_v0part, off_bscale, off_stats, off_wfold, off_chan_ms, total;
 };
 
 int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L) {
@@ -680,7 +74,8 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L) {
   L.descs.assign(T, TDesc{});
   L.dc.assign(T, -1);
   L.dr.assign(T, -1);
-  long long rowpart = 0, colpart = 0, rtab = 0, ctab = 0;
+  long long rowpart = 0, colpart = 0, fac0 = 0, fac1 = 0, term0 = 0, term1 = 0;
+  const int H = L.H;
   for (int t = 0; t < T; ++t) {
     const PyloTensorShape& s = shapes[t];
     if (s.ndim < 0 || s.ndim > PYLO_MAX_DIMS) return fail("plan: bad ndim");
@@ -718,13 +113,27 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L) {
       d.colpart_off = colpart;
       rowpart += (long long)d.n_colblk * d.R0;
       colpart += (long long)d.n_strips * d.C0;
-      d.rtab_off = rtab;
-      d.ctab_off = ctab;
-      rtab += d.len_r;
-      ctab += d.len_c;
-      d.fac_slot = (int)L.fac_list.size();
-      if (n > 0) L.fac_list.push_back(t);
-      else d.fac_slot = -1;
+      d.C0r = (d.C0 + 3) / 4 * 4;
+      d.fac0_off = fac0;
+      d.fac1_off = fac1;
+      d.term0_off = term0;
+      d.term1_off = term1;
+      fac0 += (long long)d.R0 * 4;
+      fac1 += 3ll * d.C0r;
+      term0 += (long long)d.R0 * H;
+      term1 += (long long)H * d.C0r;
+      d.fac_slot = -1;
+      if (n > 0) {
+        d.fac_slot = (int)L.fac_list.size();
+        L.fac_list.push_back(t);
+        for (int which = 0; which < 2; ++which) {
+          const int len = which ? d.C0 : d.R0;
+          d.v0a_first[which] = (int)L.v0a_items.size();
+          for (int c = 0; c * kV0aEnt < len; ++c) L.v0a_items.push_back(Item{t, c, which, 0});
+          d.v0a_n[which] = (int)L.v0a_items.size() - d.v0a_first[which];
+          for (int c = 0; c * kV0bEnt < len; ++c) L.v0b_items.push_back(Item{t, c, which, 0});
+        }
+      }
     }
     // P0 items
     if (n > 0) {
@@ -753,14 +162,20 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L) {
   L.off_dyn = take(sizeof(PyloTensorArgs) * T);
   L.off_p0_items = take(sizeof(Item) * std::max<size_t>(L.p0_items.size(), 1));
   L.off_el_items = take(sizeof(Item) * std::max<size_t>(L.el_items.size(), 1));
+  L.off_v0a_items = take(sizeof(Item) * std::max<size_t>(L.v0a_items.size(), 1));
+  L.off_v0b_items = take(sizeof(Item) * std::max<size_t>(L.v0b_items.size(), 1));
   L.off_fac_list = take(sizeof(int) * nfac);
   L.off_rowpart = take(sizeof(float) * std::max<long long>(rowpart, 1));
   L.off_colpart = take(sizeof(float) * std::max<long long>(colpart, 1));
   L.off_gsq = take(sizeof(double) * std::max<size_t>(L.p0_items.size(), 1));
   L.off_flag = take(sizeof(int) * std::max<size_t>(L.p0_items.size(), 1));
   L.off_globals = take(sizeof(Globals));
-  L.off_rtab = take(sizeof(float) * kTabW * std::max<long long>(rtab, 1));
-  L.off_ctab = take(sizeof(float) * kTabW * std::max<long long>(ctab, 1));
+  L.off_fac0 = take(sizeof(float) * std::max<long long>(fac0, 4));
+  L.off_fac1 = take(sizeof(float) * std::max<long long>(fac1, 4));
+  L.off_term0 = take(sizeof(float) * std::max<long long>(term0, 4));
+  L.off_term1 = take(sizeof(float) * std::max<long long>(term1, 4));
+  L.off_v0part = take(sizeof(double) * kNV0 * std::max<size_t>(L.v0a_items.size(), 1));
+  L.off_bscale = take(sizeof(BScale) * nfac);
   L.off_stats = take(sizeof(double) * kNStat * std::max<size_t>(L.el_items.size(), 1));
   L.off_wfold = take(sizeof(float) * kC2Fold * nfac);
   L.off_chan_ms = take(sizeof(float) * kNStat * nfac);
@@ -827,6 +242,8 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_p0_items, L.p0_items.data(), sizeof(Item) * L.p0_items.size());
   if (e == hipSuccess) e = up(L.off_el_items, L.el_items.data(), sizeof(Item) * L.el_items.size());
   if (e == hipSuccess) e = up(L.off_fac_list, L.fac_list.data(), sizeof(int) * L.fac_list.size());
+  if (e == hipSuccess) e = up(L.off_v0a_items, L.v0a_items.data(), sizeof(Item) * L.v0a_items.size());
+  if (e == hipSuccess) e = up(L.off_v0b_items, L.v0b_items.data(), sizeof(Item) * L.v0b_items.size());
   if (e == hipSuccess) e = hipStreamSynchronize(s);
   for (int i = 0; i < kStageSlots && e == hipSuccess; ++i) {
     e = hipHostMalloc(reinterpret_cast<void**>(&P->stage[i]), sizeof(PyloTensorArgs) * n_tensors, hipHostMallocDefault);
@@ -883,11 +300,12 @@ int pylo_mi355_plan_timing_end(PyloPlan* P, float* ms_out, int capacity, int* st
 
 int pylo_mi355_plan_num_launches(const PyloPlan* P) {
   if (!P) return -1;
-  return P->kind == PYLO_KIND_CELO2 ? 7 : -1;
+  return P->kind == PYLO_KIND_CELO2 ? 8 : -1;
 }
 
 const char* pylo_mi355_plan_launch_name(const PyloPlan* P, int launch) {
-  static const char* celo2[] = {"k_p0(sums)", "k_gnorm", "k_p0(exact)", "k_v0", "k_celo2_stats", "k_celo2_fold", "k_celo2_apply"};
+  static const char* celo2[] = {"k_p0(sums)", "k_gnorm", "k_p0(exact)", "k_v0a", "k_v0b",
+                                "k_celo2_stats", "k_celo2_fold", "k_celo2_apply"};
   if (!P || launch < 0 || launch >= pylo_mi355_plan_num_launches(P)) return "";
   return celo2[launch];
 }
@@ -957,8 +375,15 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   double* gsq = P->at<double>(L.off_gsq);
   int* flag = P->at<int>(L.off_flag);
   Globals* gl = P->at<Globals>(L.off_globals);
-  float* rtab = P->at<float>(L.off_rtab);
-  float* ctab = P->at<float>(L.off_ctab);
+  const Item* v0a_items = P->at<Item>(L.off_v0a_items);
+  const Item* v0b_items = P->at<Item>(L.off_v0b_items);
+  float* fac0 = P->at<float>(L.off_fac0);
+  float* fac1 = P->at<float>(L.off_fac1);
+  float* term0 = P->at<float>(L.off_term0);
+  float* term1 = P->at<float>(L.off_term1);
+  double* v0part = P->at<double>(L.off_v0part);
+  BScale* bscale = P->at<BScale>(L.off_bscale);
+  const int n_v0a = (int)L.v0a_items.size(), n_v0b = (int)L.v0b_items.size();
   double* stats = P->at<double>(L.off_stats);
   float* wfold = P->at<float>(L.off_wfold);
   float* chan_ms = P->at<float>(L.off_chan_ms);
@@ -976,15 +401,20 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   PYLO_MARK();
   if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, rowpart, colpart, gsq, flag, gl, 1);
   PYLO_MARK();
-  if (n_fac > 0)
-    hipLaunchKernelGGL(k_v0, dim3(n_fac), dim3(kV0Threads), 0, s, descs, dyn, fac_list, rowpart, colpart, gl, dec,
-                       mlp, mlp + 240, 1e-9f, rtab, ctab);
+  if (n_v0a > 0)
+    hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kThreads), 0, s, descs, dyn, v0a_items, rowpart, colpart, gl, dec, v0part);
   PYLO_MARK();
-  if (n_el > 0) hipLaunchKernelGGL(k_celo2_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, rtab, ctab, gl, dec, stats);
+  if (n_v0b > 0)
+    hipLaunchKernelGGL(k_v0b<8>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-9f, mlp,
+                       mlp + 240, fac0, fac1, term0, term1, bscale);
   PYLO_MARK();
-  if (n_fac > 0) hipLaunchKernelGGL(k_celo2_fold, dim3(n_fac), dim3(kThreads), 0, s, descs, dyn, fac_list, stats, mlp, wfold, chan_ms);
+  if (n_el > 0) hipLaunchKernelGGL(k_celo2_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac0, fac1, gl, dec, stats);
   PYLO_MARK();
-  if (n_el > 0) hipLaunchKernelGGL(k_celo2_apply, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, rtab, ctab, gl, dec, wfold);
+  if (n_fac > 0) hipLaunchKernelGGL(k_celo2_fold, dim3(n_fac), dim3(kFoldThreads), 0, s, descs, dyn, fac_list, stats, mlp, wfold, chan_ms);
+  PYLO_MARK();
+  if (n_el > 0)
+    hipLaunchKernelGGL(k_celo2_apply, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac0, fac1, term0, term1,
+                       gl, dec, wfold);
   PYLO_MARK();
 #undef PYLO_MARK
   if (timed) P->t_steps++;

@@ -103,6 +103,9 @@ def main():
     ap.add_argument("--fused-only", action="store_true",
                     help="loop the C-ABI call alone (no Newton-Schulz / apply), e.g. under rocprofv3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run a 1 GiB device-to-device tensor copy (3x) so that a counter profile of "
+                         "this command holds a kernel of known HBM traffic to scale FETCH_SIZE/WRITE_SIZE by")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
@@ -130,6 +133,13 @@ def main():
         else:
             opt.step()
 
+    if a.calib_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)                      # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(a.warmup):
         one_step()
     torch.cuda.synchronize()

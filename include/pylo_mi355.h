@@ -31,6 +31,7 @@ extern "C" {
 
 #define PYLO_MI355_ABI_VERSION 1
 #define PYLO_MAX_DIMS 8
+#define PYLO_MAX_GROUPS 8   /* parameter groups with their own step counter (VeLO) */
 
 /* optimizer kinds */
 #define PYLO_KIND_CELO2 0   /* ELO_CELO2_CUDA / CELO2_CUDA (celo2_kernel.cu)           */
@@ -76,6 +77,8 @@ typedef struct {
   float step_mult;
   float bc1;         /* CELO2 AdamW: 1 - beta1^t                                             */
   float bc2;         /* CELO2 AdamW: 1 - beta2^t                                             */
+  int32_t group;     /* VeLO: index into PyloVeloStep.frac (the tensor's parameter group)    */
+  int32_t reserved;
 } PyloTensorArgs;
 
 int pylo_mi355_abi_version(void);
@@ -122,6 +125,52 @@ const char* pylo_mi355_plan_launch_name(const PyloPlan* plan, int launch);
  */
 int pylo_mi355_celo2_step(PyloPlan* plan, const PyloTensorArgs* args, const PyloDecays* decays,
                           const float* mlp, void* stream);
+
+/*
+ * VeLO step (replaces velo_cuda_kernel.velo_kernel_simple, pylo/csrc/velo_kernel.cu:370-457, for every
+ * tensor at once, plus velo_cuda.py:183-211 (loss features), :213-252 (per-tensor LSTM features),
+ * pylo/models/VeLO_RNN.py:43-66,110-135 (mixing + LSTM cell + heads), pylo/models/VeLO_MLP.py:92-126
+ * (bank mixing) and velo_cuda.py:502-546 (accumulator updates)).
+ *
+ * All weight matrices are device pointers, fp32, stored (in, out) -- i.e. the transpose of the
+ * torch.nn.Linear weights of pylo/models/VeLO_RNN.py; `bank` is (n_bank, 159): per entry
+ * W_in (4,30) | b_in 4 | W_h (4,4) | b_h 4 | W_out (3,4) | b_out 3, each (out, in) as in VeLO_MLP.py:63-77.
+ */
+typedef struct {
+  const float* mix2_wt;   /* (30, H)   mix_layer2.weight^T        */
+  const float* mix2_b;    /* (H)                                  */
+  const float* fmix_wt;   /* (30, H)   final_mix_layer.weight^T   */
+  const float* fmix_b;    /* (H)                                  */
+  const float* lstm_wt;   /* (2H, 4H)  lstm.linear.weight^T, gate blocks i, g, f, o */
+  const float* lstm_b;    /* (4H)                                 */
+  const float* ctrl_wt;   /* (H, K)    rnn_to_controls.weight^T   */
+  const float* ctrl_b;    /* (K)                                  */
+  const float* lr_w;      /* (H)       step_size.weight           */
+  const float* lr_b;      /* (1)                                  */
+  const float* bank;      /* (K, 159)                             */
+  int32_t hidden;         /* H, multiple of 64                    */
+  int32_t n_bank;         /* K                                    */
+} PyloVeloNets;
+
+typedef struct {
+  float* lstm_h;             /* (T, H) hidden state, row r belongs to tensor T-1-r; updated in place */
+  float* lstm_c;             /* (T, H) cell state; updated in place                                   */
+  float* loss_means;         /* (10)  loss EMAs, updated in place (velo_cuda.py:183-198)              */
+  float* loss_running_min;   /* (10)  updated in place                                                */
+  const float* loss_decays;  /* (10)                                                                  */
+  int32_t* loss_iteration;   /* (1)   updated in place                                                */
+  const float* loss;         /* (1)   this step's loss, device scalar                                 */
+  float* controls_out;       /* optional (T, K): the control vectors, NULL to skip                    */
+  float* lr_mult_out;        /* optional (T): learning-rate multipliers, NULL to skip                 */
+  float frac[PYLO_MAX_GROUPS][9]; /* tanh((step/num_steps - ts) * 10) per group (velo_cuda.py:155-162) */
+} PyloVeloStep;
+
+/* Every tensor of the plan must have a gradient.  For each tensor: g <- clamp(g, +-clip_val);
+   mom / rms / fac_r / fac_c (or fac_v) EMAs; 30 features normalised over the whole tensor (eps 1e-5);
+   the tensor's own 30->4->4->3 MLP;  p -= lr * lr_mult * sqrt(mean p^2 + 1e-9) * o0 * exp(o1 * exp_mult)
+   * step_mult;  then p -= weight_decay * lr * p. */
+int pylo_mi355_velo_step(PyloPlan* plan, const PyloTensorArgs* args, const PyloDecays* decays,
+                         const PyloVeloNets* nets, const PyloVeloStep* step, void* stream);
 
 #ifdef __cplusplus
 }

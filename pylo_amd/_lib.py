@@ -27,15 +27,28 @@ class Decays(C.Structure):
     _fields_ = [("beta_m", C.c_float * 3), ("beta_rms", C.c_float), ("beta_fac", C.c_float * 3)]
 
 
-# numpy mirror of PyloTensorArgs (8 pointers, 8 floats, no padding)
+# numpy mirror of PyloTensorArgs (8 pointers, 8 floats, 2 ints, no padding)
 ARGS_DTYPE = np.dtype([
     ("grad", np.uint64), ("param", np.uint64), ("mom", np.uint64), ("rms", np.uint64),
     ("fac_r", np.uint64), ("fac_c", np.uint64), ("fac_v", np.uint64), ("step_out", np.uint64),
     ("lr", np.float32), ("weight_decay", np.float32), ("clip_norm", np.float32),
     ("clip_val", np.float32), ("exp_mult", np.float32), ("step_mult", np.float32),
-    ("bc1", np.float32), ("bc2", np.float32),
+    ("bc1", np.float32), ("bc2", np.float32), ("group", np.int32), ("reserved", np.int32),
 ])
-assert ARGS_DTYPE.itemsize == 96
+assert ARGS_DTYPE.itemsize == 104
+MAX_GROUPS = 8
+
+
+class VeloNets(C.Structure):
+    _fields_ = [(k, C.c_void_p) for k in ("mix2_wt", "mix2_b", "fmix_wt", "fmix_b", "lstm_wt", "lstm_b",
+                                          "ctrl_wt", "ctrl_b", "lr_w", "lr_b", "bank")] + \
+               [("hidden", C.c_int32), ("n_bank", C.c_int32)]
+
+
+class VeloStep(C.Structure):
+    _fields_ = [(k, C.c_void_p) for k in ("lstm_h", "lstm_c", "loss_means", "loss_running_min", "loss_decays",
+                                          "loss_iteration", "loss", "controls_out", "lr_mult_out")] + \
+               [("frac", (C.c_float * 9) * MAX_GROUPS)]
 
 _lib = None
 
@@ -66,6 +79,8 @@ def load():
     lib.pylo_mi355_plan_launch_name.restype = C.c_char_p
     lib.pylo_mi355_celo2_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.c_void_p,
                                           C.c_void_p]
+    lib.pylo_mi355_velo_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.POINTER(VeloNets),
+                                         C.POINTER(VeloStep), C.c_void_p]
     if lib.pylo_mi355_abi_version() != 1:
         raise RuntimeError("libpylo_mi355.so: ABI version mismatch, rebuild it")
     _lib = lib
@@ -148,6 +163,10 @@ class Plan:
     def celo2_step(self, decays: Decays, mlp: torch.Tensor, stream: int) -> None:
         check(load().pylo_mi355_celo2_step(self._h, self.args.ctypes.data, C.byref(decays),
                                            mlp.data_ptr(), stream), "celo2_step")
+
+    def velo_step(self, decays: Decays, nets: VeloNets, step: VeloStep, stream: int) -> None:
+        check(load().pylo_mi355_velo_step(self._h, self.args.ctypes.data, C.byref(decays), C.byref(nets),
+                                          C.byref(step), stream), "velo_step")
 
     def close(self):
         if getattr(self, "_h", None):

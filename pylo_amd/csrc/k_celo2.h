@@ -107,7 +107,7 @@ __device__ __forceinline__ void load_elems(const TDesc& d, const PyloTensorArgs&
   const float4 fa = load_f4(f0 + (size_t)x.i0 * 4);
   float fb[3][V];
 #pragma unroll
-  for (int k = 0; k < 3; ++k) load_vec<V>(f1 + (size_t)k * d.C0r + x.i1, fb[k]);
+  for (int k = 0; k < 3; ++k) load_vec<V>(f1 + (size_t)k * d.pitch[1] + x.i1, fb[k]);
 #pragma unroll
   for (int v = 0; v < V; ++v) {
     x.g[v] = clampf(x.g[v] * scale, a.clip_val);
@@ -146,8 +146,7 @@ __device__ __forceinline__ void celo2_stats_chunk(const TDesc& d, const PyloTens
 __global__ __launch_bounds__(kThreads) void k_celo2_stats(const TDesc* __restrict__ descs,
                                                           const PyloTensorArgs* __restrict__ dyn,
                                                           const Item* __restrict__ items,
-                                                          const float* __restrict__ fac0,
-                                                          const float* __restrict__ fac1,
+                                                          const float* __restrict__ fac_tab,
                                                           const Globals* __restrict__ gl, PyloDecays dec,
                                                           double* __restrict__ stats_part) {
   __shared__ float red[kWaves][kNStat];
@@ -165,8 +164,8 @@ __global__ __launch_bounds__(kThreads) void k_celo2_stats(const TDesc* __restric
   float acc[kNStat];
 #pragma unroll
   for (int c = 0; c < kNStat; ++c) acc[c] = 0.0f;
-  const float* f0 = fac0 + d.fac0_off;
-  const float* f1 = fac1 + d.fac1_off;
+  const float* f0 = fac_tab + d.fac_off[0];
+  const float* f1 = fac_tab + d.fac_off[1];
   if (d.vec == 4) celo2_stats_chunk<4>(d, a, it.a, scale, e, f0, f1, acc);
   else celo2_stats_chunk<1>(d, a, it.a, scale, e, f0, f1, acc);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -178,7 +177,7 @@ __global__ __launch_bounds__(kThreads) void k_celo2_stats(const TDesc* __restric
   __syncthreads();
   if (threadIdx.x < kNStat) {
     const int c = threadIdx.x;
-    stats_part[(size_t)blockIdx.x * kNStat + c] =
+    stats_part[(size_t)blockIdx.x * kStatW + stat_channel(c)] =
         ((double)red[0][c] + (double)red[1][c]) + ((double)red[2][c] + (double)red[3][c]);
   }
 }
@@ -202,7 +201,7 @@ __global__ __launch_bounds__(kFoldThreads) void k_celo2_fold(const TDesc* __rest
   if (gI < G) {
     double s = 0.0;
 #pragma unroll 4
-    for (int b = gI; b < d.nblk; b += G) s += stats_part[(size_t)(d.blk0 + b) * kNStat + c];
+    for (int b = gI; b < d.nblk; b += G) s += stats_part[(size_t)(d.blk0 + b) * kStatW + stat_channel(c)];
     part[gI][c] = s;
   }
   __syncthreads();
@@ -251,7 +250,7 @@ __device__ __forceinline__ void celo2_apply_chunk(const TDesc& d, const PyloTens
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         float tb[V];
-        load_vec<V>(t1 + (size_t)j * d.C0r + x.i1, tb);
+        load_vec<V>(t1 + (size_t)j * d.pitch[1] + x.i1, tb);
 #pragma unroll
         for (int v = 0; v < V; ++v) h[v][j] = ta[j] + tb[v];
       }
@@ -321,10 +320,8 @@ __device__ __forceinline__ void celo2_apply_chunk(const TDesc& d, const PyloTens
 __global__ __launch_bounds__(kThreads) void k_celo2_apply(const TDesc* __restrict__ descs,
                                                           const PyloTensorArgs* __restrict__ dyn,
                                                           const Item* __restrict__ items,
-                                                          const float* __restrict__ fac0,
-                                                          const float* __restrict__ fac1,
-                                                          const float* __restrict__ term0,
-                                                          const float* __restrict__ term1,
+                                                          const float* __restrict__ fac_tab,
+                                                          const float* __restrict__ term_tab,
                                                           const Globals* __restrict__ gl, PyloDecays dec,
                                                           const float* __restrict__ wfold) {
   const Item it = items[blockIdx.x];
@@ -336,11 +333,11 @@ __global__ __launch_bounds__(kThreads) void k_celo2_apply(const TDesc* __restric
   const EmaConsts e = make_ema(dec);
   const float* w = wfold + (size_t)d.fac_slot * kC2Fold;
   if (d.vec == 4)
-    celo2_apply_chunk<4>(d, a, it.a, scale, e, fac0 + d.fac0_off, fac1 + d.fac1_off, term0 + d.term0_off,
-                         term1 + d.term1_off, w);
+    celo2_apply_chunk<4>(d, a, it.a, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
+                         term_tab + d.term_off[0], term_tab + d.term_off[1], w);
   else
-    celo2_apply_chunk<1>(d, a, it.a, scale, e, fac0 + d.fac0_off, fac1 + d.fac1_off, term0 + d.term0_off,
-                         term1 + d.term1_off, w);
+    celo2_apply_chunk<1>(d, a, it.a, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
+                         term_tab + d.term_off[0], term_tab + d.term_off[1], w);
 }
 
 }  // namespace pylo

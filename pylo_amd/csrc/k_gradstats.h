@@ -81,8 +81,7 @@ __device__ __forceinline__ void p0_flat(const TDesc& d, const float* g, int chun
 // pass 1: only if the flag was raised: redo clip_norm > 0 tensors with scale and clamp applied.
 __global__ __launch_bounds__(kThreads) void k_p0(const TDesc* __restrict__ descs,
                                                  const PyloTensorArgs* __restrict__ dyn,
-                                                 const Item* __restrict__ items,
-                                                 float* __restrict__ rowpart, float* __restrict__ colpart,
+                                                 const Item* __restrict__ items, float* __restrict__ part,
                                                  double* __restrict__ gsq_part, int* __restrict__ flag_part,
                                                  const Globals* __restrict__ gl, int pass) {
   __shared__ float lds_col[kWaves * 256];
@@ -93,7 +92,7 @@ __global__ __launch_bounds__(kThreads) void k_p0(const TDesc* __restrict__ descs
   const TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
   const bool clip_on = a.clip_norm > 0.0f;
-  if (pass == 1 && (!clip_on || d.mode == kModeFlat || gl->flag == 0)) return;
+  if (pass == 1 && (!clip_on || d.mode != kModeFac2D || gl->flag == 0)) return;
   float gsq = 0.0f;
   int flag = 0;
   if (a.grad != nullptr) {
@@ -101,11 +100,11 @@ __global__ __launch_bounds__(kThreads) void k_p0(const TDesc* __restrict__ descs
       const bool exact = (pass == 1) || !clip_on;
       const float scale = (pass == 1) ? clip_scale(gl->gnorm, a.clip_norm) : 1.0f;
       if (d.vec == 4)
-        p0_factored<4>(d, a.grad, it.a, it.b, exact, scale, a.clip_val, rowpart + d.rowpart_off,
-                       colpart + d.colpart_off, lds_col, lds_row, gsq, flag);
+        p0_factored<4>(d, a.grad, it.a, it.b, exact, scale, a.clip_val, part + d.part_off[0],
+                       part + d.part_off[1], lds_col, lds_row, gsq, flag);
       else
-        p0_factored<1>(d, a.grad, it.a, it.b, exact, scale, a.clip_val, rowpart + d.rowpart_off,
-                       colpart + d.colpart_off, lds_col, lds_row, gsq, flag);
+        p0_factored<1>(d, a.grad, it.a, it.b, exact, scale, a.clip_val, part + d.part_off[0],
+                       part + d.part_off[1], lds_col, lds_row, gsq, flag);
     } else {
       if (d.vec == 4) p0_flat<4>(d, a.grad, it.a, a.clip_val, gsq, flag);
       else p0_flat<1>(d, a.grad, it.a, a.clip_val, gsq, flag);
@@ -142,15 +141,39 @@ __global__ __launch_bounds__(kThreads) void k_gnorm(const double* __restrict__ g
 }
 
 // =============================================================================================
-// V0a: one block per 64 entries of a row / column vector.  Finishes the sums of g^2 over the
+// Sums of g^2 over one dim of an N-D tensor (any two factored dims): one thread per entry of the
+// statistics vector, walking the removed dim.  Small tensors only (conv kernels, cls tokens); the
+// gradient is clamped directly (no global-norm scale on this path).
+// =============================================================================================
+__global__ __launch_bounds__(kThreads) void k_p0_nd(const TDesc* __restrict__ descs,
+                                                    const PyloTensorArgs* __restrict__ dyn,
+                                                    const Item* __restrict__ items, float* __restrict__ part) {
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  const int w = it.b;
+  const int i = it.a * kThreads + threadIdx.x;
+  if (i >= d.len[w]) return;
+  const int X = d.nd_size[w], sX = d.nd_stride[w];
+  const long long base = (long long)(i / sX) * X * sX + (i % sX);
+  double s = 0.0;
+  for (int x = 0; x < X; ++x) {
+    const float g = clampf(*(const gfloat*)(a.grad + base + (long long)x * sX), a.clip_val);
+    s += (double)(g * g);
+  }
+  part[d.part_off[w] + i] = (float)s;
+}
+
+// =============================================================================================
+// V0a: one block per 64 entries of a statistics vector.  Finishes the sums of g^2 over the
 // partials, advances the three Adafactor accumulators (ELO_CELO2_naive.py:152-160) and leaves
 // per-block partial sums of  f, f^2, rsqrt(f+1e-8)^2  per decay.
 // =============================================================================================
 __global__ __launch_bounds__(kThreads) void k_v0a(const TDesc* __restrict__ descs,
                                                   const PyloTensorArgs* __restrict__ dyn,
                                                   const Item* __restrict__ items,
-                                                  const float* __restrict__ rowpart,
-                                                  const float* __restrict__ colpart,
+                                                  const float* __restrict__ part,
                                                   const Globals* __restrict__ gl, PyloDecays dec,
                                                   double* __restrict__ v0part) {
   __shared__ double lds[kWaves][kV0aEnt];
@@ -159,16 +182,15 @@ __global__ __launch_bounds__(kThreads) void k_v0a(const TDesc* __restrict__ desc
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
   const int which = it.b;
-  const int len = which ? d.C0 : d.R0;       // entries of this vector
-  const int other = which ? d.R0 : d.C0;     // the dim that was summed over
-  const int npart = which ? d.n_strips : d.n_colblk;
-  const float* part = which ? colpart + d.colpart_off : rowpart + d.rowpart_off;
+  const int len = d.len[which];
+  const int npart = d.npart[which];
+  const float* pp = part + d.part_off[which];
   const int e = threadIdx.x & 63, grp = threadIdx.x >> 6;
   const int i = it.a * kV0aEnt + e;
   {
     double s = 0.0;
     if (i < len)
-      for (int q = grp; q < npart; q += kWaves) s += (double)part[(size_t)q * len + i];
+      for (int q = grp; q < npart; q += kWaves) s += (double)pp[(size_t)q * len + i];
     lds[grp][e] = s;
   }
   __syncthreads();
@@ -179,12 +201,12 @@ __global__ __launch_bounds__(kThreads) void k_v0a(const TDesc* __restrict__ desc
     const float sc = clip_scale(gl->gnorm, a.clip_norm);
     s2 = (double)sc * (double)sc;
   }
-  const bool is_r = (which == 0) == (d.r_is_dim0 != 0);
+  const bool is_r = (which == 0) == (d.vec0_is_r != 0);
   float* fac = is_r ? a.fac_r : a.fac_c;
   double s_f = 0.0, s_ff = 0.0, s_rr = 0.0;
   if (i < len) {
     const double S = ((lds[0][e] + lds[1][e]) + lds[2][e]) + lds[3][e];
-    const float q = (float)(s2 * S / (double)other) + 1e-30f;
+    const float q = (float)(s2 * S / (double)d.sumlen[which]) + 1e-30f;
     const float beta = dec.beta_fac[k];
     const float f = beta * fac[(size_t)k * len + i] + (1.0f - beta) * q;
     fac[(size_t)k * len + i] = f;
@@ -202,13 +224,56 @@ __global__ __launch_bounds__(kThreads) void k_v0a(const TDesc* __restrict__ desc
   }
 }
 
+// Where entry i of vector `which` of tensor d lives in the factor / term tables.
+__device__ __forceinline__ size_t fac_index(const TDesc& d, int which, int k, int i) {
+  return (d.mode == kModeFac2D && which == 0) ? (size_t)d.fac_off[0] + (size_t)i * 4 + k
+                                              : (size_t)d.fac_off[which] + (size_t)k * d.pitch[which] + i;
+}
+template <int H>
+__device__ __forceinline__ size_t term_index(const TDesc& d, int which, int j, int i) {
+  return (d.mode == kModeFac2D && which == 0) ? (size_t)d.term_off[0] + (size_t)i * H + j
+                                              : (size_t)d.term_off[which] + (size_t)j * d.pitch[which] + i;
+}
+
+// Row_factor / col_factor of one entry, and the two normalised broadcast features it carries
+// (accumulator value and rsqrt(value + 1e-8)).  ELO_CELO2_naive.py:161-164,202-213
+__device__ __forceinline__ void vector_entry(bool is_r, const float* fac, int len, int i, const BScale& bs,
+                                             float (&fct)[3], float (&x0)[3], float (&x1)[3]) {
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    const float f = fac[(size_t)k * len + i];
+    fct[k] = is_r ? rsq(fmaxf(f / (bs.rcm[k] + 1e-9f), 1e-9f)) : rsq(fmaxf(f, 1e-9f));
+    x0[k] = f * (is_r ? bs.s[k] : bs.s[3 + k]);
+    x1[k] = rsq(f + 1e-8f) * (is_r ? bs.s[6 + k] : bs.s[9 + k]);
+  }
+}
+
+// First-layer contribution of the channels an entry carries: t_j = (bias_j) + sum_k x0_k w[ch_f+k][j]
+// + x1_k w[ch_q+k][j], with w (30, H) row-major (in, out).
+template <int H>
+__device__ __forceinline__ void vector_terms(const TDesc& d, int which, bool is_r, int i, const float (&x0)[3],
+                                             const float (&x1)[3], const float* __restrict__ w1,
+                                             const float* __restrict__ b1, float* __restrict__ term) {
+  const int ch_f = is_r ? 15 : 18, ch_q = is_r ? 21 : 24;
+#pragma unroll
+  for (int j = 0; j < H; ++j) {
+    float t = (which == 0) ? b1[j] : 0.0f;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      t = fmaf(x0[k], w1[(ch_f + k) * H + j], t);
+      t = fmaf(x1[k], w1[(ch_q + k) * H + j], t);
+    }
+    term[term_index<H>(d, which, j, i)] = t;
+  }
+}
+
 // =============================================================================================
-// V0b: one block per 1024 entries of a row / column vector.  Reduces the V0a partials of its
-// tensor, then writes the factor tables (row_factor / col_factor, ELO_CELO2_naive.py:161-164)
-// and, when first-layer weights are given, the per-row / per-column MLP terms: the 12 feature
-// channels that depend on the row or on the column only (fac_r_k, fac_c_k and their rsqrt) are
-// normalised and pushed through the first layer once per row / column instead of once per element.
-//   w1: (30, H) row-major, (in, out); b1: (H).  Bias goes into the dim-0 terms.
+// V0b: one block per 1024 entries of a statistics vector.  Reduces the V0a partials of its
+// tensor into the normalisation scales of the 12 broadcast channels and row_col_mean (BScale),
+// writes the factor tables and, when first-layer weights are given (shared by all tensors), the
+// per-row / per-column MLP terms: the 12 feature channels that depend on the row or on the column
+// only are normalised and pushed through the first layer once per row / column instead of once
+// per element.  The bias goes into the terms of vector 0.
 // =============================================================================================
 template <int H>
 __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ descs,
@@ -216,8 +281,7 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
                                                   const Item* __restrict__ items,
                                                   const double* __restrict__ v0part, float norm_eps,
                                                   const float* __restrict__ w1, const float* __restrict__ b1,
-                                                  float* __restrict__ fac0, float* __restrict__ fac1,
-                                                  float* __restrict__ term0, float* __restrict__ term1,
+                                                  float* __restrict__ fac_tab, float* __restrict__ term_tab,
                                                   BScale* __restrict__ bscale) {
   constexpr int G = 14;  // 14 groups x 18 (vector, slot) pairs = 252 threads
   __shared__ double red[G][2 * kNV0];
@@ -242,61 +306,58 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
     }
     __syncthreads();
   }
-  // sums of the r-role vector and of the c-role vector
-  const double* tr = tot + (d.r_is_dim0 ? 0 : kNV0);
-  const double* tc = tot + (d.r_is_dim0 ? kNV0 : 0);
-  float rcm[3], s_fr[3], s_rr[3], s_fc[3], s_rc[3];
+  const int rI = d.vec0_is_r ? 0 : 1, cI = 1 - rI;
+  const double* tr = tot + rI * kNV0;
+  const double* tc = tot + cI * kNV0;
+  const double len_r = (double)d.len[rI], len_c = (double)d.len[cI];
+  BScale bs;
 #pragma unroll
   for (int k = 0; k < 3; ++k) {
-    rcm[k] = (float)(tr[k * 3 + 0] / (double)d.len_r);
-    s_fr[k] = rsq(norm_eps + (float)(tr[k * 3 + 1] / (double)d.len_r));
-    s_rr[k] = rsq(norm_eps + (float)(tr[k * 3 + 2] / (double)d.len_r));
-    s_fc[k] = rsq(norm_eps + (float)(tc[k * 3 + 1] / (double)d.len_c));
-    s_rc[k] = rsq(norm_eps + (float)(tc[k * 3 + 2] / (double)d.len_c));
+    bs.rcm[k] = (float)(tr[k * 3 + 0] / len_r);
+    bs.s[k] = rsq(norm_eps + (float)(tr[k * 3 + 1] / len_r));        // fac_r_k
+    bs.s[3 + k] = rsq(norm_eps + (float)(tc[k * 3 + 1] / len_c));    // fac_c_k
+    bs.s[6 + k] = rsq(norm_eps + (float)(tr[k * 3 + 2] / len_r));    // rsqrt(fac_r_k + 1e-8)
+    bs.s[9 + k] = rsq(norm_eps + (float)(tc[k * 3 + 2] / len_c));    // rsqrt(fac_c_k + 1e-8)
   }
+  bs.pad_ = 0.0f;
   const int which = it.b;
-  const bool is_r = (which == 0) == (d.r_is_dim0 != 0);
-  if (which == 0 && it.a == 0 && threadIdx.x == 0) {
-    BScale bs;
-#pragma unroll
-    for (int k = 0; k < 3; ++k) {
-      bs.s[k] = s_fr[k]; bs.s[3 + k] = s_fc[k]; bs.s[6 + k] = s_rr[k]; bs.s[9 + k] = s_rc[k];
-      bs.rcm[k] = rcm[k];
-    }
-    bs.pad_ = 0.0f;
-    bscale[d.fac_slot] = bs;
-  }
-  const int len = which ? d.C0 : d.R0;
+  if (which == 0 && it.a == 0 && threadIdx.x == 0) bscale[d.fac_slot] = bs;
+  const bool is_r = (which == 0) == (d.vec0_is_r != 0);
+  const int len = d.len[which];
   const float* fac = is_r ? a.fac_r : a.fac_c;
-  // channel rows of the first layer this vector feeds: accumulator value, rsqrt(value + 1e-8)
-  const int ch_f = is_r ? 15 : 18, ch_q = is_r ? 21 : 24;
   for (int i = it.a * kV0bEnt + threadIdx.x; i < min(len, (it.a + 1) * kV0bEnt); i += kThreads) {
     float fct[3], x0[3], x1[3];
+    vector_entry(is_r, fac, len, i, bs, fct, x0, x1);
 #pragma unroll
-    for (int k = 0; k < 3; ++k) {
-      const float f = fac[(size_t)k * len + i];
-      fct[k] = is_r ? rsq(fmaxf(f / (rcm[k] + 1e-9f), 1e-9f)) : rsq(fmaxf(f, 1e-9f));
-      x0[k] = f * (is_r ? s_fr[k] : s_fc[k]);
-      x1[k] = rsq(f + 1e-8f) * (is_r ? s_rr[k] : s_rc[k]);
-    }
-    if (which == 0) store_f4(fac0 + d.fac0_off + (size_t)i * 4, fct[0], fct[1], fct[2], 0.0f);
-    else {
-#pragma unroll
-      for (int k = 0; k < 3; ++k) fac1[d.fac1_off + (size_t)k * d.C0r + i] = fct[k];
-    }
-    if (w1 != nullptr) {
-#pragma unroll
-      for (int j = 0; j < H; ++j) {
-        float t = (which == 0) ? b1[j] : 0.0f;
-#pragma unroll
-        for (int k = 0; k < 3; ++k) {
-          t = fmaf(x0[k], w1[(ch_f + k) * H + j], t);
-          t = fmaf(x1[k], w1[(ch_q + k) * H + j], t);
-        }
-        if (which == 0) term0[d.term0_off + (size_t)i * H + j] = t;
-        else term1[d.term1_off + (size_t)j * d.C0r + i] = t;
-      }
-    }
+    for (int k = 0; k < 3; ++k) fac_tab[fac_index(d, which, k, i)] = fct[k];
+    if (w1 != nullptr) vector_terms<H>(d, which, is_r, i, x0, x1, w1, b1, term_tab);
+  }
+}
+
+// First-layer terms with per-tensor weights that only exist after k_v0b has run (VeLO: the LSTM
+// emits them).  w1 / b1 are per-tensor blocks `w_stride` floats apart, (30, H) then (H).
+template <int H>
+__global__ __launch_bounds__(kThreads) void k_terms(const TDesc* __restrict__ descs,
+                                                    const PyloTensorArgs* __restrict__ dyn,
+                                                    const Item* __restrict__ items,
+                                                    const BScale* __restrict__ bscale,
+                                                    const float* __restrict__ w1_all, int w_stride,
+                                                    float* __restrict__ term_tab) {
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  const BScale bs = bscale[d.fac_slot];
+  const float* w1 = w1_all + (size_t)it.tensor * w_stride;
+  const float* b1 = w1 + 30 * H;
+  const int which = it.b;
+  const bool is_r = (which == 0) == (d.vec0_is_r != 0);
+  const int len = d.len[which];
+  const float* fac = is_r ? a.fac_r : a.fac_c;
+  for (int i = it.a * kV0bEnt + threadIdx.x; i < min(len, (it.a + 1) * kV0bEnt); i += kThreads) {
+    float fct[3], x0[3], x1[3];
+    vector_entry(is_r, fac, len, i, bs, fct, x0, x1);
+    vector_terms<H>(d, which, is_r, i, x0, x1, w1, b1, term_tab);
   }
 }
 

@@ -1,0 +1,641 @@
+// VeLO: element kernels (statistics / apply for factored 2-D, factored N-D and non-factored
+// tensors), the per-tensor reduction with the LSTM input features, and the per-tensor LSTM that
+// emits each tensor's MLP weights.
+#pragma once
+
+#include "k_celo2.h"
+#include "k_gradstats.h"
+#include "pylo_common.h"
+
+namespace pylo {
+
+// Folded per-tensor weights (floats): first layer rows scaled by the channel normalisers
+// (18 per-element rows for factored tensors, all 30 rows for non-factored ones), (in, out).
+constexpr int kVW1 = 0, kVB1 = 120, kVWH = 124, kVBH = 140, kVWO = 144, kVBO = 152, kVPS = 154, kVLR = 155,
+              kVFold = 160;
+constexpr int kVCanon = 128;   // per-tensor un-scaled first layer (30,4) + bias 4, for k_terms
+constexpr int kVBank = 159;    // floats per bank entry: W_in (4,30) | b_in 4 | W_h (4,4) | b_h 4 | W_out (3,4) | b_out 3
+constexpr int kXW = 32;        // row pitch of the LSTM input features (30 used)
+constexpr int kGateBT = 8;     // tensors per k_velo_gates block
+
+struct VeloStep {              // by-value kernel argument: scalars of one step
+  float frac[PYLO_MAX_GROUPS][9];
+};
+
+// ---------------------------------------------------------------------------------------------
+// element access for factored tensors, 2-D fast path (V consecutive elements of one row) or
+// generic N-D (V == 1)
+// ---------------------------------------------------------------------------------------------
+template <int V, bool ND>
+__device__ __forceinline__ void lo_load(const TDesc& d, const PyloTensorArgs& a, long long idx,
+                                        const float* __restrict__ fac_tab, ElemIn<V>& x) {
+  if constexpr (!ND) {
+    load_elems<V>(d, a, idx, 1.0f, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1], x);
+  } else {
+    const long long n = d.n;
+    x.g[0] = clampf(*(const gfloat*)(a.grad + idx), a.clip_val);
+    x.p[0] = *(const gfloat*)(a.param + idx);
+    x.m[0][0] = *(const gfloat*)(a.mom + idx);
+    x.m[0][1] = *(const gfloat*)(a.mom + n + idx);
+    x.m[0][2] = *(const gfloat*)(a.mom + 2 * n + idx);
+    x.rms[0] = *(const gfloat*)(a.rms + idx);
+    const unsigned u = (unsigned)idx;
+    const unsigned s0 = (unsigned)d.nd_stride[0], z0 = (unsigned)d.nd_size[0] * s0;
+    const unsigned s1 = (unsigned)d.nd_stride[1], z1 = (unsigned)d.nd_size[1] * s1;
+    x.i0 = (int)((u / z0) * s0 + u % s0);
+    x.i1 = (int)((u / z1) * s1 + u % s1);
+#pragma unroll
+    for (int k = 0; k < 3; ++k)
+      x.rfcf[0][k] = fac_tab[d.fac_off[0] + (size_t)k * d.pitch[0] + x.i0] *
+                     fac_tab[d.fac_off[1] + (size_t)k * d.pitch[1] + x.i1];
+  }
+}
+
+// h[v][j] = term0[j] + term1[j] of the element's row / column
+template <int V, bool ND, int H>
+__device__ __forceinline__ void lo_terms(const TDesc& d, const ElemIn<V>& x, const float* __restrict__ term_tab,
+                                         float (&h)[V][H]) {
+  if constexpr (!ND) {
+    const float* t0 = term_tab + d.term_off[0] + (size_t)x.i0 * H;
+    const float* t1 = term_tab + d.term_off[1];
+#pragma unroll
+    for (int j = 0; j < H; ++j) {
+      float tb[V];
+      load_vec<V>(t1 + (size_t)j * d.pitch[1] + x.i1, tb);
+      const float ta = *(const gfloat*)(t0 + j);
+#pragma unroll
+      for (int v = 0; v < V; ++v) h[v][j] = ta + tb[v];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < H; ++j)
+      h[0][j] = term_tab[d.term_off[0] + (size_t)j * d.pitch[0] + x.i0] +
+                term_tab[d.term_off[1] + (size_t)j * d.pitch[1] + x.i1];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// statistics pass
+// ---------------------------------------------------------------------------------------------
+struct VeloAcc {
+  float ch[30];   // sum of squares per channel (factored tensors fill the 18 per-element ones)
+  float lstm[8];  // sum m_k, sum m_k^2, sum rms, sum rms^2 over the accumulators before the update
+};
+
+__device__ __forceinline__ void lstm_sums(const float (&m)[3], float rms, float (&s)[8]) {
+#pragma unroll
+  for (int k = 0; k < 3; ++k) { s[k] += m[k]; s[3 + k] = fmaf(m[k], m[k], s[3 + k]); }
+  s[6] += rms;
+  s[7] = fmaf(rms, rms, s[7]);
+}
+
+template <int V, bool ND>
+__device__ __forceinline__ void velo_stats_fac(const TDesc& d, const PyloTensorArgs& a, int chunk,
+                                               const EmaConsts& e, const float* __restrict__ fac_tab, VeloAcc& acc) {
+  const long long base = (long long)chunk * (kThreads * V * kElemIters);
+#pragma unroll 2
+  for (int it = 0; it < kElemIters; ++it) {
+    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
+    if (idx >= d.n) break;
+    ElemIn<V> x;
+    lo_load<V, ND>(d, a, idx, fac_tab, x);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      lstm_sums(x.m[v], x.rms[v], acc.lstm);
+      ema_update(e, x.g[v], x.m[v], x.rms[v]);
+      float f[kNStat];
+      lo_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.rfcf[v], 1e-6f, f);
+#pragma unroll
+      for (int c = 0; c < kNStat; ++c) acc.ch[stat_channel(c)] = fmaf(f[c], f[c], acc.ch[stat_channel(c)]);
+    }
+  }
+}
+
+// Non-factored tensor: the 30 channels of one element (Velo_naive.py:60-68,439-451,478-488).
+// m, rms, v are the accumulators after this step's update; fm_eps is added to v under the
+// power -1/2 of the last group (0 for VeLO, 1e-6 for AdafacLO).
+__device__ __forceinline__ void vec_features(float g, float p, const float (&m)[3], float rms,
+                                             const float (&v)[3], float fm_eps, float (&f)[30]) {
+  const float rs = rsq(rms + 1e-6f);
+  f[0] = g;
+  f[1] = fminf(fmaxf(g, -0.1f), 0.1f);
+  f[2] = p;
+  f[6] = rms;
+  f[10] = rs;
+  f[14] = g * rs;
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    f[3 + k] = m[k];
+    f[7 + k] = m[k] * rs;
+    f[11 + k] = g * rsq(fmaxf(v[k] + 1e-9f, 1e-9f));
+    f[15 + k] = v[k];
+    f[18 + k] = v[k];
+    const float q = rsq(v[k] + 1e-8f);
+    f[21 + k] = q;
+    f[24 + k] = q;
+    f[27 + k] = m[k] * rsq(v[k] + fm_eps);
+  }
+}
+
+template <int V>
+struct VecIn {
+  float g[V], p[V], m[V][3], rms[V], v[V][3];
+};
+
+template <int V>
+__device__ __forceinline__ void vec_load(const TDesc& d, const PyloTensorArgs& a, long long idx, VecIn<V>& x) {
+  const long long n = d.n;
+  float t[3][V], u[3][V];
+  load_vec<V>(a.grad + idx, x.g);
+  load_vec<V>(a.param + idx, x.p);
+  load_vec<V>(a.rms + idx, x.rms);
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    load_vec<V>(a.mom + k * n + idx, t[k]);
+    load_vec<V>(a.fac_v + k * n + idx, u[k]);
+  }
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    x.g[v] = clampf(x.g[v], a.clip_val);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { x.m[v][k] = t[k][v]; x.v[v][k] = u[k][v]; }
+  }
+}
+
+__device__ __forceinline__ void vec_update(const EmaConsts& e, const PyloDecays& dec, float g, float (&m)[3],
+                                           float& rms, float (&v)[3]) {
+  ema_update(e, g, m, rms);
+  const float q = g * g + 1e-30f;
+#pragma unroll
+  for (int k = 0; k < 3; ++k) v[k] = dec.beta_fac[k] * v[k] + (1.0f - dec.beta_fac[k]) * q;
+}
+
+template <int V>
+__device__ __forceinline__ void velo_stats_vec(const TDesc& d, const PyloTensorArgs& a, int chunk,
+                                               const EmaConsts& e, const PyloDecays& dec, VeloAcc& acc) {
+  const long long base = (long long)chunk * (kThreads * V * kElemIters);
+  for (int it = 0; it < kElemIters; ++it) {
+    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
+    if (idx >= d.n) break;
+    VecIn<V> x;
+    vec_load<V>(d, a, idx, x);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      lstm_sums(x.m[v], x.rms[v], acc.lstm);
+      vec_update(e, dec, x.g[v], x.m[v], x.rms[v], x.v[v]);
+      float f[30];
+      vec_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.v[v], 0.0f, f);
+#pragma unroll
+      for (int c = 0; c < 30; ++c) acc.ch[c] = fmaf(f[c], f[c], acc.ch[c]);
+    }
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void k_velo_stats(const TDesc* __restrict__ descs,
+                                                         const PyloTensorArgs* __restrict__ dyn,
+                                                         const Item* __restrict__ items,
+                                                         const float* __restrict__ fac_tab, PyloDecays dec,
+                                                         double* __restrict__ stats_part) {
+  __shared__ float red[kWaves][38];
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  const EmaConsts e = make_ema(dec);
+  VeloAcc acc;
+#pragma unroll
+  for (int c = 0; c < 30; ++c) acc.ch[c] = 0.0f;
+#pragma unroll
+  for (int c = 0; c < 8; ++c) acc.lstm[c] = 0.0f;
+  if (d.mode == kModeFac2D) {
+    if (d.vec == 4) velo_stats_fac<4, false>(d, a, it.a, e, fac_tab, acc);
+    else velo_stats_fac<1, false>(d, a, it.a, e, fac_tab, acc);
+  } else if (d.mode == kModeFacND) {
+    velo_stats_fac<1, true>(d, a, it.a, e, fac_tab, acc);
+  } else {
+    if (d.vec == 4) velo_stats_vec<4>(d, a, it.a, e, dec, acc);
+    else velo_stats_vec<1>(d, a, it.a, e, dec, acc);
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int c = 0; c < 30; ++c) {
+    const float s = wave_sum(acc.ch[c]);
+    if (lane == 0) red[wave][c] = s;
+  }
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    const float s = wave_sum(acc.lstm[c]);
+    if (lane == 0) red[wave][30 + c] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x < 38) {
+    const int c = threadIdx.x;
+    stats_part[(size_t)blockIdx.x * kStatW + c] =
+        ((double)red[0][c] + (double)red[1][c]) + ((double)red[2][c] + (double)red[3][c]);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// loss features (Velo_naive.py:147-175): 10 EMAs of the clipped loss, updated in place
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void k_velo_loss(float* __restrict__ means, float* __restrict__ running_min,
+                                                  const float* __restrict__ decays, int* __restrict__ iteration,
+                                                  const float* __restrict__ loss_p, float* __restrict__ lossfeat) {
+  __shared__ float cor_s[10], rmin_s[10];
+  const int dI = threadIdx.x;
+  const int it = *iteration;
+  const float loss = *loss_p;
+  float cor = -INFINITY, dec = 0.0f, mean = 0.0f, pw = 0.0f;
+  if (dI < 10) {
+    dec = decays[dI];
+    mean = means[dI];
+    pw = powf(dec, (float)(it + 1));
+    cor = mean / (1.0f - pw);
+  }
+  float mx = cor;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  const float approx_max = (it == 0) ? loss : mx;
+  const float l = fminf(fabsf(approx_max) * 2.0f, loss);
+  if (dI < 10) {
+    const float m2 = mean * dec + l * (1.0f - dec);
+    const float cor2 = m2 / (1.0f - pw);
+    const float rmin = fminf(running_min[dI], cor2);
+    means[dI] = m2;
+    running_min[dI] = rmin;
+    cor_s[dI] = cor2;
+    rmin_s[dI] = rmin;
+  }
+  __syncthreads();
+  if (dI == 0) *iteration = it + 1;
+  if (dI < 9) {
+    const float den = fmaxf(1e-8f, cor_s[dI + 1] - rmin_s[dI]);
+    float f = (cor_s[dI] - rmin_s[dI]) / den - 1.0f;
+    f = fminf(fmaxf(f, -1.0f), 1.0f);
+    lossfeat[dI] = (it + 1 <= 2) ? f * 0.0f : f;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// per-tensor totals of the statistics partials, then (VeLO) the 30 LSTM input features of the
+// tensor (Velo_naive.py:178-206), written to row T-1-t (the reference flips the tensor order).
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float clip_log_abs10(double v) {
+  const float x = (float)v;
+  return 0.5f * fminf(fmaxf(logf(1e-8f + fabsf(x * 10.0f)), -5.0f), 5.0f);
+}
+
+__global__ __launch_bounds__(kThreads) void k_lo_reduce(const TDesc* __restrict__ descs,
+                                                        const PyloTensorArgs* __restrict__ dyn, int T,
+                                                        const double* __restrict__ stats_part,
+                                                        double* __restrict__ totals,
+                                                        const float* __restrict__ lossfeat, VeloStep st,
+                                                        float* __restrict__ xfeat) {
+  constexpr int G = 6;  // 6 groups x 40 sums = 240 threads
+  __shared__ double part[G][kStatW];
+  __shared__ double tot[kStatW];
+  const int t = blockIdx.x;
+  const TDesc d = descs[t];
+  const PyloTensorArgs a = dyn[t];
+  const int c = threadIdx.x % kStatW, gI = threadIdx.x / kStatW;
+  if (gI < G) {
+    double s = 0.0;
+    if (a.grad != nullptr && c < 38)
+      for (int b = gI; b < d.nblk; b += G) s += stats_part[(size_t)(d.blk0 + b) * kStatW + c];
+    part[gI][c] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x < kStatW) {
+    double s = 0.0;
+    for (int g2 = 0; g2 < G; ++g2) s += part[g2][threadIdx.x];
+    tot[threadIdx.x] = s;
+    totals[(size_t)t * kStatW + threadIdx.x] = s;
+  }
+  __syncthreads();
+  if (xfeat == nullptr || threadIdx.x >= 30) return;
+  const int q = threadIdx.x;
+  const double n = (double)(d.n > 0 ? d.n : 1);
+  const float nu = rsq(fmaxf((float)(tot[2] / n), 1e-9f));
+  const double nu2 = (double)nu * (double)nu;
+  float val;
+  if (q < 9) {
+    val = st.frac[a.group][q];
+  } else if (q < 18) {
+    val = lossfeat[q - 9];
+  } else if (q == 18) {
+    val = clip_log_abs10((double)nu * (tot[kSumR] / n));
+  } else if (q < 24) {
+    val = (q - 19 == d.rank) ? 1.0f : 0.0f;
+  } else {
+    const int k = (q - 24) % 3;
+    const double mean_m = tot[kSumM + k] / n;
+    if (q < 27) {
+      val = clip_log_abs10(nu2 * (tot[kSumMM + k] / n - mean_m * mean_m));
+    } else {  // the reference subtracts mean_m (not mean_rms) from rms here (Velo_naive.py:198)
+      const double mean_r = tot[kSumR] / n;
+      val = clip_log_abs10(nu2 * (tot[kSumRR] / n - 2.0 * mean_m * mean_r + mean_m * mean_m));
+    }
+  }
+  xfeat[(size_t)(T - 1 - t) * kXW + q] = val;
+}
+
+// ---------------------------------------------------------------------------------------------
+// LSTM (VeLO_RNN.py:43-66,110-135).  All weights are pre-transposed to (in, out) by the host.
+// Rows are in the reference's order r = T-1-t.
+// ---------------------------------------------------------------------------------------------
+// x' = final_mix(x) + max_r relu(mix2(x));  xT[u][r] = x'[r][u], xT[H+u][r] = h[r][u]
+__global__ __launch_bounds__(kThreads) void k_velo_mix(const float* __restrict__ xfeat, int T, int Tpad, int H,
+                                                       const float* __restrict__ w2t, const float* __restrict__ b2,
+                                                       const float* __restrict__ wft, const float* __restrict__ bf,
+                                                       const float* __restrict__ h_state, float* __restrict__ xT) {
+  __shared__ float mx_s[kWaves][64];
+  const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+  const int u = blockIdx.x * 64 + lane;
+  const bool ok = u < H;
+  float mx = 0.0f;  // relu output is >= 0
+  for (int r = grp; r < T; r += kWaves) {
+    float acc = ok ? b2[u] : 0.0f;
+    const float* xr = xfeat + (size_t)r * kXW;
+    if (ok) {
+#pragma unroll
+      for (int k = 0; k < 30; ++k) acc = fmaf(xr[k], w2t[k * H + u], acc);
+    }
+    mx = fmaxf(mx, acc);
+  }
+  mx_s[grp][lane] = mx;
+  __syncthreads();
+  const float v = fmaxf(fmaxf(mx_s[0][lane], mx_s[1][lane]), fmaxf(mx_s[2][lane], mx_s[3][lane]));
+  if (!ok) return;
+  for (int r = grp; r < Tpad; r += kWaves) {
+    float acc = 0.0f, hv = 0.0f;
+    if (r < T) {
+      acc = bf[u];
+      const float* xr = xfeat + (size_t)r * kXW;
+#pragma unroll
+      for (int k = 0; k < 30; ++k) acc = fmaf(xr[k], wft[k * H + u], acc);
+      acc += v;
+      hv = h_state[(size_t)r * H + u];
+    }
+    xT[(size_t)u * Tpad + r] = acc;
+    xT[(size_t)(H + u) * Tpad + r] = hv;
+  }
+}
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// gates = [x', h] W^T + b in chunks i, g, f, o;  c = sig(f+1) c + sig(i) tanh(g);  h = sig(o) tanh(c)
+__global__ __launch_bounds__(128) void k_velo_gates(const float* __restrict__ xT, int T, int Tpad, int H,
+                                                    const float* __restrict__ wt /*(2H, 4H)*/,
+                                                    const float* __restrict__ b /*4H*/,
+                                                    float* __restrict__ h_state, float* __restrict__ c_state) {
+  const int u = blockIdx.y * 128 + threadIdx.x;
+  if (u >= H) return;
+  const int r0 = blockIdx.x * kGateBT;
+  float acc[4][kGateBT];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const float bias = b[g * H + u];
+#pragma unroll
+    for (int t = 0; t < kGateBT; ++t) acc[g][t] = bias;
+  }
+  const int K2 = 2 * H;
+  for (int k = 0; k < K2; ++k) {
+    float w[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) w[g] = wt[(size_t)k * 4 * H + g * H + u];
+    const float* xr = xT + (size_t)k * Tpad + r0;
+#pragma unroll
+    for (int t = 0; t < kGateBT; ++t) {
+      const float xv = xr[t];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) acc[g][t] = fmaf(xv, w[g], acc[g][t]);
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < kGateBT; ++t) {
+    const int r = r0 + t;
+    if (r < T) {
+      const float c_old = c_state[(size_t)r * H + u];
+      const float c_new = sigmoidf_(acc[2][t] + 1.0f) * c_old + sigmoidf_(acc[0][t]) * tanhf(acc[1][t]);
+      c_state[(size_t)r * H + u] = c_new;
+      h_state[(size_t)r * H + u] = sigmoidf_(acc[3][t]) * tanhf(c_new);
+    }
+  }
+}
+
+// One block per tensor row r: controls = h Wc^T + bc, lr_mult = h.wlr + blr, the tensor's MLP =
+// 100 * mean_i(control_i * bank_i) (VeLO_MLP.py:92-126), then the weight blocks the element
+// kernels read: un-scaled first layer for k_terms, and the folded block (first-layer rows scaled
+// by rsqrt(1e-5 + mean f_c^2), param_scale = sqrt(mean p^2 + 1e-9), lr_mult).
+__global__ __launch_bounds__(kThreads) void k_velo_heads(const TDesc* __restrict__ descs, int T, int H, int K,
+                                                         const float* __restrict__ h_state,
+                                                         const float* __restrict__ wct /*(H,K)*/,
+                                                         const float* __restrict__ bc, const float* __restrict__ wlr,
+                                                         const float* __restrict__ blr,
+                                                         const float* __restrict__ bank /*(K,159)*/,
+                                                         const double* __restrict__ totals,
+                                                         float* __restrict__ canon, float* __restrict__ wfold,
+                                                         float* __restrict__ controls_out,
+                                                         float* __restrict__ lr_mult_out) {
+  extern __shared__ float smem[];  // hs[H] | ctrl[K] | wm[160] | sc[32] | red[4]
+  float* hs = smem;
+  float* ctrl = hs + H;
+  float* wm = ctrl + K;
+  float* sc = wm + 160;
+  float* red = sc + 32;
+  const int r = blockIdx.x;
+  const int t = T - 1 - r;
+  const TDesc d = descs[t];
+  for (int u = threadIdx.x; u < H; u += kThreads) hs[u] = h_state[(size_t)r * H + u];
+  __syncthreads();
+  for (int j = threadIdx.x; j < K; j += kThreads) {
+    float acc = bc[j];
+    for (int u = 0; u < H; ++u) acc = fmaf(hs[u], wct[(size_t)u * K + j], acc);
+    ctrl[j] = acc;
+    if (controls_out != nullptr) controls_out[(size_t)r * K + j] = acc;
+  }
+  {
+    float s = 0.0f;
+    for (int u = threadIdx.x; u < H; u += kThreads) s = fmaf(hs[u], wlr[u], s);
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  }
+  if (threadIdx.x < 30) {
+    const double n = (double)(d.n > 0 ? d.n : 1);
+    sc[threadIdx.x] = rsq(1e-5f + (float)(totals[(size_t)t * kStatW + threadIdx.x] / n));
+  }
+  __syncthreads();
+  const float lr_mult = ((red[0] + red[1]) + (red[2] + red[3])) + blr[0];
+  for (int q = threadIdx.x; q < kVBank; q += kThreads) {
+    float acc = 0.0f;
+    for (int i = 0; i < K; ++i) acc = fmaf(ctrl[i], bank[(size_t)i * kVBank + q], acc);
+    wm[q] = (acc / (float)K) * 100.0f;
+  }
+  __syncthreads();
+  float* cn = canon + (size_t)t * kVCanon;
+  float* wf = wfold + (size_t)t * kVFold;
+  const bool factored = d.mode == kModeFac2D || d.mode == kModeFacND;
+  for (int i = threadIdx.x; i < 120; i += kThreads) {
+    const int k = i / 4, j = i % 4;
+    cn[i] = wm[j * 30 + k];
+    if (factored) {
+      if (k < kNStat) wf[kVW1 + i] = wm[j * 30 + stat_channel(k)] * sc[stat_channel(k)];
+    } else {
+      wf[kVW1 + i] = wm[j * 30 + k] * sc[k];
+    }
+  }
+  if (threadIdx.x < 4) { cn[120 + threadIdx.x] = wm[120 + threadIdx.x]; wf[kVB1 + threadIdx.x] = wm[120 + threadIdx.x]; }
+  if (threadIdx.x < 16) wf[kVWH + threadIdx.x] = wm[124 + (threadIdx.x % 4) * 4 + threadIdx.x / 4];   // (in,out)
+  if (threadIdx.x < 4) wf[kVBH + threadIdx.x] = wm[140 + threadIdx.x];
+  if (threadIdx.x < 8) wf[kVWO + threadIdx.x] = wm[144 + (threadIdx.x % 2) * 4 + threadIdx.x / 2];    // [k][j<2]
+  if (threadIdx.x < 2) wf[kVBO + threadIdx.x] = wm[156 + threadIdx.x];
+  if (threadIdx.x == 0) {
+    const double n = (double)(d.n > 0 ? d.n : 1);
+    wf[kVPS] = sqrtf((float)(totals[(size_t)t * kStatW + 2] / n) + 1e-9f);
+    wf[kVLR] = lr_mult;
+    if (lr_mult_out != nullptr) lr_mult_out[r] = lr_mult;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// apply pass: accumulators advanced and written, features, 30->4->4->3 MLP,
+//   p <- p - lr * lr_mult * param_scale * o0 * exp(o1 * exp_mult) * step_mult;  p <- p - wd*lr*p
+// (Velo_naive.py:491-502)
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float velo_update(float p, const float (&h1)[4], const cfloat* w, const PyloTensorArgs& a) {
+  float o0 = w[kVBO + 0], o1 = w[kVBO + 1];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float hk = fmaxf(h1[k], 0.0f);
+    o0 = fmaf(hk, w[kVWO + k * 2 + 0], o0);
+    o1 = fmaf(hk, w[kVWO + k * 2 + 1], o1);
+  }
+  float step = w[kVPS] * ((o0 * expf(o1 * a.exp_mult)) * a.step_mult);
+  step = w[kVLR] * step;
+  p = fmaf(step, -a.lr, p);
+  if (a.weight_decay > 0.0f) p = fmaf(p, -(a.weight_decay * a.lr), p);
+  return p;
+}
+
+__device__ __forceinline__ void velo_hidden(const float (&h0)[4], const cfloat* w, float (&h1)[4]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) h1[j] = w[kVBH + j];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float hk = fmaxf(h0[k], 0.0f);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) h1[j] = fmaf(hk, w[kVWH + k * 4 + j], h1[j]);
+  }
+}
+
+template <int V, bool ND>
+__device__ __forceinline__ void velo_apply_fac(const TDesc& d, const PyloTensorArgs& a, int chunk,
+                                               const EmaConsts& e, const float* __restrict__ fac_tab,
+                                               const float* __restrict__ term_tab, const float* wbase) {
+  const long long base = (long long)chunk * (kThreads * V * kElemIters);
+  const long long n = d.n;
+  for (int it = 0; it < kElemIters; ++it) {
+    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
+    if (idx >= n) break;
+    ElemIn<V> x;
+    lo_load<V, ND>(d, a, idx, fac_tab, x);
+    float h[V][4];
+    lo_terms<V, ND, 4>(d, x, term_tab, h);
+    float f[V][kNStat], m0[V], m1[V], m2[V], pn[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      ema_update(e, x.g[v], x.m[v], x.rms[v]);
+      m0[v] = x.m[v][0]; m1[v] = x.m[v][1]; m2[v] = x.m[v][2];
+      lo_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.rfcf[v], 1e-6f, f[v]);
+    }
+    const cfloat* w = launder(wbase);
+#pragma unroll
+    for (int c = 0; c < kNStat; ++c) {
+      float wc[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wc[j] = w[kVW1 + c * 4 + j];
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) h[v][j] = fmaf(f[v][c], wc[j], h[v][j]);
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      float h1[4];
+      velo_hidden(h[v], w, h1);
+      pn[v] = velo_update(x.p[v], h1, w, a);
+    }
+    store_vec<V>(a.mom + idx, m0);
+    store_vec<V>(a.mom + n + idx, m1);
+    store_vec<V>(a.mom + 2 * n + idx, m2);
+    store_vec<V>(a.rms + idx, x.rms);
+    store_vec<V>(a.param + idx, pn);
+  }
+}
+
+template <int V>
+__device__ __forceinline__ void velo_apply_vec(const TDesc& d, const PyloTensorArgs& a, int chunk,
+                                               const EmaConsts& e, const PyloDecays& dec, const float* wbase) {
+  const long long base = (long long)chunk * (kThreads * V * kElemIters);
+  const long long n = d.n;
+  for (int it = 0; it < kElemIters; ++it) {
+    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
+    if (idx >= n) break;
+    VecIn<V> x;
+    vec_load<V>(d, a, idx, x);
+    const cfloat* w = launder(wbase);
+    float pn[V], mo[3][V], vo[3][V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      vec_update(e, dec, x.g[v], x.m[v], x.rms[v], x.v[v]);
+      float f[30];
+      vec_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.v[v], 0.0f, f);
+      float h0[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) h0[j] = w[kVB1 + j];
+#pragma unroll
+      for (int c = 0; c < 30; ++c) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) h0[j] = fmaf(f[c], w[kVW1 + c * 4 + j], h0[j]);
+      }
+      float h1[4];
+      velo_hidden(h0, w, h1);
+      pn[v] = velo_update(x.p[v], h1, w, a);
+#pragma unroll
+      for (int k = 0; k < 3; ++k) { mo[k][v] = x.m[v][k]; vo[k][v] = x.v[v][k]; }
+    }
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      store_vec<V>(a.mom + k * n + idx, mo[k]);
+      store_vec<V>(a.fac_v + k * n + idx, vo[k]);
+    }
+    store_vec<V>(a.rms + idx, x.rms);
+    store_vec<V>(a.param + idx, pn);
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void k_velo_apply(const TDesc* __restrict__ descs,
+                                                         const PyloTensorArgs* __restrict__ dyn,
+                                                         const Item* __restrict__ items,
+                                                         const float* __restrict__ fac_tab,
+                                                         const float* __restrict__ term_tab, PyloDecays dec,
+                                                         const float* __restrict__ wfold) {
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  const EmaConsts e = make_ema(dec);
+  const float* w = wfold + (size_t)it.tensor * kVFold;
+  if (d.mode == kModeFac2D) {
+    if (d.vec == 4) velo_apply_fac<4, false>(d, a, it.a, e, fac_tab, term_tab, w);
+    else velo_apply_fac<1, false>(d, a, it.a, e, fac_tab, term_tab, w);
+  } else if (d.mode == kModeFacND) {
+    velo_apply_fac<1, true>(d, a, it.a, e, fac_tab, term_tab, w);
+  } else {
+    if (d.vec == 4) velo_apply_vec<4>(d, a, it.a, e, dec, w);
+    else velo_apply_vec<1>(d, a, it.a, e, dec, w);
+  }
+}
+
+}  // namespace pylo

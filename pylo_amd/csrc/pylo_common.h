@@ -31,31 +31,49 @@ __host__ __device__ constexpr int stat_channel(int c) { return c < 15 ? c : c + 
 constexpr int kC2W1 = 0, kC2WH = 144, kC2BH = 208, kC2WO = 216, kC2BO = 232, kC2Fold = 240;
 
 // ---- plan tables (device copies live in the caller's workspace) -----------------------------
-enum : int { kModeFlat = 0, kModeFac2D = 1 };
+// kModeFlat   no factored statistics, no MLP: CELO2 tensors routed to AdamW
+// kModeFac2D  2-D factored tensor, tiled fast path
+// kModeFacND  >2-D factored tensor (any two dims), generic indexing, dword accesses
+// kModeVec    VeLO / AdafacLO tensor with fewer than 2 dims: per-element accumulator fac_v
+enum : int { kModeFlat = 0, kModeFac2D = 1, kModeFacND = 2, kModeVec = 3 };
 
+// A factored tensor owns two statistics vectors.  2-D: vector 0 is indexed by the dim-0
+// coordinate (sums over dim 1), vector 1 by the dim-1 coordinate.  N-D: vector 0 is the tensor
+// with the largest dim removed (the reference's fac_vec_row), vector 1 with the 2nd-largest removed.
 struct TDesc {
   long long n;
-  int mode;        // kModeFlat: no factored statistics (CELO2 AdamW tensors); kModeFac2D: 2-D factored
-  int vec;         // 4: 128-bit loads (row length % 4 == 0); 1: dword loads
-  int R0, C0;      // sizes of dim 0 / dim 1
-  int C0r;         // C0 rounded up to a multiple of 4 (row pitch of the dim-1 tables)
-  int r_is_dim0;   // fac_r / row_factor are indexed by the dim-0 coordinate (largest dim is dim 1)
-  int len_r, len_c;
+  int mode;
+  int vec;          // 4: 128-bit accesses (2-D with C0 % 4 == 0, flat/vec with n % 4 == 0); 1: dword
+  int R0, C0;       // 2-D: sizes of dim 0 / dim 1
+  int vec0_is_r;    // vector 0 carries fac_r / row_factor (else fac_c / col_factor)
+  int len[2];       // entries of vector 0 / 1
+  int sumlen[2];    // elements summed into one entry
+  int npart[2];     // partial rows to add up per entry (2-D: column blocks / strips; N-D: 1)
+  int pitch[2];     // row pitch of the SoA tables of vector 0 / 1 (len rounded up to 4)
+  int nd_size[2];   // N-D: size and stride of the dim removed from vector 0 / 1;
+  int nd_stride[2]; //      entry = (idx / (size*stride)) * stride + idx % stride
   int n_strips, n_colblk;
-  int blk0, nblk;  // range of element-chunk blocks (rows of the statistics partials)
-  int fac_slot;    // index among factored tensors
-  long long rowpart_off, colpart_off;  // floats
-  long long fac0_off, fac1_off;        // floats: dim-0 factors [R0][4], dim-1 factors [3][C0r]
-  long long term0_off, term1_off;      // floats: dim-0 terms [R0][H], dim-1 terms [H][C0r]
-  int v0a_first[2], v0a_n[2];          // k_v0a blocks of the dim-0 / dim-1 vector
+  int blk0, nblk;   // range of element-chunk blocks (rows of the statistics partials)
+  int fac_slot;     // index among factored tensors, -1 otherwise
+  int rank;         // number of dims larger than 1 (VeLO's rank one-hot feature)
+  long long part_off[2];  // floats, partial sums of g^2
+  long long fac_off[2];   // floats, factor tables: 2-D vector 0 is AoS [len][4], everything else SoA [3][pitch]
+  long long term_off[2];  // floats, first-layer terms: 2-D vector 0 is AoS [len][H], else SoA [H][pitch]
+  int v0a_first[2], v0a_n[2];  // k_v0a blocks of vector 0 / 1
 };
 
 struct Item {
   int tensor;
-  int a;  // P0: strip (or flat chunk); element kernels: chunk; V0: chunk
-  int b;  // P0: column block; V0: 0 = dim-0 vector, 1 = dim-1 vector
+  int a;  // P0: strip (or flat chunk); element kernels: chunk; V0 / N-D sums: chunk
+  int b;  // P0: column block; V0 / N-D sums: vector 0 or 1
   int pad_;
 };
+
+// Width of one row of statistics partials (doubles): sum of squares per feature channel in the
+// reference's 30-channel order, then the per-tensor LSTM input sums of VeLO taken over the
+// accumulators *before* the update: sum m_k (30..32), sum m_k^2 (33..35), sum rms (36), sum rms^2 (37).
+constexpr int kStatW = 40;
+constexpr int kSumM = 30, kSumMM = 33, kSumR = 36, kSumRR = 37;
 
 struct Globals {
   float gnorm;  // ||all grads||_2

@@ -18,6 +18,7 @@
 
 #include "k_celo2.h"
 #include "k_gradstats.h"
+#include "k_velo.h"
 #include "pylo_common.h"
 
 // =============================================================================================
@@ -41,6 +42,7 @@ int fail(const std::string& m) {
   } while (0)
 
 size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a * a; }
+long long round4(long long x) { return (x + 3) / 4 * 4; }
 
 // (dc, dr): index of the 2nd-largest and largest dim, ties keep index order
 // (pylo/optim/CELO2_naive.py:42-47); VeLO swaps an equal pair except 4-D (0,1)
@@ -59,94 +61,115 @@ bool factored_dims(int kind, const PyloTensorShape& s, int* dc, int* dr) {
 
 struct Layout {
   std::vector<TDesc> descs;
-  std::vector<Item> p0_items, el_items, v0a_items, v0b_items;
+  std::vector<Item> p0_items, nd_items, el_items, v0a_items, v0b_items;
   std::vector<int> fac_list;
   std::vector<int> dc, dr;
   int H = 8;  // width of the first MLP layer (terms per row / column)
-  size_t off_descs, off_dyn, off_p0_items, off_el_items, off_v0a_items, off_v0b_items, off_fac_list,
-      off_rowpart, off_colpart, off_gsq, off_flag, off_globals, off_fac0, off_fac1, off_term0, off_term1,
-      off_v0part, off_bscale, off_stats, off_wfold, off_chan_ms, total;
+  int Tpad = 0;
+  size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_el_items, off_v0a_items, off_v0b_items, off_fac_list,
+      off_part, off_gsq, off_flag, off_globals, off_fac, off_term, off_v0part, off_bscale, off_stats, off_wfold,
+      off_chan_ms, off_totals, off_xfeat, off_lossfeat, off_xT, off_canon, total;
 };
 
-int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L) {
-  if (kind != PYLO_KIND_CELO2) return fail("plan: only PYLO_KIND_CELO2 is implemented");
+int first_layer_width(int kind) { return kind == PYLO_KIND_CELO2 ? 8 : kind == PYLO_KIND_VELO ? 4 : 32; }
+
+int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int velo_hidden) {
+  if (kind != PYLO_KIND_CELO2 && kind != PYLO_KIND_VELO) return fail("plan: this optimizer kind is not implemented");
   if (T <= 0 || shapes == nullptr) return fail("plan: no tensors");
+  L.H = first_layer_width(kind);
   L.descs.assign(T, TDesc{});
   L.dc.assign(T, -1);
   L.dr.assign(T, -1);
-  long long rowpart = 0, colpart = 0, fac0 = 0, fac1 = 0, term0 = 0, term1 = 0;
+  long long part = 0, fac = 0, term = 0;
   const int H = L.H;
   for (int t = 0; t < T; ++t) {
     const PyloTensorShape& s = shapes[t];
     if (s.ndim < 0 || s.ndim > PYLO_MAX_DIMS) return fail("plan: bad ndim");
     long long n = 1;
+    int rank = 0;
     for (int i = 0; i < s.ndim; ++i) {
       if (s.shape[i] < 0) return fail("plan: negative dim");
       n *= s.shape[i];
+      rank += s.shape[i] > 1;
     }
     if (n >= (1ll << 31)) return fail("plan: tensors of 2^31 or more elements are not supported");
     TDesc& d = L.descs[t];
     d.n = n;
     d.fac_slot = -1;
-    const bool adam = (s.flags & PYLO_F_ADAM) != 0 || s.ndim < 2;
-    if (kind == PYLO_KIND_CELO2 && s.ndim < 2 && !(s.flags & PYLO_F_ADAM))
-      return fail("plan: CELO2 tensors with fewer than 2 dims must carry PYLO_F_ADAM");
-    if (adam) {
-      d.mode = kModeFlat;
+    d.rank = rank < 4 ? rank : 4;
+    int dc = -1, dr = -1;
+    const bool can_factor = factored_dims(kind, s, &dc, &dr);
+    if (kind == PYLO_KIND_CELO2) {
+      const bool adam = (s.flags & PYLO_F_ADAM) != 0;
+      if (!can_factor && !adam) return fail("plan: CELO2 tensors with fewer than 2 dims must carry PYLO_F_ADAM");
+      if (adam) d.mode = kModeFlat;
+      else if (s.ndim == 2) d.mode = kModeFac2D;
+      else return fail("plan: CELO2 tensors with more than 2 dims are not supported yet");
+    } else {
+      d.mode = !can_factor ? kModeVec : (s.ndim == 2 ? kModeFac2D : kModeFacND);
+    }
+    if (d.mode == kModeFlat || d.mode == kModeVec) {
       d.vec = (n % 4 == 0) ? 4 : 1;
     } else {
-      if (s.ndim != 2) return fail("plan: CELO2 tensors with more than 2 dims are not supported yet");
-      int dc, dr;
-      factored_dims(kind, s, &dc, &dr);
       L.dc[t] = dc;
       L.dr[t] = dr;
-      d.mode = kModeFac2D;
-      d.R0 = (int)s.shape[0];
-      d.C0 = (int)s.shape[1];
-      d.vec = (d.C0 % 4 == 0) ? 4 : 1;
-      d.r_is_dim0 = (dr == 1) ? 1 : 0;
-      d.len_r = d.r_is_dim0 ? d.R0 : d.C0;
-      d.len_c = d.r_is_dim0 ? d.C0 : d.R0;
-      d.n_strips = (d.R0 + kP0Rows - 1) / kP0Rows;
-      d.n_colblk = (d.C0 + 64 * d.vec - 1) / (64 * d.vec);
-      d.rowpart_off = rowpart;
-      d.colpart_off = colpart;
-      rowpart += (long long)d.n_colblk * d.R0;
-      colpart += (long long)d.n_strips * d.C0;
-      d.C0r = (d.C0 + 3) / 4 * 4;
-      d.fac0_off = fac0;
-      d.fac1_off = fac1;
-      d.term0_off = term0;
-      d.term1_off = term1;
-      fac0 += (long long)d.R0 * 4;
-      fac1 += 3ll * d.C0r;
-      term0 += (long long)d.R0 * H;
-      term1 += (long long)H * d.C0r;
-      d.fac_slot = -1;
+      if (d.mode == kModeFac2D) {
+        d.R0 = (int)s.shape[0];
+        d.C0 = (int)s.shape[1];
+        d.vec = (d.C0 % 4 == 0) ? 4 : 1;
+        d.vec0_is_r = (dr == 1) ? 1 : 0;  // vector 0 (indexed by dim 0) results from summing over dim 1
+        d.len[0] = d.R0; d.len[1] = d.C0;
+        d.sumlen[0] = d.C0; d.sumlen[1] = d.R0;
+        d.n_strips = (d.R0 + kP0Rows - 1) / kP0Rows;
+        d.n_colblk = (d.C0 + 64 * d.vec - 1) / (64 * d.vec);
+        d.npart[0] = d.n_colblk; d.npart[1] = d.n_strips;
+      } else {
+        d.vec = 1;
+        d.vec0_is_r = 1;
+        const int rem[2] = {dr, dc};  // the dim each vector lost
+        for (int w = 0; w < 2; ++w) {
+          long long stride = 1;
+          for (int i = rem[w] + 1; i < s.ndim; ++i) stride *= s.shape[i];
+          d.nd_size[w] = (int)s.shape[rem[w]];
+          d.nd_stride[w] = (int)stride;
+          d.len[w] = d.nd_size[w] > 0 ? (int)(n / d.nd_size[w]) : 0;
+          d.sumlen[w] = d.nd_size[w];
+          d.npart[w] = 1;
+        }
+      }
+      for (int w = 0; w < 2; ++w) {
+        d.pitch[w] = (int)round4(d.len[w]);
+        d.part_off[w] = part;
+        part += round4((long long)d.npart[w] * d.len[w]);
+        const bool aos = d.mode == kModeFac2D && w == 0;
+        d.fac_off[w] = fac;
+        fac += aos ? (long long)d.len[w] * 4 : 3ll * d.pitch[w];
+        d.term_off[w] = term;
+        term += aos ? round4((long long)d.len[w] * H) : (long long)H * d.pitch[w];
+      }
       if (n > 0) {
         d.fac_slot = (int)L.fac_list.size();
         L.fac_list.push_back(t);
-        for (int which = 0; which < 2; ++which) {
-          const int len = which ? d.C0 : d.R0;
-          d.v0a_first[which] = (int)L.v0a_items.size();
-          for (int c = 0; c * kV0aEnt < len; ++c) L.v0a_items.push_back(Item{t, c, which, 0});
-          d.v0a_n[which] = (int)L.v0a_items.size() - d.v0a_first[which];
-          for (int c = 0; c * kV0bEnt < len; ++c) L.v0b_items.push_back(Item{t, c, which, 0});
+        for (int w = 0; w < 2; ++w) {
+          d.v0a_first[w] = (int)L.v0a_items.size();
+          for (int c = 0; c * kV0aEnt < d.len[w]; ++c) L.v0a_items.push_back(Item{t, c, w, 0});
+          d.v0a_n[w] = (int)L.v0a_items.size() - d.v0a_first[w];
+          for (int c = 0; c * kV0bEnt < d.len[w]; ++c) L.v0b_items.push_back(Item{t, c, w, 0});
+          if (d.mode == kModeFacND)
+            for (int c = 0; c * kThreads < d.len[w]; ++c) L.nd_items.push_back(Item{t, c, w, 0});
         }
       }
     }
-    // P0 items
+    const long long chunk = (long long)kThreads * d.vec * kElemIters;
+    // P0 items: tiles of 2-D factored tensors; flat chunks only where a global norm is needed (CELO2)
     if (n > 0) {
       if (d.mode == kModeFac2D) {
         for (int st = 0; st < d.n_strips; ++st)
           for (int cb = 0; cb < d.n_colblk; ++cb) L.p0_items.push_back(Item{t, st, cb, 0});
-      } else {
-        const long long chunk = (long long)kThreads * d.vec * kElemIters;
+      } else if (d.mode == kModeFlat) {
         for (long long c = 0; c * chunk < n; ++c) L.p0_items.push_back(Item{t, (int)c, 0, 0});
       }
     }
-    // element items
-    const long long chunk = (long long)kThreads * d.vec * kElemIters;
     d.blk0 = (int)L.el_items.size();
     for (long long c = 0; c * chunk < n; ++c) L.el_items.push_back(Item{t, (int)c, 0, 0});
     d.nblk = (int)L.el_items.size() - d.blk0;
@@ -154,36 +177,41 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L) {
   size_t off = 0;
   auto take = [&](size_t bytes) {
     size_t o = off;
-    off = align_up(off + bytes);
+    off = align_up(off + std::max<size_t>(bytes, 16));
     return o;
   };
   const size_t nfac = std::max<size_t>(L.fac_list.size(), 1);
   L.off_descs = take(sizeof(TDesc) * T);
   L.off_dyn = take(sizeof(PyloTensorArgs) * T);
-  L.off_p0_items = take(sizeof(Item) * std::max<size_t>(L.p0_items.size(), 1));
-  L.off_el_items = take(sizeof(Item) * std::max<size_t>(L.el_items.size(), 1));
-  L.off_v0a_items = take(sizeof(Item) * std::max<size_t>(L.v0a_items.size(), 1));
-  L.off_v0b_items = take(sizeof(Item) * std::max<size_t>(L.v0b_items.size(), 1));
+  L.off_p0_items = take(sizeof(Item) * L.p0_items.size());
+  L.off_nd_items = take(sizeof(Item) * L.nd_items.size());
+  L.off_el_items = take(sizeof(Item) * L.el_items.size());
+  L.off_v0a_items = take(sizeof(Item) * L.v0a_items.size());
+  L.off_v0b_items = take(sizeof(Item) * L.v0b_items.size());
   L.off_fac_list = take(sizeof(int) * nfac);
-  L.off_rowpart = take(sizeof(float) * std::max<long long>(rowpart, 1));
-  L.off_colpart = take(sizeof(float) * std::max<long long>(colpart, 1));
-  L.off_gsq = take(sizeof(double) * std::max<size_t>(L.p0_items.size(), 1));
-  L.off_flag = take(sizeof(int) * std::max<size_t>(L.p0_items.size(), 1));
+  L.off_part = take(sizeof(float) * part);
+  L.off_gsq = take(sizeof(double) * L.p0_items.size());
+  L.off_flag = take(sizeof(int) * L.p0_items.size());
   L.off_globals = take(sizeof(Globals));
-  L.off_fac0 = take(sizeof(float) * std::max<long long>(fac0, 4));
-  L.off_fac1 = take(sizeof(float) * std::max<long long>(fac1, 4));
-  L.off_term0 = take(sizeof(float) * std::max<long long>(term0, 4));
-  L.off_term1 = take(sizeof(float) * std::max<long long>(term1, 4));
-  L.off_v0part = take(sizeof(double) * kNV0 * std::max<size_t>(L.v0a_items.size(), 1));
+  L.off_fac = take(sizeof(float) * fac);
+  L.off_term = take(sizeof(float) * term);
+  L.off_v0part = take(sizeof(double) * kNV0 * L.v0a_items.size());
   L.off_bscale = take(sizeof(BScale) * nfac);
-  L.off_stats = take(sizeof(double) * kNStat * std::max<size_t>(L.el_items.size(), 1));
-  L.off_wfold = take(sizeof(float) * kC2Fold * nfac);
+  L.off_stats = take(sizeof(double) * kStatW * L.el_items.size());
+  L.off_wfold = take(sizeof(float) * (kind == PYLO_KIND_CELO2 ? kC2Fold * nfac : (size_t)kVFold * T));
   L.off_chan_ms = take(sizeof(float) * kNStat * nfac);
+  L.off_totals = take(sizeof(double) * kStatW * T);
+  L.Tpad = (T + kGateBT - 1) / kGateBT * kGateBT;
+  L.off_xfeat = take(sizeof(float) * kXW * T);
+  L.off_lossfeat = take(sizeof(float) * 16);
+  L.off_xT = take(kind == PYLO_KIND_VELO ? sizeof(float) * 2 * (size_t)velo_hidden * L.Tpad : 0);
+  L.off_canon = take(kind == PYLO_KIND_VELO ? sizeof(float) * kVCanon * (size_t)T : 0);
   L.total = off;
   return 0;
 }
 
 constexpr int kStageSlots = 4;
+constexpr int kVeloHiddenMax = 1024;  // workspace is sized for LSTM widths up to this
 
 }  // namespace
 
@@ -215,7 +243,7 @@ const char* pylo_mi355_last_error(void) { return g_err.c_str(); }
 int pylo_mi355_plan_workspace_bytes(int kind, const PyloTensorShape* shapes, int n_tensors, size_t* bytes_out) {
   if (!bytes_out) return fail("workspace_bytes: null output");
   Layout L;
-  if (int rc = build_layout(kind, shapes, n_tensors, L)) return rc;
+  if (int rc = build_layout(kind, shapes, n_tensors, L, kVeloHiddenMax)) return rc;
   *bytes_out = L.total;
   return 0;
 }
@@ -227,7 +255,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   PyloPlan* P = new PyloPlan();
   P->kind = kind;
   P->T = n_tensors;
-  if (int rc = build_layout(kind, shapes, n_tensors, P->L)) { delete P; return rc; }
+  if (int rc = build_layout(kind, shapes, n_tensors, P->L, kVeloHiddenMax)) { delete P; return rc; }
   if (workspace == nullptr || workspace_bytes < P->L.total) { delete P; return fail("plan_create: workspace too small"); }
   if (reinterpret_cast<uintptr_t>(workspace) % 256 != 0) { delete P; return fail("plan_create: workspace must be 256-byte aligned"); }
   P->ws = static_cast<char*>(workspace);
@@ -240,6 +268,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   hipError_t e = hipSuccess;
   if (e == hipSuccess) e = up(L.off_descs, L.descs.data(), sizeof(TDesc) * L.descs.size());
   if (e == hipSuccess) e = up(L.off_p0_items, L.p0_items.data(), sizeof(Item) * L.p0_items.size());
+  if (e == hipSuccess) e = up(L.off_nd_items, L.nd_items.data(), sizeof(Item) * L.nd_items.size());
   if (e == hipSuccess) e = up(L.off_el_items, L.el_items.data(), sizeof(Item) * L.el_items.size());
   if (e == hipSuccess) e = up(L.off_fac_list, L.fac_list.data(), sizeof(int) * L.fac_list.size());
   if (e == hipSuccess) e = up(L.off_v0a_items, L.v0a_items.data(), sizeof(Item) * L.v0a_items.size());
@@ -266,6 +295,22 @@ int pylo_mi355_plan_destroy(PyloPlan* P) {
   }
   delete P;
   return 0;
+}
+
+static const char* kCelo2Launches[] = {"k_p0(sums)", "k_gnorm", "k_p0(exact)", "k_v0a", "k_v0b",
+                                       "k_celo2_stats", "k_celo2_fold", "k_celo2_apply"};
+static const char* kVeloLaunches[] = {"k_p0(sums)", "k_p0_nd", "k_v0a", "k_v0b", "k_velo_stats", "k_velo_loss",
+                                      "k_lo_reduce", "k_velo_mix", "k_velo_gates", "k_velo_heads", "k_terms",
+                                      "k_velo_apply"};
+
+int pylo_mi355_plan_num_launches(const PyloPlan* P) {
+  if (!P) return -1;
+  return P->kind == PYLO_KIND_CELO2 ? 8 : P->kind == PYLO_KIND_VELO ? 12 : -1;
+}
+
+const char* pylo_mi355_plan_launch_name(const PyloPlan* P, int launch) {
+  if (!P || launch < 0 || launch >= pylo_mi355_plan_num_launches(P)) return "";
+  return P->kind == PYLO_KIND_CELO2 ? kCelo2Launches[launch] : kVeloLaunches[launch];
 }
 
 int pylo_mi355_plan_timing_begin(PyloPlan* P, int max_steps) {
@@ -298,18 +343,6 @@ int pylo_mi355_plan_timing_end(PyloPlan* P, float* ms_out, int capacity, int* st
   return 0;
 }
 
-int pylo_mi355_plan_num_launches(const PyloPlan* P) {
-  if (!P) return -1;
-  return P->kind == PYLO_KIND_CELO2 ? 8 : -1;
-}
-
-const char* pylo_mi355_plan_launch_name(const PyloPlan* P, int launch) {
-  static const char* celo2[] = {"k_p0(sums)", "k_gnorm", "k_p0(exact)", "k_v0a", "k_v0b",
-                                "k_celo2_stats", "k_celo2_fold", "k_celo2_apply"};
-  if (!P || launch < 0 || launch >= pylo_mi355_plan_num_launches(P)) return "";
-  return celo2[launch];
-}
-
 int pylo_mi355_plan_factored_dims(const PyloPlan* P, int tensor, int* dc, int* dr) {
   if (!P || tensor < 0 || tensor >= P->T || !dc || !dr) return fail("factored_dims: bad argument");
   *dc = P->L.dc[tensor];
@@ -338,22 +371,43 @@ int upload_args(PyloPlan* P, const PyloTensorArgs* args, hipStream_t s) {
   return 0;
 }
 
-int check_args(const PyloPlan* P, const PyloTensorArgs* args) {
+int check_args(const PyloPlan* P, const PyloTensorArgs* args, bool need_all_grads) {
   for (int t = 0; t < P->T; ++t) {
     const TDesc& d = P->L.descs[t];
     const PyloTensorArgs& a = args[t];
-    if (a.grad == nullptr || d.n == 0) continue;
-    if (!a.param || !a.mom || !a.rms) return fail("step: null param/mom/rms pointer at tensor " + std::to_string(t));
-    if (d.mode == kModeFac2D && (!a.fac_r || !a.fac_c || !a.step_out))
-      return fail("step: null fac_r/fac_c/step_out pointer at tensor " + std::to_string(t));
+    const std::string at = " at tensor " + std::to_string(t);
+    if (a.grad == nullptr) {
+      if (need_all_grads) return fail("step: every tensor needs a gradient" + at);
+      continue;
+    }
+    if (d.n == 0) continue;
+    if (!a.param || !a.mom || !a.rms) return fail("step: null param/mom/rms pointer" + at);
+    const bool factored = d.mode == kModeFac2D || d.mode == kModeFacND;
+    if (factored && (!a.fac_r || !a.fac_c)) return fail("step: null fac_r/fac_c pointer" + at);
+    if (factored && P->kind == PYLO_KIND_CELO2 && !a.step_out) return fail("step: null step_out pointer" + at);
+    if (d.mode == kModeVec && !a.fac_v) return fail("step: null fac_v pointer" + at);
+    if (a.group < 0 || a.group >= PYLO_MAX_GROUPS) return fail("step: group index out of range" + at);
     const uintptr_t m = reinterpret_cast<uintptr_t>(a.grad) | reinterpret_cast<uintptr_t>(a.param) |
                         reinterpret_cast<uintptr_t>(a.mom) | reinterpret_cast<uintptr_t>(a.rms) |
                         reinterpret_cast<uintptr_t>(a.fac_r) | reinterpret_cast<uintptr_t>(a.fac_c) |
-                        reinterpret_cast<uintptr_t>(a.step_out);
-    if (m % 16 != 0) return fail("step: pointers must be 16-byte aligned (tensor " + std::to_string(t) + ")");
+                        reinterpret_cast<uintptr_t>(a.fac_v) | reinterpret_cast<uintptr_t>(a.step_out);
+    if (m % (d.vec == 4 ? 16 : 4) != 0) return fail("step: misaligned pointer (16 bytes needed)" + at);
   }
   return 0;
 }
+
+struct Marks {  // per-launch HIP events when timing is on
+  PyloPlan* P;
+  hipStream_t s;
+  hipEvent_t* ev;
+  int mark = 0;
+  Marks(PyloPlan* P_, hipStream_t s_) : P(P_), s(s_) {
+    const bool timed = P->timing && P->t_steps < P->t_steps_max;
+    ev = timed ? &P->tev[(size_t)P->t_steps * P->t_per_step] : nullptr;
+  }
+  hipError_t operator()() { return ev ? hipEventRecord(ev[mark++], s) : hipSuccess; }
+  void done() { if (ev) P->t_steps++; }
+};
 
 }  // namespace
 
@@ -361,7 +415,7 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
                                      const float* mlp, void* stream) {
   if (!P || !args || !decays || !mlp) return fail("celo2_step: null argument");
   if (P->kind != PYLO_KIND_CELO2) return fail("celo2_step: plan is not a CELO2 plan");
-  if (int rc = check_args(P, args)) return rc;
+  if (int rc = check_args(P, args, false)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (int rc = upload_args(P, args, s)) return rc;
   const Layout& L = P->L;
@@ -369,55 +423,133 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   const PyloTensorArgs* dyn = P->at<PyloTensorArgs>(L.off_dyn);
   const Item* p0_items = P->at<Item>(L.off_p0_items);
   const Item* el_items = P->at<Item>(L.off_el_items);
+  const Item* v0a_items = P->at<Item>(L.off_v0a_items);
+  const Item* v0b_items = P->at<Item>(L.off_v0b_items);
   const int* fac_list = P->at<int>(L.off_fac_list);
-  float* rowpart = P->at<float>(L.off_rowpart);
-  float* colpart = P->at<float>(L.off_colpart);
+  float* part = P->at<float>(L.off_part);
   double* gsq = P->at<double>(L.off_gsq);
   int* flag = P->at<int>(L.off_flag);
   Globals* gl = P->at<Globals>(L.off_globals);
-  const Item* v0a_items = P->at<Item>(L.off_v0a_items);
-  const Item* v0b_items = P->at<Item>(L.off_v0b_items);
-  float* fac0 = P->at<float>(L.off_fac0);
-  float* fac1 = P->at<float>(L.off_fac1);
-  float* term0 = P->at<float>(L.off_term0);
-  float* term1 = P->at<float>(L.off_term1);
+  float* fac_tab = P->at<float>(L.off_fac);
+  float* term_tab = P->at<float>(L.off_term);
   double* v0part = P->at<double>(L.off_v0part);
   BScale* bscale = P->at<BScale>(L.off_bscale);
-  const int n_v0a = (int)L.v0a_items.size(), n_v0b = (int)L.v0b_items.size();
   double* stats = P->at<double>(L.off_stats);
   float* wfold = P->at<float>(L.off_wfold);
   float* chan_ms = P->at<float>(L.off_chan_ms);
   const int n_p0 = (int)L.p0_items.size(), n_el = (int)L.el_items.size(), n_fac = (int)L.fac_list.size();
+  const int n_v0a = (int)L.v0a_items.size(), n_v0b = (int)L.v0b_items.size();
   const PyloDecays dec = *decays;
+  Marks mark(P, s);
 
-  const bool timed = P->timing && P->t_steps < P->t_steps_max;
-  hipEvent_t* ev = timed ? &P->tev[(size_t)P->t_steps * P->t_per_step] : nullptr;
-  int mark = 0;
-#define PYLO_MARK() do { if (timed) HIP_TRY(hipEventRecord(ev[mark++], s)); } while (0)
-  PYLO_MARK();
-  if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, rowpart, colpart, gsq, flag, gl, 0);
-  PYLO_MARK();
+  HIP_TRY(mark());
+  if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0);
+  HIP_TRY(mark());
   hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl);
-  PYLO_MARK();
-  if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, rowpart, colpart, gsq, flag, gl, 1);
-  PYLO_MARK();
+  HIP_TRY(mark());
+  if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1);
+  HIP_TRY(mark());
   if (n_v0a > 0)
-    hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kThreads), 0, s, descs, dyn, v0a_items, rowpart, colpart, gl, dec, v0part);
-  PYLO_MARK();
+    hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
+  HIP_TRY(mark());
   if (n_v0b > 0)
     hipLaunchKernelGGL(k_v0b<8>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-9f, mlp,
-                       mlp + 240, fac0, fac1, term0, term1, bscale);
-  PYLO_MARK();
-  if (n_el > 0) hipLaunchKernelGGL(k_celo2_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac0, fac1, gl, dec, stats);
-  PYLO_MARK();
+                       mlp + 240, fac_tab, term_tab, bscale);
+  HIP_TRY(mark());
+  if (n_el > 0) hipLaunchKernelGGL(k_celo2_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, gl, dec, stats);
+  HIP_TRY(mark());
   if (n_fac > 0) hipLaunchKernelGGL(k_celo2_fold, dim3(n_fac), dim3(kFoldThreads), 0, s, descs, dyn, fac_list, stats, mlp, wfold, chan_ms);
-  PYLO_MARK();
+  HIP_TRY(mark());
   if (n_el > 0)
-    hipLaunchKernelGGL(k_celo2_apply, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac0, fac1, term0, term1,
-                       gl, dec, wfold);
-  PYLO_MARK();
-#undef PYLO_MARK
-  if (timed) P->t_steps++;
+    hipLaunchKernelGGL(k_celo2_apply, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, term_tab, gl, dec, wfold);
+  HIP_TRY(mark());
+  mark.done();
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, const PyloDecays* decays,
+                                    const PyloVeloNets* nets, const PyloVeloStep* step, void* stream) {
+  if (!P || !args || !decays || !nets || !step) return fail("velo_step: null argument");
+  if (P->kind != PYLO_KIND_VELO) return fail("velo_step: plan is not a VeLO plan");
+  const int H = nets->hidden, K = nets->n_bank, T = P->T;
+  if (H <= 0 || H % 64 != 0 || H > kVeloHiddenMax) return fail("velo_step: LSTM width must be a multiple of 64, at most 1024");
+  if (K <= 0 || K > 4096) return fail("velo_step: bank size out of range");
+  if (!nets->mix2_wt || !nets->mix2_b || !nets->fmix_wt || !nets->fmix_b || !nets->lstm_wt || !nets->lstm_b ||
+      !nets->ctrl_wt || !nets->ctrl_b || !nets->lr_w || !nets->lr_b || !nets->bank)
+    return fail("velo_step: null weight pointer");
+  if (!step->lstm_h || !step->lstm_c || !step->loss_means || !step->loss_running_min || !step->loss_decays ||
+      !step->loss_iteration || !step->loss)
+    return fail("velo_step: null state pointer");
+  if (int rc = check_args(P, args, true)) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (int rc = upload_args(P, args, s)) return rc;
+  const Layout& L = P->L;
+  const TDesc* descs = P->at<TDesc>(L.off_descs);
+  const PyloTensorArgs* dyn = P->at<PyloTensorArgs>(L.off_dyn);
+  const Item* p0_items = P->at<Item>(L.off_p0_items);
+  const Item* nd_items = P->at<Item>(L.off_nd_items);
+  const Item* el_items = P->at<Item>(L.off_el_items);
+  const Item* v0a_items = P->at<Item>(L.off_v0a_items);
+  const Item* v0b_items = P->at<Item>(L.off_v0b_items);
+  float* part = P->at<float>(L.off_part);
+  double* gsq = P->at<double>(L.off_gsq);
+  int* flag = P->at<int>(L.off_flag);
+  Globals* gl = P->at<Globals>(L.off_globals);
+  float* fac_tab = P->at<float>(L.off_fac);
+  float* term_tab = P->at<float>(L.off_term);
+  double* v0part = P->at<double>(L.off_v0part);
+  BScale* bscale = P->at<BScale>(L.off_bscale);
+  double* stats = P->at<double>(L.off_stats);
+  float* wfold = P->at<float>(L.off_wfold);
+  double* totals = P->at<double>(L.off_totals);
+  float* xfeat = P->at<float>(L.off_xfeat);
+  float* lossfeat = P->at<float>(L.off_lossfeat);
+  float* xT = P->at<float>(L.off_xT);
+  float* canon = P->at<float>(L.off_canon);
+  const int n_p0 = (int)L.p0_items.size(), n_nd = (int)L.nd_items.size(), n_el = (int)L.el_items.size();
+  const int n_v0a = (int)L.v0a_items.size(), n_v0b = (int)L.v0b_items.size();
+  const PyloDecays dec = *decays;
+  VeloStep vs;
+  std::memcpy(vs.frac, step->frac, sizeof(vs.frac));
+  Marks mark(P, s);
+
+  HIP_TRY(mark());
+  // clip_norm is 0 for VeLO tensors: k_p0 clamps directly; its norm / flag outputs are not used
+  if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0);
+  HIP_TRY(mark());
+  if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part);
+  HIP_TRY(mark());
+  if (n_v0a > 0)
+    hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
+  HIP_TRY(mark());
+  if (n_v0b > 0)
+    hipLaunchKernelGGL(k_v0b<4>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-5f,
+                       (const float*)nullptr, (const float*)nullptr, fac_tab, term_tab, bscale);
+  HIP_TRY(mark());
+  if (n_el > 0) hipLaunchKernelGGL(k_velo_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, dec, stats);
+  HIP_TRY(mark());
+  hipLaunchKernelGGL(k_velo_loss, dim3(1), dim3(64), 0, s, step->loss_means, step->loss_running_min, step->loss_decays,
+                     step->loss_iteration, step->loss, lossfeat);
+  HIP_TRY(mark());
+  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kThreads), 0, s, descs, dyn, T, stats, totals, lossfeat, vs, xfeat);
+  HIP_TRY(mark());
+  hipLaunchKernelGGL(k_velo_mix, dim3(H / 64), dim3(kThreads), 0, s, xfeat, T, L.Tpad, H, nets->mix2_wt, nets->mix2_b,
+                     nets->fmix_wt, nets->fmix_b, step->lstm_h, xT);
+  HIP_TRY(mark());
+  hipLaunchKernelGGL(k_velo_gates, dim3(L.Tpad / kGateBT, (H + 127) / 128), dim3(128), 0, s, xT, T, L.Tpad, H,
+                     nets->lstm_wt, nets->lstm_b, step->lstm_h, step->lstm_c);
+  HIP_TRY(mark());
+  hipLaunchKernelGGL(k_velo_heads, dim3(T), dim3(kThreads), sizeof(float) * (H + K + 160 + 32 + 4), s, descs, T, H, K,
+                     step->lstm_h, nets->ctrl_wt, nets->ctrl_b, nets->lr_w, nets->lr_b, nets->bank, totals, canon, wfold,
+                     step->controls_out, step->lr_mult_out);
+  HIP_TRY(mark());
+  if (n_v0b > 0)
+    hipLaunchKernelGGL(k_terms<4>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, bscale, canon, kVCanon, term_tab);
+  HIP_TRY(mark());
+  if (n_el > 0) hipLaunchKernelGGL(k_velo_apply, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, term_tab, dec, wfold);
+  HIP_TRY(mark());
+  mark.done();
   HIP_TRY(hipGetLastError());
   return 0;
 }

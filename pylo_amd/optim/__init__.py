@@ -1,7 +1,9 @@
 """Fused learned-optimizer classes (same public names as ``pylo.optim``)."""
 
 from .ELO_CELO2_cuda import ELO_CELO2_CUDA
+from .velo_cuda import VeLO_CUDA
 
 ELO_CELO2 = ELO_CELO2_CUDA
+VeLO = VeLO_CUDA
 
-__all__ = ["ELO_CELO2_CUDA", "ELO_CELO2"]
+__all__ = ["ELO_CELO2_CUDA", "ELO_CELO2", "VeLO_CUDA", "VeLO"]

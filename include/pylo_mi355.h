@@ -172,6 +172,21 @@ typedef struct {
 int pylo_mi355_velo_step(PyloPlan* plan, const PyloTensorArgs* args, const PyloDecays* decays,
                          const PyloVeloNets* nets, const PyloVeloStep* step, void* stream);
 
+/*
+ * AdafacLO step (replaces cuda_lo.learned_optimizer_kernel, pylo/csrc/learned_optimizer.cu:303-394, for
+ * every tensor at once, plus the accumulator updates of AdafacLO_cuda.py:291-373 and the weight decay
+ * of :406-407).  `net` is a device pointer to 2466 floats, every matrix stored (in, out):
+ *   w1 (30,32): first-layer rows for the 30-channel feature order g, clip(g), p, m0..2, rms, m_k*rs,
+ *               rs, g*rf_k*cf_k, g*rs, fac_r_k, fac_c_k, rsqrt(fac_r_k), rsqrt(fac_c_k), m_k*rf_k*cf_k
+ *               (AdafacLO has no clip(g) / g*rs channel: rows 1 and 14 are zero);
+ *   b1 32 | w_time (11,32): rows of the 11 tanh time features | w_h (32,32) | b_h 32 | w_o (32,2) | b_o 2
+ * (pylo_amd.models.pack_metamlp builds it from a MetaMLP).  `step` is the 0-based step counter fed to
+ * the time features (AdafacLO_cuda.py:400).  Tensors without gradient are skipped.
+ *   p -= lr * o0 * exp(o1 * exp_mult) * step_mult;  then p -= weight_decay * lr * p.
+ */
+int pylo_mi355_adafac_step(PyloPlan* plan, const PyloTensorArgs* args, const PyloDecays* decays,
+                           const float* net, float step, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

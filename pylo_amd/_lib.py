@@ -81,6 +81,8 @@ def load():
                                           C.c_void_p]
     lib.pylo_mi355_velo_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.POINTER(VeloNets),
                                          C.POINTER(VeloStep), C.c_void_p]
+    lib.pylo_mi355_adafac_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.c_void_p, C.c_float,
+                                           C.c_void_p]
     if lib.pylo_mi355_abi_version() != 1:
         raise RuntimeError("libpylo_mi355.so: ABI version mismatch, rebuild it")
     _lib = lib
@@ -167,6 +169,10 @@ class Plan:
     def velo_step(self, decays: Decays, nets: VeloNets, step: VeloStep, stream: int) -> None:
         check(load().pylo_mi355_velo_step(self._h, self.args.ctypes.data, C.byref(decays), C.byref(nets),
                                           C.byref(step), stream), "velo_step")
+
+    def adafac_step(self, decays: Decays, net: torch.Tensor, step: float, stream: int) -> None:
+        check(load().pylo_mi355_adafac_step(self._h, self.args.ctypes.data, C.byref(decays), net.data_ptr(),
+                                            float(step), stream), "adafac_step")
 
     def close(self):
         if getattr(self, "_h", None):

@@ -1,0 +1,267 @@
+// AdafacLO (small_fc_lopt): element kernels.  28 normalised features + 11 time features,
+// 39 -> 32 -> 32 -> 2 MLP, parameter updated in place (pylo/optim/AdafacLO_naive.py:187-311).
+//
+// The 28 features are the VeLO channel set without clip(g) and g*rsqrt(rms); they are kept in the
+// same 30-channel numbering so the statistics machinery is shared.  The 11 time features are the
+// same for every element of a step and are folded into the first-layer bias.
+#pragma once
+
+#include "k_velo.h"
+
+namespace pylo {
+
+// Host-packed network (floats), all (in, out):
+//   w1 (30,32) rows in the 30-channel order (rows 1 and 14 zero) | b1 32 | w_time (11,32) |
+//   w_h (32,32) | b_h 32 | w_o (32,2) | b_o 2
+constexpr int kAH = 32;
+constexpr int kAW1 = 0, kAB1 = 960, kAWT = 992, kAWH = 1344, kABH = 2368, kAWO = 2400, kABO = 2464, kANet = 2466;
+constexpr int kAFold = 960;  // per-tensor first-layer rows scaled by the channel normalisers
+
+__host__ __device__ constexpr bool adafac_channel(int c) { return c != 1 && c != 14; }
+
+// b_eff = b1 + w_time^T tanh(step / ts - 1)   (AdafacLO_naive.py:81-87,226)
+__global__ __launch_bounds__(64) void k_adafac_bias(const float* __restrict__ net, float step,
+                                                    float* __restrict__ bias_eff) {
+  const float ts[11] = {1.f, 3.f, 10.f, 30.f, 100.f, 300.f, 1000.f, 3000.f, 10000.f, 30000.f, 100000.f};
+  const int j = threadIdx.x;
+  if (j >= kAH) return;
+  float acc = net[kAB1 + j];
+#pragma unroll
+  for (int q = 0; q < 11; ++q) acc = fmaf(tanhf(step / ts[q] - 1.0f), net[kAWT + q * kAH + j], acc);
+  bias_eff[j] = acc;
+}
+
+template <int V, bool ND>
+__device__ __forceinline__ void adafac_stats_fac(const TDesc& d, const PyloTensorArgs& a, int chunk,
+                                                 const EmaConsts& e, const float* __restrict__ fac_tab, VeloAcc& acc) {
+  const long long base = (long long)chunk * (kThreads * V * kElemIters);
+#pragma unroll 2
+  for (int it = 0; it < kElemIters; ++it) {
+    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
+    if (idx >= d.n) break;
+    ElemIn<V> x;
+    lo_load<V, ND>(d, a, idx, fac_tab, x);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      ema_update(e, x.g[v], x.m[v], x.rms[v]);
+      float f[kNStat];
+      lo_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.rfcf[v], 1e-6f, f);
+#pragma unroll
+      for (int c = 0; c < kNStat; ++c)
+        if (adafac_channel(stat_channel(c))) acc.ch[stat_channel(c)] = fmaf(f[c], f[c], acc.ch[stat_channel(c)]);
+    }
+  }
+}
+
+template <int V>
+__device__ __forceinline__ void adafac_stats_vec(const TDesc& d, const PyloTensorArgs& a, int chunk,
+                                                 const EmaConsts& e, const PyloDecays& dec, VeloAcc& acc) {
+  const long long base = (long long)chunk * (kThreads * V * kElemIters);
+  for (int it = 0; it < kElemIters; ++it) {
+    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
+    if (idx >= d.n) break;
+    VecIn<V> x;
+    vec_load<V>(d, a, idx, x);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      vec_update(e, dec, x.g[v], x.m[v], x.rms[v], x.v[v]);
+      float f[30];
+      vec_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.v[v], 1e-6f, f);
+#pragma unroll
+      for (int c = 0; c < 30; ++c)
+        if (adafac_channel(c)) acc.ch[c] = fmaf(f[c], f[c], acc.ch[c]);
+    }
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void k_adafac_stats(const TDesc* __restrict__ descs,
+                                                           const PyloTensorArgs* __restrict__ dyn,
+                                                           const Item* __restrict__ items,
+                                                           const float* __restrict__ fac_tab, PyloDecays dec,
+                                                           double* __restrict__ stats_part) {
+  __shared__ float red[kWaves][30];
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  const EmaConsts e = make_ema(dec);
+  VeloAcc acc;
+#pragma unroll
+  for (int c = 0; c < 30; ++c) acc.ch[c] = 0.0f;
+  if (d.mode == kModeFac2D) {
+    if (d.vec == 4) adafac_stats_fac<4, false>(d, a, it.a, e, fac_tab, acc);
+    else adafac_stats_fac<1, false>(d, a, it.a, e, fac_tab, acc);
+  } else if (d.mode == kModeFacND) {
+    adafac_stats_fac<1, true>(d, a, it.a, e, fac_tab, acc);
+  } else {
+    if (d.vec == 4) adafac_stats_vec<4>(d, a, it.a, e, dec, acc);
+    else adafac_stats_vec<1>(d, a, it.a, e, dec, acc);
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int c = 0; c < 30; ++c) {
+    const float s = wave_sum(acc.ch[c]);
+    if (lane == 0) red[wave][c] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x < kStatW) {
+    const int c = threadIdx.x;
+    stats_part[(size_t)blockIdx.x * kStatW + c] =
+        c < 30 ? ((double)red[0][c] + (double)red[1][c]) + ((double)red[2][c] + (double)red[3][c]) : 0.0;
+  }
+}
+
+// Per tensor: first-layer rows scaled by rsqrt(1e-5 + mean f_c^2) (AdafacLO_naive.py:90-92,301).
+__global__ __launch_bounds__(kThreads) void k_adafac_fold(const TDesc* __restrict__ descs,
+                                                          const PyloTensorArgs* __restrict__ dyn,
+                                                          const double* __restrict__ totals,
+                                                          const float* __restrict__ net, float* __restrict__ wfold) {
+  __shared__ float sc[32];
+  const int t = blockIdx.x;
+  const TDesc d = descs[t];
+  if (dyn[t].grad == nullptr) return;
+  if (threadIdx.x < 30) {
+    const double n = (double)(d.n > 0 ? d.n : 1);
+    sc[threadIdx.x] = rsq(1e-5f + (float)(totals[(size_t)t * kStatW + threadIdx.x] / n));
+  }
+  __syncthreads();
+  float* w = wfold + (size_t)t * kAFold;
+  for (int i = threadIdx.x; i < 30 * kAH; i += kThreads) w[i] = net[kAW1 + i] * sc[i / kAH];
+}
+
+// One element per lane: 16 (factored) or 28 (non-factored) scaled features -> 32 -> 32 -> 2.
+// Weights are wave-uniform and come through the scalar cache, one input row at a time.
+template <int NF>
+__device__ __forceinline__ float adafac_mlp(const float (&f)[NF], const int (&row)[NF], float (&h)[kAH],
+                                            const float* wfold_t, const float* net, const PyloTensorArgs& a,
+                                            float p) {
+  const cfloat* w1 = launder(wfold_t);
+  const cfloat* nw = launder(net);
+#pragma unroll
+  for (int c = 0; c < NF; ++c) {
+#pragma unroll
+    for (int j = 0; j < kAH; ++j) h[j] = fmaf(f[c], w1[row[c] * kAH + j], h[j]);
+  }
+  float h1[kAH];
+#pragma unroll
+  for (int j = 0; j < kAH; ++j) h1[j] = nw[kABH + j];
+#pragma unroll
+  for (int k = 0; k < kAH; ++k) {
+    const float hk = fmaxf(h[k], 0.0f);
+#pragma unroll
+    for (int j = 0; j < kAH; ++j) h1[j] = fmaf(hk, nw[kAWH + k * kAH + j], h1[j]);
+  }
+  float o0 = nw[kABO + 0], o1 = nw[kABO + 1];
+#pragma unroll
+  for (int k = 0; k < kAH; ++k) {
+    const float hk = fmaxf(h1[k], 0.0f);
+    o0 = fmaf(hk, nw[kAWO + k * 2 + 0], o0);
+    o1 = fmaf(hk, nw[kAWO + k * 2 + 1], o1);
+  }
+  const float step = (o0 * expf(o1 * a.exp_mult)) * a.step_mult;
+  p = fmaf(step, -a.lr, p);
+  if (a.weight_decay > 0.0f) p = fmaf(p, -(a.weight_decay * a.lr), p);
+  return p;
+}
+
+template <bool ND>
+__device__ __forceinline__ void adafac_apply_fac(const TDesc& d, const PyloTensorArgs& a, long long base,
+                                                 long long count, const EmaConsts& e,
+                                                 const float* __restrict__ fac_tab, const float* __restrict__ term_tab,
+                                                 const float* wfold_t, const float* net) {
+  const long long n = d.n;
+  for (long long off = threadIdx.x; off < count; off += kThreads) {
+    const long long idx = base + off;
+    if (idx >= n) break;
+    ElemIn<1> x;
+    if constexpr (ND) {
+      lo_load<1, true>(d, a, idx, fac_tab, x);
+    } else {  // 2-D, one element per lane
+      x.g[0] = clampf(*(const gfloat*)(a.grad + idx), a.clip_val);
+      x.p[0] = *(const gfloat*)(a.param + idx);
+      x.m[0][0] = *(const gfloat*)(a.mom + idx);
+      x.m[0][1] = *(const gfloat*)(a.mom + n + idx);
+      x.m[0][2] = *(const gfloat*)(a.mom + 2 * n + idx);
+      x.rms[0] = *(const gfloat*)(a.rms + idx);
+      const unsigned u = (unsigned)idx;
+      x.i0 = (int)(u / (unsigned)d.C0);
+      x.i1 = (int)(u - (unsigned)x.i0 * (unsigned)d.C0);
+      const float4 fa = load_f4(fac_tab + d.fac_off[0] + (size_t)x.i0 * 4);
+      x.rfcf[0][0] = fa.x * fac_tab[d.fac_off[1] + x.i1];
+      x.rfcf[0][1] = fa.y * fac_tab[d.fac_off[1] + (size_t)d.pitch[1] + x.i1];
+      x.rfcf[0][2] = fa.z * fac_tab[d.fac_off[1] + 2 * (size_t)d.pitch[1] + x.i1];
+    }
+    float h[1][kAH];
+    lo_terms<1, ND, kAH>(d, x, term_tab, h);
+    ema_update(e, x.g[0], x.m[0], x.rms[0]);
+    float f18[kNStat];
+    lo_features(x.g[0], x.p[0], x.m[0], x.rms[0], x.rfcf[0], 1e-6f, f18);
+    // the 16 per-element channels AdafacLO uses, and their rows in the 30-channel order
+    const float f[16] = {f18[0], f18[2], f18[3], f18[4], f18[5], f18[6], f18[7], f18[8], f18[9], f18[10],
+                         f18[11], f18[12], f18[13], f18[15], f18[16], f18[17]};
+    const int row[16] = {0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 27, 28, 29};
+    const float pn = adafac_mlp<16>(f, row, h[0], wfold_t, net, a, x.p[0]);
+    *(gfloat*)(a.mom + idx) = x.m[0][0];
+    *(gfloat*)(a.mom + n + idx) = x.m[0][1];
+    *(gfloat*)(a.mom + 2 * n + idx) = x.m[0][2];
+    *(gfloat*)(a.rms + idx) = x.rms[0];
+    *(gfloat*)(a.param + idx) = pn;
+  }
+}
+
+__device__ __forceinline__ void adafac_apply_vec(const TDesc& d, const PyloTensorArgs& a, long long base,
+                                                 long long count, const EmaConsts& e, const PyloDecays& dec,
+                                                 const float* wfold_t, const float* net, const float* bias_eff) {
+  const long long n = d.n;
+  for (long long off = threadIdx.x; off < count; off += kThreads) {
+    const long long idx = base + off;
+    if (idx >= n) break;
+    VecIn<1> x;
+    vec_load<1>(d, a, idx, x);
+    vec_update(e, dec, x.g[0], x.m[0], x.rms[0], x.v[0]);
+    float f30[30];
+    vec_features(x.g[0], x.p[0], x.m[0], x.rms[0], x.v[0], 1e-6f, f30);
+    float f[28];
+    int row[28];
+    {
+      int q = 0;
+#pragma unroll
+      for (int c = 0; c < 30; ++c)
+        if (adafac_channel(c)) { f[q] = f30[c]; row[q] = c; ++q; }
+    }
+    float h[kAH];
+#pragma unroll
+    for (int j = 0; j < kAH; ++j) h[j] = bias_eff[j];
+    const float pn = adafac_mlp<28>(f, row, h, wfold_t, net, a, x.p[0]);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      *(gfloat*)(a.mom + k * n + idx) = x.m[0][k];
+      *(gfloat*)(a.fac_v + k * n + idx) = x.v[0][k];
+    }
+    *(gfloat*)(a.rms + idx) = x.rms[0];
+    *(gfloat*)(a.param + idx) = pn;
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void k_adafac_apply(const TDesc* __restrict__ descs,
+                                                           const PyloTensorArgs* __restrict__ dyn,
+                                                           const Item* __restrict__ items,
+                                                           const float* __restrict__ fac_tab,
+                                                           const float* __restrict__ term_tab, PyloDecays dec,
+                                                           const float* __restrict__ wfold,
+                                                           const float* __restrict__ net,
+                                                           const float* __restrict__ bias_eff) {
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  const EmaConsts e = make_ema(dec);
+  const float* w = wfold + (size_t)it.tensor * kAFold;
+  const long long count = (long long)kThreads * d.vec * kElemIters;
+  const long long base = (long long)it.a * count;
+  if (d.mode == kModeFac2D) adafac_apply_fac<false>(d, a, base, count, e, fac_tab, term_tab, w, net);
+  else if (d.mode == kModeFacND) adafac_apply_fac<true>(d, a, base, count, e, fac_tab, term_tab, w, net);
+  else adafac_apply_vec(d, a, base, count, e, dec, w, net, bias_eff);
+}
+
+}  // namespace pylo

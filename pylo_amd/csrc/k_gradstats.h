@@ -237,12 +237,20 @@ __device__ __forceinline__ size_t term_index(const TDesc& d, int which, int j, i
 
 // Row_factor / col_factor of one entry, and the two normalised broadcast features it carries
 // (accumulator value and rsqrt(value + 1e-8)).  ELO_CELO2_naive.py:161-164,202-213
-__device__ __forceinline__ void vector_entry(bool is_r, const float* fac, int len, int i, const BScale& bs,
-                                             float (&fct)[3], float (&x0)[3], float (&x1)[3]) {
+__device__ __forceinline__ void vector_entry(const TDesc& d, bool is_r, const float* fac, int len, int i,
+                                             const BScale& bs, float (&fct)[3], float (&x0)[3], float (&x1)[3]) {
 #pragma unroll
   for (int k = 0; k < 3; ++k) {
     const float f = fac[(size_t)k * len + i];
-    fct[k] = is_r ? rsq(fmaxf(f / (bs.rcm[k] + 1e-9f), 1e-9f)) : rsq(fmaxf(f, 1e-9f));
+    float rcm = bs.rcm[k];
+    if (is_r && d.mode == kModeFacND) {  // mean over the dc axis of this entry's slice of fac_r
+      const int sz = d.rcm_size, st = d.rcm_stride;
+      const int base = (i / (sz * st)) * (sz * st) + i % st;
+      double s = 0.0;
+      for (int x = 0; x < sz; ++x) s += (double)fac[(size_t)k * len + base + x * st];
+      rcm = (float)(s / (double)sz);
+    }
+    fct[k] = is_r ? rsq(fmaxf(f / (rcm + 1e-9f), 1e-9f)) : rsq(fmaxf(f, 1e-9f));
     x0[k] = f * (is_r ? bs.s[k] : bs.s[3 + k]);
     x1[k] = rsq(f + 1e-8f) * (is_r ? bs.s[6 + k] : bs.s[9 + k]);
   }
@@ -327,7 +335,7 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
   const float* fac = is_r ? a.fac_r : a.fac_c;
   for (int i = it.a * kV0bEnt + threadIdx.x; i < min(len, (it.a + 1) * kV0bEnt); i += kThreads) {
     float fct[3], x0[3], x1[3];
-    vector_entry(is_r, fac, len, i, bs, fct, x0, x1);
+    vector_entry(d, is_r, fac, len, i, bs, fct, x0, x1);
 #pragma unroll
     for (int k = 0; k < 3; ++k) fac_tab[fac_index(d, which, k, i)] = fct[k];
     if (w1 != nullptr) vector_terms<H>(d, which, is_r, i, x0, x1, w1, b1, term_tab);
@@ -356,7 +364,7 @@ __global__ __launch_bounds__(kThreads) void k_terms(const TDesc* __restrict__ de
   const float* fac = is_r ? a.fac_r : a.fac_c;
   for (int i = it.a * kV0bEnt + threadIdx.x; i < min(len, (it.a + 1) * kV0bEnt); i += kThreads) {
     float fct[3], x0[3], x1[3];
-    vector_entry(is_r, fac, len, i, bs, fct, x0, x1);
+    vector_entry(d, is_r, fac, len, i, bs, fct, x0, x1);
     vector_terms<H>(d, which, is_r, i, x0, x1, w1, b1, term_tab);
   }
 }

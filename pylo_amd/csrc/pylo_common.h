@@ -52,6 +52,8 @@ struct TDesc {
   int pitch[2];     // row pitch of the SoA tables of vector 0 / 1 (len rounded up to 4)
   int nd_size[2];   // N-D: size and stride of the dim removed from vector 0 / 1;
   int nd_stride[2]; //      entry = (idx / (size*stride)) * stride + idx % stride
+  int rcm_size;     // N-D: size of the 2nd-largest dim and its stride inside the row vector; row_col_mean
+  int rcm_stride;   //      is the mean over that axis, one value per slice (2-D: one value per tensor)
   int n_strips, n_colblk;
   int blk0, nblk;   // range of element-chunk blocks (rows of the statistics partials)
   int fac_slot;     // index among factored tensors, -1 otherwise

@@ -18,6 +18,7 @@
 
 #include "k_celo2.h"
 #include "k_gradstats.h"
+#include "k_adafac.h"
 #include "k_velo.h"
 #include "pylo_common.h"
 
@@ -74,7 +75,8 @@ struct Layout {
 int first_layer_width(int kind) { return kind == PYLO_KIND_CELO2 ? 8 : kind == PYLO_KIND_VELO ? 4 : 32; }
 
 int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int velo_hidden) {
-  if (kind != PYLO_KIND_CELO2 && kind != PYLO_KIND_VELO) return fail("plan: this optimizer kind is not implemented");
+  if (kind != PYLO_KIND_CELO2 && kind != PYLO_KIND_VELO && kind != PYLO_KIND_ADAFAC)
+    return fail("plan: unknown optimizer kind");
   if (T <= 0 || shapes == nullptr) return fail("plan: no tensors");
   L.H = first_layer_width(kind);
   L.descs.assign(T, TDesc{});
@@ -136,6 +138,9 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
           d.sumlen[w] = d.nd_size[w];
           d.npart[w] = 1;
         }
+        // the dc axis as it sits inside the row vector (the tensor without dim dr)
+        d.rcm_size = d.nd_size[1];
+        d.rcm_stride = dc > dr ? d.nd_stride[1] : d.nd_stride[1] / std::max(d.nd_size[0], 1);
       }
       for (int w = 0; w < 2; ++w) {
         d.pitch[w] = (int)round4(d.len[w]);
@@ -198,7 +203,8 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_v0part = take(sizeof(double) * kNV0 * L.v0a_items.size());
   L.off_bscale = take(sizeof(BScale) * nfac);
   L.off_stats = take(sizeof(double) * kStatW * L.el_items.size());
-  L.off_wfold = take(sizeof(float) * (kind == PYLO_KIND_CELO2 ? kC2Fold * nfac : (size_t)kVFold * T));
+  L.off_wfold = take(sizeof(float) * (kind == PYLO_KIND_CELO2 ? kC2Fold * nfac
+                                      : kind == PYLO_KIND_VELO ? (size_t)kVFold * T : (size_t)kAFold * T));
   L.off_chan_ms = take(sizeof(float) * kNStat * nfac);
   L.off_totals = take(sizeof(double) * kStatW * T);
   L.Tpad = (T + kGateBT - 1) / kGateBT * kGateBT;
@@ -303,14 +309,18 @@ static const char* kVeloLaunches[] = {"k_p0(sums)", "k_p0_nd", "k_v0a", "k_v0b",
                                       "k_lo_reduce", "k_velo_mix", "k_velo_gates", "k_velo_heads", "k_terms",
                                       "k_velo_apply"};
 
+static const char* kAdafacLaunches[] = {"k_p0(sums)", "k_p0_nd", "k_v0a", "k_adafac_bias", "k_v0b", "k_adafac_stats",
+                                        "k_lo_reduce", "k_adafac_fold", "k_adafac_apply"};
+
 int pylo_mi355_plan_num_launches(const PyloPlan* P) {
   if (!P) return -1;
-  return P->kind == PYLO_KIND_CELO2 ? 8 : P->kind == PYLO_KIND_VELO ? 12 : -1;
+  return P->kind == PYLO_KIND_CELO2 ? 8 : P->kind == PYLO_KIND_VELO ? 12 : P->kind == PYLO_KIND_ADAFAC ? 9 : -1;
 }
 
 const char* pylo_mi355_plan_launch_name(const PyloPlan* P, int launch) {
   if (!P || launch < 0 || launch >= pylo_mi355_plan_num_launches(P)) return "";
-  return P->kind == PYLO_KIND_CELO2 ? kCelo2Launches[launch] : kVeloLaunches[launch];
+  return P->kind == PYLO_KIND_CELO2 ? kCelo2Launches[launch]
+         : P->kind == PYLO_KIND_VELO ? kVeloLaunches[launch] : kAdafacLaunches[launch];
 }
 
 int pylo_mi355_plan_timing_begin(PyloPlan* P, int max_steps) {
@@ -548,6 +558,71 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
     hipLaunchKernelGGL(k_terms<4>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, bscale, canon, kVCanon, term_tab);
   HIP_TRY(mark());
   if (n_el > 0) hipLaunchKernelGGL(k_velo_apply, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, term_tab, dec, wfold);
+  HIP_TRY(mark());
+  mark.done();
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, const PyloDecays* decays,
+                                      const float* net, float step, void* stream) {
+  if (!P || !args || !decays || !net) return fail("adafac_step: null argument");
+  if (P->kind != PYLO_KIND_ADAFAC) return fail("adafac_step: plan is not an AdafacLO plan");
+  if (int rc = check_args(P, args, false)) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (int rc = upload_args(P, args, s)) return rc;
+  const Layout& L = P->L;
+  const TDesc* descs = P->at<TDesc>(L.off_descs);
+  const PyloTensorArgs* dyn = P->at<PyloTensorArgs>(L.off_dyn);
+  const Item* p0_items = P->at<Item>(L.off_p0_items);
+  const Item* nd_items = P->at<Item>(L.off_nd_items);
+  const Item* el_items = P->at<Item>(L.off_el_items);
+  const Item* v0a_items = P->at<Item>(L.off_v0a_items);
+  const Item* v0b_items = P->at<Item>(L.off_v0b_items);
+  float* part = P->at<float>(L.off_part);
+  double* gsq = P->at<double>(L.off_gsq);
+  int* flag = P->at<int>(L.off_flag);
+  Globals* gl = P->at<Globals>(L.off_globals);
+  float* fac_tab = P->at<float>(L.off_fac);
+  float* term_tab = P->at<float>(L.off_term);
+  double* v0part = P->at<double>(L.off_v0part);
+  BScale* bscale = P->at<BScale>(L.off_bscale);
+  double* stats = P->at<double>(L.off_stats);
+  float* wfold = P->at<float>(L.off_wfold);
+  double* totals = P->at<double>(L.off_totals);
+  float* bias_eff = P->at<float>(L.off_xfeat);  // 32 floats; the LSTM feature buffer is unused by this kind
+  const int n_p0 = (int)L.p0_items.size(), n_nd = (int)L.nd_items.size(), n_el = (int)L.el_items.size();
+  const int n_v0a = (int)L.v0a_items.size(), n_v0b = (int)L.v0b_items.size();
+  const int T = P->T;
+  const PyloDecays dec = *decays;
+  VeloStep vs;
+  std::memset(&vs, 0, sizeof(vs));
+  Marks mark(P, s);
+
+  HIP_TRY(mark());
+  if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0);
+  HIP_TRY(mark());
+  if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part);
+  HIP_TRY(mark());
+  if (n_v0a > 0)
+    hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
+  HIP_TRY(mark());
+  hipLaunchKernelGGL(k_adafac_bias, dim3(1), dim3(64), 0, s, net, step, bias_eff);
+  HIP_TRY(mark());
+  if (n_v0b > 0)
+    hipLaunchKernelGGL(k_v0b<kAH>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-5f,
+                       net + kAW1, (const float*)bias_eff, fac_tab, term_tab, bscale);
+  HIP_TRY(mark());
+  if (n_el > 0) hipLaunchKernelGGL(k_adafac_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, dec, stats);
+  HIP_TRY(mark());
+  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kThreads), 0, s, descs, dyn, T, stats, totals, (const float*)nullptr, vs,
+                     (float*)nullptr);
+  HIP_TRY(mark());
+  hipLaunchKernelGGL(k_adafac_fold, dim3(T), dim3(kThreads), 0, s, descs, dyn, totals, net, wfold);
+  HIP_TRY(mark());
+  if (n_el > 0)
+    hipLaunchKernelGGL(k_adafac_apply, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, term_tab, dec,
+                       wfold, net, (const float*)bias_eff);
   HIP_TRY(mark());
   mark.done();
   HIP_TRY(hipGetLastError());

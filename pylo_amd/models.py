@@ -186,12 +186,25 @@ def pack_celo2(net: CELO2MLP) -> torch.Tensor:
     return torch.cat([t.reshape(-1).float() for t in parts]).contiguous()
 
 
+# AdafacLO's 28 features (g, p, m0..2, rms, m_k*rs, rs, fac_g_k, row_k, col_k, rsqrt(row_k), rsqrt(col_k),
+# fac_mom_k; pylo/optim/AdafacLO_naive.py:261-300) in the kernels' 30-channel numbering, which also
+# has clip(g) at 1 and g*rs at 14.
+ADAFAC_CHANNELS = (0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 15, 16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26,
+                   27, 28, 29)
+
+
 def pack_metamlp(net: MetaMLP) -> torch.Tensor:
-    """[W_in (32,39) | b_in 32 | W_h (32,32) | b_h 32 | W_out (2,32) | b_out 2] = 2402 floats, (out,in)."""
+    """2466 floats, every matrix (in, out): w1 (30,32) in the 30-channel order (rows 1, 14 zero) | b1 32 |
+    w_time (11,32) | w_h (32,32) | b_h 32 | w_o (32,2) | b_o 2."""
     seq = net.network
-    parts = [seq.input.weight, seq.input.bias, seq.linear_0.weight, seq.linear_0.bias,
-             seq.output.weight, seq.output.bias]
-    return torch.cat([t.detach().reshape(-1).float() for t in parts]).contiguous()
+    w_in = seq.input.weight.detach().float()                 # (32, 39)
+    if tuple(w_in.shape) != (32, 39) or not hasattr(seq, "linear_0") or hasattr(seq, "linear_1"):
+        raise ValueError("the AdafacLO kernel supports MetaMLP(input_size=39, hidden_size=32, hidden_layers=1)")
+    w1 = torch.zeros(30, 32, dtype=torch.float32, device=w_in.device)
+    w1[list(ADAFAC_CHANNELS)] = w_in[:, :28].t()
+    parts = [w1, seq.input.bias, w_in[:, 28:39].t(), seq.linear_0.weight.t(), seq.linear_0.bias,
+             seq.output.weight.t(), seq.output.bias]
+    return torch.cat([t.detach().float().reshape(-1) for t in parts]).contiguous()
 
 
 def pack_velo_bank(net: VeLOMLP) -> torch.Tensor:

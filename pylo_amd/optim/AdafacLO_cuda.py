@@ -1,0 +1,187 @@
+"""AdafacLO_CUDA (small_fc_lopt) on MI355X: one multi-tensor HIP step per optimizer step.
+
+Drop-in for pylo/optim/AdafacLO_cuda.py:76-407: same constructor and ``step()``, per-parameter state
+``step`` (float64 CPU scalar), ``exp_avg (3,*s)``, ``exp_avg_sq (*s)``, ``exp_avg_sq_r``,
+``exp_avg_sq_c``.  Arithmetic follows the naive class (pylo/optim/AdafacLO_naive.py:187-311); in
+particular ``row_col_mean`` averages over the 2nd-largest parameter dim (the reference's CUDA class
+reduces the decay axis instead, AdafacLO_cuda.py:342-343), and 1-D tensors use
+``m * (v + 1e-6)^-1/2`` for the last feature group (AdafacLO_naive.py:298).
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Union
+
+import torch
+from torch.optim import Optimizer
+
+from .. import _lib
+from ..models import MetaMLP, pack_metamlp
+
+
+def _factored_dims(shape):
+    """(dc, dr): 2nd-largest and largest dim, ties by index (AdafacLO_cuda.py:52-73 with
+    min_dim_size_to_factor=1)."""
+    if len(shape) < 2:
+        return None
+    order = sorted(range(len(shape)), key=lambda i: (shape[i], i))
+    return order[-2], order[-1]
+
+
+def _decays(initial, offsets, device):
+    """clip(1 - exp(10 * (log(1 - d0) / 10 + offset)), 0, 1) in fp32 (AdafacLO_cuda.py:29-34,153-173)."""
+    off = offsets if torch.is_tensor(offsets) else torch.tensor(offsets, device=device)
+    par = torch.log(1 - torch.tensor(initial, device=device)) / 10.0 + off.to(device)
+    return torch.clip(1 - torch.exp(par * 10.0), 0.0, 1.0)
+
+
+class AdafacLO_CUDA(Optimizer):
+    def __init__(
+        self,
+        params,
+        lr: float = 1.0,
+        min_dim_size_to_factor: int = 32,
+        decay_rate: float = 0.8,
+        decay_offset: int = 0,
+        beta2_cap: float = 0.999,
+        initial_momentum_decays=(0.9, 0.99, 0.999),
+        initial_rms_decays=(0.999,),
+        initial_adafactor_decays=(0.9, 0.99, 0.999),
+        momentum_decays=[0.15216392, 0.14245212, 0.06812963],
+        rms_decays=[0.01079706],
+        adafactor_decays=[0.18621896, -0.10864615, -0.06185547],
+        momentum_dtype: Union[str, torch.dtype] = torch.float32,
+        eps: Optional[float] = None,
+        weight_decay: float = 0.0,
+        clipping_threshold: Optional[float] = None,
+        max_grad_norm: Optional[float] = None,
+        unscaled_wd: bool = False,
+        step_mult: float = 0.01,
+        exp_mult: float = 0.001,
+        load_from_file: Optional[str] = None,
+        *,
+        foreach: Optional[bool] = False,
+        hf_key: Optional[str] = "btherien/mulo",
+        network: Optional[MetaMLP] = None,
+    ):
+        if not torch.cuda.is_available():
+            raise RuntimeError("AdafacLO_CUDA requires a GPU (torch.cuda.is_available() is False).")
+        _lib.load()
+        if isinstance(momentum_dtype, str):
+            momentum_dtype = {"float16": torch.float16, "bfloat16": torch.bfloat16,
+                              "float32": torch.float32}[momentum_dtype]
+        if momentum_dtype != torch.float32:
+            raise NotImplementedError("the fused step keeps momentum in float32")
+        if foreach:
+            raise NotImplementedError("foreach=True is not implemented (neither is it in the reference)")
+        defaults = dict(lr=lr, min_dim_size_to_factor=min_dim_size_to_factor, decay_rate=decay_rate,
+                        decay_offset=decay_offset, beta2_cap=beta2_cap, momentum_dtype=momentum_dtype, eps=eps,
+                        weight_decay=weight_decay, clipping_threshold=clipping_threshold,
+                        max_grad_norm=max_grad_norm, unscaled_wd=unscaled_wd, foreach=foreach)
+        super().__init__(params, defaults)
+        first = next(p for g in self.param_groups for p in g["params"])
+        self.device = first.device if first.is_cuda else torch.device("cuda", torch.cuda.current_device())
+        self.metamlp = (network if network is not None else MetaMLP.from_pretrained(hf_key)).to(self.device)
+        if load_from_file:
+            loaded = torch.load(load_from_file, map_location=self.device, weights_only=True)
+            self.metamlp.load_state_dict(loaded["state_dict"])
+            momentum_decays = loaded["decays"]["momentum_decays"]
+            rms_decays = loaded["decays"]["rms_decays"]
+            adafactor_decays = loaded["decays"]["adafactor_decays"]
+        for prm in self.metamlp.parameters():
+            prm.requires_grad = False
+        self.beta_m = _decays(initial_momentum_decays, momentum_decays, self.device)
+        self.beta_rms = _decays(initial_rms_decays, rms_decays, self.device)
+        self.beta_adafactor = _decays(initial_adafactor_decays, adafactor_decays, self.device)
+        self.step_mult = step_mult
+        self.exp_mult = exp_mult
+        self._net = pack_metamlp(self.metamlp).to(self.device)
+        self._decays = _lib.make_decays(self.beta_m.tolist(), float(self.beta_rms[0]),
+                                        self.beta_adafactor.tolist())
+        self._plan = None
+        self._plan_key = None
+
+    def _init_state(self, state, p):
+        """pylo/optim/AdafacLO_cuda.py:227-256"""
+        shape = tuple(p.shape)
+        state["step"] = torch.tensor(0.0, dtype=torch.float64)
+        fd = _factored_dims(shape)
+        if fd is not None:
+            dc, dr = fd
+            r_shape, c_shape = list(shape), list(shape)
+            r_shape[dr] = 1
+            c_shape[dc] = 1
+            state["exp_avg_sq_r"] = torch.zeros([3] + r_shape, device=self.device)
+            state["exp_avg_sq_c"] = torch.zeros([3] + c_shape, device=self.device)
+        else:
+            state["exp_avg_sq_r"] = torch.zeros((3,) + shape, device=self.device)
+            state["exp_avg_sq_c"] = state["exp_avg_sq_r"]      # the reference keeps two identical copies
+        state["exp_avg_sq"] = torch.zeros(shape, device=self.device)
+        state["exp_avg"] = torch.zeros((3,) + shape, device=self.device)
+
+    def _ensure_plan(self, tensors):
+        key = tuple(tuple(p.shape) for _, p in tensors)
+        if key == self._plan_key:
+            return
+        for _, p in tensors:
+            if not p.is_cuda or p.device != self.device or p.dtype != torch.float32 or not p.is_contiguous():
+                raise TypeError("AdafacLO_CUDA: parameters must be contiguous float32 tensors on the optimizer's GPU")
+        if self._plan is not None:
+            self._plan.close()
+        self._plan = _lib.Plan(_lib.KIND_ADAFAC, [tuple(p.shape) for _, p in tensors], [0] * len(tensors),
+                               self.device)
+        self._plan_key = key
+
+    @torch.no_grad()
+    def step(self, loss=None):
+        tensors = [(g, p) for g in self.param_groups for p in g["params"]]
+        self._ensure_plan(tensors)
+        plan = self._plan
+        n = len(tensors)
+        keys = ("grad", "param", "mom", "rms", "fac_r", "fac_c", "fac_v")
+        cols = {k: [0] * n for k in keys}
+        fl = {k: [0.0] * n for k in ("lr", "weight_decay", "exp_mult", "step_mult")}
+        keep = []
+        step_fed = None
+        for i, (group, p) in enumerate(tensors):
+            if group["max_grad_norm"] is not None:
+                torch.nn.utils.clip_grad_norm_(p, group["max_grad_norm"])
+            g = p.grad
+            if g is None:
+                continue
+            if g.is_sparse:
+                raise RuntimeError("Sparse gradients not supported")
+            if g.dtype != torch.float32:
+                raise TypeError("AdafacLO_CUDA: gradients must be float32")
+            if not g.is_contiguous():
+                g = g.contiguous()
+                keep.append(g)
+            state = self.state[p]
+            if len(state) == 0:
+                self._init_state(state, p)
+            state["step"] += 1
+            s0 = float(state["step"]) - 1.0
+            if step_fed is None:
+                step_fed = s0
+            elif step_fed != s0:
+                raise NotImplementedError("AdafacLO_CUDA: parameters with different step counts in one call")
+            cols["grad"][i], cols["param"][i] = g.data_ptr(), p.data_ptr()
+            cols["mom"][i], cols["rms"][i] = state["exp_avg"].data_ptr(), state["exp_avg_sq"].data_ptr()
+            if _factored_dims(tuple(p.shape)) is None:
+                cols["fac_v"][i] = state["exp_avg_sq_r"].data_ptr()
+            else:
+                cols["fac_r"][i] = state["exp_avg_sq_r"].data_ptr()
+                cols["fac_c"][i] = state["exp_avg_sq_c"].data_ptr()
+            fl["lr"][i], fl["weight_decay"][i] = group["lr"], group["weight_decay"]
+            fl["exp_mult"][i], fl["step_mult"][i] = self.exp_mult, self.step_mult
+        if step_fed is None:
+            return loss
+        args = plan.args
+        for k, v in cols.items():
+            args[k] = v
+        for k, v in fl.items():
+            args[k] = v
+        with torch.cuda.device(self.device):
+            plan.adafac_step(self._decays, self._net, step_fed, torch.cuda.current_stream(self.device).cuda_stream)
+        del keep
+        return loss

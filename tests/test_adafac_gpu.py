@@ -1,0 +1,125 @@
+"""GPU parity of the fused AdafacLO step (HIP, through the C ABI) against the golden trajectories
+of the reference's naive class and against the CPU oracle on larger / odd shapes.
+
+Tolerance: rel 1e-5 / abs 1e-6 on parameters and every accumulator, every step.  The reference has
+no numerical test of its `cuda_lo` kernel for AdafacLO (only a resume test).
+"""
+
+import copy
+
+import pytest
+import torch
+
+from golden_io import Golden, max_err, trailing_to_keepdim
+
+pytestmark = pytest.mark.gpu
+
+REL, ABS = 1e-5, 1e-6
+
+
+@pytest.mark.parametrize("name", ["adafac_small", "adafac_small_wd"])
+def test_adafac_matches_reference_golden(name):
+    from oracle import pylo_oracle as O
+    from pylo_amd import AdafacLO_CUDA
+    from pylo_amd.models import MetaMLP
+
+    G = Golden(name)
+    meta, shapes = G.meta, G.shapes
+    net = MetaMLP(39, 32, 1)
+    net.load_state_dict(G.state_dict("net"))
+    gpu = [torch.nn.Parameter(G.t(f"init/{i}").cuda()) for i in range(len(shapes))]
+    opt = AdafacLO_CUDA(gpu, lr=meta["lr"], weight_decay=meta["weight_decay"], network=net)
+    worst = 0.0
+    for t in range(meta["n_steps"]):
+        for i, p in enumerate(gpu):
+            p.grad = G.t(f"grad{t}/{i}").cuda()
+        opt.step()
+        for i, p in enumerate(gpu):
+            st = opt.state[p]
+            checks = [("param", p, G.t(f"step{t}/param/{i}")), ("exp_avg", st["exp_avg"], G.t(f"step{t}/exp_avg/{i}")),
+                      ("exp_avg_sq", st["exp_avg_sq"], G.t(f"step{t}/exp_avg_sq/{i}"))]
+            if len(shapes[i]) < 2:
+                checks.append(("fac_v", st["exp_avg_sq_r"], G.t(f"step{t}/fac_vec_v/{i}")))
+            else:
+                dc, dr = O.factored_dims(shapes[i])
+                checks.append(("row", st["exp_avg_sq_r"],
+                               trailing_to_keepdim(G.t(f"step{t}/fac_vec_row_trailing/{i}"), dr)))
+                checks.append(("col", st["exp_avg_sq_c"],
+                               trailing_to_keepdim(G.t(f"step{t}/fac_vec_col_trailing/{i}"), dc)))
+            for tag, got, ref in checks:
+                e = max_err(got, ref, REL, ABS)
+                worst = max(worst, e)
+                assert e <= 1.0, (name, t, i, tag, e)
+    print(name, "worst err/tol", worst)
+
+
+def test_adafac_matches_oracle_mixed_shapes():
+    from oracle import pylo_oracle as O
+    from pylo_amd import AdafacLO_CUDA
+    from pylo_amd.models import MetaMLP
+
+    torch.manual_seed(9)
+    net = MetaMLP(39, 32, 1)
+    shapes = [(256, 516), (516, 256), (300, 260), (37, 101), (32, 16, 3, 3), (1, 1, 48), (1000,), (7,), (64, 64)]
+    gen = torch.Generator().manual_seed(23)
+    init = [torch.randn(s, generator=gen) * 0.3 for s in shapes]
+    cpu = [v.clone() for v in init]
+    gpu = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+    orc = O.AdafacOracle(cpu, net.state_dict(), lr=0.5, weight_decay=1e-3)
+    opt = AdafacLO_CUDA(gpu, lr=0.5, weight_decay=1e-3, network=copy.deepcopy(net))
+    worst = 0.0
+    for t in range(5):
+        grads = [torch.randn(s, generator=gen) * (10.0 ** (-(i % 4))) for i, s in enumerate(shapes)]
+        if t == 4:
+            grads[3] = None      # a tensor without gradient is skipped
+        for p, g in zip(gpu, grads):
+            p.grad = None if g is None else g.cuda()
+        orc.step(grads)
+        opt.step()
+        for i, p in enumerate(gpu):
+            st, so = opt.state[p], orc.state[i]
+            checks = [("param", p, cpu[i])]
+            if len(st):
+                checks += [("exp_avg", st["exp_avg"], so["exp_avg"]), ("exp_avg_sq", st["exp_avg_sq"], so["exp_avg_sq"]),
+                           ("r", st["exp_avg_sq_r"], so["exp_avg_sq_r"]), ("c", st["exp_avg_sq_c"], so["exp_avg_sq_c"])]
+            for tag, got, ref in checks:
+                e = max_err(got, ref, REL, ABS)
+                worst = max(worst, e)
+                assert e <= 1.0, (t, i, tag, e)
+    print("adafac mixed worst err/tol", worst)
+
+
+def test_adafac_state_dict_resume():
+    """tests/test_optimizer_resume.py:19-164"""
+    from pylo_amd import AdafacLO_CUDA
+    from pylo_amd.models import MetaMLP
+
+    torch.manual_seed(4)
+    net = MetaMLP(39, 32, 1)
+    shapes = [(24, 16), (16,)]
+    gen = torch.Generator().manual_seed(2)
+    init = [torch.randn(s, generator=gen) for s in shapes]
+    grads = [[torch.randn(s, generator=gen).cuda() for s in shapes] for _ in range(8)]
+
+    def run(params, opt, ts):
+        for t in ts:
+            for p, g in zip(params, grads[t]):
+                p.grad = g.clone()
+            opt.step()
+
+    a = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+    oa = AdafacLO_CUDA(a, lr=1.0, network=net)
+    run(a, oa, range(4))
+    sd = copy.deepcopy(oa.state_dict())
+    snap = [p.detach().clone() for p in a]
+    run(a, oa, range(4, 8))
+    b = [torch.nn.Parameter(v.clone()) for v in snap]
+    ob = AdafacLO_CUDA(b, lr=1.0, network=net)
+    ob.load_state_dict(sd)
+    run(b, ob, range(4, 8))
+    for x, y in zip(a, b):
+        assert torch.max(torch.abs(x - y)).item() < 1e-6
+    st = oa.state[a[0]]
+    assert set(st.keys()) == {"step", "exp_avg_sq_r", "exp_avg_sq_c", "exp_avg_sq", "exp_avg"}
+    assert st["exp_avg"].shape == (3, 24, 16) and st["exp_avg_sq_r"].shape == (3, 1, 16)
+    assert st["step"].dtype == torch.float64 and float(st["step"]) == 8.0

@@ -101,6 +101,17 @@ def decay_from_offsets(initial: Sequence[float], offsets: Sequence[float]) -> to
     return torch.clip(1 - torch.exp(par * 10.0), 0.0, 1.0)
 
 
+def _to_double(obj):
+    """Recursively converts floating tensors held in dicts / lists / tuples to fp64."""
+    if torch.is_tensor(obj):
+        return obj.double() if obj.is_floating_point() else obj
+    if isinstance(obj, dict):
+        return {k: _to_double(v) for k, v in obj.items()}
+    if isinstance(obj, (list, tuple)):
+        return type(obj)(_to_double(v) for v in obj)
+    return obj
+
+
 def _bview(beta: torch.Tensor, ndim: int) -> torch.Tensor:
     return beta.view([-1] + [1] * ndim)
 
@@ -200,18 +211,20 @@ class EloCelo2Oracle:
                  momentum_decays=(0.9, 0.99, 0.999), rms_decays=(0.95,),
                  adafactor_decays=(0.9, 0.99, 0.999), exp_mult=0.0, rmsmult=1.0,
                  param_scale_mult=False, ns_coeffs=(3.4445, -4.7750, 2.0315), ns_iters=5,
-                 ns_eps=1e-8, grad_clip_val=1000.0, is_embedding: Sequence[bool] = ()):
+                 ns_eps=1e-8, grad_clip_val=1000.0, is_embedding: Sequence[bool] = (), device="cpu"):
         self.params = params
-        self.net = {k: v.detach().to(F32).cpu() for k, v in net.items()}
+        self.device = torch.device(device)
+        self.net = {k: v.detach().to(F32).to(self.device) for k, v in net.items()}
         self.h = dict(lr=lr, weight_decay=weight_decay, clip_grad=clip_grad, clip_norm=clip_norm,
                       adam_lr_mult=adam_lr_mult,
                       adam_weight_decay=weight_decay if adam_weight_decay is None else adam_weight_decay,
                       use_adamw_for_1d=use_adamw_for_1d, orthogonalize=orthogonalize,
                       exp_mult=exp_mult, rmsmult=rmsmult, param_scale_mult=param_scale_mult,
                       grad_clip_val=grad_clip_val)
-        self.beta_m = torch.tensor(momentum_decays, dtype=F32)
-        self.beta_rms = torch.clamp(torch.tensor(rms_decays, dtype=F32), 0.0, 1.0)
-        self.beta_fac = torch.clamp(torch.tensor(adafactor_decays, dtype=F32), 0.0, 1.0)
+        dv = self.device
+        self.beta_m = torch.tensor(momentum_decays, dtype=F32, device=dv)
+        self.beta_rms = torch.clamp(torch.tensor(rms_decays, dtype=F32, device=dv), 0.0, 1.0)
+        self.beta_fac = torch.clamp(torch.tensor(adafactor_decays, dtype=F32, device=dv), 0.0, 1.0)
         self.ns = (tuple(float(c) for c in ns_coeffs), ns_iters, ns_eps)
         self.is_embedding = list(is_embedding) or [False] * len(params)
         self.t = 0
@@ -219,20 +232,28 @@ class EloCelo2Oracle:
         self.state: List[Dict[str, torch.Tensor]] = []
         for p in params:
             s = tuple(p.shape)
-            st = {"mom": torch.zeros((3,) + s), "rms": torch.zeros(s)}
+            st = {"mom": torch.zeros((3,) + s, device=dv), "rms": torch.zeros(s, device=dv)}
             fd = factored_dims(s)
             if fd is not None:
                 dc, dr = fd
                 rs_, cs_ = list(s), list(s)
                 rs_[dr] = 1
                 cs_[dc] = 1
-                st["fac_r"] = torch.zeros([3] + rs_)
-                st["fac_c"] = torch.zeros([3] + cs_)
+                st["fac_r"] = torch.zeros([3] + rs_, device=dv)
+                st["fac_c"] = torch.zeros([3] + cs_, device=dv)
             self.state.append(st)
+
+    def double_(self):
+        """Evaluate everything in fp64 from here on (the decays keep their fp32 values): the
+        reference formulas without fp32 rounding, for checks at sizes where fp32 PyTorch reductions
+        are themselves less accurate than the tolerance.  ``self.params`` must then be fp64 tensors."""
+        self.net, self.state = _to_double(self.net), _to_double(self.state)
+        self.beta_m, self.beta_rms, self.beta_fac = self.beta_m.double(), self.beta_rms.double(), self.beta_fac.double()
+        return self
 
     def grad_scale(self, grads) -> float:
         """clip_norm / max(global_norm, clip_norm).  pylo/optim/ELO_CELO2_naive.py:126-135"""
-        total = torch.zeros(())
+        total = torch.zeros((), device=self.device)
         for g in grads:
             if g is not None:
                 total = total + g.detach().float().pow(2).sum()
@@ -435,10 +456,20 @@ class VeloOracle:
                  num_steps=10000, weight_decay=0.0,
                  initial_momentum_decays=(0.9, 0.99, 0.999), initial_rms_decays=(0.999,),
                  initial_adafactor_decays=(0.9, 0.99, 0.999),
-                 momentum_decays=(0.0, 0.0, 0.0), rms_decays=(0.0,), adafactor_decays=(0.0, 0.0, 0.0)):
+                 momentum_decays=(0.0, 0.0, 0.0), rms_decays=(0.0,), adafactor_decays=(0.0, 0.0, 0.0),
+                 device="cpu"):
         self.params = params
-        self.rnn = {k: v.detach().to(F32).cpu() for k, v in rnn.items()}
-        self.mlp = {k: v.detach().to(F32).cpu() for k, v in mlp.items()}
+        self.device = torch.device(device)
+        with torch.device(self.device):
+            self._init(params, rnn, mlp, lr, exp_mult, step_mult, num_steps, weight_decay,
+                       initial_momentum_decays, initial_rms_decays, initial_adafactor_decays,
+                       momentum_decays, rms_decays, adafactor_decays)
+
+    def _init(self, params, rnn, mlp, lr, exp_mult, step_mult, num_steps, weight_decay,
+              initial_momentum_decays, initial_rms_decays, initial_adafactor_decays,
+              momentum_decays, rms_decays, adafactor_decays):
+        self.rnn = {k: v.detach().to(F32).to(self.device) for k, v in rnn.items()}
+        self.mlp = {k: v.detach().to(F32).to(self.device) for k, v in mlp.items()}
         self.lr, self.exp_mult, self.step_mult = lr, exp_mult, step_mult
         self.weight_decay, self.num_steps = weight_decay, num_steps
         self.beta_m = decay_from_offsets(initial_momentum_decays, momentum_decays)
@@ -468,9 +499,23 @@ class VeloOracle:
         self.last_lr_mult = None
         self.last_rnn_in = None
 
+    def double_(self):
+        """fp64 evaluation, see EloCelo2Oracle.double_."""
+        self.rnn, self.mlp, self.state = _to_double(self.rnn), _to_double(self.mlp), _to_double(self.state)
+        self.beta_m, self.beta_rms, self.beta_fac = self.beta_m.double(), self.beta_rms.double(), self.beta_fac.double()
+        self.h, self.c = self.h.double(), self.c.double()
+        self.loss.decays, self.loss.means, self.loss.running_min = (
+            self.loss.decays.double(), self.loss.means.double(), self.loss.running_min.double())
+        self.dtype = torch.float64
+        return self
+
     @torch.no_grad()
     def step(self, grads: List[torch.Tensor], loss: torch.Tensor) -> None:
-        self.loss.update(loss.detach().to(F32).cpu())
+        with torch.device(self.device):
+            self._step(grads, loss)
+
+    def _step(self, grads, loss):
+        self.loss.update(loss.detach().to(getattr(self, "dtype", F32)).to(self.device))
         loss_feats = self.loss.features()
         frac = self.t / self.num_steps
         feats = []
@@ -535,35 +580,45 @@ class AdafacOracle:
                  initial_adafactor_decays=(0.9, 0.99, 0.999),
                  momentum_decays=(0.15216392, 0.14245212, 0.06812963),
                  rms_decays=(0.01079706,),
-                 adafactor_decays=(0.18621896, -0.10864615, -0.06185547)):
+                 adafactor_decays=(0.18621896, -0.10864615, -0.06185547), device="cpu"):
         self.params = params
-        self.net = {k: v.detach().to(F32).cpu() for k, v in net.items()}
+        dv = self.device = torch.device(device)
+        self.net = {k: v.detach().to(F32).to(dv) for k, v in net.items()}
         self.lr, self.exp_mult, self.step_mult, self.weight_decay = lr, exp_mult, step_mult, weight_decay
-        self.beta_m = decay_from_offsets(initial_momentum_decays, momentum_decays)
-        self.beta_rms = decay_from_offsets(initial_rms_decays, rms_decays)
-        self.beta_fac = decay_from_offsets(initial_adafactor_decays, adafactor_decays)
+        self.beta_m = decay_from_offsets(initial_momentum_decays, momentum_decays).to(dv)
+        self.beta_rms = decay_from_offsets(initial_rms_decays, rms_decays).to(dv)
+        self.beta_fac = decay_from_offsets(initial_adafactor_decays, adafactor_decays).to(dv)
         self.t = 0
         self.state = []
         for p in params:
             s = tuple(p.shape)
-            st = {"exp_avg": torch.zeros((3,) + s), "exp_avg_sq": torch.zeros(s)}
+            st = {"exp_avg": torch.zeros((3,) + s, device=dv), "exp_avg_sq": torch.zeros(s, device=dv)}
             fd = factored_dims(s)
             if fd is not None:
                 dc, dr = fd
                 r_, c_ = list(s), list(s)
                 r_[dr] = 1
                 c_[dc] = 1
-                st["exp_avg_sq_r"] = torch.zeros([3] + r_)
-                st["exp_avg_sq_c"] = torch.zeros([3] + c_)
+                st["exp_avg_sq_r"] = torch.zeros([3] + r_, device=dv)
+                st["exp_avg_sq_c"] = torch.zeros([3] + c_, device=dv)
             else:
-                st["exp_avg_sq_r"] = torch.zeros((3,) + s)      # the (3,n) vector accumulator
+                st["exp_avg_sq_r"] = torch.zeros((3,) + s, device=dv)      # the (3,n) vector accumulator
                 st["exp_avg_sq_c"] = st["exp_avg_sq_r"]
             self.state.append(st)
+
+    def double_(self):
+        """fp64 evaluation, see EloCelo2Oracle.double_."""
+        self.net, self.state = _to_double(self.net), _to_double(self.state)
+        self.beta_m, self.beta_rms, self.beta_fac = self.beta_m.double(), self.beta_rms.double(), self.beta_fac.double()
+        for st in self.state:                      # keep the 1-D alias
+            if st["exp_avg_sq_r"].dim() == st["exp_avg"].dim() and st["exp_avg_sq_r"].shape == st["exp_avg"].shape:
+                st["exp_avg_sq_c"] = st["exp_avg_sq_r"]
+        return self
 
     @torch.no_grad()
     def step(self, grads: List[Optional[torch.Tensor]]) -> None:
         self.t += 1
-        tfeat = tanh_time_embedding(self.t - 1)
+        tfeat = tanh_time_embedding(self.t - 1).to(self.device)
         sd = self.net
         for p, g, st in zip(self.params, grads, self.state):
             if g is None:

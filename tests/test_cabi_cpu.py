@@ -1,0 +1,106 @@
+"""The C-ABI library loads without a GPU and exports every symbol include/pylo_mi355.h declares;
+host-only entry points (plan sizing, argument checks, error reporting) behave as documented."""
+
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "pylo_mi355.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pylo_mi355_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from pylo_amd import _lib
+
+    lib = _lib.load()
+    names = _declared()
+    assert len(names) >= 12, names
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in the header but not exported"
+    assert lib.pylo_mi355_abi_version() == 1
+
+
+def test_struct_sizes_match_header():
+    from pylo_amd import _lib
+
+    assert _lib.ARGS_DTYPE.itemsize == 8 * 8 + 8 * 4 + 2 * 4          # PyloTensorArgs
+    assert C.sizeof(_lib.TensorShape) == 8 + 8 * 8
+    assert C.sizeof(_lib.Decays) == 7 * 4
+    assert C.sizeof(_lib.VeloNets) == 11 * 8 + 2 * 4
+    assert C.sizeof(_lib.VeloStep) == 9 * 8 + 8 * 9 * 4
+
+
+def test_workspace_sizing_and_error_paths_without_gpu():
+    from pylo_amd import _lib
+
+    lib = _lib.load()
+    n = C.c_size_t(0)
+    shapes = _lib.make_shapes([(50257, 768), (768,), (768, 2304)], [0, _lib.F_ADAM, 0])
+    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, shapes, 3, C.byref(n)) == 0
+    assert 1 << 20 < n.value < 1 << 28          # partial sums + tables: a few % of the 154 MB tensor
+    # a 1-D CELO2 tensor must be routed to AdamW by the caller
+    bad = _lib.make_shapes([(768,)], [0])
+    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, bad, 1, C.byref(n)) != 0
+    assert b"PYLO_F_ADAM" in lib.pylo_mi355_last_error()
+    # >2-D tensors are fine for VeLO / AdafacLO, rejected (for now) on the CELO2 MLP path
+    nd = _lib.make_shapes([(768, 3, 16, 16)], [0])
+    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_VELO, nd, 1, C.byref(n)) == 0
+    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_ADAFAC, nd, 1, C.byref(n)) == 0
+    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, nd, 1, C.byref(n)) != 0
+    # too large
+    huge = _lib.make_shapes([(1 << 16, 1 << 16)], [0])
+    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_VELO, huge, 1, C.byref(n)) != 0
+    assert b"2^31" in lib.pylo_mi355_last_error()
+    assert lib.pylo_mi355_plan_workspace_bytes(7, shapes, 3, C.byref(n)) != 0
+    assert lib.pylo_mi355_plan_destroy(None) == 0
+
+
+def test_optimizers_fail_loudly_without_gpu():
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("this check is for GPU-less hosts")
+    from pylo_amd import AdafacLO_CUDA, ELO_CELO2_CUDA, VeLO_CUDA
+    from pylo_amd.models import CELO2MLP, MetaMLP, VeLOMLP, VeLORNN
+
+    p = [torch.nn.Parameter(torch.zeros(4, 4))]
+    with pytest.raises(RuntimeError, match="requires a GPU"):
+        ELO_CELO2_CUDA(p, network=CELO2MLP(), hf_key=None)
+    with pytest.raises(RuntimeError, match="requires a GPU"):
+        VeLO_CUDA(p, rnn=VeLORNN(lstm_hidden_size=64, param_inits=8), mlp=VeLOMLP(param_inits=8))
+    with pytest.raises(RuntimeError, match="requires a GPU"):
+        AdafacLO_CUDA(p, network=MetaMLP(39, 32, 1))
+
+
+def test_weight_containers_round_trip_through_the_reference_file_format(tmp_path):
+    """config.json + model.safetensors written by save_pretrained load back bit-identically, with
+    the reference's parameter names."""
+    import torch
+
+    from pylo_amd.models import CELO2MLP, MetaMLP, VeLOMLP, VeLORNN
+
+    torch.manual_seed(0)
+    cases = [(CELO2MLP, {}), (MetaMLP, dict(input_size=39, hidden_size=32, hidden_layers=1)),
+             (VeLOMLP, dict(param_inits=8)), (VeLORNN, dict(lstm_hidden_size=64, param_inits=8))]
+    for cls, kw in cases:
+        m = cls(**kw)
+        d = tmp_path / cls.__name__
+        m.save_pretrained(str(d))
+        assert (d / "config.json").exists() and (d / "model.safetensors").exists()
+        m2 = cls.from_pretrained(str(d))
+        for (k1, v1), (k2, v2) in zip(m.state_dict().items(), m2.state_dict().items()):
+            assert k1 == k2 and torch.equal(v1, v2), (cls.__name__, k1)
+    keys = set(CELO2MLP().state_dict().keys())
+    assert {"w0.0", "w0.13", "b0", "dense_w.0", "dense_b.1"} <= keys
+    assert "network.linear_0.weight" in MetaMLP(39, 32, 1).state_dict()
+    assert {"input_weights_", "hidden_weights_.0", "output_bias"} <= set(VeLOMLP(param_inits=4).state_dict())
+    assert {"mix_layer1.weight", "lstm.linear.bias", "lstm_init_state.1", "step_size.weight"} <= \
+        set(VeLORNN(lstm_hidden_size=64, param_inits=4).state_dict())

@@ -187,9 +187,10 @@ __device__ __forceinline__ void adafac_apply_fac(const TDesc& d, const PyloTenso
       x.i0 = (int)(u / (unsigned)d.C0);
       x.i1 = (int)(u - (unsigned)x.i0 * (unsigned)d.C0);
       const float4 fa = load_f4(fac_tab + d.fac_off[0] + (size_t)x.i0 * 4);
-      x.rfcf[0][0] = fa.x * fac_tab[d.fac_off[1] + x.i1];
-      x.rfcf[0][1] = fa.y * fac_tab[d.fac_off[1] + (size_t)d.pitch[1] + x.i1];
-      x.rfcf[0][2] = fa.z * fac_tab[d.fac_off[1] + 2 * (size_t)d.pitch[1] + x.i1];
+      const float4 fb = load_f4(fac_tab + d.fac_off[1] + (size_t)x.i1 * 4);
+      x.rfcf[0][0] = fa.x * fb.x;
+      x.rfcf[0][1] = fa.y * fb.y;
+      x.rfcf[0][2] = fa.z * fb.z;
     }
     float h[1][kAH];
     lo_terms<1, ND, kAH>(d, x, term_tab, h);

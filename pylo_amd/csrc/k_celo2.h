@@ -105,16 +105,101 @@ __device__ __forceinline__ void load_elems(const TDesc& d, const PyloTensorArgs&
   x.i0 = (int)(u / (unsigned)d.C0);
   x.i1 = (int)(u - (unsigned)x.i0 * (unsigned)d.C0);
   const float4 fa = load_f4(f0 + (size_t)x.i0 * 4);
-  float fb[3][V];
-#pragma unroll
-  for (int k = 0; k < 3; ++k) load_vec<V>(f1 + (size_t)k * d.pitch[1] + x.i1, fb[k]);
 #pragma unroll
   for (int v = 0; v < V; ++v) {
+    const float4 fb = load_f4(f1 + (size_t)(x.i1 + v) * 4);
     x.g[v] = clampf(x.g[v] * scale, a.clip_val);
     x.m[v][0] = m0[v]; x.m[v][1] = m1[v]; x.m[v][2] = m2[v];
-    x.rfcf[v][0] = fa.x * fb[0][v];
-    x.rfcf[v][1] = fa.y * fb[1][v];
-    x.rfcf[v][2] = fa.z * fb[2][v];
+    x.rfcf[v][0] = fa.x * fb.x;
+    x.rfcf[v][1] = fa.y * fb.y;
+    x.rfcf[v][2] = fa.z * fb.z;
+  }
+}
+
+// Position of a lane inside one chunk of consecutive elements of a 2-D tensor: element
+// offset from the chunk's first element, row and column.  Advancing by a whole block stride costs
+// three or four instructions (no division); every access is "uniform base + 32-bit lane offset".
+// V = elements per lane and access, VC = the tensor's vector width (which fixes the chunk size).
+template <int V, int VC = V>
+struct Cursor {
+  static constexpr int kChunkElems = kThreads * VC * kElemIters;
+  static constexpr int kIters = kElemIters * VC / V;
+  unsigned off, i0, i1;  // lane's vector: element offset in the chunk, row, column
+  unsigned lim;          // elements of the chunk that exist
+  unsigned C0, sq, sr;   // row length; block stride = sq rows + sr columns
+  unsigned c_i0, c_i1;   // coordinates of the chunk's first element (always valid)
+
+  __device__ __forceinline__ Cursor(const TDesc& d, long long base) {
+    off = threadIdx.x * V;
+    const long long left = d.n - base;
+    lim = left < (long long)kChunkElems ? (unsigned)left : (unsigned)kChunkElems;
+    C0 = (unsigned)d.C0;
+    const unsigned ub = (unsigned)base;  // n < 2^31
+    c_i0 = ub / C0;
+    c_i1 = ub - c_i0 * C0;
+    const unsigned q = off / C0;
+    i0 = c_i0 + q;
+    i1 = c_i1 + (off - q * C0);
+    if (i1 >= C0) { i1 -= C0; ++i0; }
+    constexpr unsigned step = kThreads * V;
+    sq = step / C0;
+    sr = step - sq * C0;
+  }
+  __device__ __forceinline__ bool live() const { return off < lim; }
+  __device__ __forceinline__ void advance() {
+    off += kThreads * V;
+    i0 += sq;
+    i1 += sr;
+    if (i1 >= C0) { i1 -= C0; ++i0; }
+  }
+};
+
+// Base pointers of one chunk (all wave-uniform).
+struct ChunkPtrs {
+  const float *g, *p;
+  float *m0, *m1, *m2, *rms, *out;
+  __device__ __forceinline__ ChunkPtrs(const TDesc& d, const PyloTensorArgs& a, long long base) {
+    g = a.grad + base; p = a.param + base;
+    m0 = a.mom + base; m1 = a.mom + d.n + base; m2 = a.mom + 2 * d.n + base;
+    rms = a.rms + base; out = a.step_out + base;
+  }
+};
+
+// eight consecutive floats of row i of a table with eight floats per row
+__device__ __forceinline__ void load_row8(const float* tab, unsigned i, float (&t)[8]) {
+  float lo[4], hi[4];
+  load_vec_o<4>(tab, i * 32u, lo);
+  load_vec_o<4>(tab + 4, i * 32u, hi);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) { t[j] = lo[j]; t[4 + j] = hi[j]; }
+}
+
+// load_elems through a cursor; (off, i0, i1) are the lane's (possibly substituted) coordinates.
+template <int V>
+__device__ __forceinline__ void load_elems_at(const TDesc& d, const PyloTensorArgs& a, const ChunkPtrs& cp,
+                                              unsigned off, unsigned i0, unsigned i1, float scale,
+                                              const float* f0, const float* f1, ElemIn<V>& x) {
+  float m0[V], m1[V], m2[V];
+  const unsigned bo = off * 4u;
+  load_vec_o<V>(cp.g, bo, x.g);
+  load_vec_o<V>(cp.p, bo, x.p);
+  load_vec_o<V>(cp.m0, bo, m0);
+  load_vec_o<V>(cp.m1, bo, m1);
+  load_vec_o<V>(cp.m2, bo, m2);
+  load_vec_o<V>(cp.rms, bo, x.rms);
+  x.i0 = (int)i0;
+  x.i1 = (int)i1;
+  float fa[4];
+  load_vec_o<4>(f0, i0 * 16u, fa);
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    float fb[4];
+    load_vec_o<4>(f1 + v * 4, i1 * 16u, fb);
+    x.g[v] = clampf(x.g[v] * scale, a.clip_val);
+    x.m[v][0] = m0[v]; x.m[v][1] = m1[v]; x.m[v][2] = m2[v];
+    x.rfcf[v][0] = fa[0] * fb[0];
+    x.rfcf[v][1] = fa[1] * fb[1];
+    x.rfcf[v][2] = fa[2] * fb[2];
   }
 }
 
@@ -123,12 +208,13 @@ __device__ __forceinline__ void celo2_stats_chunk(const TDesc& d, const PyloTens
                                                   float scale, const EmaConsts& e, const float* f0,
                                                   const float* f1, float (&acc)[kNStat]) {
   const long long base = (long long)chunk * (kThreads * V * kElemIters);
+  Cursor<V> cur(d, base);
+  const ChunkPtrs cp(d, a, base);
 #pragma unroll 2
-  for (int it = 0; it < kElemIters; ++it) {
-    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
-    if (idx >= d.n) break;
+  for (int it = 0; it < kElemIters; ++it, cur.advance()) {
+    if (!cur.live()) break;
     ElemIn<V> x;
-    load_elems<V>(d, a, idx, scale, f0, f1, x);
+    load_elems_at<V>(d, a, cp, cur.off, cur.i0, cur.i1, scale, f0, f1, x);
 #pragma unroll
     for (int v = 0; v < V; ++v) {
       ema_update(e, x.g[v], x.m[v], x.rms[v]);
@@ -225,8 +311,8 @@ __global__ __launch_bounds__(kFoldThreads) void k_celo2_fold(const TDesc* __rest
   }
   for (int i = threadIdx.x; i < 64; i += kFoldThreads) w[kC2WH + i] = w_h[i];
   for (int i = threadIdx.x; i < 8; i += kFoldThreads) w[kC2BH + i] = b_h[i];
-  for (int i = threadIdx.x; i < 16; i += kFoldThreads) w[kC2WO + i] = w_out[(i / 2) * 3 + (i % 2)];
-  for (int i = threadIdx.x; i < 2; i += kFoldThreads) w[kC2BO + i] = b_out[i];
+  for (int i = threadIdx.x; i < 32; i += kFoldThreads) w[kC2WO + i] = (i % 4) < 2 ? w_out[(i / 4) * 3 + (i % 4)] : 0.0f;
+  for (int i = threadIdx.x; i < 4; i += kFoldThreads) w[kC2BO + i] = i < 2 ? b_out[i] : 0.0f;
 }
 
 template <int V>
@@ -235,24 +321,24 @@ __device__ __forceinline__ void celo2_apply_chunk(const TDesc& d, const PyloTens
                                                   const float* f1, const float* t0, const float* t1,
                                                   const float* wbase) {
   const long long base = (long long)chunk * (kThreads * V * kElemIters);
-  const long long n = d.n;
   const bool use_exp = a.exp_mult != 0.0f;
-  for (int it = 0; it < kElemIters; ++it) {
-    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
-    if (idx >= n) break;
+  Cursor<V> cur(d, base);
+  const ChunkPtrs cp(d, a, base);
+  for (int it = 0; it < kElemIters; ++it, cur.advance()) {
+    if (!cur.live()) break;
     ElemIn<V> x;
-    load_elems<V>(d, a, idx, scale, f0, f1, x);
+    load_elems_at<V>(d, a, cp, cur.off, cur.i0, cur.i1, scale, f0, f1, x);
     float f[V][kNStat], h[V][8];
     float m0[V], m1[V], m2[V];
     {
-      const float4 a0 = load_f4(t0 + (size_t)x.i0 * 8), a1 = load_f4(t0 + (size_t)x.i0 * 8 + 4);
-      const float ta[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+      float ta[8];
+      load_row8(t0, cur.i0, ta);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        float tb[V];
-        load_vec<V>(t1 + (size_t)j * d.pitch[1] + x.i1, tb);
+      for (int v = 0; v < V; ++v) {
+        float tb[8];
+        load_row8(t1 + v * 8, cur.i1, tb);
 #pragma unroll
-        for (int v = 0; v < V; ++v) h[v][j] = ta[j] + tb[v];
+        for (int j = 0; j < 8; ++j) h[v][j] = ta[j] + tb[j];
       }
     }
 #pragma unroll
@@ -261,10 +347,10 @@ __device__ __forceinline__ void celo2_apply_chunk(const TDesc& d, const PyloTens
       m0[v] = x.m[v][0]; m1[v] = x.m[v][1]; m2[v] = x.m[v][2];
       lo_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.rfcf[v], 1e-8f, f[v]);
     }
-    store_vec<V>(a.mom + idx, m0);
-    store_vec<V>(a.mom + n + idx, m1);
-    store_vec<V>(a.mom + 2 * n + idx, m2);
-    store_vec<V>(a.rms + idx, x.rms);
+    store_vec_o<V>(cp.m0, cur.off * 4u, m0);
+    store_vec_o<V>(cp.m1, cur.off * 4u, m1);
+    store_vec_o<V>(cp.m2, cur.off * 4u, m2);
+    store_vec_o<V>(cp.rms, cur.off * 4u, x.rms);
     // The weights are wave-uniform: they are fetched through the scalar cache into SGPRs one input
     // row at a time and shared by the P elements processed together (channel-outer loop order).
     constexpr int P = V >= 2 ? 2 : 1;
@@ -306,18 +392,124 @@ __device__ __forceinline__ void celo2_apply_chunk(const TDesc& d, const PyloTens
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
           const float hk = fmaxf(h1[q][k], 0.0f);
-          o0 = fmaf(hk, w[kC2WO + k * 2 + 0], o0);
-          if (use_exp) o1 = fmaf(hk, w[kC2WO + k * 2 + 1], o1);
+          o0 = fmaf(hk, w[kC2WO + k * 4 + 0], o0);
+          o1 = fmaf(hk, w[kC2WO + k * 4 + 1], o1);
         }
         out[v0 + q] = use_exp ? o0 * expf(o1 * a.exp_mult) : o0;
       }
     }
-    store_vec<V>(a.step_out + idx, out);
+    store_vec_o<V>(cp.out, cur.off * 4u, out);
+  }
+}
+
+#ifndef PYLO_MFMA_V
+#define PYLO_MFMA_V 2
+#endif
+#ifndef PYLO_APPLY_WAVES
+#define PYLO_APPLY_WAVES 4
+#endif
+constexpr int kMfmaV = PYLO_MFMA_V;   // elements per lane and iteration on the matrix-pipe path
+
+// The same pass with the three layers on the matrix pipe (128-bit-aligned tensors only).  The folded
+// weight block is 63 groups of four consecutive floats; lane l of register r holds float r*64 + l,
+// so group v sits in lanes 4*(v%16).. of register v/16 and is selected with abid = v % 16.  Four
+// VGPRs hold every weight.  Biases enter as a rank-1 update with the constant 1.
+template <int V>
+__device__ __forceinline__ void celo2_apply_chunk_mfma(const TDesc& d, const PyloTensorArgs& a, int chunk,
+                                                       float scale, const EmaConsts& e, const float* f0,
+                                                       const float* f1, const float* t0, const float* t1,
+                                                       const float* wbase) {
+  const long long base = (long long)chunk * (kThreads * 4 * kElemIters);   // chunks are sized for vec == 4
+  const bool use_exp = a.exp_mult != 0.0f;
+  const float exp_scale = a.exp_mult * 1.44269504088896341f;
+  const int lane = threadIdx.x & 63;
+  float wreg[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) wreg[r] = *(const gfloat*)(wbase + r * 64 + lane);
+  constexpr int gWH = kC2WH / 4, gBH = kC2BH / 4, gWO = kC2WO / 4, gBO = kC2BO / 4;
+  const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
+  Cursor<V, 4> cur(d, base);
+  const ChunkPtrs cp(d, a, base);
+  for (int it = 0; it < Cursor<V, 4>::kIters; ++it, cur.advance()) {
+    // no early exit: every lane of the wave must reach the matrix instructions; lanes past the end
+    // work on the chunk's first element and store nothing
+    const bool live = cur.live();
+    const unsigned off = live ? cur.off : 0u, i0 = live ? cur.i0 : cur.c_i0, i1 = live ? cur.i1 : cur.c_i1;
+    ElemIn<V> x;
+    load_elems_at<V>(d, a, cp, off, i0, i1, scale, f0, f1, x);
+    v4f ha[V], hb[V];
+    {
+      float ta[8];
+      load_row8(t0, i0, ta);
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        float tb[8];
+        load_row8(t1 + v * 8, i1, tb);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { ha[v][j] = ta[j] + tb[j]; hb[v][j] = ta[4 + j] + tb[4 + j]; }
+      }
+    }
+    float f[V][kNStat], m0[V], m1[V], m2[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      ema_update(e, x.g[v], x.m[v], x.rms[v]);
+      m0[v] = x.m[v][0]; m1[v] = x.m[v][1]; m2[v] = x.m[v][2];
+      lo_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.rfcf[v], 1e-8f, f[v]);
+    }
+    if (live) {
+      store_vec_o<V>(cp.m0, off * 4u, m0);
+      store_vec_o<V>(cp.m1, off * 4u, m1);
+      store_vec_o<V>(cp.m2, off * 4u, m2);
+      store_vec_o<V>(cp.rms, off * 4u, x.rms);
+    }
+    // layer 1: 18 rank-1 updates per half (hidden units 0-3 / 4-7)
+#pragma unroll
+    for (int c = 0; c < kNStat; ++c) {
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        ha[v] = mfma_w4(wreg[(2 * c) / 16], f[v][c], ha[v], (2 * c) % 16);
+        hb[v] = mfma_w4(wreg[(2 * c + 1) / 16], f[v][c], hb[v], (2 * c + 1) % 16);
+      }
+    }
+    // layer 2: bias, then 8 rank-1 updates per half
+    v4f ga[V], gb[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      ga[v] = mfma_w4(wreg[gBH / 16], 1.0f, zero, gBH % 16);
+      gb[v] = mfma_w4(wreg[(gBH + 1) / 16], 1.0f, zero, (gBH + 1) % 16);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        const float hk = relu(k < 4 ? ha[v][k] : hb[v][k - 4]);
+        ga[v] = mfma_w4(wreg[(gWH + 2 * k) / 16], hk, ga[v], (gWH + 2 * k) % 16);
+        gb[v] = mfma_w4(wreg[(gWH + 2 * k + 1) / 16], hk, gb[v], (gWH + 2 * k + 1) % 16);
+      }
+    }
+    // layer 3: the two outputs sit in elements 0 and 1 of the accumulator
+    v4f o[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) o[v] = mfma_w4(wreg[gBO / 16], 1.0f, zero, gBO % 16);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        const float hk = relu(k < 4 ? ga[v][k] : gb[v][k - 4]);
+        o[v] = mfma_w4(wreg[(gWO + k) / 16], hk, o[v], (gWO + k) % 16);
+      }
+    }
+    float out[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v)
+      out[v] = use_exp ? o[v][0] * __builtin_amdgcn_exp2f(o[v][1] * exp_scale) : o[v][0];
+    if (live) store_vec_o<V>(cp.out, off * 4u, out);
   }
 }
 
 // Apply pass: accumulators advanced and written, features, MLP, raw step.
-__global__ __launch_bounds__(kThreads) void k_celo2_apply(const TDesc* __restrict__ descs,
+template <bool MFMA>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PYLO_APPLY_WAVES))) void k_celo2_apply(const TDesc* __restrict__ descs,
                                                           const PyloTensorArgs* __restrict__ dyn,
                                                           const Item* __restrict__ items,
                                                           const float* __restrict__ fac_tab,
@@ -332,7 +524,10 @@ __global__ __launch_bounds__(kThreads) void k_celo2_apply(const TDesc* __restric
   const float scale = clip_scale(gl->gnorm, a.clip_norm);
   const EmaConsts e = make_ema(dec);
   const float* w = wfold + (size_t)d.fac_slot * kC2Fold;
-  if (d.vec == 4)
+  if (MFMA && d.vec == 4)
+    celo2_apply_chunk_mfma<kMfmaV>(d, a, it.a, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
+                                   term_tab + d.term_off[0], term_tab + d.term_off[1], w);
+  else if (d.vec == 4)
     celo2_apply_chunk<4>(d, a, it.a, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
                          term_tab + d.term_off[0], term_tab + d.term_off[1], w);
   else

@@ -141,28 +141,37 @@ __global__ __launch_bounds__(kThreads) void k_gnorm(const double* __restrict__ g
 }
 
 // =============================================================================================
-// Sums of g^2 over one dim of an N-D tensor (any two factored dims): one thread per entry of the
-// statistics vector, walking the removed dim.  Small tensors only (conv kernels, cls tokens); the
-// gradient is clamped directly (no global-norm scale on this path).
+// Sums of g^2 over one dim of an N-D tensor (any two factored dims): a block takes 64 entries of
+// the statistics vector and 64 positions of the removed dim and writes one partial row; k_v0a adds
+// the partial rows up.  Small tensors only (conv kernels, cls tokens); the gradient is clamped
+// directly (no global-norm scale on this path).
 // =============================================================================================
 __global__ __launch_bounds__(kThreads) void k_p0_nd(const TDesc* __restrict__ descs,
                                                     const PyloTensorArgs* __restrict__ dyn,
                                                     const Item* __restrict__ items, float* __restrict__ part) {
+  __shared__ float lds[kWaves][kV0aEnt];
   const Item it = items[blockIdx.x];
   const TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
   const int w = it.b;
-  const int i = it.a * kThreads + threadIdx.x;
-  if (i >= d.len[w]) return;
+  const int e = threadIdx.x & 63, grp = threadIdx.x >> 6;
+  const int i = it.a * kV0aEnt + e;
   const int X = d.nd_size[w], sX = d.nd_stride[w];
-  const long long base = (long long)(i / sX) * X * sX + (i % sX);
-  double s = 0.0;
-  for (int x = 0; x < X; ++x) {
-    const float g = clampf(*(const gfloat*)(a.grad + base + (long long)x * sX), a.clip_val);
-    s += (double)(g * g);
+  float s = 0.0f;
+  if (i < d.len[w]) {
+    const long long base = (long long)(i / sX) * X * sX + (i % sX);
+    const int x0 = it.c * kNdX + grp * (kNdX / kWaves);
+    const int x1 = min(X, x0 + kNdX / kWaves);
+    for (int x = x0; x < x1; ++x) {
+      const float g = clampf(*(const gfloat*)(a.grad + base + (long long)x * sX), a.clip_val);
+      s = fmaf(g, g, s);
+    }
   }
-  part[d.part_off[w] + i] = (float)s;
+  lds[grp][e] = s;
+  __syncthreads();
+  if (grp == 0 && i < d.len[w])
+    part[d.part_off[w] + (size_t)it.c * d.len[w] + i] = ((lds[0][e] + lds[1][e]) + lds[2][e]) + lds[3][e];
 }
 
 // =============================================================================================
@@ -226,13 +235,13 @@ __global__ __launch_bounds__(kThreads) void k_v0a(const TDesc* __restrict__ desc
 
 // Where entry i of vector `which` of tensor d lives in the factor / term tables.
 __device__ __forceinline__ size_t fac_index(const TDesc& d, int which, int k, int i) {
-  return (d.mode == kModeFac2D && which == 0) ? (size_t)d.fac_off[0] + (size_t)i * 4 + k
-                                              : (size_t)d.fac_off[which] + (size_t)k * d.pitch[which] + i;
+  return d.mode == kModeFac2D ? (size_t)d.fac_off[which] + (size_t)i * 4 + k
+                              : (size_t)d.fac_off[which] + (size_t)k * d.pitch[which] + i;
 }
 template <int H>
 __device__ __forceinline__ size_t term_index(const TDesc& d, int which, int j, int i) {
-  return (d.mode == kModeFac2D && which == 0) ? (size_t)d.term_off[0] + (size_t)i * H + j
-                                              : (size_t)d.term_off[which] + (size_t)j * d.pitch[which] + i;
+  return d.mode == kModeFac2D ? (size_t)d.term_off[which] + (size_t)i * H + j
+                              : (size_t)d.term_off[which] + (size_t)j * d.pitch[which] + i;
 }
 
 // Row_factor / col_factor of one entry, and the two normalised broadcast features it carries

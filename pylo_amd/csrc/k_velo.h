@@ -56,15 +56,18 @@ template <int V, bool ND, int H>
 __device__ __forceinline__ void lo_terms(const TDesc& d, const ElemIn<V>& x, const float* __restrict__ term_tab,
                                          float (&h)[V][H]) {
   if constexpr (!ND) {
+    static_assert(H % 4 == 0, "term tables are read four floats at a time");
     const float* t0 = term_tab + d.term_off[0] + (size_t)x.i0 * H;
-    const float* t1 = term_tab + d.term_off[1];
+    const float* t1 = term_tab + d.term_off[1] + (size_t)x.i1 * H;
 #pragma unroll
-    for (int j = 0; j < H; ++j) {
-      float tb[V];
-      load_vec<V>(t1 + (size_t)j * d.pitch[1] + x.i1, tb);
-      const float ta = *(const gfloat*)(t0 + j);
+    for (int q = 0; q < H / 4; ++q) {
+      const float4 ta = load_f4(t0 + q * 4);
 #pragma unroll
-      for (int v = 0; v < V; ++v) h[v][j] = ta + tb[v];
+      for (int v = 0; v < V; ++v) {
+        const float4 tb = load_f4(t1 + v * H + q * 4);
+        h[v][q * 4 + 0] = ta.x + tb.x; h[v][q * 4 + 1] = ta.y + tb.y;
+        h[v][q * 4 + 2] = ta.z + tb.z; h[v][q * 4 + 3] = ta.w + tb.w;
+      }
     }
   } else {
 #pragma unroll
@@ -285,13 +288,13 @@ __device__ __forceinline__ float clip_log_abs10(double v) {
   return 0.5f * fminf(fmaxf(logf(1e-8f + fabsf(x * 10.0f)), -5.0f), 5.0f);
 }
 
-__global__ __launch_bounds__(kThreads) void k_lo_reduce(const TDesc* __restrict__ descs,
+__global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restrict__ descs,
                                                         const PyloTensorArgs* __restrict__ dyn, int T,
                                                         const double* __restrict__ stats_part,
                                                         double* __restrict__ totals,
                                                         const float* __restrict__ lossfeat, VeloStep st,
                                                         float* __restrict__ xfeat) {
-  constexpr int G = 6;  // 6 groups x 40 sums = 240 threads
+  constexpr int G = kFoldThreads / kStatW;  // 25 groups x 40 sums = 1000 threads
   __shared__ double part[G][kStatW];
   __shared__ double tot[kStatW];
   const int t = blockIdx.x;
@@ -384,42 +387,57 @@ __global__ __launch_bounds__(kThreads) void k_velo_mix(const float* __restrict__
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
 
 // gates = [x', h] W^T + b in chunks i, g, f, o;  c = sig(f+1) c + sig(i) tanh(g);  h = sig(o) tanh(c)
-__global__ __launch_bounds__(128) void k_velo_gates(const float* __restrict__ xT, int T, int Tpad, int H,
-                                                    const float* __restrict__ wt /*(2H, 4H)*/,
-                                                    const float* __restrict__ b /*4H*/,
-                                                    float* __restrict__ h_state, float* __restrict__ c_state) {
-  const int u = blockIdx.y * 128 + threadIdx.x;
-  if (u >= H) return;
+// Block = 32 hidden units x 8 slices of the 2H-long contraction, 8 tensors; the slices are added
+// in LDS in a fixed order.
+constexpr int kGateU = 32, kGateS = 8;
+__global__ __launch_bounds__(kThreads) void k_velo_gates(const float* __restrict__ xT, int T, int Tpad, int H,
+                                                         const float* __restrict__ wt /*(2H, 4H)*/,
+                                                         const float* __restrict__ b /*4H*/,
+                                                         float* __restrict__ h_state, float* __restrict__ c_state) {
+  __shared__ float red[kGateS][4 * kGateBT][kGateU];
+  const int ul = threadIdx.x % kGateU, sl = threadIdx.x / kGateU;
+  const int u = blockIdx.y * kGateU + ul;
   const int r0 = blockIdx.x * kGateBT;
   float acc[4][kGateBT];
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const float bias = b[g * H + u];
+  for (int g = 0; g < 4; ++g)
 #pragma unroll
-    for (int t = 0; t < kGateBT; ++t) acc[g][t] = bias;
-  }
+    for (int t = 0; t < kGateBT; ++t) acc[g][t] = 0.0f;
   const int K2 = 2 * H;
-  for (int k = 0; k < K2; ++k) {
-    float w[4];
+  if (u < H) {
+#pragma unroll 2
+    for (int k = sl; k < K2; k += kGateS) {
+      float w[4];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) w[g] = wt[(size_t)k * 4 * H + g * H + u];
-    const float* xr = xT + (size_t)k * Tpad + r0;
+      for (int g = 0; g < 4; ++g) w[g] = wt[(size_t)k * 4 * H + g * H + u];
+      const float4 xa = load_f4(xT + (size_t)k * Tpad + r0), xb = load_f4(xT + (size_t)k * Tpad + r0 + 4);
+      const float xv[kGateBT] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
 #pragma unroll
-    for (int t = 0; t < kGateBT; ++t) {
-      const float xv = xr[t];
+      for (int t = 0; t < kGateBT; ++t)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) acc[g][t] = fmaf(xv, w[g], acc[g][t]);
+        for (int g = 0; g < 4; ++g) acc[g][t] = fmaf(xv[t], w[g], acc[g][t]);
     }
   }
 #pragma unroll
-  for (int t = 0; t < kGateBT; ++t) {
-    const int r = r0 + t;
-    if (r < T) {
-      const float c_old = c_state[(size_t)r * H + u];
-      const float c_new = sigmoidf_(acc[2][t] + 1.0f) * c_old + sigmoidf_(acc[0][t]) * tanhf(acc[1][t]);
-      c_state[(size_t)r * H + u] = c_new;
-      h_state[(size_t)r * H + u] = sigmoidf_(acc[3][t]) * tanhf(c_new);
+  for (int g = 0; g < 4; ++g)
+#pragma unroll
+    for (int t = 0; t < kGateBT; ++t) red[sl][g * kGateBT + t][ul] = acc[g][t];
+  __syncthreads();
+  // thread (ul, sl) finishes tensor t = sl of unit ul
+  const int t = sl, r = r0 + t;
+  if (u < H && r < T) {
+    float gate[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      float s = b[g * H + u];
+#pragma unroll
+      for (int q = 0; q < kGateS; ++q) s += red[q][g * kGateBT + t][ul];
+      gate[g] = s;
     }
+    const float c_old = c_state[(size_t)r * H + u];
+    const float c_new = sigmoidf_(gate[2] + 1.0f) * c_old + sigmoidf_(gate[0]) * tanhf(gate[1]);
+    c_state[(size_t)r * H + u] = c_new;
+    h_state[(size_t)r * H + u] = sigmoidf_(gate[3]) * tanhf(c_new);
   }
 }
 

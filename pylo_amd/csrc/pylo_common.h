@@ -21,6 +21,7 @@ constexpr int kV0aEnt = 64;     // vector entries per k_v0a block
 constexpr int kV0bEnt = 1024;   // vector entries per k_v0b block
 constexpr int kNV0 = 9;         // partial sums per k_v0a block
 constexpr int kFoldThreads = 1024;
+constexpr int kNdX = 64;        // elements of the summed dim one k_p0_nd block covers (one partial row)
 
 // Per-element channels, as indices into the reference's 30-channel order
 // (pylo/csrc/celo2_kernel.cu:86-124): g, clip(g), p, m0..2, rms, m_k*rs, rs, g*rf_k*cf_k, g*rs,
@@ -28,7 +29,8 @@ constexpr int kFoldThreads = 1024;
 __host__ __device__ constexpr int stat_channel(int c) { return c < 15 ? c : c + 12; }
 
 // Folded per-tensor MLP weights for CELO2 (floats): w1[18][8] | w_h[8][8] | b_h[8] | w_out[8][2] | b_out[2]
-constexpr int kC2W1 = 0, kC2WH = 144, kC2BH = 208, kC2WO = 216, kC2BO = 232, kC2Fold = 240;
+// folded per-tensor weights: W1 (18,8) | WH (8,8) | bH 8 | WO (8,4: two outputs, two zeros) | bO 4 (same padding)
+constexpr int kC2W1 = 0, kC2WH = 144, kC2BH = 208, kC2WO = 216, kC2BO = 248, kC2Fold = 256;
 
 // ---- plan tables (device copies live in the caller's workspace) -----------------------------
 // kModeFlat   no factored statistics, no MLP: CELO2 tensors routed to AdamW
@@ -49,7 +51,7 @@ struct TDesc {
   int len[2];       // entries of vector 0 / 1
   int sumlen[2];    // elements summed into one entry
   int npart[2];     // partial rows to add up per entry (2-D: column blocks / strips; N-D: 1)
-  int pitch[2];     // row pitch of the SoA tables of vector 0 / 1 (len rounded up to 4)
+  int pitch[2];     // row pitch of the SoA tables of vector 0 / 1 (len rounded up to 4); 2-D tensors use [index][k] tables
   int nd_size[2];   // N-D: size and stride of the dim removed from vector 0 / 1;
   int nd_stride[2]; //      entry = (idx / (size*stride)) * stride + idx % stride
   int rcm_size;     // N-D: size of the 2nd-largest dim and its stride inside the row vector; row_col_mean
@@ -66,9 +68,9 @@ struct TDesc {
 
 struct Item {
   int tensor;
-  int a;  // P0: strip (or flat chunk); element kernels: chunk; V0 / N-D sums: chunk
+  int a;  // P0: strip (or flat chunk); element kernels: chunk; V0 / N-D sums: chunk of entries
   int b;  // P0: column block; V0 / N-D sums: vector 0 or 1
-  int pad_;
+  int c;  // N-D sums: chunk of the summed dim (= partial row)
 };
 
 // Width of one row of statistics partials (doubles): sum of squares per feature channel in the
@@ -123,12 +125,17 @@ __device__ __forceinline__ float rsq(float x) { return __builtin_amdgcn_rsqf(x);
 typedef __attribute__((address_space(1))) float gfloat;
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) v4f gv4f;
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(1))) v2f gv2f;
 
 template <int V>
 __device__ __forceinline__ void load_vec(const float* p, float (&x)[V]) {
   if constexpr (V == 4) {
     const v4f t = *(const gv4f*)(p);
     x[0] = t.x; x[1] = t.y; x[2] = t.z; x[3] = t.w;
+  } else if constexpr (V == 2) {
+    const v2f t = *(const gv2f*)(p);
+    x[0] = t.x; x[1] = t.y;
   } else {
     x[0] = *(const gfloat*)(p);
   }
@@ -140,8 +147,46 @@ __device__ __forceinline__ void store_vec(float* p, const float (&x)[V]) {
     v4f t;
     t.x = x[0]; t.y = x[1]; t.z = x[2]; t.w = x[3];
     *(gv4f*)(p) = t;
+  } else if constexpr (V == 2) {
+    v2f t;
+    t.x = x[0]; t.y = x[1];
+    *(gv2f*)(p) = t;
   } else {
     *(gfloat*)(p) = x[0];
+  }
+}
+
+// The same through a wave-uniform base and a 32-bit byte offset per lane: one scalar base register
+// pair plus one offset VGPR per access instead of a 64-bit address per lane.
+typedef __attribute__((address_space(1))) char gchar;
+
+template <int V>
+__device__ __forceinline__ void load_vec_o(const float* sbase, unsigned byte_off, float (&x)[V]) {
+  const gchar* p = (const gchar*)sbase + byte_off;
+  if constexpr (V == 4) {
+    const v4f t = *(const gv4f*)p;
+    x[0] = t.x; x[1] = t.y; x[2] = t.z; x[3] = t.w;
+  } else if constexpr (V == 2) {
+    const v2f t = *(const gv2f*)p;
+    x[0] = t.x; x[1] = t.y;
+  } else {
+    x[0] = *(const gfloat*)p;
+  }
+}
+
+template <int V>
+__device__ __forceinline__ void store_vec_o(float* sbase, unsigned byte_off, const float (&x)[V]) {
+  gchar* p = (gchar*)sbase + byte_off;
+  if constexpr (V == 4) {
+    v4f t;
+    t.x = x[0]; t.y = x[1]; t.z = x[2]; t.w = x[3];
+    *(gv4f*)p = t;
+  } else if constexpr (V == 2) {
+    v2f t;
+    t.x = x[0]; t.y = x[1];
+    *(gv2f*)p = t;
+  } else {
+    *(gfloat*)p = x[0];
   }
 }
 
@@ -155,6 +200,36 @@ __device__ __forceinline__ void store_f4(float* p, float a, float b, float c, fl
   t.x = a; t.y = b; t.z = c; t.w = d;
   *(gv4f*)(p) = t;
 }
+
+// D(4x4, 16 blocks) += A(4x1) B(1x4) per block, fp32.  Lane l = 4*block + j holds B[j] (src1) and the
+// column D[0..3][j] (4 VGPRs); with cbsz = 4 the four A values are taken from lanes 4*abid .. 4*abid+3
+// of src0 for every block.  Used as a lane-local FMA engine: B = a value of the lane's own element,
+// A = four weights, D = four hidden units of the lane's own element -- nothing crosses lanes except
+// the weights.  `abid` must be a compile-time constant after unrolling.
+__device__ __forceinline__ v4f mfma_w4(float wreg, float b, v4f c, int abid) {
+  switch (abid & 15) {
+    case 0: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 0, 0);
+    case 1: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 1, 0);
+    case 2: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 2, 0);
+    case 3: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 3, 0);
+    case 4: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 4, 0);
+    case 5: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 5, 0);
+    case 6: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 6, 0);
+    case 7: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 7, 0);
+    case 8: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 8, 0);
+    case 9: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 9, 0);
+    case 10: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 10, 0);
+    case 11: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 11, 0);
+    case 12: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 12, 0);
+    case 13: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 13, 0);
+    case 14: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 14, 0);
+    default: return __builtin_amdgcn_mfma_f32_4x4x1f32(wreg, b, c, 4, 15, 0);
+  }
+}
+
+// max(x, 0) for finite x as one median-of-three (no NaN-quieting pre-pass as fmaxf needs; written
+// with a compiler builtin so the hazard recogniser sees an ordinary VALU instruction after an MFMA)
+__device__ __forceinline__ float relu(float x) { return __builtin_amdgcn_fmed3f(x, 0.0f, 3.0e38f); }
 
 // Makes the compiler forget what it knows about a (wave-uniform) pointer, so loads through it
 // are re-issued where they are written instead of being hoisted out of the enclosing loop; the

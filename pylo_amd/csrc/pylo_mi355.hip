@@ -13,6 +13,7 @@
 //   k_celo2_apply   accumulators advanced and written, features, MLP, step_out             44 B/elem
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -136,7 +137,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
           d.nd_stride[w] = (int)stride;
           d.len[w] = d.nd_size[w] > 0 ? (int)(n / d.nd_size[w]) : 0;
           d.sumlen[w] = d.nd_size[w];
-          d.npart[w] = 1;
+          d.npart[w] = std::max(1, (d.nd_size[w] + kNdX - 1) / kNdX);
         }
         // the dc axis as it sits inside the row vector (the tensor without dim dr)
         d.rcm_size = d.nd_size[1];
@@ -146,7 +147,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
         d.pitch[w] = (int)round4(d.len[w]);
         d.part_off[w] = part;
         part += round4((long long)d.npart[w] * d.len[w]);
-        const bool aos = d.mode == kModeFac2D && w == 0;
+        const bool aos = d.mode == kModeFac2D;  // 2-D: both tables are [index][4] / [index][H]
         d.fac_off[w] = fac;
         fac += aos ? (long long)d.len[w] * 4 : 3ll * d.pitch[w];
         d.term_off[w] = term;
@@ -161,7 +162,8 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
           d.v0a_n[w] = (int)L.v0a_items.size() - d.v0a_first[w];
           for (int c = 0; c * kV0bEnt < d.len[w]; ++c) L.v0b_items.push_back(Item{t, c, w, 0});
           if (d.mode == kModeFacND)
-            for (int c = 0; c * kThreads < d.len[w]; ++c) L.nd_items.push_back(Item{t, c, w, 0});
+            for (int c = 0; c * kV0aEnt < d.len[w]; ++c)
+              for (int q = 0; q < d.npart[w]; ++q) L.nd_items.push_back(Item{t, c, w, q});
         }
       }
     }
@@ -231,6 +233,10 @@ struct PyloPlan {
   int slot = 0;
   std::vector<PyloTensorArgs> last;
   bool have_last = false;
+  // The hidden layers run as lane-local 4x4x1 fp32 outer products on the matrix pipe; setting the
+  // environment variable PYLO_MI355_VALU_MLP=1 before the plan is created keeps them on the VALU
+  // (same results up to rounding; for A/B measurements).
+  bool mlp_on_matrix_pipe = true;
   // optional per-launch timing (pylo_mi355_plan_timing_begin/end)
   std::vector<hipEvent_t> tev;
   int t_steps_max = 0, t_steps = 0, t_per_step = 0;
@@ -261,6 +267,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   PyloPlan* P = new PyloPlan();
   P->kind = kind;
   P->T = n_tensors;
+  if (const char* v = std::getenv("PYLO_MI355_VALU_MLP")) P->mlp_on_matrix_pipe = !(v[0] == '1');
   if (int rc = build_layout(kind, shapes, n_tensors, P->L, kVeloHiddenMax)) { delete P; return rc; }
   if (workspace == nullptr || workspace_bytes < P->L.total) { delete P; return fail("plan_create: workspace too small"); }
   if (reinterpret_cast<uintptr_t>(workspace) % 256 != 0) { delete P; return fail("plan_create: workspace must be 256-byte aligned"); }
@@ -470,8 +477,14 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   HIP_TRY(mark());
   if (n_fac > 0) hipLaunchKernelGGL(k_celo2_fold, dim3(n_fac), dim3(kFoldThreads), 0, s, descs, dyn, fac_list, stats, mlp, wfold, chan_ms);
   HIP_TRY(mark());
-  if (n_el > 0)
-    hipLaunchKernelGGL(k_celo2_apply, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, term_tab, gl, dec, wfold);
+  if (n_el > 0) {
+    if (P->mlp_on_matrix_pipe)
+      hipLaunchKernelGGL(k_celo2_apply<true>, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab,
+                         term_tab, gl, dec, wfold);
+    else
+      hipLaunchKernelGGL(k_celo2_apply<false>, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab,
+                         term_tab, gl, dec, wfold);
+  }
   HIP_TRY(mark());
   mark.done();
   HIP_TRY(hipGetLastError());
@@ -542,12 +555,12 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
   hipLaunchKernelGGL(k_velo_loss, dim3(1), dim3(64), 0, s, step->loss_means, step->loss_running_min, step->loss_decays,
                      step->loss_iteration, step->loss, lossfeat);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kThreads), 0, s, descs, dyn, T, stats, totals, lossfeat, vs, xfeat);
+  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, totals, lossfeat, vs, xfeat);
   HIP_TRY(mark());
   hipLaunchKernelGGL(k_velo_mix, dim3(H / 64), dim3(kThreads), 0, s, xfeat, T, L.Tpad, H, nets->mix2_wt, nets->mix2_b,
                      nets->fmix_wt, nets->fmix_b, step->lstm_h, xT);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_velo_gates, dim3(L.Tpad / kGateBT, (H + 127) / 128), dim3(128), 0, s, xT, T, L.Tpad, H,
+  hipLaunchKernelGGL(k_velo_gates, dim3(L.Tpad / kGateBT, H / kGateU), dim3(kThreads), 0, s, xT, T, L.Tpad, H,
                      nets->lstm_wt, nets->lstm_b, step->lstm_h, step->lstm_c);
   HIP_TRY(mark());
   hipLaunchKernelGGL(k_velo_heads, dim3(T), dim3(kThreads), sizeof(float) * (H + K + 160 + 32 + 4), s, descs, T, H, K,
@@ -615,7 +628,7 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   HIP_TRY(mark());
   if (n_el > 0) hipLaunchKernelGGL(k_adafac_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, dec, stats);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kThreads), 0, s, descs, dyn, T, stats, totals, (const float*)nullptr, vs,
+  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, totals, (const float*)nullptr, vs,
                      (float*)nullptr);
   HIP_TRY(mark());
   hipLaunchKernelGGL(k_adafac_fold, dim3(T), dim3(kThreads), 0, s, descs, dyn, totals, net, wfold);

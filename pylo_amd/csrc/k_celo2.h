@@ -226,6 +226,60 @@ __device__ __forceinline__ void celo2_stats_chunk(const TDesc& d, const PyloTens
   }
 }
 
+// Geometry of one wave task of the column-resident walk.
+struct TileTask {
+  int r0, r1;          // rows
+  unsigned col;        // the lane's first column
+  long long first;     // element index of (r0, first column of the wave)
+  __device__ __forceinline__ TileTask(const TDesc& d, int task) {
+    const int ct = task % d.tile_nct, rr = task / d.tile_nct;
+    r0 = rr * kTileRows;
+    r1 = r0 + kTileRows < d.R0 ? r0 + kTileRows : d.R0;
+    col = (unsigned)ct * kTileCols + (threadIdx.x & 63) * kTileV;
+    first = (long long)r0 * d.C0 + (long long)ct * kTileCols;
+  }
+};
+
+// Statistics of one wave task: the column factors stay in registers, the row factors arrive through
+// the scalar cache, and the only per-row vector memory traffic is the six streams.
+__device__ __forceinline__ void celo2_stats_tile(const TDesc& d, const PyloTensorArgs& a, int task, float scale,
+                                                 const EmaConsts& e, const float* f0, const float* f1,
+                                                 float (&acc)[kNStat]) {
+  constexpr int V = kTileV;
+  const TileTask tk(d, task);
+  float fb[V][4];
+#pragma unroll
+  for (int v = 0; v < V; ++v) load_vec_o<4>(f1 + v * 4, tk.col * 16u, fb[v]);
+  const unsigned lo = (threadIdx.x & 63) * (V * 4u);
+  const float *g = a.grad + tk.first, *p = a.param + tk.first, *m0 = a.mom + tk.first,
+              *m1 = a.mom + d.n + tk.first, *m2 = a.mom + 2 * d.n + tk.first, *rms = a.rms + tk.first;
+  const float* fr = f0 + (size_t)tk.r0 * 4;
+#pragma unroll 2
+  for (int r = tk.r0; r < tk.r1; ++r) {
+    float xg[V], xp[V], x0[V], x1[V], x2[V], xr[V], fa[4];
+    load_vec_nt<V>(g, lo, xg);
+    load_vec_nt<V>(p, lo, xp);
+    load_vec_nt<V>(m0, lo, x0);
+    load_vec_nt<V>(m1, lo, x1);
+    load_vec_nt<V>(m2, lo, x2);
+    load_vec_nt<V>(rms, lo, xr);
+    load_uniform<4>(fr, fa);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      const float gg = clampf(xg[v] * scale, a.clip_val);
+      float m[3] = {x0[v], x1[v], x2[v]};
+      float rr = xr[v];
+      ema_update(e, gg, m, rr);
+      const float rfcf[3] = {fa[0] * fb[v][0], fa[1] * fb[v][1], fa[2] * fb[v][2]};
+      float f[kNStat];
+      lo_features(gg, xp[v], m, rr, rfcf, 1e-8f, f);
+#pragma unroll
+      for (int c = 0; c < kNStat; ++c) acc[c] = fmaf(f[c], f[c], acc[c]);
+    }
+    g += d.C0; p += d.C0; m0 += d.C0; m1 += d.C0; m2 += d.C0; rms += d.C0; fr += 4;
+  }
+}
+
 // Statistics pass: sum of squares of the 18 per-element channels of every MLP tensor, with the
 // accumulators advanced in registers only (nothing is written back).  AdamW tensors are updated
 // completely here.
@@ -252,9 +306,15 @@ __global__ __launch_bounds__(kThreads) void k_celo2_stats(const TDesc* __restric
   for (int c = 0; c < kNStat; ++c) acc[c] = 0.0f;
   const float* f0 = fac_tab + d.fac_off[0];
   const float* f1 = fac_tab + d.fac_off[1];
-  if (d.vec == 4) celo2_stats_chunk<4>(d, a, it.a, scale, e, f0, f1, acc);
-  else celo2_stats_chunk<1>(d, a, it.a, scale, e, f0, f1, acc);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (d.tile_nct > 0) {
+    const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(wave);
+    if (task < d.tile_ntask) celo2_stats_tile(d, a, task, scale, e, f0, f1, acc);
+  } else if (d.vec == 4) {
+    celo2_stats_chunk<4>(d, a, it.a, scale, e, f0, f1, acc);
+  } else {
+    celo2_stats_chunk<1>(d, a, it.a, scale, e, f0, f1, acc);
+  }
 #pragma unroll
   for (int c = 0; c < kNStat; ++c) {
     const float s = wave_sum(acc[c]);
@@ -507,6 +567,104 @@ __device__ __forceinline__ void celo2_apply_chunk_mfma(const TDesc& d, const Pyl
   }
 }
 
+// The matrix-pipe apply pass over one wave task of the column-resident walk: column factors and
+// column terms stay in registers, row factors and row terms arrive through the scalar cache.
+__device__ __forceinline__ void celo2_apply_tile(const TDesc& d, const PyloTensorArgs& a, int task, float scale,
+                                                 const EmaConsts& e, const float* f0, const float* f1,
+                                                 const float* t0, const float* t1, const float* wbase) {
+  constexpr int V = kTileV;
+  const TileTask tk(d, task);
+  const bool use_exp = a.exp_mult != 0.0f;
+  const float exp_scale = a.exp_mult * 1.44269504088896341f;
+  const int lane = threadIdx.x & 63;
+  float wreg[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) wreg[r] = *(const gfloat*)(wbase + r * 64 + lane);
+  constexpr int gWH = kC2WH / 4, gBH = kC2BH / 4, gWO = kC2WO / 4, gBO = kC2BO / 4;
+  const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
+  float fb[V][4], tb[V][8];
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    load_vec_o<4>(f1 + v * 4, tk.col * 16u, fb[v]);
+    load_row8(t1 + v * 8, tk.col, tb[v]);
+  }
+  const unsigned lo = lane * (V * 4u);
+  const float *g = a.grad + tk.first, *p = a.param + tk.first;
+  float *m0 = a.mom + tk.first, *m1 = a.mom + d.n + tk.first, *m2 = a.mom + 2 * d.n + tk.first,
+        *rms = a.rms + tk.first, *out = a.step_out + tk.first;
+  const float* fr = f0 + (size_t)tk.r0 * 4;
+  const float* tr = t0 + (size_t)tk.r0 * 8;
+  for (int r = tk.r0; r < tk.r1; ++r) {
+    float xg[V], xp[V], x0[V], x1[V], x2[V], xr[V], fa[4], ta[8];
+    load_vec_nt<V>(g, lo, xg);
+    load_vec_nt<V>(p, lo, xp);
+    load_vec_nt<V>(m0, lo, x0);
+    load_vec_nt<V>(m1, lo, x1);
+    load_vec_nt<V>(m2, lo, x2);
+    load_vec_nt<V>(rms, lo, xr);
+    load_uniform<4>(fr, fa);
+    load_uniform<8>(tr, ta);
+    float f[V][kNStat];
+    v4f ha[V], hb[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      const float gg = clampf(xg[v] * scale, a.clip_val);
+      float m[3] = {x0[v], x1[v], x2[v]};
+      ema_update(e, gg, m, xr[v]);
+      x0[v] = m[0]; x1[v] = m[1]; x2[v] = m[2];
+      const float rfcf[3] = {fa[0] * fb[v][0], fa[1] * fb[v][1], fa[2] * fb[v][2]};
+      lo_features(gg, xp[v], m, xr[v], rfcf, 1e-8f, f[v]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { ha[v][j] = ta[j] + tb[v][j]; hb[v][j] = ta[4 + j] + tb[v][4 + j]; }
+    }
+    store_vec_nt<V>(m0, lo, x0);
+    store_vec_nt<V>(m1, lo, x1);
+    store_vec_nt<V>(m2, lo, x2);
+    store_vec_nt<V>(rms, lo, xr);
+#pragma unroll
+    for (int c = 0; c < kNStat; ++c) {
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        ha[v] = mfma_w4(wreg[(2 * c) / 16], f[v][c], ha[v], (2 * c) % 16);
+        hb[v] = mfma_w4(wreg[(2 * c + 1) / 16], f[v][c], hb[v], (2 * c + 1) % 16);
+      }
+    }
+    v4f ga[V], gb[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      ga[v] = mfma_w4(wreg[gBH / 16], 1.0f, zero, gBH % 16);
+      gb[v] = mfma_w4(wreg[(gBH + 1) / 16], 1.0f, zero, (gBH + 1) % 16);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        const float hk = relu(k < 4 ? ha[v][k] : hb[v][k - 4]);
+        ga[v] = mfma_w4(wreg[(gWH + 2 * k) / 16], hk, ga[v], (gWH + 2 * k) % 16);
+        gb[v] = mfma_w4(wreg[(gWH + 2 * k + 1) / 16], hk, gb[v], (gWH + 2 * k + 1) % 16);
+      }
+    }
+    v4f o[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) o[v] = mfma_w4(wreg[gBO / 16], 1.0f, zero, gBO % 16);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        const float hk = relu(k < 4 ? ga[v][k] : gb[v][k - 4]);
+        o[v] = mfma_w4(wreg[(gWO + k) / 16], hk, o[v], (gWO + k) % 16);
+      }
+    }
+    float res[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v)
+      res[v] = use_exp ? o[v][0] * __builtin_amdgcn_exp2f(o[v][1] * exp_scale) : o[v][0];
+    store_vec_o<V>(out, lo, res);
+    g += d.C0; p += d.C0; m0 += d.C0; m1 += d.C0; m2 += d.C0; rms += d.C0; out += d.C0;
+    fr += 4; tr += 8;
+  }
+}
+
 // Apply pass: accumulators advanced and written, features, MLP, raw step.
 template <bool MFMA>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PYLO_APPLY_WAVES))) void k_celo2_apply(const TDesc* __restrict__ descs,
@@ -524,7 +682,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PYLO_A
   const float scale = clip_scale(gl->gnorm, a.clip_norm);
   const EmaConsts e = make_ema(dec);
   const float* w = wfold + (size_t)d.fac_slot * kC2Fold;
-  if (MFMA && d.vec == 4)
+  if (MFMA && d.tile_nct > 0) {
+    const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (task < d.tile_ntask)
+      celo2_apply_tile(d, a, task, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
+                       term_tab + d.term_off[0], term_tab + d.term_off[1], w);
+  } else if (MFMA && d.vec == 4)
     celo2_apply_chunk_mfma<kMfmaV>(d, a, it.a, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
                                    term_tab + d.term_off[0], term_tab + d.term_off[1], w);
   else if (d.vec == 4)

@@ -9,11 +9,11 @@ namespace pylo {
 // =============================================================================================
 // P0: row / column sums of g^2 for 2-D factored tensors; sum g^2 and clamp flag for everything
 // =============================================================================================
-template <int V>
-__device__ __forceinline__ void p0_factored(const TDesc& d, const float* g, int strip, int cb, bool exact,
+template <int V, bool exact>
+__device__ __forceinline__ void p0_factored(const TDesc& d, const float* g, int strip, int cb,
                                             float scale, float clipv, float* __restrict__ rowpart,
                                             float* __restrict__ colpart, float* lds_col, float* lds_row,
-                                            float& gsq, int& flag) {
+                                            float& gsq, float& amax) {
   constexpr int TC = 64 * V;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int C0 = d.C0, R0 = d.R0;
@@ -24,27 +24,40 @@ __device__ __forceinline__ void p0_factored(const TDesc& d, const float* g, int 
   float col[V];
 #pragma unroll
   for (int v = 0; v < V; ++v) col[v] = 0.0f;
-  for (int r = r0 + wave; r < r1; r += kWaves) {
-    float x[V];
-    if (in) {
-      load_vec<V>(g + (size_t)r * C0 + c, x);
-    } else {
+  // Four rows per wave and trip (rows rb, rb+4, rb+8, rb+12): the loads are independent and issued
+  // together, and the four row sums are reduced jointly.  lds_row is [wave][trip][16-lane group][u].
+  int trip = 0;
+  for (int rb = r0 + wave; rb < r1; rb += 4 * kWaves, ++trip) {
+    float x[4][V];
 #pragma unroll
-      for (int v = 0; v < V; ++v) x[v] = 0.0f;
-    }
-    float rs = 0.0f;
+    for (int u = 0; u < 4; ++u) {
+      const int r = rb + u * kWaves;
+      const float* src = g + (size_t)(r < r1 ? r : rb) * C0 + (in ? c : 0);
+      load_vec<V>(src, x[u]);
+      if (!(in && r < r1)) {
 #pragma unroll
-    for (int v = 0; v < V; ++v) {
-      const float raw = x[v];
-      gsq = fmaf(raw, raw, gsq);
-      if (!exact) flag |= (fabsf(raw) > clipv && clipv > 0.0f) ? 1 : 0;
-      const float y = exact ? clampf(raw * scale, clipv) : raw;
-      const float sq = y * y;
-      col[v] += sq;
-      rs += sq;
+        for (int v = 0; v < V; ++v) x[u][v] = 0.0f;
+      }
     }
-    rs = wave_sum(rs);
-    if (lane == 0) lds_row[r - r0] = rs;
+    float rs[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      float sq[V];
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        const float raw = x[u][v];
+        amax = fmaxf(amax, fabsf(raw));
+        if (exact) gsq = fmaf(raw, raw, gsq);
+        const float y = exact ? clampf(raw * scale, clipv) : raw;
+        sq[v] = y * y;
+        col[v] += sq[v];
+      }
+      if constexpr (V == 4) rs[u] = (sq[0] + sq[1]) + (sq[2] + sq[3]);
+      else rs[u] = sq[0];
+      if (!exact) gsq += rs[u];
+    }
+    const float tot = reduce4_rows16(rs[0], rs[1], rs[2], rs[3]);
+    if ((lane & 12) == 0) lds_row[((wave * (kP0Rows / 16) + trip) * 4 + (lane >> 4)) * 4 + (lane & 3)] = tot;
   }
 #pragma unroll
   for (int v = 0; v < V; ++v) lds_col[wave * TC + lane * V + v] = col[v];
@@ -54,12 +67,16 @@ __device__ __forceinline__ void p0_factored(const TDesc& d, const float* g, int 
     const int cc = cb * TC + j;
     if (cc < C0) colpart[(size_t)strip * C0 + cc] = s;
   }
-  for (int j = threadIdx.x; j < r1 - r0; j += kThreads) rowpart[(size_t)cb * R0 + r0 + j] = lds_row[j];
+  for (int j = threadIdx.x; j < r1 - r0; j += kThreads) {
+    // row r0 + j was handled by wave j % 4 in trip (j / 4) / 4 as its row u = (j / 4) % 4
+    const int w = j % kWaves, q = j / kWaves;
+    const float* t = lds_row + ((w * (kP0Rows / 16) + q / 4) * 4) * 4 + (q % 4);
+    rowpart[(size_t)cb * R0 + r0 + j] = (t[0] + t[4]) + (t[8] + t[12]);
+  }
 }
 
 template <int V>
-__device__ __forceinline__ void p0_flat(const TDesc& d, const float* g, int chunk, float clipv,
-                                        float& gsq, int& flag) {
+__device__ __forceinline__ void p0_flat(const TDesc& d, const float* g, int chunk, float& gsq, float& amax) {
   const long long base = (long long)chunk * (kThreads * V * kElemIters);
 #pragma unroll
   for (int it = 0; it < kElemIters; ++it) {
@@ -70,7 +87,7 @@ __device__ __forceinline__ void p0_flat(const TDesc& d, const float* g, int chun
 #pragma unroll
       for (int v = 0; v < V; ++v) {
         gsq = fmaf(x[v], x[v], gsq);
-        flag |= (fabsf(x[v]) > clipv && clipv > 0.0f) ? 1 : 0;
+        amax = fmaxf(amax, fabsf(x[v]));
       }
     }
   }
@@ -85,7 +102,7 @@ __global__ __launch_bounds__(kThreads) void k_p0(const TDesc* __restrict__ descs
                                                  double* __restrict__ gsq_part, int* __restrict__ flag_part,
                                                  const Globals* __restrict__ gl, int pass) {
   __shared__ float lds_col[kWaves * 256];
-  __shared__ float lds_row[kP0Rows];
+  __shared__ float lds_row[kWaves * (kP0Rows / 16) * 16];
   __shared__ float lds_red[kWaves];
   __shared__ int lds_flag[kWaves];
   const Item it = items[blockIdx.x];
@@ -93,26 +110,26 @@ __global__ __launch_bounds__(kThreads) void k_p0(const TDesc* __restrict__ descs
   const PyloTensorArgs a = dyn[it.tensor];
   const bool clip_on = a.clip_norm > 0.0f;
   if (pass == 1 && (!clip_on || d.mode != kModeFac2D || gl->flag == 0)) return;
-  float gsq = 0.0f;
-  int flag = 0;
+  float gsq = 0.0f, amax = 0.0f;
   if (a.grad != nullptr) {
     if (d.mode == kModeFac2D) {
       const bool exact = (pass == 1) || !clip_on;
       const float scale = (pass == 1) ? clip_scale(gl->gnorm, a.clip_norm) : 1.0f;
-      if (d.vec == 4)
-        p0_factored<4>(d, a.grad, it.a, it.b, exact, scale, a.clip_val, part + d.part_off[0],
-                       part + d.part_off[1], lds_col, lds_row, gsq, flag);
-      else
-        p0_factored<1>(d, a.grad, it.a, it.b, exact, scale, a.clip_val, part + d.part_off[0],
-                       part + d.part_off[1], lds_col, lds_row, gsq, flag);
+      float* p0r = part + d.part_off[0];
+      float* p0c = part + d.part_off[1];
+      if (d.vec == 4 && exact) p0_factored<4, true>(d, a.grad, it.a, it.b, scale, a.clip_val, p0r, p0c, lds_col, lds_row, gsq, amax);
+      else if (d.vec == 4) p0_factored<4, false>(d, a.grad, it.a, it.b, scale, a.clip_val, p0r, p0c, lds_col, lds_row, gsq, amax);
+      else if (exact) p0_factored<1, true>(d, a.grad, it.a, it.b, scale, a.clip_val, p0r, p0c, lds_col, lds_row, gsq, amax);
+      else p0_factored<1, false>(d, a.grad, it.a, it.b, scale, a.clip_val, p0r, p0c, lds_col, lds_row, gsq, amax);
     } else {
-      if (d.vec == 4) p0_flat<4>(d, a.grad, it.a, a.clip_val, gsq, flag);
-      else p0_flat<1>(d, a.grad, it.a, a.clip_val, gsq, flag);
+      if (d.vec == 4) p0_flat<4>(d, a.grad, it.a, gsq, amax);
+      else p0_flat<1>(d, a.grad, it.a, gsq, amax);
     }
   }
   if (pass == 1) return;
   gsq = wave_sum(gsq);
-  flag = __any(flag) ? 1 : 0;
+  // some element lies beyond the clamp (fmaxf drops NaNs, which therefore never raise the flag)
+  const int flag = __any(a.clip_val > 0.0f && !(amax <= a.clip_val)) ? 1 : 0;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   if (lane == 0) { lds_red[wave] = gsq; lds_flag[wave] = flag; }
   __syncthreads();
@@ -179,13 +196,14 @@ __global__ __launch_bounds__(kThreads) void k_p0_nd(const TDesc* __restrict__ de
 // partials, advances the three Adafactor accumulators (ELO_CELO2_naive.py:152-160) and leaves
 // per-block partial sums of  f, f^2, rsqrt(f+1e-8)^2  per decay.
 // =============================================================================================
-__global__ __launch_bounds__(kThreads) void k_v0a(const TDesc* __restrict__ descs,
+__global__ __launch_bounds__(kV0aThreads) void k_v0a(const TDesc* __restrict__ descs,
                                                   const PyloTensorArgs* __restrict__ dyn,
                                                   const Item* __restrict__ items,
                                                   const float* __restrict__ part,
                                                   const Globals* __restrict__ gl, PyloDecays dec,
                                                   double* __restrict__ v0part) {
-  __shared__ double lds[kWaves][kV0aEnt];
+  constexpr int G = kV0aThreads / 64;
+  __shared__ double lds[G][kV0aEnt];
   const Item it = items[blockIdx.x];
   const TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
@@ -198,8 +216,10 @@ __global__ __launch_bounds__(kThreads) void k_v0a(const TDesc* __restrict__ desc
   const int i = it.a * kV0aEnt + e;
   {
     double s = 0.0;
-    if (i < len)
-      for (int q = grp; q < npart; q += kWaves) s += (double)pp[(size_t)q * len + i];
+    if (i < len) {
+#pragma unroll 8
+      for (int q = grp; q < npart; q += G) s += (double)*(const gfloat*)(pp + (size_t)q * len + i);
+    }
     lds[grp][e] = s;
   }
   __syncthreads();
@@ -214,7 +234,9 @@ __global__ __launch_bounds__(kThreads) void k_v0a(const TDesc* __restrict__ desc
   float* fac = is_r ? a.fac_r : a.fac_c;
   double s_f = 0.0, s_ff = 0.0, s_rr = 0.0;
   if (i < len) {
-    const double S = ((lds[0][e] + lds[1][e]) + lds[2][e]) + lds[3][e];
+    double S = 0.0;
+#pragma unroll
+    for (int q = 0; q < G; ++q) S += lds[q][e];
     const float q = (float)(s2 * S / (double)d.sumlen[which]) + 1e-30f;
     const float beta = dec.beta_fac[k];
     const float f = beta * fac[(size_t)k * len + i] + (1.0f - beta) * q;

@@ -15,11 +15,15 @@ constexpr int kThreads = 256;   // 4 waves of 64 lanes
 constexpr int kWaves = 4;
 constexpr int kP0Rows = 128;    // rows of one row/column-sum tile; tile columns = 64 * vec
 constexpr int kElemIters = 8;   // an element chunk is kThreads * vec * kElemIters elements
+constexpr int kTileV = 2;       // column-resident walk: a wave owns 64 * kTileV columns ...
+constexpr int kTileCols = 64 * kTileV;
+constexpr int kTileRows = 32;   // ... and walks this many rows of them
 constexpr int kNStat = 18;      // feature channels that vary per element (the other 12 are
                                 // functions of the row or of the column only)
 constexpr int kV0aEnt = 64;     // vector entries per k_v0a block
 constexpr int kV0bEnt = 1024;   // vector entries per k_v0b block
 constexpr int kNV0 = 9;         // partial sums per k_v0a block
+constexpr int kV0aThreads = 256;   // groups of 64 lanes share the partial rows of 64 entries
 constexpr int kFoldThreads = 1024;
 constexpr int kNdX = 64;        // elements of the summed dim one k_p0_nd block covers (one partial row)
 
@@ -64,6 +68,10 @@ struct TDesc {
   long long fac_off[2];   // floats, factor tables: 2-D vector 0 is AoS [len][4], everything else SoA [3][pitch]
   long long term_off[2];  // floats, first-layer terms: 2-D vector 0 is AoS [len][H], else SoA [H][pitch]
   int v0a_first[2], v0a_n[2];  // k_v0a blocks of vector 0 / 1
+  // Column-resident walk (wide 2-D tensors, C0 % kTileCols == 0): wave task w covers columns
+  // [ (w % tile_nct) * kTileCols, +kTileCols ) of rows [ (w / tile_nct) * kTileRows, +kTileRows );
+  // element block a holds tasks 4a .. 4a+3.  tile_nct == 0: linear chunks instead.
+  int tile_nct, tile_ntask;
 };
 
 struct Item {
@@ -99,15 +107,64 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Sum over the wave without the LDS crossbar (six DPP adds); the total is valid in lane 63 only.
+__device__ __forceinline__ float wave_sum_to_last(float v) {
+  auto dpp = [](float x, int ctrl, int row_mask) {
+    int r;
+    switch (ctrl) {  // the control word must be an immediate
+      case 0xB1: r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, false); break;   // quad_perm [1,0,3,2]
+      case 0x4E: r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, false); break;   // quad_perm [2,3,0,1]
+      case 0x141: r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, false); break; // row_half_mirror
+      case 0x140: r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, false); break; // row_mirror
+      case 0x142: r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xA, 0xF, false); break; // row_bcast:15 into rows 1, 3
+      default: r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x143, 0xC, 0xF, false); break;    // row_bcast:31 into rows 2, 3
+    }
+    (void)row_mask;
+    return __builtin_bit_cast(float, r);
+  };
+  v += dpp(v, 0xB1, 0xF);
+  v += dpp(v, 0x4E, 0xF);
+  v += dpp(v, 0x141, 0xF);
+  v += dpp(v, 0x140, 0xF);
+  v += dpp(v, 0x142, 0xA);
+  v += dpp(v, 0x143, 0xC);
+  return v;
+}
+
+// DPP moves with the control word as a template argument (it must be an immediate).
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, false));
+}
+
+// Four values per lane (one per row u) -> per 16-lane group, lane 4q + u holds the sum of row u over
+// the group's 16 lanes (q = 0..3 all hold it).  Fourteen VALU instructions instead of four full
+// wave reductions; lane-pair exchanges first, so every lane ends up owning one row.
+__device__ __forceinline__ float reduce4_rows16(float a0, float a1, float a2, float a3) {
+  const int lane = threadIdx.x & 63;
+  const bool b0 = lane & 1, b1 = lane & 2;
+  const float k01 = b0 ? a1 : a0, s01 = b0 ? a0 : a1;
+  const float k23 = b0 ? a3 : a2, s23 = b0 ? a2 : a3;
+  const float p01 = k01 + dpp_mov<0xB1>(s01);  // quad_perm [1,0,3,2]
+  const float p23 = k23 + dpp_mov<0xB1>(s23);
+  const float k = b1 ? p23 : p01, s = b1 ? p01 : p23;
+  float v = k + dpp_mov<0x4E>(s);              // quad_perm [2,3,0,1]: lane%4 = u holds row u of its quad
+  v += dpp_mov<0x124>(v);                      // row_ror:4
+  v += dpp_mov<0x128>(v);                      // row_ror:8
+  return v;
+}
+
 __device__ __forceinline__ double wave_sum(double v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
   return v;
 }
 
-// torch.clamp semantics (NaN propagates); c <= 0 disables the clamp.
+// torch.clamp semantics (NaN propagates); c <= 0 disables the clamp.  Branch-free: the bound is a
+// wave-uniform select that the compiler hoists out of element loops.
 __device__ __forceinline__ float clampf(float x, float c) {
-  return (c > 0.0f) ? (x < -c ? -c : (x > c ? c : x)) : x;
+  const float hi = c > 0.0f ? c : __builtin_inff();
+  return x < -hi ? -hi : (x > hi ? hi : x);
 }
 
 // clip_norm / max(norm, clip_norm); 1 when clipping is off (ELO_CELO2_naive.py:126-135).
@@ -190,6 +247,37 @@ __device__ __forceinline__ void store_vec_o(float* sbase, unsigned byte_off, con
   }
 }
 
+// Streaming variants: the data is not needed again before it would be evicted anyway.
+template <int V>
+__device__ __forceinline__ void load_vec_nt(const float* sbase, unsigned byte_off, float (&x)[V]) {
+  const gchar* p = (const gchar*)sbase + byte_off;
+  if constexpr (V == 4) {
+    const v4f t = __builtin_nontemporal_load((const gv4f*)p);
+    x[0] = t.x; x[1] = t.y; x[2] = t.z; x[3] = t.w;
+  } else if constexpr (V == 2) {
+    const v2f t = __builtin_nontemporal_load((const gv2f*)p);
+    x[0] = t.x; x[1] = t.y;
+  } else {
+    x[0] = __builtin_nontemporal_load((const gfloat*)p);
+  }
+}
+
+template <int V>
+__device__ __forceinline__ void store_vec_nt(float* sbase, unsigned byte_off, const float (&x)[V]) {
+  gchar* p = (gchar*)sbase + byte_off;
+  if constexpr (V == 4) {
+    v4f t;
+    t.x = x[0]; t.y = x[1]; t.z = x[2]; t.w = x[3];
+    __builtin_nontemporal_store(t, (gv4f*)p);
+  } else if constexpr (V == 2) {
+    v2f t;
+    t.x = x[0]; t.y = x[1];
+    __builtin_nontemporal_store(t, (gv2f*)p);
+  } else {
+    __builtin_nontemporal_store(x[0], (gfloat*)p);
+  }
+}
+
 __device__ __forceinline__ float4 load_f4(const float* p) {
   const v4f t = *(const gv4f*)(p);
   return make_float4(t.x, t.y, t.z, t.w);
@@ -238,6 +326,15 @@ typedef __attribute__((address_space(4))) float cfloat;
 __device__ __forceinline__ const cfloat* launder(const float* p) {
   asm volatile("" : "+s"(p));
   return (const cfloat*)p;
+}
+
+// N consecutive floats at a wave-uniform address, through the scalar cache into SGPRs.  The memory
+// must not be written by the running kernel.
+template <int N>
+__device__ __forceinline__ void load_uniform(const float* p, float (&x)[N]) {
+  const cfloat* q = (const cfloat*)p;
+#pragma unroll
+  for (int i = 0; i < N; ++i) x[i] = q[i];
 }
 
 }  // namespace pylo

@@ -75,6 +75,14 @@ struct Layout {
 
 int first_layer_width(int kind) { return kind == PYLO_KIND_CELO2 ? 8 : kind == PYLO_KIND_VELO ? 4 : 32; }
 
+// The hidden layers of ELO-CELO2 run as lane-local 4x4x1 fp32 outer products on the matrix pipe and
+// wide 2-D tensors are walked column-resident; PYLO_MI355_VALU_MLP=1 in the environment keeps the
+// earlier all-VALU kernels over linear chunks (same results up to rounding; for A/B measurements).
+bool env_matrix_pipe() {
+  const char* v = std::getenv("PYLO_MI355_VALU_MLP");
+  return !(v && v[0] == '1');
+}
+
 int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int velo_hidden) {
   if (kind != PYLO_KIND_CELO2 && kind != PYLO_KIND_VELO && kind != PYLO_KIND_ADAFAC)
     return fail("plan: unknown optimizer kind");
@@ -178,7 +186,13 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       }
     }
     d.blk0 = (int)L.el_items.size();
-    for (long long c = 0; c * chunk < n; ++c) L.el_items.push_back(Item{t, (int)c, 0, 0});
+    if (kind == PYLO_KIND_CELO2 && d.mode == kModeFac2D && n > 0 && d.C0 % kTileCols == 0 && env_matrix_pipe()) {
+      d.tile_nct = d.C0 / kTileCols;
+      d.tile_ntask = d.tile_nct * ((d.R0 + kTileRows - 1) / kTileRows);
+      for (int b = 0; b * 4 < d.tile_ntask; ++b) L.el_items.push_back(Item{t, b, 0, 0});
+    } else {
+      for (long long c = 0; c * chunk < n; ++c) L.el_items.push_back(Item{t, (int)c, 0, 0});
+    }
     d.nblk = (int)L.el_items.size() - d.blk0;
   }
   size_t off = 0;
@@ -233,10 +247,7 @@ struct PyloPlan {
   int slot = 0;
   std::vector<PyloTensorArgs> last;
   bool have_last = false;
-  // The hidden layers run as lane-local 4x4x1 fp32 outer products on the matrix pipe; setting the
-  // environment variable PYLO_MI355_VALU_MLP=1 before the plan is created keeps them on the VALU
-  // (same results up to rounding; for A/B measurements).
-  bool mlp_on_matrix_pipe = true;
+  bool mlp_on_matrix_pipe = true;  // env_matrix_pipe() when the plan was created
   // optional per-launch timing (pylo_mi355_plan_timing_begin/end)
   std::vector<hipEvent_t> tev;
   int t_steps_max = 0, t_steps = 0, t_per_step = 0;
@@ -267,7 +278,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   PyloPlan* P = new PyloPlan();
   P->kind = kind;
   P->T = n_tensors;
-  if (const char* v = std::getenv("PYLO_MI355_VALU_MLP")) P->mlp_on_matrix_pipe = !(v[0] == '1');
+  P->mlp_on_matrix_pipe = env_matrix_pipe();
   if (int rc = build_layout(kind, shapes, n_tensors, P->L, kVeloHiddenMax)) { delete P; return rc; }
   if (workspace == nullptr || workspace_bytes < P->L.total) { delete P; return fail("plan_create: workspace too small"); }
   if (reinterpret_cast<uintptr_t>(workspace) % 256 != 0) { delete P; return fail("plan_create: workspace must be 256-byte aligned"); }
@@ -467,7 +478,7 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1);
   HIP_TRY(mark());
   if (n_v0a > 0)
-    hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
+    hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kV0aThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
   HIP_TRY(mark());
   if (n_v0b > 0)
     hipLaunchKernelGGL(k_v0b<8>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-9f, mlp,
@@ -544,7 +555,7 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
   if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part);
   HIP_TRY(mark());
   if (n_v0a > 0)
-    hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
+    hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kV0aThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
   HIP_TRY(mark());
   if (n_v0b > 0)
     hipLaunchKernelGGL(k_v0b<4>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-5f,
@@ -618,7 +629,7 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part);
   HIP_TRY(mark());
   if (n_v0a > 0)
-    hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
+    hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kV0aThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
   HIP_TRY(mark());
   hipLaunchKernelGGL(k_adafac_bias, dim3(1), dim3(64), 0, s, net, step, bias_eff);
   HIP_TRY(mark());

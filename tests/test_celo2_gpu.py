@@ -63,6 +63,9 @@ def _check_states(opt, orc, gpu, t, tag=""):
     ([(40, 56), (7,)], 0.5, dict(lr=1e-2, clip_grad=False, adam_lr_mult=1.0)),
     ([(37, 4099), (4099, 37), (5, 3), (1, 9), (1,), (130, 1)], 0.1, dict(lr=1e-3)),    # dword path, ragged
     ([(256, 1028), (1028, 256), (300, 260)], 2.0, dict(lr=1e-3)),                      # several tiles
+    # column-resident walk (row length a multiple of 128): ragged row ranges, a single row, a
+    # task count that does not fill the last block, next to narrow tensors on the chunked path
+    ([(70, 384), (33, 128), (1, 128), (2100, 256), (300,), (64, 130)], 1.0, dict(lr=1e-3, exp_mult=0.01)),
 ])
 def test_fused_kernel_matches_oracle_per_step(shapes, gscale, cfg):
     """Raw step (what celo2_kernel.cu writes to step_out) and all accumulators, every step, with

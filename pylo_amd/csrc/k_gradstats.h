@@ -174,9 +174,9 @@ __global__ __launch_bounds__(kThreads) void k_p0_nd(const TDesc* __restrict__ de
   const int w = it.b;
   const int e = threadIdx.x & 63, grp = threadIdx.x >> 6;
   const int i = it.a * kV0aEnt + e;
-  const int X = d.nd_size[w], sX = d.nd_stride[w];
+  const int X = pick(d.nd_size, w), sX = pick(d.nd_stride, w);
   float s = 0.0f;
-  if (i < d.len[w]) {
+  if (i < pick(d.len, w)) {
     const long long base = (long long)(i / sX) * X * sX + (i % sX);
     const int x0 = it.c * kNdX + grp * (kNdX / kWaves);
     const int x1 = min(X, x0 + kNdX / kWaves);
@@ -187,8 +187,8 @@ __global__ __launch_bounds__(kThreads) void k_p0_nd(const TDesc* __restrict__ de
   }
   lds[grp][e] = s;
   __syncthreads();
-  if (grp == 0 && i < d.len[w])
-    part[d.part_off[w] + (size_t)it.c * d.len[w] + i] = ((lds[0][e] + lds[1][e]) + lds[2][e]) + lds[3][e];
+  if (grp == 0 && i < pick(d.len, w))
+    part[pick(d.part_off, w) + (size_t)it.c * pick(d.len, w) + i] = ((lds[0][e] + lds[1][e]) + lds[2][e]) + lds[3][e];
 }
 
 // =============================================================================================
@@ -209,9 +209,9 @@ __global__ __launch_bounds__(kV0aThreads) void k_v0a(const TDesc* __restrict__ d
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
   const int which = it.b;
-  const int len = d.len[which];
-  const int npart = d.npart[which];
-  const float* pp = part + d.part_off[which];
+  const int len = pick(d.len, which);
+  const int npart = pick(d.npart, which);
+  const float* pp = part + pick(d.part_off, which);
   const int e = threadIdx.x & 63, grp = threadIdx.x >> 6;
   const int i = it.a * kV0aEnt + e;
   {
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(kV0aThreads) void k_v0a(const TDesc* __restrict__ d
     double S = 0.0;
 #pragma unroll
     for (int q = 0; q < G; ++q) S += lds[q][e];
-    const float q = (float)(s2 * S / (double)d.sumlen[which]) + 1e-30f;
+    const float q = (float)(s2 * S / (double)pick(d.sumlen, which)) + 1e-30f;
     const float beta = dec.beta_fac[k];
     const float f = beta * fac[(size_t)k * len + i] + (1.0f - beta) * q;
     fac[(size_t)k * len + i] = f;
@@ -257,13 +257,13 @@ __global__ __launch_bounds__(kV0aThreads) void k_v0a(const TDesc* __restrict__ d
 
 // Where entry i of vector `which` of tensor d lives in the factor / term tables.
 __device__ __forceinline__ size_t fac_index(const TDesc& d, int which, int k, int i) {
-  return d.mode == kModeFac2D ? (size_t)d.fac_off[which] + (size_t)i * 4 + k
-                              : (size_t)d.fac_off[which] + (size_t)k * d.pitch[which] + i;
+  return d.mode == kModeFac2D ? (size_t)pick(d.fac_off, which) + (size_t)i * 4 + k
+                              : (size_t)pick(d.fac_off, which) + (size_t)k * pick(d.pitch, which) + i;
 }
 template <int H>
 __device__ __forceinline__ size_t term_index(const TDesc& d, int which, int j, int i) {
-  return d.mode == kModeFac2D ? (size_t)d.term_off[which] + (size_t)i * H + j
-                              : (size_t)d.term_off[which] + (size_t)j * d.pitch[which] + i;
+  return d.mode == kModeFac2D ? (size_t)pick(d.term_off, which) + (size_t)i * H + j
+                              : (size_t)pick(d.term_off, which) + (size_t)j * pick(d.pitch, which) + i;
 }
 
 // Row_factor / col_factor of one entry, and the two normalised broadcast features it carries
@@ -334,7 +334,9 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
     if (gI < G) {
       const int vecI = pair / kNV0, slot = pair % kNV0;
       double s = 0.0;
-      for (int b = gI; b < d.v0a_n[vecI]; b += G) s += v0part[(size_t)(d.v0a_first[vecI] + b) * kNV0 + slot];
+      const int nb = vecI ? d.v0a_n[1] : d.v0a_n[0], first = vecI ? d.v0a_first[1] : d.v0a_first[0];
+#pragma unroll 8
+      for (int b = gI; b < nb; b += G) s += v0part[(size_t)(first + b) * kNV0 + slot];
       red[gI][pair] = s;
     }
     __syncthreads();
@@ -362,7 +364,7 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
   const int which = it.b;
   if (which == 0 && it.a == 0 && threadIdx.x == 0) bscale[d.fac_slot] = bs;
   const bool is_r = (which == 0) == (d.vec0_is_r != 0);
-  const int len = d.len[which];
+  const int len = pick(d.len, which);
   const float* fac = is_r ? a.fac_r : a.fac_c;
   for (int i = it.a * kV0bEnt + threadIdx.x; i < min(len, (it.a + 1) * kV0bEnt); i += kThreads) {
     float fct[3], x0[3], x1[3];
@@ -391,7 +393,7 @@ __global__ __launch_bounds__(kThreads) void k_terms(const TDesc* __restrict__ de
   const float* b1 = w1 + 30 * H;
   const int which = it.b;
   const bool is_r = (which == 0) == (d.vec0_is_r != 0);
-  const int len = d.len[which];
+  const int len = pick(d.len, which);
   const float* fac = is_r ? a.fac_r : a.fac_c;
   for (int i = it.a * kV0bEnt + threadIdx.x; i < min(len, (it.a + 1) * kV0bEnt); i += kThreads) {
     float fct[3], x0[3], x1[3];

@@ -74,6 +74,11 @@ struct TDesc {
   int tile_nct, tile_ntask;
 };
 
+// Field of vector 0 or 1 chosen at run time.  Indexing the by-value descriptor with a run-time
+// index would force the whole struct into scratch memory; a select keeps it in registers.
+template <class T>
+__device__ __forceinline__ T pick(const T (&a)[2], int w) { return w ? a[1] : a[0]; }
+
 struct Item {
   int tensor;
   int a;  // P0: strip (or flat chunk); element kernels: chunk; V0 / N-D sums: chunk of entries

@@ -11,8 +11,10 @@ namespace pylo {
 
 // Folded per-tensor weights (floats): first layer rows scaled by the channel normalisers
 // (18 per-element rows for factored tensors, all 30 rows for non-factored ones), (in, out).
-constexpr int kVW1 = 0, kVB1 = 120, kVWH = 124, kVBH = 140, kVWO = 144, kVBO = 152, kVPS = 154, kVLR = 155,
-              kVFold = 160;
+// W1 (30,4) | b1 4 | WH (4,4) | bH 4 | WO (4,4: two outputs, two zeros) | bO 4 (same padding) |
+// param_scale | lr_mult; padded to three 64-float registers for the matrix-pipe path
+constexpr int kVW1 = 0, kVB1 = 120, kVWH = 124, kVBH = 140, kVWO = 144, kVBO = 160, kVPS = 164, kVLR = 165,
+              kVFold = 192;
 constexpr int kVCanon = 128;   // per-tensor un-scaled first layer (30,4) + bias 4, for k_terms
 constexpr int kVBank = 159;    // floats per bank entry: W_in (4,30) | b_in 4 | W_h (4,4) | b_h 4 | W_out (3,4) | b_out 3
 constexpr int kXW = 32;        // row pitch of the LSTM input features (30 used)
@@ -114,6 +116,49 @@ __device__ __forceinline__ void velo_stats_fac(const TDesc& d, const PyloTensorA
   }
 }
 
+// Column-resident walk of one wave task (wide 2-D tensors): column factors in registers, row
+// factors through the scalar cache, six streams per row.
+__device__ __forceinline__ void velo_stats_tile(const TDesc& d, const PyloTensorArgs& a, int task,
+                                                const EmaConsts& e, const float* __restrict__ fac_tab,
+                                                VeloAcc& acc) {
+  constexpr int V = kTileV;
+  const TileTask tk(d, task);
+  const float* f0 = fac_tab + d.fac_off[0];
+  const float* f1 = fac_tab + d.fac_off[1];
+  float fb[V][4];
+#pragma unroll
+  for (int v = 0; v < V; ++v) load_vec_o<4>(f1 + v * 4, tk.col * 16u, fb[v]);
+  const unsigned lo = (threadIdx.x & 63) * (V * 4u);
+  const float *g = a.grad + tk.first, *p = a.param + tk.first, *m0 = a.mom + tk.first,
+              *m1 = a.mom + d.n + tk.first, *m2 = a.mom + 2 * d.n + tk.first, *rms = a.rms + tk.first;
+  const float* fr = f0 + (size_t)tk.r0 * 4;
+#pragma unroll 2
+  for (int r = tk.r0; r < tk.r1; ++r) {
+    float xg[V], xp[V], x0[V], x1[V], x2[V], xr[V], fa[4];
+    load_vec_nt<V>(g, lo, xg);
+    load_vec_nt<V>(p, lo, xp);
+    load_vec_nt<V>(m0, lo, x0);
+    load_vec_nt<V>(m1, lo, x1);
+    load_vec_nt<V>(m2, lo, x2);
+    load_vec_nt<V>(rms, lo, xr);
+    load_uniform<4>(fr, fa);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      const float gg = clampf(xg[v], a.clip_val);
+      float m[3] = {x0[v], x1[v], x2[v]};
+      float rr = xr[v];
+      lstm_sums(m, rr, acc.lstm);
+      ema_update(e, gg, m, rr);
+      const float rfcf[3] = {fa[0] * fb[v][0], fa[1] * fb[v][1], fa[2] * fb[v][2]};
+      float f[kNStat];
+      lo_features(gg, xp[v], m, rr, rfcf, 1e-6f, f);
+#pragma unroll
+      for (int c = 0; c < kNStat; ++c) acc.ch[stat_channel(c)] = fmaf(f[c], f[c], acc.ch[stat_channel(c)]);
+    }
+    g += d.C0; p += d.C0; m0 += d.C0; m1 += d.C0; m2 += d.C0; rms += d.C0; fr += 4;
+  }
+}
+
 // Non-factored tensor: the 30 channels of one element (Velo_naive.py:60-68,439-451,478-488).
 // m, rms, v are the accumulators after this step's update; fm_eps is added to v under the
 // power -1/2 of the last group (0 for VeLO, 1e-6 for AdafacLO).
@@ -210,7 +255,10 @@ __global__ __launch_bounds__(kThreads) void k_velo_stats(const TDesc* __restrict
   for (int c = 0; c < 30; ++c) acc.ch[c] = 0.0f;
 #pragma unroll
   for (int c = 0; c < 8; ++c) acc.lstm[c] = 0.0f;
-  if (d.mode == kModeFac2D) {
+  if (d.tile_nct > 0) {
+    const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (task < d.tile_ntask) velo_stats_tile(d, a, task, e, fac_tab, acc);
+  } else if (d.mode == kModeFac2D) {
     if (d.vec == 4) velo_stats_fac<4, false>(d, a, it.a, e, fac_tab, acc);
     else velo_stats_fac<1, false>(d, a, it.a, e, fac_tab, acc);
   } else if (d.mode == kModeFacND) {
@@ -352,17 +400,24 @@ __global__ __launch_bounds__(kThreads) void k_velo_mix(const float* __restrict__
                                                        const float* __restrict__ wft, const float* __restrict__ bf,
                                                        const float* __restrict__ h_state, float* __restrict__ xT) {
   __shared__ float mx_s[kWaves][64];
-  const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, grp = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int u = blockIdx.x * 64 + lane;
   const bool ok = u < H;
+  // the lane's weight columns stay in registers; the feature rows are wave-uniform (scalar loads)
+  float w2[30], wf[30];
+#pragma unroll
+  for (int k = 0; k < 30; ++k) {
+    w2[k] = ok ? w2t[k * H + u] : 0.0f;
+    wf[k] = ok ? wft[k * H + u] : 0.0f;
+  }
+  const float b2u = ok ? b2[u] : 0.0f, bfu = ok ? bf[u] : 0.0f;
   float mx = 0.0f;  // relu output is >= 0
   for (int r = grp; r < T; r += kWaves) {
-    float acc = ok ? b2[u] : 0.0f;
-    const float* xr = xfeat + (size_t)r * kXW;
-    if (ok) {
+    float xr[30];
+    load_uniform<30>(xfeat + (size_t)r * kXW, xr);
+    float acc = b2u;
 #pragma unroll
-      for (int k = 0; k < 30; ++k) acc = fmaf(xr[k], w2t[k * H + u], acc);
-    }
+    for (int k = 0; k < 30; ++k) acc = fmaf(xr[k], w2[k], acc);
     mx = fmaxf(mx, acc);
   }
   mx_s[grp][lane] = mx;
@@ -372,10 +427,11 @@ __global__ __launch_bounds__(kThreads) void k_velo_mix(const float* __restrict__
   for (int r = grp; r < Tpad; r += kWaves) {
     float acc = 0.0f, hv = 0.0f;
     if (r < T) {
-      acc = bf[u];
-      const float* xr = xfeat + (size_t)r * kXW;
+      float xr[30];
+      load_uniform<30>(xfeat + (size_t)r * kXW, xr);
+      acc = bfu;
 #pragma unroll
-      for (int k = 0; k < 30; ++k) acc = fmaf(xr[k], wft[k * H + u], acc);
+      for (int k = 0; k < 30; ++k) acc = fmaf(xr[k], wf[k], acc);
       acc += v;
       hv = h_state[(size_t)r * H + u];
     }
@@ -468,6 +524,7 @@ __global__ __launch_bounds__(kThreads) void k_velo_heads(const TDesc* __restrict
   __syncthreads();
   for (int j = threadIdx.x; j < K; j += kThreads) {
     float acc = bc[j];
+#pragma unroll 16
     for (int u = 0; u < H; ++u) acc = fmaf(hs[u], wct[(size_t)u * K + j], acc);
     ctrl[j] = acc;
     if (controls_out != nullptr) controls_out[(size_t)r * K + j] = acc;
@@ -486,6 +543,7 @@ __global__ __launch_bounds__(kThreads) void k_velo_heads(const TDesc* __restrict
   const float lr_mult = ((red[0] + red[1]) + (red[2] + red[3])) + blr[0];
   for (int q = threadIdx.x; q < kVBank; q += kThreads) {
     float acc = 0.0f;
+#pragma unroll 16
     for (int i = 0; i < K; ++i) acc = fmaf(ctrl[i], bank[(size_t)i * kVBank + q], acc);
     wm[q] = (acc / (float)K) * 100.0f;
   }
@@ -505,8 +563,9 @@ __global__ __launch_bounds__(kThreads) void k_velo_heads(const TDesc* __restrict
   if (threadIdx.x < 4) { cn[120 + threadIdx.x] = wm[120 + threadIdx.x]; wf[kVB1 + threadIdx.x] = wm[120 + threadIdx.x]; }
   if (threadIdx.x < 16) wf[kVWH + threadIdx.x] = wm[124 + (threadIdx.x % 4) * 4 + threadIdx.x / 4];   // (in,out)
   if (threadIdx.x < 4) wf[kVBH + threadIdx.x] = wm[140 + threadIdx.x];
-  if (threadIdx.x < 8) wf[kVWO + threadIdx.x] = wm[144 + (threadIdx.x % 2) * 4 + threadIdx.x / 2];    // [k][j<2]
-  if (threadIdx.x < 2) wf[kVBO + threadIdx.x] = wm[156 + threadIdx.x];
+  if (threadIdx.x < 16)   // [k][j], j < 2 used
+    wf[kVWO + threadIdx.x] = (threadIdx.x % 4) < 2 ? wm[144 + (threadIdx.x % 4) * 4 + threadIdx.x / 4] : 0.0f;
+  if (threadIdx.x < 4) wf[kVBO + threadIdx.x] = threadIdx.x < 2 ? wm[156 + threadIdx.x] : 0.0f;
   if (threadIdx.x == 0) {
     const double n = (double)(d.n > 0 ? d.n : 1);
     wf[kVPS] = sqrtf((float)(totals[(size_t)t * kStatW + 2] / n) + 1e-9f);
@@ -525,8 +584,8 @@ __device__ __forceinline__ float velo_update(float p, const float (&h1)[4], cons
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     const float hk = fmaxf(h1[k], 0.0f);
-    o0 = fmaf(hk, w[kVWO + k * 2 + 0], o0);
-    o1 = fmaf(hk, w[kVWO + k * 2 + 1], o1);
+    o0 = fmaf(hk, w[kVWO + k * 4 + 0], o0);
+    o1 = fmaf(hk, w[kVWO + k * 4 + 1], o1);
   }
   float step = w[kVPS] * ((o0 * expf(o1 * a.exp_mult)) * a.step_mult);
   step = w[kVLR] * step;
@@ -592,6 +651,103 @@ __device__ __forceinline__ void velo_apply_fac(const TDesc& d, const PyloTensorA
   }
 }
 
+// The apply pass over one wave task of the column-resident walk, with the 30->4->4->2 MLP as
+// lane-local 4x4x1 fp32 outer products on the matrix pipe: weight group v (four consecutive floats
+// of the folded block) sits in lanes 4*(v%16).. of register v/16; biases enter as a rank-1 update
+// with the constant 1.
+__device__ __forceinline__ void velo_apply_tile(const TDesc& d, const PyloTensorArgs& a, int task,
+                                                const EmaConsts& e, const float* __restrict__ fac_tab,
+                                                const float* __restrict__ term_tab, const float* wbase) {
+  constexpr int V = kTileV;
+  const TileTask tk(d, task);
+  const int lane = threadIdx.x & 63;
+  float wreg[3];
+#pragma unroll
+  for (int r = 0; r < 3; ++r) wreg[r] = *(const gfloat*)(wbase + r * 64 + lane);
+  const cfloat* ws = launder(wbase);
+  const float pscale = ws[kVPS], lr_mult = ws[kVLR];
+  const float exp_scale = a.exp_mult * 1.44269504088896341f;
+  constexpr int gWH = kVWH / 4, gBH = kVBH / 4, gWO = kVWO / 4, gBO = kVBO / 4;
+  const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
+  const float* f0 = fac_tab + d.fac_off[0];
+  const float* f1 = fac_tab + d.fac_off[1];
+  const float* t0 = term_tab + d.term_off[0];
+  const float* t1 = term_tab + d.term_off[1];
+  float fb[V][4], tb[V][4];
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    load_vec_o<4>(f1 + v * 4, tk.col * 16u, fb[v]);
+    load_vec_o<4>(t1 + v * 4, tk.col * 16u, tb[v]);
+  }
+  const unsigned lo = lane * (V * 4u);
+  const float* g = a.grad + tk.first;
+  float *p = a.param + tk.first, *m0 = a.mom + tk.first, *m1 = a.mom + d.n + tk.first,
+        *m2 = a.mom + 2 * d.n + tk.first, *rms = a.rms + tk.first;
+  const float* fr = f0 + (size_t)tk.r0 * 4;
+  const float* tr = t0 + (size_t)tk.r0 * 4;
+  const float wd_lr = a.weight_decay * a.lr;
+  for (int r = tk.r0; r < tk.r1; ++r) {
+    float xg[V], xp[V], x0[V], x1[V], x2[V], xr[V], fa[4], ta[4];
+    load_vec_nt<V>(g, lo, xg);
+    load_vec_nt<V>(p, lo, xp);
+    load_vec_nt<V>(m0, lo, x0);
+    load_vec_nt<V>(m1, lo, x1);
+    load_vec_nt<V>(m2, lo, x2);
+    load_vec_nt<V>(rms, lo, xr);
+    load_uniform<4>(fr, fa);
+    load_uniform<4>(tr, ta);
+    float f[V][kNStat];
+    v4f h[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      const float gg = clampf(xg[v], a.clip_val);
+      float m[3] = {x0[v], x1[v], x2[v]};
+      ema_update(e, gg, m, xr[v]);
+      x0[v] = m[0]; x1[v] = m[1]; x2[v] = m[2];
+      const float rfcf[3] = {fa[0] * fb[v][0], fa[1] * fb[v][1], fa[2] * fb[v][2]};
+      lo_features(gg, xp[v], m, xr[v], rfcf, 1e-6f, f[v]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) h[v][j] = ta[j] + tb[v][j];
+    }
+    store_vec_nt<V>(m0, lo, x0);
+    store_vec_nt<V>(m1, lo, x1);
+    store_vec_nt<V>(m2, lo, x2);
+    store_vec_nt<V>(rms, lo, xr);
+#pragma unroll
+    for (int c = 0; c < kNStat; ++c) {
+#pragma unroll
+      for (int v = 0; v < V; ++v) h[v] = mfma_w4(wreg[c / 16], f[v][c], h[v], c % 16);
+    }
+    v4f g2[V], o[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) g2[v] = mfma_w4(wreg[gBH / 16], 1.0f, zero, gBH % 16);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+#pragma unroll
+      for (int v = 0; v < V; ++v) g2[v] = mfma_w4(wreg[(gWH + k) / 16], relu(h[v][k]), g2[v], (gWH + k) % 16);
+    }
+#pragma unroll
+    for (int v = 0; v < V; ++v) o[v] = mfma_w4(wreg[gBO / 16], 1.0f, zero, gBO % 16);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+#pragma unroll
+      for (int v = 0; v < V; ++v) o[v] = mfma_w4(wreg[(gWO + k) / 16], relu(g2[v][k]), o[v], (gWO + k) % 16);
+    }
+    float pn[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      float step = pscale * ((o[v][0] * __builtin_amdgcn_exp2f(o[v][1] * exp_scale)) * a.step_mult);
+      step = lr_mult * step;
+      float q = fmaf(step, -a.lr, xp[v]);
+      if (a.weight_decay > 0.0f) q = fmaf(q, -wd_lr, q);
+      pn[v] = q;
+    }
+    store_vec_o<V>(p, lo, pn);
+    g += d.C0; p += d.C0; m0 += d.C0; m1 += d.C0; m2 += d.C0; rms += d.C0;
+    fr += 4; tr += 4;
+  }
+}
+
 template <int V>
 __device__ __forceinline__ void velo_apply_vec(const TDesc& d, const PyloTensorArgs& a, int chunk,
                                                const EmaConsts& e, const PyloDecays& dec, const float* wbase) {
@@ -645,7 +801,10 @@ __global__ __launch_bounds__(kThreads) void k_velo_apply(const TDesc* __restrict
   if (a.grad == nullptr) return;
   const EmaConsts e = make_ema(dec);
   const float* w = wfold + (size_t)it.tensor * kVFold;
-  if (d.mode == kModeFac2D) {
+  if (d.tile_nct > 0) {
+    const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (task < d.tile_ntask) velo_apply_tile(d, a, task, e, fac_tab, term_tab, w);
+  } else if (d.mode == kModeFac2D) {
     if (d.vec == 4) velo_apply_fac<4, false>(d, a, it.a, e, fac_tab, term_tab, w);
     else velo_apply_fac<1, false>(d, a, it.a, e, fac_tab, term_tab, w);
   } else if (d.mode == kModeFacND) {

@@ -186,7 +186,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       }
     }
     d.blk0 = (int)L.el_items.size();
-    if (kind == PYLO_KIND_CELO2 && d.mode == kModeFac2D && n > 0 && d.C0 % kTileCols == 0 && env_matrix_pipe()) {
+    if ((kind == PYLO_KIND_CELO2 || kind == PYLO_KIND_VELO) && d.mode == kModeFac2D && n > 0 && d.C0 % kTileCols == 0 && env_matrix_pipe()) {
       d.tile_nct = d.C0 / kTileCols;
       d.tile_ntask = d.tile_nct * ((d.R0 + kTileRows - 1) / kTileRows);
       for (int b = 0; b * 4 < d.tile_ntask; ++b) L.el_items.push_back(Item{t, b, 0, 0});

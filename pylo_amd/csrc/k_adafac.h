@@ -53,6 +53,48 @@ __device__ __forceinline__ void adafac_stats_fac(const TDesc& d, const PyloTenso
   }
 }
 
+// Column-resident walk of one wave task (wide 2-D tensors), as in VeLO's statistics pass.
+__device__ __forceinline__ void adafac_stats_tile(const TDesc& d, const PyloTensorArgs& a, int task,
+                                                  const EmaConsts& e, const float* __restrict__ fac_tab,
+                                                  VeloAcc& acc) {
+  constexpr int V = kTileV;
+  const TileTask tk(d, task);
+  const float* f0 = fac_tab + d.fac_off[0];
+  const float* f1 = fac_tab + d.fac_off[1];
+  float fb[V][4];
+#pragma unroll
+  for (int v = 0; v < V; ++v) load_vec_o<4>(f1 + v * 4, tk.col * 16u, fb[v]);
+  const unsigned lo = (threadIdx.x & 63) * (V * 4u);
+  const float *g = a.grad + tk.first, *p = a.param + tk.first, *m0 = a.mom + tk.first,
+              *m1 = a.mom + d.n + tk.first, *m2 = a.mom + 2 * d.n + tk.first, *rms = a.rms + tk.first;
+  const float* fr = f0 + (size_t)tk.r0 * 4;
+#pragma unroll 2
+  for (int r = tk.r0; r < tk.r1; ++r) {
+    float xg[V], xp[V], x0[V], x1[V], x2[V], xr[V], fa[4];
+    load_vec_nt<V>(g, lo, xg);
+    load_vec_nt<V>(p, lo, xp);
+    load_vec_nt<V>(m0, lo, x0);
+    load_vec_nt<V>(m1, lo, x1);
+    load_vec_nt<V>(m2, lo, x2);
+    load_vec_nt<V>(rms, lo, xr);
+    load_uniform<4>(fr, fa);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      const float gg = clampf(xg[v], a.clip_val);
+      float m[3] = {x0[v], x1[v], x2[v]};
+      float rr = xr[v];
+      ema_update(e, gg, m, rr);
+      const float rfcf[3] = {fa[0] * fb[v][0], fa[1] * fb[v][1], fa[2] * fb[v][2]};
+      float f[kNStat];
+      lo_features(gg, xp[v], m, rr, rfcf, 1e-6f, f);
+#pragma unroll
+      for (int c = 0; c < kNStat; ++c)
+        if (adafac_channel(stat_channel(c))) acc.ch[stat_channel(c)] = fmaf(f[c], f[c], acc.ch[stat_channel(c)]);
+    }
+    g += d.C0; p += d.C0; m0 += d.C0; m1 += d.C0; m2 += d.C0; rms += d.C0; fr += 4;
+  }
+}
+
 template <int V>
 __device__ __forceinline__ void adafac_stats_vec(const TDesc& d, const PyloTensorArgs& a, int chunk,
                                                  const EmaConsts& e, const PyloDecays& dec, VeloAcc& acc) {
@@ -88,7 +130,10 @@ __global__ __launch_bounds__(kThreads) void k_adafac_stats(const TDesc* __restri
   VeloAcc acc;
 #pragma unroll
   for (int c = 0; c < 30; ++c) acc.ch[c] = 0.0f;
-  if (d.mode == kModeFac2D) {
+  if (d.tile_nct > 0) {
+    const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (task < d.tile_ntask) adafac_stats_tile(d, a, task, e, fac_tab, acc);
+  } else if (d.mode == kModeFac2D) {
     if (d.vec == 4) adafac_stats_fac<4, false>(d, a, it.a, e, fac_tab, acc);
     else adafac_stats_fac<1, false>(d, a, it.a, e, fac_tab, acc);
   } else if (d.mode == kModeFacND) {
@@ -244,6 +289,112 @@ __device__ __forceinline__ void adafac_apply_vec(const TDesc& d, const PyloTenso
   }
 }
 
+// Row of the 30-channel first layer that per-element channel c (0..15) of a factored tensor uses:
+// {0, 2..13, 27, 28, 29}.
+__device__ __forceinline__ int adafac_elem_row(int c) { return c == 0 ? 0 : (c <= 12 ? c + 1 : c + 14); }
+
+// The apply pass over one wave task of the column-resident walk (one column per lane), with the
+// 16 -> 32 -> 32 -> 2 element MLP as lane-local 4x4x1 fp32 outer products on the matrix pipe.
+// Weight group v (four consecutive outputs of one input) sits in lanes 4*(v%16).. of register v/16:
+// 8 registers hold the scaled first layer of this tensor, 16 the hidden layer, 2 the output layer
+// (padded to four outputs) and one the hidden bias (groups 0..7) and output bias (group 8).  The
+// kernel is bound by the fp32 matrix rate (425 instructions of 256 FMAs per 64 elements).
+__device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTensorArgs& a, int task,
+                                                  const EmaConsts& e, const float* __restrict__ fac_tab,
+                                                  const float* __restrict__ term_tab, const float* wfold_t,
+                                                  const float* net) {
+  const TileTask tk(d, task, d.atile_nct, 1);
+  const int lane = threadIdx.x & 63;
+  float w1r[8], whr[16], wor[2], br;
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const int i = r * 64 + lane;  // compact (16, 32) index
+    w1r[r] = *(const gfloat*)(wfold_t + adafac_elem_row(i / kAH) * kAH + (i % kAH));
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) whr[r] = *(const gfloat*)(net + kAWH + r * 64 + lane);
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int i = r * 64 + lane, k = i / 4, j = i % 4;
+    wor[r] = j < 2 ? *(const gfloat*)(net + kAWO + k * 2 + j) : 0.0f;
+  }
+  br = lane < kAH ? *(const gfloat*)(net + kABH + lane) : (lane < kAH + 2 ? *(const gfloat*)(net + kABO + lane - kAH) : 0.0f);
+  const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
+  const float exp_scale = a.exp_mult * 1.44269504088896341f;
+  const float wd_lr = a.weight_decay * a.lr;
+  // the column's 32 first-layer terms are re-read from the cache every row (the registers are
+  // needed for a third wave per SIMD: one wave issues a 4x4x1 MFMA at most every 16 cycles)
+  float fb[4];
+  load_vec_o<4>(fac_tab + d.fac_off[1], tk.col * 16u, fb);
+  const float* tcol = term_tab + d.term_off[1];
+  const unsigned lo = lane * 4u;
+  const float* g = a.grad + tk.first;
+  float *p = a.param + tk.first, *m0 = a.mom + tk.first, *m1 = a.mom + d.n + tk.first,
+        *m2 = a.mom + 2 * d.n + tk.first, *rms = a.rms + tk.first;
+  const float* fr = fac_tab + d.fac_off[0] + (size_t)tk.r0 * 4;
+  const float* tr = term_tab + d.term_off[0] + (size_t)tk.r0 * kAH;
+  for (int r = tk.r0; r < tk.r1; ++r) {
+    float xg[1], xp[1], x0[1], x1[1], x2[1], xr[1], fa[4], ta[kAH];
+    load_vec_nt<1>(g, lo, xg);
+    load_vec_nt<1>(p, lo, xp);
+    load_vec_nt<1>(m0, lo, x0);
+    load_vec_nt<1>(m1, lo, x1);
+    load_vec_nt<1>(m2, lo, x2);
+    load_vec_nt<1>(rms, lo, xr);
+    load_uniform<4>(fr, fa);
+    load_uniform<kAH>(tr, ta);
+    const float gg = clampf(xg[0], a.clip_val);
+    float m[3] = {x0[0], x1[0], x2[0]};
+    ema_update(e, gg, m, xr[0]);
+    x0[0] = m[0]; x1[0] = m[1]; x2[0] = m[2];
+    store_vec_nt<1>(m0, lo, x0);
+    store_vec_nt<1>(m1, lo, x1);
+    store_vec_nt<1>(m2, lo, x2);
+    store_vec_nt<1>(rms, lo, xr);
+    const float rfcf[3] = {fa[0] * fb[0], fa[1] * fb[1], fa[2] * fb[2]};
+    float f18[kNStat];
+    lo_features(gg, xp[0], m, xr[0], rfcf, 1e-6f, f18);
+    const float f[16] = {f18[0], f18[2], f18[3], f18[4], f18[5], f18[6], f18[7], f18[8], f18[9], f18[10],
+                         f18[11], f18[12], f18[13], f18[15], f18[16], f18[17]};
+    v4f h[8], g2[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      float t4[4];
+      load_vec_o<4>(tcol + q * 4, tk.col * (kAH * 4u), t4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) h[q][j] = ta[q * 4 + j] + t4[j];
+    }
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) h[q] = mfma_w4(w1r[(c * 8 + q) / 16], f[c], h[q], (c * 8 + q) % 16);
+    }
+#pragma unroll
+    for (int q = 0; q < 8; ++q) g2[q] = mfma_w4(br, 1.0f, zero, q);
+#pragma unroll
+    for (int k = 0; k < kAH; ++k) {
+      const float hk = relu(h[k / 4][k % 4]);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) g2[q] = mfma_w4(whr[(k * 8 + q) / 16], hk, g2[q], (k * 8 + q) % 16);
+    }
+    // two accumulators halve the dependent chain of the output layer
+    v4f oa = mfma_w4(br, 1.0f, zero, 8), ob = zero;
+#pragma unroll
+    for (int k = 0; k < kAH; k += 2) {
+      oa = mfma_w4(wor[k / 16], relu(g2[k / 4][k % 4]), oa, k % 16);
+      ob = mfma_w4(wor[(k + 1) / 16], relu(g2[(k + 1) / 4][(k + 1) % 4]), ob, (k + 1) % 16);
+    }
+    const float o0 = oa[0] + ob[0], o1 = oa[1] + ob[1];
+    const float step = (o0 * __builtin_amdgcn_exp2f(o1 * exp_scale)) * a.step_mult;
+    float pn[1];
+    pn[0] = fmaf(step, -a.lr, xp[0]);
+    if (a.weight_decay > 0.0f) pn[0] = fmaf(pn[0], -wd_lr, pn[0]);
+    store_vec_o<1>(p, lo, pn);
+    g += d.C0; p += d.C0; m0 += d.C0; m1 += d.C0; m2 += d.C0; rms += d.C0;
+    fr += 4; tr += kAH;
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void k_adafac_apply(const TDesc* __restrict__ descs,
                                                            const PyloTensorArgs* __restrict__ dyn,
                                                            const Item* __restrict__ items,
@@ -263,6 +414,21 @@ __global__ __launch_bounds__(kThreads) void k_adafac_apply(const TDesc* __restri
   if (d.mode == kModeFac2D) adafac_apply_fac<false>(d, a, base, count, e, fac_tab, term_tab, w, net);
   else if (d.mode == kModeFacND) adafac_apply_fac<true>(d, a, base, count, e, fac_tab, term_tab, w, net);
   else adafac_apply_vec(d, a, base, count, e, dec, w, net, bias_eff);
+}
+
+// The apply pass for tensors walked column-resident (items hold four wave tasks each).
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3)))
+void k_adafac_apply_tile(const TDesc* __restrict__ descs, const PyloTensorArgs* __restrict__ dyn,
+                         const Item* __restrict__ items, const float* __restrict__ fac_tab,
+                         const float* __restrict__ term_tab, PyloDecays dec, const float* __restrict__ wfold,
+                         const float* __restrict__ net) {
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (task >= d.atile_ntask) return;
+  adafac_apply_tile(d, a, task, make_ema(dec), fac_tab, term_tab, wfold + (size_t)it.tensor * kAFold, net);
 }
 
 }  // namespace pylo

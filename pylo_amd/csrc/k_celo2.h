@@ -226,18 +226,19 @@ __device__ __forceinline__ void celo2_stats_chunk(const TDesc& d, const PyloTens
   }
 }
 
-// Geometry of one wave task of the column-resident walk.
+// Geometry of one wave task of the column-resident walk: V columns per lane, nct column tiles.
 struct TileTask {
   int r0, r1;          // rows
   unsigned col;        // the lane's first column
   long long first;     // element index of (r0, first column of the wave)
-  __device__ __forceinline__ TileTask(const TDesc& d, int task) {
-    const int ct = task % d.tile_nct, rr = task / d.tile_nct;
+  __device__ __forceinline__ TileTask(const TDesc& d, int task, int nct, int V) {
+    const int ct = task % nct, rr = task / nct;
     r0 = rr * kTileRows;
     r1 = r0 + kTileRows < d.R0 ? r0 + kTileRows : d.R0;
-    col = (unsigned)ct * kTileCols + (threadIdx.x & 63) * kTileV;
-    first = (long long)r0 * d.C0 + (long long)ct * kTileCols;
+    col = (unsigned)ct * (64 * V) + (threadIdx.x & 63) * V;
+    first = (long long)r0 * d.C0 + (long long)ct * (64 * V);
   }
+  __device__ __forceinline__ TileTask(const TDesc& d, int task) : TileTask(d, task, d.tile_nct, kTileV) {}
 };
 
 // Statistics of one wave task: the column factors stay in registers, the row factors arrive through

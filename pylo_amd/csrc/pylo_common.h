@@ -72,6 +72,9 @@ struct TDesc {
   // [ (w % tile_nct) * kTileCols, +kTileCols ) of rows [ (w / tile_nct) * kTileRows, +kTileRows );
   // element block a holds tasks 4a .. 4a+3.  tile_nct == 0: linear chunks instead.
   int tile_nct, tile_ntask;
+  // AdafacLO's apply pass walks one column per lane (its 32-wide MLP leaves no registers for two):
+  // same scheme with 64 columns per wave task; apply block a holds tasks 4a .. 4a+3.
+  int atile_nct, atile_ntask;
 };
 
 // Field of vector 0 or 1 chosen at run time.  Indexing the by-value descriptor with a run-time

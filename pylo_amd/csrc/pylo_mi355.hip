@@ -63,12 +63,12 @@ bool factored_dims(int kind, const PyloTensorShape& s, int* dc, int* dr) {
 
 struct Layout {
   std::vector<TDesc> descs;
-  std::vector<Item> p0_items, nd_items, el_items, v0a_items, v0b_items;
+  std::vector<Item> p0_items, nd_items, el_items, ap_items, ga_items, v0a_items, v0b_items;
   std::vector<int> fac_list;
   std::vector<int> dc, dr;
   int H = 8;  // width of the first MLP layer (terms per row / column)
   int Tpad = 0;
-  size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_el_items, off_v0a_items, off_v0b_items, off_fac_list,
+  size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_el_items, off_ap_items, off_ga_items, off_v0a_items, off_v0b_items, off_fac_list,
       off_part, off_gsq, off_flag, off_globals, off_fac, off_term, off_v0part, off_bscale, off_stats, off_wfold,
       off_chan_ms, off_totals, off_xfeat, off_lossfeat, off_xT, off_canon, total;
 };
@@ -186,7 +186,8 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       }
     }
     d.blk0 = (int)L.el_items.size();
-    if ((kind == PYLO_KIND_CELO2 || kind == PYLO_KIND_VELO) && d.mode == kModeFac2D && n > 0 && d.C0 % kTileCols == 0 && env_matrix_pipe()) {
+    const bool wide = d.mode == kModeFac2D && n > 0 && env_matrix_pipe();
+    if (wide && d.C0 % kTileCols == 0) {
       d.tile_nct = d.C0 / kTileCols;
       d.tile_ntask = d.tile_nct * ((d.R0 + kTileRows - 1) / kTileRows);
       for (int b = 0; b * 4 < d.tile_ntask; ++b) L.el_items.push_back(Item{t, b, 0, 0});
@@ -194,6 +195,17 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       for (long long c = 0; c * chunk < n; ++c) L.el_items.push_back(Item{t, (int)c, 0, 0});
     }
     d.nblk = (int)L.el_items.size() - d.blk0;
+    // blocks of AdafacLO's apply pass: one column per lane where the tensor allows it (ap_items,
+    // k_adafac_apply_tile), linear chunks otherwise (ga_items, k_adafac_apply)
+    if (kind == PYLO_KIND_ADAFAC) {
+      if (wide && d.C0 % 64 == 0) {
+        d.atile_nct = d.C0 / 64;
+        d.atile_ntask = d.atile_nct * ((d.R0 + kTileRows - 1) / kTileRows);
+        for (int b = 0; b * 4 < d.atile_ntask; ++b) L.ap_items.push_back(Item{t, b, 0, 0});
+      } else {
+        for (long long c = 0; c * chunk < n; ++c) L.ga_items.push_back(Item{t, (int)c, 0, 0});
+      }
+    }
   }
   size_t off = 0;
   auto take = [&](size_t bytes) {
@@ -207,6 +219,8 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_p0_items = take(sizeof(Item) * L.p0_items.size());
   L.off_nd_items = take(sizeof(Item) * L.nd_items.size());
   L.off_el_items = take(sizeof(Item) * L.el_items.size());
+  L.off_ap_items = take(sizeof(Item) * L.ap_items.size());
+  L.off_ga_items = take(sizeof(Item) * L.ga_items.size());
   L.off_v0a_items = take(sizeof(Item) * L.v0a_items.size());
   L.off_v0b_items = take(sizeof(Item) * L.v0b_items.size());
   L.off_fac_list = take(sizeof(int) * nfac);
@@ -294,6 +308,8 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_p0_items, L.p0_items.data(), sizeof(Item) * L.p0_items.size());
   if (e == hipSuccess) e = up(L.off_nd_items, L.nd_items.data(), sizeof(Item) * L.nd_items.size());
   if (e == hipSuccess) e = up(L.off_el_items, L.el_items.data(), sizeof(Item) * L.el_items.size());
+  if (e == hipSuccess) e = up(L.off_ap_items, L.ap_items.data(), sizeof(Item) * L.ap_items.size());
+  if (e == hipSuccess) e = up(L.off_ga_items, L.ga_items.data(), sizeof(Item) * L.ga_items.size());
   if (e == hipSuccess) e = up(L.off_fac_list, L.fac_list.data(), sizeof(int) * L.fac_list.size());
   if (e == hipSuccess) e = up(L.off_v0a_items, L.v0a_items.data(), sizeof(Item) * L.v0a_items.size());
   if (e == hipSuccess) e = up(L.off_v0b_items, L.v0b_items.data(), sizeof(Item) * L.v0b_items.size());
@@ -644,9 +660,15 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   HIP_TRY(mark());
   hipLaunchKernelGGL(k_adafac_fold, dim3(T), dim3(kThreads), 0, s, descs, dyn, totals, net, wfold);
   HIP_TRY(mark());
-  if (n_el > 0)
-    hipLaunchKernelGGL(k_adafac_apply, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, term_tab, dec,
+  const Item* ap_items = P->at<Item>(L.off_ap_items);
+  const Item* ga_items = P->at<Item>(L.off_ga_items);
+  const int n_ap = (int)L.ap_items.size(), n_ga = (int)L.ga_items.size();
+  if (n_ga > 0)
+    hipLaunchKernelGGL(k_adafac_apply, dim3(n_ga), dim3(kThreads), 0, s, descs, dyn, ga_items, fac_tab, term_tab, dec,
                        wfold, net, (const float*)bias_eff);
+  if (n_ap > 0)
+    hipLaunchKernelGGL(k_adafac_apply_tile, dim3(n_ap), dim3(kThreads), 0, s, descs, dyn, ap_items, fac_tab, term_tab,
+                       dec, wfold, net);
   HIP_TRY(mark());
   mark.done();
   HIP_TRY(hipGetLastError());

@@ -30,6 +30,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 B_P0, B_STATS, B_APPLY = 4, 24, 44   # algorithmic bytes per element of a >=2-D tensor, per pass
 B_ADAM = 44                    # 1-D AdamW branch: read g,p,m0..2,rms; write m0..2,rms,p
+# HBM bytes of one k_celo2_apply launch on the GPT-2-small set, from rocprofv3 FETCH_SIZE x 2.000 KiB +
+# WRITE_SIZE x 1.000 KiB (factors calibrated on a 1 GiB copy in the same runs; --calib-copy)
+TRAFFIC_APPLY_GPT2S = 5.528e9
 
 
 def gpt2_small_shapes():
@@ -196,7 +199,8 @@ def main():
         "whole_step_note": "optimizer.step(): fused path + torch Newton-Schulz (fp32 GEMMs), normalise, apply",
         "launch_ms": {nm: float(v) for nm, v in zip(names, mean)},
         "roofline": {"bound": "hbm", "kernel": "k_celo2_apply", "achieved": apply_gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": apply_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "unit": "GB/s", "frac": apply_gbs / HBM_PEAK_GBS,
+                     "traffic": TRAFFIC_APPLY_GPT2S if a.workload == "gpt2s" else None,
                      "algorithmic_bytes_per_launch": n2d * B_APPLY, "avg_launch_ms": apply_ms},
     }
     if not a.no_cpu_baseline:
@@ -264,7 +268,8 @@ def other_workload(a):
         "whole_step_ms": wall_ms,
         "launch_ms": {nm: float(v) for nm, v in zip(names, mean)},
         "roofline": {"bound": "hbm", "kernel": apply_kernel, "achieved": apply_gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": apply_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "unit": "GB/s", "frac": apply_gbs / HBM_PEAK_GBS,
+                     "traffic": TRAFFIC_APPLY_GPT2S if a.workload == "gpt2s" else None,
                      "avg_launch_ms": float(mean[k])},
     }
     print(json.dumps(out))

@@ -13,6 +13,9 @@ namespace pylo {
 // Host-packed network (floats), all (in, out):
 //   w1 (30,32) rows in the 30-channel order (rows 1 and 14 zero) | b1 32 | w_time (11,32) |
 //   w_h (32,32) | b_h 32 | w_o (32,2) | b_o 2
+#ifndef PYLO_ADAFAC_WAVES
+#define PYLO_ADAFAC_WAVES 3
+#endif
 constexpr int kAH = 32;
 constexpr int kAW1 = 0, kAB1 = 960, kAWT = 992, kAWH = 1344, kABH = 2368, kAWO = 2400, kABO = 2464, kANet = 2466;
 constexpr int kAFold = 960;  // per-tensor first-layer rows scaled by the channel normalisers
@@ -293,98 +296,148 @@ __device__ __forceinline__ void adafac_apply_vec(const TDesc& d, const PyloTenso
 // {0, 2..13, 27, 28, 29}.
 __device__ __forceinline__ int adafac_elem_row(int c) { return c == 0 ? 0 : (c <= 12 ? c + 1 : c + 14); }
 
-// The apply pass over one wave task of the column-resident walk (one column per lane), with the
-// 16 -> 32 -> 32 -> 2 element MLP as lane-local 4x4x1 fp32 outer products on the matrix pipe.
-// Weight group v (four consecutive outputs of one input) sits in lanes 4*(v%16).. of register v/16:
-// 8 registers hold the scaled first layer of this tensor, 16 the hidden layer, 2 the output layer
-// (padded to four outputs) and one the hidden bias (groups 0..7) and output bias (group 8).  The
-// kernel is bound by the fp32 matrix rate (425 instructions of 256 FMAs per 64 elements).
+// The apply pass over one wave task of the column-resident walk (one column per lane).  The
+// 16 -> 32 -> 32 -> 2 element MLP runs as v_mfma_f32_16x16x4_f32 products with the *elements* as the
+// N dimension: D(16 units x 16 elements) += A(16 units x 4 inputs) B(4 inputs x 16 elements).
+// Operand layouts (lane = 16 q + e): A holds unit e, input q; B holds input q of element e; D holds
+// units 4q..4q+3 of element e.  The D layout of one layer is a valid B layout of the next (input
+// slot (q, r) = unit 16 b + 4 q + r), so activations never move between lanes; only the 16 features
+// of the 64 elements a wave holds (one element per lane) are regrouped once per row through LDS
+// into four groups of 16 elements.  Per row of 64 elements: 32 + 64 MFMAs for the two layers and 8
+// that sum the output layer's per-lane partial products over q (A = 1); 1 600 FMAs per element in
+// all, bound by the fp32 matrix rate.
+__device__ __forceinline__ v4f mfma16(float a, float b, v4f c) {
+  return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
 __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTensorArgs& a, int task,
                                                   const EmaConsts& e, const float* __restrict__ fac_tab,
                                                   const float* __restrict__ term_tab, const float* wfold_t,
-                                                  const float* net) {
+                                                  const float* net, float* xch /* LDS [16][64] of this wave */) {
   const TileTask tk(d, task, d.atile_nct, 1);
-  const int lane = threadIdx.x & 63;
-  float w1r[8], whr[16], wor[2], br;
+  const int lane = threadIdx.x & 63, q = lane >> 4, el = lane & 15;
+  // A operands: first layer [b][c'] (inputs 4c'+q), hidden layer [bo][b][r] (input 16b+4q+r)
+  float a1[2][4], a2[2][2][4], wo[2][4][2];
+  v4f bh[2];
 #pragma unroll
-  for (int r = 0; r < 8; ++r) {
-    const int i = r * 64 + lane;  // compact (16, 32) index
-    w1r[r] = *(const gfloat*)(wfold_t + adafac_elem_row(i / kAH) * kAH + (i % kAH));
+  for (int b = 0; b < 2; ++b) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      a1[b][c] = *(const gfloat*)(wfold_t + adafac_elem_row(4 * c + q) * kAH + 16 * b + el);
+#pragma unroll
+    for (int bi = 0; bi < 2; ++bi) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) a2[b][bi][r] = *(const gfloat*)(net + kAWH + (16 * bi + 4 * q + r) * kAH + 16 * b + el);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      bh[b][r] = *(const gfloat*)(net + kABH + 16 * b + 4 * q + r);
+      wo[b][r][0] = *(const gfloat*)(net + kAWO + (16 * b + 4 * q + r) * 2 + 0);
+      wo[b][r][1] = *(const gfloat*)(net + kAWO + (16 * b + 4 * q + r) * 2 + 1);
+    }
   }
-#pragma unroll
-  for (int r = 0; r < 16; ++r) whr[r] = *(const gfloat*)(net + kAWH + r * 64 + lane);
-#pragma unroll
-  for (int r = 0; r < 2; ++r) {
-    const int i = r * 64 + lane, k = i / 4, j = i % 4;
-    wor[r] = j < 2 ? *(const gfloat*)(net + kAWO + k * 2 + j) : 0.0f;
-  }
-  br = lane < kAH ? *(const gfloat*)(net + kABH + lane) : (lane < kAH + 2 ? *(const gfloat*)(net + kABO + lane - kAH) : 0.0f);
+  const cfloat* nw = launder(net);
+  const float bo0 = nw[kABO + 0], bo1 = nw[kABO + 1];
   const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
   const float exp_scale = a.exp_mult * 1.44269504088896341f;
   const float wd_lr = a.weight_decay * a.lr;
-  // the column's 32 first-layer terms are re-read from the cache every row (the registers are
-  // needed for a third wave per SIMD: one wave issues a 4x4x1 MFMA at most every 16 cycles)
   float fb[4];
   load_vec_o<4>(fac_tab + d.fac_off[1], tk.col * 16u, fb);
+  // column terms of element (16 g + el), units 16 b + 4 q ..: one voffset, immediates per (g, b)
   const float* tcol = term_tab + d.term_off[1];
+  const unsigned tcol_off = ((tk.col - lane + el) * kAH + 4 * q) * 4u;
+  const unsigned trow_off = 4 * q * 4u;
   const unsigned lo = lane * 4u;
+  float* xw = xch + lane;                 // feature c of this lane's element goes to xch[c][lane]
+  const float* xr = xch + q * 64 + el;    // input 4c'+q of element 16g+el is xch[4c'+q][16g+el]
   const float* g = a.grad + tk.first;
   float *p = a.param + tk.first, *m0 = a.mom + tk.first, *m1 = a.mom + d.n + tk.first,
         *m2 = a.mom + 2 * d.n + tk.first, *rms = a.rms + tk.first;
   const float* fr = fac_tab + d.fac_off[0] + (size_t)tk.r0 * 4;
   const float* tr = term_tab + d.term_off[0] + (size_t)tk.r0 * kAH;
   for (int r = tk.r0; r < tk.r1; ++r) {
-    float xg[1], xp[1], x0[1], x1[1], x2[1], xr[1], fa[4], ta[kAH];
+    float xg[1], xp[1], x0[1], x1[1], x2[1], xr_[1], fa[4];
     load_vec_nt<1>(g, lo, xg);
     load_vec_nt<1>(p, lo, xp);
     load_vec_nt<1>(m0, lo, x0);
     load_vec_nt<1>(m1, lo, x1);
     load_vec_nt<1>(m2, lo, x2);
-    load_vec_nt<1>(rms, lo, xr);
+    load_vec_nt<1>(rms, lo, xr_);
     load_uniform<4>(fr, fa);
-    load_uniform<kAH>(tr, ta);
+    float ta[2][4];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) load_vec_o<4>(tr + 16 * b, trow_off, ta[b]);
     const float gg = clampf(xg[0], a.clip_val);
     float m[3] = {x0[0], x1[0], x2[0]};
-    ema_update(e, gg, m, xr[0]);
+    ema_update(e, gg, m, xr_[0]);
     x0[0] = m[0]; x1[0] = m[1]; x2[0] = m[2];
     store_vec_nt<1>(m0, lo, x0);
     store_vec_nt<1>(m1, lo, x1);
     store_vec_nt<1>(m2, lo, x2);
-    store_vec_nt<1>(rms, lo, xr);
+    store_vec_nt<1>(rms, lo, xr_);
     const float rfcf[3] = {fa[0] * fb[0], fa[1] * fb[1], fa[2] * fb[2]};
     float f18[kNStat];
-    lo_features(gg, xp[0], m, xr[0], rfcf, 1e-6f, f18);
+    lo_features(gg, xp[0], m, xr_[0], rfcf, 1e-6f, f18);
     const float f[16] = {f18[0], f18[2], f18[3], f18[4], f18[5], f18[6], f18[7], f18[8], f18[9], f18[10],
                          f18[11], f18[12], f18[13], f18[15], f18[16], f18[17]};
-    v4f h[8], g2[8];
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      float t4[4];
-      load_vec_o<4>(tcol + q * 4, tk.col * (kAH * 4u), t4);
+    for (int c = 0; c < 16; ++c) xw[c * 64] = f[c];
+    float o0 = 0.0f, o1 = 0.0f;
+    // two groups of 16 elements at a time: four independent accumulator chains
 #pragma unroll
-      for (int j = 0; j < 4; ++j) h[q][j] = ta[q * 4 + j] + t4[j];
+    for (int gP = 0; gP < 4; gP += 2) {
+      v4f h[2][2], g2[2][2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          float tb[4];
+          load_vec_o<4>(tcol + (16 * (gP + u)) * kAH + 16 * b, tcol_off, tb);
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) h[u][b][rr] = ta[b][rr] + tb[rr];
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const float bv = xr[(4 * c) * 64 + 16 * (gP + u)];
+          h[u][0] = mfma16(a1[0][c], bv, h[u][0]);
+          h[u][1] = mfma16(a1[1][c], bv, h[u][1]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u) { g2[u][0] = bh[0]; g2[u][1] = bh[1]; }
+#pragma unroll
+      for (int bi = 0; bi < 2; ++bi) {
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const float hv = relu(h[u][bi][rr]);
+            g2[u][0] = mfma16(a2[0][bi][rr], hv, g2[u][0]);
+            g2[u][1] = mfma16(a2[1][bi][rr], hv, g2[u][1]);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        float p0 = 0.0f, p1 = 0.0f;
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+            const float gv = relu(g2[u][b][rr]);
+            p0 = fmaf(gv, wo[b][rr][0], p0);
+            p1 = fmaf(gv, wo[b][rr][1], p1);
+          }
+        }
+        const v4f t0 = mfma16(1.0f, p0, zero), t1 = mfma16(1.0f, p1, zero);  // sums over q, in every lane
+        if (q == gP + u) { o0 = t0[0]; o1 = t1[0]; }
+      }
     }
-#pragma unroll
-    for (int c = 0; c < 16; ++c) {
-#pragma unroll
-      for (int q = 0; q < 8; ++q) h[q] = mfma_w4(w1r[(c * 8 + q) / 16], f[c], h[q], (c * 8 + q) % 16);
-    }
-#pragma unroll
-    for (int q = 0; q < 8; ++q) g2[q] = mfma_w4(br, 1.0f, zero, q);
-#pragma unroll
-    for (int k = 0; k < kAH; ++k) {
-      const float hk = relu(h[k / 4][k % 4]);
-#pragma unroll
-      for (int q = 0; q < 8; ++q) g2[q] = mfma_w4(whr[(k * 8 + q) / 16], hk, g2[q], (k * 8 + q) % 16);
-    }
-    // two accumulators halve the dependent chain of the output layer
-    v4f oa = mfma_w4(br, 1.0f, zero, 8), ob = zero;
-#pragma unroll
-    for (int k = 0; k < kAH; k += 2) {
-      oa = mfma_w4(wor[k / 16], relu(g2[k / 4][k % 4]), oa, k % 16);
-      ob = mfma_w4(wor[(k + 1) / 16], relu(g2[(k + 1) / 4][(k + 1) % 4]), ob, (k + 1) % 16);
-    }
-    const float o0 = oa[0] + ob[0], o1 = oa[1] + ob[1];
+    o0 += bo0;
+    o1 += bo1;
     const float step = (o0 * __builtin_amdgcn_exp2f(o1 * exp_scale)) * a.step_mult;
     float pn[1];
     pn[0] = fmaf(step, -a.lr, xp[0]);
@@ -417,7 +470,7 @@ __global__ __launch_bounds__(kThreads) void k_adafac_apply(const TDesc* __restri
 }
 
 // The apply pass for tensors walked column-resident (items hold four wave tasks each).
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3)))
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PYLO_ADAFAC_WAVES)))
 void k_adafac_apply_tile(const TDesc* __restrict__ descs, const PyloTensorArgs* __restrict__ dyn,
                          const Item* __restrict__ items, const float* __restrict__ fac_tab,
                          const float* __restrict__ term_tab, PyloDecays dec, const float* __restrict__ wfold,
@@ -426,9 +479,12 @@ void k_adafac_apply_tile(const TDesc* __restrict__ descs, const PyloTensorArgs* 
   const TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
-  const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  __shared__ float xch[kWaves][16 * 64];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int task = it.a * 4 + wave;
   if (task >= d.atile_ntask) return;
-  adafac_apply_tile(d, a, task, make_ema(dec), fac_tab, term_tab, wfold + (size_t)it.tensor * kAFold, net);
+  adafac_apply_tile(d, a, task, make_ema(dec), fac_tab, term_tab, wfold + (size_t)it.tensor * kAFold, net,
+                    xch[wave]);
 }
 
 }  // namespace pylo

@@ -17,7 +17,7 @@ constexpr int kP0Rows = 128;    // rows of one row/column-sum tile; tile columns
 constexpr int kElemIters = 8;   // an element chunk is kThreads * vec * kElemIters elements
 constexpr int kTileV = 2;       // column-resident walk: a wave owns 64 * kTileV columns ...
 constexpr int kTileCols = 64 * kTileV;
-constexpr int kTileRows = 32;   // ... and walks this many rows of them
+constexpr int kTileRows = 16;   // ... and walks this many rows of them
 constexpr int kNStat = 18;      // feature channels that vary per element (the other 12 are
                                 // functions of the row or of the column only)
 constexpr int kV0aEnt = 64;     // vector entries per k_v0a block

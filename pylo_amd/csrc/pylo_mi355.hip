@@ -348,7 +348,10 @@ static const char* kAdafacLaunches[] = {"k_p0(sums)", "k_p0_nd", "k_v0a", "k_ada
 
 int pylo_mi355_plan_num_launches(const PyloPlan* P) {
   if (!P) return -1;
-  return P->kind == PYLO_KIND_CELO2 ? 8 : P->kind == PYLO_KIND_VELO ? 12 : P->kind == PYLO_KIND_ADAFAC ? 9 : -1;
+  constexpr int n_celo2 = sizeof(kCelo2Launches) / sizeof(kCelo2Launches[0]);
+  constexpr int n_velo = sizeof(kVeloLaunches) / sizeof(kVeloLaunches[0]);
+  constexpr int n_adafac = sizeof(kAdafacLaunches) / sizeof(kAdafacLaunches[0]);
+  return P->kind == PYLO_KIND_CELO2 ? n_celo2 : P->kind == PYLO_KIND_VELO ? n_velo : P->kind == PYLO_KIND_ADAFAC ? n_adafac : -1;
 }
 
 const char* pylo_mi355_plan_launch_name(const PyloPlan* P, int launch) {

@@ -60,7 +60,8 @@ def test_adafac_matches_oracle_mixed_shapes():
 
     torch.manual_seed(9)
     net = MetaMLP(39, 32, 1)
-    shapes = [(256, 516), (516, 256), (300, 260), (37, 101), (32, 16, 3, 3), (1, 1, 48), (1000,), (7,), (64, 64)]
+    shapes = [(256, 516), (516, 256), (300, 260), (37, 101), (32, 16, 3, 3), (1, 1, 48), (1000,), (7,), (64, 64),
+              (70, 384), (33, 128), (1, 128), (130, 192), (3, 64)]  # column-resident walks (128 / 64 columns a wave)
     gen = torch.Generator().manual_seed(23)
     init = [torch.randn(s, generator=gen) * 0.3 for s in shapes]
     cpu = [v.clone() for v in init]

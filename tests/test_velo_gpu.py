@@ -78,7 +78,8 @@ def test_velo_matches_oracle_full_size():
         rnn.lstm_init_state[0].normal_(0, 0.1)
         rnn.lstm_init_state[1].normal_(0, 0.1)
     mlp = VeLOMLP()
-    shapes = [(256, 1028), (1028, 256), (300, 260), (37, 101), (32, 16, 3, 3), (1, 1, 48), (1000,), (7,), (1,),
+    shapes = [(70, 384), (33, 128), (1, 128), (130, 192),  # column-resident walk: ragged row ranges, one row
+              (256, 1028), (1028, 256), (300, 260), (37, 101), (32, 16, 3, 3), (1, 1, 48), (1000,), (7,), (1,),
               (64, 64), (2, 3, 64, 64)]
     gen = torch.Generator().manual_seed(17)
     init = [torch.randn(s, generator=gen) * 0.3 for s in shapes]

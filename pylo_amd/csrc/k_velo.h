@@ -351,8 +351,10 @@ __global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restr
   const int c = threadIdx.x % kStatW, gI = threadIdx.x / kStatW;
   if (gI < G) {
     double s = 0.0;
-    if (a.grad != nullptr && c < 38)
+    if (a.grad != nullptr && c < 38) {
+#pragma unroll 16
       for (int b = gI; b < d.nblk; b += G) s += stats_part[(size_t)(d.blk0 + b) * kStatW + c];
+    }
     part[gI][c] = s;
   }
   __syncthreads();

@@ -25,15 +25,22 @@ _IN, _HID = 30, 8
 
 
 def newton_schulz(x: torch.Tensor, coeffs, iters: int, eps: float) -> torch.Tensor:
-    """Quintic Newton-Schulz over the last two dims (pylo/optim/CELO2_naive.py:59-73)."""
+    """Quintic Newton-Schulz over the last two dims (pylo/optim/CELO2_naive.py:59-73).  A leading
+    batch dim runs as strided-batched library GEMMs with the scalings folded into them."""
     tall = x.shape[-2] > x.shape[-1]
     if tall:
         x = x.transpose(-2, -1)
     x = x / (torch.linalg.norm(x, dim=(-2, -1), keepdim=True) + eps)
     c0, c1, c2 = coeffs
-    for _ in range(iters):
-        a = x @ x.transpose(-2, -1)
-        x = c0 * x + (c1 * a + c2 * (a @ a)) @ x
+    if x.dim() == 3:
+        for _ in range(iters):
+            a = torch.bmm(x, x.transpose(-2, -1))
+            b = torch.baddbmm(a, a, a, beta=c1, alpha=c2)         # c1 A + c2 A A
+            x = torch.baddbmm(x, b, x, beta=c0, alpha=1.0)        # c0 X + B X
+    else:
+        for _ in range(iters):
+            a = x @ x.transpose(-2, -1)
+            x = c0 * x + (c1 * a + c2 * (a @ a)) @ x
     return x.transpose(-2, -1) if tall else x
 
 
@@ -149,16 +156,19 @@ class ELO_CELO2_CUDA(Optimizer):
         flags = [_lib.F_ADAM if adam else 0 for _, _p, adam in tensors]
         self._plan = _lib.Plan(_lib.KIND_CELO2, shapes, flags, self.device)
         self._plan_key = key
-        # one flat buffer for the raw steps of all MLP tensors, 256-byte aligned slices
-        offs, total = [], 0
-        for _, p, adam in tensors:
-            offs.append(total)
+        # Raw steps of the MLP tensors: tensors of one parameter group and one shape share a
+        # contiguous (count, *shape) buffer, so Newton-Schulz and the normalisation run batched.
+        buckets = {}
+        for i, (group, p, adam) in enumerate(tensors):
             if not adam:
-                total += (p.numel() + 63) // 64 * 64
-        flat = torch.empty(max(total, 1), dtype=torch.float32, device=self.device)
-        self._raw = [None if adam else flat[o:o + p.numel()].view(p.shape)
-                     for o, (_, p, adam) in zip(offs, tensors)]
-        self._raw_flat = flat
+                buckets.setdefault((id(group), tuple(p.shape)), []).append(i)
+        self._raw = [None] * len(tensors)
+        self._raw_groups = []
+        for (_gid, shape), idx in buckets.items():
+            buf = torch.empty((len(idx),) + shape, dtype=torch.float32, device=self.device)
+            for j, i in enumerate(idx):
+                self._raw[i] = buf[j]
+            self._raw_groups.append((buf, idx))
 
     def _init_state(self, state, p):
         shape = tuple(p.shape)
@@ -293,16 +303,34 @@ class ELO_CELO2_CUDA(Optimizer):
     def finish_step(self, tensors):
         """Newton-Schulz, RMS normalisation and the parameter update of the MLP tensors
         (pylo/optim/ELO_CELO2_cuda.py:288-296)."""
-        for i, (group, p, adam) in enumerate(tensors):
-            if adam or p.grad is None:
+        for buf, idx in self._raw_groups:
+            group = tensors[idx[0]][0]
+            ps = [tensors[i][1] for i in idx]
+            if any(p.grad is None for p in ps):
+                # a tensor of the bucket sat this step out: one by one
+                for i in idx:
+                    p = tensors[i][1]
+                    if p.grad is None:
+                        continue
+                    step = self._raw[i]
+                    if group["param_scale_mult"]:
+                        step = step * torch.sqrt(torch.mean(p * p) + 1e-9)
+                    if group["orthogonalize"]:
+                        step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
+                    step = rms_normalize(step, [-2, -1]) * group["rmsmult"]
+                    p.add_(step + group["weight_decay"] * p, alpha=-group["lr"])
                 continue
-            step = self._raw[i]
+            step = buf
             if group["param_scale_mult"]:
-                step = step * torch.sqrt(torch.mean(p * p) + 1e-9)
+                n = ps[0].numel()
+                sq = torch.stack(torch._foreach_norm(ps)) ** 2 / n
+                step = step * torch.sqrt(sq + 1e-9).view(-1, 1, 1)
             if group["orthogonalize"]:
                 step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
-            step = rms_normalize(step, list(range(p.dim()))[-2:]) * group["rmsmult"]
-            p.add_(step + group["weight_decay"] * p, alpha=-group["lr"])
+            step = rms_normalize(step, [-2, -1]) * group["rmsmult"]
+            upd = torch._foreach_mul(ps, group["weight_decay"])
+            torch._foreach_add_(upd, list(step.unbind(0)))
+            torch._foreach_add_(ps, upd, alpha=-group["lr"])
 
 
 def _factored_dims_host(shape):

@@ -127,6 +127,18 @@ int pylo_mi355_celo2_step(PyloPlan* plan, const PyloTensorArgs* args, const Pylo
                           const float* mlp, void* stream);
 
 /*
+ * ELO-CELO2 finishing pass (replaces the last two lines of the per-tensor loop in
+ * ELO_CELO2_cuda.py:288-296 / CELO2_naive.py:54-56): for every non-ADAM tensor with a gradient,
+ * with x = the step after Newton-Schulz (read from `step_out`, same shape as the parameter, contiguous):
+ *     step = x * rsqrt(1e-9 + mean(x^2 over the tensor)) * step_mult      (step_mult carries rmsmult)
+ *     param <- param - lr * (step + weight_decay * param)
+ * Fields read per tensor: grad (only as "takes part" flag), param, step_out, lr, weight_decay,
+ * step_mult.  PYLO_F_ADAM tensors are skipped.  Three launches: sum of squares per 8192-element
+ * block, per-tensor scale (fixed-order fp64 sum), update.  16 bytes per element.
+ */
+int pylo_mi355_celo2_finish(PyloPlan* plan, const PyloTensorArgs* args, void* stream);
+
+/*
  * VeLO step (replaces velo_cuda_kernel.velo_kernel_simple, pylo/csrc/velo_kernel.cu:370-457, for every
  * tensor at once, plus velo_cuda.py:183-211 (loss features), :213-252 (per-tensor LSTM features),
  * pylo/models/VeLO_RNN.py:43-66,110-135 (mixing + LSTM cell + heads), pylo/models/VeLO_MLP.py:92-126

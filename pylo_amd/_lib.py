@@ -79,6 +79,7 @@ def load():
     lib.pylo_mi355_plan_launch_name.restype = C.c_char_p
     lib.pylo_mi355_celo2_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.c_void_p,
                                           C.c_void_p]
+    lib.pylo_mi355_celo2_finish.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
     lib.pylo_mi355_velo_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.POINTER(VeloNets),
                                          C.POINTER(VeloStep), C.c_void_p]
     lib.pylo_mi355_adafac_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.c_void_p, C.c_float,
@@ -165,6 +166,10 @@ class Plan:
     def celo2_step(self, decays: Decays, mlp: torch.Tensor, stream: int) -> None:
         check(load().pylo_mi355_celo2_step(self._h, self.args.ctypes.data, C.byref(decays),
                                            mlp.data_ptr(), stream), "celo2_step")
+
+    def celo2_finish(self, args: np.ndarray, stream: int) -> None:
+        """Normalise + apply after Newton-Schulz; `args` is a table like `self.args` (own array)."""
+        check(load().pylo_mi355_celo2_finish(self._h, args.ctypes.data, stream), "celo2_finish")
 
     def velo_step(self, decays: Decays, nets: VeloNets, step: VeloStep, stream: int) -> None:
         check(load().pylo_mi355_velo_step(self._h, self.args.ctypes.data, C.byref(decays), C.byref(nets),

@@ -699,4 +699,104 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PYLO_A
                          term_tab + d.term_off[0], term_tab + d.term_off[1], w);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Finishing pass of ELO-CELO2 (after Newton-Schulz): x = step_out,
+//   step = x * rsqrt(1e-9 + mean x^2) * rmsmult;  p <- p - lr * (step + wd * p)
+// (CELO2_naive.py:54-56, ELO_CELO2_cuda.py:294-296).  Linear 8192-element blocks.
+// ---------------------------------------------------------------------------------------------
+constexpr int kFinElems = kThreads * 4 * kElemIters;
+
+__global__ __launch_bounds__(kThreads) void k_celo2_sumsq(const TDesc* __restrict__ descs,
+                                                          const PyloTensorArgs* __restrict__ dyn,
+                                                          const Item* __restrict__ items,
+                                                          double* __restrict__ fin_part) {
+  __shared__ float red[kWaves];
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  const long long base = (long long)it.a * kFinElems;
+  const long long left = d.n - base;
+  const unsigned lim = left < (long long)kFinElems ? (unsigned)left : (unsigned)kFinElems;
+  const float* x = a.step_out + base;
+  float s = 0.0f;
+  if (d.n % 4 == 0) {
+#pragma unroll
+    for (int i = 0; i < kElemIters; ++i) {
+      const unsigned off = (i * kThreads + threadIdx.x) * 4u;
+      if (off < lim) {
+        float v[4];
+        load_vec_nt<4>(x, off * 4u, v);
+        s += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+      }
+    }
+  } else {
+    for (unsigned off = threadIdx.x; off < lim; off += kThreads) {
+      const float v = *(const gfloat*)(x + off);
+      s = fmaf(v, v, s);
+    }
+  }
+  s = wave_sum(s);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0)
+    fin_part[blockIdx.x] = ((double)red[0] + (double)red[1]) + ((double)red[2] + (double)red[3]);
+}
+
+__global__ __launch_bounds__(kThreads) void k_celo2_finscale(const TDesc* __restrict__ descs,
+                                                             const PyloTensorArgs* __restrict__ dyn,
+                                                             const int* __restrict__ fac_list,
+                                                             const double* __restrict__ fin_part,
+                                                             float* __restrict__ fin_scale) {
+  __shared__ double red[kWaves];
+  const int t = fac_list[blockIdx.x];
+  const TDesc d = descs[t];
+  if (dyn[t].grad == nullptr) return;
+  double s = 0.0;
+#pragma unroll 8
+  for (int b = threadIdx.x; b < d.fin_nblk; b += kThreads) s += fin_part[d.fin_blk0 + b];
+  s = wave_sum(s);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const float ms = (float)(((red[0] + red[1]) + (red[2] + red[3])) / (double)d.n);
+    fin_scale[t] = rsq(1e-9f + ms);
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void k_celo2_update(const TDesc* __restrict__ descs,
+                                                           const PyloTensorArgs* __restrict__ dyn,
+                                                           const Item* __restrict__ items,
+                                                           const float* __restrict__ fin_scale) {
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  const long long base = (long long)it.a * kFinElems;
+  const long long left = d.n - base;
+  const unsigned lim = left < (long long)kFinElems ? (unsigned)left : (unsigned)kFinElems;
+  const float* x = a.step_out + base;
+  float* p = a.param + base;
+  const float sc = fin_scale[it.tensor], rm = a.step_mult, wd = a.weight_decay, nlr = -a.lr;
+  if (d.n % 4 == 0) {
+#pragma unroll
+    for (int i = 0; i < kElemIters; ++i) {
+      const unsigned off = (i * kThreads + threadIdx.x) * 4u;
+      if (off < lim) {
+        float v[4], q[4];
+        load_vec_nt<4>(x, off * 4u, v);
+        load_vec_o<4>(p, off * 4u, q);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) q[j] = fmaf(nlr, (v[j] * sc) * rm + wd * q[j], q[j]);
+        store_vec_o<4>(p, off * 4u, q);
+      }
+    }
+  } else {
+    for (unsigned off = threadIdx.x; off < lim; off += kThreads) {
+      const float v = *(const gfloat*)(x + off), q = *(const gfloat*)(p + off);
+      *(gfloat*)(p + off) = fmaf(nlr, (v * sc) * rm + wd * q, q);
+    }
+  }
+}
+
 }  // namespace pylo

@@ -75,6 +75,7 @@ struct TDesc {
   // AdafacLO's apply pass walks one column per lane (its 32-wide MLP leaves no registers for two):
   // same scheme with 64 columns per wave task; apply block a holds tasks 4a .. 4a+3.
   int atile_nct, atile_ntask;
+  int fin_blk0, fin_nblk;  // ELO-CELO2 finishing pass: range of 8192-element blocks (rows of its partials)
 };
 
 // Field of vector 0 or 1 chosen at run time.  Indexing the by-value descriptor with a run-time

@@ -63,12 +63,12 @@ bool factored_dims(int kind, const PyloTensorShape& s, int* dc, int* dr) {
 
 struct Layout {
   std::vector<TDesc> descs;
-  std::vector<Item> p0_items, nd_items, el_items, ap_items, ga_items, v0a_items, v0b_items;
+  std::vector<Item> p0_items, nd_items, el_items, ap_items, ga_items, fin_items, v0a_items, v0b_items;
   std::vector<int> fac_list;
   std::vector<int> dc, dr;
   int H = 8;  // width of the first MLP layer (terms per row / column)
   int Tpad = 0;
-  size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_el_items, off_ap_items, off_ga_items, off_v0a_items, off_v0b_items, off_fac_list,
+  size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_el_items, off_ap_items, off_ga_items, off_fin_items, off_finpart, off_finscale, off_v0a_items, off_v0b_items, off_fac_list,
       off_part, off_gsq, off_flag, off_globals, off_fac, off_term, off_v0part, off_bscale, off_stats, off_wfold,
       off_chan_ms, off_totals, off_xfeat, off_lossfeat, off_xT, off_canon, total;
 };
@@ -195,6 +195,12 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       for (long long c = 0; c * chunk < n; ++c) L.el_items.push_back(Item{t, (int)c, 0, 0});
     }
     d.nblk = (int)L.el_items.size() - d.blk0;
+    // blocks of ELO-CELO2's finishing pass (after Newton-Schulz): linear 8192-element pieces of the MLP tensors
+    if (kind == PYLO_KIND_CELO2 && d.mode != kModeFlat) {
+      d.fin_blk0 = (int)L.fin_items.size();
+      for (long long c = 0; c * kFinElems < n; ++c) L.fin_items.push_back(Item{t, (int)c, 0, 0});
+      d.fin_nblk = (int)L.fin_items.size() - d.fin_blk0;
+    }
     // blocks of AdafacLO's apply pass: one column per lane where the tensor allows it (ap_items,
     // k_adafac_apply_tile), linear chunks otherwise (ga_items, k_adafac_apply)
     if (kind == PYLO_KIND_ADAFAC) {
@@ -221,6 +227,9 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_el_items = take(sizeof(Item) * L.el_items.size());
   L.off_ap_items = take(sizeof(Item) * L.ap_items.size());
   L.off_ga_items = take(sizeof(Item) * L.ga_items.size());
+  L.off_fin_items = take(sizeof(Item) * L.fin_items.size());
+  L.off_finpart = take(sizeof(double) * L.fin_items.size());
+  L.off_finscale = take(sizeof(float) * T);
   L.off_v0a_items = take(sizeof(Item) * L.v0a_items.size());
   L.off_v0b_items = take(sizeof(Item) * L.v0b_items.size());
   L.off_fac_list = take(sizeof(int) * nfac);
@@ -310,6 +319,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_el_items, L.el_items.data(), sizeof(Item) * L.el_items.size());
   if (e == hipSuccess) e = up(L.off_ap_items, L.ap_items.data(), sizeof(Item) * L.ap_items.size());
   if (e == hipSuccess) e = up(L.off_ga_items, L.ga_items.data(), sizeof(Item) * L.ga_items.size());
+  if (e == hipSuccess) e = up(L.off_fin_items, L.fin_items.data(), sizeof(Item) * L.fin_items.size());
   if (e == hipSuccess) e = up(L.off_fac_list, L.fac_list.data(), sizeof(int) * L.fac_list.size());
   if (e == hipSuccess) e = up(L.off_v0a_items, L.v0a_items.data(), sizeof(Item) * L.v0a_items.size());
   if (e == hipSuccess) e = up(L.off_v0b_items, L.v0b_items.data(), sizeof(Item) * L.v0b_items.size());
@@ -530,6 +540,35 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   }
   HIP_TRY(mark());
   mark.done();
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+extern "C" int pylo_mi355_celo2_finish(PyloPlan* P, const PyloTensorArgs* args, void* stream) {
+  if (!P || P->kind != PYLO_KIND_CELO2) return fail("celo2_finish: not an ELO-CELO2 plan");
+  if (!args) return fail("celo2_finish: null argument");
+  const Layout& L = P->L;
+  for (int t = 0; t < P->T; ++t) {
+    const TDesc& d = L.descs[t];
+    const PyloTensorArgs& a = args[t];
+    if (a.grad == nullptr || d.mode == kModeFlat || d.n == 0) continue;
+    if (!a.param || !a.step_out) return fail("celo2_finish: null param/step_out pointer at tensor " + std::to_string(t));
+    const uintptr_t m = reinterpret_cast<uintptr_t>(a.param) | reinterpret_cast<uintptr_t>(a.step_out);
+    if (m % (d.n % 4 == 0 ? 16 : 4) != 0) return fail("celo2_finish: misaligned pointer at tensor " + std::to_string(t));
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (int rc = upload_args(P, args, s)) return rc;
+  const TDesc* descs = P->at<TDesc>(L.off_descs);
+  const PyloTensorArgs* dyn = P->at<PyloTensorArgs>(L.off_dyn);
+  const Item* fin_items = P->at<Item>(L.off_fin_items);
+  const int* fac_list = P->at<int>(L.off_fac_list);
+  double* fin_part = P->at<double>(L.off_finpart);
+  float* fin_scale = P->at<float>(L.off_finscale);
+  const int n_fin = (int)L.fin_items.size(), n_fac = (int)L.fac_list.size();
+  if (n_fin == 0) return 0;
+  hipLaunchKernelGGL(k_celo2_sumsq, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_part);
+  hipLaunchKernelGGL(k_celo2_finscale, dim3(n_fac), dim3(kThreads), 0, s, descs, dyn, fac_list, fin_part, fin_scale);
+  hipLaunchKernelGGL(k_celo2_update, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_scale);
   HIP_TRY(hipGetLastError());
   return 0;
 }

@@ -26,22 +26,25 @@ _IN, _HID = 30, 8
 
 def newton_schulz(x: torch.Tensor, coeffs, iters: int, eps: float) -> torch.Tensor:
     """Quintic Newton-Schulz over the last two dims (pylo/optim/CELO2_naive.py:59-73).  A leading
-    batch dim runs as strided-batched library GEMMs with the scalings folded into them."""
+    batch dim runs as strided-batched library GEMMs with the scalings folded into them.  The reference
+    transposes tall matrices so that the Gram matrix is the small one; the same products are taken
+    here on the untransposed matrix (A = X^T X, X <- c0 X + X B), which keeps the result contiguous."""
     tall = x.shape[-2] > x.shape[-1]
-    if tall:
-        x = x.transpose(-2, -1)
     x = x / (torch.linalg.norm(x, dim=(-2, -1), keepdim=True) + eps)
     c0, c1, c2 = coeffs
     if x.dim() == 3:
         for _ in range(iters):
-            a = torch.bmm(x, x.transpose(-2, -1))
+            xt = x.transpose(-2, -1)
+            a = torch.bmm(xt, x) if tall else torch.bmm(x, xt)
             b = torch.baddbmm(a, a, a, beta=c1, alpha=c2)         # c1 A + c2 A A
-            x = torch.baddbmm(x, b, x, beta=c0, alpha=1.0)        # c0 X + B X
-    else:
-        for _ in range(iters):
-            a = x @ x.transpose(-2, -1)
-            x = c0 * x + (c1 * a + c2 * (a @ a)) @ x
-    return x.transpose(-2, -1) if tall else x
+            x = torch.baddbmm(x, x, b, beta=c0) if tall else torch.baddbmm(x, b, x, beta=c0)
+        return x
+    for _ in range(iters):
+        xt = x.transpose(-2, -1)
+        a = xt @ x if tall else x @ xt
+        b = c1 * a + c2 * (a @ a)
+        x = c0 * x + (x @ b if tall else b @ x)
+    return x
 
 
 def rms_normalize(x: torch.Tensor, dims, eps: float = 1e-9) -> torch.Tensor:
@@ -169,6 +172,7 @@ class ELO_CELO2_CUDA(Optimizer):
             for j, i in enumerate(idx):
                 self._raw[i] = buf[j]
             self._raw_groups.append((buf, idx))
+        self._fin_args = np.zeros(len(tensors), dtype=_lib.ARGS_DTYPE)
 
     def _init_state(self, state, p):
         shape = tuple(p.shape)
@@ -303,6 +307,9 @@ class ELO_CELO2_CUDA(Optimizer):
     def finish_step(self, tensors):
         """Newton-Schulz, RMS normalisation and the parameter update of the MLP tensors
         (pylo/optim/ELO_CELO2_cuda.py:288-296)."""
+        fin = self._fin_args
+        fin["grad"] = 0
+        keep, any_fin = [], False   # post-Newton-Schulz matrices must outlive the launch
         for buf, idx in self._raw_groups:
             group = tensors[idx[0]][0]
             ps = [tensors[i][1] for i in idx]
@@ -327,10 +334,21 @@ class ELO_CELO2_CUDA(Optimizer):
                 step = step * torch.sqrt(sq + 1e-9).view(-1, 1, 1)
             if group["orthogonalize"]:
                 step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
-            step = rms_normalize(step, [-2, -1]) * group["rmsmult"]
-            upd = torch._foreach_mul(ps, group["weight_decay"])
-            torch._foreach_add_(upd, list(step.unbind(0)))
-            torch._foreach_add_(ps, upd, alpha=-group["lr"])
+            step = step.contiguous()
+            keep.append(step)
+            base, stride = step.data_ptr(), step[0].numel() * 4
+            for j, i in enumerate(idx):
+                fin["grad"][i] = 1          # "takes part"; the gradient itself is not read
+                fin["param"][i] = ps[j].data_ptr()
+                fin["step_out"][i] = base + j * stride
+                fin["lr"][i] = group["lr"]
+                fin["weight_decay"][i] = group["weight_decay"]
+                fin["step_mult"][i] = group["rmsmult"]
+            any_fin = True
+        if any_fin:
+            with torch.cuda.device(self.device):
+                self._plan.celo2_finish(fin, torch.cuda.current_stream(self.device).cuda_stream)
+        del keep
 
 
 def _factored_dims_host(shape):

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define PYLO_MI355_ABI_VERSION 1
+#define PYLO_MI355_ABI_VERSION 2
 #define PYLO_MAX_DIMS 8
 #define PYLO_MAX_GROUPS 8   /* parameter groups with their own step counter (VeLO) */
 
@@ -41,6 +41,9 @@ extern "C" {
 /* PyloTensorShape.flags */
 #define PYLO_F_ADAM 1 /* CELO2: update with AdamW on mom[0] / rms (1-D tensors, is_embedding groups;
                          ELO_CELO2_cuda.py:246-253) */
+#define PYLO_F_ADAM_INDEP 2 /* CELO2: AdamW with the tensor's own moments (CELO2_cuda.py:234-253): `mom`
+                               points to exp_avg (n), `rms` to exp_avg_sq (n); betas and eps come from
+                               PyloDecays.adam_*; bc1 / bc2 carry 1 - beta^adam_step of the tensor */
 
 typedef struct PyloPlan PyloPlan; /* opaque, host memory owned by the library */
 
@@ -56,6 +59,7 @@ typedef struct {
   float beta_m[3];
   float beta_rms;
   float beta_fac[3];
+  float adam_beta1, adam_beta2, adam_eps; /* PYLO_F_ADAM_INDEP tensors only (CELO2_cuda.py:113-114) */
 } PyloDecays;
 
 /* Per-tensor, per-step arguments.  Pointers are device pointers; the table itself is host

@@ -211,7 +211,12 @@ class EloCelo2Oracle:
                  momentum_decays=(0.9, 0.99, 0.999), rms_decays=(0.95,),
                  adafactor_decays=(0.9, 0.99, 0.999), exp_mult=0.0, rmsmult=1.0,
                  param_scale_mult=False, ns_coeffs=(3.4445, -4.7750, 2.0315), ns_iters=5,
-                 ns_eps=1e-8, grad_clip_val=1000.0, is_embedding: Sequence[bool] = (), device="cpu"):
+                 ns_eps=1e-8, grad_clip_val=1000.0, is_embedding: Sequence[bool] = (), device="cpu",
+                 independent_adam=None):
+        # independent_adam = (beta1, beta2, eps): the AdamW branch keeps its own exp_avg / exp_avg_sq /
+        # adam_step per tensor as CELO2_naive does (pylo/optim/CELO2_naive.py:263-283) instead of
+        # reading mom[0] / rms of the shared accumulators.
+        self.independent_adam = independent_adam
         self.params = params
         self.device = torch.device(device)
         self.net = {k: v.detach().to(F32).to(self.device) for k, v in net.items()}
@@ -309,7 +314,19 @@ class EloCelo2Oracle:
             if scale != 1.0:
                 g = g * scale
             g = torch.clamp(g, -h["grad_clip_val"], h["grad_clip_val"])
-            if h["use_adamw_for_1d"] and (p.dim() <= 1 or self.is_embedding[i]):
+            if h["use_adamw_for_1d"] and (p.dim() <= 1 or self.is_embedding[i]) and self.independent_adam:
+                b1, b2, eps = self.independent_adam
+                st = self.state[i]
+                if "exp_avg" not in st:
+                    st["exp_avg"], st["exp_avg_sq"], st["adam_step"] = torch.zeros_like(p), torch.zeros_like(p), 0
+                st["adam_step"] += 1
+                ta = st["adam_step"]
+                st["exp_avg"].mul_(b1).add_(g, alpha=1 - b1)
+                st["exp_avg_sq"].mul_(b2).addcmul_(g, g, value=1 - b2)
+                m_hat = st["exp_avg"] / (1.0 - b1 ** ta)
+                v_hat = st["exp_avg_sq"] / (1.0 - b2 ** ta)
+                p.add_(m_hat / (torch.sqrt(v_hat) + eps) + h["adam_weight_decay"] * p, alpha=-adam_lr)
+            elif h["use_adamw_for_1d"] and (p.dim() <= 1 or self.is_embedding[i]):
                 st = self.state[i]
                 _ema_(st["mom"], _bview(self.beta_m, p.dim()), g[None])
                 _ema_(st["rms"], self.beta_rms[-1], g * g)

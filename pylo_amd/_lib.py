@@ -17,6 +17,7 @@ from .build import LIB_PATH
 MAX_DIMS = 8
 KIND_CELO2, KIND_VELO, KIND_ADAFAC = 0, 1, 2
 F_ADAM = 1
+F_ADAM_INDEP = 2
 
 
 class TensorShape(C.Structure):
@@ -24,7 +25,8 @@ class TensorShape(C.Structure):
 
 
 class Decays(C.Structure):
-    _fields_ = [("beta_m", C.c_float * 3), ("beta_rms", C.c_float), ("beta_fac", C.c_float * 3)]
+    _fields_ = [("beta_m", C.c_float * 3), ("beta_rms", C.c_float), ("beta_fac", C.c_float * 3),
+                ("adam_beta1", C.c_float), ("adam_beta2", C.c_float), ("adam_eps", C.c_float)]
 
 
 # numpy mirror of PyloTensorArgs (8 pointers, 8 floats, 2 ints, no padding)
@@ -84,7 +86,7 @@ def load():
                                          C.POINTER(VeloStep), C.c_void_p]
     lib.pylo_mi355_adafac_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.c_void_p, C.c_float,
                                            C.c_void_p]
-    if lib.pylo_mi355_abi_version() != 1:
+    if lib.pylo_mi355_abi_version() != 2:
         raise RuntimeError("libpylo_mi355.so: ABI version mismatch, rebuild it")
     _lib = lib
     return lib
@@ -107,8 +109,9 @@ def make_shapes(shapes: Sequence[Sequence[int]], flags: Sequence[int]):
     return arr
 
 
-def make_decays(beta_m, beta_rms, beta_fac) -> Decays:
+def make_decays(beta_m, beta_rms, beta_fac, adam_betas=(0.9, 0.95), adam_eps=1e-8) -> Decays:
     d = Decays()
+    d.adam_beta1, d.adam_beta2, d.adam_eps = float(adam_betas[0]), float(adam_betas[1]), float(adam_eps)
     for k in range(3):
         d.beta_m[k] = float(beta_m[k])
         d.beta_fac[k] = float(beta_fac[k])

@@ -82,6 +82,38 @@ __device__ __forceinline__ void celo2_adam_chunk(const TDesc& d, const PyloTenso
   }
 }
 
+// AdamW with the tensor's own moments (CELO2_cuda.py:234-253): a.mom = exp_avg, a.rms = exp_avg_sq.
+template <int V>
+__device__ __forceinline__ void celo2_adam_indep_chunk(const TDesc& d, const PyloTensorArgs& a, int chunk,
+                                                       float scale, const PyloDecays& dec) {
+  const long long base = (long long)chunk * (kThreads * V * kElemIters);
+  const long long n = d.n;
+  const float b1 = dec.adam_beta1, ob1 = 1.0f - dec.adam_beta1, b2 = dec.adam_beta2, ob2 = 1.0f - dec.adam_beta2;
+#pragma unroll 2
+  for (int it = 0; it < kElemIters; ++it) {
+    const long long idx = base + (long long)(it * kThreads + threadIdx.x) * V;
+    if (idx >= n) break;
+    float g[V], p[V], m[V], v[V];
+    load_vec<V>(a.grad + idx, g);
+    load_vec<V>(a.param + idx, p);
+    load_vec<V>(a.mom + idx, m);
+    load_vec<V>(a.rms + idx, v);
+#pragma unroll
+    for (int q = 0; q < V; ++q) {
+      const float gg = clampf(g[q] * scale, a.clip_val);
+      m[q] = m[q] * b1 + ob1 * gg;
+      v[q] = v[q] * b2 + (ob2 * gg) * gg;
+      const float mh = m[q] / a.bc1;
+      const float vh = v[q] / a.bc2;
+      const float upd = mh / (sqrtf(vh) + dec.adam_eps);
+      p[q] = fmaf(upd + a.weight_decay * p[q], -a.lr, p[q]);
+    }
+    store_vec<V>(a.mom + idx, m);
+    store_vec<V>(a.rms + idx, v);
+    store_vec<V>(a.param + idx, p);
+  }
+}
+
 // One vector of V consecutive elements (same dim-0 index i0, dim-1 indices i1..i1+V-1).
 template <int V>
 struct ElemIn {
@@ -298,8 +330,13 @@ __global__ __launch_bounds__(kThreads) void k_celo2_stats(const TDesc* __restric
   const float scale = clip_scale(gl->gnorm, a.clip_norm);
   const EmaConsts e = make_ema(dec);
   if (d.mode == kModeFlat) {
-    if (d.vec == 4) celo2_adam_chunk<4>(d, a, it.a, scale, e);
-    else celo2_adam_chunk<1>(d, a, it.a, scale, e);
+    if (d.adam_indep) {
+      if (d.vec == 4) celo2_adam_indep_chunk<4>(d, a, it.a, scale, dec);
+      else celo2_adam_indep_chunk<1>(d, a, it.a, scale, dec);
+    } else {
+      if (d.vec == 4) celo2_adam_chunk<4>(d, a, it.a, scale, e);
+      else celo2_adam_chunk<1>(d, a, it.a, scale, e);
+    }
     return;
   }
   float acc[kNStat];

@@ -75,6 +75,7 @@ struct TDesc {
   // AdafacLO's apply pass walks one column per lane (its 32-wide MLP leaves no registers for two):
   // same scheme with 64 columns per wave task; apply block a holds tasks 4a .. 4a+3.
   int atile_nct, atile_ntask;
+  int adam_indep;          // kModeFlat: AdamW on the tensor's own two moments instead of mom[0] / rms
   int fin_blk0, fin_nblk;  // ELO-CELO2 finishing pass: range of 8192-element blocks (rows of its partials)
 };
 

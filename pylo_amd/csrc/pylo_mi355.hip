@@ -111,8 +111,9 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     int dc = -1, dr = -1;
     const bool can_factor = factored_dims(kind, s, &dc, &dr);
     if (kind == PYLO_KIND_CELO2) {
-      const bool adam = (s.flags & PYLO_F_ADAM) != 0;
+      const bool adam = (s.flags & (PYLO_F_ADAM | PYLO_F_ADAM_INDEP)) != 0;
       if (!can_factor && !adam) return fail("plan: CELO2 tensors with fewer than 2 dims must carry PYLO_F_ADAM");
+      d.adam_indep = (s.flags & PYLO_F_ADAM_INDEP) != 0;
       if (adam) d.mode = kModeFlat;
       else if (s.ndim == 2) d.mode = kModeFac2D;
       else return fail("plan: CELO2 tensors with more than 2 dims are not supported yet");

@@ -56,6 +56,8 @@ class ELO_CELO2_CUDA(Optimizer):
     """Inference-time ELO-CELO2: CELO2 MLP steps for >=2-D tensors, shared-accumulator AdamW for
     1-D tensors and ``is_embedding`` groups."""
 
+    _ADAM_FLAG = _lib.F_ADAM
+
     def __init__(
         self,
         params,
@@ -156,7 +158,7 @@ class ELO_CELO2_CUDA(Optimizer):
         if self._plan is not None:
             self._plan.close()
         shapes = [tuple(p.shape) for _, p, _a in tensors]
-        flags = [_lib.F_ADAM if adam else 0 for _, _p, adam in tensors]
+        flags = [self._ADAM_FLAG if adam else 0 for _, _p, adam in tensors]
         self._plan = _lib.Plan(_lib.KIND_CELO2, shapes, flags, self.device)
         self._plan_key = key
         # Raw steps of the MLP tensors: tensors of one parameter group and one shape share a
@@ -174,7 +176,7 @@ class ELO_CELO2_CUDA(Optimizer):
             self._raw_groups.append((buf, idx))
         self._fin_args = np.zeros(len(tensors), dtype=_lib.ARGS_DTYPE)
 
-    def _init_state(self, state, p):
+    def _init_state(self, state, p, adam):
         shape = tuple(p.shape)
         state["mom"] = torch.zeros((self.n_mom,) + shape, device=self.device)
         state["rms"] = torch.zeros(shape, device=self.device)
@@ -205,6 +207,18 @@ class ELO_CELO2_CUDA(Optimizer):
         self._fast = None
         return super().add_param_group(param_group)
 
+    # AdamW branch: which two moment buffers a tensor uses and its bias corrections this step
+    def _adam_row(self, group, state):
+        t = group["step"]
+        beta1, beta2 = float(self.beta_m[0]), float(self.beta_rms[-1])
+        return state["mom"].data_ptr(), state["rms"].data_ptr(), 1.0 - beta1 ** t, 1.0 - beta2 ** t
+
+    def _adam_corrections_fast(self, fast, per_group):
+        beta1, beta2 = float(self.beta_m[0]), float(self.beta_rms[-1])
+        adam = fast["adam"]
+        return (np.where(adam, per_group(lambda g: 1.0 - beta1 ** g["step"]), 0.0),
+                np.where(adam, per_group(lambda g: 1.0 - beta2 ** g["step"]), 0.0))
+
     def _fused_step_fast(self, fast):
         grads = [p.grad for p in fast["params"]]
         f32 = torch.float32
@@ -231,8 +245,7 @@ class ELO_CELO2_CUDA(Optimizer):
         args["exp_mult"] = per_group(lambda g: g["exp_mult"])
         args["lr"] = np.where(adam, per_group(lambda g: g["adam_lr_mult"] * g["lr"]), 0.0)
         args["weight_decay"] = np.where(adam, per_group(lambda g: g["adam_weight_decay"]), 0.0)
-        args["bc1"] = np.where(adam, per_group(lambda g: 1.0 - beta1 ** g["step"]), 0.0)
-        args["bc2"] = np.where(adam, per_group(lambda g: 1.0 - beta2 ** g["step"]), 0.0)
+        args["bc1"], args["bc2"] = self._adam_corrections_fast(fast, per_group)
         with torch.cuda.device(self.device):
             self._plan.celo2_step(self._decays, self._mlp, torch.cuda.current_stream(self.device).cuda_stream)
         return fast["tensors"]
@@ -270,19 +283,18 @@ class ELO_CELO2_CUDA(Optimizer):
                 keep.append(g)
             state = self.state[p]
             if len(state) == 0:
-                self._init_state(state, p)
+                self._init_state(state, p, adam)
             t = group["step"]
             cols["grad"][i], cols["param"][i] = g.data_ptr(), p.data_ptr()
-            cols["mom"][i], cols["rms"][i] = state["mom"].data_ptr(), state["rms"].data_ptr()
             fl["clip_norm"][i] = group["clip_norm"] if group["clip_grad"] else 0.0
             fl["clip_val"][i] = group["grad_clip_val"]
             fl["exp_mult"][i] = group["exp_mult"]
             if adam:
+                cols["mom"][i], cols["rms"][i], fl["bc1"][i], fl["bc2"][i] = self._adam_row(group, state)
                 fl["lr"][i] = group["adam_lr_mult"] * group["lr"]
                 fl["weight_decay"][i] = group["adam_weight_decay"]
-                fl["bc1"][i] = 1.0 - beta1 ** t
-                fl["bc2"][i] = 1.0 - beta2 ** t
             else:
+                cols["mom"][i], cols["rms"][i] = state["mom"].data_ptr(), state["rms"].data_ptr()
                 cols["fac_r"][i], cols["fac_c"][i] = state["fac_r"].data_ptr(), state["fac_c"].data_ptr()
                 cols["step_out"][i] = self._raw[i].data_ptr()
         args = plan.args

@@ -41,6 +41,7 @@ def _load_reference():
         VeLOMLP=m("pylo.models.VeLO_MLP").VeLOMLP,
         VeLORNN=m("pylo.models.VeLO_RNN").VeLORNN,
         ELO_CELO2_naive=m("pylo.optim.ELO_CELO2_naive").ELO_CELO2_naive,
+        CELO2_naive=m("pylo.optim.CELO2_naive").CELO2_naive,
         VeLO_naive=m("pylo.optim.Velo_naive").VeLO_naive,
         AdafacLO_naive=m("pylo.optim.AdafacLO_naive").AdafacLO_naive,
     )
@@ -69,16 +70,16 @@ def _sd_arrays(prefix, module, arrays):
 
 # ------------------------------------------------------------------ ELO-CELO2
 def celo2_case(R, name, shapes, n_steps, grad_scale, seed, cfg, net_seed=1, full=True, sample=4099,
-               init_std=1.0):
+               init_std=1.0, cls="ELO_CELO2_naive"):
     torch.manual_seed(net_seed)
     net = R["CELO2MLP"]()
     gen = torch.Generator().manual_seed(seed)
     init = [torch.randn(s, generator=gen) * init_std for s in shapes]
     params = [torch.nn.Parameter(v.clone()) for v in init]
-    opt = R["ELO_CELO2_naive"](params, network=net, hf_key=None, **cfg)
+    opt = R[cls](params, network=net, hf_key=None, **cfg)
     arrays = {}
     _sd_arrays("net", net, arrays)
-    meta = dict(kind="elo_celo2", shapes=[list(s) for s in shapes], n_steps=n_steps, cfg=cfg,
+    meta = dict(kind="elo_celo2" if cls == "ELO_CELO2_naive" else "celo2", shapes=[list(s) for s in shapes], n_steps=n_steps, cfg=cfg,
                 grad_scale=grad_scale, seed=seed, net_seed=net_seed, full=full, sample=sample,
                 init_std=init_std)
     if full:
@@ -91,9 +92,12 @@ def celo2_case(R, name, shapes, n_steps, grad_scale, seed, cfg, net_seed=1, full
         opt.step()
         for i, p in enumerate(params):
             st = opt.state[p]
-            rec = {"param": p.detach(), "mom": _to_leading(st["mom"], p.dim()),
-                   "rms": st["rms"][..., 0]}
-            if p.dim() >= 2:
+            if "exp_avg" in st:   # CELO2_naive: tensors on the AdamW branch keep their own two moments
+                rec = {"param": p.detach(), "exp_avg": st["exp_avg"], "exp_avg_sq": st["exp_avg_sq"]}
+            else:
+                rec = {"param": p.detach(), "mom": _to_leading(st["mom"], p.dim()),
+                       "rms": st["rms"][..., 0]}
+            if p.dim() >= 2 and "exp_avg" not in st:
                 # naive fac_vec_row (mean over dr, decay last) -> (3,*s with dr->1)
                 sorted_dims = np.argsort(p.shape)
                 dc, dr = int(sorted_dims[-2]), int(sorted_dims[-1])
@@ -218,6 +222,14 @@ def ctor_checksums(R):
 def main():
     R = _load_reference()
     torch.set_num_threads(8)
+    # CELO2_naive (independent AdamW moments on 1-D tensors and is_embedding groups; CELO2_naive.py:263-283)
+    celo2_case(R, "celo2_small", [(64, 32), (32, 64), (32,), (48, 24), (5,)], 8, 1.0, 12,
+               dict(lr=1e-2, adam_lr_mult=3.0, weight_decay=0.02, adam_betas=(0.8, 0.9), adam_eps=1e-6,
+                    clip_grad=True, clip_norm=2.0), cls="CELO2_naive")
+    celo2_case(R, "celo2_small_defaults", [(40, 56), (7,), (24, 24)], 6, 0.1, 13, dict(lr=1e-3),
+               cls="CELO2_naive")
+    if "--celo2-only" in sys.argv:
+        return
     ctor_checksums(R)
     # shapes of the reference's own CUDA-vs-naive test (tests/test_celo2_cuda.py:38,116)
     celo2_case(R, "elo_celo2_small_clip", [(64, 32), (32, 64), (32,), (48, 24)], 10, 3.0, 2,

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     assert len(names) >= 12, names
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in the header but not exported"
-    assert lib.pylo_mi355_abi_version() == 1
+    assert lib.pylo_mi355_abi_version() == 2
 
 
 def test_struct_sizes_match_header():
@@ -33,7 +33,7 @@ def test_struct_sizes_match_header():
 
     assert _lib.ARGS_DTYPE.itemsize == 8 * 8 + 8 * 4 + 2 * 4          # PyloTensorArgs
     assert C.sizeof(_lib.TensorShape) == 8 + 8 * 8
-    assert C.sizeof(_lib.Decays) == 7 * 4
+    assert C.sizeof(_lib.Decays) == 10 * 4            # 7 accumulator decays + adam_beta1/2, adam_eps
     assert C.sizeof(_lib.VeloNets) == 11 * 8 + 2 * 4
     assert C.sizeof(_lib.VeloStep) == 9 * 8 + 8 * 9 * 4
 
@@ -50,6 +50,9 @@ def test_workspace_sizing_and_error_paths_without_gpu():
     bad = _lib.make_shapes([(768,)], [0])
     assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, bad, 1, C.byref(n)) != 0
     assert b"PYLO_F_ADAM" in lib.pylo_mi355_last_error()
+    # the independent-moment AdamW branch (CELO2_CUDA) is a tensor flag of its own
+    indep = _lib.make_shapes([(768,), (64, 16)], [_lib.F_ADAM_INDEP, _lib.F_ADAM_INDEP])
+    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, indep, 2, C.byref(n)) == 0
     # >2-D tensors are fine for VeLO / AdafacLO, rejected (for now) on the CELO2 MLP path
     nd = _lib.make_shapes([(768, 3, 16, 16)], [0])
     assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_VELO, nd, 1, C.byref(n)) == 0
@@ -68,12 +71,14 @@ def test_optimizers_fail_loudly_without_gpu():
 
     if torch.cuda.is_available():
         pytest.skip("this check is for GPU-less hosts")
-    from pylo_amd import AdafacLO_CUDA, ELO_CELO2_CUDA, VeLO_CUDA
+    from pylo_amd import AdafacLO_CUDA, CELO2_CUDA, ELO_CELO2_CUDA, VeLO_CUDA
     from pylo_amd.models import CELO2MLP, MetaMLP, VeLOMLP, VeLORNN
 
     p = [torch.nn.Parameter(torch.zeros(4, 4))]
     with pytest.raises(RuntimeError, match="requires a GPU"):
         ELO_CELO2_CUDA(p, network=CELO2MLP(), hf_key=None)
+    with pytest.raises(RuntimeError, match="requires a GPU"):
+        CELO2_CUDA(p, network=CELO2MLP(), hf_key=None)
     with pytest.raises(RuntimeError, match="requires a GPU"):
         VeLO_CUDA(p, rnn=VeLORNN(lstm_hidden_size=64, param_inits=8), mlp=VeLOMLP(param_inits=8))
     with pytest.raises(RuntimeError, match="requires a GPU"):

@@ -58,6 +58,34 @@ def test_elo_celo2_oracle_matches_reference(name):
     print(name, "worst err / tol =", worst)
 
 
+@pytest.mark.parametrize("name", ["celo2_small", "celo2_small_defaults"])
+def test_celo2_oracle_matches_reference(name):
+    """CELO2_naive: the ELO-CELO2 arithmetic with independent AdamW moments on the AdamW branch."""
+    G = Golden(name)
+    meta, shapes = G.meta, G.shapes
+    init = [G.t(f"init/{i}") for i in range(len(shapes))]
+    params = [v.clone() for v in init]
+    cfg = dict(meta["cfg"])
+    betas, eps = cfg.pop("adam_betas", (0.9, 0.95)), cfg.pop("adam_eps", 1e-8)
+    for k, v in dict(weight_decay=0.0, clip_grad=False, adam_lr_mult=1.0).items():   # CELO2_naive defaults
+        cfg.setdefault(k, v)
+    opt = O.EloCelo2Oracle(params, G.state_dict("net"), independent_adam=(betas[0], betas[1], eps), **cfg)
+    worst = 0.0
+    for t in range(meta["n_steps"]):
+        opt.step([G.t(f"grad{t}/{i}") for i in range(len(shapes))])
+        for i, p in enumerate(params):
+            st = opt.state[i]
+            if p.dim() >= 2:
+                got = {"param": p, "mom": st["mom"], "rms": st["rms"], "fac_r": st["fac_r"], "fac_c": st["fac_c"]}
+            else:
+                got = {"param": p, "exp_avg": st["exp_avg"], "exp_avg_sq": st["exp_avg_sq"]}
+            for k, v in got.items():
+                e = max_err(v, G.t(f"step{t}/{k}/{i}"), REL, ABS)
+                worst = max(worst, e)
+                assert e <= 1.0, (name, t, k, i, e)
+    print(name, "worst err / tol =", worst)
+
+
 @pytest.mark.parametrize("name", ["velo_small", "velo_small_wd"])
 def test_velo_oracle_matches_reference(name):
     G = Golden(name)

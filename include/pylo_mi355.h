@@ -45,6 +45,17 @@ extern "C" {
                                points to exp_avg (n), `rms` to exp_avg_sq (n); betas and eps come from
                                PyloDecays.adam_*; bc1 / bc2 carry 1 - beta^adam_step of the tensor */
 
+#define PYLO_F_NAN_TO_NUM 4 /* AdafacLO kind: the (clip-scaled) gradient passes through torch.nan_to_num
+                              (ELO_cuda.py:208-211): NaN -> 0; give the tensor clip_val = FLT_MAX so that
+                              +-inf map to +-FLT_MAX as torch maps them */
+#define PYLO_F_WD_PRESTEP 8 /* AdafacLO kind: p -= lr * (step + weight_decay * p) against the pre-step
+                               parameter (ELO_naive.py:236-237; ELO_cuda.py:244-247,285-286) instead of
+                               the two-stage AdafacLO update */
+
+#define PYLO_F_GLOBAL_NORM 16 /* AdafacLO kind: the tensor's gradient is summed into the global norm of the
+                                 call; required on every tensor of a plan whose steps pass clip_norm > 0
+                                 (CELO2 plans always take the norm over all their tensors) */
+
 typedef struct PyloPlan PyloPlan; /* opaque, host memory owned by the library */
 
 typedef struct {
@@ -75,7 +86,8 @@ typedef struct {
   float* step_out;   /* (n)     CELO2: raw per-element step (celo2_kernel.cu:280), else NULL */
   float lr;          /* VeLO / AdafacLO: lr applied in-kernel; CELO2 AdamW branch: adam lr   */
   float weight_decay;/* VeLO / AdafacLO: p -= wd*lr*p after the update; CELO2 AdamW: adam wd */
-  float clip_norm;   /* CELO2: global-norm clip threshold, 0 = clipping off for this tensor  */
+  float clip_norm;   /* CELO2, AdafacLO kind (ELO_cuda.py:153-161): global-norm clip threshold over
+                        the gradients of the call, 0 = clipping off for this tensor            */
   float clip_val;    /* element-wise clamp of the gradient (1000 in the reference), 0 = off  */
   float exp_mult;
   float step_mult;
@@ -199,6 +211,8 @@ int pylo_mi355_velo_step(PyloPlan* plan, const PyloTensorArgs* args, const PyloD
  * (pylo_amd.models.pack_metamlp builds it from a MetaMLP).  `step` is the 0-based step counter fed to
  * the time features (AdafacLO_cuda.py:400).  Tensors without gradient are skipped.
  *   p -= lr * o0 * exp(o1 * exp_mult) * step_mult;  then p -= weight_decay * lr * p.
+ * ELO_CUDA (pylo/optim/ELO_cuda.py:179-288) runs on the same call: raw decays in `decays`, step_mult = 1,
+ * clip_norm > 0 for global-norm clipping, and the tensor flags PYLO_F_NAN_TO_NUM | PYLO_F_WD_PRESTEP.
  */
 int pylo_mi355_adafac_step(PyloPlan* plan, const PyloTensorArgs* args, const PyloDecays* decays,
                            const float* net, float step, void* stream);

@@ -632,11 +632,22 @@ class AdafacOracle:
                 st["exp_avg_sq_c"] = st["exp_avg_sq_r"]
         return self
 
+    def condition_grads(self, grads):
+        """AdafacLO_naive feeds the gradients as they are (max_grad_norm is applied by the caller)."""
+        return grads
+
+    def apply(self, p: torch.Tensor, unit_step: torch.Tensor) -> None:
+        """pylo/optim/AdafacLO_naive.py:305-310 (`unit_step` = direction * exp(magnitude * exp_mult))"""
+        p.add_(unit_step * self.step_mult, alpha=-self.lr)
+        if self.weight_decay > 0:
+            p.add_(p, alpha=-self.weight_decay * self.lr)
+
     @torch.no_grad()
     def step(self, grads: List[Optional[torch.Tensor]]) -> None:
         self.t += 1
         tfeat = tanh_time_embedding(self.t - 1).to(self.device)
         sd = self.net
+        grads = self.condition_grads(grads)
         for p, g, st in zip(self.params, grads, self.state):
             if g is None:
                 continue
@@ -667,7 +678,47 @@ class AdafacOracle:
             hcur = torch.relu(x @ sd["network.input.weight"].t() + sd["network.input.bias"])
             hcur = torch.relu(hcur @ sd["network.linear_0.weight"].t() + sd["network.linear_0.bias"])
             out = hcur @ sd["network.output.weight"].t() + sd["network.output.bias"]
-            step = out[..., 0] * torch.exp(out[..., 1] * self.exp_mult) * self.step_mult
-            p.add_(step, alpha=-self.lr)
-            if self.weight_decay > 0:
-                p.add_(p, alpha=-self.weight_decay * self.lr)
+            self.apply(p, out[..., 0] * torch.exp(out[..., 1] * self.exp_mult))
+
+
+class EloOracle(AdafacOracle):
+    """ELO_naive.step restated (pylo/optim/ELO_naive.py:127-238): the AdafacLO feature set and MLP with
+    the accumulator decays used as given (:76-99, no offset re-parameterisation), optional global-norm
+    clipping followed by ``nan_to_num`` of every gradient (:118-125,141-146), and the update
+    ``p -= lr * (step + weight_decay * p)`` against the pre-step parameter (:236-237).  State in
+    ELO_cuda.py:162-178's layout, which is AdafacLO_cuda's."""
+
+    def __init__(self, params, net, lr=1e-3, exp_mult=0.001, weight_decay=0.0,
+                 initial_momentum_decays=(0.9, 0.99, 0.999), initial_rms_decays=(0.999,),
+                 initial_adafactor_decays=(0.9, 0.99, 0.999), clip_grad=False, clip_norm=1.0, device="cpu"):
+        super().__init__(params, net, lr=lr, exp_mult=exp_mult, step_mult=1.0, weight_decay=weight_decay,
+                         device=device)
+        dv = self.device
+
+        def raw(v):
+            return torch.clamp(torch.tensor(v, dtype=F32, device=dv), 0.0, 1.0)
+
+        self.beta_m, self.beta_rms, self.beta_fac = (raw(initial_momentum_decays), raw(initial_rms_decays),
+                                                     raw(initial_adafactor_decays))
+        self.clip_grad, self.clip_norm = clip_grad, clip_norm
+
+    def condition_grads(self, grads):
+        scale = 1.0
+        if self.clip_grad:
+            total = torch.zeros((), device=self.device)
+            for g in grads:
+                if g is not None:
+                    total = total + g.detach().float().pow(2).sum()
+            denom = torch.clamp(torch.sqrt(total), min=self.clip_norm)
+            scale = (self.clip_norm / denom).item() if denom > 0 else 1.0
+        out = []
+        for g in grads:
+            if g is not None:
+                if scale != 1.0:
+                    g = g * scale
+                g = torch.nan_to_num(g)
+            out.append(g)
+        return out
+
+    def apply(self, p: torch.Tensor, unit_step: torch.Tensor) -> None:
+        p.add_(unit_step + self.weight_decay * p, alpha=-self.lr)

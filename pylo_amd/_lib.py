@@ -18,6 +18,7 @@ MAX_DIMS = 8
 KIND_CELO2, KIND_VELO, KIND_ADAFAC = 0, 1, 2
 F_ADAM = 1
 F_ADAM_INDEP = 2
+F_NAN_TO_NUM, F_WD_PRESTEP, F_GLOBAL_NORM = 4, 8, 16
 
 
 class TensorShape(C.Structure):

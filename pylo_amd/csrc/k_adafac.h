@@ -83,7 +83,7 @@ __device__ __forceinline__ void adafac_stats_tile(const TDesc& d, const PyloTens
     load_uniform<4>(fr, fa);
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-      const float gg = clampf(xg[v], a.clip_val);
+      const float gg = cond_grad(xg[v], d.gscale, a.clip_val, d.nan0);
       float m[3] = {x0[v], x1[v], x2[v]};
       float rr = xr[v];
       ema_update(e, gg, m, rr);
@@ -123,12 +123,14 @@ __global__ __launch_bounds__(kThreads) void k_adafac_stats(const TDesc* __restri
                                                            const PyloTensorArgs* __restrict__ dyn,
                                                            const Item* __restrict__ items,
                                                            const float* __restrict__ fac_tab, PyloDecays dec,
-                                                           double* __restrict__ stats_part) {
+                                                           double* __restrict__ stats_part,
+                                                           const Globals* __restrict__ gl) {
   __shared__ float red[kWaves][30];
   const Item it = items[blockIdx.x];
-  const TDesc d = descs[it.tensor];
+  TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
+  set_grad_scale(d, a, gl);
   const EmaConsts e = make_ema(dec);
   VeloAcc acc;
 #pragma unroll
@@ -177,12 +179,23 @@ __global__ __launch_bounds__(kThreads) void k_adafac_fold(const TDesc* __restric
   for (int i = threadIdx.x; i < 30 * kAH; i += kThreads) w[i] = net[kAW1 + i] * sc[i / kAH];
 }
 
+// Parameter update from the unit step direction * exp(magnitude * exp_mult).  AdafacLO
+// (AdafacLO_naive.py:305-310): p -= lr * step_mult * step, then p -= wd * lr * p on the updated value.
+// ELO (ELO_naive.py:236-237): p -= lr * (step + wd * p) against the pre-step parameter.
+__device__ __forceinline__ float adafac_update(const TDesc& d, const PyloTensorArgs& a, float unit_step, float p) {
+  const float step = unit_step * a.step_mult;
+  if (d.wd_prestep) return fmaf(step + a.weight_decay * p, -a.lr, p);
+  p = fmaf(step, -a.lr, p);
+  if (a.weight_decay > 0.0f) p = fmaf(p, -(a.weight_decay * a.lr), p);
+  return p;
+}
+
 // One element per lane: 16 (factored) or 28 (non-factored) scaled features -> 32 -> 32 -> 2.
 // Weights are wave-uniform and come through the scalar cache, one input row at a time.
 template <int NF>
 __device__ __forceinline__ float adafac_mlp(const float (&f)[NF], const int (&row)[NF], float (&h)[kAH],
-                                            const float* wfold_t, const float* net, const PyloTensorArgs& a,
-                                            float p) {
+                                            const float* wfold_t, const float* net, const TDesc& d,
+                                            const PyloTensorArgs& a, float p) {
   const cfloat* w1 = launder(wfold_t);
   const cfloat* nw = launder(net);
 #pragma unroll
@@ -206,10 +219,7 @@ __device__ __forceinline__ float adafac_mlp(const float (&f)[NF], const int (&ro
     o0 = fmaf(hk, nw[kAWO + k * 2 + 0], o0);
     o1 = fmaf(hk, nw[kAWO + k * 2 + 1], o1);
   }
-  const float step = (o0 * expf(o1 * a.exp_mult)) * a.step_mult;
-  p = fmaf(step, -a.lr, p);
-  if (a.weight_decay > 0.0f) p = fmaf(p, -(a.weight_decay * a.lr), p);
-  return p;
+  return adafac_update(d, a, o0 * expf(o1 * a.exp_mult), p);
 }
 
 template <bool ND>
@@ -225,7 +235,7 @@ __device__ __forceinline__ void adafac_apply_fac(const TDesc& d, const PyloTenso
     if constexpr (ND) {
       lo_load<1, true>(d, a, idx, fac_tab, x);
     } else {  // 2-D, one element per lane
-      x.g[0] = clampf(*(const gfloat*)(a.grad + idx), a.clip_val);
+      x.g[0] = cond_grad(*(const gfloat*)(a.grad + idx), d.gscale, a.clip_val, d.nan0);
       x.p[0] = *(const gfloat*)(a.param + idx);
       x.m[0][0] = *(const gfloat*)(a.mom + idx);
       x.m[0][1] = *(const gfloat*)(a.mom + n + idx);
@@ -249,7 +259,7 @@ __device__ __forceinline__ void adafac_apply_fac(const TDesc& d, const PyloTenso
     const float f[16] = {f18[0], f18[2], f18[3], f18[4], f18[5], f18[6], f18[7], f18[8], f18[9], f18[10],
                          f18[11], f18[12], f18[13], f18[15], f18[16], f18[17]};
     const int row[16] = {0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 27, 28, 29};
-    const float pn = adafac_mlp<16>(f, row, h[0], wfold_t, net, a, x.p[0]);
+    const float pn = adafac_mlp<16>(f, row, h[0], wfold_t, net, d, a, x.p[0]);
     *(gfloat*)(a.mom + idx) = x.m[0][0];
     *(gfloat*)(a.mom + n + idx) = x.m[0][1];
     *(gfloat*)(a.mom + 2 * n + idx) = x.m[0][2];
@@ -281,7 +291,7 @@ __device__ __forceinline__ void adafac_apply_vec(const TDesc& d, const PyloTenso
     float h[kAH];
 #pragma unroll
     for (int j = 0; j < kAH; ++j) h[j] = bias_eff[j];
-    const float pn = adafac_mlp<28>(f, row, h, wfold_t, net, a, x.p[0]);
+    const float pn = adafac_mlp<28>(f, row, h, wfold_t, net, d, a, x.p[0]);
 #pragma unroll
     for (int k = 0; k < 3; ++k) {
       *(gfloat*)(a.mom + k * n + idx) = x.m[0][k];
@@ -340,7 +350,6 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
   const float bo0 = nw[kABO + 0], bo1 = nw[kABO + 1];
   const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
   const float exp_scale = a.exp_mult * 1.44269504088896341f;
-  const float wd_lr = a.weight_decay * a.lr;
   float fb[4];
   load_vec_o<4>(fac_tab + d.fac_off[1], tk.col * 16u, fb);
   // column terms of element (16 g + el), units 16 b + 4 q ..: one voffset, immediates per (g, b)
@@ -367,7 +376,7 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
     float ta[2][4];
 #pragma unroll
     for (int b = 0; b < 2; ++b) load_vec_o<4>(tr + 16 * b, trow_off, ta[b]);
-    const float gg = clampf(xg[0], a.clip_val);
+    const float gg = cond_grad(xg[0], d.gscale, a.clip_val, d.nan0);
     float m[3] = {x0[0], x1[0], x2[0]};
     ema_update(e, gg, m, xr_[0]);
     x0[0] = m[0]; x1[0] = m[1]; x2[0] = m[2];
@@ -438,10 +447,8 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
     }
     o0 += bo0;
     o1 += bo1;
-    const float step = (o0 * __builtin_amdgcn_exp2f(o1 * exp_scale)) * a.step_mult;
     float pn[1];
-    pn[0] = fmaf(step, -a.lr, xp[0]);
-    if (a.weight_decay > 0.0f) pn[0] = fmaf(pn[0], -wd_lr, pn[0]);
+    pn[0] = adafac_update(d, a, o0 * __builtin_amdgcn_exp2f(o1 * exp_scale), xp[0]);
     store_vec_o<1>(p, lo, pn);
     g += d.C0; p += d.C0; m0 += d.C0; m1 += d.C0; m2 += d.C0; rms += d.C0;
     fr += 4; tr += kAH;
@@ -455,11 +462,13 @@ __global__ __launch_bounds__(kThreads) void k_adafac_apply(const TDesc* __restri
                                                            const float* __restrict__ term_tab, PyloDecays dec,
                                                            const float* __restrict__ wfold,
                                                            const float* __restrict__ net,
-                                                           const float* __restrict__ bias_eff) {
+                                                           const float* __restrict__ bias_eff,
+                                                           const Globals* __restrict__ gl) {
   const Item it = items[blockIdx.x];
-  const TDesc d = descs[it.tensor];
+  TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
+  set_grad_scale(d, a, gl);
   const EmaConsts e = make_ema(dec);
   const float* w = wfold + (size_t)it.tensor * kAFold;
   const long long count = (long long)kThreads * d.vec * kElemIters;
@@ -474,11 +483,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PYLO_A
 void k_adafac_apply_tile(const TDesc* __restrict__ descs, const PyloTensorArgs* __restrict__ dyn,
                          const Item* __restrict__ items, const float* __restrict__ fac_tab,
                          const float* __restrict__ term_tab, PyloDecays dec, const float* __restrict__ wfold,
-                         const float* __restrict__ net) {
+                         const float* __restrict__ net, const Globals* __restrict__ gl) {
   const Item it = items[blockIdx.x];
-  const TDesc d = descs[it.tensor];
+  TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
+  set_grad_scale(d, a, gl);
   __shared__ float xch[kWaves][16 * 64];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int task = it.a * 4 + wave;

@@ -140,7 +140,7 @@ __device__ __forceinline__ void load_elems(const TDesc& d, const PyloTensorArgs&
 #pragma unroll
   for (int v = 0; v < V; ++v) {
     const float4 fb = load_f4(f1 + (size_t)(x.i1 + v) * 4);
-    x.g[v] = clampf(x.g[v] * scale, a.clip_val);
+    x.g[v] = cond_grad(x.g[v], scale, a.clip_val, d.nan0);
     x.m[v][0] = m0[v]; x.m[v][1] = m1[v]; x.m[v][2] = m2[v];
     x.rfcf[v][0] = fa.x * fb.x;
     x.rfcf[v][1] = fa.y * fb.y;

@@ -9,9 +9,16 @@ namespace pylo {
 // =============================================================================================
 // P0: row / column sums of g^2 for 2-D factored tensors; sum g^2 and clamp flag for everything
 // =============================================================================================
+// |x|; NaN counts as infinity on tensors whose NaNs are replaced (fmaxf alone would drop it), so
+// that the flag for the exact pass is raised.
+__device__ __forceinline__ float abs_or_inf(float x, int nan0) {
+  const float ax = fabsf(x);
+  return (nan0 && ax != ax) ? __builtin_inff() : ax;
+}
+
 template <int V, bool exact>
 __device__ __forceinline__ void p0_factored(const TDesc& d, const float* g, int strip, int cb,
-                                            float scale, float clipv, float* __restrict__ rowpart,
+                                            float scale, float clipv, int nan0, float* __restrict__ rowpart,
                                             float* __restrict__ colpart, float* lds_col, float* lds_row,
                                             float& gsq, float& amax) {
   constexpr int TC = 64 * V;
@@ -46,9 +53,9 @@ __device__ __forceinline__ void p0_factored(const TDesc& d, const float* g, int 
 #pragma unroll
       for (int v = 0; v < V; ++v) {
         const float raw = x[u][v];
-        amax = fmaxf(amax, fabsf(raw));
+        amax = fmaxf(amax, abs_or_inf(raw, nan0));
         if (exact) gsq = fmaf(raw, raw, gsq);
-        const float y = exact ? clampf(raw * scale, clipv) : raw;
+        const float y = exact ? cond_grad(raw, scale, clipv, nan0) : raw;
         sq[v] = y * y;
         col[v] += sq[v];
       }
@@ -77,6 +84,7 @@ __device__ __forceinline__ void p0_factored(const TDesc& d, const float* g, int 
 
 template <int V>
 __device__ __forceinline__ void p0_flat(const TDesc& d, const float* g, int chunk, float& gsq, float& amax) {
+  const int nan0 = d.nan0;
   const long long base = (long long)chunk * (kThreads * V * kElemIters);
 #pragma unroll
   for (int it = 0; it < kElemIters; ++it) {
@@ -87,7 +95,7 @@ __device__ __forceinline__ void p0_flat(const TDesc& d, const float* g, int chun
 #pragma unroll
       for (int v = 0; v < V; ++v) {
         gsq = fmaf(x[v], x[v], gsq);
-        amax = fmaxf(amax, fabsf(x[v]));
+        amax = fmaxf(amax, abs_or_inf(x[v], nan0));
       }
     }
   }
@@ -117,10 +125,10 @@ __global__ __launch_bounds__(kThreads) void k_p0(const TDesc* __restrict__ descs
       const float scale = (pass == 1) ? clip_scale(gl->gnorm, a.clip_norm) : 1.0f;
       float* p0r = part + d.part_off[0];
       float* p0c = part + d.part_off[1];
-      if (d.vec == 4 && exact) p0_factored<4, true>(d, a.grad, it.a, it.b, scale, a.clip_val, p0r, p0c, lds_col, lds_row, gsq, amax);
-      else if (d.vec == 4) p0_factored<4, false>(d, a.grad, it.a, it.b, scale, a.clip_val, p0r, p0c, lds_col, lds_row, gsq, amax);
-      else if (exact) p0_factored<1, true>(d, a.grad, it.a, it.b, scale, a.clip_val, p0r, p0c, lds_col, lds_row, gsq, amax);
-      else p0_factored<1, false>(d, a.grad, it.a, it.b, scale, a.clip_val, p0r, p0c, lds_col, lds_row, gsq, amax);
+      if (d.vec == 4 && exact) p0_factored<4, true>(d, a.grad, it.a, it.b, scale, a.clip_val, d.nan0, p0r, p0c, lds_col, lds_row, gsq, amax);
+      else if (d.vec == 4) p0_factored<4, false>(d, a.grad, it.a, it.b, scale, a.clip_val, d.nan0, p0r, p0c, lds_col, lds_row, gsq, amax);
+      else if (exact) p0_factored<1, true>(d, a.grad, it.a, it.b, scale, a.clip_val, d.nan0, p0r, p0c, lds_col, lds_row, gsq, amax);
+      else p0_factored<1, false>(d, a.grad, it.a, it.b, scale, a.clip_val, d.nan0, p0r, p0c, lds_col, lds_row, gsq, amax);
     } else {
       if (d.vec == 4) p0_flat<4>(d, a.grad, it.a, gsq, amax);
       else p0_flat<1>(d, a.grad, it.a, gsq, amax);
@@ -160,12 +168,13 @@ __global__ __launch_bounds__(kThreads) void k_gnorm(const double* __restrict__ g
 // =============================================================================================
 // Sums of g^2 over one dim of an N-D tensor (any two factored dims): a block takes 64 entries of
 // the statistics vector and 64 positions of the removed dim and writes one partial row; k_v0a adds
-// the partial rows up.  Small tensors only (conv kernels, cls tokens); the gradient is clamped
-// directly (no global-norm scale on this path).
+// the partial rows up.  Small tensors only (conv kernels, cls tokens); runs after the global norm is
+// known and takes the sums of the conditioned gradient directly.
 // =============================================================================================
 __global__ __launch_bounds__(kThreads) void k_p0_nd(const TDesc* __restrict__ descs,
                                                     const PyloTensorArgs* __restrict__ dyn,
-                                                    const Item* __restrict__ items, float* __restrict__ part) {
+                                                    const Item* __restrict__ items, float* __restrict__ part,
+                                                    const Globals* __restrict__ gl) {
   __shared__ float lds[kWaves][kV0aEnt];
   const Item it = items[blockIdx.x];
   const TDesc d = descs[it.tensor];
@@ -175,13 +184,14 @@ __global__ __launch_bounds__(kThreads) void k_p0_nd(const TDesc* __restrict__ de
   const int e = threadIdx.x & 63, grp = threadIdx.x >> 6;
   const int i = it.a * kV0aEnt + e;
   const int X = pick(d.nd_size, w), sX = pick(d.nd_stride, w);
+  const float scale = a.clip_norm > 0.0f ? clip_scale(gl->gnorm, a.clip_norm) : 1.0f;
   float s = 0.0f;
   if (i < pick(d.len, w)) {
     const long long base = (long long)(i / sX) * X * sX + (i % sX);
     const int x0 = it.c * kNdX + grp * (kNdX / kWaves);
     const int x1 = min(X, x0 + kNdX / kWaves);
     for (int x = x0; x < x1; ++x) {
-      const float g = clampf(*(const gfloat*)(a.grad + base + (long long)x * sX), a.clip_val);
+      const float g = cond_grad(*(const gfloat*)(a.grad + base + (long long)x * sX), scale, a.clip_val, d.nan0);
       s = fmaf(g, g, s);
     }
   }
@@ -226,7 +236,7 @@ __global__ __launch_bounds__(kV0aThreads) void k_v0a(const TDesc* __restrict__ d
   const int k = grp;  // waves 0..2 take one decay each
   if (k >= 3) return;
   double s2 = 1.0;
-  if (a.clip_norm > 0.0f && gl->flag == 0) {
+  if (a.clip_norm > 0.0f && gl->flag == 0 && d.mode == kModeFac2D) {  // other modes sum the scaled gradient
     const float sc = clip_scale(gl->gnorm, a.clip_norm);
     s2 = (double)sc * (double)sc;
   }

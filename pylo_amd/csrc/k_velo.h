@@ -32,10 +32,10 @@ template <int V, bool ND>
 __device__ __forceinline__ void lo_load(const TDesc& d, const PyloTensorArgs& a, long long idx,
                                         const float* __restrict__ fac_tab, ElemIn<V>& x) {
   if constexpr (!ND) {
-    load_elems<V>(d, a, idx, 1.0f, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1], x);
+    load_elems<V>(d, a, idx, d.gscale, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1], x);
   } else {
     const long long n = d.n;
-    x.g[0] = clampf(*(const gfloat*)(a.grad + idx), a.clip_val);
+    x.g[0] = cond_grad(*(const gfloat*)(a.grad + idx), d.gscale, a.clip_val, d.nan0);
     x.p[0] = *(const gfloat*)(a.param + idx);
     x.m[0][0] = *(const gfloat*)(a.mom + idx);
     x.m[0][1] = *(const gfloat*)(a.mom + n + idx);
@@ -204,7 +204,7 @@ __device__ __forceinline__ void vec_load(const TDesc& d, const PyloTensorArgs& a
   }
 #pragma unroll
   for (int v = 0; v < V; ++v) {
-    x.g[v] = clampf(x.g[v], a.clip_val);
+    x.g[v] = cond_grad(x.g[v], d.gscale, a.clip_val, d.nan0);
 #pragma unroll
     for (int k = 0; k < 3; ++k) { x.m[v][k] = t[k][v]; x.v[v][k] = u[k][v]; }
   }

@@ -77,6 +77,9 @@ struct TDesc {
   int atile_nct, atile_ntask;
   int adam_indep;          // kModeFlat: AdamW on the tensor's own two moments instead of mom[0] / rms
   int fin_blk0, fin_nblk;  // ELO-CELO2 finishing pass: range of 8192-element blocks (rows of its partials)
+  int nan0;                // gradients pass through torch.nan_to_num (PYLO_F_NAN_TO_NUM)
+  int wd_prestep;          // p -= lr * (step + wd * p) against the pre-step parameter (PYLO_F_WD_PRESTEP)
+  float gscale;            // 1 in the plan; AdafacLO-family kernels overwrite their copy with the clip scale
 };
 
 // Field of vector 0 or 1 chosen at run time.  Indexing the by-value descriptor with a run-time
@@ -182,6 +185,20 @@ __device__ __forceinline__ float clip_scale(float gnorm, float clip_norm) {
   if (!(clip_norm > 0.0f)) return 1.0f;
   float denom = fmaxf(gnorm, clip_norm);
   return denom > 0.0f ? clip_norm / denom : 1.0f;
+}
+
+// The descriptor copy of a kernel carries the tensor's global-norm clip factor for cond_grad.
+__device__ __forceinline__ void set_grad_scale(TDesc& d, const PyloTensorArgs& a, const Globals* gl) {
+  d.gscale = a.clip_norm > 0.0f ? clip_scale(gl->gnorm, a.clip_norm) : 1.0f;
+}
+
+// The gradient as the optimizer sees it (ELO_naive.py:141-146): scaled by the global-norm clip factor,
+// NaN -> 0 where the tensor asks for torch.nan_to_num (its clip_val is FLT_MAX then, which maps
+// +-inf as torch does), clamped to +-clip_val.
+__device__ __forceinline__ float cond_grad(float raw, float scale, float clip_val, int nan0) {
+  float x = raw * scale;
+  if (nan0) x = (x == x) ? x : 0.0f;
+  return clampf(x, clip_val);
 }
 
 // 1/sqrt(x) for x in the normal range (callers add an epsilon >= 1e-9 first): v_rsq_f32, 1 ulp.

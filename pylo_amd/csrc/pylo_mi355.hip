@@ -68,6 +68,7 @@ struct Layout {
   std::vector<int> dc, dr;
   int H = 8;  // width of the first MLP layer (terms per row / column)
   int Tpad = 0;
+  bool global_norm = false;  // AdafacLO kind: every tensor has P0 items, the call may clip by global norm
   size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_el_items, off_ap_items, off_ga_items, off_fin_items, off_finpart, off_finscale, off_v0a_items, off_v0b_items, off_fac_list,
       off_part, off_gsq, off_flag, off_globals, off_fac, off_term, off_v0part, off_bscale, off_stats, off_wfold,
       off_chan_ms, off_totals, off_xfeat, off_lossfeat, off_xT, off_canon, total;
@@ -93,6 +94,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.dr.assign(T, -1);
   long long part = 0, fac = 0, term = 0;
   const int H = L.H;
+  L.global_norm = (shapes[0].flags & PYLO_F_GLOBAL_NORM) != 0;
   for (int t = 0; t < T; ++t) {
     const PyloTensorShape& s = shapes[t];
     if (s.ndim < 0 || s.ndim > PYLO_MAX_DIMS) return fail("plan: bad ndim");
@@ -106,6 +108,13 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     if (n >= (1ll << 31)) return fail("plan: tensors of 2^31 or more elements are not supported");
     TDesc& d = L.descs[t];
     d.n = n;
+    d.gscale = 1.0f;
+    if ((s.flags & (PYLO_F_NAN_TO_NUM | PYLO_F_WD_PRESTEP | PYLO_F_GLOBAL_NORM)) && kind != PYLO_KIND_ADAFAC)
+      return fail("plan: PYLO_F_NAN_TO_NUM / PYLO_F_WD_PRESTEP / PYLO_F_GLOBAL_NORM belong to AdafacLO plans");
+    if (((s.flags & PYLO_F_GLOBAL_NORM) != 0) != L.global_norm)
+      return fail("plan: PYLO_F_GLOBAL_NORM must be set on every tensor of the plan or on none");
+    d.nan0 = (s.flags & PYLO_F_NAN_TO_NUM) != 0;
+    d.wd_prestep = (s.flags & PYLO_F_WD_PRESTEP) != 0;
     d.fac_slot = -1;
     d.rank = rank < 4 ? rank : 4;
     int dc = -1, dr = -1;
@@ -177,12 +186,13 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       }
     }
     const long long chunk = (long long)kThreads * d.vec * kElemIters;
-    // P0 items: tiles of 2-D factored tensors; flat chunks only where a global norm is needed (CELO2)
+    // P0 items: tiles of 2-D factored tensors; flat chunks only where a global norm is needed
+    // (CELO2's AdamW tensors, every other tensor of a PYLO_F_GLOBAL_NORM plan)
     if (n > 0) {
       if (d.mode == kModeFac2D) {
         for (int st = 0; st < d.n_strips; ++st)
           for (int cb = 0; cb < d.n_colblk; ++cb) L.p0_items.push_back(Item{t, st, cb, 0});
-      } else if (d.mode == kModeFlat) {
+      } else if (d.mode == kModeFlat || (s.flags & PYLO_F_GLOBAL_NORM)) {
         for (long long c = 0; c * chunk < n; ++c) L.p0_items.push_back(Item{t, (int)c, 0, 0});
       }
     }
@@ -624,7 +634,7 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
   // clip_norm is 0 for VeLO tensors: k_p0 clamps directly; its norm / flag outputs are not used
   if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0);
   HIP_TRY(mark());
-  if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part);
+  if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part, gl);
   HIP_TRY(mark());
   if (n_v0a > 0)
     hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kV0aThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
@@ -695,10 +705,19 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   std::memset(&vs, 0, sizeof(vs));
   Marks mark(P, s);
 
+  // ELO's global-norm clipping (ELO_cuda.py:153-161): the norm, then the exact sums where an element
+  // is not a fixed point of the conditioning.  Plain AdafacLO steps skip both launches.
+  bool clips = false;
+  for (int t = 0; t < T; ++t) clips = clips || (args[t].grad != nullptr && args[t].clip_norm > 0.0f);
+  if (clips && !L.global_norm) return fail("adafac_step: clip_norm > 0 needs a plan built with PYLO_F_GLOBAL_NORM");
   HIP_TRY(mark());
   if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0);
+  if (clips) {
+    hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl);
+    if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1);
+  }
   HIP_TRY(mark());
-  if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part);
+  if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part, gl);
   HIP_TRY(mark());
   if (n_v0a > 0)
     hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kV0aThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
@@ -709,7 +728,7 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
     hipLaunchKernelGGL(k_v0b<kAH>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-5f,
                        net + kAW1, (const float*)bias_eff, fac_tab, term_tab, bscale);
   HIP_TRY(mark());
-  if (n_el > 0) hipLaunchKernelGGL(k_adafac_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, dec, stats);
+  if (n_el > 0) hipLaunchKernelGGL(k_adafac_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, dec, stats, gl);
   HIP_TRY(mark());
   hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, totals, (const float*)nullptr, vs,
                      (float*)nullptr);
@@ -721,10 +740,10 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   const int n_ap = (int)L.ap_items.size(), n_ga = (int)L.ga_items.size();
   if (n_ga > 0)
     hipLaunchKernelGGL(k_adafac_apply, dim3(n_ga), dim3(kThreads), 0, s, descs, dyn, ga_items, fac_tab, term_tab, dec,
-                       wfold, net, (const float*)bias_eff);
+                       wfold, net, (const float*)bias_eff, gl);
   if (n_ap > 0)
     hipLaunchKernelGGL(k_adafac_apply_tile, dim3(n_ap), dim3(kThreads), 0, s, descs, dyn, ap_items, fac_tab, term_tab,
-                       dec, wfold, net);
+                       dec, wfold, net, gl);
   HIP_TRY(mark());
   mark.done();
   HIP_TRY(hipGetLastError());

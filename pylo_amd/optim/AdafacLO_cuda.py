@@ -36,6 +36,8 @@ def _decays(initial, offsets, device):
 
 
 class AdafacLO_CUDA(Optimizer):
+    _PLAN_FLAGS = 0      # PyloTensorShape.flags of every tensor
+
     def __init__(
         self,
         params,
@@ -128,9 +130,19 @@ class AdafacLO_CUDA(Optimizer):
                 raise TypeError("AdafacLO_CUDA: parameters must be contiguous float32 tensors on the optimizer's GPU")
         if self._plan is not None:
             self._plan.close()
-        self._plan = _lib.Plan(_lib.KIND_ADAFAC, [tuple(p.shape) for _, p in tensors], [0] * len(tensors),
-                               self.device)
+        self._plan = _lib.Plan(_lib.KIND_ADAFAC, [tuple(p.shape) for _, p in tensors],
+                               [self._PLAN_FLAGS] * len(tensors), self.device)
         self._plan_key = key
+
+    def _pre_clip(self, group, p):
+        """Per-parameter norm clipping of the gradient, in place (AdafacLO_naive.py:200-201)."""
+        if group["max_grad_norm"] is not None:
+            torch.nn.utils.clip_grad_norm_(p, group["max_grad_norm"])
+
+    def _scalars(self, group):
+        """Per-tensor scalar columns of the argument table."""
+        return dict(lr=group["lr"], weight_decay=group["weight_decay"], exp_mult=self.exp_mult,
+                    step_mult=self.step_mult)
 
     @torch.no_grad()
     def step(self, loss=None):
@@ -140,12 +152,11 @@ class AdafacLO_CUDA(Optimizer):
         n = len(tensors)
         keys = ("grad", "param", "mom", "rms", "fac_r", "fac_c", "fac_v")
         cols = {k: [0] * n for k in keys}
-        fl = {k: [0.0] * n for k in ("lr", "weight_decay", "exp_mult", "step_mult")}
+        fl = {k: [0.0] * n for k in ("lr", "weight_decay", "exp_mult", "step_mult", "clip_norm", "clip_val")}
         keep = []
         step_fed = None
         for i, (group, p) in enumerate(tensors):
-            if group["max_grad_norm"] is not None:
-                torch.nn.utils.clip_grad_norm_(p, group["max_grad_norm"])
+            self._pre_clip(group, p)
             g = p.grad
             if g is None:
                 continue
@@ -164,7 +175,7 @@ class AdafacLO_CUDA(Optimizer):
             if step_fed is None:
                 step_fed = s0
             elif step_fed != s0:
-                raise NotImplementedError("AdafacLO_CUDA: parameters with different step counts in one call")
+                raise NotImplementedError(f"{type(self).__name__}: parameters with different step counts in one call")
             cols["grad"][i], cols["param"][i] = g.data_ptr(), p.data_ptr()
             cols["mom"][i], cols["rms"][i] = state["exp_avg"].data_ptr(), state["exp_avg_sq"].data_ptr()
             if _factored_dims(tuple(p.shape)) is None:
@@ -172,8 +183,8 @@ class AdafacLO_CUDA(Optimizer):
             else:
                 cols["fac_r"][i] = state["exp_avg_sq_r"].data_ptr()
                 cols["fac_c"][i] = state["exp_avg_sq_c"].data_ptr()
-            fl["lr"][i], fl["weight_decay"][i] = group["lr"], group["weight_decay"]
-            fl["exp_mult"][i], fl["step_mult"][i] = self.exp_mult, self.step_mult
+            for k, v in self._scalars(group).items():
+                fl[k][i] = v
         if step_fed is None:
             return loss
         args = plan.args

@@ -44,6 +44,7 @@ def _load_reference():
         CELO2_naive=m("pylo.optim.CELO2_naive").CELO2_naive,
         VeLO_naive=m("pylo.optim.Velo_naive").VeLO_naive,
         AdafacLO_naive=m("pylo.optim.AdafacLO_naive").AdafacLO_naive,
+        ELO_naive=m("pylo.optim.ELO_naive").ELO_naive,
     )
 
 
@@ -172,7 +173,10 @@ def velo_case(R, name, shapes, n_steps, grad_scale, seed, num_steps, weight_deca
 
 
 # ------------------------------------------------------------------- AdafacLO
-def adafac_case(R, name, shapes, n_steps, grad_scale, seed, weight_decay, lr):
+def adafac_case(R, name, shapes, n_steps, grad_scale, seed, weight_decay, lr, cls="AdafacLO_naive", extra=None,
+                nan_at=()):
+    """`extra`: further constructor arguments (ELO_naive: exp_mult, clip_grad, clip_norm, decays);
+    `nan_at`: (step, tensor, flat index) triples where the gradient is NaN (ELO_naive zeroes them)."""
     torch.manual_seed(21)
     net = R["MetaMLP"](39, 32, 1)
     tmp = tempfile.mkdtemp()
@@ -180,15 +184,19 @@ def adafac_case(R, name, shapes, n_steps, grad_scale, seed, weight_decay, lr):
     gen = torch.Generator().manual_seed(seed)
     init = [torch.randn(s, generator=gen) * 0.5 for s in shapes]
     params = [torch.nn.Parameter(v.clone()) for v in init]
-    opt = R["AdafacLO_naive"](params, lr=lr, weight_decay=weight_decay, hf_key=os.path.join(tmp, "mlp"))
+    extra = dict(extra or {})
+    opt = R[cls](params, lr=lr, weight_decay=weight_decay, hf_key=os.path.join(tmp, "mlp"), **extra)
     arrays = {}
     _sd_arrays("net", net, arrays)
-    meta = dict(kind="adafac", shapes=[list(s) for s in shapes], n_steps=n_steps, seed=seed,
-                weight_decay=weight_decay, lr=lr, grad_scale=grad_scale)
+    meta = dict(kind="adafac" if cls == "AdafacLO_naive" else "elo", shapes=[list(s) for s in shapes],
+                n_steps=n_steps, seed=seed, weight_decay=weight_decay, lr=lr, grad_scale=grad_scale, extra=extra)
     for i, v in enumerate(init):
         arrays[f"init/{i}"] = _np(v)
     for t in range(n_steps):
         grads = [torch.randn(s, generator=gen) * grad_scale for s in shapes]
+        for tt, ti, fi in nan_at:
+            if tt == t:
+                grads[ti].view(-1)[fi] = float("nan")
         for p, g in zip(params, grads):
             p.grad = g.clone()
         opt.step()
@@ -229,6 +237,14 @@ def main():
     celo2_case(R, "celo2_small_defaults", [(40, 56), (7,), (24, 24)], 6, 0.1, 13, dict(lr=1e-3),
                cls="CELO2_naive")
     if "--celo2-only" in sys.argv:
+        return
+    # ELO_naive: AdafacLO's features and MLP, raw decays, global-norm clipping, nan_to_num, ELO update rule
+    adafac_case(R, "elo_small", [(20, 10), (20,), (5, 20), (6, 3, 4, 4), (16, 16), (40, 128)], 6, 0.3, 31,
+                weight_decay=0.05, lr=1e-2, cls="ELO_naive",
+                extra=dict(exp_mult=0.01, clip_grad=True, clip_norm=2.0, initial_rms_decays=(0.99,)))
+    adafac_case(R, "elo_small_nan", [(33, 17), (17,), (4, 3, 5)], 5, 1.0, 32, weight_decay=0.0, lr=1e-3,
+                cls="ELO_naive", nan_at=((1, 0, 7), (1, 1, 3), (3, 2, 11), (3, 0, 100)))
+    if "--elo-only" in sys.argv:
         return
     ctor_checksums(R)
     # shapes of the reference's own CUDA-vs-naive test (tests/test_celo2_cuda.py:38,116)

@@ -53,6 +53,16 @@ def test_workspace_sizing_and_error_paths_without_gpu():
     # the independent-moment AdamW branch (CELO2_CUDA) is a tensor flag of its own
     indep = _lib.make_shapes([(768,), (64, 16)], [_lib.F_ADAM_INDEP, _lib.F_ADAM_INDEP])
     assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, indep, 2, C.byref(n)) == 0
+    # ELO_CUDA's tensor flags belong to AdafacLO plans; the global-norm flag is all-or-none
+    elo = _lib.F_NAN_TO_NUM | _lib.F_WD_PRESTEP | _lib.F_GLOBAL_NORM
+    ok = _lib.make_shapes([(64, 128), (128,), (4, 3, 5)], [elo, elo, elo])
+    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_ADAFAC, ok, 3, C.byref(n)) == 0
+    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, ok, 1, C.byref(n)) != 0
+    assert b"AdafacLO plans" in lib.pylo_mi355_last_error()
+    for fl in ([elo, 0, elo], [0, elo, elo]):
+        mixed = _lib.make_shapes([(64, 128), (128,), (4, 3, 5)], fl)
+        assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_ADAFAC, mixed, 3, C.byref(n)) != 0
+        assert b"PYLO_F_GLOBAL_NORM" in lib.pylo_mi355_last_error()
     # >2-D tensors are fine for VeLO / AdafacLO, rejected (for now) on the CELO2 MLP path
     nd = _lib.make_shapes([(768, 3, 16, 16)], [0])
     assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_VELO, nd, 1, C.byref(n)) == 0
@@ -71,7 +81,7 @@ def test_optimizers_fail_loudly_without_gpu():
 
     if torch.cuda.is_available():
         pytest.skip("this check is for GPU-less hosts")
-    from pylo_amd import AdafacLO_CUDA, CELO2_CUDA, ELO_CELO2_CUDA, VeLO_CUDA
+    from pylo_amd import AdafacLO_CUDA, CELO2_CUDA, ELO_CELO2_CUDA, ELO_CUDA, VeLO_CUDA
     from pylo_amd.models import CELO2MLP, MetaMLP, VeLOMLP, VeLORNN
 
     p = [torch.nn.Parameter(torch.zeros(4, 4))]
@@ -83,6 +93,8 @@ def test_optimizers_fail_loudly_without_gpu():
         VeLO_CUDA(p, rnn=VeLORNN(lstm_hidden_size=64, param_inits=8), mlp=VeLOMLP(param_inits=8))
     with pytest.raises(RuntimeError, match="requires a GPU"):
         AdafacLO_CUDA(p, network=MetaMLP(39, 32, 1))
+    with pytest.raises(RuntimeError, match="requires a GPU"):
+        ELO_CUDA(p, network=MetaMLP(39, 32, 1))
 
 
 def test_weight_containers_round_trip_through_the_reference_file_format(tmp_path):

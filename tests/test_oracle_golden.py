@@ -139,6 +139,36 @@ def test_adafac_oracle_matches_reference(name):
                 assert max_err(st["exp_avg_sq_c"], ref_c, REL, ABS) <= 1.0, (t, i, "col")
 
 
+@pytest.mark.parametrize("name", ["elo_small", "elo_small_nan"])
+def test_elo_oracle_matches_reference(name):
+    """ELO_naive: raw decays, global-norm clipping, NaN gradients zeroed, pre-step weight decay."""
+    G = Golden(name)
+    meta = G.meta
+    shapes = G.shapes
+    params = [G.t(f"init/{i}").clone() for i in range(len(shapes))]
+    opt = O.EloOracle(params, G.state_dict("net"), lr=meta["lr"], weight_decay=meta["weight_decay"], **meta["extra"])
+    saw_nan = False
+    for t in range(meta["n_steps"]):
+        grads = [G.t(f"grad{t}/{i}") for i in range(len(shapes))]
+        saw_nan |= any(bool(torch.isnan(g).any()) for g in grads)
+        opt.step(grads)
+        for i, p in enumerate(params):
+            st = opt.state[i]
+            assert max_err(p, G.t(f"step{t}/param/{i}"), REL, ABS) <= 1.0, (t, i, "param")
+            assert max_err(st["exp_avg"], G.t(f"step{t}/exp_avg/{i}"), REL, ABS) <= 1.0, (t, i)
+            assert max_err(st["exp_avg_sq"], G.t(f"step{t}/exp_avg_sq/{i}"), REL, ABS) <= 1.0, (t, i)
+            if len(shapes[i]) < 2:
+                assert max_err(st["exp_avg_sq_r"], G.t(f"step{t}/fac_vec_v/{i}"), REL, ABS) <= 1.0
+            else:
+                dc, dr = O.factored_dims(shapes[i])
+                ref_r = trailing_to_keepdim(G.t(f"step{t}/fac_vec_row_trailing/{i}"), dr)
+                ref_c = trailing_to_keepdim(G.t(f"step{t}/fac_vec_col_trailing/{i}"), dc)
+                assert max_err(st["exp_avg_sq_r"], ref_r, REL, ABS) <= 1.0, (t, i, "row")
+                assert max_err(st["exp_avg_sq_c"], ref_c, REL, ABS) <= 1.0, (t, i, "col")
+    assert saw_nan == (name == "elo_small_nan")
+    assert all(bool(torch.isfinite(p).all()) for p in params)
+
+
 def test_constructor_rng_order_matches_reference():
     """Freshly constructed product meta-nets under seed 1234 have the reference's weights."""
     from pylo_amd import models as M

@@ -130,6 +130,8 @@ class ELO_CELO2_CUDA(Optimizer):
         self._mlp = pack_celo2(self.network).to(self.device)
         bm, bf = self.beta_m.tolist(), self.beta_fac.tolist()
         self._decays = _lib.make_decays(bm, float(self.beta_rms[-1]), bf)
+        # host copies: reading an element of a device tensor synchronises with the GPU
+        self._adam_b1, self._adam_b2 = float(bm[0]), float(self.beta_rms[-1])
         self._plan = None
         self._plan_key = None
 
@@ -210,11 +212,11 @@ class ELO_CELO2_CUDA(Optimizer):
     # AdamW branch: which two moment buffers a tensor uses and its bias corrections this step
     def _adam_row(self, group, state):
         t = group["step"]
-        beta1, beta2 = float(self.beta_m[0]), float(self.beta_rms[-1])
-        return state["mom"].data_ptr(), state["rms"].data_ptr(), 1.0 - beta1 ** t, 1.0 - beta2 ** t
+        return (state["mom"].data_ptr(), state["rms"].data_ptr(), 1.0 - self._adam_b1 ** t,
+                1.0 - self._adam_b2 ** t)
 
     def _adam_corrections_fast(self, fast, per_group):
-        beta1, beta2 = float(self.beta_m[0]), float(self.beta_rms[-1])
+        beta1, beta2 = self._adam_b1, self._adam_b2
         adam = fast["adam"]
         return (np.where(adam, per_group(lambda g: 1.0 - beta1 ** g["step"]), 0.0),
                 np.where(adam, per_group(lambda g: 1.0 - beta2 ** g["step"]), 0.0))
@@ -230,8 +232,6 @@ class ELO_CELO2_CUDA(Optimizer):
             return None
         for group in groups:
             group["step"] = group.get("step", 0) + 1
-        beta1 = float(self.beta_m[0])
-        beta2 = float(self.beta_rms[-1])
         gidx, adam = fast["gidx"], fast["adam"]
 
         def per_group(fn):
@@ -264,8 +264,6 @@ class ELO_CELO2_CUDA(Optimizer):
         plan = self._plan
         for group in self.param_groups:
             group["step"] = group.get("step", 0) + 1
-        beta1 = float(self.beta_m[0])
-        beta2 = float(self.beta_rms[-1])
         n = len(tensors)
         cols = {k: [0] * n for k in ("grad", "param", "mom", "rms", "fac_r", "fac_c", "step_out")}
         fl = {k: [0.0] * n for k in ("lr", "weight_decay", "clip_norm", "clip_val", "exp_mult", "bc1", "bc2")}
@@ -284,7 +282,6 @@ class ELO_CELO2_CUDA(Optimizer):
             state = self.state[p]
             if len(state) == 0:
                 self._init_state(state, p, adam)
-            t = group["step"]
             cols["grad"][i], cols["param"][i] = g.data_ptr(), p.data_ptr()
             fl["clip_norm"][i] = group["clip_norm"] if group["clip_grad"] else 0.0
             fl["clip_val"][i] = group["grad_clip_val"]

@@ -133,9 +133,13 @@ const char* pylo_mi355_plan_launch_name(const PyloPlan* plan, int launch);
  * For every tensor with a gradient:  g <- clamp(g * clip_scale, +-clip_val) with
  * clip_scale = clip_norm / max(||all grads||_2, clip_norm); mom/rms EMAs; then
  *   - PYLO_F_ADAM tensors: AdamW on mom[0] / rms, parameter updated in place;
- *   - other (>=2-D) tensors: fac_r / fac_c EMAs, 30 features, per-channel RMS normalisation
- *     over the tensor, the 30->8->8->3 MLP; step_out = o0 * exp(o1 * exp_mult).  The parameter
- *     is NOT touched (Newton-Schulz, normalise and apply follow, ELO_CELO2_cuda.py:288-296).
+ *   - other tensors: fac_r / fac_c EMAs, 30 features, per-channel RMS normalisation over the last
+ *     two dims (the whole tensor when it is 2-D; one set of normalisers per slice when it has more
+ *     dims, ELO_CELO2_naive.py:217-218), the 30->8->8->3 MLP; step_out = o0 * exp(o1 * exp_mult).
+ *     The parameter is NOT touched (Newton-Schulz, normalise and apply follow,
+ *     ELO_CELO2_cuda.py:288-296).  A tensor of fewer than two dims without an AdamW flag takes the
+ *     same path with the per-element accumulator fac_v and the first nine feature groups
+ *     (use_adamw_for_1d=False, ELO_CELO2_naive.py:166-169,180-191).
  * `mlp` is a device pointer to 347 floats: w_in (30,8) | b_in 8 | w_h (8,8) | b_h 8 | w_out (8,3) | b_out 3,
  * weights stored (in, out) as in pylo/models/CELO2_MLP.py:72-86.
  */

@@ -246,6 +246,8 @@ class EloCelo2Oracle:
                 cs_[dc] = 1
                 st["fac_r"] = torch.zeros([3] + rs_, device=dv)
                 st["fac_c"] = torch.zeros([3] + cs_, device=dv)
+            elif not use_adamw_for_1d:
+                st["fac_v"] = torch.zeros((3,) + s, device=dv)     # ELO_CELO2_naive.py:254-256
             self.state.append(st)
 
     def double_(self):
@@ -275,9 +277,20 @@ class EloCelo2Oracle:
         nd = p.dim()
         _ema_(st["mom"], _bview(self.beta_m, nd), g[None])
         _ema_(st["rms"], self.beta_rms[-1], g * g)
-        dc, dr = factored_dims(tuple(p.shape))
-        rf, cf = _factored_update(st, g, self.beta_fac, dc, dr, "fac_r", "fac_c")
-        groups = celo2_feature_groups(p, g, st["mom"], st["rms"], st["fac_r"], st["fac_c"], rf, cf)
+        fd = factored_dims(tuple(p.shape))
+        if fd is not None:
+            dc, dr = fd
+            rf, cf = _factored_update(st, g, self.beta_fac, dc, dr, "fac_r", "fac_c")
+            groups = celo2_feature_groups(p, g, st["mom"], st["rms"], st["fac_r"], st["fac_c"], rf, cf)
+        else:
+            # fewer than two dims on the MLP path (use_adamw_for_1d=False): the accumulator is per
+            # element and only the first nine feature groups exist; the split first layer adds up
+            # the groups it is given (ELO_CELO2_naive.py:166-169,180-191; CELO2_MLP.py:100-110)
+            b = _bview(self.beta_fac, nd)
+            st["fac_v"] = b * st["fac_v"] + (1 - b) * (g * g + 1e-30)[None]
+            rs = torch.rsqrt(st["rms"] + 1e-8)
+            groups = [g[None], torch.clamp(g, -0.1, 0.1)[None], p[None], st["mom"], st["rms"][None],
+                      st["mom"] * rs[None], rs[None], g[None] * safe_rsqrt(st["fac_v"] + 1e-9), (g * rs)[None]]
         axes = [nd - 1, nd] if nd >= 2 else [nd]      # last two param dims (decay axis leads)
         groups = [rms_normalize(x, axes, 1e-9) for x in groups]
         out = celo2_mlp(groups, self.net)

@@ -782,13 +782,12 @@ __global__ __launch_bounds__(kThreads) void k_celo2_sumsq(const TDesc* __restric
 
 __global__ __launch_bounds__(kThreads) void k_celo2_finscale(const TDesc* __restrict__ descs,
                                                              const PyloTensorArgs* __restrict__ dyn,
-                                                             const int* __restrict__ fac_list,
                                                              const double* __restrict__ fin_part,
                                                              float* __restrict__ fin_scale) {
   __shared__ double red[kWaves];
-  const int t = fac_list[blockIdx.x];
+  const int t = blockIdx.x;  // one block per tensor of the plan; AdamW tensors have no finishing blocks
   const TDesc d = descs[t];
-  if (dyn[t].grad == nullptr) return;
+  if (dyn[t].grad == nullptr || d.fin_nblk == 0) return;
   double s = 0.0;
 #pragma unroll 8
   for (int b = threadIdx.x; b < d.fin_nblk; b += kThreads) s += fin_part[d.fin_blk0 + b];

@@ -77,6 +77,7 @@ struct TDesc {
   int atile_nct, atile_ntask;
   int adam_indep;          // kModeFlat: AdamW on the tensor's own two moments instead of mom[0] / rms
   int fin_blk0, fin_nblk;  // ELO-CELO2 finishing pass: range of 8192-element blocks (rows of its partials)
+  int slice_len;           // CELO2, N-D or fewer than two dims: elements per slice of the last two dims (or n)
   int nan0;                // gradients pass through torch.nan_to_num (PYLO_F_NAN_TO_NUM)
   int wd_prestep;          // p -= lr * (step + wd * p) against the pre-step parameter (PYLO_F_WD_PRESTEP)
   float gscale;            // 1 in the plan; AdafacLO-family kernels overwrite their copy with the clip scale

@@ -21,6 +21,7 @@
 #include "k_gradstats.h"
 #include "k_adafac.h"
 #include "k_velo.h"
+#include "k_celo2_slices.h"
 #include "pylo_common.h"
 
 // =============================================================================================
@@ -63,13 +64,13 @@ bool factored_dims(int kind, const PyloTensorShape& s, int* dc, int* dr) {
 
 struct Layout {
   std::vector<TDesc> descs;
-  std::vector<Item> p0_items, nd_items, el_items, ap_items, ga_items, fin_items, v0a_items, v0b_items;
+  std::vector<Item> p0_items, nd_items, sl_items, el_items, ap_items, ga_items, fin_items, v0a_items, v0b_items;
   std::vector<int> fac_list;
   std::vector<int> dc, dr;
   int H = 8;  // width of the first MLP layer (terms per row / column)
   int Tpad = 0;
   bool global_norm = false;  // AdafacLO kind: every tensor has P0 items, the call may clip by global norm
-  size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_el_items, off_ap_items, off_ga_items, off_fin_items, off_finpart, off_finscale, off_v0a_items, off_v0b_items, off_fac_list,
+  size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_sl_items, off_el_items, off_ap_items, off_ga_items, off_fin_items, off_finpart, off_finscale, off_v0a_items, off_v0b_items, off_fac_list,
       off_part, off_gsq, off_flag, off_globals, off_fac, off_term, off_v0part, off_bscale, off_stats, off_wfold,
       off_chan_ms, off_totals, off_xfeat, off_lossfeat, off_xT, off_canon, total;
 };
@@ -121,11 +122,12 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     const bool can_factor = factored_dims(kind, s, &dc, &dr);
     if (kind == PYLO_KIND_CELO2) {
       const bool adam = (s.flags & (PYLO_F_ADAM | PYLO_F_ADAM_INDEP)) != 0;
-      if (!can_factor && !adam) return fail("plan: CELO2 tensors with fewer than 2 dims must carry PYLO_F_ADAM");
       d.adam_indep = (s.flags & PYLO_F_ADAM_INDEP) != 0;
       if (adam) d.mode = kModeFlat;
-      else if (s.ndim == 2) d.mode = kModeFac2D;
-      else return fail("plan: CELO2 tensors with more than 2 dims are not supported yet");
+      else if (!can_factor) d.mode = kModeVec;  // the MLP on a tensor with fewer than two dims
+      else d.mode = s.ndim == 2 ? kModeFac2D : kModeFacND;
+      if (d.mode == kModeVec) d.slice_len = (int)std::max<long long>(n, 1);
+      if (d.mode == kModeFacND) d.slice_len = (int)std::max<long long>(s.shape[s.ndim - 2] * s.shape[s.ndim - 1], 1);
     } else {
       d.mode = !can_factor ? kModeVec : (s.ndim == 2 ? kModeFac2D : kModeFacND);
     }
@@ -192,13 +194,18 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       if (d.mode == kModeFac2D) {
         for (int st = 0; st < d.n_strips; ++st)
           for (int cb = 0; cb < d.n_colblk; ++cb) L.p0_items.push_back(Item{t, st, cb, 0});
-      } else if (d.mode == kModeFlat || (s.flags & PYLO_F_GLOBAL_NORM)) {
+      } else if (kind == PYLO_KIND_CELO2 || (s.flags & PYLO_F_GLOBAL_NORM)) {
         for (long long c = 0; c * chunk < n; ++c) L.p0_items.push_back(Item{t, (int)c, 0, 0});
       }
     }
     d.blk0 = (int)L.el_items.size();
     const bool wide = d.mode == kModeFac2D && n > 0 && env_matrix_pipe();
-    if (wide && d.C0 % kTileCols == 0) {
+    if (kind == PYLO_KIND_CELO2 && (d.mode == kModeFacND || d.mode == kModeVec)) {
+      // one pass per slice of the last two dims (k_celo2_slices): 256 slices a block, or 4
+      const long long n_slices = n / d.slice_len, per = d.slice_len <= kSliceLaneMax ? kThreads : kWaves;
+      if (n_slices >= (1ll << 31)) return fail("plan: too many slices");
+      for (long long s0 = 0; s0 < n_slices && n > 0; s0 += per) L.sl_items.push_back(Item{t, (int)s0, 0, 0});
+    } else if (wide && d.C0 % kTileCols == 0) {
       d.tile_nct = d.C0 / kTileCols;
       d.tile_ntask = d.tile_nct * ((d.R0 + kTileRows - 1) / kTileRows);
       for (int b = 0; b * 4 < d.tile_ntask; ++b) L.el_items.push_back(Item{t, b, 0, 0});
@@ -235,6 +242,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_dyn = take(sizeof(PyloTensorArgs) * T);
   L.off_p0_items = take(sizeof(Item) * L.p0_items.size());
   L.off_nd_items = take(sizeof(Item) * L.nd_items.size());
+  L.off_sl_items = take(sizeof(Item) * L.sl_items.size());
   L.off_el_items = take(sizeof(Item) * L.el_items.size());
   L.off_ap_items = take(sizeof(Item) * L.ap_items.size());
   L.off_ga_items = take(sizeof(Item) * L.ga_items.size());
@@ -327,6 +335,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_descs, L.descs.data(), sizeof(TDesc) * L.descs.size());
   if (e == hipSuccess) e = up(L.off_p0_items, L.p0_items.data(), sizeof(Item) * L.p0_items.size());
   if (e == hipSuccess) e = up(L.off_nd_items, L.nd_items.data(), sizeof(Item) * L.nd_items.size());
+  if (e == hipSuccess) e = up(L.off_sl_items, L.sl_items.data(), sizeof(Item) * L.sl_items.size());
   if (e == hipSuccess) e = up(L.off_el_items, L.el_items.data(), sizeof(Item) * L.el_items.size());
   if (e == hipSuccess) e = up(L.off_ap_items, L.ap_items.data(), sizeof(Item) * L.ap_items.size());
   if (e == hipSuccess) e = up(L.off_ga_items, L.ga_items.data(), sizeof(Item) * L.ga_items.size());
@@ -465,7 +474,8 @@ int check_args(const PyloPlan* P, const PyloTensorArgs* args, bool need_all_grad
     if (!a.param || !a.mom || !a.rms) return fail("step: null param/mom/rms pointer" + at);
     const bool factored = d.mode == kModeFac2D || d.mode == kModeFacND;
     if (factored && (!a.fac_r || !a.fac_c)) return fail("step: null fac_r/fac_c pointer" + at);
-    if (factored && P->kind == PYLO_KIND_CELO2 && !a.step_out) return fail("step: null step_out pointer" + at);
+    if ((factored || d.mode == kModeVec) && P->kind == PYLO_KIND_CELO2 && !a.step_out)
+      return fail("step: null step_out pointer" + at);
     if (d.mode == kModeVec && !a.fac_v) return fail("step: null fac_v pointer" + at);
     if (a.group < 0 || a.group >= PYLO_MAX_GROUPS) return fail("step: group index out of range" + at);
     const uintptr_t m = reinterpret_cast<uintptr_t>(a.grad) | reinterpret_cast<uintptr_t>(a.param) |
@@ -506,6 +516,9 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   const Item* el_items = P->at<Item>(L.off_el_items);
   const Item* v0a_items = P->at<Item>(L.off_v0a_items);
   const Item* v0b_items = P->at<Item>(L.off_v0b_items);
+  const Item* nd_items = P->at<Item>(L.off_nd_items);
+  const Item* sl_items = P->at<Item>(L.off_sl_items);
+  const int n_nd = (int)L.nd_items.size(), n_sl = (int)L.sl_items.size();
   const int* fac_list = P->at<int>(L.off_fac_list);
   float* part = P->at<float>(L.off_part);
   double* gsq = P->at<double>(L.off_gsq);
@@ -529,6 +542,7 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl);
   HIP_TRY(mark());
   if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1);
+  if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part, gl);
   HIP_TRY(mark());
   if (n_v0a > 0)
     hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kV0aThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
@@ -549,6 +563,8 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
       hipLaunchKernelGGL(k_celo2_apply<false>, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab,
                          term_tab, gl, dec, wfold);
   }
+  if (n_sl > 0)
+    hipLaunchKernelGGL(k_celo2_slices, dim3(n_sl), dim3(kThreads), 0, s, descs, dyn, sl_items, fac_tab, gl, dec, mlp);
   HIP_TRY(mark());
   mark.done();
   HIP_TRY(hipGetLastError());
@@ -563,6 +579,9 @@ extern "C" int pylo_mi355_celo2_finish(PyloPlan* P, const PyloTensorArgs* args, 
     const TDesc& d = L.descs[t];
     const PyloTensorArgs& a = args[t];
     if (a.grad == nullptr || d.mode == kModeFlat || d.n == 0) continue;
+    if (d.mode == kModeFacND)
+      return fail("celo2_finish: tensors with more than two dims are normalised per slice of the last two dims, "
+                  "not by this tensor-wide pass (tensor " + std::to_string(t) + ")");
     if (!a.param || !a.step_out) return fail("celo2_finish: null param/step_out pointer at tensor " + std::to_string(t));
     const uintptr_t m = reinterpret_cast<uintptr_t>(a.param) | reinterpret_cast<uintptr_t>(a.step_out);
     if (m % (d.n % 4 == 0 ? 16 : 4) != 0) return fail("celo2_finish: misaligned pointer at tensor " + std::to_string(t));
@@ -572,13 +591,12 @@ extern "C" int pylo_mi355_celo2_finish(PyloPlan* P, const PyloTensorArgs* args, 
   const TDesc* descs = P->at<TDesc>(L.off_descs);
   const PyloTensorArgs* dyn = P->at<PyloTensorArgs>(L.off_dyn);
   const Item* fin_items = P->at<Item>(L.off_fin_items);
-  const int* fac_list = P->at<int>(L.off_fac_list);
   double* fin_part = P->at<double>(L.off_finpart);
   float* fin_scale = P->at<float>(L.off_finscale);
-  const int n_fin = (int)L.fin_items.size(), n_fac = (int)L.fac_list.size();
+  const int n_fin = (int)L.fin_items.size();
   if (n_fin == 0) return 0;
   hipLaunchKernelGGL(k_celo2_sumsq, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_part);
-  hipLaunchKernelGGL(k_celo2_finscale, dim3(n_fac), dim3(kThreads), 0, s, descs, dyn, fac_list, fin_part, fin_scale);
+  hipLaunchKernelGGL(k_celo2_finscale, dim3(P->T), dim3(kThreads), 0, s, descs, dyn, fin_part, fin_scale);
   hipLaunchKernelGGL(k_celo2_update, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_scale);
   HIP_TRY(hipGetLastError());
   return 0;

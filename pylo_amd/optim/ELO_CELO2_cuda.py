@@ -7,7 +7,10 @@ Drop-in for pylo/optim/ELO_CELO2_cuda.py:39-298: same constructor, ``step()``,
 accumulator update, the 1-D AdamW branch and the feature/MLP pass of all tensors run in
 seven launches of ``libpylo_mi355.so``; only Newton-Schulz (library GEMMs), the final RMS
 normalisation and the parameter update remain in PyTorch.  Arithmetic follows the
-reference's naive class (pylo/optim/ELO_CELO2_naive.py:126-306).
+reference's naive class (pylo/optim/ELO_CELO2_naive.py:126-306), also where the reference's CUDA class
+differs or fails: tensors with more than two dims normalise features and steps per slice of the last two
+dims, and ``use_adamw_for_1d=False`` sends 1-D tensors through the MLP with a per-element accumulator
+(state ``fac_v (3,*s)``).
 """
 
 from __future__ import annotations
@@ -29,6 +32,8 @@ def newton_schulz(x: torch.Tensor, coeffs, iters: int, eps: float) -> torch.Tens
     batch dim runs as strided-batched library GEMMs with the scalings folded into them.  The reference
     transposes tall matrices so that the Gram matrix is the small one; the same products are taken
     here on the untransposed matrix (A = X^T X, X <- c0 X + X B), which keeps the result contiguous."""
+    if x.dim() > 3:     # more leading dims: one batch of matrices
+        return newton_schulz(x.reshape((-1,) + tuple(x.shape[-2:])), coeffs, iters, eps).reshape(x.shape)
     tall = x.shape[-2] > x.shape[-1]
     x = x / (torch.linalg.norm(x, dim=(-2, -1), keepdim=True) + eps)
     c0, c1, c2 = coeffs
@@ -140,11 +145,9 @@ class ELO_CELO2_CUDA(Optimizer):
         out = []
         for group in self.param_groups:
             for p in group["params"]:
-                adam = p.dim() <= 1 or group["is_embedding"]
-                if adam and not group["use_adamw_for_1d"]:
-                    raise NotImplementedError(
-                        "use_adamw_for_1d=False (CELO2 MLP on 1-D / embedding tensors) is not supported "
-                        "by the fused step")
+                # ELO_CELO2_naive.py:291-292: AdamW for tensors with fewer than two dims and for
+                # is_embedding groups, unless the group turns that off
+                adam = (p.dim() <= 1 or group["is_embedding"]) and group["use_adamw_for_1d"]
                 out.append((group, p, adam))
         return out
 
@@ -189,6 +192,8 @@ class ELO_CELO2_CUDA(Optimizer):
             c_shape[dc] = 1
             state["fac_r"] = torch.zeros([self.n_fac] + r_shape, device=self.device)
             state["fac_c"] = torch.zeros([self.n_fac] + c_shape, device=self.device)
+        elif not adam:   # the MLP on a tensor with fewer than two dims: per-element Adafactor accumulator
+            state["fac_v"] = torch.zeros((self.n_fac,) + shape, device=self.device)
 
     # ------------------------------------------------------------------ step
     @torch.no_grad()
@@ -265,7 +270,7 @@ class ELO_CELO2_CUDA(Optimizer):
         for group in self.param_groups:
             group["step"] = group.get("step", 0) + 1
         n = len(tensors)
-        cols = {k: [0] * n for k in ("grad", "param", "mom", "rms", "fac_r", "fac_c", "step_out")}
+        cols = {k: [0] * n for k in ("grad", "param", "mom", "rms", "fac_r", "fac_c", "fac_v", "step_out")}
         fl = {k: [0.0] * n for k in ("lr", "weight_decay", "clip_norm", "clip_val", "exp_mult", "bc1", "bc2")}
         keep = []   # contiguous copies of non-contiguous grads must outlive the launch
         for i, (group, p, adam) in enumerate(tensors):
@@ -292,7 +297,10 @@ class ELO_CELO2_CUDA(Optimizer):
                 fl["weight_decay"][i] = group["adam_weight_decay"]
             else:
                 cols["mom"][i], cols["rms"][i] = state["mom"].data_ptr(), state["rms"].data_ptr()
-                cols["fac_r"][i], cols["fac_c"][i] = state["fac_r"].data_ptr(), state["fac_c"].data_ptr()
+                if p.dim() >= 2:
+                    cols["fac_r"][i], cols["fac_c"][i] = state["fac_r"].data_ptr(), state["fac_c"].data_ptr()
+                else:
+                    cols["fac_v"][i] = state["fac_v"].data_ptr()
                 cols["step_out"][i] = self._raw[i].data_ptr()
         args = plan.args
         for k, v in cols.items():
@@ -331,18 +339,26 @@ class ELO_CELO2_CUDA(Optimizer):
                     step = self._raw[i]
                     if group["param_scale_mult"]:
                         step = step * torch.sqrt(torch.mean(p * p) + 1e-9)
-                    if group["orthogonalize"]:
+                    if group["orthogonalize"] and step.dim() >= 2:
                         step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
-                    step = rms_normalize(step, [-2, -1]) * group["rmsmult"]
+                    step = rms_normalize(step, list(range(step.dim()))[-2:]) * group["rmsmult"]
                     p.add_(step + group["weight_decay"] * p, alpha=-group["lr"])
                 continue
             step = buf
+            nd = buf.dim() - 1
             if group["param_scale_mult"]:
                 n = ps[0].numel()
                 sq = torch.stack(torch._foreach_norm(ps)) ** 2 / n
-                step = step * torch.sqrt(sq + 1e-9).view(-1, 1, 1)
-            if group["orthogonalize"]:
+                step = step * torch.sqrt(sq + 1e-9).view([-1] + [1] * nd)
+            if group["orthogonalize"] and nd >= 2:
                 step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
+            if nd > 2:
+                # more than two dims: the normaliser is per slice of the last two dims
+                # (ELO_CELO2_naive.py:217-218,235), which the tensor-wide finishing kernels do not do
+                step = rms_normalize(step, [-2, -1]) * group["rmsmult"]
+                for j, p in enumerate(ps):
+                    p.add_(step[j] + group["weight_decay"] * p, alpha=-group["lr"])
+                continue
             step = step.contiguous()
             keep.append(step)
             base, stride = step.data_ptr(), step[0].numel() * 4

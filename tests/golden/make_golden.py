@@ -98,6 +98,8 @@ def celo2_case(R, name, shapes, n_steps, grad_scale, seed, cfg, net_seed=1, full
             else:
                 rec = {"param": p.detach(), "mom": _to_leading(st["mom"], p.dim()),
                        "rms": st["rms"][..., 0]}
+            if "exp_avg" not in st and st["fac_vec_v"].numel():
+                rec["fac_v"] = st["fac_vec_v"].movedim(-1, 0)
             if p.dim() >= 2 and "exp_avg" not in st:
                 # naive fac_vec_row (mean over dr, decay last) -> (3,*s with dr->1)
                 sorted_dims = np.argsort(p.shape)
@@ -237,6 +239,14 @@ def main():
     celo2_case(R, "celo2_small_defaults", [(40, 56), (7,), (24, 24)], 6, 0.1, 13, dict(lr=1e-3),
                cls="CELO2_naive")
     if "--celo2-only" in sys.argv:
+        return
+    # ELO_CELO2_naive on tensors with more than two dims (feature normalisers and Newton-Schulz per
+    # slice of the last two dims) and with the MLP on 1-D tensors (use_adamw_for_1d=False)
+    celo2_case(R, "elo_celo2_nd", [(6, 3, 4, 4), (2, 5, 3), (3, 16, 8), (12,), (20, 10), (4, 3, 70)], 6, 0.5, 41,
+               dict(lr=1e-2, adam_lr_mult=5.0, exp_mult=0.01))
+    celo2_case(R, "elo_celo2_mlp1d", [(20, 10), (12,), (5,), (200,), (3, 2, 2)], 6, 2.0, 42,
+               dict(lr=1e-2, use_adamw_for_1d=False, clip_norm=3.0))
+    if "--celo2-nd-only" in sys.argv:
         return
     # ELO_naive: AdafacLO's features and MLP, raw decays, global-norm clipping, nan_to_num, ELO update rule
     adafac_case(R, "elo_small", [(20, 10), (20,), (5, 20), (6, 3, 4, 4), (16, 16), (40, 128)], 6, 0.3, 31,

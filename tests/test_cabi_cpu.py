@@ -46,10 +46,9 @@ def test_workspace_sizing_and_error_paths_without_gpu():
     shapes = _lib.make_shapes([(50257, 768), (768,), (768, 2304)], [0, _lib.F_ADAM, 0])
     assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, shapes, 3, C.byref(n)) == 0
     assert 1 << 20 < n.value < 1 << 28          # partial sums + tables: a few % of the 154 MB tensor
-    # a 1-D CELO2 tensor must be routed to AdamW by the caller
-    bad = _lib.make_shapes([(768,)], [0])
-    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, bad, 1, C.byref(n)) != 0
-    assert b"PYLO_F_ADAM" in lib.pylo_mi355_last_error()
+    # a CELO2 tensor with fewer than two dims and no AdamW flag takes the MLP (use_adamw_for_1d=False)
+    mlp1d = _lib.make_shapes([(768,)], [0])
+    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, mlp1d, 1, C.byref(n)) == 0
     # the independent-moment AdamW branch (CELO2_CUDA) is a tensor flag of its own
     indep = _lib.make_shapes([(768,), (64, 16)], [_lib.F_ADAM_INDEP, _lib.F_ADAM_INDEP])
     assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, indep, 2, C.byref(n)) == 0
@@ -63,11 +62,10 @@ def test_workspace_sizing_and_error_paths_without_gpu():
         mixed = _lib.make_shapes([(64, 128), (128,), (4, 3, 5)], fl)
         assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_ADAFAC, mixed, 3, C.byref(n)) != 0
         assert b"PYLO_F_GLOBAL_NORM" in lib.pylo_mi355_last_error()
-    # >2-D tensors are fine for VeLO / AdafacLO, rejected (for now) on the CELO2 MLP path
+    # tensors with more than two dims are fine for every kind
     nd = _lib.make_shapes([(768, 3, 16, 16)], [0])
-    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_VELO, nd, 1, C.byref(n)) == 0
-    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_ADAFAC, nd, 1, C.byref(n)) == 0
-    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, nd, 1, C.byref(n)) != 0
+    for kind in (_lib.KIND_VELO, _lib.KIND_ADAFAC, _lib.KIND_CELO2):
+        assert lib.pylo_mi355_plan_workspace_bytes(kind, nd, 1, C.byref(n)) == 0
     # too large
     huge = _lib.make_shapes([(1 << 16, 1 << 16)], [0])
     assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_VELO, huge, 1, C.byref(n)) != 0

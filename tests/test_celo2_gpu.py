@@ -92,7 +92,7 @@ def test_fused_kernel_matches_oracle_per_step(shapes, gscale, cfg):
 
 
 @pytest.mark.parametrize("name", ["elo_celo2_small_clip", "elo_celo2_small_noclip_exp",
-                                  "elo_celo2_small_noortho"])
+                                  "elo_celo2_small_noortho", "elo_celo2_nd", "elo_celo2_mlp1d"])
 def test_full_step_matches_reference_golden(name):
     """Whole step() trajectories (NS, normalise, apply included) against the reference's naive class."""
     from pylo_amd import ELO_CELO2_CUDA
@@ -113,12 +113,58 @@ def test_full_step_matches_reference_golden(name):
         opt.step()
         for i, p in enumerate(gpu):
             keys = ["param", "mom", "rms"] + (["fac_r", "fac_c"] if p.dim() >= 2 else [])
+            if p.dim() < 2 and not cfg.get("use_adamw_for_1d", True):
+                keys.append("fac_v")          # the MLP on a 1-D tensor keeps a per-element accumulator
             for k in keys:
                 got = p if k == "param" else opt.state[p][k]
                 e = max_err(got, G.t(f"step{t}/{k}/{i}"), REL, ABS)
                 worst = max(worst, e)
                 assert e <= 1.0, (name, t, i, k, e)
     print(name, "worst err/tol", worst)
+
+
+@pytest.mark.parametrize("adam_1d", [True, False])
+def test_tensors_with_more_than_two_dims_and_mlp_on_1d(adam_1d):
+    """Per-slice normalisers (last two dims) on N-D tensors: short slices walked by one lane (3x3, 5x5),
+    long ones by a wave (4x70, 40x33), next to 2-D tensors on the ordinary passes; with
+    use_adamw_for_1d=False the 1-D tensors take the MLP with their per-element accumulator.  Raw steps,
+    accumulators and whole-step parameters against the oracle, clipping active."""
+    from oracle import pylo_oracle as O
+    from pylo_amd import ELO_CELO2_CUDA
+
+    shapes = [(32, 16, 3, 3), (8, 4, 70), (3, 40, 33), (5, 5, 5, 5), (300,), (64, 32), (2, 1, 7), (1,), (40, 128),
+              (2, 3, 4, 2, 3)]
+    net = _net(5)
+    init, gen = _mk(shapes, 17)
+    cfg = dict(lr=1e-2, exp_mult=0.01, clip_norm=4.0, use_adamw_for_1d=adam_1d, adam_lr_mult=2.0)
+    cpu = [v.clone() for v in init]
+    gpu = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+    orc = O.EloCelo2Oracle(cpu, net.state_dict(), **cfg)
+    opt = ELO_CELO2_CUDA(gpu, network=net, hf_key=None, **cfg)
+    worst = 0.0
+    for t in range(5):
+        grads = [torch.randn(s, generator=gen) * (0.3 if i % 2 else 3.0) for i, s in enumerate(shapes)]
+        if t == 3:
+            grads[1] = None
+        raw = {}
+        for p, g in zip(gpu, grads):
+            p.grad = None if g is None else g.cuda()
+        orc.step(grads, keep_raw=raw)
+        opt.step()
+        for i, r in raw.items():
+            e = max_err(opt._raw[i], r, REL, ABS)
+            worst = max(worst, e)
+            assert e <= 1.0, ("raw step", adam_1d, t, i, shapes[i], e)
+        for i, p in enumerate(gpu):
+            for k, v in orc.state[i].items():
+                if k in opt.state[p]:
+                    e = max_err(opt.state[p][k], v, REL, ABS)
+                    assert e <= 1.0, (adam_1d, t, i, k, e)
+            e = max_err(p, cpu[i], REL, ABS)
+            assert e <= 1.0, ("param", adam_1d, t, i, shapes[i], e)
+            p.data.copy_(cpu[i])
+        assert ("fac_v" in opt.state[gpu[4]]) == (not adam_1d)
+    print("nd / 1-d mlp worst raw err/tol", worst)
 
 
 def test_config1_trajectory():

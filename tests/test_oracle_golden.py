@@ -24,7 +24,8 @@ def _regen_inputs(meta):
 
 
 @pytest.mark.parametrize("name", ["elo_celo2_small_clip", "elo_celo2_small_noclip_exp",
-                                  "elo_celo2_small_noortho", "elo_celo2_cfg1"])
+                                  "elo_celo2_small_noortho", "elo_celo2_cfg1", "elo_celo2_nd",
+                                  "elo_celo2_mlp1d"])
 def test_elo_celo2_oracle_matches_reference(name):
     G = Golden(name)
     meta = G.meta
@@ -45,6 +46,8 @@ def test_elo_celo2_oracle_matches_reference(name):
             got = {"param": p, "mom": opt.state[i]["mom"], "rms": opt.state[i]["rms"]}
             if p.dim() >= 2:
                 got["fac_r"], got["fac_c"] = opt.state[i]["fac_r"], opt.state[i]["fac_c"]
+            elif not cfg.get("use_adamw_for_1d", True):
+                got["fac_v"] = opt.state[i]["fac_v"]
             for k, v in got.items():
                 if meta["full"]:
                     e = max_err(v, G.t(f"step{t}/{k}/{i}"), REL, ABS)

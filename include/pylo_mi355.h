@@ -91,7 +91,8 @@ typedef struct {
   float clip_val;    /* element-wise clamp of the gradient (1000 in the reference), 0 = off  */
   float exp_mult;
   float step_mult;
-  float bc1;         /* CELO2 AdamW: 1 - beta1^t                                             */
+  float bc1;         /* CELO2 AdamW: 1 - beta1^t; AdafacLO kind: the tensor's step counter when
+                        the call passes step < 0                                             */
   float bc2;         /* CELO2 AdamW: 1 - beta2^t                                             */
   int32_t group;     /* VeLO: index into PyloVeloStep.frac (the tensor's parameter group)    */
   int32_t reserved;
@@ -213,7 +214,9 @@ int pylo_mi355_velo_step(PyloPlan* plan, const PyloTensorArgs* args, const PyloD
  *               (AdafacLO has no clip(g) / g*rs channel: rows 1 and 14 are zero);
  *   b1 32 | w_time (11,32): rows of the 11 tanh time features | w_h (32,32) | b_h 32 | w_o (32,2) | b_o 2
  * (pylo_amd.models.pack_metamlp builds it from a MetaMLP).  `step` is the 0-based step counter fed to
- * the time features (AdafacLO_cuda.py:400).  Tensors without gradient are skipped.
+ * the time features (AdafacLO_cuda.py:400) of every tensor; a negative `step` takes each tensor's own
+ * counter from its `bc1` field (the reference keeps one per parameter, AdafacLO_cuda.py:304-305, and
+ * parameters that sat steps out lag behind).  Tensors without gradient are skipped.
  *   p -= lr * o0 * exp(o1 * exp_mult) * step_mult;  then p -= weight_decay * lr * p.
  * ELO_CUDA (pylo/optim/ELO_cuda.py:179-288) runs on the same call: raw decays in `decays`, step_mult = 1,
  * clip_norm > 0 for global-norm clipping, and the tensor flags PYLO_F_NAN_TO_NUM | PYLO_F_WD_PRESTEP.

@@ -610,7 +610,13 @@ class AdafacOracle:
                  initial_adafactor_decays=(0.9, 0.99, 0.999),
                  momentum_decays=(0.15216392, 0.14245212, 0.06812963),
                  rms_decays=(0.01079706,),
-                 adafactor_decays=(0.18621896, -0.10864615, -0.06185547), device="cpu"):
+                 adafactor_decays=(0.18621896, -0.10864615, -0.06185547), device="cpu",
+                 per_param_step=False):
+        # per_param_step: the time features follow each parameter's own step counter, as the CUDA
+        # class keeps it (AdafacLO_cuda.py:304-305,400), instead of the group's counter of the naive
+        # class (AdafacLO_naive.py:194-197,226); the two differ only for a parameter that sat steps out.
+        self.per_param_step = per_param_step
+        self.steps = [0] * len(params)
         self.params = params
         dv = self.device = torch.device(device)
         self.net = {k: v.detach().to(F32).to(dv) for k, v in net.items()}
@@ -661,9 +667,12 @@ class AdafacOracle:
         tfeat = tanh_time_embedding(self.t - 1).to(self.device)
         sd = self.net
         grads = self.condition_grads(grads)
-        for p, g, st in zip(self.params, grads, self.state):
+        for i, (p, g, st) in enumerate(zip(self.params, grads, self.state)):
             if g is None:
                 continue
+            self.steps[i] += 1
+            if self.per_param_step:
+                tfeat = tanh_time_embedding(self.steps[i] - 1).to(self.device)
             nd = p.dim()
             mom = st["exp_avg"]
             _ema_(mom, _bview(self.beta_m, nd), g[None])

@@ -23,11 +23,16 @@ constexpr int kAFold = 960;  // per-tensor first-layer rows scaled by the channe
 __host__ __device__ constexpr bool adafac_channel(int c) { return c != 1 && c != 14; }
 
 // b_eff = b1 + w_time^T tanh(step / ts - 1)   (AdafacLO_naive.py:81-87,226)
+// One block per tensor: `step` >= 0 is the counter of every tensor, a negative `step` takes each
+// tensor's own counter from its argument record (bc1; AdafacLO_cuda.py:304-305,400 keeps one per parameter).
 __global__ __launch_bounds__(64) void k_adafac_bias(const float* __restrict__ net, float step,
-                                                    float* __restrict__ bias_eff) {
+                                                    const PyloTensorArgs* __restrict__ dyn,
+                                                    float* __restrict__ bias_all) {
   const float ts[11] = {1.f, 3.f, 10.f, 30.f, 100.f, 300.f, 1000.f, 3000.f, 10000.f, 30000.f, 100000.f};
   const int j = threadIdx.x;
   if (j >= kAH) return;
+  if (step < 0.0f) step = dyn[blockIdx.x].bc1;
+  float* bias_eff = bias_all + (size_t)blockIdx.x * kAH;
   float acc = net[kAB1 + j];
 #pragma unroll
   for (int q = 0; q < 11; ++q) acc = fmaf(tanhf(step / ts[q] - 1.0f), net[kAWT + q * kAH + j], acc);
@@ -475,7 +480,7 @@ __global__ __launch_bounds__(kThreads) void k_adafac_apply(const TDesc* __restri
   const long long base = (long long)it.a * count;
   if (d.mode == kModeFac2D) adafac_apply_fac<false>(d, a, base, count, e, fac_tab, term_tab, w, net);
   else if (d.mode == kModeFacND) adafac_apply_fac<true>(d, a, base, count, e, fac_tab, term_tab, w, net);
-  else adafac_apply_vec(d, a, base, count, e, dec, w, net, bias_eff);
+  else adafac_apply_vec(d, a, base, count, e, dec, w, net, bias_eff + (size_t)it.tensor * kAH);
 }
 
 // The apply pass for tensors walked column-resident (items hold four wave tasks each).

@@ -330,6 +330,7 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
                                                   const Item* __restrict__ items,
                                                   const double* __restrict__ v0part, float norm_eps,
                                                   const float* __restrict__ w1, const float* __restrict__ b1,
+                                                  int b1_stride /* floats between the tensors' biases, 0: shared */,
                                                   float* __restrict__ fac_tab, float* __restrict__ term_tab,
                                                   BScale* __restrict__ bscale) {
   constexpr int G = 14;  // 14 groups x 18 (vector, slot) pairs = 252 threads
@@ -381,7 +382,7 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
     vector_entry(d, is_r, fac, len, i, bs, fct, x0, x1);
 #pragma unroll
     for (int k = 0; k < 3; ++k) fac_tab[fac_index(d, which, k, i)] = fct[k];
-    if (w1 != nullptr) vector_terms<H>(d, which, is_r, i, x0, x1, w1, b1, term_tab);
+    if (w1 != nullptr) vector_terms<H>(d, which, is_r, i, x0, x1, w1, b1 + (size_t)it.tensor * b1_stride, term_tab);
   }
 }
 

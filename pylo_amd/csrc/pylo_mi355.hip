@@ -549,7 +549,7 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   HIP_TRY(mark());
   if (n_v0b > 0)
     hipLaunchKernelGGL(k_v0b<8>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-9f, mlp,
-                       mlp + 240, fac_tab, term_tab, bscale);
+                       mlp + 240, 0, fac_tab, term_tab, bscale);
   HIP_TRY(mark());
   if (n_el > 0) hipLaunchKernelGGL(k_celo2_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, gl, dec, stats);
   HIP_TRY(mark());
@@ -659,7 +659,7 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
   HIP_TRY(mark());
   if (n_v0b > 0)
     hipLaunchKernelGGL(k_v0b<4>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-5f,
-                       (const float*)nullptr, (const float*)nullptr, fac_tab, term_tab, bscale);
+                       (const float*)nullptr, (const float*)nullptr, 0, fac_tab, term_tab, bscale);
   HIP_TRY(mark());
   if (n_el > 0) hipLaunchKernelGGL(k_velo_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, dec, stats);
   HIP_TRY(mark());
@@ -714,7 +714,7 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   double* stats = P->at<double>(L.off_stats);
   float* wfold = P->at<float>(L.off_wfold);
   double* totals = P->at<double>(L.off_totals);
-  float* bias_eff = P->at<float>(L.off_xfeat);  // 32 floats; the LSTM feature buffer is unused by this kind
+  float* bias_eff = P->at<float>(L.off_xfeat);  // [T][32]; the LSTM feature buffer is unused by this kind
   const int n_p0 = (int)L.p0_items.size(), n_nd = (int)L.nd_items.size(), n_el = (int)L.el_items.size();
   const int n_v0a = (int)L.v0a_items.size(), n_v0b = (int)L.v0b_items.size();
   const int T = P->T;
@@ -740,11 +740,11 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   if (n_v0a > 0)
     hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kV0aThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_adafac_bias, dim3(1), dim3(64), 0, s, net, step, bias_eff);
+  hipLaunchKernelGGL(k_adafac_bias, dim3(T), dim3(64), 0, s, net, step, dyn, bias_eff);
   HIP_TRY(mark());
   if (n_v0b > 0)
     hipLaunchKernelGGL(k_v0b<kAH>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-5f,
-                       net + kAW1, (const float*)bias_eff, fac_tab, term_tab, bscale);
+                       net + kAW1, (const float*)bias_eff, kAH, fac_tab, term_tab, bscale);
   HIP_TRY(mark());
   if (n_el > 0) hipLaunchKernelGGL(k_adafac_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, dec, stats, gl);
   HIP_TRY(mark());

@@ -152,7 +152,7 @@ class AdafacLO_CUDA(Optimizer):
         n = len(tensors)
         keys = ("grad", "param", "mom", "rms", "fac_r", "fac_c", "fac_v")
         cols = {k: [0] * n for k in keys}
-        fl = {k: [0.0] * n for k in ("lr", "weight_decay", "exp_mult", "step_mult", "clip_norm", "clip_val")}
+        fl = {k: [0.0] * n for k in ("lr", "weight_decay", "exp_mult", "step_mult", "clip_norm", "clip_val", "bc1")}
         keep = []
         step_fed = None
         for i, (group, p) in enumerate(tensors):
@@ -171,11 +171,14 @@ class AdafacLO_CUDA(Optimizer):
             if len(state) == 0:
                 self._init_state(state, p)
             state["step"] += 1
+            # the time features take each parameter's own counter (pylo/optim/AdafacLO_cuda.py:304-305,400):
+            # one that sat steps out lags behind the others
             s0 = float(state["step"]) - 1.0
+            fl["bc1"][i] = s0
             if step_fed is None:
                 step_fed = s0
             elif step_fed != s0:
-                raise NotImplementedError(f"{type(self).__name__}: parameters with different step counts in one call")
+                step_fed = -1.0      # counters differ: the library reads them per tensor
             cols["grad"][i], cols["param"][i] = g.data_ptr(), p.data_ptr()
             cols["mom"][i], cols["rms"][i] = state["exp_avg"].data_ptr(), state["exp_avg_sq"].data_ptr()
             if _factored_dims(tuple(p.shape)) is None:

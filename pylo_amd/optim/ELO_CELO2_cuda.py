@@ -4,9 +4,10 @@ loop and CUDA extension replaced by one multi-tensor HIP step.
 Drop-in for pylo/optim/ELO_CELO2_cuda.py:39-298: same constructor, ``step()``,
 ``param_groups`` keys and per-parameter state (``mom (3,*s)``, ``rms (*s)``, ``fac_r``,
 ``fac_c``).  What differs is *where* the work happens: gradient clipping, every
-accumulator update, the 1-D AdamW branch and the feature/MLP pass of all tensors run in
-seven launches of ``libpylo_mi355.so``; only Newton-Schulz (library GEMMs), the final RMS
-normalisation and the parameter update remain in PyTorch.  Arithmetic follows the
+accumulator update, the 1-D AdamW branch and the feature/MLP pass of all tensors run in one
+call into ``libpylo_mi355.so`` (eight launches); Newton-Schulz runs as batched library GEMMs over
+buckets of equally shaped tensors, and a second call normalises the steps and updates the
+parameters.  Arithmetic follows the
 reference's naive class (pylo/optim/ELO_CELO2_naive.py:126-306), also where the reference's CUDA class
 differs or fails: tensors with more than two dims normalise features and steps per slice of the last two
 dims, and ``use_adamw_for_1d=False`` sends 1-D tensors through the MLP with a per-element accumulator

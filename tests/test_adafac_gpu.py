@@ -90,6 +90,39 @@ def test_adafac_matches_oracle_mixed_shapes():
     print("adafac mixed worst err/tol", worst)
 
 
+def test_parameter_that_sat_steps_out_keeps_its_own_step_counter():
+    """AdafacLO_cuda.py:304-305,400: the time features come from each parameter's own ``state["step"]``;
+    a parameter without gradient on some steps lags behind and the call carries per-tensor counters."""
+    from oracle import pylo_oracle as O
+    from pylo_amd import AdafacLO_CUDA
+    from pylo_amd.models import MetaMLP
+
+    torch.manual_seed(12)
+    net = MetaMLP(39, 32, 1)
+    shapes = [(40, 128), (24, 20), (50,), (3, 4, 5)]
+    gen = torch.Generator().manual_seed(5)
+    init = [torch.randn(s, generator=gen) * 0.3 for s in shapes]
+    cpu = [v.clone() for v in init]
+    gpu = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+    orc = O.AdafacOracle(cpu, net.state_dict(), lr=0.5, per_param_step=True)
+    opt = AdafacLO_CUDA(gpu, lr=0.5, network=copy.deepcopy(net))
+    for t in range(6):
+        grads = [torch.randn(s, generator=gen) * 0.1 for s in shapes]
+        if t in (1, 2):
+            grads[0] = None
+        if t == 3:
+            grads[2] = grads[3] = None
+        for p, g in zip(gpu, grads):
+            p.grad = None if g is None else g.cuda()
+        orc.step(grads)
+        opt.step()
+        for i, p in enumerate(gpu):
+            assert float(opt.state[p]["step"]) == orc.steps[i]
+            e = max_err(p, cpu[i], REL, ABS)
+            assert e <= 1.0, (t, i, e)
+    assert [float(opt.state[p]["step"]) for p in gpu] == [4.0, 6.0, 5.0, 5.0]
+
+
 def test_adafac_state_dict_resume():
     """tests/test_optimizer_resume.py:19-164"""
     from pylo_amd import AdafacLO_CUDA

@@ -174,7 +174,8 @@ typedef struct {
   const float* mix2_b;    /* (H)                                  */
   const float* fmix_wt;   /* (30, H)   final_mix_layer.weight^T   */
   const float* fmix_b;    /* (H)                                  */
-  const float* lstm_wt;   /* (2H, 4H)  lstm.linear.weight^T, gate blocks i, g, f, o */
+  const float* lstm_wt;   /* (2H, H, 4) lstm.linear.weight^T with the four gates (i, g, f, o) of a
+                             unit adjacent: [k][u][q] = weight[q*H + u][k] */
   const float* lstm_b;    /* (4H)                                 */
   const float* ctrl_wt;   /* (H, K)    rnn_to_controls.weight^T   */
   const float* ctrl_b;    /* (K)                                  */

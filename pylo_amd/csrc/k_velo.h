@@ -336,38 +336,11 @@ __device__ __forceinline__ float clip_log_abs10(double v) {
   return 0.5f * fminf(fmaxf(logf(1e-8f + fabsf(x * 10.0f)), -5.0f), 5.0f);
 }
 
-__global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restrict__ descs,
-                                                        const PyloTensorArgs* __restrict__ dyn, int T,
-                                                        const double* __restrict__ stats_part,
-                                                        double* __restrict__ totals,
-                                                        const float* __restrict__ lossfeat, VeloStep st,
-                                                        float* __restrict__ xfeat) {
-  constexpr int G = kFoldThreads / kStatW;  // 25 groups x 40 sums = 1000 threads
-  __shared__ double part[G][kStatW];
-  __shared__ double tot[kStatW];
-  const int t = blockIdx.x;
-  const TDesc d = descs[t];
-  const PyloTensorArgs a = dyn[t];
-  const int c = threadIdx.x % kStatW, gI = threadIdx.x / kStatW;
-  if (gI < G) {
-    double s = 0.0;
-    if (a.grad != nullptr && c < 38) {
-#pragma unroll 16
-      for (int b = gI; b < d.nblk; b += G) s += stats_part[(size_t)(d.blk0 + b) * kStatW + c];
-    }
-    part[gI][c] = s;
-  }
-  __syncthreads();
-  if (threadIdx.x < kStatW) {
-    double s = 0.0;
-    for (int g2 = 0; g2 < G; ++g2) s += part[g2][threadIdx.x];
-    tot[threadIdx.x] = s;
-    totals[(size_t)t * kStatW + threadIdx.x] = s;
-  }
-  __syncthreads();
-  if (xfeat == nullptr || threadIdx.x >= 30) return;
-  const int q = threadIdx.x;
+// Feature q of the 30 LSTM inputs of one tensor from its totals (Velo_naive.py:178-206).
+__device__ __forceinline__ float lo_lstm_feature(const TDesc& d, const PyloTensorArgs& a, const double* tot,
+                                                 const float* __restrict__ lossfeat, const VeloStep& st, int q) {
   const double n = (double)(d.n > 0 ? d.n : 1);
+
   const float nu = rsq(fmaxf((float)(tot[2] / n), 1e-9f));
   const double nu2 = (double)nu * (double)nu;
   float val;
@@ -389,52 +362,86 @@ __global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restr
       val = clip_log_abs10(nu2 * (tot[kSumRR] / n - 2.0 * mean_m * mean_r + mean_m * mean_m));
     }
   }
-  xfeat[(size_t)(T - 1 - t) * kXW + q] = val;
+  return val;
+}
+
+
+__global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restrict__ descs,
+                                                        const PyloTensorArgs* __restrict__ dyn, int T,
+                                                        const double* __restrict__ stats_part,
+                                                        double* __restrict__ totals,
+                                                        const float* __restrict__ lossfeat, VeloStep st,
+                                                        float* __restrict__ xfeat, int H,
+                                                        const float* __restrict__ w2t, const float* __restrict__ b2,
+                                                        const float* __restrict__ wft, const float* __restrict__ bf,
+                                                        float* __restrict__ mixbuf /* [2][T][H]: relu(mix2 x), final_mix x */) {
+  constexpr int G = kFoldThreads / kStatW;  // 25 groups x 40 sums = 1000 threads
+  __shared__ double part[G][kStatW];
+  __shared__ double tot[kStatW];
+  __shared__ float xs[32];
+  const int t = blockIdx.x;
+  const TDesc d = descs[t];
+  const PyloTensorArgs a = dyn[t];
+  const int c = threadIdx.x % kStatW, gI = threadIdx.x / kStatW;
+  if (gI < G) {
+    double s = 0.0;
+    if (a.grad != nullptr && c < 38) {
+#pragma unroll 16
+      for (int b = gI; b < d.nblk; b += G) s += stats_part[(size_t)(d.blk0 + b) * kStatW + c];
+    }
+    part[gI][c] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x < kStatW) {
+    double s = 0.0;
+    for (int g2 = 0; g2 < G; ++g2) s += part[g2][threadIdx.x];
+    tot[threadIdx.x] = s;
+    totals[(size_t)t * kStatW + threadIdx.x] = s;
+  }
+  __syncthreads();
+  if (xfeat == nullptr) return;
+  const int row = T - 1 - t;
+  if (threadIdx.x < 30) xs[threadIdx.x] = lo_lstm_feature(d, a, tot, lossfeat, st, threadIdx.x);
+  __syncthreads();
+  if (threadIdx.x < 30) xfeat[(size_t)row * kXW + threadIdx.x] = xs[threadIdx.x];
+  // the row's share of the LSTM input mixing (VeLO_RNN.py:110-122): relu(mix2 x) and final_mix x for every
+  // hidden unit; the maximum over rows and the sum follow in k_velo_mix
+  for (int i = threadIdx.x; i < 2 * H; i += kFoldThreads) {
+    const int u = i < H ? i : i - H;
+    const float* w = i < H ? w2t : wft;
+    float acc = i < H ? b2[u] : bf[u];
+#pragma unroll
+    for (int k = 0; k < 30; ++k) acc = fmaf(xs[k], w[k * H + u], acc);
+    mixbuf[((size_t)(i < H ? 0 : 1) * T + row) * H + u] = i < H ? fmaxf(acc, 0.0f) : acc;
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
 // LSTM (VeLO_RNN.py:43-66,110-135).  All weights are pre-transposed to (in, out) by the host.
 // Rows are in the reference's order r = T-1-t.
 // ---------------------------------------------------------------------------------------------
-// x' = final_mix(x) + max_r relu(mix2(x));  xT[u][r] = x'[r][u], xT[H+u][r] = h[r][u]
-__global__ __launch_bounds__(kThreads) void k_velo_mix(const float* __restrict__ xfeat, int T, int Tpad, int H,
-                                                       const float* __restrict__ w2t, const float* __restrict__ b2,
-                                                       const float* __restrict__ wft, const float* __restrict__ bf,
+// x' = final_mix(x) + max_r relu(mix2(x));  xT[u][r] = x'[r][u], xT[H+u][r] = h[r][u].  The per-row
+// products are in mixbuf (written by k_lo_reduce).  Block (x, y): 64 hidden units (one per lane) and
+// the 8 rows 8y .. 8y+7, two per wave; every block takes the maximum over all rows itself.
+__global__ __launch_bounds__(kThreads) void k_velo_mix(const float* __restrict__ mixbuf, int T, int Tpad, int H,
                                                        const float* __restrict__ h_state, float* __restrict__ xT) {
   __shared__ float mx_s[kWaves][64];
   const int lane = threadIdx.x & 63, grp = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int u = blockIdx.x * 64 + lane;
-  const bool ok = u < H;
-  // the lane's weight columns stay in registers; the feature rows are wave-uniform (scalar loads)
-  float w2[30], wf[30];
-#pragma unroll
-  for (int k = 0; k < 30; ++k) {
-    w2[k] = ok ? w2t[k * H + u] : 0.0f;
-    wf[k] = ok ? wft[k * H + u] : 0.0f;
-  }
-  const float b2u = ok ? b2[u] : 0.0f, bfu = ok ? bf[u] : 0.0f;
+  const int u = blockIdx.x * 64 + lane;  // H is a multiple of 64
+  const float* m2 = mixbuf;
+  const float* fm = mixbuf + (size_t)T * H;
   float mx = 0.0f;  // relu output is >= 0
-  for (int r = grp; r < T; r += kWaves) {
-    float xr[30];
-    load_uniform<30>(xfeat + (size_t)r * kXW, xr);
-    float acc = b2u;
-#pragma unroll
-    for (int k = 0; k < 30; ++k) acc = fmaf(xr[k], w2[k], acc);
-    mx = fmaxf(mx, acc);
-  }
+#pragma unroll 8
+  for (int r = grp; r < T; r += kWaves) mx = fmaxf(mx, m2[(size_t)r * H + u]);
   mx_s[grp][lane] = mx;
   __syncthreads();
   const float v = fmaxf(fmaxf(mx_s[0][lane], mx_s[1][lane]), fmaxf(mx_s[2][lane], mx_s[3][lane]));
-  if (!ok) return;
-  for (int r = grp; r < Tpad; r += kWaves) {
+#pragma unroll
+  for (int q = 0; q < kGateBT / kWaves; ++q) {
+    const int r = blockIdx.y * kGateBT + q * kWaves + grp;  // < Tpad
     float acc = 0.0f, hv = 0.0f;
     if (r < T) {
-      float xr[30];
-      load_uniform<30>(xfeat + (size_t)r * kXW, xr);
-      acc = bfu;
-#pragma unroll
-      for (int k = 0; k < 30; ++k) acc = fmaf(xr[k], wf[k], acc);
-      acc += v;
+      acc = fm[(size_t)r * H + u] + v;
       hv = h_state[(size_t)r * H + u];
     }
     xT[(size_t)u * Tpad + r] = acc;
@@ -446,36 +453,70 @@ __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf
 
 // gates = [x', h] W^T + b in chunks i, g, f, o;  c = sig(f+1) c + sig(i) tanh(g);  h = sig(o) tanh(c)
 // Block = 32 hidden units x 8 slices of the 2H-long contraction, 8 tensors; the slices are added
-// in LDS in a fixed order.
+// in LDS in a fixed order.  The weights arrive with the four gates of a unit adjacent, wt[k][u][4],
+// so a thread fetches its unit's four gate weights of one input with a single 16-byte load; the
+// inputs of the block's 8 tensors (32 B per k, the same for every unit) are staged in LDS once and
+// read back as broadcasts, which leaves the weight stream as the only vector-memory traffic of the
+// loop.  Blocks are numbered so that the blocks one XCD receives (block id modulo 8) share their
+// unit blocks: each XCD's L2 then holds its 1/8 of the 8 MB weight matrix instead of all of it.
 constexpr int kGateU = 32, kGateS = 8;
 __global__ __launch_bounds__(kThreads) void k_velo_gates(const float* __restrict__ xT, int T, int Tpad, int H,
-                                                         const float* __restrict__ wt /*(2H, 4H)*/,
+                                                         const float* __restrict__ wt /*(2H, H, 4)*/,
                                                          const float* __restrict__ b /*4H*/,
                                                          float* __restrict__ h_state, float* __restrict__ c_state) {
-  __shared__ float red[kGateS][4 * kGateBT][kGateU];
+  // x tile [2H][8] during the loop (2H <= 2048: 64 KB would not fit, so it is staged in two halves),
+  // then the partial sums [kGateS][4 * kGateBT][kGateU]
+  constexpr int kHalf = 1024;
+  __shared__ float lds[kGateS * 4 * kGateBT * kGateU];
+  static_assert(kHalf * kGateBT <= kGateS * 4 * kGateBT * kGateU, "x tile must fit the reduction buffer");
   const int ul = threadIdx.x % kGateU, sl = threadIdx.x / kGateU;
-  const int u = blockIdx.y * kGateU + ul;
-  const int r0 = blockIdx.x * kGateBT;
+  const int n_ub = H / kGateU;
+  int ub, rb;
+  if (n_ub % 8 == 0) {
+    const int per = n_ub / 8, xcd = blockIdx.x % 8, j = blockIdx.x / 8;
+    ub = xcd * per + j % per;
+    rb = j / per;
+  } else {
+    ub = blockIdx.x % n_ub;
+    rb = blockIdx.x / n_ub;
+  }
+  const int u = ub * kGateU + ul;
+  const int r0 = rb * kGateBT;
   float acc[4][kGateBT];
 #pragma unroll
   for (int g = 0; g < 4; ++g)
 #pragma unroll
     for (int t = 0; t < kGateBT; ++t) acc[g][t] = 0.0f;
   const int K2 = 2 * H;
-  if (u < H) {
-#pragma unroll 2
-    for (int k = sl; k < K2; k += kGateS) {
-      float w[4];
+  for (int k0 = 0; k0 < K2; k0 += kHalf) {
+    const int kn = min(kHalf, K2 - k0);
+    __syncthreads();
+    for (int i = threadIdx.x; i < kn * 2; i += kThreads) {  // 2 float4 per k
+      const int k = i >> 1, h4 = (i & 1) * 4;
+      *(float4*)(lds + k * kGateBT + h4) = load_f4(xT + (size_t)(k0 + k) * Tpad + r0 + h4);
+    }
+    __syncthreads();
+    // eight weight loads are issued before the first is used: the loop is bound by how many bytes a
+    // block keeps in flight, not by arithmetic (kn is a multiple of 8 * kGateS: H is a multiple of 64)
+    for (int kb = sl; kb < kn; kb += 8 * kGateS) {
+      float4 wv[8];
 #pragma unroll
-      for (int g = 0; g < 4; ++g) w[g] = wt[(size_t)k * 4 * H + g * H + u];
-      const float4 xa = load_f4(xT + (size_t)k * Tpad + r0), xb = load_f4(xT + (size_t)k * Tpad + r0 + 4);
-      const float xv[kGateBT] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+      for (int i = 0; i < 8; ++i) wv[i] = load_f4(wt + ((size_t)(k0 + kb + i * kGateS) * H + u) * 4);
 #pragma unroll
-      for (int t = 0; t < kGateBT; ++t)
+      for (int i = 0; i < 8; ++i) {
+        const int k = kb + i * kGateS;
+        const float w[4] = {wv[i].x, wv[i].y, wv[i].z, wv[i].w};
+        const float4 xa = *(const float4*)(lds + k * kGateBT), xb = *(const float4*)(lds + k * kGateBT + 4);
+        const float xv[kGateBT] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
 #pragma unroll
-        for (int g = 0; g < 4; ++g) acc[g][t] = fmaf(xv[t], w[g], acc[g][t]);
+        for (int t = 0; t < kGateBT; ++t)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) acc[g][t] = fmaf(xv[t], w[g], acc[g][t]);
+      }
     }
   }
+  __syncthreads();
+  float (*red)[4 * kGateBT][kGateU] = reinterpret_cast<float (*)[4 * kGateBT][kGateU]>(lds);
 #pragma unroll
   for (int g = 0; g < 4; ++g)
 #pragma unroll
@@ -483,7 +524,7 @@ __global__ __launch_bounds__(kThreads) void k_velo_gates(const float* __restrict
   __syncthreads();
   // thread (ul, sl) finishes tensor t = sl of unit ul
   const int t = sl, r = r0 + t;
-  if (u < H && r < T) {
+  if (r < T) {
     float gate[4];
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
@@ -503,37 +544,49 @@ __global__ __launch_bounds__(kThreads) void k_velo_gates(const float* __restrict
 // 100 * mean_i(control_i * bank_i) (VeLO_MLP.py:92-126), then the weight blocks the element
 // kernels read: un-scaled first layer for k_terms, and the folded block (first-layer rows scaled
 // by rsqrt(1e-5 + mean f_c^2), param_scale = sqrt(mean p^2 + 1e-9), lr_mult).
-__global__ __launch_bounds__(kThreads) void k_velo_heads(const TDesc* __restrict__ descs, int T, int H, int K,
-                                                         const float* __restrict__ h_state,
-                                                         const float* __restrict__ wct /*(H,K)*/,
-                                                         const float* __restrict__ bc, const float* __restrict__ wlr,
-                                                         const float* __restrict__ blr,
-                                                         const float* __restrict__ bank /*(K,159)*/,
-                                                         const double* __restrict__ totals,
-                                                         float* __restrict__ canon, float* __restrict__ wfold,
-                                                         float* __restrict__ controls_out,
-                                                         float* __restrict__ lr_mult_out) {
-  extern __shared__ float smem[];  // hs[H] | ctrl[K] | wm[160] | sc[32] | red[4]
+__global__ __launch_bounds__(kFoldThreads) void k_velo_heads(const TDesc* __restrict__ descs, int T, int H, int K,
+                                                             const float* __restrict__ h_state,
+                                                             const float* __restrict__ wct /*(H,K)*/,
+                                                             const float* __restrict__ bc, const float* __restrict__ wlr,
+                                                             const float* __restrict__ blr,
+                                                             const float* __restrict__ bank /*(K,159)*/,
+                                                             const double* __restrict__ totals,
+                                                             float* __restrict__ canon, float* __restrict__ wfold,
+                                                             float* __restrict__ controls_out,
+                                                             float* __restrict__ lr_mult_out) {
+  // Both contractions (controls over the H hidden units, the bank mix over the K controls) are cut
+  // into four slices that run side by side and are added in a fixed order; eight loads are issued
+  // before the first is used, since a block is bound by the bytes it keeps in flight.
+  constexpr int kSl = 4;
+  extern __shared__ float smem[];  // hs[H] | ctrl[K] | wm[160] | sc[32] | red[16] | part[kSl][max(K,160)]
   float* hs = smem;
   float* ctrl = hs + H;
   float* wm = ctrl + K;
   float* sc = wm + 160;
   float* red = sc + 32;
+  float* part = red + 16;
+  const int pitch = K > 160 ? K : 160;
   const int r = blockIdx.x;
   const int t = T - 1 - r;
   const TDesc d = descs[t];
-  for (int u = threadIdx.x; u < H; u += kThreads) hs[u] = h_state[(size_t)r * H + u];
+  for (int u = threadIdx.x; u < H; u += kFoldThreads) hs[u] = h_state[(size_t)r * H + u];
   __syncthreads();
-  for (int j = threadIdx.x; j < K; j += kThreads) {
-    float acc = bc[j];
-#pragma unroll 16
-    for (int u = 0; u < H; ++u) acc = fmaf(hs[u], wct[(size_t)u * K + j], acc);
-    ctrl[j] = acc;
-    if (controls_out != nullptr) controls_out[(size_t)r * K + j] = acc;
+  for (int i = threadIdx.x; i < K * kSl; i += kFoldThreads) {
+    const int j = i % K, sl = i / K;
+    const int u0 = sl * (H / kSl), u1 = u0 + H / kSl;  // H is a multiple of 64
+    float acc = 0.0f;
+    for (int u = u0; u < u1; u += 8) {
+      float w[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) w[q] = wct[(size_t)(u + q) * K + j];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) acc = fmaf(hs[u + q], w[q], acc);
+    }
+    part[sl * pitch + j] = acc;
   }
   {
     float s = 0.0f;
-    for (int u = threadIdx.x; u < H; u += kThreads) s = fmaf(hs[u], wlr[u], s);
+    for (int u = threadIdx.x; u < H; u += kFoldThreads) s = fmaf(hs[u], wlr[u], s);
     s = wave_sum(s);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
   }
@@ -542,18 +595,47 @@ __global__ __launch_bounds__(kThreads) void k_velo_heads(const TDesc* __restrict
     sc[threadIdx.x] = rsq(1e-5f + (float)(totals[(size_t)t * kStatW + threadIdx.x] / n));
   }
   __syncthreads();
-  const float lr_mult = ((red[0] + red[1]) + (red[2] + red[3])) + blr[0];
-  for (int q = threadIdx.x; q < kVBank; q += kThreads) {
+  for (int j = threadIdx.x; j < K; j += kFoldThreads) {
+    const float acc = bc[j] + ((part[j] + part[pitch + j]) + (part[2 * pitch + j] + part[3 * pitch + j]));
+    ctrl[j] = acc;
+    if (controls_out != nullptr) controls_out[(size_t)r * K + j] = acc;
+  }
+  float lr_mult = blr[0];
+  {
+    float s = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kFoldThreads / 64; ++w) s += red[w];
+    lr_mult += s;
+  }
+  __syncthreads();
+  const int Kq = (K + kSl - 1) / kSl;
+  for (int i = threadIdx.x; i < 160 * kSl; i += kFoldThreads) {
+    const int q = i % 160, sl = i / 160;
     float acc = 0.0f;
-#pragma unroll 16
-    for (int i = 0; i < K; ++i) acc = fmaf(ctrl[i], bank[(size_t)i * kVBank + q], acc);
+    if (q < kVBank) {
+      const int i0 = sl * Kq, i1 = min(K, i0 + Kq);
+      int c = i0;
+      for (; c + 8 <= i1; c += 8) {
+        float b8[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) b8[e] = bank[(size_t)(c + e) * kVBank + q];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc = fmaf(ctrl[c + e], b8[e], acc);
+      }
+      for (; c < i1; ++c) acc = fmaf(ctrl[c], bank[(size_t)c * kVBank + q], acc);
+    }
+    part[sl * pitch + q] = acc;
+  }
+  __syncthreads();
+  for (int q = threadIdx.x; q < kVBank; q += kFoldThreads) {
+    const float acc = (part[q] + part[pitch + q]) + (part[2 * pitch + q] + part[3 * pitch + q]);
     wm[q] = (acc / (float)K) * 100.0f;
   }
   __syncthreads();
   float* cn = canon + (size_t)t * kVCanon;
   float* wf = wfold + (size_t)t * kVFold;
   const bool factored = d.mode == kModeFac2D || d.mode == kModeFacND;
-  for (int i = threadIdx.x; i < 120; i += kThreads) {
+  for (int i = threadIdx.x; i < 120; i += kFoldThreads) {
     const int k = i / 4, j = i % 4;
     cn[i] = wm[j * 30 + k];
     if (factored) {

@@ -72,7 +72,7 @@ struct Layout {
   bool global_norm = false;  // AdafacLO kind: every tensor has P0 items, the call may clip by global norm
   size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_sl_items, off_el_items, off_ap_items, off_ga_items, off_fin_items, off_finpart, off_finscale, off_v0a_items, off_v0b_items, off_fac_list,
       off_part, off_gsq, off_flag, off_globals, off_fac, off_term, off_v0part, off_bscale, off_stats, off_wfold,
-      off_chan_ms, off_totals, off_xfeat, off_lossfeat, off_xT, off_canon, total;
+      off_chan_ms, off_totals, off_xfeat, off_lossfeat, off_xT, off_mixbuf, off_canon, total;
 };
 
 int first_layer_width(int kind) { return kind == PYLO_KIND_CELO2 ? 8 : kind == PYLO_KIND_VELO ? 4 : 32; }
@@ -269,6 +269,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_xfeat = take(sizeof(float) * kXW * T);
   L.off_lossfeat = take(sizeof(float) * 16);
   L.off_xT = take(kind == PYLO_KIND_VELO ? sizeof(float) * 2 * (size_t)velo_hidden * L.Tpad : 0);
+  L.off_mixbuf = take(kind == PYLO_KIND_VELO ? sizeof(float) * 2 * (size_t)velo_hidden * T : 0);
   L.off_canon = take(kind == PYLO_KIND_VELO ? sizeof(float) * kVCanon * (size_t)T : 0);
   L.total = off;
   return 0;
@@ -641,6 +642,7 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
   float* lossfeat = P->at<float>(L.off_lossfeat);
   float* xT = P->at<float>(L.off_xT);
   float* canon = P->at<float>(L.off_canon);
+  float* mixbuf = P->at<float>(L.off_mixbuf);
   const int n_p0 = (int)L.p0_items.size(), n_nd = (int)L.nd_items.size(), n_el = (int)L.el_items.size();
   const int n_v0a = (int)L.v0a_items.size(), n_v0b = (int)L.v0b_items.size();
   const PyloDecays dec = *decays;
@@ -666,15 +668,16 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
   hipLaunchKernelGGL(k_velo_loss, dim3(1), dim3(64), 0, s, step->loss_means, step->loss_running_min, step->loss_decays,
                      step->loss_iteration, step->loss, lossfeat);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, totals, lossfeat, vs, xfeat);
+  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, totals, lossfeat, vs, xfeat,
+                     H, nets->mix2_wt, nets->mix2_b, nets->fmix_wt, nets->fmix_b, mixbuf);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_velo_mix, dim3(H / 64), dim3(kThreads), 0, s, xfeat, T, L.Tpad, H, nets->mix2_wt, nets->mix2_b,
-                     nets->fmix_wt, nets->fmix_b, step->lstm_h, xT);
+  hipLaunchKernelGGL(k_velo_mix, dim3(H / 64, L.Tpad / kGateBT), dim3(kThreads), 0, s, (const float*)mixbuf, T, L.Tpad, H, step->lstm_h, xT);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_velo_gates, dim3(L.Tpad / kGateBT, H / kGateU), dim3(kThreads), 0, s, xT, T, L.Tpad, H,
+  hipLaunchKernelGGL(k_velo_gates, dim3((L.Tpad / kGateBT) * (H / kGateU)), dim3(kThreads), 0, s, xT, T, L.Tpad, H,
                      nets->lstm_wt, nets->lstm_b, step->lstm_h, step->lstm_c);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_velo_heads, dim3(T), dim3(kThreads), sizeof(float) * (H + K + 160 + 32 + 4), s, descs, T, H, K,
+  hipLaunchKernelGGL(k_velo_heads, dim3(T), dim3(kFoldThreads),
+                     sizeof(float) * (H + K + 160 + 32 + 16 + 4 * (size_t)std::max(K, 160)), s, descs, T, H, K,
                      step->lstm_h, nets->ctrl_wt, nets->ctrl_b, nets->lr_w, nets->lr_b, nets->bank, totals, canon, wfold,
                      step->controls_out, step->lr_mult_out);
   HIP_TRY(mark());
@@ -749,7 +752,8 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   if (n_el > 0) hipLaunchKernelGGL(k_adafac_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, dec, stats, gl);
   HIP_TRY(mark());
   hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, totals, (const float*)nullptr, vs,
-                     (float*)nullptr);
+                     (float*)nullptr, 0, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
+                     (const float*)nullptr, (float*)nullptr);
   HIP_TRY(mark());
   hipLaunchKernelGGL(k_adafac_fold, dim3(T), dim3(kThreads), 0, s, descs, dyn, totals, net, wfold);
   HIP_TRY(mark());

@@ -200,10 +200,15 @@ class VeLO_CUDA(Optimizer):
         def v(b):
             return b.detach().float().contiguous().to(self.device)
 
+        def gates_last(w):
+            # (4H, 2H) with gate blocks i, g, f, o -> (2H, H, 4): a unit's four gate weights side by side
+            h4, k2 = w.shape
+            return w.detach().float().reshape(4, h4 // 4, k2).permute(2, 1, 0).contiguous().to(self.device)
+
         self._w = dict(
             mix2_wt=t(r.mix_layer2.weight), mix2_b=v(r.mix_layer2.bias),
             fmix_wt=t(r.final_mix_layer.weight), fmix_b=v(r.final_mix_layer.bias),
-            lstm_wt=t(r.lstm.linear.weight), lstm_b=v(r.lstm.linear.bias),
+            lstm_wt=gates_last(r.lstm.linear.weight), lstm_b=v(r.lstm.linear.bias),
             ctrl_wt=t(r.rnn_to_controls.weight), ctrl_b=v(r.rnn_to_controls.bias),
             lr_w=v(r.step_size.weight.reshape(-1)), lr_b=v(r.step_size.bias),
             bank=pack_velo_bank(self.network_stack).to(self.device))

@@ -373,6 +373,7 @@ __global__ __launch_bounds__(kFoldThreads) void k_celo2_fold(const TDesc* __rest
                                                              const PyloTensorArgs* __restrict__ dyn,
                                                              const int* __restrict__ fac_list,
                                                              const double* __restrict__ stats_part,
+                                                             const double* __restrict__ seg_tot,
                                                              const float* __restrict__ mlp,
                                                              float* __restrict__ wfold, float* __restrict__ chan_ms) {
   constexpr int G = kFoldThreads / kNStat;  // 56 groups x 18 channels
@@ -383,9 +384,11 @@ __global__ __launch_bounds__(kFoldThreads) void k_celo2_fold(const TDesc* __rest
   if (dyn[t].grad == nullptr) return;
   const int c = threadIdx.x % kNStat, gI = threadIdx.x / kNStat;
   if (gI < G) {
+    int n_rows;
+    const double* rows = stat_rows(d, stats_part, seg_tot, n_rows);
     double s = 0.0;
 #pragma unroll 16
-    for (int b = gI; b < d.nblk; b += G) s += stats_part[(size_t)(d.blk0 + b) * kStatW + stat_channel(c)];
+    for (int b = gI; b < n_rows; b += G) s += rows[(size_t)b * kStatW + stat_channel(c)];
     part[gI][c] = s;
   }
   __syncthreads();

@@ -154,7 +154,19 @@ __global__ __launch_bounds__(kThreads) void k_gnorm(const double* __restrict__ g
   __shared__ int fred[kWaves];
   double s = 0.0;
   int f = 0;
-  for (int i = threadIdx.x; i < nblk; i += kThreads) { s += gsq_part[i]; f |= flag_part[i]; }
+  // sixteen partials are fetched before the first is added: the one block is bound by load latency
+  for (int i0 = threadIdx.x; i0 < nblk; i0 += 16 * kThreads) {
+    double sv[16];
+    int fv[16];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int i = i0 + q * kThreads;
+      sv[q] = i < nblk ? gsq_part[i] : 0.0;
+      fv[q] = i < nblk ? flag_part[i] : 0;
+    }
+#pragma unroll
+    for (int q = 0; q < 16; ++q) { s += sv[q]; f |= fv[q]; }
+  }
   s = wave_sum(s);
   f = __any(f) ? 1 : 0;
   if ((threadIdx.x & 63) == 0) { red[threadIdx.x >> 6] = s; fred[threadIdx.x >> 6] = f; }
@@ -199,6 +211,44 @@ __global__ __launch_bounds__(kThreads) void k_p0_nd(const TDesc* __restrict__ de
   __syncthreads();
   if (grp == 0 && i < pick(d.len, w))
     part[pick(d.part_off, w) + (size_t)it.c * pick(d.len, w) + i] = ((lds[0][e] + lds[1][e]) + lds[2][e]) + lds[3][e];
+}
+
+// =============================================================================================
+// First stage of the per-tensor reduction of the statistics partials, for tensors with thousands
+// of rows: one block adds up kSegRows rows, so that the per-tensor block that follows (one block,
+// hence one CU's bandwidth) reads a few dozen rows instead of thousands.  Fixed order throughout.
+// Item: tensor, first row (relative to the tensor's rows), number of rows.
+// =============================================================================================
+__global__ __launch_bounds__(kThreads) void k_stat_segsum(const TDesc* __restrict__ descs,
+                                                          const Item* __restrict__ items,
+                                                          const double* __restrict__ stats_part,
+                                                          double* __restrict__ seg_tot) {
+  constexpr int G = kThreads / kStatW;  // 6 groups x 40 channels
+  __shared__ double part[G][kStatW];
+  const Item it = items[blockIdx.x];
+  const int blk0 = descs[it.tensor].blk0 + it.a;
+  const int c = threadIdx.x % kStatW, gI = threadIdx.x / kStatW;
+  if (gI < G) {
+    double s = 0.0;
+    for (int b0 = gI; b0 < it.b; b0 += 16 * G) {
+      double v[16];
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int b = b0 + q * G;
+        v[q] = b < it.b ? stats_part[(size_t)(blk0 + b) * kStatW + c] : 0.0;
+      }
+#pragma unroll
+      for (int q = 0; q < 16; ++q) s += v[q];
+    }
+    part[gI][c] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x < kStatW) {
+    double s = 0.0;
+#pragma unroll
+    for (int g2 = 0; g2 < G; ++g2) s += part[g2][threadIdx.x];
+    seg_tot[(size_t)blockIdx.x * kStatW + threadIdx.x] = s;
+  }
 }
 
 // =============================================================================================

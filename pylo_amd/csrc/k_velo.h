@@ -369,6 +369,7 @@ __device__ __forceinline__ float lo_lstm_feature(const TDesc& d, const PyloTenso
 __global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restrict__ descs,
                                                         const PyloTensorArgs* __restrict__ dyn, int T,
                                                         const double* __restrict__ stats_part,
+                                                        const double* __restrict__ seg_tot,
                                                         double* __restrict__ totals,
                                                         const float* __restrict__ lossfeat, VeloStep st,
                                                         float* __restrict__ xfeat, int H,
@@ -386,8 +387,10 @@ __global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restr
   if (gI < G) {
     double s = 0.0;
     if (a.grad != nullptr && c < 38) {
+      int n_rows;
+      const double* rows = stat_rows(d, stats_part, seg_tot, n_rows);
 #pragma unroll 16
-      for (int b = gI; b < d.nblk; b += G) s += stats_part[(size_t)(d.blk0 + b) * kStatW + c];
+      for (int b = gI; b < n_rows; b += G) s += rows[(size_t)b * kStatW + c];
     }
     part[gI][c] = s;
   }
@@ -420,22 +423,41 @@ __global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restr
 // LSTM (VeLO_RNN.py:43-66,110-135).  All weights are pre-transposed to (in, out) by the host.
 // Rows are in the reference's order r = T-1-t.
 // ---------------------------------------------------------------------------------------------
+// Maximum of relu(mix2 x) over a chunk of rows: many tensors only (T > kMixRows), so that the blocks of
+// k_velo_mix do not each walk every row.  Block (x, y): 64 hidden units, rows y*kMixRows .. +kMixRows.
+constexpr int kMixRows = 256;
+__device__ __forceinline__ float mix_colmax(const float* __restrict__ m2, int r0, int r1, int H, int u,
+                                            float (*mx_s)[64]) {
+  const int lane = threadIdx.x & 63, grp = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  float mx = 0.0f;  // relu output is >= 0
+#pragma unroll 8
+  for (int r = r0 + grp; r < r1; r += kWaves) mx = fmaxf(mx, m2[(size_t)r * H + u]);
+  mx_s[grp][lane] = mx;
+  __syncthreads();
+  return fmaxf(fmaxf(mx_s[0][lane], mx_s[1][lane]), fmaxf(mx_s[2][lane], mx_s[3][lane]));
+}
+
+__global__ __launch_bounds__(kThreads) void k_velo_colmax(const float* __restrict__ mixbuf, int T, int H,
+                                                          float* __restrict__ pmax /* [chunks][H] */) {
+  __shared__ float mx_s[kWaves][64];
+  const int u = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int r0 = blockIdx.y * kMixRows;
+  const float v = mix_colmax(mixbuf, r0, min(T, r0 + kMixRows), H, u, mx_s);
+  if (threadIdx.x < 64) pmax[(size_t)blockIdx.y * H + u] = v;
+}
+
 // x' = final_mix(x) + max_r relu(mix2(x));  xT[u][r] = x'[r][u], xT[H+u][r] = h[r][u].  The per-row
 // products are in mixbuf (written by k_lo_reduce).  Block (x, y): 64 hidden units (one per lane) and
-// the 8 rows 8y .. 8y+7, two per wave; every block takes the maximum over all rows itself.
+// the 8 rows 8y .. 8y+7, two per wave; the maximum over all rows is taken by every block itself, or
+// from the per-chunk maxima of k_velo_colmax when there are many rows.
 __global__ __launch_bounds__(kThreads) void k_velo_mix(const float* __restrict__ mixbuf, int T, int Tpad, int H,
+                                                       const float* __restrict__ pmax, int n_chunks,
                                                        const float* __restrict__ h_state, float* __restrict__ xT) {
   __shared__ float mx_s[kWaves][64];
   const int lane = threadIdx.x & 63, grp = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int u = blockIdx.x * 64 + lane;  // H is a multiple of 64
-  const float* m2 = mixbuf;
   const float* fm = mixbuf + (size_t)T * H;
-  float mx = 0.0f;  // relu output is >= 0
-#pragma unroll 8
-  for (int r = grp; r < T; r += kWaves) mx = fmaxf(mx, m2[(size_t)r * H + u]);
-  mx_s[grp][lane] = mx;
-  __syncthreads();
-  const float v = fmaxf(fmaxf(mx_s[0][lane], mx_s[1][lane]), fmaxf(mx_s[2][lane], mx_s[3][lane]));
+  const float v = pmax != nullptr ? mix_colmax(pmax, 0, n_chunks, H, u, mx_s) : mix_colmax(mixbuf, 0, T, H, u, mx_s);
 #pragma unroll
   for (int q = 0; q < kGateBT / kWaves; ++q) {
     const int r = blockIdx.y * kGateBT + q * kWaves + grp;  // < Tpad

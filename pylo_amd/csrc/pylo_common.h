@@ -62,6 +62,7 @@ struct TDesc {
   int rcm_stride;   //      is the mean over that axis, one value per slice (2-D: one value per tensor)
   int n_strips, n_colblk;
   int blk0, nblk;   // range of element-chunk blocks (rows of the statistics partials)
+  int seg0, nseg;   // tensors with many rows: their rows are first summed in segments of kSegRows (k_stat_segsum)
   int fac_slot;     // index among factored tensors, -1 otherwise
   int rank;         // number of dims larger than 1 (VeLO's rank one-hot feature)
   long long part_off[2];  // floats, partial sums of g^2
@@ -99,6 +100,17 @@ struct Item {
 // reference's 30-channel order, then the per-tensor LSTM input sums of VeLO taken over the
 // accumulators *before* the update: sum m_k (30..32), sum m_k^2 (33..35), sum rms (36), sum rms^2 (37).
 constexpr int kStatW = 40;
+constexpr int kSegRows = 256;   // rows of statistics partials one k_stat_segsum block adds up
+constexpr int kSegMin = 1024;   // tensors with more rows than this are reduced in two stages
+
+// Where a per-tensor reduction finds the tensor's rows: its segment sums if it has any, else its partials.
+__device__ __forceinline__ const double* stat_rows(const TDesc& d, const double* stats_part, const double* seg_tot,
+                                                   int& n_rows) {
+  if (d.nseg > 0) { n_rows = d.nseg; return seg_tot + (size_t)d.seg0 * kStatW; }
+  n_rows = d.nblk;
+  return stats_part + (size_t)d.blk0 * kStatW;
+}
+
 constexpr int kSumM = 30, kSumMM = 33, kSumR = 36, kSumRR = 37;
 
 struct Globals {

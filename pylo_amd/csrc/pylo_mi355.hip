@@ -64,15 +64,15 @@ bool factored_dims(int kind, const PyloTensorShape& s, int* dc, int* dr) {
 
 struct Layout {
   std::vector<TDesc> descs;
-  std::vector<Item> p0_items, nd_items, sl_items, el_items, ap_items, ga_items, fin_items, v0a_items, v0b_items;
+  std::vector<Item> p0_items, nd_items, sl_items, seg_items, el_items, ap_items, ga_items, fin_items, v0a_items, v0b_items;
   std::vector<int> fac_list;
   std::vector<int> dc, dr;
   int H = 8;  // width of the first MLP layer (terms per row / column)
   int Tpad = 0;
   bool global_norm = false;  // AdafacLO kind: every tensor has P0 items, the call may clip by global norm
-  size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_sl_items, off_el_items, off_ap_items, off_ga_items, off_fin_items, off_finpart, off_finscale, off_v0a_items, off_v0b_items, off_fac_list,
+  size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_sl_items, off_seg_items, off_segtot, off_el_items, off_ap_items, off_ga_items, off_fin_items, off_finpart, off_finscale, off_v0a_items, off_v0b_items, off_fac_list,
       off_part, off_gsq, off_flag, off_globals, off_fac, off_term, off_v0part, off_bscale, off_stats, off_wfold,
-      off_chan_ms, off_totals, off_xfeat, off_lossfeat, off_xT, off_mixbuf, off_canon, total;
+      off_chan_ms, off_totals, off_xfeat, off_lossfeat, off_xT, off_mixbuf, off_pmax, off_canon, total;
 };
 
 int first_layer_width(int kind) { return kind == PYLO_KIND_CELO2 ? 8 : kind == PYLO_KIND_VELO ? 4 : 32; }
@@ -213,6 +213,11 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       for (long long c = 0; c * chunk < n; ++c) L.el_items.push_back(Item{t, (int)c, 0, 0});
     }
     d.nblk = (int)L.el_items.size() - d.blk0;
+    if (d.nblk > kSegMin) {  // two-stage reduction of the statistics partials (k_stat_segsum)
+      d.seg0 = (int)L.seg_items.size();
+      for (int r = 0; r < d.nblk; r += kSegRows) L.seg_items.push_back(Item{t, r, std::min(kSegRows, d.nblk - r), 0});
+      d.nseg = (int)L.seg_items.size() - d.seg0;
+    }
     // blocks of ELO-CELO2's finishing pass (after Newton-Schulz): linear 8192-element pieces of the MLP tensors
     if (kind == PYLO_KIND_CELO2 && d.mode != kModeFlat) {
       d.fin_blk0 = (int)L.fin_items.size();
@@ -243,6 +248,8 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_p0_items = take(sizeof(Item) * L.p0_items.size());
   L.off_nd_items = take(sizeof(Item) * L.nd_items.size());
   L.off_sl_items = take(sizeof(Item) * L.sl_items.size());
+  L.off_seg_items = take(sizeof(Item) * L.seg_items.size());
+  L.off_segtot = take(sizeof(double) * kStatW * L.seg_items.size());
   L.off_el_items = take(sizeof(Item) * L.el_items.size());
   L.off_ap_items = take(sizeof(Item) * L.ap_items.size());
   L.off_ga_items = take(sizeof(Item) * L.ga_items.size());
@@ -270,6 +277,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_lossfeat = take(sizeof(float) * 16);
   L.off_xT = take(kind == PYLO_KIND_VELO ? sizeof(float) * 2 * (size_t)velo_hidden * L.Tpad : 0);
   L.off_mixbuf = take(kind == PYLO_KIND_VELO ? sizeof(float) * 2 * (size_t)velo_hidden * T : 0);
+  L.off_pmax = take(kind == PYLO_KIND_VELO ? sizeof(float) * (size_t)velo_hidden * ((T + kMixRows - 1) / kMixRows) : 0);
   L.off_canon = take(kind == PYLO_KIND_VELO ? sizeof(float) * kVCanon * (size_t)T : 0);
   L.total = off;
   return 0;
@@ -337,6 +345,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_p0_items, L.p0_items.data(), sizeof(Item) * L.p0_items.size());
   if (e == hipSuccess) e = up(L.off_nd_items, L.nd_items.data(), sizeof(Item) * L.nd_items.size());
   if (e == hipSuccess) e = up(L.off_sl_items, L.sl_items.data(), sizeof(Item) * L.sl_items.size());
+  if (e == hipSuccess) e = up(L.off_seg_items, L.seg_items.data(), sizeof(Item) * L.seg_items.size());
   if (e == hipSuccess) e = up(L.off_el_items, L.el_items.data(), sizeof(Item) * L.el_items.size());
   if (e == hipSuccess) e = up(L.off_ap_items, L.ap_items.data(), sizeof(Item) * L.ap_items.size());
   if (e == hipSuccess) e = up(L.off_ga_items, L.ga_items.data(), sizeof(Item) * L.ga_items.size());
@@ -554,7 +563,13 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   HIP_TRY(mark());
   if (n_el > 0) hipLaunchKernelGGL(k_celo2_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, gl, dec, stats);
   HIP_TRY(mark());
-  if (n_fac > 0) hipLaunchKernelGGL(k_celo2_fold, dim3(n_fac), dim3(kFoldThreads), 0, s, descs, dyn, fac_list, stats, mlp, wfold, chan_ms);
+  const Item* seg_items = P->at<Item>(L.off_seg_items);
+  double* seg_tot = P->at<double>(L.off_segtot);
+  const int n_seg = (int)L.seg_items.size();
+  if (n_seg > 0) hipLaunchKernelGGL(k_stat_segsum, dim3(n_seg), dim3(kThreads), 0, s, descs, seg_items, stats, seg_tot);
+  if (n_fac > 0)
+    hipLaunchKernelGGL(k_celo2_fold, dim3(n_fac), dim3(kFoldThreads), 0, s, descs, dyn, fac_list, stats, seg_tot, mlp, wfold,
+                       chan_ms);
   HIP_TRY(mark());
   if (n_el > 0) {
     if (P->mlp_on_matrix_pipe)
@@ -668,10 +683,19 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
   hipLaunchKernelGGL(k_velo_loss, dim3(1), dim3(64), 0, s, step->loss_means, step->loss_running_min, step->loss_decays,
                      step->loss_iteration, step->loss, lossfeat);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, totals, lossfeat, vs, xfeat,
+  const Item* seg_items = P->at<Item>(L.off_seg_items);
+  double* seg_tot = P->at<double>(L.off_segtot);
+  const int n_seg = (int)L.seg_items.size();
+  if (n_seg > 0) hipLaunchKernelGGL(k_stat_segsum, dim3(n_seg), dim3(kThreads), 0, s, descs, seg_items, stats, seg_tot);
+  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, seg_tot, totals, lossfeat, vs, xfeat,
                      H, nets->mix2_wt, nets->mix2_b, nets->fmix_wt, nets->fmix_b, mixbuf);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_velo_mix, dim3(H / 64, L.Tpad / kGateBT), dim3(kThreads), 0, s, (const float*)mixbuf, T, L.Tpad, H, step->lstm_h, xT);
+  const int n_chunks = (T + kMixRows - 1) / kMixRows;
+  float* pmax = n_chunks > 1 ? P->at<float>(L.off_pmax) : nullptr;
+  if (pmax != nullptr)
+    hipLaunchKernelGGL(k_velo_colmax, dim3(H / 64, n_chunks), dim3(kThreads), 0, s, (const float*)mixbuf, T, H, pmax);
+  hipLaunchKernelGGL(k_velo_mix, dim3(H / 64, L.Tpad / kGateBT), dim3(kThreads), 0, s, (const float*)mixbuf, T, L.Tpad, H,
+                     (const float*)pmax, n_chunks, step->lstm_h, xT);
   HIP_TRY(mark());
   hipLaunchKernelGGL(k_velo_gates, dim3((L.Tpad / kGateBT) * (H / kGateU)), dim3(kThreads), 0, s, xT, T, L.Tpad, H,
                      nets->lstm_wt, nets->lstm_b, step->lstm_h, step->lstm_c);
@@ -751,7 +775,11 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   HIP_TRY(mark());
   if (n_el > 0) hipLaunchKernelGGL(k_adafac_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, dec, stats, gl);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, totals, (const float*)nullptr, vs,
+  const Item* seg_items = P->at<Item>(L.off_seg_items);
+  double* seg_tot = P->at<double>(L.off_segtot);
+  const int n_seg = (int)L.seg_items.size();
+  if (n_seg > 0) hipLaunchKernelGGL(k_stat_segsum, dim3(n_seg), dim3(kThreads), 0, s, descs, seg_items, stats, seg_tot);
+  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, seg_tot, totals, (const float*)nullptr, vs,
                      (float*)nullptr, 0, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
                      (const float*)nullptr, (float*)nullptr);
   HIP_TRY(mark());

@@ -147,9 +147,11 @@ __global__ __launch_bounds__(kThreads) void k_p0(const TDesc* __restrict__ descs
   }
 }
 
+// use_flags == 0: the caller has shown that no element can exceed its clamp after scaling (the scaled
+// gradient is bounded by clip_norm), so the exact pass never runs and the flags are ignored.
 __global__ __launch_bounds__(kThreads) void k_gnorm(const double* __restrict__ gsq_part,
                                                     const int* __restrict__ flag_part, int nblk,
-                                                    Globals* __restrict__ gl) {
+                                                    Globals* __restrict__ gl, int use_flags) {
   __shared__ double red[kWaves];
   __shared__ int fred[kWaves];
   double s = 0.0;
@@ -173,7 +175,7 @@ __global__ __launch_bounds__(kThreads) void k_gnorm(const double* __restrict__ g
   __syncthreads();
   if (threadIdx.x == 0) {
     gl->gnorm = (float)sqrt((red[0] + red[1]) + (red[2] + red[3]));
-    gl->flag = fred[0] | fred[1] | fred[2] | fred[3];
+    gl->flag = use_flags ? (fred[0] | fred[1] | fred[2] | fred[3]) : 0;
   }
 }
 
@@ -354,15 +356,29 @@ __device__ __forceinline__ void vector_terms(const TDesc& d, int which, bool is_
                                              const float (&x1)[3], const float* __restrict__ w1,
                                              const float* __restrict__ b1, float* __restrict__ term) {
   const int ch_f = is_r ? 15 : 18, ch_q = is_r ? 21 : 24;
+  // The weight rows are the same for every lane: eight outputs at a time they arrive as a few wide
+  // scalar loads (w1 and b1 are not written by the running kernel).
+  static_assert(H % 4 == 0, "first-layer width");
+  constexpr int JB = H < 8 ? H : 8;
 #pragma unroll
-  for (int j = 0; j < H; ++j) {
-    float t = (which == 0) ? b1[j] : 0.0f;
+  for (int j0 = 0; j0 < H; j0 += JB) {
+    float wf[3][JB], wq[3][JB], bb[JB];
 #pragma unroll
     for (int k = 0; k < 3; ++k) {
-      t = fmaf(x0[k], w1[(ch_f + k) * H + j], t);
-      t = fmaf(x1[k], w1[(ch_q + k) * H + j], t);
+      load_uniform<JB>(w1 + (ch_f + k) * H + j0, wf[k]);
+      load_uniform<JB>(w1 + (ch_q + k) * H + j0, wq[k]);
     }
-    term[term_index<H>(d, which, j, i)] = t;
+    load_uniform<JB>(b1 + j0, bb);
+#pragma unroll
+    for (int j = 0; j < JB; ++j) {
+      float t = (which == 0) ? bb[j] : 0.0f;
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        t = fmaf(x0[k], wf[k][j], t);
+        t = fmaf(x1[k], wq[k][j], t);
+      }
+      term[term_index<H>(d, which, j0 + j, i)] = t;
+    }
   }
 }
 
@@ -411,15 +427,16 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
   const int rI = d.vec0_is_r ? 0 : 1, cI = 1 - rI;
   const double* tr = tot + rI * kNV0;
   const double* tc = tot + cI * kNV0;
-  const double len_r = (double)d.len[rI], len_c = (double)d.len[cI];
+  // means as sum * (1 / len): one double division per vector instead of nine
+  const double inv_r = 1.0 / (double)d.len[rI], inv_c = 1.0 / (double)d.len[cI];
   BScale bs;
 #pragma unroll
   for (int k = 0; k < 3; ++k) {
-    bs.rcm[k] = (float)(tr[k * 3 + 0] / len_r);
-    bs.s[k] = rsq(norm_eps + (float)(tr[k * 3 + 1] / len_r));        // fac_r_k
-    bs.s[3 + k] = rsq(norm_eps + (float)(tc[k * 3 + 1] / len_c));    // fac_c_k
-    bs.s[6 + k] = rsq(norm_eps + (float)(tr[k * 3 + 2] / len_r));    // rsqrt(fac_r_k + 1e-8)
-    bs.s[9 + k] = rsq(norm_eps + (float)(tc[k * 3 + 2] / len_c));    // rsqrt(fac_c_k + 1e-8)
+    bs.rcm[k] = (float)(tr[k * 3 + 0] * inv_r);
+    bs.s[k] = rsq(norm_eps + (float)(tr[k * 3 + 1] * inv_r));        // fac_r_k
+    bs.s[3 + k] = rsq(norm_eps + (float)(tc[k * 3 + 1] * inv_c));    // fac_c_k
+    bs.s[6 + k] = rsq(norm_eps + (float)(tr[k * 3 + 2] * inv_r));    // rsqrt(fac_r_k + 1e-8)
+    bs.s[9 + k] = rsq(norm_eps + (float)(tc[k * 3 + 2] * inv_c));    // rsqrt(fac_c_k + 1e-8)
   }
   bs.pad_ = 0.0f;
   const int which = it.b;

@@ -497,6 +497,21 @@ int check_args(const PyloPlan* P, const PyloTensorArgs* args, bool need_all_grad
   return 0;
 }
 
+// The sums of g^2 of a globally clipped 2-D tensor are taken on the raw gradient and scaled afterwards;
+// that is exact unless some scaled element lies beyond the tensor's clamp, in which case a second
+// pass redoes them (k_p0, pass 1).  The scaled gradient is bounded by the global norm times the scale,
+// i.e. by clip_norm, so with clip_norm below clip_val (1.0 against 1000 by default) the second pass can
+// never be needed and is not launched.  Tensors whose NaNs are replaced always keep it.
+bool exact_pass_possible(const PyloPlan* P, const PyloTensorArgs* args) {
+  for (int t = 0; t < P->T; ++t) {
+    const PyloTensorArgs& a = args[t];
+    if (a.grad == nullptr || !(a.clip_norm > 0.0f)) continue;
+    if (P->L.descs[t].nan0) return true;
+    if (a.clip_val > 0.0f && !(a.clip_norm <= 0.99f * a.clip_val)) return true;
+  }
+  return false;
+}
+
 struct Marks {  // per-launch HIP events when timing is on
   PyloPlan* P;
   hipStream_t s;
@@ -546,12 +561,14 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   const PyloDecays dec = *decays;
   Marks mark(P, s);
 
+  const bool exact_pass = exact_pass_possible(P, args);
   HIP_TRY(mark());
   if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl);
+  hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl, exact_pass ? 1 : 0);
   HIP_TRY(mark());
-  if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1);
+  if (n_p0 > 0 && exact_pass)
+    hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1);
   if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part, gl);
   HIP_TRY(mark());
   if (n_v0a > 0)
@@ -758,8 +775,10 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   HIP_TRY(mark());
   if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0);
   if (clips) {
-    hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl);
-    if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1);
+    const bool exact_pass = exact_pass_possible(P, args);
+    hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl, exact_pass ? 1 : 0);
+    if (n_p0 > 0 && exact_pass)
+      hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1);
   }
   HIP_TRY(mark());
   if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part, gl);

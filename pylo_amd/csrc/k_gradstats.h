@@ -369,6 +369,7 @@ __device__ __forceinline__ void vector_terms(const TDesc& d, int which, bool is_
       load_uniform<JB>(w1 + (ch_q + k) * H + j0, wq[k]);
     }
     load_uniform<JB>(b1 + j0, bb);
+    float tv[JB];
 #pragma unroll
     for (int j = 0; j < JB; ++j) {
       float t = (which == 0) ? bb[j] : 0.0f;
@@ -377,7 +378,15 @@ __device__ __forceinline__ void vector_terms(const TDesc& d, int which, bool is_
         t = fmaf(x0[k], wf[k][j], t);
         t = fmaf(x1[k], wq[k][j], t);
       }
-      term[term_index<H>(d, which, j0 + j, i)] = t;
+      tv[j] = t;
+    }
+    if (d.mode == kModeFac2D) {  // [index][H]: the entry's outputs are adjacent, 16 bytes a store
+#pragma unroll
+      for (int j = 0; j < JB; j += 4)
+        *(float4*)(term + term_index<H>(d, which, j0 + j, i)) = make_float4(tv[j], tv[j + 1], tv[j + 2], tv[j + 3]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < JB; ++j) term[term_index<H>(d, which, j0 + j, i)] = tv[j];
     }
   }
 }
@@ -447,8 +456,12 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
   for (int i = it.a * kV0bEnt + threadIdx.x; i < min(len, (it.a + 1) * kV0bEnt); i += kThreads) {
     float fct[3], x0[3], x1[3];
     vector_entry(d, is_r, fac, len, i, bs, fct, x0, x1);
+    if (d.mode == kModeFac2D) {  // [index][4]: one 16-byte store
+      *(float4*)(fac_tab + fac_index(d, which, 0, i)) = make_float4(fct[0], fct[1], fct[2], 0.0f);
+    } else {
 #pragma unroll
-    for (int k = 0; k < 3; ++k) fac_tab[fac_index(d, which, k, i)] = fct[k];
+      for (int k = 0; k < 3; ++k) fac_tab[fac_index(d, which, k, i)] = fct[k];
+    }
     if (w1 != nullptr) vector_terms<H>(d, which, is_r, i, x0, x1, w1, b1 + (size_t)it.tensor * b1_stride, term_tab);
   }
 }

@@ -33,6 +33,8 @@ B_ADAM = 44                    # 1-D AdamW branch: read g,p,m0..2,rms; write m0.
 # HBM bytes of one k_celo2_apply launch on the GPT-2-small set, from rocprofv3 FETCH_SIZE x 2.000 KiB +
 # WRITE_SIZE x 1.000 KiB (factors calibrated on a 1 GiB copy in the same runs; --calib-copy)
 TRAFFIC_APPLY_GPT2S = 5.528e9
+# the same for one k_velo_apply launch on the ViT-B/16 set (1 030 664 x 2 KiB fetched + 1 689 522 KiB written)
+TRAFFIC_APPLY_VITB16 = 3.841e9
 
 
 def gpt2_small_shapes():
@@ -270,7 +272,9 @@ def other_workload(a):
     k = names.index(apply_kernel)
     apply_gbs = (n2d * B_APPLY + n1d * 68) / (float(mean[k]) * 1e-3) / 1e9
     roof = {"bound": "hbm", "kernel": apply_kernel, "achieved": apply_gbs, "peak": HBM_PEAK_GBS,
-            "unit": "GB/s", "frac": apply_gbs / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": float(mean[k])}
+            "unit": "GB/s", "frac": apply_gbs / HBM_PEAK_GBS,
+            "traffic": TRAFFIC_APPLY_VITB16 if a.workload == "vit_velo" else None,
+            "algorithmic_bytes_per_launch": n2d * B_APPLY + n1d * 68, "avg_launch_ms": float(mean[k])}
     if a.workload == "llama_adafac":
         # the 16 -> 32 -> 32 -> 2 element MLP: 1 600 FMAs per element of a >= 2-D tensor, fp32 matrix pipe
         tflops = n2d * 3200.0 / (float(mean[k]) * 1e-3) / 1e12

@@ -157,3 +157,44 @@ def test_adafac_state_dict_resume():
     assert set(st.keys()) == {"step", "exp_avg_sq_r", "exp_avg_sq_c", "exp_avg_sq", "exp_avg"}
     assert st["exp_avg"].shape == (3, 24, 16) and st["exp_avg_sq_r"].shape == (3, 1, 16)
     assert st["step"].dtype == torch.float64 and float(st["step"]) == 8.0
+
+
+def test_mulo_wrapper_runs_the_fused_step_with_per_group_learning_rates():
+    """MuLO_CUDA (pylo/optim/MuLO_cuda.py:12-61) = AdafacLO_CUDA over groups split by muP width multiplier
+    with lr / multiplier: same parameters, bit for bit, as AdafacLO_CUDA given those groups directly."""
+    from pylo_amd import AdafacLO_CUDA, MuLO_CUDA
+    from pylo_amd.models import MetaMLP
+
+    class Inf:
+        def __init__(self, n, w):
+            self.n, self.w = n, w
+
+        def ninf(self):
+            return self.n
+
+        def width_mult(self):
+            return self.w
+
+    torch.manual_seed(2)
+    net = MetaMLP(39, 32, 1)
+    shapes, infs = [(40, 128), (24, 20), (50,), (16, 16)], [Inf(2, 4.0), Inf(2, 2.0), Inf(1, 1.0), Inf(2, 4.0)]
+    gen = torch.Generator().manual_seed(8)
+    init = [torch.randn(s, generator=gen) * 0.3 for s in shapes]
+    grads = [[torch.randn(s, generator=gen).cuda() * 0.1 for s in shapes] for _ in range(3)]
+    a = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+    for p, i in zip(a, infs):
+        p.infshape = i
+    oa = MuLO_CUDA(a, lr=0.8, network=copy.deepcopy(net))
+    assert [g["lr"] for g in oa.param_groups] == [0.2, 0.4, 0.8]
+    b = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+    ob = AdafacLO_CUDA([dict(params=[b[0], b[3]], lr=0.2), dict(params=[b[1]], lr=0.4), dict(params=[b[2]], lr=0.8)],
+                       lr=0.8, network=copy.deepcopy(net))
+    for t in range(3):
+        for ps in (a, b):
+            for p, g in zip(ps, grads[t]):
+                p.grad = g.clone()
+        oa.step()
+        ob.step()
+    for x, y, v in zip(a, b, init):
+        assert torch.equal(x, y)
+        assert not torch.equal(x.cpu(), v)

@@ -17,6 +17,12 @@ state, ``torch.optim.AdamW`` for the 1-D branch, ``torch.nn.LSTMCell`` with
 permuted gates for the LSTM, fp64 brute force for Newton-Schulz and the feature
 list, ``numpy.argsort`` for ``factored_dims``.
 
+Parity unpinned: ``AdafacOracle(per_param_step=True)``.  That switch restates the CUDA class's
+per-parameter step counter (AdafacLO_cuda.py:304-305,400), and the CUDA class cannot run here, so
+no golden trajectory covers a parameter that sat steps out.  It only selects which step number
+feeds the time features; the time features themselves, and everything else in the class, are
+pinned by the golden trajectories of AdafacLO_naive and ELO_naive.
+
 Every function cites the reference lines it restates.
 """
 

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define PYLO_MI355_ABI_VERSION 2
+#define PYLO_MI355_ABI_VERSION 3
 #define PYLO_MAX_DIMS 8
 #define PYLO_MAX_GROUPS 8   /* parameter groups with their own step counter (VeLO) */
 
@@ -154,8 +154,11 @@ int pylo_mi355_celo2_step(PyloPlan* plan, const PyloTensorArgs* args, const Pylo
  *     step = x * rsqrt(1e-9 + mean(x^2 over the tensor)) * step_mult      (step_mult carries rmsmult)
  *     param <- param - lr * (step + weight_decay * param)
  * Fields read per tensor: grad (only as "takes part" flag), param, step_out, lr, weight_decay,
- * step_mult.  PYLO_F_ADAM tensors are skipped.  Three launches: sum of squares per 8192-element
- * block, per-tensor scale (fixed-order fp64 sum), update.  16 bytes per element.
+ * step_mult.  PYLO_F_ADAM tensors are skipped; tensors of fewer than two dims on the MLP path are
+ * handled like matrices (their normaliser is over the whole vector); tensors with more than two dims
+ * are refused, since their normaliser is per slice of the last two dims (ELO_CELO2_naive.py:217-218,235).
+ * Three launches: sum of squares per 8192-element block, per-tensor scale (fixed-order fp64 sum),
+ * update.  16 bytes per element.
  */
 int pylo_mi355_celo2_finish(PyloPlan* plan, const PyloTensorArgs* args, void* stream);
 
@@ -166,7 +169,8 @@ int pylo_mi355_celo2_finish(PyloPlan* plan, const PyloTensorArgs* args, void* st
  * (bank mixing) and velo_cuda.py:502-546 (accumulator updates)).
  *
  * All weight matrices are device pointers, fp32, stored (in, out) -- i.e. the transpose of the
- * torch.nn.Linear weights of pylo/models/VeLO_RNN.py; `bank` is (n_bank, 159): per entry
+ * torch.nn.Linear weights of pylo/models/VeLO_RNN.py (lstm_wt additionally with the gates innermost,
+ * see the field); `bank` is (n_bank, 159): per entry
  * W_in (4,30) | b_in 4 | W_h (4,4) | b_h 4 | W_out (3,4) | b_out 3, each (out, in) as in VeLO_MLP.py:63-77.
  */
 typedef struct {

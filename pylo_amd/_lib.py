@@ -87,7 +87,7 @@ def load():
                                          C.POINTER(VeloStep), C.c_void_p]
     lib.pylo_mi355_adafac_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.c_void_p, C.c_float,
                                            C.c_void_p]
-    if lib.pylo_mi355_abi_version() != 2:
+    if lib.pylo_mi355_abi_version() != 3:
         raise RuntimeError("libpylo_mi355.so: ABI version mismatch, rebuild it")
     _lib = lib
     return lib

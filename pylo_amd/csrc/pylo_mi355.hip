@@ -477,7 +477,8 @@ int check_args(const PyloPlan* P, const PyloTensorArgs* args, bool need_all_grad
     const PyloTensorArgs& a = args[t];
     const std::string at = " at tensor " + std::to_string(t);
     if (a.grad == nullptr) {
-      if (need_all_grads) return fail("step: every tensor needs a gradient" + at);
+      // an empty tensor has no gradient buffer to point to; its LSTM row sees zero statistics
+      if (need_all_grads && d.n > 0) return fail("step: every tensor needs a gradient" + at);
       continue;
     }
     if (d.n == 0) continue;

@@ -318,9 +318,9 @@ __device__ __forceinline__ int adafac_elem_row(int c) { return c == 0 ? 0 : (c <
 // units 4q..4q+3 of element e.  The D layout of one layer is a valid B layout of the next (input
 // slot (q, r) = unit 16 b + 4 q + r), so activations never move between lanes; only the 16 features
 // of the 64 elements a wave holds (one element per lane) are regrouped once per row through LDS
-// into four groups of 16 elements.  Per row of 64 elements: 32 + 64 MFMAs for the two layers and 8
-// that sum the output layer's per-lane partial products over q (A = 1); 1 600 FMAs per element in
-// all, bound by the fp32 matrix rate.
+// into four groups of 16 elements.  Per row of 64 elements: 32 + 64 MFMAs for the two layers; the
+// output layer's per-lane partial products are summed over q with two cross-lane moves each.
+// 1 536 matrix FMAs + 64 VALU FMAs per element, bound by the fp32 matrix rate.
 __device__ __forceinline__ v4f mfma16(float a, float b, v4f c) {
   return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
@@ -353,7 +353,6 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
   }
   const cfloat* nw = launder(net);
   const float bo0 = nw[kABO + 0], bo1 = nw[kABO + 1];
-  const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
   const float exp_scale = a.exp_mult * 1.44269504088896341f;
   float fb[4];
   load_vec_o<4>(fac_tab + d.fac_off[1], tk.col * 16u, fb);
@@ -446,8 +445,12 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
             p1 = fmaf(gv, wo[b][rr][1], p1);
           }
         }
-        const v4f t0 = mfma16(1.0f, p0, zero), t1 = mfma16(1.0f, p1, zero);  // sums over q, in every lane
-        if (q == gP + u) { o0 = t0[0]; o1 = t1[0]; }
+        // sum of the per-lane partial products over the four lane groups q (lanes el, el+16, el+32, el+48)
+        p0 += __shfl_xor(p0, 16, 64);
+        p1 += __shfl_xor(p1, 16, 64);
+        p0 += __shfl_xor(p0, 32, 64);
+        p1 += __shfl_xor(p1, 32, 64);
+        if (q == gP + u) { o0 = p0; o1 = p1; }
       }
     }
     o0 += bo0;

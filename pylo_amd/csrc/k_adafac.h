@@ -321,6 +321,10 @@ __device__ __forceinline__ int adafac_elem_row(int c) { return c == 0 ? 0 : (c <
 // into four groups of 16 elements.  Per row of 64 elements: 32 + 64 MFMAs for the two layers; the
 // output layer's per-lane partial products are summed over q with two cross-lane moves each.
 // 1 536 matrix FMAs + 64 VALU FMAs per element, bound by the fp32 matrix rate.
+// Row pitch of the feature exchange buffer: 64 elements plus 16 floats, so that the four lane groups
+// of a read (rows 4c'+q, q = 0..3, same 16 columns) fall into different LDS banks; with a pitch of 64
+// they collided and every read took twice as long.
+constexpr int kXPitch = 80;
 __device__ __forceinline__ v4f mfma16(float a, float b, v4f c) {
   return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
@@ -328,7 +332,7 @@ __device__ __forceinline__ v4f mfma16(float a, float b, v4f c) {
 __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTensorArgs& a, int task,
                                                   const EmaConsts& e, const float* __restrict__ fac_tab,
                                                   const float* __restrict__ term_tab, const float* wfold_t,
-                                                  const float* net, float* xch /* LDS [16][64] of this wave */) {
+                                                  const float* net, float* xch /* LDS [16][kXPitch] of this wave */) {
   const TileTask tk(d, task, d.atile_nct, 1);
   const int lane = threadIdx.x & 63, q = lane >> 4, el = lane & 15;
   // A operands: first layer [b][c'] (inputs 4c'+q), hidden layer [bo][b][r] (input 16b+4q+r)
@@ -362,7 +366,7 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
   const unsigned trow_off = 4 * q * 4u;
   const unsigned lo = lane * 4u;
   float* xw = xch + lane;                 // feature c of this lane's element goes to xch[c][lane]
-  const float* xr = xch + q * 64 + el;    // input 4c'+q of element 16g+el is xch[4c'+q][16g+el]
+  const float* xr = xch + q * kXPitch + el;  // input 4c'+q of element 16g+el is xch[4c'+q][16g+el]
   const float* g = a.grad + tk.first;
   float *p = a.param + tk.first, *m0 = a.mom + tk.first, *m1 = a.mom + d.n + tk.first,
         *m2 = a.mom + 2 * d.n + tk.first, *rms = a.rms + tk.first;
@@ -394,7 +398,7 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
     const float f[16] = {f18[0], f18[2], f18[3], f18[4], f18[5], f18[6], f18[7], f18[8], f18[9], f18[10],
                          f18[11], f18[12], f18[13], f18[15], f18[16], f18[17]};
 #pragma unroll
-    for (int c = 0; c < 16; ++c) xw[c * 64] = f[c];
+    for (int c = 0; c < 16; ++c) xw[c * kXPitch] = f[c];
     float o0 = 0.0f, o1 = 0.0f;
     // two groups of 16 elements at a time: four independent accumulator chains
 #pragma unroll
@@ -414,7 +418,7 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
       for (int c = 0; c < 4; ++c) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-          const float bv = xr[(4 * c) * 64 + 16 * (gP + u)];
+          const float bv = xr[(4 * c) * kXPitch + 16 * (gP + u)];
           h[u][0] = mfma16(a1[0][c], bv, h[u][0]);
           h[u][1] = mfma16(a1[1][c], bv, h[u][1]);
         }
@@ -497,7 +501,7 @@ void k_adafac_apply_tile(const TDesc* __restrict__ descs, const PyloTensorArgs* 
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
   set_grad_scale(d, a, gl);
-  __shared__ float xch[kWaves][16 * 64];
+  __shared__ float xch[kWaves][16 * kXPitch];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int task = it.a * 4 + wave;
   if (task >= d.atile_ntask) return;

@@ -330,12 +330,16 @@ __device__ __forceinline__ size_t term_index(const TDesc& d, int which, int j, i
 
 // Row_factor / col_factor of one entry, and the two normalised broadcast features it carries
 // (accumulator value and rsqrt(value + 1e-8)).  ELO_CELO2_naive.py:161-164,202-213
+// rcm: row_col_mean per decay; s0 / s1: normalisation scales of the vector's two broadcast channels.
+// (They arrive as plain arrays: indexing a BScale held in registers with `is_r ? k : 3 + k` makes the
+// compiler move the struct to LDS, 64 bytes a thread with bank conflicts on every access.)
 __device__ __forceinline__ void vector_entry(const TDesc& d, bool is_r, const float* fac, int len, int i,
-                                             const BScale& bs, float (&fct)[3], float (&x0)[3], float (&x1)[3]) {
+                                             const float (&rcm3)[3], const float (&s0)[3], const float (&s1)[3],
+                                             float (&fct)[3], float (&x0)[3], float (&x1)[3]) {
 #pragma unroll
   for (int k = 0; k < 3; ++k) {
     const float f = fac[(size_t)k * len + i];
-    float rcm = bs.rcm[k];
+    float rcm = rcm3[k];
     if (is_r && d.mode == kModeFacND) {  // mean over the dc axis of this entry's slice of fac_r
       const int sz = d.rcm_size, st = d.rcm_stride;
       const int base = (i / (sz * st)) * (sz * st) + i % st;
@@ -344,8 +348,8 @@ __device__ __forceinline__ void vector_entry(const TDesc& d, bool is_r, const fl
       rcm = (float)(s / (double)sz);
     }
     fct[k] = is_r ? rsq(fmaxf(f / (rcm + 1e-9f), 1e-9f)) : rsq(fmaxf(f, 1e-9f));
-    x0[k] = f * (is_r ? bs.s[k] : bs.s[3 + k]);
-    x1[k] = rsq(f + 1e-8f) * (is_r ? bs.s[6 + k] : bs.s[9 + k]);
+    x0[k] = f * s0[k];
+    x1[k] = rsq(f + 1e-8f) * s1[k];
   }
 }
 
@@ -438,24 +442,36 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
   const double* tc = tot + cI * kNV0;
   // means as sum * (1 / len): one double division per vector instead of nine
   const double inv_r = 1.0 / (double)d.len[rI], inv_c = 1.0 / (double)d.len[cI];
-  BScale bs;
+  const int which = it.b;
+  if (which == 0 && it.a == 0 && threadIdx.x == 0) {  // the tensor's scales, for k_terms
+    BScale bs;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      bs.rcm[k] = (float)(tr[k * 3 + 0] * inv_r);
+      bs.s[k] = rsq(norm_eps + (float)(tr[k * 3 + 1] * inv_r));        // fac_r_k
+      bs.s[3 + k] = rsq(norm_eps + (float)(tc[k * 3 + 1] * inv_c));    // fac_c_k
+      bs.s[6 + k] = rsq(norm_eps + (float)(tr[k * 3 + 2] * inv_r));    // rsqrt(fac_r_k + 1e-8)
+      bs.s[9 + k] = rsq(norm_eps + (float)(tc[k * 3 + 2] * inv_c));    // rsqrt(fac_c_k + 1e-8)
+    }
+    bs.pad_ = 0.0f;
+    bscale[d.fac_slot] = bs;
+  }
+  // this block's vector: its own sums sit at tot + which * kNV0
+  const double* own = tot + which * kNV0;
+  const double inv_own = 1.0 / (double)pick(d.len, which);
+  float rcm3[3], s0[3], s1[3];
 #pragma unroll
   for (int k = 0; k < 3; ++k) {
-    bs.rcm[k] = (float)(tr[k * 3 + 0] * inv_r);
-    bs.s[k] = rsq(norm_eps + (float)(tr[k * 3 + 1] * inv_r));        // fac_r_k
-    bs.s[3 + k] = rsq(norm_eps + (float)(tc[k * 3 + 1] * inv_c));    // fac_c_k
-    bs.s[6 + k] = rsq(norm_eps + (float)(tr[k * 3 + 2] * inv_r));    // rsqrt(fac_r_k + 1e-8)
-    bs.s[9 + k] = rsq(norm_eps + (float)(tc[k * 3 + 2] * inv_c));    // rsqrt(fac_c_k + 1e-8)
+    rcm3[k] = (float)(tr[k * 3 + 0] * inv_r);
+    s0[k] = rsq(norm_eps + (float)(own[k * 3 + 1] * inv_own));
+    s1[k] = rsq(norm_eps + (float)(own[k * 3 + 2] * inv_own));
   }
-  bs.pad_ = 0.0f;
-  const int which = it.b;
-  if (which == 0 && it.a == 0 && threadIdx.x == 0) bscale[d.fac_slot] = bs;
   const bool is_r = (which == 0) == (d.vec0_is_r != 0);
   const int len = pick(d.len, which);
   const float* fac = is_r ? a.fac_r : a.fac_c;
   for (int i = it.a * kV0bEnt + threadIdx.x; i < min(len, (it.a + 1) * kV0bEnt); i += kThreads) {
     float fct[3], x0[3], x1[3];
-    vector_entry(d, is_r, fac, len, i, bs, fct, x0, x1);
+    vector_entry(d, is_r, fac, len, i, rcm3, s0, s1, fct, x0, x1);
     if (d.mode == kModeFac2D) {  // [index][4]: one 16-byte store
       *(float4*)(fac_tab + fac_index(d, which, 0, i)) = make_float4(fct[0], fct[1], fct[2], 0.0f);
     } else {
@@ -479,16 +495,21 @@ __global__ __launch_bounds__(kThreads) void k_terms(const TDesc* __restrict__ de
   const TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
-  const BScale bs = bscale[d.fac_slot];
   const float* w1 = w1_all + (size_t)it.tensor * w_stride;
   const float* b1 = w1 + 30 * H;
   const int which = it.b;
   const bool is_r = (which == 0) == (d.vec0_is_r != 0);
   const int len = pick(d.len, which);
   const float* fac = is_r ? a.fac_r : a.fac_c;
+  // the tensor's scales, written by k_v0b: wave-uniform, through the scalar cache
+  const BScale* bs = bscale + d.fac_slot;
+  float rcm3[3], s0[3], s1[3];
+  load_uniform<3>(bs->rcm, rcm3);
+  load_uniform<3>(bs->s + (is_r ? 0 : 3), s0);
+  load_uniform<3>(bs->s + (is_r ? 6 : 9), s1);
   for (int i = it.a * kV0bEnt + threadIdx.x; i < min(len, (it.a + 1) * kV0bEnt); i += kThreads) {
     float fct[3], x0[3], x1[3];
-    vector_entry(d, is_r, fac, len, i, bs, fct, x0, x1);
+    vector_entry(d, is_r, fac, len, i, rcm3, s0, s1, fct, x0, x1);
     vector_terms<H>(d, which, is_r, i, x0, x1, w1, b1, term_tab);
   }
 }

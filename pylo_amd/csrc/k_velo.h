@@ -474,14 +474,15 @@ __global__ __launch_bounds__(kThreads) void k_velo_mix(const float* __restrict__
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
 
 // gates = [x', h] W^T + b in chunks i, g, f, o;  c = sig(f+1) c + sig(i) tanh(g);  h = sig(o) tanh(c)
-// Block = 32 hidden units x 8 slices of the 2H-long contraction, 8 tensors; the slices are added
-// in LDS in a fixed order.  The weights arrive with the four gates of a unit adjacent, wt[k][u][4],
+// Block = 16 hidden units x 16 slices of the 2H-long contraction, 8 tensors; the slices are added
+// in LDS in a fixed order.  (A block streams its units' weights with a fixed number of bytes in flight:
+// 16 units a block instead of 32 halves the bytes per block and doubles the blocks, 416 for 256 CUs.)  The weights arrive with the four gates of a unit adjacent, wt[k][u][4],
 // so a thread fetches its unit's four gate weights of one input with a single 16-byte load; the
 // inputs of the block's 8 tensors (32 B per k, the same for every unit) are staged in LDS once and
 // read back as broadcasts, which leaves the weight stream as the only vector-memory traffic of the
 // loop.  Blocks are numbered so that the blocks one XCD receives (block id modulo 8) share their
 // unit blocks: each XCD's L2 then holds its 1/8 of the 8 MB weight matrix instead of all of it.
-constexpr int kGateU = 32, kGateS = 8;
+constexpr int kGateU = 16, kGateS = 16;
 __global__ __launch_bounds__(kThreads) void k_velo_gates(const float* __restrict__ xT, int T, int Tpad, int H,
                                                          const float* __restrict__ wt /*(2H, H, 4)*/,
                                                          const float* __restrict__ b /*4H*/,
@@ -491,6 +492,8 @@ __global__ __launch_bounds__(kThreads) void k_velo_gates(const float* __restrict
   constexpr int kHalf = 1024;
   __shared__ float lds[kGateS * 4 * kGateBT * kGateU];
   static_assert(kHalf * kGateBT <= kGateS * 4 * kGateBT * kGateU, "x tile must fit the reduction buffer");
+  static_assert(8 * kGateS <= 128 && kHalf % (8 * kGateS) == 0,
+                "a batch of eight weight loads per slice must divide 2H for every H that is a multiple of 64");
   const int ul = threadIdx.x % kGateU, sl = threadIdx.x / kGateU;
   const int n_ub = H / kGateU;
   int ub, rb;
@@ -544,9 +547,9 @@ __global__ __launch_bounds__(kThreads) void k_velo_gates(const float* __restrict
 #pragma unroll
     for (int t = 0; t < kGateBT; ++t) red[sl][g * kGateBT + t][ul] = acc[g][t];
   __syncthreads();
-  // thread (ul, sl) finishes tensor t = sl of unit ul
+  // thread (ul, sl), sl < 8, finishes tensor t = sl of unit ul
   const int t = sl, r = r0 + t;
-  if (r < T) {
+  if (sl < kGateBT && r < T) {
     float gate[4];
 #pragma unroll
     for (int g = 0; g < 4; ++g) {

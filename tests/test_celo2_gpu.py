@@ -254,3 +254,33 @@ def test_state_dict_resume():
     assert set(oa.state[a[0]].keys()) == {"mom", "rms", "fac_r", "fac_c"}
     assert oa.state[a[0]]["mom"].shape == (3, 32, 24) and oa.state[a[0]]["fac_r"].shape == (3, 1, 24)
     assert set(oa.state[a[1]].keys()) == {"mom", "rms"}
+
+
+def test_runs_on_the_callers_stream():
+    """The library enqueues on torch's current stream (the reference launches on the legacy default
+    stream): stepping under a side stream gives bit-identical parameters, and work queued on that stream
+    before the step is ordered before it."""
+    from pylo_amd import ELO_CELO2_CUDA
+
+    shapes = [(70, 384), (48, 40), (40,)]
+    net = _net(2)
+    init, gen = _mk(shapes, 4)
+    grads = [[torch.randn(s, generator=gen) for s in shapes] for _ in range(3)]
+
+    def run(stream):
+        ps = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+        opt = ELO_CELO2_CUDA(ps, lr=1e-2, network=net, hf_key=None)
+        gs = [[g.cuda() for g in step] for step in grads]
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            for t in range(3):
+                for p, g in zip(ps, gs[t]):
+                    p.grad = g * 1.0          # produced on the same stream right before the step
+                opt.step()
+        stream.synchronize()
+        return [p.detach().clone() for p in ps]
+
+    a = run(torch.cuda.current_stream())
+    b = run(torch.cuda.Stream())
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)

@@ -276,6 +276,18 @@ __global__ __launch_bounds__(kV0aThreads) void k_v0a(const TDesc* __restrict__ d
   const float* pp = part + pick(d.part_off, which);
   const int e = threadIdx.x & 63, grp = threadIdx.x >> 6;
   const int i = it.a * kV0aEnt + e;
+  const int k = grp;  // after the sums: waves 0..2 take one decay each
+  // everything the second half needs from memory is requested before the partial sums are read, so that
+  // the block pays one memory round trip instead of two (kernels start with cold caches)
+  const bool is_r = (which == 0) == (d.vec0_is_r != 0);
+  float* fac = is_r ? a.fac_r : a.fac_c;
+  float fac_old = 0.0f;
+  if (k < 3 && i < len) fac_old = *(const gfloat*)(fac + (size_t)k * len + i);
+  double s2 = 1.0;
+  if (a.clip_norm > 0.0f && gl->flag == 0 && d.mode == kModeFac2D) {  // other modes sum the scaled gradient
+    const float sc = clip_scale(gl->gnorm, a.clip_norm);
+    s2 = (double)sc * (double)sc;
+  }
   {
     double s = 0.0;
     if (i < len) {
@@ -285,15 +297,7 @@ __global__ __launch_bounds__(kV0aThreads) void k_v0a(const TDesc* __restrict__ d
     lds[grp][e] = s;
   }
   __syncthreads();
-  const int k = grp;  // waves 0..2 take one decay each
   if (k >= 3) return;
-  double s2 = 1.0;
-  if (a.clip_norm > 0.0f && gl->flag == 0 && d.mode == kModeFac2D) {  // other modes sum the scaled gradient
-    const float sc = clip_scale(gl->gnorm, a.clip_norm);
-    s2 = (double)sc * (double)sc;
-  }
-  const bool is_r = (which == 0) == (d.vec0_is_r != 0);
-  float* fac = is_r ? a.fac_r : a.fac_c;
   double s_f = 0.0, s_ff = 0.0, s_rr = 0.0;
   if (i < len) {
     double S = 0.0;
@@ -301,7 +305,7 @@ __global__ __launch_bounds__(kV0aThreads) void k_v0a(const TDesc* __restrict__ d
     for (int q = 0; q < G; ++q) S += lds[q][e];
     const float q = (float)(s2 * S / (double)pick(d.sumlen, which)) + 1e-30f;
     const float beta = dec.beta_fac[k];
-    const float f = beta * fac[(size_t)k * len + i] + (1.0f - beta) * q;
+    const float f = beta * fac_old + (1.0f - beta) * q;
     fac[(size_t)k * len + i] = f;
     const float rq = rsq(f + 1e-8f);
     s_f = (double)f;
@@ -333,12 +337,13 @@ __device__ __forceinline__ size_t term_index(const TDesc& d, int which, int j, i
 // rcm: row_col_mean per decay; s0 / s1: normalisation scales of the vector's two broadcast channels.
 // (They arrive as plain arrays: indexing a BScale held in registers with `is_r ? k : 3 + k` makes the
 // compiler move the struct to LDS, 64 bytes a thread with bank conflicts on every access.)
+// fv: the entry's three accumulator values (fac[k * len + i]), loaded by the caller.
 __device__ __forceinline__ void vector_entry(const TDesc& d, bool is_r, const float* fac, int len, int i,
-                                             const float (&rcm3)[3], const float (&s0)[3], const float (&s1)[3],
-                                             float (&fct)[3], float (&x0)[3], float (&x1)[3]) {
+                                             const float (&fv)[3], const float (&rcm3)[3], const float (&s0)[3],
+                                             const float (&s1)[3], float (&fct)[3], float (&x0)[3], float (&x1)[3]) {
 #pragma unroll
   for (int k = 0; k < 3; ++k) {
-    const float f = fac[(size_t)k * len + i];
+    const float f = fv[k];
     float rcm = rcm3[k];
     if (is_r && d.mode == kModeFacND) {  // mean over the dc axis of this entry's slice of fac_r
       const int sz = d.rcm_size, st = d.rcm_stride;
@@ -419,6 +424,21 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
   const TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
+  // the entries' accumulator values are requested before the reduction below waits on its own loads:
+  // one memory round trip for the block instead of two (kernels start with cold caches)
+  constexpr int kPer = kV0bEnt / kThreads;
+  const int which = it.b;
+  const bool is_r = (which == 0) == (d.vec0_is_r != 0);
+  const int len = pick(d.len, which);
+  const float* fac = is_r ? a.fac_r : a.fac_c;
+  const int i_end = min(len, (it.a + 1) * kV0bEnt);
+  float fpre[kPer][3];
+#pragma unroll
+  for (int q = 0; q < kPer; ++q) {
+    const int i = it.a * kV0bEnt + q * kThreads + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) fpre[q][k] = i < i_end ? *(const gfloat*)(fac + (size_t)k * len + i) : 0.0f;
+  }
   {
     const int pair = threadIdx.x % (2 * kNV0), gI = threadIdx.x / (2 * kNV0);
     if (gI < G) {
@@ -442,7 +462,6 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
   const double* tc = tot + cI * kNV0;
   // means as sum * (1 / len): one double division per vector instead of nine
   const double inv_r = 1.0 / (double)d.len[rI], inv_c = 1.0 / (double)d.len[cI];
-  const int which = it.b;
   if (which == 0 && it.a == 0 && threadIdx.x == 0) {  // the tensor's scales, for k_terms
     BScale bs;
 #pragma unroll
@@ -466,12 +485,12 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
     s0[k] = rsq(norm_eps + (float)(own[k * 3 + 1] * inv_own));
     s1[k] = rsq(norm_eps + (float)(own[k * 3 + 2] * inv_own));
   }
-  const bool is_r = (which == 0) == (d.vec0_is_r != 0);
-  const int len = pick(d.len, which);
-  const float* fac = is_r ? a.fac_r : a.fac_c;
-  for (int i = it.a * kV0bEnt + threadIdx.x; i < min(len, (it.a + 1) * kV0bEnt); i += kThreads) {
+#pragma unroll
+  for (int q = 0; q < kPer; ++q) {
+    const int i = it.a * kV0bEnt + q * kThreads + threadIdx.x;
+    if (i >= i_end) break;
     float fct[3], x0[3], x1[3];
-    vector_entry(d, is_r, fac, len, i, rcm3, s0, s1, fct, x0, x1);
+    vector_entry(d, is_r, fac, len, i, fpre[q], rcm3, s0, s1, fct, x0, x1);
     if (d.mode == kModeFac2D) {  // [index][4]: one 16-byte store
       *(float4*)(fac_tab + fac_index(d, which, 0, i)) = make_float4(fct[0], fct[1], fct[2], 0.0f);
     } else {
@@ -508,8 +527,10 @@ __global__ __launch_bounds__(kThreads) void k_terms(const TDesc* __restrict__ de
   load_uniform<3>(bs->s + (is_r ? 0 : 3), s0);
   load_uniform<3>(bs->s + (is_r ? 6 : 9), s1);
   for (int i = it.a * kV0bEnt + threadIdx.x; i < min(len, (it.a + 1) * kV0bEnt); i += kThreads) {
-    float fct[3], x0[3], x1[3];
-    vector_entry(d, is_r, fac, len, i, rcm3, s0, s1, fct, x0, x1);
+    float fct[3], x0[3], x1[3], fv[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) fv[k] = *(const gfloat*)(fac + (size_t)k * len + i);
+    vector_entry(d, is_r, fac, len, i, fv, rcm3, s0, s1, fct, x0, x1);
     vector_terms<H>(d, which, is_r, i, x0, x1, w1, b1, term_tab);
   }
 }

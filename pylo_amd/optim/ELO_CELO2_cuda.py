@@ -236,6 +236,9 @@ class ELO_CELO2_CUDA(Optimizer):
         groups = self.param_groups
         if len(groups) != fast["n_groups"] or len(self.state) != fast["n_state"]:
             return None
+        for st, key, t in fast["alive"]:
+            if st.get(key) is not t:      # a state tensor was replaced: the cached pointers are stale
+                return None
         for group in groups:
             group["step"] = group.get("step", 0) + 1
         gidx, adam = fast["gidx"], fast["adam"]
@@ -313,7 +316,8 @@ class ELO_CELO2_CUDA(Optimizer):
         if not keep and all(p.grad is not None for _, p, _a in tensors):
             index = {id(g): i for i, g in enumerate(self.param_groups)}
             # the cached rows point into the state tensors: hold them, and notice a cleared state
-            alive = [t for _, p, _a in tensors for t in self.state[p].values() if torch.is_tensor(t)]
+            alive = [(self.state[p], k, t) for _, p, _a in tensors for k, t in self.state[p].items()
+                     if torch.is_tensor(t)]
             self._fast = dict(tensors=tensors, params=[p for _, p, _a in tensors], n_groups=len(self.param_groups),
                               n_state=len(self.state), alive=alive,
                               gidx=np.asarray([index[id(g)] for g, _p, _a in tensors], dtype=np.int64),

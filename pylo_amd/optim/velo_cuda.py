@@ -286,6 +286,14 @@ class VeLO_CUDA(Optimizer):
                     fast = self._fast = None
                     break
         if fast is not None:
+            for state, key, t in fast["alive"]:
+                if state.get(key) is not t:   # a state tensor was replaced: the cached pointers are stale
+                    fast = self._fast = None
+                    break
+            else:
+                if any(a is not p for a, (_, _, p) in zip(fast["params"], tensors)):
+                    fast = self._fast = None
+        if fast is not None:
             args = plan.args
             gidx = fast["gidx"]
             args["grad"] = [g.data_ptr() for g in grads]
@@ -328,8 +336,10 @@ class VeLO_CUDA(Optimizer):
                 args[k] = v
             args["group"] = grp
             if not keep:
-                alive = [t for _, _, p in tensors for t in self.state[p].values() if torch.is_tensor(t)]
+                alive = [(self.state[p], k, t) for _, _, p in tensors for k, t in self.state[p].items()
+                         if torch.is_tensor(t)]
                 self._fast = dict(key=self._plan_key, n_state=len(self.state), alive=alive,
+                                  params=[p for _, _, p in tensors],
                                   gidx=np.asarray(grp, dtype=np.int64))
 
         h, c = self.lstm_hidden_state

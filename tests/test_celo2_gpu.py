@@ -284,3 +284,36 @@ def test_runs_on_the_callers_stream():
     b = run(torch.cuda.Stream())
     for x, y in zip(a, b):
         assert torch.equal(x, y)
+
+
+def test_replaced_state_tensor_is_picked_up():
+    """The step caches its argument table between calls; a state tensor swapped for a copy (what a
+    user-side checkpoint restore or a dtype/device round trip does) must be the one updated from then
+    on, with the trajectory unchanged."""
+    from pylo_amd import ELO_CELO2_CUDA
+
+    shapes = [(40, 24), (24,), (24, 8)]
+    net = _net(3)
+    init, gen = _mk(shapes, 9)
+    grads = [[torch.randn(s, generator=gen).cuda() for s in shapes] for _ in range(6)]
+
+    def run(swap):
+        ps = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+        opt = ELO_CELO2_CUDA(ps, lr=1e-2, network=net, hf_key=None)
+        for t in range(6):
+            for p, g in zip(ps, grads[t]):
+                p.grad = g.clone()
+            opt.step()
+            if swap and t == 2:
+                for p in ps:
+                    for k, v in list(opt.state[p].items()):
+                        if torch.is_tensor(v):
+                            opt.state[p][k] = v.clone()
+                            v.fill_(float("nan"))      # the old storage must not be read again
+        return ps, opt
+
+    a, _ = run(False)
+    b, ob = run(True)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    assert all(bool(torch.isfinite(v).all()) for p in b for v in ob.state[p].values() if torch.is_tensor(v))

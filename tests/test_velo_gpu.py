@@ -146,3 +146,35 @@ def test_velo_state_dict_resume():
     assert st["mom"].shape == (3, 24, 16) and st["rms"].shape == (1, 24, 16)
     assert st["fac_vec_row"].shape == (3, 1, 16) and st["fac_vec_col"].shape == (3, 24, 1)
     assert oa.state[a[1]]["fac_vec_v"].shape == (3, 16)
+
+
+def test_velo_replaced_state_tensor_is_picked_up():
+    """A state tensor swapped for a copy between steps is the one the next step updates (the argument
+    table cached between calls must notice), with the trajectory unchanged."""
+    from pylo_amd import VeLO_CUDA
+    from pylo_amd.models import VeLOMLP, VeLORNN
+
+    torch.manual_seed(6)
+    rnn, mlp = VeLORNN(lstm_hidden_size=64, param_inits=32), VeLOMLP(param_inits=32)
+    shapes = [(24, 16), (16,), (8, 24)]
+    gen = torch.Generator().manual_seed(3)
+    init = [torch.randn(s, generator=gen) for s in shapes]
+    grads = [[torch.randn(s, generator=gen).cuda() for s in shapes] for _ in range(6)]
+
+    def run(swap):
+        ps = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+        opt = VeLO_CUDA(ps, lr=1e-2, num_steps=20, rnn=rnn, mlp=mlp)
+        for t in range(6):
+            for p, g in zip(ps, grads[t]):
+                p.grad = g.clone()
+            opt.step(torch.tensor(2.0 / (1 + t)).cuda())
+            if swap and t == 2:
+                for p in ps:
+                    for k, v in list(opt.state[p].items()):
+                        if torch.is_tensor(v):
+                            opt.state[p][k] = v.clone()
+                            v.fill_(float("nan"))
+        return ps
+
+    for x, y in zip(run(False), run(True)):
+        assert torch.equal(x, y)

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define PYLO_MI355_ABI_VERSION 3
+#define PYLO_MI355_ABI_VERSION 4
 #define PYLO_MAX_DIMS 8
 #define PYLO_MAX_GROUPS 8   /* parameter groups with their own step counter (VeLO) */
 
@@ -126,6 +126,37 @@ int pylo_mi355_plan_timing_end(PyloPlan* plan, float* ms_out, int capacity, int*
 
 /* Names of the launches of one step, in launch order (static strings). */
 const char* pylo_mi355_plan_launch_name(const PyloPlan* plan, int launch);
+
+/* ---- Steps that a HIP graph can replay.  No counterpart in the reference, whose step() waits for
+ * the device once per step or per tensor (ELO_CELO2_cuda.py:154-162, velo_cuda.py:747) and counts
+ * steps on the host (ELO_CELO2_cuda.py:224, AdafacLO_cuda.py:304-305). ------------------------- */
+
+/* The plan's own argument tables: pinned host memory, `n_tensors` records each, slot 0..3.  A step /
+   finish call whose `args` IS such a pointer does no host-side staging (no comparison with the
+   previous table, no events, no waits): it enqueues one small kernel that reads the table when it
+   RUNS.  Recorded into a HIP graph, every replay therefore takes the table's contents at that moment.
+   The caller must not write a table while a run that reads it may be in flight.  A slot that has been
+   handed out is no longer used for staging ordinary calls (which need at least one free slot). */
+#define PYLO_ARG_TABLES 4
+int pylo_mi355_plan_arg_table(PyloPlan* plan, int slot, PyloTensorArgs** table_out);
+
+/* Step counters kept on the device.  With `counters` set, every *_step call on the plan first runs a
+   small kernel that advances them and derives from them what the host otherwise supplies per step:
+     CELO2 kind    counters[t] += 1 for every tensor (a PYLO_F_ADAM_INDEP tensor: only when it has a
+                   gradient), then bc1 / bc2 of an AdamW tensor's record = 1 - beta1^counters[t] /
+                   1 - beta2^counters[t];
+     VeLO kind     frac of group g = tanh((counters[g] / num_steps - ts) * 10), then counters[g] += 1;
+                   PyloVeloStep.frac is ignored; `counters` holds PYLO_MAX_GROUPS entries;
+     AdafacLO kind bc1 of record t = counters[t], then counters[t] += 1 when tensor t has a gradient;
+                   the call's `step` is ignored.
+   `counters` is device memory owned by the caller (int32, one per tensor except for VeLO); NULL
+   switches the mechanism off. */
+typedef struct {
+  int32_t* counters;
+  double beta1, beta2; /* CELO2 kind */
+  double num_steps;    /* VeLO kind  */
+} PyloDeviceSteps;
+int pylo_mi355_plan_device_steps(PyloPlan* plan, const PyloDeviceSteps* steps);
 
 /*
  * ELO-CELO2 / CELO2 step (replaces celo2_cuda_kernel.celo2_kernel, pylo/csrc/celo2_kernel.cu:284-350,

@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes as C
 import os
-from typing import List, Sequence
+from typing import List, Optional, Sequence
 
 import numpy as np
 import torch
@@ -56,6 +56,11 @@ class VeloStep(C.Structure):
 _lib = None
 
 
+class DeviceSteps(C.Structure):
+    _fields_ = [("counters", C.c_void_p), ("beta1", C.c_double), ("beta2", C.c_double),
+                ("num_steps", C.c_double)]
+
+
 def load():
     """Loads the shared library once; raises if it has not been built."""
     global _lib
@@ -87,7 +92,9 @@ def load():
                                          C.POINTER(VeloStep), C.c_void_p]
     lib.pylo_mi355_adafac_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.c_void_p, C.c_float,
                                            C.c_void_p]
-    if lib.pylo_mi355_abi_version() != 3:
+    lib.pylo_mi355_plan_arg_table.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_void_p)]
+    lib.pylo_mi355_plan_device_steps.argtypes = [C.c_void_p, C.POINTER(DeviceSteps)]
+    if lib.pylo_mi355_abi_version() != 4:
         raise RuntimeError("libpylo_mi355.so: ABI version mismatch, rebuild it")
     _lib = lib
     return lib
@@ -167,20 +174,49 @@ class Plan:
         nl = self.num_launches
         return np.array(buf[:steps.value * nl], dtype=np.float64).reshape(steps.value, nl)
 
-    def celo2_step(self, decays: Decays, mlp: torch.Tensor, stream: int) -> None:
-        check(load().pylo_mi355_celo2_step(self._h, self.args.ctypes.data, C.byref(decays),
+    def pinned_table(self, slot: int) -> np.ndarray:
+        """The plan's own pinned argument table `slot` as a structured array.  A call given this
+        array reads it in place when it runs on the device, which is what a HIP graph needs: every
+        replay sees the table as it is then.  Do not write it while such a run may be in flight."""
+        tabs = self.__dict__.setdefault("_tables", {})
+        if slot not in tabs:
+            ptr = C.c_void_p()
+            check(load().pylo_mi355_plan_arg_table(self._h, slot, C.byref(ptr)), "plan_arg_table")
+            buf = (C.c_char * (ARGS_DTYPE.itemsize * self.n)).from_address(ptr.value)
+            tabs[slot] = np.frombuffer(buf, dtype=ARGS_DTYPE, count=self.n)
+        return tabs[slot]
+
+    def device_steps(self, counters: Optional[torch.Tensor], beta1: float = 0.0, beta2: float = 0.0,
+                     num_steps: float = 1.0) -> None:
+        """Keep the step counters in `counters` (int32, on the device; held by the plan) and let
+        the library derive bias corrections / time features from them; None switches that off."""
+        ds = DeviceSteps()
+        if counters is not None:
+            if counters.dtype != torch.int32 or not counters.is_cuda or not counters.is_contiguous():
+                raise TypeError("step counters must be a contiguous int32 tensor on the GPU")
+            ds.counters, ds.beta1, ds.beta2, ds.num_steps = counters.data_ptr(), beta1, beta2, num_steps
+        check(load().pylo_mi355_plan_device_steps(self._h, C.byref(ds)), "plan_device_steps")
+        self._counters = counters
+
+    def _table_ptr(self, args: Optional[np.ndarray]) -> int:
+        return (self.args if args is None else args).ctypes.data
+
+    def celo2_step(self, decays: Decays, mlp: torch.Tensor, stream: int, args: Optional[np.ndarray] = None) -> None:
+        check(load().pylo_mi355_celo2_step(self._h, self._table_ptr(args), C.byref(decays),
                                            mlp.data_ptr(), stream), "celo2_step")
 
     def celo2_finish(self, args: np.ndarray, stream: int) -> None:
         """Normalise + apply after Newton-Schulz; `args` is a table like `self.args` (own array)."""
         check(load().pylo_mi355_celo2_finish(self._h, args.ctypes.data, stream), "celo2_finish")
 
-    def velo_step(self, decays: Decays, nets: VeloNets, step: VeloStep, stream: int) -> None:
-        check(load().pylo_mi355_velo_step(self._h, self.args.ctypes.data, C.byref(decays), C.byref(nets),
+    def velo_step(self, decays: Decays, nets: VeloNets, step: VeloStep, stream: int,
+                  args: Optional[np.ndarray] = None) -> None:
+        check(load().pylo_mi355_velo_step(self._h, self._table_ptr(args), C.byref(decays), C.byref(nets),
                                           C.byref(step), stream), "velo_step")
 
-    def adafac_step(self, decays: Decays, net: torch.Tensor, step: float, stream: int) -> None:
-        check(load().pylo_mi355_adafac_step(self._h, self.args.ctypes.data, C.byref(decays), net.data_ptr(),
+    def adafac_step(self, decays: Decays, net: torch.Tensor, step: float, stream: int,
+                    args: Optional[np.ndarray] = None) -> None:
+        check(load().pylo_mi355_adafac_step(self._h, self._table_ptr(args), C.byref(decays), net.data_ptr(),
                                             float(step), stream), "adafac_step")
 
     def close(self):

@@ -22,6 +22,7 @@ constexpr int kGateBT = 8;     // tensors per k_velo_gates block
 
 struct VeloStep {              // by-value kernel argument: scalars of one step
   float frac[PYLO_MAX_GROUPS][9];
+  const float* frac_dev;       // the same table in device memory when the step counters live there, else null
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -345,7 +346,7 @@ __device__ __forceinline__ float lo_lstm_feature(const TDesc& d, const PyloTenso
   const double nu2 = (double)nu * (double)nu;
   float val;
   if (q < 9) {
-    val = st.frac[a.group][q];
+    val = st.frac_dev ? st.frac_dev[a.group * 9 + q] : st.frac[a.group][q];
   } else if (q < 18) {
     val = lossfeat[q - 9];
   } else if (q == 18) {

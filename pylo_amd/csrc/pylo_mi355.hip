@@ -72,7 +72,7 @@ struct Layout {
   bool global_norm = false;  // AdafacLO kind: every tensor has P0 items, the call may clip by global norm
   size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_sl_items, off_seg_items, off_segtot, off_el_items, off_ap_items, off_ga_items, off_fin_items, off_finpart, off_finscale, off_v0a_items, off_v0b_items, off_fac_list,
       off_part, off_gsq, off_flag, off_globals, off_fac, off_term, off_v0part, off_bscale, off_stats, off_wfold,
-      off_chan_ms, off_totals, off_xfeat, off_lossfeat, off_xT, off_mixbuf, off_pmax, off_canon, total;
+      off_chan_ms, off_totals, off_xfeat, off_lossfeat, off_xT, off_mixbuf, off_pmax, off_canon, off_frac, total;
 };
 
 int first_layer_width(int kind) { return kind == PYLO_KIND_CELO2 ? 8 : kind == PYLO_KIND_VELO ? 4 : 32; }
@@ -279,11 +279,12 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_mixbuf = take(kind == PYLO_KIND_VELO ? sizeof(float) * 2 * (size_t)velo_hidden * T : 0);
   L.off_pmax = take(kind == PYLO_KIND_VELO ? sizeof(float) * (size_t)velo_hidden * ((T + kMixRows - 1) / kMixRows) : 0);
   L.off_canon = take(kind == PYLO_KIND_VELO ? sizeof(float) * kVCanon * (size_t)T : 0);
+  L.off_frac = take(kind == PYLO_KIND_VELO ? sizeof(float) * 9 * PYLO_MAX_GROUPS : 0);
   L.total = off;
   return 0;
 }
 
-constexpr int kStageSlots = 4;
+constexpr int kStageSlots = PYLO_ARG_TABLES;
 constexpr int kVeloHiddenMax = 1024;  // workspace is sized for LSTM widths up to this
 
 }  // namespace
@@ -295,7 +296,9 @@ struct PyloPlan {
   PyloTensorArgs* stage[kStageSlots] = {nullptr, nullptr, nullptr, nullptr};
   hipEvent_t ev[kStageSlots] = {nullptr, nullptr, nullptr, nullptr};
   bool ev_used[kStageSlots] = {false, false, false, false};
+  bool handed[kStageSlots] = {false, false, false, false};  // given to the caller by plan_arg_table
   int slot = 0;
+  PyloDeviceSteps dsteps = {nullptr, 0.0, 0.0, 1.0};
   std::vector<PyloTensorArgs> last;
   bool have_last = false;
   bool mlp_on_matrix_pipe = true;  // env_matrix_pipe() when the plan was created
@@ -431,6 +434,27 @@ int pylo_mi355_plan_timing_end(PyloPlan* P, float* ms_out, int capacity, int* st
   return 0;
 }
 
+int pylo_mi355_plan_arg_table(PyloPlan* P, int slot, PyloTensorArgs** table_out) {
+  if (!P || !table_out || slot < 0 || slot >= kStageSlots) return fail("plan_arg_table: bad argument");
+  // a staged copy out of this slot may still be pending on the device
+  if (P->ev_used[slot]) HIP_TRY(hipEventSynchronize(P->ev[slot]));
+  P->handed[slot] = true;
+  *table_out = P->stage[slot];
+  return 0;
+}
+
+int pylo_mi355_plan_device_steps(PyloPlan* P, const PyloDeviceSteps* steps) {
+  if (!P) return fail("plan_device_steps: null plan");
+  if (!steps || !steps->counters) {
+    P->dsteps = PyloDeviceSteps{nullptr, 0.0, 0.0, 1.0};
+    return 0;
+  }
+  if (reinterpret_cast<uintptr_t>(steps->counters) % 4 != 0) return fail("plan_device_steps: misaligned counters");
+  if (P->kind == PYLO_KIND_VELO && !(steps->num_steps > 0.0)) return fail("plan_device_steps: num_steps must be positive");
+  P->dsteps = *steps;
+  return 0;
+}
+
 int pylo_mi355_plan_factored_dims(const PyloPlan* P, int tensor, int* dc, int* dr) {
   if (!P || tensor < 0 || tensor >= P->T || !dc || !dr) return fail("factored_dims: bad argument");
   *dc = P->L.dc[tensor];
@@ -453,22 +477,83 @@ __global__ __launch_bounds__(256) void k_copy_args(const uint4* __restrict__ src
 
 int upload_args(PyloPlan* P, const PyloTensorArgs* args, hipStream_t s) {
   const size_t bytes = sizeof(PyloTensorArgs) * P->T;
+  static_assert(sizeof(PyloTensorArgs) % 8 == 0, "argument records are copied in 16-byte pieces");
+  const int n16 = (int)((bytes + 15) / 16);
+  const dim3 grid(std::min(64, (n16 + 255) / 256));
+  for (int j = 0; j < kStageSlots; ++j) {
+    if (args != P->stage[j]) continue;
+    // one of the plan's own pinned tables: read in place when the kernel runs (a graph replay sees the
+    // table as it is then); nothing on the host side depends on earlier calls
+    void* src_dev = nullptr;
+    HIP_TRY(hipHostGetDevicePointer(&src_dev, P->stage[j], 0));
+    hipLaunchKernelGGL(k_copy_args, grid, dim3(256), 0, s, static_cast<const uint4*>(src_dev),
+                       reinterpret_cast<uint4*>(P->ws + P->L.off_dyn), n16);
+    P->have_last = false;
+    return 0;
+  }
   if (P->have_last && std::memcmp(P->last.data(), args, bytes) == 0) return 0;
-  const int i = P->slot;
-  P->slot = (P->slot + 1) % kStageSlots;
+  int i = -1;
+  for (int k = 0; k < kStageSlots && i < 0; ++k) {
+    const int c = (P->slot + k) % kStageSlots;
+    if (!P->handed[c]) i = c;
+  }
+  if (i < 0) return fail("step: every argument table of the plan has been handed out; call with one of them");
+  P->slot = (i + 1) % kStageSlots;
   if (P->ev_used[i]) HIP_TRY(hipEventSynchronize(P->ev[i]));
   std::memcpy(P->stage[i], args, bytes);
-  static_assert(sizeof(PyloTensorArgs) % 8 == 0, "argument records are copied in 16-byte pieces");
   void* src_dev = nullptr;
   HIP_TRY(hipHostGetDevicePointer(&src_dev, P->stage[i], 0));
-  const int n16 = (int)((bytes + 15) / 16);
-  hipLaunchKernelGGL(k_copy_args, dim3(std::min(64, (n16 + 255) / 256)), dim3(256), 0, s,
+  hipLaunchKernelGGL(k_copy_args, grid, dim3(256), 0, s,
                      static_cast<const uint4*>(src_dev), reinterpret_cast<uint4*>(P->ws + P->L.off_dyn), n16);
   HIP_TRY(hipEventRecord(P->ev[i], s));
   P->ev_used[i] = true;
   P->last.assign(args, args + P->T);
   P->have_last = true;
   return 0;
+}
+
+// Step counters kept on the device: advances them and writes what the host otherwise supplies per
+// step into the device copy of the argument table (bias corrections, AdafacLO's counter) or into
+// the VeLO time-feature buffer.  One thread per tensor (VeLO: per group).
+__global__ __launch_bounds__(256) void k_advance_steps(int kind, int T, const TDesc* __restrict__ descs,
+                                                       PyloTensorArgs* __restrict__ dyn, PyloDeviceSteps ds,
+                                                       float* __restrict__ frac_out) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (kind == PYLO_KIND_VELO) {
+    if (t >= PYLO_MAX_GROUPS) return;
+    const float ts[9] = {0.03f, 0.1f, 0.2f, 0.4f, 0.6f, 0.8f, 0.9f, 1.0f, 1.1f};
+    const int c = ds.counters[t];
+    const float x = (float)((double)c / ds.num_steps);
+#pragma unroll
+    for (int q = 0; q < 9; ++q) frac_out[t * 9 + q] = tanhf((x - ts[q]) * 10.0f);
+    ds.counters[t] = c + 1;
+    return;
+  }
+  if (t >= T) return;
+  const bool has_grad = dyn[t].grad != nullptr;
+  if (kind == PYLO_KIND_ADAFAC) {
+    if (!has_grad) return;
+    const int c = ds.counters[t];
+    dyn[t].bc1 = (float)c;
+    ds.counters[t] = c + 1;
+    return;
+  }
+  // CELO2 kind: a per-parameter counter (independent AdamW moments) sits a step out with its tensor,
+  // the others count the calls like the reference's per-group counter
+  if (descs[t].adam_indep && !has_grad) return;
+  const int c = ds.counters[t] + 1;
+  ds.counters[t] = c;
+  if (descs[t].mode != kModeFlat) return;
+  dyn[t].bc1 = (float)(1.0 - pow(ds.beta1, (double)c));
+  dyn[t].bc2 = (float)(1.0 - pow(ds.beta2, (double)c));
+}
+
+void advance_steps(PyloPlan* P, hipStream_t s) {
+  if (!P->dsteps.counters) return;
+  const int n = P->kind == PYLO_KIND_VELO ? PYLO_MAX_GROUPS : P->T;
+  hipLaunchKernelGGL(k_advance_steps, dim3((n + 255) / 256), dim3(256), 0, s, P->kind, P->T,
+                     P->at<TDesc>(P->L.off_descs), P->at<PyloTensorArgs>(P->L.off_dyn), P->dsteps,
+                     P->kind == PYLO_KIND_VELO ? P->at<float>(P->L.off_frac) : nullptr);
 }
 
 int check_args(const PyloPlan* P, const PyloTensorArgs* args, bool need_all_grads) {
@@ -535,6 +620,7 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   if (int rc = check_args(P, args, false)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (int rc = upload_args(P, args, s)) return rc;
+  advance_steps(P, s);
   const Layout& L = P->L;
   const TDesc* descs = P->at<TDesc>(L.off_descs);
   const PyloTensorArgs* dyn = P->at<PyloTensorArgs>(L.off_dyn);
@@ -652,6 +738,7 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
   if (int rc = check_args(P, args, true)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (int rc = upload_args(P, args, s)) return rc;
+  advance_steps(P, s);
   const Layout& L = P->L;
   const TDesc* descs = P->at<TDesc>(L.off_descs);
   const PyloTensorArgs* dyn = P->at<PyloTensorArgs>(L.off_dyn);
@@ -681,6 +768,7 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
   const PyloDecays dec = *decays;
   VeloStep vs;
   std::memcpy(vs.frac, step->frac, sizeof(vs.frac));
+  vs.frac_dev = P->dsteps.counters ? P->at<float>(L.off_frac) : nullptr;
   Marks mark(P, s);
 
   HIP_TRY(mark());
@@ -740,6 +828,7 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   if (int rc = check_args(P, args, false)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (int rc = upload_args(P, args, s)) return rc;
+  advance_steps(P, s);
   const Layout& L = P->L;
   const TDesc* descs = P->at<TDesc>(L.off_descs);
   const PyloTensorArgs* dyn = P->at<PyloTensorArgs>(L.off_dyn);
@@ -787,7 +876,7 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   if (n_v0a > 0)
     hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kV0aThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_adafac_bias, dim3(T), dim3(64), 0, s, net, step, dyn, bias_eff);
+  hipLaunchKernelGGL(k_adafac_bias, dim3(T), dim3(64), 0, s, net, P->dsteps.counters ? -1.0f : step, dyn, bias_eff);
   HIP_TRY(mark());
   if (n_v0b > 0)
     hipLaunchKernelGGL(k_v0b<kAH>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-5f,

@@ -56,6 +56,7 @@ class CELO2_CUDA(ELO_CELO2_CUDA):
         hf_key: Optional[str] = "DiamondXL/celo2",
         checkpoint_path: Optional[str] = None,
         network: Optional[CELO2MLP] = None,
+        capturable: bool = False,
     ):
         super().__init__(
             params, lr=lr, weight_decay=weight_decay, clip_grad=clip_grad, clip_norm=clip_norm,
@@ -65,7 +66,8 @@ class CELO2_CUDA(ELO_CELO2_CUDA):
             initial_momentum_decays=initial_momentum_decays, initial_rms_decays=initial_rms_decays,
             initial_adafactor_decays=initial_adafactor_decays, exp_mult=exp_mult, rmsmult=rmsmult,
             param_scale_mult=param_scale_mult, ns_coeffs=ns_coeffs, ns_iters=ns_iters, ns_eps=ns_eps,
-            grad_clip_val=grad_clip_val, hf_key=hf_key, checkpoint_path=checkpoint_path, network=network)
+            grad_clip_val=grad_clip_val, hf_key=hf_key, checkpoint_path=checkpoint_path, network=network,
+            capturable=capturable)
         self.adam_beta1, self.adam_beta2 = (float(b) for b in adam_betas)
         self.adam_eps = adam_eps
         self._decays = _lib.make_decays(self.beta_m.tolist(), float(self.beta_rms[-1]), self.beta_fac.tolist(),
@@ -81,10 +83,23 @@ class CELO2_CUDA(ELO_CELO2_CUDA):
     # pylo/optim/CELO2_cuda.py:241-251: the counter is per parameter and advances only on steps in
     # which the parameter has a gradient
     def _adam_row(self, group, state):
-        state["adam_step"] += 1
+        if not self.capturable:
+            state["adam_step"] += 1
         t = state["adam_step"]
         return (state["exp_avg"].data_ptr(), state["exp_avg_sq"].data_ptr(),
                 1.0 - self.adam_beta1 ** t, 1.0 - self.adam_beta2 ** t)
+
+    # device-side counters (capturable=True): one per AdamW parameter
+    def _step_values(self, tensors):
+        return [self.state[p].get("adam_step", 0) if a else 0 for _g, p, a in tensors]
+
+    def _step_betas(self):
+        return self.adam_beta1, self.adam_beta2
+
+    def _store_step_values(self, tensors, values):
+        for (_g, p, a), v in zip(tensors, values):
+            if a and "adam_step" in self.state[p]:
+                self.state[p]["adam_step"] = v
 
     def _adam_corrections_fast(self, fast, per_group):
         steps = fast.get("adam_states")

@@ -90,9 +90,15 @@ class ELO_CELO2_CUDA(Optimizer):
         hf_key: Optional[str] = "DiamondXL/elo-celo2",
         checkpoint_path: Optional[str] = None,
         network: Optional[CELO2MLP] = None,
+        capturable: bool = False,
     ):
         if not torch.cuda.is_available():
             raise RuntimeError("ELO_CELO2_CUDA requires a GPU (torch.cuda.is_available() is False).")
+        # capturable: step counters live on the device and ``step()`` can be recorded into a HIP graph
+        # (torch.cuda.graph) and replayed; ``group["step"]`` is then refreshed by ``state_dict()`` /
+        # ``sync_step_counters()`` only.  The reference has no such mode.
+        self.capturable = bool(capturable)
+        self._dev_steps = None
         _lib.load()
         defaults = dict(
             lr=lr, weight_decay=weight_decay, adam_lr_mult=adam_lr_mult,
@@ -181,6 +187,50 @@ class ELO_CELO2_CUDA(Optimizer):
                 self._raw[i] = buf[j]
             self._raw_groups.append((buf, idx))
         self._fin_args = np.zeros(len(tensors), dtype=_lib.ARGS_DTYPE)
+        if self.capturable:
+            self._reset_device_steps(tensors)
+
+    # ------------------------------------------------------------------ device-side step counters
+    def _step_values(self, tensors):
+        return [g.get("step", 0) for g, _p, _a in tensors]
+
+    def _step_betas(self):
+        return self._adam_b1, self._adam_b2
+
+    def _store_step_values(self, tensors, values):
+        for (g, _p, _a), v in zip(tensors, values):
+            g["step"] = v
+
+    def _reset_device_steps(self, tensors):
+        values = torch.tensor(self._step_values(tensors), dtype=torch.int32)
+        if self._dev_steps is None or self._dev_steps.numel() != len(tensors):
+            self._dev_steps = torch.zeros(len(tensors), dtype=torch.int32, device=self.device)
+        self._dev_steps.copy_(values)       # in place: a recorded graph keeps pointing at this tensor
+        beta1, beta2 = self._step_betas()
+        self._plan.device_steps(self._dev_steps, beta1, beta2)
+        self._plan.pinned_table(0), self._plan.pinned_table(1)   # handed out now, not while a capture is open
+
+    def sync_step_counters(self):
+        """capturable mode: read the device counters back into ``group["step"]`` (waits for the GPU)."""
+        if self.capturable and self._dev_steps is not None and self._plan is not None:
+            self._store_step_values(self._tensors(), self._dev_steps.tolist())
+
+    def state_dict(self):
+        self.sync_step_counters()
+        return super().state_dict()
+
+    def _capturing(self):
+        return self.capturable and torch.cuda.is_current_stream_capturing()
+
+    def _launch_step(self):
+        plan = self._plan
+        table = None
+        if self._capturing():
+            # the recorded call reads the plan's pinned table in place on every replay
+            table = plan.pinned_table(0)
+            table[:] = plan.args
+        with torch.cuda.device(self.device):
+            plan.celo2_step(self._decays, self._mlp, torch.cuda.current_stream(self.device).cuda_stream, args=table)
 
     def _init_state(self, state, p, adam):
         shape = tuple(p.shape)
@@ -209,7 +259,10 @@ class ELO_CELO2_CUDA(Optimizer):
     # the per-group scalars are refreshed, which keeps the host ahead of a ~1.7 ms GPU step.
     def load_state_dict(self, state_dict):
         self._fast = None
-        return super().load_state_dict(state_dict)
+        out = super().load_state_dict(state_dict)
+        if self.capturable and self._plan is not None:
+            self._reset_device_steps(self._tensors())
+        return out
 
     def add_param_group(self, param_group):
         self._fast = None
@@ -217,7 +270,7 @@ class ELO_CELO2_CUDA(Optimizer):
 
     # AdamW branch: which two moment buffers a tensor uses and its bias corrections this step
     def _adam_row(self, group, state):
-        t = group["step"]
+        t = group.get("step", 0)
         return (state["mom"].data_ptr(), state["rms"].data_ptr(), 1.0 - self._adam_b1 ** t,
                 1.0 - self._adam_b2 ** t)
 
@@ -239,8 +292,9 @@ class ELO_CELO2_CUDA(Optimizer):
         for st, key, t in fast["alive"]:
             if st.get(key) is not t:      # a state tensor was replaced: the cached pointers are stale
                 return None
-        for group in groups:
-            group["step"] = group.get("step", 0) + 1
+        if not self.capturable:
+            for group in groups:
+                group["step"] = group.get("step", 0) + 1
         gidx, adam = fast["gidx"], fast["adam"]
 
         def per_group(fn):
@@ -254,9 +308,9 @@ class ELO_CELO2_CUDA(Optimizer):
         args["exp_mult"] = per_group(lambda g: g["exp_mult"])
         args["lr"] = np.where(adam, per_group(lambda g: g["adam_lr_mult"] * g["lr"]), 0.0)
         args["weight_decay"] = np.where(adam, per_group(lambda g: g["adam_weight_decay"]), 0.0)
-        args["bc1"], args["bc2"] = self._adam_corrections_fast(fast, per_group)
-        with torch.cuda.device(self.device):
-            self._plan.celo2_step(self._decays, self._mlp, torch.cuda.current_stream(self.device).cuda_stream)
+        if not self.capturable:     # else the library derives them from its device counters
+            args["bc1"], args["bc2"] = self._adam_corrections_fast(fast, per_group)
+        self._launch_step()
         return fast["tensors"]
 
     @torch.no_grad()
@@ -271,8 +325,9 @@ class ELO_CELO2_CUDA(Optimizer):
         tensors = self._tensors()
         self._ensure_plan(tensors)
         plan = self._plan
-        for group in self.param_groups:
-            group["step"] = group.get("step", 0) + 1
+        if not self.capturable:
+            for group in self.param_groups:
+                group["step"] = group.get("step", 0) + 1
         n = len(tensors)
         cols = {k: [0] * n for k in ("grad", "param", "mom", "rms", "fac_r", "fac_c", "fac_v", "step_out")}
         fl = {k: [0.0] * n for k in ("lr", "weight_decay", "clip_norm", "clip_val", "exp_mult", "bc1", "bc2")}
@@ -311,8 +366,7 @@ class ELO_CELO2_CUDA(Optimizer):
             args[k] = v
         for k, v in fl.items():
             args[k] = v
-        with torch.cuda.device(self.device):
-            plan.celo2_step(self._decays, self._mlp, torch.cuda.current_stream(self.device).cuda_stream)
+        self._launch_step()
         if not keep and all(p.grad is not None for _, p, _a in tensors):
             index = {id(g): i for i, g in enumerate(self.param_groups)}
             # the cached rows point into the state tensors: hold them, and notice a cleared state
@@ -376,6 +430,10 @@ class ELO_CELO2_CUDA(Optimizer):
                 fin["step_mult"][i] = group["rmsmult"]
             any_fin = True
         if any_fin:
+            if self._capturing():
+                table = self._plan.pinned_table(1)
+                table[:] = fin
+                fin = table
             with torch.cuda.device(self.device):
                 self._plan.celo2_finish(fin, torch.cuda.current_stream(self.device).cuda_stream)
         del keep

@@ -37,6 +37,11 @@ def _decays(initial, offsets, device):
 
 class AdafacLO_CUDA(Optimizer):
     _PLAN_FLAGS = 0      # PyloTensorShape.flags of every tensor
+    # capturable=True: the per-parameter step counters live on the device and ``step()`` can be recorded
+    # into a HIP graph (torch.cuda.graph) and replayed; ``state[p]["step"]`` is then refreshed by
+    # ``state_dict()`` / ``sync_step_counters()`` only.  The reference has no such mode.
+    capturable = False
+    _dev_steps = None
 
     def __init__(
         self,
@@ -65,9 +70,11 @@ class AdafacLO_CUDA(Optimizer):
         foreach: Optional[bool] = False,
         hf_key: Optional[str] = "btherien/mulo",
         network: Optional[MetaMLP] = None,
+        capturable: bool = False,
     ):
         if not torch.cuda.is_available():
             raise RuntimeError("AdafacLO_CUDA requires a GPU (torch.cuda.is_available() is False).")
+        self.capturable = bool(capturable)
         _lib.load()
         if isinstance(momentum_dtype, str):
             momentum_dtype = {"float16": torch.float16, "bfloat16": torch.bfloat16,
@@ -133,6 +140,36 @@ class AdafacLO_CUDA(Optimizer):
         self._plan = _lib.Plan(_lib.KIND_ADAFAC, [tuple(p.shape) for _, p in tensors],
                                [self._PLAN_FLAGS] * len(tensors), self.device)
         self._plan_key = key
+        if self.capturable:
+            self._reset_device_steps(tensors)
+
+    # ------------------------------------------------------------------ device-side step counters
+    def _reset_device_steps(self, tensors):
+        values = [int(self.state[p]["step"]) if "step" in self.state[p] else 0 for _, p in tensors]
+        if self._dev_steps is None or self._dev_steps.numel() != len(tensors):
+            self._dev_steps = torch.zeros(len(tensors), dtype=torch.int32, device=self.device)
+        self._dev_steps.copy_(torch.tensor(values, dtype=torch.int32))   # in place: graphs keep the pointer
+        self._plan.device_steps(self._dev_steps)
+        self._plan.pinned_table(0)        # handed out now, not while a capture is open
+
+    def sync_step_counters(self):
+        """capturable mode: read the device counters back into ``state[p]["step"]`` (waits for the GPU)."""
+        if self.capturable and self._dev_steps is not None and self._plan is not None:
+            values = self._dev_steps.tolist()
+            tensors = [(g, p) for g in self.param_groups for p in g["params"]]
+            for (_, p), v in zip(tensors, values):
+                if "step" in self.state[p]:
+                    self.state[p]["step"] = torch.tensor(float(v), dtype=torch.float64)
+
+    def state_dict(self):
+        self.sync_step_counters()
+        return super().state_dict()
+
+    def load_state_dict(self, state_dict):
+        out = super().load_state_dict(state_dict)
+        if self.capturable and self._plan is not None:
+            self._reset_device_steps([(g, p) for g in self.param_groups for p in g["params"]])
+        return out
 
     def _pre_clip(self, group, p):
         """Per-parameter norm clipping of the gradient, in place (AdafacLO_naive.py:200-201)."""
@@ -170,10 +207,11 @@ class AdafacLO_CUDA(Optimizer):
             state = self.state[p]
             if len(state) == 0:
                 self._init_state(state, p)
-            state["step"] += 1
+            if not self.capturable:     # else counted on the device
+                state["step"] += 1
             # the time features take each parameter's own counter (pylo/optim/AdafacLO_cuda.py:304-305,400):
             # one that sat steps out lags behind the others
-            s0 = float(state["step"]) - 1.0
+            s0 = float(state["step"]) - 1.0 if not self.capturable else 0.0
             fl["bc1"][i] = s0
             if step_fed is None:
                 step_fed = s0
@@ -195,7 +233,13 @@ class AdafacLO_CUDA(Optimizer):
             args[k] = v
         for k, v in fl.items():
             args[k] = v
+        table = None
+        if self.capturable and torch.cuda.is_current_stream_capturing():
+            # the recorded call reads the plan's pinned table in place on every replay
+            table = plan.pinned_table(0)
+            table[:] = args
         with torch.cuda.device(self.device):
-            plan.adafac_step(self._decays, self._net, step_fed, torch.cuda.current_stream(self.device).cuda_stream)
+            plan.adafac_step(self._decays, self._net, step_fed, torch.cuda.current_stream(self.device).cuda_stream,
+                             args=table)
         del keep
         return loss

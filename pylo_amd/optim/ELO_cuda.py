@@ -48,9 +48,11 @@ class ELO_CUDA(AdafacLO_CUDA):
         hf_key: Optional[str] = "DiamondXL/elo",
         checkpoint_path: Optional[str] = None,
         network: Optional[MetaMLP] = None,
+        capturable: bool = False,
     ):
         if not torch.cuda.is_available():
             raise RuntimeError("ELO_CUDA requires a GPU (torch.cuda.is_available() is False).")
+        self.capturable = bool(capturable)
         _lib.load()
         defaults = dict(lr=lr, exp_mult=exp_mult, weight_decay=weight_decay, clip_grad=clip_grad,
                         clip_norm=clip_norm)

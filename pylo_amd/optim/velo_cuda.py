@@ -80,7 +80,13 @@ class VeLO_CUDA(Optimizer):
         legacy=False,
         rnn: VeLORNN = None,
         mlp: VeLOMLP = None,
+        capturable: bool = False,
     ):
+        # capturable: the per-group step counters live on the device and ``step(loss)`` can be recorded
+        # into a HIP graph (torch.cuda.graph) and replayed; ``group["step"]`` is then refreshed by
+        # ``state_dict()`` / ``sync_step_counters()`` only.  The reference has no such mode.
+        self.capturable = bool(capturable)
+        self._dev_steps = None
         if legacy:
             raise NotImplementedError("legacy=True (the pure-PyTorch parameter loop) is not provided")
         if not torch.cuda.is_available():
@@ -172,7 +178,26 @@ class VeLO_CUDA(Optimizer):
             self.lstm_init_state[1].detach().repeat(layer_idx, 1).to(self.device).contiguous(),
         )
 
+    # ------------------------------------------------------------------ device-side step counters
+    def _reset_device_steps(self):
+        values = [0] * _lib.MAX_GROUPS
+        for gi, group in enumerate(self.param_groups):
+            values[gi] = int(group["step"])
+        if self._dev_steps is None:
+            self._dev_steps = torch.zeros(_lib.MAX_GROUPS, dtype=torch.int32, device=self.device)
+        self._dev_steps.copy_(torch.tensor(values, dtype=torch.int32))   # in place: graphs keep the pointer
+        self._plan.device_steps(self._dev_steps, num_steps=float(self.num_steps))
+        self._plan.pinned_table(0)        # handed out now, not while a capture is open
+
+    def sync_step_counters(self):
+        """capturable mode: read the device counters back into ``group["step"]`` (waits for the GPU)."""
+        if self.capturable and self._dev_steps is not None and self._plan is not None:
+            values = self._dev_steps.tolist()
+            for gi, group in enumerate(self.param_groups):
+                group["step"] = values[gi]
+
     def state_dict(self):
+        self.sync_step_counters()
         sd = super().state_dict()
         sd["loss_buffer"] = self.loss_buffer
         sd["lstm_hidden_state"] = self.lstm_hidden_state
@@ -188,6 +213,8 @@ class VeLO_CUDA(Optimizer):
         self.loss_buffer = {k: (v.to(self.device) if torch.is_tensor(v) else v) for k, v in loss_buffer.items()}
         self.lstm_hidden_state = tuple(t.to(self.device).contiguous() for t in lstm_hidden_state)
         self.num_steps = num_steps
+        if self.capturable and self._plan is not None:
+            self._reset_device_steps()
 
     # ------------------------------------------------------------------ networks
     def _pack_networks(self):
@@ -249,6 +276,8 @@ class VeLO_CUDA(Optimizer):
         self._plan = _lib.Plan(_lib.KIND_VELO, [tuple(p.shape) for _, _, p in tensors], [0] * len(tensors),
                                self.device)
         self._plan_key = key
+        if self.capturable:
+            self._reset_device_steps()
 
     @torch.no_grad()
     def step(self, loss):
@@ -267,8 +296,9 @@ class VeLO_CUDA(Optimizer):
             frac = fractional_tanh_embed(group["step"] / self.num_steps).tolist()
             for q in range(9):
                 st.frac[gi][q] = frac[q]
-        for group in self.param_groups:
-            group["step"] += 1
+        if not self.capturable:     # else counted on the device, which also forms the time features
+            for group in self.param_groups:
+                group["step"] += 1
 
         fast = getattr(self, "_fast", None)
         if fast is not None and (fast["key"] is not self._plan_key or len(self.state) != fast["n_state"]):
@@ -349,9 +379,14 @@ class VeLO_CUDA(Optimizer):
         st.loss_decays, st.loss_iteration = lb["decays"].data_ptr(), lb["iteration"].data_ptr()
         st.loss = loss_dev.data_ptr()
         st.controls_out = st.lr_mult_out = None
+        table = None
+        if self.capturable and torch.cuda.is_current_stream_capturing():
+            # the recorded call reads the plan's pinned table in place on every replay
+            table = plan.pinned_table(0)
+            table[:] = plan.args
         with torch.cuda.device(self.device):
             plan.velo_step(self._decays_struct(), self._nets, st,
-                           torch.cuda.current_stream(self.device).cuda_stream)
+                           torch.cuda.current_stream(self.device).cuda_stream, args=table)
         del keep, loss_dev
         return
 

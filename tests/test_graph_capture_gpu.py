@@ -134,3 +134,51 @@ def test_capturable_checkpoint_resumes_the_counters():
     run(ob, b, range(3, 6))
     _close(a, c, "device counters vs host counters")
     _close(b, c, "resumed")
+
+
+def test_velo_step_replays_from_a_graph():
+    """The time features (tanh embedding of step / num_steps), the loss EMAs and the LSTM state all
+    advance on the device; the loss is read from a static device scalar."""
+    from pylo_amd import VeLO_CUDA
+    from pylo_amd.models import VeLOMLP, VeLORNN
+
+    torch.manual_seed(8)
+    rnn, mlp = VeLORNN(lstm_hidden_size=64, param_inits=32), VeLOMLP(param_inits=32)
+    shapes = [(40, 24), (24,), (8, 3, 5, 5), (24, 56)]
+    loss = torch.zeros((), device="cuda")
+    losses = iter([2.0, 1.7, 1.5, 1.45, 1.2, 1.1])
+
+    def make(params, capturable):
+        return VeLO_CUDA(params, lr=1e-2, num_steps=20, weight_decay=0.01, rnn=rnn, mlp=mlp, capturable=capturable)
+
+    def step(opt):
+        # the reference optimizer steps first in every round and draws the loss; the capturable one reuses it
+        if not opt.capturable:
+            loss.fill_(next(losses))
+        opt.step(loss)
+
+    ref, cap, n = _graph_vs_eager(make, step, shapes)
+    assert cap.state_dict()["param_groups"][0]["step"] == n == ref.param_groups[0]["step"]
+    for a, b in zip(cap.lstm_hidden_state, ref.lstm_hidden_state):
+        assert max_err(a.cpu(), b.cpu(), REL, ABS) <= 1.0
+
+
+@pytest.mark.parametrize("which", ["adafac", "elo"])
+def test_adafac_family_step_replays_from_a_graph(which):
+    from pylo_amd import AdafacLO_CUDA, ELO_CUDA
+    from pylo_amd.models import MetaMLP
+
+    torch.manual_seed(9)
+    net = MetaMLP(39, 32, 1)
+    shapes = [(48, 40), (40,), (6, 4, 3, 3), (40, 72)]
+
+    def make(params, capturable):
+        if which == "adafac":
+            return AdafacLO_CUDA(params, lr=0.5, weight_decay=0.01, network=net, hf_key=None, capturable=capturable)
+        return ELO_CUDA(params, lr=1e-2, weight_decay=0.01, clip_grad=True, clip_norm=0.5, network=net, hf_key=None,
+                        capturable=capturable)
+
+    ref, cap, n = _graph_vs_eager(make, lambda o: o.step(), shapes)
+    cap.sync_step_counters()
+    p0 = cap.param_groups[0]["params"][0]
+    assert float(cap.state[p0]["step"]) == n == float(ref.state[ref.param_groups[0]["params"][0]]["step"])

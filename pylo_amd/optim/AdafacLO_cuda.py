@@ -161,6 +161,17 @@ class AdafacLO_CUDA(Optimizer):
                 if "step" in self.state[p]:
                     self.state[p]["step"] = torch.tensor(float(v), dtype=torch.float64)
 
+    def refresh_graph_tables(self):
+        """capturable mode: copy the groups' learning rates and weight decays into the pinned table
+        that a recorded ``step()`` reads, e.g. after a scheduler step.  Call it while no replay is in
+        flight."""
+        if not self.capturable or self._plan is None:
+            return
+        table = self._plan.pinned_table(0)
+        for i, (group, _p) in enumerate((g, p) for g in self.param_groups for p in g["params"]):
+            for k, v in self._scalars(group).items():
+                table[k][i] = v
+
     def state_dict(self):
         self.sync_step_counters()
         return super().state_dict()

@@ -219,6 +219,22 @@ class ELO_CELO2_CUDA(Optimizer):
         self.sync_step_counters()
         return super().state_dict()
 
+    def refresh_graph_tables(self):
+        """capturable mode: copy the groups' learning rates and weight decays into the pinned tables
+        that a recorded ``step()`` reads, e.g. after a scheduler step.  Call it while no replay is in
+        flight.  Tensors that the recorded step finishes with torch operations (more than two dims)
+        keep the values they were recorded with."""
+        if not self.capturable or self._plan is None:
+            return
+        step_tab, fin_tab = self._plan.pinned_table(0), self._plan.pinned_table(1)
+        for i, (group, _p, adam) in enumerate(self._tensors()):
+            if adam:
+                step_tab["lr"][i] = group["adam_lr_mult"] * group["lr"]
+                step_tab["weight_decay"][i] = group["adam_weight_decay"]
+            elif fin_tab["grad"][i]:
+                fin_tab["lr"][i], fin_tab["weight_decay"][i] = group["lr"], group["weight_decay"]
+                fin_tab["step_mult"][i] = group["rmsmult"]
+
     def _capturing(self):
         return self.capturable and torch.cuda.is_current_stream_capturing()
 

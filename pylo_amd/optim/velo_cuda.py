@@ -196,6 +196,17 @@ class VeLO_CUDA(Optimizer):
             for gi, group in enumerate(self.param_groups):
                 group["step"] = values[gi]
 
+    def refresh_graph_tables(self):
+        """capturable mode: copy the groups' lr / weight_decay / exp_mult / step_mult into the pinned
+        table that a recorded ``step()`` reads, e.g. after a scheduler step.  Call it while no replay
+        is in flight."""
+        if not self.capturable or self._plan is None:
+            return
+        table = self._plan.pinned_table(0)
+        for i, (_gi, group, _p) in enumerate(self._tensors()):
+            for k in ("lr", "weight_decay", "exp_mult", "step_mult"):
+                table[k][i] = group[k]
+
     def state_dict(self):
         self.sync_step_counters()
         sd = super().state_dict()

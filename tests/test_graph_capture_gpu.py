@@ -182,3 +182,54 @@ def test_adafac_family_step_replays_from_a_graph(which):
     cap.sync_step_counters()
     p0 = cap.param_groups[0]["params"][0]
     assert float(cap.state[p0]["step"]) == n == float(ref.state[ref.param_groups[0]["params"][0]]["step"])
+
+
+@pytest.mark.parametrize("which", ["elo_celo2", "velo", "adafac"])
+def test_learning_rate_change_between_replays(which):
+    """A scheduler step between replays reaches the recorded step through the pinned tables."""
+    from pylo_amd import AdafacLO_CUDA, ELO_CELO2_CUDA, VeLO_CUDA
+    from pylo_amd.models import MetaMLP, VeLOMLP, VeLORNN
+
+    torch.manual_seed(10)
+    shapes = [(40, 24), (24,), (24, 56)]
+    loss = torch.tensor(1.3, device="cuda")
+    if which == "elo_celo2":
+        net = _celo2_net(6)
+        make = lambda ps, cap: ELO_CELO2_CUDA(ps, lr=1e-2, network=net, hf_key=None, capturable=cap)
+        step = lambda o: o.step()
+    elif which == "velo":
+        rnn, mlp = VeLORNN(lstm_hidden_size=64, param_inits=32), VeLOMLP(param_inits=32)
+        make = lambda ps, cap: VeLO_CUDA(ps, lr=1e-2, num_steps=20, rnn=rnn, mlp=mlp, capturable=cap)
+        step = lambda o: o.step(loss)
+    else:
+        net = MetaMLP(39, 32, 1)
+        make = lambda ps, cap: AdafacLO_CUDA(ps, lr=0.5, network=net, hf_key=None, capturable=cap)
+        step = lambda o: o.step()
+    gen = torch.Generator().manual_seed(2)
+    init = [torch.randn(s, generator=gen) * 0.1 for s in shapes]
+    grads = [[(torch.randn(s, generator=gen) * 0.05).cuda() for s in shapes] for _ in range(5)]
+    ref_p = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+    cap_p = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+    ref, cap = make(ref_p, False), make(cap_p, True)
+    for p in cap_p:
+        p.grad = torch.zeros_like(p)
+    graph = None
+    for t in range(5):
+        for p, q, g in zip(ref_p, cap_p, grads[t]):
+            p.grad = g.clone()
+            q.grad.copy_(g)
+        if t >= 3:                                   # the schedule: a third of the rate from step 3 on
+            for o in (ref, cap):
+                o.param_groups[0]["lr"] = o.defaults["lr"] / 3
+            cap.refresh_graph_tables()
+        step(ref)
+        if t == 0:
+            step(cap)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step(cap)
+        else:
+            graph.replay()
+        torch.cuda.synchronize()
+        _close(cap_p, ref_p, f"{which} step {t}")

@@ -72,6 +72,13 @@ def test_workspace_sizing_and_error_paths_without_gpu():
     assert b"2^31" in lib.pylo_mi355_last_error()
     assert lib.pylo_mi355_plan_workspace_bytes(7, shapes, 3, C.byref(n)) != 0
     assert lib.pylo_mi355_plan_destroy(None) == 0
+    # the graph-replay entry points refuse a null plan with a message instead of touching it
+    table = C.c_void_p()
+    assert lib.pylo_mi355_plan_arg_table(None, 0, C.byref(table)) != 0
+    assert b"plan_arg_table" in lib.pylo_mi355_last_error()
+    assert lib.pylo_mi355_plan_device_steps(None, None) != 0
+    assert b"plan_device_steps" in lib.pylo_mi355_last_error()
+    assert C.sizeof(_lib.DeviceSteps) == 8 + 3 * 8
 
 
 def test_optimizers_fail_loudly_without_gpu():
@@ -97,7 +104,7 @@ def test_optimizers_fail_loudly_without_gpu():
 
 def test_weight_containers_round_trip_through_the_reference_file_format(tmp_path):
     """config.json + model.safetensors written by save_pretrained load back bit-identically, with
-    the reference's parameter names (SURVEY row S)."""
+    the reference's parameter names."""
     import torch
 
     from pylo_amd.models import CELO2MLP, MetaMLP, VeLOMLP, VeLORNN

@@ -260,6 +260,54 @@ int pylo_mi355_velo_step(PyloPlan* plan, const PyloTensorArgs* args, const PyloD
 int pylo_mi355_adafac_step(PyloPlan* plan, const PyloTensorArgs* args, const PyloDecays* decays,
                            const float* net, float step, void* stream);
 
+/* ---- Single-tensor calls with the argument lists of the reference's extension functions ------------
+ * For callers that keep the reference's per-tensor loop (its optimizer classes update the accumulators
+ * and form row_factor / col_factor with tensor operations, then call one function per tensor).  All
+ * pointers are device pointers to contiguous fp32 data of the shapes the reference passes; `shape` /
+ * `ndim` describe the parameter (the reference reads them off the tensor); dc / dr are the factored
+ * dims (ignored when vector_like != 0).  `second_moment` must arrive zeroed and is accumulated into
+ * (30 / 28 / 30 floats).  Factor vectors of tensors with more than two dims are addressed as
+ * velo_kernel.cu:109-120 does, which for up to two dims is the `col_idx + k * num_cols` form of
+ * celo2_kernel.cu:67-84 / learned_optimizer.cu:55-72.  Launches go to `stream` (the reference uses
+ * the legacy default stream).  The plans above are the fast path: these calls cost two launches per
+ * tensor and leave the accumulator updates to the caller. */
+
+/* celo2_cuda_kernel.celo2_kernel (pylo/csrc/celo2_kernel.cu:284-357): step_out = o0 * exp(o1 * exp_mult)
+   of the 30 -> 8 -> 8 -> 3 MLP (weights stored (in, out)) on features normalised with eps 1e-9; p is
+   not modified. */
+int pylo_mi355_celo2_kernel(const float* g, const float* p, const float* m, const float* v,
+                            const float* fac_r, const float* fac_c, const float* row_factor,
+                            const float* col_factor, float* second_moment, const float* w_in,
+                            const float* b_in, const float* w_h, const float* b_h, const float* w_out,
+                            const float* b_out, float* step_out, float exp_mult, const int64_t* shape,
+                            int ndim, int dc, int dr, int vector_like, void* stream);
+
+/* cuda_lo.learned_optimizer_kernel (pylo/csrc/learned_optimizer.cu:303-404): 28 features (eps 1e-5) +
+   11 tanh(step / ts - 1) features, 39 -> 32 -> 32 -> 2 MLP with (out, in) weights;
+   p -= lr * o0 * exp(o1 * exp_mult) * step_mult.  `weight_decay` is accepted and unused, as in the
+   reference (its callers apply the decay themselves). */
+int pylo_mi355_learned_optimizer_kernel(const float* g, float* p, const float* m, const float* v,
+                                        const float* fac_r, const float* fac_c, const float* row_factor,
+                                        const float* col_factor, float* second_moment,
+                                        const float* input_weights, const float* input_bias,
+                                        const float* hidden_weights, const float* hidden_bias,
+                                        const float* output_weights, const float* output_bias, float lr,
+                                        float step_mult, float exp_mult, float epsilon, float step,
+                                        float weight_decay, const int64_t* shape, int ndim, int dc, int dr,
+                                        int vector_like, void* stream);
+
+/* velo_cuda_kernel.velo_kernel_simple (pylo/csrc/velo_kernel.cu:370-462; note the factor arguments
+   come in a different order than above): 30 features (eps 1e-5), 30 -> 4 -> 4 -> 3 MLP with (out, in)
+   weights; p -= lr * sqrt(mean p^2 + 1e-9) * o0 * exp(o1 * exp_mult) * step_mult, then
+   p -= weight_decay * lr * p when weight_decay > 0. */
+int pylo_mi355_velo_kernel_simple(const float* grad, float* param, const float* momentum, const float* rms,
+                                  const float* row_factor, const float* col_factor, const float* fac_vec_row,
+                                  const float* fac_vec_col, float* second_moment, const float* input_weights,
+                                  const float* input_bias, const float* hidden_weights, const float* hidden_bias,
+                                  const float* output_weights, const float* output_bias, float lr,
+                                  float step_mult, float exp_mult, float epsilon, float weight_decay,
+                                  const int64_t* shape, int ndim, int dc, int dr, int vector_like, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -480,6 +480,66 @@ def lo_feature_groups_1d(g, mom, rms, fac_v, rs_eps: float, fac_mom_eps: float):
     return rs, fac_g, fac_v, fac_v, torch.rsqrt(fac_v + 1e-8), torch.rsqrt(fac_v + 1e-8), fac_mom
 
 
+def velo_feature_groups(p, g, mom, rms, fac_row, fac_col, row_factor, col_factor):
+    """The 30 un-normalised VeLO channels as groups with a leading channel axis; ``fac_col is None``
+    marks a non-factored tensor whose accumulator ``fac_row`` is ``fac_vec_v (3,*s)``.
+
+    pylo/optim/Velo_naive.py:421-488 (the order of pylo/csrc/velo_kernel.cu:124-162)
+    """
+    if fac_col is not None:
+        rs = torch.rsqrt(rms + 1e-6)
+        full = (3,) + tuple(p.shape)
+        rowf, colf = fac_row.expand(full), fac_col.expand(full)
+        tail = [g[None] * row_factor * col_factor, (g * rs)[None], rowf, colf,
+                torch.rsqrt(rowf + 1e-8), torch.rsqrt(colf + 1e-8), mom * row_factor * col_factor]
+    else:
+        rs, fac_g, a, b_, c_, d_, fac_mom = lo_feature_groups_1d(g, mom, rms, fac_row, 1e-6, 0.0)
+        tail = [fac_g, (g * rs)[None], a, b_, c_, d_, fac_mom]
+    return [g[None], torch.clip(g, -0.1, 0.1)[None], p[None], mom, rms[None], mom * rs[None], rs[None]] + tail
+
+
+def velo_element_mlp(groups, weights):
+    """Normalise every channel over the whole tensor (eps 1e-5) and run the tensor's 30 -> 4 -> 4 -> 3
+    MLP, weights stored (out, in); returns (*shape, 3).  pylo/optim/Velo_naive.py:489-497"""
+    nd = groups[0].dim() - 1
+    axes = list(range(1, nd + 1))
+    x30 = torch.cat([rms_normalize(v, axes, 1e-5) for v in groups], dim=0)   # (30,*s)
+    w_in, b_in, w_h, b_h, w_out, b_out = weights
+    hcur = torch.relu(x30.movedim(0, -1) @ w_in.t() + b_in)
+    hcur = torch.relu(hcur @ w_h.t() + b_h)
+    return hcur @ w_out.t() + b_out
+
+
+def adafac_feature_groups(p, g, mom, rms, fac_r, fac_c, row_factor, col_factor):
+    """The 28 un-normalised AdafacLO channels; ``fac_c is None`` marks a non-factored tensor whose
+    accumulator ``fac_r`` is ``(3,*s)``.
+
+    pylo/optim/AdafacLO_naive.py:262-299 (the order of pylo/csrc/learned_optimizer.cu:59-97)
+    """
+    if fac_c is not None:
+        rs = torch.rsqrt(rms + 1e-6)
+        full = (3,) + tuple(p.shape)
+        rowf, colf = fac_r.expand(full), fac_c.expand(full)
+        tail = [g[None] * row_factor * col_factor, rowf, colf, torch.rsqrt(rowf + 1e-8),
+                torch.rsqrt(colf + 1e-8), mom * row_factor * col_factor]
+    else:
+        rs, fac_g, a, b_, c_, d_, fac_mom = lo_feature_groups_1d(g, mom, rms, fac_r, 1e-6, 1e-6)
+        tail = [fac_g, a, b_, c_, d_, fac_mom]
+    return [g[None], p[None], mom, rms[None], mom * rs[None], rs[None]] + tail
+
+
+def adafac_element_mlp(groups, tfeat, sd):
+    """Normalise the 28 channels over the whole tensor (eps 1e-5), append the 11 time features and run
+    the 39 -> 32 -> 32 -> 2 MetaMLP; returns (*shape, 2).  pylo/optim/AdafacLO_naive.py:300-307"""
+    shape = tuple(groups[0].shape[1:])
+    nd = len(shape)
+    x28 = rms_normalize(torch.cat(groups, dim=0), list(range(1, nd + 1)), 1e-5)
+    x = torch.cat([x28.movedim(0, -1), tfeat.expand(shape + (11,))], dim=-1)
+    hcur = torch.relu(x @ sd["network.input.weight"].t() + sd["network.input.bias"])
+    hcur = torch.relu(hcur @ sd["network.linear_0.weight"].t() + sd["network.linear_0.bias"])
+    return hcur @ sd["network.output.weight"].t() + sd["network.output.bias"]
+
+
 class VeloOracle:
     """VeLO_naive.step restated (pylo/optim/Velo_naive.py:384-503).
 
@@ -573,25 +633,12 @@ class VeloOracle:
             if fd is not None:
                 dc, dr = fd
                 rf, cf = _factored_update(st, g, self.beta_fac, dc, dr, "fac_vec_row", "fac_vec_col")
-                rs = torch.rsqrt(rms + 1e-6)
-                full = (3,) + tuple(p.shape)
-                rowf, colf = st["fac_vec_row"].expand(full), st["fac_vec_col"].expand(full)
-                tail = [g[None] * rf * cf, (g * rs)[None], rowf, colf,
-                        torch.rsqrt(rowf + 1e-8), torch.rsqrt(colf + 1e-8), st["mom"] * rf * cf]
+                groups = velo_feature_groups(p, g, st["mom"], rms, st["fac_vec_row"], st["fac_vec_col"], rf, cf)
             else:
                 b = _bview(self.beta_fac, nd)
                 st["fac_vec_v"] = b * st["fac_vec_v"] + (1 - b) * (g * g + 1e-30)[None]
-                rs, fac_g, a, b_, c_, d_, fac_mom = lo_feature_groups_1d(
-                    g, st["mom"], rms, st["fac_vec_v"], 1e-6, 0.0)
-                tail = [fac_g, (g * rs)[None], a, b_, c_, d_, fac_mom]
-            groups = [g[None], torch.clip(g, -0.1, 0.1)[None], p[None], st["mom"], rms[None],
-                      st["mom"] * rs[None], rs[None]] + tail
-            axes = list(range(1, nd + 1))
-            x30 = torch.cat([rms_normalize(v, axes, 1e-5) for v in groups], dim=0)   # (30,*s)
-            w_in, b_in, w_h, b_h, w_out, b_out = velo_mix_bank(controls[-(1 + i)], self.mlp)
-            hcur = torch.relu(x30.movedim(0, -1) @ w_in.t() + b_in)
-            hcur = torch.relu(hcur @ w_h.t() + b_h)
-            out = hcur @ w_out.t() + b_out
+                groups = velo_feature_groups(p, g, st["mom"], rms, st["fac_vec_v"], None, None, None)
+            out = velo_element_mlp(groups, velo_mix_bank(controls[-(1 + i)], self.mlp))
             param_scale = torch.sqrt(torch.mean(p ** 2) + 1e-9)
             step = param_scale * (out[..., 0] * torch.exp(out[..., 1] * self.exp_mult) * self.step_mult)
             step = lr_mult[-(1 + i)] * step
@@ -688,24 +735,13 @@ class AdafacOracle:
             if fd is not None:
                 dc, dr = fd
                 rf, cf = _factored_update(st, g, self.beta_fac, dc, dr, "exp_avg_sq_r", "exp_avg_sq_c")
-                rs = torch.rsqrt(rms + 1e-6)
-                full = (3,) + tuple(p.shape)
-                rowf, colf = st["exp_avg_sq_r"].expand(full), st["exp_avg_sq_c"].expand(full)
-                tail = [g[None] * rf * cf, rowf, colf, torch.rsqrt(rowf + 1e-8),
-                        torch.rsqrt(colf + 1e-8), mom * rf * cf]
+                groups = adafac_feature_groups(p, g, mom, rms, st["exp_avg_sq_r"], st["exp_avg_sq_c"], rf, cf)
             else:
                 b = _bview(self.beta_fac, nd)
                 st["exp_avg_sq_r"] = b * st["exp_avg_sq_r"] + (1 - b) * (g * g + 1e-30)[None]
                 st["exp_avg_sq_c"] = st["exp_avg_sq_r"]
-                rs, fac_g, a, b_, c_, d_, fac_mom = lo_feature_groups_1d(
-                    g, mom, rms, st["exp_avg_sq_r"], 1e-6, 1e-6)
-                tail = [fac_g, a, b_, c_, d_, fac_mom]
-            groups = [g[None], p[None], mom, rms[None], mom * rs[None], rs[None]] + tail
-            x28 = rms_normalize(torch.cat(groups, dim=0), list(range(1, nd + 1)), 1e-5)
-            x = torch.cat([x28.movedim(0, -1), tfeat.expand(tuple(p.shape) + (11,))], dim=-1)
-            hcur = torch.relu(x @ sd["network.input.weight"].t() + sd["network.input.bias"])
-            hcur = torch.relu(hcur @ sd["network.linear_0.weight"].t() + sd["network.linear_0.bias"])
-            out = hcur @ sd["network.output.weight"].t() + sd["network.output.bias"]
+                groups = adafac_feature_groups(p, g, mom, rms, st["exp_avg_sq_r"], None, None, None)
+            out = adafac_element_mlp(groups, tfeat, sd)
             self.apply(p, out[..., 0] * torch.exp(out[..., 1] * self.exp_mult))
 
 

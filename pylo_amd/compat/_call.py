@@ -1,0 +1,60 @@
+"""Shared argument handling of the single-tensor calls."""
+
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from .. import _lib
+
+_F = C.c_float
+_P = C.c_void_p
+_TAIL = [C.POINTER(C.c_int64), C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+_SIGS = {
+    "pylo_mi355_celo2_kernel": [_P] * 16 + [_F] + _TAIL,
+    "pylo_mi355_learned_optimizer_kernel": [_P] * 15 + [_F] * 6 + _TAIL,
+    "pylo_mi355_velo_kernel_simple": [_P] * 15 + [_F] * 5 + _TAIL,
+}
+_bound = set()
+
+
+def entry(name: str):
+    lib = _lib.load()
+    fn = getattr(lib, name)
+    if name not in _bound:
+        fn.argtypes = _SIGS[name]
+        fn.restype = C.c_int
+        _bound.add(name)
+    return fn
+
+
+def pointers(who: str, device: torch.device, **tensors) -> list:
+    """Device pointers of contiguous float32 tensors on `device`; an empty tensor gives a null pointer
+    (the reference passes nullptr for empty factor tensors, velo_kernel.cu:411-414)."""
+    out = []
+    for name, t in tensors.items():
+        if not torch.is_tensor(t):
+            raise TypeError(f"{who}: {name} must be a tensor")
+        if t.numel() == 0:
+            out.append(None)
+            continue
+        if not t.is_cuda or t.device != device:
+            raise RuntimeError(f"{who}: {name} must live on {device}")
+        if t.dtype != torch.float32:
+            raise TypeError(f"{who}: {name} must be float32 (got {t.dtype})")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{who}: {name} must be contiguous")
+        out.append(t.data_ptr())
+    return out
+
+
+def shape_args(p: torch.Tensor):
+    arr = (C.c_int64 * max(p.dim(), 1))(*p.shape)
+    return arr, p.dim()
+
+
+def run(who: str, name: str, p: torch.Tensor, args: list) -> None:
+    with torch.cuda.device(p.device):
+        stream = torch.cuda.current_stream(p.device).cuda_stream
+        _lib.check(entry(name)(*args, stream), who)

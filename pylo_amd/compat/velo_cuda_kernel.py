@@ -1,0 +1,20 @@
+"""``velo_cuda_kernel`` of the reference (pylo/csrc/velo_kernel.cu:370-462) on the HIP library."""
+
+from ._call import pointers, run, shape_args
+
+
+def velo_kernel_simple(grad, param, momentum, rms, row_factor, col_factor, fac_vec_row, fac_vec_col, second_moment,
+                       input_weights, input_bias, hidden_weights, hidden_bias, output_weights, output_bias, lr,
+                       step_mult, exp_mult, epsilon, weight_decay, dc, dr, vector_like):
+    """Adds the sums of squared features into ``second_moment`` (30, zeroed by the caller) and updates
+    ``param`` in place, weight decay included."""
+    who = "velo_kernel_simple"
+    ptrs = pointers(who, param.device, grad=grad, param=param, momentum=momentum, rms=rms, row_factor=row_factor,
+                    col_factor=col_factor, fac_vec_row=fac_vec_row, fac_vec_col=fac_vec_col,
+                    second_moment=second_moment, input_weights=input_weights, input_bias=input_bias,
+                    hidden_weights=hidden_weights, hidden_bias=hidden_bias, output_weights=output_weights,
+                    output_bias=output_bias)
+    shape, ndim = shape_args(param)
+    run(who, "pylo_mi355_velo_kernel_simple", param,
+        ptrs + [float(lr), float(step_mult), float(exp_mult), float(epsilon), float(weight_decay),
+                shape, ndim, int(dc), int(dr), int(vector_like)])

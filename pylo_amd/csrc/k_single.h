@@ -1,0 +1,206 @@
+// Single-tensor kernels behind the entry points that keep the argument lists of the reference's three
+// extension functions (celo2_cuda_kernel.celo2_kernel, cuda_lo.learned_optimizer_kernel,
+// velo_cuda_kernel.velo_kernel_simple): the caller has already updated the accumulators and formed
+// row_factor / col_factor; one launch adds the per-channel sums of squared features into
+// `second_moment`, a second one normalises, runs the MLP and writes the step or the parameter.
+// These are the compatibility path for per-tensor callers; the multi-tensor plans are the fast path.
+#pragma once
+
+#include "pylo_common.h"
+
+namespace pylo {
+
+enum { kFamCelo2 = 0, kFamLo = 1, kFamVelo = 2 };
+
+template <int F> struct Fam;
+// CELO2: 30 channels, 30 -> 8 -> 8 -> 3, weights stored (in, out)          (celo2_kernel.cu:33-40,214-219)
+template <> struct Fam<kFamCelo2> { static constexpr int NSTAT = 30, NIN = 30, H = 8, NOUT = 3; static constexpr bool in_major = true; };
+// AdafacLO / ELO: 28 channels + 11 time features, 39 -> 32 -> 32 -> 2, (out, in)   (learned_optimizer.cu:10-13)
+template <> struct Fam<kFamLo> { static constexpr int NSTAT = 28, NIN = 39, H = 32, NOUT = 2; static constexpr bool in_major = false; };
+// VeLO: 30 channels, 30 -> 4 -> 4 -> 3, (out, in)                                   (velo_kernel.cu:10-13)
+template <> struct Fam<kFamVelo> { static constexpr int NSTAT = 30, NIN = 30, H = 4, NOUT = 3; static constexpr bool in_major = false; };
+
+struct SingleArgs {
+  const float *g, *m, *v, *fac_r, *fac_c, *row_factor, *col_factor;
+  float* p;              // read by every family; updated in place by the lo / velo families
+  float* second_moment;  // NSTAT floats, accumulated into (the caller zeroes it)
+  const float *w_in, *b_in, *w_h, *b_h, *w_out, *b_out;
+  float* step_out;       // celo2 only
+  int n, num_rows, num_cols, row_stride, col_stride, vector_like;
+  float lr, step_mult, exp_mult, epsilon, step, weight_decay;
+};
+
+constexpr int kSingleThreads = 256;
+constexpr int kSingleMaxBlocks = 2048;
+
+// Offsets of element idx into the row vectors (row_factor, fac_r: the tensor's shape with the largest
+// dim dr removed) and the column vectors (col_factor, fac_c: dim dc removed), and their decay strides.
+// For tensors of up to two dims this is the reference's `col_idx + k * num_cols` / `row_idx + k * num_rows`
+// (celo2_kernel.cu:67-84, learned_optimizer.cu:55-72); with more dims it is velo_kernel.cu:109-120.
+struct FacOfs { int r, c, stride_r, stride_c; };
+__device__ __forceinline__ FacOfs fac_offsets(const SingleArgs& a, int idx) {
+  FacOfs o;
+  if (a.vector_like) {
+    o.r = o.c = idx;
+    o.stride_r = o.stride_c = a.n;
+  } else {
+    o.stride_r = a.n / a.num_rows;
+    o.stride_c = a.n / a.num_cols;
+    o.r = (idx / (a.num_rows * a.row_stride)) * a.row_stride + idx % a.row_stride;
+    o.c = (idx / (a.num_cols * a.col_stride)) * a.col_stride + idx % a.col_stride;
+  }
+  return o;
+}
+
+template <int F>
+__device__ __forceinline__ void single_features(const SingleArgs& a, int idx, float (&f)[Fam<F>::NSTAT]) {
+  const FacOfs o = fac_offsets(a, idx);
+  const float g = a.g[idx], p = a.p[idx];
+  const float m0 = a.m[idx], m1 = a.m[idx + (size_t)a.n], m2 = a.m[idx + 2 * (size_t)a.n];
+  const float v = a.v[idx];
+  const bool vl = a.vector_like != 0;
+  const float rf0 = a.row_factor[o.r], rf1 = a.row_factor[o.r + (size_t)o.stride_r],
+              rf2 = a.row_factor[o.r + 2 * (size_t)o.stride_r];
+  const float cf0 = vl ? 1.0f : a.col_factor[o.c], cf1 = vl ? 1.0f : a.col_factor[o.c + (size_t)o.stride_c],
+              cf2 = vl ? 1.0f : a.col_factor[o.c + 2 * (size_t)o.stride_c];
+  if constexpr (F == kFamLo) {
+    // learned_optimizer.cu:34-98
+    const float rs = rsq(v + a.epsilon);
+    f[0] = g; f[1] = p; f[2] = m0; f[3] = m1; f[4] = m2; f[5] = v;
+    f[6] = m0 * rs; f[7] = m1 * rs; f[8] = m2 * rs; f[9] = rs;
+    f[10] = rf0 * cf0 * g; f[11] = rf1 * cf1 * g; f[12] = rf2 * cf2 * g;
+    const float r0 = a.fac_r[o.r], r1 = a.fac_r[o.r + (size_t)o.stride_r], r2 = a.fac_r[o.r + 2 * (size_t)o.stride_r];
+    const float c0 = a.fac_c[o.c], c1 = a.fac_c[o.c + (size_t)o.stride_c], c2 = a.fac_c[o.c + 2 * (size_t)o.stride_c];
+    f[13] = r0; f[14] = r1; f[15] = r2; f[16] = c0; f[17] = c1; f[18] = c2;
+    f[19] = rsq(r0 + 1e-8f); f[20] = rsq(r1 + 1e-8f); f[21] = rsq(r2 + 1e-8f);
+    f[22] = rsq(c0 + 1e-8f); f[23] = rsq(c1 + 1e-8f); f[24] = rsq(c2 + 1e-8f);
+    f[25] = rf0 * cf0 * m0; f[26] = rf1 * cf1 * m1; f[27] = rf2 * cf2 * m2;
+  } else {
+    // celo2_kernel.cu:48-125 (rsqrt epsilon fixed at 1e-8), velo_kernel.cu:72-164 (epsilon argument)
+    const float rs = rsq(v + (F == kFamCelo2 ? 1e-8f : a.epsilon));
+    f[0] = g; f[1] = fminf(fmaxf(g, -0.1f), 0.1f); f[2] = p; f[3] = m0; f[4] = m1; f[5] = m2; f[6] = v;
+    f[7] = m0 * rs; f[8] = m1 * rs; f[9] = m2 * rs; f[10] = rs;
+    f[11] = g * rf0 * cf0; f[12] = g * rf1 * cf1; f[13] = g * rf2 * cf2;
+    f[14] = g * rs;
+    if (F == kFamCelo2 && vl) {   // only the first nine feature groups exist for a vector-like tensor
+#pragma unroll
+      for (int c = 15; c < 30; ++c) f[c] = 0.0f;
+      return;
+    }
+    const float r0 = a.fac_r[o.r], r1 = a.fac_r[o.r + (size_t)o.stride_r], r2 = a.fac_r[o.r + 2 * (size_t)o.stride_r];
+    const float c0 = a.fac_c[o.c], c1 = a.fac_c[o.c + (size_t)o.stride_c], c2 = a.fac_c[o.c + 2 * (size_t)o.stride_c];
+    f[15] = r0; f[16] = r1; f[17] = r2; f[18] = c0; f[19] = c1; f[20] = c2;
+    f[21] = rsq(r0 + 1e-8f); f[22] = rsq(r1 + 1e-8f); f[23] = rsq(r2 + 1e-8f);
+    f[24] = rsq(c0 + 1e-8f); f[25] = rsq(c1 + 1e-8f); f[26] = rsq(c2 + 1e-8f);
+    f[27] = m0 * rf0 * cf0; f[28] = m1 * rf1 * cf1; f[29] = m2 * rf2 * cf2;
+  }
+}
+
+// second_moment[c] += sum over the elements of feature_c^2: per-thread and per-wave sums, then one
+// float atomic per channel and block, as the reference does (celo2_kernel.cu:129-199).
+template <int F>
+__global__ __launch_bounds__(kSingleThreads) void k_single_moment(SingleArgs a) {
+  constexpr int NS = Fam<F>::NSTAT;
+  float acc[NS];
+#pragma unroll
+  for (int c = 0; c < NS; ++c) acc[c] = 0.0f;
+  for (long long i = (long long)blockIdx.x * kSingleThreads + threadIdx.x; i < a.n;
+       i += (long long)gridDim.x * kSingleThreads) {
+    float f[NS];
+    single_features<F>(a, (int)i, f);
+#pragma unroll
+    for (int c = 0; c < NS; ++c) acc[c] = fmaf(f[c], f[c], acc[c]);
+  }
+  __shared__ float s[kSingleThreads / 64][NS];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+  for (int c = 0; c < NS; ++c) {
+    const float t = wave_sum(acc[c]);
+    if (lane == 0) s[wave][c] = t;
+  }
+  __syncthreads();
+  if (threadIdx.x < NS) {
+    float t = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kSingleThreads / 64; ++w) t += s[w][threadIdx.x];
+    atomicAdd(a.second_moment + threadIdx.x, t);
+  }
+}
+
+// Normalise by rsqrt(second_moment / n + eps), MLP, output.  The weights are staged in LDS once per
+// block with the channel normalisers folded into the first layer ([k][j] layout, read as broadcasts);
+// AdafacLO's eleven time features are the same for every element and go into the first bias.
+template <int F>
+__global__ __launch_bounds__(kSingleThreads) void k_single_apply(SingleArgs a) {
+  using Fm = Fam<F>;
+  constexpr int NS = Fm::NSTAT, NIN = Fm::NIN, H = Fm::H, NO = Fm::NOUT;
+  __shared__ float s_norm[NS];
+  __shared__ float w1[NS * H], w2[H * H], w3[H * NO], b1[H], b2[H], b3[NO];
+  const int tid = threadIdx.x;
+  const float nf = (float)a.n;
+  if (tid < NS) s_norm[tid] = rsq(a.second_moment[tid] / nf + (F == kFamCelo2 ? 1e-9f : 1e-5f));
+  __syncthreads();
+  for (int i = tid; i < NS * H; i += kSingleThreads) {
+    const int k = i / H, j = i % H;
+    w1[i] = (Fm::in_major ? a.w_in[k * H + j] : a.w_in[j * NIN + k]) * s_norm[k];
+  }
+  for (int i = tid; i < H * H; i += kSingleThreads) {
+    const int k = i / H, j = i % H;
+    w2[i] = Fm::in_major ? a.w_h[k * H + j] : a.w_h[j * H + k];
+  }
+  for (int i = tid; i < H * NO; i += kSingleThreads) {
+    const int k = i / NO, j = i % NO;
+    w3[i] = Fm::in_major ? a.w_out[k * NO + j] : a.w_out[j * H + k];
+  }
+  if (tid < H) {
+    float b = a.b_in[tid];
+    if constexpr (F == kFamLo) {   // tanh(step / ts - 1), learned_optimizer.cu:27-32
+      const float ts[11] = {1.f, 3.f, 10.f, 30.f, 100.f, 300.f, 1000.f, 3000.f, 10000.f, 30000.f, 100000.f};
+#pragma unroll
+      for (int q = 0; q < 11; ++q) b = fmaf(tanhf(a.step / ts[q] - 1.0f), a.w_in[tid * NIN + NS + q], b);
+    }
+    b1[tid] = b;
+    b2[tid] = a.b_h[tid];
+  }
+  if (tid < NO) b3[tid] = a.b_out[tid];
+  __syncthreads();
+  const float pscale = F == kFamVelo ? sqrtf(a.second_moment[2] / nf + 1e-9f) : 1.0f;   // channel 2 is p
+
+  for (long long i = (long long)blockIdx.x * kSingleThreads + tid; i < a.n; i += (long long)gridDim.x * kSingleThreads) {
+    float f[NS];
+    single_features<F>(a, (int)i, f);
+    float h0[H], h1[H], out[NO];
+#pragma unroll
+    for (int j = 0; j < H; ++j) h0[j] = b1[j];
+#pragma unroll
+    for (int k = 0; k < NS; ++k)
+#pragma unroll
+      for (int j = 0; j < H; ++j) h0[j] = fmaf(f[k], w1[k * H + j], h0[j]);
+#pragma unroll
+    for (int j = 0; j < H; ++j) { h0[j] = fmaxf(h0[j], 0.0f); h1[j] = b2[j]; }
+#pragma unroll
+    for (int k = 0; k < H; ++k)
+#pragma unroll
+      for (int j = 0; j < H; ++j) h1[j] = fmaf(h0[k], w2[k * H + j], h1[j]);
+#pragma unroll
+    for (int j = 0; j < NO; ++j) out[j] = b3[j];
+#pragma unroll
+    for (int k = 0; k < H; ++k) {
+      const float hk = fmaxf(h1[k], 0.0f);
+#pragma unroll
+      for (int j = 0; j < NO; ++j) out[j] = fmaf(hk, w3[k * NO + j], out[j]);
+    }
+    const float step = out[0] * expf(out[1] * a.exp_mult);
+    if constexpr (F == kFamCelo2) {
+      a.step_out[i] = step;                                   // celo2_kernel.cu:280; p is left untouched
+    } else if constexpr (F == kFamLo) {
+      a.p[i] = f[1] - a.lr * (step * a.step_mult);            // learned_optimizer.cu:296-299
+    } else {
+      float pn = f[2] - a.lr * (pscale * step * a.step_mult); // velo_kernel.cu:352-362
+      if (a.weight_decay > 0.0f) pn = pn - a.weight_decay * a.lr * pn;
+      a.p[i] = pn;
+    }
+  }
+}
+
+}  // namespace pylo

@@ -20,6 +20,7 @@
 #include "k_celo2.h"
 #include "k_gradstats.h"
 #include "k_adafac.h"
+#include "k_single.h"
 #include "k_velo.h"
 #include "k_celo2_slices.h"
 #include "pylo_common.h"
@@ -907,4 +908,111 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   mark.done();
   HIP_TRY(hipGetLastError());
   return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Single-tensor calls with the reference's argument lists
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+// Geometry as the reference launchers derive it from the parameter tensor (celo2_kernel.cu:306-312):
+// sizes and strides of dims dr / dc of a contiguous tensor.
+int single_geometry(const char* who, const int64_t* shape, int ndim, int dc, int dr, int vector_like, SingleArgs& a) {
+  const std::string w(who);
+  if (ndim < 0 || ndim > PYLO_MAX_DIMS || (ndim > 0 && !shape)) return fail(w + ": bad shape");
+  long long n = 1;
+  for (int i = 0; i < ndim; ++i) {
+    if (shape[i] < 0) return fail(w + ": negative dim");
+    n *= shape[i];
+    if (n >= (1LL << 31)) return fail(w + ": tensors of 2^31 elements or more are not supported");
+  }
+  a.n = (int)n;
+  a.vector_like = vector_like ? 1 : 0;
+  if (vector_like) {
+    a.num_rows = a.num_cols = a.n;
+    a.row_stride = a.col_stride = 1;
+    return 0;
+  }
+  if (dc < 0 || dr < 0 || dc >= ndim || dr >= ndim || dc == dr) return fail(w + ": dc / dr are not two dims of the tensor");
+  auto stride = [&](int d) {
+    long long st = 1;
+    for (int i = d + 1; i < ndim; ++i) st *= shape[i];
+    return (int)st;
+  };
+  a.num_rows = (int)shape[dr];
+  a.num_cols = (int)shape[dc];
+  a.row_stride = stride(dr);
+  a.col_stride = stride(dc);
+  return 0;
+}
+
+template <int F>
+int single_launch(const char* who, const SingleArgs& a, void* stream) {
+  if (a.n == 0) return 0;
+  if (!a.g || !a.p || !a.m || !a.v || !a.fac_r || !a.fac_c || !a.row_factor || !a.second_moment || !a.w_in ||
+      !a.b_in || !a.w_h || !a.b_h || !a.w_out || !a.b_out || (!a.vector_like && !a.col_factor) ||
+      (F == kFamCelo2 && !a.step_out))
+    return fail(std::string(who) + ": null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int blocks = std::min((a.n + kSingleThreads - 1) / kSingleThreads, kSingleMaxBlocks);
+  hipLaunchKernelGGL(k_single_moment<F>, dim3(blocks), dim3(kSingleThreads), 0, s, a);
+  hipLaunchKernelGGL(k_single_apply<F>, dim3(blocks), dim3(kSingleThreads), 0, s, a);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int pylo_mi355_celo2_kernel(const float* g, const float* p, const float* m, const float* v,
+                                       const float* fac_r, const float* fac_c, const float* row_factor,
+                                       const float* col_factor, float* second_moment, const float* w_in,
+                                       const float* b_in, const float* w_h, const float* b_h, const float* w_out,
+                                       const float* b_out, float* step_out, float exp_mult, const int64_t* shape,
+                                       int ndim, int dc, int dr, int vector_like, void* stream) {
+  SingleArgs a{};
+  if (int rc = single_geometry("celo2_kernel", shape, ndim, dc, dr, vector_like, a)) return rc;
+  a.g = g; a.p = const_cast<float*>(p); a.m = m; a.v = v; a.fac_r = fac_r; a.fac_c = fac_c;
+  a.row_factor = row_factor; a.col_factor = col_factor; a.second_moment = second_moment;
+  a.w_in = w_in; a.b_in = b_in; a.w_h = w_h; a.b_h = b_h; a.w_out = w_out; a.b_out = b_out;
+  a.step_out = step_out; a.exp_mult = exp_mult;
+  return single_launch<kFamCelo2>("celo2_kernel", a, stream);
+}
+
+extern "C" int pylo_mi355_learned_optimizer_kernel(const float* g, float* p, const float* m, const float* v,
+                                                   const float* fac_r, const float* fac_c, const float* row_factor,
+                                                   const float* col_factor, float* second_moment,
+                                                   const float* input_weights, const float* input_bias,
+                                                   const float* hidden_weights, const float* hidden_bias,
+                                                   const float* output_weights, const float* output_bias, float lr,
+                                                   float step_mult, float exp_mult, float epsilon, float step,
+                                                   float weight_decay, const int64_t* shape, int ndim, int dc, int dr,
+                                                   int vector_like, void* stream) {
+  SingleArgs a{};
+  if (int rc = single_geometry("learned_optimizer_kernel", shape, ndim, dc, dr, vector_like, a)) return rc;
+  a.g = g; a.p = p; a.m = m; a.v = v; a.fac_r = fac_r; a.fac_c = fac_c;
+  a.row_factor = row_factor; a.col_factor = col_factor; a.second_moment = second_moment;
+  a.w_in = input_weights; a.b_in = input_bias; a.w_h = hidden_weights; a.b_h = hidden_bias;
+  a.w_out = output_weights; a.b_out = output_bias;
+  a.lr = lr; a.step_mult = step_mult; a.exp_mult = exp_mult; a.epsilon = epsilon; a.step = step;
+  a.weight_decay = weight_decay;
+  return single_launch<kFamLo>("learned_optimizer_kernel", a, stream);
+}
+
+extern "C" int pylo_mi355_velo_kernel_simple(const float* grad, float* param, const float* momentum, const float* rms,
+                                             const float* row_factor, const float* col_factor,
+                                             const float* fac_vec_row, const float* fac_vec_col, float* second_moment,
+                                             const float* input_weights, const float* input_bias,
+                                             const float* hidden_weights, const float* hidden_bias,
+                                             const float* output_weights, const float* output_bias, float lr,
+                                             float step_mult, float exp_mult, float epsilon, float weight_decay,
+                                             const int64_t* shape, int ndim, int dc, int dr, int vector_like,
+                                             void* stream) {
+  SingleArgs a{};
+  if (int rc = single_geometry("velo_kernel_simple", shape, ndim, dc, dr, vector_like, a)) return rc;
+  a.g = grad; a.p = param; a.m = momentum; a.v = rms; a.fac_r = fac_vec_row; a.fac_c = fac_vec_col;
+  a.row_factor = row_factor; a.col_factor = col_factor; a.second_moment = second_moment;
+  a.w_in = input_weights; a.b_in = input_bias; a.w_h = hidden_weights; a.b_h = hidden_bias;
+  a.w_out = output_weights; a.b_out = output_bias;
+  a.lr = lr; a.step_mult = step_mult; a.exp_mult = exp_mult; a.epsilon = epsilon; a.weight_decay = weight_decay;
+  return single_launch<kFamVelo>("velo_kernel_simple", a, stream);
 }

@@ -126,3 +126,28 @@ def test_weight_containers_round_trip_through_the_reference_file_format(tmp_path
     assert {"input_weights_", "hidden_weights_.0", "output_bias"} <= set(VeLOMLP(param_inits=4).state_dict())
     assert {"mix_layer1.weight", "lstm.linear.bias", "lstm_init_state.1", "step_size.weight"} <= \
         set(VeLORNN(lstm_hidden_size=64, param_inits=4).state_dict())
+
+
+def test_reference_module_names_resolve_after_install():
+    """``pylo_amd.compat.install()`` registers modules under the reference's extension-module names with
+    its function names and argument lists (pylo/csrc/celo2_kernel.cu:352-357, learned_optimizer.cu:396-403,
+    velo_kernel.cu:459-462)."""
+    import importlib
+    import inspect
+
+    from pylo_amd import compat
+
+    compat.install()
+    want = {
+        "celo2_cuda_kernel": ("celo2_kernel", 20),
+        "cuda_lo": ("learned_optimizer_kernel", 24),
+        "velo_cuda_kernel": ("velo_kernel_simple", 23),
+    }
+    for mod, (fn, nargs) in want.items():
+        f = getattr(importlib.import_module(mod), fn)
+        assert len(inspect.signature(f).parameters) == nargs, (mod, fn)
+    import torch
+
+    with pytest.raises((RuntimeError, TypeError)):       # CPU tensors are refused before anything is launched
+        z = torch.zeros(4, 4)
+        importlib.import_module("celo2_cuda_kernel").celo2_kernel(*([z] * 16), 0.0, 1, 0, 0)

@@ -1,0 +1,182 @@
+"""The single-tensor calls that keep the reference's extension-module signatures
+(``celo2_cuda_kernel.celo2_kernel``, ``cuda_lo.learned_optimizer_kernel``,
+``velo_cuda_kernel.velo_kernel_simple``) against the oracle's per-tensor feature / MLP functions, which
+the golden trajectories pin through the oracle classes.
+
+The caller supplies already-updated accumulators and the row / column factors, as the reference's
+optimizer classes do (ELO_CELO2_cuda.py:187-202,265-286; AdafacLO_cuda.py:335-405; velo_cuda.py:693-755).
+For non-factored tensors the kernels' single ``row_factor`` multiplies both the gradient and the momentum
+channels, so the expected momentum channels are ``mom * row_factor`` there (the CUDA classes' form; the
+naive classes use a different epsilon for them).  Tolerance rel 1e-5 / abs 1e-6 on outputs, rel 1e-5 on
+``second_moment``.
+"""
+
+import pytest
+import torch
+
+from golden_io import max_err
+from oracle import pylo_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+REL, ABS = 1e-5, 1e-6
+
+
+def _state(shape, seed, factored_dims):
+    gen = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=gen)
+    st = dict(g=r(*shape) * 0.05, p=r(*shape) * 0.1, mom=r(3, *shape) * 0.03, rms=r(*shape).abs() * 2e-3 + 1e-6)
+    fd = factored_dims(tuple(shape))
+    if fd is not None:
+        dc, dr = fd
+        rs, cs = list(shape), list(shape)
+        rs[dr], cs[dc] = 1, 1
+        st["fac_r"] = r(3, *rs).abs() * 2e-3 + 1e-7
+        st["fac_c"] = r(3, *cs).abs() * 2e-3 + 1e-7
+        st["rf"], st["cf"] = O._row_col_factors(st["fac_r"], st["fac_c"], dc)
+        st["dims"] = (dc, dr, 0)
+    else:
+        st["fac_r"] = st["fac_c"] = r(3, *shape).abs() * 2e-3 + 1e-7
+        st["rf"] = O.safe_rsqrt(st["fac_r"] + 1e-9)
+        st["cf"] = torch.ones_like(st["rf"])
+        st["dims"] = (0, 0, 1)
+    return st
+
+
+def _cuda(st, *keys):
+    return [st[k].contiguous().cuda() for k in keys]
+
+
+def _check_moment(second_moment, groups):
+    ref = torch.cat([(x.double() ** 2).reshape(x.shape[0], -1).sum(1) for x in groups])
+    got = second_moment.cpu().double()[: ref.numel()]
+    assert torch.all((got - ref).abs() <= 1e-5 * ref.abs() + 1e-30), (got, ref)
+
+
+@pytest.mark.parametrize("shape", [(48, 40), (40, 72), (333,), (1, 17)])
+def test_celo2_kernel_signature(shape):
+    from pylo_amd.compat import celo2_cuda_kernel
+    from pylo_amd.models import CELO2MLP
+
+    torch.manual_seed(11)
+    net = CELO2MLP()
+    sd = net.state_dict()
+    st = _state(shape, 1, O.factored_dims)
+    dc, dr, vl = st["dims"]
+    if vl:
+        rs = torch.rsqrt(st["rms"] + 1e-8)
+        groups = [st["g"][None], torch.clamp(st["g"], -0.1, 0.1)[None], st["p"][None], st["mom"], st["rms"][None],
+                  st["mom"] * rs[None], rs[None], st["g"][None] * st["rf"], (st["g"] * rs)[None]]
+    else:
+        groups = O.celo2_feature_groups(st["p"], st["g"], st["mom"], st["rms"], st["fac_r"], st["fac_c"],
+                                        st["rf"], st["cf"])
+    axes = list(range(1, len(shape) + 1))
+    out = O.celo2_mlp([O.rms_normalize(x, axes, 1e-9) for x in groups], sd)
+    exp_mult = 0.3
+    want = out[..., 0] * torch.exp(out[..., 1] * exp_mult)
+
+    g, p, m, v, fr, fc, rf, cf = _cuda(st, "g", "p", "mom", "rms", "fac_r", "fac_c", "rf", "cf")
+    w_in = torch.cat([sd[f"w0.{i}"] for i in range(14)]).contiguous().cuda()
+    ws = [w_in] + [sd[k].contiguous().cuda() for k in ("b0", "dense_w.0", "dense_b.0", "dense_w.1", "dense_b.1")]
+    sm = torch.zeros(30, device="cuda")
+    step_out = torch.full(shape, float("nan"), device="cuda")
+    p_before = p.clone()
+    celo2_cuda_kernel.celo2_kernel(g, p, m, v, fr, fc, rf, cf, sm, *ws, step_out, exp_mult, dc, dr, vl)
+    assert max_err(step_out.cpu(), want, REL, ABS) <= 1.0
+    assert torch.equal(p, p_before)
+    _check_moment(sm, groups)
+
+
+@pytest.mark.parametrize("shape", [(48, 40), (40, 72), (333,), (6, 4, 3, 3)])
+def test_learned_optimizer_kernel_signature(shape):
+    from pylo_amd.compat import cuda_lo
+    from pylo_amd.models import MetaMLP
+
+    torch.manual_seed(12)
+    sd = MetaMLP(39, 32, 1).state_dict()
+    st = _state(shape, 2, O.factored_dims)
+    dc, dr, vl = st["dims"]
+    if vl:
+        groups = O.adafac_feature_groups(st["p"], st["g"], st["mom"], st["rms"], st["fac_r"], None, None, None)
+        groups[-1] = st["mom"] * st["rf"]
+    else:
+        groups = O.adafac_feature_groups(st["p"], st["g"], st["mom"], st["rms"], st["fac_r"], st["fac_c"],
+                                         st["rf"], st["cf"])
+    step, lr, step_mult, exp_mult = 7.0, 0.5, 0.01, 0.001
+    out = O.adafac_element_mlp(groups, O.tanh_time_embedding(step), sd)
+    want = st["p"] - lr * (out[..., 0] * torch.exp(out[..., 1] * exp_mult) * step_mult)
+
+    g, p, m, v, fr, fc, rf, cf = _cuda(st, "g", "p", "mom", "rms", "fac_r", "fac_c", "rf", "cf")
+    ws = [sd[k].contiguous().cuda() for k in ("network.input.weight", "network.input.bias", "network.linear_0.weight",
+                                              "network.linear_0.bias", "network.output.weight", "network.output.bias")]
+    sm = torch.zeros(28, device="cuda")
+    cuda_lo.learned_optimizer_kernel(g, p, m, v, fr, fc, rf, cf, sm, *ws, lr, step_mult, exp_mult, 1e-6, step, 0.0,
+                                     dc, dr, vl)
+    assert max_err(p.cpu(), want, REL, ABS) <= 1.0
+    _check_moment(sm, groups)
+
+
+@pytest.mark.parametrize("shape,wd", [((48, 40), 0.0), ((40, 72), 0.02), ((333,), 0.02), ((6, 4, 3, 3), 0.0),
+                                      ((5, 3, 7), 0.1)])
+def test_velo_kernel_simple_signature(shape, wd):
+    from pylo_amd.compat import velo_cuda_kernel
+
+    gen = torch.Generator().manual_seed(13)
+    weights = [torch.randn(s, generator=gen) * sc for s, sc in
+               (((4, 30), 0.3), ((4,), 0.1), ((4, 4), 0.5), ((4,), 0.1), ((3, 4), 0.5), ((3,), 0.1))]
+    st = _state(shape, 3, O.factored_dims_velo)
+    dc, dr, vl = st["dims"]
+    if vl:
+        groups = O.velo_feature_groups(st["p"], st["g"], st["mom"], st["rms"], st["fac_r"], None, None, None)
+        groups[-1] = st["mom"] * st["rf"]
+    else:
+        groups = O.velo_feature_groups(st["p"], st["g"], st["mom"], st["rms"], st["fac_r"], st["fac_c"],
+                                       st["rf"], st["cf"])
+    lr, step_mult, exp_mult = 0.03, 0.001, 0.001
+    out = O.velo_element_mlp(groups, weights)
+    scale = torch.sqrt(torch.mean(st["p"] ** 2) + 1e-9)
+    want = st["p"] - lr * (scale * (out[..., 0] * torch.exp(out[..., 1] * exp_mult) * step_mult))
+    if wd > 0:
+        want = want - wd * lr * want
+
+    g, p, m, v, fr, fc, rf, cf = _cuda(st, "g", "p", "mom", "rms", "fac_r", "fac_c", "rf", "cf")
+    sm = torch.zeros(30, device="cuda")
+    velo_cuda_kernel.velo_kernel_simple(g, p, m, v, rf, cf, fr, fc, sm, *[w.cuda() for w in weights], lr, step_mult,
+                                        exp_mult, 1e-6, wd, dc, dr, vl)
+    assert max_err(p.cpu(), want, REL, ABS) <= 1.0
+    _check_moment(sm, groups)
+
+
+def test_large_tensor_and_argument_errors():
+    """A tensor that needs the grid-stride loop (more elements than 2048 blocks cover), and the
+    Python-side checks: wrong dtype / device / layout raise instead of launching."""
+    from pylo_amd.compat import velo_cuda_kernel
+
+    shape = (1500, 700)
+    gen = torch.Generator().manual_seed(14)
+    weights = [torch.randn(s, generator=gen) * sc for s, sc in
+               (((4, 30), 0.3), ((4,), 0.1), ((4, 4), 0.5), ((4,), 0.1), ((3, 4), 0.5), ((3,), 0.1))]
+    st = _state(shape, 4, O.factored_dims_velo)
+    dc, dr, vl = st["dims"]
+    groups = O.velo_feature_groups(st["p"], st["g"], st["mom"], st["rms"], st["fac_r"], st["fac_c"], st["rf"], st["cf"])
+    out = O.velo_element_mlp(groups, weights)
+    scale = torch.sqrt(torch.mean(st["p"] ** 2) + 1e-9)
+    want = st["p"] - 0.03 * (scale * (out[..., 0] * torch.exp(out[..., 1] * 0.001) * 0.001))
+    g, p, m, v, fr, fc, rf, cf = _cuda(st, "g", "p", "mom", "rms", "fac_r", "fac_c", "rf", "cf")
+    sm = torch.zeros(30, device="cuda")
+    ws = [w.cuda() for w in weights]
+    velo_cuda_kernel.velo_kernel_simple(g, p, m, v, rf, cf, fr, fc, sm, *ws, 0.03, 0.001, 0.001, 1e-6, 0.0, dc, dr, vl)
+    assert max_err(p.cpu(), want, REL, ABS) <= 1.0
+    _check_moment(sm, groups)
+    with pytest.raises(TypeError, match="float32"):
+        velo_cuda_kernel.velo_kernel_simple(g.double(), p, m, v, rf, cf, fr, fc, sm, *ws, 0.03, 0.001, 0.001, 1e-6,
+                                            0.0, dc, dr, vl)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        velo_cuda_kernel.velo_kernel_simple(g.t(), p, m, v, rf, cf, fr, fc, sm, *ws, 0.03, 0.001, 0.001, 1e-6,
+                                            0.0, dc, dr, vl)
+    with pytest.raises(RuntimeError, match="must live on"):
+        velo_cuda_kernel.velo_kernel_simple(g.cpu(), p, m, v, rf, cf, fr, fc, sm, *ws, 0.03, 0.001, 0.001, 1e-6,
+                                            0.0, dc, dr, vl)
+    with pytest.raises(RuntimeError, match="dc / dr"):
+        velo_cuda_kernel.velo_kernel_simple(g, p, m, v, rf, cf, fr, fc, sm, *ws, 0.03, 0.001, 0.001, 1e-6,
+                                            0.0, 1, 1, 0)

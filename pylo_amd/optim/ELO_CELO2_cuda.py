@@ -386,8 +386,11 @@ class ELO_CELO2_CUDA(Optimizer):
         if not keep and all(p.grad is not None for _, p, _a in tensors):
             index = {id(g): i for i, g in enumerate(self.param_groups)}
             # the cached rows point into the state tensors: hold them, and notice a cleared state
-            alive = [(self.state[p], k, t) for _, p, _a in tensors for k, t in self.state[p].items()
-                     if torch.is_tensor(t)]
+            # one (state, key, tensor) per parameter, its first state tensor: replacing a parameter's
+            # state replaces that one too, and a walk over every tensor costs milliseconds with
+            # thousands of parameters
+            alive = [(self.state[p],) + next(((k, t) for k, t in self.state[p].items() if torch.is_tensor(t)), (None, None))
+                     for _, p, _a in tensors]
             self._fast = dict(tensors=tensors, params=[p for _, p, _a in tensors], n_groups=len(self.param_groups),
                               n_state=len(self.state), alive=alive,
                               gidx=np.asarray([index[id(g)] for g, _p, _a in tensors], dtype=np.int64),

@@ -377,8 +377,11 @@ class VeLO_CUDA(Optimizer):
                 args[k] = v
             args["group"] = grp
             if not keep:
-                alive = [(self.state[p], k, t) for _, _, p in tensors for k, t in self.state[p].items()
-                         if torch.is_tensor(t)]
+                # one (state, key, tensor) per parameter, its first state tensor: replacing a parameter's
+                # state replaces that one too, and a walk over every tensor costs milliseconds with
+                # thousands of parameters
+                alive = [(self.state[p],) + next(((k, t) for k, t in self.state[p].items() if torch.is_tensor(t)), (None, None))
+                         for _, _, p in tensors]
                 self._fast = dict(key=self._plan_key, n_state=len(self.state), alive=alive,
                                   params=[p for _, _, p in tensors],
                                   gidx=np.asarray(grp, dtype=np.int64))

@@ -220,6 +220,7 @@ class Plan:
                                             float(step), stream), "adafac_step")
 
     def close(self):
+        self.__dict__.pop("_tables", None)     # views of pinned memory that dies with the plan
         if getattr(self, "_h", None):
             load().pylo_mi355_plan_destroy(self._h)
             self._h = None

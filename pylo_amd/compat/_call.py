@@ -49,6 +49,33 @@ def pointers(who: str, device: torch.device, **tensors) -> list:
     return out
 
 
+def check_sizes(who: str, p: torch.Tensor, dc: int, dr: int, vector_like: int, n_stat: int, sizes: dict,
+                weights: dict) -> None:
+    """Element counts the kernels rely on (they index without bounds checks): per-element arrays, the
+    three-decay accumulators, factor vectors with the dr / dc dim removed, `second_moment`, MLP arrays.
+    `sizes` maps a name to (tensor, kind), kind in {"n", "3n", "row", "col", "stat"}."""
+    n = p.numel()
+    if vector_like:
+        row = col = 3 * n
+    else:
+        if not (0 <= dc < p.dim() and 0 <= dr < p.dim()) or dc == dr:
+            raise RuntimeError(f"{who}: dc / dr are not two dims of the tensor")
+        row = 3 * n // max(p.shape[dr], 1)
+        col = 3 * n // max(p.shape[dc], 1)
+    want = {"n": n, "3n": 3 * n, "row": row, "col": col}
+    for name, (t, kind) in sizes.items():
+        if kind == "stat":
+            if t.numel() < n_stat:
+                raise RuntimeError(f"{who}: {name} needs at least {n_stat} elements")
+        elif kind == "col" and vector_like:
+            continue                      # not read for a vector-like tensor
+        elif t.numel() != want[kind] and n > 0:
+            raise RuntimeError(f"{who}: {name} has {t.numel()} elements, expected {want[kind]}")
+    for name, (t, count) in weights.items():
+        if t.numel() != count:
+            raise RuntimeError(f"{who}: {name} has {t.numel()} elements, expected {count}")
+
+
 def shape_args(p: torch.Tensor):
     arr = (C.c_int64 * max(p.dim(), 1))(*p.shape)
     return arr, p.dim()

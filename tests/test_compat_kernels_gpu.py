@@ -177,6 +177,12 @@ def test_large_tensor_and_argument_errors():
     with pytest.raises(RuntimeError, match="must live on"):
         velo_cuda_kernel.velo_kernel_simple(g.cpu(), p, m, v, rf, cf, fr, fc, sm, *ws, 0.03, 0.001, 0.001, 1e-6,
                                             0.0, dc, dr, vl)
+    with pytest.raises(RuntimeError, match="expected"):      # a momentum buffer of one decay instead of three
+        velo_cuda_kernel.velo_kernel_simple(g, p, m[0].contiguous(), v, rf, cf, fr, fc, sm, *ws, 0.03, 0.001, 0.001,
+                                            1e-6, 0.0, dc, dr, vl)
+    with pytest.raises(RuntimeError, match="at least 30"):
+        velo_cuda_kernel.velo_kernel_simple(g, p, m, v, rf, cf, fr, fc, sm[:10], *ws, 0.03, 0.001, 0.001, 1e-6,
+                                            0.0, dc, dr, vl)
     with pytest.raises(RuntimeError, match="dc / dr"):
         velo_cuda_kernel.velo_kernel_simple(g, p, m, v, rf, cf, fr, fc, sm, *ws, 0.03, 0.001, 0.001, 1e-6,
                                             0.0, 1, 1, 0)

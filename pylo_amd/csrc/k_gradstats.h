@@ -101,6 +101,38 @@ __device__ __forceinline__ void p0_flat(const TDesc& d, const float* g, int chun
   }
 }
 
+// Sums of g^2 of a tensor with more than two dims over one of its two factored dims, one block per
+// (chunk of 64 entries, slab of kNdX positions along the removed dim); used by k_p0_nd and, when no
+// global norm has to be known first, by the tail blocks of k_p0.  `lds` holds kWaves * 64 floats.
+__device__ __forceinline__ void p0_nd_block(const TDesc* __restrict__ descs, const PyloTensorArgs* __restrict__ dyn,
+                                            const Item it, float* __restrict__ part,
+                                            const Globals* __restrict__ gl, float* lds) {
+  static_assert(kV0aEnt == 64, "one lane per entry");
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  const int w = it.b;
+  const int e = threadIdx.x & 63, grp = threadIdx.x >> 6;
+  const int i = it.a * kV0aEnt + e;
+  const int X = pick(d.nd_size, w), sX = pick(d.nd_stride, w);
+  const float scale = a.clip_norm > 0.0f ? clip_scale(gl->gnorm, a.clip_norm) : 1.0f;
+  float s = 0.0f;
+  if (i < pick(d.len, w)) {
+    const long long base = (long long)(i / sX) * X * sX + (i % sX);
+    const int x0 = it.c * kNdX + grp * (kNdX / kWaves);
+    const int x1 = min(X, x0 + kNdX / kWaves);
+    for (int x = x0; x < x1; ++x) {
+      const float g = cond_grad(*(const gfloat*)(a.grad + base + (long long)x * sX), scale, a.clip_val, d.nan0);
+      s = fmaf(g, g, s);
+    }
+  }
+  lds[grp * kV0aEnt + e] = s;
+  __syncthreads();
+  if (grp == 0 && i < pick(d.len, w))
+    part[pick(d.part_off, w) + (size_t)it.c * pick(d.len, w) + i] =
+        ((lds[e] + lds[kV0aEnt + e]) + lds[2 * kV0aEnt + e]) + lds[3 * kV0aEnt + e];
+}
+
 // pass 0: tensors with clip_norm > 0 are summed raw (the scale factors out of g^2) and flag
 //         elements beyond the clamp; tensors without global-norm clipping are clamped directly.
 // pass 1: only if the flag was raised: redo clip_norm > 0 tensors with scale and clamp applied.
@@ -108,11 +140,18 @@ __global__ __launch_bounds__(kThreads) void k_p0(const TDesc* __restrict__ descs
                                                  const PyloTensorArgs* __restrict__ dyn,
                                                  const Item* __restrict__ items, float* __restrict__ part,
                                                  double* __restrict__ gsq_part, int* __restrict__ flag_part,
-                                                 const Globals* __restrict__ gl, int pass) {
+                                                 const Globals* __restrict__ gl, int pass,
+                                                 const Item* __restrict__ nd_items, int n_main) {
   __shared__ float lds_col[kWaves * 256];
   __shared__ float lds_row[kWaves * (kP0Rows / 16) * 16];
   __shared__ float lds_red[kWaves];
   __shared__ int lds_flag[kWaves];
+  // blocks past the main items: the N-D tensors' sums, when the launcher appended them (it does when
+  // no tensor is clipped by the global norm, which they would have to wait for)
+  if ((int)blockIdx.x >= n_main) {
+    p0_nd_block(descs, dyn, nd_items[blockIdx.x - n_main], part, gl, lds_col);
+    return;
+  }
   const Item it = items[blockIdx.x];
   const TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
@@ -189,30 +228,8 @@ __global__ __launch_bounds__(kThreads) void k_p0_nd(const TDesc* __restrict__ de
                                                     const PyloTensorArgs* __restrict__ dyn,
                                                     const Item* __restrict__ items, float* __restrict__ part,
                                                     const Globals* __restrict__ gl) {
-  __shared__ float lds[kWaves][kV0aEnt];
-  const Item it = items[blockIdx.x];
-  const TDesc d = descs[it.tensor];
-  const PyloTensorArgs a = dyn[it.tensor];
-  if (a.grad == nullptr) return;
-  const int w = it.b;
-  const int e = threadIdx.x & 63, grp = threadIdx.x >> 6;
-  const int i = it.a * kV0aEnt + e;
-  const int X = pick(d.nd_size, w), sX = pick(d.nd_stride, w);
-  const float scale = a.clip_norm > 0.0f ? clip_scale(gl->gnorm, a.clip_norm) : 1.0f;
-  float s = 0.0f;
-  if (i < pick(d.len, w)) {
-    const long long base = (long long)(i / sX) * X * sX + (i % sX);
-    const int x0 = it.c * kNdX + grp * (kNdX / kWaves);
-    const int x1 = min(X, x0 + kNdX / kWaves);
-    for (int x = x0; x < x1; ++x) {
-      const float g = cond_grad(*(const gfloat*)(a.grad + base + (long long)x * sX), scale, a.clip_val, d.nan0);
-      s = fmaf(g, g, s);
-    }
-  }
-  lds[grp][e] = s;
-  __syncthreads();
-  if (grp == 0 && i < pick(d.len, w))
-    part[pick(d.part_off, w) + (size_t)it.c * pick(d.len, w) + i] = ((lds[0][e] + lds[1][e]) + lds[2][e]) + lds[3][e];
+  __shared__ float lds[kWaves * kV0aEnt];
+  p0_nd_block(descs, dyn, items[blockIdx.x], part, gl, lds);
 }
 
 // =============================================================================================

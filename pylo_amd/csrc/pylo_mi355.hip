@@ -651,12 +651,15 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
 
   const bool exact_pass = exact_pass_possible(P, args);
   HIP_TRY(mark());
-  if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0);
+  if (n_p0 > 0)
+    hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0,
+                       (const Item*)nullptr, n_p0);
   HIP_TRY(mark());
   hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl, exact_pass ? 1 : 0);
   HIP_TRY(mark());
   if (n_p0 > 0 && exact_pass)
-    hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1);
+    hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1,
+                       (const Item*)nullptr, n_p0);
   if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part, gl);
   HIP_TRY(mark());
   if (n_v0a > 0)
@@ -774,9 +777,11 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
 
   HIP_TRY(mark());
   // clip_norm is 0 for VeLO tensors: k_p0 clamps directly; its norm / flag outputs are not used
-  if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0);
+  // no global norm to wait for: the N-D tensors' sums ride in the tail blocks of the same launch
+  if (n_p0 + n_nd > 0)
+    hipLaunchKernelGGL(k_p0, dim3(n_p0 + n_nd), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0,
+                       nd_items, n_p0);
   HIP_TRY(mark());
-  if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part, gl);
   HIP_TRY(mark());
   if (n_v0a > 0)
     hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kV0aThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
@@ -864,15 +869,20 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   for (int t = 0; t < T; ++t) clips = clips || (args[t].grad != nullptr && args[t].clip_norm > 0.0f);
   if (clips && !L.global_norm) return fail("adafac_step: clip_norm > 0 needs a plan built with PYLO_F_GLOBAL_NORM");
   HIP_TRY(mark());
-  if (n_p0 > 0) hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0);
+  // without global-norm clipping the N-D tensors' sums ride in the tail blocks of the first launch
+  const int n_tail = clips ? 0 : n_nd;
+  if (n_p0 + n_tail > 0)
+    hipLaunchKernelGGL(k_p0, dim3(n_p0 + n_tail), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0,
+                       nd_items, n_p0);
   if (clips) {
     const bool exact_pass = exact_pass_possible(P, args);
     hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl, exact_pass ? 1 : 0);
     if (n_p0 > 0 && exact_pass)
-      hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1);
+      hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1,
+                         (const Item*)nullptr, n_p0);
   }
   HIP_TRY(mark());
-  if (n_nd > 0) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part, gl);
+  if (n_nd > 0 && clips) hipLaunchKernelGGL(k_p0_nd, dim3(n_nd), dim3(kThreads), 0, s, descs, dyn, nd_items, part, gl);
   HIP_TRY(mark());
   if (n_v0a > 0)
     hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kV0aThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);

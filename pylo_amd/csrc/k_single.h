@@ -127,31 +127,20 @@ __global__ __launch_bounds__(kSingleThreads) void k_single_moment(SingleArgs a) 
   }
 }
 
-// Normalise by rsqrt(second_moment / n + eps), MLP, output.  The weights are staged in LDS once per
-// block with the channel normalisers folded into the first layer ([k][j] layout, read as broadcasts);
-// AdafacLO's eleven time features are the same for every element and go into the first bias.
+// Normalise by rsqrt(second_moment / n + eps), MLP, output.  The weights are the same for every lane:
+// they are read through the scalar cache into SGPRs where they are used (the pointer is laundered once
+// per element so that the loads stay inside the loop instead of being hoisted into a register file they
+// do not fit), which leaves the vector pipe with the multiply-adds only.  AdafacLO's eleven time features
+// are the same for every element and go into the first bias, once per block.
 template <int F>
 __global__ __launch_bounds__(kSingleThreads) void k_single_apply(SingleArgs a) {
   using Fm = Fam<F>;
   constexpr int NS = Fm::NSTAT, NIN = Fm::NIN, H = Fm::H, NO = Fm::NOUT;
   __shared__ float s_norm[NS];
-  __shared__ float w1[NS * H], w2[H * H], w3[H * NO], b1[H], b2[H], b3[NO];
+  __shared__ float b1[H];
   const int tid = threadIdx.x;
   const float nf = (float)a.n;
   if (tid < NS) s_norm[tid] = rsq(a.second_moment[tid] / nf + (F == kFamCelo2 ? 1e-9f : 1e-5f));
-  __syncthreads();
-  for (int i = tid; i < NS * H; i += kSingleThreads) {
-    const int k = i / H, j = i % H;
-    w1[i] = (Fm::in_major ? a.w_in[k * H + j] : a.w_in[j * NIN + k]) * s_norm[k];
-  }
-  for (int i = tid; i < H * H; i += kSingleThreads) {
-    const int k = i / H, j = i % H;
-    w2[i] = Fm::in_major ? a.w_h[k * H + j] : a.w_h[j * H + k];
-  }
-  for (int i = tid; i < H * NO; i += kSingleThreads) {
-    const int k = i / NO, j = i % NO;
-    w3[i] = Fm::in_major ? a.w_out[k * NO + j] : a.w_out[j * H + k];
-  }
   if (tid < H) {
     float b = a.b_in[tid];
     if constexpr (F == kFamLo) {   // tanh(step / ts - 1), learned_optimizer.cu:27-32
@@ -160,43 +149,73 @@ __global__ __launch_bounds__(kSingleThreads) void k_single_apply(SingleArgs a) {
       for (int q = 0; q < 11; ++q) b = fmaf(tanhf(a.step / ts[q] - 1.0f), a.w_in[tid * NIN + NS + q], b);
     }
     b1[tid] = b;
-    b2[tid] = a.b_h[tid];
   }
-  if (tid < NO) b3[tid] = a.b_out[tid];
   __syncthreads();
   const float pscale = F == kFamVelo ? sqrtf(a.second_moment[2] / nf + 1e-9f) : 1.0f;   // channel 2 is p
 
   for (long long i = (long long)blockIdx.x * kSingleThreads + tid; i < a.n; i += (long long)gridDim.x * kSingleThreads) {
     float f[NS];
     single_features<F>(a, (int)i, f);
+    const float p_old = f[F == kFamLo ? 1 : 2];
+#pragma unroll
+    for (int k = 0; k < NS; ++k) f[k] *= s_norm[k];
+    const cfloat* w1 = launder(a.w_in);
+    const cfloat* w2 = launder(a.w_h);
+    const cfloat* w3 = launder(a.w_out);
+    const cfloat* bh = launder(a.b_h);
+    const cfloat* bo = launder(a.b_out);
     float h0[H], h1[H], out[NO];
+    if constexpr (Fm::in_major) {
 #pragma unroll
-    for (int j = 0; j < H; ++j) h0[j] = b1[j];
+      for (int j = 0; j < H; ++j) h0[j] = b1[j];
 #pragma unroll
-    for (int k = 0; k < NS; ++k)
+      for (int k = 0; k < NS; ++k)
 #pragma unroll
-      for (int j = 0; j < H; ++j) h0[j] = fmaf(f[k], w1[k * H + j], h0[j]);
+        for (int j = 0; j < H; ++j) h0[j] = fmaf(f[k], w1[k * H + j], h0[j]);
 #pragma unroll
-    for (int j = 0; j < H; ++j) { h0[j] = fmaxf(h0[j], 0.0f); h1[j] = b2[j]; }
+      for (int j = 0; j < H; ++j) { h0[j] = fmaxf(h0[j], 0.0f); h1[j] = bh[j]; }
 #pragma unroll
-    for (int k = 0; k < H; ++k)
+      for (int k = 0; k < H; ++k)
 #pragma unroll
-      for (int j = 0; j < H; ++j) h1[j] = fmaf(h0[k], w2[k * H + j], h1[j]);
+        for (int j = 0; j < H; ++j) h1[j] = fmaf(h0[k], w2[k * H + j], h1[j]);
 #pragma unroll
-    for (int j = 0; j < NO; ++j) out[j] = b3[j];
+      for (int j = 0; j < NO; ++j) out[j] = bo[j];
 #pragma unroll
-    for (int k = 0; k < H; ++k) {
-      const float hk = fmaxf(h1[k], 0.0f);
+      for (int k = 0; k < H; ++k) {
+        const float hk = fmaxf(h1[k], 0.0f);
 #pragma unroll
-      for (int j = 0; j < NO; ++j) out[j] = fmaf(hk, w3[k * NO + j], out[j]);
+        for (int j = 0; j < NO; ++j) out[j] = fmaf(hk, w3[k * NO + j], out[j]);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < H; ++j) {
+        float acc = b1[j];
+#pragma unroll
+        for (int k = 0; k < NS; ++k) acc = fmaf(f[k], w1[j * NIN + k], acc);
+        h0[j] = fmaxf(acc, 0.0f);
+      }
+#pragma unroll
+      for (int j = 0; j < H; ++j) {
+        float acc = bh[j];
+#pragma unroll
+        for (int k = 0; k < H; ++k) acc = fmaf(h0[k], w2[j * H + k], acc);
+        h1[j] = fmaxf(acc, 0.0f);
+      }
+#pragma unroll
+      for (int j = 0; j < NO; ++j) {
+        float acc = bo[j];
+#pragma unroll
+        for (int k = 0; k < H; ++k) acc = fmaf(h1[k], w3[j * H + k], acc);
+        out[j] = acc;
+      }
     }
     const float step = out[0] * expf(out[1] * a.exp_mult);
     if constexpr (F == kFamCelo2) {
       a.step_out[i] = step;                                   // celo2_kernel.cu:280; p is left untouched
     } else if constexpr (F == kFamLo) {
-      a.p[i] = f[1] - a.lr * (step * a.step_mult);            // learned_optimizer.cu:296-299
+      a.p[i] = p_old - a.lr * (step * a.step_mult);           // learned_optimizer.cu:296-299
     } else {
-      float pn = f[2] - a.lr * (pscale * step * a.step_mult); // velo_kernel.cu:352-362
+      float pn = p_old - a.lr * (pscale * step * a.step_mult); // velo_kernel.cu:352-362
       if (a.weight_decay > 0.0f) pn = pn - a.weight_decay * a.lr * pn;
       a.p[i] = pn;
     }

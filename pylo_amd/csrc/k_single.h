@@ -20,6 +20,28 @@ template <> struct Fam<kFamLo> { static constexpr int NSTAT = 28, NIN = 39, H = 
 // VeLO: 30 channels, 30 -> 4 -> 4 -> 3, (out, in)                                   (velo_kernel.cu:10-13)
 template <> struct Fam<kFamVelo> { static constexpr int NSTAT = 30, NIN = 30, H = 4, NOUT = 3; static constexpr bool in_major = false; };
 
+// Division of an element index (< 2^31) by a divisor fixed for the launch: q = (n * m) >> (31 + s) with
+// s = ceil(log2 d), m = floor(2^(31+s) / d) + 1 < 2^32, exact for every n < 2^31 (the error of m is at
+// most d / 2^(31+s) per unit of n).  s < 0 marks d == 1.  Four of these per element replace four integer
+// divisions of some twenty instructions each.
+struct FastDiv {
+  unsigned m;
+  int s;
+  unsigned d;
+};
+inline FastDiv make_fastdiv(unsigned d) {
+  FastDiv f{0u, -1, d};
+  if (d <= 1) return f;
+  int s = 0;
+  while ((1ull << s) < d) ++s;
+  f.s = s;
+  f.m = (unsigned)((1ull << (31 + s)) / d + 1);
+  return f;
+}
+__device__ __forceinline__ unsigned fd_div(unsigned n, const FastDiv& f) {
+  return f.s < 0 ? n : (__umulhi(n, f.m) >> (f.s - 1));
+}
+
 struct SingleArgs {
   const float *g, *m, *v, *fac_r, *fac_c, *row_factor, *col_factor;
   float* p;              // read by every family; updated in place by the lo / velo families
@@ -27,6 +49,8 @@ struct SingleArgs {
   const float *w_in, *b_in, *w_h, *b_h, *w_out, *b_out;
   float* step_out;       // celo2 only
   int n, num_rows, num_cols, row_stride, col_stride, vector_like;
+  int stride_r, stride_c;                        // decay strides of the row / column vectors
+  FastDiv div_rblock, div_rstride, div_cblock, div_cstride;   // num_rows*row_stride, row_stride, num_cols*col_stride, col_stride
   float lr, step_mult, exp_mult, epsilon, step, weight_decay;
 };
 
@@ -36,7 +60,8 @@ constexpr int kSingleMaxBlocks = 2048;
 // Offsets of element idx into the row vectors (row_factor, fac_r: the tensor's shape with the largest
 // dim dr removed) and the column vectors (col_factor, fac_c: dim dc removed), and their decay strides.
 // For tensors of up to two dims this is the reference's `col_idx + k * num_cols` / `row_idx + k * num_rows`
-// (celo2_kernel.cu:67-84, learned_optimizer.cu:55-72); with more dims it is velo_kernel.cu:109-120.
+// (celo2_kernel.cu:67-84, learned_optimizer.cu:55-72); with more dims it is velo_kernel.cu:109-120:
+//   ofs_row = (idx / (num_rows * row_stride)) * row_stride + idx % row_stride, likewise for columns.
 struct FacOfs { int r, c, stride_r, stride_c; };
 __device__ __forceinline__ FacOfs fac_offsets(const SingleArgs& a, int idx) {
   FacOfs o;
@@ -44,10 +69,11 @@ __device__ __forceinline__ FacOfs fac_offsets(const SingleArgs& a, int idx) {
     o.r = o.c = idx;
     o.stride_r = o.stride_c = a.n;
   } else {
-    o.stride_r = a.n / a.num_rows;
-    o.stride_c = a.n / a.num_cols;
-    o.r = (idx / (a.num_rows * a.row_stride)) * a.row_stride + idx % a.row_stride;
-    o.c = (idx / (a.num_cols * a.col_stride)) * a.col_stride + idx % a.col_stride;
+    const unsigned u = (unsigned)idx;
+    o.stride_r = a.stride_r;
+    o.stride_c = a.stride_c;
+    o.r = (int)(fd_div(u, a.div_rblock) * (unsigned)a.row_stride + (u - fd_div(u, a.div_rstride) * (unsigned)a.row_stride));
+    o.c = (int)(fd_div(u, a.div_cblock) * (unsigned)a.col_stride + (u - fd_div(u, a.div_cstride) * (unsigned)a.col_stride));
   }
   return o;
 }

@@ -953,6 +953,14 @@ int single_geometry(const char* who, const int64_t* shape, int ndim, int dc, int
   a.num_cols = (int)shape[dc];
   a.row_stride = stride(dr);
   a.col_stride = stride(dc);
+  if (a.n > 0) {   // then every dim is at least 1
+    a.stride_r = a.n / a.num_rows;
+    a.stride_c = a.n / a.num_cols;
+    a.div_rblock = make_fastdiv((unsigned)a.num_rows * (unsigned)a.row_stride);
+    a.div_rstride = make_fastdiv((unsigned)a.row_stride);
+    a.div_cblock = make_fastdiv((unsigned)a.num_cols * (unsigned)a.col_stride);
+    a.div_cstride = make_fastdiv((unsigned)a.col_stride);
+  }
   return 0;
 }
 

@@ -357,19 +357,39 @@ __device__ __forceinline__ size_t term_index(const TDesc& d, int which, int j, i
 // fv: the entry's three accumulator values (fac[k * len + i]), loaded by the caller.
 __device__ __forceinline__ void vector_entry(const TDesc& d, bool is_r, const float* fac, int len, int i,
                                              const float (&fv)[3], const float (&rcm3)[3], const float (&s0)[3],
-                                             const float (&s1)[3], float (&fct)[3], float (&x0)[3], float (&x1)[3]) {
+                                             const float (&s1)[3], float (&fct)[3], float (&x0)[3], float (&x1)[3],
+                                             const float* rcm_slices = nullptr, int slice = 0) {
+  float rcm[3] = {rcm3[0], rcm3[1], rcm3[2]};
+  if (is_r && d.mode == kModeFacND) {  // mean over the dc axis of this entry's slice of fac_r
+    if (rcm_slices != nullptr) {       // the block has it in its per-slice table
+#pragma unroll
+      for (int k = 0; k < 3; ++k) rcm[k] = rcm_slices[k * kRcmSlots + slice];
+    } else {
+      const int sz = d.rcm_size, st = d.rcm_stride;
+      const int base = (i / (sz * st)) * (sz * st) + i % st;
+      double s[3] = {0.0, 0.0, 0.0};
+      // sixteen positions of all three decays are requested before any is added (addresses clamped,
+      // values past the end dropped afterwards, so that the loads stay unconditional)
+      for (int xb = 0; xb < sz; xb += 16) {
+        float v[3][16];
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+#pragma unroll
+          for (int q = 0; q < 16; ++q)
+            v[k][q] = *(const gfloat*)(fac + (size_t)k * len + base + (size_t)min(xb + q, sz - 1) * st);
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+#pragma unroll
+          for (int q = 0; q < 16; ++q) s[k] += xb + q < sz ? (double)v[k][q] : 0.0;
+      }
+#pragma unroll
+      for (int k = 0; k < 3; ++k) rcm[k] = (float)(s[k] / (double)sz);
+    }
+  }
 #pragma unroll
   for (int k = 0; k < 3; ++k) {
     const float f = fv[k];
-    float rcm = rcm3[k];
-    if (is_r && d.mode == kModeFacND) {  // mean over the dc axis of this entry's slice of fac_r
-      const int sz = d.rcm_size, st = d.rcm_stride;
-      const int base = (i / (sz * st)) * (sz * st) + i % st;
-      double s = 0.0;
-      for (int x = 0; x < sz; ++x) s += (double)fac[(size_t)k * len + base + x * st];
-      rcm = (float)(s / (double)sz);
-    }
-    fct[k] = is_r ? rsq(fmaxf(f / (rcm + 1e-9f), 1e-9f)) : rsq(fmaxf(f, 1e-9f));
+    fct[k] = is_r ? rsq(fmaxf(f / (rcm[k] + 1e-9f), 1e-9f)) : rsq(fmaxf(f, 1e-9f));
     x0[k] = f * s0[k];
     x1[k] = rsq(f + 1e-8f) * s1[k];
   }
@@ -462,8 +482,18 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
       const int vecI = pair / kNV0, slot = pair % kNV0;
       double s = 0.0;
       const int nb = vecI ? d.v0a_n[1] : d.v0a_n[0], first = vecI ? d.v0a_first[1] : d.v0a_first[0];
-#pragma unroll 8
-      for (int b = gI; b < nb; b += G) s += v0part[(size_t)(first + b) * kNV0 + slot];
+      // up to 32 partial rows per thread requested at once (same order of addition as a plain loop): a
+      // vector of tens of thousands of entries has hundreds of rows, and every batch is a memory round trip
+      for (int b0 = gI; b0 < nb; b0 += 32 * G) {
+        double v[32];
+#pragma unroll
+        for (int q = 0; q < 32; ++q) {
+          const int b = b0 + q * G;
+          v[q] = b < nb ? v0part[(size_t)(first + b) * kNV0 + slot] : 0.0;
+        }
+#pragma unroll
+        for (int q = 0; q < 32; ++q) s += v[q];
+      }
       red[gI][pair] = s;
     }
     __syncthreads();
@@ -502,12 +532,68 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
     s0[k] = rsq(norm_eps + (float)(own[k * 3 + 1] * inv_own));
     s1[k] = rsq(norm_eps + (float)(own[k * 3 + 2] * inv_own));
   }
+  // N-D row vector: row_col_mean is a mean over the dc axis inside the vector, one value per slice
+  // (o, r) of its [o][dc][r] view.  The slices this block's entries belong to are reduced once, here,
+  // into a table in LDS (a thread per slice while the axis is short, a wave per slice otherwise; fixed
+  // order either way) instead of once per entry, which costs the axis length in loads per entry.
+  __shared__ float rcm_tab[3 * kRcmSlots];
+  const float* rcm_slices = nullptr;
+  int o_first = 0;
+  if (is_r && d.mode == kModeFacND) {
+    const int sz = d.rcm_size, st = d.rcm_stride, blk = sz * st;
+    const int i0 = it.a * kV0bEnt;
+    o_first = i0 / blk;
+    const int count = ((i_end - 1) / blk - o_first + 1) * st;
+    if (count <= kRcmSlots) {
+      const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+      if (sz < 64) {
+        for (int sl = threadIdx.x; sl < count; sl += kThreads) {
+          const int base = (o_first + sl / st) * blk + sl % st;
+          double sk[3] = {0.0, 0.0, 0.0};
+          for (int xb = 0; xb < sz; xb += 16) {
+            float v[3][16];
+#pragma unroll
+            for (int k = 0; k < 3; ++k)
+#pragma unroll
+              for (int q = 0; q < 16; ++q)
+                v[k][q] = *(const gfloat*)(fac + (size_t)k * len + base + (size_t)min(xb + q, sz - 1) * st);
+#pragma unroll
+            for (int k = 0; k < 3; ++k)
+#pragma unroll
+              for (int q = 0; q < 16; ++q) sk[k] += xb + q < sz ? (double)v[k][q] : 0.0;
+          }
+#pragma unroll
+          for (int k = 0; k < 3; ++k) rcm_tab[k * kRcmSlots + sl] = (float)(sk[k] / (double)sz);
+        }
+      } else {
+        for (int sl = wave; sl < count; sl += kWaves) {
+          const int base = (o_first + sl / st) * blk + sl % st;
+          double sk[3] = {0.0, 0.0, 0.0};
+          for (int x = lane; x < sz; x += 64)
+#pragma unroll
+            for (int k = 0; k < 3; ++k) sk[k] += (double)*(const gfloat*)(fac + (size_t)k * len + base + (size_t)x * st);
+#pragma unroll
+          for (int k = 0; k < 3; ++k) {
+            const double t = wave_sum(sk[k]);
+            if (lane == 0) rcm_tab[k * kRcmSlots + sl] = (float)(t / (double)sz);
+          }
+        }
+      }
+      __syncthreads();
+      rcm_slices = rcm_tab;
+    }
+  }
 #pragma unroll
   for (int q = 0; q < kPer; ++q) {
     const int i = it.a * kV0bEnt + q * kThreads + threadIdx.x;
     if (i >= i_end) break;
     float fct[3], x0[3], x1[3];
-    vector_entry(d, is_r, fac, len, i, fpre[q], rcm3, s0, s1, fct, x0, x1);
+    int slice = 0;
+    if (rcm_slices != nullptr) {
+      const int st = d.rcm_stride, blk = d.rcm_size * st;
+      slice = (i / blk - o_first) * st + i % st;
+    }
+    vector_entry(d, is_r, fac, len, i, fpre[q], rcm3, s0, s1, fct, x0, x1, rcm_slices, slice);
     if (d.mode == kModeFac2D) {  // [index][4]: one 16-byte store
       *(float4*)(fac_tab + fac_index(d, which, 0, i)) = make_float4(fct[0], fct[1], fct[2], 0.0f);
     } else {

@@ -25,6 +25,7 @@ constexpr int kV0bEnt = 1024;   // vector entries per k_v0b block
 constexpr int kNV0 = 9;         // partial sums per k_v0a block
 constexpr int kV0aThreads = 256;   // groups of 64 lanes share the partial rows of 64 entries
 constexpr int kFoldThreads = 1024;
+constexpr int kRcmSlots = 1024; // slices of an N-D row vector whose row_col_mean one k_v0b block tabulates
 constexpr int kNdX = 64;        // elements of the summed dim one k_p0_nd block covers (one partial row)
 
 // Per-element channels, as indices into the reference's 30-channel order

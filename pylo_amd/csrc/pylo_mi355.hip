@@ -132,16 +132,32 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     } else {
       d.mode = !can_factor ? kModeVec : (s.ndim == 2 ? kModeFac2D : kModeFacND);
     }
+    // Geometry is laid out over the dims that matter: dims of size 1 other than the two factored ones
+    // change neither strides nor sums, so a (O, I, 1, 1) convolution kernel or a (1, 1, C) token is a
+    // plain 2-D tensor for the kernels (vectorised loads, column-resident walk).  Not for CELO2, whose
+    // normalisers run over slices of the last two dims as given.
+    PyloTensorShape e = s;
+    int edc = dc, edr = dr;
+    if (can_factor && kind != PYLO_KIND_CELO2 && n > 0) {
+      e.ndim = 0;
+      for (int i = 0; i < s.ndim; ++i) {
+        if (s.shape[i] == 1 && i != dc && i != dr) continue;
+        if (i == dc) edc = e.ndim;
+        if (i == dr) edr = e.ndim;
+        e.shape[e.ndim++] = s.shape[i];
+      }
+      d.mode = e.ndim == 2 ? kModeFac2D : kModeFacND;
+    }
     if (d.mode == kModeFlat || d.mode == kModeVec) {
       d.vec = (n % 4 == 0) ? 4 : 1;
     } else {
       L.dc[t] = dc;
       L.dr[t] = dr;
       if (d.mode == kModeFac2D) {
-        d.R0 = (int)s.shape[0];
-        d.C0 = (int)s.shape[1];
+        d.R0 = (int)e.shape[0];
+        d.C0 = (int)e.shape[1];
         d.vec = (d.C0 % 4 == 0) ? 4 : 1;
-        d.vec0_is_r = (dr == 1) ? 1 : 0;  // vector 0 (indexed by dim 0) results from summing over dim 1
+        d.vec0_is_r = (edr == 1) ? 1 : 0;  // vector 0 (indexed by dim 0) results from summing over dim 1
         d.len[0] = d.R0; d.len[1] = d.C0;
         d.sumlen[0] = d.C0; d.sumlen[1] = d.R0;
         d.n_strips = (d.R0 + kP0Rows - 1) / kP0Rows;
@@ -150,11 +166,11 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       } else {
         d.vec = 1;
         d.vec0_is_r = 1;
-        const int rem[2] = {dr, dc};  // the dim each vector lost
+        const int rem[2] = {edr, edc};  // the dim each vector lost
         for (int w = 0; w < 2; ++w) {
           long long stride = 1;
-          for (int i = rem[w] + 1; i < s.ndim; ++i) stride *= s.shape[i];
-          d.nd_size[w] = (int)s.shape[rem[w]];
+          for (int i = rem[w] + 1; i < e.ndim; ++i) stride *= e.shape[i];
+          d.nd_size[w] = (int)e.shape[rem[w]];
           d.nd_stride[w] = (int)stride;
           d.len[w] = d.nd_size[w] > 0 ? (int)(n / d.nd_size[w]) : 0;
           d.sumlen[w] = d.nd_size[w];
@@ -162,7 +178,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
         }
         // the dc axis as it sits inside the row vector (the tensor without dim dr)
         d.rcm_size = d.nd_size[1];
-        d.rcm_stride = dc > dr ? d.nd_stride[1] : d.nd_stride[1] / std::max(d.nd_size[0], 1);
+        d.rcm_stride = edc > edr ? d.nd_stride[1] : d.nd_stride[1] / std::max(d.nd_size[0], 1);
       }
       for (int w = 0; w < 2; ++w) {
         d.pitch[w] = (int)round4(d.len[w]);

@@ -20,28 +20,6 @@ template <> struct Fam<kFamLo> { static constexpr int NSTAT = 28, NIN = 39, H = 
 // VeLO: 30 channels, 30 -> 4 -> 4 -> 3, (out, in)                                   (velo_kernel.cu:10-13)
 template <> struct Fam<kFamVelo> { static constexpr int NSTAT = 30, NIN = 30, H = 4, NOUT = 3; static constexpr bool in_major = false; };
 
-// Division of an element index (< 2^31) by a divisor fixed for the launch: q = (n * m) >> (31 + s) with
-// s = ceil(log2 d), m = floor(2^(31+s) / d) + 1 < 2^32, exact for every n < 2^31 (the error of m is at
-// most d / 2^(31+s) per unit of n).  s < 0 marks d == 1.  Four of these per element replace four integer
-// divisions of some twenty instructions each.
-struct FastDiv {
-  unsigned m;
-  int s;
-  unsigned d;
-};
-inline FastDiv make_fastdiv(unsigned d) {
-  FastDiv f{0u, -1, d};
-  if (d <= 1) return f;
-  int s = 0;
-  while ((1ull << s) < d) ++s;
-  f.s = s;
-  f.m = (unsigned)((1ull << (31 + s)) / d + 1);
-  return f;
-}
-__device__ __forceinline__ unsigned fd_div(unsigned n, const FastDiv& f) {
-  return f.s < 0 ? n : (__umulhi(n, f.m) >> (f.s - 1));
-}
-
 struct SingleArgs {
   const float *g, *m, *v, *fac_r, *fac_c, *row_factor, *col_factor;
   float* p;              // read by every family; updated in place by the lo / velo families

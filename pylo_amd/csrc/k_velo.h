@@ -43,10 +43,9 @@ __device__ __forceinline__ void lo_load(const TDesc& d, const PyloTensorArgs& a,
     x.m[0][2] = *(const gfloat*)(a.mom + 2 * n + idx);
     x.rms[0] = *(const gfloat*)(a.rms + idx);
     const unsigned u = (unsigned)idx;
-    const unsigned s0 = (unsigned)d.nd_stride[0], z0 = (unsigned)d.nd_size[0] * s0;
-    const unsigned s1 = (unsigned)d.nd_stride[1], z1 = (unsigned)d.nd_size[1] * s1;
-    x.i0 = (int)((u / z0) * s0 + u % s0);
-    x.i1 = (int)((u / z1) * s1 + u % s1);
+    const unsigned s0 = (unsigned)d.nd_stride[0], s1 = (unsigned)d.nd_stride[1];
+    x.i0 = (int)(fd_div(u, d.nd_div_blk[0]) * s0 + (u - fd_div(u, d.nd_div_st[0]) * s0));
+    x.i1 = (int)(fd_div(u, d.nd_div_blk[1]) * s1 + (u - fd_div(u, d.nd_div_st[1]) * s1));
 #pragma unroll
     for (int k = 0; k < 3; ++k)
       x.rfcf[0][k] = fac_tab[d.fac_off[0] + (size_t)k * d.pitch[0] + x.i0] *

@@ -47,6 +47,28 @@ enum : int { kModeFlat = 0, kModeFac2D = 1, kModeFacND = 2, kModeVec = 3 };
 // A factored tensor owns two statistics vectors.  2-D: vector 0 is indexed by the dim-0
 // coordinate (sums over dim 1), vector 1 by the dim-1 coordinate.  N-D: vector 0 is the tensor
 // with the largest dim removed (the reference's fac_vec_row), vector 1 with the 2nd-largest removed.
+// Division of an element index (< 2^31) by a divisor fixed for the launch or the plan: q = (n * m) >> (31 + s) with
+// s = ceil(log2 d), m = floor(2^(31+s) / d) + 1 < 2^32, exact for every n < 2^31 (the error of m is at
+// most d / 2^(31+s) per unit of n).  s < 0 marks d == 1.  Four of these per element replace four integer
+// divisions of some twenty instructions each.
+struct FastDiv {
+  unsigned m;
+  int s;
+  unsigned d;
+};
+__host__ inline FastDiv make_fastdiv(unsigned d) {
+  FastDiv f{0u, -1, d};
+  if (d <= 1) return f;
+  int s = 0;
+  while ((1ull << s) < d) ++s;
+  f.s = s;
+  f.m = (unsigned)((1ull << (31 + s)) / d + 1);
+  return f;
+}
+__device__ __forceinline__ unsigned fd_div(unsigned n, const FastDiv& f) {
+  return f.s < 0 ? n : (__umulhi(n, f.m) >> (f.s - 1));
+}
+
 struct TDesc {
   long long n;
   int mode;
@@ -59,6 +81,7 @@ struct TDesc {
   int pitch[2];     // row pitch of the SoA tables of vector 0 / 1 (len rounded up to 4); 2-D tensors use [index][k] tables
   int nd_size[2];   // N-D: size and stride of the dim removed from vector 0 / 1;
   int nd_stride[2]; //      entry = (idx / (size*stride)) * stride + idx % stride
+  FastDiv nd_div_blk[2], nd_div_st[2];  // the two divisors of that formula per vector, as multiply-and-shift
   int rcm_size;     // N-D: size of the 2nd-largest dim and its stride inside the row vector; row_col_mean
   int rcm_stride;   //      is the mean over that axis, one value per slice (2-D: one value per tensor)
   int n_strips, n_colblk;

@@ -172,6 +172,8 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
           for (int i = rem[w] + 1; i < e.ndim; ++i) stride *= e.shape[i];
           d.nd_size[w] = (int)e.shape[rem[w]];
           d.nd_stride[w] = (int)stride;
+          d.nd_div_blk[w] = make_fastdiv((unsigned)std::max<long long>(e.shape[rem[w]] * stride, 1));
+          d.nd_div_st[w] = make_fastdiv((unsigned)std::max<long long>(stride, 1));
           d.len[w] = d.nd_size[w] > 0 ? (int)(n / d.nd_size[w]) : 0;
           d.sumlen[w] = d.nd_size[w];
           d.npart[w] = std::max(1, (d.nd_size[w] + kNdX - 1) / kNdX);

@@ -84,14 +84,37 @@ __device__ __forceinline__ void lo_terms(const TDesc& d, const ElemIn<V>& x, con
 // ---------------------------------------------------------------------------------------------
 struct VeloAcc {
   float ch[30];   // sum of squares per channel (factored tensors fill the 18 per-element ones)
-  float lstm[8];  // sum m_k, sum m_k^2, sum rms, sum rms^2 over the accumulators before the update
+  // The LSTM's variance features are taken over the accumulators before the update.  Their sums are
+  // shifted by a pivot per tensor (its first element): sum (m_k - c_k), sum (m_k - c_k)^2, sum (rms - c_r),
+  // sum (rms - c_r)^2.  Plain sums of m and m^2 cancel catastrophically where the spread is small
+  // against the mean -- a one-element tensor has variance exactly 0 in the reference, and the rounding
+  // of its m^2, scaled by 1 / mean p^2, used to land far above the feature's clamp at exp(-5).
+  float lstm[8];
+  float piv[4];   // c_0, c_1, c_2, c_r
 };
 
-__device__ __forceinline__ void lstm_sums(const float (&m)[3], float rms, float (&s)[8]) {
+// First element of each accumulator of a tensor (0 for an empty one); the same for every block.
+__device__ __forceinline__ void lstm_pivots(const TDesc& d, const PyloTensorArgs& a, float (&piv)[4]) {
+  if (d.n > 0) {
+    piv[0] = *(const gfloat*)(a.mom);
+    piv[1] = *(const gfloat*)(a.mom + d.n);
+    piv[2] = *(const gfloat*)(a.mom + 2 * d.n);
+    piv[3] = *(const gfloat*)(a.rms);
+  } else {
+    piv[0] = piv[1] = piv[2] = piv[3] = 0.0f;
+  }
+}
+
+__device__ __forceinline__ void lstm_sums(const float (&m)[3], float rms, VeloAcc& acc) {
 #pragma unroll
-  for (int k = 0; k < 3; ++k) { s[k] += m[k]; s[3 + k] = fmaf(m[k], m[k], s[3 + k]); }
-  s[6] += rms;
-  s[7] = fmaf(rms, rms, s[7]);
+  for (int k = 0; k < 3; ++k) {
+    const float dm = m[k] - acc.piv[k];
+    acc.lstm[k] += dm;
+    acc.lstm[3 + k] = fmaf(dm, dm, acc.lstm[3 + k]);
+  }
+  const float dr = rms - acc.piv[3];
+  acc.lstm[6] += dr;
+  acc.lstm[7] = fmaf(dr, dr, acc.lstm[7]);
 }
 
 template <int V, bool ND>
@@ -106,7 +129,7 @@ __device__ __forceinline__ void velo_stats_fac(const TDesc& d, const PyloTensorA
     lo_load<V, ND>(d, a, idx, fac_tab, x);
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-      lstm_sums(x.m[v], x.rms[v], acc.lstm);
+      lstm_sums(x.m[v], x.rms[v], acc);
       ema_update(e, x.g[v], x.m[v], x.rms[v]);
       float f[kNStat];
       lo_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.rfcf[v], 1e-6f, f);
@@ -147,7 +170,7 @@ __device__ __forceinline__ void velo_stats_tile(const TDesc& d, const PyloTensor
       const float gg = clampf(xg[v], a.clip_val);
       float m[3] = {x0[v], x1[v], x2[v]};
       float rr = xr[v];
-      lstm_sums(m, rr, acc.lstm);
+      lstm_sums(m, rr, acc);
       ema_update(e, gg, m, rr);
       const float rfcf[3] = {fa[0] * fb[v][0], fa[1] * fb[v][1], fa[2] * fb[v][2]};
       float f[kNStat];
@@ -229,7 +252,7 @@ __device__ __forceinline__ void velo_stats_vec(const TDesc& d, const PyloTensorA
     vec_load<V>(d, a, idx, x);
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-      lstm_sums(x.m[v], x.rms[v], acc.lstm);
+      lstm_sums(x.m[v], x.rms[v], acc);
       vec_update(e, dec, x.g[v], x.m[v], x.rms[v], x.v[v]);
       float f[30];
       vec_features(x.g[v], x.p[v], x.m[v], x.rms[v], x.v[v], 0.0f, f);
@@ -255,6 +278,7 @@ __global__ __launch_bounds__(kThreads) void k_velo_stats(const TDesc* __restrict
   for (int c = 0; c < 30; ++c) acc.ch[c] = 0.0f;
 #pragma unroll
   for (int c = 0; c < 8; ++c) acc.lstm[c] = 0.0f;
+  lstm_pivots(d, a, acc.piv);
   if (d.tile_nct > 0) {
     const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (task < d.tile_ntask) velo_stats_tile(d, a, task, e, fac_tab, acc);
@@ -348,18 +372,27 @@ __device__ __forceinline__ float lo_lstm_feature(const TDesc& d, const PyloTenso
     val = st.frac_dev ? st.frac_dev[a.group * 9 + q] : st.frac[a.group][q];
   } else if (q < 18) {
     val = lossfeat[q - 9];
-  } else if (q == 18) {
-    val = clip_log_abs10((double)nu * (tot[kSumR] / n));
-  } else if (q < 24) {
-    val = (q - 19 == d.rank) ? 1.0f : 0.0f;
   } else {
-    const int k = (q - 24) % 3;
-    const double mean_m = tot[kSumM + k] / n;
-    if (q < 27) {
-      val = clip_log_abs10(nu2 * (tot[kSumMM + k] / n - mean_m * mean_m));
-    } else {  // the reference subtracts mean_m (not mean_rms) from rms here (Velo_naive.py:198)
-      const double mean_r = tot[kSumR] / n;
-      val = clip_log_abs10(nu2 * (tot[kSumRR] / n - 2.0 * mean_m * mean_r + mean_m * mean_m));
+    // totals are of the accumulators shifted by the tensor's pivots (VeloAcc)
+    float piv[4];
+    lstm_pivots(d, a, piv);
+    const double dr = tot[kSumR] / n;
+    const double mean_r = (double)piv[3] + dr;
+    if (q == 18) {
+      val = clip_log_abs10((double)nu * mean_r);
+    } else if (q < 24) {
+      val = (q - 19 == d.rank) ? 1.0f : 0.0f;
+    } else {
+      const int k = (q - 24) % 3;
+      const double dm = tot[kSumM + k] / n;
+      const double mean_m = (double)(k == 0 ? piv[0] : k == 1 ? piv[1] : piv[2]) + dm;
+      if (q < 27) {
+        val = clip_log_abs10(nu2 * (tot[kSumMM + k] / n - dm * dm));
+      } else {  // the reference subtracts mean_m (not mean_rms) from rms here (Velo_naive.py:198):
+                // mean (rms - mean_m)^2 = var(rms) + (mean_rms - mean_m)^2
+        const double var_r = tot[kSumRR] / n - dr * dr;
+        val = clip_log_abs10(nu2 * (var_r + (mean_r - mean_m) * (mean_r - mean_m)));
+      }
     }
   }
   return val;

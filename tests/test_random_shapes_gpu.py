@@ -76,3 +76,6 @@ def test_random_tensor_lists_match_the_oracle(seed):
         for i, (g, c) in enumerate(zip(gpu, cpu)):
             e = max_err(g.detach().cpu(), c, 1e-5, 1e-6)
             assert e <= 1.0, (name, seed, i, shapes[i], e)
+        if name == "velo":     # the steps are small against the parameters: the LSTM state is the sharper check
+            assert max_err(opt.lstm_hidden_state[0].cpu(), orc.h, 1e-5, 1e-6) <= 1.0, (name, seed, "lstm h")
+            assert max_err(opt.lstm_hidden_state[1].cpu(), orc.c, 1e-5, 1e-6) <= 1.0, (name, seed, "lstm c")

@@ -178,3 +178,41 @@ def test_velo_replaced_state_tensor_is_picked_up():
 
     for x, y in zip(run(False), run(True)):
         assert torch.equal(x, y)
+
+
+def test_velo_variance_features_where_the_spread_is_tiny():
+    """The LSTM sees log-variances of the momentum / rms accumulators of every tensor.  A one-element
+    tensor, or one whose gradient is the same for every element, has variance exactly zero in the
+    reference (the feature sits at its lower clamp); large gradients on a small parameter make that a
+    cancellation of order 1e2 in single precision unless the sums are shifted.  The LSTM mixes tensors
+    through a max-pool, so one wrong row shows in every tensor's state."""
+    from oracle import pylo_oracle as O
+    from pylo_amd import VeLO_CUDA
+    from pylo_amd.models import VeLOMLP, VeLORNN
+
+    torch.manual_seed(4)
+    rnn, mlp = VeLORNN(lstm_hidden_size=64, param_inits=32), VeLOMLP(param_inits=32)
+    shapes = [(1, 1), (1,), (6, 40), (33,), (129, 257)]
+    gen = torch.Generator().manual_seed(8)
+    init = [torch.randn(s, generator=gen) * 0.01 for s in shapes]
+    grads = []
+    for t in range(4):
+        gs = [torch.randn(s, generator=gen) * 30.0 for s in shapes]
+        gs[2] = torch.full(shapes[2], 17.0 + t)          # the same gradient for every element
+        gs[3] = torch.full(shapes[3], -250.0) + torch.randn(shapes[3], generator=gen) * 1e-3
+        grads.append(gs)
+    gpu = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+    cpu = [v.clone() for v in init]
+    opt = VeLO_CUDA(gpu, lr=1e-2, num_steps=10, rnn=rnn, mlp=mlp)
+    orc = O.VeloOracle(cpu, rnn.state_dict(), mlp.state_dict(), lr=1e-2, num_steps=10)
+    loss = torch.tensor(1.0)
+    for t in range(4):
+        for p, g in zip(gpu, grads[t]):
+            p.grad = g.cuda()
+        opt.step(loss)
+        orc.step([g.clone() for g in grads[t]], loss)
+        torch.cuda.synchronize()
+        assert max_err(opt.lstm_hidden_state[0].cpu(), orc.h, REL, ABS) <= 1.0, (t, "h")
+        assert max_err(opt.lstm_hidden_state[1].cpu(), orc.c, REL, ABS) <= 1.0, (t, "c")
+        for i, (p, c) in enumerate(zip(gpu, cpu)):
+            assert max_err(p.detach().cpu(), c, REL, ABS) <= 1.0, (t, i)

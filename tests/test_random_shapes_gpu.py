@@ -79,3 +79,68 @@ def test_random_tensor_lists_match_the_oracle(seed):
         if name == "velo":     # the steps are small against the parameters: the LSTM state is the sharper check
             assert max_err(opt.lstm_hidden_state[0].cpu(), orc.h, 1e-5, 1e-6) <= 1.0, (name, seed, "lstm h")
             assert max_err(opt.lstm_hidden_state[1].cpu(), orc.c, 1e-5, 1e-6) <= 1.0, (name, seed, "lstm c")
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_steps_are_as_accurate_as_the_fp32_reference(seed):
+    """The parameter tolerance is loose where steps are small against the parameters (VeLO, AdafacLO), so
+    this looks at the steps themselves: the oracle evaluated in fp64 is the yardstick, and the error of the
+    HIP step, relative to the largest step of the tensor, may not exceed five times the error of the same
+    oracle evaluated in fp32 (plus what an fp32 parameter cannot resolve).  Over 120 seeds of this sweep
+    the HIP error stayed below 0.6 of that bound's first term."""
+    from oracle import pylo_oracle as O
+    from pylo_amd import AdafacLO_CUDA, CELO2_CUDA, ELO_CELO2_CUDA, ELO_CUDA, VeLO_CUDA
+    from pylo_amd.models import CELO2MLP, MetaMLP, VeLOMLP, VeLORNN
+
+    torch.manual_seed(1)
+    cnet, mnet = CELO2MLP(), MetaMLP(39, 32, 1)
+    rnn, mlp = VeLORNN(lstm_hidden_size=64, param_inits=32), VeLOMLP(param_inits=32)
+    rng = random.Random(seed)
+    shapes = [_rand_shape(rng) for _ in range(rng.randint(2, 6))]
+    gscale = rng.choice([1e-3, 0.05, 1.0, 30.0])
+    gen = torch.Generator().manual_seed(seed)
+    init = [torch.randn(s, generator=gen) * 0.1 for s in shapes]
+    grads = [[torch.randn(s, generator=gen) * gscale for s in shapes] for _ in range(2)]
+    adam_1d = seed % 2 == 0
+    ck = dict(lr=1e-2, weight_decay=0.0, clip_grad=False, independent_adam=(0.9, 0.95, 1e-8), use_adamw_for_1d=adam_1d)
+    cases = [
+        ("elo_celo2", lambda g: ELO_CELO2_CUDA(g, lr=1e-2, network=cnet, hf_key=None),
+         lambda c: O.EloCelo2Oracle(c, cnet.state_dict(), lr=1e-2, adam_lr_mult=20.0), None),
+        ("celo2", lambda g: CELO2_CUDA(g, lr=1e-2, network=cnet, hf_key=None, use_adamw_for_1d=adam_1d),
+         lambda c: O.EloCelo2Oracle(c, cnet.state_dict(), **ck), None),
+        ("adafac", lambda g: AdafacLO_CUDA(g, lr=0.5, network=copy.deepcopy(mnet), hf_key=None),
+         lambda c: O.AdafacOracle(c, mnet.state_dict(), lr=0.5), None),
+        ("elo", lambda g: ELO_CUDA(g, lr=1e-2, network=copy.deepcopy(mnet), hf_key=None, clip_grad=True),
+         lambda c: O.EloOracle(c, mnet.state_dict(), lr=1e-2, clip_grad=True), None),
+        ("velo", lambda g: VeLO_CUDA(g, lr=1e-2, num_steps=10, rnn=copy.deepcopy(rnn), mlp=copy.deepcopy(mlp)),
+         lambda c: O.VeloOracle(c, rnn.state_dict(), mlp.state_dict(), lr=1e-2, num_steps=10), torch.tensor(1.0)),
+    ]
+    for name, make_opt, make_orc, loss in cases:
+        print(f"seed {seed} {name} shapes {shapes} gscale {gscale}", flush=True)
+        gpu = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+        c32 = [v.clone() for v in init]
+        c64 = [v.clone().double() for v in init]
+        opt, o32, o64 = make_opt(gpu), make_orc(c32), make_orc(c64).double_()
+        for t in range(2):
+            before = ([p.detach().cpu().double().clone() for p in gpu], [c.double().clone() for c in c32],
+                      [c.clone() for c in c64])
+            for p, g in zip(gpu, grads[t]):
+                p.grad = g.cuda()
+            g32, g64 = [g.clone() for g in grads[t]], [g.double() for g in grads[t]]
+            if loss is None:
+                opt.step()
+                o32.step(g32)
+                o64.step(g64)
+            else:
+                opt.step(loss)
+                o32.step(g32, loss)
+                o64.step(g64, loss.double())
+        torch.cuda.synchronize()
+        for i, s in enumerate(shapes):
+            s64 = c64[i] - before[2][i]
+            s_hip = gpu[i].detach().cpu().double() - before[0][i]
+            s32 = c32[i].double() - before[1][i]
+            scale = float(s64.abs().max()) + 1e-30
+            e_hip, e_32 = float((s_hip - s64).abs().max()) / scale, float((s32 - s64).abs().max()) / scale
+            ulp = float(c64[i].abs().max()) * 6e-8 / scale
+            assert e_hip <= 5 * e_32 + 4 * ulp + 2e-4, (name, seed, s, e_hip, e_32, ulp)

@@ -216,3 +216,39 @@ def test_velo_variance_features_where_the_spread_is_tiny():
         assert max_err(opt.lstm_hidden_state[1].cpu(), orc.c, REL, ABS) <= 1.0, (t, "c")
         for i, (p, c) in enumerate(zip(gpu, cpu)):
             assert max_err(p.detach().cpu(), c, REL, ABS) <= 1.0, (t, i)
+
+
+def test_velo_loss_accumulators_follow_the_reference():
+    """The ten loss EMAs, their running minima and the iteration counter (Velo_naive.py:129-175) over a
+    loss sequence with a spike (clipped to twice the largest corrected mean), a plateau and a rise; the
+    nine loss features feed the LSTM from the third step on, so its state is compared as well."""
+    from oracle import pylo_oracle as O
+    from pylo_amd import VeLO_CUDA
+    from pylo_amd.models import VeLOMLP, VeLORNN
+
+    torch.manual_seed(9)
+    rnn, mlp = VeLORNN(lstm_hidden_size=64, param_inits=32), VeLOMLP(param_inits=32)
+    shapes = [(12, 20), (20,)]
+    gen = torch.Generator().manual_seed(3)
+    init = [torch.randn(s, generator=gen) * 0.1 for s in shapes]
+    losses = [2.3, 1.9, 1.7, 40.0, 1.5, 1.5, 1.5, 0.9, 1.2, 2.0, 0.05, 0.04]
+    gpu = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+    cpu = [v.clone() for v in init]
+    opt = VeLO_CUDA(gpu, lr=1e-2, num_steps=30, rnn=rnn, mlp=mlp)
+    orc = O.VeloOracle(cpu, rnn.state_dict(), mlp.state_dict(), lr=1e-2, num_steps=30)
+    for t, lv in enumerate(losses):
+        grads = [torch.randn(s, generator=gen) * 0.1 for s in shapes]
+        for p, g in zip(gpu, grads):
+            p.grad = g.cuda()
+        loss = torch.tensor(lv)
+        opt.step(loss.cuda())
+        orc.step(grads, loss)
+        torch.cuda.synchronize()
+        lb = opt.loss_buffer
+        assert int(lb["iteration"]) == int(orc.loss.iteration) == t + 1
+        assert max_err(lb["means"].cpu(), orc.loss.means, REL, ABS) <= 1.0, (t, "means")
+        assert max_err(lb["running_min"].cpu(), orc.loss.running_min, REL, ABS) <= 1.0, (t, "running_min")
+        assert max_err(opt.lstm_hidden_state[0].cpu(), orc.h, REL, ABS) <= 1.0, (t, "h")
+        assert max_err(opt.lstm_hidden_state[1].cpu(), orc.c, REL, ABS) <= 1.0, (t, "c")
+        for i, (p, c) in enumerate(zip(gpu, cpu)):
+            assert max_err(p.detach().cpu(), c, REL, ABS) <= 1.0, (t, i)

@@ -340,13 +340,11 @@ __global__ __launch_bounds__(kV0aThreads) void k_v0a(const TDesc* __restrict__ d
 
 // Where entry i of vector `which` of tensor d lives in the factor / term tables.
 __device__ __forceinline__ size_t fac_index(const TDesc& d, int which, int k, int i) {
-  return d.mode == kModeFac2D ? (size_t)pick(d.fac_off, which) + (size_t)i * 4 + k
-                              : (size_t)pick(d.fac_off, which) + (size_t)k * pick(d.pitch, which) + i;
+  return (size_t)pick(d.fac_off, which) + (size_t)i * 4 + k;   // [entry][4]: one 16-byte access per entry
 }
 template <int H>
 __device__ __forceinline__ size_t term_index(const TDesc& d, int which, int j, int i) {
-  return d.mode == kModeFac2D ? (size_t)pick(d.term_off, which) + (size_t)i * H + j
-                              : (size_t)pick(d.term_off, which) + (size_t)j * pick(d.pitch, which) + i;
+  return (size_t)pick(d.term_off, which) + (size_t)i * H + j;   // [entry][H]
 }
 
 // Row_factor / col_factor of one entry, and the two normalised broadcast features it carries
@@ -426,14 +424,10 @@ __device__ __forceinline__ void vector_terms(const TDesc& d, int which, bool is_
       }
       tv[j] = t;
     }
-    if (d.mode == kModeFac2D) {  // [index][H]: the entry's outputs are adjacent, 16 bytes a store
+    // [entry][H]: the entry's outputs are adjacent, 16 bytes a store
 #pragma unroll
-      for (int j = 0; j < JB; j += 4)
-        *(float4*)(term + term_index<H>(d, which, j0 + j, i)) = make_float4(tv[j], tv[j + 1], tv[j + 2], tv[j + 3]);
-    } else {
-#pragma unroll
-      for (int j = 0; j < JB; ++j) term[term_index<H>(d, which, j0 + j, i)] = tv[j];
-    }
+    for (int j = 0; j < JB; j += 4)
+      *(float4*)(term + term_index<H>(d, which, j0 + j, i)) = make_float4(tv[j], tv[j + 1], tv[j + 2], tv[j + 3]);
   }
 }
 
@@ -594,12 +588,7 @@ __global__ __launch_bounds__(kThreads) void k_v0b(const TDesc* __restrict__ desc
       slice = (i / blk - o_first) * st + i % st;
     }
     vector_entry(d, is_r, fac, len, i, fpre[q], rcm3, s0, s1, fct, x0, x1, rcm_slices, slice);
-    if (d.mode == kModeFac2D) {  // [index][4]: one 16-byte store
-      *(float4*)(fac_tab + fac_index(d, which, 0, i)) = make_float4(fct[0], fct[1], fct[2], 0.0f);
-    } else {
-#pragma unroll
-      for (int k = 0; k < 3; ++k) fac_tab[fac_index(d, which, k, i)] = fct[k];
-    }
+    *(float4*)(fac_tab + fac_index(d, which, 0, i)) = make_float4(fct[0], fct[1], fct[2], 0.0f);
     if (w1 != nullptr) vector_terms<H>(d, which, is_r, i, x0, x1, w1, b1 + (size_t)it.tensor * b1_stride, term_tab);
   }
 }

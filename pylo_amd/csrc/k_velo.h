@@ -46,10 +46,11 @@ __device__ __forceinline__ void lo_load(const TDesc& d, const PyloTensorArgs& a,
     const unsigned s0 = (unsigned)d.nd_stride[0], s1 = (unsigned)d.nd_stride[1];
     x.i0 = (int)(fd_div(u, d.nd_div_blk[0]) * s0 + (u - fd_div(u, d.nd_div_st[0]) * s0));
     x.i1 = (int)(fd_div(u, d.nd_div_blk[1]) * s1 + (u - fd_div(u, d.nd_div_st[1]) * s1));
-#pragma unroll
-    for (int k = 0; k < 3; ++k)
-      x.rfcf[0][k] = fac_tab[d.fac_off[0] + (size_t)k * d.pitch[0] + x.i0] *
-                     fac_tab[d.fac_off[1] + (size_t)k * d.pitch[1] + x.i1];
+    const float4 fa = load_f4(fac_tab + d.fac_off[0] + (size_t)x.i0 * 4);
+    const float4 fb = load_f4(fac_tab + d.fac_off[1] + (size_t)x.i1 * 4);
+    x.rfcf[0][0] = fa.x * fb.x;
+    x.rfcf[0][1] = fa.y * fb.y;
+    x.rfcf[0][2] = fa.z * fb.z;
   }
 }
 
@@ -72,10 +73,15 @@ __device__ __forceinline__ void lo_terms(const TDesc& d, const ElemIn<V>& x, con
       }
     }
   } else {
+    static_assert(H % 4 == 0, "term tables are read four floats at a time");
+    const float* t0 = term_tab + d.term_off[0] + (size_t)x.i0 * H;
+    const float* t1 = term_tab + d.term_off[1] + (size_t)x.i1 * H;
 #pragma unroll
-    for (int j = 0; j < H; ++j)
-      h[0][j] = term_tab[d.term_off[0] + (size_t)j * d.pitch[0] + x.i0] +
-                term_tab[d.term_off[1] + (size_t)j * d.pitch[1] + x.i1];
+    for (int q = 0; q < H / 4; ++q) {
+      const float4 ta = load_f4(t0 + q * 4), tb = load_f4(t1 + q * 4);
+      h[0][q * 4 + 0] = ta.x + tb.x; h[0][q * 4 + 1] = ta.y + tb.y;
+      h[0][q * 4 + 2] = ta.z + tb.z; h[0][q * 4 + 3] = ta.w + tb.w;
+    }
   }
 }
 

@@ -78,7 +78,7 @@ struct TDesc {
   int len[2];       // entries of vector 0 / 1
   int sumlen[2];    // elements summed into one entry
   int npart[2];     // partial rows to add up per entry (2-D: column blocks / strips; N-D: 1)
-  int pitch[2];     // row pitch of the SoA tables of vector 0 / 1 (len rounded up to 4); 2-D tensors use [index][k] tables
+  int pitch[2];     // len rounded up to 4
   int nd_size[2];   // N-D: size and stride of the dim removed from vector 0 / 1;
   int nd_stride[2]; //      entry = (idx / (size*stride)) * stride + idx % stride
   FastDiv nd_div_blk[2], nd_div_st[2];  // the two divisors of that formula per vector, as multiply-and-shift
@@ -90,8 +90,8 @@ struct TDesc {
   int fac_slot;     // index among factored tensors, -1 otherwise
   int rank;         // number of dims larger than 1 (VeLO's rank one-hot feature)
   long long part_off[2];  // floats, partial sums of g^2
-  long long fac_off[2];   // floats, factor tables: 2-D vector 0 is AoS [len][4], everything else SoA [3][pitch]
-  long long term_off[2];  // floats, first-layer terms: 2-D vector 0 is AoS [len][H], else SoA [H][pitch]
+  long long fac_off[2];   // floats, factor tables [entry][4] (three decays + padding: one 16-byte access per entry)
+  long long term_off[2];  // floats, first-layer terms [entry][H]
   int v0a_first[2], v0a_n[2];  // k_v0a blocks of vector 0 / 1
   // Column-resident walk (wide 2-D tensors, C0 % kTileCols == 0): wave task w covers columns
   // [ (w % tile_nct) * kTileCols, +kTileCols ) of rows [ (w / tile_nct) * kTileRows, +kTileRows );

@@ -186,11 +186,10 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
         d.pitch[w] = (int)round4(d.len[w]);
         d.part_off[w] = part;
         part += round4((long long)d.npart[w] * d.len[w]);
-        const bool aos = d.mode == kModeFac2D;  // 2-D: both tables are [index][4] / [index][H]
-        d.fac_off[w] = fac;
-        fac += aos ? (long long)d.len[w] * 4 : 3ll * d.pitch[w];
-        d.term_off[w] = term;
-        term += aos ? round4((long long)d.len[w] * H) : (long long)H * d.pitch[w];
+        d.fac_off[w] = fac;              // [entry][4]
+        fac += (long long)d.len[w] * 4;
+        d.term_off[w] = term;            // [entry][H]
+        term += round4((long long)d.len[w] * H);
       }
       if (n > 0) {
         d.fac_slot = (int)L.fac_list.size();

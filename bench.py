@@ -208,7 +208,7 @@ def main():
         "hbm_GBps_fused_path": bytes_fused / (fused_ms * 1e-3) / 1e9,
         "hbm_roofline_frac_fused_path": bytes_fused / (fused_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "whole_step_ms": wall_ms,
-        "whole_step_note": "optimizer.step(): fused path + Newton-Schulz as batched library fp32 GEMMs + the HIP finishing pass "
+        "whole_step_note": "optimizer.step(): fused path + Newton-Schulz as batched library fp32 GEMMs (rocBLAS) + the HIP finishing pass "
                            "(normalise, apply)",
         "launch_ms": {nm: float(v) for nm, v in zip(names, mean)},
         "roofline": {"bound": "hbm", "kernel": "k_celo2_apply", "achieved": apply_gbs, "peak": HBM_PEAK_GBS,

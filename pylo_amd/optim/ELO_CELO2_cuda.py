@@ -18,6 +18,8 @@ from __future__ import annotations
 
 from typing import Optional
 
+import os
+
 import numpy as np
 import torch
 from torch.optim import Optimizer
@@ -36,14 +38,34 @@ def newton_schulz(x: torch.Tensor, coeffs, iters: int, eps: float) -> torch.Tens
     if x.dim() > 3:     # more leading dims: one batch of matrices
         return newton_schulz(x.reshape((-1,) + tuple(x.shape[-2:])), coeffs, iters, eps).reshape(x.shape)
     tall = x.shape[-2] > x.shape[-1]
-    x = x / (torch.linalg.norm(x, dim=(-2, -1), keepdim=True) + eps)
+    if x.dim() == 3 and x.is_cuda:
+        # Frobenius norms through the multi-tensor kernels: a reduction to one value per matrix runs on a
+        # handful of blocks (0.27 ms for a 50257 x 768 matrix), the multi-tensor one on all of them
+        norm = torch.stack(torch._foreach_norm(list(x.unbind(0)))).view(-1, 1, 1)
+    else:
+        norm = torch.linalg.norm(x, dim=(-2, -1), keepdim=True)
+    x = x / (norm + eps)
     c0, c1, c2 = coeffs
     if x.dim() == 3:
+        split = _gram_split(x.shape[-2] if tall else x.shape[-1], min(x.shape[-2:]), x.shape[0])
         for _ in range(iters):
             xt = x.transpose(-2, -1)
-            a = torch.bmm(xt, x) if tall else torch.bmm(x, xt)
-            b = torch.baddbmm(a, a, a, beta=c1, alpha=c2)         # c1 A + c2 A A
-            x = torch.baddbmm(x, x, b, beta=c0) if tall else torch.baddbmm(x, b, x, beta=c0)
+            if split > 1 and tall:
+                # Gram matrix of a very tall matrix (an embedding: 50257 x 768): one GEMM with a 768 x 768
+                # output and a reduction 50257 long leaves most of the GPU idle; the rows are cut into
+                # `split` slabs whose Gram matrices are one batched GEMM, added up afterwards
+                xs = x.reshape(x.shape[0] * split, x.shape[1] // split, x.shape[2])
+                a = torch.bmm(xs.transpose(-2, -1), xs).view(x.shape[0], split, x.shape[2], x.shape[2]).sum(1)
+            else:
+                a = torch.bmm(xt, x) if tall else torch.bmm(x, xt)
+            # c1 A + c2 A A = (c2 A + c1 I) A and c0 X + B X = (B + c0 I) X: the scalings ride on the
+            # diagonals of the small matrices, so every product is a plain GEMM (a GEMM that accumulates
+            # into c0 X first copies X, half a gigabyte per iteration on this parameter set)
+            a2 = a * c2
+            a2.diagonal(dim1=-2, dim2=-1).add_(c1)
+            b = torch.bmm(a2, a)
+            b.diagonal(dim1=-2, dim2=-1).add_(c0)
+            x = torch.bmm(x, b) if tall else torch.bmm(b, x)
         return x
     for _ in range(iters):
         xt = x.transpose(-2, -1)
@@ -51,6 +73,39 @@ def newton_schulz(x: torch.Tensor, coeffs, iters: int, eps: float) -> torch.Tens
         b = c1 * a + c2 * (a @ a)
         x = c0 * x + (x @ b if tall else b @ x)
     return x
+
+
+class _ns_blas:
+    """Newton-Schulz GEMMs through rocBLAS for the duration of the block: on the shapes of a transformer's
+    matrices (768 .. 3072 wide, batches of 12) its fp32 kernels run at 122 TFLOP/s where hipBLASLt's choices
+    give 110 (768^3 batched: 55).  ``PYLO_MI355_NS_BLAS=default`` leaves torch's setting alone."""
+
+    def __enter__(self):
+        self.prev = None
+        if os.environ.get("PYLO_MI355_NS_BLAS", "rocblas") == "rocblas":
+            try:
+                self.prev = torch.backends.cuda.preferred_blas_library()
+                torch.backends.cuda.preferred_blas_library("cublas")      # torch's name for rocBLAS
+            except Exception:
+                self.prev = None
+        return self
+
+    def __exit__(self, *exc):
+        if self.prev is not None:
+            torch.backends.cuda.preferred_blas_library(self.prev)
+        return False
+
+
+def _gram_split(k: int, small: int, batch: int) -> int:
+    """Number of slabs to cut a reduction of length k into for the Gram product of `batch` matrices whose
+    other dim is `small`: 1 unless the reduction is long against the output and the batch is too small to
+    fill the GPU by itself; else the largest divisor of k up to 64 that leaves slabs of 512 or more."""
+    if batch * small * small >= 8 * 1024 * 1024 or k < 16 * small or k < 8192:
+        return 1
+    for s in range(64, 1, -1):
+        if k % s == 0 and k // s >= 512:
+            return s
+    return 1
 
 
 def rms_normalize(x: torch.Tensor, dims, eps: float = 1e-9) -> torch.Tensor:
@@ -402,6 +457,10 @@ class ELO_CELO2_CUDA(Optimizer):
     def finish_step(self, tensors):
         """Newton-Schulz, RMS normalisation and the parameter update of the MLP tensors
         (pylo/optim/ELO_CELO2_cuda.py:288-296)."""
+        with _ns_blas():
+            self._finish_step(tensors)
+
+    def _finish_step(self, tensors):
         fin = self._fin_args
         fin["grad"] = 0
         keep, any_fin = [], False   # post-Newton-Schulz matrices must outlive the launch

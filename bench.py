@@ -1,6 +1,6 @@
 """Benchmark of the fused learned-optimizer step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gpt2s|cfg1] [--fused-only]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gpt2s|cfg1|vit_velo|llama_adafac|stream_ceiling] [--fused-only]
 
 Workload (default): BASELINE config 2 -- ELO-CELO2 on a GPT-2-small-shaped fp32 parameter set
 (98 tensors, 124 355 328 parameters), synthetic per-tensor Gaussian gradients with log-uniform
@@ -121,7 +121,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gpt2s", choices=["gpt2s", "cfg1", "vit_velo", "llama_adafac"])
+    ap.add_argument("--workload", default="gpt2s", choices=["gpt2s", "cfg1", "vit_velo", "llama_adafac", "stream_ceiling"])
     ap.add_argument("--fused-only", action="store_true",
                     help="loop the C-ABI call alone (no Newton-Schulz / apply), e.g. under rocprofv3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -139,6 +139,8 @@ def main():
 
     if a.workload in ("vit_velo", "llama_adafac"):
         return other_workload(a)
+    if a.workload == "stream_ceiling":
+        return stream_ceiling(a)
     dev = torch.device("cuda:0")
     shapes = gpt2_small_shapes() if a.workload == "gpt2s" else cfg1_shapes()
     torch.manual_seed(1)
@@ -219,6 +221,43 @@ def main():
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
+
+
+def stream_ceiling(a):
+    """What the memory system delivers for the access mixes of the element passes, with nothing computed:
+    the library's bare streaming kernel over arrays of the GPT-2-small matrices' size.  Not a benchmark of
+    the optimizer; it is the yardstick the roofline fractions of its kernels are read against."""
+    import ctypes as C
+
+    import torch
+
+    from pylo_amd import _lib
+
+    lib = _lib.load()
+    lib.pylo_mi355_stream_probe.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    dev = torch.device("cuda:0")
+    n = 124318464
+    src = torch.zeros(6 * n, device=dev)
+    dst = torch.zeros(5 * n, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    out = {}
+    for name, r, w in (("read6 (statistics pass)", 6, 0), ("read6 write5 (apply pass)", 6, 5), ("read1 write1 (copy)", 1, 1),
+                       ("read1 (gradient pass)", 1, 0), ("write5", 1, 5)):
+        for nt in (0, 1):
+            call = lambda: _lib.check(lib.pylo_mi355_stream_probe(src.data_ptr(), dst.data_ptr(), n, r, w, nt, stream),
+                                      "stream_probe")
+            for _ in range(max(a.warmup, 3)):
+                call()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(a.steps):
+                call()
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / a.steps
+            out[f"{name}{', non-temporal' if nt else ''}"] = {"ms": ms, "GBps": (r + w) * 4.0 * n / ms / 1e6}
+    print(json.dumps({"metric": "attainable_hbm_rate_by_access_mix", "unit": "GB/s", "n_gpus": 1, "steps": a.steps,
+                      "warmup": a.warmup, "elements_per_array": n, "peak_GBps": HBM_PEAK_GBS, "mixes": out}))
 
 
 def other_workload(a):

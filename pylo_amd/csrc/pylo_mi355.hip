@@ -1051,3 +1051,60 @@ extern "C" int pylo_mi355_velo_kernel_simple(const float* grad, float* param, co
   a.lr = lr; a.step_mult = step_mult; a.exp_mult = exp_mult; a.epsilon = epsilon; a.weight_decay = weight_decay;
   return single_launch<kFamVelo>("velo_kernel_simple", a, stream);
 }
+
+// ---------------------------------------------------------------------------------------------
+// Bare streaming kernel (benchmark instrumentation): the rate the memory system gives an access mix
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+template <int R, int W, bool NT>
+__global__ __launch_bounds__(kThreads) void k_stream_probe(const float* __restrict__ in, float* __restrict__ out,
+                                                           size_t n) {
+  constexpr int kIters = 8;
+  const size_t base = (size_t)blockIdx.x * kThreads * 4 * kIters;
+  for (int it = 0; it < kIters; ++it) {
+    const size_t i = base + ((size_t)it * kThreads + threadIdx.x) * 4;
+    if (i >= n) break;
+    v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const gv4f* p = (const gv4f*)(in + (size_t)r * n + i);
+      acc += NT ? __builtin_nontemporal_load(p) : *p;
+    }
+#pragma unroll
+    for (int w = 0; w < W; ++w) {
+      gv4f* p = (gv4f*)(out + (size_t)w * n + i);
+      const v4f v = acc * (float)(w + 1);
+      if (NT) __builtin_nontemporal_store(v, p);
+      else *p = v;
+    }
+    if (W == 0 && acc.x == 123.456f) out[0] = acc.y;   // keeps the loads of a read-only mix alive
+  }
+}
+
+template <int R, int W>
+void stream_launch(const float* in, float* out, size_t n, bool nt, hipStream_t s) {
+  const unsigned grid = (unsigned)((n + (size_t)kThreads * 4 * 8 - 1) / ((size_t)kThreads * 4 * 8));
+  if (nt) hipLaunchKernelGGL((k_stream_probe<R, W, true>), dim3(grid), dim3(kThreads), 0, s, in, out, n);
+  else hipLaunchKernelGGL((k_stream_probe<R, W, false>), dim3(grid), dim3(kThreads), 0, s, in, out, n);
+}
+
+}  // namespace
+
+extern "C" int pylo_mi355_stream_probe(const float* in, float* out, size_t n, int reads, int writes, int nontemporal,
+                                       void* stream) {
+  if (!in || !out || n == 0 || n % 4 != 0) return fail("stream_probe: null pointer or n not a multiple of 4");
+  if ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) % 16 != 0)
+    return fail("stream_probe: 16-byte alignment needed");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool nt = nontemporal != 0;
+  if (reads == 6 && writes == 5) stream_launch<6, 5>(in, out, n, nt, s);
+  else if (reads == 6 && writes == 0) stream_launch<6, 0>(in, out, n, nt, s);
+  else if (reads == 6 && writes == 1) stream_launch<6, 1>(in, out, n, nt, s);
+  else if (reads == 1 && writes == 1) stream_launch<1, 1>(in, out, n, nt, s);
+  else if (reads == 1 && writes == 0) stream_launch<1, 0>(in, out, n, nt, s);
+  else if (reads == 1 && writes == 5) stream_launch<1, 5>(in, out, n, nt, s);
+  else return fail("stream_probe: reads must be 1 or 6, writes 0, 1 or 5");
+  HIP_TRY(hipGetLastError());
+  return 0;
+}

@@ -79,6 +79,9 @@ def test_workspace_sizing_and_error_paths_without_gpu():
     assert lib.pylo_mi355_plan_device_steps(None, None) != 0
     assert b"plan_device_steps" in lib.pylo_mi355_last_error()
     assert C.sizeof(_lib.DeviceSteps) == 8 + 3 * 8
+    lib.pylo_mi355_stream_probe.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    assert lib.pylo_mi355_stream_probe(None, None, 1024, 6, 5, 0, None) != 0
+    assert b"stream_probe" in lib.pylo_mi355_last_error()
 
 
 def test_optimizers_fail_loudly_without_gpu():

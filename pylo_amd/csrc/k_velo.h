@@ -20,6 +20,14 @@ constexpr int kVBank = 159;    // floats per bank entry: W_in (4,30) | b_in 4 | 
 constexpr int kXW = 32;        // row pitch of the LSTM input features (30 used)
 constexpr int kGateBT = 8;     // tensors per k_velo_gates block
 
+struct LossState {             // by-value kernel argument: the caller's loss accumulators (PyloVeloStep)
+  float* means;
+  float* running_min;
+  const float* decays;
+  int* iteration;
+  const float* loss;
+};
+
 struct VeloStep {              // by-value kernel argument: scalars of one step
   float frac[PYLO_MAX_GROUPS][9];
   const float* frac_dev;       // the same table in device memory when the step counters live there, else null
@@ -319,42 +327,53 @@ __global__ __launch_bounds__(kThreads) void k_velo_stats(const TDesc* __restrict
 // ---------------------------------------------------------------------------------------------
 // loss features (Velo_naive.py:147-175): 10 EMAs of the clipped loss, updated in place
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void k_velo_loss(float* __restrict__ means, float* __restrict__ running_min,
-                                                  const float* __restrict__ decays, int* __restrict__ iteration,
-                                                  const float* __restrict__ loss_p, float* __restrict__ lossfeat) {
-  __shared__ float cor_s[10], rmin_s[10];
+// One step of the loss accumulators (Velo_naive.py:129-175), by a whole block (its first wave works, the
+// others keep the barriers): ten EMAs of the loss clipped to twice the largest corrected mean, their running
+// minima, the iteration counter, and the nine features clamp((cm_i - rmin_i) / max(1e-8, cm_{i+1} - rmin_i) - 1,
+// +-1), zero while iteration <= 2, left in feat_s[0..8].  write == false only reads the state: every block of
+// k_lo_reduce derives the features that way, and one block of the launch after it advances the state.
+__device__ __forceinline__ void loss_step(float* __restrict__ means, float* __restrict__ running_min,
+                                          const float* __restrict__ decays, int* __restrict__ iteration,
+                                          const float* __restrict__ loss_p, bool write, float* cor_s /*10*/,
+                                          float* rmin_s /*10*/, float* feat_s /*9*/) {
   const int dI = threadIdx.x;
-  const int it = *iteration;
-  const float loss = *loss_p;
-  float cor = -INFINITY, dec = 0.0f, mean = 0.0f, pw = 0.0f;
-  if (dI < 10) {
-    dec = decays[dI];
-    mean = means[dI];
-    pw = powf(dec, (float)(it + 1));
-    cor = mean / (1.0f - pw);
-  }
-  float mx = cor;
+  int it = 0;
+  if (dI < 64) {
+    it = *iteration;
+    const float loss = *loss_p;
+    float cor = -INFINITY, dec = 0.0f, mean = 0.0f, pw = 0.0f;
+    if (dI < 10) {
+      dec = decays[dI];
+      mean = means[dI];
+      pw = powf(dec, (float)(it + 1));
+      cor = mean / (1.0f - pw);
+    }
+    float mx = cor;
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-  const float approx_max = (it == 0) ? loss : mx;
-  const float l = fminf(fabsf(approx_max) * 2.0f, loss);
-  if (dI < 10) {
-    const float m2 = mean * dec + l * (1.0f - dec);
-    const float cor2 = m2 / (1.0f - pw);
-    const float rmin = fminf(running_min[dI], cor2);
-    means[dI] = m2;
-    running_min[dI] = rmin;
-    cor_s[dI] = cor2;
-    rmin_s[dI] = rmin;
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    const float approx_max = (it == 0) ? loss : mx;
+    const float l = fminf(fabsf(approx_max) * 2.0f, loss);
+    if (dI < 10) {
+      const float m2 = mean * dec + l * (1.0f - dec);
+      const float cor2 = m2 / (1.0f - pw);
+      const float rmin = fminf(running_min[dI], cor2);
+      if (write) {
+        means[dI] = m2;
+        running_min[dI] = rmin;
+      }
+      cor_s[dI] = cor2;
+      rmin_s[dI] = rmin;
+    }
   }
   __syncthreads();
-  if (dI == 0) *iteration = it + 1;
+  if (write && dI == 0) *iteration = it + 1;
   if (dI < 9) {
     const float den = fmaxf(1e-8f, cor_s[dI + 1] - rmin_s[dI]);
     float f = (cor_s[dI] - rmin_s[dI]) / den - 1.0f;
     f = fminf(fmaxf(f, -1.0f), 1.0f);
-    lossfeat[dI] = (it + 1 <= 2) ? f * 0.0f : f;
+    feat_s[dI] = (it + 1 <= 2) ? f * 0.0f : f;
   }
+  __syncthreads();
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -410,7 +429,7 @@ __global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restr
                                                         const double* __restrict__ stats_part,
                                                         const double* __restrict__ seg_tot,
                                                         double* __restrict__ totals,
-                                                        const float* __restrict__ lossfeat, VeloStep st,
+                                                        LossState ls, VeloStep st,
                                                         float* __restrict__ xfeat, int H,
                                                         const float* __restrict__ w2t, const float* __restrict__ b2,
                                                         const float* __restrict__ wft, const float* __restrict__ bf,
@@ -443,6 +462,8 @@ __global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restr
   __syncthreads();
   if (xfeat == nullptr) return;
   const int row = T - 1 - t;
+  __shared__ float cor_s[10], rmin_s[10], lossfeat[9];
+  loss_step(ls.means, ls.running_min, ls.decays, ls.iteration, ls.loss, false, cor_s, rmin_s, lossfeat);
   if (threadIdx.x < 30) xs[threadIdx.x] = lo_lstm_feature(d, a, tot, lossfeat, st, threadIdx.x);
   __syncthreads();
   if (threadIdx.x < 30) xfeat[(size_t)row * kXW + threadIdx.x] = xs[threadIdx.x];
@@ -491,8 +512,14 @@ __global__ __launch_bounds__(kThreads) void k_velo_colmax(const float* __restric
 // from the per-chunk maxima of k_velo_colmax when there are many rows.
 __global__ __launch_bounds__(kThreads) void k_velo_mix(const float* __restrict__ mixbuf, int T, int Tpad, int H,
                                                        const float* __restrict__ pmax, int n_chunks,
-                                                       const float* __restrict__ h_state, float* __restrict__ xT) {
+                                                       const float* __restrict__ h_state, float* __restrict__ xT,
+                                                       LossState ls) {
   __shared__ float mx_s[kWaves][64];
+  // every block of k_lo_reduce has read the loss accumulators by now: one block advances them
+  if (blockIdx.x == 0 && blockIdx.y == 0) {
+    __shared__ float cor_s[10], rmin_s[10], feat_s[9];
+    loss_step(ls.means, ls.running_min, ls.decays, ls.iteration, ls.loss, true, cor_s, rmin_s, feat_s);
+  }
   const int lane = threadIdx.x & 63, grp = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int u = blockIdx.x * 64 + lane;  // H is a multiple of 64
   const float* fm = mixbuf + (size_t)T * H;

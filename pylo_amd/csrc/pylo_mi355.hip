@@ -401,7 +401,7 @@ int pylo_mi355_plan_destroy(PyloPlan* P) {
 
 static const char* kCelo2Launches[] = {"k_p0(sums)", "k_gnorm", "k_p0(exact)", "k_v0a", "k_v0b",
                                        "k_celo2_stats", "k_celo2_fold", "k_celo2_apply"};
-static const char* kVeloLaunches[] = {"k_p0(sums)", "k_p0_nd", "k_v0a", "k_v0b", "k_velo_stats", "k_velo_loss",
+static const char* kVeloLaunches[] = {"k_p0(sums)", "k_p0_nd", "k_v0a", "k_v0b", "k_velo_stats",
                                       "k_lo_reduce", "k_velo_mix", "k_velo_gates", "k_velo_heads", "k_terms",
                                       "k_velo_apply"};
 
@@ -780,7 +780,6 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
   float* wfold = P->at<float>(L.off_wfold);
   double* totals = P->at<double>(L.off_totals);
   float* xfeat = P->at<float>(L.off_xfeat);
-  float* lossfeat = P->at<float>(L.off_lossfeat);
   float* xT = P->at<float>(L.off_xT);
   float* canon = P->at<float>(L.off_canon);
   float* mixbuf = P->at<float>(L.off_mixbuf);
@@ -809,14 +808,12 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
   HIP_TRY(mark());
   if (n_el > 0) hipLaunchKernelGGL(k_velo_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, dec, stats);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_velo_loss, dim3(1), dim3(64), 0, s, step->loss_means, step->loss_running_min, step->loss_decays,
-                     step->loss_iteration, step->loss, lossfeat);
-  HIP_TRY(mark());
+  const LossState ls{step->loss_means, step->loss_running_min, step->loss_decays, step->loss_iteration, step->loss};
   const Item* seg_items = P->at<Item>(L.off_seg_items);
   double* seg_tot = P->at<double>(L.off_segtot);
   const int n_seg = (int)L.seg_items.size();
   if (n_seg > 0) hipLaunchKernelGGL(k_stat_segsum, dim3(n_seg), dim3(kThreads), 0, s, descs, seg_items, stats, seg_tot);
-  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, seg_tot, totals, lossfeat, vs, xfeat,
+  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, seg_tot, totals, ls, vs, xfeat,
                      H, nets->mix2_wt, nets->mix2_b, nets->fmix_wt, nets->fmix_b, mixbuf);
   HIP_TRY(mark());
   const int n_chunks = (T + kMixRows - 1) / kMixRows;
@@ -824,7 +821,7 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
   if (pmax != nullptr)
     hipLaunchKernelGGL(k_velo_colmax, dim3(H / 64, n_chunks), dim3(kThreads), 0, s, (const float*)mixbuf, T, H, pmax);
   hipLaunchKernelGGL(k_velo_mix, dim3(H / 64, L.Tpad / kGateBT), dim3(kThreads), 0, s, (const float*)mixbuf, T, L.Tpad, H,
-                     (const float*)pmax, n_chunks, step->lstm_h, xT);
+                     (const float*)pmax, n_chunks, step->lstm_h, xT, ls);
   HIP_TRY(mark());
   hipLaunchKernelGGL(k_velo_gates, dim3((L.Tpad / kGateBT) * (H / kGateU)), dim3(kThreads), 0, s, xT, T, L.Tpad, H,
                      nets->lstm_wt, nets->lstm_b, step->lstm_h, step->lstm_c);
@@ -916,7 +913,7 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   double* seg_tot = P->at<double>(L.off_segtot);
   const int n_seg = (int)L.seg_items.size();
   if (n_seg > 0) hipLaunchKernelGGL(k_stat_segsum, dim3(n_seg), dim3(kThreads), 0, s, descs, seg_items, stats, seg_tot);
-  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, seg_tot, totals, (const float*)nullptr, vs,
+  hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, seg_tot, totals, LossState{}, vs,
                      (float*)nullptr, 0, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
                      (const float*)nullptr, (float*)nullptr);
   HIP_TRY(mark());

@@ -71,12 +71,17 @@ def _graph_vs_eager(make_opt, step, shapes, n_warm=2, n_replay=4, seed=0):
     return ref, cap, n_warm + n_replay
 
 
-@pytest.mark.parametrize("whole_step", [False, True])
+@pytest.mark.parametrize("whole_step", [False, True, "tall"])
 def test_elo_celo2_step_replays_from_a_graph(whole_step):
     from pylo_amd import ELO_CELO2_CUDA
 
     net = _celo2_net(3)
     shapes = [(96, 64), (64,), (64, 160), (160,), (33, 7)]
+    if whole_step == "tall":
+        # a very tall matrix: Newton-Schulz takes its Gram product over 25 row slabs and adds them up with a
+        # library reduction, the Frobenius norm runs over a million elements -- both inside the graph
+        shapes = [(16400, 64), (64,)]
+        whole_step = True
 
     def make(params, capturable):
         return ELO_CELO2_CUDA(params, lr=1e-2, weight_decay=0.05, network=net, hf_key=None,

@@ -48,6 +48,7 @@ def newton_schulz(x: torch.Tensor, coeffs, iters: int, eps: float) -> torch.Tens
     c0, c1, c2 = coeffs
     if x.dim() == 3:
         split = _gram_split(x.shape[-2] if tall else x.shape[-1], min(x.shape[-2:]), x.shape[0])
+        eye_c1 = torch.eye(min(x.shape[-2:]), device=x.device, dtype=x.dtype) * c1
         for _ in range(iters):
             xt = x.transpose(-2, -1)
             if split > 1 and tall:
@@ -61,8 +62,7 @@ def newton_schulz(x: torch.Tensor, coeffs, iters: int, eps: float) -> torch.Tens
             # c1 A + c2 A A = (c2 A + c1 I) A and c0 X + B X = (B + c0 I) X: the scalings ride on the
             # diagonals of the small matrices, so every product is a plain GEMM (a GEMM that accumulates
             # into c0 X first copies X, half a gigabyte per iteration on this parameter set)
-            a2 = a * c2
-            a2.diagonal(dim1=-2, dim2=-1).add_(c1)
+            a2 = torch.add(eye_c1, a, alpha=c2)      # c2 A + c1 I in one pass
             b = torch.bmm(a2, a)
             b.diagonal(dim1=-2, dim2=-1).add_(c0)
             x = torch.bmm(x, b) if tall else torch.bmm(b, x)

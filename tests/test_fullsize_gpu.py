@@ -185,3 +185,122 @@ def test_adafac_llama_tensors():
                 worst = max(worst, e)
                 assert e <= 1.0, (t, i, shapes[i], tag, e)
     print("adafac full-size tensors worst err/tol", worst)
+
+
+def test_adafac_llama_embedding_and_block():
+    """cfg4's largest tensor, the 32000x2048 embedding (65.5 M elements: 8 000 blocks of statistics
+    partials, i.e. the two-stage segment sums, and 250 row strips of gradient sums), next to one Llama
+    block, bf16-rounded gradients, two steps against the oracle in fp64."""
+    from oracle import pylo_oracle as O
+    from pylo_amd import AdafacLO_CUDA
+    from pylo_amd.models import MetaMLP
+
+    torch.manual_seed(8)
+    net = MetaMLP(39, 32, 1)
+    shapes = [(32000, 2048), (2048,), (2048, 2048), (2048, 256), (2048, 5632), (5632, 2048)]
+    init, grads = _inputs(shapes, 11, lambda i: 1e-3)
+    grads = [[g.bfloat16().float() for g in gs] for gs in grads]
+    ref = [v.double() for v in init]
+    gpu = [torch.nn.Parameter(v.clone()) for v in init]
+    orc = O.AdafacOracle(ref, net.state_dict(), lr=1.0, device="cuda").double_()
+    opt = AdafacLO_CUDA(gpu, lr=1.0, network=copy.deepcopy(net))
+    worst = 0.0
+    for t in range(2):
+        for p, g in zip(gpu, grads[t]):
+            p.grad = g
+        orc.step([g.double() for g in grads[t]])
+        opt.step()
+        for i, p in enumerate(gpu):
+            st, so = opt.state[p], orc.state[i]
+            for tag, got, want in [("param", p, ref[i]), ("exp_avg", st["exp_avg"], so["exp_avg"]),
+                                   ("exp_avg_sq", st["exp_avg_sq"], so["exp_avg_sq"]),
+                                   ("r", st["exp_avg_sq_r"], so["exp_avg_sq_r"]),
+                                   ("c", st["exp_avg_sq_c"], so["exp_avg_sq_c"])]:
+                e = max_err(got, want, REL, ABS)
+                worst = max(worst, e)
+                assert e <= 1.0, (t, i, shapes[i], tag, e)
+    print("adafac embedding + block worst err/tol", worst)
+
+
+def _ortho_step(p_new, p_old, lr, wd):
+    """The orthogonalised, normalised step a parameter update implies: p_new = p_old - lr (s + wd p_old)."""
+    return (p_old.double() - p_new.double()) / lr - wd * p_old.double()
+
+
+def test_celo2_whole_step_at_gpt2_size():
+    """The whole ``step()`` -- fused pass, Newton-Schulz, normalise, apply -- on cfg2's embedding (the
+    tensor whose Gram product is cut into row slabs), a wide and a tall matrix and a vector, two
+    free-running steps against the oracle's literal Newton-Schulz (pylo/optim/CELO2_naive.py:59-73)
+    in fp64.  Parameters at the rel 1e-5 / abs 1e-6 bar; since lr = 3.16e-4 makes that bar loose for the
+    orthogonalised step itself, the step recovered from the update is also held to 2e-4 of its RMS."""
+    from oracle import pylo_oracle as O
+    from pylo_amd import ELO_CELO2_CUDA
+    from pylo_amd.models import CELO2MLP
+
+    torch.manual_seed(1)
+    net = CELO2MLP()
+    shapes = [(50257, 768), (768, 2304), (3072, 768), (768,)]
+    lr, wd = 3.16e-4, 0.1
+    init, grads = _inputs(shapes, 13, lambda i: 10.0 ** (-2 - i % 3))
+    ref = [v.double() for v in init]
+    gpu = [torch.nn.Parameter(v.clone()) for v in init]
+    orc = O.EloCelo2Oracle(ref, net.state_dict(), lr=lr, weight_decay=wd, adam_lr_mult=20.0, device="cuda").double_()
+    opt = ELO_CELO2_CUDA(gpu, lr=lr, weight_decay=wd, adam_lr_mult=20.0, network=net, hf_key=None)
+    worst = worst_step = 0.0
+    for t in range(2):
+        before = [(p.detach().clone(), r.clone()) for p, r in zip(gpu, ref)]
+        for p, g in zip(gpu, grads[t]):
+            p.grad = g
+        orc.step([g.double() for g in grads[t]])
+        opt.step()
+        for i, p in enumerate(gpu):
+            e = max_err(p, ref[i], REL, ABS)
+            worst = max(worst, e)
+            assert e <= 1.0, (t, i, shapes[i], "param", e)
+            if p.dim() >= 2:
+                got = _ortho_step(p.detach(), before[i][0], lr, wd)
+                want = _ortho_step(ref[i], before[i][1], lr, wd)
+                rms = float(want.pow(2).mean().sqrt())
+                assert 0.9 < rms < 1.1, (t, i, rms)                     # normalised to unit RMS
+                # fp32 parameters quantise the recovered step to ~ ulp(p) / lr; leave room for that
+                quant = float(before[i][0].abs().max()) * 2.0 ** -23 / lr
+                es = float((got - want).abs().max()) / rms
+                worst_step = max(worst_step, es)
+                assert es <= 2e-4 + 2 * quant, (t, i, shapes[i], "orthogonalised step", es, quant)
+    print("celo2 whole step worst err/tol", worst, "step err / rms", worst_step)
+
+
+def test_celo2_block_twenty_free_running_steps():
+    """One full-size GPT-2 block, 20 whole steps without ever re-synchronising parameters or state with
+    the oracle: drift stays inside the bar."""
+    from oracle import pylo_oracle as O
+    from pylo_amd import ELO_CELO2_CUDA
+    from pylo_amd.models import CELO2MLP
+
+    torch.manual_seed(1)
+    net = CELO2MLP()
+    shapes = [(768,), (768,), (768, 2304), (768, 768), (768,), (768,), (768, 3072), (3072, 768)]
+    gen = torch.Generator(device="cuda").manual_seed(17)
+    init = [torch.randn(s, generator=gen, device="cuda") * 0.02 for s in shapes]
+    ref = [v.double() for v in init]
+    gpu = [torch.nn.Parameter(v.clone()) for v in init]
+    kw = dict(lr=3.16e-4, weight_decay=0.1, adam_lr_mult=20.0)
+    orc = O.EloCelo2Oracle(ref, net.state_dict(), device="cuda", **kw).double_()
+    opt = ELO_CELO2_CUDA(gpu, network=net, hf_key=None, **kw)
+    worst = 0.0
+    for t in range(20):
+        grads = [torch.randn(s, generator=gen, device="cuda") * 10.0 ** (-2 - i % 3) for i, s in enumerate(shapes)]
+        for p, g in zip(gpu, grads):
+            p.grad = g
+        orc.step([g.double() for g in grads])
+        opt.step()
+        for i, p in enumerate(gpu):
+            e = max_err(p, ref[i], REL, ABS)
+            worst = max(worst, e)
+            assert e <= 1.0, (t, i, shapes[i], e)
+    for i, p in enumerate(gpu):
+        st, so = opt.state[p], orc.state[i]
+        for k in ("mom", "rms", "fac_r", "fac_c"):
+            if k in so and k in st:
+                assert max_err(st[k], so[k], REL, ABS) <= 1.0, (i, k)
+    print("celo2 block, 20 free-running steps: worst err/tol", worst)

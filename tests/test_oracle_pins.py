@@ -259,3 +259,42 @@ def test_loss_accumulators_closed_forms():
     acc2.update(torch.tensor(1000.0))                    # clipped to 2 * max corrected mean = 2
     cor2 = acc2.means / (1 - acc2.decays ** 2)
     assert float(cor2.max()) <= 2.0 + 1e-5
+
+
+# ---------------------------------------------------------------- per-parameter step counters (AdafacLO)
+def test_adafac_per_param_step_equals_single_parameter_runs():
+    """AdafacLO_cuda.py:304-305,400: every parameter's time features follow its own step counter.
+    AdafacLO tensors do not interact, so the switch is fixed by a property that needs no second
+    implementation: a parameter that sat steps out must end exactly where a single-parameter run, fed
+    only the steps it took part in (and counting per group, the golden-pinned default), ends."""
+    from pylo_amd.models import MetaMLP
+
+    torch.manual_seed(21)
+    net = MetaMLP(39, 32, 1).state_dict()
+    shapes = [(6, 10), (7,), (3, 4, 5)]
+    gen = torch.Generator().manual_seed(9)
+    init = [torch.randn(s, generator=gen) * 0.3 for s in shapes]
+    sat_out = {0: {1, 2}, 1: {4}, 2: set()}          # parameter -> steps without a gradient
+    steps = 6
+    grads = [[None if t in sat_out[i] else torch.randn(s, generator=gen) * 0.1 for i, s in enumerate(shapes)]
+             for t in range(steps)]
+    both = [v.clone() for v in init]
+    orc = O.AdafacOracle(both, net, lr=0.5, per_param_step=True)
+    for t in range(steps):
+        orc.step(grads[t])
+    assert orc.steps == [4, 5, 6]
+    for i in range(len(shapes)):
+        alone = [init[i].clone()]
+        solo = O.AdafacOracle(alone, net, lr=0.5)     # per group: t counts the calls it received
+        for t in range(steps):
+            if grads[t][i] is not None:
+                solo.step([grads[t][i]])
+        assert torch.equal(both[i], alone[0]), i
+        for k in ("exp_avg", "exp_avg_sq", "exp_avg_sq_r", "exp_avg_sq_c"):
+            assert torch.equal(orc.state[i][k], solo.state[0][k]), (i, k)
+    # and the switch matters: counting per group moves the lagging parameter elsewhere
+    grp = [v.clone() for v in init]
+    orc_g = O.AdafacOracle(grp, net, lr=0.5)
+    for t in range(steps):
+        orc_g.step(grads[t])
+    assert not torch.equal(grp[0], both[0]) and torch.equal(grp[2], both[2])

@@ -290,6 +290,22 @@ int pylo_mi355_celo2_kernel(const float* g, const float* p, const float* m, cons
                             const float* b_out, float* step_out, float exp_mult, const int64_t* shape,
                             int ndim, int dc, int dr, int vector_like, void* stream);
 
+/* pylo_mi355_celo2_kernel without the `second_moment` argument.  No counterpart in the reference: it is
+   for callers that cannot allocate device memory -- code under HIP graph capture, tight serving loops,
+   harnesses that forbid hipMalloc -- and so cannot supply (and zero) that buffer per call.  The per-channel
+   sums live in a 256-byte device array inside the library (one copy per GPU, held until the process ends)
+   that the call clears with a small kernel before it accumulates into it; the call itself allocates and
+   frees nothing.  Limit: tensors of up to 2^31 - 1 elements, as for pylo_mi355_celo2_kernel (the array does
+   not grow with the tensor); larger ones are refused with an error.  Every call on a GPU shares that GPU's
+   array: calls that may overlap on one GPU (two streams, two threads) race on the sums and must be
+   serialised by the caller.  The GPU used is the calling thread's current device. */
+int pylo_mi355_celo2_kernel_noalloc(const float* g, const float* p, const float* m, const float* v,
+                                    const float* fac_r, const float* fac_c, const float* row_factor,
+                                    const float* col_factor, const float* w_in, const float* b_in,
+                                    const float* w_h, const float* b_h, const float* w_out, const float* b_out,
+                                    float* step_out, float exp_mult, const int64_t* shape, int ndim, int dc,
+                                    int dr, int vector_like, void* stream);
+
 /* cuda_lo.learned_optimizer_kernel (pylo/csrc/learned_optimizer.cu:303-404): 28 features (eps 1e-5) +
    11 tanh(step / ts - 1) features, 39 -> 32 -> 32 -> 2 MLP with (out, in) weights;
    p -= lr * o0 * exp(o1 * exp_mult) * step_mult.  `weight_decay` is accepted and unused, as in the

@@ -15,6 +15,8 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
+#include <string>
 #include <vector>
 
 #include "k_celo2.h"
@@ -979,12 +981,19 @@ int single_geometry(const char* who, const int64_t* shape, int ndim, int dc, int
 }
 
 template <int F>
-int single_launch(const char* who, const SingleArgs& a, void* stream) {
+int single_check(const char* who, const SingleArgs& a) {
   if (a.n == 0) return 0;
   if (!a.g || !a.p || !a.m || !a.v || !a.fac_r || !a.fac_c || !a.row_factor || !a.second_moment || !a.w_in ||
       !a.b_in || !a.w_h || !a.b_h || !a.w_out || !a.b_out || (!a.vector_like && !a.col_factor) ||
       (F == kFamCelo2 && !a.step_out))
     return fail(std::string(who) + ": null pointer");
+  return 0;
+}
+
+template <int F>
+int single_launch(const char* who, const SingleArgs& a, void* stream) {
+  if (a.n == 0) return 0;
+  if (int rc = single_check<F>(who, a)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int blocks = std::min((a.n + kSingleThreads - 1) / kSingleThreads, kSingleMaxBlocks);
   hipLaunchKernelGGL(k_single_moment<F>, dim3(blocks), dim3(kSingleThreads), 0, s, a);
@@ -1047,6 +1056,63 @@ extern "C" int pylo_mi355_velo_kernel_simple(const float* grad, float* param, co
   a.w_out = output_weights; a.b_out = output_bias;
   a.lr = lr; a.step_mult = step_mult; a.exp_mult = exp_mult; a.epsilon = epsilon; a.weight_decay = weight_decay;
   return single_launch<kFamVelo>("velo_kernel_simple", a, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// celo2_kernel for callers that cannot allocate: the per-channel sums live in the library's own
+// device array instead of a caller-supplied `second_moment`
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+constexpr int kScratchFloats = 64;   // 30 channel sums, padded to one 256-byte line
+static __device__ __align__(256) float scratch[kScratchFloats];
+
+constexpr int kMaxDevices = 64;
+float* g_scratch_ptr[kMaxDevices];   // device address of `scratch` per GPU, resolved on first use
+std::mutex g_scratch_mu;
+
+// The array's name is a host-side stand-in, not a device address: each GPU holds its own copy at its
+// own address, looked up once per device with that device current.
+int scratch_on_current_device(float** out) {
+  int dev = -1;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail("celo2_kernel_noalloc: device index out of range");
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) return fail("celo2_kernel_noalloc: no device address for the scratch array");
+    g_scratch_ptr[dev] = static_cast<float*>(ptr);
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+// a fill kernel rather than a memset node: callers may record the call into a HIP graph
+__global__ __launch_bounds__(64) void k_scratch_clear(float* __restrict__ s) { s[threadIdx.x] = 0.0f; }
+
+}  // namespace
+
+extern "C" int pylo_mi355_celo2_kernel_noalloc(const float* g, const float* p, const float* m, const float* v,
+                                               const float* fac_r, const float* fac_c, const float* row_factor,
+                                               const float* col_factor, const float* w_in, const float* b_in,
+                                               const float* w_h, const float* b_h, const float* w_out,
+                                               const float* b_out, float* step_out, float exp_mult,
+                                               const int64_t* shape, int ndim, int dc, int dr, int vector_like,
+                                               void* stream) {
+  SingleArgs a{};
+  if (int rc = single_geometry("celo2_kernel_noalloc", shape, ndim, dc, dr, vector_like, a)) return rc;
+  float* sums = nullptr;
+  if (int rc = scratch_on_current_device(&sums)) return rc;
+  a.g = g; a.p = const_cast<float*>(p); a.m = m; a.v = v; a.fac_r = fac_r; a.fac_c = fac_c;
+  a.row_factor = row_factor; a.col_factor = col_factor; a.second_moment = sums;
+  a.w_in = w_in; a.b_in = b_in; a.w_h = w_h; a.b_h = b_h; a.w_out = w_out; a.b_out = b_out;
+  a.step_out = step_out; a.exp_mult = exp_mult;
+  if (a.n == 0) return 0;
+  if (int rc = single_check<kFamCelo2>("celo2_kernel_noalloc", a)) return rc;
+  // the array keeps the previous call's sums: they start at zero on every call
+  hipLaunchKernelGGL(k_scratch_clear, dim3(1), dim3(kScratchFloats), 0, static_cast<hipStream_t>(stream), sums);
+  return single_launch<kFamCelo2>("celo2_kernel_noalloc", a, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -3,6 +3,10 @@
 
 #include "pylo_common.h"
 
+#ifndef PYLO_STATS_UNROLL
+#define PYLO_STATS_UNROLL 2   // rows of the statistics walk whose loads are issued together
+#endif
+
 namespace pylo {
 
 struct EmaConsts {
@@ -265,8 +269,8 @@ struct TileTask {
   long long first;     // element index of (r0, first column of the wave)
   __device__ __forceinline__ TileTask(const TDesc& d, int task, int nct, int V) {
     const int ct = task % nct, rr = task / nct;
-    r0 = rr * kTileRows;
-    r1 = r0 + kTileRows < d.R0 ? r0 + kTileRows : d.R0;
+    r0 = rr * d.tile_rows;
+    r1 = r0 + d.tile_rows < d.R0 ? r0 + d.tile_rows : d.R0;
     col = (unsigned)ct * (64 * V) + (threadIdx.x & 63) * V;
     first = (long long)r0 * d.C0 + (long long)ct * (64 * V);
   }
@@ -275,6 +279,10 @@ struct TileTask {
 
 // Statistics of one wave task: the column factors stay in registers, the row factors arrive through
 // the scalar cache, and the only per-row vector memory traffic is the six streams.
+// KEEP: plain loads, which leave the lines in the memory-side cache for the apply items that follow a
+// few thousand blocks later (k_celo2_elem); otherwise non-temporal loads, the faster way to stream
+// data that will have been evicted before anyone reads it again.
+template <bool KEEP>
 __device__ __forceinline__ void celo2_stats_tile(const TDesc& d, const PyloTensorArgs& a, int task, float scale,
                                                  const EmaConsts& e, const float* f0, const float* f1,
                                                  float (&acc)[kNStat]) {
@@ -287,15 +295,24 @@ __device__ __forceinline__ void celo2_stats_tile(const TDesc& d, const PyloTenso
   const float *g = a.grad + tk.first, *p = a.param + tk.first, *m0 = a.mom + tk.first,
               *m1 = a.mom + d.n + tk.first, *m2 = a.mom + 2 * d.n + tk.first, *rms = a.rms + tk.first;
   const float* fr = f0 + (size_t)tk.r0 * 4;
-#pragma unroll 2
+#pragma unroll PYLO_STATS_UNROLL
   for (int r = tk.r0; r < tk.r1; ++r) {
     float xg[V], xp[V], x0[V], x1[V], x2[V], xr[V], fa[4];
-    load_vec_nt<V>(g, lo, xg);
-    load_vec_nt<V>(p, lo, xp);
-    load_vec_nt<V>(m0, lo, x0);
-    load_vec_nt<V>(m1, lo, x1);
-    load_vec_nt<V>(m2, lo, x2);
-    load_vec_nt<V>(rms, lo, xr);
+    if constexpr (KEEP) {
+      load_vec_o<V>(g, lo, xg);
+      load_vec_o<V>(p, lo, xp);
+      load_vec_o<V>(m0, lo, x0);
+      load_vec_o<V>(m1, lo, x1);
+      load_vec_o<V>(m2, lo, x2);
+      load_vec_o<V>(rms, lo, xr);
+    } else {
+      load_vec_nt<V>(g, lo, xg);
+      load_vec_nt<V>(p, lo, xp);
+      load_vec_nt<V>(m0, lo, x0);
+      load_vec_nt<V>(m1, lo, x1);
+      load_vec_nt<V>(m2, lo, x2);
+      load_vec_nt<V>(rms, lo, xr);
+    }
     load_uniform<4>(fr, fa);
 #pragma unroll
     for (int v = 0; v < V; ++v) {
@@ -313,20 +330,13 @@ __device__ __forceinline__ void celo2_stats_tile(const TDesc& d, const PyloTenso
   }
 }
 
-// Statistics pass: sum of squares of the 18 per-element channels of every MLP tensor, with the
-// accumulators advanced in registers only (nothing is written back).  AdamW tensors are updated
-// completely here.
-__global__ __launch_bounds__(kThreads) void k_celo2_stats(const TDesc* __restrict__ descs,
-                                                          const PyloTensorArgs* __restrict__ dyn,
-                                                          const Item* __restrict__ items,
-                                                          const float* __restrict__ fac_tab,
-                                                          const Globals* __restrict__ gl, PyloDecays dec,
-                                                          double* __restrict__ stats_part) {
-  __shared__ float red[kWaves][kNStat];
-  const Item it = items[blockIdx.x];
-  const TDesc d = descs[it.tensor];
-  const PyloTensorArgs a = dyn[it.tensor];
-  if (a.grad == nullptr) return;
+// One block of the statistics pass: sum of squares of the 18 per-element channels over the block's
+// elements, with the accumulators advanced in registers only (nothing is written back); an AdamW tensor
+// is updated completely instead.  Returns true when `red` holds the four waves' sums (after a barrier).
+template <bool KEEP>
+__device__ __forceinline__ bool celo2_stats_block(const TDesc& d, const PyloTensorArgs& a, const Item& it,
+                                                  const float* __restrict__ fac_tab, const Globals* __restrict__ gl,
+                                                  const PyloDecays& dec, float (*red)[kNStat]) {
   const float scale = clip_scale(gl->gnorm, a.clip_norm);
   const EmaConsts e = make_ema(dec);
   if (d.mode == kModeFlat) {
@@ -337,7 +347,7 @@ __global__ __launch_bounds__(kThreads) void k_celo2_stats(const TDesc* __restric
       if (d.vec == 4) celo2_adam_chunk<4>(d, a, it.a, scale, e);
       else celo2_adam_chunk<1>(d, a, it.a, scale, e);
     }
-    return;
+    return false;
   }
   float acc[kNStat];
 #pragma unroll
@@ -347,7 +357,7 @@ __global__ __launch_bounds__(kThreads) void k_celo2_stats(const TDesc* __restric
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   if (d.tile_nct > 0) {
     const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(wave);
-    if (task < d.tile_ntask) celo2_stats_tile(d, a, task, scale, e, f0, f1, acc);
+    if (task < d.tile_ntask) celo2_stats_tile<KEEP>(d, a, task, scale, e, f0, f1, acc);
   } else if (d.vec == 4) {
     celo2_stats_chunk<4>(d, a, it.a, scale, e, f0, f1, acc);
   } else {
@@ -359,36 +369,61 @@ __global__ __launch_bounds__(kThreads) void k_celo2_stats(const TDesc* __restric
     if (lane == 0) red[wave][c] = s;
   }
   __syncthreads();
-  if (threadIdx.x < kNStat) {
-    const int c = threadIdx.x;
-    stats_part[(size_t)blockIdx.x * kStatW + stat_channel(c)] =
-        ((double)red[0][c] + (double)red[1][c]) + ((double)red[2][c] + (double)red[3][c]);
-  }
+  return true;
+}
+
+__device__ __forceinline__ double stats_block_total(const float (*red)[kNStat], int c) {
+  return ((double)red[0][c] + (double)red[1][c]) + ((double)red[2][c] + (double)red[3][c]);
+}
+
+// Statistics pass as a launch of its own (each pass over all tensors; the fused element pass,
+// k_celo2_elem, is the default).
+__global__ __launch_bounds__(kThreads) void k_celo2_stats(const TDesc* __restrict__ descs,
+                                                          const PyloTensorArgs* __restrict__ dyn,
+                                                          const Item* __restrict__ items,
+                                                          const float* __restrict__ fac_tab,
+                                                          const Globals* __restrict__ gl, PyloDecays dec,
+                                                          double* __restrict__ stats_part) {
+  __shared__ float red[kWaves][kNStat];
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  if (!celo2_stats_block<false>(d, a, it, fac_tab, gl, dec, red)) return;
+  if (threadIdx.x < kNStat)
+    stats_part[(size_t)blockIdx.x * kStatW + stat_channel(threadIdx.x)] = stats_block_total(red, threadIdx.x);
 }
 
 // Per factored tensor: s_c = rsqrt(1e-9 + mean f_c^2) folded into the first-layer rows of the 18
-// per-element channels; the remaining layers are copied behind them so the apply kernel reads one
-// contiguous block per tensor.
-__global__ __launch_bounds__(kFoldThreads) void k_celo2_fold(const TDesc* __restrict__ descs,
-                                                             const PyloTensorArgs* __restrict__ dyn,
-                                                             const int* __restrict__ fac_list,
-                                                             const double* __restrict__ stats_part,
-                                                             const double* __restrict__ seg_tot,
-                                                             const float* __restrict__ mlp,
-                                                             float* __restrict__ wfold, float* __restrict__ chan_ms) {
-  constexpr int G = kFoldThreads / kNStat;  // 56 groups x 18 channels
-  __shared__ double part[G][kNStat];
-  __shared__ float scale_c[kNStat];
-  const int t = fac_list[blockIdx.x];
-  const TDesc d = descs[t];
-  if (dyn[t].grad == nullptr) return;
+// per-element channels; the remaining layers are copied behind them so the apply pass reads one
+// contiguous block per tensor.  NT threads; `rows` are n_rows rows of kStatW doubles, added in a fixed
+// order.  COH: the rows were written by other blocks of the running kernel and the results are for
+// such blocks (see coh_store_wait).
+template <int NT, bool COH>
+__device__ __forceinline__ void celo2_fold_tensor(const TDesc& d, const double* __restrict__ rows, int n_rows,
+                                                  const float* __restrict__ mlp, float* __restrict__ w,
+                                                  float* __restrict__ chan_ms, double (*part)[kNStat],
+                                                  float* scale_c) {
+  constexpr int G = NT / kNStat;
   const int c = threadIdx.x % kNStat, gI = threadIdx.x / kNStat;
   if (gI < G) {
-    int n_rows;
-    const double* rows = stat_rows(d, stats_part, seg_tot, n_rows);
     double s = 0.0;
+    if constexpr (COH) {
+      // every load is a round trip to the memory side: sixteen are in flight before the first is added
+      for (int b0 = gI; b0 < n_rows; b0 += 16 * G) {
+        double v[16];
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+          const int b = b0 + q * G;
+          v[q] = b < n_rows ? coh_load(rows + (size_t)b * kStatW + stat_channel(c)) : 0.0;
+        }
+#pragma unroll
+        for (int q = 0; q < 16; ++q) s += v[q];
+      }
+    } else {
 #pragma unroll 16
-    for (int b = gI; b < n_rows; b += G) s += rows[(size_t)b * kStatW + stat_channel(c)];
+      for (int b = gI; b < n_rows; b += G) s += rows[(size_t)b * kStatW + stat_channel(c)];
+    }
     part[gI][c] = s;
   }
   __syncthreads();
@@ -400,20 +435,38 @@ __global__ __launch_bounds__(kFoldThreads) void k_celo2_fold(const TDesc* __rest
     scale_c[threadIdx.x] = rsq(1e-9f + ms);
   }
   __syncthreads();
-  float* w = wfold + (size_t)d.fac_slot * kC2Fold;
   const float* w_in = mlp;                  // (30,8)
   const float* w_h = mlp + 240 + 8;         // (8,8)
   const float* b_h = w_h + 64;              // 8
   const float* w_out = b_h + 8;             // (8,3)
   const float* b_out = w_out + 24;          // 3
-  for (int i = threadIdx.x; i < kNStat * 8; i += kFoldThreads) {
-    const int cc = i / 8, j = i % 8;
-    w[kC2W1 + i] = w_in[stat_channel(cc) * 8 + j] * scale_c[cc];
+  for (int i = threadIdx.x; i < kC2Fold; i += NT) {
+    float v;
+    if (i < kC2WH) v = w_in[stat_channel(i / 8) * 8 + i % 8] * scale_c[i / 8];
+    else if (i < kC2BH) v = w_h[i - kC2WH];
+    else if (i < kC2WO) v = b_h[i - kC2BH];
+    else if (i < kC2BO) v = ((i - kC2WO) % 4) < 2 ? w_out[((i - kC2WO) / 4) * 3 + ((i - kC2WO) % 4)] : 0.0f;
+    else v = (i - kC2BO) < 2 ? b_out[i - kC2BO] : 0.0f;
+    if constexpr (COH) coh_store_wait(w + i, v);
+    else w[i] = v;
   }
-  for (int i = threadIdx.x; i < 64; i += kFoldThreads) w[kC2WH + i] = w_h[i];
-  for (int i = threadIdx.x; i < 8; i += kFoldThreads) w[kC2BH + i] = b_h[i];
-  for (int i = threadIdx.x; i < 32; i += kFoldThreads) w[kC2WO + i] = (i % 4) < 2 ? w_out[(i / 4) * 3 + (i % 4)] : 0.0f;
-  for (int i = threadIdx.x; i < 4; i += kFoldThreads) w[kC2BO + i] = i < 2 ? b_out[i] : 0.0f;
+}
+
+__global__ __launch_bounds__(kFoldThreads) void k_celo2_fold(const TDesc* __restrict__ descs,
+                                                             const PyloTensorArgs* __restrict__ dyn,
+                                                             const int* __restrict__ fac_list,
+                                                             const double* __restrict__ stats_part,
+                                                             const double* __restrict__ seg_tot,
+                                                             const float* __restrict__ mlp,
+                                                             float* __restrict__ wfold, float* __restrict__ chan_ms) {
+  __shared__ double part[kFoldThreads / kNStat][kNStat];
+  __shared__ float scale_c[kNStat];
+  const int t = fac_list[blockIdx.x];
+  const TDesc d = descs[t];
+  if (dyn[t].grad == nullptr) return;
+  int n_rows;
+  const double* rows = stat_rows(d, stats_part, seg_tot, n_rows);
+  celo2_fold_tensor<kFoldThreads, false>(d, rows, n_rows, mlp, wfold + (size_t)d.fac_slot * kC2Fold, chan_ms, part, scale_c);
 }
 
 template <int V>
@@ -515,7 +568,7 @@ constexpr int kMfmaV = PYLO_MFMA_V;   // elements per lane and iteration on the 
 // weight block is 63 groups of four consecutive floats; lane l of register r holds float r*64 + l,
 // so group v sits in lanes 4*(v%16).. of register v/16 and is selected with abid = v % 16.  Four
 // VGPRs hold every weight.  Biases enter as a rank-1 update with the constant 1.
-template <int V>
+template <int V, bool COH>
 __device__ __forceinline__ void celo2_apply_chunk_mfma(const TDesc& d, const PyloTensorArgs& a, int chunk,
                                                        float scale, const EmaConsts& e, const float* f0,
                                                        const float* f1, const float* t0, const float* t1,
@@ -526,7 +579,7 @@ __device__ __forceinline__ void celo2_apply_chunk_mfma(const TDesc& d, const Pyl
   const int lane = threadIdx.x & 63;
   float wreg[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) wreg[r] = *(const gfloat*)(wbase + r * 64 + lane);
+  for (int r = 0; r < 4; ++r) wreg[r] = COH ? coh_load(wbase + r * 64 + lane) : *(const gfloat*)(wbase + r * 64 + lane);
   constexpr int gWH = kC2WH / 4, gBH = kC2BH / 4, gWO = kC2WO / 4, gBO = kC2BO / 4;
   const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
   Cursor<V, 4> cur(d, base);
@@ -610,6 +663,7 @@ __device__ __forceinline__ void celo2_apply_chunk_mfma(const TDesc& d, const Pyl
 
 // The matrix-pipe apply pass over one wave task of the column-resident walk: column factors and
 // column terms stay in registers, row factors and row terms arrive through the scalar cache.
+template <bool COH>
 __device__ __forceinline__ void celo2_apply_tile(const TDesc& d, const PyloTensorArgs& a, int task, float scale,
                                                  const EmaConsts& e, const float* f0, const float* f1,
                                                  const float* t0, const float* t1, const float* wbase) {
@@ -620,7 +674,7 @@ __device__ __forceinline__ void celo2_apply_tile(const TDesc& d, const PyloTenso
   const int lane = threadIdx.x & 63;
   float wreg[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) wreg[r] = *(const gfloat*)(wbase + r * 64 + lane);
+  for (int r = 0; r < 4; ++r) wreg[r] = COH ? coh_load(wbase + r * 64 + lane) : *(const gfloat*)(wbase + r * 64 + lane);
   constexpr int gWH = kC2WH / 4, gBH = kC2BH / 4, gWO = kC2WO / 4, gBO = kC2BO / 4;
   const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
   float fb[V][4], tb[V][8];
@@ -700,13 +754,39 @@ __device__ __forceinline__ void celo2_apply_tile(const TDesc& d, const PyloTenso
 #pragma unroll
     for (int v = 0; v < V; ++v)
       res[v] = use_exp ? o[v][0] * __builtin_amdgcn_exp2f(o[v][1] * exp_scale) : o[v][0];
-    store_vec_o<V>(out, lo, res);
+    store_vec_nt<V>(out, lo, res);
     g += d.C0; p += d.C0; m0 += d.C0; m1 += d.C0; m2 += d.C0; rms += d.C0; out += d.C0;
     fr += 4; tr += 8;
   }
 }
 
-// Apply pass: accumulators advanced and written, features, MLP, raw step.
+// One block of the apply pass: accumulators advanced and written, features, MLP, raw step.
+// COH: the tensor's folded weights were written by another block of the running kernel.
+template <bool MFMA, bool COH>
+__device__ __forceinline__ void celo2_apply_block(const TDesc& d, const PyloTensorArgs& a, const Item& it,
+                                                  const float* __restrict__ fac_tab,
+                                                  const float* __restrict__ term_tab, const Globals* __restrict__ gl,
+                                                  const PyloDecays& dec, const float* __restrict__ wfold) {
+  const float scale = clip_scale(gl->gnorm, a.clip_norm);
+  const EmaConsts e = make_ema(dec);
+  const float* w = wfold + (size_t)d.fac_slot * kC2Fold;
+  if (MFMA && d.tile_nct > 0) {
+    const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (task < d.tile_ntask)
+      celo2_apply_tile<COH>(d, a, task, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
+                            term_tab + d.term_off[0], term_tab + d.term_off[1], w);
+  } else if (MFMA && d.vec == 4)
+    celo2_apply_chunk_mfma<kMfmaV, COH>(d, a, it.a, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
+                                        term_tab + d.term_off[0], term_tab + d.term_off[1], w);
+  else if (d.vec == 4)
+    celo2_apply_chunk<4>(d, a, it.a, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
+                         term_tab + d.term_off[0], term_tab + d.term_off[1], w);
+  else
+    celo2_apply_chunk<1>(d, a, it.a, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
+                         term_tab + d.term_off[0], term_tab + d.term_off[1], w);
+}
+
+// Apply pass as a launch of its own (see k_celo2_stats).
 template <bool MFMA>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PYLO_APPLY_WAVES))) void k_celo2_apply(const TDesc* __restrict__ descs,
                                                           const PyloTensorArgs* __restrict__ dyn,
@@ -720,23 +800,92 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PYLO_A
   if (d.mode == kModeFlat) return;
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
-  const float scale = clip_scale(gl->gnorm, a.clip_norm);
-  const EmaConsts e = make_ema(dec);
-  const float* w = wfold + (size_t)d.fac_slot * kC2Fold;
-  if (MFMA && d.tile_nct > 0) {
-    const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (task < d.tile_ntask)
-      celo2_apply_tile(d, a, task, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
-                       term_tab + d.term_off[0], term_tab + d.term_off[1], w);
-  } else if (MFMA && d.vec == 4)
-    celo2_apply_chunk_mfma<kMfmaV>(d, a, it.a, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
-                                   term_tab + d.term_off[0], term_tab + d.term_off[1], w);
-  else if (d.vec == 4)
-    celo2_apply_chunk<4>(d, a, it.a, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
-                         term_tab + d.term_off[0], term_tab + d.term_off[1], w);
-  else
-    celo2_apply_chunk<1>(d, a, it.a, scale, e, fac_tab + d.fac_off[0], fac_tab + d.fac_off[1],
-                         term_tab + d.term_off[0], term_tab + d.term_off[1], w);
+  celo2_apply_block<MFMA, false>(d, a, it, fac_tab, term_tab, gl, dec, wfold);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The fused element pass: statistics, weight folding and apply pass of every tensor in ONE launch.
+//
+// The plan orders the items slab by slab (a slab is a run of whole tensors of a few million elements):
+//   stats(slab 0) stats(slab 1) stats(slab 2) apply(slab 0) stats(slab 3) apply(slab 1) ...
+// Blocks are dispatched in index order, so at any time the GPU works on the statistics of one slab
+// and on the apply items of the slab two before it, whose six input streams (24 of the apply pass's 44
+// bytes per element) are then still in the 256 MB memory-side cache: they are read from HBM once
+// instead of twice.  A launch per slab and pass does not get there: a slab fills a fraction of the
+// GPU, and every launch boundary drains it.
+//
+// What makes one launch possible is a hand-over between running blocks, per tensor:
+//   - a statistics block leaves its row of partial sums with coh_store_wait and then counts itself in
+//     (sync[t], an agent-scope atomic); the block that completes the count folds the tensor's weights
+//     (rows added in index order, whichever block comes last: results stay bit-reproducible), leaves
+//     them the same way and raises sync[T + t];
+//   - an apply block polls that flag first.  Every block it can be waiting for has a lower index, was
+//     therefore dispatched earlier and waits for nothing itself, so the wait ends; the plan puts two
+//     slabs of statistics items (hundreds of blocks, tens of microseconds) between a tensor's last
+//     statistics item and its first apply item, so it rarely begins.  A block that has polled
+//     kSpinLimit times (seconds) gives up and writes NaN steps, which no caller can overlook,
+//     rather than hang the GPU.
+// k_gnorm zeroes `sync` before every launch.
+// ---------------------------------------------------------------------------------------------
+template <bool MFMA>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PYLO_APPLY_WAVES))) void k_celo2_elem(
+    const TDesc* __restrict__ descs, const PyloTensorArgs* __restrict__ dyn, const Item* __restrict__ items,
+    const float* __restrict__ fac_tab, const float* __restrict__ term_tab, const Globals* __restrict__ gl,
+    PyloDecays dec, const float* __restrict__ mlp, float* __restrict__ wfold, float* __restrict__ chan_ms,
+    double* __restrict__ stats_part, int* __restrict__ sync, int n_tensors) {
+  __shared__ float red[kWaves][kNStat];
+  __shared__ double part[kThreads / kNStat][kNStat];
+  __shared__ float scale_c[kNStat];
+  __shared__ int s_flag;
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  if (it.c & kElemApply) {
+    if (threadIdx.x == 0) {
+      const int* ready = sync + n_tensors + it.tensor;
+      int ok = coh_load(ready);
+      for (int spin = 0; !ok && spin < kSpinLimit; ++spin) {
+        __builtin_amdgcn_s_sleep(16);
+        ok = coh_load(ready);
+      }
+      s_flag = ok;
+    }
+    __syncthreads();
+    if (s_flag) {
+      celo2_apply_block<MFMA, true>(d, a, it, fac_tab, term_tab, gl, dec, wfold);
+    } else {
+      // gave up: NaN steps for this block's elements (tile items: the wave tasks' rows; else the chunk)
+      const float nan = __builtin_nanf("");
+      if (d.tile_nct > 0) {
+        const int task = it.a * 4 + (threadIdx.x >> 6);
+        if (task < d.tile_ntask) {
+          const TileTask tk(d, task);
+          for (int r = tk.r0; r < tk.r1; ++r)
+            for (int v = 0; v < kTileV; ++v) a.step_out[(size_t)r * d.C0 + tk.col + v] = nan;
+        }
+      } else {
+        const long long chunk = (long long)kThreads * d.vec * kElemIters, base = (long long)it.a * chunk;
+        for (long long i = base + threadIdx.x; i < base + chunk && i < d.n; i += kThreads) a.step_out[i] = nan;
+      }
+    }
+    return;
+  }
+  const bool counted = (it.c & kElemKeep) ? celo2_stats_block<true>(d, a, it, fac_tab, gl, dec, red)
+                                          : celo2_stats_block<false>(d, a, it, fac_tab, gl, dec, red);
+  if (!counted) return;
+  if (threadIdx.x < kNStat)
+    coh_store_wait(stats_part + (size_t)it.b * kStatW + stat_channel(threadIdx.x), stats_block_total(red, threadIdx.x));
+  __syncthreads();   // every row entry of this block has been performed
+  if (threadIdx.x == 0)
+    s_flag = __hip_atomic_fetch_add(sync + it.tensor, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == d.nblk - 1;
+  __syncthreads();
+  if (!s_flag) return;
+  // the tensor's last statistics block: fold its weights
+  celo2_fold_tensor<kThreads, true>(d, stats_part + (size_t)d.blk0 * kStatW, d.nblk, mlp,
+                                    wfold + (size_t)d.fac_slot * kC2Fold, chan_ms, part, scale_c);
+  __syncthreads();   // every folded weight has been performed
+  if (threadIdx.x == 0) __hip_atomic_store(sync + n_tensors + it.tensor, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -190,9 +190,12 @@ __global__ __launch_bounds__(kThreads) void k_p0(const TDesc* __restrict__ descs
 // gradient is bounded by clip_norm), so the exact pass never runs and the flags are ignored.
 __global__ __launch_bounds__(kThreads) void k_gnorm(const double* __restrict__ gsq_part,
                                                     const int* __restrict__ flag_part, int nblk,
-                                                    Globals* __restrict__ gl, int use_flags) {
+                                                    Globals* __restrict__ gl, int use_flags,
+                                                    int* __restrict__ sync, int n_sync) {
   __shared__ double red[kWaves];
   __shared__ int fred[kWaves];
+  // the counters and flags of the fused element pass that follows (k_celo2_elem) start at zero
+  for (int i = threadIdx.x; i < n_sync; i += kThreads) sync[i] = 0;
   double s = 0.0;
   int f = 0;
   // sixteen partials are fetched before the first is added: the one block is bound by load latency

@@ -17,7 +17,7 @@ constexpr int kP0Rows = 128;    // rows of one row/column-sum tile; tile columns
 constexpr int kElemIters = 8;   // an element chunk is kThreads * vec * kElemIters elements
 constexpr int kTileV = 2;       // column-resident walk: a wave owns 64 * kTileV columns ...
 constexpr int kTileCols = 64 * kTileV;
-constexpr int kTileRows = 16;   // ... and walks this many rows of them
+constexpr int kTileRows = 16;   // ... and walks this many rows of them (TDesc::tile_rows; ELO-CELO2 plans may choose fewer)
 constexpr int kNStat = 18;      // feature channels that vary per element (the other 12 are
                                 // functions of the row or of the column only)
 constexpr int kV0aEnt = 64;     // vector entries per k_v0a block
@@ -94,9 +94,9 @@ struct TDesc {
   long long term_off[2];  // floats, first-layer terms [entry][H]
   int v0a_first[2], v0a_n[2];  // k_v0a blocks of vector 0 / 1
   // Column-resident walk (wide 2-D tensors, C0 % kTileCols == 0): wave task w covers columns
-  // [ (w % tile_nct) * kTileCols, +kTileCols ) of rows [ (w / tile_nct) * kTileRows, +kTileRows );
+  // [ (w % tile_nct) * kTileCols, +kTileCols ) of rows [ (w / tile_nct) * tile_rows, +tile_rows );
   // element block a holds tasks 4a .. 4a+3.  tile_nct == 0: linear chunks instead.
-  int tile_nct, tile_ntask;
+  int tile_nct, tile_ntask, tile_rows;
   // AdafacLO's apply pass walks one column per lane (its 32-wide MLP leaves no registers for two):
   // same scheme with 64 columns per wave task; apply block a holds tasks 4a .. 4a+3.
   int atile_nct, atile_ntask;
@@ -141,6 +141,11 @@ struct Globals {
   float gnorm;  // ||all grads||_2
   int flag;     // some |g| exceeded clip_val on a tensor whose sums were taken un-clamped
 };
+
+// Item::c of the fused element pass of ELO-CELO2 (k_celo2_elem)
+constexpr int kElemApply = 1;   // apply item (else statistics item); Item::b is the row of the statistics partials
+constexpr int kElemKeep = 2;    // statistics item whose inputs the apply pass re-reads from the memory-side cache
+constexpr int kSpinLimit = 2000000;   // polls of a tensor's "folded weights ready" flag before a block gives up
 
 // Per factored tensor, written by k_v0b: normalisation scales of the 12 broadcast channels in the
 // reference's channel order 15..26 (fac_r_k, fac_c_k, rsqrt(fac_r_k+1e-8), rsqrt(fac_c_k+1e-8)).
@@ -382,6 +387,34 @@ __device__ __forceinline__ v4f mfma_w4(float wreg, float b, v4f c, int abid) {
 // max(x, 0) for finite x as one median-of-three (no NaN-quieting pre-pass as fmaxf needs; written
 // with a compiler builtin so the hazard recogniser sees an ordinary VALU instruction after an MFMA)
 __device__ __forceinline__ float relu(float x) { return __builtin_amdgcn_fmed3f(x, 0.0f, 3.0e38f); }
+
+// ---- values handed from one running block to another (the fused element pass of ELO-CELO2) -------
+// Ordinary loads and stores go through an L2 that is private to each of the eight XCDs, so a value
+// written by a block on one XCD is not seen by a block on another before the kernel ends.  Agent-scope
+// atomics are performed at the memory side, which all XCDs share.  A producer writes its values with
+// atomic exchanges, whose returned old values it waits for (then the writes have been performed), and
+// only then announces them with a counter or flag, again an atomic; a consumer reads with atomic loads.
+// No fence is used: a release fence writes back the XCD's whole L2 and costs microseconds per block.
+__device__ __forceinline__ void coh_store_wait(float* p, float v) {
+  const float old = __hip_atomic_exchange(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  asm volatile("" ::"v"(old) : "memory");   // the old value has arrived: the exchange has been performed
+}
+__device__ __forceinline__ void coh_store_wait(double* p, double v) {
+  const unsigned long long old = __hip_atomic_exchange(reinterpret_cast<unsigned long long*>(p),
+                                                       __builtin_bit_cast(unsigned long long, v), __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT);
+  asm volatile("" ::"v"(old) : "memory");
+}
+__device__ __forceinline__ float coh_load(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ double coh_load(const double* p) {
+  return __builtin_bit_cast(double, __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED,
+                                                      __HIP_MEMORY_SCOPE_AGENT));
+}
+__device__ __forceinline__ int coh_load(const int* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 // Makes the compiler forget what it knows about a (wave-uniform) pointer, so loads through it
 // are re-issued where they are written instead of being hoisted out of the enclosing loop; the

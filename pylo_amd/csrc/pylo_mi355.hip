@@ -1,16 +1,20 @@
 // Fused learned-optimizer step for MI355X (gfx950): the C ABI of include/pylo_mi355.h.
 //
-// Pipeline of one ELO-CELO2 step over all tensors of a plan (8 launches, no host sync):
+// Pipeline of one ELO-CELO2 step over all tensors of a plan (6 launches, no host sync):
 //   k_p0 (pass 0)   row / column sums of g^2 per tile, sum g^2 and clamp flag per block     4 B/elem
 //   k_gnorm         global gradient norm, clamp flag
 //   k_p0 (pass 1)   exits at once unless some |g| exceeded the clamp: redoes the sums exactly
 //   k_v0a           fac_r / fac_c EMAs per 64 vector entries, partial sums of their statistics
 //   k_v0b           row / column factor tables; the 12 row-only / column-only feature channels
 //                   normalised and folded into 8-float first-layer terms per row / column
-//   k_celo2_stats   sum of squares of the 18 per-element channels (accumulators advanced in
+//   k_celo2_elem    one launch, items ordered slab by slab (k_celo2.h):
+//     statistics    sum of squares of the 18 per-element channels (accumulators advanced in
 //                   registers, nothing written); AdamW tensors are fully updated here      24 B/elem
-//   k_celo2_fold    per tensor: normalisation scales folded into the first-layer weights
-//   k_celo2_apply   accumulators advanced and written, features, MLP, step_out             44 B/elem
+//     fold          per tensor, by its last statistics block: normalisation scales folded into the
+//                   first-layer weights
+//     apply         accumulators advanced and written, features, MLP, step_out             44 B/elem
+//   (PYLO_MI355_SLAB_ELEMS=0: k_celo2_stats, k_stat_segsum, k_celo2_fold, k_celo2_apply as launches
+//   of their own, each over all tensors)
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
@@ -66,6 +70,8 @@ bool factored_dims(int kind, const PyloTensorShape& s, int* dc, int* dr) {
 }
 
 struct Layout {
+  std::vector<Item> mx_items;   // ELO-CELO2: statistics and apply items in slab order (k_celo2_elem)
+  size_t off_mx_items = 0, off_sync = 0;
   std::vector<TDesc> descs;
   std::vector<Item> p0_items, nd_items, sl_items, seg_items, el_items, ap_items, ga_items, fin_items, v0a_items, v0b_items;
   std::vector<int> fac_list;
@@ -86,6 +92,86 @@ int first_layer_width(int kind) { return kind == PYLO_KIND_CELO2 ? 8 : kind == P
 bool env_matrix_pipe() {
   const char* v = std::getenv("PYLO_MI355_VALU_MLP");
   return !(v && v[0] == '1');
+}
+
+// Elements per slab of the fused element pass of ELO-CELO2 (k_celo2_elem).  While the apply items of one
+// slab run, the statistics items of the third slab after it do, with the slabs between them resident
+// as well: four slabs of 24 bytes per element plus the 20 bytes per element the apply items write
+// must fit the 256 MB memory-side cache (measured on the GPT-2-small set: 1.2 M elements 1.51 ms a step,
+// 2.4 M 1.48, 3.6 M 1.48, 4.8 M 1.72).  PYLO_MI355_SLAB_ELEMS=0 in the environment (read at plan
+// creation) runs each pass over all tensors as a launch of its own instead.
+long long env_slab_elems() {
+  const char* v = std::getenv("PYLO_MI355_SLAB_ELEMS");
+  if (v && v[0]) return std::atoll(v);
+  return 2400000;
+}
+int env_slab_depth() {   // slabs of statistics items between a slab's statistics and its apply items
+  const char* v = std::getenv("PYLO_MI355_SLAB_DEPTH");
+  return (v && v[0]) ? std::max(1, std::atoi(v)) : 3;
+}
+long long env_keep_elems() {   // largest tensor whose inputs are still expected in the cache when its apply items run
+  const char* v = std::getenv("PYLO_MI355_KEEP_ELEMS");
+  return (v && v[0]) ? std::atoll(v) : 8000000;
+}
+
+int tile_rows_for(int kind) {
+  const char* v = std::getenv("PYLO_MI355_TILE_ROWS");
+  if (kind == PYLO_KIND_CELO2 && v && v[0] && std::atoi(v) > 0) return std::atoi(v);
+  return kTileRows;
+}
+
+// Items of k_celo2_elem.  Slabs are runs of whole tensors, last tensors first (their gradients are what
+// k_p0 read last).  A tensor too large to stay cached is streamed: its statistics items are cut into
+// slab-sized pieces (so that the apply items of the slabs before it keep their place two pieces behind),
+// and its apply items follow its last piece, last item first: they start on what was read last.
+void build_elem_items(Layout& L, int T) {
+  struct Piece { int st0, st1, ap0, ap1; bool keep; };   // statistics items [st0, st1); apply items [ap0, ap1) or none
+  const long long cap = env_slab_elems(), keep_max = env_keep_elems();
+  if (cap <= 0) return;
+  std::vector<Piece> pieces;
+  long long elems = 0;
+  int el_hi = -1, el_lo = -1;
+  auto close = [&]() {
+    if (el_hi > el_lo) pieces.push_back(Piece{el_lo, el_hi, el_lo, el_hi, true});
+    el_hi = el_lo = -1;
+    elems = 0;
+  };
+  for (int t = T - 1; t >= 0; --t) {
+    const TDesc& d = L.descs[t];
+    if (d.nblk == 0) continue;
+    if (d.n > keep_max) {
+      close();
+      const long long per_item = std::max<long long>(d.n / d.nblk, 1);
+      const int step = (int)std::max<long long>(cap / per_item, 1);
+      for (int i = d.blk0; i < d.blk0 + d.nblk; i += step) {
+        const int e = std::min(i + step, d.blk0 + d.nblk);
+        const bool last = e == d.blk0 + d.nblk;
+        pieces.push_back(Piece{i, e, last ? d.blk0 : 0, last ? d.blk0 + d.nblk : 0, false});
+      }
+      continue;
+    }
+    if (elems > 0 && elems + d.n > cap) close();
+    if (el_hi < 0) el_hi = d.blk0 + d.nblk;
+    el_lo = d.blk0;   // tensors are visited in descending order: the run grows downwards
+    elems += d.n;
+  }
+  close();
+  const int np = (int)pieces.size(), depth = env_slab_depth();
+  auto push = [&](int i0, int i1, bool apply, bool keep) {
+    const int n0 = (int)L.mx_items.size();
+    for (int i = i0; i < i1; ++i) {
+      Item it = L.el_items[i];
+      if (apply && L.descs[it.tensor].mode == kModeFlat) continue;   // AdamW tensors are finished by their statistics items
+      it.b = i;
+      it.c = apply ? kElemApply : (keep ? kElemKeep : 0);
+      L.mx_items.push_back(it);
+    }
+    if (apply && !keep) std::reverse(L.mx_items.begin() + n0, L.mx_items.end());
+  };
+  for (int k = 0; k < np + depth; ++k) {
+    if (k < np) push(pieces[k].st0, pieces[k].st1, false, pieces[k].keep);
+    if (k >= depth) push(pieces[k - depth].ap0, pieces[k - depth].ap1, true, pieces[k - depth].keep);
+  }
 }
 
 int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int velo_hidden) {
@@ -227,7 +313,8 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       for (long long s0 = 0; s0 < n_slices && n > 0; s0 += per) L.sl_items.push_back(Item{t, (int)s0, 0, 0});
     } else if (wide && d.C0 % kTileCols == 0) {
       d.tile_nct = d.C0 / kTileCols;
-      d.tile_ntask = d.tile_nct * ((d.R0 + kTileRows - 1) / kTileRows);
+      d.tile_rows = tile_rows_for(kind);
+      d.tile_ntask = d.tile_nct * ((d.R0 + d.tile_rows - 1) / d.tile_rows);
       for (int b = 0; b * 4 < d.tile_ntask; ++b) L.el_items.push_back(Item{t, b, 0, 0});
     } else {
       for (long long c = 0; c * chunk < n; ++c) L.el_items.push_back(Item{t, (int)c, 0, 0});
@@ -249,13 +336,15 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     if (kind == PYLO_KIND_ADAFAC) {
       if (wide && d.C0 % 64 == 0) {
         d.atile_nct = d.C0 / 64;
-        d.atile_ntask = d.atile_nct * ((d.R0 + kTileRows - 1) / kTileRows);
+        if (d.tile_rows == 0) d.tile_rows = tile_rows_for(kind);
+        d.atile_ntask = d.atile_nct * ((d.R0 + d.tile_rows - 1) / d.tile_rows);
         for (int b = 0; b * 4 < d.atile_ntask; ++b) L.ap_items.push_back(Item{t, b, 0, 0});
       } else {
         for (long long c = 0; c * chunk < n; ++c) L.ga_items.push_back(Item{t, (int)c, 0, 0});
       }
     }
   }
+  if (kind == PYLO_KIND_CELO2) build_elem_items(L, T);
   size_t off = 0;
   auto take = [&](size_t bytes) {
     size_t o = off;
@@ -300,6 +389,8 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_pmax = take(kind == PYLO_KIND_VELO ? sizeof(float) * (size_t)velo_hidden * ((T + kMixRows - 1) / kMixRows) : 0);
   L.off_canon = take(kind == PYLO_KIND_VELO ? sizeof(float) * kVCanon * (size_t)T : 0);
   L.off_frac = take(kind == PYLO_KIND_VELO ? sizeof(float) * 9 * PYLO_MAX_GROUPS : 0);
+  L.off_mx_items = take(sizeof(Item) * L.mx_items.size());
+  L.off_sync = take(sizeof(int) * 2 * (size_t)T);
   L.total = off;
   return 0;
 }
@@ -376,6 +467,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_fac_list, L.fac_list.data(), sizeof(int) * L.fac_list.size());
   if (e == hipSuccess) e = up(L.off_v0a_items, L.v0a_items.data(), sizeof(Item) * L.v0a_items.size());
   if (e == hipSuccess) e = up(L.off_v0b_items, L.v0b_items.data(), sizeof(Item) * L.v0b_items.size());
+  if (e == hipSuccess) e = up(L.off_mx_items, L.mx_items.data(), sizeof(Item) * L.mx_items.size());
   if (e == hipSuccess) e = hipStreamSynchronize(s);
   for (int i = 0; i < kStageSlots && e == hipSuccess; ++i) {
     e = hipHostMalloc(reinterpret_cast<void**>(&P->stage[i]), (sizeof(PyloTensorArgs) * n_tensors + 15) / 16 * 16,
@@ -403,6 +495,8 @@ int pylo_mi355_plan_destroy(PyloPlan* P) {
 
 static const char* kCelo2Launches[] = {"k_p0(sums)", "k_gnorm", "k_p0(exact)", "k_v0a", "k_v0b",
                                        "k_celo2_stats", "k_celo2_fold", "k_celo2_apply"};
+static const char* kCelo2FusedLaunches[] = {"k_p0(sums)", "k_gnorm", "k_p0(exact)", "k_v0a", "k_v0b",
+                                            "k_celo2_elem", "k_celo2_slices"};
 static const char* kVeloLaunches[] = {"k_p0(sums)", "k_p0_nd", "k_v0a", "k_v0b", "k_velo_stats",
                                       "k_lo_reduce", "k_velo_mix", "k_velo_gates", "k_velo_heads", "k_terms",
                                       "k_velo_apply"};
@@ -412,7 +506,8 @@ static const char* kAdafacLaunches[] = {"k_p0(sums)", "k_p0_nd", "k_v0a", "k_ada
 
 int pylo_mi355_plan_num_launches(const PyloPlan* P) {
   if (!P) return -1;
-  constexpr int n_celo2 = sizeof(kCelo2Launches) / sizeof(kCelo2Launches[0]);
+  const int n_celo2 = P->L.mx_items.empty() ? (int)(sizeof(kCelo2Launches) / sizeof(kCelo2Launches[0]))
+                                            : (int)(sizeof(kCelo2FusedLaunches) / sizeof(kCelo2FusedLaunches[0]));
   constexpr int n_velo = sizeof(kVeloLaunches) / sizeof(kVeloLaunches[0]);
   constexpr int n_adafac = sizeof(kAdafacLaunches) / sizeof(kAdafacLaunches[0]);
   return P->kind == PYLO_KIND_CELO2 ? n_celo2 : P->kind == PYLO_KIND_VELO ? n_velo : P->kind == PYLO_KIND_ADAFAC ? n_adafac : -1;
@@ -420,7 +515,7 @@ int pylo_mi355_plan_num_launches(const PyloPlan* P) {
 
 const char* pylo_mi355_plan_launch_name(const PyloPlan* P, int launch) {
   if (!P || launch < 0 || launch >= pylo_mi355_plan_num_launches(P)) return "";
-  return P->kind == PYLO_KIND_CELO2 ? kCelo2Launches[launch]
+  return P->kind == PYLO_KIND_CELO2 ? (P->L.mx_items.empty() ? kCelo2Launches[launch] : kCelo2FusedLaunches[launch])
          : P->kind == PYLO_KIND_VELO ? kVeloLaunches[launch] : kAdafacLaunches[launch];
 }
 
@@ -674,7 +769,8 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
     hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0,
                        (const Item*)nullptr, n_p0);
   HIP_TRY(mark());
-  hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl, exact_pass ? 1 : 0);
+  hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl, exact_pass ? 1 : 0,
+                     P->at<int>(L.off_sync), 2 * P->T);
   HIP_TRY(mark());
   if (n_p0 > 0 && exact_pass)
     hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1,
@@ -688,23 +784,36 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
     hipLaunchKernelGGL(k_v0b<8>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-9f, mlp,
                        mlp + 240, 0, fac_tab, term_tab, bscale);
   HIP_TRY(mark());
-  if (n_el > 0) hipLaunchKernelGGL(k_celo2_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, gl, dec, stats);
-  HIP_TRY(mark());
-  const Item* seg_items = P->at<Item>(L.off_seg_items);
-  double* seg_tot = P->at<double>(L.off_segtot);
-  const int n_seg = (int)L.seg_items.size();
-  if (n_seg > 0) hipLaunchKernelGGL(k_stat_segsum, dim3(n_seg), dim3(kThreads), 0, s, descs, seg_items, stats, seg_tot);
-  if (n_fac > 0)
-    hipLaunchKernelGGL(k_celo2_fold, dim3(n_fac), dim3(kFoldThreads), 0, s, descs, dyn, fac_list, stats, seg_tot, mlp, wfold,
-                       chan_ms);
-  HIP_TRY(mark());
-  if (n_el > 0) {
+  const int n_mx = (int)L.mx_items.size();
+  if (n_mx > 0) {
+    const Item* mx_items = P->at<Item>(L.off_mx_items);
+    int* sync = P->at<int>(L.off_sync);
     if (P->mlp_on_matrix_pipe)
-      hipLaunchKernelGGL(k_celo2_apply<true>, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab,
-                         term_tab, gl, dec, wfold);
+      hipLaunchKernelGGL(k_celo2_elem<true>, dim3(n_mx), dim3(kThreads), 0, s, descs, dyn, mx_items, fac_tab, term_tab,
+                         gl, dec, mlp, wfold, chan_ms, stats, sync, P->T);
     else
-      hipLaunchKernelGGL(k_celo2_apply<false>, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab,
-                         term_tab, gl, dec, wfold);
+      hipLaunchKernelGGL(k_celo2_elem<false>, dim3(n_mx), dim3(kThreads), 0, s, descs, dyn, mx_items, fac_tab, term_tab,
+                         gl, dec, mlp, wfold, chan_ms, stats, sync, P->T);
+    HIP_TRY(mark());
+  } else {
+    if (n_el > 0) hipLaunchKernelGGL(k_celo2_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, gl, dec, stats);
+    HIP_TRY(mark());
+    const Item* seg_items = P->at<Item>(L.off_seg_items);
+    double* seg_tot = P->at<double>(L.off_segtot);
+    const int n_seg = (int)L.seg_items.size();
+    if (n_seg > 0) hipLaunchKernelGGL(k_stat_segsum, dim3(n_seg), dim3(kThreads), 0, s, descs, seg_items, stats, seg_tot);
+    if (n_fac > 0)
+      hipLaunchKernelGGL(k_celo2_fold, dim3(n_fac), dim3(kFoldThreads), 0, s, descs, dyn, fac_list, stats, seg_tot, mlp, wfold,
+                         chan_ms);
+    HIP_TRY(mark());
+    if (n_el > 0) {
+      if (P->mlp_on_matrix_pipe)
+        hipLaunchKernelGGL(k_celo2_apply<true>, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab,
+                           term_tab, gl, dec, wfold);
+      else
+        hipLaunchKernelGGL(k_celo2_apply<false>, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab,
+                           term_tab, gl, dec, wfold);
+    }
   }
   if (n_sl > 0)
     hipLaunchKernelGGL(k_celo2_slices, dim3(n_sl), dim3(kThreads), 0, s, descs, dyn, sl_items, fac_tab, gl, dec, mlp);
@@ -892,7 +1001,7 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
                        nd_items, n_p0);
   if (clips) {
     const bool exact_pass = exact_pass_possible(P, args);
-    hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl, exact_pass ? 1 : 0);
+    hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl, exact_pass ? 1 : 0, (int*)nullptr, 0);
     if (n_p0 > 0 && exact_pass)
       hipLaunchKernelGGL(k_p0, dim3(n_p0), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 1,
                          (const Item*)nullptr, n_p0);

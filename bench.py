@@ -6,12 +6,14 @@ Workload (default): BASELINE config 2 -- ELO-CELO2 on a GPT-2-small-shaped fp32 
 (98 tensors, 124 355 328 parameters), synthetic per-tensor Gaussian gradients with log-uniform
 scale in [1e-5, 1e-2], random-init CELO2MLP, everything resident in HBM before timing starts.
 
-A *step* of the metric is one pass of the fused hot path: the single C-ABI call
-``pylo_mi355_celo2_step`` (7 launches: gradient statistics, accumulator updates, features, MLP,
-raw step for the 2-D tensors, AdamW for the 1-D tensors).  Its duration is measured with HIP
-events recorded by the library on the launch stream, inside full ``optimizer.step()`` calls; the
-whole ``step()`` (which adds library-GEMM Newton-Schulz, normalisation and the parameter update)
-is reported next to it as ``whole_step_ms``.
+A *step* of the metric is one whole ``optimizer.step()``: the single C-ABI call
+``pylo_mi355_celo2_step`` (gradient statistics, accumulator updates, features, MLP, raw step for the
+2-D tensors, AdamW for the 1-D tensors), Newton-Schulz on every raw step, and the finishing pass that
+normalises the steps and updates the matrices.  ``value`` is parameters updated per second by that.
+The HBM-bound part -- the C-ABI call -- is timed inside the same steps with HIP events recorded by the
+library on the launch stream (``fused_pass``, ``roofline``), and once more alone, back to back; VeLO on
+the ViT-B/16 set and AdafacLO on the Llama-1.1B set are measured after it (``velo_vitb16``,
+``llama_adafac``).
 
 Prints ONE JSON line.
 """
@@ -30,11 +32,6 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 B_P0, B_STATS, B_APPLY = 4, 24, 44   # algorithmic bytes per element of a >=2-D tensor, per pass
 B_ADAM = 44                    # 1-D AdamW branch: read g,p,m0..2,rms; write m0..2,rms,p
-# HBM bytes of one k_celo2_apply launch on the GPT-2-small set, from rocprofv3 FETCH_SIZE x 2.000 KiB +
-# WRITE_SIZE x 1.000 KiB (factors calibrated on a 1 GiB copy in the same runs; --calib-copy)
-TRAFFIC_APPLY_GPT2S = 5.528e9
-# the same for one k_velo_apply launch on the ViT-B/16 set (1 030 664 x 2 KiB fetched + 1 689 522 KiB written)
-TRAFFIC_APPLY_VITB16 = 3.841e9
 
 
 def gpt2_small_shapes():
@@ -107,13 +104,38 @@ def cpu_baseline(steps=6):
             t_all += dt
             t_fused += dt - orc.finish_seconds
     return {
-        "value": n * steps / t_fused, "unit": "params/s", "cores": torch.get_num_threads(),
+        "value": n * steps / t_all, "unit": "params/s", "cores": torch.get_num_threads(),
         "kind": "port",
         "sample": f"oracle (torch-CPU restatement of ELO_CELO2_naive) on one GPT-2-small layer "
-                  f"({n} params, {steps} steps after 1 warm-up): accumulators+features+MLP+AdamW only; "
-                  f"with Newton-Schulz/normalise/apply {n * steps / t_all:.3e} params/s",
+                  f"({n} params, {steps} whole steps after 1 warm-up: accumulators, features, MLP, AdamW, "
+                  f"Newton-Schulz, normalise, apply); without Newton-Schulz/normalise/apply "
+                  f"{n * steps / t_fused:.3e} params/s",
         "os_cpu_count": os.cpu_count(),
     }
+
+
+def ns_flops(shapes, iters=5):
+    """fp32 FLOPs of the Newton-Schulz iterations of one step (pylo/optim/CELO2_naive.py:59-73): per iteration
+    and matrix with small dim m and large dim n, A = X X^T (2 m^2 n), (c2 A + c1 I) A (2 m^3), (B + c0 I) X (2 m^2 n)."""
+    total = 0.0
+    for s in shapes:
+        if len(s) == 2:
+            m, n = min(s), max(s)
+            total += iters * (4.0 * m * m * n + 2.0 * m ** 3)
+    return total
+
+
+def traffic_from_profile(fname, kernel):
+    """HBM bytes per launch of `kernel` as the counter summary under profiles/ states them
+    (a line `traffic_bytes_per_launch <kernel> = <bytes>`); None when the file does not hold it."""
+    import re
+
+    try:
+        text = open(os.path.join(ROOT, "profiles", fname)).read()
+    except OSError:
+        return None
+    m = re.search(r"^traffic_bytes_per_launch\s+%s\s*=\s*([0-9.eE+]+)" % re.escape(kernel), text, re.M)
+    return float(m.group(1)) if m else None
 
 
 def main():
@@ -125,6 +147,8 @@ def main():
     ap.add_argument("--fused-only", action="store_true",
                     help="loop the C-ABI call alone (no Newton-Schulz / apply), e.g. under rocprofv3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra-workloads", action="store_true",
+                    help="skip the VeLO / AdafacLO sub-objects of the default line")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a 1 GiB device-to-device tensor copy (3x) so that a counter profile of "
                          "this command holds a kernel of known HBM traffic to scale FETCH_SIZE/WRITE_SIZE by")
@@ -132,13 +156,15 @@ def main():
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
 
+    import numpy as np
     import torch
 
     from pylo_amd import ELO_CELO2_CUDA
     from pylo_amd.models import CELO2MLP
 
     if a.workload in ("vit_velo", "llama_adafac"):
-        return other_workload(a)
+        print(json.dumps(other_workload(a.workload, a.steps, a.warmup)))
+        return
     if a.workload == "stream_ceiling":
         return stream_ceiling(a)
     dev = torch.device("cuda:0")
@@ -152,6 +178,7 @@ def main():
     n_params = sum(p.numel() for p in params)
     n2d = sum(p.numel() for p in params if p.dim() >= 2)
     n1d = n_params - n2d
+    bytes_fused = n2d * (B_P0 + B_STATS + B_APPLY) + n1d * B_ADAM
 
     if a.calib_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -160,64 +187,106 @@ def main():
             dst.copy_(src)                      # reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
         del src, dst
-    # 1) the timed region: K back-to-back fused steps (the C-ABI call), synchronised on both sides
-    for _ in range(a.warmup):
-        opt.fused_step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(a.steps):
-        opt.fused_step()
-    torch.cuda.synchronize()
-    fused_ms = (time.perf_counter() - t0) * 1e3 / a.steps
-    # 2) per-launch breakdown: the same steps again with the library's HIP events around every launch
-    plan = opt._plan
-    plan.timing_begin(a.steps)
-    for _ in range(a.steps):
-        opt.fused_step()
-    torch.cuda.synchronize()
-    per = plan.timing_end()                       # (steps, launches) ms
-    # 3) the whole optimizer.step() (fused path + torch Newton-Schulz / normalise / apply), a few times
-    wall_ms = None
-    if not a.fused_only:
-        opt.step()
+    plan = None
+
+    def fused_loop(k):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(5):
-            opt.step()
+        for _ in range(k):
+            opt.fused_step()
         torch.cuda.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3 / 5
+        return (time.perf_counter() - t0) * 1e3 / k
+
+    if a.fused_only:
+        for _ in range(a.warmup):
+            opt.fused_step()
+        ms = fused_loop(a.steps)
+        print(json.dumps({"metric": "fused C-ABI call alone", "ms_per_step": ms, "steps": a.steps, "warmup": a.warmup,
+                          "hbm_roofline_frac_fused_path": bytes_fused / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}))
+        return
+
+    # 1) the timed region: K whole optimizer steps.  step() is fused_step() + finish_step(); they are called one
+    #    after the other here so that events on the launch stream can mark where one ends.  The library records
+    #    its own HIP events around every launch of the C-ABI call during these same steps.
+    for _ in range(a.warmup):
+        opt.step()
+    plan = opt._plan
     names = plan.launch_names()
+    plan.timing_begin(a.steps)
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(a.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(a.steps):
+        marks[k][0].record()
+        tensors = opt.fused_step()
+        marks[k][1].record()
+        opt.finish_step(tensors)
+        marks[k][2].record()
+    torch.cuda.synchronize()
+    whole_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    per = plan.timing_end()                       # (steps, launches) ms
     mean = per.mean(axis=0)
-    bytes_fused = n2d * (B_P0 + B_STATS + B_APPLY) + n1d * B_ADAM
-    k_apply = names.index("k_celo2_apply")
-    apply_ms = float(mean[k_apply])
-    apply_gbs = n2d * B_APPLY / (apply_ms * 1e-3) / 1e9
+    fused_in_step_ms = float(np.mean([m[0].elapsed_time(m[1]) for m in marks]))
+    finish_ms = float(np.mean([m[1].elapsed_time(m[2]) for m in marks]))
+    # 2) the C-ABI call alone, back to back (no Newton-Schulz between two calls)
+    fused_alone_ms = fused_loop(a.steps)
+
+    flops = ns_flops(shapes)
+    elem = "k_celo2_elem" if "k_celo2_elem" in names else "k_celo2_apply"
+    b_elem = (B_STATS + B_APPLY) if elem == "k_celo2_elem" else B_APPLY
+    elem_ms = float(mean[names.index(elem)])
+    elem_gbs = n2d * b_elem / (elem_ms * 1e-3) / 1e9
+    fused_ms = float(per.sum(axis=1).mean())
     out = {
-        "metric": "params_updated_per_sec (fused ELO-CELO2 step, C-ABI call)",
-        "value": n_params / (fused_ms * 1e-3),
+        "metric": "optimizer step ms + params updated/sec, % of MI355X HBM roofline (124M params)",
+        "value": n_params / (whole_ms * 1e-3),
         "unit": "params/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": fused_ms,
+        "ms_per_step": whole_ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": ("ELO_CELO2 fused step, GPT-2-small fp32 parameter set (98 tensors)"
-                                if a.workload == "gpt2s" else "ELO_CELO2 fused step, 1024x1024 + 1024"),
-                   "params": n_params, "tensors": len(shapes), "launches_per_step": len(names),
-                   "timed": "wall clock over `steps` back-to-back C-ABI calls between two device synchronisations; "
-                            "launch_ms and roofline from a second pass with HIP events around every launch"},
-        "sum_of_launch_intervals_ms": float(per.sum(axis=1).mean()),
-        "hbm_algorithmic_GB_per_step": bytes_fused / 1e9,
-        "hbm_GBps_fused_path": bytes_fused / (fused_ms * 1e-3) / 1e9,
+        "config": {"workload": ("ELO_CELO2 optimizer.step(), GPT-2-small fp32 parameter set (98 tensors)"
+                                if a.workload == "gpt2s" else "ELO_CELO2 optimizer.step(), 1024x1024 + 1024"),
+                   "params": n_params, "tensors": len(shapes),
+                   "timed": "wall clock over `steps` whole optimizer steps (fused C-ABI call, Newton-Schulz, "
+                            "finishing pass) between two device synchronisations; every parameter is updated "
+                            "in every timed step"},
+        # the HBM-bound part of the step: the one C-ABI call (gradient statistics, accumulators, features, MLP,
+        # raw step; AdamW for the 1-D tensors), timed inside the same steps by the library's events
+        "fused_pass": {
+            "ms": fused_ms, "ms_by_stream_events_around_the_call": fused_in_step_ms,
+            "ms_alone_back_to_back": fused_alone_ms,
+            "hbm_algorithmic_GB": bytes_fused / 1e9,
+            "hbm_GBps": bytes_fused / (fused_ms * 1e-3) / 1e9,
+            "hbm_roofline_frac": bytes_fused / (fused_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "hbm_roofline_frac_alone_back_to_back": bytes_fused / (fused_alone_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "params_per_sec_through_the_pass": n_params / (fused_ms * 1e-3),
+            "note": "updates the 1-D (AdamW) parameters and writes the raw steps of the matrices; the matrices "
+                    "themselves are updated by the finishing pass after Newton-Schulz",
+            "launches_per_step": len(names),
+            "launch_ms": {nm: float(v) for nm, v in zip(names, mean)},
+        },
         "hbm_roofline_frac_fused_path": bytes_fused / (fused_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        "whole_step_ms": wall_ms,
-        "whole_step_note": "optimizer.step(): fused path + Newton-Schulz as batched library fp32 GEMMs (rocBLAS) + the HIP finishing pass "
-                           "(normalise, apply)",
-        "launch_ms": {nm: float(v) for nm, v in zip(names, mean)},
-        "roofline": {"bound": "hbm", "kernel": "k_celo2_apply", "achieved": apply_gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": apply_gbs / HBM_PEAK_GBS,
-                     "traffic": TRAFFIC_APPLY_GPT2S if a.workload == "gpt2s" else None,
-                     "algorithmic_bytes_per_launch": n2d * B_APPLY, "avg_launch_ms": apply_ms},
+        # Newton-Schulz + normalise + apply: fp32 matrix products
+        "whole_step": {
+            "ms": whole_ms, "params_per_sec": n_params / (whole_ms * 1e-3),
+            "finish_ms": finish_ms, "newton_schulz_TFLOP": flops / 1e12,
+            "roofline": {"bound": "mfma", "kernel": "Newton-Schulz products + finishing pass", "achieved": flops / (finish_ms * 1e-3) / 1e12,
+                         "peak": 157.3, "unit": "TFLOP/s", "frac": flops / (finish_ms * 1e-3) / 1e12 / 157.3,
+                         "traffic": None},
+        },
+        "roofline": {"bound": "hbm", "kernel": elem, "achieved": elem_gbs, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": elem_gbs / HBM_PEAK_GBS,
+                     "traffic": traffic_from_profile("celo2_fused_step_gpt2s_hbm_traffic.txt", elem) if a.workload == "gpt2s" else None,
+                     "algorithmic_bytes_per_launch": n2d * b_elem, "avg_launch_ms": elem_ms},
     }
+    del opt, params, grads, plan
+    torch.cuda.empty_cache()
+    if a.workload == "gpt2s" and not a.no_extra_workloads:
+        out["velo_vitb16"] = other_workload("vit_velo", a.steps, a.warmup)
+        torch.cuda.empty_cache()
+        out["llama_adafac"] = other_workload("llama_adafac", max(5, a.steps // 5), max(2, a.warmup // 5))
+        torch.cuda.empty_cache()
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
@@ -260,7 +329,7 @@ def stream_ceiling(a):
                       "warmup": a.warmup, "elements_per_array": n, "peak_GBps": HBM_PEAK_GBS, "mixes": out}))
 
 
-def other_workload(a):
+def other_workload(workload, steps, warmup):
     """VeLO on the ViT-B/16 set (config 3) or AdafacLO on the Llama-1.1B set (config 4): same JSON
     line, the whole optimizer step is the fused C-ABI call for these two optimizers."""
     import torch
@@ -270,7 +339,7 @@ def other_workload(a):
 
     dev = torch.device("cuda:0")
     torch.manual_seed(1)
-    if a.workload == "vit_velo":
+    if workload == "vit_velo":
         shapes = vit_b16_shapes()
         params, grads = make_inputs(shapes, dev)
         opt = VeLO_CUDA(params, lr=1e-3, num_steps=10000, rnn=VeLORNN(), mlp=VeLOMLP())
@@ -291,17 +360,17 @@ def other_workload(a):
     n_params = sum(p.numel() for p in params)
     n2d = sum(p.numel() for p in params if p.dim() >= 2)
     n1d = n_params - n2d
-    for _ in range(a.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(a.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
-    fused_ms = (time.perf_counter() - t0) * 1e3 / a.steps   # the timed region: K back-to-back steps
+    fused_ms = (time.perf_counter() - t0) * 1e3 / steps   # the timed region: K back-to-back steps
     plan = opt._plan
-    plan.timing_begin(a.steps)                               # second pass: HIP events around every launch
-    for _ in range(a.steps):
+    plan.timing_begin(steps)                               # second pass: HIP events around every launch
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
     per = plan.timing_end()
@@ -313,9 +382,9 @@ def other_workload(a):
     apply_gbs = (n2d * B_APPLY + n1d * 68) / (float(mean[k]) * 1e-3) / 1e9
     roof = {"bound": "hbm", "kernel": apply_kernel, "achieved": apply_gbs, "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": apply_gbs / HBM_PEAK_GBS,
-            "traffic": TRAFFIC_APPLY_VITB16 if a.workload == "vit_velo" else None,
+            "traffic": traffic_from_profile("velo_fused_step_vitb16_kernel_trace_and_traffic.txt", apply_kernel) if workload == "vit_velo" else None,
             "algorithmic_bytes_per_launch": n2d * B_APPLY + n1d * 68, "avg_launch_ms": float(mean[k])}
-    if a.workload == "llama_adafac":
+    if workload == "llama_adafac":
         # the 16 -> 32 -> 32 -> 2 element MLP: 1 600 FMAs per element of a >= 2-D tensor, fp32 matrix pipe
         tflops = n2d * 3200.0 / (float(mean[k]) * 1e-3) / 1e12
         roof = {"bound": "mfma", "kernel": "k_adafac_apply_tile", "achieved": tflops, "peak": 157.3,
@@ -323,7 +392,7 @@ def other_workload(a):
                 "hbm_GBps": apply_gbs}
     out = {
         "metric": "params_updated_per_sec (fused step, C-ABI call)", "value": n_params / (fused_ms * 1e-3),
-        "unit": "params/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": fused_ms,
+        "unit": "params/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": fused_ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": label, "params": n_params, "tensors": len(shapes), "launches_per_step": len(names)},
         "hbm_algorithmic_GB_per_step": bytes_fused / 1e9,
@@ -333,7 +402,8 @@ def other_workload(a):
         "launch_ms": {nm: float(v) for nm, v in zip(names, mean)},
         "roofline": roof,
     }
-    print(json.dumps(out))
+    del opt, params, grads, plan
+    return out
 
 
 if __name__ == "__main__":

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define PYLO_MI355_ABI_VERSION 4
+#define PYLO_MI355_ABI_VERSION 5
 #define PYLO_MAX_DIMS 8
 #define PYLO_MAX_GROUPS 8   /* parameter groups with their own step counter (VeLO) */
 
@@ -95,8 +95,12 @@ typedef struct {
                         the call passes step < 0                                             */
   float bc2;         /* CELO2 AdamW: 1 - beta2^t                                             */
   int32_t group;     /* VeLO: index into PyloVeloStep.frac (the tensor's parameter group)    */
-  int32_t reserved;
+  int32_t flags;     /* PYLO_ARG_* bits, 0 for the step calls                                */
 } PyloTensorArgs;
+
+/* PyloTensorArgs.flags, pylo_mi355_celo2_orthogonalize_finish: `step_out` holds the tensor's raw step and the
+   call orthogonalises it first (the group's `orthogonalize`, ELO_CELO2_cuda.py:288-292) */
+#define PYLO_ARG_ORTHOGONALIZE 1
 
 int pylo_mi355_abi_version(void);
 const char* pylo_mi355_last_error(void);
@@ -200,6 +204,24 @@ int pylo_mi355_celo2_step(PyloPlan* plan, const PyloTensorArgs* args, const Pylo
  * update.  16 bytes per element.
  */
 int pylo_mi355_celo2_finish(PyloPlan* plan, const PyloTensorArgs* args, void* stream);
+
+/*
+ * Newton-Schulz and the finishing pass in one call (replaces `step = newton_schulz(step, ...)` of the
+ * per-tensor loop, ELO_CELO2_cuda.py:288-292 / CELO2_naive.py:59-73, for all tensors at once, followed by
+ * what pylo_mi355_celo2_finish does).  For every tensor with PYLO_ARG_ORTHOGONALIZE in `flags`, with
+ * X = step_out / (||step_out||_F + ns_eps) and (c0, c1, c2) = ns_coeffs, `ns_iters` times
+ *     A = X X^T (the Gram matrix over the smaller dim);  X <- c0 X + (c1 A + c2 A A) X
+ * as fp32 matrix-pipe products that compute the symmetric A and c1 A + c2 A A once per pair of tiles; then
+ * every tensor is normalised and applied as by pylo_mi355_celo2_finish (tensors without the flag from
+ * `step_out` as it stands).  `step_out` of a flagged tensor is overwritten with intermediate results.
+ * A tensor can carry the flag when pylo_mi355_plan_orthogonalize_supported says so: two dims, the last
+ * and the smaller of the two multiples of 4; others (and tensors whose step is orthogonalised per slice of more leading dims) are
+ * orthogonalised by the caller and passed without the flag.  The plan's workspace holds the second copy of
+ * X and the two small matrices per tensor.
+ */
+int pylo_mi355_celo2_orthogonalize_finish(PyloPlan* plan, const PyloTensorArgs* args, const float* ns_coeffs,
+                                          int ns_iters, float ns_eps, void* stream);
+int pylo_mi355_plan_orthogonalize_supported(const PyloPlan* plan, int tensor);
 
 /*
  * VeLO step (replaces velo_cuda_kernel.velo_kernel_simple, pylo/csrc/velo_kernel.cu:370-457, for every

@@ -19,6 +19,7 @@ KIND_CELO2, KIND_VELO, KIND_ADAFAC = 0, 1, 2
 F_ADAM = 1
 F_ADAM_INDEP = 2
 F_NAN_TO_NUM, F_WD_PRESTEP, F_GLOBAL_NORM = 4, 8, 16
+ARG_ORTHOGONALIZE = 1      # PyloTensorArgs.flags
 
 
 class TensorShape(C.Structure):
@@ -36,7 +37,7 @@ ARGS_DTYPE = np.dtype([
     ("fac_r", np.uint64), ("fac_c", np.uint64), ("fac_v", np.uint64), ("step_out", np.uint64),
     ("lr", np.float32), ("weight_decay", np.float32), ("clip_norm", np.float32),
     ("clip_val", np.float32), ("exp_mult", np.float32), ("step_mult", np.float32),
-    ("bc1", np.float32), ("bc2", np.float32), ("group", np.int32), ("reserved", np.int32),
+    ("bc1", np.float32), ("bc2", np.float32), ("group", np.int32), ("flags", np.int32),
 ])
 assert ARGS_DTYPE.itemsize == 104
 MAX_GROUPS = 8
@@ -88,13 +89,16 @@ def load():
     lib.pylo_mi355_celo2_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.c_void_p,
                                           C.c_void_p]
     lib.pylo_mi355_celo2_finish.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.pylo_mi355_celo2_orthogonalize_finish.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_float), C.c_int,
+                                                         C.c_float, C.c_void_p]
+    lib.pylo_mi355_plan_orthogonalize_supported.argtypes = [C.c_void_p, C.c_int]
     lib.pylo_mi355_velo_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.POINTER(VeloNets),
                                          C.POINTER(VeloStep), C.c_void_p]
     lib.pylo_mi355_adafac_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.c_void_p, C.c_float,
                                            C.c_void_p]
     lib.pylo_mi355_plan_arg_table.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_void_p)]
     lib.pylo_mi355_plan_device_steps.argtypes = [C.c_void_p, C.POINTER(DeviceSteps)]
-    if lib.pylo_mi355_abi_version() != 4:
+    if lib.pylo_mi355_abi_version() != 5:
         raise RuntimeError("libpylo_mi355.so: ABI version mismatch, rebuild it")
     _lib = lib
     return lib
@@ -208,6 +212,15 @@ class Plan:
     def celo2_finish(self, args: np.ndarray, stream: int) -> None:
         """Normalise + apply after Newton-Schulz; `args` is a table like `self.args` (own array)."""
         check(load().pylo_mi355_celo2_finish(self._h, args.ctypes.data, stream), "celo2_finish")
+
+    def orthogonalize_supported(self, i: int) -> bool:
+        return load().pylo_mi355_plan_orthogonalize_supported(self._h, i) == 1
+
+    def celo2_orthogonalize_finish(self, args: np.ndarray, coeffs, iters: int, eps: float, stream: int) -> None:
+        """Newton-Schulz on the tensors flagged in `args["flags"]`, then normalise + apply for all of them."""
+        c = (C.c_float * 3)(*[float(v) for v in coeffs])
+        check(load().pylo_mi355_celo2_orthogonalize_finish(self._h, args.ctypes.data, c, int(iters), float(eps), stream),
+              "celo2_orthogonalize_finish")
 
     def velo_step(self, decays: Decays, nets: VeloNets, step: VeloStep, stream: int,
                   args: Optional[np.ndarray] = None) -> None:

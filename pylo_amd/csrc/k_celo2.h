@@ -895,10 +895,21 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PYLO_A
 // ---------------------------------------------------------------------------------------------
 constexpr int kFinElems = kThreads * 4 * kElemIters;
 
+// Where the finishing pass finds a tensor's step: `step_out`, or -- for a tensor the same call has
+// orthogonalised with an odd number of Newton-Schulz iterations -- the second X buffer in the workspace
+// (x_alt[tensor] floats into `ws`; x_alt == nullptr: always `step_out`).
+__device__ __forceinline__ const float* fin_source(const PyloTensorArgs& a, int tensor, const long long* x_alt,
+                                                   const float* ws) {
+  if (x_alt != nullptr && (a.flags & PYLO_ARG_ORTHOGONALIZE) && x_alt[tensor] >= 0) return ws + x_alt[tensor];
+  return a.step_out;
+}
+
 __global__ __launch_bounds__(kThreads) void k_celo2_sumsq(const TDesc* __restrict__ descs,
                                                           const PyloTensorArgs* __restrict__ dyn,
                                                           const Item* __restrict__ items,
-                                                          double* __restrict__ fin_part) {
+                                                          double* __restrict__ fin_part,
+                                                          const long long* __restrict__ x_alt,
+                                                          const float* __restrict__ ws) {
   __shared__ float red[kWaves];
   const Item it = items[blockIdx.x];
   const TDesc d = descs[it.tensor];
@@ -907,7 +918,7 @@ __global__ __launch_bounds__(kThreads) void k_celo2_sumsq(const TDesc* __restric
   const long long base = (long long)it.a * kFinElems;
   const long long left = d.n - base;
   const unsigned lim = left < (long long)kFinElems ? (unsigned)left : (unsigned)kFinElems;
-  const float* x = a.step_out + base;
+  const float* x = fin_source(a, it.tensor, x_alt, ws) + base;
   float s = 0.0f;
   if (d.n % 4 == 0) {
 #pragma unroll
@@ -955,7 +966,9 @@ __global__ __launch_bounds__(kThreads) void k_celo2_finscale(const TDesc* __rest
 __global__ __launch_bounds__(kThreads) void k_celo2_update(const TDesc* __restrict__ descs,
                                                            const PyloTensorArgs* __restrict__ dyn,
                                                            const Item* __restrict__ items,
-                                                           const float* __restrict__ fin_scale) {
+                                                           const float* __restrict__ fin_scale,
+                                                           const long long* __restrict__ x_alt,
+                                                           const float* __restrict__ ws) {
   const Item it = items[blockIdx.x];
   const TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
@@ -963,7 +976,7 @@ __global__ __launch_bounds__(kThreads) void k_celo2_update(const TDesc* __restri
   const long long base = (long long)it.a * kFinElems;
   const long long left = d.n - base;
   const unsigned lim = left < (long long)kFinElems ? (unsigned)left : (unsigned)kFinElems;
-  const float* x = a.step_out + base;
+  const float* x = fin_source(a, it.tensor, x_alt, ws) + base;
   float* p = a.param + base;
   const float sc = fin_scale[it.tensor], rm = a.step_mult, wd = a.weight_decay, nlr = -a.lr;
   if (d.n % 4 == 0) {

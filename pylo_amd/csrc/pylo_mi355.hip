@@ -29,6 +29,7 @@
 #include "k_single.h"
 #include "k_velo.h"
 #include "k_celo2_slices.h"
+#include "k_ns.h"
 #include "pylo_common.h"
 
 // =============================================================================================
@@ -72,6 +73,15 @@ bool factored_dims(int kind, const PyloTensorShape& s, int* dc, int* dr) {
 struct Layout {
   std::vector<Item> mx_items;   // ELO-CELO2: statistics and apply items in slab order (k_celo2_elem)
   size_t off_mx_items = 0, off_sync = 0;
+  // ELO-CELO2: Newton-Schulz on the 2-D tensors (k_ns.h)
+  std::vector<NsMat> ns_mats;
+  std::vector<NsItem> ns_gram, ns_poly, ns_upd;
+  std::vector<int> ns_split;          // matrices whose Gram product is split (k_ns_gram_reduce)
+  std::vector<long long> ns_xalt;     // per tensor: offset of its second X buffer, -1 without one
+  std::vector<int> ns_of_tensor;      // per tensor: index into ns_mats, -1
+  int ns_max_m = 0;
+  size_t off_ns_mats = 0, off_ns_gram = 0, off_ns_poly = 0, off_ns_upd = 0, off_ns_split = 0, off_ns_xalt = 0,
+         off_ns_scale = 0, off_ns_ws = 0;
   std::vector<TDesc> descs;
   std::vector<Item> p0_items, nd_items, sl_items, seg_items, el_items, ap_items, ga_items, fin_items, v0a_items, v0b_items;
   std::vector<int> fac_list;
@@ -172,6 +182,56 @@ void build_elem_items(Layout& L, int T) {
     if (k < np) push(pieces[k].st0, pieces[k].st1, false, pieces[k].keep);
     if (k >= depth) push(pieces[k - depth].ap0, pieces[k - depth].ap1, true, pieces[k - depth].keep);
   }
+}
+
+// Newton-Schulz tables: every 2-D MLP tensor whose rows (C) and whose smaller dim (the rows of A and B')
+// are multiples of 4: the kernels load 16 bytes at a time along the contiguous dim of X, A and B'.  The
+// number of rows of a tall matrix is free (50257 x 768).  `ws_floats` returns the floats of workspace behind off_ns_ws.
+void build_ns_tables(Layout& L, int T, long long& ws_floats) {
+  ws_floats = 0;
+  L.ns_xalt.assign(T, -1);
+  L.ns_of_tensor.assign(T, -1);
+  auto take = [&](long long n) { const long long o = ws_floats; ws_floats += (n + 63) / 64 * 64; return o; };
+  for (int t = 0; t < T; ++t) {
+    const TDesc& d = L.descs[t];
+    if (d.mode != kModeFac2D || d.n == 0 || d.C0 % 4 != 0 || std::min(d.R0, d.C0) % 4 != 0) continue;
+    NsMat mt{};
+    mt.tensor = t;
+    mt.R = d.R0; mt.C = d.C0;
+    mt.tall = d.R0 > d.C0;
+    mt.m = std::min(d.R0, d.C0);
+    const int K = mt.tall ? mt.R : mt.C;
+    mt.n_slabs = K >= kNsSplitMin ? (K + kNsSlabK - 1) / kNsSlabK : 1;
+    mt.off_x1 = take(d.n);
+    mt.off_a = take((long long)mt.m * mt.m);
+    mt.off_b = take((long long)mt.m * mt.m);
+    mt.off_part = mt.n_slabs > 1 ? take((long long)mt.n_slabs * mt.m * mt.m) : 0;
+    const int q = (int)L.ns_mats.size();
+    L.ns_of_tensor[t] = q;
+    L.ns_xalt[t] = mt.off_x1;
+    L.ns_max_m = std::max(L.ns_max_m, mt.m);
+    const int nt = (mt.m + kNsTile - 1) / kNsTile;
+    for (int tm = 0; tm < nt; ++tm)
+      for (int tn = tm; tn < nt; ++tn) {
+        if (mt.n_slabs > 1) {
+          for (int sl = 0; sl < mt.n_slabs; ++sl)
+            L.ns_gram.push_back(NsItem{q, tm, tn, sl * kNsSlabK, std::min(K, (sl + 1) * kNsSlabK), sl});
+        } else {
+          L.ns_gram.push_back(NsItem{q, tm, tn, 0, K, -1});
+        }
+        L.ns_poly.push_back(NsItem{q, tm, tn, 0, mt.m, -1});
+      }
+    const int ni = ((mt.tall ? mt.R : mt.m) + kNsTile - 1) / kNsTile, nj = ((mt.tall ? mt.m : mt.C) + kNsTile - 1) / kNsTile;
+    for (int tm = 0; tm < ni; ++tm)
+      for (int tn = 0; tn < nj; ++tn) L.ns_upd.push_back(NsItem{q, tm, tn, 0, mt.m, -1});
+    if (mt.n_slabs > 1) L.ns_split.push_back(q);
+    L.ns_mats.push_back(mt);
+  }
+  // longest jobs first: the launch ends when its last block does
+  auto longer = [](const NsItem& x, const NsItem& y) { return x.k1 - x.k0 > y.k1 - y.k0; };
+  std::stable_sort(L.ns_gram.begin(), L.ns_gram.end(), longer);
+  std::stable_sort(L.ns_poly.begin(), L.ns_poly.end(), longer);
+  std::stable_sort(L.ns_upd.begin(), L.ns_upd.end(), longer);
 }
 
 int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int velo_hidden) {
@@ -391,6 +451,18 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_frac = take(kind == PYLO_KIND_VELO ? sizeof(float) * 9 * PYLO_MAX_GROUPS : 0);
   L.off_mx_items = take(sizeof(Item) * L.mx_items.size());
   L.off_sync = take(sizeof(int) * 2 * (size_t)T);
+  if (kind == PYLO_KIND_CELO2) {
+    long long ns_floats = 0;
+    build_ns_tables(L, T, ns_floats);
+    L.off_ns_mats = take(sizeof(NsMat) * L.ns_mats.size());
+    L.off_ns_gram = take(sizeof(NsItem) * L.ns_gram.size());
+    L.off_ns_poly = take(sizeof(NsItem) * L.ns_poly.size());
+    L.off_ns_upd = take(sizeof(NsItem) * L.ns_upd.size());
+    L.off_ns_split = take(sizeof(int) * L.ns_split.size());
+    L.off_ns_xalt = take(sizeof(long long) * (size_t)T);
+    L.off_ns_scale = take(sizeof(float) * L.ns_mats.size());
+    L.off_ns_ws = take(sizeof(float) * (size_t)ns_floats);
+  }
   L.total = off;
   return 0;
 }
@@ -468,6 +540,12 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_v0a_items, L.v0a_items.data(), sizeof(Item) * L.v0a_items.size());
   if (e == hipSuccess) e = up(L.off_v0b_items, L.v0b_items.data(), sizeof(Item) * L.v0b_items.size());
   if (e == hipSuccess) e = up(L.off_mx_items, L.mx_items.data(), sizeof(Item) * L.mx_items.size());
+  if (e == hipSuccess) e = up(L.off_ns_mats, L.ns_mats.data(), sizeof(NsMat) * L.ns_mats.size());
+  if (e == hipSuccess) e = up(L.off_ns_gram, L.ns_gram.data(), sizeof(NsItem) * L.ns_gram.size());
+  if (e == hipSuccess) e = up(L.off_ns_poly, L.ns_poly.data(), sizeof(NsItem) * L.ns_poly.size());
+  if (e == hipSuccess) e = up(L.off_ns_upd, L.ns_upd.data(), sizeof(NsItem) * L.ns_upd.size());
+  if (e == hipSuccess) e = up(L.off_ns_split, L.ns_split.data(), sizeof(int) * L.ns_split.size());
+  if (e == hipSuccess && kind == PYLO_KIND_CELO2) e = up(L.off_ns_xalt, L.ns_xalt.data(), sizeof(long long) * L.ns_xalt.size());
   if (e == hipSuccess) e = hipStreamSynchronize(s);
   for (int i = 0; i < kStageSlots && e == hipSuccess; ++i) {
     e = hipHostMalloc(reinterpret_cast<void**>(&P->stage[i]), (sizeof(PyloTensorArgs) * n_tensors + 15) / 16 * 16,
@@ -823,20 +901,31 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   return 0;
 }
 
-extern "C" int pylo_mi355_celo2_finish(PyloPlan* P, const PyloTensorArgs* args, void* stream) {
-  if (!P || P->kind != PYLO_KIND_CELO2) return fail("celo2_finish: not an ELO-CELO2 plan");
-  if (!args) return fail("celo2_finish: null argument");
+namespace {
+
+// Newton-Schulz (ns_iters > 0, on the tensors flagged PYLO_ARG_ORTHOGONALIZE) and the finishing pass.
+int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, int ns_iters, float ns_eps, void* stream,
+                const char* who) {
+  const std::string w(who);
+  if (!P || P->kind != PYLO_KIND_CELO2) return fail(w + ": not an ELO-CELO2 plan");
+  if (!args) return fail(w + ": null argument");
   const Layout& L = P->L;
+  bool any_ns = false;
   for (int t = 0; t < P->T; ++t) {
     const TDesc& d = L.descs[t];
     const PyloTensorArgs& a = args[t];
     if (a.grad == nullptr || d.mode == kModeFlat || d.n == 0) continue;
+    const std::string at = " (tensor " + std::to_string(t) + ")";
     if (d.mode == kModeFacND)
-      return fail("celo2_finish: tensors with more than two dims are normalised per slice of the last two dims, "
-                  "not by this tensor-wide pass (tensor " + std::to_string(t) + ")");
-    if (!a.param || !a.step_out) return fail("celo2_finish: null param/step_out pointer at tensor " + std::to_string(t));
+      return fail(w + ": tensors with more than two dims are normalised per slice of the last two dims, "
+                  "not by this tensor-wide pass" + at);
+    if (!a.param || !a.step_out) return fail(w + ": null param/step_out pointer" + at);
     const uintptr_t m = reinterpret_cast<uintptr_t>(a.param) | reinterpret_cast<uintptr_t>(a.step_out);
-    if (m % (d.n % 4 == 0 ? 16 : 4) != 0) return fail("celo2_finish: misaligned pointer at tensor " + std::to_string(t));
+    if (m % (d.n % 4 == 0 ? 16 : 4) != 0) return fail(w + ": misaligned pointer" + at);
+    if (ns_iters > 0 && (a.flags & PYLO_ARG_ORTHOGONALIZE)) {
+      if (L.ns_of_tensor[t] < 0) return fail(w + ": PYLO_ARG_ORTHOGONALIZE on a tensor the library cannot orthogonalise" + at);
+      any_ns = true;
+    }
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (int rc = upload_args(P, args, s)) return rc;
@@ -847,11 +936,60 @@ extern "C" int pylo_mi355_celo2_finish(PyloPlan* P, const PyloTensorArgs* args, 
   float* fin_scale = P->at<float>(L.off_finscale);
   const int n_fin = (int)L.fin_items.size();
   if (n_fin == 0) return 0;
-  hipLaunchKernelGGL(k_celo2_sumsq, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_part);
+  const long long* x_alt = nullptr;
+  float* ns_ws = nullptr;
+  if (any_ns) {
+    const NsMat* mats = P->at<NsMat>(L.off_ns_mats);
+    const NsItem* gram = P->at<NsItem>(L.off_ns_gram);
+    const NsItem* poly = P->at<NsItem>(L.off_ns_poly);
+    const NsItem* upd = P->at<NsItem>(L.off_ns_upd);
+    const int* split = P->at<int>(L.off_ns_split);
+    float* scale = P->at<float>(L.off_ns_scale);
+    ns_ws = P->at<float>(L.off_ns_ws);
+    const int n_mats = (int)L.ns_mats.size(), n_gram = (int)L.ns_gram.size(), n_poly = (int)L.ns_poly.size(),
+              n_upd = (int)L.ns_upd.size(), n_split = (int)L.ns_split.size();
+    // ||raw||: the finishing pass's sums of squares, taken on the raw steps
+    hipLaunchKernelGGL(k_celo2_sumsq, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_part,
+                       (const long long*)nullptr, (const float*)nullptr);
+    hipLaunchKernelGGL(k_ns_scale, dim3(n_mats), dim3(256), 0, s, mats, n_mats, descs, fin_part, ns_eps, scale);
+    for (int it = 0; it < ns_iters; ++it) {
+      const int first = it == 0, par = it & 1;
+      hipLaunchKernelGGL(k_ns_gemm<kNsGram>, dim3(n_gram), dim3(256), 0, s, mats, gram, dyn, ns_ws, scale, first, par,
+                         coeffs[0], coeffs[1], coeffs[2]);
+      if (n_split > 0)
+        hipLaunchKernelGGL(k_ns_gram_reduce, dim3(((size_t)L.ns_max_m * L.ns_max_m + 255) / 256, n_split), dim3(256), 0, s,
+                           mats, split, dyn, ns_ws);
+      hipLaunchKernelGGL(k_ns_gemm<kNsPoly>, dim3(n_poly), dim3(256), 0, s, mats, poly, dyn, ns_ws, scale, first, par,
+                         coeffs[0], coeffs[1], coeffs[2]);
+      hipLaunchKernelGGL(k_ns_gemm<kNsUpdate>, dim3(n_upd), dim3(256), 0, s, mats, upd, dyn, ns_ws, scale, first, par,
+                         coeffs[0], coeffs[1], coeffs[2]);
+    }
+    if (ns_iters & 1) x_alt = P->at<long long>(L.off_ns_xalt);   // the last iteration wrote the second buffer
+  }
+  hipLaunchKernelGGL(k_celo2_sumsq, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_part, x_alt,
+                     (const float*)ns_ws);
   hipLaunchKernelGGL(k_celo2_finscale, dim3(P->T), dim3(kThreads), 0, s, descs, dyn, fin_part, fin_scale);
-  hipLaunchKernelGGL(k_celo2_update, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_scale);
+  hipLaunchKernelGGL(k_celo2_update, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_scale, x_alt,
+                     (const float*)ns_ws);
   HIP_TRY(hipGetLastError());
   return 0;
+}
+
+}  // namespace
+
+extern "C" int pylo_mi355_celo2_finish(PyloPlan* P, const PyloTensorArgs* args, void* stream) {
+  return finish_impl(P, args, nullptr, 0, 0.0f, stream, "celo2_finish");
+}
+
+extern "C" int pylo_mi355_celo2_orthogonalize_finish(PyloPlan* P, const PyloTensorArgs* args, const float* ns_coeffs,
+                                                     int ns_iters, float ns_eps, void* stream) {
+  if (ns_iters < 0 || (ns_iters > 0 && !ns_coeffs)) return fail("celo2_orthogonalize_finish: bad Newton-Schulz arguments");
+  return finish_impl(P, args, ns_coeffs, ns_iters, ns_eps, stream, "celo2_orthogonalize_finish");
+}
+
+extern "C" int pylo_mi355_plan_orthogonalize_supported(const PyloPlan* P, int tensor) {
+  if (!P || tensor < 0 || tensor >= P->T || P->kind != PYLO_KIND_CELO2) return 0;
+  return P->L.ns_of_tensor[tensor] >= 0 ? 1 : 0;
 }
 
 extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, const PyloDecays* decays,

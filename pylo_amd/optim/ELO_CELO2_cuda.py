@@ -76,18 +76,16 @@ def newton_schulz(x: torch.Tensor, coeffs, iters: int, eps: float) -> torch.Tens
 
 
 class _ns_blas:
-    """Newton-Schulz GEMMs through rocBLAS for the duration of the block: on the shapes of a transformer's
-    matrices (768 .. 3072 wide, batches of 12) its fp32 kernels run at 122 TFLOP/s where hipBLASLt's choices
-    give 110 (768^3 batched: 55).  ``PYLO_MI355_NS_BLAS=default`` leaves torch's setting alone."""
+    """The torch path of Newton-Schulz (shapes the library's own kernels do not take) with torch's BLAS choice
+    left alone.  ``PYLO_MI355_NS_BLAS=rocblas`` in the environment opts in to rocBLAS for the duration of the
+    block (on 768 .. 3072 wide matrices in batches of 12 its fp32 kernels run at 122 TFLOP/s where hipBLASLt's
+    choices give 110); that switch is process-wide in torch, so it is never made unasked."""
 
     def __enter__(self):
         self.prev = None
-        if os.environ.get("PYLO_MI355_NS_BLAS", "rocblas") == "rocblas":
-            try:
-                self.prev = torch.backends.cuda.preferred_blas_library()
-                torch.backends.cuda.preferred_blas_library("cublas")      # torch's name for rocBLAS
-            except Exception:
-                self.prev = None
+        if os.environ.get("PYLO_MI355_NS_BLAS", "default") == "rocblas":
+            self.prev = torch.backends.cuda.preferred_blas_library()
+            torch.backends.cuda.preferred_blas_library("cublas")      # torch's name for rocBLAS
         return self
 
     def __exit__(self, *exc):
@@ -201,6 +199,7 @@ class ELO_CELO2_CUDA(Optimizer):
         self._adam_b1, self._adam_b2 = float(bm[0]), float(self.beta_rms[-1])
         self._plan = None
         self._plan_key = None
+        self._lib_ns = os.environ.get("PYLO_MI355_NS", "lib") != "torch"
 
     # ------------------------------------------------------------------ plan
     def _tensors(self):
@@ -242,6 +241,7 @@ class ELO_CELO2_CUDA(Optimizer):
                 self._raw[i] = buf[j]
             self._raw_groups.append((buf, idx))
         self._fin_args = np.zeros(len(tensors), dtype=_lib.ARGS_DTYPE)
+        self._ns_ok = [self._plan.orthogonalize_supported(i) for i in range(len(tensors))]
         if self.capturable:
             self._reset_device_steps(tensors)
 
@@ -456,13 +456,17 @@ class ELO_CELO2_CUDA(Optimizer):
     @torch.no_grad()
     def finish_step(self, tensors):
         """Newton-Schulz, RMS normalisation and the parameter update of the MLP tensors
-        (pylo/optim/ELO_CELO2_cuda.py:288-296)."""
-        with _ns_blas():
-            self._finish_step(tensors)
+        (pylo/optim/ELO_CELO2_cuda.py:288-296).  Matrices whose dims are multiples of 4 are orthogonalised by
+        the library's own fp32 matrix-pipe kernels inside the finishing call; other shapes, tensors with more
+        than two dims and buckets in which a tensor sat the step out go through the batched torch products
+        (also with ``PYLO_MI355_NS=torch`` in the environment, for comparisons)."""
+        self._finish_step(tensors)
 
     def _finish_step(self, tensors):
         fin = self._fin_args
         fin["grad"] = 0
+        fin["flags"] = 0
+        lib_ns = self._lib_ns
         keep, any_fin = [], False   # post-Newton-Schulz matrices must outlive the launch
         for buf, idx in self._raw_groups:
             group = tensors[idx[0]][0]
@@ -477,7 +481,8 @@ class ELO_CELO2_CUDA(Optimizer):
                     if group["param_scale_mult"]:
                         step = step * torch.sqrt(torch.mean(p * p) + 1e-9)
                     if group["orthogonalize"] and step.dim() >= 2:
-                        step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
+                        with _ns_blas():
+                            step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
                     step = rms_normalize(step, list(range(step.dim()))[-2:]) * group["rmsmult"]
                     p.add_(step + group["weight_decay"] * p, alpha=-group["lr"])
                 continue
@@ -486,9 +491,14 @@ class ELO_CELO2_CUDA(Optimizer):
             if group["param_scale_mult"]:
                 n = ps[0].numel()
                 sq = torch.stack(torch._foreach_norm(ps)) ** 2 / n
-                step = step * torch.sqrt(sq + 1e-9).view([-1] + [1] * nd)
+                step = step.mul_(torch.sqrt(sq + 1e-9).view([-1] + [1] * nd))   # the raw steps are scratch
+            flag = 0
             if group["orthogonalize"] and nd >= 2:
-                step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
+                if lib_ns and nd == 2 and self.ns_iters > 0 and all(self._ns_ok[i] for i in idx):
+                    flag = _lib.ARG_ORTHOGONALIZE
+                else:
+                    with _ns_blas():
+                        step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
             if nd > 2:
                 # more than two dims: the normaliser is per slice of the last two dims
                 # (ELO_CELO2_naive.py:217-218,235), which the tensor-wide finishing kernels do not do
@@ -506,6 +516,7 @@ class ELO_CELO2_CUDA(Optimizer):
                 fin["lr"][i] = group["lr"]
                 fin["weight_decay"][i] = group["weight_decay"]
                 fin["step_mult"][i] = group["rmsmult"]
+                fin["flags"][i] = flag
             any_fin = True
         if any_fin:
             if self._capturing():
@@ -513,7 +524,8 @@ class ELO_CELO2_CUDA(Optimizer):
                 table[:] = fin
                 fin = table
             with torch.cuda.device(self.device):
-                self._plan.celo2_finish(fin, torch.cuda.current_stream(self.device).cuda_stream)
+                self._plan.celo2_orthogonalize_finish(fin, self.ns_coeffs, self.ns_iters, self.ns_eps,
+                                                      torch.cuda.current_stream(self.device).cuda_stream)
         del keep
 
 

@@ -45,3 +45,13 @@ def max_err(a: torch.Tensor, b: torch.Tensor, rel=1e-5, abs_=1e-6) -> float:
 def trailing_to_keepdim(vec: torch.Tensor, drop_dim: int) -> torch.Tensor:
     """naive factored accumulator (param dims minus one, decay last) -> (3, *shape with dim->1)."""
     return vec.movedim(-1, 0).unsqueeze(drop_dim + 1)
+
+
+def step_keeping_raw(opt):
+    """``opt.step()`` of an ELO-CELO2-family optimizer, returning copies of the raw per-element steps (what
+    celo2_kernel.cu:280 writes to ``step_out``) taken between the fused call and the finishing call, which
+    orthogonalises in place and leaves intermediate results in those buffers."""
+    tensors = opt.fused_step()
+    kept = [None if r is None else r.clone() for r in opt._raw]
+    opt.finish_step(tensors)
+    return kept

@@ -14,7 +14,7 @@ import os
 import pytest
 import torch
 
-from golden_io import max_err
+from golden_io import max_err, step_keeping_raw
 
 pytestmark = pytest.mark.gpu
 
@@ -52,8 +52,7 @@ def _run(env, steps=3, seed=0, shapes=SHAPES):
         for t in range(steps):
             for i, p in enumerate(params):
                 p.grad = torch.randn(p.shape, generator=gen, device="cuda") * 10.0 ** (-1 - i % 3)
-            opt.step()
-            raws.append([None if r is None else r.clone() for r in opt._raw])
+            raws.append(step_keeping_raw(opt))
         names = opt._plan.launch_names()
     torch.cuda.synchronize()
     return params, opt, raws, names

@@ -1,0 +1,128 @@
+"""The library's own Newton-Schulz kernels (``pylo_mi355_celo2_orthogonalize_finish``: symmetric products on
+tiles on and above the diagonal, split Gram product of very tall matrices, scalings folded into the first
+iteration) against the oracle's literal formula (pylo/optim/CELO2_naive.py:59-73) evaluated in fp64, through
+whole optimizer steps.  The orthogonalised, normalised step is recovered from the parameter update,
+``p_new = p_old - lr (s + wd p_old)``, and held to 2e-4 of its RMS (the library's fp32 products sit at
+2e-5 .. 5e-5, the same as the batched torch products they replace); parameters at rel 1e-5 / abs 1e-6.
+"""
+
+import pytest
+import torch
+
+from golden_io import max_err
+
+pytestmark = pytest.mark.gpu
+
+LR, WD = 1e-2, 0.1
+
+
+def _run(shapes, steps=2, seed=0, **kw):
+    from oracle import pylo_oracle as O
+    from pylo_amd import ELO_CELO2_CUDA
+    from pylo_amd.models import CELO2MLP
+
+    torch.manual_seed(1)
+    net = CELO2MLP()
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    init = [torch.randn(s, generator=gen, device="cuda") * 0.05 for s in shapes]
+    ref = [v.double() for v in init]
+    gpu = [torch.nn.Parameter(v.clone()) for v in init]
+    cfg = dict(lr=LR, weight_decay=WD, adam_lr_mult=20.0)
+    cfg.update(kw)
+    orc = O.EloCelo2Oracle(ref, net.state_dict(), device="cuda", **cfg).double_()
+    opt = ELO_CELO2_CUDA(gpu, network=net, hf_key=None, **cfg)
+    worst = 0.0
+    for t in range(steps):
+        before = [(p.detach().clone(), r.clone()) for p, r in zip(gpu, ref)]
+        grads = [torch.randn(s, generator=gen, device="cuda") * 10.0 ** (-1 - i % 3) for i, s in enumerate(shapes)]
+        for p, g in zip(gpu, grads):
+            p.grad = g
+        orc.step([g.double() for g in grads])
+        opt.step()
+        torch.cuda.synchronize()
+        for i, p in enumerate(gpu):
+            assert torch.isfinite(p).all(), (t, i, shapes[i])
+            assert max_err(p, ref[i], 1e-5, 1e-6) <= 1.0, (t, i, shapes[i])
+            if p.dim() == 2:
+                got = (before[i][0].double() - p.detach().double()) / LR - WD * before[i][0].double()
+                want = (before[i][1] - ref[i]) / LR - WD * before[i][1]
+                rms = float(want.pow(2).mean().sqrt())
+                quant = float(before[i][0].abs().max()) * 2.0 ** -23 / LR     # fp32 parameters quantise the recovered step
+                e = float((got - want).abs().max()) / rms
+                worst = max(worst, e)
+                assert e <= 2e-4 + 2 * quant / rms, (t, i, shapes[i], e)
+    return opt, worst
+
+
+def test_library_kernels_take_these_shapes():
+    shapes = [(256, 384), (384, 256), (128, 128), (132, 260), (260, 132), (4, 8), (8, 4), (36, 36), (1, 64), (64, 1),
+              (130, 6), (6, 130), (10, 12), (12, 10), (9, 16), (16, 9)]
+    opt, _ = _run(shapes, steps=1)
+    # the last dim and the smaller dim must be multiples of 4; everything else goes through torch
+    for s, got in zip(shapes, opt._ns_ok):
+        r, c = s
+        assert got == (c % 4 == 0 and min(r, c) % 4 == 0), s
+    assert opt._ns_ok[:8] == [True] * 8 and not any(opt._ns_ok[8:])
+
+
+@pytest.mark.parametrize("shapes", [
+    [(256, 384), (384, 256), (128, 128), (768,)],                       # whole tiles
+    [(132, 260), (260, 132), (4, 8), (8, 4), (36, 36), (200, 4)],        # ragged tiles, a single MFMA column
+    [(8201, 128), (128, 8200), (16385, 64)],                             # split Gram product, odd reduction length
+    [(130, 6), (6, 130), (9, 16), (64, 64)],                             # library and torch side by side
+    [(300, 260), (300, 260), (300, 260), (64,)],                         # a bucket of equal shapes
+])
+def test_library_newton_schulz_matches_oracle(shapes):
+    _, worst = _run(shapes, steps=2, seed=len(shapes))
+    print("orthogonalised step err / rms", worst)
+
+
+@pytest.mark.parametrize("iters", [0, 1, 2, 4])
+def test_iteration_counts_and_result_buffer(iters):
+    """An even number of iterations leaves the result in the raw-step buffer, an odd one in the workspace."""
+    _run([(256, 384), (384, 256), (132, 260)], steps=2, ns_iters=iters)
+
+
+def test_groups_without_orthogonalisation_and_with_param_scale():
+    from pylo_amd import ELO_CELO2_CUDA
+    from pylo_amd.models import CELO2MLP
+    from oracle import pylo_oracle as O
+
+    _run([(256, 384), (132, 260), (64,)], orthogonalize=False)
+    _run([(256, 384), (132, 260), (64,)], param_scale_mult=True)
+    _run([(256, 384), (132, 260), (64,)], ns_coeffs=(3.0, -3.2, 1.2), ns_eps=1e-6)
+    # a tensor of a bucket sits a step out: that bucket takes the torch path, the others the library's
+    torch.manual_seed(1)
+    net = CELO2MLP()
+    shapes = [(256, 128), (256, 128), (128, 256)]
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    init = [torch.randn(s, generator=gen, device="cuda") * 0.05 for s in shapes]
+    ref = [v.double() for v in init]
+    gpu = [torch.nn.Parameter(v.clone()) for v in init]
+    orc = O.EloCelo2Oracle(ref, net.state_dict(), lr=LR, weight_decay=WD, device="cuda").double_()
+    opt = ELO_CELO2_CUDA(gpu, lr=LR, weight_decay=WD, network=net, hf_key=None)
+    for t in range(3):
+        grads = [None if (t == 1 and i == 1) else torch.randn(s, generator=gen, device="cuda") * 0.01
+                 for i, s in enumerate(shapes)]
+        for p, g in zip(gpu, grads):
+            p.grad = g
+        orc.step([None if g is None else g.double() for g in grads])
+        opt.step()
+        for i, p in enumerate(gpu):
+            assert max_err(p, ref[i], 1e-5, 1e-6) <= 1.0, (t, i)
+
+
+def test_flag_on_an_unsupported_tensor_is_refused():
+    import numpy as np
+
+    from pylo_amd import _lib
+
+    plan = _lib.Plan(_lib.KIND_CELO2, [(130, 6), (64, 64)], [0, 0], torch.device("cuda:0"))
+    assert not plan.orthogonalize_supported(0) and plan.orthogonalize_supported(1)
+    x = torch.zeros(130 * 6 + 64 * 64, device="cuda")
+    fin = np.zeros(2, dtype=_lib.ARGS_DTYPE)
+    fin["grad"], fin["param"], fin["step_out"] = 1, x.data_ptr(), x.data_ptr()
+    fin["flags"][0] = _lib.ARG_ORTHOGONALIZE
+    with pytest.raises(RuntimeError, match="cannot orthogonalise"):
+        plan.celo2_orthogonalize_finish(fin, (3.4445, -4.775, 2.0315), 5, 1e-8, 0)
+    plan.close()

@@ -378,12 +378,15 @@ def other_workload(workload, steps, warmup):
     mean = per.mean(axis=0)
     # 1-D tensors also carry the per-element accumulator fac_v: +3 reads in both passes, +3 writes
     bytes_fused = n2d * (B_P0 + B_STATS + B_APPLY) + n1d * (36 + 36 + 32)
+    b_elem, b_vec = B_APPLY, 68
+    if "k_velo_elem" in names:        # statistics and apply items of all tensors in one launch
+        apply_kernel, b_elem, b_vec = "k_velo_elem", B_STATS + B_APPLY, 36 + 68
     k = names.index(apply_kernel)
-    apply_gbs = (n2d * B_APPLY + n1d * 68) / (float(mean[k]) * 1e-3) / 1e9
+    apply_gbs = (n2d * b_elem + n1d * b_vec) / (float(mean[k]) * 1e-3) / 1e9
     roof = {"bound": "hbm", "kernel": apply_kernel, "achieved": apply_gbs, "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": apply_gbs / HBM_PEAK_GBS,
             "traffic": traffic_from_profile("velo_fused_step_vitb16_kernel_trace_and_traffic.txt", apply_kernel) if workload == "vit_velo" else None,
-            "algorithmic_bytes_per_launch": n2d * B_APPLY + n1d * 68, "avg_launch_ms": float(mean[k])}
+            "algorithmic_bytes_per_launch": n2d * b_elem + n1d * b_vec, "avg_launch_ms": float(mean[k])}
     if workload == "llama_adafac":
         # the 16 -> 32 -> 32 -> 2 element MLP: 1 600 FMAs per element of a >= 2-D tensor, fp32 matrix pipe
         tflops = n2d * 3200.0 / (float(mean[k]) * 1e-3) / 1e12

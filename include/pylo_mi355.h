@@ -271,6 +271,17 @@ typedef struct {
 int pylo_mi355_velo_step(PyloPlan* plan, const PyloTensorArgs* args, const PyloDecays* decays,
                          const PyloVeloNets* nets, const PyloVeloStep* step, void* stream);
 
+/* The per-tensor LSTM reads sums over every tensor's parameter, momentum and rms values as they stand
+   BEFORE the step (velo_cuda.py:213-252).  From its second step on a plan does not read the tensors for
+   them: the apply items of step t sum up the values they write, which are the values step t+1 starts from,
+   so the LSTM of step t+1 runs ahead of its statistics pass (next to the gradient sums, on a stream of the
+   plan's own) and statistics and apply items run as one launch.  That holds as long as nobody else writes
+   `param`, `mom` or `rms` of a tensor between two steps of the plan.  A caller who does (loads a checkpoint
+   into them, edits parameters in place, swaps a state tensor) calls this first; the next step then takes the
+   sums from the tensors again, each pass a launch of its own.  No counterpart in the reference, which
+   recomputes everything every step. */
+int pylo_mi355_plan_invalidate_statistics(PyloPlan* plan);
+
 /*
  * AdafacLO step (replaces cuda_lo.learned_optimizer_kernel, pylo/csrc/learned_optimizer.cu:303-394, for
  * every tensor at once, plus the accumulator updates of AdafacLO_cuda.py:291-373 and the weight decay

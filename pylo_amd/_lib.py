@@ -96,6 +96,7 @@ def load():
                                          C.POINTER(VeloStep), C.c_void_p]
     lib.pylo_mi355_adafac_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.c_void_p, C.c_float,
                                            C.c_void_p]
+    lib.pylo_mi355_plan_invalidate_statistics.argtypes = [C.c_void_p]
     lib.pylo_mi355_plan_arg_table.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_void_p)]
     lib.pylo_mi355_plan_device_steps.argtypes = [C.c_void_p, C.POINTER(DeviceSteps)]
     if lib.pylo_mi355_abi_version() != 5:
@@ -212,6 +213,10 @@ class Plan:
     def celo2_finish(self, args: np.ndarray, stream: int) -> None:
         """Normalise + apply after Newton-Schulz; `args` is a table like `self.args` (own array)."""
         check(load().pylo_mi355_celo2_finish(self._h, args.ctypes.data, stream), "celo2_finish")
+
+    def invalidate_statistics(self) -> None:
+        """VeLO: parameters or accumulators were written by someone else since the plan's last step."""
+        check(load().pylo_mi355_plan_invalidate_statistics(self._h), "plan_invalidate_statistics")
 
     def orthogonalize_supported(self, i: int) -> bool:
         return load().pylo_mi355_plan_orthogonalize_supported(self._h, i) == 1

@@ -119,6 +119,48 @@ __device__ __forceinline__ void lstm_pivots(const TDesc& d, const PyloTensorArgs
   }
 }
 
+// What the apply pass adds up over the values it WRITES, for the LSTM features of the next step (they are
+// that step's "accumulators before the update"): sum p^2, then the shifted sums as in VeloAcc::lstm.  The
+// pivots are the tensor's first elements AFTER this step's update -- what the next step finds there --
+// which every block derives for itself from the first elements before the update (kept per tensor by the
+// kernel that formed the LSTM's inputs, since the apply pass overwrites them while it runs) and the
+// tensor's first gradient element; they are wave-uniform and live in scalar registers.
+constexpr int kNewSumW = 10;    // doubles per row of those partial sums (9 used)
+struct NewSums {
+  float v[9];
+  float piv[4];
+  __device__ __forceinline__ void clear(const TDesc& d, const PyloTensorArgs& a, const EmaConsts& e,
+                                        const float* __restrict__ old_first) {
+#pragma unroll
+    for (int c = 0; c < 9; ++c) v[c] = 0.0f;
+    float of[4];
+    load_uniform<4>(old_first, of);
+    const float g0 = d.n > 0 ? cond_grad(*(const cfloat*)a.grad, d.gscale, a.clip_val, d.nan0) : 0.0f;
+    float m[3] = {of[0], of[1], of[2]};
+    float r = of[3];
+    ema_update(e, g0, m, r);
+    auto uniform = [](float x) {   // the value is the same in every lane: keep it in a scalar register
+      return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
+    };
+    piv[0] = uniform(m[0]);
+    piv[1] = uniform(m[1]);
+    piv[2] = uniform(m[2]);
+    piv[3] = uniform(r);
+  }
+  __device__ __forceinline__ void add(float p_new, const float (&m)[3], float rms) {
+    v[0] = fmaf(p_new, p_new, v[0]);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      const float dm = m[k] - piv[k];
+      v[1 + k] += dm;
+      v[4 + k] = fmaf(dm, dm, v[4 + k]);
+    }
+    const float dr = rms - piv[3];
+    v[7] += dr;
+    v[8] = fmaf(dr, dr, v[8]);
+  }
+};
+
 __device__ __forceinline__ void lstm_sums(const float (&m)[3], float rms, VeloAcc& acc) {
 #pragma unroll
   for (int k = 0; k < 3; ++k) {
@@ -155,6 +197,9 @@ __device__ __forceinline__ void velo_stats_fac(const TDesc& d, const PyloTensorA
 
 // Column-resident walk of one wave task (wide 2-D tensors): column factors in registers, row
 // factors through the scalar cache, six streams per row.
+// KEEP: plain loads, which leave the lines in the memory-side cache for the apply items that follow
+// (k_velo_elem); otherwise non-temporal loads (see celo2_stats_tile).
+template <bool KEEP>
 __device__ __forceinline__ void velo_stats_tile(const TDesc& d, const PyloTensorArgs& a, int task,
                                                 const EmaConsts& e, const float* __restrict__ fac_tab,
                                                 VeloAcc& acc) {
@@ -172,12 +217,21 @@ __device__ __forceinline__ void velo_stats_tile(const TDesc& d, const PyloTensor
 #pragma unroll 2
   for (int r = tk.r0; r < tk.r1; ++r) {
     float xg[V], xp[V], x0[V], x1[V], x2[V], xr[V], fa[4];
-    load_vec_nt<V>(g, lo, xg);
-    load_vec_nt<V>(p, lo, xp);
-    load_vec_nt<V>(m0, lo, x0);
-    load_vec_nt<V>(m1, lo, x1);
-    load_vec_nt<V>(m2, lo, x2);
-    load_vec_nt<V>(rms, lo, xr);
+    if constexpr (KEEP) {
+      load_vec_o<V>(g, lo, xg);
+      load_vec_o<V>(p, lo, xp);
+      load_vec_o<V>(m0, lo, x0);
+      load_vec_o<V>(m1, lo, x1);
+      load_vec_o<V>(m2, lo, x2);
+      load_vec_o<V>(rms, lo, xr);
+    } else {
+      load_vec_nt<V>(g, lo, xg);
+      load_vec_nt<V>(p, lo, xp);
+      load_vec_nt<V>(m0, lo, x0);
+      load_vec_nt<V>(m1, lo, x1);
+      load_vec_nt<V>(m2, lo, x2);
+      load_vec_nt<V>(rms, lo, xr);
+    }
     load_uniform<4>(fr, fa);
 #pragma unroll
     for (int v = 0; v < V; ++v) {
@@ -276,16 +330,12 @@ __device__ __forceinline__ void velo_stats_vec(const TDesc& d, const PyloTensorA
   }
 }
 
-__global__ __launch_bounds__(kThreads) void k_velo_stats(const TDesc* __restrict__ descs,
-                                                         const PyloTensorArgs* __restrict__ dyn,
-                                                         const Item* __restrict__ items,
-                                                         const float* __restrict__ fac_tab, PyloDecays dec,
-                                                         double* __restrict__ stats_part) {
-  __shared__ float red[kWaves][38];
-  const Item it = items[blockIdx.x];
-  const TDesc d = descs[it.tensor];
-  const PyloTensorArgs a = dyn[it.tensor];
-  if (a.grad == nullptr) return;
+// One block of the statistics pass (channel sums and, when nobody carried them over, the LSTM's sums).
+// Returns after a barrier with the four waves' sums in `red`.
+template <bool LSTM_SUMS, bool KEEP>
+__device__ __forceinline__ void velo_stats_block(const TDesc& d, const PyloTensorArgs& a, const Item& it,
+                                                 const float* __restrict__ fac_tab, const PyloDecays& dec,
+                                                 float (*red)[38]) {
   const EmaConsts e = make_ema(dec);
   VeloAcc acc;
 #pragma unroll
@@ -295,7 +345,7 @@ __global__ __launch_bounds__(kThreads) void k_velo_stats(const TDesc* __restrict
   lstm_pivots(d, a, acc.piv);
   if (d.tile_nct > 0) {
     const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (task < d.tile_ntask) velo_stats_tile(d, a, task, e, fac_tab, acc);
+    if (task < d.tile_ntask) velo_stats_tile<KEEP>(d, a, task, e, fac_tab, acc);
   } else if (d.mode == kModeFac2D) {
     if (d.vec == 4) velo_stats_fac<4, false>(d, a, it.a, e, fac_tab, acc);
     else velo_stats_fac<1, false>(d, a, it.a, e, fac_tab, acc);
@@ -311,12 +361,27 @@ __global__ __launch_bounds__(kThreads) void k_velo_stats(const TDesc* __restrict
     const float s = wave_sum(acc.ch[c]);
     if (lane == 0) red[wave][c] = s;
   }
+  if (LSTM_SUMS) {
 #pragma unroll
-  for (int c = 0; c < 8; ++c) {
-    const float s = wave_sum(acc.lstm[c]);
-    if (lane == 0) red[wave][30 + c] = s;
+    for (int c = 0; c < 8; ++c) {
+      const float s = wave_sum(acc.lstm[c]);
+      if (lane == 0) red[wave][30 + c] = s;
+    }
   }
   __syncthreads();
+}
+
+__global__ __launch_bounds__(kThreads) void k_velo_stats(const TDesc* __restrict__ descs,
+                                                         const PyloTensorArgs* __restrict__ dyn,
+                                                         const Item* __restrict__ items,
+                                                         const float* __restrict__ fac_tab, PyloDecays dec,
+                                                         double* __restrict__ stats_part) {
+  __shared__ float red[kWaves][38];
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  velo_stats_block<true, false>(d, a, it, fac_tab, dec, red);
   if (threadIdx.x < 38) {
     const int c = threadIdx.x;
     stats_part[(size_t)blockIdx.x * kStatW + c] =
@@ -386,8 +451,11 @@ __device__ __forceinline__ float clip_log_abs10(double v) {
 }
 
 // Feature q of the 30 LSTM inputs of one tensor from its totals (Velo_naive.py:178-206).
+// piv_in: the pivots the totals were shifted by when they are not the tensor's first elements as they stand
+// (totals carried over from the previous step's apply pass), else null.
 __device__ __forceinline__ float lo_lstm_feature(const TDesc& d, const PyloTensorArgs& a, const double* tot,
-                                                 const float* __restrict__ lossfeat, const VeloStep& st, int q) {
+                                                 const float* __restrict__ lossfeat, const VeloStep& st, int q,
+                                                 const float* piv_in = nullptr) {
   const double n = (double)(d.n > 0 ? d.n : 1);
 
   const float nu = rsq(fmaxf((float)(tot[2] / n), 1e-9f));
@@ -400,7 +468,8 @@ __device__ __forceinline__ float lo_lstm_feature(const TDesc& d, const PyloTenso
   } else {
     // totals are of the accumulators shifted by the tensor's pivots (VeloAcc)
     float piv[4];
-    lstm_pivots(d, a, piv);
+    if (piv_in != nullptr) { piv[0] = piv_in[0]; piv[1] = piv_in[1]; piv[2] = piv_in[2]; piv[3] = piv_in[3]; }
+    else lstm_pivots(d, a, piv);
     const double dr = tot[kSumR] / n;
     const double mean_r = (double)piv[3] + dr;
     if (q == 18) {
@@ -424,6 +493,38 @@ __device__ __forceinline__ float lo_lstm_feature(const TDesc& d, const PyloTenso
 }
 
 
+// Row T-1-t of the LSTM input: the tensor's 30 features from its totals and its share of the input mixing
+// (VeLO_RNN.py:110-122): relu(mix2 x) and final_mix x for every hidden unit; the maximum over rows and the sum
+// follow in k_velo_mix.  Afterwards the tensor's pivots for the sums its apply pass will take are stored
+// (its accumulators' first elements as they stand now; the apply pass overwrites them while it runs).
+__device__ __forceinline__ void velo_row_features(const TDesc& d, const PyloTensorArgs& a, int t, int T,
+                                                  const double* tot, const float* piv_in, float* __restrict__ piv_out,
+                                                  const LossState& ls, const VeloStep& st, float* __restrict__ xfeat,
+                                                  int H, const float* __restrict__ w2t, const float* __restrict__ b2,
+                                                  const float* __restrict__ wft, const float* __restrict__ bf,
+                                                  float* __restrict__ mixbuf, float* xs) {
+  const int row = T - 1 - t;
+  __shared__ float cor_s[10], rmin_s[10], lossfeat[9];
+  loss_step(ls.means, ls.running_min, ls.decays, ls.iteration, ls.loss, false, cor_s, rmin_s, lossfeat);
+  if (threadIdx.x < 30) xs[threadIdx.x] = lo_lstm_feature(d, a, tot, lossfeat, st, threadIdx.x, piv_in);
+  __syncthreads();
+  if (piv_out != nullptr && threadIdx.x == 0) {
+    float pv[4];
+    lstm_pivots(d, a, pv);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) piv_out[(size_t)t * 4 + q] = pv[q];
+  }
+  if (threadIdx.x < 30) xfeat[(size_t)row * kXW + threadIdx.x] = xs[threadIdx.x];
+  for (int i = threadIdx.x; i < 2 * H; i += kFoldThreads) {
+    const int u = i < H ? i : i - H;
+    const float* w = i < H ? w2t : wft;
+    float acc = i < H ? b2[u] : bf[u];
+#pragma unroll
+    for (int k = 0; k < 30; ++k) acc = fmaf(xs[k], w[k * H + u], acc);
+    mixbuf[((size_t)(i < H ? 0 : 1) * T + row) * H + u] = i < H ? fmaxf(acc, 0.0f) : acc;
+  }
+}
+
 __global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restrict__ descs,
                                                         const PyloTensorArgs* __restrict__ dyn, int T,
                                                         const double* __restrict__ stats_part,
@@ -433,7 +534,8 @@ __global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restr
                                                         float* __restrict__ xfeat, int H,
                                                         const float* __restrict__ w2t, const float* __restrict__ b2,
                                                         const float* __restrict__ wft, const float* __restrict__ bf,
-                                                        float* __restrict__ mixbuf /* [2][T][H]: relu(mix2 x), final_mix x */) {
+                                                        float* __restrict__ mixbuf /* [2][T][H]: relu(mix2 x), final_mix x */,
+                                                        float* __restrict__ piv_out /* [T][4], VeLO: see velo_row_features */) {
   constexpr int G = kFoldThreads / kStatW;  // 25 groups x 40 sums = 1000 threads
   __shared__ double part[G][kStatW];
   __shared__ double tot[kStatW];
@@ -461,22 +563,55 @@ __global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restr
   }
   __syncthreads();
   if (xfeat == nullptr) return;
-  const int row = T - 1 - t;
-  __shared__ float cor_s[10], rmin_s[10], lossfeat[9];
-  loss_step(ls.means, ls.running_min, ls.decays, ls.iteration, ls.loss, false, cor_s, rmin_s, lossfeat);
-  if (threadIdx.x < 30) xs[threadIdx.x] = lo_lstm_feature(d, a, tot, lossfeat, st, threadIdx.x);
-  __syncthreads();
-  if (threadIdx.x < 30) xfeat[(size_t)row * kXW + threadIdx.x] = xs[threadIdx.x];
-  // the row's share of the LSTM input mixing (VeLO_RNN.py:110-122): relu(mix2 x) and final_mix x for every
-  // hidden unit; the maximum over rows and the sum follow in k_velo_mix
-  for (int i = threadIdx.x; i < 2 * H; i += kFoldThreads) {
-    const int u = i < H ? i : i - H;
-    const float* w = i < H ? w2t : wft;
-    float acc = i < H ? b2[u] : bf[u];
+  velo_row_features(d, a, t, T, tot, nullptr, piv_out, ls, st, xfeat, H, w2t, b2, wft, bf, mixbuf, xs);
+}
+
+// The same from the sums the previous step's apply pass left (rows of kNewSumW doubles per element
+// block, shifted by the tensor's first elements as that pass wrote them, i.e. as they stand now): the
+// LSTM does not wait for this step's statistics pass.
+__global__ __launch_bounds__(kFoldThreads) void k_velo_feat(const TDesc* __restrict__ descs,
+                                                            const PyloTensorArgs* __restrict__ dyn, int T,
+                                                            const double* __restrict__ newsum_part,
+                                                            float* __restrict__ piv, LossState ls, VeloStep st,
+                                                            float* __restrict__ xfeat, int H,
+                                                            const float* __restrict__ w2t, const float* __restrict__ b2,
+                                                            const float* __restrict__ wft, const float* __restrict__ bf,
+                                                            float* __restrict__ mixbuf, int* __restrict__ sync) {
+  constexpr int G = kFoldThreads / kNewSumW;
+  __shared__ double part[G][kNewSumW];
+  __shared__ double tot[kStatW];
+  __shared__ float xs[32];
+  const int t = blockIdx.x;
+  const TDesc d = descs[t];
+  const PyloTensorArgs a = dyn[t];
+  const int c = threadIdx.x % kNewSumW, gI = threadIdx.x / kNewSumW;
+  if (gI < G) {
+    double s = 0.0;
+    const double* rows = newsum_part + (size_t)d.blk0 * kNewSumW;
+    for (int b0 = gI; b0 < d.nblk; b0 += 16 * G) {
+      double v[16];
 #pragma unroll
-    for (int k = 0; k < 30; ++k) acc = fmaf(xs[k], w[k * H + u], acc);
-    mixbuf[((size_t)(i < H ? 0 : 1) * T + row) * H + u] = i < H ? fmaxf(acc, 0.0f) : acc;
+      for (int q = 0; q < 16; ++q) {
+        const int b = b0 + q * G;
+        v[q] = b < d.nblk ? rows[(size_t)b * kNewSumW + c] : 0.0;
+      }
+#pragma unroll
+      for (int q = 0; q < 16; ++q) s += v[q];
+    }
+    part[gI][c] = s;
   }
+  if (threadIdx.x < kStatW) tot[threadIdx.x] = 0.0;
+  // the tensor's counter and flag of the fused element pass that follows (k_velo_elem) start at zero
+  if (threadIdx.x == 0) { sync[t] = 0; sync[T + t] = 0; }
+  __syncthreads();
+  if (threadIdx.x < 9) {
+    double s = 0.0;
+    for (int g2 = 0; g2 < G; ++g2) s += part[g2][threadIdx.x];
+    const int q = threadIdx.x;   // 0: sum p^2 | 1..3: m | 4..6: m^2 | 7: rms | 8: rms^2
+    tot[q == 0 ? 2 : q < 4 ? kSumM + q - 1 : q < 7 ? kSumMM + q - 4 : q == 7 ? kSumR : kSumRR] = s;
+  }
+  __syncthreads();
+  velo_row_features(d, a, t, T, tot, nullptr, piv, ls, st, xfeat, H, w2t, b2, wft, bf, mixbuf, xs);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -631,6 +766,27 @@ __global__ __launch_bounds__(kThreads) void k_velo_gates(const float* __restrict
   }
 }
 
+// Entry i of a tensor's folded weight block (layout at the top of this file) from its un-scaled MLP `wm`
+// (a bank entry's layout, kVBank floats), the channel normalisers sc[30], param_scale and lr_mult.
+// Entries the layout leaves unused read as zero.
+__device__ __forceinline__ float velo_fold_entry(const TDesc& d, const float* wm, const float* sc, float pscale,
+                                                 float lr_mult, int i) {
+  const bool factored = d.mode == kModeFac2D || d.mode == kModeFacND;
+  if (i < kVB1) {
+    const int k = i / 4, j = i % 4;
+    if (factored) return k < kNStat ? wm[j * 30 + stat_channel(k)] * sc[stat_channel(k)] : 0.0f;
+    return wm[j * 30 + k] * sc[k];
+  }
+  if (i < kVWH) return wm[120 + (i - kVB1)];
+  if (i < kVBH) return wm[124 + ((i - kVWH) % 4) * 4 + (i - kVWH) / 4];   // (in, out)
+  if (i < kVWO) return wm[140 + (i - kVBH)];
+  if (i < kVBO) return ((i - kVWO) % 4) < 2 ? wm[144 + ((i - kVWO) % 4) * 4 + (i - kVWO) / 4] : 0.0f;   // [k][j], j < 2 used
+  if (i < kVPS) return (i - kVBO) < 2 ? wm[156 + (i - kVBO)] : 0.0f;
+  if (i == kVPS) return pscale;
+  if (i == kVLR) return lr_mult;
+  return 0.0f;
+}
+
 // One block per tensor row r: controls = h Wc^T + bc, lr_mult = h.wlr + blr, the tensor's MLP =
 // 100 * mean_i(control_i * bank_i) (VeLO_MLP.py:92-126), then the weight blocks the element
 // kernels read: un-scaled first layer for k_terms, and the folded block (first-layer rows scaled
@@ -644,7 +800,11 @@ __global__ __launch_bounds__(kFoldThreads) void k_velo_heads(const TDesc* __rest
                                                              const double* __restrict__ totals,
                                                              float* __restrict__ canon, float* __restrict__ wfold,
                                                              float* __restrict__ controls_out,
-                                                             float* __restrict__ lr_mult_out) {
+                                                             float* __restrict__ lr_mult_out,
+                                                             float* __restrict__ wmix) {
+  // totals == nullptr: the channel sums of this step are not known yet (the LSTM runs ahead of the
+  // statistics pass); the tensor's un-scaled MLP (159 floats) and lr_mult go to wmix[t][160] and the
+  // folded block is written later, by the tensor's last statistics block (k_velo_elem)
   // Both contractions (controls over the H hidden units, the bank mix over the K controls) are cut
   // into four slices that run side by side and are added in a fixed order; eight loads are issued
   // before the first is used, since a block is bound by the bytes it keeps in flight.
@@ -681,7 +841,7 @@ __global__ __launch_bounds__(kFoldThreads) void k_velo_heads(const TDesc* __rest
     s = wave_sum(s);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
   }
-  if (threadIdx.x < 30) {
+  if (threadIdx.x < 30 && totals != nullptr) {
     const double n = (double)(d.n > 0 ? d.n : 1);
     sc[threadIdx.x] = rsq(1e-5f + (float)(totals[(size_t)t * kStatW + threadIdx.x] / n));
   }
@@ -724,28 +884,18 @@ __global__ __launch_bounds__(kFoldThreads) void k_velo_heads(const TDesc* __rest
   }
   __syncthreads();
   float* cn = canon + (size_t)t * kVCanon;
-  float* wf = wfold + (size_t)t * kVFold;
-  const bool factored = d.mode == kModeFac2D || d.mode == kModeFacND;
-  for (int i = threadIdx.x; i < 120; i += kFoldThreads) {
-    const int k = i / 4, j = i % 4;
-    cn[i] = wm[j * 30 + k];
-    if (factored) {
-      if (k < kNStat) wf[kVW1 + i] = wm[j * 30 + stat_channel(k)] * sc[stat_channel(k)];
-    } else {
-      wf[kVW1 + i] = wm[j * 30 + k] * sc[k];
-    }
+  for (int i = threadIdx.x; i < 124; i += kFoldThreads) cn[i] = i < 120 ? wm[(i % 4) * 30 + i / 4] : wm[i];
+  if (threadIdx.x == 0 && lr_mult_out != nullptr) lr_mult_out[r] = lr_mult;
+  if (totals == nullptr) {
+    float* o = wmix + (size_t)t * 160;
+    for (int i = threadIdx.x; i < 160; i += kFoldThreads) o[i] = i < kVBank ? wm[i] : lr_mult;
+    return;
   }
-  if (threadIdx.x < 4) { cn[120 + threadIdx.x] = wm[120 + threadIdx.x]; wf[kVB1 + threadIdx.x] = wm[120 + threadIdx.x]; }
-  if (threadIdx.x < 16) wf[kVWH + threadIdx.x] = wm[124 + (threadIdx.x % 4) * 4 + threadIdx.x / 4];   // (in,out)
-  if (threadIdx.x < 4) wf[kVBH + threadIdx.x] = wm[140 + threadIdx.x];
-  if (threadIdx.x < 16)   // [k][j], j < 2 used
-    wf[kVWO + threadIdx.x] = (threadIdx.x % 4) < 2 ? wm[144 + (threadIdx.x % 4) * 4 + threadIdx.x / 4] : 0.0f;
-  if (threadIdx.x < 4) wf[kVBO + threadIdx.x] = threadIdx.x < 2 ? wm[156 + threadIdx.x] : 0.0f;
-  if (threadIdx.x == 0) {
-    const double n = (double)(d.n > 0 ? d.n : 1);
-    wf[kVPS] = sqrtf((float)(totals[(size_t)t * kStatW + 2] / n) + 1e-9f);
-    wf[kVLR] = lr_mult;
-    if (lr_mult_out != nullptr) lr_mult_out[r] = lr_mult;
+  const double n = (double)(d.n > 0 ? d.n : 1);
+  const float pscale = sqrtf((float)(totals[(size_t)t * kStatW + 2] / n) + 1e-9f);
+  for (int i = threadIdx.x; i < kVFold; i += kFoldThreads) {
+    const float v = velo_fold_entry(d, wm, sc, pscale, lr_mult, i);
+    if (i < kVLR + 1) wfold[(size_t)t * kVFold + i] = v;
   }
 }
 
@@ -783,7 +933,7 @@ __device__ __forceinline__ void velo_hidden(const float (&h0)[4], const cfloat* 
 template <int V, bool ND>
 __device__ __forceinline__ void velo_apply_fac(const TDesc& d, const PyloTensorArgs& a, int chunk,
                                                const EmaConsts& e, const float* __restrict__ fac_tab,
-                                               const float* __restrict__ term_tab, const float* wbase) {
+                                               const float* __restrict__ term_tab, const float* wbase, NewSums& ns) {
   const long long base = (long long)chunk * (kThreads * V * kElemIters);
   const long long n = d.n;
   for (int it = 0; it < kElemIters; ++it) {
@@ -817,6 +967,7 @@ __device__ __forceinline__ void velo_apply_fac(const TDesc& d, const PyloTensorA
       float h1[4];
       velo_hidden(h[v], w, h1);
       pn[v] = velo_update(x.p[v], h1, w, a);
+      ns.add(pn[v], x.m[v], x.rms[v]);
     }
     store_vec<V>(a.mom + idx, m0);
     store_vec<V>(a.mom + n + idx, m1);
@@ -832,15 +983,17 @@ __device__ __forceinline__ void velo_apply_fac(const TDesc& d, const PyloTensorA
 // with the constant 1.
 __device__ __forceinline__ void velo_apply_tile(const TDesc& d, const PyloTensorArgs& a, int task,
                                                 const EmaConsts& e, const float* __restrict__ fac_tab,
-                                                const float* __restrict__ term_tab, const float* wbase) {
+                                                const float* __restrict__ term_tab, const float* wbase, NewSums& ns,
+                                                bool coh) {
+  // coh: the folded block was written by another block of the running kernel (see coh_store_wait)
   constexpr int V = kTileV;
   const TileTask tk(d, task);
   const int lane = threadIdx.x & 63;
   float wreg[3];
 #pragma unroll
-  for (int r = 0; r < 3; ++r) wreg[r] = *(const gfloat*)(wbase + r * 64 + lane);
-  const cfloat* ws = launder(wbase);
-  const float pscale = ws[kVPS], lr_mult = ws[kVLR];
+  for (int r = 0; r < 3; ++r) wreg[r] = coh ? coh_load(wbase + r * 64 + lane) : *(const gfloat*)(wbase + r * 64 + lane);
+  // param_scale and lr_mult sit in floats 164 / 165 of the block, i.e. in lanes 36 / 37 of register 2
+  const float pscale = __shfl(wreg[2], kVPS - 128, 64), lr_mult = __shfl(wreg[2], kVLR - 128, 64);
   const float exp_scale = a.exp_mult * 1.44269504088896341f;
   constexpr int gWH = kVWH / 4, gBH = kVBH / 4, gWO = kVWO / 4, gBO = kVBO / 4;
   const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -916,6 +1069,8 @@ __device__ __forceinline__ void velo_apply_tile(const TDesc& d, const PyloTensor
       float q = fmaf(step, -a.lr, xp[v]);
       if (a.weight_decay > 0.0f) q = fmaf(q, -wd_lr, q);
       pn[v] = q;
+      const float mm[3] = {x0[v], x1[v], x2[v]};
+      ns.add(q, mm, xr[v]);
     }
     store_vec_o<V>(p, lo, pn);
     g += d.C0; p += d.C0; m0 += d.C0; m1 += d.C0; m2 += d.C0; rms += d.C0;
@@ -925,7 +1080,8 @@ __device__ __forceinline__ void velo_apply_tile(const TDesc& d, const PyloTensor
 
 template <int V>
 __device__ __forceinline__ void velo_apply_vec(const TDesc& d, const PyloTensorArgs& a, int chunk,
-                                               const EmaConsts& e, const PyloDecays& dec, const float* wbase) {
+                                               const EmaConsts& e, const PyloDecays& dec, const float* wbase,
+                                               NewSums& ns) {
   const long long base = (long long)chunk * (kThreads * V * kElemIters);
   const long long n = d.n;
   for (int it = 0; it < kElemIters; ++it) {
@@ -951,6 +1107,7 @@ __device__ __forceinline__ void velo_apply_vec(const TDesc& d, const PyloTensorA
       float h1[4];
       velo_hidden(h0, w, h1);
       pn[v] = velo_update(x.p[v], h1, w, a);
+      ns.add(pn[v], x.m[v], x.rms[v]);
 #pragma unroll
       for (int k = 0; k < 3; ++k) { mo[k][v] = x.m[v][k]; vo[k][v] = x.v[v][k]; }
     }
@@ -964,30 +1121,164 @@ __device__ __forceinline__ void velo_apply_vec(const TDesc& d, const PyloTensorA
   }
 }
 
-__global__ __launch_bounds__(kThreads) void k_velo_apply(const TDesc* __restrict__ descs,
+// One block of the apply pass; its sums over the written values go to row `row` of newsum_part.
+__device__ __forceinline__ void velo_apply_block(const TDesc& d, const PyloTensorArgs& a, const Item& it,
+                                                 const float* __restrict__ fac_tab,
+                                                 const float* __restrict__ term_tab, const PyloDecays& dec,
+                                                 const float* __restrict__ wfold, const float* __restrict__ piv,
+                                                 double* __restrict__ newsum_part, int row, bool coh, float (*red)[9]) {
+  const EmaConsts e = make_ema(dec);
+  const float* w = wfold + (size_t)it.tensor * kVFold;
+  NewSums ns;
+  ns.clear(d, a, e, piv + (size_t)it.tensor * 4);
+  if (d.tile_nct > 0) {
+    const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (task < d.tile_ntask) velo_apply_tile(d, a, task, e, fac_tab, term_tab, w, ns, coh);
+  } else if (d.mode == kModeFac2D) {
+    if (d.vec == 4) velo_apply_fac<4, false>(d, a, it.a, e, fac_tab, term_tab, w, ns);
+    else velo_apply_fac<1, false>(d, a, it.a, e, fac_tab, term_tab, w, ns);
+  } else if (d.mode == kModeFacND) {
+    velo_apply_fac<1, true>(d, a, it.a, e, fac_tab, term_tab, w, ns);
+  } else {
+    if (d.vec == 4) velo_apply_vec<4>(d, a, it.a, e, dec, w, ns);
+    else velo_apply_vec<1>(d, a, it.a, e, dec, w, ns);
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int c = 0; c < 9; ++c) {
+    const float sc = wave_sum(ns.v[c]);
+    if (lane == 0) red[wave][c] = sc;
+  }
+  __syncthreads();
+  if (threadIdx.x < 9) {
+    const int c = threadIdx.x;
+    newsum_part[(size_t)row * kNewSumW + c] =
+        ((double)red[0][c] + (double)red[1][c]) + ((double)red[2][c] + (double)red[3][c]);
+  }
+}
+
+// Apply pass as a launch of its own.
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void k_velo_apply(const TDesc* __restrict__ descs,
                                                          const PyloTensorArgs* __restrict__ dyn,
                                                          const Item* __restrict__ items,
                                                          const float* __restrict__ fac_tab,
                                                          const float* __restrict__ term_tab, PyloDecays dec,
-                                                         const float* __restrict__ wfold) {
+                                                         const float* __restrict__ wfold,
+                                                         const float* __restrict__ piv,
+                                                         double* __restrict__ newsum_part) {
+  __shared__ float red[kWaves][9];
   const Item it = items[blockIdx.x];
   const TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
-  const EmaConsts e = make_ema(dec);
-  const float* w = wfold + (size_t)it.tensor * kVFold;
-  if (d.tile_nct > 0) {
-    const int task = it.a * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (task < d.tile_ntask) velo_apply_tile(d, a, task, e, fac_tab, term_tab, w);
-  } else if (d.mode == kModeFac2D) {
-    if (d.vec == 4) velo_apply_fac<4, false>(d, a, it.a, e, fac_tab, term_tab, w);
-    else velo_apply_fac<1, false>(d, a, it.a, e, fac_tab, term_tab, w);
-  } else if (d.mode == kModeFacND) {
-    velo_apply_fac<1, true>(d, a, it.a, e, fac_tab, term_tab, w);
-  } else {
-    if (d.vec == 4) velo_apply_vec<4>(d, a, it.a, e, dec, w);
-    else velo_apply_vec<1>(d, a, it.a, e, dec, w);
+  velo_apply_block(d, a, it, fac_tab, term_tab, dec, wfold, piv, newsum_part, (int)blockIdx.x, false, red);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The fused element pass of VeLO: statistics, weight folding and apply items of every tensor in ONE
+// launch, ordered slab by slab, exactly as k_celo2_elem does it (see there for the ordering, the
+// hand-over between running blocks and why a wait ends).  It needs the tensors' MLPs before it starts,
+// i.e. an LSTM that does not depend on this step's statistics pass: the LSTM's inputs are sums over the
+// parameters and accumulators as they stand BEFORE the step, which are the values the previous step's
+// apply items wrote and summed up on the way (NewSums, k_velo_feat).  The tensor's last statistics
+// block folds this step's channel normalisers, param_scale and lr_mult into the block the apply
+// items read.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void k_velo_elem(const TDesc* __restrict__ descs,
+                                                        const PyloTensorArgs* __restrict__ dyn,
+                                                        const Item* __restrict__ items,
+                                                        const float* __restrict__ fac_tab,
+                                                        const float* __restrict__ term_tab, PyloDecays dec,
+                                                        const float* __restrict__ wmix, float* __restrict__ wfold,
+                                                        double* __restrict__ stats_part, const float* __restrict__ piv,
+                                                        double* __restrict__ newsum_part, int* __restrict__ sync,
+                                                        int n_tensors) {
+  __shared__ float red[kWaves][38];
+  __shared__ double part[kThreads / 30][30];
+  __shared__ float sc[30];
+  __shared__ int s_flag;
+  const Item it = items[blockIdx.x];
+  const TDesc d = descs[it.tensor];
+  const PyloTensorArgs a = dyn[it.tensor];
+  if (a.grad == nullptr) return;
+  if (it.c & kElemApply) {
+    if (threadIdx.x == 0) {
+      const int* ready = sync + n_tensors + it.tensor;
+      int ok = coh_load(ready);
+      for (int spin = 0; !ok && spin < kSpinLimit; ++spin) {
+        __builtin_amdgcn_s_sleep(16);
+        ok = coh_load(ready);
+      }
+      s_flag = ok;
+    }
+    __syncthreads();
+    if (s_flag) {
+      velo_apply_block(d, a, it, fac_tab, term_tab, dec, wfold, piv, newsum_part, it.b, true,
+                       reinterpret_cast<float(*)[9]>(&red[0][0]));
+    } else {
+      // gave up waiting (see k_celo2_elem): NaN parameters for this block's elements rather than a hang
+      const float nan = __builtin_nanf("");
+      if (d.tile_nct > 0) {
+        const int task = it.a * 4 + (threadIdx.x >> 6);
+        if (task < d.tile_ntask) {
+          const TileTask tk(d, task);
+          for (int r = tk.r0; r < tk.r1; ++r)
+            for (int v = 0; v < kTileV; ++v) a.param[(size_t)r * d.C0 + tk.col + v] = nan;
+        }
+      } else {
+        const long long chunk = (long long)kThreads * d.vec * kElemIters, base = (long long)it.a * chunk;
+        for (long long i = base + threadIdx.x; i < base + chunk && i < d.n; i += kThreads) a.param[i] = nan;
+      }
+    }
+    return;
   }
+  // the LSTM's sums were carried over: nobody reads them here
+  if (it.c & kElemKeep) velo_stats_block<false, true>(d, a, it, fac_tab, dec, red);
+  else velo_stats_block<false, false>(d, a, it, fac_tab, dec, red);
+  if (threadIdx.x < 30) {
+    const int c = threadIdx.x;
+    coh_store_wait(stats_part + (size_t)it.b * kStatW + c,
+                   ((double)red[0][c] + (double)red[1][c]) + ((double)red[2][c] + (double)red[3][c]));
+  }
+  __syncthreads();
+  if (threadIdx.x == 0)
+    s_flag = __hip_atomic_fetch_add(sync + it.tensor, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == d.nblk - 1;
+  __syncthreads();
+  if (!s_flag) return;
+  // the tensor's last statistics block: channel sums in row order, then the folded block
+  constexpr int G = kThreads / 30;
+  const int c = threadIdx.x % 30, gI = threadIdx.x / 30;
+  if (gI < G) {
+    const double* rows = stats_part + (size_t)d.blk0 * kStatW;
+    double s = 0.0;
+    for (int b0 = gI; b0 < d.nblk; b0 += 16 * G) {
+      double v[16];
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int b = b0 + q * G;
+        v[q] = b < d.nblk ? coh_load(rows + (size_t)b * kStatW + c) : 0.0;
+      }
+#pragma unroll
+      for (int q = 0; q < 16; ++q) s += v[q];
+    }
+    part[gI][c] = s;
+  }
+  __syncthreads();
+  __shared__ float pscale_s;
+  if (threadIdx.x < 30) {
+    double s = 0.0;
+    for (int g2 = 0; g2 < G; ++g2) s += part[g2][threadIdx.x];
+    const double n = (double)(d.n > 0 ? d.n : 1);
+    sc[threadIdx.x] = rsq(1e-5f + (float)(s / n));
+    if (threadIdx.x == 2) pscale_s = sqrtf((float)(s / n) + 1e-9f);   // channel 2 is the parameter
+  }
+  __syncthreads();
+  const float* wm = wmix + (size_t)it.tensor * 160;
+  if (threadIdx.x < kVFold)
+    coh_store_wait(wfold + (size_t)it.tensor * kVFold + threadIdx.x,
+                   velo_fold_entry(d, wm, sc, pscale_s, wm[kVBank], threadIdx.x));
+  __syncthreads();   // every folded weight has been performed
+  if (threadIdx.x == 0) __hip_atomic_store(sync + n_tensors + it.tensor, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace pylo

@@ -73,6 +73,7 @@ bool factored_dims(int kind, const PyloTensorShape& s, int* dc, int* dr) {
 struct Layout {
   std::vector<Item> mx_items;   // ELO-CELO2: statistics and apply items in slab order (k_celo2_elem)
   size_t off_mx_items = 0, off_sync = 0;
+  size_t off_newsum = 0, off_piv = 0, off_wmix = 0;   // VeLO: sums carried to the next step, pivots, un-folded MLPs
   // ELO-CELO2: Newton-Schulz on the 2-D tensors (k_ns.h)
   std::vector<NsMat> ns_mats;
   std::vector<NsItem> ns_gram, ns_poly, ns_upd;
@@ -115,9 +116,11 @@ long long env_slab_elems() {
   if (v && v[0]) return std::atoll(v);
   return 2400000;
 }
-int env_slab_depth() {   // slabs of statistics items between a slab's statistics and its apply items
+// Slabs of statistics items between a slab's statistics and its apply items (measured: ELO-CELO2 on the
+// GPT-2-small set 1.49 / 1.48 ms a step with 2 / 3, VeLO on the ViT-B/16 set 1.06 / 1.00 / 1.04 ms with 1 / 2 / 3).
+int env_slab_depth(int kind) {
   const char* v = std::getenv("PYLO_MI355_SLAB_DEPTH");
-  return (v && v[0]) ? std::max(1, std::atoi(v)) : 3;
+  return (v && v[0]) ? std::max(1, std::atoi(v)) : (kind == PYLO_KIND_VELO ? 2 : 3);
 }
 long long env_keep_elems() {   // largest tensor whose inputs are still expected in the cache when its apply items run
   const char* v = std::getenv("PYLO_MI355_KEEP_ELEMS");
@@ -134,7 +137,7 @@ int tile_rows_for(int kind) {
 // k_p0 read last).  A tensor too large to stay cached is streamed: its statistics items are cut into
 // slab-sized pieces (so that the apply items of the slabs before it keep their place two pieces behind),
 // and its apply items follow its last piece, last item first: they start on what was read last.
-void build_elem_items(Layout& L, int T) {
+void build_elem_items(Layout& L, int T, int kind) {
   struct Piece { int st0, st1, ap0, ap1; bool keep; };   // statistics items [st0, st1); apply items [ap0, ap1) or none
   const long long cap = env_slab_elems(), keep_max = env_keep_elems();
   if (cap <= 0) return;
@@ -166,7 +169,7 @@ void build_elem_items(Layout& L, int T) {
     elems += d.n;
   }
   close();
-  const int np = (int)pieces.size(), depth = env_slab_depth();
+  const int np = (int)pieces.size(), depth = env_slab_depth(kind);
   auto push = [&](int i0, int i1, bool apply, bool keep) {
     const int n0 = (int)L.mx_items.size();
     for (int i = i0; i < i1; ++i) {
@@ -404,7 +407,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       }
     }
   }
-  if (kind == PYLO_KIND_CELO2) build_elem_items(L, T);
+  if (kind == PYLO_KIND_CELO2 || kind == PYLO_KIND_VELO) build_elem_items(L, T, kind);
   size_t off = 0;
   auto take = [&](size_t bytes) {
     size_t o = off;
@@ -451,6 +454,9 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_frac = take(kind == PYLO_KIND_VELO ? sizeof(float) * 9 * PYLO_MAX_GROUPS : 0);
   L.off_mx_items = take(sizeof(Item) * L.mx_items.size());
   L.off_sync = take(sizeof(int) * 2 * (size_t)T);
+  L.off_newsum = take(kind == PYLO_KIND_VELO ? sizeof(double) * kNewSumW * L.el_items.size() : 0);
+  L.off_piv = take(kind == PYLO_KIND_VELO ? sizeof(float) * 4 * (size_t)T : 0);
+  L.off_wmix = take(kind == PYLO_KIND_VELO ? sizeof(float) * 160 * (size_t)T : 0);
   if (kind == PYLO_KIND_CELO2) {
     long long ns_floats = 0;
     build_ns_tables(L, T, ns_floats);
@@ -489,6 +495,11 @@ struct PyloPlan {
   std::vector<hipEvent_t> tev;
   int t_steps_max = 0, t_steps = 0, t_per_step = 0;
   bool timing = false;
+  // VeLO: the LSTM's input sums were left by the previous step's apply items (see k_velo_elem); false
+  // until a step has run and after pylo_mi355_plan_invalidate_statistics
+  bool stats_carried = false;
+  hipStream_t side = nullptr;            // the LSTM runs next to the gradient sums on a stream of the plan's own
+  hipEvent_t ev_fork = nullptr, ev_join = nullptr;
 
   template <class Tp>
   Tp* at(size_t off) const { return reinterpret_cast<Tp*>(ws + off); }
@@ -552,6 +563,11 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
                       hipHostMallocDefault);
     if (e == hipSuccess) e = hipEventCreateWithFlags(&P->ev[i], hipEventDisableTiming);
   }
+  if (e == hipSuccess && kind == PYLO_KIND_VELO && !P->L.mx_items.empty()) {
+    e = hipStreamCreateWithFlags(&P->side, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&P->ev_fork, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&P->ev_join, hipEventDisableTiming);
+  }
   if (e != hipSuccess) {
     pylo_mi355_plan_destroy(P);
     return fail(std::string("plan_create: ") + hipGetErrorString(e));
@@ -563,6 +579,9 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
 int pylo_mi355_plan_destroy(PyloPlan* P) {
   if (!P) return 0;
   for (hipEvent_t e : P->tev) (void)hipEventDestroy(e);
+  if (P->ev_fork) (void)hipEventDestroy(P->ev_fork);
+  if (P->ev_join) (void)hipEventDestroy(P->ev_join);
+  if (P->side) (void)hipStreamDestroy(P->side);
   for (int i = 0; i < kStageSlots; ++i) {
     if (P->ev[i]) (void)hipEventDestroy(P->ev[i]);
     if (P->stage[i]) (void)hipHostFree(P->stage[i]);
@@ -579,6 +598,7 @@ static const char* kVeloLaunches[] = {"k_p0(sums)", "k_p0_nd", "k_v0a", "k_v0b",
                                       "k_lo_reduce", "k_velo_mix", "k_velo_gates", "k_velo_heads", "k_terms",
                                       "k_velo_apply"};
 
+static const char* kVeloFusedLaunches[] = {"k_p0(sums) | LSTM", "k_v0a", "k_v0b", "k_terms", "k_velo_elem"};
 static const char* kAdafacLaunches[] = {"k_p0(sums)", "k_p0_nd", "k_v0a", "k_adafac_bias", "k_v0b", "k_adafac_stats",
                                         "k_lo_reduce", "k_adafac_fold", "k_adafac_apply"};
 
@@ -586,7 +606,8 @@ int pylo_mi355_plan_num_launches(const PyloPlan* P) {
   if (!P) return -1;
   const int n_celo2 = P->L.mx_items.empty() ? (int)(sizeof(kCelo2Launches) / sizeof(kCelo2Launches[0]))
                                             : (int)(sizeof(kCelo2FusedLaunches) / sizeof(kCelo2FusedLaunches[0]));
-  constexpr int n_velo = sizeof(kVeloLaunches) / sizeof(kVeloLaunches[0]);
+  const int n_velo = P->L.mx_items.empty() ? (int)(sizeof(kVeloLaunches) / sizeof(kVeloLaunches[0]))
+                                           : (int)(sizeof(kVeloFusedLaunches) / sizeof(kVeloFusedLaunches[0]));
   constexpr int n_adafac = sizeof(kAdafacLaunches) / sizeof(kAdafacLaunches[0]);
   return P->kind == PYLO_KIND_CELO2 ? n_celo2 : P->kind == PYLO_KIND_VELO ? n_velo : P->kind == PYLO_KIND_ADAFAC ? n_adafac : -1;
 }
@@ -594,7 +615,8 @@ int pylo_mi355_plan_num_launches(const PyloPlan* P) {
 const char* pylo_mi355_plan_launch_name(const PyloPlan* P, int launch) {
   if (!P || launch < 0 || launch >= pylo_mi355_plan_num_launches(P)) return "";
   return P->kind == PYLO_KIND_CELO2 ? (P->L.mx_items.empty() ? kCelo2Launches[launch] : kCelo2FusedLaunches[launch])
-         : P->kind == PYLO_KIND_VELO ? kVeloLaunches[launch] : kAdafacLaunches[launch];
+         : P->kind == PYLO_KIND_VELO ? (P->L.mx_items.empty() ? kVeloLaunches[launch] : kVeloFusedLaunches[launch])
+                                     : kAdafacLaunches[launch];
 }
 
 int pylo_mi355_plan_timing_begin(PyloPlan* P, int max_steps) {
@@ -1039,54 +1061,102 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
   std::memcpy(vs.frac, step->frac, sizeof(vs.frac));
   vs.frac_dev = P->dsteps.counters ? P->at<float>(L.off_frac) : nullptr;
   Marks mark(P, s);
-
-  HIP_TRY(mark());
+  float* piv = P->at<float>(L.off_piv);
+  double* newsum = P->at<double>(L.off_newsum);
+  float* wmix = P->at<float>(L.off_wmix);
+  const LossState ls{step->loss_means, step->loss_running_min, step->loss_decays, step->loss_iteration, step->loss};
+  const int n_chunks = (T + kMixRows - 1) / kMixRows;
+  float* pmax = n_chunks > 1 ? P->at<float>(L.off_pmax) : nullptr;
+  const size_t heads_lds = sizeof(float) * (H + K + 160 + 32 + 16 + 4 * (size_t)std::max(K, 160));
+  // The LSTM from the tensors' 30 input features on: input mixing across tensors, cell, heads.
+  auto lstm = [&](hipStream_t q, const double* tot, bool timed) {
+    if (pmax != nullptr)
+      hipLaunchKernelGGL(k_velo_colmax, dim3(H / 64, n_chunks), dim3(kThreads), 0, q, (const float*)mixbuf, T, H, pmax);
+    hipLaunchKernelGGL(k_velo_mix, dim3(H / 64, L.Tpad / kGateBT), dim3(kThreads), 0, q, (const float*)mixbuf, T, L.Tpad, H,
+                       (const float*)pmax, n_chunks, step->lstm_h, xT, ls);
+    if (timed) (void)mark();
+    hipLaunchKernelGGL(k_velo_gates, dim3((L.Tpad / kGateBT) * (H / kGateU)), dim3(kThreads), 0, q, xT, T, L.Tpad, H,
+                       nets->lstm_wt, nets->lstm_b, step->lstm_h, step->lstm_c);
+    if (timed) (void)mark();
+    hipLaunchKernelGGL(k_velo_heads, dim3(T), dim3(kFoldThreads), heads_lds, q, descs, T, H, K, step->lstm_h,
+                       nets->ctrl_wt, nets->ctrl_b, nets->lr_w, nets->lr_b, nets->bank, tot, canon, wfold,
+                       step->controls_out, step->lr_mult_out, wmix);
+    if (timed) (void)mark();
+  };
   // clip_norm is 0 for VeLO tensors: k_p0 clamps directly; its norm / flag outputs are not used
   // no global norm to wait for: the N-D tensors' sums ride in the tail blocks of the same launch
-  if (n_p0 + n_nd > 0)
-    hipLaunchKernelGGL(k_p0, dim3(n_p0 + n_nd), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0,
-                       nd_items, n_p0);
+  auto gradient_sums = [&]() {
+    if (n_p0 + n_nd > 0)
+      hipLaunchKernelGGL(k_p0, dim3(n_p0 + n_nd), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0,
+                         nd_items, n_p0);
+  };
+  auto factor_tables = [&]() {
+    if (n_v0a > 0)
+      hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kV0aThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
+    HIP_TRY(mark());
+    if (n_v0b > 0)
+      hipLaunchKernelGGL(k_v0b<4>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-5f,
+                         (const float*)nullptr, (const float*)nullptr, 0, fac_tab, term_tab, bscale);
+    HIP_TRY(mark());
+    return 0;
+  };
+  const int n_mx = (int)L.mx_items.size();
   HIP_TRY(mark());
+  if (n_mx > 0 && P->stats_carried) {
+    // The LSTM's inputs are sums over the parameters and accumulators as they stand before the step: the
+    // previous step's apply items left them.  It runs next to the gradient sums, on the plan's own stream.
+    HIP_TRY(hipEventRecord(P->ev_fork, s));
+    HIP_TRY(hipStreamWaitEvent(P->side, P->ev_fork, 0));
+    hipLaunchKernelGGL(k_velo_feat, dim3(T), dim3(kFoldThreads), 0, P->side, descs, dyn, T, (const double*)newsum, piv, ls, vs,
+                       xfeat, H, nets->mix2_wt, nets->mix2_b, nets->fmix_wt, nets->fmix_b, mixbuf, P->at<int>(L.off_sync));
+    lstm(P->side, nullptr, false);
+    HIP_TRY(hipEventRecord(P->ev_join, P->side));
+    gradient_sums();
+    HIP_TRY(mark());
+    if (int rc = factor_tables()) return rc;
+    HIP_TRY(hipStreamWaitEvent(s, P->ev_join, 0));
+    if (n_v0b > 0)
+      hipLaunchKernelGGL(k_terms<4>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, bscale, canon, kVCanon, term_tab);
+    HIP_TRY(mark());
+    hipLaunchKernelGGL(k_velo_elem, dim3(n_mx), dim3(kThreads), 0, s, descs, dyn, P->at<Item>(L.off_mx_items), fac_tab, term_tab,
+                       dec, (const float*)wmix, wfold, stats, (const float*)piv, newsum, P->at<int>(L.off_sync), T);
+    HIP_TRY(mark());
+    mark.done();
+    HIP_TRY(hipGetLastError());
+    return 0;
+  }
+  // Each pass as a launch of its own: the first step of a plan, a step after its carried sums were
+  // invalidated, and every step with PYLO_MI355_SLAB_ELEMS=0.
+  gradient_sums();
   HIP_TRY(mark());
-  if (n_v0a > 0)
-    hipLaunchKernelGGL(k_v0a, dim3(n_v0a), dim3(kV0aThreads), 0, s, descs, dyn, v0a_items, part, gl, dec, v0part);
-  HIP_TRY(mark());
-  if (n_v0b > 0)
-    hipLaunchKernelGGL(k_v0b<4>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, v0part, 1e-5f,
-                       (const float*)nullptr, (const float*)nullptr, 0, fac_tab, term_tab, bscale);
-  HIP_TRY(mark());
+  if (n_mx == 0) HIP_TRY(mark());
+  if (int rc = factor_tables()) return rc;
   if (n_el > 0) hipLaunchKernelGGL(k_velo_stats, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, dec, stats);
-  HIP_TRY(mark());
-  const LossState ls{step->loss_means, step->loss_running_min, step->loss_decays, step->loss_iteration, step->loss};
+  if (n_mx == 0) HIP_TRY(mark());
   const Item* seg_items = P->at<Item>(L.off_seg_items);
   double* seg_tot = P->at<double>(L.off_segtot);
   const int n_seg = (int)L.seg_items.size();
   if (n_seg > 0) hipLaunchKernelGGL(k_stat_segsum, dim3(n_seg), dim3(kThreads), 0, s, descs, seg_items, stats, seg_tot);
   hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, seg_tot, totals, ls, vs, xfeat,
-                     H, nets->mix2_wt, nets->mix2_b, nets->fmix_wt, nets->fmix_b, mixbuf);
-  HIP_TRY(mark());
-  const int n_chunks = (T + kMixRows - 1) / kMixRows;
-  float* pmax = n_chunks > 1 ? P->at<float>(L.off_pmax) : nullptr;
-  if (pmax != nullptr)
-    hipLaunchKernelGGL(k_velo_colmax, dim3(H / 64, n_chunks), dim3(kThreads), 0, s, (const float*)mixbuf, T, H, pmax);
-  hipLaunchKernelGGL(k_velo_mix, dim3(H / 64, L.Tpad / kGateBT), dim3(kThreads), 0, s, (const float*)mixbuf, T, L.Tpad, H,
-                     (const float*)pmax, n_chunks, step->lstm_h, xT, ls);
-  HIP_TRY(mark());
-  hipLaunchKernelGGL(k_velo_gates, dim3((L.Tpad / kGateBT) * (H / kGateU)), dim3(kThreads), 0, s, xT, T, L.Tpad, H,
-                     nets->lstm_wt, nets->lstm_b, step->lstm_h, step->lstm_c);
-  HIP_TRY(mark());
-  hipLaunchKernelGGL(k_velo_heads, dim3(T), dim3(kFoldThreads),
-                     sizeof(float) * (H + K + 160 + 32 + 16 + 4 * (size_t)std::max(K, 160)), s, descs, T, H, K,
-                     step->lstm_h, nets->ctrl_wt, nets->ctrl_b, nets->lr_w, nets->lr_b, nets->bank, totals, canon, wfold,
-                     step->controls_out, step->lr_mult_out);
-  HIP_TRY(mark());
+                     H, nets->mix2_wt, nets->mix2_b, nets->fmix_wt, nets->fmix_b, mixbuf, piv);
+  if (n_mx == 0) HIP_TRY(mark());
+  lstm(s, totals, n_mx == 0);   // the LSTM's launches have intervals of their own only in the launch list without k_velo_elem
   if (n_v0b > 0)
     hipLaunchKernelGGL(k_terms<4>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, bscale, canon, kVCanon, term_tab);
   HIP_TRY(mark());
-  if (n_el > 0) hipLaunchKernelGGL(k_velo_apply, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, term_tab, dec, wfold);
+  if (n_el > 0)
+    hipLaunchKernelGGL(k_velo_apply, dim3(n_el), dim3(kThreads), 0, s, descs, dyn, el_items, fac_tab, term_tab, dec, wfold,
+                       (const float*)piv, newsum);
   HIP_TRY(mark());
   mark.done();
   HIP_TRY(hipGetLastError());
+  P->stats_carried = n_mx > 0;
+  return 0;
+}
+
+extern "C" int pylo_mi355_plan_invalidate_statistics(PyloPlan* P) {
+  if (!P) return fail("plan_invalidate_statistics: null plan");
+  P->stats_carried = false;
   return 0;
 }
 
@@ -1164,7 +1234,7 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   if (n_seg > 0) hipLaunchKernelGGL(k_stat_segsum, dim3(n_seg), dim3(kThreads), 0, s, descs, seg_items, stats, seg_tot);
   hipLaunchKernelGGL(k_lo_reduce, dim3(T), dim3(kFoldThreads), 0, s, descs, dyn, T, stats, seg_tot, totals, LossState{}, vs,
                      (float*)nullptr, 0, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
-                     (const float*)nullptr, (float*)nullptr);
+                     (const float*)nullptr, (float*)nullptr, (float*)nullptr);
   HIP_TRY(mark());
   hipLaunchKernelGGL(k_adafac_fold, dim3(T), dim3(kThreads), 0, s, descs, dyn, totals, net, wfold);
   HIP_TRY(mark());

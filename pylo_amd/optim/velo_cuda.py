@@ -327,12 +327,15 @@ class VeLO_CUDA(Optimizer):
                     fast = self._fast = None
                     break
         if fast is not None:
-            for state, key, t in fast["alive"]:
-                if state.get(key) is not t:   # a state tensor was replaced: the cached pointers are stale
+            for state, mom, rms in fast["alive"]:
+                # a state tensor was replaced: the cached pointers are stale (and so are the carried sums)
+                if state.get("mom") is not mom or state.get("rms") is not rms:
                     fast = self._fast = None
                     break
             else:
-                if any(a is not p for a, (_, _, p) in zip(fast["params"], tensors)):
+                # a parameter object was swapped, or written in place through torch since the last step
+                # (the library's own writes do not count in `_version`)
+                if any(a is not p or v != p._version for a, v, (_, _, p) in zip(fast["params"], fast["versions"], tensors)):
                     fast = self._fast = None
         if fast is not None:
             args = plan.args
@@ -370,6 +373,10 @@ class VeLO_CUDA(Optimizer):
             fl["exp_mult"][i], fl["step_mult"][i] = group["exp_mult"], group["step_mult"]
             grp[i] = gi
         if fast is None:
+            # anything that sends the step down this path (first step, a loaded checkpoint, a replaced
+            # state tensor or parameter, a parameter written in place) may have changed what the LSTM's
+            # input sums are taken over: the library takes them from the tensors again
+            plan.invalidate_statistics()
             args = plan.args
             for k, v in cols.items():
                 args[k] = v
@@ -377,13 +384,12 @@ class VeLO_CUDA(Optimizer):
                 args[k] = v
             args["group"] = grp
             if not keep:
-                # one (state, key, tensor) per parameter, its first state tensor: replacing a parameter's
-                # state replaces that one too, and a walk over every tensor costs milliseconds with
-                # thousands of parameters
-                alive = [(self.state[p],) + next(((k, t) for k, t in self.state[p].items() if torch.is_tensor(t)), (None, None))
-                         for _, _, p in tensors]
+                # the two state tensors whose sums are carried from step to step, per parameter (a walk over
+                # every state tensor costs milliseconds with thousands of parameters; replacing a parameter's
+                # whole state replaces these too)
+                alive = [(self.state[p], self.state[p]["mom"], self.state[p]["rms"]) for _, _, p in tensors]
                 self._fast = dict(key=self._plan_key, n_state=len(self.state), alive=alive,
-                                  params=[p for _, _, p in tensors],
+                                  params=[p for _, _, p in tensors], versions=[p._version for _, _, p in tensors],
                                   gidx=np.asarray(grp, dtype=np.int64))
 
         h, c = self.lstm_hidden_state
@@ -403,6 +409,14 @@ class VeLO_CUDA(Optimizer):
                            torch.cuda.current_stream(self.device).cuda_stream, args=table)
         del keep, loss_dev
         return
+
+    def invalidate_statistics(self):
+        """Call after writing parameters or ``mom`` / ``rms`` state tensors in a way the optimizer cannot see
+        (through ``.data`` or a custom kernel): the next step then reads every tensor for the LSTM's input
+        statistics, as the reference does on every step, instead of using the sums the previous step left."""
+        self._fast = None
+        if self._plan is not None:
+            self._plan.invalidate_statistics()
 
     def _decays_struct(self):
         g0 = self.param_groups[0]

@@ -176,8 +176,12 @@ def test_velo_replaced_state_tensor_is_picked_up():
                             v.fill_(float("nan"))
         return ps
 
+    # Not bit for bit: the step after the swap takes the LSTM's input sums from the tensors again (fp32
+    # partial sums around the tensors' first elements), the undisturbed run from what its previous step
+    # carried over (fp64 around the first elements of a step earlier); both are the same sums up to rounding.
     for x, y in zip(run(False), run(True)):
-        assert torch.equal(x, y)
+        assert torch.isfinite(y).all()
+        assert max_err(y, x, REL, ABS) <= 1.0
 
 
 def test_velo_variance_features_where_the_spread_is_tiny():

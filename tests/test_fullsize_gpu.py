@@ -222,6 +222,50 @@ def test_adafac_llama_embedding_and_block():
     print("adafac embedding + block worst err/tol", worst)
 
 
+def test_adafac_whole_llama_set():
+    """All of cfg4: the 200 tensors of Llama-1.1B (1 100 046 336 elements, both 32000x2048 embeddings,
+    22 blocks) through one plan, bf16-rounded gradients, two steps, every tensor and every state against
+    the oracle in fp64 on the device.  What the one-block cases above cannot show: launch tables and
+    workspace offsets of the whole set (more than 2^31 bytes of tensors behind one argument table)."""
+    from oracle import pylo_oracle as O
+    from pylo_amd import AdafacLO_CUDA
+    from pylo_amd.models import MetaMLP
+
+    torch.manual_seed(9)
+    net = MetaMLP(39, 32, 1)
+    shapes = [(32000, 2048)]
+    for _ in range(22):
+        shapes += [(2048,), (2048, 2048), (2048, 256), (2048, 256), (2048, 2048), (2048,),
+                   (2048, 5632), (2048, 5632), (5632, 2048)]
+    shapes += [(32000, 2048)]
+    assert len(shapes) == 200 and sum(torch.Size(s).numel() for s in shapes) == 1100046336
+    gen = torch.Generator(device="cuda").manual_seed(13)
+    init = [torch.randn(s, generator=gen, device="cuda") * 0.02 for s in shapes]
+    ref = [v.double() for v in init]
+    gpu = [torch.nn.Parameter(v) for v in init]
+    orc = O.AdafacOracle(ref, net.state_dict(), lr=1.0, device="cuda").double_()
+    opt = AdafacLO_CUDA(gpu, lr=1.0, network=copy.deepcopy(net))
+    worst = 0.0
+    for t in range(2):
+        grads = [(torch.randn(s, generator=gen, device="cuda") * 1e-3).bfloat16().float() for s in shapes]
+        for p, g in zip(gpu, grads):
+            p.grad = g
+        orc.step([g.double() for g in grads])
+        opt.step()
+        torch.cuda.synchronize()
+        del grads
+        for i, p in enumerate(gpu):
+            st, so = opt.state[p], orc.state[i]
+            for tag, got, want in [("param", p, ref[i]), ("exp_avg", st["exp_avg"], so["exp_avg"]),
+                                   ("exp_avg_sq", st["exp_avg_sq"], so["exp_avg_sq"]),
+                                   ("r", st["exp_avg_sq_r"], so["exp_avg_sq_r"]),
+                                   ("c", st["exp_avg_sq_c"], so["exp_avg_sq_c"])]:
+                e = max_err(got, want, REL, ABS)
+                worst = max(worst, e)
+                assert e <= 1.0, (t, i, shapes[i], tag, e)
+    print("adafac whole Llama-1.1B set worst err/tol", worst)
+
+
 def _ortho_step(p_new, p_old, lr, wd):
     """The orthogonalised, normalised step a parameter update implies: p_new = p_old - lr (s + wd p_old)."""
     return (p_old.double() - p_new.double()) / lr - wd * p_old.double()

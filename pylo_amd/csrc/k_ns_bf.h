@@ -1,0 +1,408 @@
+// Newton-Schulz products at fp32 accuracy on the bf16 matrix pipe.
+//
+// An fp32 number is the exact sum of three bf16 numbers, x = h + m + l (h = bf16(x), m = bf16(x - h),
+// l = x - h - m: 8 + 8 + 8 significand bits).  A product of two such numbers is nine bf16 products; the
+// three smallest (m l, l m, l l) are below 2^-25 |x y| together, less than the rounding of an fp32
+// multiply-add, and are dropped.  The other six are exact in fp32 and are accumulated in fp32 by
+// v_mfma_f32_32x32x16_bf16, which does sixteen times the multiply-adds of v_mfma_f32_32x32x2_f32 per
+// instruction slot: six of them replace eight fp32 instructions' worth of work at 2.7 times the rate.
+//
+// Operands therefore live as *planes*: three bf16 matrices (h, m, l) with the reduction index contiguous,
+// written by the kernel that produces the matrix (never converted inside a product's main loop).
+// With X of m x n or n x m (m the smaller dim), Xs = X as [m][n] and Xl = X as [n][m]:
+//     A   = Xs Xs^T                      (reduction over n; symmetric, tiles on and above the diagonal)
+//     B'  = c2 A A + c1 A + c0 I         (reduction over m; symmetric)
+//     Xl' = Xl B'                        (reduction over m), written as planes of Xl' and of Xs' = Xl'^T,
+//                                         or as fp32 in the tensor's own layout after the last iteration
+// for wide and tall matrices alike (B' is symmetric, so (B' X)^T = X^T B').
+//
+// Tile job: 128 x 128 outputs by 256 threads = 2 x 2 waves of 64 x 64 = 2 x 2 accumulators of 32 x 32;
+// 16 reduction steps per stage, double buffered in LDS (48 KB), one 16-byte read per lane, plane and
+// 32-row block per stage.
+#pragma once
+
+#include "k_ns.h"
+
+namespace pylo {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned short bfbits;   // a bf16 in memory
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) u32x4 luint4;
+
+constexpr int kBfBK = 16;                     // reduction steps per stage
+constexpr int kBfOperandLds = kNsTile * 96;   // bytes of one operand's stage: 128 rows x 3 planes x 32 B
+constexpr int kBfStageLds = 2 * kBfOperandLds;   // 24 KB
+
+// Planes of one matrix with `rows` rows and a (padded) reduction length: stored in blocks of 16 reduction
+// steps, [k / 16][row][plane][k % 16], so that the 128 rows x 3 planes x 16 steps a tile job stages at a
+// time are 12 KB of consecutive memory (whole cache lines; with row-major planes a stage was 32 bytes
+// out of every row and each 128-byte line was fetched from L2 four times).
+struct BfPlanes {
+  const bfbits* base;
+  int rows;   // rows that exist; a tile's rows past them read as zero
+};
+
+// element offset of (row, k) in plane 0; planes 1 and 2 are 16 and 32 elements further
+__device__ __forceinline__ size_t bf_off(int rows, int row, int k) {
+  return ((size_t)(k >> 4) * rows + row) * 48 + (k & 15);
+}
+
+struct NsBfMat {
+  int tensor;
+  int R, C, m, n, tall;      // X is R x C row-major; m = min, n = max; tall: R > C
+  int pad_m, pad_n;          // m and n rounded up to the 16 reduction steps of a stage (the padding holds zeros)
+  int n_slabs;
+  long long off_xs;          // elements (bfbits) into the plane workspace: planes of Xs (m rows, reduction n)
+  long long off_xl[2];       // planes of Xl (n rows, reduction m), two buffers (a product reads one and writes the other)
+  long long off_pa, off_pb;  // planes of A and B' (m rows, reduction m)
+  long long off_a;           // floats into the fp32 workspace: A (m x m)
+  long long off_part;        // floats: partial matrices of a split Gram product
+};
+
+__device__ __forceinline__ float bf_to_float(bfbits b) { return __uint_as_float((unsigned)b << 16); }
+
+// x = h + m + l
+__device__ __forceinline__ void bf_split(float x, bfbits& h, bfbits& m, bfbits& l) {
+  const __bf16 hb = (__bf16)x;
+  const float r1 = x - (float)hb;
+  const __bf16 mb = (__bf16)r1;
+  const float r2 = r1 - (float)mb;
+  const __bf16 lb = (__bf16)r2;
+  h = __builtin_bit_cast(bfbits, hb);
+  m = __builtin_bit_cast(bfbits, mb);
+  l = __builtin_bit_cast(bfbits, lb);
+}
+
+// A stage of one operand in LDS: [row][plane][half], 96 bytes a row, as in memory, except that the two
+// 16-byte halves are swapped for every other group of eight rows (rows 8 apart would share banks).
+__device__ __forceinline__ int bf_lds_piece(int row, int plane, int half) {
+  return row * 96 + plane * 32 + 16 * (half ^ ((row >> 3) & 1));
+}
+
+// One operand's stage from global memory into registers: the 768 pieces of 16 bytes are consecutive in
+// memory; thread t takes pieces t, t + 256, t + 512.
+__device__ __forceinline__ void bf_load_stage(const BfPlanes& P, int row0, int k, u32x4 (&reg)[3]) {
+  const bfbits* p = P.base + ((size_t)(k >> 4) * P.rows + row0) * 48;
+#pragma unroll
+  for (int j = 0; j < 3; ++j) {
+    const int g = threadIdx.x + 256 * j;
+    reg[j] = row0 + g / 6 < P.rows ? *(const u32x4*)(p + (size_t)g * 8) : u32x4{0u, 0u, 0u, 0u};
+  }
+}
+
+__device__ __forceinline__ void bf_store_stage(char __attribute__((address_space(3)))* lds, const u32x4 (&reg)[3]) {
+#pragma unroll
+  for (int j = 0; j < 3; ++j) {
+    const int g = threadIdx.x + 256 * j, row = g / 6, rem = g - 6 * row;
+    *(luint4*)(lds + bf_lds_piece(row, rem >> 1, rem & 1)) = reg[j];
+  }
+}
+
+// acc[hi][hj] += (rows i0.. of P1) x (rows j0.. of P2)^T over the reduction range [k0, k1) (multiples of 16)
+__device__ __forceinline__ void bf_tile_product(const BfPlanes& P1, int i0, const BfPlanes& P2, int j0, int k0, int k1,
+                                                char __attribute__((address_space(3)))* lds, v16f (&acc)[2][2]) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;
+  const int kg = lane >> 5, lo = lane & 31;
+  u32x4 ra[3], rb[3];
+  bf_load_stage(P1, i0, k0, ra);
+  bf_load_stage(P2, j0, k0, rb);
+  bf_store_stage(lds, ra);
+  bf_store_stage(lds + kBfOperandLds, rb);
+  __syncthreads();
+  int cur = 0;
+  const int oa0 = bf_lds_piece(wi + lo, 0, kg), oa1 = bf_lds_piece(wi + 32 + lo, 0, kg);
+  const int ob0 = kBfOperandLds + bf_lds_piece(wj + lo, 0, kg), ob1 = kBfOperandLds + bf_lds_piece(wj + 32 + lo, 0, kg);
+  for (int k = k0; k < k1; k += kBfBK) {
+    const bool more = k + kBfBK < k1;
+    if (more) {
+      bf_load_stage(P1, i0, k + kBfBK, ra);
+      bf_load_stage(P2, j0, k + kBfBK, rb);
+    }
+    bf16x8 a[2][3], b[2][3];
+#pragma unroll
+    for (int q = 0; q < 3; ++q) {
+      a[0][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + q * 32 + oa0));
+      a[1][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + q * 32 + oa1));
+      b[0][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + q * 32 + ob0));
+      b[1][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + q * 32 + ob1));
+    }
+    // smallest terms first: l h, h l, m m, m h, h m, h h
+#pragma unroll
+    for (int term = 0; term < 6; ++term) {
+      constexpr int pa[6] = {2, 0, 1, 1, 0, 0}, pb[6] = {0, 2, 1, 0, 1, 0};
+#pragma unroll
+      for (int hi = 0; hi < 2; ++hi)
+#pragma unroll
+        for (int hj = 0; hj < 2; ++hj)
+          acc[hi][hj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[hi][pa[term]], b[hj][pb[term]], acc[hi][hj], 0, 0, 0);
+    }
+    if (more) {
+      bf_store_stage(lds + (kBfStageLds - cur), ra);
+      bf_store_stage(lds + (kBfStageLds - cur) + kBfOperandLds, rb);
+    }
+    __syncthreads();
+    cur = kBfStageLds - cur;
+  }
+}
+
+// Four values at consecutive reduction indices k .. k + 3 (k a multiple of 4) of one row: one 8-byte store per plane.
+__device__ __forceinline__ void bf_store4(bfbits* base, int rows, int row, int k, const float (&v)[4]) {
+  bfbits h[4], m[4], l[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) bf_split(v[r], h[r], m[r], l[r]);
+  typedef unsigned long long u64;
+  bfbits* p = base + bf_off(rows, row, k);
+  *(u64*)p = (u64)h[0] | (u64)h[1] << 16 | (u64)h[2] << 32 | (u64)h[3] << 48;
+  *(u64*)(p + 16) = (u64)m[0] | (u64)m[1] << 16 | (u64)m[2] << 32 | (u64)m[3] << 48;
+  *(u64*)(p + 32) = (u64)l[0] | (u64)l[1] << 16 | (u64)l[2] << 32 | (u64)l[3] << 48;
+}
+
+__device__ __forceinline__ void bf_store1(bfbits* base, int rows, int row, int k, float v) {
+  bfbits h, m, l;
+  bf_split(v, h, m, l);
+  bfbits* p = base + bf_off(rows, row, k);
+  p[0] = h;
+  p[16] = m;
+  p[32] = l;
+}
+
+// The block's 128 x 128 values (accumulator layout) into planes whose reduction index is the tile's column
+// index.  Four passes of 16 rows per wave: every lane splits its values and drops the halves into the
+// wave's own LDS patch ([row][plane][64 columns], 2 bytes each), then the wave reads the patch back as
+// 16-byte pieces in the order the planes have in memory ([16 columns][row][plane][half]) and stores them.
+constexpr int kBfPatchPlane = 144;                 // bytes: 64 columns x 2 + 16 (bank spread)
+constexpr int kBfPatchRow = 3 * kBfPatchPlane;
+constexpr int kBfPatchWave = 16 * kBfPatchRow;     // 6912 bytes per wave
+
+__device__ __forceinline__ void bf_store_direct(char __attribute__((address_space(3)))* lds, const v16f (&acc)[2][2],
+                                                bfbits* __restrict__ D, int rows_total, int i0, int j0, int n_rows,
+                                                int n_cols) {
+  typedef __attribute__((address_space(3))) bfbits lbf;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  char __attribute__((address_space(3)))* patch = lds + wave * kBfPatchWave;
+  const int wi = i0 + (wave >> 1) * 64, wj = j0 + (wave & 1) * 64;   // origin of the wave's values
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass) {
+    const int hi = pass >> 1, half = pass & 1;   // rows 32 hi + 16 half .. + 15 of the wave's 64
+    __syncthreads();   // the patch is free (first pass: every wave has left the product's last stage)
+#pragma unroll
+    for (int hj = 0; hj < 2; ++hj)
+#pragma unroll
+      for (int r8 = 0; r8 < 8; ++r8) {
+        const int r = 8 * half + r8;
+        const int row_l = 8 * (r8 >> 2) + 4 * (lane >> 5) + (r8 & 3), col_l = 32 * hj + (lane & 31);
+        bfbits h, m, l;
+        bf_split(acc[hi][hj][r], h, m, l);
+        lbf* q = (lbf*)(patch + row_l * kBfPatchRow + col_l * 2);
+        q[0] = h;
+        q[kBfPatchPlane / 2] = m;
+        q[kBfPatchPlane] = l;
+      }
+    __syncthreads();
+    const int row_w0 = wi + 32 * hi + 16 * half;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {          // 16 columns = one block of the planes' layout
+      const int col = wj + 16 * c;
+      if (col >= n_cols) continue;
+      bfbits* dst = D + bf_off(rows_total, row_w0, col);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {        // 96 pieces: [row][plane][half]
+        const int pc = lane + 64 * j;
+        if (pc >= 96) continue;
+        const int row_l = pc / 6, rem = pc - 6 * row_l, plane = rem >> 1, hf = rem & 1;
+        if (row_w0 + row_l >= n_rows) continue;
+        const u32x4 w = *(const luint4*)(patch + row_l * kBfPatchRow + plane * kBfPatchPlane + (16 * c + 8 * hf) * 2);
+        *(u32x4*)(dst + (size_t)pc * 8) = w;
+      }
+    }
+  }
+}
+
+// One launch = one product of one iteration, for every tensor (see the head of this file).
+//   kNsGram    A = Xs Xs^T as fp32 and planes, both halves; a slab of a split product: fp32 partial tile only
+//   kNsPoly    B' = c2 A A + c1 A + c0 I as planes, both halves
+//   kNsUpdate  Xl' = Xl B': planes of Xl' (buffer 1 - par) and Xs', or fp32 X in place of the raw step (`last`)
+template <int OP>
+__global__ __launch_bounds__(256) void k_ns_bf_gemm(const NsBfMat* __restrict__ mats, const NsItem* __restrict__ items,
+                                                    const PyloTensorArgs* __restrict__ dyn, float* __restrict__ ws,
+                                                    bfbits* __restrict__ pw, int par, int last, float c0, float c1,
+                                                    float c2) {
+  __shared__ __attribute__((aligned(16))) char lds_[2 * kBfStageLds];
+  char __attribute__((address_space(3)))* lds = (char __attribute__((address_space(3)))*)lds_;
+  const NsItem it = items[blockIdx.x];
+  if (it.mat < 0) return;   // a filler job
+  const NsBfMat mt = mats[it.mat];
+  const PyloTensorArgs a = dyn[mt.tensor];
+  if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
+  const int m = mt.m, n = mt.n;
+  v16f acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  const int i0 = it.tm * kNsTile, j0 = it.tn * kNsTile;
+  if (OP == kNsGram) {
+    const BfPlanes X{pw + mt.off_xs, m};
+    bf_tile_product(X, i0, X, j0, it.k0, it.k1, lds, acc);
+  } else if (OP == kNsPoly) {
+    const BfPlanes A{pw + mt.off_pa, m};
+    bf_tile_product(A, i0, A, j0, it.k0, it.k1, lds, acc);
+  } else {
+    const BfPlanes X{pw + mt.off_xl[par], n};
+    const BfPlanes B{pw + mt.off_pb, m};
+    bf_tile_product(X, i0, B, j0, it.k0, it.k1, lds, acc);
+  }
+  float* A32 = ws + mt.off_a;
+  const int n_i = OP == kNsUpdate ? n : m;   // rows of the output; its columns are always m
+  const bool partial = OP == kNsGram && it.slab >= 0;
+  const bool mirror = OP != kNsUpdate && !partial && it.tm != it.tn;
+  // what the registers can store well: fp32 outputs, and the planes in which four consecutive rows of a
+  // lane are four consecutive reduction indices (the mirrored tile, Xs')
+#pragma unroll
+  for (int hi = 0; hi < 2; ++hi)
+#pragma unroll
+    for (int hj = 0; hj < 2; ++hj) {
+      const int col = j0 + ns_acc_col(hj);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = i0 + ns_acc_row(hi, 4 * q);   // rows row .. row + 3
+        if (col >= m || row >= n_i) continue;
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float x = acc[hi][hj][4 * q + r];
+          if (OP == kNsPoly) {
+            const float aij = row + r < m ? A32[(size_t)(row + r) * m + col] : 0.0f;
+            x = c2 * x + c1 * aij + ((row + r) == col ? c0 : 0.0f);
+            acc[hi][hj][4 * q + r] = x;
+          }
+          v[r] = x;
+        }
+        if (OP == kNsGram) {
+          float* out = partial ? ws + mt.off_part + (size_t)it.slab * m * m : A32;
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (row + r < m) out[(size_t)(row + r) * m + col] = v[r];
+          if (mirror) *(gv4f*)(out + (size_t)col * m + row) = v4f{v[0], v[1], v[2], v[3]};
+        }
+        if (OP == kNsGram || OP == kNsPoly) {
+          if (mirror) bf_store4(pw + (OP == kNsGram ? mt.off_pa : mt.off_pb), m, col, row, v);
+        } else if (!last) {
+          bf_store4(pw + mt.off_xs, m, col, row, v);   // values past n are zeros, into the padding
+        } else if (mt.tall) {   // X = Xl, n x m
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (row + r < n) a.step_out[(size_t)(row + r) * m + col] = v[r];
+        } else {                // X = Xs, m x n: four consecutive columns of row `col` (n is a multiple of 4)
+          *(gv4f*)(a.step_out + (size_t)col * n + row) = v4f{v[0], v[1], v[2], v[3]};
+        }
+      }
+    }
+  // the planes in which a lane's column is the reduction index (A, B', Xl'): through LDS, 16 rows of each
+  // wave's 64 x 64 values at a time, so that memory sees 16-byte pieces in the planes' own order
+  if (partial || (OP == kNsUpdate && last)) return;
+  bfbits* D = pw + (OP == kNsGram ? mt.off_pa : OP == kNsPoly ? mt.off_pb : mt.off_xl[1 - par]);
+  bf_store_direct(lds, acc, D, n_i, i0, j0, n_i, m);
+}
+
+// A = sum over the slabs' partial matrices, in slab order, as fp32 and as planes (both halves).
+__global__ __launch_bounds__(256) void k_ns_bf_gram_reduce(const NsBfMat* __restrict__ mats, const int* __restrict__ split_mats,
+                                                           const PyloTensorArgs* __restrict__ dyn, float* __restrict__ ws,
+                                                           bfbits* __restrict__ pw) {
+  const NsBfMat mt = mats[split_mats[blockIdx.y]];
+  const PyloTensorArgs a = dyn[mt.tensor];
+  if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
+  const int m = mt.m;
+  const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (long long)m * m) return;
+  const int i = (int)(e / m), j = (int)(e - (long long)i * m);
+  if (i / kNsTile > j / kNsTile) return;
+  const size_t mm = (size_t)m * m;
+  const float* p = ws + mt.off_part + (size_t)i * m + j;
+  float s = 0.0f;
+  for (int q0 = 0; q0 < mt.n_slabs; q0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) v[q] = q0 + q < mt.n_slabs ? *(const gfloat*)(p + (size_t)(q0 + q) * mm) : 0.0f;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) s += v[q];
+  }
+  float* A = ws + mt.off_a;
+  bfbits* P = pw + mt.off_pa;
+  A[(size_t)i * m + j] = s;
+  bf_store1(P, m, i, j, s);
+  if (i / kNsTile != j / kNsTile) {
+    A[(size_t)j * m + i] = s;
+    bf_store1(P, m, j, i, s);
+  }
+}
+
+// X0 = raw * s (s = 1 / (||raw|| + eps), scale[mat]) as planes in both layouts.  One block = one 64 x 64
+// tile of the raw step (R x C): the planes in which the tensor's rows stay rows are written straight from
+// the loaded values, the transposed planes through LDS.
+struct NsTileItem { int mat, tr, tc; };
+
+__global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__ mats, const NsTileItem* __restrict__ items,
+                                                     const PyloTensorArgs* __restrict__ dyn, const float* __restrict__ scale,
+                                                     bfbits* __restrict__ pw) {
+  __shared__ bfbits tile[3][64][66];
+  const NsTileItem it = items[blockIdx.x];
+  const NsBfMat mt = mats[it.mat];
+  const PyloTensorArgs a = dyn[mt.tensor];
+  if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
+  const float s = scale[it.mat];
+  const int R = mt.R, C = mt.C;
+  // direct planes: the tensor's rows are the planes' rows; transposed planes: its columns are
+  bfbits* direct = pw + (mt.tall ? mt.off_xl[0] : mt.off_xs);
+  bfbits* transp = pw + (mt.tall ? mt.off_xs : mt.off_xl[0]);
+  const int r0 = it.tr * 64, c0 = it.tc * 64;
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass) {
+    const int lr = pass * 16 + (t >> 4), lc = 4 * (t & 15);
+    const int r = r0 + lr, c = c0 + lc;
+    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const bool in = r < R && c < C;   // C is a multiple of 4
+    if (in) {
+      const v4f x = *(const gv4f*)(a.step_out + (size_t)r * C + c);
+      v[0] = x.x * s; v[1] = x.y * s; v[2] = x.z * s; v[3] = x.w * s;
+    }
+    bfbits h[4], m[4], l[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      bf_split(v[q], h[q], m[q], l[q]);
+      tile[0][lr][lc + q] = h[q];
+      tile[1][lr][lc + q] = m[q];
+      tile[2][lr][lc + q] = l[q];
+    }
+    if (in) {
+      typedef unsigned long long u64;
+      bfbits* p = direct + bf_off(R, r, c);
+      *(u64*)p = (u64)h[0] | (u64)h[1] << 16 | (u64)h[2] << 32 | (u64)h[3] << 48;
+      *(u64*)(p + 16) = (u64)m[0] | (u64)m[1] << 16 | (u64)m[2] << 32 | (u64)m[3] << 48;
+      *(u64*)(p + 32) = (u64)l[0] | (u64)l[1] << 16 | (u64)l[2] << 32 | (u64)l[3] << 48;
+    }
+  }
+  __syncthreads();
+  // transposed: thread takes column lc2 and four consecutive rows (rows past R were stored as zeros: padding)
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass) {
+    const int lc2 = pass * 16 + (t >> 4), lr2 = 4 * (t & 15);
+    const int c = c0 + lc2, r = r0 + lr2;
+    if (c >= C || r >= R) continue;
+    typedef unsigned long long u64;
+    bfbits* p = transp + bf_off(C, c, r);
+#pragma unroll
+    for (int q = 0; q < 3; ++q) {
+      const u64 w = (u64)tile[q][lr2][lc2] | (u64)tile[q][lr2 + 1][lc2] << 16 | (u64)tile[q][lr2 + 2][lc2] << 32 |
+                    (u64)tile[q][lr2 + 3][lc2] << 48;
+      *(u64*)(p + 16 * q) = w;
+    }
+  }
+}
+
+}  // namespace pylo

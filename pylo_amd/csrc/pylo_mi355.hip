@@ -30,6 +30,7 @@
 #include "k_velo.h"
 #include "k_celo2_slices.h"
 #include "k_ns.h"
+#include "k_ns_bf.h"
 #include "pylo_common.h"
 
 // =============================================================================================
@@ -81,6 +82,12 @@ struct Layout {
   std::vector<long long> ns_xalt;     // per tensor: offset of its second X buffer, -1 without one
   std::vector<int> ns_of_tensor;      // per tensor: index into ns_mats, -1
   int ns_max_m = 0;
+  // Newton-Schulz on the bf16 matrix pipe (three-way split operands): tables of their own
+  bool ns_bf = false;
+  std::vector<NsBfMat> nsb_mats;
+  std::vector<NsTileItem> nsb_split_items;
+  size_t off_nsb_mats = 0, off_nsb_split_items = 0, off_ns_pw = 0;
+  long long nsb_plane_elems = 0;
   size_t off_ns_mats = 0, off_ns_gram = 0, off_ns_poly = 0, off_ns_upd = 0, off_ns_split = 0, off_ns_xalt = 0,
          off_ns_scale = 0, off_ns_ws = 0;
   std::vector<TDesc> descs;
@@ -187,6 +194,47 @@ void build_elem_items(Layout& L, int T, int kind) {
   }
 }
 
+// PYLO_MI355_NS_F32=1 keeps the Newton-Schulz products on the fp32 matrix instructions (k_ns.h) instead of
+// the split-bf16 ones (k_ns_bf.h); read at plan creation.
+bool env_ns_xcd() {
+  const char* e = getenv("PYLO_MI355_NS_XCD");
+  return !(e && e[0] == '0');
+}
+
+bool env_ns_bf() {
+  const char* e = getenv("PYLO_MI355_NS_F32");
+  return !(e && e[0] == '1');
+}
+
+// Workgroups go to the eight XCDs in turn (block b runs on XCD b % 8) and every XCD has an L2 of its own:
+// tile jobs that read the same operands should share an XCD.  `units` are runs of jobs that belong together
+// (count, work per job); the run sequence is cut into eight stretches of about equal work, stretch x becomes
+// the jobs 8 i + x.  Stretches are filled up with jobs that do nothing (mat = -1).
+constexpr int kXcds = 8;
+void xcd_interleave(std::vector<NsItem>& items, const std::vector<std::pair<int, long long>>& units) {
+  long long total = 0;
+  for (const auto& u : units) total += u.first * u.second;
+  std::vector<std::vector<NsItem>> lane(kXcds);
+  long long done = 0;
+  size_t pos = 0;
+  int x = 0;
+  for (const auto& u : units) {
+    // a unit goes to the stretch in which its middle falls
+    const long long mid = done + u.first * u.second / 2;
+    x = std::max(x, (int)std::min<long long>(kXcds - 1, total > 0 ? mid * kXcds / total : 0));
+    for (int i = 0; i < u.first; ++i) lane[x].push_back(items[pos + i]);
+    pos += u.first;
+    done += u.first * u.second;
+  }
+  size_t longest = 0;
+  for (const auto& l : lane) longest = std::max(longest, l.size());
+  std::vector<NsItem> out;
+  out.reserve(longest * kXcds);
+  for (size_t i = 0; i < longest; ++i)
+    for (int q = 0; q < kXcds; ++q) out.push_back(i < lane[q].size() ? lane[q][i] : NsItem{-1, 0, 0, 0, 0, -1});
+  items.swap(out);
+}
+
 // Newton-Schulz tables: every 2-D MLP tensor whose rows (C) and whose smaller dim (the rows of A and B')
 // are multiples of 4: the kernels load 16 bytes at a time along the contiguous dim of X, A and B'.  The
 // number of rows of a tall matrix is free (50257 x 768).  `ws_floats` returns the floats of workspace behind off_ns_ws.
@@ -229,6 +277,69 @@ void build_ns_tables(Layout& L, int T, long long& ws_floats) {
       for (int tn = 0; tn < nj; ++tn) L.ns_upd.push_back(NsItem{q, tm, tn, 0, mt.m, -1});
     if (mt.n_slabs > 1) L.ns_split.push_back(q);
     L.ns_mats.push_back(mt);
+  }
+  if (L.ns_bf) {
+    // same matrices, operands as bf16 planes; the item tables are rebuilt for the uniform (n x m) orientation
+    L.ns_gram.clear(); L.ns_poly.clear(); L.ns_upd.clear();
+    ws_floats = 0;
+    long long pw = 0;
+    auto take_p = [&](long long n) { const long long o = pw; pw += (n + 63) / 64 * 64; return o; };
+    auto up16 = [](int x) { return (x + kBfBK - 1) / kBfBK * kBfBK; };
+    // job runs that read the same operands: per matrix (slab), and finer, per row of tiles, for sets of few matrices
+    std::vector<std::pair<int, long long>> gram_units, poly_units, upd_units, gram_rows, poly_rows;
+    for (size_t q = 0; q < L.ns_mats.size(); ++q) {
+      const NsMat& f = L.ns_mats[q];
+      NsBfMat b{};
+      b.tensor = f.tensor; b.R = f.R; b.C = f.C; b.m = f.m; b.n = std::max(f.R, f.C); b.tall = f.tall;
+      b.pad_m = up16(b.m);
+      b.pad_n = up16(b.n);
+      b.n_slabs = f.n_slabs;
+      b.off_xs = take_p(3ll * b.m * b.pad_n);
+      b.off_xl[0] = take_p(3ll * b.n * b.pad_m);
+      b.off_xl[1] = take_p(3ll * b.n * b.pad_m);
+      b.off_pa = take_p(3ll * b.m * b.pad_m);
+      b.off_pb = take_p(3ll * b.m * b.pad_m);
+      b.off_a = take((long long)b.m * b.m);
+      b.off_part = b.n_slabs > 1 ? take((long long)b.n_slabs * b.m * b.m) : 0;
+      L.ns_mats[q].off_a = b.off_a;   // the fp32 tables stay consistent for k_ns_scale (tensor index only)
+      const int nt = (b.m + kNsTile - 1) / kNsTile, n_upper = nt * (nt + 1) / 2;
+      // Gram: the tiles of one matrix (of one slab of it) read the same rows of Xs; Poly: the same A
+      for (int sl = 0; sl < b.n_slabs; ++sl) {
+        const int k0 = b.n_slabs > 1 ? sl * kNsSlabK : 0;
+        const int k1 = b.n_slabs > 1 ? up16(std::min(b.n, (sl + 1) * kNsSlabK)) : up16(b.n);
+        for (int tm = 0; tm < nt; ++tm)
+          for (int tn = tm; tn < nt; ++tn) L.ns_gram.push_back(NsItem{(int)q, tm, tn, k0, k1, b.n_slabs > 1 ? sl : -1});
+        gram_units.push_back({n_upper, (long long)(k1 - k0)});
+        for (int tm = 0; tm < nt; ++tm) gram_rows.push_back({nt - tm, (long long)(k1 - k0)});
+      }
+      for (int tm = 0; tm < nt; ++tm)
+        for (int tn = tm; tn < nt; ++tn) L.ns_poly.push_back(NsItem{(int)q, tm, tn, 0, up16(b.m), -1});
+      poly_units.push_back({n_upper, (long long)up16(b.m)});
+      for (int tm = 0; tm < nt; ++tm) poly_rows.push_back({nt - tm, (long long)up16(b.m)});
+      // Update: the tiles of one row block read the same rows of Xl, all of them the same B'
+      const int ni = (b.n + kNsTile - 1) / kNsTile;
+      for (int tm = 0; tm < ni; ++tm) {
+        for (int tn = 0; tn < nt; ++tn) L.ns_upd.push_back(NsItem{(int)q, tm, tn, 0, up16(b.m), -1});
+        upd_units.push_back({nt, (long long)up16(b.m)});
+      }
+      for (int tr = 0; tr < (b.R + 63) / 64; ++tr)
+        for (int tc = 0; tc < (b.C + 63) / 64; ++tc) L.nsb_split_items.push_back(NsTileItem{(int)q, tr, tc});
+      L.nsb_mats.push_back(b);
+    }
+    L.nsb_plane_elems = pw;
+    std::fill(L.ns_xalt.begin(), L.ns_xalt.end(), -1);   // the result always replaces the raw step
+    if (env_ns_xcd()) {
+      // with fewer runs than a few per XCD the stretches would be uneven: take the finer runs, or leave the order
+      auto pick = [](std::vector<NsItem>& items, const std::vector<std::pair<int, long long>>& coarse,
+                     const std::vector<std::pair<int, long long>>& fine) {
+        if (coarse.size() >= 4 * kXcds) xcd_interleave(items, coarse);
+        else if (fine.size() >= 4 * kXcds) xcd_interleave(items, fine);
+      };
+      pick(L.ns_gram, gram_units, gram_rows);
+      pick(L.ns_poly, poly_units, poly_rows);
+      pick(L.ns_upd, upd_units, upd_units);
+    }
+    return;
   }
   // longest jobs first: the launch ends when its last block does
   auto longer = [](const NsItem& x, const NsItem& y) { return x.k1 - x.k0 > y.k1 - y.k0; };
@@ -459,6 +570,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_wmix = take(kind == PYLO_KIND_VELO ? sizeof(float) * 160 * (size_t)T : 0);
   if (kind == PYLO_KIND_CELO2) {
     long long ns_floats = 0;
+    L.ns_bf = env_ns_bf();
     build_ns_tables(L, T, ns_floats);
     L.off_ns_mats = take(sizeof(NsMat) * L.ns_mats.size());
     L.off_ns_gram = take(sizeof(NsItem) * L.ns_gram.size());
@@ -468,6 +580,9 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     L.off_ns_xalt = take(sizeof(long long) * (size_t)T);
     L.off_ns_scale = take(sizeof(float) * L.ns_mats.size());
     L.off_ns_ws = take(sizeof(float) * (size_t)ns_floats);
+    L.off_nsb_mats = take(sizeof(NsBfMat) * L.nsb_mats.size());
+    L.off_nsb_split_items = take(sizeof(NsTileItem) * L.nsb_split_items.size());
+    L.off_ns_pw = take(sizeof(bfbits) * (size_t)L.nsb_plane_elems);
   }
   L.total = off;
   return 0;
@@ -557,6 +672,11 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_ns_upd, L.ns_upd.data(), sizeof(NsItem) * L.ns_upd.size());
   if (e == hipSuccess) e = up(L.off_ns_split, L.ns_split.data(), sizeof(int) * L.ns_split.size());
   if (e == hipSuccess && kind == PYLO_KIND_CELO2) e = up(L.off_ns_xalt, L.ns_xalt.data(), sizeof(long long) * L.ns_xalt.size());
+  if (e == hipSuccess) e = up(L.off_nsb_mats, L.nsb_mats.data(), sizeof(NsBfMat) * L.nsb_mats.size());
+  if (e == hipSuccess) e = up(L.off_nsb_split_items, L.nsb_split_items.data(), sizeof(NsTileItem) * L.nsb_split_items.size());
+  // the padding of the operand planes is read by the products and written by nobody: zero, once
+  if (e == hipSuccess && L.nsb_plane_elems > 0)
+    e = hipMemsetAsync(P->ws + L.off_ns_pw, 0, sizeof(bfbits) * (size_t)L.nsb_plane_elems, s);
   if (e == hipSuccess) e = hipStreamSynchronize(s);
   for (int i = 0; i < kStageSlots && e == hipSuccess; ++i) {
     e = hipHostMalloc(reinterpret_cast<void**>(&P->stage[i]), (sizeof(PyloTensorArgs) * n_tensors + 15) / 16 * 16,
@@ -974,6 +1094,25 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
     hipLaunchKernelGGL(k_celo2_sumsq, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_part,
                        (const long long*)nullptr, (const float*)nullptr);
     hipLaunchKernelGGL(k_ns_scale, dim3(n_mats), dim3(256), 0, s, mats, n_mats, descs, fin_part, ns_eps, scale);
+    if (L.ns_bf) {
+      const NsBfMat* bmats = P->at<NsBfMat>(L.off_nsb_mats);
+      const NsTileItem* sitems = P->at<NsTileItem>(L.off_nsb_split_items);
+      bfbits* pw = P->at<bfbits>(L.off_ns_pw);
+      hipLaunchKernelGGL(k_ns_bf_split, dim3((unsigned)L.nsb_split_items.size()), dim3(256), 0, s, bmats, sitems, dyn,
+                         (const float*)scale, pw);
+      for (int it = 0; it < ns_iters; ++it) {
+        const int par = it & 1, last = it == ns_iters - 1;
+        hipLaunchKernelGGL(k_ns_bf_gemm<kNsGram>, dim3(n_gram), dim3(256), 0, s, bmats, gram, dyn, ns_ws, pw, par, last,
+                           coeffs[0], coeffs[1], coeffs[2]);
+        if (n_split > 0)
+          hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)L.ns_max_m * L.ns_max_m + 255) / 256, n_split), dim3(256),
+                             0, s, bmats, split, dyn, ns_ws, pw);
+        hipLaunchKernelGGL(k_ns_bf_gemm<kNsPoly>, dim3(n_poly), dim3(256), 0, s, bmats, poly, dyn, ns_ws, pw, par, last,
+                           coeffs[0], coeffs[1], coeffs[2]);
+        hipLaunchKernelGGL(k_ns_bf_gemm<kNsUpdate>, dim3(n_upd), dim3(256), 0, s, bmats, upd, dyn, ns_ws, pw, par, last,
+                           coeffs[0], coeffs[1], coeffs[2]);
+      }
+    } else
     for (int it = 0; it < ns_iters; ++it) {
       const int first = it == 0, par = it & 1;
       hipLaunchKernelGGL(k_ns_gemm<kNsGram>, dim3(n_gram), dim3(256), 0, s, mats, gram, dyn, ns_ws, scale, first, par,
@@ -986,7 +1125,8 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
       hipLaunchKernelGGL(k_ns_gemm<kNsUpdate>, dim3(n_upd), dim3(256), 0, s, mats, upd, dyn, ns_ws, scale, first, par,
                          coeffs[0], coeffs[1], coeffs[2]);
     }
-    if (ns_iters & 1) x_alt = P->at<long long>(L.off_ns_xalt);   // the last iteration wrote the second buffer
+    // fp32 kernels: an odd number of iterations leaves the result in the second buffer
+    if (!L.ns_bf && (ns_iters & 1)) x_alt = P->at<long long>(L.off_ns_xalt);
   }
   hipLaunchKernelGGL(k_celo2_sumsq, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_part, x_alt,
                      (const float*)ns_ws);

@@ -72,14 +72,23 @@ def test_library_kernels_take_these_shapes():
     [(130, 6), (6, 130), (9, 16), (64, 64)],                             # library and torch side by side
     [(300, 260), (300, 260), (300, 260), (64,)],                         # a bucket of equal shapes
 ])
-def test_library_newton_schulz_matches_oracle(shapes):
+@pytest.mark.parametrize("pipe", ["bf16x3", "fp32"])
+def test_library_newton_schulz_matches_oracle(shapes, pipe, monkeypatch):
+    """Both sets of product kernels: the default (operands split into three bf16 planes, six bf16 matrix
+    products per fp32 product) and the fp32 matrix instructions (PYLO_MI355_NS_F32=1, read at plan creation)."""
+    if pipe == "fp32":
+        monkeypatch.setenv("PYLO_MI355_NS_F32", "1")
     _, worst = _run(shapes, steps=2, seed=len(shapes))
     print("orthogonalised step err / rms", worst)
 
 
 @pytest.mark.parametrize("iters", [0, 1, 2, 4])
-def test_iteration_counts_and_result_buffer(iters):
-    """An even number of iterations leaves the result in the raw-step buffer, an odd one in the workspace."""
+@pytest.mark.parametrize("pipe", ["bf16x3", "fp32"])
+def test_iteration_counts_and_result_buffer(iters, pipe, monkeypatch):
+    """fp32 kernels: an even number of iterations leaves the result in the raw-step buffer, an odd one in the
+    workspace; split-bf16 kernels: the last update writes fp32 over the raw step whatever the count."""
+    if pipe == "fp32":
+        monkeypatch.setenv("PYLO_MI355_NS_F32", "1")
     _run([(256, 384), (384, 256), (132, 260)], steps=2, ns_iters=iters)
 
 

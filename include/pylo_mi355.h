@@ -12,9 +12,11 @@
  * Conventions
  *   - every function returns 0 on success, non-zero on failure;
  *     pylo_mi355_last_error() then returns a thread-local message;
- *   - all device buffers are caller-owned fp32, contiguous, 16-byte aligned;
- *     nothing is allocated on the device by the library (the caller passes a
- *     workspace of pylo_mi355_plan_workspace_bytes() bytes, 256-byte aligned);
+ *   - all device buffers are caller-owned, contiguous, 16-byte aligned and fp32,
+ *     except `grad` and `param` of tensors whose PyloTensorShape carries a
+ *     PYLO_F_STORE_* tag; nothing is allocated on the device by the library
+ *     (the caller passes a workspace of pylo_mi355_plan_workspace_bytes()
+ *     bytes, 256-byte aligned);
  *   - `stream` is a hipStream_t (NULL = the null stream); calls only enqueue
  *     work and never synchronise the device;
  *   - a plan must not be used from two host threads, or on two streams, at once.
@@ -29,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PYLO_MI355_ABI_VERSION 5
+#define PYLO_MI355_ABI_VERSION 6
 #define PYLO_MAX_DIMS 8
 #define PYLO_MAX_GROUPS 8   /* parameter groups with their own step counter (VeLO) */
 
@@ -56,6 +58,22 @@ extern "C" {
                                  call; required on every tensor of a plan whose steps pass clip_norm > 0
                                  (CELO2 plans always take the norm over all their tensors) */
 
+/* Storage type of the tensor's `grad` and `param` buffers (bits 8-9 of PyloTensorShape.flags).  The reference's
+   kernels are instantiated for float, double and half (AT_DISPATCH_FLOATING_TYPES_AND_HALF,
+   celo2_kernel.cu:314,328, velo_kernel.cu:405,427, learned_optimizer.cu:338,364): they widen every value to
+   float on load (celo2_kernel.cu:70-75), compute in float and narrow on store (:280).  Here likewise: the
+   gradient and the parameter are widened exactly to fp32 when read, every accumulator (mom, rms, fac_*,
+   step_out) stays fp32 as the reference's classes keep them (ELO_CELO2_cuda.py:167-177), all arithmetic is
+   that of an fp32 tensor holding the widened values (fp64 values are rounded to fp32 first, as
+   static_cast<float> does), and the updated parameter is rounded to nearest-even into its storage type.
+   bf16 is an addition (the reference's dispatch has no bf16 case).  Mixed plans are fine: the tag is per
+   tensor. */
+#define PYLO_F_STORE_F32 0
+#define PYLO_F_STORE_F16 0x100
+#define PYLO_F_STORE_BF16 0x200
+#define PYLO_F_STORE_F64 0x300
+#define PYLO_F_STORE_MASK 0x300
+
 typedef struct PyloPlan PyloPlan; /* opaque, host memory owned by the library */
 
 typedef struct {
@@ -76,8 +94,9 @@ typedef struct {
 /* Per-tensor, per-step arguments.  Pointers are device pointers; the table itself is host
    memory and is copied by the call. */
 typedef struct {
-  const float* grad; /* NULL: the tensor is skipped this step (p.grad is None)               */
-  float* param;      /* (n)                                                                  */
+  const float* grad; /* NULL: the tensor is skipped this step (p.grad is None); elements of the
+                        tensor's storage type (PYLO_F_STORE_*), fp32 without a tag            */
+  float* param;      /* (n)     of the tensor's storage type                                  */
   float* mom;        /* (3, n)  momentum accumulators, decay axis leading                    */
   float* rms;        /* (n)     second-moment accumulator                                    */
   float* fac_r;      /* (3, n/size(dr)) row accumulator (mean of g^2 over the largest dim)   */
@@ -364,6 +383,38 @@ int pylo_mi355_velo_kernel_simple(const float* grad, float* param, const float* 
                                   const float* output_weights, const float* output_bias, float lr,
                                   float step_mult, float exp_mult, float epsilon, float weight_decay,
                                   const int64_t* shape, int ndim, int dc, int dr, int vector_like, void* stream);
+
+/* The three calls above for arrays of another element type: what the reference's
+   AT_DISPATCH_FLOATING_TYPES_AND_HALF over p.scalar_type() selects (celo2_kernel.cu:314,328,
+   learned_optimizer.cu:338,364, velo_kernel.cu:405,427).  `dtype` is one of PYLO_F_STORE_*; every array holds
+   elements of that type except `second_moment`, which is float as in the reference
+   (second_moment.data_ptr<float>(), celo2_kernel.cu:324).  Values are widened to float on load, the arithmetic is
+   float, results are rounded to nearest-even on store (celo2_kernel.cu:70-75,280).  PYLO_F_STORE_BF16 is an
+   addition: the reference's dispatch has no bfloat16 case. */
+int pylo_mi355_celo2_kernel_typed(int dtype, const void* g, const void* p, const void* m, const void* v,
+                                  const void* fac_r, const void* fac_c, const void* row_factor,
+                                  const void* col_factor, float* second_moment, const void* w_in, const void* b_in,
+                                  const void* w_h, const void* b_h, const void* w_out, const void* b_out,
+                                  void* step_out, float exp_mult, const int64_t* shape, int ndim, int dc, int dr,
+                                  int vector_like, void* stream);
+int pylo_mi355_learned_optimizer_kernel_typed(int dtype, const void* g, void* p, const void* m, const void* v,
+                                              const void* fac_r, const void* fac_c, const void* row_factor,
+                                              const void* col_factor, float* second_moment,
+                                              const void* input_weights, const void* input_bias,
+                                              const void* hidden_weights, const void* hidden_bias,
+                                              const void* output_weights, const void* output_bias, float lr,
+                                              float step_mult, float exp_mult, float epsilon, float step,
+                                              float weight_decay, const int64_t* shape, int ndim, int dc, int dr,
+                                              int vector_like, void* stream);
+int pylo_mi355_velo_kernel_simple_typed(int dtype, const void* grad, void* param, const void* momentum,
+                                        const void* rms, const void* row_factor, const void* col_factor,
+                                        const void* fac_vec_row, const void* fac_vec_col, float* second_moment,
+                                        const void* input_weights, const void* input_bias,
+                                        const void* hidden_weights, const void* hidden_bias,
+                                        const void* output_weights, const void* output_bias, float lr,
+                                        float step_mult, float exp_mult, float epsilon, float weight_decay,
+                                        const int64_t* shape, int ndim, int dc, int dr, int vector_like,
+                                        void* stream);
 
 #ifdef __cplusplus
 }

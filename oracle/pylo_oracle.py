@@ -17,11 +17,18 @@ state, ``torch.optim.AdamW`` for the 1-D branch, ``torch.nn.LSTMCell`` with
 permuted gates for the LSTM, fp64 brute force for Newton-Schulz and the feature
 list, ``numpy.argsort`` for ``factored_dims``.
 
-Parity unpinned: ``AdafacOracle(per_param_step=True)``.  That switch restates the CUDA class's
-per-parameter step counter (AdafacLO_cuda.py:304-305,400), and the CUDA class cannot run here, so
-no golden trajectory covers a parameter that sat steps out.  It only selects which step number
-feeds the time features; the time features themselves, and everything else in the class, are
-pinned by the golden trajectories of AdafacLO_naive and ELO_naive.
+``AdafacOracle(per_param_step=True)`` restates the CUDA class's per-parameter step counter
+(AdafacLO_cuda.py:304-305,400); the CUDA class cannot run here and the naive class counts per group, so
+no golden trajectory covers a parameter that sat steps out.  The switch is pinned by a property instead
+(tests/test_oracle_pins.py): AdafacLO tensors do not interact, so such a parameter must end bit-exactly
+where a single-parameter run fed only the steps it took part in ends.  Nothing here is unpinned.
+
+Parameters stored as float16 / bfloat16 / float64 need no code of their own: the contract is the float32
+step on the widened values with the result rounded into the storage type, so the tests feed these classes
+widened inputs and round.  (Of the reference's naive classes, ELO_CELO2_naive and CELO2_naive raise a dtype
+error on any parameter that is not float32 and all of them on float64; AdafacLO_naive, ELO_naive and
+VeLO_naive run on 16-bit parameters with float32 accumulators and a few operations, g*g among them, in the
+16-bit type.)
 
 Every function cites the reference lines it restates.
 """

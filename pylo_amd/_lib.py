@@ -20,6 +20,16 @@ F_ADAM = 1
 F_ADAM_INDEP = 2
 F_NAN_TO_NUM, F_WD_PRESTEP, F_GLOBAL_NORM = 4, 8, 16
 ARG_ORTHOGONALIZE = 1      # PyloTensorArgs.flags
+# storage type of a tensor's grad / param buffers (PYLO_F_STORE_*); accumulators and arithmetic stay fp32
+STORE_FLAG = {torch.float32: 0, torch.float16: 0x100, torch.bfloat16: 0x200, torch.float64: 0x300}
+
+
+def store_flag(p: torch.Tensor, who: str) -> int:
+    """The PYLO_F_STORE_* tag of a parameter; its gradient must have the same type (torch sees to that)."""
+    try:
+        return STORE_FLAG[p.dtype]
+    except KeyError:
+        raise TypeError(f"{who}: parameters must be float32, float16, bfloat16 or float64, got {p.dtype}") from None
 
 
 class TensorShape(C.Structure):
@@ -99,7 +109,7 @@ def load():
     lib.pylo_mi355_plan_invalidate_statistics.argtypes = [C.c_void_p]
     lib.pylo_mi355_plan_arg_table.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_void_p)]
     lib.pylo_mi355_plan_device_steps.argtypes = [C.c_void_p, C.POINTER(DeviceSteps)]
-    if lib.pylo_mi355_abi_version() != 5:
+    if lib.pylo_mi355_abi_version() != 6:
         raise RuntimeError("libpylo_mi355.so: ABI version mismatch, rebuild it")
     _lib = lib
     return lib

@@ -16,6 +16,8 @@ _SIGS = {
     "pylo_mi355_learned_optimizer_kernel": [_P] * 15 + [_F] * 6 + _TAIL,
     "pylo_mi355_velo_kernel_simple": [_P] * 15 + [_F] * 5 + _TAIL,
 }
+# the same calls with a leading element-type argument (what the reference's dispatch macro selects)
+_SIGS.update({k + "_typed": [C.c_int] + v for k, v in list(_SIGS.items())})
 _bound = set()
 
 
@@ -29,9 +31,10 @@ def entry(name: str):
     return fn
 
 
-def pointers(who: str, device: torch.device, **tensors) -> list:
-    """Device pointers of contiguous float32 tensors on `device`; an empty tensor gives a null pointer
-    (the reference passes nullptr for empty factor tensors, velo_kernel.cu:411-414)."""
+def pointers(who: str, device: torch.device, dtype: torch.dtype = torch.float32, **tensors) -> list:
+    """Device pointers of contiguous tensors of `dtype` on `device` (``second_moment`` is always float32, as
+    in the reference: celo2_kernel.cu:324); an empty tensor gives a null pointer (the reference passes nullptr
+    for empty factor tensors, velo_kernel.cu:411-414)."""
     out = []
     for name, t in tensors.items():
         if not torch.is_tensor(t):
@@ -41,8 +44,10 @@ def pointers(who: str, device: torch.device, **tensors) -> list:
             continue
         if not t.is_cuda or t.device != device:
             raise RuntimeError(f"{who}: {name} must live on {device}")
-        if t.dtype != torch.float32:
-            raise TypeError(f"{who}: {name} must be float32 (got {t.dtype})")
+        want = torch.float32 if name == "second_moment" else dtype
+        if t.dtype != want:
+            raise TypeError(f"{who}: {name} must be {want} (got {t.dtype}); every array has the parameter's "
+                            "element type, second_moment is float32")
         if not t.is_contiguous():
             raise RuntimeError(f"{who}: {name} must be contiguous")
         out.append(t.data_ptr())
@@ -82,6 +87,11 @@ def shape_args(p: torch.Tensor):
 
 
 def run(who: str, name: str, p: torch.Tensor, args: list) -> None:
+    """Dispatch on the parameter's element type like the reference's AT_DISPATCH_FLOATING_TYPES_AND_HALF
+    (celo2_kernel.cu:314): float32 takes the plain entry point, float16 / float64 (and bfloat16) the typed one."""
     with torch.cuda.device(p.device):
         stream = torch.cuda.current_stream(p.device).cuda_stream
-        _lib.check(entry(name)(*args, stream), who)
+        if p.dtype == torch.float32:
+            _lib.check(entry(name)(*args, stream), who)
+        else:
+            _lib.check(entry(name + "_typed")(_lib.store_flag(p, who), *args, stream), who)

@@ -13,7 +13,7 @@ def celo2_kernel(g, p, m, v, fac_r, fac_c, row_factor, col_factor, second_moment
                      row_factor=(row_factor, "row"), col_factor=(col_factor, "col"),
                      second_moment=(second_moment, "stat"), step_out=(step_out, "n")),
                 dict(w_in=(w_in, 240), b_in=(b_in, 8), w_h=(w_h, 64), b_h=(b_h, 8), w_out=(w_out, 24), b_out=(b_out, 3)))
-    ptrs = pointers(who, p.device, g=g, p=p, m=m, v=v, fac_r=fac_r, fac_c=fac_c, row_factor=row_factor,
+    ptrs = pointers(who, p.device, p.dtype, g=g, p=p, m=m, v=v, fac_r=fac_r, fac_c=fac_c, row_factor=row_factor,
                     col_factor=col_factor, second_moment=second_moment, w_in=w_in, b_in=b_in, w_h=w_h, b_h=b_h,
                     w_out=w_out, b_out=b_out, step_out=step_out)
     shape, ndim = shape_args(p)

@@ -16,7 +16,7 @@ def learned_optimizer_kernel(g, p, m, v, fac_r, fac_c, row_factor, col_factor, s
                 dict(input_weights=(input_weights, 32 * 39), input_bias=(input_bias, 32),
                      hidden_weights=(hidden_weights, 32 * 32), hidden_bias=(hidden_bias, 32),
                      output_weights=(output_weights, 64), output_bias=(output_bias, 2)))
-    ptrs = pointers(who, p.device, g=g, p=p, m=m, v=v, fac_r=fac_r, fac_c=fac_c, row_factor=row_factor,
+    ptrs = pointers(who, p.device, p.dtype, g=g, p=p, m=m, v=v, fac_r=fac_r, fac_c=fac_c, row_factor=row_factor,
                     col_factor=col_factor, second_moment=second_moment, input_weights=input_weights,
                     input_bias=input_bias, hidden_weights=hidden_weights, hidden_bias=hidden_bias,
                     output_weights=output_weights, output_bias=output_bias)

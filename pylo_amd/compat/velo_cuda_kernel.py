@@ -15,7 +15,7 @@ def velo_kernel_simple(grad, param, momentum, rms, row_factor, col_factor, fac_v
                      second_moment=(second_moment, "stat")),
                 dict(input_weights=(input_weights, 120), input_bias=(input_bias, 4), hidden_weights=(hidden_weights, 16),
                      hidden_bias=(hidden_bias, 4), output_weights=(output_weights, 12), output_bias=(output_bias, 3)))
-    ptrs = pointers(who, param.device, grad=grad, param=param, momentum=momentum, rms=rms, row_factor=row_factor,
+    ptrs = pointers(who, param.device, param.dtype, grad=grad, param=param, momentum=momentum, rms=rms, row_factor=row_factor,
                     col_factor=col_factor, fac_vec_row=fac_vec_row, fac_vec_col=fac_vec_col,
                     second_moment=second_moment, input_weights=input_weights, input_bias=input_bias,
                     hidden_weights=hidden_weights, hidden_bias=hidden_bias, output_weights=output_weights,

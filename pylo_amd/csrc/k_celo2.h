@@ -2,6 +2,7 @@
 #pragma once
 
 #include "pylo_common.h"
+#include "k_cast.h"
 
 #ifndef PYLO_STATS_UNROLL
 #define PYLO_STATS_UNROLL 2   // rows of the statistics walk whose loads are issued together
@@ -979,6 +980,14 @@ __global__ __launch_bounds__(kThreads) void k_celo2_update(const TDesc* __restri
   const float* x = fin_source(a, it.tensor, x_alt, ws) + base;
   float* p = a.param + base;
   const float sc = fin_scale[it.tensor], rm = a.step_mult, wd = a.weight_decay, nlr = -a.lr;
+  if (d.store != 0) {
+    // the parameter in its storage type (fp16, bf16, fp64): widened, updated in fp32, rounded to nearest-even
+    for (unsigned off = threadIdx.x; off < lim; off += kThreads) {
+      const float v = *(const gfloat*)(x + off), q = load_stored(a.param, base + off, d.store);
+      store_stored(a.param, base + off, d.store, fmaf(nlr, (v * sc) * rm + wd * q, q));
+    }
+    return;
+  }
   if (d.n % 4 == 0) {
 #pragma unroll
     for (int i = 0; i < kElemIters; ++i) {

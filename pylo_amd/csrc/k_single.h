@@ -7,6 +7,7 @@
 #pragma once
 
 #include "pylo_common.h"
+#include "k_cast.h"
 
 namespace pylo {
 
@@ -20,6 +21,9 @@ template <> struct Fam<kFamLo> { static constexpr int NSTAT = 28, NIN = 39, H = 
 // VeLO: 30 channels, 30 -> 4 -> 4 -> 3, (out, in)                                   (velo_kernel.cu:10-13)
 template <> struct Fam<kFamVelo> { static constexpr int NSTAT = 30, NIN = 30, H = 4, NOUT = 3; static constexpr bool in_major = false; };
 
+// Every array except `second_moment` holds elements of the call's element type (float unless the typed
+// entry points say otherwise; the reference instantiates its kernels for float, double and half and passes
+// all of them as scalar_t, celo2_kernel.cu:314-347): the members are typed float* and read through ld<ST>.
 struct SingleArgs {
   const float *g, *m, *v, *fac_r, *fac_c, *row_factor, *col_factor;
   float* p;              // read by every family; updated in place by the lo / velo families
@@ -56,25 +60,38 @@ __device__ __forceinline__ FacOfs fac_offsets(const SingleArgs& a, int idx) {
   return o;
 }
 
-template <int F>
+// Element i of an array of the call's element type ST (kStore*), widened to float as the reference's
+// static_cast<float> does (celo2_kernel.cu:70-75), and the narrowing store (celo2_kernel.cu:280).
+template <int ST>
+__device__ __forceinline__ float ld(const float* base, size_t i) {
+  if constexpr (ST == kStoreF32) return base[i];
+  else return load_stored(base, (long long)i, ST);
+}
+template <int ST>
+__device__ __forceinline__ void st(float* base, size_t i, float x) {
+  if constexpr (ST == kStoreF32) base[i] = x;
+  else store_stored(base, (long long)i, ST, x);
+}
+
+template <int F, int ST>
 __device__ __forceinline__ void single_features(const SingleArgs& a, int idx, float (&f)[Fam<F>::NSTAT]) {
   const FacOfs o = fac_offsets(a, idx);
-  const float g = a.g[idx], p = a.p[idx];
-  const float m0 = a.m[idx], m1 = a.m[idx + (size_t)a.n], m2 = a.m[idx + 2 * (size_t)a.n];
-  const float v = a.v[idx];
+  const float g = ld<ST>(a.g, idx), p = ld<ST>(a.p, idx);
+  const float m0 = ld<ST>(a.m, idx), m1 = ld<ST>(a.m, idx + (size_t)a.n), m2 = ld<ST>(a.m, idx + 2 * (size_t)a.n);
+  const float v = ld<ST>(a.v, idx);
   const bool vl = a.vector_like != 0;
-  const float rf0 = a.row_factor[o.r], rf1 = a.row_factor[o.r + (size_t)o.stride_r],
-              rf2 = a.row_factor[o.r + 2 * (size_t)o.stride_r];
-  const float cf0 = vl ? 1.0f : a.col_factor[o.c], cf1 = vl ? 1.0f : a.col_factor[o.c + (size_t)o.stride_c],
-              cf2 = vl ? 1.0f : a.col_factor[o.c + 2 * (size_t)o.stride_c];
+  const float rf0 = ld<ST>(a.row_factor, o.r), rf1 = ld<ST>(a.row_factor, o.r + (size_t)o.stride_r),
+              rf2 = ld<ST>(a.row_factor, o.r + 2 * (size_t)o.stride_r);
+  const float cf0 = vl ? 1.0f : ld<ST>(a.col_factor, o.c), cf1 = vl ? 1.0f : ld<ST>(a.col_factor, o.c + (size_t)o.stride_c),
+              cf2 = vl ? 1.0f : ld<ST>(a.col_factor, o.c + 2 * (size_t)o.stride_c);
   if constexpr (F == kFamLo) {
     // learned_optimizer.cu:34-98
     const float rs = rsq(v + a.epsilon);
     f[0] = g; f[1] = p; f[2] = m0; f[3] = m1; f[4] = m2; f[5] = v;
     f[6] = m0 * rs; f[7] = m1 * rs; f[8] = m2 * rs; f[9] = rs;
     f[10] = rf0 * cf0 * g; f[11] = rf1 * cf1 * g; f[12] = rf2 * cf2 * g;
-    const float r0 = a.fac_r[o.r], r1 = a.fac_r[o.r + (size_t)o.stride_r], r2 = a.fac_r[o.r + 2 * (size_t)o.stride_r];
-    const float c0 = a.fac_c[o.c], c1 = a.fac_c[o.c + (size_t)o.stride_c], c2 = a.fac_c[o.c + 2 * (size_t)o.stride_c];
+    const float r0 = ld<ST>(a.fac_r, o.r), r1 = ld<ST>(a.fac_r, o.r + (size_t)o.stride_r), r2 = ld<ST>(a.fac_r, o.r + 2 * (size_t)o.stride_r);
+    const float c0 = ld<ST>(a.fac_c, o.c), c1 = ld<ST>(a.fac_c, o.c + (size_t)o.stride_c), c2 = ld<ST>(a.fac_c, o.c + 2 * (size_t)o.stride_c);
     f[13] = r0; f[14] = r1; f[15] = r2; f[16] = c0; f[17] = c1; f[18] = c2;
     f[19] = rsq(r0 + 1e-8f); f[20] = rsq(r1 + 1e-8f); f[21] = rsq(r2 + 1e-8f);
     f[22] = rsq(c0 + 1e-8f); f[23] = rsq(c1 + 1e-8f); f[24] = rsq(c2 + 1e-8f);
@@ -91,8 +108,8 @@ __device__ __forceinline__ void single_features(const SingleArgs& a, int idx, fl
       for (int c = 15; c < 30; ++c) f[c] = 0.0f;
       return;
     }
-    const float r0 = a.fac_r[o.r], r1 = a.fac_r[o.r + (size_t)o.stride_r], r2 = a.fac_r[o.r + 2 * (size_t)o.stride_r];
-    const float c0 = a.fac_c[o.c], c1 = a.fac_c[o.c + (size_t)o.stride_c], c2 = a.fac_c[o.c + 2 * (size_t)o.stride_c];
+    const float r0 = ld<ST>(a.fac_r, o.r), r1 = ld<ST>(a.fac_r, o.r + (size_t)o.stride_r), r2 = ld<ST>(a.fac_r, o.r + 2 * (size_t)o.stride_r);
+    const float c0 = ld<ST>(a.fac_c, o.c), c1 = ld<ST>(a.fac_c, o.c + (size_t)o.stride_c), c2 = ld<ST>(a.fac_c, o.c + 2 * (size_t)o.stride_c);
     f[15] = r0; f[16] = r1; f[17] = r2; f[18] = c0; f[19] = c1; f[20] = c2;
     f[21] = rsq(r0 + 1e-8f); f[22] = rsq(r1 + 1e-8f); f[23] = rsq(r2 + 1e-8f);
     f[24] = rsq(c0 + 1e-8f); f[25] = rsq(c1 + 1e-8f); f[26] = rsq(c2 + 1e-8f);
@@ -102,7 +119,7 @@ __device__ __forceinline__ void single_features(const SingleArgs& a, int idx, fl
 
 // second_moment[c] += sum over the elements of feature_c^2: per-thread and per-wave sums, then one
 // float atomic per channel and block, as the reference does (celo2_kernel.cu:129-199).
-template <int F>
+template <int F, int ST>
 __global__ __launch_bounds__(kSingleThreads) void k_single_moment(SingleArgs a) {
   constexpr int NS = Fam<F>::NSTAT;
   float acc[NS];
@@ -111,7 +128,7 @@ __global__ __launch_bounds__(kSingleThreads) void k_single_moment(SingleArgs a) 
   for (long long i = (long long)blockIdx.x * kSingleThreads + threadIdx.x; i < a.n;
        i += (long long)gridDim.x * kSingleThreads) {
     float f[NS];
-    single_features<F>(a, (int)i, f);
+    single_features<F, ST>(a, (int)i, f);
 #pragma unroll
     for (int c = 0; c < NS; ++c) acc[c] = fmaf(f[c], f[c], acc[c]);
   }
@@ -131,97 +148,115 @@ __global__ __launch_bounds__(kSingleThreads) void k_single_moment(SingleArgs a) 
   }
 }
 
+// The MLP of one element on normalised features; WP is the pointer type the weights are read through.
+template <int F, class WP>
+__device__ __forceinline__ void single_mlp(const float (&f)[Fam<F>::NSTAT], const float* b1, WP w1, WP w2, WP w3, WP bh,
+                                           WP bo, float (&out)[Fam<F>::NOUT]) {
+  using Fm = Fam<F>;
+  constexpr int NS = Fm::NSTAT, NIN = Fm::NIN, H = Fm::H, NO = Fm::NOUT;
+  float h0[H], h1[H];
+  if constexpr (Fm::in_major) {
+#pragma unroll
+    for (int j = 0; j < H; ++j) h0[j] = b1[j];
+#pragma unroll
+    for (int k = 0; k < NS; ++k)
+#pragma unroll
+      for (int j = 0; j < H; ++j) h0[j] = fmaf(f[k], w1[k * H + j], h0[j]);
+#pragma unroll
+    for (int j = 0; j < H; ++j) { h0[j] = fmaxf(h0[j], 0.0f); h1[j] = bh[j]; }
+#pragma unroll
+    for (int k = 0; k < H; ++k)
+#pragma unroll
+      for (int j = 0; j < H; ++j) h1[j] = fmaf(h0[k], w2[k * H + j], h1[j]);
+#pragma unroll
+    for (int j = 0; j < NO; ++j) out[j] = bo[j];
+#pragma unroll
+    for (int k = 0; k < H; ++k) {
+      const float hk = fmaxf(h1[k], 0.0f);
+#pragma unroll
+      for (int j = 0; j < NO; ++j) out[j] = fmaf(hk, w3[k * NO + j], out[j]);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < H; ++j) {
+      float acc = b1[j];
+#pragma unroll
+      for (int k = 0; k < NS; ++k) acc = fmaf(f[k], w1[j * NIN + k], acc);
+      h0[j] = fmaxf(acc, 0.0f);
+    }
+#pragma unroll
+    for (int j = 0; j < H; ++j) {
+      float acc = bh[j];
+#pragma unroll
+      for (int k = 0; k < H; ++k) acc = fmaf(h0[k], w2[j * H + k], acc);
+      h1[j] = fmaxf(acc, 0.0f);
+    }
+#pragma unroll
+    for (int j = 0; j < NO; ++j) {
+      float acc = bo[j];
+#pragma unroll
+      for (int k = 0; k < H; ++k) acc = fmaf(h1[k], w3[j * H + k], acc);
+      out[j] = acc;
+    }
+  }
+}
+
 // Normalise by rsqrt(second_moment / n + eps), MLP, output.  The weights are the same for every lane:
-// they are read through the scalar cache into SGPRs where they are used (the pointer is laundered once
-// per element so that the loads stay inside the loop instead of being hoisted into a register file they
-// do not fit), which leaves the vector pipe with the multiply-adds only.  AdafacLO's eleven time features
-// are the same for every element and go into the first bias, once per block.
-template <int F>
+// float weights are read through the scalar cache into SGPRs where they are used (the pointer is laundered
+// once per element so that the loads stay inside the loop instead of being hoisted into a register file they
+// do not fit), which leaves the vector pipe with the multiply-adds only; weights of another element type are
+// widened into LDS once per block and read from there.  AdafacLO's eleven time features are the same for
+// every element and go into the first bias, once per block.
+template <int F, int ST>
 __global__ __launch_bounds__(kSingleThreads) void k_single_apply(SingleArgs a) {
   using Fm = Fam<F>;
   constexpr int NS = Fm::NSTAT, NIN = Fm::NIN, H = Fm::H, NO = Fm::NOUT;
+  constexpr int kW1 = 0, kW2 = NIN * H, kW3 = kW2 + H * H, kBH = kW3 + H * NO, kBO = kBH + H, kWTot = kBO + NO;
   __shared__ float s_norm[NS];
   __shared__ float b1[H];
+  __shared__ float wl[ST == kStoreF32 ? 1 : kWTot];
   const int tid = threadIdx.x;
   const float nf = (float)a.n;
   if (tid < NS) s_norm[tid] = rsq(a.second_moment[tid] / nf + (F == kFamCelo2 ? 1e-9f : 1e-5f));
   if (tid < H) {
-    float b = a.b_in[tid];
+    float b = ld<ST>(a.b_in, tid);
     if constexpr (F == kFamLo) {   // tanh(step / ts - 1), learned_optimizer.cu:27-32
       const float ts[11] = {1.f, 3.f, 10.f, 30.f, 100.f, 300.f, 1000.f, 3000.f, 10000.f, 30000.f, 100000.f};
 #pragma unroll
-      for (int q = 0; q < 11; ++q) b = fmaf(tanhf(a.step / ts[q] - 1.0f), a.w_in[tid * NIN + NS + q], b);
+      for (int q = 0; q < 11; ++q) b = fmaf(tanhf(a.step / ts[q] - 1.0f), ld<ST>(a.w_in, tid * NIN + NS + q), b);
     }
     b1[tid] = b;
+  }
+  if constexpr (ST != kStoreF32) {
+    for (int i = tid; i < NIN * H; i += kSingleThreads) wl[kW1 + i] = ld<ST>(a.w_in, i);
+    for (int i = tid; i < H * H; i += kSingleThreads) wl[kW2 + i] = ld<ST>(a.w_h, i);
+    for (int i = tid; i < H * NO; i += kSingleThreads) wl[kW3 + i] = ld<ST>(a.w_out, i);
+    for (int i = tid; i < H; i += kSingleThreads) wl[kBH + i] = ld<ST>(a.b_h, i);
+    for (int i = tid; i < NO; i += kSingleThreads) wl[kBO + i] = ld<ST>(a.b_out, i);
   }
   __syncthreads();
   const float pscale = F == kFamVelo ? sqrtf(a.second_moment[2] / nf + 1e-9f) : 1.0f;   // channel 2 is p
 
   for (long long i = (long long)blockIdx.x * kSingleThreads + tid; i < a.n; i += (long long)gridDim.x * kSingleThreads) {
     float f[NS];
-    single_features<F>(a, (int)i, f);
+    single_features<F, ST>(a, (int)i, f);
     const float p_old = f[F == kFamLo ? 1 : 2];
 #pragma unroll
     for (int k = 0; k < NS; ++k) f[k] *= s_norm[k];
-    const cfloat* w1 = launder(a.w_in);
-    const cfloat* w2 = launder(a.w_h);
-    const cfloat* w3 = launder(a.w_out);
-    const cfloat* bh = launder(a.b_h);
-    const cfloat* bo = launder(a.b_out);
-    float h0[H], h1[H], out[NO];
-    if constexpr (Fm::in_major) {
-#pragma unroll
-      for (int j = 0; j < H; ++j) h0[j] = b1[j];
-#pragma unroll
-      for (int k = 0; k < NS; ++k)
-#pragma unroll
-        for (int j = 0; j < H; ++j) h0[j] = fmaf(f[k], w1[k * H + j], h0[j]);
-#pragma unroll
-      for (int j = 0; j < H; ++j) { h0[j] = fmaxf(h0[j], 0.0f); h1[j] = bh[j]; }
-#pragma unroll
-      for (int k = 0; k < H; ++k)
-#pragma unroll
-        for (int j = 0; j < H; ++j) h1[j] = fmaf(h0[k], w2[k * H + j], h1[j]);
-#pragma unroll
-      for (int j = 0; j < NO; ++j) out[j] = bo[j];
-#pragma unroll
-      for (int k = 0; k < H; ++k) {
-        const float hk = fmaxf(h1[k], 0.0f);
-#pragma unroll
-        for (int j = 0; j < NO; ++j) out[j] = fmaf(hk, w3[k * NO + j], out[j]);
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < H; ++j) {
-        float acc = b1[j];
-#pragma unroll
-        for (int k = 0; k < NS; ++k) acc = fmaf(f[k], w1[j * NIN + k], acc);
-        h0[j] = fmaxf(acc, 0.0f);
-      }
-#pragma unroll
-      for (int j = 0; j < H; ++j) {
-        float acc = bh[j];
-#pragma unroll
-        for (int k = 0; k < H; ++k) acc = fmaf(h0[k], w2[j * H + k], acc);
-        h1[j] = fmaxf(acc, 0.0f);
-      }
-#pragma unroll
-      for (int j = 0; j < NO; ++j) {
-        float acc = bo[j];
-#pragma unroll
-        for (int k = 0; k < H; ++k) acc = fmaf(h1[k], w3[j * H + k], acc);
-        out[j] = acc;
-      }
-    }
+    float out[NO];
+    if constexpr (ST == kStoreF32)
+      single_mlp<F>(f, b1, launder(a.w_in), launder(a.w_h), launder(a.w_out), launder(a.b_h), launder(a.b_out), out);
+    else
+      single_mlp<F, const float*>(f, b1, wl + kW1, wl + kW2, wl + kW3, wl + kBH, wl + kBO, out);
     const float step = out[0] * expf(out[1] * a.exp_mult);
     if constexpr (F == kFamCelo2) {
-      a.step_out[i] = step;                                   // celo2_kernel.cu:280; p is left untouched
+      st<ST>(a.step_out, i, step);                             // celo2_kernel.cu:280; p is left untouched
     } else if constexpr (F == kFamLo) {
-      a.p[i] = p_old - a.lr * (step * a.step_mult);           // learned_optimizer.cu:296-299
+      st<ST>(a.p, i, p_old - a.lr * (step * a.step_mult));    // learned_optimizer.cu:296-299
     } else {
       float pn = p_old - a.lr * (pscale * step * a.step_mult); // velo_kernel.cu:352-362
       if (a.weight_decay > 0.0f) pn = pn - a.weight_decay * a.lr * pn;
-      a.p[i] = pn;
+      st<ST>(a.p, i, pn);
     }
   }
 }

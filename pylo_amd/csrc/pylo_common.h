@@ -105,6 +105,7 @@ struct TDesc {
   int slice_len;           // CELO2, N-D or fewer than two dims: elements per slice of the last two dims (or n)
   int nan0;                // gradients pass through torch.nan_to_num (PYLO_F_NAN_TO_NUM)
   int wd_prestep;          // p -= lr * (step + wd * p) against the pre-step parameter (PYLO_F_WD_PRESTEP)
+  int store;               // storage type of the caller's grad / param buffers (kStore*, k_cast.h); 0 = fp32
   float gscale;            // 1 in the plan; AdafacLO-family kernels overwrite their copy with the clip scale
 };
 

@@ -31,6 +31,7 @@
 #include "k_celo2_slices.h"
 #include "k_ns.h"
 #include "k_ns_bf.h"
+#include "k_cast.h"
 #include "pylo_common.h"
 
 // =============================================================================================
@@ -90,6 +91,12 @@ struct Layout {
   long long nsb_plane_elems = 0;
   size_t off_ns_mats = 0, off_ns_gram = 0, off_ns_poly = 0, off_ns_upd = 0, off_ns_split = 0, off_ns_xalt = 0,
          off_ns_scale = 0, off_ns_ws = 0;
+  // tensors whose grad / param are not fp32 (PYLO_F_STORE_*): fp32 staging, pieces of the cast kernels
+  bool typed = false;
+  std::vector<StageOfs> stage_ofs;
+  std::vector<Item> cast_items;
+  long long stage_floats = 0;
+  size_t off_dyn_user = 0, off_stage_ofs = 0, off_cast_items = 0, off_stage = 0;
   std::vector<TDesc> descs;
   std::vector<Item> p0_items, nd_items, sl_items, seg_items, el_items, ap_items, ga_items, fin_items, v0a_items, v0b_items;
   std::vector<int> fac_list;
@@ -378,6 +385,15 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     if (((s.flags & PYLO_F_GLOBAL_NORM) != 0) != L.global_norm)
       return fail("plan: PYLO_F_GLOBAL_NORM must be set on every tensor of the plan or on none");
     d.nan0 = (s.flags & PYLO_F_NAN_TO_NUM) != 0;
+    d.store = (s.flags & PYLO_F_STORE_MASK) >> 8;
+    L.stage_ofs.push_back(StageOfs{-1, -1});
+    if (d.store != kStoreF32 && n > 0) {
+      const long long pitch = (n + 63) / 64 * 64;
+      L.stage_ofs.back() = StageOfs{L.stage_floats, L.stage_floats + pitch};
+      L.stage_floats += 2 * pitch;
+      for (long long c = 0; c * kCastElems < n; ++c) L.cast_items.push_back(Item{t, (int)c, 0, 0});
+      L.typed = true;
+    }
     d.wd_prestep = (s.flags & PYLO_F_WD_PRESTEP) != 0;
     d.fac_slot = -1;
     d.rank = rank < 4 ? rank : 4;
@@ -528,6 +544,10 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   const size_t nfac = std::max<size_t>(L.fac_list.size(), 1);
   L.off_descs = take(sizeof(TDesc) * T);
   L.off_dyn = take(sizeof(PyloTensorArgs) * T);
+  L.off_dyn_user = L.typed ? take(sizeof(PyloTensorArgs) * T) : L.off_dyn;
+  L.off_stage_ofs = take(L.typed ? sizeof(StageOfs) * T : 0);
+  L.off_cast_items = take(sizeof(Item) * L.cast_items.size());
+  L.off_stage = take(sizeof(float) * (size_t)L.stage_floats);
   L.off_p0_items = take(sizeof(Item) * L.p0_items.size());
   L.off_nd_items = take(sizeof(Item) * L.nd_items.size());
   L.off_sl_items = take(sizeof(Item) * L.sl_items.size());
@@ -604,6 +624,7 @@ struct PyloPlan {
   int slot = 0;
   PyloDeviceSteps dsteps = {nullptr, 0.0, 0.0, 1.0};
   std::vector<PyloTensorArgs> last;
+  size_t last_dst = 0;   // where `last` was copied to
   bool have_last = false;
   bool mlp_on_matrix_pipe = true;  // env_matrix_pipe() when the plan was created
   // optional per-launch timing (pylo_mi355_plan_timing_begin/end)
@@ -655,6 +676,8 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   hipError_t e = hipSuccess;
   if (e == hipSuccess) e = up(L.off_descs, L.descs.data(), sizeof(TDesc) * L.descs.size());
   if (e == hipSuccess) e = up(L.off_p0_items, L.p0_items.data(), sizeof(Item) * L.p0_items.size());
+  if (e == hipSuccess && L.typed) e = up(L.off_stage_ofs, L.stage_ofs.data(), sizeof(StageOfs) * L.stage_ofs.size());
+  if (e == hipSuccess) e = up(L.off_cast_items, L.cast_items.data(), sizeof(Item) * L.cast_items.size());
   if (e == hipSuccess) e = up(L.off_nd_items, L.nd_items.data(), sizeof(Item) * L.nd_items.size());
   if (e == hipSuccess) e = up(L.off_sl_items, L.sl_items.data(), sizeof(Item) * L.sl_items.size());
   if (e == hipSuccess) e = up(L.off_seg_items, L.seg_items.data(), sizeof(Item) * L.seg_items.size());
@@ -810,7 +833,9 @@ __global__ __launch_bounds__(256) void k_copy_args(const uint4* __restrict__ src
   for (int i = blockIdx.x * 256 + threadIdx.x; i < n16; i += gridDim.x * 256) dst[i] = src[i];
 }
 
-int upload_args(PyloPlan* P, const PyloTensorArgs* args, hipStream_t s) {
+// `dst_off`: where the table goes, the records the kernels read (off_dyn) or, for a step of a plan with
+// tensors of other storage types, the caller's records that k_stage_args copies from (off_dyn_user).
+int upload_args(PyloPlan* P, const PyloTensorArgs* args, hipStream_t s, size_t dst_off) {
   const size_t bytes = sizeof(PyloTensorArgs) * P->T;
   static_assert(sizeof(PyloTensorArgs) % 8 == 0, "argument records are copied in 16-byte pieces");
   const int n16 = (int)((bytes + 15) / 16);
@@ -822,11 +847,11 @@ int upload_args(PyloPlan* P, const PyloTensorArgs* args, hipStream_t s) {
     void* src_dev = nullptr;
     HIP_TRY(hipHostGetDevicePointer(&src_dev, P->stage[j], 0));
     hipLaunchKernelGGL(k_copy_args, grid, dim3(256), 0, s, static_cast<const uint4*>(src_dev),
-                       reinterpret_cast<uint4*>(P->ws + P->L.off_dyn), n16);
+                       reinterpret_cast<uint4*>(P->ws + dst_off), n16);
     P->have_last = false;
     return 0;
   }
-  if (P->have_last && std::memcmp(P->last.data(), args, bytes) == 0) return 0;
+  if (P->have_last && P->last_dst == dst_off && std::memcmp(P->last.data(), args, bytes) == 0) return 0;
   int i = -1;
   for (int k = 0; k < kStageSlots && i < 0; ++k) {
     const int c = (P->slot + k) % kStageSlots;
@@ -839,12 +864,34 @@ int upload_args(PyloPlan* P, const PyloTensorArgs* args, hipStream_t s) {
   void* src_dev = nullptr;
   HIP_TRY(hipHostGetDevicePointer(&src_dev, P->stage[i], 0));
   hipLaunchKernelGGL(k_copy_args, grid, dim3(256), 0, s,
-                     static_cast<const uint4*>(src_dev), reinterpret_cast<uint4*>(P->ws + P->L.off_dyn), n16);
+                     static_cast<const uint4*>(src_dev), reinterpret_cast<uint4*>(P->ws + dst_off), n16);
   HIP_TRY(hipEventRecord(P->ev[i], s));
   P->ev_used[i] = true;
   P->last.assign(args, args + P->T);
+  P->last_dst = dst_off;
   P->have_last = true;
   return 0;
+}
+
+// Step of a plan with tagged tensors: the records the kernels read are the caller's with grad / param of the
+// tagged tensors redirected into the staging, which is filled here.  `what`: 1 gradient, 2 parameter, 3 both.
+void stage_in(PyloPlan* P, hipStream_t s, int what) {
+  const Layout& L = P->L;
+  if (!L.typed) return;
+  hipLaunchKernelGGL(k_stage_args, dim3((P->T + 255) / 256), dim3(256), 0, s, P->T, P->at<TDesc>(L.off_descs),
+                     P->at<PyloTensorArgs>(L.off_dyn_user), P->at<PyloTensorArgs>(L.off_dyn),
+                     P->at<StageOfs>(L.off_stage_ofs), P->at<float>(L.off_stage));
+  hipLaunchKernelGGL(k_cast_in, dim3((unsigned)L.cast_items.size()), dim3(kThreads), 0, s, P->at<TDesc>(L.off_descs),
+                     P->at<PyloTensorArgs>(L.off_dyn_user), P->at<Item>(L.off_cast_items),
+                     P->at<StageOfs>(L.off_stage_ofs), P->at<float>(L.off_stage), what);
+}
+
+void stage_out(PyloPlan* P, hipStream_t s, int flat_only) {
+  const Layout& L = P->L;
+  if (!L.typed) return;
+  hipLaunchKernelGGL(k_cast_out, dim3((unsigned)L.cast_items.size()), dim3(kThreads), 0, s, P->at<TDesc>(L.off_descs),
+                     P->at<PyloTensorArgs>(L.off_dyn_user), P->at<Item>(L.off_cast_items),
+                     P->at<StageOfs>(L.off_stage_ofs), P->at<float>(L.off_stage), flat_only);
 }
 
 // Step counters kept on the device: advances them and writes what the host otherwise supplies per
@@ -914,6 +961,9 @@ int check_args(const PyloPlan* P, const PyloTensorArgs* args, bool need_all_grad
                         reinterpret_cast<uintptr_t>(a.fac_r) | reinterpret_cast<uintptr_t>(a.fac_c) |
                         reinterpret_cast<uintptr_t>(a.fac_v) | reinterpret_cast<uintptr_t>(a.step_out);
     if (m % (d.vec == 4 ? 16 : 4) != 0) return fail("step: misaligned pointer (16 bytes needed)" + at);
+    const uintptr_t gp = reinterpret_cast<uintptr_t>(a.grad) | reinterpret_cast<uintptr_t>(a.param);
+    if (d.store != kStoreF32 && gp % 16 != 0)
+      return fail("step: grad / param of a tensor with a storage type tag must be 16-byte aligned" + at);
   }
   return 0;
 }
@@ -954,7 +1004,8 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   if (P->kind != PYLO_KIND_CELO2) return fail("celo2_step: plan is not a CELO2 plan");
   if (int rc = check_args(P, args, false)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (int rc = upload_args(P, args, s)) return rc;
+  if (int rc = upload_args(P, args, s, P->L.off_dyn_user)) return rc;
+  stage_in(P, s, 3);
   advance_steps(P, s);
   const Layout& L = P->L;
   const TDesc* descs = P->at<TDesc>(L.off_descs);
@@ -1039,6 +1090,7 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
     hipLaunchKernelGGL(k_celo2_slices, dim3(n_sl), dim3(kThreads), 0, s, descs, dyn, sl_items, fac_tab, gl, dec, mlp);
   HIP_TRY(mark());
   mark.done();
+  stage_out(P, s, 1);   // only the AdamW tensors were updated
   HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -1070,7 +1122,8 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
     }
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (int rc = upload_args(P, args, s)) return rc;
+  // the caller's records as they are: the update kernel reads and writes the parameter in its storage type
+  if (int rc = upload_args(P, args, s, L.off_dyn)) return rc;
   const TDesc* descs = P->at<TDesc>(L.off_descs);
   const PyloTensorArgs* dyn = P->at<PyloTensorArgs>(L.off_dyn);
   const Item* fin_items = P->at<Item>(L.off_fin_items);
@@ -1169,8 +1222,12 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
     return fail("velo_step: null state pointer");
   if (int rc = check_args(P, args, true)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (int rc = upload_args(P, args, s)) return rc;
+  if (int rc = upload_args(P, args, s, P->L.off_dyn_user)) return rc;
+  stage_in(P, s, 3);
   advance_steps(P, s);
+  // the sums the apply items carry over are taken on the fp32 parameter they write; the next step starts
+  // from that value rounded to the tensor's storage type
+  if (P->L.typed) P->stats_carried = false;
   const Layout& L = P->L;
   const TDesc* descs = P->at<TDesc>(L.off_descs);
   const PyloTensorArgs* dyn = P->at<PyloTensorArgs>(L.off_dyn);
@@ -1262,6 +1319,7 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
                        dec, (const float*)wmix, wfold, stats, (const float*)piv, newsum, P->at<int>(L.off_sync), T);
     HIP_TRY(mark());
     mark.done();
+    stage_out(P, s, 0);
     HIP_TRY(hipGetLastError());
     return 0;
   }
@@ -1289,6 +1347,7 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
                        (const float*)piv, newsum);
   HIP_TRY(mark());
   mark.done();
+  stage_out(P, s, 0);
   HIP_TRY(hipGetLastError());
   P->stats_carried = n_mx > 0;
   return 0;
@@ -1306,7 +1365,8 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   if (P->kind != PYLO_KIND_ADAFAC) return fail("adafac_step: plan is not an AdafacLO plan");
   if (int rc = check_args(P, args, false)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (int rc = upload_args(P, args, s)) return rc;
+  if (int rc = upload_args(P, args, s, P->L.off_dyn_user)) return rc;
+  stage_in(P, s, 3);
   advance_steps(P, s);
   const Layout& L = P->L;
   const TDesc* descs = P->at<TDesc>(L.off_descs);
@@ -1389,6 +1449,7 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
                        dec, wfold, net, gl);
   HIP_TRY(mark());
   mark.done();
+  stage_out(P, s, 0);
   HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -1447,14 +1508,26 @@ int single_check(const char* who, const SingleArgs& a) {
   return 0;
 }
 
+template <int F, int ST>
+void single_enqueue(const SingleArgs& a, int blocks, hipStream_t s) {
+  hipLaunchKernelGGL((k_single_moment<F, ST>), dim3(blocks), dim3(kSingleThreads), 0, s, a);
+  hipLaunchKernelGGL((k_single_apply<F, ST>), dim3(blocks), dim3(kSingleThreads), 0, s, a);
+}
+
+// `dtype`: PYLO_F_STORE_* of every array but `second_moment` (the reference's scalar_t)
 template <int F>
-int single_launch(const char* who, const SingleArgs& a, void* stream) {
+int single_launch(const char* who, const SingleArgs& a, void* stream, int dtype = PYLO_F_STORE_F32) {
+  if (dtype & ~PYLO_F_STORE_MASK) return fail(std::string(who) + ": dtype must be one of PYLO_F_STORE_*");
   if (a.n == 0) return 0;
   if (int rc = single_check<F>(who, a)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int blocks = std::min((a.n + kSingleThreads - 1) / kSingleThreads, kSingleMaxBlocks);
-  hipLaunchKernelGGL(k_single_moment<F>, dim3(blocks), dim3(kSingleThreads), 0, s, a);
-  hipLaunchKernelGGL(k_single_apply<F>, dim3(blocks), dim3(kSingleThreads), 0, s, a);
+  switch (dtype >> 8) {
+    case kStoreF16: single_enqueue<F, kStoreF16>(a, blocks, s); break;
+    case kStoreBF16: single_enqueue<F, kStoreBF16>(a, blocks, s); break;
+    case kStoreF64: single_enqueue<F, kStoreF64>(a, blocks, s); break;
+    default: single_enqueue<F, kStoreF32>(a, blocks, s);
+  }
   HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -1514,6 +1587,69 @@ extern "C" int pylo_mi355_velo_kernel_simple(const float* grad, float* param, co
   a.lr = lr; a.step_mult = step_mult; a.exp_mult = exp_mult; a.epsilon = epsilon; a.weight_decay = weight_decay;
   return single_launch<kFamVelo>("velo_kernel_simple", a, stream);
 }
+
+// The same three calls for arrays of another element type (the reference's AT_DISPATCH_FLOATING_TYPES_AND_HALF
+// over p.scalar_type(), celo2_kernel.cu:314,328, learned_optimizer.cu:338,364, velo_kernel.cu:405,427): every
+// array but `second_moment` holds elements of `dtype`.
+#define PYLO_AS_F(x) static_cast<const float*>(x)
+extern "C" int pylo_mi355_celo2_kernel_typed(int dtype, const void* g, const void* p, const void* m, const void* v,
+                                             const void* fac_r, const void* fac_c, const void* row_factor,
+                                             const void* col_factor, float* second_moment, const void* w_in,
+                                             const void* b_in, const void* w_h, const void* b_h, const void* w_out,
+                                             const void* b_out, void* step_out, float exp_mult, const int64_t* shape,
+                                             int ndim, int dc, int dr, int vector_like, void* stream) {
+  SingleArgs a{};
+  if (int rc = single_geometry("celo2_kernel", shape, ndim, dc, dr, vector_like, a)) return rc;
+  a.g = PYLO_AS_F(g); a.p = const_cast<float*>(PYLO_AS_F(p)); a.m = PYLO_AS_F(m); a.v = PYLO_AS_F(v);
+  a.fac_r = PYLO_AS_F(fac_r); a.fac_c = PYLO_AS_F(fac_c);
+  a.row_factor = PYLO_AS_F(row_factor); a.col_factor = PYLO_AS_F(col_factor); a.second_moment = second_moment;
+  a.w_in = PYLO_AS_F(w_in); a.b_in = PYLO_AS_F(b_in); a.w_h = PYLO_AS_F(w_h); a.b_h = PYLO_AS_F(b_h);
+  a.w_out = PYLO_AS_F(w_out); a.b_out = PYLO_AS_F(b_out);
+  a.step_out = static_cast<float*>(step_out); a.exp_mult = exp_mult;
+  return single_launch<kFamCelo2>("celo2_kernel", a, stream, dtype);
+}
+
+extern "C" int pylo_mi355_learned_optimizer_kernel_typed(int dtype, const void* g, void* p, const void* m, const void* v,
+                                                         const void* fac_r, const void* fac_c, const void* row_factor,
+                                                         const void* col_factor, float* second_moment,
+                                                         const void* input_weights, const void* input_bias,
+                                                         const void* hidden_weights, const void* hidden_bias,
+                                                         const void* output_weights, const void* output_bias, float lr,
+                                                         float step_mult, float exp_mult, float epsilon, float step,
+                                                         float weight_decay, const int64_t* shape, int ndim, int dc,
+                                                         int dr, int vector_like, void* stream) {
+  SingleArgs a{};
+  if (int rc = single_geometry("learned_optimizer_kernel", shape, ndim, dc, dr, vector_like, a)) return rc;
+  a.g = PYLO_AS_F(g); a.p = static_cast<float*>(p); a.m = PYLO_AS_F(m); a.v = PYLO_AS_F(v);
+  a.fac_r = PYLO_AS_F(fac_r); a.fac_c = PYLO_AS_F(fac_c);
+  a.row_factor = PYLO_AS_F(row_factor); a.col_factor = PYLO_AS_F(col_factor); a.second_moment = second_moment;
+  a.w_in = PYLO_AS_F(input_weights); a.b_in = PYLO_AS_F(input_bias); a.w_h = PYLO_AS_F(hidden_weights);
+  a.b_h = PYLO_AS_F(hidden_bias); a.w_out = PYLO_AS_F(output_weights); a.b_out = PYLO_AS_F(output_bias);
+  a.lr = lr; a.step_mult = step_mult; a.exp_mult = exp_mult; a.epsilon = epsilon; a.step = step;
+  a.weight_decay = weight_decay;
+  return single_launch<kFamLo>("learned_optimizer_kernel", a, stream, dtype);
+}
+
+extern "C" int pylo_mi355_velo_kernel_simple_typed(int dtype, const void* grad, void* param, const void* momentum,
+                                                   const void* rms, const void* row_factor, const void* col_factor,
+                                                   const void* fac_vec_row, const void* fac_vec_col,
+                                                   float* second_moment, const void* input_weights,
+                                                   const void* input_bias, const void* hidden_weights,
+                                                   const void* hidden_bias, const void* output_weights,
+                                                   const void* output_bias, float lr, float step_mult, float exp_mult,
+                                                   float epsilon, float weight_decay, const int64_t* shape, int ndim,
+                                                   int dc, int dr, int vector_like, void* stream) {
+  SingleArgs a{};
+  if (int rc = single_geometry("velo_kernel_simple", shape, ndim, dc, dr, vector_like, a)) return rc;
+  a.g = PYLO_AS_F(grad); a.p = static_cast<float*>(param); a.m = PYLO_AS_F(momentum); a.v = PYLO_AS_F(rms);
+  a.fac_r = PYLO_AS_F(fac_vec_row); a.fac_c = PYLO_AS_F(fac_vec_col);
+  a.row_factor = PYLO_AS_F(row_factor); a.col_factor = PYLO_AS_F(col_factor); a.second_moment = second_moment;
+  a.w_in = PYLO_AS_F(input_weights); a.b_in = PYLO_AS_F(input_bias); a.w_h = PYLO_AS_F(hidden_weights);
+  a.b_h = PYLO_AS_F(hidden_bias); a.w_out = PYLO_AS_F(output_weights); a.b_out = PYLO_AS_F(output_bias);
+  a.lr = lr; a.step_mult = step_mult; a.exp_mult = exp_mult; a.epsilon = epsilon; a.weight_decay = weight_decay;
+  return single_launch<kFamVelo>("velo_kernel_simple", a, stream, dtype);
+}
+#undef PYLO_AS_F
 
 // ---------------------------------------------------------------------------------------------
 // celo2_kernel for callers that cannot allocate: the per-channel sums live in the library's own

@@ -129,16 +129,18 @@ class AdafacLO_CUDA(Optimizer):
         state["exp_avg"] = torch.zeros((3,) + shape, device=self.device)
 
     def _ensure_plan(self, tensors):
-        key = tuple(tuple(p.shape) for _, p in tensors)
+        key = tuple((tuple(p.shape), p.dtype) for _, p in tensors)
         if key == self._plan_key:
             return
         for _, p in tensors:
-            if not p.is_cuda or p.device != self.device or p.dtype != torch.float32 or not p.is_contiguous():
-                raise TypeError("AdafacLO_CUDA: parameters must be contiguous float32 tensors on the optimizer's GPU")
+            if not p.is_cuda or p.device != self.device or not p.is_contiguous():
+                raise TypeError("AdafacLO_CUDA: parameters must be contiguous tensors on the optimizer's GPU")
         if self._plan is not None:
             self._plan.close()
+        # parameters and gradients may be float16 / bfloat16 / float64 (the reference's kernels dispatch on the
+        # element type, learned_optimizer.cu:338,364); the accumulators stay float32
         self._plan = _lib.Plan(_lib.KIND_ADAFAC, [tuple(p.shape) for _, p in tensors],
-                               [self._PLAN_FLAGS] * len(tensors), self.device)
+                               [self._PLAN_FLAGS | _lib.store_flag(p, "AdafacLO_CUDA") for _, p in tensors], self.device)
         self._plan_key = key
         if self.capturable:
             self._reset_device_steps(tensors)
@@ -210,8 +212,8 @@ class AdafacLO_CUDA(Optimizer):
                 continue
             if g.is_sparse:
                 raise RuntimeError("Sparse gradients not supported")
-            if g.dtype != torch.float32:
-                raise TypeError("AdafacLO_CUDA: gradients must be float32")
+            if g.dtype != p.dtype:
+                raise TypeError("AdafacLO_CUDA: a gradient must have its parameter's dtype")
             if not g.is_contiguous():
                 g = g.contiguous()
                 keep.append(g)

@@ -111,6 +111,16 @@ def rms_normalize(x: torch.Tensor, dims, eps: float = 1e-9) -> torch.Tensor:
     return x * torch.rsqrt(eps + torch.mean(x * x, dim=dims, keepdim=True))
 
 
+def _apply(p, step, weight_decay, lr):
+    """p <- p - lr (step + wd p) in fp32 on the widened parameter, rounded into p's own dtype
+    (what the library's update kernel does for the tensors it finishes itself)."""
+    if p.dtype == torch.float32:
+        p.add_(step + weight_decay * p, alpha=-lr)
+    else:
+        pf = p.float()
+        p.copy_(pf.add_(step + weight_decay * pf, alpha=-lr))
+
+
 class ELO_CELO2_CUDA(Optimizer):
     """Inference-time ELO-CELO2: CELO2 MLP steps for >=2-D tensors, shared-accumulator AdamW for
     1-D tensors and ``is_embedding`` groups."""
@@ -213,18 +223,20 @@ class ELO_CELO2_CUDA(Optimizer):
         return out
 
     def _ensure_plan(self, tensors):
-        key = tuple((tuple(p.shape), adam) for _, p, adam in tensors)
+        key = tuple((tuple(p.shape), adam, p.dtype) for _, p, adam in tensors)
         if key == self._plan_key:
             return
         for _, p, _a in tensors:
             if not p.is_cuda or p.device != self.device:
                 raise RuntimeError("ELO_CELO2_CUDA: every parameter must live on the optimizer's GPU")
-            if p.dtype != torch.float32 or not p.is_contiguous():
-                raise TypeError("ELO_CELO2_CUDA: parameters must be contiguous float32 tensors")
+            if not p.is_contiguous():
+                raise TypeError("ELO_CELO2_CUDA: parameters must be contiguous tensors")
         if self._plan is not None:
             self._plan.close()
         shapes = [tuple(p.shape) for _, p, _a in tensors]
-        flags = [self._ADAM_FLAG if adam else 0 for _, _p, adam in tensors]
+        # parameters and gradients may be float16 / bfloat16 / float64 (the reference's kernel dispatches on the
+        # element type, celo2_kernel.cu:314,328); accumulators and raw steps stay float32 (ELO_CELO2_cuda.py:167-177)
+        flags = [(self._ADAM_FLAG if adam else 0) | _lib.store_flag(p, type(self).__name__) for _, p, adam in tensors]
         self._plan = _lib.Plan(_lib.KIND_CELO2, shapes, flags, self.device)
         self._plan_key = key
         # Raw steps of the MLP tensors: tensors of one parameter group and one shape share a
@@ -353,9 +365,8 @@ class ELO_CELO2_CUDA(Optimizer):
 
     def _fused_step_fast(self, fast):
         grads = [p.grad for p in fast["params"]]
-        f32 = torch.float32
-        for g in grads:
-            if g is None or g.dtype is not f32 or g.layout is not torch.strided or not g.is_contiguous():
+        for g in grads:     # a dense gradient has its parameter's dtype (torch enforces it on assignment)
+            if g is None or g.layout is not torch.strided or not g.is_contiguous():
                 return None
         groups = self.param_groups
         if len(groups) != fast["n_groups"] or len(self.state) != fast["n_state"]:
@@ -409,8 +420,8 @@ class ELO_CELO2_CUDA(Optimizer):
                 continue
             if g.is_sparse:
                 raise RuntimeError("ELO_CELO2_CUDA does not support sparse gradients")
-            if g.dtype != torch.float32:
-                raise TypeError("ELO_CELO2_CUDA: gradients must be float32")
+            if g.dtype != p.dtype:
+                raise TypeError("ELO_CELO2_CUDA: a gradient must have its parameter's dtype")
             if not g.is_contiguous():
                 g = g.contiguous()
                 keep.append(g)
@@ -479,18 +490,19 @@ class ELO_CELO2_CUDA(Optimizer):
                         continue
                     step = self._raw[i]
                     if group["param_scale_mult"]:
-                        step = step * torch.sqrt(torch.mean(p * p) + 1e-9)
+                        pf = p.float()
+                        step = step * torch.sqrt(torch.mean(pf * pf) + 1e-9)
                     if group["orthogonalize"] and step.dim() >= 2:
                         with _ns_blas():
                             step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
                     step = rms_normalize(step, list(range(step.dim()))[-2:]) * group["rmsmult"]
-                    p.add_(step + group["weight_decay"] * p, alpha=-group["lr"])
+                    _apply(p, step, group["weight_decay"], group["lr"])
                 continue
             step = buf
             nd = buf.dim() - 1
             if group["param_scale_mult"]:
                 n = ps[0].numel()
-                sq = torch.stack(torch._foreach_norm(ps)) ** 2 / n
+                sq = torch.stack(torch._foreach_norm([p.float() for p in ps] if ps[0].dtype != torch.float32 else ps)) ** 2 / n
                 step = step.mul_(torch.sqrt(sq + 1e-9).view([-1] + [1] * nd))   # the raw steps are scratch
             flag = 0
             if group["orthogonalize"] and nd >= 2:
@@ -504,7 +516,7 @@ class ELO_CELO2_CUDA(Optimizer):
                 # (ELO_CELO2_naive.py:217-218,235), which the tensor-wide finishing kernels do not do
                 step = rms_normalize(step, [-2, -1]) * group["rmsmult"]
                 for j, p in enumerate(ps):
-                    p.add_(step[j] + group["weight_decay"] * p, alpha=-group["lr"])
+                    _apply(p, step[j], group["weight_decay"], group["lr"])
                 continue
             step = step.contiguous()
             keep.append(step)

@@ -274,18 +274,20 @@ class VeLO_CUDA(Optimizer):
         return out
 
     def _ensure_plan(self, tensors):
-        key = tuple(tuple(p.shape) for _, _, p in tensors)
+        key = tuple((tuple(p.shape), p.dtype) for _, _, p in tensors)
         if key == self._plan_key:
             return
         if len(self.param_groups) > _lib.MAX_GROUPS:
             raise ValueError(f"VeLO_CUDA supports at most {_lib.MAX_GROUPS} parameter groups")
         for _, _, p in tensors:
-            if not p.is_cuda or p.device != self.device or p.dtype != torch.float32 or not p.is_contiguous():
-                raise TypeError("VeLO_CUDA: parameters must be contiguous float32 tensors on the optimizer's GPU")
+            if not p.is_cuda or p.device != self.device or not p.is_contiguous():
+                raise TypeError("VeLO_CUDA: parameters must be contiguous tensors on the optimizer's GPU")
         if self._plan is not None:
             self._plan.close()
-        self._plan = _lib.Plan(_lib.KIND_VELO, [tuple(p.shape) for _, _, p in tensors], [0] * len(tensors),
-                               self.device)
+        # parameters and gradients may be float16 / bfloat16 / float64 (the reference's kernels dispatch on the
+        # element type, velo_kernel.cu:405,427); the accumulators stay float32
+        self._plan = _lib.Plan(_lib.KIND_VELO, [tuple(p.shape) for _, _, p in tensors],
+                               [_lib.store_flag(p, "VeLO_CUDA") for _, _, p in tensors], self.device)
         self._plan_key = key
         if self.capturable:
             self._reset_device_steps()
@@ -321,9 +323,8 @@ class VeLO_CUDA(Optimizer):
             # static columns (state pointers, group index) are still in the table from an earlier
             # step: refresh gradient / parameter pointers and the per-group scalars only
             grads = [p.grad for _, _, p in tensors]
-            f32 = torch.float32
-            for g in grads:
-                if g is None or g.dtype is not f32 or g.layout is not torch.strided or not g.is_contiguous():
+            for g in grads:     # a dense gradient has its parameter's dtype (torch enforces it on assignment)
+                if g is None or g.layout is not torch.strided or not g.is_contiguous():
                     fast = self._fast = None
                     break
         if fast is not None:
@@ -353,8 +354,8 @@ class VeLO_CUDA(Optimizer):
             g = p.grad
             if g is None:
                 raise RuntimeError("VeLO_CUDA.step: every parameter needs a gradient")
-            if g.dtype != torch.float32 or g.is_sparse:
-                raise TypeError("VeLO_CUDA: gradients must be dense float32")
+            if g.dtype != p.dtype or g.is_sparse:
+                raise TypeError("VeLO_CUDA: gradients must be dense and of their parameter's dtype")
             if not g.is_contiguous():
                 g = g.contiguous()
                 keep.append(g)

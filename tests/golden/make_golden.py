@@ -120,8 +120,14 @@ def celo2_case(R, name, shapes, n_steps, grad_scale, seed, cfg, net_seed=1, full
 
 
 # ---------------------------------------------------------------------- VeLO
+_DTYPES = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}
+
+
 def velo_case(R, name, shapes, n_steps, grad_scale, seed, num_steps, weight_decay, lr,
-              lstm_hidden=64, param_inits=32):
+              lstm_hidden=64, param_inits=32, dtype="float32"):
+    """`dtype`: the parameters' and gradients' element type.  The naive class keeps its accumulators in
+    float32 and computes in whatever torch's type promotion gives; arrays are stored widened to float32."""
+    dt = _DTYPES[dtype]
     # A reduced LSTM width / bank size keeps the fixture small; both classes read the sizes
     # from the saved config.json, and the arithmetic does not depend on them.
     torch.manual_seed(11)
@@ -139,7 +145,7 @@ def velo_case(R, name, shapes, n_steps, grad_scale, seed, num_steps, weight_deca
     rnn.save_pretrained(os.path.join(tmp, "rnn"))
     mlp.save_pretrained(os.path.join(tmp, "mlp"))
     gen = torch.Generator().manual_seed(seed)
-    init = [torch.randn(s, generator=gen) * 0.5 for s in shapes]
+    init = [(torch.randn(s, generator=gen) * 0.5).to(dt) for s in shapes]
     params = [torch.nn.Parameter(v.clone()) for v in init]
     opt = R["VeLO_naive"](params, lr=lr, num_steps=num_steps, weight_decay=weight_decay,
                           hf_key_rnn=os.path.join(tmp, "rnn"), hf_key_mlp=os.path.join(tmp, "mlp"))
@@ -148,11 +154,11 @@ def velo_case(R, name, shapes, n_steps, grad_scale, seed, num_steps, weight_deca
     _sd_arrays("mlp", mlp, arrays)
     meta = dict(kind="velo", shapes=[list(s) for s in shapes], n_steps=n_steps, seed=seed,
                 num_steps=num_steps, weight_decay=weight_decay, lr=lr, grad_scale=grad_scale,
-                lstm_hidden=lstm_hidden, param_inits=param_inits)
+                lstm_hidden=lstm_hidden, param_inits=param_inits, dtype=dtype)
     for i, v in enumerate(init):
-        arrays[f"init/{i}"] = _np(v)
+        arrays[f"init/{i}"] = _np(v.float())
     for t in range(n_steps):
-        grads = [torch.randn(s, generator=gen) * grad_scale for s in shapes]
+        grads = [(torch.randn(s, generator=gen) * grad_scale).to(dt) for s in shapes]
         loss = torch.tensor(2.0 * np.exp(-t / 5.0) + 0.1 + 0.05 * ((t * 7) % 3), dtype=torch.float32)
         for p, g in zip(params, grads):
             p.grad = g.clone()
@@ -162,8 +168,8 @@ def velo_case(R, name, shapes, n_steps, grad_scale, seed, num_steps, weight_deca
         arrays[f"step{t}/lstm_c"] = _np(opt.lstm_hidden_state[1])
         for i, p in enumerate(params):
             st = opt.state[p]
-            arrays[f"grad{t}/{i}"] = _np(grads[i])
-            arrays[f"step{t}/param/{i}"] = _np(p)
+            arrays[f"grad{t}/{i}"] = _np(grads[i].float())
+            arrays[f"step{t}/param/{i}"] = _np(p.float())
             arrays[f"step{t}/mom/{i}"] = _np(st["mom"].movedim(-1, 0))
             arrays[f"step{t}/rms/{i}"] = _np(st["rms"].movedim(-1, 0))
             if st["fac_vec_v"].numel():
@@ -176,7 +182,7 @@ def velo_case(R, name, shapes, n_steps, grad_scale, seed, num_steps, weight_deca
 
 # ------------------------------------------------------------------- AdafacLO
 def adafac_case(R, name, shapes, n_steps, grad_scale, seed, weight_decay, lr, cls="AdafacLO_naive", extra=None,
-                nan_at=()):
+                nan_at=(), dtype="float32"):
     """`extra`: further constructor arguments (ELO_naive: exp_mult, clip_grad, clip_norm, decays);
     `nan_at`: (step, tensor, flat index) triples where the gradient is NaN (ELO_naive zeroes them)."""
     torch.manual_seed(21)
@@ -184,18 +190,20 @@ def adafac_case(R, name, shapes, n_steps, grad_scale, seed, weight_decay, lr, cl
     tmp = tempfile.mkdtemp()
     net.save_pretrained(os.path.join(tmp, "mlp"))
     gen = torch.Generator().manual_seed(seed)
-    init = [torch.randn(s, generator=gen) * 0.5 for s in shapes]
+    dt = _DTYPES[dtype]
+    init = [(torch.randn(s, generator=gen) * 0.5).to(dt) for s in shapes]
     params = [torch.nn.Parameter(v.clone()) for v in init]
     extra = dict(extra or {})
     opt = R[cls](params, lr=lr, weight_decay=weight_decay, hf_key=os.path.join(tmp, "mlp"), **extra)
     arrays = {}
     _sd_arrays("net", net, arrays)
     meta = dict(kind="adafac" if cls == "AdafacLO_naive" else "elo", shapes=[list(s) for s in shapes],
-                n_steps=n_steps, seed=seed, weight_decay=weight_decay, lr=lr, grad_scale=grad_scale, extra=extra)
+                n_steps=n_steps, seed=seed, weight_decay=weight_decay, lr=lr, grad_scale=grad_scale, extra=extra,
+                dtype=dtype)
     for i, v in enumerate(init):
-        arrays[f"init/{i}"] = _np(v)
+        arrays[f"init/{i}"] = _np(v.float())
     for t in range(n_steps):
-        grads = [torch.randn(s, generator=gen) * grad_scale for s in shapes]
+        grads = [(torch.randn(s, generator=gen) * grad_scale).to(dt) for s in shapes]
         for tt, ti, fi in nan_at:
             if tt == t:
                 grads[ti].view(-1)[fi] = float("nan")
@@ -204,8 +212,8 @@ def adafac_case(R, name, shapes, n_steps, grad_scale, seed, weight_decay, lr, cl
         opt.step()
         for i, p in enumerate(params):
             st = opt.state[p]
-            arrays[f"grad{t}/{i}"] = _np(grads[i])
-            arrays[f"step{t}/param/{i}"] = _np(p)
+            arrays[f"grad{t}/{i}"] = _np(grads[i].float())
+            arrays[f"step{t}/param/{i}"] = _np(p.float())
             arrays[f"step{t}/exp_avg/{i}"] = _np(st["mom"].movedim(-1, 0))
             arrays[f"step{t}/exp_avg_sq/{i}"] = _np(st["rms"][..., 0])
             if st["fac_vec_v"].numel():
@@ -229,9 +237,24 @@ def ctor_checksums(R):
     _save("ctor_checksums", arrays, dict(kind="ctor", seed=1234))
 
 
+def stored_type_cases(R):
+    """The naive classes on 16-bit parameters, where they run: AdafacLO_naive, ELO_naive and VeLO_naive keep
+    float32 accumulators and let torch's type promotion decide the rest (g * g and the means over it are taken
+    in the 16-bit type).  ELO_CELO2_naive and CELO2_naive raise a dtype error on any non-float32 parameter,
+    and every naive class does on float64, so there is nothing to record for those."""
+    adafac_case(R, "adafac_bf16", [(20, 10), (20,), (5, 20), (6, 3, 4, 4), (16, 16), (64, 128)], 5, 0.3, 51,
+                weight_decay=0.01, lr=0.5, dtype="bfloat16")
+    adafac_case(R, "elo_f16", [(20, 10), (20,), (6, 3, 4, 4), (40, 128)], 5, 0.3, 52, weight_decay=0.05, lr=1e-2,
+                cls="ELO_naive", extra=dict(exp_mult=0.01, clip_grad=True, clip_norm=2.0), dtype="float16")
+    velo_case(R, "velo_bf16", [(20, 10), (20,), (5, 20), (6, 3, 4, 4), (64, 128)], 5, 0.3, 53, num_steps=40,
+              weight_decay=0.01, lr=1e-2, dtype="bfloat16")
+
+
 def main():
     R = _load_reference()
     torch.set_num_threads(8)
+    if "--stored-types-only" in sys.argv:
+        return stored_type_cases(R)
     # CELO2_naive (independent AdamW moments on 1-D tensors and is_embedding groups; CELO2_naive.py:263-283)
     celo2_case(R, "celo2_small", [(64, 32), (32, 64), (32,), (48, 24), (5,)], 8, 1.0, 12,
                dict(lr=1e-2, adam_lr_mult=3.0, weight_decay=0.02, adam_betas=(0.8, 0.9), adam_eps=1e-6,
@@ -273,6 +296,7 @@ def main():
     adafac_case(R, "adafac_small", [(20, 10), (20,), (5, 20), (6, 3, 4, 4), (16, 16)], 6, 0.3, 7,
                 weight_decay=0.0, lr=1.0)
     adafac_case(R, "adafac_small_wd", [(33, 17), (17,)], 5, 1e-3, 8, weight_decay=0.01, lr=0.5)
+    stored_type_cases(R)
 
 
 if __name__ == "__main__":

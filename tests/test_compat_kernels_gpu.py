@@ -186,3 +186,116 @@ def test_large_tensor_and_argument_errors():
     with pytest.raises(RuntimeError, match="dc / dr"):
         velo_cuda_kernel.velo_kernel_simple(g, p, m, v, rf, cf, fr, fc, sm, *ws, 0.03, 0.001, 0.001, 1e-6,
                                             0.0, 1, 1, 0)
+
+
+# ---------------------------------------------------------------- other element types
+# The reference's three functions dispatch on p.scalar_type() over float, double and half
+# (AT_DISPATCH_FLOATING_TYPES_AND_HALF, celo2_kernel.cu:314,328; learned_optimizer.cu:338,364;
+# velo_kernel.cu:405,427): every array but second_moment has that type, values are widened to float on load
+# and narrowed on store.  Expected results: the oracle's float32 functions on the widened inputs; outputs
+# rounded into the type (float64: rel 1e-5 / abs 1e-6; 16-bit: at most one spacing away, at most 0.3 % of the
+# values above 1e-3 not bit-identical); second_moment at rel 1e-5 as above.  bfloat16 is an addition.
+TYPES = [torch.float16, torch.bfloat16, torch.float64]
+
+
+def _as_stored(st, dtype):
+    """The case with every array rounded into `dtype`, plus the widened float32 view the kernels compute with."""
+    stored = {k: (v.to(dtype) if torch.is_tensor(v) else v) for k, v in st.items()}
+    wide = {k: (v.float() if torch.is_tensor(v) else v) for k, v in stored.items()}
+    return stored, wide
+
+
+def _check_stored(got, want32, dtype):
+    assert got.dtype == dtype
+    if dtype == torch.float64:
+        assert max_err(got.cpu(), want32, REL, ABS) <= 1.0
+        return
+    bits = {torch.bfloat16: 7, torch.float16: 10}[dtype]
+    g, w = got.cpu().reshape(-1), want32.to(dtype).reshape(-1)
+    spacing = torch.pow(2.0, torch.floor(torch.log2(w.double().abs().clamp_min(1e-3))) - bits)
+    assert float(((g.double() - w.double()).abs() / spacing).max()) <= 1.0
+    differ = int(((g != w) & (w.float().abs() > 1e-3)).sum())
+    assert differ <= max(1, int(g.numel() * 3e-3)), (differ, g.numel())
+
+
+@pytest.mark.parametrize("dtype", TYPES)
+@pytest.mark.parametrize("shape", [(48, 40), (333,)])
+def test_celo2_kernel_element_types(shape, dtype):
+    from pylo_amd.compat import celo2_cuda_kernel
+    from pylo_amd.models import CELO2MLP
+
+    torch.manual_seed(11)
+    sd = {k: v.to(dtype) for k, v in CELO2MLP().state_dict().items()}
+    sdw = {k: v.float() for k, v in sd.items()}
+    stored, st = _as_stored(_state(shape, 1, O.factored_dims), dtype)
+    dc, dr, vl = st["dims"]
+    if vl:
+        rs = torch.rsqrt(st["rms"] + 1e-8)
+        groups = [st["g"][None], torch.clamp(st["g"], -0.1, 0.1)[None], st["p"][None], st["mom"], st["rms"][None],
+                  st["mom"] * rs[None], rs[None], st["g"][None] * st["rf"], (st["g"] * rs)[None]]
+    else:
+        groups = O.celo2_feature_groups(st["p"], st["g"], st["mom"], st["rms"], st["fac_r"], st["fac_c"],
+                                        st["rf"], st["cf"])
+    axes = list(range(1, len(shape) + 1))
+    out = O.celo2_mlp([O.rms_normalize(x, axes, 1e-9) for x in groups], sdw)
+    want = out[..., 0] * torch.exp(out[..., 1] * 0.3)
+    g, p, m, v, fr, fc, rf, cf = _cuda(stored, "g", "p", "mom", "rms", "fac_r", "fac_c", "rf", "cf")
+    w_in = torch.cat([sd[f"w0.{i}"] for i in range(14)]).contiguous().cuda()
+    ws = [w_in] + [sd[k].contiguous().cuda() for k in ("b0", "dense_w.0", "dense_b.0", "dense_w.1", "dense_b.1")]
+    sm = torch.zeros(30, device="cuda")
+    step_out = torch.full(shape, float("nan"), device="cuda", dtype=dtype)
+    celo2_cuda_kernel.celo2_kernel(g, p, m, v, fr, fc, rf, cf, sm, *ws, step_out, 0.3, dc, dr, vl)
+    _check_stored(step_out, want, dtype)
+    _check_moment(sm, groups)
+
+
+@pytest.mark.parametrize("dtype", TYPES)
+@pytest.mark.parametrize("shape", [(40, 72), (6, 4, 3, 3)])
+def test_learned_optimizer_kernel_element_types(shape, dtype):
+    from pylo_amd.compat import cuda_lo
+    from pylo_amd.models import MetaMLP
+
+    torch.manual_seed(12)
+    sd = {k: v.to(dtype) for k, v in MetaMLP(39, 32, 1).state_dict().items()}
+    sdw = {k: v.float() for k, v in sd.items()}
+    stored, st = _as_stored(_state(shape, 2, O.factored_dims), dtype)
+    dc, dr, vl = st["dims"]
+    groups = O.adafac_feature_groups(st["p"], st["g"], st["mom"], st["rms"], st["fac_r"], st["fac_c"], st["rf"], st["cf"])
+    step, lr, step_mult, exp_mult = 7.0, 0.5, 0.01, 0.001
+    out = O.adafac_element_mlp(groups, O.tanh_time_embedding(step), sdw)
+    want = st["p"] - lr * (out[..., 0] * torch.exp(out[..., 1] * exp_mult) * step_mult)
+    g, p, m, v, fr, fc, rf, cf = _cuda(stored, "g", "p", "mom", "rms", "fac_r", "fac_c", "rf", "cf")
+    ws = [sd[k].contiguous().cuda() for k in ("network.input.weight", "network.input.bias", "network.linear_0.weight",
+                                              "network.linear_0.bias", "network.output.weight", "network.output.bias")]
+    sm = torch.zeros(28, device="cuda")
+    cuda_lo.learned_optimizer_kernel(g, p, m, v, fr, fc, rf, cf, sm, *ws, lr, step_mult, exp_mult, 1e-6, step, 0.0,
+                                     dc, dr, vl)
+    _check_stored(p, want, dtype)
+    _check_moment(sm, groups)
+
+
+@pytest.mark.parametrize("dtype", TYPES)
+@pytest.mark.parametrize("shape,wd", [((40, 72), 0.02), ((5, 3, 7), 0.1)])
+def test_velo_kernel_simple_element_types(shape, wd, dtype):
+    from pylo_amd.compat import velo_cuda_kernel
+
+    gen = torch.Generator().manual_seed(13)
+    weights = [(torch.randn(s, generator=gen) * sc).to(dtype) for s, sc in
+               (((4, 30), 0.3), ((4,), 0.1), ((4, 4), 0.5), ((4,), 0.1), ((3, 4), 0.5), ((3,), 0.1))]
+    stored, st = _as_stored(_state(shape, 3, O.factored_dims_velo), dtype)
+    dc, dr, vl = st["dims"]
+    groups = O.velo_feature_groups(st["p"], st["g"], st["mom"], st["rms"], st["fac_r"], st["fac_c"], st["rf"], st["cf"])
+    lr, step_mult, exp_mult = 0.03, 0.001, 0.001
+    out = O.velo_element_mlp(groups, [w.float() for w in weights])
+    scale = torch.sqrt(torch.mean(st["p"] ** 2) + 1e-9)
+    want = st["p"] - lr * (scale * (out[..., 0] * torch.exp(out[..., 1] * exp_mult) * step_mult))
+    want = want - wd * lr * want
+    g, p, m, v, fr, fc, rf, cf = _cuda(stored, "g", "p", "mom", "rms", "fac_r", "fac_c", "rf", "cf")
+    sm = torch.zeros(30, device="cuda")
+    velo_cuda_kernel.velo_kernel_simple(g, p, m, v, rf, cf, fr, fc, sm, *[w.cuda() for w in weights], lr, step_mult,
+                                        exp_mult, 1e-6, wd, dc, dr, vl)
+    _check_stored(p, want, dtype)
+    _check_moment(sm, groups)
+    with pytest.raises(TypeError, match="second_moment is float32"):      # one array of another type than the parameter
+        velo_cuda_kernel.velo_kernel_simple(g.float(), p, m, v, rf, cf, fr, fc, sm, *[w.cuda() for w in weights], lr,
+                                            step_mult, exp_mult, 1e-6, wd, dc, dr, vl)

@@ -138,6 +138,30 @@ def ns_flops_executed(shapes, iters=5, tile=128):
     return total
 
 
+def whole_step_object(whole_ms, finish_ms, n_params, flops, flops_exec):
+    """The matrix-pipe part of the step against the peak of the pipe it runs on.  By default the products run
+    on the bf16 matrix instructions with every fp32 operand split into three bf16 planes: six bf16 products
+    per fp32 product, so the executed work is 6 x the fp32 FLOPs against the 2.5 PFLOP/s of dense bf16;
+    PYLO_MI355_NS_F32=1 runs them on the fp32 matrix instructions (157.3 TFLOP/s).  `achieved` counts the FLOPs
+    the kernels execute (the symmetric halves they skip earn nothing); by the reference's full fp32 products the
+    same time is `nominal_fp32_TFLOPs`."""
+    f32 = os.environ.get("PYLO_MI355_NS_F32") == "1"
+    t = finish_ms * 1e-3
+    mult, peak = (1.0, 157.3) if f32 else (6.0, 2500.0)
+    return {
+        "ms": whole_ms, "params_per_sec": n_params / (whole_ms * 1e-3), "finish_ms": finish_ms,
+        "newton_schulz_TFLOP": flops / 1e12, "newton_schulz_TFLOP_executed": flops_exec / 1e12,
+        "roofline": {"bound": "mfma",
+                     "kernel": ("k_ns_gemm (fp32 matrix instructions)" if f32 else
+                                "k_ns_bf_gemm (bf16 matrix instructions, 6 products per fp32 product)")
+                               + " + finishing pass",
+                     "achieved": mult * flops_exec / t / 1e12, "peak": peak, "unit": "TFLOP/s",
+                     "frac": mult * flops_exec / t / 1e12 / peak,
+                     "fp32_equivalent_TFLOPs": flops_exec / t / 1e12,
+                     "nominal_fp32_TFLOPs": flops / t / 1e12, "traffic": None},
+    }
+
+
 def traffic_from_profile(fname, kernel):
     """HBM bytes per launch of `kernel` as the counter summary under profiles/ states them
     (a line `traffic_bytes_per_launch <kernel> = <bytes>`); None when the file does not hold it."""
@@ -281,18 +305,8 @@ def main():
             "launch_ms": {nm: float(v) for nm, v in zip(names, mean)},
         },
         "hbm_roofline_frac_fused_path": bytes_fused / (fused_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        # Newton-Schulz + normalise + apply: fp32 matrix products
-        "whole_step": {
-            "ms": whole_ms, "params_per_sec": n_params / (whole_ms * 1e-3),
-            "finish_ms": finish_ms, "newton_schulz_TFLOP": flops / 1e12,
-            "newton_schulz_TFLOP_executed": flops_exec / 1e12,
-            # `achieved` counts the FLOPs the kernels execute (the symmetric halves they skip earn nothing);
-            # by the reference's full products the same time is `nominal_TFLOPs`
-            "roofline": {"bound": "mfma", "kernel": "k_ns_gemm (Newton-Schulz products) + finishing pass",
-                         "achieved": flops_exec / (finish_ms * 1e-3) / 1e12,
-                         "peak": 157.3, "unit": "TFLOP/s", "frac": flops_exec / (finish_ms * 1e-3) / 1e12 / 157.3,
-                         "nominal_TFLOPs": flops / (finish_ms * 1e-3) / 1e12, "traffic": None},
-        },
+        # Newton-Schulz + normalise + apply
+        "whole_step": whole_step_object(whole_ms, finish_ms, n_params, flops, flops_exec),
         "roofline": {"bound": "hbm", "kernel": elem, "achieved": elem_gbs, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": elem_gbs / HBM_PEAK_GBS,
                      "traffic": traffic_from_profile("celo2_fused_step_gpt2s_hbm_traffic.txt", elem) if a.workload == "gpt2s" else None,

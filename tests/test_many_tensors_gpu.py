@@ -1,9 +1,8 @@
-"""Many-tensor and odd-shape stress (BASELINE config 5): 1500 tensors with sizes drawn log-uniform
+"""Many-tensor and odd-shape stress (BASELINE config 5): 3000 tensors with sizes drawn log-uniform
 in [1, 65536] elements, mixing 1-D and 2-D shapes with non-power-of-two dims (37x4099 among them),
 plus one 32000x4096 embedding; heavy-tailed Student-t (df = 3) gradients scaled by 1e-3.  Checks the
 multi-tensor launch tables and every per-tensor reduction against the oracle evaluated in fp64 on the
-GPU (tolerance rel 1e-5 / abs 1e-6).  Half of config 5's 3000 tensors keep the oracle's Python loop
-within a minute; the launch-table code does not depend on the count.
+GPU (tolerance rel 1e-5 / abs 1e-6).
 """
 
 import copy
@@ -49,7 +48,7 @@ def test_celo2_many_tensors():
 
     torch.manual_seed(1)
     net = CELO2MLP()
-    shapes = _shapes(1500, 11, (32000, 4096))
+    shapes = _shapes(3000, 11, (32000, 4096))
     init, grads = _inputs(shapes, 12, 2)
     ref = [v.double() for v in init]
     gpu = [torch.nn.Parameter(v.clone()) for v in init]
@@ -87,20 +86,23 @@ def test_velo_many_tensors():
 
     torch.manual_seed(2)
     rnn, mlp = VeLORNN(), VeLOMLP()
-    shapes = _shapes(1500, 21, (32000, 4096))
+    shapes = _shapes(3000, 21, (32000, 4096))
     init, grads = _inputs(shapes, 22, 2)
     ref = [v.double() for v in init]
     ref32 = [v.clone() for v in init]
     gpu = [torch.nn.Parameter(v.clone()) for v in init]
     kw = dict(lr=1e-2, num_steps=100, weight_decay=1e-4)
-    # The oracle twice: evaluated in fp64 and in the reference's own fp32.  With Student-t (df = 3)
-    # gradients the fp32 evaluation itself leaves the fp64 one by up to 1.4 tolerances on the largest
-    # updates of the 131 M-element embedding (57 elements); a value passes when it is within the
-    # tolerance of either evaluation.
+    # The oracle twice: in the reference's own fp32 arithmetic, and in fp64 to say how far that arithmetic itself
+    # is from the exact value.  With Student-t (df = 3) gradients the fp32 evaluation leaves the fp64 one by up
+    # to 1.4 tolerances on the largest updates of the 131 M-element embedding (its fp32 means over 131 M
+    # elements), where the HIP path, whose reductions run in fp64 across blocks, stays with the fp64 value.
+    # One criterion for every value: |hip - fp64| <= tolerance + |fp32 - fp64|, i.e. the tolerance around the
+    # exact value, widened at each element by the error the reference's arithmetic makes there.  The error
+    # against the fp32 evaluation alone and against the fp64 evaluation alone are printed.
     orc = O.VeloOracle(ref, rnn.state_dict(), mlp.state_dict(), device="cuda", **kw).double_()
     orc32 = O.VeloOracle(ref32, rnn.state_dict(), mlp.state_dict(), device="cuda", **kw)
     opt = VeLO_CUDA(gpu, rnn=copy.deepcopy(rnn), mlp=copy.deepcopy(mlp), **kw)
-    worst64 = worst = 0.0
+    worst64 = worst32 = worst = 0.0
     for t in range(2):
         loss = torch.tensor(2.0 - 0.3 * t, device="cuda")
         for p, g in zip(gpu, grads[t]):
@@ -117,10 +119,14 @@ def test_velo_many_tensors():
                 if k in so:
                     checks.append((f"{k}{i}", st[k], so[k], s32[k]))
         for tag, got, want, want32 in checks:
-            e = max_err(got, want, REL, ABS)
-            worst64 = max(worst64, e)
-            if e > 1.0:
-                e = min(e, max_err(got, want32, REL, ABS))
+            g64, w64, w32 = (x.detach().double().reshape(-1) for x in (got, want, want32))
+            if g64.numel() == 0:
+                continue
+            own = (w32 - w64).abs()
+            e = float(((g64 - w64).abs() / (ABS + REL * w64.abs() + own)).max())
             worst = max(worst, e)
+            worst64 = max(worst64, max_err(got, want, REL, ABS))
+            worst32 = max(worst32, max_err(got, want32, REL, ABS))
             assert e <= 1.0, (t, tag, e)
-    print("velo many tensors worst err/tol", worst, "(against the fp64 evaluation alone:", worst64, ")")
+    print("velo many tensors worst err/tol", worst, "(against the fp64 evaluation alone:", worst64,
+          ", against the fp32 evaluation alone:", worst32, ")")

@@ -111,6 +111,9 @@ def rms_normalize(x: torch.Tensor, dims, eps: float = 1e-9) -> torch.Tensor:
     return x * torch.rsqrt(eps + torch.mean(x * x, dim=dims, keepdim=True))
 
 
+_WATCH_ALL = 512   # parameter lists up to this length have every state tensor checked for replacement each step
+
+
 def _apply(p, step, weight_decay, lr):
     """p <- p - lr (step + wd p) in fp32 on the widened parameter, rounded into p's own dtype
     (what the library's update kernel does for the tensors it finishes itself)."""
@@ -374,6 +377,8 @@ class ELO_CELO2_CUDA(Optimizer):
         for st, key, t in fast["alive"]:
             if st.get(key) is not t:      # a state tensor was replaced: the cached pointers are stale
                 return None
+        if fast["routing"] != [(g["use_adamw_for_1d"], g["is_embedding"]) for g in groups]:
+            return None                   # a group changed which branch its tensors take: new plan
         if not self.capturable:
             for group in groups:
                 group["step"] = group.get("step", 0) + 1
@@ -451,14 +456,18 @@ class ELO_CELO2_CUDA(Optimizer):
         self._launch_step()
         if not keep and all(p.grad is not None for _, p, _a in tensors):
             index = {id(g): i for i, g in enumerate(self.param_groups)}
-            # the cached rows point into the state tensors: hold them, and notice a cleared state
-            # one (state, key, tensor) per parameter, its first state tensor: replacing a parameter's
-            # state replaces that one too, and a walk over every tensor costs milliseconds with
-            # thousands of parameters
-            alive = [(self.state[p],) + next(((k, t) for k, t in self.state[p].items() if torch.is_tensor(t)), (None, None))
-                     for _, p, _a in tensors]
+            # the cached rows point into the state tensors: hold them, and notice a replaced or cleared one.
+            # Every state tensor of every parameter is watched (a few hundred identity checks a step for a
+            # transformer's parameter list); beyond _WATCH_ALL parameters only the first state tensor of each
+            # is, because the walk then costs milliseconds a step: there, state tensors must be updated in place
+            # or through load_state_dict().
+            def watched(state):
+                items = [(k, t) for k, t in state.items() if torch.is_tensor(t) and t.dim() > 0]
+                return items if len(tensors) <= _WATCH_ALL else items[:1]
+            alive = [(self.state[p], k, t) for _, p, _a in tensors for k, t in watched(self.state[p])]
             self._fast = dict(tensors=tensors, params=[p for _, p, _a in tensors], n_groups=len(self.param_groups),
                               n_state=len(self.state), alive=alive,
+                              routing=[(g["use_adamw_for_1d"], g["is_embedding"]) for g in self.param_groups],
                               gidx=np.asarray([index[id(g)] for g, _p, _a in tensors], dtype=np.int64),
                               adam=np.asarray([a for _g, _p, a in tensors], dtype=bool))
         del keep

@@ -328,9 +328,9 @@ class VeLO_CUDA(Optimizer):
                     fast = self._fast = None
                     break
         if fast is not None:
-            for state, mom, rms in fast["alive"]:
+            for state, key, t in fast["alive"]:
                 # a state tensor was replaced: the cached pointers are stale (and so are the carried sums)
-                if state.get("mom") is not mom or state.get("rms") is not rms:
+                if state.get(key) is not t:
                     fast = self._fast = None
                     break
             else:
@@ -385,10 +385,12 @@ class VeLO_CUDA(Optimizer):
                 args[k] = v
             args["group"] = grp
             if not keep:
-                # the two state tensors whose sums are carried from step to step, per parameter (a walk over
-                # every state tensor costs milliseconds with thousands of parameters; replacing a parameter's
-                # whole state replaces these too)
-                alive = [(self.state[p], self.state[p]["mom"], self.state[p]["rms"]) for _, _, p in tensors]
+                # every accumulator of every parameter is watched for replacement (a few hundred identity checks
+                # a step); beyond 512 parameters only the two whose sums are carried from step to step, because
+                # the walk then costs milliseconds a step: there, the factored accumulators must be updated in
+                # place or through load_state_dict()
+                keys = ("mom", "rms", "fac_vec_row", "fac_vec_col", "fac_vec_v") if n <= 512 else ("mom", "rms")
+                alive = [(self.state[p], k, self.state[p][k]) for _, _, p in tensors for k in keys]
                 self._fast = dict(key=self._plan_key, n_state=len(self.state), alive=alive,
                                   params=[p for _, _, p in tensors], versions=[p._version for _, _, p in tensors],
                                   gidx=np.asarray(grp, dtype=np.int64))

@@ -317,3 +317,32 @@ def test_replaced_state_tensor_is_picked_up():
     for x, y in zip(a, b):
         assert torch.equal(x, y)
     assert all(bool(torch.isfinite(v).all()) for p in b for v in ob.state[p].values() if torch.is_tensor(v))
+
+
+def test_replaced_state_tensors_are_noticed():
+    """The step caches device pointers of the state tensors between calls; a state tensor swapped for another
+    object (any of them, not only the first) must be picked up by the next step, which then updates the new
+    tensor and leaves the orphaned one alone."""
+    net = _net()
+    shapes = [(64, 32), (32,), (48, 24)]
+    init, gen = _mk(shapes, 9)
+    orc, opt, cpu, gpu = _pair(shapes, init, net, dict(lr=1e-2))
+    for t in range(4):
+        grads = [torch.randn(s, generator=gen) * 0.3 for s in shapes]
+        for p, g in zip(gpu, grads):
+            p.grad = g.cuda()
+        orphans = []
+        if t == 2:      # after two steps on the fast path
+            for p in gpu:
+                st = opt.state[p]
+                for k in ("rms", "fac_c") if "fac_c" in st else ("rms",):
+                    orphans.append((st[k], st[k].clone()))
+                    st[k] = st[k].clone()
+        orc.step(grads)
+        opt.step()
+        torch.cuda.synchronize()
+        _check_states(opt, orc, gpu, t, "after swap" if t >= 2 else "")
+        for old, before in orphans:
+            assert torch.equal(old, before)
+        for pc, pg in zip(cpu, gpu):
+            assert max_err(pg, pc, REL, ABS) <= 1.0, t

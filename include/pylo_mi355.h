@@ -140,24 +140,6 @@ int pylo_mi355_plan_destroy(PyloPlan* plan);
 int pylo_mi355_plan_num_launches(const PyloPlan* plan);
 int pylo_mi355_plan_factored_dims(const PyloPlan* plan, int tensor, int* dc, int* dr);
 
-/* Optional per-launch timing, for benchmarks (no counterpart in the reference).  Between begin and
-   end every *_step call records one HIP event before its first launch and one after each launch,
-   on the call's stream, for at most `max_steps` calls.  end synchronises the last event and
-   writes steps x num_launches durations in milliseconds (row-major) into ms_out. */
-int pylo_mi355_plan_timing_begin(PyloPlan* plan, int max_steps);
-int pylo_mi355_plan_timing_end(PyloPlan* plan, float* ms_out, int capacity, int* steps_out);
-
-/* Names of the launches of one step, in launch order (static strings). */
-const char* pylo_mi355_plan_launch_name(const PyloPlan* plan, int launch);
-
-/* Bare streaming kernel, for benchmarks (no counterpart in the reference): per element, `reads` arrays of n
-   floats are read (in[r * n + i]) and `writes` arrays written (out[w * n + i]), 16 bytes per lane and access,
-   nothing computed.  It measures what the memory system delivers for an access mix -- 6 reads and 5 writes
-   is the apply pass of the ELO-CELO2 step, 6 reads its statistics pass.  reads in {1, 6}, writes in
-   {0, 1, 5}; n a multiple of 4; nontemporal != 0 uses non-temporal loads and stores. */
-int pylo_mi355_stream_probe(const float* in, float* out, size_t n, int reads, int writes, int nontemporal,
-                            void* stream);
-
 /* ---- Steps that a HIP graph can replay.  No counterpart in the reference, whose step() waits for
  * the device once per step or per tensor (ELO_CELO2_cuda.py:154-162, velo_cuda.py:747) and counts
  * steps on the host (ELO_CELO2_cuda.py:224, AdafacLO_cuda.py:304-305). ------------------------- */

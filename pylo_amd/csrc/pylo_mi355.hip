@@ -33,6 +33,7 @@
 #include "k_ns_bf.h"
 #include "k_cast.h"
 #include "pylo_common.h"
+#include "pylo_mi355_bench.h"
 
 // =============================================================================================
 // Host side: plan construction and the C ABI

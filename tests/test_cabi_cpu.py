@@ -1,4 +1,5 @@
-"""The C-ABI library loads without a GPU and exports every symbol include/pylo_mi355.h declares;
+"""The C-ABI library loads without a GPU and exports every symbol include/*.h declare (the boundary,
+pylo_mi355.h, and the measurement instrumentation, pylo_mi355_bench.h);
 host-only entry points (plan sizing, argument checks, error reporting) behave as documented."""
 
 import ctypes as C
@@ -8,11 +9,11 @@ import re
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "pylo_mi355.h")
+HEADERS = [os.path.join(ROOT, "include", n) for n in ("pylo_mi355.h", "pylo_mi355_bench.h")]
 
 
 def _declared():
-    text = open(HEADER).read()
+    text = "".join(open(h).read() for h in HEADERS)
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(pylo_mi355_\w+)\s*\(", text)))
 

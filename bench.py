@@ -420,11 +420,23 @@ def other_workload(workload, steps, warmup):
             "traffic": traffic_from_profile("velo_fused_step_vitb16_kernel_trace_and_traffic.txt", apply_kernel) if workload == "vit_velo" else None,
             "algorithmic_bytes_per_launch": n2d * b_elem + n1d * b_vec, "avg_launch_ms": float(mean[k])}
     if workload == "llama_adafac":
-        # the 16 -> 32 -> 32 -> 2 element MLP: 1 600 FMAs per element of a >= 2-D tensor, fp32 matrix pipe
-        tflops = n2d * 3200.0 / (float(mean[k]) * 1e-3) / 1e12
-        roof = {"bound": "mfma", "kernel": "k_adafac_apply_tile", "achieved": tflops, "peak": 157.3,
-                "unit": "TFLOP/s", "frac": tflops / 157.3, "traffic": None, "avg_launch_ms": float(mean[k]),
-                "hbm_GBps": apply_gbs}
+        # The 16 -> 32 -> 32 -> 2 element MLP: 1 600 FMAs per element of a >= 2-D tensor.  By default its two
+        # wide layers (1 536 FMAs) run on the bf16 matrix instructions with three-plane operands, six bf16
+        # products per fp32 product, and the kernel is bound by what one SIMD can issue: matrix and vector
+        # instructions do not overlap on it (the splitting of the activations is vector work);
+        # PYLO_MI355_ADAFAC_F32=1 runs the layers on the fp32 matrix instructions.
+        t = float(mean[k]) * 1e-3
+        f32 = os.environ.get("PYLO_MI355_ADAFAC_F32") == "1"
+        fp32_tflops = n2d * 3200.0 / t / 1e12
+        if f32:
+            roof = {"bound": "mfma", "kernel": "k_adafac_apply_tile (fp32 matrix instructions)", "achieved": fp32_tflops,
+                    "peak": 157.3, "unit": "TFLOP/s", "frac": fp32_tflops / 157.3}
+        else:
+            bf = n2d * 6 * 1536 * 2.0 / t / 1e12
+            roof = {"bound": "mfma", "kernel": "k_adafac_apply_tile (bf16 matrix instructions, 6 products per fp32 product)",
+                    "achieved": bf, "peak": 2500.0, "unit": "TFLOP/s", "frac": bf / 2500.0,
+                    "fp32_equivalent_TFLOPs": fp32_tflops, "fp32_matrix_peak_TFLOPs": 157.3}
+        roof.update({"traffic": None, "avg_launch_ms": float(mean[k]), "hbm_GBps": apply_gbs})
     out = {
         "metric": "params_updated_per_sec (fused step, C-ABI call)", "value": n_params / (fused_ms * 1e-3),
         "unit": "params/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": fused_ms,

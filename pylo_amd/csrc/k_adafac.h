@@ -467,6 +467,215 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
   }
 }
 
+// ---- the same pass with the element MLP on the bf16 matrix instructions at fp32 accuracy ----------------
+// An fp32 number is the exact sum of three bf16 numbers (8 + 8 + 8 significand bits; taken by truncation:
+// h = x & 0xffff0000, m = (x - h) & 0xffff0000, l = x - h - m, every step exact), and a product of two such
+// sums is, up to 2^-25 of itself, the six products h h, h m, m h, m m, h l, l h, each exact in fp32.  One
+// v_mfma_f32_32x32x16_bf16 does sixteen times the multiply-adds of v_mfma_f32_16x16x4_f32 in the same 32
+// cycles, so six of them per fp32 product leave 36 matrix instructions per row of 64 elements where the
+// fp32 instructions need 96; the price is vector work (this SIMD executes either kind, never both at once):
+// splitting the 16 features and the 2 x 16 hidden values a lane holds costs 5.5 instructions a value.
+//
+// Layouts (lane = 32 half + e): units are the M dimension, elements the N dimension, inputs the K
+// dimension.  A operand: lane holds inputs 8 half .. 8 half + 7 of unit e.  B operand: lane holds inputs
+// 8 half .. + 7 of element e of the group (two groups of 32 elements per wave row; a lane owns element
+// 32 half + e, i.e. the lanes of one half own one group).  D: lane holds units 8 j + 4 half + i (j, i = 0..3)
+// of element e.  Lanes e and e + 32 hold complementary halves of what the other needs, both for the features
+// (own element, all 16 inputs) and for the hidden values (D -> B of the next layer): one
+// v_permlane32_swap per register (lanes 32..63 of the first operand change places with lanes 0..31 of the
+// second) puts everything where the next matrix instruction reads it; nothing goes through LDS.
+typedef __bf16 abf16x8 __attribute__((ext_vector_type(8)));
+typedef float av16f __attribute__((ext_vector_type(16)));
+typedef unsigned int au32x4 __attribute__((ext_vector_type(4)));
+
+struct Bf3 { unsigned h, m, l; };   // fp32 bit patterns whose upper halves are the three bf16 planes
+
+__device__ __forceinline__ Bf3 bf3_split(float x) {
+  Bf3 r;
+  r.h = __float_as_uint(x) & 0xffff0000u;
+  const float r1 = x - __uint_as_float(r.h);
+  r.m = __float_as_uint(r1) & 0xffff0000u;
+  r.l = __float_as_uint(r1 - __uint_as_float(r.m));   // at most 8 significant bits left: its lower half is zero
+  return r;
+}
+// upper halves of two fp32 patterns as one dword, `lo` in the lower half
+__device__ __forceinline__ unsigned bf_pack(unsigned lo, unsigned hi) { return __builtin_amdgcn_perm(hi, lo, 0x07060302u); }
+
+// eight values (consecutive inputs of a matrix operand) as three planes of eight bf16
+__device__ __forceinline__ void bf3_pack8(const float (&x)[8], au32x4 (&pl)[3]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const Bf3 a = bf3_split(x[2 * i]), b = bf3_split(x[2 * i + 1]);
+    pl[0][i] = bf_pack(a.h, b.h);
+    pl[1][i] = bf_pack(a.m, b.m);
+    pl[2][i] = bf_pack(a.l, b.l);
+  }
+}
+
+// lanes 32..63 of `a` change places with lanes 0..31 of `b`
+__device__ __forceinline__ void half_swap(unsigned& a, unsigned& b) {
+  const auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+  a = r[0];
+  b = r[1];
+}
+
+// acc += W (three planes) x act (three planes), smallest terms first
+__device__ __forceinline__ av16f bf3_mfma(const au32x4 (&w)[3], const au32x4 (&x)[3], av16f acc) {
+  constexpr int pw[6] = {2, 0, 1, 1, 0, 0}, px[6] = {0, 2, 1, 0, 1, 0};
+#pragma unroll
+  for (int t = 0; t < 6; ++t)
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(abf16x8, w[pw[t]]), __builtin_bit_cast(abf16x8, x[px[t]]),
+                                                  acc, 0, 0, 0);
+  return acc;
+}
+
+__device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloTensorArgs& a, int task,
+                                                     const EmaConsts& e, const float* __restrict__ fac_tab,
+                                                     const float* __restrict__ term_tab, const float* wfold_t,
+                                                     const float* net) {
+  const TileTask tk(d, task, d.atile_nct, 1);
+  const int lane = threadIdx.x & 63, half = lane >> 5, el = lane & 31;
+  // A operands: first layer (unit el, inputs 8 half ..), hidden layer per reduction step s (inputs 16 s + 8 half ..)
+  au32x4 w1[3], w2[2][3];
+  {
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = *(const gfloat*)(wfold_t + adafac_elem_row(8 * half + i) * kAH + el);
+    bf3_pack8(x, w1);
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = *(const gfloat*)(net + kAWH + (16 * s + 8 * half + i) * kAH + el);
+      bf3_pack8(x, w2[s]);
+    }
+  }
+  // what belongs to the units this lane holds in D: hidden bias, output weights
+  av16f bh;
+  float wo[16][2];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int unit = 8 * (r >> 2) + 4 * half + (r & 3);
+    bh[r] = *(const gfloat*)(net + kABH + unit);
+    wo[r][0] = *(const gfloat*)(net + kAWO + unit * 2 + 0);
+    wo[r][1] = *(const gfloat*)(net + kAWO + unit * 2 + 1);
+  }
+  const cfloat* nw = launder(net);
+  const float bo0 = nw[kABO + 0], bo1 = nw[kABO + 1];
+  const float exp_scale = a.exp_mult * 1.44269504088896341f;
+  float fb[4];
+  load_vec_o<4>(fac_tab + d.fac_off[1], tk.col * 16u, fb);
+  // column terms of element e of group g (column: the wave's first + 32 g + e), units 8 j + 4 half ..: one
+  // offset per lane, immediates per (g, j); row terms likewise from the row's table entry
+  const float* tcol = term_tab + d.term_off[1];
+  const unsigned tcol_off = ((tk.col - lane + el) * kAH + 4 * half) * 4u;
+  const unsigned trow_off = 4 * half * 4u;
+  const unsigned lo = lane * 4u;
+  const float* g = a.grad + tk.first;
+  float *p = a.param + tk.first, *m0 = a.mom + tk.first, *m1 = a.mom + d.n + tk.first,
+        *m2 = a.mom + 2 * d.n + tk.first, *rms = a.rms + tk.first;
+  const float* fr = fac_tab + d.fac_off[0] + (size_t)tk.r0 * 4;
+  const float* tr = term_tab + d.term_off[0] + (size_t)tk.r0 * kAH;
+  for (int r = tk.r0; r < tk.r1; ++r) {
+    float xg[1], xp[1], x0[1], x1[1], x2[1], xr_[1], fa[4];
+    load_vec_nt<1>(g, lo, xg);
+    load_vec_nt<1>(p, lo, xp);
+    load_vec_nt<1>(m0, lo, x0);
+    load_vec_nt<1>(m1, lo, x1);
+    load_vec_nt<1>(m2, lo, x2);
+    load_vec_nt<1>(rms, lo, xr_);
+    load_uniform<4>(fr, fa);
+    float ta[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) load_vec_o<4>(tr + 8 * j, trow_off, ta[j]);
+    const float gg = cond_grad(xg[0], d.gscale, a.clip_val, d.nan0);
+    float m[3] = {x0[0], x1[0], x2[0]};
+    ema_update(e, gg, m, xr_[0]);
+    x0[0] = m[0]; x1[0] = m[1]; x2[0] = m[2];
+    store_vec_nt<1>(m0, lo, x0);
+    store_vec_nt<1>(m1, lo, x1);
+    store_vec_nt<1>(m2, lo, x2);
+    store_vec_nt<1>(rms, lo, xr_);
+    const float rfcf[3] = {fa[0] * fb[0], fa[1] * fb[1], fa[2] * fb[2]};
+    float f18[kNStat];
+    lo_features(gg, xp[0], m, xr_[0], rfcf, 1e-6f, f18);
+    const float flo[8] = {f18[0], f18[2], f18[3], f18[4], f18[5], f18[6], f18[7], f18[8]};
+    const float fhi[8] = {f18[9], f18[10], f18[11], f18[12], f18[13], f18[15], f18[16], f18[17]};
+    // B operands of the first layer: after the swap xb[0] serves group 0 (lanes 0..31: their own inputs 0..7,
+    // lanes 32..63: inputs 8..15 of the element 32 lanes below), xb[1] group 1
+    au32x4 xb[2][3];
+    bf3_pack8(flo, xb[0]);
+    bf3_pack8(fhi, xb[1]);
+#pragma unroll
+    for (int q = 0; q < 3; ++q)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        unsigned u = xb[0][q][i], v = xb[1][q][i];
+        half_swap(u, v);
+        xb[0][q][i] = u;
+        xb[1][q][i] = v;
+      }
+    float part[2][2];
+#pragma unroll
+    for (int gq = 0; gq < 2; ++gq) {
+      av16f h;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float tb[4];
+        load_vec_o<4>(tcol + (32 * gq) * kAH + 8 * j, tcol_off, tb);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) h[4 * j + i] = ta[j][i] + tb[i];
+      }
+      h = bf3_mfma(w1, xb[gq], h);
+      // hidden values of the units this lane holds -> planes, four units (two dwords) per block j
+      unsigned hp[3][4][2];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const Bf3 u0 = bf3_split(relu(h[4 * j + 2 * i])), u1 = bf3_split(relu(h[4 * j + 2 * i + 1]));
+          hp[0][j][i] = bf_pack(u0.h, u1.h);
+          hp[1][j][i] = bf_pack(u0.m, u1.m);
+          hp[2][j][i] = bf_pack(u0.l, u1.l);
+        }
+      // blocks (0, 1) and (2, 3) trade halves: afterwards lanes 0..31 hold units 16 s + 0..7, lanes 32..63
+      // units 16 s + 8..15 of their element, in order
+      av16f g2 = bh;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        au32x4 hb[3];
+#pragma unroll
+        for (int q = 0; q < 3; ++q) {
+#pragma unroll
+          for (int i = 0; i < 2; ++i) half_swap(hp[q][2 * s2][i], hp[q][2 * s2 + 1][i]);
+          hb[q] = au32x4{hp[q][2 * s2][0], hp[q][2 * s2][1], hp[q][2 * s2 + 1][0], hp[q][2 * s2 + 1][1]};
+        }
+        g2 = bf3_mfma(w2[s2], hb, g2);
+      }
+      float p0 = 0.0f, p1 = 0.0f;
+#pragma unroll
+      for (int r2 = 0; r2 < 16; ++r2) {
+        const float gv = relu(g2[r2]);
+        p0 = fmaf(gv, wo[r2][0], p0);
+        p1 = fmaf(gv, wo[r2][1], p1);
+      }
+      part[gq][0] = p0;
+      part[gq][1] = p1;
+    }
+    // a lane's element belongs to group `half`; its other 16 units sit 32 lanes away
+    unsigned a0 = __float_as_uint(part[0][0]), b0 = __float_as_uint(part[1][0]);
+    unsigned a1 = __float_as_uint(part[0][1]), b1 = __float_as_uint(part[1][1]);
+    half_swap(a0, b0);
+    half_swap(a1, b1);
+    const float o0 = (__uint_as_float(a0) + __uint_as_float(b0)) + bo0;
+    const float o1 = (__uint_as_float(a1) + __uint_as_float(b1)) + bo1;
+    float pn[1];
+    pn[0] = adafac_update(d, a, o0 * __builtin_amdgcn_exp2f(o1 * exp_scale), xp[0]);
+    store_vec_o<1>(p, lo, pn);
+    g += d.C0; p += d.C0; m0 += d.C0; m1 += d.C0; m2 += d.C0; rms += d.C0;
+    fr += 4; tr += kAH;
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void k_adafac_apply(const TDesc* __restrict__ descs,
                                                            const PyloTensorArgs* __restrict__ dyn,
                                                            const Item* __restrict__ items,
@@ -490,8 +699,10 @@ __global__ __launch_bounds__(kThreads) void k_adafac_apply(const TDesc* __restri
   else adafac_apply_vec(d, a, base, count, e, dec, w, net, bias_eff + (size_t)it.tensor * kAH);
 }
 
-// The apply pass for tensors walked column-resident (items hold four wave tasks each).
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PYLO_ADAFAC_WAVES)))
+// The apply pass for tensors walked column-resident (items hold four wave tasks each).  BF: the element MLP on
+// the bf16 matrix instructions (three-plane operands), else on the fp32 ones.
+template <bool BF>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(BF ? 2 : PYLO_ADAFAC_WAVES)))
 void k_adafac_apply_tile(const TDesc* __restrict__ descs, const PyloTensorArgs* __restrict__ dyn,
                          const Item* __restrict__ items, const float* __restrict__ fac_tab,
                          const float* __restrict__ term_tab, PyloDecays dec, const float* __restrict__ wfold,
@@ -501,12 +712,14 @@ void k_adafac_apply_tile(const TDesc* __restrict__ descs, const PyloTensorArgs* 
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
   set_grad_scale(d, a, gl);
-  __shared__ float xch[kWaves][16 * kXPitch];
+  __shared__ float xch[BF ? 1 : kWaves][BF ? 1 : 16 * kXPitch];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int task = it.a * 4 + wave;
   if (task >= d.atile_ntask) return;
-  adafac_apply_tile(d, a, task, make_ema(dec), fac_tab, term_tab, wfold + (size_t)it.tensor * kAFold, net,
-                    xch[wave]);
+  if constexpr (BF)
+    adafac_apply_tile_bf(d, a, task, make_ema(dec), fac_tab, term_tab, wfold + (size_t)it.tensor * kAFold, net);
+  else
+    adafac_apply_tile(d, a, task, make_ema(dec), fac_tab, term_tab, wfold + (size_t)it.tensor * kAFold, net, xch[wave]);
 }
 
 }  // namespace pylo

@@ -628,6 +628,7 @@ struct PyloPlan {
   size_t last_dst = 0;   // where `last` was copied to
   bool have_last = false;
   bool mlp_on_matrix_pipe = true;  // env_matrix_pipe() when the plan was created
+  bool adafac_bf = true;           // AdafacLO's element MLP on the bf16 matrix instructions (PYLO_MI355_ADAFAC_F32=1: fp32 ones)
   // optional per-launch timing (pylo_mi355_plan_timing_begin/end)
   std::vector<hipEvent_t> tev;
   int t_steps_max = 0, t_steps = 0, t_per_step = 0;
@@ -664,6 +665,10 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   P->kind = kind;
   P->T = n_tensors;
   P->mlp_on_matrix_pipe = env_matrix_pipe();
+  {
+    const char* e = getenv("PYLO_MI355_ADAFAC_F32");
+    P->adafac_bf = !(e && e[0] == '1');
+  }
   if (int rc = build_layout(kind, shapes, n_tensors, P->L, kVeloHiddenMax)) { delete P; return rc; }
   if (workspace == nullptr || workspace_bytes < P->L.total) { delete P; return fail("plan_create: workspace too small"); }
   if (reinterpret_cast<uintptr_t>(workspace) % 256 != 0) { delete P; return fail("plan_create: workspace must be 256-byte aligned"); }
@@ -1445,9 +1450,14 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   if (n_ga > 0)
     hipLaunchKernelGGL(k_adafac_apply, dim3(n_ga), dim3(kThreads), 0, s, descs, dyn, ga_items, fac_tab, term_tab, dec,
                        wfold, net, (const float*)bias_eff, gl);
-  if (n_ap > 0)
-    hipLaunchKernelGGL(k_adafac_apply_tile, dim3(n_ap), dim3(kThreads), 0, s, descs, dyn, ap_items, fac_tab, term_tab,
-                       dec, wfold, net, gl);
+  if (n_ap > 0) {
+    if (P->adafac_bf)
+      hipLaunchKernelGGL(k_adafac_apply_tile<true>, dim3(n_ap), dim3(kThreads), 0, s, descs, dyn, ap_items, fac_tab,
+                         term_tab, dec, wfold, net, gl);
+    else
+      hipLaunchKernelGGL(k_adafac_apply_tile<false>, dim3(n_ap), dim3(kThreads), 0, s, descs, dyn, ap_items, fac_tab,
+                         term_tab, dec, wfold, net, gl);
+  }
   HIP_TRY(mark());
   mark.done();
   stage_out(P, s, 0);

@@ -73,12 +73,16 @@ def test_velo_valu(monkeypatch):
             assert max_err(p, cpu[i], REL, ABS) <= 1.0, (t, i)
 
 
-def test_adafac_valu(monkeypatch):
+@pytest.mark.parametrize("switch", ["PYLO_MI355_VALU_MLP", "PYLO_MI355_ADAFAC_F32"])
+def test_adafac_valu(monkeypatch, switch):
+    """AdafacLO's element MLP runs on the bf16 matrix instructions by default (operands split into three
+    bf16 planes, six products per fp32 product); PYLO_MI355_ADAFAC_F32=1 keeps it on the fp32 matrix
+    instructions, PYLO_MI355_VALU_MLP=1 on the vector pipe."""
     from oracle import pylo_oracle as O
     from pylo_amd import AdafacLO_CUDA
     from pylo_amd.models import MetaMLP
 
-    monkeypatch.setenv("PYLO_MI355_VALU_MLP", "1")
+    monkeypatch.setenv(switch, "1")
     torch.manual_seed(3)
     net = MetaMLP(39, 32, 1)
     init, grads = _inputs(5)
@@ -95,3 +99,36 @@ def test_adafac_valu(monkeypatch):
             assert max_err(p, cpu[i], REL, ABS) <= 1.0, (t, i)
             for k in ("exp_avg", "exp_avg_sq", "exp_avg_sq_r", "exp_avg_sq_c"):
                 assert max_err(opt.state[p][k], orc.state[i][k], REL, ABS) <= 1.0, (t, i, k)
+
+
+def test_adafac_matrix_pipes_against_fp64(monkeypatch):
+    """The split-bf16 MLP gives up no accuracy: the parameter steps of both matrix-pipe variants against the
+    oracle evaluated in fp64, relative to the error the fp32 oracle itself makes (both stay below it)."""
+    from oracle import pylo_oracle as O
+    from pylo_amd import AdafacLO_CUDA
+    from pylo_amd.models import MetaMLP
+
+    torch.manual_seed(3)
+    net = MetaMLP(39, 32, 1)
+    shapes = [(256, 512), (96, 1024)]
+    gen = torch.Generator().manual_seed(8)
+    init = [torch.randn(s, generator=gen) * 0.01 for s in shapes]     # small against the step: p's own rounding stays out of the way
+    grads = [torch.randn(s, generator=gen) * 0.1 for s in shapes]
+    ref64 = [v.double().cuda() for v in init]
+    ref32 = [v.clone().cuda() for v in init]
+    kw = dict(lr=1.0, step_mult=1.0, exp_mult=0.1)
+    O.AdafacOracle(ref64, net.state_dict(), device="cuda", **kw).double_().step([g.double().cuda() for g in grads])
+    O.AdafacOracle(ref32, net.state_dict(), device="cuda", **kw).step([g.cuda() for g in grads])
+    own = max(float((a.double() - b).abs().max()) for a, b in zip(ref32, ref64))
+    errs = {}
+    for name, env in (("bf16x3", "0"), ("fp32", "1")):
+        monkeypatch.setenv("PYLO_MI355_ADAFAC_F32", env)
+        gpu = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+        opt = AdafacLO_CUDA(gpu, network=copy.deepcopy(net), **kw)
+        for p, g in zip(gpu, grads):
+            p.grad = g.cuda()
+        opt.step()
+        torch.cuda.synchronize()
+        errs[name] = max(float((p.detach().double() - b).abs().max()) for p, b in zip(gpu, ref64))
+    print("max |p - fp64 oracle|: fp32 oracle", own, " HIP", errs)
+    assert errs["bf16x3"] <= 1.5 * max(own, errs["fp32"]), (errs, own)

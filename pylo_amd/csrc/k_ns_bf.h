@@ -373,11 +373,14 @@ __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__
     }
     bfbits h[4], m[4], l[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      bf_split(v[q], h[q], m[q], l[q]);
-      tile[0][lr][lc + q] = h[q];
-      tile[1][lr][lc + q] = m[q];
-      tile[2][lr][lc + q] = l[q];
+    for (int q = 0; q < 4; ++q) bf_split(v[q], h[q], m[q], l[q]);
+    // two values a store (lc is even and the row pitch is 33 dwords: 4-byte aligned)
+    typedef unsigned int u32;
+#pragma unroll
+    for (int q = 0; q < 4; q += 2) {
+      *(u32*)&tile[0][lr][lc + q] = (u32)h[q] | (u32)h[q + 1] << 16;
+      *(u32*)&tile[1][lr][lc + q] = (u32)m[q] | (u32)m[q + 1] << 16;
+      *(u32*)&tile[2][lr][lc + q] = (u32)l[q] | (u32)l[q + 1] << 16;
     }
     if (in) {
       typedef unsigned long long u64;

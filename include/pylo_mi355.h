@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PYLO_MI355_ABI_VERSION 6
+#define PYLO_MI355_ABI_VERSION 7
 #define PYLO_MAX_DIMS 8
 #define PYLO_MAX_GROUPS 8   /* parameter groups with their own step counter (VeLO) */
 
@@ -57,6 +57,12 @@ extern "C" {
 #define PYLO_F_GLOBAL_NORM 16 /* AdafacLO kind: the tensor's gradient is summed into the global norm of the
                                  call; required on every tensor of a plan whose steps pass clip_norm > 0
                                  (CELO2 plans always take the norm over all their tensors) */
+#define PYLO_F_TENSOR_NORM 32 /* AdafacLO kind: clip_norm > 0 bounds the norm of this tensor's gradient alone, as
+                                 torch.nn.utils.clip_grad_norm_(p, clip_norm) does on one parameter
+                                 (AdafacLO_naive.py:199-200, AdafacLO_cuda.py:214-215): the step sees
+                                 g * min(1, clip_norm / (||g||_2 + 1e-6)).  The gradient buffer itself is not
+                                 modified (the reference scales p.grad in place).  On every tensor of the plan or
+                                 on none; not with PYLO_F_GLOBAL_NORM or PYLO_F_NAN_TO_NUM; clip_val must be 0 */
 
 /* Storage type of the tensor's `grad` and `param` buffers (bits 8-9 of PyloTensorShape.flags).  The reference's
    kernels are instantiated for float, double and half (AT_DISPATCH_FLOATING_TYPES_AND_HALF,

@@ -671,7 +671,8 @@ class AdafacOracle:
                  momentum_decays=(0.15216392, 0.14245212, 0.06812963),
                  rms_decays=(0.01079706,),
                  adafactor_decays=(0.18621896, -0.10864615, -0.06185547), device="cpu",
-                 per_param_step=False):
+                 per_param_step=False, max_grad_norm=None):
+        self.max_grad_norm = max_grad_norm
         # per_param_step: the time features follow each parameter's own step counter, as the CUDA
         # class keeps it (AdafacLO_cuda.py:304-305,400), instead of the group's counter of the naive
         # class (AdafacLO_naive.py:194-197,226); the two differ only for a parameter that sat steps out.
@@ -712,8 +713,18 @@ class AdafacOracle:
         return self
 
     def condition_grads(self, grads):
-        """AdafacLO_naive feeds the gradients as they are (max_grad_norm is applied by the caller)."""
-        return grads
+        """``max_grad_norm``: every gradient is clipped against its own 2-norm before anything else sees it
+        (AdafacLO_naive.py:199-200, ``torch.nn.utils.clip_grad_norm_(p, max_grad_norm)`` on one parameter:
+        the factor is ``min(1, max_norm / (norm + 1e-6))``).  The caller's tensors are left as they are."""
+        if self.max_grad_norm is None:
+            return grads
+        out = []
+        for g in grads:
+            if g is not None:
+                coef = self.max_grad_norm / (torch.linalg.vector_norm(g) + 1e-6)
+                g = g * torch.clamp(coef, max=1.0)
+            out.append(g)
+        return out
 
     def apply(self, p: torch.Tensor, unit_step: torch.Tensor) -> None:
         """pylo/optim/AdafacLO_naive.py:305-310 (`unit_step` = direction * exp(magnitude * exp_mult))"""

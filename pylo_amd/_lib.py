@@ -18,7 +18,7 @@ MAX_DIMS = 8
 KIND_CELO2, KIND_VELO, KIND_ADAFAC = 0, 1, 2
 F_ADAM = 1
 F_ADAM_INDEP = 2
-F_NAN_TO_NUM, F_WD_PRESTEP, F_GLOBAL_NORM = 4, 8, 16
+F_NAN_TO_NUM, F_WD_PRESTEP, F_GLOBAL_NORM, F_TENSOR_NORM = 4, 8, 16, 32
 ARG_ORTHOGONALIZE = 1      # PyloTensorArgs.flags
 # storage type of a tensor's grad / param buffers (PYLO_F_STORE_*); accumulators and arithmetic stay fp32
 STORE_FLAG = {torch.float32: 0, torch.float16: 0x100, torch.bfloat16: 0x200, torch.float64: 0x300}
@@ -109,7 +109,7 @@ def load():
     lib.pylo_mi355_plan_invalidate_statistics.argtypes = [C.c_void_p]
     lib.pylo_mi355_plan_arg_table.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_void_p)]
     lib.pylo_mi355_plan_device_steps.argtypes = [C.c_void_p, C.POINTER(DeviceSteps)]
-    if lib.pylo_mi355_abi_version() != 6:
+    if lib.pylo_mi355_abi_version() != 7:
         raise RuntimeError("libpylo_mi355.so: ABI version mismatch, rebuild it")
     _lib = lib
     return lib

@@ -135,7 +135,7 @@ __global__ __launch_bounds__(kThreads) void k_adafac_stats(const TDesc* __restri
   TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
-  set_grad_scale(d, a, gl);
+  set_grad_scale(d, a, gl, it.tensor);
   const EmaConsts e = make_ema(dec);
   VeloAcc acc;
 #pragma unroll
@@ -689,7 +689,7 @@ __global__ __launch_bounds__(kThreads) void k_adafac_apply(const TDesc* __restri
   TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
-  set_grad_scale(d, a, gl);
+  set_grad_scale(d, a, gl, it.tensor);
   const EmaConsts e = make_ema(dec);
   const float* w = wfold + (size_t)it.tensor * kAFold;
   const long long count = (long long)kThreads * d.vec * kElemIters;
@@ -711,7 +711,7 @@ void k_adafac_apply_tile(const TDesc* __restrict__ descs, const PyloTensorArgs* 
   TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
-  set_grad_scale(d, a, gl);
+  set_grad_scale(d, a, gl, it.tensor);
   __shared__ float xch[BF ? 1 : kWaves][BF ? 1 : 16 * kXPitch];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int task = it.a * 4 + wave;

@@ -148,7 +148,7 @@ __global__ __launch_bounds__(kThreads) void k_celo2_slices(const TDesc* __restri
   TDesc d = descs[it.tensor];
   const PyloTensorArgs a = dyn[it.tensor];
   if (a.grad == nullptr) return;
-  set_grad_scale(d, a, gl);
+  set_grad_scale(d, a, gl, it.tensor);
   const EmaConsts e = make_ema(dec);
   const cfloat* w = launder(mlp);
   const int S = d.slice_len;

@@ -115,7 +115,7 @@ __device__ __forceinline__ void p0_nd_block(const TDesc* __restrict__ descs, con
   const int e = threadIdx.x & 63, grp = threadIdx.x >> 6;
   const int i = it.a * kV0aEnt + e;
   const int X = pick(d.nd_size, w), sX = pick(d.nd_stride, w);
-  const float scale = a.clip_norm > 0.0f ? clip_scale(gl->gnorm, a.clip_norm) : 1.0f;
+  const float scale = grad_scale(d, a, gl, it.tensor);
   float s = 0.0f;
   if (i < pick(d.len, w)) {
     const long long base = (long long)(i / sX) * X * sX + (i % sX);
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(kThreads) void k_p0(const TDesc* __restrict__ descs
   if (a.grad != nullptr) {
     if (d.mode == kModeFac2D) {
       const bool exact = (pass == 1) || !clip_on;
-      const float scale = (pass == 1) ? clip_scale(gl->gnorm, a.clip_norm) : 1.0f;
+      const float scale = (pass == 1) ? grad_scale(d, a, gl, it.tensor) : 1.0f;
       float* p0r = part + d.part_off[0];
       float* p0c = part + d.part_off[1];
       if (d.vec == 4 && exact) p0_factored<4, true>(d, a.grad, it.a, it.b, scale, a.clip_val, d.nan0, p0r, p0c, lds_col, lds_row, gsq, amax);
@@ -218,6 +218,44 @@ __global__ __launch_bounds__(kThreads) void k_gnorm(const double* __restrict__ g
   if (threadIdx.x == 0) {
     gl->gnorm = (float)sqrt((red[0] + red[1]) + (red[2] + red[3]));
     gl->flag = use_flags ? (fred[0] | fred[1] | fred[2] | fred[3]) : 0;
+  }
+}
+
+// Per-tensor norm clipping (PYLO_F_TENSOR_NORM; AdafacLO_naive.py:199-200 calls torch.nn.utils.clip_grad_norm_
+// on each parameter by itself): one block per tensor adds up the tensor's sum-of-squares partials in a fixed
+// order and leaves  min(1, clip_norm / (norm + 1e-6))  in tscale[t], torch's clip coefficient.  Such tensors
+// carry no clamp (the launcher checks), so the exact pass never runs: flag = 0.
+__global__ __launch_bounds__(kThreads) void k_tnorm(const TDesc* __restrict__ descs,
+                                                    const PyloTensorArgs* __restrict__ dyn,
+                                                    const double* __restrict__ gsq_part, Globals* __restrict__ gl,
+                                                    float* __restrict__ tscale) {
+  __shared__ double red[kWaves];
+  const int t = blockIdx.x;
+  if (t == 0 && threadIdx.x == 0) {
+    gl->gnorm = 0.0f;
+    gl->flag = 0;
+    gl->tscale = tscale;
+  }
+  const int first = descs[t].p0_first, n = descs[t].p0_n;
+  const float clip = dyn[t].clip_norm;
+  double s = 0.0;
+  for (int i0 = threadIdx.x; i0 < n; i0 += 16 * kThreads) {
+    double sv[16];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int i = i0 + q * kThreads;
+      sv[q] = i < n ? gsq_part[first + i] : 0.0;
+    }
+#pragma unroll
+    for (int q = 0; q < 16; ++q) s += sv[q];
+  }
+  s = wave_sum(s);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const float norm = (float)sqrt((red[0] + red[1]) + (red[2] + red[3]));
+    const float c = clip / (norm + 1e-6f);
+    tscale[t] = clip > 0.0f ? (c > 1.0f ? 1.0f : c) : 1.0f;   // a NaN norm gives a NaN factor, as torch.clamp does
   }
 }
 
@@ -305,7 +343,7 @@ __global__ __launch_bounds__(kV0aThreads) void k_v0a(const TDesc* __restrict__ d
   if (k < 3 && i < len) fac_old = *(const gfloat*)(fac + (size_t)k * len + i);
   double s2 = 1.0;
   if (a.clip_norm > 0.0f && gl->flag == 0 && d.mode == kModeFac2D) {  // other modes sum the scaled gradient
-    const float sc = clip_scale(gl->gnorm, a.clip_norm);
+    const float sc = grad_scale(d, a, gl, it.tensor);
     s2 = (double)sc * (double)sc;
   }
   {

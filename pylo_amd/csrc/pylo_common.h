@@ -106,6 +106,8 @@ struct TDesc {
   int nan0;                // gradients pass through torch.nan_to_num (PYLO_F_NAN_TO_NUM)
   int wd_prestep;          // p -= lr * (step + wd * p) against the pre-step parameter (PYLO_F_WD_PRESTEP)
   int store;               // storage type of the caller's grad / param buffers (kStore*, k_cast.h); 0 = fp32
+  int own_norm;            // clip_norm bounds the tensor's own gradient norm (PYLO_F_TENSOR_NORM), not the call's
+  int p0_first, p0_n;      // the tensor's blocks of the first statistics launch (rows of its sum-of-squares partials)
   float gscale;            // 1 in the plan; AdafacLO-family kernels overwrite their copy with the clip scale
 };
 
@@ -141,6 +143,7 @@ constexpr int kSumM = 30, kSumMM = 33, kSumR = 36, kSumRR = 37;
 struct Globals {
   float gnorm;  // ||all grads||_2
   int flag;     // some |g| exceeded clip_val on a tensor whose sums were taken un-clamped
+  const float* tscale;  // plans with per-tensor norm clipping: the clip factor of every tensor (k_tnorm)
 };
 
 // Item::c of the fused element pass of ELO-CELO2 (k_celo2_elem)
@@ -230,9 +233,16 @@ __device__ __forceinline__ float clip_scale(float gnorm, float clip_norm) {
   return denom > 0.0f ? clip_norm / denom : 1.0f;
 }
 
-// The descriptor copy of a kernel carries the tensor's global-norm clip factor for cond_grad.
-__device__ __forceinline__ void set_grad_scale(TDesc& d, const PyloTensorArgs& a, const Globals* gl) {
-  d.gscale = a.clip_norm > 0.0f ? clip_scale(gl->gnorm, a.clip_norm) : 1.0f;
+// Factor on tensor t's gradient from norm clipping: by the norm of all gradients of the call, or, on tensors
+// flagged PYLO_F_TENSOR_NORM, by the tensor's own (k_tnorm has left the factor in gl->tscale).
+__device__ __forceinline__ float grad_scale(const TDesc& d, const PyloTensorArgs& a, const Globals* gl, int t) {
+  if (!(a.clip_norm > 0.0f)) return 1.0f;
+  return d.own_norm ? gl->tscale[t] : clip_scale(gl->gnorm, a.clip_norm);
+}
+
+// The descriptor copy of a kernel carries the tensor's clip factor for cond_grad.
+__device__ __forceinline__ void set_grad_scale(TDesc& d, const PyloTensorArgs& a, const Globals* gl, int t) {
+  d.gscale = grad_scale(d, a, gl, t);
 }
 
 // The gradient as the optimizer sees it (ELO_naive.py:141-146): scaled by the global-norm clip factor,

@@ -105,7 +105,8 @@ struct Layout {
   int H = 8;  // width of the first MLP layer (terms per row / column)
   int Tpad = 0;
   bool global_norm = false;  // AdafacLO kind: every tensor has P0 items, the call may clip by global norm
-  size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_sl_items, off_seg_items, off_segtot, off_el_items, off_ap_items, off_ga_items, off_fin_items, off_finpart, off_finscale, off_v0a_items, off_v0b_items, off_fac_list,
+  bool tensor_norm = false;  // ... or every tensor by its own norm (PYLO_F_TENSOR_NORM)
+  size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_sl_items, off_seg_items, off_segtot, off_el_items, off_ap_items, off_ga_items, off_fin_items, off_finpart, off_finscale, off_tscale, off_v0a_items, off_v0b_items, off_fac_list,
       off_part, off_gsq, off_flag, off_globals, off_fac, off_term, off_v0part, off_bscale, off_stats, off_wfold,
       off_chan_ms, off_totals, off_xfeat, off_lossfeat, off_xT, off_mixbuf, off_pmax, off_canon, off_frac, total;
 };
@@ -366,7 +367,8 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.dr.assign(T, -1);
   long long part = 0, fac = 0, term = 0;
   const int H = L.H;
-  L.global_norm = (shapes[0].flags & PYLO_F_GLOBAL_NORM) != 0;
+  L.tensor_norm = (shapes[0].flags & PYLO_F_TENSOR_NORM) != 0;
+  L.global_norm = (shapes[0].flags & PYLO_F_GLOBAL_NORM) != 0 || L.tensor_norm;
   for (int t = 0; t < T; ++t) {
     const PyloTensorShape& s = shapes[t];
     if (s.ndim < 0 || s.ndim > PYLO_MAX_DIMS) return fail("plan: bad ndim");
@@ -381,10 +383,17 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     TDesc& d = L.descs[t];
     d.n = n;
     d.gscale = 1.0f;
-    if ((s.flags & (PYLO_F_NAN_TO_NUM | PYLO_F_WD_PRESTEP | PYLO_F_GLOBAL_NORM)) && kind != PYLO_KIND_ADAFAC)
-      return fail("plan: PYLO_F_NAN_TO_NUM / PYLO_F_WD_PRESTEP / PYLO_F_GLOBAL_NORM belong to AdafacLO plans");
-    if (((s.flags & PYLO_F_GLOBAL_NORM) != 0) != L.global_norm)
+    if ((s.flags & (PYLO_F_NAN_TO_NUM | PYLO_F_WD_PRESTEP | PYLO_F_GLOBAL_NORM | PYLO_F_TENSOR_NORM)) &&
+        kind != PYLO_KIND_ADAFAC)
+      return fail("plan: PYLO_F_NAN_TO_NUM / PYLO_F_WD_PRESTEP / PYLO_F_GLOBAL_NORM / PYLO_F_TENSOR_NORM belong to "
+                  "AdafacLO plans");
+    if (((s.flags & PYLO_F_TENSOR_NORM) != 0) != L.tensor_norm)
+      return fail("plan: PYLO_F_TENSOR_NORM must be set on every tensor of the plan or on none");
+    if (L.tensor_norm && (s.flags & (PYLO_F_GLOBAL_NORM | PYLO_F_NAN_TO_NUM)))
+      return fail("plan: PYLO_F_TENSOR_NORM does not combine with PYLO_F_GLOBAL_NORM or PYLO_F_NAN_TO_NUM");
+    if (!L.tensor_norm && ((s.flags & PYLO_F_GLOBAL_NORM) != 0) != L.global_norm)
       return fail("plan: PYLO_F_GLOBAL_NORM must be set on every tensor of the plan or on none");
+    d.own_norm = L.tensor_norm ? 1 : 0;
     d.nan0 = (s.flags & PYLO_F_NAN_TO_NUM) != 0;
     d.store = (s.flags & PYLO_F_STORE_MASK) >> 8;
     L.stage_ofs.push_back(StageOfs{-1, -1});
@@ -487,14 +496,16 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     const long long chunk = (long long)kThreads * d.vec * kElemIters;
     // P0 items: tiles of 2-D factored tensors; flat chunks only where a global norm is needed
     // (CELO2's AdamW tensors, every other tensor of a PYLO_F_GLOBAL_NORM plan)
+    d.p0_first = (int)L.p0_items.size();
     if (n > 0) {
       if (d.mode == kModeFac2D) {
         for (int st = 0; st < d.n_strips; ++st)
           for (int cb = 0; cb < d.n_colblk; ++cb) L.p0_items.push_back(Item{t, st, cb, 0});
-      } else if (kind == PYLO_KIND_CELO2 || (s.flags & PYLO_F_GLOBAL_NORM)) {
+      } else if (kind == PYLO_KIND_CELO2 || L.global_norm) {
         for (long long c = 0; c * chunk < n; ++c) L.p0_items.push_back(Item{t, (int)c, 0, 0});
       }
     }
+    d.p0_n = (int)L.p0_items.size() - d.p0_first;
     d.blk0 = (int)L.el_items.size();
     const bool wide = d.mode == kModeFac2D && n > 0 && env_matrix_pipe();
     if (kind == PYLO_KIND_CELO2 && (d.mode == kModeFacND || d.mode == kModeVec)) {
@@ -567,6 +578,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_gsq = take(sizeof(double) * L.p0_items.size());
   L.off_flag = take(sizeof(int) * L.p0_items.size());
   L.off_globals = take(sizeof(Globals));
+  L.off_tscale = take(sizeof(float) * (L.tensor_norm ? T : 0));
   L.off_fac = take(sizeof(float) * fac);
   L.off_term = take(sizeof(float) * term);
   L.off_v0part = take(sizeof(double) * kNV0 * L.v0a_items.size());
@@ -1406,14 +1418,22 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   // is not a fixed point of the conditioning.  Plain AdafacLO steps skip both launches.
   bool clips = false;
   for (int t = 0; t < T; ++t) clips = clips || (args[t].grad != nullptr && args[t].clip_norm > 0.0f);
-  if (clips && !L.global_norm) return fail("adafac_step: clip_norm > 0 needs a plan built with PYLO_F_GLOBAL_NORM");
+  if (clips && !L.global_norm)
+    return fail("adafac_step: clip_norm > 0 needs a plan built with PYLO_F_GLOBAL_NORM or PYLO_F_TENSOR_NORM");
+  if (clips && L.tensor_norm)
+    for (int t = 0; t < T; ++t)
+      if (args[t].grad != nullptr && args[t].clip_norm > 0.0f && args[t].clip_val != 0.0f)
+        return fail("adafac_step: a tensor clipped by its own norm (PYLO_F_TENSOR_NORM) takes no clip_val");
   HIP_TRY(mark());
   // without global-norm clipping the N-D tensors' sums ride in the tail blocks of the first launch
   const int n_tail = clips ? 0 : n_nd;
   if (n_p0 + n_tail > 0)
     hipLaunchKernelGGL(k_p0, dim3(n_p0 + n_tail), dim3(kThreads), 0, s, descs, dyn, p0_items, part, gsq, flag, gl, 0,
                        nd_items, n_p0);
-  if (clips) {
+  if (clips && L.tensor_norm) {
+    // every tensor against its own norm (AdafacLO_naive.py:199-200): no clamp on such tensors, no exact pass
+    hipLaunchKernelGGL(k_tnorm, dim3(T), dim3(kThreads), 0, s, descs, dyn, gsq, gl, P->at<float>(L.off_tscale));
+  } else if (clips) {
     const bool exact_pass = exact_pass_possible(P, args);
     hipLaunchKernelGGL(k_gnorm, dim3(1), dim3(kThreads), 0, s, gsq, flag, n_p0, gl, exact_pass ? 1 : 0, (int*)nullptr, 0);
     if (n_p0 > 0 && exact_pass)

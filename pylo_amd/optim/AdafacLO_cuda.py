@@ -129,7 +129,8 @@ class AdafacLO_CUDA(Optimizer):
         state["exp_avg"] = torch.zeros((3,) + shape, device=self.device)
 
     def _ensure_plan(self, tensors):
-        key = tuple((tuple(p.shape), p.dtype) for _, p in tensors)
+        flags = self._PLAN_FLAGS | self._norm_flags()
+        key = (flags,) + tuple((tuple(p.shape), p.dtype) for _, p in tensors)
         if key == self._plan_key:
             return
         for _, p in tensors:
@@ -140,7 +141,7 @@ class AdafacLO_CUDA(Optimizer):
         # parameters and gradients may be float16 / bfloat16 / float64 (the reference's kernels dispatch on the
         # element type, learned_optimizer.cu:338,364); the accumulators stay float32
         self._plan = _lib.Plan(_lib.KIND_ADAFAC, [tuple(p.shape) for _, p in tensors],
-                               [self._PLAN_FLAGS | _lib.store_flag(p, "AdafacLO_CUDA") for _, p in tensors], self.device)
+                               [flags | _lib.store_flag(p, "AdafacLO_CUDA") for _, p in tensors], self.device)
         self._plan_key = key
         if self.capturable:
             self._reset_device_steps(tensors)
@@ -184,15 +185,19 @@ class AdafacLO_CUDA(Optimizer):
             self._reset_device_steps([(g, p) for g in self.param_groups for p in g["params"]])
         return out
 
-    def _pre_clip(self, group, p):
-        """Per-parameter norm clipping of the gradient, in place (AdafacLO_naive.py:200-201)."""
-        if group["max_grad_norm"] is not None:
-            torch.nn.utils.clip_grad_norm_(p, group["max_grad_norm"])
+    def _norm_flags(self):
+        """``max_grad_norm`` bounds every parameter's own gradient norm (AdafacLO_naive.py:199-200 and
+        AdafacLO_cuda.py:214-215 call ``torch.nn.utils.clip_grad_norm_`` per parameter): the fused step takes the
+        norms from its statistics pass and scales the gradients as it reads them (PYLO_F_TENSOR_NORM), so nothing
+        is launched per parameter.  Unlike the reference, ``p.grad`` itself is left as it was."""
+        on = any(g["max_grad_norm"] is not None for g in self.param_groups)
+        return _lib.F_TENSOR_NORM if on else 0
 
     def _scalars(self, group):
         """Per-tensor scalar columns of the argument table."""
+        mx = group["max_grad_norm"]
         return dict(lr=group["lr"], weight_decay=group["weight_decay"], exp_mult=self.exp_mult,
-                    step_mult=self.step_mult)
+                    step_mult=self.step_mult, clip_norm=0.0 if mx is None else float(mx))
 
     @torch.no_grad()
     def step(self, loss=None):
@@ -206,7 +211,6 @@ class AdafacLO_CUDA(Optimizer):
         keep = []
         step_fed = None
         for i, (group, p) in enumerate(tensors):
-            self._pre_clip(group, p)
             g = p.grad
             if g is None:
                 continue

@@ -88,8 +88,8 @@ class ELO_CUDA(AdafacLO_CUDA):
         self._plan = None
         self._plan_key = None
 
-    def _pre_clip(self, group, p):
-        pass            # global-norm clipping happens inside the step (ELO_cuda.py:153-161)
+    def _norm_flags(self):
+        return 0        # global-norm clipping (ELO_cuda.py:153-161): _PLAN_FLAGS
 
     def _scalars(self, group):
         return dict(lr=group["lr"], weight_decay=group["weight_decay"], exp_mult=group["exp_mult"], step_mult=1.0,

@@ -224,6 +224,13 @@ def adafac_case(R, name, shapes, n_steps, grad_scale, seed, weight_decay, lr, cl
     _save(name, arrays, meta)
 
 
+def adafac_max_norm_case(R):
+    """AdafacLO_naive with max_grad_norm (clip_grad_norm_ per parameter, AdafacLO_naive.py:199-200): gradients of
+    N(0, 0.1) against a bound of 1.0 clip four tensors (norms 1.4 .. 3.8) and leave the two small ones alone."""
+    adafac_case(R, "adafac_max_norm", [(20, 10), (20,), (40, 36), (6, 3, 4, 4), (16, 16), (3,)], 5, 0.1, 9,
+                weight_decay=0.01, lr=0.5, extra=dict(max_grad_norm=1.0))
+
+
 def ctor_checksums(R):
     """Sum and sum of squares (fp64) of every freshly constructed meta-net parameter under a fixed
     seed: pins the order in which the constructors draw from the RNG."""
@@ -255,6 +262,8 @@ def main():
     torch.set_num_threads(8)
     if "--stored-types-only" in sys.argv:
         return stored_type_cases(R)
+    if "--max-norm-only" in sys.argv:
+        return adafac_max_norm_case(R)
     # CELO2_naive (independent AdamW moments on 1-D tensors and is_embedding groups; CELO2_naive.py:263-283)
     celo2_case(R, "celo2_small", [(64, 32), (32, 64), (32,), (48, 24), (5,)], 8, 1.0, 12,
                dict(lr=1e-2, adam_lr_mult=3.0, weight_decay=0.02, adam_betas=(0.8, 0.9), adam_eps=1e-6,
@@ -296,6 +305,7 @@ def main():
     adafac_case(R, "adafac_small", [(20, 10), (20,), (5, 20), (6, 3, 4, 4), (16, 16)], 6, 0.3, 7,
                 weight_decay=0.0, lr=1.0)
     adafac_case(R, "adafac_small_wd", [(33, 17), (17,)], 5, 1e-3, 8, weight_decay=0.01, lr=0.5)
+    adafac_max_norm_case(R)
     stored_type_cases(R)
 
 

@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 REL, ABS = 1e-5, 1e-6
 
 
-@pytest.mark.parametrize("name", ["adafac_small", "adafac_small_wd"])
+@pytest.mark.parametrize("name", ["adafac_small", "adafac_small_wd", "adafac_max_norm"])
 def test_adafac_matches_reference_golden(name):
     from oracle import pylo_oracle as O
     from pylo_amd import AdafacLO_CUDA
@@ -28,7 +28,8 @@ def test_adafac_matches_reference_golden(name):
     net = MetaMLP(39, 32, 1)
     net.load_state_dict(G.state_dict("net"))
     gpu = [torch.nn.Parameter(G.t(f"init/{i}").cuda()) for i in range(len(shapes))]
-    opt = AdafacLO_CUDA(gpu, lr=meta["lr"], weight_decay=meta["weight_decay"], network=net)
+    # adafac_max_norm: max_grad_norm=1.0, per-parameter norm clipping inside the fused step
+    opt = AdafacLO_CUDA(gpu, lr=meta["lr"], weight_decay=meta["weight_decay"], network=net, **(meta.get("extra") or {}))
     worst = 0.0
     for t in range(meta["n_steps"]):
         for i, p in enumerate(gpu):
@@ -53,7 +54,11 @@ def test_adafac_matches_reference_golden(name):
     print(name, "worst err/tol", worst)
 
 
-def test_adafac_matches_oracle_mixed_shapes():
+@pytest.mark.parametrize("max_norm", [None, 0.7, "second group only"])
+def test_adafac_matches_oracle_mixed_shapes(max_norm):
+    """max_norm: ``max_grad_norm`` of the class (every gradient clipped against its own norm inside the fused step;
+    gradient norms here run from 0.003 to 360, so some tensors are scaled and some are not), for all parameters or
+    for the second of two parameter groups only."""
     from oracle import pylo_oracle as O
     from pylo_amd import AdafacLO_CUDA
     from pylo_amd.models import MetaMLP
@@ -66,8 +71,16 @@ def test_adafac_matches_oracle_mixed_shapes():
     init = [torch.randn(s, generator=gen) * 0.3 for s in shapes]
     cpu = [v.clone() for v in init]
     gpu = [torch.nn.Parameter(v.clone().cuda()) for v in init]
-    orc = O.AdafacOracle(cpu, net.state_dict(), lr=0.5, weight_decay=1e-3)
-    opt = AdafacLO_CUDA(gpu, lr=0.5, weight_decay=1e-3, network=copy.deepcopy(net))
+    if max_norm == "second group only":
+        half = len(shapes) // 2
+        orc = O.AdafacOracle(cpu, net.state_dict(), lr=0.5, weight_decay=1e-3, max_grad_norm=0.7)
+        clip = orc.condition_grads
+        orc.condition_grads = lambda gs: gs[:half] + clip(gs[half:])
+        groups = [{"params": gpu[:half]}, {"params": gpu[half:], "max_grad_norm": 0.7}]
+        opt = AdafacLO_CUDA(groups, lr=0.5, weight_decay=1e-3, network=copy.deepcopy(net))
+    else:
+        orc = O.AdafacOracle(cpu, net.state_dict(), lr=0.5, weight_decay=1e-3, max_grad_norm=max_norm)
+        opt = AdafacLO_CUDA(gpu, lr=0.5, weight_decay=1e-3, network=copy.deepcopy(net), max_grad_norm=max_norm)
     worst = 0.0
     for t in range(5):
         grads = [torch.randn(s, generator=gen) * (10.0 ** (-(i % 4))) for i, s in enumerate(shapes)]
@@ -77,6 +90,8 @@ def test_adafac_matches_oracle_mixed_shapes():
             p.grad = None if g is None else g.cuda()
         orc.step(grads)
         opt.step()
+        for p, g in zip(gpu, grads):     # the fused step scales what it reads, never the caller's buffer
+            assert g is None or torch.equal(p.grad.cpu(), g)
         for i, p in enumerate(gpu):
             st, so = opt.state[p], orc.state[i]
             checks = [("param", p, cpu[i])]

@@ -117,13 +117,14 @@ def test_velo_oracle_matches_reference(name):
                 assert max_err(st["fac_vec_col"], ref_c, REL, ABS) <= 1.0, (t, i, "col")
 
 
-@pytest.mark.parametrize("name", ["adafac_small", "adafac_small_wd"])
+@pytest.mark.parametrize("name", ["adafac_small", "adafac_small_wd", "adafac_max_norm"])
 def test_adafac_oracle_matches_reference(name):
     G = Golden(name)
     meta = G.meta
     shapes = G.shapes
     params = [G.t(f"init/{i}").clone() for i in range(len(shapes))]
-    opt = O.AdafacOracle(params, G.state_dict("net"), lr=meta["lr"], weight_decay=meta["weight_decay"])
+    opt = O.AdafacOracle(params, G.state_dict("net"), lr=meta["lr"], weight_decay=meta["weight_decay"],
+                         **(meta.get("extra") or {}))
     for t in range(meta["n_steps"]):
         grads = [G.t(f"grad{t}/{i}") for i in range(len(shapes))]
         opt.step(grads)

@@ -21,7 +21,9 @@ list, ``numpy.argsort`` for ``factored_dims``.
 (AdafacLO_cuda.py:304-305,400); the CUDA class cannot run here and the naive class counts per group, so
 no golden trajectory covers a parameter that sat steps out.  The switch is pinned by a property instead
 (tests/test_oracle_pins.py): AdafacLO tensors do not interact, so such a parameter must end bit-exactly
-where a single-parameter run fed only the steps it took part in ends.  Nothing here is unpinned.
+where a single-parameter run fed only the steps it took part in ends.  ``AdafacOracle(max_grad_norm=...)``
+(norm clipping of every gradient by itself) is pinned by a golden trajectory of the naive class with that
+argument (tests/golden/adafac_max_norm.npz).  Nothing here is unpinned.
 
 Parameters stored as float16 / bfloat16 / float64 need no code of their own: the contract is the float32
 step on the widened values with the result rounded into the storage type, so the tests feed these classes

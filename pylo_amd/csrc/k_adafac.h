@@ -529,6 +529,10 @@ __device__ __forceinline__ av16f bf3_mfma(const au32x4 (&w)[3], const au32x4 (&x
   return acc;
 }
 
+// PER: the tensor is an (O, I, k, ..) one walked as the matrix (O, I * P) (TDesc::aper): the vector that is not
+// indexed by the column has an entry per (row, column mod P), so a lane fetches the row's factor and first-layer
+// terms for its own columns (one per element group) instead of sharing one entry with the wave.
+template <bool PER>
 __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloTensorArgs& a, int task,
                                                      const EmaConsts& e, const float* __restrict__ fac_tab,
                                                      const float* __restrict__ term_tab, const float* wfold_t,
@@ -562,19 +566,27 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
   const cfloat* nw = launder(net);
   const float bo0 = nw[kABO + 0], bo1 = nw[kABO + 1];
   const float exp_scale = a.exp_mult * 1.44269504088896341f;
+  const int cv = PER ? d.aper_col : 1, pv = 1 - cv;   // the vector the column indexes, and the other one
+  const int per = PER ? d.aper : 1;
   float fb[4];
-  load_vec_o<4>(fac_tab + d.fac_off[1], tk.col * 16u, fb);
+  load_vec_o<4>(fac_tab + pick(d.fac_off, cv), tk.col * 16u, fb);
   // column terms of element e of group g (column: the wave's first + 32 g + e), units 8 j + 4 half ..: one
   // offset per lane, immediates per (g, j); row terms likewise from the row's table entry
-  const float* tcol = term_tab + d.term_off[1];
+  const float* tcol = term_tab + pick(d.term_off, cv);
   const unsigned tcol_off = ((tk.col - lane + el) * kAH + 4 * half) * 4u;
-  const unsigned trow_off = 4 * half * 4u;
+  // row side: byte offsets of the lane's entries relative to the row's first (zero unless PER)
+  unsigned fa_off = 0, trow_off[2] = {4 * half * 4u, 4 * half * 4u};
+  if constexpr (PER) {
+    fa_off = (tk.col % (unsigned)per) * 16u;
+#pragma unroll
+    for (int gq = 0; gq < 2; ++gq) trow_off[gq] += ((tk.col - lane + 32 * gq + el) % (unsigned)per) * (kAH * 4u);
+  }
   const unsigned lo = lane * 4u;
   const float* g = a.grad + tk.first;
   float *p = a.param + tk.first, *m0 = a.mom + tk.first, *m1 = a.mom + d.n + tk.first,
         *m2 = a.mom + 2 * d.n + tk.first, *rms = a.rms + tk.first;
-  const float* fr = fac_tab + d.fac_off[0] + (size_t)tk.r0 * 4;
-  const float* tr = term_tab + d.term_off[0] + (size_t)tk.r0 * kAH;
+  const float* fr = fac_tab + pick(d.fac_off, pv) + (size_t)tk.r0 * 4 * per;
+  const float* tr = term_tab + pick(d.term_off, pv) + (size_t)tk.r0 * kAH * per;
   for (int r = tk.r0; r < tk.r1; ++r) {
     float xg[1], xp[1], x0[1], x1[1], x2[1], xr_[1], fa[4];
     load_vec_nt<1>(g, lo, xg);
@@ -583,10 +595,13 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
     load_vec_nt<1>(m1, lo, x1);
     load_vec_nt<1>(m2, lo, x2);
     load_vec_nt<1>(rms, lo, xr_);
-    load_uniform<4>(fr, fa);
-    float ta[4][4];
+    if constexpr (PER) load_vec_o<4>(fr, fa_off, fa);
+    else load_uniform<4>(fr, fa);
+    float ta[PER ? 2 : 1][4][4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) load_vec_o<4>(tr + 8 * j, trow_off, ta[j]);
+    for (int gq = 0; gq < (PER ? 2 : 1); ++gq)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) load_vec_o<4>(tr + 8 * j, trow_off[gq], ta[gq][j]);
     const float gg = cond_grad(xg[0], d.gscale, a.clip_val, d.nan0);
     float m[3] = {x0[0], x1[0], x2[0]};
     ema_update(e, gg, m, xr_[0]);
@@ -623,7 +638,7 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
         float tb[4];
         load_vec_o<4>(tcol + (32 * gq) * kAH + 8 * j, tcol_off, tb);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) h[4 * j + i] = ta[j][i] + tb[i];
+        for (int i = 0; i < 4; ++i) h[4 * j + i] = ta[PER ? gq : 0][j][i] + tb[i];
       }
       h = bf3_mfma(w1, xb[gq], h);
       // hidden values of the units this lane holds -> planes, four units (two dwords) per block j
@@ -672,7 +687,7 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
     pn[0] = adafac_update(d, a, o0 * __builtin_amdgcn_exp2f(o1 * exp_scale), xp[0]);
     store_vec_o<1>(p, lo, pn);
     g += d.C0; p += d.C0; m0 += d.C0; m1 += d.C0; m2 += d.C0; rms += d.C0;
-    fr += 4; tr += kAH;
+    fr += 4 * per; tr += kAH * per;
   }
 }
 
@@ -701,7 +716,7 @@ __global__ __launch_bounds__(kThreads) void k_adafac_apply(const TDesc* __restri
 
 // The apply pass for tensors walked column-resident (items hold four wave tasks each).  BF: the element MLP on
 // the bf16 matrix instructions (three-plane operands), else on the fp32 ones.
-template <bool BF>
+template <bool BF, bool PER = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(BF ? 2 : PYLO_ADAFAC_WAVES)))
 void k_adafac_apply_tile(const TDesc* __restrict__ descs, const PyloTensorArgs* __restrict__ dyn,
                          const Item* __restrict__ items, const float* __restrict__ fac_tab,
@@ -716,8 +731,9 @@ void k_adafac_apply_tile(const TDesc* __restrict__ descs, const PyloTensorArgs* 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int task = it.a * 4 + wave;
   if (task >= d.atile_ntask) return;
+  static_assert(BF || !PER, "tensors with more than two dims are walked by the bf16 variant only");
   if constexpr (BF)
-    adafac_apply_tile_bf(d, a, task, make_ema(dec), fac_tab, term_tab, wfold + (size_t)it.tensor * kAFold, net);
+    adafac_apply_tile_bf<PER>(d, a, task, make_ema(dec), fac_tab, term_tab, wfold + (size_t)it.tensor * kAFold, net);
   else
     adafac_apply_tile(d, a, task, make_ema(dec), fac_tab, term_tab, wfold + (size_t)it.tensor * kAFold, net, xch[wave]);
 }

@@ -100,6 +100,11 @@ struct TDesc {
   // AdafacLO's apply pass walks one column per lane (its 32-wide MLP leaves no registers for two):
   // same scheme with 64 columns per wave task; apply block a holds tasks 4a .. 4a+3.
   int atile_nct, atile_ntask;
+  // ... and an (O, I, k, ..) tensor whose factored dims are the two leading ones is walked the same way as the
+  // matrix (O, I * P), P = product of the trailing dims: one vector is indexed by the matrix column, the other by
+  // (row, column mod P).  aper = P (0: not walked so), aper_col = which vector the column indexes; R0 / C0 hold
+  // the matrix view.
+  int aper, aper_col;
   int adam_indep;          // kModeFlat: AdamW on the tensor's own two moments instead of mom[0] / rms
   int fin_blk0, fin_nblk;  // ELO-CELO2 finishing pass: range of 8192-element blocks (rows of its partials)
   int slice_len;           // CELO2, N-D or fewer than two dims: elements per slice of the last two dims (or n)

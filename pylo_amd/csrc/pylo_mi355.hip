@@ -99,14 +99,14 @@ struct Layout {
   long long stage_floats = 0;
   size_t off_dyn_user = 0, off_stage_ofs = 0, off_cast_items = 0, off_stage = 0;
   std::vector<TDesc> descs;
-  std::vector<Item> p0_items, nd_items, sl_items, seg_items, el_items, ap_items, ga_items, fin_items, v0a_items, v0b_items;
+  std::vector<Item> p0_items, nd_items, sl_items, seg_items, el_items, ap_items, pp_items, ga_items, fin_items, v0a_items, v0b_items;
   std::vector<int> fac_list;
   std::vector<int> dc, dr;
   int H = 8;  // width of the first MLP layer (terms per row / column)
   int Tpad = 0;
   bool global_norm = false;  // AdafacLO kind: every tensor has P0 items, the call may clip by global norm
   bool tensor_norm = false;  // ... or every tensor by its own norm (PYLO_F_TENSOR_NORM)
-  size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_sl_items, off_seg_items, off_segtot, off_el_items, off_ap_items, off_ga_items, off_fin_items, off_finpart, off_finscale, off_tscale, off_v0a_items, off_v0b_items, off_fac_list,
+  size_t off_descs, off_dyn, off_p0_items, off_nd_items, off_sl_items, off_seg_items, off_segtot, off_el_items, off_ap_items, off_pp_items, off_ga_items, off_fin_items, off_finpart, off_finscale, off_tscale, off_v0a_items, off_v0b_items, off_fac_list,
       off_part, off_gsq, off_flag, off_globals, off_fac, off_term, off_v0part, off_bscale, off_stats, off_wfold,
       off_chan_ms, off_totals, off_xfeat, off_lossfeat, off_xT, off_mixbuf, off_pmax, off_canon, off_frac, total;
 };
@@ -118,6 +118,13 @@ int first_layer_width(int kind) { return kind == PYLO_KIND_CELO2 ? 8 : kind == P
 // earlier all-VALU kernels over linear chunks (same results up to rounding; for A/B measurements).
 bool env_matrix_pipe() {
   const char* v = std::getenv("PYLO_MI355_VALU_MLP");
+  return !(v && v[0] == '1');
+}
+
+// AdafacLO's element MLP on the bf16 matrix instructions (three-plane operands); PYLO_MI355_ADAFAC_F32=1 keeps
+// the fp32 matrix instructions.
+bool env_adafac_bf() {
+  const char* v = std::getenv("PYLO_MI355_ADAFAC_F32");
   return !(v && v[0] == '1');
 }
 
@@ -536,11 +543,26 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     // blocks of AdafacLO's apply pass: one column per lane where the tensor allows it (ap_items,
     // k_adafac_apply_tile), linear chunks otherwise (ga_items, k_adafac_apply)
     if (kind == PYLO_KIND_ADAFAC) {
-      if (wide && d.C0 % 64 == 0) {
+      // an (O, I, k, ..) tensor factored over its two leading dims (convolution kernels) is the matrix (O, I * P)
+      // for this pass, P = product of the trailing dims (pp_items)
+      bool periodic = false;
+      if (d.mode == kModeFacND && n > 0 && env_matrix_pipe() && env_adafac_bf() && e.ndim >= 3 &&
+          ((edr == 0 && edc == 1) || (edr == 1 && edc == 0))) {
+        long long P = 1;
+        for (int i = 2; i < e.ndim; ++i) P *= e.shape[i];
+        if ((e.shape[1] * P) % 64 == 0) {
+          periodic = true;
+          d.aper = (int)P;
+          d.aper_col = edr == 0 ? 0 : 1;   // vector 0 lost dim edr: it is indexed by the column if that dim is O
+          d.R0 = (int)e.shape[0];
+          d.C0 = (int)(e.shape[1] * P);
+        }
+      }
+      if ((wide && d.C0 % 64 == 0) || periodic) {
         d.atile_nct = d.C0 / 64;
         if (d.tile_rows == 0) d.tile_rows = tile_rows_for(kind);
         d.atile_ntask = d.atile_nct * ((d.R0 + d.tile_rows - 1) / d.tile_rows);
-        for (int b = 0; b * 4 < d.atile_ntask; ++b) L.ap_items.push_back(Item{t, b, 0, 0});
+        for (int b = 0; b * 4 < d.atile_ntask; ++b) (periodic ? L.pp_items : L.ap_items).push_back(Item{t, b, 0, 0});
       } else {
         for (long long c = 0; c * chunk < n; ++c) L.ga_items.push_back(Item{t, (int)c, 0, 0});
       }
@@ -567,6 +589,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_segtot = take(sizeof(double) * kStatW * L.seg_items.size());
   L.off_el_items = take(sizeof(Item) * L.el_items.size());
   L.off_ap_items = take(sizeof(Item) * L.ap_items.size());
+  L.off_pp_items = take(sizeof(Item) * L.pp_items.size());
   L.off_ga_items = take(sizeof(Item) * L.ga_items.size());
   L.off_fin_items = take(sizeof(Item) * L.fin_items.size());
   L.off_finpart = take(sizeof(double) * L.fin_items.size());
@@ -677,10 +700,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   P->kind = kind;
   P->T = n_tensors;
   P->mlp_on_matrix_pipe = env_matrix_pipe();
-  {
-    const char* e = getenv("PYLO_MI355_ADAFAC_F32");
-    P->adafac_bf = !(e && e[0] == '1');
-  }
+  P->adafac_bf = env_adafac_bf();
   if (int rc = build_layout(kind, shapes, n_tensors, P->L, kVeloHiddenMax)) { delete P; return rc; }
   if (workspace == nullptr || workspace_bytes < P->L.total) { delete P; return fail("plan_create: workspace too small"); }
   if (reinterpret_cast<uintptr_t>(workspace) % 256 != 0) { delete P; return fail("plan_create: workspace must be 256-byte aligned"); }
@@ -701,6 +721,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_seg_items, L.seg_items.data(), sizeof(Item) * L.seg_items.size());
   if (e == hipSuccess) e = up(L.off_el_items, L.el_items.data(), sizeof(Item) * L.el_items.size());
   if (e == hipSuccess) e = up(L.off_ap_items, L.ap_items.data(), sizeof(Item) * L.ap_items.size());
+  if (e == hipSuccess) e = up(L.off_pp_items, L.pp_items.data(), sizeof(Item) * L.pp_items.size());
   if (e == hipSuccess) e = up(L.off_ga_items, L.ga_items.data(), sizeof(Item) * L.ga_items.size());
   if (e == hipSuccess) e = up(L.off_fin_items, L.fin_items.data(), sizeof(Item) * L.fin_items.size());
   if (e == hipSuccess) e = up(L.off_fac_list, L.fac_list.data(), sizeof(int) * L.fac_list.size());
@@ -1466,10 +1487,14 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
   HIP_TRY(mark());
   const Item* ap_items = P->at<Item>(L.off_ap_items);
   const Item* ga_items = P->at<Item>(L.off_ga_items);
-  const int n_ap = (int)L.ap_items.size(), n_ga = (int)L.ga_items.size();
+  const Item* pp_items = P->at<Item>(L.off_pp_items);
+  const int n_ap = (int)L.ap_items.size(), n_ga = (int)L.ga_items.size(), n_pp = (int)L.pp_items.size();
   if (n_ga > 0)
     hipLaunchKernelGGL(k_adafac_apply, dim3(n_ga), dim3(kThreads), 0, s, descs, dyn, ga_items, fac_tab, term_tab, dec,
                        wfold, net, (const float*)bias_eff, gl);
+  if (n_pp > 0)
+    hipLaunchKernelGGL((k_adafac_apply_tile<true, true>), dim3(n_pp), dim3(kThreads), 0, s, descs, dyn, pp_items, fac_tab,
+                       term_tab, dec, wfold, net, gl);
   if (n_ap > 0) {
     if (P->adafac_bf)
       hipLaunchKernelGGL(k_adafac_apply_tile<true>, dim3(n_ap), dim3(kThreads), 0, s, descs, dyn, ap_items, fac_tab,

@@ -213,3 +213,48 @@ def test_mulo_wrapper_runs_the_fused_step_with_per_group_learning_rates():
     for x, y, v in zip(a, b, init):
         assert torch.equal(x, y)
         assert not torch.equal(x.cpu(), v)
+
+
+@pytest.mark.parametrize("cls_name", ["AdafacLO_CUDA", "ELO_CUDA"])
+def test_convolution_kernels_walked_as_matrices(cls_name):
+    """(O, I, k, ..) tensors whose two largest dims are the leading ones take the column-resident apply pass as the
+    matrix (O, I * k..): one statistics vector is indexed by the matrix column, the other by (row, column mod k..).
+    Covered: O > I, O < I, O == I (the tie goes to I), one and three trailing dims, a size-1 dim in between, rows
+    that do not fill the last tile; (8, 128, 3, 64) and (32, 16, 3, 3) stay on the generic path (factored dims
+    not leading / I * k * k not a multiple of 64)."""
+    from oracle import pylo_oracle as O
+    import pylo_amd
+    from pylo_amd.models import MetaMLP
+
+    torch.manual_seed(5)
+    net = MetaMLP(39, 32, 1)
+    shapes = [(64, 64, 3, 3), (96, 128, 3, 3), (128, 64, 3, 3), (40, 64, 5), (256, 32, 2, 2, 2), (8, 128, 3, 64),
+              (130, 64, 1, 3), (32, 16, 3, 3), (64, 128)]
+    gen = torch.Generator().manual_seed(31)
+    init = [torch.randn(s, generator=gen) * 0.3 for s in shapes]
+    cpu = [v.clone() for v in init]
+    gpu = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+    if cls_name == "ELO_CUDA":
+        kw = dict(lr=1e-2, weight_decay=0.05, exp_mult=0.01, clip_grad=True, clip_norm=2.0)
+        orc = O.EloOracle(cpu, net.state_dict(), **kw)
+        opt = pylo_amd.ELO_CUDA(gpu, network=copy.deepcopy(net), hf_key=None, **kw)
+    else:
+        orc = O.AdafacOracle(cpu, net.state_dict(), lr=0.5, weight_decay=1e-3)
+        opt = pylo_amd.AdafacLO_CUDA(gpu, lr=0.5, weight_decay=1e-3, network=copy.deepcopy(net))
+    worst = 0.0
+    for t in range(4):
+        grads = [torch.randn(s, generator=gen) * (10.0 ** (-(i % 3))) for i, s in enumerate(shapes)]
+        for p, g in zip(gpu, grads):
+            p.grad = g.cuda()
+        orc.step(grads)
+        opt.step()
+        for i, p in enumerate(gpu):
+            st, so = opt.state[p], orc.state[i]
+            checks = [("param", p, cpu[i]), ("exp_avg", st["exp_avg"], so["exp_avg"]),
+                      ("exp_avg_sq", st["exp_avg_sq"], so["exp_avg_sq"]),
+                      ("r", st["exp_avg_sq_r"], so["exp_avg_sq_r"]), ("c", st["exp_avg_sq_c"], so["exp_avg_sq_c"])]
+            for tag, got, ref in checks:
+                e = max_err(got, ref, REL, ABS)
+                worst = max(worst, e)
+                assert e <= 1.0, (cls_name, t, i, shapes[i], tag, e)
+    print(cls_name, "convolution kernels worst err/tol", worst)

@@ -477,13 +477,17 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
 // splitting the 16 features and the 2 x 16 hidden values a lane holds costs 5.5 instructions a value.
 //
 // Layouts (lane = 32 half + e): units are the M dimension, elements the N dimension, inputs the K
-// dimension.  A operand: lane holds inputs 8 half .. 8 half + 7 of unit e.  B operand: lane holds inputs
-// 8 half .. + 7 of element e of the group (two groups of 32 elements per wave row; a lane owns element
+// dimension.  A operand: lane holds reduction slots 8 half .. 8 half + 7 of unit e.  B operand: lane holds
+// slots 8 half .. + 7 of element e of the group (two groups of 32 elements per wave row; a lane owns element
 // 32 half + e, i.e. the lanes of one half own one group).  D: lane holds units 8 j + 4 half + i (j, i = 0..3)
-// of element e.  Lanes e and e + 32 hold complementary halves of what the other needs, both for the features
-// (own element, all 16 inputs) and for the hidden values (D -> B of the next layer): one
-// v_permlane32_swap per register (lanes 32..63 of the first operand change places with lanes 0..31 of the
-// second) puts everything where the next matrix instruction reads it; nothing goes through LDS.
+// of element e.
+// First layer: slot = input.  A lane has all 16 features of its own element and needs, per group, half of the
+// features of element e of that group: lanes e and e + 32 trade the halves the other needs, eight
+// v_permlane32_swap on the fp32 values (lanes 32..63 of the first operand change places with lanes 0..31 of the
+// second), before the split.
+// Hidden layer: which hidden unit a reduction slot stands for is free as long as both operands agree, so slot
+// 8 half + 4 q + i of step s is unit 8 (2 s + q) + 4 half + i: exactly the sixteen units the lane holds in D
+// after the first layer.  The hidden values never leave their lane; nothing goes through LDS.
 typedef __bf16 abf16x8 __attribute__((ext_vector_type(8)));
 typedef float av16f __attribute__((ext_vector_type(16)));
 typedef unsigned int au32x4 __attribute__((ext_vector_type(4)));
@@ -539,7 +543,8 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
                                                      const float* net) {
   const TileTask tk(d, task, d.atile_nct, 1);
   const int lane = threadIdx.x & 63, half = lane >> 5, el = lane & 31;
-  // A operands: first layer (unit el, inputs 8 half ..), hidden layer per reduction step s (inputs 16 s + 8 half ..)
+  // A operands: first layer (unit el, inputs 8 half ..), hidden layer per reduction step s (slot 8 half + 4 q + i:
+  // hidden unit 8 (2 s + q) + 4 half + i)
   au32x4 w1[3], w2[2][3];
   {
     float x[8];
@@ -549,7 +554,8 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) x[i] = *(const gfloat*)(net + kAWH + (16 * s + 8 * half + i) * kAH + el);
+      for (int i = 0; i < 8; ++i)
+        x[i] = *(const gfloat*)(net + kAWH + (8 * (2 * s + (i >> 2)) + 4 * half + (i & 3)) * kAH + el);
       bf3_pack8(x, w2[s]);
     }
   }
@@ -587,21 +593,36 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
         *m2 = a.mom + 2 * d.n + tk.first, *rms = a.rms + tk.first;
   const float* fr = fac_tab + pick(d.fac_off, pv) + (size_t)tk.r0 * 4 * per;
   const float* tr = term_tab + pick(d.term_off, pv) + (size_t)tk.r0 * kAH * per;
-  for (int r = tk.r0; r < tk.r1; ++r) {
-    float xg[1], xp[1], x0[1], x1[1], x2[1], xr_[1], fa[4];
-    load_vec_nt<1>(g, lo, xg);
-    load_vec_nt<1>(p, lo, xp);
-    load_vec_nt<1>(m0, lo, x0);
-    load_vec_nt<1>(m1, lo, x1);
-    load_vec_nt<1>(m2, lo, x2);
-    load_vec_nt<1>(rms, lo, xr_);
-    if constexpr (PER) load_vec_o<4>(fr, fa_off, fa);
-    else load_uniform<4>(fr, fa);
-    float ta[PER ? 2 : 1][4][4];
+  // Everything a row reads from memory.  The loop keeps one row in flight: the loads of row r + 1 are issued
+  // before row r is worked on (a wave shares its SIMD with one other wave only, too few to cover a memory round
+  // trip per row otherwise).
+  struct RowIn { float g[1], p[1], m0[1], m1[1], m2[1], rms[1], fa[4], ta[PER ? 2 : 1][4][4]; };
+  auto fetch = [&](RowIn& x, long long eo, const float* fr_, const float* tr_) {
+    load_vec_nt<1>(g + eo, lo, x.g);
+    load_vec_nt<1>(p + eo, lo, x.p);
+    load_vec_nt<1>(m0 + eo, lo, x.m0);
+    load_vec_nt<1>(m1 + eo, lo, x.m1);
+    load_vec_nt<1>(m2 + eo, lo, x.m2);
+    load_vec_nt<1>(rms + eo, lo, x.rms);
+    if constexpr (PER) load_vec_o<4>(fr_, fa_off, x.fa);
+    else load_uniform<4>(fr_, x.fa);
 #pragma unroll
     for (int gq = 0; gq < (PER ? 2 : 1); ++gq)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) load_vec_o<4>(tr + 8 * j, trow_off[gq], ta[gq][j]);
+      for (int j = 0; j < 4; ++j) load_vec_o<4>(tr_ + 8 * j, trow_off[gq], x.ta[gq][j]);
+  };
+  RowIn cur;
+  fetch(cur, 0, fr, tr);
+  for (int r = tk.r0; r < tk.r1; ++r) {
+    RowIn nxt;
+    {   // past the last row: the same row again, discarded
+      const bool more = r + 1 < tk.r1;
+      fetch(nxt, more ? d.C0 : 0, fr + (more ? 4 * per : 0), tr + (more ? kAH * per : 0));
+    }
+    float xg[1] = {cur.g[0]}, xp[1] = {cur.p[0]}, x0[1] = {cur.m0[0]}, x1[1] = {cur.m1[0]}, x2[1] = {cur.m2[0]},
+          xr_[1] = {cur.rms[0]};
+    const float (&fa)[4] = cur.fa;
+    const float (&ta)[PER ? 2 : 1][4][4] = cur.ta;
     const float gg = cond_grad(xg[0], d.gscale, a.clip_val, d.nan0);
     float m[3] = {x0[0], x1[0], x2[0]};
     ema_update(e, gg, m, xr_[0]);
@@ -613,22 +634,20 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
     const float rfcf[3] = {fa[0] * fb[0], fa[1] * fb[1], fa[2] * fb[2]};
     float f18[kNStat];
     lo_features(gg, xp[0], m, xr_[0], rfcf, 1e-6f, f18);
-    const float flo[8] = {f18[0], f18[2], f18[3], f18[4], f18[5], f18[6], f18[7], f18[8]};
-    const float fhi[8] = {f18[9], f18[10], f18[11], f18[12], f18[13], f18[15], f18[16], f18[17]};
-    // B operands of the first layer: after the swap xb[0] serves group 0 (lanes 0..31: their own inputs 0..7,
-    // lanes 32..63: inputs 8..15 of the element 32 lanes below), xb[1] group 1
+    float flo[8] = {f18[0], f18[2], f18[3], f18[4], f18[5], f18[6], f18[7], f18[8]};
+    float fhi[8] = {f18[9], f18[10], f18[11], f18[12], f18[13], f18[15], f18[16], f18[17]};
+    // B operands of the first layer: after the swap flo serves group 0 (lanes 0..31: their own inputs 0..7,
+    // lanes 32..63: inputs 8..15 of the element 32 lanes below), fhi group 1
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      unsigned u = __float_as_uint(flo[i]), v = __float_as_uint(fhi[i]);
+      half_swap(u, v);
+      flo[i] = __uint_as_float(u);
+      fhi[i] = __uint_as_float(v);
+    }
     au32x4 xb[2][3];
     bf3_pack8(flo, xb[0]);
     bf3_pack8(fhi, xb[1]);
-#pragma unroll
-    for (int q = 0; q < 3; ++q)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        unsigned u = xb[0][q][i], v = xb[1][q][i];
-        half_swap(u, v);
-        xb[0][q][i] = u;
-        xb[1][q][i] = v;
-      }
     float part[2][2];
 #pragma unroll
     for (int gq = 0; gq < 2; ++gq) {
@@ -652,18 +671,14 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
           hp[1][j][i] = bf_pack(u0.m, u1.m);
           hp[2][j][i] = bf_pack(u0.l, u1.l);
         }
-      // blocks (0, 1) and (2, 3) trade halves: afterwards lanes 0..31 hold units 16 s + 0..7, lanes 32..63
-      // units 16 s + 8..15 of their element, in order
+      // blocks 2 s and 2 s + 1 are the lane's eight slots of reduction step s as they stand
       av16f g2 = bh;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         au32x4 hb[3];
 #pragma unroll
-        for (int q = 0; q < 3; ++q) {
-#pragma unroll
-          for (int i = 0; i < 2; ++i) half_swap(hp[q][2 * s2][i], hp[q][2 * s2 + 1][i]);
+        for (int q = 0; q < 3; ++q)
           hb[q] = au32x4{hp[q][2 * s2][0], hp[q][2 * s2][1], hp[q][2 * s2 + 1][0], hp[q][2 * s2 + 1][1]};
-        }
         g2 = bf3_mfma(w2[s2], hb, g2);
       }
       float p0 = 0.0f, p1 = 0.0f;
@@ -688,6 +703,7 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
     store_vec_o<1>(p, lo, pn);
     g += d.C0; p += d.C0; m0 += d.C0; m1 += d.C0; m2 += d.C0; rms += d.C0;
     fr += 4 * per; tr += kAH * per;
+    cur = nxt;
   }
 }
 

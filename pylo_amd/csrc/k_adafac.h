@@ -648,43 +648,53 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
     au32x4 xb[2][3];
     bf3_pack8(flo, xb[0]);
     bf3_pack8(fhi, xb[1]);
-    float part[2][2];
+    // The two groups of 32 elements go through the layers a phase apart, so that the matrix instructions of one
+    // have the vector work of the other to run under: first layer of both, then per group split -> hidden layer,
+    // then the output layer (on the vector pipe) of both.
+    av16f h[2];
 #pragma unroll
     for (int gq = 0; gq < 2; ++gq) {
-      av16f h;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         float tb[4];
         load_vec_o<4>(tcol + (32 * gq) * kAH + 8 * j, tcol_off, tb);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) h[4 * j + i] = ta[PER ? gq : 0][j][i] + tb[i];
+        for (int i = 0; i < 4; ++i) h[gq][4 * j + i] = ta[PER ? gq : 0][j][i] + tb[i];
       }
-      h = bf3_mfma(w1, xb[gq], h);
+      h[gq] = bf3_mfma(w1, xb[gq], h[gq]);
+    }
+    av16f g2[2];
+#pragma unroll
+    for (int gq = 0; gq < 2; ++gq) {
       // hidden values of the units this lane holds -> planes, four units (two dwords) per block j
       unsigned hp[3][4][2];
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-          const Bf3 u0 = bf3_split(relu(h[4 * j + 2 * i])), u1 = bf3_split(relu(h[4 * j + 2 * i + 1]));
+          const Bf3 u0 = bf3_split(relu(h[gq][4 * j + 2 * i])), u1 = bf3_split(relu(h[gq][4 * j + 2 * i + 1]));
           hp[0][j][i] = bf_pack(u0.h, u1.h);
           hp[1][j][i] = bf_pack(u0.m, u1.m);
           hp[2][j][i] = bf_pack(u0.l, u1.l);
         }
       // blocks 2 s and 2 s + 1 are the lane's eight slots of reduction step s as they stand
-      av16f g2 = bh;
+      g2[gq] = bh;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         au32x4 hb[3];
 #pragma unroll
         for (int q = 0; q < 3; ++q)
           hb[q] = au32x4{hp[q][2 * s2][0], hp[q][2 * s2][1], hp[q][2 * s2 + 1][0], hp[q][2 * s2 + 1][1]};
-        g2 = bf3_mfma(w2[s2], hb, g2);
+        g2[gq] = bf3_mfma(w2[s2], hb, g2[gq]);
       }
+    }
+    float part[2][2];
+#pragma unroll
+    for (int gq = 0; gq < 2; ++gq) {
       float p0 = 0.0f, p1 = 0.0f;
 #pragma unroll
       for (int r2 = 0; r2 < 16; ++r2) {
-        const float gv = relu(g2[r2]);
+        const float gv = relu(g2[gq][r2]);
         p0 = fmaf(gv, wo[r2][0], p0);
         p1 = fmaf(gv, wo[r2][1], p1);
       }

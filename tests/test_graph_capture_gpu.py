@@ -168,7 +168,7 @@ def test_velo_step_replays_from_a_graph():
         assert max_err(a.cpu(), b.cpu(), REL, ABS) <= 1.0
 
 
-@pytest.mark.parametrize("which", ["adafac", "elo"])
+@pytest.mark.parametrize("which", ["adafac", "adafac max_grad_norm", "elo"])
 def test_adafac_family_step_replays_from_a_graph(which):
     from pylo_amd import AdafacLO_CUDA, ELO_CUDA
     from pylo_amd.models import MetaMLP
@@ -178,8 +178,9 @@ def test_adafac_family_step_replays_from_a_graph(which):
     shapes = [(48, 40), (40,), (6, 4, 3, 3), (40, 72)]
 
     def make(params, capturable):
-        if which == "adafac":
-            return AdafacLO_CUDA(params, lr=0.5, weight_decay=0.01, network=net, hf_key=None, capturable=capturable)
+        if which.startswith("adafac"):      # with max_grad_norm every tensor is clipped against its own norm in the call
+            return AdafacLO_CUDA(params, lr=0.5, weight_decay=0.01, network=net, hf_key=None, capturable=capturable,
+                                 max_grad_norm=0.3 if "max_grad_norm" in which else None)
         return ELO_CUDA(params, lr=1e-2, weight_decay=0.01, clip_grad=True, clip_norm=0.5, network=net, hf_key=None,
                         capturable=capturable)
 

@@ -66,6 +66,18 @@ def test_workspace_sizing_and_error_paths_without_gpu():
         mixed = _lib.make_shapes([(64, 128), (128,), (4, 3, 5)], fl)
         assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_ADAFAC, mixed, 3, C.byref(n)) != 0
         assert b"PYLO_F_GLOBAL_NORM" in lib.pylo_mi355_last_error()
+    # per-tensor norm clipping (AdafacLO's max_grad_norm): all-or-none too, AdafacLO plans only, and not together
+    # with the global norm or nan_to_num
+    tn = _lib.F_TENSOR_NORM
+    ok = _lib.make_shapes([(64, 128), (128,), (4, 3, 5)], [tn, tn, tn])
+    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_ADAFAC, ok, 3, C.byref(n)) == 0
+    assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_VELO, ok, 3, C.byref(n)) != 0
+    assert b"AdafacLO plans" in lib.pylo_mi355_last_error()
+    for fl, msg in (([tn, 0, tn], b"every tensor"), ([0, tn, tn], b"every tensor"),
+                    ([tn | _lib.F_GLOBAL_NORM] * 3, b"does not combine"), ([tn | _lib.F_NAN_TO_NUM] * 3, b"does not combine")):
+        bad = _lib.make_shapes([(64, 128), (128,), (4, 3, 5)], fl)
+        assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_ADAFAC, bad, 3, C.byref(n)) != 0
+        assert b"PYLO_F_TENSOR_NORM" in lib.pylo_mi355_last_error() and msg in lib.pylo_mi355_last_error()
     # tensors with more than two dims are fine for every kind
     nd = _lib.make_shapes([(768, 3, 16, 16)], [0])
     for kind in (_lib.KIND_VELO, _lib.KIND_ADAFAC, _lib.KIND_CELO2):

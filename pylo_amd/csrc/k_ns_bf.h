@@ -349,7 +349,8 @@ struct NsTileItem { int mat, tr, tc; };
 __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__ mats, const NsTileItem* __restrict__ items,
                                                      const PyloTensorArgs* __restrict__ dyn, const float* __restrict__ scale,
                                                      bfbits* __restrict__ pw) {
-  __shared__ bfbits tile[3][64][66];
+  constexpr int RP = 72;   // bf16 per row of the tile in LDS: 64 + 8, rows stay 16-byte aligned
+  __shared__ __attribute__((aligned(16))) bfbits tile[3][64][RP];
   const NsTileItem it = items[blockIdx.x];
   const NsBfMat mt = mats[it.mat];
   const PyloTensorArgs a = dyn[mt.tensor];
@@ -361,49 +362,61 @@ __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__
   bfbits* transp = pw + (mt.tall ? mt.off_xs : mt.off_xl[0]);
   const int r0 = it.tr * 64, c0 = it.tc * 64;
   const int t = threadIdx.x;
+  // Eight consecutive columns of one row a lane and pass: 32 bytes read, one 16-byte piece per plane written
+  // to the direct planes (the two lanes of a 16-column block fill its 96 bytes) and to the tile in LDS.
+  // Columns and rows past the matrix read as zero; where a piece straddles the edge (C or R a multiple of 4
+  // only) the zeros land in the planes' padding, which holds zeros anyway.
 #pragma unroll
-  for (int pass = 0; pass < 4; ++pass) {
-    const int lr = pass * 16 + (t >> 4), lc = 4 * (t & 15);
+  for (int pass = 0; pass < 2; ++pass) {
+    const int u = pass * 256 + t, lr = u >> 3, lc = 8 * (u & 7);
     const int r = r0 + lr, c = c0 + lc;
-    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    const bool in = r < R && c < C;   // C is a multiple of 4
+    float v[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    const bool in = r < R && c < C;
     if (in) {
-      const v4f x = *(const gv4f*)(a.step_out + (size_t)r * C + c);
+      const float* src = a.step_out + (size_t)r * C + c;
+      const v4f x = *(const gv4f*)src;
       v[0] = x.x * s; v[1] = x.y * s; v[2] = x.z * s; v[3] = x.w * s;
+      if (c + 4 < C) {
+        const v4f y = *(const gv4f*)(src + 4);
+        v[4] = y.x * s; v[5] = y.y * s; v[6] = y.z * s; v[7] = y.w * s;
+      }
     }
-    bfbits h[4], m[4], l[4];
+    u32x4 pl[3];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) bf_split(v[q], h[q], m[q], l[q]);
-    // two values a store (lc is even and the row pitch is 33 dwords: 4-byte aligned)
-    typedef unsigned int u32;
-#pragma unroll
-    for (int q = 0; q < 4; q += 2) {
-      *(u32*)&tile[0][lr][lc + q] = (u32)h[q] | (u32)h[q + 1] << 16;
-      *(u32*)&tile[1][lr][lc + q] = (u32)m[q] | (u32)m[q + 1] << 16;
-      *(u32*)&tile[2][lr][lc + q] = (u32)l[q] | (u32)l[q + 1] << 16;
+    for (int q = 0; q < 4; ++q) {
+      bfbits h0, m0, l0, h1, m1, l1;
+      bf_split(v[2 * q], h0, m0, l0);
+      bf_split(v[2 * q + 1], h1, m1, l1);
+      pl[0][q] = (unsigned)h0 | (unsigned)h1 << 16;
+      pl[1][q] = (unsigned)m0 | (unsigned)m1 << 16;
+      pl[2][q] = (unsigned)l0 | (unsigned)l1 << 16;
     }
+#pragma unroll
+    for (int q = 0; q < 3; ++q) *(luint4*)&tile[q][lr][lc] = pl[q];
     if (in) {
-      typedef unsigned long long u64;
       bfbits* p = direct + bf_off(R, r, c);
-      *(u64*)p = (u64)h[0] | (u64)h[1] << 16 | (u64)h[2] << 32 | (u64)h[3] << 48;
-      *(u64*)(p + 16) = (u64)m[0] | (u64)m[1] << 16 | (u64)m[2] << 32 | (u64)m[3] << 48;
-      *(u64*)(p + 32) = (u64)l[0] | (u64)l[1] << 16 | (u64)l[2] << 32 | (u64)l[3] << 48;
+#pragma unroll
+      for (int q = 0; q < 3; ++q) *(u32x4*)(p + 16 * q) = pl[q];
     }
   }
   __syncthreads();
-  // transposed: thread takes column lc2 and four consecutive rows (rows past R were stored as zeros: padding)
+  // transposed: a lane takes one column and sixteen rows of the tile, i.e. one row and one 16-step block of
+  // the transposed planes: 96 consecutive bytes, and the lanes of a wave (consecutive columns) the next 96
+  {
+    const int lc = t & 63, rb = t >> 6;
+    const int c = c0 + lc, r = r0 + 16 * rb;
+    if (c < C && r < R) {
+      bfbits* p = transp + bf_off(C, c, r);
 #pragma unroll
-  for (int pass = 0; pass < 4; ++pass) {
-    const int lc2 = pass * 16 + (t >> 4), lr2 = 4 * (t & 15);
-    const int c = c0 + lc2, r = r0 + lr2;
-    if (c >= C || r >= R) continue;
-    typedef unsigned long long u64;
-    bfbits* p = transp + bf_off(C, c, r);
+      for (int q = 0; q < 3; ++q)
 #pragma unroll
-    for (int q = 0; q < 3; ++q) {
-      const u64 w = (u64)tile[q][lr2][lc2] | (u64)tile[q][lr2 + 1][lc2] << 16 | (u64)tile[q][lr2 + 2][lc2] << 32 |
-                    (u64)tile[q][lr2 + 3][lc2] << 48;
-      *(u64*)(p + 16 * q) = w;
+        for (int hf = 0; hf < 2; ++hf) {
+          u32x4 w;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            w[i] = (unsigned)tile[q][16 * rb + 8 * hf + 2 * i][lc] | (unsigned)tile[q][16 * rb + 8 * hf + 2 * i + 1][lc] << 16;
+          *(u32x4*)(p + 16 * q + 8 * hf) = w;
+        }
     }
   }
 }

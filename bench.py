@@ -79,7 +79,7 @@ def make_inputs(shapes, device, seed=0):
     return params, grads
 
 
-def cpu_baseline(steps=6):
+def cpu_baseline(steps=14):
     """The oracle (CPU restatement of the reference's naive PyTorch path) on one transformer
     layer of the same workload, host cores of this box."""
     import torch

@@ -1,6 +1,6 @@
 """Benchmark of the fused learned-optimizer step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gpt2s|cfg1|vit_velo|llama_adafac|stream_ceiling] [--fused-only]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gpt2s|cfg1|vit_velo|llama_adafac|stress_velo|stress_celo2|stream_ceiling] [--fused-only]
 
 Workload (default): BASELINE config 2 -- ELO-CELO2 on a GPT-2-small-shaped fp32 parameter set
 (98 tensors, 124 355 328 parameters), synthetic per-tensor Gaussian gradients with log-uniform
@@ -60,6 +60,25 @@ def llama_1b_shapes(layers=22):
         shapes += [(2048,), (2048, 2048), (2048, 256), (2048, 256), (2048, 2048), (2048,),
                    (2048, 5632), (2048, 5632), (5632, 2048)]
     return shapes + [(32000, 2048)]
+
+
+def stress_shapes(n_tensors=3000, seed=11, embedding=(32000, 4096)):
+    """BASELINE config 5: tensors of 1 .. 65 536 elements drawn log-uniform, 1-D and 2-D with odd dims mixed, plus one
+    32000 x 4096 embedding (the generator of tests/test_many_tensors_gpu.py)."""
+    import math
+
+    import torch
+
+    gen = torch.Generator().manual_seed(seed)
+    shapes = [(37, 4099), (4099, 37)]
+    while len(shapes) < n_tensors:
+        n = max(int(math.exp(float(torch.rand((), generator=gen)) * math.log(65536.0))), 1)
+        if float(torch.rand((), generator=gen)) < 0.4:
+            shapes.append((n,))
+        else:
+            r = max(1, int(math.exp(float(torch.rand((), generator=gen)) * math.log(n))))
+            shapes.append((r, max(1, n // r)))
+    return shapes + [embedding]
 
 
 def layer_sample_shapes():
@@ -180,7 +199,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gpt2s", choices=["gpt2s", "cfg1", "vit_velo", "llama_adafac", "stream_ceiling"])
+    ap.add_argument("--workload", default="gpt2s", choices=["gpt2s", "cfg1", "vit_velo", "llama_adafac", "stress_velo", "stress_celo2", "stream_ceiling"])
     ap.add_argument("--fused-only", action="store_true",
                     help="loop the C-ABI call alone (no Newton-Schulz / apply), e.g. under rocprofv3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -199,6 +218,9 @@ def main():
     from pylo_amd import ELO_CELO2_CUDA
     from pylo_amd.models import CELO2MLP
 
+    if a.workload in ("stress_velo", "stress_celo2"):
+        print(json.dumps(stress_workload(a.workload, a.steps, a.warmup)))
+        return
     if a.workload in ("vit_velo", "llama_adafac"):
         print(json.dumps(other_workload(a.workload, a.steps, a.warmup)))
         return
@@ -359,6 +381,61 @@ def stream_ceiling(a):
             out[f"{name}{', non-temporal' if nt else ''}"] = {"ms": ms, "GBps": (r + w) * 4.0 * n / ms / 1e6}
     print(json.dumps({"metric": "attainable_hbm_rate_by_access_mix", "unit": "GB/s", "n_gpus": 1, "steps": a.steps,
                       "warmup": a.warmup, "elements_per_array": n, "peak_GBps": HBM_PEAK_GBS, "mixes": out}))
+
+
+def stress_workload(workload, steps, warmup):
+    """Config 5 (3 000 small tensors + one 32000 x 4096 embedding, Student-t gradients): the fused VeLO step or the
+    fused ELO-CELO2 element call.  What it measures is the multi-tensor launch table: how long the host takes to
+    enqueue a step (argument table of 3 001 rows) against how long the GPU takes to run it, and the launches."""
+    import torch
+
+    from pylo_amd import ELO_CELO2_CUDA, VeLO_CUDA
+    from pylo_amd.models import CELO2MLP, VeLOMLP, VeLORNN
+
+    dev = torch.device("cuda:0")
+    shapes = stress_shapes()
+    gen = torch.Generator(device=dev).manual_seed(1)
+    params = [torch.nn.Parameter(torch.randn(s, generator=gen, device=dev) * 0.02) for s in shapes]
+    torch.manual_seed(2)
+    t3 = torch.distributions.StudentT(torch.tensor(3.0, device=dev))
+    for p in params:
+        p.grad = t3.sample(p.shape) * 1e-3
+    torch.manual_seed(1)
+    if workload == "stress_velo":
+        opt = VeLO_CUDA(params, lr=1e-3, num_steps=1000, rnn=VeLORNN(), mlp=VeLOMLP())
+        loss = torch.tensor(1.0, device=dev)
+        step = lambda: opt.step(loss)
+        label = "VeLO fused step"
+    else:
+        opt = ELO_CELO2_CUDA(params, lr=3e-4, network=CELO2MLP(), hf_key=None)
+        step = opt.fused_step
+        label = "ELO_CELO2 fused element call (no Newton-Schulz)"
+    # (one call around the tenth in flight takes 0.1 s on the host, once; it is kept out of the timed region)
+    for _ in range(max(warmup, 16)):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    t1 = time.perf_counter()
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    plan = opt._plan
+    plan.timing_begin(steps)
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    per = plan.timing_end()
+    n = sum(p.numel() for p in params)
+    ms = (t2 - t0) * 1e3 / steps
+    return {"metric": "params_updated_per_sec (fused step, C-ABI call)", "value": n / (ms * 1e-3), "unit": "params/s",
+            "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": f"{label}, stress set of {len(shapes)} tensors (3 000 of 1 - 65 536 elements, 1-D and odd "
+                                   f"2-D, plus 32000 x 4096)", "params": n, "tensors": len(shapes)},
+            "host_enqueue_ms_per_step": (t1 - t0) * 1e3 / steps,
+            "sum_of_launch_intervals_ms": float(per.sum(axis=1).mean()),
+            "launch_ms": {nm: float(v) for nm, v in zip(plan.launch_names(), per.mean(axis=0))}}
 
 
 def other_workload(workload, steps, warmup):

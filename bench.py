@@ -499,8 +499,8 @@ def other_workload(workload, steps, warmup):
     if workload == "llama_adafac":
         # The 16 -> 32 -> 32 -> 2 element MLP: 1 600 FMAs per element of a >= 2-D tensor.  By default its two
         # wide layers (1 536 FMAs) run on the bf16 matrix instructions with three-plane operands, six bf16
-        # products per fp32 product, and the kernel is bound by what one SIMD can issue: matrix and vector
-        # instructions do not overlap on it (the splitting of the activations is vector work);
+        # products per fp32 product, and the kernel is bound by its vector instructions (the splitting of the
+        # activations is vector work; the bf16 matrix instructions run under it about half of the time);
         # PYLO_MI355_ADAFAC_F32=1 runs the layers on the fp32 matrix instructions.
         t = float(mean[k]) * 1e-3
         f32 = os.environ.get("PYLO_MI355_ADAFAC_F32") == "1"

@@ -473,7 +473,8 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
 // sums is, up to 2^-25 of itself, the six products h h, h m, m h, m m, h l, l h, each exact in fp32.  One
 // v_mfma_f32_32x32x16_bf16 does sixteen times the multiply-adds of v_mfma_f32_16x16x4_f32 in the same 32
 // cycles, so six of them per fp32 product leave 36 matrix instructions per row of 64 elements where the
-// fp32 instructions need 96; the price is vector work (this SIMD executes either kind, never both at once):
+// fp32 instructions need 96; the price is vector work (bf16 matrix instructions run under vector instructions of
+// the SIMD's waves about half of the time, fp32 ones never did, but the vector pipe is what fills up):
 // splitting the 16 features and the 2 x 16 hidden values a lane holds costs 5.5 instructions a value.
 //
 // Layouts (lane = 32 half + e): units are the M dimension, elements the N dimension, inputs the K

@@ -470,7 +470,8 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
 // ---- the same pass with the element MLP on the bf16 matrix instructions at fp32 accuracy ----------------
 // An fp32 number is the exact sum of three bf16 numbers (8 + 8 + 8 significand bits; taken by truncation:
 // h = x & 0xffff0000, m = (x - h) & 0xffff0000, l = x - h - m, every step exact), and a product of two such
-// sums is, up to 2^-25 of itself, the six products h h, h m, m h, m m, h l, l h, each exact in fp32.  One
+// sums is, up to 2^-23 of itself (2^-25 on average), the six products h h, h m, m h, m m, h l, l h, each exact
+// in fp32.  One
 // v_mfma_f32_32x32x16_bf16 does sixteen times the multiply-adds of v_mfma_f32_16x16x4_f32 in the same 32
 // cycles, so six of them per fp32 product leave 36 matrix instructions per row of 64 elements where the
 // fp32 instructions need 96; the price is vector work (bf16 matrix instructions run under vector instructions of

@@ -112,7 +112,9 @@ typedef struct {
   float lr;          /* VeLO / AdafacLO: lr applied in-kernel; CELO2 AdamW branch: adam lr   */
   float weight_decay;/* VeLO / AdafacLO: p -= wd*lr*p after the update; CELO2 AdamW: adam wd */
   float clip_norm;   /* CELO2, AdafacLO kind (ELO_cuda.py:153-161): global-norm clip threshold over
-                        the gradients of the call, 0 = clipping off for this tensor            */
+                        the gradients of the call, 0 = clipping off for this tensor; on tensors
+                        flagged PYLO_F_TENSOR_NORM: the bound on the tensor's own gradient norm
+                        (AdafacLO_cuda.py:214-215)                                              */
   float clip_val;    /* element-wise clamp of the gradient (1000 in the reference), 0 = off  */
   float exp_mult;
   float step_mult;
@@ -304,6 +306,8 @@ int pylo_mi355_plan_invalidate_statistics(PyloPlan* plan);
  *   p -= lr * o0 * exp(o1 * exp_mult) * step_mult;  then p -= weight_decay * lr * p.
  * ELO_CUDA (pylo/optim/ELO_cuda.py:179-288) runs on the same call: raw decays in `decays`, step_mult = 1,
  * clip_norm > 0 for global-norm clipping, and the tensor flags PYLO_F_NAN_TO_NUM | PYLO_F_WD_PRESTEP.
+ * AdafacLO_CUDA's max_grad_norm (AdafacLO_cuda.py:214-215): clip_norm = max_grad_norm on a plan whose tensors
+ * carry PYLO_F_TENSOR_NORM.
  */
 int pylo_mi355_adafac_step(PyloPlan* plan, const PyloTensorArgs* args, const PyloDecays* decays,
                            const float* net, float step, void* stream);

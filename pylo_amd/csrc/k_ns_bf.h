@@ -16,9 +16,13 @@
 //                                         or as fp32 in the tensor's own layout after the last iteration
 // for wide and tall matrices alike (B' is symmetric, so (B' X)^T = X^T B').
 //
-// Tile job: 128 x 128 outputs by 256 threads = 2 x 2 waves of 64 x 64 = 2 x 2 accumulators of 32 x 32;
-// 16 reduction steps per stage, double buffered in LDS (48 KB), one 16-byte read per lane, plane and
-// 32-row block per stage.
+// Tile job: 128 x 128 (Gram, Poly, narrow updates) or 128 x 256 outputs (updates with m > 128) by 256 threads =
+// 2 x 2 waves of 64 x 64 / 64 x 128 = 2 x 2 / 2 x 4 accumulators of 32 x 32; 16 reduction steps per stage,
+// double buffered in LDS (48 / 72 KB), staged from global memory straight into LDS (global_load_lds_dwordx4: no
+// staging registers, no LDS store instructions), one 16-byte read per lane, plane and 32-row block per stage.
+// The planes are allocated with their rows rounded up to whole tiles and the padding holds zeros, so the main
+// loop has no bounds checks; any two dims are taken (the raw step is read and the result written per element
+// where the tensor's rows are not 16-byte aligned).
 #pragma once
 
 #include "k_ns.h"
@@ -31,8 +35,8 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) u32x4 luint4;
 
 constexpr int kBfBK = 16;                     // reduction steps per stage
-constexpr int kBfOperandLds = kNsTile * 96;   // bytes of one operand's stage: 128 rows x 3 planes x 32 B
-constexpr int kBfStageLds = 2 * kBfOperandLds;   // 24 KB
+// LDS of a tile job with 64 WN columns: two stages of (128 + 64 WN) rows x 3 planes x 32 bytes
+constexpr int bf_gemm_lds(int wn) { return 2 * (128 + 64 * wn) * 96; }
 
 // Planes of one matrix with `rows` rows and a (padded) reduction length: stored in blocks of 16 reduction
 // steps, [k / 16][row][plane][k % 16], so that the 128 rows x 3 planes x 16 steps a tile job stages at a
@@ -40,7 +44,7 @@ constexpr int kBfStageLds = 2 * kBfOperandLds;   // 24 KB
 // out of every row and each 128-byte line was fetched from L2 four times).
 struct BfPlanes {
   const bfbits* base;
-  int rows;   // rows that exist; a tile's rows past them read as zero
+  int rows;   // rows allocated (a multiple of the tiles' rows; rows past the matrix hold zeros)
 };
 
 // element offset of (row, k) in plane 0; planes 1 and 2 are 16 and 32 elements further
@@ -52,12 +56,15 @@ struct NsBfMat {
   int tensor;
   int R, C, m, n, tall;      // X is R x C row-major; m = min, n = max; tall: R > C
   int pad_m, pad_n;          // m and n rounded up to the 16 reduction steps of a stage (the padding holds zeros)
+  int rows_m, rows_n;        // rows allocated for the planes whose rows are the m / n index (whole tiles)
+  int lda;                   // row pitch of the fp32 A and of the partial matrices: m rounded up to 4
   int n_slabs;
   long long off_xs;          // elements (bfbits) into the plane workspace: planes of Xs (m rows, reduction n)
   long long off_xl[2];       // planes of Xl (n rows, reduction m), two buffers (a product reads one and writes the other)
   long long off_pa, off_pb;  // planes of A and B' (m rows, reduction m)
   long long off_a;           // floats into the fp32 workspace: A (m x m)
   long long off_part;        // floats: partial matrices of a split Gram product
+  long long elem_off;        // elements from the tensor's raw step to this matrix (a slice of a tensor with more dims)
 };
 
 __device__ __forceinline__ float bf_to_float(bfbits b) { return __uint_as_float((unsigned)b << 16); }
@@ -76,57 +83,65 @@ __device__ __forceinline__ void bf_split(float x, bfbits& h, bfbits& m, bfbits& 
 
 // A stage of one operand in LDS: [row][plane][half], 96 bytes a row, as in memory, except that the two
 // 16-byte halves are swapped for every other group of eight rows (rows 8 apart would share banks).
-__device__ __forceinline__ int bf_lds_piece(int row, int plane, int half) {
-  return row * 96 + plane * 32 + 16 * (half ^ ((row >> 3) & 1));
-}
+// A wave-wide load instruction moves 64 consecutive 16-byte pieces of the stage from global memory into LDS
+// (the hardware puts lane l's piece at the instruction's LDS base + 16 l); the swap is done on the global
+// side: lane l fetches the piece whose place in LDS it fills.  ROWS x 6 pieces = ROWS x 6 / 256 instructions
+// per thread; `off[]` holds the lane's byte offsets into the stage in memory (they do not change with k).
+#define PYLO_LDS __attribute__((address_space(3)))
+#define PYLO_GLB __attribute__((address_space(1)))
 
-// One operand's stage from global memory into registers: the 768 pieces of 16 bytes are consecutive in
-// memory; thread t takes pieces t, t + 256, t + 512.
-__device__ __forceinline__ void bf_load_stage(const BfPlanes& P, int row0, int k, u32x4 (&reg)[3]) {
-  const bfbits* p = P.base + ((size_t)(k >> 4) * P.rows + row0) * 48;
+template <int ROWS>
+__device__ __forceinline__ void bf_stage_offsets(int wave, int lane, int (&off)[ROWS * 6 / 256]) {
 #pragma unroll
-  for (int j = 0; j < 3; ++j) {
-    const int g = threadIdx.x + 256 * j;
-    reg[j] = row0 + g / 6 < P.rows ? *(const u32x4*)(p + (size_t)g * 8) : u32x4{0u, 0u, 0u, 0u};
+  for (int j = 0; j < ROWS * 6 / 256; ++j) {
+    const int p = (j * 4 + wave) * 64 + lane;
+    off[j] = (p ^ (((p / 6) >> 3) & 1)) * 16;
   }
 }
 
-__device__ __forceinline__ void bf_store_stage(char __attribute__((address_space(3)))* lds, const u32x4 (&reg)[3]) {
+template <int ROWS>
+__device__ __forceinline__ void bf_stage_issue(const char* g, const int (&off)[ROWS * 6 / 256], PYLO_LDS char* lds, int wave) {
 #pragma unroll
-  for (int j = 0; j < 3; ++j) {
-    const int g = threadIdx.x + 256 * j, row = g / 6, rem = g - 6 * row;
-    *(luint4*)(lds + bf_lds_piece(row, rem >> 1, rem & 1)) = reg[j];
-  }
+  for (int j = 0; j < ROWS * 6 / 256; ++j)
+    __builtin_amdgcn_global_load_lds((const PYLO_GLB void*)(g + off[j]), (PYLO_LDS void*)(lds + (j * 4 + wave) * 1024), 16, 0, 0);
 }
 
-// acc[hi][hj] += (rows i0.. of P1) x (rows j0.. of P2)^T over the reduction range [k0, k1) (multiples of 16)
+// acc[hi][hj] += (rows i0.. of P1) x (rows j0.. of P2)^T over the reduction range [k0, k1) (multiples of 16);
+// 128 rows of P1, 64 WN rows of P2.  LDS: two stages of (128 + 64 WN) x 96 bytes.
+template <int WN>
 __device__ __forceinline__ void bf_tile_product(const BfPlanes& P1, int i0, const BfPlanes& P2, int j0, int k0, int k1,
-                                                char __attribute__((address_space(3)))* lds, v16f (&acc)[2][2]) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;
+                                                PYLO_LDS char* lds, v16f (&acc)[2][WN]) {
+  constexpr int RB = 64 * WN, SA = 128 * 96, STAGE = SA + RB * 96;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wi = (wave >> 1) * 64, wj = (wave & 1) * 32 * WN;
   const int kg = lane >> 5, lo = lane & 31;
-  u32x4 ra[3], rb[3];
-  bf_load_stage(P1, i0, k0, ra);
-  bf_load_stage(P2, j0, k0, rb);
-  bf_store_stage(lds, ra);
-  bf_store_stage(lds + kBfOperandLds, rb);
+  int offa[3], offb[RB * 6 / 256];
+  bf_stage_offsets<128>(wave, lane, offa);
+  bf_stage_offsets<RB>(wave, lane, offb);
+  const char* ga = (const char*)P1.base + ((size_t)(k0 >> 4) * P1.rows + i0) * 96;
+  const char* gb = (const char*)P2.base + ((size_t)(k0 >> 4) * P2.rows + j0) * 96;
+  const size_t sa = (size_t)P1.rows * 96, sb = (size_t)P2.rows * 96;
+  bf_stage_issue<128>(ga, offa, lds, wave);
+  bf_stage_issue<RB>(gb, offb, lds + SA, wave);
+  __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
+  const int sw = 16 * (kg ^ ((lo >> 3) & 1));
+  const int oa = (wi + lo) * 96 + sw, ob = SA + (wj + lo) * 96 + sw;
   int cur = 0;
-  const int oa0 = bf_lds_piece(wi + lo, 0, kg), oa1 = bf_lds_piece(wi + 32 + lo, 0, kg);
-  const int ob0 = kBfOperandLds + bf_lds_piece(wj + lo, 0, kg), ob1 = kBfOperandLds + bf_lds_piece(wj + 32 + lo, 0, kg);
   for (int k = k0; k < k1; k += kBfBK) {
-    const bool more = k + kBfBK < k1;
-    if (more) {
-      bf_load_stage(P1, i0, k + kBfBK, ra);
-      bf_load_stage(P2, j0, k + kBfBK, rb);
+    if (k + kBfBK < k1) {
+      ga += sa;
+      gb += sb;
+      bf_stage_issue<128>(ga, offa, lds + (STAGE - cur), wave);
+      bf_stage_issue<RB>(gb, offb, lds + (STAGE - cur) + SA, wave);
     }
-    bf16x8 a[2][3], b[2][3];
+    bf16x8 a[2][3], b[WN][3];
 #pragma unroll
     for (int q = 0; q < 3; ++q) {
-      a[0][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + q * 32 + oa0));
-      a[1][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + q * 32 + oa1));
-      b[0][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + q * 32 + ob0));
-      b[1][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + q * 32 + ob1));
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[i][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + oa + i * 32 * 96 + q * 32));
+#pragma unroll
+      for (int j = 0; j < WN; ++j) b[j][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + ob + j * 32 * 96 + q * 32));
     }
     // smallest terms first: l h, h l, m m, m h, h m, h h
 #pragma unroll
@@ -135,15 +150,14 @@ __device__ __forceinline__ void bf_tile_product(const BfPlanes& P1, int i0, cons
 #pragma unroll
       for (int hi = 0; hi < 2; ++hi)
 #pragma unroll
-        for (int hj = 0; hj < 2; ++hj)
+        for (int hj = 0; hj < WN; ++hj)
           acc[hi][hj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[hi][pa[term]], b[hj][pb[term]], acc[hi][hj], 0, 0, 0);
     }
-    if (more) {
-      bf_store_stage(lds + (kBfStageLds - cur), ra);
-      bf_store_stage(lds + (kBfStageLds - cur) + kBfOperandLds, rb);
-    }
+    // the loads into the other stage have landed (they are counted like any other vector-memory load) and
+    // every wave has read this one
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    cur = kBfStageLds - cur;
+    cur = STAGE - cur;
   }
 }
 
@@ -168,42 +182,40 @@ __device__ __forceinline__ void bf_store1(bfbits* base, int rows, int row, int k
   p[32] = l;
 }
 
-// The block's 128 x 128 values (accumulator layout) into planes whose reduction index is the tile's column
+// The block's 128 x 64 WN values (accumulator layout) into planes whose reduction index is the tile's column
 // index.  Four passes of 16 rows per wave: every lane splits its values and drops the halves into the
-// wave's own LDS patch ([row][plane][64 columns], 2 bytes each), then the wave reads the patch back as
+// wave's own LDS patch ([row][plane][32 WN columns], 2 bytes each), then the wave reads the patch back as
 // 16-byte pieces in the order the planes have in memory ([16 columns][row][plane][half]) and stores them.
-constexpr int kBfPatchPlane = 144;                 // bytes: 64 columns x 2 + 16 (bank spread)
-constexpr int kBfPatchRow = 3 * kBfPatchPlane;
-constexpr int kBfPatchWave = 16 * kBfPatchRow;     // 6912 bytes per wave
-
-__device__ __forceinline__ void bf_store_direct(char __attribute__((address_space(3)))* lds, const v16f (&acc)[2][2],
-                                                bfbits* __restrict__ D, int rows_total, int i0, int j0, int n_rows,
-                                                int n_cols) {
-  typedef __attribute__((address_space(3))) bfbits lbf;
+template <int WN>
+__device__ __forceinline__ void bf_store_direct(PYLO_LDS char* lds, const v16f (&acc)[2][WN], bfbits* __restrict__ D,
+                                                int rows_total, int i0, int j0, int n_rows, int n_cols) {
+  constexpr int kPlane = 64 * WN + 16;        // bytes: 32 WN columns x 2 + 16 (bank spread)
+  constexpr int kRow = 3 * kPlane, kWave = 16 * kRow;
+  typedef PYLO_LDS bfbits lbf;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  char __attribute__((address_space(3)))* patch = lds + wave * kBfPatchWave;
-  const int wi = i0 + (wave >> 1) * 64, wj = j0 + (wave & 1) * 64;   // origin of the wave's values
+  PYLO_LDS char* patch = lds + wave * kWave;
+  const int wi = i0 + (wave >> 1) * 64, wj = j0 + (wave & 1) * 32 * WN;   // origin of the wave's values
 #pragma unroll
   for (int pass = 0; pass < 4; ++pass) {
     const int hi = pass >> 1, half = pass & 1;   // rows 32 hi + 16 half .. + 15 of the wave's 64
     __syncthreads();   // the patch is free (first pass: every wave has left the product's last stage)
 #pragma unroll
-    for (int hj = 0; hj < 2; ++hj)
+    for (int hj = 0; hj < WN; ++hj)
 #pragma unroll
       for (int r8 = 0; r8 < 8; ++r8) {
         const int r = 8 * half + r8;
         const int row_l = 8 * (r8 >> 2) + 4 * (lane >> 5) + (r8 & 3), col_l = 32 * hj + (lane & 31);
         bfbits h, m, l;
         bf_split(acc[hi][hj][r], h, m, l);
-        lbf* q = (lbf*)(patch + row_l * kBfPatchRow + col_l * 2);
+        lbf* q = (lbf*)(patch + row_l * kRow + col_l * 2);
         q[0] = h;
-        q[kBfPatchPlane / 2] = m;
-        q[kBfPatchPlane] = l;
+        q[kPlane / 2] = m;
+        q[kPlane] = l;
       }
     __syncthreads();
     const int row_w0 = wi + 32 * hi + 16 * half;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {          // 16 columns = one block of the planes' layout
+    for (int c = 0; c < 2 * WN; ++c) {     // 16 columns = one block of the planes' layout
       const int col = wj + 16 * c;
       if (col >= n_cols) continue;
       bfbits* dst = D + bf_off(rows_total, row_w0, col);
@@ -213,7 +225,7 @@ __device__ __forceinline__ void bf_store_direct(char __attribute__((address_spac
         if (pc >= 96) continue;
         const int row_l = pc / 6, rem = pc - 6 * row_l, plane = rem >> 1, hf = rem & 1;
         if (row_w0 + row_l >= n_rows) continue;
-        const u32x4 w = *(const luint4*)(patch + row_l * kBfPatchRow + plane * kBfPatchPlane + (16 * c + 8 * hf) * 2);
+        const u32x4 w = *(const luint4*)(patch + row_l * kRow + plane * kPlane + (16 * c + 8 * hf) * 2);
         *(u32x4*)(dst + (size_t)pc * 8) = w;
       }
     }
@@ -224,49 +236,55 @@ __device__ __forceinline__ void bf_store_direct(char __attribute__((address_spac
 //   kNsGram    A = Xs Xs^T as fp32 and planes, both halves; a slab of a split product: fp32 partial tile only
 //   kNsPoly    B' = c2 A A + c1 A + c0 I as planes, both halves
 //   kNsUpdate  Xl' = Xl B': planes of Xl' (buffer 1 - par) and Xs', or fp32 X in place of the raw step (`last`)
-template <int OP>
-__global__ __launch_bounds__(256) void k_ns_bf_gemm(const NsBfMat* __restrict__ mats, const NsItem* __restrict__ items,
+// WN: the tile has 64 WN columns (Gram and Poly: 2; updates: 2 or 4, a table of jobs each).
+// Registers: 64 / 128 accumulator registers plus what the epilogues need; tiles of 256 columns are held to two
+// waves per SIMD (256 registers: left alone the epilogue takes 296 and a CU runs one job at a time).
+template <int OP, int WN>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2 : 3))) void k_ns_bf_gemm(const NsBfMat* __restrict__ mats, const NsItem* __restrict__ items,
                                                     const PyloTensorArgs* __restrict__ dyn, float* __restrict__ ws,
                                                     bfbits* __restrict__ pw, int par, int last, float c0, float c1,
                                                     float c2) {
-  __shared__ __attribute__((aligned(16))) char lds_[2 * kBfStageLds];
-  char __attribute__((address_space(3)))* lds = (char __attribute__((address_space(3)))*)lds_;
+  extern __shared__ __attribute__((aligned(16))) char lds_[];
+  PYLO_LDS char* lds = (PYLO_LDS char*)lds_;
   const NsItem it = items[blockIdx.x];
   if (it.mat < 0) return;   // a filler job
   const NsBfMat mt = mats[it.mat];
   const PyloTensorArgs a = dyn[mt.tensor];
   if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
-  const int m = mt.m, n = mt.n;
-  v16f acc[2][2];
+  const int m = mt.m, n = mt.n, lda = mt.lda;
+  v16f acc[2][WN];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-  const int i0 = it.tm * kNsTile, j0 = it.tn * kNsTile;
+  const int i0 = it.tm * kNsTile, j0 = it.tn * 64 * WN;
   if (OP == kNsGram) {
-    const BfPlanes X{pw + mt.off_xs, m};
-    bf_tile_product(X, i0, X, j0, it.k0, it.k1, lds, acc);
+    const BfPlanes X{pw + mt.off_xs, mt.rows_m};
+    bf_tile_product<WN>(X, i0, X, j0, it.k0, it.k1, lds, acc);
   } else if (OP == kNsPoly) {
-    const BfPlanes A{pw + mt.off_pa, m};
-    bf_tile_product(A, i0, A, j0, it.k0, it.k1, lds, acc);
+    const BfPlanes A{pw + mt.off_pa, mt.rows_m};
+    bf_tile_product<WN>(A, i0, A, j0, it.k0, it.k1, lds, acc);
   } else {
-    const BfPlanes X{pw + mt.off_xl[par], n};
-    const BfPlanes B{pw + mt.off_pb, m};
-    bf_tile_product(X, i0, B, j0, it.k0, it.k1, lds, acc);
+    const BfPlanes X{pw + (par ? mt.off_xl[1] : mt.off_xl[0]), mt.rows_n};   // no run-time index: the struct stays in registers
+    const BfPlanes B{pw + mt.off_pb, mt.rows_m};
+    bf_tile_product<WN>(X, i0, B, j0, it.k0, it.k1, lds, acc);
   }
   float* A32 = ws + mt.off_a;
   const int n_i = OP == kNsUpdate ? n : m;   // rows of the output; its columns are always m
   const bool partial = OP == kNsGram && it.slab >= 0;
   const bool mirror = OP != kNsUpdate && !partial && it.tm != it.tn;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float* xout = a.step_out + mt.elem_off;
+  const bool vec_out = (mt.C & 3) == 0;   // rows of the tensor are 16-byte aligned
   // what the registers can store well: fp32 outputs, and the planes in which four consecutive rows of a
   // lane are four consecutive reduction indices (the mirrored tile, Xs')
 #pragma unroll
   for (int hi = 0; hi < 2; ++hi)
 #pragma unroll
-    for (int hj = 0; hj < 2; ++hj) {
-      const int col = j0 + ns_acc_col(hj);
+    for (int hj = 0; hj < WN; ++hj) {
+      const int col = j0 + (wave & 1) * 32 * WN + hj * 32 + (lane & 31);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int row = i0 + ns_acc_row(hi, 4 * q);   // rows row .. row + 3
@@ -276,37 +294,42 @@ __global__ __launch_bounds__(256) void k_ns_bf_gemm(const NsBfMat* __restrict__ 
         for (int r = 0; r < 4; ++r) {
           float x = acc[hi][hj][4 * q + r];
           if (OP == kNsPoly) {
-            const float aij = row + r < m ? A32[(size_t)(row + r) * m + col] : 0.0f;
-            x = c2 * x + c1 * aij + ((row + r) == col ? c0 : 0.0f);
+            const bool in = row + r < m;
+            const float aij = in ? A32[(size_t)(row + r) * lda + col] : 0.0f;
+            x = in ? c2 * x + c1 * aij + ((row + r) == col ? c0 : 0.0f) : 0.0f;
             acc[hi][hj][4 * q + r] = x;
           }
           v[r] = x;
         }
         if (OP == kNsGram) {
-          float* out = partial ? ws + mt.off_part + (size_t)it.slab * m * m : A32;
+          float* out = partial ? ws + mt.off_part + (size_t)it.slab * m * lda : A32;
 #pragma unroll
           for (int r = 0; r < 4; ++r)
-            if (row + r < m) out[(size_t)(row + r) * m + col] = v[r];
-          if (mirror) *(gv4f*)(out + (size_t)col * m + row) = v4f{v[0], v[1], v[2], v[3]};
+            if (row + r < m) out[(size_t)(row + r) * lda + col] = v[r];
+          if (mirror) *(gv4f*)(out + (size_t)col * lda + row) = v4f{v[0], v[1], v[2], v[3]};   // past m: zeros into the pitch's padding
         }
         if (OP == kNsGram || OP == kNsPoly) {
-          if (mirror) bf_store4(pw + (OP == kNsGram ? mt.off_pa : mt.off_pb), m, col, row, v);
+          if (mirror) bf_store4(pw + (OP == kNsGram ? mt.off_pa : mt.off_pb), mt.rows_m, col, row, v);
         } else if (!last) {
-          bf_store4(pw + mt.off_xs, m, col, row, v);   // values past n are zeros, into the padding
+          bf_store4(pw + mt.off_xs, mt.rows_m, col, row, v);   // values past n are zeros, into the padding
         } else if (mt.tall) {   // X = Xl, n x m
 #pragma unroll
           for (int r = 0; r < 4; ++r)
-            if (row + r < n) a.step_out[(size_t)(row + r) * m + col] = v[r];
-        } else {                // X = Xs, m x n: four consecutive columns of row `col` (n is a multiple of 4)
-          *(gv4f*)(a.step_out + (size_t)col * n + row) = v4f{v[0], v[1], v[2], v[3]};
+            if (row + r < n) xout[(size_t)(row + r) * m + col] = v[r];
+        } else if (vec_out) {   // X = Xs, m x n: four consecutive columns of row `col` (n is a multiple of 4)
+          *(gv4f*)(xout + (size_t)col * n + row) = v4f{v[0], v[1], v[2], v[3]};
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (row + r < n) xout[(size_t)col * n + row + r] = v[r];
         }
       }
     }
   // the planes in which a lane's column is the reduction index (A, B', Xl'): through LDS, 16 rows of each
-  // wave's 64 x 64 values at a time, so that memory sees 16-byte pieces in the planes' own order
+  // wave's 64 x 32 WN values at a time, so that memory sees 16-byte pieces in the planes' own order
   if (partial || (OP == kNsUpdate && last)) return;
-  bfbits* D = pw + (OP == kNsGram ? mt.off_pa : OP == kNsPoly ? mt.off_pb : mt.off_xl[1 - par]);
-  bf_store_direct(lds, acc, D, n_i, i0, j0, n_i, m);
+  bfbits* D = pw + (OP == kNsGram ? mt.off_pa : OP == kNsPoly ? mt.off_pb : par ? mt.off_xl[0] : mt.off_xl[1]);
+  bf_store_direct<WN>(lds, acc, D, OP == kNsUpdate ? mt.rows_n : mt.rows_m, i0, j0, n_i, m);
 }
 
 // A = sum over the slabs' partial matrices, in slab order, as fp32 and as planes (both halves).
@@ -316,13 +339,13 @@ __global__ __launch_bounds__(256) void k_ns_bf_gram_reduce(const NsBfMat* __rest
   const NsBfMat mt = mats[split_mats[blockIdx.y]];
   const PyloTensorArgs a = dyn[mt.tensor];
   if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
-  const int m = mt.m;
+  const int m = mt.m, lda = mt.lda;
   const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
   if (e >= (long long)m * m) return;
   const int i = (int)(e / m), j = (int)(e - (long long)i * m);
   if (i / kNsTile > j / kNsTile) return;
-  const size_t mm = (size_t)m * m;
-  const float* p = ws + mt.off_part + (size_t)i * m + j;
+  const size_t mm = (size_t)m * lda;
+  const float* p = ws + mt.off_part + (size_t)i * lda + j;
   float s = 0.0f;
   for (int q0 = 0; q0 < mt.n_slabs; q0 += 8) {
     float v[8];
@@ -333,11 +356,11 @@ __global__ __launch_bounds__(256) void k_ns_bf_gram_reduce(const NsBfMat* __rest
   }
   float* A = ws + mt.off_a;
   bfbits* P = pw + mt.off_pa;
-  A[(size_t)i * m + j] = s;
-  bf_store1(P, m, i, j, s);
+  A[(size_t)i * lda + j] = s;
+  bf_store1(P, mt.rows_m, i, j, s);
   if (i / kNsTile != j / kNsTile) {
-    A[(size_t)j * m + i] = s;
-    bf_store1(P, m, j, i, s);
+    A[(size_t)j * lda + i] = s;
+    bf_store1(P, mt.rows_m, j, i, s);
   }
 }
 
@@ -357,15 +380,18 @@ __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__
   if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
   const float s = scale[it.mat];
   const int R = mt.R, C = mt.C;
+  const float* raw = a.step_out + mt.elem_off;
+  const bool vec_in = (C & 3) == 0;
   // direct planes: the tensor's rows are the planes' rows; transposed planes: its columns are
   bfbits* direct = pw + (mt.tall ? mt.off_xl[0] : mt.off_xs);
   bfbits* transp = pw + (mt.tall ? mt.off_xs : mt.off_xl[0]);
+  const int rows_d = mt.tall ? mt.rows_n : mt.rows_m, rows_t = mt.tall ? mt.rows_m : mt.rows_n;
   const int r0 = it.tr * 64, c0 = it.tc * 64;
   const int t = threadIdx.x;
   // Eight consecutive columns of one row a lane and pass: 32 bytes read, one 16-byte piece per plane written
   // to the direct planes (the two lanes of a 16-column block fill its 96 bytes) and to the tile in LDS.
-  // Columns and rows past the matrix read as zero; where a piece straddles the edge (C or R a multiple of 4
-  // only) the zeros land in the planes' padding, which holds zeros anyway.
+  // Columns and rows past the matrix read as zero; where a piece straddles the edge the zeros land in the
+  // planes' padding, which holds zeros anyway.
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
     const int u = pass * 256 + t, lr = u >> 3, lc = 8 * (u & 7);
@@ -373,12 +399,18 @@ __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__
     float v[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     const bool in = r < R && c < C;
     if (in) {
-      const float* src = a.step_out + (size_t)r * C + c;
-      const v4f x = *(const gv4f*)src;
-      v[0] = x.x * s; v[1] = x.y * s; v[2] = x.z * s; v[3] = x.w * s;
-      if (c + 4 < C) {
-        const v4f y = *(const gv4f*)(src + 4);
-        v[4] = y.x * s; v[5] = y.y * s; v[6] = y.z * s; v[7] = y.w * s;
+      const float* src = raw + (size_t)r * C + c;
+      if (vec_in) {
+        const v4f x = *(const gv4f*)src;
+        v[0] = x.x * s; v[1] = x.y * s; v[2] = x.z * s; v[3] = x.w * s;
+        if (c + 4 < C) {
+          const v4f y = *(const gv4f*)(src + 4);
+          v[4] = y.x * s; v[5] = y.y * s; v[6] = y.z * s; v[7] = y.w * s;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (c + e < C) v[e] = *(const gfloat*)(src + e) * s;
       }
     }
     u32x4 pl[3];
@@ -394,7 +426,7 @@ __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__
 #pragma unroll
     for (int q = 0; q < 3; ++q) *(luint4*)&tile[q][lr][lc] = pl[q];
     if (in) {
-      bfbits* p = direct + bf_off(R, r, c);
+      bfbits* p = direct + bf_off(rows_d, r, c);
 #pragma unroll
       for (int q = 0; q < 3; ++q) *(u32x4*)(p + 16 * q) = pl[q];
     }
@@ -406,7 +438,7 @@ __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__
     const int lc = t & 63, rb = t >> 6;
     const int c = c0 + lc, r = r0 + 16 * rb;
     if (c < C && r < R) {
-      bfbits* p = transp + bf_off(C, c, r);
+      bfbits* p = transp + bf_off(rows_t, c, r);
 #pragma unroll
       for (int q = 0; q < 3; ++q)
 #pragma unroll

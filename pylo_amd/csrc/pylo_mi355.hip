@@ -80,6 +80,7 @@ struct Layout {
   // ELO-CELO2: Newton-Schulz on the 2-D tensors (k_ns.h)
   std::vector<NsMat> ns_mats;
   std::vector<NsItem> ns_gram, ns_poly, ns_upd;
+  std::vector<NsItem> ns_upd4;        // split-bf16 kernels: update jobs with 256-column tiles
   std::vector<int> ns_split;          // matrices whose Gram product is split (k_ns_gram_reduce)
   std::vector<long long> ns_xalt;     // per tensor: offset of its second X buffer, -1 without one
   std::vector<int> ns_of_tensor;      // per tensor: index into ns_mats, -1
@@ -88,7 +89,7 @@ struct Layout {
   bool ns_bf = false;
   std::vector<NsBfMat> nsb_mats;
   std::vector<NsTileItem> nsb_split_items;
-  size_t off_nsb_mats = 0, off_nsb_split_items = 0, off_ns_pw = 0;
+  size_t off_nsb_mats = 0, off_nsb_split_items = 0, off_ns_pw = 0, off_ns_upd4 = 0;
   long long nsb_plane_elems = 0;
   size_t off_ns_mats = 0, off_ns_gram = 0, off_ns_poly = 0, off_ns_upd = 0, off_ns_split = 0, off_ns_xalt = 0,
          off_ns_scale = 0, off_ns_ws = 0;
@@ -251,9 +252,8 @@ void xcd_interleave(std::vector<NsItem>& items, const std::vector<std::pair<int,
   items.swap(out);
 }
 
-// Newton-Schulz tables: every 2-D MLP tensor whose rows (C) and whose smaller dim (the rows of A and B')
-// are multiples of 4: the kernels load 16 bytes at a time along the contiguous dim of X, A and B'.  The
-// number of rows of a tall matrix is free (50257 x 768).  `ws_floats` returns the floats of workspace behind off_ns_ws.
+// Newton-Schulz tables: every 2-D MLP tensor (the fp32 kernels: those whose rows (C) and whose smaller dim are
+// multiples of 4).  `ws_floats` returns the floats of workspace behind off_ns_ws.
 void build_ns_tables(Layout& L, int T, long long& ws_floats) {
   ws_floats = 0;
   L.ns_xalt.assign(T, -1);
@@ -261,7 +261,9 @@ void build_ns_tables(Layout& L, int T, long long& ws_floats) {
   auto take = [&](long long n) { const long long o = ws_floats; ws_floats += (n + 63) / 64 * 64; return o; };
   for (int t = 0; t < T; ++t) {
     const TDesc& d = L.descs[t];
-    if (d.mode != kModeFac2D || d.n == 0 || d.C0 % 4 != 0 || std::min(d.R0, d.C0) % 4 != 0) continue;
+    if (d.mode != kModeFac2D || d.n == 0) continue;
+    // the fp32 kernels load 16 bytes at a time along the contiguous dim of X, A and B'
+    if (!L.ns_bf && (d.C0 % 4 != 0 || std::min(d.R0, d.C0) % 4 != 0)) continue;
     NsMat mt{};
     mt.tensor = t;
     mt.R = d.R0; mt.C = d.C0;
@@ -296,27 +298,34 @@ void build_ns_tables(Layout& L, int T, long long& ws_floats) {
   }
   if (L.ns_bf) {
     // same matrices, operands as bf16 planes; the item tables are rebuilt for the uniform (n x m) orientation
-    L.ns_gram.clear(); L.ns_poly.clear(); L.ns_upd.clear();
+    L.ns_gram.clear(); L.ns_poly.clear(); L.ns_upd.clear(); L.ns_upd4.clear();
     ws_floats = 0;
     long long pw = 0;
     auto take_p = [&](long long n) { const long long o = pw; pw += (n + 63) / 64 * 64; return o; };
-    auto up16 = [](int x) { return (x + kBfBK - 1) / kBfBK * kBfBK; };
+    auto up = [](int x, int q) { return (x + q - 1) / q * q; };
+    auto up16 = [&](int x) { return up(x, kBfBK); };
     // job runs that read the same operands: per matrix (slab), and finer, per row of tiles, for sets of few matrices
-    std::vector<std::pair<int, long long>> gram_units, poly_units, upd_units, gram_rows, poly_rows;
+    std::vector<std::pair<int, long long>> gram_units, poly_units, upd_units, upd4_units, gram_rows, poly_rows;
     for (size_t q = 0; q < L.ns_mats.size(); ++q) {
       const NsMat& f = L.ns_mats[q];
       NsBfMat b{};
       b.tensor = f.tensor; b.R = f.R; b.C = f.C; b.m = f.m; b.n = std::max(f.R, f.C); b.tall = f.tall;
       b.pad_m = up16(b.m);
       b.pad_n = up16(b.n);
+      // update tiles of 256 columns where that does not compute much more padding than tiles of 128 would
+      const bool wide_tiles = up(b.m, 256) <= 1.06 * up(b.m, 128);
+      b.rows_m = up(b.m, wide_tiles ? 256 : kNsTile);
+      b.rows_n = up(b.n, kNsTile);
+      b.lda = up(b.m, 4);
       b.n_slabs = f.n_slabs;
-      b.off_xs = take_p(3ll * b.m * b.pad_n);
-      b.off_xl[0] = take_p(3ll * b.n * b.pad_m);
-      b.off_xl[1] = take_p(3ll * b.n * b.pad_m);
-      b.off_pa = take_p(3ll * b.m * b.pad_m);
-      b.off_pb = take_p(3ll * b.m * b.pad_m);
-      b.off_a = take((long long)b.m * b.m);
-      b.off_part = b.n_slabs > 1 ? take((long long)b.n_slabs * b.m * b.m) : 0;
+      b.off_xs = take_p(3ll * b.rows_m * b.pad_n);
+      b.off_xl[0] = take_p(3ll * b.rows_n * b.pad_m);
+      b.off_xl[1] = take_p(3ll * b.rows_n * b.pad_m);
+      b.off_pa = take_p(3ll * b.rows_m * b.pad_m);
+      b.off_pb = take_p(3ll * b.rows_m * b.pad_m);
+      b.off_a = take((long long)b.m * b.lda);
+      b.off_part = b.n_slabs > 1 ? take((long long)b.n_slabs * b.m * b.lda) : 0;
+      b.elem_off = 0;
       L.ns_mats[q].off_a = b.off_a;   // the fp32 tables stay consistent for k_ns_scale (tensor index only)
       const int nt = (b.m + kNsTile - 1) / kNsTile, n_upper = nt * (nt + 1) / 2;
       // Gram: the tiles of one matrix (of one slab of it) read the same rows of Xs; Poly: the same A
@@ -333,10 +342,12 @@ void build_ns_tables(Layout& L, int T, long long& ws_floats) {
       poly_units.push_back({n_upper, (long long)up16(b.m)});
       for (int tm = 0; tm < nt; ++tm) poly_rows.push_back({nt - tm, (long long)up16(b.m)});
       // Update: the tiles of one row block read the same rows of Xl, all of them the same B'
-      const int ni = (b.n + kNsTile - 1) / kNsTile;
+      const int ni = (b.n + kNsTile - 1) / kNsTile, ntu = wide_tiles ? (b.m + 255) / 256 : nt;
+      std::vector<NsItem>& upd = wide_tiles ? L.ns_upd4 : L.ns_upd;
+      std::vector<std::pair<int, long long>>& units = wide_tiles ? upd4_units : upd_units;
       for (int tm = 0; tm < ni; ++tm) {
-        for (int tn = 0; tn < nt; ++tn) L.ns_upd.push_back(NsItem{(int)q, tm, tn, 0, up16(b.m), -1});
-        upd_units.push_back({nt, (long long)up16(b.m)});
+        for (int tn = 0; tn < ntu; ++tn) upd.push_back(NsItem{(int)q, tm, tn, 0, up16(b.m), -1});
+        units.push_back({ntu, (long long)up16(b.m)});
       }
       for (int tr = 0; tr < (b.R + 63) / 64; ++tr)
         for (int tc = 0; tc < (b.C + 63) / 64; ++tc) L.nsb_split_items.push_back(NsTileItem{(int)q, tr, tc});
@@ -354,6 +365,7 @@ void build_ns_tables(Layout& L, int T, long long& ws_floats) {
       pick(L.ns_gram, gram_units, gram_rows);
       pick(L.ns_poly, poly_units, poly_rows);
       pick(L.ns_upd, upd_units, upd_units);
+      pick(L.ns_upd4, upd4_units, upd4_units);
     }
     return;
   }
@@ -632,6 +644,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     L.off_ns_gram = take(sizeof(NsItem) * L.ns_gram.size());
     L.off_ns_poly = take(sizeof(NsItem) * L.ns_poly.size());
     L.off_ns_upd = take(sizeof(NsItem) * L.ns_upd.size());
+    L.off_ns_upd4 = take(sizeof(NsItem) * L.ns_upd4.size());
     L.off_ns_split = take(sizeof(int) * L.ns_split.size());
     L.off_ns_xalt = take(sizeof(long long) * (size_t)T);
     L.off_ns_scale = take(sizeof(float) * L.ns_mats.size());
@@ -732,6 +745,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_ns_gram, L.ns_gram.data(), sizeof(NsItem) * L.ns_gram.size());
   if (e == hipSuccess) e = up(L.off_ns_poly, L.ns_poly.data(), sizeof(NsItem) * L.ns_poly.size());
   if (e == hipSuccess) e = up(L.off_ns_upd, L.ns_upd.data(), sizeof(NsItem) * L.ns_upd.size());
+  if (e == hipSuccess) e = up(L.off_ns_upd4, L.ns_upd4.data(), sizeof(NsItem) * L.ns_upd4.size());
   if (e == hipSuccess) e = up(L.off_ns_split, L.ns_split.data(), sizeof(int) * L.ns_split.size());
   if (e == hipSuccess && kind == PYLO_KIND_CELO2) e = up(L.off_ns_xalt, L.ns_xalt.data(), sizeof(long long) * L.ns_xalt.size());
   if (e == hipSuccess) e = up(L.off_nsb_mats, L.nsb_mats.data(), sizeof(NsBfMat) * L.nsb_mats.size());
@@ -1136,6 +1150,24 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
 
 namespace {
 
+// The split-bf16 product kernels take their LDS as dynamic shared memory; tiles of 256 columns need more than
+// the 64 KB a kernel may have without asking.
+int ns_bf_lds_once() {
+  static std::mutex mu;
+  static std::vector<int> done;   // devices on which the attribute has been set
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(mu);
+  for (int d : done)
+    if (d == dev) return 0;
+  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsGram, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(2)));
+  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsPoly, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(2)));
+  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsUpdate, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(2)));
+  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsUpdate, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(4)));
+  done.push_back(dev);
+  return 0;
+}
+
 // Newton-Schulz (ns_iters > 0, on the tensors flagged PYLO_ARG_ORTHOGONALIZE) and the finishing pass.
 int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, int ns_iters, float ns_eps, void* stream,
                 const char* who) {
@@ -1192,17 +1224,24 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
       bfbits* pw = P->at<bfbits>(L.off_ns_pw);
       hipLaunchKernelGGL(k_ns_bf_split, dim3((unsigned)L.nsb_split_items.size()), dim3(256), 0, s, bmats, sitems, dyn,
                          (const float*)scale, pw);
+      const NsItem* upd4 = P->at<NsItem>(L.off_ns_upd4);
+      const int n_upd4 = (int)L.ns_upd4.size();
+      if (int rc = ns_bf_lds_once()) return rc;
       for (int it = 0; it < ns_iters; ++it) {
         const int par = it & 1, last = it == ns_iters - 1;
-        hipLaunchKernelGGL(k_ns_bf_gemm<kNsGram>, dim3(n_gram), dim3(256), 0, s, bmats, gram, dyn, ns_ws, pw, par, last,
-                           coeffs[0], coeffs[1], coeffs[2]);
+        hipLaunchKernelGGL((k_ns_bf_gemm<kNsGram, 2>), dim3(n_gram), dim3(256), bf_gemm_lds(2), s, bmats, gram, dyn, ns_ws,
+                           pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
         if (n_split > 0)
           hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)L.ns_max_m * L.ns_max_m + 255) / 256, n_split), dim3(256),
                              0, s, bmats, split, dyn, ns_ws, pw);
-        hipLaunchKernelGGL(k_ns_bf_gemm<kNsPoly>, dim3(n_poly), dim3(256), 0, s, bmats, poly, dyn, ns_ws, pw, par, last,
-                           coeffs[0], coeffs[1], coeffs[2]);
-        hipLaunchKernelGGL(k_ns_bf_gemm<kNsUpdate>, dim3(n_upd), dim3(256), 0, s, bmats, upd, dyn, ns_ws, pw, par, last,
-                           coeffs[0], coeffs[1], coeffs[2]);
+        hipLaunchKernelGGL((k_ns_bf_gemm<kNsPoly, 2>), dim3(n_poly), dim3(256), bf_gemm_lds(2), s, bmats, poly, dyn, ns_ws,
+                           pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+        if (n_upd4 > 0)
+          hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 4>), dim3(n_upd4), dim3(256), bf_gemm_lds(4), s, bmats, upd4, dyn,
+                             ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+        if (n_upd > 0)
+          hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 2>), dim3(n_upd), dim3(256), bf_gemm_lds(2), s, bmats, upd, dyn,
+                             ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
       }
     } else
     for (int it = 0; it < ns_iters; ++it) {

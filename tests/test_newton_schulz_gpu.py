@@ -54,11 +54,18 @@ def _run(shapes, steps=2, seed=0, **kw):
     return opt, worst
 
 
-def test_library_kernels_take_these_shapes():
+@pytest.mark.parametrize("pipe", ["bf16x3", "fp32"])
+def test_library_kernels_take_these_shapes(pipe, monkeypatch):
+    if pipe == "fp32":
+        monkeypatch.setenv("PYLO_MI355_NS_F32", "1")
     shapes = [(256, 384), (384, 256), (128, 128), (132, 260), (260, 132), (4, 8), (8, 4), (36, 36), (1, 64), (64, 1),
-              (130, 6), (6, 130), (10, 12), (12, 10), (9, 16), (16, 9)]
-    opt, _ = _run(shapes, steps=1)
-    # the last dim and the smaller dim must be multiples of 4; everything else goes through torch
+              (130, 6), (6, 130), (10, 12), (12, 10), (9, 16), (16, 9), (37, 131), (131, 37), (1, 1), (3, 5)]
+    opt, _ = _run(shapes, steps=2)
+    if pipe == "bf16x3":
+        # the split-bf16 kernels take any two dims
+        assert all(opt._ns_ok), opt._ns_ok
+        return
+    # fp32 kernels: the last dim and the smaller dim must be multiples of 4; everything else goes through torch
     for s, got in zip(shapes, opt._ns_ok):
         r, c = s
         assert got == (c % 4 == 0 and min(r, c) % 4 == 0), s
@@ -69,7 +76,8 @@ def test_library_kernels_take_these_shapes():
     [(256, 384), (384, 256), (128, 128), (768,)],                       # whole tiles
     [(132, 260), (260, 132), (4, 8), (8, 4), (36, 36), (200, 4)],        # ragged tiles, a single MFMA column
     [(8201, 128), (128, 8200), (16385, 64)],                             # split Gram product, odd reduction length
-    [(130, 6), (6, 130), (9, 16), (64, 64)],                             # library and torch side by side
+    [(130, 6), (6, 130), (9, 16), (64, 64)],                             # dims that are not multiples of 4 (fp32 kernels: torch)
+    [(37, 4099), (4099, 37), (255, 257), (129, 129), (1, 300), (300, 1), (2, 3)],   # odd dims, single rows and columns
     [(300, 260), (300, 260), (300, 260), (64,)],                         # a bucket of equal shapes
 ])
 @pytest.mark.parametrize("pipe", ["bf16x3", "fp32"])
@@ -121,11 +129,12 @@ def test_groups_without_orthogonalisation_and_with_param_scale():
             assert max_err(p, ref[i], 1e-5, 1e-6) <= 1.0, (t, i)
 
 
-def test_flag_on_an_unsupported_tensor_is_refused():
+def test_flag_on_an_unsupported_tensor_is_refused(monkeypatch):
     import numpy as np
 
     from pylo_amd import _lib
 
+    monkeypatch.setenv("PYLO_MI355_NS_F32", "1")   # the fp32 kernels refuse dims that are not multiples of 4
     plan = _lib.Plan(_lib.KIND_CELO2, [(130, 6), (64, 64)], [0, 0], torch.device("cuda:0"))
     assert not plan.orthogonalize_supported(0) and plan.orthogonalize_supported(1)
     x = torch.zeros(130 * 6 + 64 * 64, device="cuda")

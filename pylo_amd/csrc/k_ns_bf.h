@@ -182,37 +182,55 @@ __device__ __forceinline__ void bf_store1(bfbits* base, int rows, int row, int k
   p[32] = l;
 }
 
-// The block's 128 x 64 WN values (accumulator layout) into planes whose reduction index is the tile's column
-// index.  Four passes of 16 rows per wave: every lane splits its values and drops the halves into the
-// wave's own LDS patch ([row][plane][32 WN columns], 2 bytes each), then the wave reads the patch back as
-// 16-byte pieces in the order the planes have in memory ([16 columns][row][plane][half]) and stores them.
+// The block's 128 x 64 WN values (accumulator layout) into planes, in one or both orientations, every value
+// split once.
+//   D   planes whose reduction index is the tile's column index: through the wave's own LDS patch
+//       ([row][plane][32 WN columns], 2 bytes each), 16 rows at a time; the wave reads the patch back as
+//       16-byte pieces in the order the planes have in memory ([16 columns][row][plane][half]).
+//   D4  (when not null) planes whose reduction index is the tile's row index: four consecutive rows of a
+//       lane are four consecutive reduction indices, one 8-byte store per plane straight from the registers.
+// Only the lanes of one wave meet in a patch and a wave's LDS instructions execute in order, so the passes
+// need no barrier, just the compiler kept from moving the reads over the writes.
 template <int WN>
-__device__ __forceinline__ void bf_store_direct(PYLO_LDS char* lds, const v16f (&acc)[2][WN], bfbits* __restrict__ D,
-                                                int rows_total, int i0, int j0, int n_rows, int n_cols) {
+__device__ __forceinline__ void bf_store_planes(PYLO_LDS char* lds, const v16f (&acc)[2][WN], bfbits* __restrict__ D,
+                                                int rows_total, int i0, int j0, int n_rows, int n_cols,
+                                                bfbits* __restrict__ D4, int rows4) {
   constexpr int kPlane = 64 * WN + 16;        // bytes: 32 WN columns x 2 + 16 (bank spread)
   constexpr int kRow = 3 * kPlane, kWave = 16 * kRow;
   typedef PYLO_LDS bfbits lbf;
+  typedef unsigned long long u64;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   PYLO_LDS char* patch = lds + wave * kWave;
   const int wi = i0 + (wave >> 1) * 64, wj = j0 + (wave & 1) * 32 * WN;   // origin of the wave's values
 #pragma unroll
   for (int pass = 0; pass < 4; ++pass) {
     const int hi = pass >> 1, half = pass & 1;   // rows 32 hi + 16 half .. + 15 of the wave's 64
-    __syncthreads();   // the patch is free (first pass: every wave has left the product's last stage)
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // the patch is free: the previous pass has read it
 #pragma unroll
     for (int hj = 0; hj < WN; ++hj)
 #pragma unroll
-      for (int r8 = 0; r8 < 8; ++r8) {
-        const int r = 8 * half + r8;
-        const int row_l = 8 * (r8 >> 2) + 4 * (lane >> 5) + (r8 & 3), col_l = 32 * hj + (lane & 31);
-        bfbits h, m, l;
-        bf_split(acc[hi][hj][r], h, m, l);
-        lbf* q = (lbf*)(patch + row_l * kRow + col_l * 2);
-        q[0] = h;
-        q[kPlane / 2] = m;
-        q[kPlane] = l;
+      for (int g4 = 0; g4 < 2; ++g4) {
+        bfbits h[4], m[4], l[4];
+        const int col_l = 32 * hj + (lane & 31);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          bf_split(acc[hi][hj][8 * half + 4 * g4 + r], h[r], m[r], l[r]);
+          lbf* q = (lbf*)(patch + (8 * g4 + 4 * (lane >> 5) + r) * kRow + col_l * 2);
+          q[0] = h[r];
+          q[kPlane / 2] = m[r];
+          q[kPlane] = l[r];
+        }
+        if (D4 != nullptr) {
+          const int row = wi + 32 * hi + 16 * half + 8 * g4 + 4 * (lane >> 5), col = wj + col_l;
+          if (col < n_cols && row < n_rows) {   // values past n_rows are zeros, into the padding
+            bfbits* p = D4 + bf_off(rows4, col, row);
+            *(u64*)p = (u64)h[0] | (u64)h[1] << 16 | (u64)h[2] << 32 | (u64)h[3] << 48;
+            *(u64*)(p + 16) = (u64)m[0] | (u64)m[1] << 16 | (u64)m[2] << 32 | (u64)m[3] << 48;
+            *(u64*)(p + 32) = (u64)l[0] | (u64)l[1] << 16 | (u64)l[2] << 32 | (u64)l[3] << 48;
+          }
+        }
       }
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     const int row_w0 = wi + 32 * hi + 16 * half;
 #pragma unroll
     for (int c = 0; c < 2 * WN; ++c) {     // 16 columns = one block of the planes' layout
@@ -278,58 +296,60 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float* xout = a.step_out + mt.elem_off;
   const bool vec_out = (mt.C & 3) == 0;   // rows of the tensor are 16-byte aligned
-  // what the registers can store well: fp32 outputs, and the planes in which four consecutive rows of a
-  // lane are four consecutive reduction indices (the mirrored tile, Xs')
+  // fp32 outputs (and Poly's transform of the accumulators) straight from the registers
+  if (OP != kNsUpdate || last) {
 #pragma unroll
-  for (int hi = 0; hi < 2; ++hi)
+    for (int hi = 0; hi < 2; ++hi)
 #pragma unroll
-    for (int hj = 0; hj < WN; ++hj) {
-      const int col = j0 + (wave & 1) * 32 * WN + hj * 32 + (lane & 31);
+      for (int hj = 0; hj < WN; ++hj) {
+        const int col = j0 + (wave & 1) * 32 * WN + hj * 32 + (lane & 31);
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int row = i0 + ns_acc_row(hi, 4 * q);   // rows row .. row + 3
-        if (col >= m || row >= n_i) continue;
-        float v[4];
+        for (int q = 0; q < 4; ++q) {
+          const int row = i0 + ns_acc_row(hi, 4 * q);   // rows row .. row + 3
+          if (col >= m || row >= n_i) continue;
+          float v[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float x = acc[hi][hj][4 * q + r];
-          if (OP == kNsPoly) {
-            const bool in = row + r < m;
-            const float aij = in ? A32[(size_t)(row + r) * lda + col] : 0.0f;
-            x = in ? c2 * x + c1 * aij + ((row + r) == col ? c0 : 0.0f) : 0.0f;
-            acc[hi][hj][4 * q + r] = x;
+          for (int r = 0; r < 4; ++r) {
+            float x = acc[hi][hj][4 * q + r];
+            if (OP == kNsPoly) {
+              const bool in = row + r < m;
+              const float aij = in ? A32[(size_t)(row + r) * lda + col] : 0.0f;
+              x = in ? c2 * x + c1 * aij + ((row + r) == col ? c0 : 0.0f) : 0.0f;
+              acc[hi][hj][4 * q + r] = x;
+            }
+            v[r] = x;
           }
-          v[r] = x;
-        }
-        if (OP == kNsGram) {
-          float* out = partial ? ws + mt.off_part + (size_t)it.slab * m * lda : A32;
+          if (OP == kNsGram) {
+            float* out = partial ? ws + mt.off_part + (size_t)it.slab * m * lda : A32;
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (row + r < m) out[(size_t)(row + r) * lda + col] = v[r];
-          if (mirror) *(gv4f*)(out + (size_t)col * lda + row) = v4f{v[0], v[1], v[2], v[3]};   // past m: zeros into the pitch's padding
-        }
-        if (OP == kNsGram || OP == kNsPoly) {
-          if (mirror) bf_store4(pw + (OP == kNsGram ? mt.off_pa : mt.off_pb), mt.rows_m, col, row, v);
-        } else if (!last) {
-          bf_store4(pw + mt.off_xs, mt.rows_m, col, row, v);   // values past n are zeros, into the padding
-        } else if (mt.tall) {   // X = Xl, n x m
+            for (int r = 0; r < 4; ++r)
+              if (row + r < m) out[(size_t)(row + r) * lda + col] = v[r];
+            if (mirror) *(gv4f*)(out + (size_t)col * lda + row) = v4f{v[0], v[1], v[2], v[3]};   // past m: zeros into the pitch's padding
+          } else if (OP == kNsUpdate) {
+            if (mt.tall) {   // X = Xl, n x m
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (row + r < n) xout[(size_t)(row + r) * m + col] = v[r];
-        } else if (vec_out) {   // X = Xs, m x n: four consecutive columns of row `col` (n is a multiple of 4)
-          *(gv4f*)(xout + (size_t)col * n + row) = v4f{v[0], v[1], v[2], v[3]};
-        } else {
+              for (int r = 0; r < 4; ++r)
+                if (row + r < n) xout[(size_t)(row + r) * m + col] = v[r];
+            } else if (vec_out) {   // X = Xs, m x n: four consecutive columns of row `col` (n is a multiple of 4)
+              *(gv4f*)(xout + (size_t)col * n + row) = v4f{v[0], v[1], v[2], v[3]};
+            } else {
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (row + r < n) xout[(size_t)col * n + row + r] = v[r];
+              for (int r = 0; r < 4; ++r)
+                if (row + r < n) xout[(size_t)col * n + row + r] = v[r];
+            }
+          }
         }
       }
-    }
-  // the planes in which a lane's column is the reduction index (A, B', Xl'): through LDS, 16 rows of each
-  // wave's 64 x 32 WN values at a time, so that memory sees 16-byte pieces in the planes' own order
+  }
+  // planes: A and B' in both halves (the tile itself through LDS, the mirrored tile from the registers), Xl'
+  // (through LDS) and Xs' (registers)
   if (partial || (OP == kNsUpdate && last)) return;
-  bfbits* D = pw + (OP == kNsGram ? mt.off_pa : OP == kNsPoly ? mt.off_pb : par ? mt.off_xl[0] : mt.off_xl[1]);
-  bf_store_direct<WN>(lds, acc, D, OP == kNsUpdate ? mt.rows_n : mt.rows_m, i0, j0, n_i, m);
+  if (OP == kNsUpdate) {
+    bf_store_planes<WN>(lds, acc, pw + (par ? mt.off_xl[0] : mt.off_xl[1]), mt.rows_n, i0, j0, n, m, pw + mt.off_xs, mt.rows_m);
+  } else {
+    bfbits* D = pw + (OP == kNsGram ? mt.off_pa : mt.off_pb);
+    bf_store_planes<WN>(lds, acc, D, mt.rows_m, i0, j0, m, m, mirror ? D : nullptr, mt.rows_m);
+  }
 }
 
 // A = sum over the slabs' partial matrices, in slab order, as fp32 and as planes (both halves).

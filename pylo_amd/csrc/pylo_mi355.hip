@@ -73,6 +73,9 @@ bool factored_dims(int kind, const PyloTensorShape& s, int* dc, int* dr) {
   return true;
 }
 
+// One group of matrices of the split-bf16 Newton-Schulz kernels: its ranges in the job tables.
+struct NsGroup { int gram0, n_gram, poly0, n_poly, upd0, n_upd, upd40, n_upd4, split0, n_split, split_max_m; };
+
 struct Layout {
   std::vector<Item> mx_items;   // ELO-CELO2: statistics and apply items in slab order (k_celo2_elem)
   size_t off_mx_items = 0, off_sync = 0;
@@ -81,6 +84,7 @@ struct Layout {
   std::vector<NsMat> ns_mats;
   std::vector<NsItem> ns_gram, ns_poly, ns_upd;
   std::vector<NsItem> ns_upd4;        // split-bf16 kernels: update jobs with 256-column tiles
+  std::vector<NsGroup> ns_groups;     // split-bf16 kernels: ranges of the job tables, one per group of matrices
   std::vector<int> ns_split;          // matrices whose Gram product is split (k_ns_gram_reduce)
   std::vector<long long> ns_xalt;     // per tensor: offset of its second X buffer, -1 without one
   std::vector<int> ns_of_tensor;      // per tensor: index into ns_mats, -1
@@ -218,6 +222,13 @@ bool env_ns_xcd() {
   return !(e && e[0] == '0');
 }
 
+// PYLO_MI355_NS_GROUPS: into how many groups (streams) the matrices of a plan are dealt, 1 to 4; read at plan creation.
+int env_ns_groups() {
+  const char* e = getenv("PYLO_MI355_NS_GROUPS");
+  const int g = e ? atoi(e) : 2;
+  return std::max(1, std::min(g, 4));
+}
+
 bool env_ns_bf() {
   const char* e = getenv("PYLO_MI355_NS_F32");
   return !(e && e[0] == '1');
@@ -304,8 +315,7 @@ void build_ns_tables(Layout& L, int T, long long& ws_floats) {
     auto take_p = [&](long long n) { const long long o = pw; pw += (n + 63) / 64 * 64; return o; };
     auto up = [](int x, int q) { return (x + q - 1) / q * q; };
     auto up16 = [&](int x) { return up(x, kBfBK); };
-    // job runs that read the same operands: per matrix (slab), and finer, per row of tiles, for sets of few matrices
-    std::vector<std::pair<int, long long>> gram_units, poly_units, upd_units, upd4_units, gram_rows, poly_rows;
+    // planes and fp32 matrices of every matrix
     for (size_t q = 0; q < L.ns_mats.size(); ++q) {
       const NsMat& f = L.ns_mats[q];
       NsBfMat b{};
@@ -327,45 +337,91 @@ void build_ns_tables(Layout& L, int T, long long& ws_floats) {
       b.off_part = b.n_slabs > 1 ? take((long long)b.n_slabs * b.m * b.lda) : 0;
       b.elem_off = 0;
       L.ns_mats[q].off_a = b.off_a;   // the fp32 tables stay consistent for k_ns_scale (tensor index only)
-      const int nt = (b.m + kNsTile - 1) / kNsTile, n_upper = nt * (nt + 1) / 2;
-      // Gram: the tiles of one matrix (of one slab of it) read the same rows of Xs; Poly: the same A
-      for (int sl = 0; sl < b.n_slabs; ++sl) {
-        const int k0 = b.n_slabs > 1 ? sl * kNsSlabK : 0;
-        const int k1 = b.n_slabs > 1 ? up16(std::min(b.n, (sl + 1) * kNsSlabK)) : up16(b.n);
-        for (int tm = 0; tm < nt; ++tm)
-          for (int tn = tm; tn < nt; ++tn) L.ns_gram.push_back(NsItem{(int)q, tm, tn, k0, k1, b.n_slabs > 1 ? sl : -1});
-        gram_units.push_back({n_upper, (long long)(k1 - k0)});
-        for (int tm = 0; tm < nt; ++tm) gram_rows.push_back({nt - tm, (long long)(k1 - k0)});
-      }
-      for (int tm = 0; tm < nt; ++tm)
-        for (int tn = tm; tn < nt; ++tn) L.ns_poly.push_back(NsItem{(int)q, tm, tn, 0, up16(b.m), -1});
-      poly_units.push_back({n_upper, (long long)up16(b.m)});
-      for (int tm = 0; tm < nt; ++tm) poly_rows.push_back({nt - tm, (long long)up16(b.m)});
-      // Update: the tiles of one row block read the same rows of Xl, all of them the same B'
-      const int ni = (b.n + kNsTile - 1) / kNsTile, ntu = wide_tiles ? (b.m + 255) / 256 : nt;
-      std::vector<NsItem>& upd = wide_tiles ? L.ns_upd4 : L.ns_upd;
-      std::vector<std::pair<int, long long>>& units = wide_tiles ? upd4_units : upd_units;
-      for (int tm = 0; tm < ni; ++tm) {
-        for (int tn = 0; tn < ntu; ++tn) upd.push_back(NsItem{(int)q, tm, tn, 0, up16(b.m), -1});
-        units.push_back({ntu, (long long)up16(b.m)});
-      }
       for (int tr = 0; tr < (b.R + 63) / 64; ++tr)
         for (int tc = 0; tc < (b.C + 63) / 64; ++tc) L.nsb_split_items.push_back(NsTileItem{(int)q, tr, tc});
       L.nsb_mats.push_back(b);
     }
     L.nsb_plane_elems = pw;
     std::fill(L.ns_xalt.begin(), L.ns_xalt.end(), -1);   // the result always replaces the raw step
-    if (env_ns_xcd()) {
-      // with fewer runs than a few per XCD the stretches would be uneven: take the finer runs, or leave the order
-      auto pick = [](std::vector<NsItem>& items, const std::vector<std::pair<int, long long>>& coarse,
-                     const std::vector<std::pair<int, long long>>& fine) {
-        if (coarse.size() >= 4 * kXcds) xcd_interleave(items, coarse);
-        else if (fine.size() >= 4 * kXcds) xcd_interleave(items, fine);
+    // Groups of matrices.  The products of one matrix depend on each other, those of different matrices do not:
+    // each group runs its chain of launches on a stream of its own, so that the blocks of one group's launch
+    // fill the CUs that the tail of the other's leaves idle.  Matrices are dealt to the groups heaviest first.
+    int n_groups = std::min<int>(env_ns_groups(), std::max<size_t>(L.nsb_mats.size() / 8, 1));
+    std::vector<std::vector<int>> members(n_groups);
+    {
+      std::vector<int> order(L.nsb_mats.size());
+      for (size_t q = 0; q < order.size(); ++q) order[q] = (int)q;
+      auto work = [&](int q) { const NsBfMat& b = L.nsb_mats[q]; return (double)b.m * b.m * b.n; };
+      std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return work(x) > work(y); });
+      std::vector<double> load(n_groups, 0.0);
+      for (int q : order) {
+        const int g = (int)(std::min_element(load.begin(), load.end()) - load.begin());
+        members[g].push_back(q);
+        load[g] += work(q);
+      }
+      for (auto& mm : members) std::sort(mm.begin(), mm.end());   // neighbours in memory stay neighbours in the tables
+    }
+    L.ns_groups.clear();
+    L.ns_split.clear();
+    for (int g = 0; g < n_groups; ++g) {
+      // job runs that read the same operands: per matrix (slab), and finer, per row of tiles, for sets of few matrices
+      std::vector<std::pair<int, long long>> gram_units, poly_units, upd_units, upd4_units, gram_rows, poly_rows;
+      std::vector<NsItem> gram, poly, upd, upd4;
+      NsGroup grp{};
+      grp.split0 = (int)L.ns_split.size();
+      for (int q : members[g]) {
+        const NsBfMat& b = L.nsb_mats[q];
+        const bool wide_tiles = b.rows_m % 256 == 0 && up(b.m, 256) <= 1.06 * up(b.m, 128);
+        const int nt = (b.m + kNsTile - 1) / kNsTile, n_upper = nt * (nt + 1) / 2;
+        // Gram: the tiles of one matrix (of one slab of it) read the same rows of Xs; Poly: the same A
+        for (int sl = 0; sl < b.n_slabs; ++sl) {
+          const int k0 = b.n_slabs > 1 ? sl * kNsSlabK : 0;
+          const int k1 = b.n_slabs > 1 ? up16(std::min(b.n, (sl + 1) * kNsSlabK)) : up16(b.n);
+          for (int tm = 0; tm < nt; ++tm)
+            for (int tn = tm; tn < nt; ++tn) gram.push_back(NsItem{q, tm, tn, k0, k1, b.n_slabs > 1 ? sl : -1});
+          gram_units.push_back({n_upper, (long long)(k1 - k0)});
+          for (int tm = 0; tm < nt; ++tm) gram_rows.push_back({nt - tm, (long long)(k1 - k0)});
+        }
+        for (int tm = 0; tm < nt; ++tm)
+          for (int tn = tm; tn < nt; ++tn) poly.push_back(NsItem{q, tm, tn, 0, up16(b.m), -1});
+        poly_units.push_back({n_upper, (long long)up16(b.m)});
+        for (int tm = 0; tm < nt; ++tm) poly_rows.push_back({nt - tm, (long long)up16(b.m)});
+        // Update: the tiles of one row block read the same rows of Xl, all of them the same B'
+        const int ni = (b.n + kNsTile - 1) / kNsTile, ntu = wide_tiles ? (b.m + 255) / 256 : nt;
+        std::vector<NsItem>& u = wide_tiles ? upd4 : upd;
+        std::vector<std::pair<int, long long>>& units = wide_tiles ? upd4_units : upd_units;
+        for (int tm = 0; tm < ni; ++tm) {
+          for (int tn = 0; tn < ntu; ++tn) u.push_back(NsItem{q, tm, tn, 0, up16(b.m), -1});
+          units.push_back({ntu, (long long)up16(b.m)});
+        }
+        if (b.n_slabs > 1) {
+          L.ns_split.push_back(q);
+          grp.split_max_m = std::max(grp.split_max_m, b.m);
+        }
+      }
+      if (env_ns_xcd()) {
+        // with fewer runs than a few per XCD the stretches would be uneven: take the finer runs, or leave the order
+        auto pick = [](std::vector<NsItem>& items, const std::vector<std::pair<int, long long>>& coarse,
+                       const std::vector<std::pair<int, long long>>& fine) {
+          if (coarse.size() >= 4 * kXcds) xcd_interleave(items, coarse);
+          else if (fine.size() >= 4 * kXcds) xcd_interleave(items, fine);
+        };
+        pick(gram, gram_units, gram_rows);
+        pick(poly, poly_units, poly_rows);
+        pick(upd, upd_units, upd_units);
+        pick(upd4, upd4_units, upd4_units);
+      }
+      auto append = [](std::vector<NsItem>& all, const std::vector<NsItem>& part, int& first, int& count) {
+        first = (int)all.size();
+        count = (int)part.size();
+        all.insert(all.end(), part.begin(), part.end());
       };
-      pick(L.ns_gram, gram_units, gram_rows);
-      pick(L.ns_poly, poly_units, poly_rows);
-      pick(L.ns_upd, upd_units, upd_units);
-      pick(L.ns_upd4, upd4_units, upd4_units);
+      append(L.ns_gram, gram, grp.gram0, grp.n_gram);
+      append(L.ns_poly, poly, grp.poly0, grp.n_poly);
+      append(L.ns_upd, upd, grp.upd0, grp.n_upd);
+      append(L.ns_upd4, upd4, grp.upd40, grp.n_upd4);
+      grp.n_split = (int)L.ns_split.size() - grp.split0;
+      L.ns_groups.push_back(grp);
     }
     return;
   }
@@ -686,6 +742,9 @@ struct PyloPlan {
   bool stats_carried = false;
   hipStream_t side = nullptr;            // the LSTM runs next to the gradient sums on a stream of the plan's own
   hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+  // ELO-CELO2: the Newton-Schulz chains of the groups of matrices after the first run on streams of the plan's own
+  hipStream_t ns_side[3] = {nullptr, nullptr, nullptr};
+  hipEvent_t ns_fork = nullptr, ns_join[3] = {nullptr, nullptr, nullptr};
 
   template <class Tp>
   Tp* at(size_t off) const { return reinterpret_cast<Tp*>(ws + off); }
@@ -764,6 +823,11 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
     if (e == hipSuccess) e = hipEventCreateWithFlags(&P->ev_fork, hipEventDisableTiming);
     if (e == hipSuccess) e = hipEventCreateWithFlags(&P->ev_join, hipEventDisableTiming);
   }
+  for (size_t g = 1; g < L.ns_groups.size() && e == hipSuccess; ++g) {
+    if (g == 1) e = hipEventCreateWithFlags(&P->ns_fork, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&P->ns_side[g - 1], hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&P->ns_join[g - 1], hipEventDisableTiming);
+  }
   if (e != hipSuccess) {
     pylo_mi355_plan_destroy(P);
     return fail(std::string("plan_create: ") + hipGetErrorString(e));
@@ -778,6 +842,11 @@ int pylo_mi355_plan_destroy(PyloPlan* P) {
   if (P->ev_fork) (void)hipEventDestroy(P->ev_fork);
   if (P->ev_join) (void)hipEventDestroy(P->ev_join);
   if (P->side) (void)hipStreamDestroy(P->side);
+  if (P->ns_fork) (void)hipEventDestroy(P->ns_fork);
+  for (int g = 0; g < 3; ++g) {
+    if (P->ns_join[g]) (void)hipEventDestroy(P->ns_join[g]);
+    if (P->ns_side[g]) (void)hipStreamDestroy(P->ns_side[g]);
+  }
   for (int i = 0; i < kStageSlots; ++i) {
     if (P->ev[i]) (void)hipEventDestroy(P->ev[i]);
     if (P->stage[i]) (void)hipHostFree(P->stage[i]);
@@ -1225,24 +1294,40 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
       hipLaunchKernelGGL(k_ns_bf_split, dim3((unsigned)L.nsb_split_items.size()), dim3(256), 0, s, bmats, sitems, dyn,
                          (const float*)scale, pw);
       const NsItem* upd4 = P->at<NsItem>(L.off_ns_upd4);
-      const int n_upd4 = (int)L.ns_upd4.size();
       if (int rc = ns_bf_lds_once()) return rc;
+      // every group of matrices on a stream of its own, the first on the caller's
+      const int n_groups = (int)L.ns_groups.size();
+      if (n_groups > 1 && ns_iters > 0) {
+        HIP_TRY(hipEventRecord(P->ns_fork, s));
+        for (int g = 1; g < n_groups; ++g) HIP_TRY(hipStreamWaitEvent(P->ns_side[g - 1], P->ns_fork, 0));
+      }
       for (int it = 0; it < ns_iters; ++it) {
         const int par = it & 1, last = it == ns_iters - 1;
-        hipLaunchKernelGGL((k_ns_bf_gemm<kNsGram, 2>), dim3(n_gram), dim3(256), bf_gemm_lds(2), s, bmats, gram, dyn, ns_ws,
-                           pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
-        if (n_split > 0)
-          hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)L.ns_max_m * L.ns_max_m + 255) / 256, n_split), dim3(256),
-                             0, s, bmats, split, dyn, ns_ws, pw);
-        hipLaunchKernelGGL((k_ns_bf_gemm<kNsPoly, 2>), dim3(n_poly), dim3(256), bf_gemm_lds(2), s, bmats, poly, dyn, ns_ws,
-                           pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
-        if (n_upd4 > 0)
-          hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 4>), dim3(n_upd4), dim3(256), bf_gemm_lds(4), s, bmats, upd4, dyn,
-                             ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
-        if (n_upd > 0)
-          hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 2>), dim3(n_upd), dim3(256), bf_gemm_lds(2), s, bmats, upd, dyn,
-                             ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+        for (int g = 0; g < n_groups; ++g) {
+          const NsGroup& G = L.ns_groups[g];
+          hipStream_t sg = g == 0 ? s : P->ns_side[g - 1];
+          if (G.n_gram > 0)
+            hipLaunchKernelGGL((k_ns_bf_gemm<kNsGram, 2>), dim3(G.n_gram), dim3(256), bf_gemm_lds(2), sg, bmats, gram + G.gram0,
+                               dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+          if (G.n_split > 0)
+            hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)G.split_max_m * G.split_max_m + 255) / 256, G.n_split),
+                               dim3(256), 0, sg, bmats, split + G.split0, dyn, ns_ws, pw);
+          if (G.n_poly > 0)
+            hipLaunchKernelGGL((k_ns_bf_gemm<kNsPoly, 2>), dim3(G.n_poly), dim3(256), bf_gemm_lds(2), sg, bmats, poly + G.poly0,
+                               dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+          if (G.n_upd4 > 0)
+            hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 4>), dim3(G.n_upd4), dim3(256), bf_gemm_lds(4), sg, bmats,
+                               upd4 + G.upd40, dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+          if (G.n_upd > 0)
+            hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 2>), dim3(G.n_upd), dim3(256), bf_gemm_lds(2), sg, bmats,
+                               upd + G.upd0, dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+        }
       }
+      if (n_groups > 1 && ns_iters > 0)
+        for (int g = 1; g < n_groups; ++g) {
+          HIP_TRY(hipEventRecord(P->ns_join[g - 1], P->ns_side[g - 1]));
+          HIP_TRY(hipStreamWaitEvent(s, P->ns_join[g - 1], 0));
+        }
     } else
     for (int it = 0; it < ns_iters; ++it) {
       const int first = it == 0, par = it & 1;

@@ -1,6 +1,6 @@
 """Benchmark of the fused learned-optimizer step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gpt2s|cfg1|vit_velo|llama_adafac|stress_velo|stress_celo2|stream_ceiling] [--fused-only]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gpt2s|cfg1|vit_velo|llama_adafac|stress_velo|stress_celo2|stream_ceiling|matrix_ceiling] [--fused-only]
 
 Workload (default): BASELINE config 2 -- ELO-CELO2 on a GPT-2-small-shaped fp32 parameter set
 (98 tensors, 124 355 328 parameters), synthetic per-tensor Gaussian gradients with log-uniform
@@ -199,7 +199,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gpt2s", choices=["gpt2s", "cfg1", "vit_velo", "llama_adafac", "stress_velo", "stress_celo2", "stream_ceiling"])
+    ap.add_argument("--workload", default="gpt2s", choices=["gpt2s", "cfg1", "vit_velo", "llama_adafac", "stress_velo", "stress_celo2", "stream_ceiling", "matrix_ceiling"])
     ap.add_argument("--fused-only", action="store_true",
                     help="loop the C-ABI call alone (no Newton-Schulz / apply), e.g. under rocprofv3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -226,6 +226,8 @@ def main():
         return
     if a.workload == "stream_ceiling":
         return stream_ceiling(a)
+    if a.workload == "matrix_ceiling":
+        return matrix_ceiling(a)
     dev = torch.device("cuda:0")
     shapes = gpt2_small_shapes() if a.workload == "gpt2s" else cfg1_shapes()
     torch.manual_seed(1)
@@ -383,6 +385,55 @@ def stream_ceiling(a):
                       "warmup": a.warmup, "elements_per_array": n, "peak_GBps": HBM_PEAK_GBS, "mixes": out}))
 
 
+def matrix_ceiling(a):
+    """What the bf16 matrix pipe delivers for the instruction mix of the Newton-Schulz products: the library's
+    bare matrix-pipe kernel (the update product's main loop, 128 x 256 tiles, reduction length 768) on planes of
+    the GPT-2-small set's size, with the data path taken away in steps, on random data and on zeros (the pipe's
+    power, and with it the clock, depends on the operands).  The yardstick next to the data sheet's 2.5 PFLOP/s."""
+    import ctypes as C
+
+    import torch
+
+    from pylo_amd import _lib
+
+    lib = _lib.load()
+    lib.pylo_mi355_matrix_probe.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    dev = torch.device("cuda:0")
+    rows_x, rows_b, k = 163840, 768, 768          # 125.8 M elements of X against a 768 x 768 matrix
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    res = {}
+    for data in ("random", "zeros"):
+        gen = torch.Generator(device=dev).manual_seed(0)
+        mk = (lambda n: torch.randint(-32768, 32767, (n,), generator=gen, device=dev, dtype=torch.int16)) if data == "random" \
+            else (lambda n: torch.zeros(n, device=dev, dtype=torch.int16))
+        # random bit patterns with the exponents of numbers around 1 (no NaN or infinity): sign, exponent 120..127, 7 mantissa bits
+        def planes(n):
+            t = mk(n)
+            if data == "random":
+                t = (t & -32641) | (((t.to(torch.int32) >> 7) & 7) + 120).to(torch.int16) << 7
+            return t
+        x = planes(rows_x * k * 3)
+        b = planes(rows_b * k * 3)
+        out = torch.zeros((rows_x // 128) * (rows_b // 256) * 256, device=dev)
+        for mode, name in ((0, "product loop"), (1, "LDS reads + matrix instructions"), (2, "matrix instructions only")):
+            call = lambda: _lib.check(lib.pylo_mi355_matrix_probe(x.data_ptr(), rows_x, b.data_ptr(), rows_b, k, mode,
+                                                                  out.data_ptr(), stream), "matrix_probe")
+            for _ in range(max(a.warmup, 3)):
+                call()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(a.steps):
+                call()
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / a.steps
+            res[f"{name}, {data}"] = {"ms": ms, "PFLOPs": 12.0 * rows_x * rows_b * k / ms / 1e12}
+        del x, b, out
+    print(json.dumps({"metric": "attainable_bf16_matrix_rate", "unit": "PFLOP/s", "n_gpus": 1, "steps": a.steps,
+                      "warmup": a.warmup, "tile": "128x256, 6 x v_mfma_f32_32x32x16_bf16 per fp32 tile product",
+                      "peak_PFLOPs": 2.5, "cases": res}))
+
+
 def stress_workload(workload, steps, warmup):
     """Config 5 (3 000 small tensors + one 32000 x 4096 embedding, Student-t gradients): the fused VeLO step or the
     fused ELO-CELO2 element call.  What it measures is the multi-tensor launch table: how long the host takes to
@@ -408,8 +459,8 @@ def stress_workload(workload, steps, warmup):
         label = "VeLO fused step"
     else:
         opt = ELO_CELO2_CUDA(params, lr=3e-4, network=CELO2MLP(), hf_key=None)
-        step = opt.fused_step
-        label = "ELO_CELO2 fused element call (no Newton-Schulz)"
+        step = opt.step
+        label = "ELO_CELO2 whole optimizer.step() (fused call, Newton-Schulz of every matrix incl. 32000 x 4096, update)"
     # (one call around the tenth in flight takes 0.1 s on the host, once; it is kept out of the timed region)
     for _ in range(max(warmup, 16)):
         step()
@@ -428,12 +479,37 @@ def stress_workload(workload, steps, warmup):
     per = plan.timing_end()
     n = sum(p.numel() for p in params)
     ms = (t2 - t0) * 1e3 / steps
-    return {"metric": "params_updated_per_sec (fused step, C-ABI call)", "value": n / (ms * 1e-3), "unit": "params/s",
+    extra = {}
+    if workload == "stress_celo2":
+        # the fused element call alone, and the same step with the 32000 x 4096 matrix in an is_embedding group
+        # (AdamW, no Newton-Schulz on it): what the 3 000 small tensors cost by themselves
+        extra["fused_call_ms"] = float(per.sum(axis=1).mean())
+        del opt
+        torch.cuda.empty_cache()
+        opt2 = ELO_CELO2_CUDA([{"params": params[:-1]}, {"params": params[-1:], "is_embedding": True}], lr=3e-4,
+                              network=CELO2MLP(), hf_key=None)
+        for _ in range(max(warmup, 16)):
+            opt2.step()
+        torch.cuda.synchronize()
+        t3a = time.perf_counter()
+        for _ in range(steps):
+            opt2.step()
+        t3b = time.perf_counter()
+        torch.cuda.synchronize()
+        t3c = time.perf_counter()
+        extra["embedding_as_adamw_group"] = {"ms_per_step": (t3c - t3a) * 1e3 / steps,
+                                             "host_enqueue_ms_per_step": (t3b - t3a) * 1e3 / steps}
+        n_mats = sum(1 for s_ in shapes if len(s_) == 2)
+        extra["matrices_orthogonalised_by_library_kernels"] = n_mats
+        extra["matrices_left_to_torch_products"] = sum(1 for i, s_ in enumerate(shapes[:-1]) if len(s_) == 2 and not opt2._ns_ok[i])
+        plan = opt2._plan
+    return {"metric": "params_updated_per_sec (fused step, C-ABI call)" if workload == "stress_velo" else
+            "params_updated_per_sec (whole optimizer.step())", "value": n / (ms * 1e-3), "unit": "params/s",
             "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "f32", "data": "synthetic",
             "config": {"workload": f"{label}, stress set of {len(shapes)} tensors (3 000 of 1 - 65 536 elements, 1-D and odd "
                                    f"2-D, plus 32000 x 4096)", "params": n, "tensors": len(shapes)},
-            "host_enqueue_ms_per_step": (t1 - t0) * 1e3 / steps,
+            "host_enqueue_ms_per_step": (t1 - t0) * 1e3 / steps, **extra,
             "sum_of_launch_intervals_ms": float(per.sum(axis=1).mean()),
             "launch_ms": {nm: float(v) for nm, v in zip(plan.launch_names(), per.mean(axis=0))}}
 

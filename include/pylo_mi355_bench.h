@@ -33,6 +33,18 @@ const char* pylo_mi355_plan_launch_name(const PyloPlan* plan, int launch);
 int pylo_mi355_stream_probe(const float* in, float* out, size_t n, int reads, int writes, int nontemporal,
                             void* stream);
 
+/* Bare matrix-pipe kernel, for benchmarks (no counterpart in the reference): the main loop of the Newton-Schulz
+   update product (tiles of 128 x 256 outputs, six v_mfma_f32_32x32x16_bf16 per fp32 tile product) over caller-
+   provided operand planes, every tile job over k_steps reduction steps.  x_planes: rows_x rows (a multiple of
+   128), b_planes: rows_b rows (a multiple of 256), both laid out [k_steps / 16][rows][3 planes][16] bf16
+   (96 bytes a row and block of 16 steps).  mode 0: the product's own loop (operands staged from memory into
+   LDS every 16 steps); 1: the operands of the first 16 steps staged once and read from LDS in every step;
+   2: their fragments kept in registers, matrix instructions only.  out: (rows_x / 128) (rows_b / 256) x 256
+   floats.  What the planes hold decides the power the matrix pipe draws and with it the clock: zeros run
+   faster than data. */
+int pylo_mi355_matrix_probe(const void* x_planes, int rows_x, const void* b_planes, int rows_b, int k_steps, int mode,
+                            float* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1944,3 +1944,102 @@ extern "C" int pylo_mi355_stream_probe(const float* in, float* out, size_t n, in
   HIP_TRY(hipGetLastError());
   return 0;
 }
+
+// ---------------------------------------------------------------------------------------------
+// Bare matrix-pipe kernel (benchmark instrumentation): what the bf16 matrix instructions deliver for the
+// instruction mix of the Newton-Schulz update product, with parts of its data path taken away
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+// The main loop of k_ns_bf_gemm<kNsUpdate, 4> (128 x 256 outputs, six v_mfma_f32_32x32x16_bf16 per pair of
+// 32 x 32 blocks and 16 reduction steps) over synthetic planes.  MODE 0: as in the product (operands staged
+// from memory into LDS every 16 steps); 1: the first stage is staged once and read from LDS in every step (no
+// global loads, no barriers); 2: the first stage's fragments stay in registers (matrix instructions only).
+template <int MODE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k_matrix_probe(
+    const bfbits* __restrict__ X, int rows_x, const bfbits* __restrict__ B, int rows_b, int K, float* __restrict__ out) {
+  extern __shared__ __attribute__((aligned(16))) char lds_[];
+  PYLO_LDS char* lds = (PYLO_LDS char*)lds_;
+  constexpr int WN = 4, RB = 64 * WN, SA = 128 * 96;
+  const int nj = rows_b / RB, i0 = (blockIdx.x / nj) * 128, j0 = (blockIdx.x % nj) * RB;
+  v16f acc[2][WN];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  const BfPlanes PX{X, rows_x}, PB{B, rows_b};
+  if (MODE == 0) {
+    bf_tile_product<WN>(PX, i0, PB, j0, 0, K, lds, acc);
+  } else {
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wi = (wave >> 1) * 64, wj = (wave & 1) * 32 * WN;
+    const int kg = lane >> 5, lo = lane & 31;
+    int offa[3], offb[RB * 6 / 256];
+    bf_stage_offsets<128>(wave, lane, offa);
+    bf_stage_offsets<RB>(wave, lane, offb);
+    bf_stage_issue<128>((const char*)X + (size_t)i0 * 96, offa, lds, wave);
+    bf_stage_issue<RB>((const char*)B + (size_t)j0 * 96, offb, lds + SA, wave);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    const int sw = 16 * (kg ^ ((lo >> 3) & 1));
+    const int oa = (wi + lo) * 96 + sw, ob = SA + (wj + lo) * 96 + sw;
+    bf16x8 a[2][3], b[WN][3];
+    for (int k = 0; k < K; k += kBfBK) {
+      if (MODE == 1 || k == 0) {
+#pragma unroll
+        for (int q = 0; q < 3; ++q) {
+#pragma unroll
+          for (int i = 0; i < 2; ++i) a[i][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + oa + i * 32 * 96 + q * 32));
+#pragma unroll
+          for (int j = 0; j < WN; ++j) b[j][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + ob + j * 32 * 96 + q * 32));
+        }
+      }
+#pragma unroll
+      for (int term = 0; term < 6; ++term) {
+        constexpr int pa[6] = {2, 0, 1, 1, 0, 0}, pb[6] = {0, 2, 1, 0, 1, 0};
+#pragma unroll
+        for (int hi = 0; hi < 2; ++hi)
+#pragma unroll
+          for (int hj = 0; hj < WN; ++hj)
+            acc[hi][hj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[hi][pa[term]], b[hj][pb[term]], acc[hi][hj], 0, 0, 0);
+      }
+      if (MODE == 1) asm volatile("" ::: "memory");   // the fragments are read again in the next step
+    }
+  }
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sum += acc[i][j][r];
+  out[(size_t)blockIdx.x * 256 + threadIdx.x] = sum;
+}
+
+}  // namespace
+
+extern "C" int pylo_mi355_matrix_probe(const void* x_planes, int rows_x, const void* b_planes, int rows_b, int k_steps,
+                                       int mode, float* out, void* stream) {
+  if (!x_planes || !b_planes || !out) return fail("matrix_probe: null pointer");
+  if (rows_x <= 0 || rows_x % 128 != 0 || rows_b <= 0 || rows_b % 256 != 0 || k_steps <= 0 || k_steps % 16 != 0)
+    return fail("matrix_probe: rows_x must be a multiple of 128, rows_b of 256, k_steps of 16");
+  if (mode < 0 || mode > 2) return fail("matrix_probe: mode must be 0, 1 or 2");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const unsigned grid = (unsigned)(rows_x / 128) * (unsigned)(rows_b / 256);
+  static std::mutex mu;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<0>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(4)));
+    HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<1>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(4)));
+    HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(4)));
+  }
+  const bfbits* X = static_cast<const bfbits*>(x_planes);
+  const bfbits* B = static_cast<const bfbits*>(b_planes);
+  if (mode == 0) hipLaunchKernelGGL(k_matrix_probe<0>, dim3(grid), dim3(256), bf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
+  else if (mode == 1) hipLaunchKernelGGL(k_matrix_probe<1>, dim3(grid), dim3(256), bf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
+  else hipLaunchKernelGGL(k_matrix_probe<2>, dim3(grid), dim3(256), bf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}

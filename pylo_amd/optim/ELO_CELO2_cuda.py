@@ -212,6 +212,8 @@ class ELO_CELO2_CUDA(Optimizer):
         self._adam_b1, self._adam_b2 = float(bm[0]), float(self.beta_rms[-1])
         self._plan = None
         self._plan_key = None
+        self._fast_taken = False
+        self._fin_fast = None
         self._lib_ns = os.environ.get("PYLO_MI355_NS", "lib") != "torch"
 
     # ------------------------------------------------------------------ plan
@@ -256,6 +258,7 @@ class ELO_CELO2_CUDA(Optimizer):
                 self._raw[i] = buf[j]
             self._raw_groups.append((buf, idx))
         self._fin_args = np.zeros(len(tensors), dtype=_lib.ARGS_DTYPE)
+        self._fin_fast = None
         self._ns_ok = [self._plan.orthogonalize_supported(i) for i in range(len(tensors))]
         if self.capturable:
             self._reset_device_steps(tensors)
@@ -398,6 +401,7 @@ class ELO_CELO2_CUDA(Optimizer):
         if not self.capturable:     # else the library derives them from its device counters
             args["bc1"], args["bc2"] = self._adam_corrections_fast(fast, per_group)
         self._launch_step()
+        self._fast_taken = True
         return fast["tensors"]
 
     @torch.no_grad()
@@ -409,6 +413,7 @@ class ELO_CELO2_CUDA(Optimizer):
             if done is not None:
                 return done
             self._fast = None
+        self._fast_taken = False
         tensors = self._tensors()
         self._ensure_plan(tensors)
         plan = self._plan
@@ -476,13 +481,69 @@ class ELO_CELO2_CUDA(Optimizer):
     @torch.no_grad()
     def finish_step(self, tensors):
         """Newton-Schulz, RMS normalisation and the parameter update of the MLP tensors
-        (pylo/optim/ELO_CELO2_cuda.py:288-296).  Matrices whose dims are multiples of 4 are orthogonalised by
-        the library's own fp32 matrix-pipe kernels inside the finishing call; other shapes, tensors with more
+        (pylo/optim/ELO_CELO2_cuda.py:288-296).  Matrices are orthogonalised by the library's own matrix-pipe
+        kernels inside the finishing call (fp32 accuracy on the bf16 matrix instructions, any two dims; with
+        ``PYLO_MI355_NS_F32=1`` the fp32 matrix instructions, dims that are multiples of 4); tensors with more
         than two dims and buckets in which a tensor sat the step out go through the batched torch products
-        (also with ``PYLO_MI355_NS=torch`` in the environment, for comparisons)."""
+        (also everything with ``PYLO_MI355_NS=torch`` in the environment, for comparisons)."""
         self._finish_step(tensors)
 
+    # The finishing call's table has one row per tensor as well.  When the step went through the cached rows of
+    # the fused call (every tensor has a gradient) and the library finishes every MLP tensor itself (no tensor
+    # with more than two dims, no param_scale_mult, no torch products), its static columns are kept too and a
+    # step refreshes parameter pointers and the groups' scalars with a few array operations, whatever the
+    # number of tensors.
+    def _fin_fast_key(self):
+        return (self.ns_iters, self._lib_ns,
+                tuple((g["orthogonalize"], g["param_scale_mult"]) for g in self.param_groups))
+
+    def _build_fin_fast(self, tensors):
+        if any(g["param_scale_mult"] for g in self.param_groups):
+            return None
+        idx, flags = [], []
+        for i, (group, p, adam) in enumerate(tensors):
+            if adam:
+                continue
+            if p.dim() > 2:
+                return None
+            orth = bool(group["orthogonalize"]) and p.dim() == 2 and self.ns_iters > 0
+            if orth and not (self._lib_ns and self._ns_ok[i]):
+                return None
+            idx.append(i)
+            flags.append(_lib.ARG_ORTHOGONALIZE if orth else 0)
+        if not idx:
+            return None
+        idx = np.asarray(idx, dtype=np.int64)
+        fin = self._fin_args
+        fin[:] = 0
+        fin["grad"][idx] = 1          # "takes part"; the gradient itself is not read
+        fin["step_out"][idx] = [self._raw[i].data_ptr() for i in idx]
+        fin["flags"][idx] = flags
+        return dict(key=self._fin_fast_key(), idx=idx, gidx=self._fast["gidx"][idx])
+
+    def _finish_step_fast(self, ff):
+        groups = self.param_groups
+        fin, idx, gidx = self._fin_args, ff["idx"], ff["gidx"]
+        fin["param"][idx] = self._plan.args["param"][idx]
+        fin["lr"][idx] = np.asarray([g["lr"] for g in groups], dtype=np.float64)[gidx]
+        fin["weight_decay"][idx] = np.asarray([g["weight_decay"] for g in groups], dtype=np.float64)[gidx]
+        fin["step_mult"][idx] = np.asarray([g["rmsmult"] for g in groups], dtype=np.float64)[gidx]
+        if self._capturing():
+            table = self._plan.pinned_table(1)
+            table[:] = fin
+            fin = table
+        with torch.cuda.device(self.device):
+            self._plan.celo2_orthogonalize_finish(fin, self.ns_coeffs, self.ns_iters, self.ns_eps,
+                                                  torch.cuda.current_stream(self.device).cuda_stream)
+
     def _finish_step(self, tensors):
+        if getattr(self, "_fast", None) is not None and self._fast_taken:
+            ff = getattr(self, "_fin_fast", None)
+            if ff is None or ff["key"] != self._fin_fast_key():
+                ff = self._fin_fast = self._build_fin_fast(tensors) or dict(key=self._fin_fast_key(), idx=None)
+            if ff["idx"] is not None:
+                return self._finish_step_fast(ff)
+        self._fin_fast = None      # the general path below rewrites the table
         fin = self._fin_args
         fin["grad"] = 0
         fin["flags"] = 0

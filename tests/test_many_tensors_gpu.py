@@ -42,6 +42,9 @@ def _inputs(shapes, seed, steps):
 
 
 def test_celo2_many_tensors():
+    """Whole ``ELO_CELO2_CUDA.step()`` on the 3 001 tensors, free-running: Newton-Schulz of the ~1 800 odd-shaped
+    matrices and of the 32000 x 4096 one by the library's kernels, normalisation and the parameter update;
+    parameters are never re-synchronised with the oracle."""
     from oracle import pylo_oracle as O
     from pylo_amd import ELO_CELO2_CUDA
     from pylo_amd.models import CELO2MLP
@@ -49,34 +52,39 @@ def test_celo2_many_tensors():
     torch.manual_seed(1)
     net = CELO2MLP()
     shapes = _shapes(3000, 11, (32000, 4096))
-    init, grads = _inputs(shapes, 12, 2)
+    steps = 3
+    init, grads = _inputs(shapes, 12, steps)
     ref = [v.double() for v in init]
     gpu = [torch.nn.Parameter(v.clone()) for v in init]
     orc = O.EloCelo2Oracle(ref, net.state_dict(), lr=3.16e-4, adam_lr_mult=20.0, device="cuda").double_()
     opt = ELO_CELO2_CUDA(gpu, lr=3.16e-4, adam_lr_mult=20.0, network=net, hf_key=None)
-    worst = 0.0
-    for t in range(2):
+    worst = worst_p = 0.0
+    for t in range(steps):
         raw = {}
         for p, g in zip(gpu, grads[t]):
             p.grad = g
         orc.step([g.double() for g in grads[t]], keep_raw=raw)
-        opt.fused_step()
+        tensors = opt.fused_step()
+        if t >= 1:
+            assert opt._fast_taken      # the cached argument rows
         for i, p in enumerate(gpu):
             st, so = opt.state[p], orc.state[i]
             checks = [("mom", st["mom"], so["mom"]), ("rms", st["rms"], so["rms"])]
             if p.dim() >= 2:
                 checks += [("fac_r", st["fac_r"], so["fac_r"]), ("fac_c", st["fac_c"], so["fac_c"]),
                            ("raw", opt._raw[i], raw[i])]
-            else:
-                checks.append(("param", p, ref[i]))
             for tag, got, want in checks:
                 e = max_err(got, want, REL, ABS)
                 worst = max(worst, e)
                 assert e <= 1.0, (t, i, shapes[i], tag, e)
-            p.data.copy_(ref[i].float())   # keep both on the oracle's parameters (Newton-Schulz runs only there)
-            ref[i].copy_(p.data.double())
         del raw
-    print("celo2 many tensors worst err/tol", worst)
+        opt.finish_step(tensors)
+        assert all(opt._ns_ok[i] for i, s in enumerate(shapes) if len(s) == 2)   # no torch product on this set
+        for i, p in enumerate(gpu):
+            e = max_err(p, ref[i], REL, ABS)
+            worst_p = max(worst_p, e)
+            assert e <= 1.0, (t, i, shapes[i], "param", e)
+    print("celo2 many tensors worst err/tol: states and raw steps", worst, ", parameters (free-running)", worst_p)
 
 
 def test_velo_many_tensors():
@@ -130,3 +138,13 @@ def test_velo_many_tensors():
             assert e <= 1.0, (t, tag, e)
     print("velo many tensors worst err/tol", worst, "(against the fp64 evaluation alone:", worst64,
           ", against the fp32 evaluation alone:", worst32, ")")
+    # the plain bars, kept as numbers: against the exact (fp64) value the HIP path stays within 1.5 tolerances
+    # on every value of the set, closer than the reference's own fp32 arithmetic is to it
+    assert worst64 <= 1.5, worst64
+    import json
+    import os
+    out = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+    if os.path.isdir(out):
+        with open(os.path.join(out, "velo_many_tensors_errors.json"), "w") as f:
+            json.dump({"worst_widened": worst, "worst_vs_fp64": worst64, "worst_vs_fp32_oracle": worst32,
+                       "rel": REL, "abs": ABS}, f)

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PYLO_MI355_ABI_VERSION 7
+#define PYLO_MI355_ABI_VERSION 8
 #define PYLO_MAX_DIMS 8
 #define PYLO_MAX_GROUPS 8   /* parameter groups with their own step counter (VeLO) */
 
@@ -290,6 +290,19 @@ int pylo_mi355_velo_step(PyloPlan* plan, const PyloTensorArgs* args, const PyloD
    sums from the tensors again, each pass a launch of its own.  No counterpart in the reference, which
    recomputes everything every step. */
 int pylo_mi355_plan_invalidate_statistics(PyloPlan* plan);
+
+/* The guard of those carried sums.  A step that runs on them also takes the sum of p^2 of every tensor from
+   the tensor itself (its statistics items read the parameter anyway) and holds it against the carried one.
+   Where they differ by more than 1e-3 relative -- the parameter was written by somebody else since the last
+   step and the plan was not told -- the LSTM of that step has already run on the stale sum: the tensor's
+   step of that call is NaN (loud, like the fused pass's bounded wait) and the plan's flag is raised.  This
+   call returns 0, or 1 + the index of a tensor the guard caught since the last
+   pylo_mi355_plan_invalidate_statistics; it reads a pinned copy that every step refreshes at its end and does
+   not wait for the GPU, so it may lag the step that raised the flag by the steps still in flight.  Writes
+   that leave sum p^2 within 1e-3 also leave the LSTM's input feature within that, and are not flagged; the
+   sums over `mom` and `rms` are not guarded (the Python class watches those tensors' identity and version
+   counters).  No counterpart in the reference, which recomputes everything every step. */
+int pylo_mi355_plan_statistics_stale(const PyloPlan* plan);
 
 /*
  * AdafacLO step (replaces cuda_lo.learned_optimizer_kernel, pylo/csrc/learned_optimizer.cu:303-394, for

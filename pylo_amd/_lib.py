@@ -107,9 +107,10 @@ def load():
     lib.pylo_mi355_adafac_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.c_void_p, C.c_float,
                                            C.c_void_p]
     lib.pylo_mi355_plan_invalidate_statistics.argtypes = [C.c_void_p]
+    lib.pylo_mi355_plan_statistics_stale.argtypes = [C.c_void_p]
     lib.pylo_mi355_plan_arg_table.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_void_p)]
     lib.pylo_mi355_plan_device_steps.argtypes = [C.c_void_p, C.POINTER(DeviceSteps)]
-    if lib.pylo_mi355_abi_version() != 7:
+    if lib.pylo_mi355_abi_version() != 8:
         raise RuntimeError("libpylo_mi355.so: ABI version mismatch, rebuild it")
     _lib = lib
     return lib
@@ -227,6 +228,10 @@ class Plan:
     def invalidate_statistics(self) -> None:
         """VeLO: parameters or accumulators were written by someone else since the plan's last step."""
         check(load().pylo_mi355_plan_invalidate_statistics(self._h), "plan_invalidate_statistics")
+
+    def statistics_stale(self) -> int:
+        """VeLO: 0, or 1 + the index of a tensor whose carried sum of p^2 did not match the tensor (no wait)."""
+        return load().pylo_mi355_plan_statistics_stale(self._h)
 
     def orthogonalize_supported(self, i: int) -> bool:
         return load().pylo_mi355_plan_orthogonalize_supported(self._h, i) == 1

@@ -576,7 +576,8 @@ __global__ __launch_bounds__(kFoldThreads) void k_velo_feat(const TDesc* __restr
                                                             float* __restrict__ xfeat, int H,
                                                             const float* __restrict__ w2t, const float* __restrict__ b2,
                                                             const float* __restrict__ wft, const float* __restrict__ bf,
-                                                            float* __restrict__ mixbuf, int* __restrict__ sync) {
+                                                            float* __restrict__ mixbuf, int* __restrict__ sync,
+                                                            double* __restrict__ carried_p2) {
   constexpr int G = kFoldThreads / kNewSumW;
   __shared__ double part[G][kNewSumW];
   __shared__ double tot[kStatW];
@@ -609,6 +610,7 @@ __global__ __launch_bounds__(kFoldThreads) void k_velo_feat(const TDesc* __restr
     for (int g2 = 0; g2 < G; ++g2) s += part[g2][threadIdx.x];
     const int q = threadIdx.x;   // 0: sum p^2 | 1..3: m | 4..6: m^2 | 7: rms | 8: rms^2
     tot[q == 0 ? 2 : q < 4 ? kSumM + q - 1 : q < 7 ? kSumMM + q - 4 : q == 7 ? kSumR : kSumRR] = s;
+    if (q == 0) carried_p2[t] = s;   // the statistics items of this step hold it against the sum they take themselves
   }
   __syncthreads();
   velo_row_features(d, a, t, T, tot, nullptr, piv, ls, st, xfeat, H, w2t, b2, wft, bf, mixbuf, xs);
@@ -1192,7 +1194,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                                                         const float* __restrict__ wmix, float* __restrict__ wfold,
                                                         double* __restrict__ stats_part, const float* __restrict__ piv,
                                                         double* __restrict__ newsum_part, int* __restrict__ sync,
-                                                        int n_tensors) {
+                                                        int n_tensors, const double* __restrict__ carried_p2,
+                                                        int* __restrict__ stale, int stale_gen) {
   __shared__ float red[kWaves][38];
   __shared__ double part[kThreads / 30][30];
   __shared__ float sc[30];
@@ -1246,6 +1249,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
   __syncthreads();
   if (!s_flag) return;
   // the tensor's last statistics block: channel sums in row order, then the folded block
+  __shared__ int poison_s;
+  if (threadIdx.x == 0) poison_s = 0;
   constexpr int G = kThreads / 30;
   const int c = threadIdx.x % 30, gI = threadIdx.x / 30;
   if (gI < G) {
@@ -1270,13 +1275,25 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     for (int g2 = 0; g2 < G; ++g2) s += part[g2][threadIdx.x];
     const double n = (double)(d.n > 0 ? d.n : 1);
     sc[threadIdx.x] = rsq(1e-5f + (float)(s / n));
-    if (threadIdx.x == 2) pscale_s = sqrtf((float)(s / n) + 1e-9f);   // channel 2 is the parameter
+    if (threadIdx.x == 2) {   // channel 2 is the parameter
+      pscale_s = sqrtf((float)(s / n) + 1e-9f);
+      // The LSTM of this step was fed the sum of p^2 that the previous step's apply items carried over; `s` is
+      // the same sum over the parameter as it stands now.  They differ (beyond the rounding of two summation
+      // orders) only if somebody else wrote the parameter in between without the plan being told: the
+      // tensor's step is poisoned and the plan's flag raised rather than a step taken on stale statistics.
+      const double carried = carried_p2[it.tensor], big = fmax(fabs(s), fabs(carried));
+      if (!(fabs(s - carried) <= 1e-3 * big)) {
+        poison_s = 1;
+        __hip_atomic_store(stale + 1, it.tensor, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(stale, stale_gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
   }
   __syncthreads();
   const float* wm = wmix + (size_t)it.tensor * 160;
   if (threadIdx.x < kVFold)
     coh_store_wait(wfold + (size_t)it.tensor * kVFold + threadIdx.x,
-                   velo_fold_entry(d, wm, sc, pscale_s, wm[kVBank], threadIdx.x));
+                   poison_s ? __builtin_nanf("") : velo_fold_entry(d, wm, sc, pscale_s, wm[kVBank], threadIdx.x));
   __syncthreads();   // every folded weight has been performed
   if (threadIdx.x == 0) __hip_atomic_store(sync + n_tensors + it.tensor, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }

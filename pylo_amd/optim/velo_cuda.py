@@ -298,6 +298,17 @@ class VeLO_CUDA(Optimizer):
         self._ensure_plan(tensors)
         plan = self._plan
         n = len(tensors)
+        bad = plan.statistics_stale()
+        if bad:
+            # the device-side guard of the carried sums (see invalidate_statistics) caught a parameter that was
+            # written from outside between two steps: that step's update of the tensor is NaN
+            self.invalidate_statistics()
+            raise RuntimeError(
+                f"VeLO_CUDA: parameter {bad - 1} was written between two steps in a way the optimizer does not see "
+                "(through .data or by a custom kernel) and the step after it ran on the LSTM input statistics "
+                "carried over from before the write; that step's update of the tensor was set to NaN. Call "
+                "invalidate_statistics() after such writes, or write through in-place torch operations on the "
+                "parameter itself.")
         if self.lstm_hidden_state[0].shape[0] != n:
             raise RuntimeError("VeLO_CUDA: the LSTM state does not match the number of parameters")
         if not torch.is_tensor(loss):
@@ -328,9 +339,10 @@ class VeLO_CUDA(Optimizer):
                     fast = self._fast = None
                     break
         if fast is not None:
-            for state, key, t in fast["alive"]:
-                # a state tensor was replaced: the cached pointers are stale (and so are the carried sums)
-                if state.get(key) is not t:
+            for state, key, t, version in fast["alive"]:
+                # a state tensor was replaced (the cached pointers are stale) or written in place through torch
+                # (the carried sums over mom / rms are): the library's own writes do not count in `_version`
+                if state.get(key) is not t or t._version != version:
                     fast = self._fast = None
                     break
             else:
@@ -390,7 +402,7 @@ class VeLO_CUDA(Optimizer):
                 # the walk then costs milliseconds a step: there, the factored accumulators must be updated in
                 # place or through load_state_dict()
                 keys = ("mom", "rms", "fac_vec_row", "fac_vec_col", "fac_vec_v") if n <= 512 else ("mom", "rms")
-                alive = [(self.state[p], k, self.state[p][k]) for _, _, p in tensors for k in keys]
+                alive = [(self.state[p], k, self.state[p][k], self.state[p][k]._version) for _, _, p in tensors for k in keys]
                 self._fast = dict(key=self._plan_key, n_state=len(self.state), alive=alive,
                                   params=[p for _, _, p in tensors], versions=[p._version for _, _, p in tensors],
                                   gidx=np.asarray(grp, dtype=np.int64))
@@ -416,7 +428,15 @@ class VeLO_CUDA(Optimizer):
     def invalidate_statistics(self):
         """Call after writing parameters or ``mom`` / ``rms`` state tensors in a way the optimizer cannot see
         (through ``.data`` or a custom kernel): the next step then reads every tensor for the LSTM's input
-        statistics, as the reference does on every step, instead of using the sums the previous step left."""
+        statistics, as the reference does on every step, instead of using the sums the previous step left.
+
+        What the optimizer sees by itself: a parameter or state tensor object that was replaced, in-place torch
+        operations on a parameter or on ``mom`` / ``rms`` (their version counters), ``load_state_dict``.  What it
+        catches after the fact: a parameter written through ``.data`` or by a custom kernel.  The statistics
+        items of every step re-sum p^2 of every tensor (they read the parameter anyway) and compare it with the
+        carried sum; on a mismatch that step's update of the tensor is NaN and the next ``step()`` whose call
+        sees the flag raises ``RuntimeError`` (the flag is read without waiting for the GPU, so up to the steps
+        in flight later).  Not caught: writes to ``mom`` / ``rms`` through ``.data``."""
         self._fast = None
         if self._plan is not None:
             self._plan.invalidate_statistics()

@@ -64,6 +64,14 @@ extern "C" {
                                  modified (the reference scales p.grad in place).  On every tensor of the plan or
                                  on none; not with PYLO_F_GLOBAL_NORM or PYLO_F_NAN_TO_NUM; clip_val must be 0 */
 
+#define PYLO_F_NO_ORTHOGONALIZE 64 /* CELO2 kind: the tensor is never passed to
+                                 pylo_mi355_celo2_orthogonalize_finish with PYLO_ARG_ORTHOGONALIZE (its group does not
+                                 orthogonalise, or the caller does that itself): no Newton-Schulz workspace is
+                                 reserved for it.  That workspace is 18 bytes per element of every other 2-D
+                                 MLP tensor (three bf16 planes of X in both orientations, twice for the one the
+                                 update product writes), about 4.5 times the tensor's fp32 size, and makes up most
+                                 of what pylo_mi355_plan_workspace_bytes reports for an ELO-CELO2 plan */
+
 /* Storage type of the tensor's `grad` and `param` buffers (bits 8-9 of PyloTensorShape.flags).  The reference's
    kernels are instantiated for float, double and half (AT_DISPATCH_FLOATING_TYPES_AND_HALF,
    celo2_kernel.cu:314,328, velo_kernel.cu:405,427, learned_optimizer.cu:338,364): they widen every value to
@@ -220,13 +228,21 @@ int pylo_mi355_celo2_finish(PyloPlan* plan, const PyloTensorArgs* args, void* st
  * what pylo_mi355_celo2_finish does).  For every tensor with PYLO_ARG_ORTHOGONALIZE in `flags`, with
  * X = step_out / (||step_out||_F + ns_eps) and (c0, c1, c2) = ns_coeffs, `ns_iters` times
  *     A = X X^T (the Gram matrix over the smaller dim);  X <- c0 X + (c1 A + c2 A A) X
- * as fp32 matrix-pipe products that compute the symmetric A and c1 A + c2 A A once per pair of tiles; then
- * every tensor is normalised and applied as by pylo_mi355_celo2_finish (tensors without the flag from
- * `step_out` as it stands).  `step_out` of a flagged tensor is overwritten with intermediate results.
- * A tensor can carry the flag when pylo_mi355_plan_orthogonalize_supported says so: two dims, the last
- * and the smaller of the two multiples of 4; others (and tensors whose step is orthogonalised per slice of more leading dims) are
- * orthogonalised by the caller and passed without the flag.  The plan's workspace holds the second copy of
- * X and the two small matrices per tensor.
+ * as matrix-pipe products of the library's own that compute the symmetric A and c0 I + c1 A + c2 A A once per
+ * pair of tiles -- by default on the bf16 matrix instructions at fp32 accuracy (every fp32 operand is the exact
+ * sum of three bf16 numbers, six bf16 products per fp32 product, fp32 accumulation; what is dropped is below
+ * 2^-24 of a product), with PYLO_MI355_NS_F32=1 in the environment at plan creation on the fp32 matrix
+ * instructions; then every tensor is normalised and applied as by pylo_mi355_celo2_finish (tensors without the
+ * flag from `step_out` as it stands).  `step_out` of a flagged tensor is overwritten (with the orthogonalised
+ * step).  A tensor can carry the flag when pylo_mi355_plan_orthogonalize_supported says so: two dims (any two;
+ * the fp32 instructions: the last and the smaller dim multiples of 4) and no PYLO_F_NO_ORTHOGONALIZE in its
+ * shape flags; others (and tensors whose step is orthogonalised per slice of more leading dims) are
+ * orthogonalised by the caller and passed without the flag.  The plan's workspace holds the operand planes:
+ * 18 bytes per element of every such tensor (X as three bf16 planes in both orientations, the orientation
+ * that the update product writes twice) plus 16 bytes per element of its m x m matrices -- 2.2 GB for a
+ * GPT-2-small set, all tensors resident at once; pylo_mi355_plan_workspace_bytes reports the total.  The
+ * products of groups of tensors run on streams of the plan's own next to the caller's (forked and joined
+ * with events, default priority); the call returns with the caller's stream waiting for them.
  */
 int pylo_mi355_celo2_orthogonalize_finish(PyloPlan* plan, const PyloTensorArgs* args, const float* ns_coeffs,
                                           int ns_iters, float ns_eps, void* stream);

@@ -18,6 +18,7 @@ MAX_DIMS = 8
 KIND_CELO2, KIND_VELO, KIND_ADAFAC = 0, 1, 2
 F_ADAM = 1
 F_ADAM_INDEP = 2
+F_NO_ORTHOGONALIZE = 64   # CELO2: no Newton-Schulz workspace for this tensor
 F_NAN_TO_NUM, F_WD_PRESTEP, F_GLOBAL_NORM, F_TENSOR_NORM = 4, 8, 16, 32
 ARG_ORTHOGONALIZE = 1      # PyloTensorArgs.flags
 # storage type of a tensor's grad / param buffers (PYLO_F_STORE_*); accumulators and arithmetic stay fp32

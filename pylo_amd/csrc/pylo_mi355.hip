@@ -75,6 +75,8 @@ bool factored_dims(int kind, const PyloTensorShape& s, int* dc, int* dr) {
 
 // One group of matrices of the split-bf16 Newton-Schulz kernels: its ranges in the job tables.
 struct NsGroup { int gram0, n_gram, poly0, n_poly, upd0, n_upd, upd40, n_upd4, split0, n_split, split_max_m; };
+// One batch of matrices: those whose operand planes share the plane workspace at one time.
+struct NsBatch { int mat0, n_mats, split_item0, n_split_items, group0, n_groups; long long plane_elems; };
 
 struct Layout {
   std::vector<Item> mx_items;   // ELO-CELO2: statistics and apply items in slab order (k_celo2_elem)
@@ -85,6 +87,7 @@ struct Layout {
   std::vector<NsItem> ns_gram, ns_poly, ns_upd;
   std::vector<NsItem> ns_upd4;        // split-bf16 kernels: update jobs with 256-column tiles
   std::vector<NsGroup> ns_groups;     // split-bf16 kernels: ranges of the job tables, one per group of matrices
+  std::vector<NsBatch> ns_batches;    // split-bf16 kernels: batches of matrices that run one after another
   std::vector<int> ns_split;          // matrices whose Gram product is split (k_ns_gram_reduce)
   std::vector<long long> ns_xalt;     // per tensor: offset of its second X buffer, -1 without one
   std::vector<int> ns_of_tensor;      // per tensor: index into ns_mats, -1
@@ -229,6 +232,14 @@ int env_ns_groups() {
   return std::max(1, std::min(g, 4));
 }
 
+// PYLO_MI355_NS_WORKSPACE_MB: what the operand planes of the matrices that are orthogonalised at one time may take
+// (in bf16 elements here); read at plan creation.
+long long env_ns_budget_elems() {
+  const char* e = getenv("PYLO_MI355_NS_WORKSPACE_MB");
+  const long long mb = e ? atoll(e) : 8192;
+  return std::max(1ll, mb) * (1ll << 20) / 2;
+}
+
 bool env_ns_bf() {
   const char* e = getenv("PYLO_MI355_NS_F32");
   return !(e && e[0] == '1');
@@ -265,14 +276,14 @@ void xcd_interleave(std::vector<NsItem>& items, const std::vector<std::pair<int,
 
 // Newton-Schulz tables: every 2-D MLP tensor (the fp32 kernels: those whose rows (C) and whose smaller dim are
 // multiples of 4).  `ws_floats` returns the floats of workspace behind off_ns_ws.
-void build_ns_tables(Layout& L, int T, long long& ws_floats) {
+void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long& ws_floats) {
   ws_floats = 0;
   L.ns_xalt.assign(T, -1);
   L.ns_of_tensor.assign(T, -1);
   auto take = [&](long long n) { const long long o = ws_floats; ws_floats += (n + 63) / 64 * 64; return o; };
   for (int t = 0; t < T; ++t) {
     const TDesc& d = L.descs[t];
-    if (d.mode != kModeFac2D || d.n == 0) continue;
+    if (d.mode != kModeFac2D || d.n == 0 || (shapes[t].flags & PYLO_F_NO_ORTHOGONALIZE)) continue;
     // the fp32 kernels load 16 bytes at a time along the contiguous dim of X, A and B'
     if (!L.ns_bf && (d.C0 % 4 != 0 || std::min(d.R0, d.C0) % 4 != 0)) continue;
     NsMat mt{};
@@ -315,7 +326,16 @@ void build_ns_tables(Layout& L, int T, long long& ws_floats) {
     auto take_p = [&](long long n) { const long long o = pw; pw += (n + 63) / 64 * 64; return o; };
     auto up = [](int x, int q) { return (x + q - 1) / q * q; };
     auto up16 = [&](int x) { return up(x, kBfBK); };
-    // planes and fp32 matrices of every matrix
+    // Planes and fp32 matrices of every matrix.  The planes are only live during a matrix's own products, so
+    // the matrices are cut into batches (in tensor order) whose planes fit PYLO_MI355_NS_WORKSPACE_MB (8192 by
+    // default); the batches run one after another in the same memory.  A plan whose matrices fit in one batch
+    // has its planes' padding zeroed once, at plan creation; with several batches every batch starts by zeroing
+    // the region (one fill at HBM write speed: the padding of one batch's planes lies in another's data).
+    const long long budget = env_ns_budget_elems();
+    long long pw_max = 0, ws_max = 0;
+    std::vector<int> batch_of;
+    L.ns_batches.clear();
+    NsBatch batch{};
     for (size_t q = 0; q < L.ns_mats.size(); ++q) {
       const NsMat& f = L.ns_mats[q];
       NsBfMat b{};
@@ -328,6 +348,16 @@ void build_ns_tables(Layout& L, int T, long long& ws_floats) {
       b.rows_n = up(b.n, kNsTile);
       b.lda = up(b.m, 4);
       b.n_slabs = f.n_slabs;
+      const long long need = 3ll * b.rows_m * b.pad_n + 6ll * b.rows_n * b.pad_m + 6ll * b.rows_m * b.pad_m + 5 * 64;
+      if (pw > 0 && pw + need > budget) {   // this matrix opens the next batch
+        batch.plane_elems = pw;
+        L.ns_batches.push_back(batch);
+        batch = NsBatch{};
+        batch.mat0 = (int)q;
+        batch.split_item0 = (int)L.nsb_split_items.size();
+        pw = 0;
+        ws_floats = 0;
+      }
       b.off_xs = take_p(3ll * b.rows_m * b.pad_n);
       b.off_xl[0] = take_p(3ll * b.rows_n * b.pad_m);
       b.off_xl[1] = take_p(3ll * b.rows_n * b.pad_m);
@@ -340,17 +370,31 @@ void build_ns_tables(Layout& L, int T, long long& ws_floats) {
       for (int tr = 0; tr < (b.R + 63) / 64; ++tr)
         for (int tc = 0; tc < (b.C + 63) / 64; ++tc) L.nsb_split_items.push_back(NsTileItem{(int)q, tr, tc});
       L.nsb_mats.push_back(b);
+      batch_of.push_back((int)L.ns_batches.size());
+      batch.n_mats = (int)q + 1 - batch.mat0;
+      batch.n_split_items = (int)L.nsb_split_items.size() - batch.split_item0;
+      pw_max = std::max(pw_max, pw);
+      ws_max = std::max(ws_max, ws_floats);
     }
+    if (batch.n_mats > 0) {
+      batch.plane_elems = pw;
+      L.ns_batches.push_back(batch);
+    }
+    pw = pw_max;
+    ws_floats = ws_max;
     L.nsb_plane_elems = pw;
     std::fill(L.ns_xalt.begin(), L.ns_xalt.end(), -1);   // the result always replaces the raw step
     // Groups of matrices.  The products of one matrix depend on each other, those of different matrices do not:
     // each group runs its chain of launches on a stream of its own, so that the blocks of one group's launch
     // fill the CUs that the tail of the other's leaves idle.  Matrices are dealt to the groups heaviest first.
-    int n_groups = std::min<int>(env_ns_groups(), std::max<size_t>(L.nsb_mats.size() / 8, 1));
+    L.ns_groups.clear();
+    L.ns_split.clear();
+    for (NsBatch& bt : L.ns_batches) {
+    const int n_groups = std::min<int>(env_ns_groups(), std::max(bt.n_mats / 8, 1));
     std::vector<std::vector<int>> members(n_groups);
     {
-      std::vector<int> order(L.nsb_mats.size());
-      for (size_t q = 0; q < order.size(); ++q) order[q] = (int)q;
+      std::vector<int> order(bt.n_mats);
+      for (int q = 0; q < bt.n_mats; ++q) order[q] = bt.mat0 + q;
       auto work = [&](int q) { const NsBfMat& b = L.nsb_mats[q]; return (double)b.m * b.m * b.n; };
       std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return work(x) > work(y); });
       std::vector<double> load(n_groups, 0.0);
@@ -361,8 +405,8 @@ void build_ns_tables(Layout& L, int T, long long& ws_floats) {
       }
       for (auto& mm : members) std::sort(mm.begin(), mm.end());   // neighbours in memory stay neighbours in the tables
     }
-    L.ns_groups.clear();
-    L.ns_split.clear();
+    bt.group0 = (int)L.ns_groups.size();
+    bt.n_groups = n_groups;
     for (int g = 0; g < n_groups; ++g) {
       // job runs that read the same operands: per matrix (slab), and finer, per row of tiles, for sets of few matrices
       std::vector<std::pair<int, long long>> gram_units, poly_units, upd_units, upd4_units, gram_rows, poly_rows;
@@ -422,6 +466,7 @@ void build_ns_tables(Layout& L, int T, long long& ws_floats) {
       append(L.ns_upd4, upd4, grp.upd40, grp.n_upd4);
       grp.n_split = (int)L.ns_split.size() - grp.split0;
       L.ns_groups.push_back(grp);
+    }
     }
     return;
   }
@@ -697,7 +742,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   if (kind == PYLO_KIND_CELO2) {
     long long ns_floats = 0;
     L.ns_bf = env_ns_bf();
-    build_ns_tables(L, T, ns_floats);
+    build_ns_tables(L, shapes, T, ns_floats);
     L.off_ns_mats = take(sizeof(NsMat) * L.ns_mats.size());
     L.off_ns_gram = take(sizeof(NsItem) * L.ns_gram.size());
     L.off_ns_poly = take(sizeof(NsItem) * L.ns_poly.size());
@@ -835,7 +880,9 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
     if (e == hipSuccess) e = hipEventCreateWithFlags(&P->ev_fork, hipEventDisableTiming);
     if (e == hipSuccess) e = hipEventCreateWithFlags(&P->ev_join, hipEventDisableTiming);
   }
-  for (size_t g = 1; g < L.ns_groups.size() && e == hipSuccess; ++g) {
+  size_t ns_streams = 0;
+  for (const NsBatch& bt : L.ns_batches) ns_streams = std::max<size_t>(ns_streams, bt.n_groups);
+  for (size_t g = 1; g < ns_streams && e == hipSuccess; ++g) {
     if (g == 1) e = hipEventCreateWithFlags(&P->ns_fork, hipEventDisableTiming);
     if (e == hipSuccess) e = hipStreamCreateWithFlags(&P->ns_side[g - 1], hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreateWithFlags(&P->ns_join[g - 1], hipEventDisableTiming);
@@ -1250,6 +1297,10 @@ int ns_bf_lds_once() {
   return 0;
 }
 
+__global__ __launch_bounds__(256) void k_ns_zero(u32x4* __restrict__ p, size_t n16) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) p[i] = u32x4{0u, 0u, 0u, 0u};
+}
+
 // Newton-Schulz (ns_iters > 0, on the tensors flagged PYLO_ARG_ORTHOGONALIZE) and the finishing pass.
 int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, int ns_iters, float ns_eps, void* stream,
                 const char* who) {
@@ -1304,43 +1355,52 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
       const NsBfMat* bmats = P->at<NsBfMat>(L.off_nsb_mats);
       const NsTileItem* sitems = P->at<NsTileItem>(L.off_nsb_split_items);
       bfbits* pw = P->at<bfbits>(L.off_ns_pw);
-      hipLaunchKernelGGL(k_ns_bf_split, dim3((unsigned)L.nsb_split_items.size()), dim3(256), 0, s, bmats, sitems, dyn,
-                         (const float*)scale, pw);
       const NsItem* upd4 = P->at<NsItem>(L.off_ns_upd4);
       if (int rc = ns_bf_lds_once()) return rc;
-      // every group of matrices on a stream of its own, the first on the caller's
-      const int n_groups = (int)L.ns_groups.size();
-      if (n_groups > 1 && ns_iters > 0) {
-        HIP_TRY(hipEventRecord(P->ns_fork, s));
-        for (int g = 1; g < n_groups; ++g) HIP_TRY(hipStreamWaitEvent(P->ns_side[g - 1], P->ns_fork, 0));
-      }
-      for (int it = 0; it < ns_iters; ++it) {
-        const int par = it & 1, last = it == ns_iters - 1;
-        for (int g = 0; g < n_groups; ++g) {
-          const NsGroup& G = L.ns_groups[g];
-          hipStream_t sg = g == 0 ? s : P->ns_side[g - 1];
-          if (G.n_gram > 0)
-            hipLaunchKernelGGL((k_ns_bf_gemm<kNsGram, 2>), dim3(G.n_gram), dim3(256), bf_gemm_lds(2), sg, bmats, gram + G.gram0,
-                               dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
-          if (G.n_split > 0)
-            hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)G.split_max_m * G.split_max_m + 255) / 256, G.n_split),
-                               dim3(256), 0, sg, bmats, split + G.split0, dyn, ns_ws, pw);
-          if (G.n_poly > 0)
-            hipLaunchKernelGGL((k_ns_bf_gemm<kNsPoly, 2>), dim3(G.n_poly), dim3(256), bf_gemm_lds(2), sg, bmats, poly + G.poly0,
-                               dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
-          if (G.n_upd4 > 0)
-            hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 4>), dim3(G.n_upd4), dim3(256), bf_gemm_lds(4), sg, bmats,
-                               upd4 + G.upd40, dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
-          if (G.n_upd > 0)
-            hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 2>), dim3(G.n_upd), dim3(256), bf_gemm_lds(2), sg, bmats,
-                               upd + G.upd0, dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+      const bool several = L.ns_batches.size() > 1;
+      for (const NsBatch& bt : L.ns_batches) {
+        // the planes' padding: zero from plan creation on when one batch has the memory to itself
+        if (several) {
+          const size_t n16 = (size_t)bt.plane_elems * sizeof(bfbits) / 16;
+          hipLaunchKernelGGL(k_ns_zero, dim3((unsigned)std::min<size_t>((n16 + 255) / 256, 1u << 16)), dim3(256), 0, s,
+                             reinterpret_cast<u32x4*>(pw), n16);
         }
-      }
-      if (n_groups > 1 && ns_iters > 0)
-        for (int g = 1; g < n_groups; ++g) {
-          HIP_TRY(hipEventRecord(P->ns_join[g - 1], P->ns_side[g - 1]));
-          HIP_TRY(hipStreamWaitEvent(s, P->ns_join[g - 1], 0));
+        hipLaunchKernelGGL(k_ns_bf_split, dim3((unsigned)bt.n_split_items), dim3(256), 0, s, bmats, sitems + bt.split_item0,
+                           dyn, (const float*)scale, pw);
+        // every group of matrices on a stream of its own, the first on the caller's
+        const int n_groups = bt.n_groups;
+        if (n_groups > 1 && ns_iters > 0) {
+          HIP_TRY(hipEventRecord(P->ns_fork, s));
+          for (int g = 1; g < n_groups; ++g) HIP_TRY(hipStreamWaitEvent(P->ns_side[g - 1], P->ns_fork, 0));
         }
+        for (int it = 0; it < ns_iters; ++it) {
+          const int par = it & 1, last = it == ns_iters - 1;
+          for (int g = 0; g < n_groups; ++g) {
+            const NsGroup& G = L.ns_groups[bt.group0 + g];
+            hipStream_t sg = g == 0 ? s : P->ns_side[g - 1];
+            if (G.n_gram > 0)
+              hipLaunchKernelGGL((k_ns_bf_gemm<kNsGram, 2>), dim3(G.n_gram), dim3(256), bf_gemm_lds(2), sg, bmats,
+                                 gram + G.gram0, dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+            if (G.n_split > 0)
+              hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)G.split_max_m * G.split_max_m + 255) / 256, G.n_split),
+                                 dim3(256), 0, sg, bmats, split + G.split0, dyn, ns_ws, pw);
+            if (G.n_poly > 0)
+              hipLaunchKernelGGL((k_ns_bf_gemm<kNsPoly, 2>), dim3(G.n_poly), dim3(256), bf_gemm_lds(2), sg, bmats,
+                                 poly + G.poly0, dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+            if (G.n_upd4 > 0)
+              hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 4>), dim3(G.n_upd4), dim3(256), bf_gemm_lds(4), sg, bmats,
+                                 upd4 + G.upd40, dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+            if (G.n_upd > 0)
+              hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 2>), dim3(G.n_upd), dim3(256), bf_gemm_lds(2), sg, bmats,
+                                 upd + G.upd0, dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+          }
+        }
+        if (n_groups > 1 && ns_iters > 0)
+          for (int g = 1; g < n_groups; ++g) {
+            HIP_TRY(hipEventRecord(P->ns_join[g - 1], P->ns_side[g - 1]));
+            HIP_TRY(hipStreamWaitEvent(s, P->ns_join[g - 1], 0));
+          }
+      }
     } else
     for (int it = 0; it < ns_iters; ++it) {
       const int first = it == 0, par = it & 1;

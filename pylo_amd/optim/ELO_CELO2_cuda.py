@@ -228,7 +228,10 @@ class ELO_CELO2_CUDA(Optimizer):
         return out
 
     def _ensure_plan(self, tensors):
-        key = tuple((tuple(p.shape), adam, p.dtype) for _, p, adam in tensors)
+        # the plan reserves Newton-Schulz workspace (18 bytes per element) only for the tensors whose group
+        # orthogonalises through the library
+        no_ns = [not (group["orthogonalize"] and self._lib_ns and self.ns_iters > 0) for group, _p, _a in tensors]
+        key = tuple((tuple(p.shape), adam, p.dtype, skip) for (_, p, adam), skip in zip(tensors, no_ns))
         if key == self._plan_key:
             return
         for _, p, _a in tensors:
@@ -241,7 +244,8 @@ class ELO_CELO2_CUDA(Optimizer):
         shapes = [tuple(p.shape) for _, p, _a in tensors]
         # parameters and gradients may be float16 / bfloat16 / float64 (the reference's kernel dispatches on the
         # element type, celo2_kernel.cu:314,328); accumulators and raw steps stay float32 (ELO_CELO2_cuda.py:167-177)
-        flags = [(self._ADAM_FLAG if adam else 0) | _lib.store_flag(p, type(self).__name__) for _, p, adam in tensors]
+        flags = [(self._ADAM_FLAG if adam else 0) | _lib.store_flag(p, type(self).__name__) |
+                 (_lib.F_NO_ORTHOGONALIZE if skip else 0) for (_, p, adam), skip in zip(tensors, no_ns)]
         self._plan = _lib.Plan(_lib.KIND_CELO2, shapes, flags, self.device)
         self._plan_key = key
         # Raw steps of the MLP tensors: tensors of one parameter group and one shape share a
@@ -506,8 +510,9 @@ class ELO_CELO2_CUDA(Optimizer):
                 continue
             if p.dim() > 2:
                 return None
-            orth = bool(group["orthogonalize"]) and p.dim() == 2 and self.ns_iters > 0
-            if orth and not (self._lib_ns and self._ns_ok[i]):
+            orth = bool(group["orthogonalize"]) and p.dim() == 2
+            # (zero iterations still divide by the Frobenius norm, which the normaliser's epsilon sees: torch path)
+            if orth and not (self._lib_ns and self._ns_ok[i] and self.ns_iters > 0):
                 return None
             idx.append(i)
             flags.append(_lib.ARG_ORTHOGONALIZE if orth else 0)

@@ -100,6 +100,24 @@ def test_iteration_counts_and_result_buffer(iters, pipe, monkeypatch):
     _run([(256, 384), (384, 256), (132, 260)], steps=2, ns_iters=iters)
 
 
+def test_workspace_budget_and_unflagged_tensors(monkeypatch):
+    """The operand planes live only during a matrix's own products: under a small PYLO_MI355_NS_WORKSPACE_MB the
+    matrices run in batches that share the memory (same arithmetic, bit-identical parameters, smaller workspace);
+    a group that does not orthogonalise reserves none."""
+    shapes = [(300, 260), (132, 260), (260, 132), (8201, 128), (37, 131), (256, 384), (64,), (129, 129), (96, 1024)]
+    opt_all, _ = _run(shapes, steps=2, seed=3)
+    monkeypatch.setenv("PYLO_MI355_NS_WORKSPACE_MB", "4")
+    opt_few, _ = _run(shapes, steps=2, seed=3)
+    monkeypatch.delenv("PYLO_MI355_NS_WORKSPACE_MB")
+    assert opt_few._plan.workspace.numel() < 0.7 * opt_all._plan.workspace.numel()
+    for group_a, group_b in zip(opt_all.param_groups, opt_few.param_groups):
+        for a, b in zip(group_a["params"], group_b["params"]):
+            assert torch.equal(a, b)
+    opt_none, _ = _run(shapes, steps=1, seed=3, orthogonalize=False)
+    assert opt_none._plan.workspace.numel() < 0.3 * opt_all._plan.workspace.numel()
+    assert not any(opt_none._ns_ok)
+
+
 def test_groups_without_orthogonalisation_and_with_param_scale():
     from pylo_amd import ELO_CELO2_CUDA
     from pylo_amd.models import CELO2MLP

@@ -470,8 +470,14 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
 // ---- the same pass with the element MLP on the bf16 matrix instructions at fp32 accuracy ----------------
 // An fp32 number is the exact sum of three bf16 numbers (8 + 8 + 8 significand bits; taken by truncation:
 // h = x & 0xffff0000, m = (x - h) & 0xffff0000, l = x - h - m, every step exact), and a product of two such
-// sums is, up to 2^-23 of itself (2^-25 on average), the six products h h, h m, m h, m m, h l, l h, each exact
-// in fp32.  One
+// sums is the six products h h, h m, m h, m m, h l, l h, each exact in fp32, plus m l + l m + l l, which are
+// dropped.  With truncation |m| < 2^-7 |x| and |l| < 2^-14 |x|, and the three planes have the sign of x: what is
+// dropped is below 2^-20 of |x y| in the worst case (2^-22 on average over the mantissas) and one-signed, a bias
+// towards zero per product; in a dot product of the MLP's width it stays below the rounding of the fp32
+// accumulation, which is what the comparisons with the fp64 evaluation show (the steps of this kernel and of the
+// fp32-instruction one sit at the same distance from it).  The split by rounding that the Newton-Schulz planes
+// use (|m| <= 2^-8, |l| <= 2^-16, signs mixed: 2^-23, unbiased) costs 7 vector instructions a value against
+// 5.5 here, in a kernel that is bound by exactly these instructions.  One
 // v_mfma_f32_32x32x16_bf16 does sixteen times the multiply-adds of v_mfma_f32_16x16x4_f32 in the same 32
 // cycles, so six of them per fp32 product leave 36 matrix instructions per row of 64 elements where the
 // fp32 instructions need 96; the price is vector work (bf16 matrix instructions run under vector instructions of

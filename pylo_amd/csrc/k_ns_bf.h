@@ -16,6 +16,19 @@
 //                                         or as fp32 in the tensor's own layout after the last iteration
 // for wide and tall matrices alike (B' is symmetric, so (B' X)^T = X^T B').
 //
+// Two iterations can share the two products over the long dim.  Every B'_t is a polynomial in A_t, so it
+// commutes with A_t and is symmetric, and A_{t+1} = X_{t+1} X_{t+1}^T = B'_t A_t B'_t needs no X:
+//     A_t (Gram), B'_t = p(A_t) (Poly), T = A_t B'_t (Prod), A_{t+1} = B'_t T (ProdA), B'_{t+1} = p(A_{t+1}) (Poly),
+//     Q = B'_{t+1} B'_t (Prod), X_{t+2} = Q X_t (Update)
+// i.e. four products of m^3 / 2 multiply-adds in place of one Gram product (m^2 n / 2) and one update (m^2 n).
+// What it costs in accuracy is bounded whatever the spectrum of X: A_t as computed is off by eps ||A_t|| in
+// absolute terms, which A_{t+1} = B'_t A_t B'_t inherits relative to its small eigenvalues -- they grow by
+// p(0)^2 = c0^2 in the step, so the error of p(A_{t+1}) in those directions is c1 c0^2 eps sigma_max^2, about
+// 12 times that of p of a freshly formed Gram matrix and about 1e-6 of B' itself; a second chained step would
+// multiply it by c0^2 again, which is why only pairs are merged and the next pair starts from a Gram product
+// of the X it was handed.  PYLO_MI355_NS_PAIRS=0 in the environment keeps one Gram product and one update
+// per iteration.
+//
 // Tile job: 128 x 128 (Gram, Poly, narrow updates) or 128 x 256 outputs (updates with m > 128) by 256 threads =
 // 2 x 2 waves of 64 x 64 / 64 x 128 = 2 x 2 / 2 x 4 accumulators of 32 x 32; 16 reduction steps per stage,
 // double buffered in LDS (48 / 72 KB), staged from global memory straight into LDS (global_load_lds_dwordx4: no
@@ -61,11 +74,17 @@ struct NsBfMat {
   int n_slabs;
   long long off_xs;          // elements (bfbits) into the plane workspace: planes of Xs (m rows, reduction n)
   long long off_xl[2];       // planes of Xl (n rows, reduction m), two buffers (a product reads one and writes the other)
-  long long off_pa, off_pb;  // planes of A and B' (m rows, reduction m)
+  long long off_p, p_stride; // planes of the m x m matrices (m rows, reduction m): buffer b at off_p + b p_stride
   long long off_a;           // floats into the fp32 workspace: A (m x m)
   long long off_part;        // floats: partial matrices of a split Gram product
   long long elem_off;        // elements from the tensor's raw step to this matrix (a slice of a tensor with more dims)
 };
+
+// the m x m plane buffers, and the two products on planes in and planes out (k_ns_bf_gemm's OP, after
+// kNsGram / kNsPoly / kNsUpdate)
+enum : int { kNsBufA = 0, kNsBufB = 1, kNsBufT = 2, kNsBufC = 3, kNsBufs = 4 };
+enum : int { kNsProd = 3, kNsProdA = 4 };
+struct NsBufs { int s1, s2, d; };   // operand and result buffers of an m x m product; the update's B' is s1
 
 __device__ __forceinline__ float bf_to_float(bfbits b) { return __uint_as_float((unsigned)b << 16); }
 
@@ -252,16 +271,18 @@ __device__ __forceinline__ void bf_store_planes(PYLO_LDS char* lds, const v16f (
 
 // One launch = one product of one iteration, for every tensor (see the head of this file).
 //   kNsGram    A = Xs Xs^T as fp32 and planes, both halves; a slab of a split product: fp32 partial tile only
-//   kNsPoly    B' = c2 A A + c1 A + c0 I as planes, both halves
-//   kNsUpdate  Xl' = Xl B': planes of Xl' (buffer 1 - par) and Xs', or fp32 X in place of the raw step (`last`)
+//   kNsPoly    c2 A A + c1 A + c0 I as planes (buffer bufs.d), both halves; A: buffer kNsBufA and its fp32 copy
+//   kNsProd    (buffer s1) (buffer s2) as planes (buffer d), both halves
+//   kNsProdA   the same, into buffer d and into the fp32 copy of A
+//   kNsUpdate  Xl' = Xl (buffer s1): planes of Xl' (buffer 1 - par) and Xs', or fp32 X in place of the raw step (`last`)
 // WN: the tile has 64 WN columns (Gram and Poly: 2; updates: 2 or 4, a table of jobs each).
 // Registers: 64 / 128 accumulator registers plus what the epilogues need; tiles of 256 columns are held to two
 // waves per SIMD (256 registers: left alone the epilogue takes 296 and a CU runs one job at a time).
 template <int OP, int WN>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2 : 3))) void k_ns_bf_gemm(const NsBfMat* __restrict__ mats, const NsItem* __restrict__ items,
                                                     const PyloTensorArgs* __restrict__ dyn, float* __restrict__ ws,
-                                                    bfbits* __restrict__ pw, int par, int last, float c0, float c1,
-                                                    float c2) {
+                                                    bfbits* __restrict__ pw, int par, int last, NsBufs bufs, float c0,
+                                                    float c1, float c2) {
   extern __shared__ __attribute__((aligned(16))) char lds_[];
   PYLO_LDS char* lds = (PYLO_LDS char*)lds_;
   const NsItem it = items[blockIdx.x];
@@ -282,12 +303,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
     const BfPlanes X{pw + mt.off_xs, mt.rows_m};
     bf_tile_product<WN>(X, i0, X, j0, it.k0, it.k1, lds, acc);
   } else if (OP == kNsPoly) {
-    const BfPlanes A{pw + mt.off_pa, mt.rows_m};
+    const BfPlanes A{pw + mt.off_p, mt.rows_m};
     bf_tile_product<WN>(A, i0, A, j0, it.k0, it.k1, lds, acc);
-  } else {
+  } else if (OP == kNsUpdate) {
     const BfPlanes X{pw + (par ? mt.off_xl[1] : mt.off_xl[0]), mt.rows_n};   // no run-time index: the struct stays in registers
-    const BfPlanes B{pw + mt.off_pb, mt.rows_m};
+    const BfPlanes B{pw + mt.off_p + bufs.s1 * mt.p_stride, mt.rows_m};
     bf_tile_product<WN>(X, i0, B, j0, it.k0, it.k1, lds, acc);
+  } else {
+    const BfPlanes P1{pw + mt.off_p + bufs.s1 * mt.p_stride, mt.rows_m};
+    const BfPlanes P2{pw + mt.off_p + bufs.s2 * mt.p_stride, mt.rows_m};
+    bf_tile_product<WN>(P1, i0, P2, j0, it.k0, it.k1, lds, acc);
   }
   float* A32 = ws + mt.off_a;
   const int n_i = OP == kNsUpdate ? n : m;   // rows of the output; its columns are always m
@@ -297,7 +322,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
   float* xout = a.step_out + mt.elem_off;
   const bool vec_out = (mt.C & 3) == 0;   // rows of the tensor are 16-byte aligned
   // fp32 outputs (and Poly's transform of the accumulators) straight from the registers
-  if (OP != kNsUpdate || last) {
+  if (OP == kNsGram || OP == kNsPoly || OP == kNsProdA || (OP == kNsUpdate && last)) {
 #pragma unroll
     for (int hi = 0; hi < 2; ++hi)
 #pragma unroll
@@ -319,7 +344,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
             }
             v[r] = x;
           }
-          if (OP == kNsGram) {
+          if (OP == kNsGram || OP == kNsProdA) {
             float* out = partial ? ws + mt.off_part + (size_t)it.slab * m * lda : A32;
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -347,7 +372,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
   if (OP == kNsUpdate) {
     bf_store_planes<WN>(lds, acc, pw + (par ? mt.off_xl[0] : mt.off_xl[1]), mt.rows_n, i0, j0, n, m, pw + mt.off_xs, mt.rows_m);
   } else {
-    bfbits* D = pw + (OP == kNsGram ? mt.off_pa : mt.off_pb);
+    bfbits* D = pw + mt.off_p + (OP == kNsGram ? (int)kNsBufA : bufs.d) * mt.p_stride;
     bf_store_planes<WN>(lds, acc, D, mt.rows_m, i0, j0, m, m, mirror ? D : nullptr, mt.rows_m);
   }
 }
@@ -375,7 +400,7 @@ __global__ __launch_bounds__(256) void k_ns_bf_gram_reduce(const NsBfMat* __rest
     for (int q = 0; q < 8; ++q) s += v[q];
   }
   float* A = ws + mt.off_a;
-  bfbits* P = pw + mt.off_pa;
+  bfbits* P = pw + mt.off_p;   // buffer A
   A[(size_t)i * lda + j] = s;
   bf_store1(P, mt.rows_m, i, j, s);
   if (i / kNsTile != j / kNsTile) {

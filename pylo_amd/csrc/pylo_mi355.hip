@@ -240,6 +240,13 @@ long long env_ns_budget_elems() {
   return std::max(1ll, mb) * (1ll << 20) / 2;
 }
 
+// PYLO_MI355_NS_PAIRS=0: one Gram product and one update per Newton-Schulz iteration, as the formula is written,
+// instead of one of each per pair of iterations (k_ns_bf.h); read when the products are enqueued.
+bool env_ns_pairs() {
+  const char* e = getenv("PYLO_MI355_NS_PAIRS");
+  return !(e && e[0] == '0');
+}
+
 bool env_ns_bf() {
   const char* e = getenv("PYLO_MI355_NS_F32");
   return !(e && e[0] == '1');
@@ -348,7 +355,8 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       b.rows_n = up(b.n, kNsTile);
       b.lda = up(b.m, 4);
       b.n_slabs = f.n_slabs;
-      const long long need = 3ll * b.rows_m * b.pad_n + 6ll * b.rows_n * b.pad_m + 6ll * b.rows_m * b.pad_m + 5 * 64;
+      b.p_stride = (3ll * b.rows_m * b.pad_m + 63) / 64 * 64;
+      const long long need = 3ll * b.rows_m * b.pad_n + 6ll * b.rows_n * b.pad_m + kNsBufs * b.p_stride + 4 * 64;
       if (pw > 0 && pw + need > budget) {   // this matrix opens the next batch
         batch.plane_elems = pw;
         L.ns_batches.push_back(batch);
@@ -361,8 +369,7 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       b.off_xs = take_p(3ll * b.rows_m * b.pad_n);
       b.off_xl[0] = take_p(3ll * b.rows_n * b.pad_m);
       b.off_xl[1] = take_p(3ll * b.rows_n * b.pad_m);
-      b.off_pa = take_p(3ll * b.rows_m * b.pad_m);
-      b.off_pb = take_p(3ll * b.rows_m * b.pad_m);
+      b.off_p = take_p(kNsBufs * b.p_stride);
       b.off_a = take((long long)b.m * b.lda);
       b.off_part = b.n_slabs > 1 ? take((long long)b.n_slabs * b.m * b.lda) : 0;
       b.elem_off = 0;
@@ -1291,6 +1298,8 @@ int ns_bf_lds_once() {
     if (d == dev) return 0;
   HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsGram, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(2)));
   HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsPoly, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(2)));
+  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsProd, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(2)));
+  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsProdA, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(2)));
   HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsUpdate, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(2)));
   HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsUpdate, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(4)));
   done.push_back(dev);
@@ -1373,27 +1382,45 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
           HIP_TRY(hipEventRecord(P->ns_fork, s));
           for (int g = 1; g < n_groups; ++g) HIP_TRY(hipStreamWaitEvent(P->ns_side[g - 1], P->ns_fork, 0));
         }
-        for (int it = 0; it < ns_iters; ++it) {
-          const int par = it & 1, last = it == ns_iters - 1;
+        const float c0 = coeffs[0], c1 = coeffs[1], c2 = coeffs[2];
+        const bool pairs = env_ns_pairs();
+        int par = 0;   // which Xl buffer the next update reads
+        for (int it = 0; it < ns_iters;) {
+          // two iterations as one Gram product, four m x m products and one update (k_ns_bf.h), or one iteration
+          const bool pair = pairs && it + 1 < ns_iters;
+          const int last = (it + (pair ? 2 : 1)) == ns_iters;
           for (int g = 0; g < n_groups; ++g) {
             const NsGroup& G = L.ns_groups[bt.group0 + g];
             hipStream_t sg = g == 0 ? s : P->ns_side[g - 1];
+            auto small = [&](auto kern, NsBufs b) {
+              if (G.n_poly > 0)
+                hipLaunchKernelGGL(kern, dim3(G.n_poly), dim3(256), bf_gemm_lds(2), sg, bmats, poly + G.poly0, dyn, ns_ws, pw,
+                                   par, last, b, c0, c1, c2);
+            };
             if (G.n_gram > 0)
               hipLaunchKernelGGL((k_ns_bf_gemm<kNsGram, 2>), dim3(G.n_gram), dim3(256), bf_gemm_lds(2), sg, bmats,
-                                 gram + G.gram0, dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+                                 gram + G.gram0, dyn, ns_ws, pw, par, last, NsBufs{0, 0, kNsBufA}, c0, c1, c2);
             if (G.n_split > 0)
               hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)G.split_max_m * G.split_max_m + 255) / 256, G.n_split),
                                  dim3(256), 0, sg, bmats, split + G.split0, dyn, ns_ws, pw);
-            if (G.n_poly > 0)
-              hipLaunchKernelGGL((k_ns_bf_gemm<kNsPoly, 2>), dim3(G.n_poly), dim3(256), bf_gemm_lds(2), sg, bmats,
-                                 poly + G.poly0, dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+            small(k_ns_bf_gemm<kNsPoly, 2>, NsBufs{kNsBufA, kNsBufA, kNsBufB});            // B'_t
+            int bq = kNsBufB;
+            if (pair) {
+              small(k_ns_bf_gemm<kNsProd, 2>, NsBufs{kNsBufA, kNsBufB, kNsBufT});          // T = A_t B'_t
+              small(k_ns_bf_gemm<kNsProdA, 2>, NsBufs{kNsBufB, kNsBufT, kNsBufA});         // A_{t+1} = B'_t T
+              small(k_ns_bf_gemm<kNsPoly, 2>, NsBufs{kNsBufA, kNsBufA, kNsBufC});          // B'_{t+1}
+              small(k_ns_bf_gemm<kNsProd, 2>, NsBufs{kNsBufC, kNsBufB, kNsBufT});          // Q = B'_{t+1} B'_t
+              bq = kNsBufT;
+            }
             if (G.n_upd4 > 0)
               hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 4>), dim3(G.n_upd4), dim3(256), bf_gemm_lds(4), sg, bmats,
-                                 upd4 + G.upd40, dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+                                 upd4 + G.upd40, dyn, ns_ws, pw, par, last, NsBufs{bq, 0, 0}, c0, c1, c2);
             if (G.n_upd > 0)
               hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 2>), dim3(G.n_upd), dim3(256), bf_gemm_lds(2), sg, bmats,
-                                 upd + G.upd0, dyn, ns_ws, pw, par, last, coeffs[0], coeffs[1], coeffs[2]);
+                                 upd + G.upd0, dyn, ns_ws, pw, par, last, NsBufs{bq, 0, 0}, c0, c1, c2);
           }
+          par ^= 1;
+          it += pair ? 2 : 1;
         }
         if (n_groups > 1 && ns_iters > 0)
           for (int g = 1; g < n_groups; ++g) {

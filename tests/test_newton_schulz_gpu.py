@@ -80,12 +80,16 @@ def test_library_kernels_take_these_shapes(pipe, monkeypatch):
     [(37, 4099), (4099, 37), (255, 257), (129, 129), (1, 300), (300, 1), (2, 3)],   # odd dims, single rows and columns
     [(300, 260), (300, 260), (300, 260), (64,)],                         # a bucket of equal shapes
 ])
-@pytest.mark.parametrize("pipe", ["bf16x3", "fp32"])
+@pytest.mark.parametrize("pipe", ["bf16x3", "bf16x3-literal", "fp32"])
 def test_library_newton_schulz_matches_oracle(shapes, pipe, monkeypatch):
-    """Both sets of product kernels: the default (operands split into three bf16 planes, six bf16 matrix
-    products per fp32 product) and the fp32 matrix instructions (PYLO_MI355_NS_F32=1, read at plan creation)."""
+    """The sets of product kernels: the default (operands split into three bf16 planes, six bf16 matrix products
+    per fp32 product, two iterations sharing one Gram product and one update), the same with one Gram product and
+    one update per iteration (PYLO_MI355_NS_PAIRS=0), and the fp32 matrix instructions (PYLO_MI355_NS_F32=1, read
+    at plan creation)."""
     if pipe == "fp32":
         monkeypatch.setenv("PYLO_MI355_NS_F32", "1")
+    if pipe == "bf16x3-literal":
+        monkeypatch.setenv("PYLO_MI355_NS_PAIRS", "0")
     _, worst = _run(shapes, steps=2, seed=len(shapes))
     print("orthogonalised step err / rms", worst)
 
@@ -98,6 +102,80 @@ def test_iteration_counts_and_result_buffer(iters, pipe, monkeypatch):
     if pipe == "fp32":
         monkeypatch.setenv("PYLO_MI355_NS_F32", "1")
     _run([(256, 384), (384, 256), (132, 260)], steps=2, ns_iters=iters)
+
+
+def _orthogonalise_direct(mats, iters=5):
+    """rms_normalize(newton_schulz(x)) of every matrix through the finishing call alone: p = 0, lr = -1."""
+    import numpy as np
+
+    from pylo_amd import _lib
+
+    shapes = [tuple(x.shape) for x in mats]
+    plan = _lib.Plan(_lib.KIND_CELO2, shapes, [0] * len(shapes), torch.device("cuda:0"))
+    steps = [x.clone().contiguous() for x in mats]
+    params = [torch.zeros_like(x) for x in mats]
+    fin = np.zeros(len(mats), dtype=_lib.ARGS_DTYPE)
+    for i in range(len(mats)):
+        fin["grad"][i], fin["param"][i], fin["step_out"][i] = 1, params[i].data_ptr(), steps[i].data_ptr()
+        fin["lr"][i], fin["weight_decay"][i], fin["step_mult"][i] = -1.0, 0.0, 1.0
+        fin["flags"][i] = _lib.ARG_ORTHOGONALIZE
+    plan.celo2_orthogonalize_finish(fin, (3.4445, -4.775, 2.0315), iters, 1e-8, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    plan.close()
+    return params
+
+
+def _reference_direct(x, iters=5, dtype=torch.float64):
+    """The literal formula (pylo/optim/CELO2_naive.py:59-73) and the RMS normaliser, in fp64 or, as the reference
+    runs it, in fp32 torch products."""
+    c0, c1, c2 = 3.4445, -4.775, 2.0315
+    x = x.to(dtype)
+    t = x.shape[0] > x.shape[1]
+    if t:
+        x = x.T
+    x = x / (x.norm() + 1e-8)
+    for _ in range(iters):
+        a = x @ x.T
+        x = c0 * x + (c1 * a + c2 * (a @ a)) @ x
+    if t:
+        x = x.T
+    return x * torch.rsqrt(1e-9 + (x * x).mean())
+
+
+@pytest.mark.parametrize("pairs", ["1", "0"])
+def test_spectra_with_a_dominant_direction(pairs, monkeypatch):
+    """Matrices whose singular values span several decades (one dominant direction over a flat or a decaying
+    rest): where a Gram matrix loses its small eigenvalues to rounding and five iterations amplify what the first
+    ones round off.  On such input the formula in fp32 torch products -- what the reference runs -- is itself
+    1e-4 .. 5e-3 of the result's RMS away from its fp64 evaluation; the library's kernels, with two iterations
+    sharing one Gram product (the default) or with one Gram product per iteration, must be no further away than
+    1.5 times that (plus 5e-5, the level of well-conditioned inputs)."""
+    monkeypatch.setenv("PYLO_MI355_NS_PAIRS", pairs)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    rnd = lambda *s: torch.randn(*s, generator=gen, device="cuda")
+    mats = []
+    for (r, c), rest in (((256, 384), 5e-3), ((384, 256), 5e-3), ((768, 768), 1e-3), ((130, 1000), 1e-4),
+                         ((256, 2048), 3e-2), ((256, 384), 1.0), ((768, 3072), 1.0)):
+        u, v = rnd(r, 1), rnd(1, c)
+        mats.append(u @ v / (u.norm() * v.norm()) + rest * rnd(r, c) / (r * c) ** 0.5)
+    q1, _ = torch.linalg.qr(rnd(256, 256))
+    q2, _ = torch.linalg.qr(rnd(512, 256))
+    mats.append((q1 * torch.logspace(0, -4, 256, device="cuda")) @ q2.T)     # singular values 1 .. 1e-4
+    mats.append(rnd(768, 768))
+    got = _orthogonalise_direct(mats)
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    rows = []
+    try:
+        for x, y in zip(mats, got):
+            want = _reference_direct(x)
+            e = float((y.double() - want).abs().max())       # the result has unit RMS
+            e32 = float((_reference_direct(x, dtype=torch.float32).double() - want).abs().max())
+            rows.append((tuple(x.shape), e, e32))
+            assert e <= 1.5 * e32 + 5e-5, rows[-1]
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+    print("pairs", pairs, "(shape, library error / rms, fp32 torch formula error / rms):", rows)
 
 
 def test_workspace_budget_and_unflagged_tensors(monkeypatch):

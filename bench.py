@@ -145,15 +145,19 @@ def ns_flops(shapes, iters=5):
 
 
 def ns_flops_executed(shapes, iters=5, tile=128):
-    """What the library's kernels execute of ns_flops(): the two symmetric products only on the output tiles
-    on and above the diagonal (tile x tile outputs, whole tiles)."""
+    """FLOPs (fp32 multiply-adds x 2) that the library's kernels execute: symmetric m x m results on the tiles on
+    and above the diagonal only, and, unless PYLO_MI355_NS_PAIRS=0 (or the fp32 kernels are selected), two
+    iterations sharing one Gram product and one update: per pair one Gram product, five m x m products
+    (2 x Poly, 2 x Prod, ProdA) and one update; an unpaired iteration one Gram product, Poly and one update."""
+    pairs = os.environ.get("PYLO_MI355_NS_PAIRS", "1") != "0" and os.environ.get("PYLO_MI355_NS_F32") != "1"
+    n_pairs, singles = (iters // 2, iters % 2) if pairs else (0, iters)
     total = 0.0
     for s in shapes:
         if len(s) == 2:
             m, n = min(s), max(s)
             nt = -(-m // tile)
             upper = nt * (nt + 1) / 2 * tile * tile
-            total += iters * (2.0 * upper * n + 2.0 * upper * m + 2.0 * m * m * n)
+            total += (n_pairs + singles) * (2.0 * upper * n + 2.0 * m * m * n) + (5 * n_pairs + singles) * 2.0 * upper * m
     return total
 
 
@@ -329,6 +333,10 @@ def main():
             "launch_ms": {nm: float(v) for nm, v in zip(names, mean)},
         },
         "hbm_roofline_frac_fused_path": bytes_fused / (fused_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        # which part of ms_per_step each roofline speaks for: `roofline` below (HBM) is the fused call's dominant
+        # kernel, `whole_step.roofline` (matrix pipe) is Newton-Schulz and the finishing pass
+        "share_of_step": {"fused_pass (hbm roofline)": fused_in_step_ms / whole_ms,
+                          "newton_schulz + finishing pass (mfma roofline, whole_step.roofline)": finish_ms / whole_ms},
         # Newton-Schulz + normalise + apply
         "whole_step": whole_step_object(whole_ms, finish_ms, n_params, flops, flops_exec),
         "roofline": {"bound": "hbm", "kernel": elem, "achieved": elem_gbs, "peak": HBM_PEAK_GBS,
@@ -598,6 +606,10 @@ def other_workload(workload, steps, warmup):
         "hbm_algorithmic_GB_per_step": bytes_fused / 1e9,
         "hbm_GBps_fused_path": bytes_fused / (fused_ms * 1e-3) / 1e9,
         "hbm_roofline_frac_fused_path": bytes_fused / (fused_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        # which part of ms_per_step each roofline speaks for: `roofline` below (HBM) is the fused call's dominant
+        # kernel, `whole_step.roofline` (matrix pipe) is Newton-Schulz and the finishing pass
+        "share_of_step": {"fused_pass (hbm roofline)": fused_in_step_ms / whole_ms,
+                          "newton_schulz + finishing pass (mfma roofline, whole_step.roofline)": finish_ms / whole_ms},
         "sum_of_launch_intervals_ms": float(per.sum(axis=1).mean()),
         "launch_ms": {nm: float(v) for nm, v in zip(names, mean)},
         "roofline": roof,

@@ -606,10 +606,7 @@ def other_workload(workload, steps, warmup):
         "hbm_algorithmic_GB_per_step": bytes_fused / 1e9,
         "hbm_GBps_fused_path": bytes_fused / (fused_ms * 1e-3) / 1e9,
         "hbm_roofline_frac_fused_path": bytes_fused / (fused_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        # which part of ms_per_step each roofline speaks for: `roofline` below (HBM) is the fused call's dominant
-        # kernel, `whole_step.roofline` (matrix pipe) is Newton-Schulz and the finishing pass
-        "share_of_step": {"fused_pass (hbm roofline)": fused_in_step_ms / whole_ms,
-                          "newton_schulz + finishing pass (mfma roofline, whole_step.roofline)": finish_ms / whole_ms},
+
         "sum_of_launch_intervals_ms": float(per.sum(axis=1).mean()),
         "launch_ms": {nm: float(v) for nm, v in zip(names, mean)},
         "roofline": roof,

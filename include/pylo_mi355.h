@@ -313,8 +313,9 @@ int pylo_mi355_plan_invalidate_statistics(PyloPlan* plan);
    step and the plan was not told -- the LSTM of that step has already run on the stale sum: the tensor's
    step of that call is NaN (loud, like the fused pass's bounded wait) and the plan's flag is raised.  This
    call returns 0, or 1 + the index of a tensor the guard caught since the last
-   pylo_mi355_plan_invalidate_statistics; it reads a pinned copy that every step refreshes at its end and does
-   not wait for the GPU, so it may lag the step that raised the flag by the steps still in flight.  Writes
+   pylo_mi355_plan_invalidate_statistics; it reads pinned host memory that the kernel writes when it catches a
+   mismatch and does not wait for the GPU, so it may lag the step that raised the flag by the steps still in
+   flight.  Writes
    that leave sum p^2 within 1e-3 also leave the LSTM's input feature within that, and are not flagged; the
    sums over `mom` and `rms` are not guarded (the Python class watches those tensors' identity and version
    counters).  No counterpart in the reference, which recomputes everything every step. */

@@ -566,6 +566,15 @@ __global__ __launch_bounds__(kFoldThreads) void k_lo_reduce(const TDesc* __restr
   velo_row_features(d, a, t, T, tot, nullptr, piv_out, ls, st, xfeat, H, w2t, b2, wft, bf, mixbuf, xs);
 }
 
+// Behind the 2 T counters and flags of `sync` (rounded up to 16 bytes) the workspace holds the guard of the carried
+// sums: the address of the plan's flag in pinned host memory, then per tensor the sum of p^2 that the LSTM of the
+// current step was fed.
+__device__ __forceinline__ long long* velo_guard_base(int* sync, int T) {
+  return reinterpret_cast<long long*>(sync + ((2 * T + 3) & ~3));
+}
+__device__ __forceinline__ int* velo_guard_flag(int* sync, int T) { return reinterpret_cast<int*>(velo_guard_base(sync, T)[0]); }
+__device__ __forceinline__ double* velo_guard_sums(int* sync, int T) { return reinterpret_cast<double*>(velo_guard_base(sync, T) + 2); }
+
 // The same from the sums the previous step's apply pass left (rows of kNewSumW doubles per element
 // block, shifted by the tensor's first elements as that pass wrote them, i.e. as they stand now): the
 // LSTM does not wait for this step's statistics pass.
@@ -576,8 +585,7 @@ __global__ __launch_bounds__(kFoldThreads) void k_velo_feat(const TDesc* __restr
                                                             float* __restrict__ xfeat, int H,
                                                             const float* __restrict__ w2t, const float* __restrict__ b2,
                                                             const float* __restrict__ wft, const float* __restrict__ bf,
-                                                            float* __restrict__ mixbuf, int* __restrict__ sync,
-                                                            double* __restrict__ carried_p2) {
+                                                            float* __restrict__ mixbuf, int* __restrict__ sync) {
   constexpr int G = kFoldThreads / kNewSumW;
   __shared__ double part[G][kNewSumW];
   __shared__ double tot[kStatW];
@@ -610,7 +618,7 @@ __global__ __launch_bounds__(kFoldThreads) void k_velo_feat(const TDesc* __restr
     for (int g2 = 0; g2 < G; ++g2) s += part[g2][threadIdx.x];
     const int q = threadIdx.x;   // 0: sum p^2 | 1..3: m | 4..6: m^2 | 7: rms | 8: rms^2
     tot[q == 0 ? 2 : q < 4 ? kSumM + q - 1 : q < 7 ? kSumMM + q - 4 : q == 7 ? kSumR : kSumRR] = s;
-    if (q == 0) carried_p2[t] = s;   // the statistics items of this step hold it against the sum they take themselves
+    if (q == 0) velo_guard_sums(sync, T)[t] = s;   // the statistics items of this step hold it against the sum they take themselves
   }
   __syncthreads();
   velo_row_features(d, a, t, T, tot, nullptr, piv, ls, st, xfeat, H, w2t, b2, wft, bf, mixbuf, xs);
@@ -1194,8 +1202,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                                                         const float* __restrict__ wmix, float* __restrict__ wfold,
                                                         double* __restrict__ stats_part, const float* __restrict__ piv,
                                                         double* __restrict__ newsum_part, int* __restrict__ sync,
-                                                        int n_tensors, const double* __restrict__ carried_p2,
-                                                        int* __restrict__ stale, int stale_gen) {
+                                                        int n_tensors) {
   __shared__ float red[kWaves][38];
   __shared__ double part[kThreads / 30][30];
   __shared__ float sc[30];
@@ -1249,8 +1256,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
   __syncthreads();
   if (!s_flag) return;
   // the tensor's last statistics block: channel sums in row order, then the folded block
-  __shared__ int poison_s;
-  if (threadIdx.x == 0) poison_s = 0;
   constexpr int G = kThreads / 30;
   const int c = threadIdx.x % 30, gI = threadIdx.x / 30;
   if (gI < G) {
@@ -1276,24 +1281,24 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     const double n = (double)(d.n > 0 ? d.n : 1);
     sc[threadIdx.x] = rsq(1e-5f + (float)(s / n));
     if (threadIdx.x == 2) {   // channel 2 is the parameter
-      pscale_s = sqrtf((float)(s / n) + 1e-9f);
       // The LSTM of this step was fed the sum of p^2 that the previous step's apply items carried over; `s` is
       // the same sum over the parameter as it stands now.  They differ (beyond the rounding of two summation
       // orders) only if somebody else wrote the parameter in between without the plan being told: the
-      // tensor's step is poisoned and the plan's flag raised rather than a step taken on stale statistics.
-      const double carried = carried_p2[it.tensor], big = fmax(fabs(s), fabs(carried));
-      if (!(fabs(s - carried) <= 1e-3 * big)) {
-        poison_s = 1;
-        __hip_atomic_store(stale + 1, it.tensor, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(stale, stale_gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
+      // tensor's step is poisoned (a NaN param_scale multiplies it) and the plan's flag raised rather than a
+      // step taken on stale statistics.  The flag is pinned host memory (a system-scope store of 1 + tensor).
+      // Both addresses are found behind the counters of `sync` rather than passed as arguments: the kernel's
+      // scalar registers are spilled as it is, and three more live arguments cost its hot loops 7 %.
+      const double carried = velo_guard_sums(sync, n_tensors)[it.tensor];
+      const bool ok = fabs(s - carried) <= 1e-3 * fmax(fabs(s), fabs(carried));
+      pscale_s = ok ? sqrtf((float)(s / n) + 1e-9f) : __builtin_nanf("");
+      if (!ok) __hip_atomic_store(velo_guard_flag(sync, n_tensors), it.tensor + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
   }
   __syncthreads();
   const float* wm = wmix + (size_t)it.tensor * 160;
   if (threadIdx.x < kVFold)
     coh_store_wait(wfold + (size_t)it.tensor * kVFold + threadIdx.x,
-                   poison_s ? __builtin_nanf("") : velo_fold_entry(d, wm, sc, pscale_s, wm[kVBank], threadIdx.x));
+                   velo_fold_entry(d, wm, sc, pscale_s, wm[kVBank], threadIdx.x));
   __syncthreads();   // every folded weight has been performed
   if (threadIdx.x == 0) __hip_atomic_store(sync + n_tensors + it.tensor, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }

@@ -81,7 +81,7 @@ struct NsBatch { int mat0, n_mats, split_item0, n_split_items, group0, n_groups;
 struct Layout {
   std::vector<Item> mx_items;   // ELO-CELO2: statistics and apply items in slab order (k_celo2_elem)
   size_t off_mx_items = 0, off_sync = 0;
-  size_t off_newsum = 0, off_piv = 0, off_wmix = 0, off_carried = 0, off_stale = 0;   // VeLO: sums carried to the next step, pivots, un-folded MLPs
+  size_t off_newsum = 0, off_piv = 0, off_wmix = 0;   // VeLO: sums carried to the next step, pivots, un-folded MLPs
   // ELO-CELO2: Newton-Schulz on the 2-D tensors (k_ns.h)
   std::vector<NsMat> ns_mats;
   std::vector<NsItem> ns_gram, ns_poly, ns_upd;
@@ -740,12 +740,11 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_canon = take(kind == PYLO_KIND_VELO ? sizeof(float) * kVCanon * (size_t)T : 0);
   L.off_frac = take(kind == PYLO_KIND_VELO ? sizeof(float) * 9 * PYLO_MAX_GROUPS : 0);
   L.off_mx_items = take(sizeof(Item) * L.mx_items.size());
-  L.off_sync = take(sizeof(int) * 2 * (size_t)T);
+  // (VeLO: behind the counters, the guard of the carried sums: flag address, padding, T doubles -- k_velo.h)
+  L.off_sync = take(sizeof(int) * (size_t)((2 * T + 3) & ~3) + (kind == PYLO_KIND_VELO ? 16 + sizeof(double) * (size_t)T : 0));
   L.off_newsum = take(kind == PYLO_KIND_VELO ? sizeof(double) * kNewSumW * L.el_items.size() : 0);
   L.off_piv = take(kind == PYLO_KIND_VELO ? sizeof(float) * 4 * (size_t)T : 0);
   L.off_wmix = take(kind == PYLO_KIND_VELO ? sizeof(float) * 160 * (size_t)T : 0);
-  L.off_carried = take(kind == PYLO_KIND_VELO ? sizeof(double) * (size_t)T : 0);
-  L.off_stale = take(kind == PYLO_KIND_VELO ? sizeof(int) * 2 : 0);
   if (kind == PYLO_KIND_CELO2) {
     long long ns_floats = 0;
     L.ns_bf = env_ns_bf();
@@ -794,10 +793,11 @@ struct PyloPlan {
   // VeLO: the LSTM's input sums were left by the previous step's apply items (see k_velo_elem); false
   // until a step has run and after pylo_mi355_plan_invalidate_statistics
   bool stats_carried = false;
-  // the guard of those sums: {generation, tensor} as the device left them (pinned; copied at the end of every step)
-  // and the generation that counts (pylo_mi355_plan_invalidate_statistics starts a new one)
+  // the guard of those sums: 1 + tensor in pinned host memory that the kernel writes straight into when it catches a
+  // mismatch (nothing is copied on the steps that find none; pylo_mi355_plan_invalidate_statistics clears it), and
+  // its address as the device sees it
   int* stale_host = nullptr;
-  int stale_gen = 1;
+  int* stale_dev = nullptr;
   hipStream_t side = nullptr;            // the LSTM runs next to the gradient sums on a stream of the plan's own
   hipEvent_t ev_fork = nullptr, ev_join = nullptr;
   // ELO-CELO2: the Newton-Schulz chains of the groups of matrices after the first run on streams of the plan's own
@@ -877,10 +877,15 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
     if (e == hipSuccess) e = hipEventCreateWithFlags(&P->ev[i], hipEventDisableTiming);
   }
   if (e == hipSuccess && kind == PYLO_KIND_VELO) {
-    e = hipHostMalloc(reinterpret_cast<void**>(&P->stale_host), 64, hipHostMallocDefault);
+    e = hipHostMalloc(reinterpret_cast<void**>(&P->stale_host), 64, hipHostMallocMapped);
     if (e == hipSuccess) P->stale_host[0] = P->stale_host[1] = 0;
-    if (e == hipSuccess) e = hipMemsetAsync(P->ws + L.off_stale, 0, 2 * sizeof(int), s);
-    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e == hipSuccess) e = hipHostGetDevicePointer(reinterpret_cast<void**>(&P->stale_dev), P->stale_host, 0);
+    if (e == hipSuccess) {   // its address, where the kernels look for it (behind the counters of `sync`)
+      const long long addr = reinterpret_cast<long long>(P->stale_dev);
+      e = hipMemcpyAsync(P->ws + L.off_sync + sizeof(int) * (size_t)((2 * n_tensors + 3) & ~3), &addr, sizeof(addr),
+                         hipMemcpyHostToDevice, s);
+      if (e == hipSuccess) e = hipStreamSynchronize(s);
+    }
   }
   if (e == hipSuccess && kind == PYLO_KIND_VELO && !P->L.mx_items.empty()) {
     e = hipStreamCreateWithFlags(&P->side, hipStreamNonBlocking);
@@ -1568,8 +1573,7 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
     HIP_TRY(hipEventRecord(P->ev_fork, s));
     HIP_TRY(hipStreamWaitEvent(P->side, P->ev_fork, 0));
     hipLaunchKernelGGL(k_velo_feat, dim3(T), dim3(kFoldThreads), 0, P->side, descs, dyn, T, (const double*)newsum, piv, ls, vs,
-                       xfeat, H, nets->mix2_wt, nets->mix2_b, nets->fmix_wt, nets->fmix_b, mixbuf, P->at<int>(L.off_sync),
-                       P->at<double>(L.off_carried));
+                       xfeat, H, nets->mix2_wt, nets->mix2_b, nets->fmix_wt, nets->fmix_b, mixbuf, P->at<int>(L.off_sync));
     lstm(P->side, nullptr, false);
     HIP_TRY(hipEventRecord(P->ev_join, P->side));
     gradient_sums();
@@ -1580,12 +1584,9 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
       hipLaunchKernelGGL(k_terms<4>, dim3(n_v0b), dim3(kThreads), 0, s, descs, dyn, v0b_items, bscale, canon, kVCanon, term_tab);
     HIP_TRY(mark());
     hipLaunchKernelGGL(k_velo_elem, dim3(n_mx), dim3(kThreads), 0, s, descs, dyn, P->at<Item>(L.off_mx_items), fac_tab, term_tab,
-                       dec, (const float*)wmix, wfold, stats, (const float*)piv, newsum, P->at<int>(L.off_sync), T,
-                       (const double*)P->at<double>(L.off_carried), P->at<int>(L.off_stale), P->stale_gen);
+                       dec, (const float*)wmix, wfold, stats, (const float*)piv, newsum, P->at<int>(L.off_sync), T);
     HIP_TRY(mark());
     mark.done();
-    // what the guard of the carried sums found, for pylo_mi355_plan_statistics_stale (read without waiting)
-    HIP_TRY(hipMemcpyAsync(P->stale_host, P->at<int>(L.off_stale), 2 * sizeof(int), hipMemcpyDeviceToHost, s));
     stage_out(P, s, 0);
     HIP_TRY(hipGetLastError());
     return 0;
@@ -1623,14 +1624,13 @@ extern "C" int pylo_mi355_velo_step(PyloPlan* P, const PyloTensorArgs* args, con
 extern "C" int pylo_mi355_plan_invalidate_statistics(PyloPlan* P) {
   if (!P) return fail("plan_invalidate_statistics: null plan");
   P->stats_carried = false;
-  ++P->stale_gen;   // what the guard found before this call no longer counts
+  if (P->stale_host) *static_cast<volatile int*>(P->stale_host) = 0;   // what the guard found before this call no longer counts
   return 0;
 }
 
 extern "C" int pylo_mi355_plan_statistics_stale(const PyloPlan* P) {
   if (!P || !P->stale_host) return 0;
-  const volatile int* h = P->stale_host;
-  return h[0] == P->stale_gen ? h[1] + 1 : 0;
+  return *static_cast<const volatile int*>(P->stale_host);
 }
 
 extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, const PyloDecays* decays,

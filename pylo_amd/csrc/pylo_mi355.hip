@@ -228,7 +228,7 @@ bool env_ns_xcd() {
 // PYLO_MI355_NS_GROUPS: into how many groups (streams) the matrices of a plan are dealt, 1 to 4; read at plan creation.
 int env_ns_groups() {
   const char* e = getenv("PYLO_MI355_NS_GROUPS");
-  const int g = e ? atoi(e) : 2;
+  const int g = e ? atoi(e) : 4;
   return std::max(1, std::min(g, 4));
 }
 

@@ -231,15 +231,17 @@ int pylo_mi355_celo2_finish(PyloPlan* plan, const PyloTensorArgs* args, void* st
  * as matrix-pipe products of the library's own that compute the symmetric A and c0 I + c1 A + c2 A A once per
  * pair of tiles -- by default on the bf16 matrix instructions at fp32 accuracy (every fp32 operand is the exact
  * sum of three bf16 numbers, six bf16 products per fp32 product, fp32 accumulation; what is dropped is below
- * 2^-24 of a product), with PYLO_MI355_NS_F32=1 in the environment at plan creation on the fp32 matrix
- * instructions; then every tensor is normalised and applied as by pylo_mi355_celo2_finish (tensors without the
+ * 2^-24 of a product; two iterations share one Gram product and one update, A' = B' A B' and
+ * X'' = (B'' B') X, which costs about 1e-6 of B' in accuracy whatever the spectrum of X -- PYLO_MI355_NS_PAIRS=0
+ * in the environment keeps one of each per iteration), with PYLO_MI355_NS_F32=1 in the environment at plan
+ * creation on the fp32 matrix instructions; then every tensor is normalised and applied as by pylo_mi355_celo2_finish (tensors without the
  * flag from `step_out` as it stands).  `step_out` of a flagged tensor is overwritten (with the orthogonalised
  * step).  A tensor can carry the flag when pylo_mi355_plan_orthogonalize_supported says so: two dims (any two;
  * the fp32 instructions: the last and the smaller dim multiples of 4) and no PYLO_F_NO_ORTHOGONALIZE in its
  * shape flags; others (and tensors whose step is orthogonalised per slice of more leading dims) are
  * orthogonalised by the caller and passed without the flag.  The plan's workspace holds the operand planes:
  * 18 bytes per element of every such tensor (X as three bf16 planes in both orientations, the orientation
- * that the update product writes twice) plus 16 bytes per element of its m x m matrices -- 2.2 GB for a
+ * that the update product writes twice) plus 28 bytes per element of its m x m matrices -- 2.3 GB for a
  * GPT-2-small set, all tensors resident at once; pylo_mi355_plan_workspace_bytes reports the total.  The
  * products of groups of tensors run on streams of the plan's own next to the caller's (forked and joined
  * with events, default priority); the call returns with the caller's stream waiting for them.

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define PYLO_MI355_ABI_VERSION 8
+#define PYLO_MI355_ABI_VERSION 9
 #define PYLO_MAX_DIMS 8
 #define PYLO_MAX_GROUPS 8   /* parameter groups with their own step counter (VeLO) */
 
@@ -215,12 +215,16 @@ int pylo_mi355_celo2_step(PyloPlan* plan, const PyloTensorArgs* args, const Pylo
  *     param <- param - lr * (step + weight_decay * param)
  * Fields read per tensor: grad (only as "takes part" flag), param, step_out, lr, weight_decay,
  * step_mult.  PYLO_F_ADAM tensors are skipped; tensors of fewer than two dims on the MLP path are
- * handled like matrices (their normaliser is over the whole vector); tensors with more than two dims
- * are refused, since their normaliser is per slice of the last two dims (ELO_CELO2_naive.py:217-218,235).
+ * handled like matrices (their normaliser is over the whole vector).  A tensor with more than two dims
+ * has one normaliser per slice of its last two dims (ELO_CELO2_naive.py:217-218,235): its slices are
+ * normalised and applied by one more launch, each slice held in LDS by the lanes that own it, when
+ * pylo_mi355_plan_finish_supported says that a slice fits (X twice and two m x m fp32 matrices in 128 KB:
+ * every convolution kernel); otherwise the tensor is refused and left to the caller.
  * Three launches: sum of squares per 8192-element block, per-tensor scale (fixed-order fp64 sum),
  * update.  16 bytes per element.
  */
 int pylo_mi355_celo2_finish(PyloPlan* plan, const PyloTensorArgs* args, void* stream);
+int pylo_mi355_plan_finish_supported(const PyloPlan* plan, int tensor);
 
 /*
  * Newton-Schulz and the finishing pass in one call (replaces `step = newton_schulz(step, ...)` of the
@@ -238,8 +242,10 @@ int pylo_mi355_celo2_finish(PyloPlan* plan, const PyloTensorArgs* args, void* st
  * flag from `step_out` as it stands).  `step_out` of a flagged tensor is overwritten (with the orthogonalised
  * step).  A tensor can carry the flag when pylo_mi355_plan_orthogonalize_supported says so: two dims (any two;
  * the fp32 instructions: the last and the smaller dim multiples of 4) and no PYLO_F_NO_ORTHOGONALIZE in its
- * shape flags; others (and tensors whose step is orthogonalised per slice of more leading dims) are
- * orthogonalised by the caller and passed without the flag.  The plan's workspace holds the operand planes:
+ * shape flags; a tensor with more than two dims whose slices fit (pylo_mi355_plan_finish_supported) is
+ * orthogonalised slice by slice in the launch that normalises and applies it (fp32 FMA in LDS, `ns_iters`
+ * may be 0 there: division by the norm only; `step_out` is left as it was); others are orthogonalised by
+ * the caller and passed without the flag.  The plan's workspace holds the operand planes:
  * 18 bytes per element of every such tensor (X as three bf16 planes in both orientations, the orientation
  * that the update product writes twice) plus 28 bytes per element of its m x m matrices -- 2.3 GB for a
  * GPT-2-small set, all tensors resident at once; pylo_mi355_plan_workspace_bytes reports the total.  The

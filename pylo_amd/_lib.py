@@ -103,6 +103,7 @@ def load():
     lib.pylo_mi355_celo2_orthogonalize_finish.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_float), C.c_int,
                                                          C.c_float, C.c_void_p]
     lib.pylo_mi355_plan_orthogonalize_supported.argtypes = [C.c_void_p, C.c_int]
+    lib.pylo_mi355_plan_finish_supported.argtypes = [C.c_void_p, C.c_int]
     lib.pylo_mi355_velo_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.POINTER(VeloNets),
                                          C.POINTER(VeloStep), C.c_void_p]
     lib.pylo_mi355_adafac_step.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(Decays), C.c_void_p, C.c_float,
@@ -111,7 +112,7 @@ def load():
     lib.pylo_mi355_plan_statistics_stale.argtypes = [C.c_void_p]
     lib.pylo_mi355_plan_arg_table.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_void_p)]
     lib.pylo_mi355_plan_device_steps.argtypes = [C.c_void_p, C.POINTER(DeviceSteps)]
-    if lib.pylo_mi355_abi_version() != 8:
+    if lib.pylo_mi355_abi_version() != 9:
         raise RuntimeError("libpylo_mi355.so: ABI version mismatch, rebuild it")
     _lib = lib
     return lib
@@ -236,6 +237,9 @@ class Plan:
 
     def orthogonalize_supported(self, i: int) -> bool:
         return load().pylo_mi355_plan_orthogonalize_supported(self._h, i) == 1
+
+    def finish_supported(self, i: int) -> bool:
+        return load().pylo_mi355_plan_finish_supported(self._h, i) == 1
 
     def celo2_orthogonalize_finish(self, args: np.ndarray, coeffs, iters: int, eps: float, stream: int) -> None:
         """Newton-Schulz on the tensors flagged in `args["flags"]`, then normalise + apply for all of them."""

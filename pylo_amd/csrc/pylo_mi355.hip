@@ -31,6 +31,7 @@
 #include "k_celo2_slices.h"
 #include "k_ns.h"
 #include "k_ns_bf.h"
+#include "k_slice_finish.h"
 #include "k_cast.h"
 #include "pylo_common.h"
 #include "pylo_mi355_bench.h"
@@ -91,6 +92,14 @@ struct Layout {
   std::vector<int> ns_split;          // matrices whose Gram product is split (k_ns_gram_reduce)
   std::vector<long long> ns_xalt;     // per tensor: offset of its second X buffer, -1 without one
   std::vector<int> ns_of_tensor;      // per tensor: index into ns_mats, -1
+  // ELO-CELO2: tensors with more than two dims, finished per slice of the last two dims (k_slice_finish.h)
+  std::vector<SliceMat> slice_mats;
+  // blocks of the lane-owned slices (in registers: 1 x 1, 3 x 3, 5 x 5, 7 x 7; in LDS: up to 12, 28, 64 KB a wave),
+  // of the wave-owned and of the block-owned ones
+  std::vector<Item> slice_items_l[kSliceLaneSets], slice_items_w, slice_items_b;
+  std::vector<int> slice_of_tensor;   // per tensor: index into slice_mats, -1
+  int slice_lds_l[kSliceLaneSets] = {}, slice_lds_w = 0, slice_lds_b = 0;
+  size_t off_slice_mats = 0, off_slice_items_l[kSliceLaneSets] = {}, off_slice_items_w = 0, off_slice_items_b = 0;
   int ns_max_m = 0;
   // Newton-Schulz on the bf16 matrix pipe (three-way split operands): tables of their own
   bool ns_bf = false;
@@ -484,6 +493,44 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
   std::stable_sort(L.ns_upd.begin(), L.ns_upd.end(), longer);
 }
 
+// ELO-CELO2 tensors with more than two dims on the MLP path: the slices of their last two dims, where one fits the
+// LDS of the lanes that would own it (k_slice_finish.h).
+void build_slice_tables(Layout& L, const PyloTensorShape* shapes, int T) {
+  L.slice_of_tensor.assign(T, -1);
+  L.slice_mats.clear(); L.slice_items_w.clear(); L.slice_items_b.clear();
+  for (int k = 0; k < kSliceLaneSets; ++k) { L.slice_items_l[k].clear(); L.slice_lds_l[k] = 0; }
+  L.slice_lds_w = L.slice_lds_b = 0;
+  for (int t = 0; t < T; ++t) {
+    const TDesc& d = L.descs[t];
+    const PyloTensorShape& sh = shapes[t];
+    if (d.mode != kModeFacND || d.n == 0 || sh.ndim < 3) continue;
+    SliceMat sm{};
+    sm.tensor = t;
+    sm.R = (int)sh.shape[sh.ndim - 2];
+    sm.C = (int)sh.shape[sh.ndim - 1];
+    sm.slices = d.n / ((long long)sm.R * sm.C);
+    sm.no_orth = (sh.flags & PYLO_F_NO_ORTHOGONALIZE) != 0;
+    if (!slice_geometry(sm)) continue;
+    const int per_block = sm.lanes == 1 ? 64 : 256 / sm.lanes;
+    const long long blocks = (sm.slices + per_block - 1) / per_block;
+    if (blocks >= (1ll << 31)) continue;
+    const int q = (int)L.slice_mats.size();
+    L.slice_of_tensor[t] = q;
+    // lane-owned slices: one launch per register size, and per LDS size class of the others (a wave's LDS share
+    // decides how many waves a CU holds)
+    int set = 0;
+    if (sm.lanes == 1) {
+      const long long need = slice_lane_lds(sm.m, sm.n);
+      set = slice_in_registers(sm.m, sm.n) ? sm.m / 2 : need <= 12 * 1024 ? 4 : need <= 28 * 1024 ? 5 : 6;
+    }
+    std::vector<Item>& items = sm.lanes == 1 ? L.slice_items_l[set] : sm.lanes == 256 ? L.slice_items_b : L.slice_items_w;
+    int& lds = sm.lanes == 1 ? L.slice_lds_l[set] : sm.lanes == 256 ? L.slice_lds_b : L.slice_lds_w;
+    lds = std::max(lds, sm.lanes == 1 ? (int)slice_lane_lds(sm.m, sm.n) : (int)sizeof(float) * sm.per_floats * per_block);
+    for (long long b = 0; b < blocks; ++b) items.push_back(Item{q, (int)b, 0, 0});
+    L.slice_mats.push_back(sm);
+  }
+}
+
 int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int velo_hidden) {
   if (kind != PYLO_KIND_CELO2 && kind != PYLO_KIND_VELO && kind != PYLO_KIND_ADAFAC)
     return fail("plan: unknown optimizer kind");
@@ -655,7 +702,8 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       d.nseg = (int)L.seg_items.size() - d.seg0;
     }
     // blocks of ELO-CELO2's finishing pass (after Newton-Schulz): linear 8192-element pieces of the MLP tensors
-    if (kind == PYLO_KIND_CELO2 && d.mode != kModeFlat) {
+    // (tensors with more dims are finished per slice, k_slice_finish.h)
+    if (kind == PYLO_KIND_CELO2 && d.mode != kModeFlat && d.mode != kModeFacND) {
       d.fin_blk0 = (int)L.fin_items.size();
       for (long long c = 0; c * kFinElems < n; ++c) L.fin_items.push_back(Item{t, (int)c, 0, 0});
       d.fin_nblk = (int)L.fin_items.size() - d.fin_blk0;
@@ -761,6 +809,11 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     L.off_nsb_mats = take(sizeof(NsBfMat) * L.nsb_mats.size());
     L.off_nsb_split_items = take(sizeof(NsTileItem) * L.nsb_split_items.size());
     L.off_ns_pw = take(sizeof(bfbits) * (size_t)L.nsb_plane_elems);
+    build_slice_tables(L, shapes, T);
+    L.off_slice_mats = take(sizeof(SliceMat) * L.slice_mats.size());
+    for (int k = 0; k < kSliceLaneSets; ++k) L.off_slice_items_l[k] = take(sizeof(Item) * L.slice_items_l[k].size());
+    L.off_slice_items_w = take(sizeof(Item) * L.slice_items_w.size());
+    L.off_slice_items_b = take(sizeof(Item) * L.slice_items_b.size());
   }
   L.total = off;
   return 0;
@@ -867,6 +920,11 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess && kind == PYLO_KIND_CELO2) e = up(L.off_ns_xalt, L.ns_xalt.data(), sizeof(long long) * L.ns_xalt.size());
   if (e == hipSuccess) e = up(L.off_nsb_mats, L.nsb_mats.data(), sizeof(NsBfMat) * L.nsb_mats.size());
   if (e == hipSuccess) e = up(L.off_nsb_split_items, L.nsb_split_items.data(), sizeof(NsTileItem) * L.nsb_split_items.size());
+  if (e == hipSuccess) e = up(L.off_slice_mats, L.slice_mats.data(), sizeof(SliceMat) * L.slice_mats.size());
+  for (int k = 0; k < kSliceLaneSets; ++k)
+    if (e == hipSuccess) e = up(L.off_slice_items_l[k], L.slice_items_l[k].data(), sizeof(Item) * L.slice_items_l[k].size());
+  if (e == hipSuccess) e = up(L.off_slice_items_w, L.slice_items_w.data(), sizeof(Item) * L.slice_items_w.size());
+  if (e == hipSuccess) e = up(L.off_slice_items_b, L.slice_items_b.data(), sizeof(Item) * L.slice_items_b.size());
   // the padding of the operand planes is read by the products and written by nobody: zero, once
   if (e == hipSuccess && L.nsb_plane_elems > 0)
     e = hipMemsetAsync(P->ws + L.off_ns_pw, 0, sizeof(bfbits) * (size_t)L.nsb_plane_elems, s);
@@ -1311,6 +1369,19 @@ int ns_bf_lds_once() {
   return 0;
 }
 
+int slice_lds_once() {
+  static std::mutex mu;
+  static std::vector<int> done;
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(mu);
+  for (int d : done)
+    if (d == dev) return 0;
+  HIP_TRY(hipFuncSetAttribute((const void*)k_celo2_slice_finish<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kSliceLdsBlock));
+  done.push_back(dev);
+  return 0;
+}
+
 __global__ __launch_bounds__(256) void k_ns_zero(u32x4* __restrict__ p, size_t n16) {
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) p[i] = u32x4{0u, 0u, 0u, 0u};
 }
@@ -1322,17 +1393,25 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
   if (!P || P->kind != PYLO_KIND_CELO2) return fail(w + ": not an ELO-CELO2 plan");
   if (!args) return fail(w + ": null argument");
   const Layout& L = P->L;
-  bool any_ns = false;
+  bool any_ns = false, any_slices = false;
   for (int t = 0; t < P->T; ++t) {
     const TDesc& d = L.descs[t];
     const PyloTensorArgs& a = args[t];
     if (a.grad == nullptr || d.mode == kModeFlat || d.n == 0) continue;
     const std::string at = " (tensor " + std::to_string(t) + ")";
-    if (d.mode == kModeFacND)
-      return fail(w + ": tensors with more than two dims are normalised per slice of the last two dims, "
-                  "not by this tensor-wide pass" + at);
     if (!a.param || !a.step_out) return fail(w + ": null param/step_out pointer" + at);
     const uintptr_t m = reinterpret_cast<uintptr_t>(a.param) | reinterpret_cast<uintptr_t>(a.step_out);
+    if (d.mode == kModeFacND) {
+      if (L.slice_of_tensor[t] < 0)
+        return fail(w + ": a tensor with more than two dims whose slices of the last two dims do not fit the "
+                    "per-slice pass (pylo_mi355_plan_finish_supported)" + at);
+      if (reinterpret_cast<uintptr_t>(a.step_out) % 4 != 0 || reinterpret_cast<uintptr_t>(a.param) % (d.store != 0 ? 2 : 4) != 0)
+        return fail(w + ": misaligned pointer" + at);
+      if (coeffs && (a.flags & PYLO_ARG_ORTHOGONALIZE) && L.slice_mats[L.slice_of_tensor[t]].no_orth)
+        return fail(w + ": PYLO_ARG_ORTHOGONALIZE on a tensor whose shape carries PYLO_F_NO_ORTHOGONALIZE" + at);
+      any_slices = true;
+      continue;
+    }
     if (m % (d.n % 4 == 0 ? 16 : 4) != 0) return fail(w + ": misaligned pointer" + at);
     if (ns_iters > 0 && (a.flags & PYLO_ARG_ORTHOGONALIZE)) {
       if (L.ns_of_tensor[t] < 0) return fail(w + ": PYLO_ARG_ORTHOGONALIZE on a tensor the library cannot orthogonalise" + at);
@@ -1348,7 +1427,33 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
   double* fin_part = P->at<double>(L.off_finpart);
   float* fin_scale = P->at<float>(L.off_finscale);
   const int n_fin = (int)L.fin_items.size();
-  if (n_fin == 0) return 0;
+  if (any_slices) {
+    // tensors with more than two dims: everything per slice, in LDS (k_slice_finish.h)
+    if (int rc = slice_lds_once()) return rc;
+    const SliceMat* smats = P->at<SliceMat>(L.off_slice_mats);
+    const float c0 = coeffs ? coeffs[0] : 0.0f, c1 = coeffs ? coeffs[1] : 0.0f, c2 = coeffs ? coeffs[2] : 0.0f;
+    const int orth_call = coeffs != nullptr;
+    auto lanes = [&](auto kern, int set) {
+      if (!L.slice_items_l[set].empty())
+        hipLaunchKernelGGL(kern, dim3((unsigned)L.slice_items_l[set].size()), dim3(64), L.slice_lds_l[set], s, smats,
+                           P->at<Item>(L.off_slice_items_l[set]), descs, dyn, orth_call, ns_iters, ns_eps, c0, c1, c2);
+    };
+    lanes(k_celo2_slice_finish_lane<1>, 0);
+    lanes(k_celo2_slice_finish_lane<3>, 1);
+    lanes(k_celo2_slice_finish_lane<5>, 2);
+    lanes(k_celo2_slice_finish_lane<7>, 3);
+    for (int set = 4; set < kSliceLaneSets; ++set) lanes(k_celo2_slice_finish_lane<0>, set);
+    if (!L.slice_items_w.empty())
+      hipLaunchKernelGGL(k_celo2_slice_finish<false>, dim3((unsigned)L.slice_items_w.size()), dim3(256), L.slice_lds_w, s,
+                         smats, P->at<Item>(L.off_slice_items_w), descs, dyn, orth_call, ns_iters, ns_eps, c0, c1, c2);
+    if (!L.slice_items_b.empty())
+      hipLaunchKernelGGL(k_celo2_slice_finish<true>, dim3((unsigned)L.slice_items_b.size()), dim3(256), L.slice_lds_b, s,
+                         smats, P->at<Item>(L.off_slice_items_b), descs, dyn, orth_call, ns_iters, ns_eps, c0, c1, c2);
+  }
+  if (n_fin == 0) {
+    HIP_TRY(hipGetLastError());
+    return 0;
+  }
   const long long* x_alt = nullptr;
   float* ns_ws = nullptr;
   if (any_ns) {
@@ -1470,8 +1575,17 @@ extern "C" int pylo_mi355_celo2_orthogonalize_finish(PyloPlan* P, const PyloTens
   return finish_impl(P, args, ns_coeffs, ns_iters, ns_eps, stream, "celo2_orthogonalize_finish");
 }
 
+extern "C" int pylo_mi355_plan_finish_supported(const PyloPlan* P, int tensor) {
+  if (!P || tensor < 0 || tensor >= P->T || P->kind != PYLO_KIND_CELO2) return 0;
+  const TDesc& d = P->L.descs[tensor];
+  if (d.mode == kModeFlat) return 0;
+  return d.mode != kModeFacND || P->L.slice_of_tensor[tensor] >= 0 ? 1 : 0;
+}
+
 extern "C" int pylo_mi355_plan_orthogonalize_supported(const PyloPlan* P, int tensor) {
   if (!P || tensor < 0 || tensor >= P->T || P->kind != PYLO_KIND_CELO2) return 0;
+  if (P->L.descs[tensor].mode == kModeFacND)
+    return P->L.slice_of_tensor[tensor] >= 0 && !P->L.slice_mats[P->L.slice_of_tensor[tensor]].no_orth ? 1 : 0;
   return P->L.ns_of_tensor[tensor] >= 0 ? 1 : 0;
 }
 

@@ -5,9 +5,9 @@ Drop-in for pylo/optim/ELO_CELO2_cuda.py:39-298: same constructor, ``step()``,
 ``param_groups`` keys and per-parameter state (``mom (3,*s)``, ``rms (*s)``, ``fac_r``,
 ``fac_c``).  What differs is *where* the work happens: gradient clipping, every
 accumulator update, the 1-D AdamW branch and the feature/MLP pass of all tensors run in one
-call into ``libpylo_mi355.so`` (eight launches); Newton-Schulz runs as batched library GEMMs over
-buckets of equally shaped tensors, and a second call normalises the steps and updates the
-parameters.  Arithmetic follows the
+call into ``libpylo_mi355.so`` (seven launches); a second call orthogonalises the steps of all
+matrices (Newton-Schulz as matrix-pipe products of the library's own; the slices of a tensor with more
+than two dims each in LDS), normalises them and updates the parameters.  Arithmetic follows the
 reference's naive class (pylo/optim/ELO_CELO2_naive.py:126-306), also where the reference's CUDA class
 differs or fails: tensors with more than two dims normalise features and steps per slice of the last two
 dims, and ``use_adamw_for_1d=False`` sends 1-D tensors through the MLP with a per-element accumulator
@@ -264,6 +264,7 @@ class ELO_CELO2_CUDA(Optimizer):
         self._fin_args = np.zeros(len(tensors), dtype=_lib.ARGS_DTYPE)
         self._fin_fast = None
         self._ns_ok = [self._plan.orthogonalize_supported(i) for i in range(len(tensors))]
+        self._fin_ok = [self._plan.finish_supported(i) for i in range(len(tensors))]
         if self.capturable:
             self._reset_device_steps(tensors)
 
@@ -494,7 +495,7 @@ class ELO_CELO2_CUDA(Optimizer):
 
     # The finishing call's table has one row per tensor as well.  When the step went through the cached rows of
     # the fused call (every tensor has a gradient) and the library finishes every MLP tensor itself (no tensor
-    # with more than two dims, no param_scale_mult, no torch products), its static columns are kept too and a
+    # with slices too large for the per-slice launch, no param_scale_mult, no torch products), its static columns are kept too and a
     # step refreshes parameter pointers and the groups' scalars with a few array operations, whatever the
     # number of tensors.
     def _fin_fast_key(self):
@@ -508,11 +509,13 @@ class ELO_CELO2_CUDA(Optimizer):
         for i, (group, p, adam) in enumerate(tensors):
             if adam:
                 continue
+            orth = bool(group["orthogonalize"]) and p.dim() >= 2
             if p.dim() > 2:
-                return None
-            orth = bool(group["orthogonalize"]) and p.dim() == 2
+                # per slice of the last two dims, all of it in one launch of the library's (any ns_iters)
+                if not self._fin_ok[i] or (orth and not (self._lib_ns and self._ns_ok[i])):
+                    return None
             # (zero iterations still divide by the Frobenius norm, which the normaliser's epsilon sees: torch path)
-            if orth and not (self._lib_ns and self._ns_ok[i] and self.ns_iters > 0):
+            elif orth and not (self._lib_ns and self._ns_ok[i] and self.ns_iters > 0):
                 return None
             idx.append(i)
             flags.append(_lib.ARG_ORTHOGONALIZE if orth else 0)
@@ -580,15 +583,18 @@ class ELO_CELO2_CUDA(Optimizer):
                 sq = torch.stack(torch._foreach_norm([p.float() for p in ps] if ps[0].dtype != torch.float32 else ps)) ** 2 / n
                 step = step.mul_(torch.sqrt(sq + 1e-9).view([-1] + [1] * nd))   # the raw steps are scratch
             flag = 0
+            # more than two dims: Newton-Schulz and the normaliser are per slice of the last two dims
+            # (ELO_CELO2_naive.py:217-218,235); the library does both where a slice fits its per-slice launch
+            nd_lib = nd > 2 and all(self._fin_ok[i] for i in idx) and (
+                not group["orthogonalize"] or (lib_ns and all(self._ns_ok[i] for i in idx)))
             if group["orthogonalize"] and nd >= 2:
-                if lib_ns and nd == 2 and self.ns_iters > 0 and all(self._ns_ok[i] for i in idx):
+                if nd_lib or (lib_ns and nd == 2 and self.ns_iters > 0 and all(self._ns_ok[i] for i in idx)):
                     flag = _lib.ARG_ORTHOGONALIZE
                 else:
                     with _ns_blas():
                         step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
-            if nd > 2:
-                # more than two dims: the normaliser is per slice of the last two dims
-                # (ELO_CELO2_naive.py:217-218,235), which the tensor-wide finishing kernels do not do
+            if nd > 2 and not nd_lib:
+                # slices too large for the library's per-slice launch
                 step = rms_normalize(step, [-2, -1]) * group["rmsmult"]
                 for j, p in enumerate(ps):
                     _apply(p, step[j], group["weight_decay"], group["lr"])

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     assert len(names) >= 12, names
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in the header but not exported"
-    assert lib.pylo_mi355_abi_version() == 8
+    assert lib.pylo_mi355_abi_version() == 9
 
 
 def test_struct_sizes_match_header():

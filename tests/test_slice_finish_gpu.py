@@ -1,0 +1,166 @@
+"""Tensors with more than two dims in ``pylo_mi355_celo2_orthogonalize_finish`` / ``pylo_mi355_celo2_finish``:
+Newton-Schulz, the normaliser and the parameter update per slice of the last two dims
+(pylo/optim/CELO2_naive.py:59-73 "over the last two dims"; pylo/optim/ELO_CELO2_naive.py:231-235), each slice
+held in LDS by one lane, a wave or a block.  Against the literal formula in fp64 slice by slice through the
+C-ABI, and through whole optimizer steps against the oracle (parameters at rel 1e-5 / abs 1e-6).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from golden_io import max_err
+
+pytestmark = pytest.mark.gpu
+
+COEFFS = (3.4445, -4.775, 2.0315)
+
+# (shape, lanes that own a slice)
+SHAPES = [((32, 16, 3, 3), 1), ((6, 4, 1, 1), 1), ((5, 4, 8), 1), ((3, 8, 4), 1), ((2, 1, 7), 1), ((5, 5, 5, 5), 1),
+          ((4, 6, 6), 1), ((70, 7, 7), 1), ((3, 2, 100), 1), ((130, 3, 3), 1),
+          ((7, 16, 16), 64), ((2, 3, 4, 70), 64), ((3, 70, 4), 64), ((5, 8, 8), 64),
+          ((3, 40, 33), 256), ((2, 64, 128), 256), ((2, 128, 64), 256), ((1, 2, 33, 200), 256)]
+
+
+def _formula(x, iters, dtype=torch.float64, orthogonalise=True):
+    """orthogonalize_via_newton_schulz and the normaliser over the last two dims, batched over the leading ones."""
+    c0, c1, c2 = COEFFS
+    x = x.to(dtype)
+    if orthogonalise:
+        t = x.shape[-2] > x.shape[-1]
+        if t:
+            x = x.transpose(-2, -1)
+        x = x / (torch.linalg.norm(x, dim=(-2, -1), keepdim=True) + 1e-8)
+        for _ in range(iters):
+            a = x @ x.transpose(-2, -1)
+            x = c0 * x + (c1 * a + c2 * (a @ a)) @ x
+        if t:
+            x = x.transpose(-2, -1)
+    return x * torch.rsqrt(1e-9 + (x * x).mean(dim=(-2, -1), keepdim=True))
+
+
+def _finish_direct(mats, iters, flag=True, entry="orthogonalize_finish"):
+    from pylo_amd import _lib
+
+    shapes = [tuple(x.shape) for x in mats]
+    plan = _lib.Plan(_lib.KIND_CELO2, shapes, [0] * len(shapes), torch.device("cuda:0"))
+    assert all(plan.finish_supported(i) and plan.orthogonalize_supported(i) for i in range(len(mats)))
+    steps = [x.clone().contiguous() for x in mats]
+    params = [torch.zeros_like(x) for x in mats]
+    fin = np.zeros(len(mats), dtype=_lib.ARGS_DTYPE)
+    for i in range(len(mats)):
+        fin["grad"][i], fin["param"][i], fin["step_out"][i] = 1, params[i].data_ptr(), steps[i].data_ptr()
+        fin["lr"][i], fin["weight_decay"][i], fin["step_mult"][i] = -1.0, 0.0, 1.0
+        fin["flags"][i] = _lib.ARG_ORTHOGONALIZE if flag else 0
+    stream = torch.cuda.current_stream().cuda_stream
+    if entry == "finish":
+        plan.celo2_finish(fin, stream)
+    else:
+        plan.celo2_orthogonalize_finish(fin, COEFFS, iters, 1e-8, stream)
+    torch.cuda.synchronize()
+    plan.close()
+    for x, s in zip(mats, steps):
+        assert torch.equal(x, s)      # the raw step is left as it was
+    return params
+
+
+@pytest.mark.parametrize("iters", [5, 1, 0])
+def test_slices_against_the_formula_in_fp64(iters):
+    """With p = 0, lr = -1 the parameter is the normalised, orthogonalised step (unit RMS per slice).  A slice of a
+    few elements can be nearly singular, where five iterations amplify rounding by up to 3.4445^5: the bar is the
+    error of the same formula in fp32 torch products times 1.5, plus 5e-5."""
+    gen = torch.Generator(device="cuda").manual_seed(11 + iters)
+    mats = [torch.randn(s, generator=gen, device="cuda") * 10.0 ** (-(i % 4)) for i, (s, _l) in enumerate(SHAPES)]
+    got = _finish_direct(mats, iters)
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    rows = []
+    try:
+        for x, y in zip(mats, got):
+            want = _formula(x, iters)
+            e = float((y.double() - want).abs().max())
+            e32 = float((_formula(x, iters, torch.float32).double() - want).abs().max())
+            rows.append((tuple(x.shape), e, e32))
+            assert e <= 1.5 * e32 + 5e-5, rows[-1]
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+    print("iters", iters, "(shape, library error, fp32 torch formula error):", rows)
+
+
+@pytest.mark.parametrize("entry", ["finish", "orthogonalize_finish"])
+def test_slices_without_the_flag_are_normalised_only(entry):
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    mats = [torch.randn(s, generator=gen, device="cuda") * 0.1 for s, _l in SHAPES]
+    # pylo_mi355_celo2_finish ignores the flag; the other entry point honours its absence
+    got = _finish_direct(mats, 5, flag=(entry == "finish"), entry=entry)
+    for x, y in zip(mats, got):
+        want = _formula(x, 0, orthogonalise=False)
+        assert float((y.double() - want).abs().max()) <= 2e-6, tuple(x.shape)
+
+
+def test_lanes_per_slice_and_slices_that_do_not_fit():
+    from pylo_amd import _lib
+
+    shapes = [s for s, _l in SHAPES] + [(2, 128, 128), (3, 64, 300), (64, 64)]
+    plan = _lib.Plan(_lib.KIND_CELO2, shapes, [0] * len(shapes), torch.device("cuda:0"))
+    n = len(SHAPES)
+    assert all(plan.finish_supported(i) for i in range(n))
+    assert not plan.finish_supported(n) and not plan.finish_supported(n + 1) and plan.finish_supported(n + 2)
+    assert not plan.orthogonalize_supported(n) and plan.orthogonalize_supported(n + 2)
+    x = torch.zeros(2 * 128 * 128, device="cuda")
+    fin = np.zeros(len(shapes), dtype=_lib.ARGS_DTYPE)
+    fin["grad"][n], fin["param"][n], fin["step_out"][n] = 1, x.data_ptr(), x.data_ptr()
+    with pytest.raises(RuntimeError, match="do not fit"):
+        plan.celo2_orthogonalize_finish(fin, COEFFS, 5, 1e-8, 0)
+    plan.close()
+    # a shape flagged as never orthogonalised: finished per slice, the flag refused
+    flags = [_lib.F_NO_ORTHOGONALIZE, 0]
+    plan = _lib.Plan(_lib.KIND_CELO2, [(4, 3, 3), (4, 3, 3)], flags, torch.device("cuda:0"))
+    assert plan.finish_supported(0) and not plan.orthogonalize_supported(0) and plan.orthogonalize_supported(1)
+    fin = np.zeros(2, dtype=_lib.ARGS_DTYPE)
+    fin["grad"][0], fin["param"][0], fin["step_out"][0] = 1, x.data_ptr(), x.data_ptr()
+    fin["flags"][0] = _lib.ARG_ORTHOGONALIZE
+    with pytest.raises(RuntimeError, match="PYLO_F_NO_ORTHOGONALIZE"):
+        plan.celo2_orthogonalize_finish(fin, COEFFS, 5, 1e-8, 0)
+    plan.close()
+
+
+@pytest.mark.parametrize("kw,with_large_slices,cached_table", [
+    (dict(), False, True), (dict(), True, False), (dict(ns_iters=0), False, False),
+    (dict(orthogonalize=False), False, True), (dict(param_scale_mult=True), False, False)])
+def test_whole_steps_against_the_oracle(kw, with_large_slices, cached_table):
+    """ELO_CELO2_CUDA.step() on convolution-shaped tensors next to matrices and vectors, free-running for four
+    steps against the fp64 oracle.  Slices of 128 x 128 do not fit the per-slice launch and stay on torch
+    products.  When the library finishes every tensor itself the finishing table is the cached one (no per-step
+    Python over the tensors); a matrix with zero iterations, large slices or param_scale_mult take the general path.
+    lr = 1e-3: among 512 random 3 x 3 slices some are nearly singular, where five iterations amplify the fp32
+    rounding of the raw step by up to 3.4445^5 in any fp32 evaluation (the accuracy of the orthogonalised step
+    itself is held by test_slices_against_the_formula_in_fp64)."""
+    from oracle import pylo_oracle as O
+    from pylo_amd import ELO_CELO2_CUDA
+    from pylo_amd.models import CELO2MLP
+
+    torch.manual_seed(1)
+    net = CELO2MLP()
+    shapes = [(32, 16, 3, 3), (7, 16, 16), (256, 384), (64,), (3, 40, 33), (2, 64, 128), (6, 4, 1, 1), (5, 4, 8)]
+    if with_large_slices:
+        shapes.append((2, 128, 128))
+    gen = torch.Generator(device="cuda").manual_seed(21)
+    init = [torch.randn(s, generator=gen, device="cuda") * 0.05 for s in shapes]
+    ref = [v.double() for v in init]
+    gpu = [torch.nn.Parameter(v.clone()) for v in init]
+    cfg = dict(lr=1e-3, weight_decay=0.1, adam_lr_mult=20.0)
+    cfg.update(kw)
+    orc = O.EloCelo2Oracle(ref, net.state_dict(), device="cuda", **cfg).double_()
+    opt = ELO_CELO2_CUDA(gpu, network=net, hf_key=None, **cfg)
+    for t in range(4):
+        grads = [torch.randn(s, generator=gen, device="cuda") * 10.0 ** (-1 - i % 3) for i, s in enumerate(shapes)]
+        for p, g in zip(gpu, grads):
+            p.grad = g
+        orc.step([g.double() for g in grads])
+        opt.step()
+        torch.cuda.synchronize()
+        for i, p in enumerate(gpu):
+            assert max_err(p, ref[i], 1e-5, 1e-6) <= 1.0, (kw, t, i, shapes[i])
+    cached = getattr(opt, "_fin_fast", None)
+    assert (cached is not None and cached["idx"] is not None) == cached_table

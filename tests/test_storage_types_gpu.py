@@ -80,7 +80,7 @@ def _grads(shapes, gen, dtype, scales):
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_elo_celo2_steps_on_stored_types(dtype):
     """Whole ELO_CELO2_CUDA.step(): matrices (column walk, linear chunks, ragged), a tensor with more than two
-    dims (torch finish), AdamW vectors, an is_embedding group; one tensor stays float32 (mixed plan)."""
+    dims (the per-slice launch), AdamW vectors, an is_embedding group; one tensor stays float32 (mixed plan)."""
     from oracle import pylo_oracle as O
     from pylo_amd import ELO_CELO2_CUDA
     from pylo_amd.models import CELO2MLP

@@ -216,10 +216,11 @@ int pylo_mi355_celo2_step(PyloPlan* plan, const PyloTensorArgs* args, const Pylo
  * Fields read per tensor: grad (only as "takes part" flag), param, step_out, lr, weight_decay,
  * step_mult.  PYLO_F_ADAM tensors are skipped; tensors of fewer than two dims on the MLP path are
  * handled like matrices (their normaliser is over the whole vector).  A tensor with more than two dims
- * has one normaliser per slice of its last two dims (ELO_CELO2_naive.py:217-218,235): its slices are
- * normalised and applied by one more launch, each slice held in LDS by the lanes that own it, when
- * pylo_mi355_plan_finish_supported says that a slice fits (X twice and two m x m fp32 matrices in 128 KB:
- * every convolution kernel); otherwise the tensor is refused and left to the caller.
+ * has one normaliser per slice of its last two dims (ELO_CELO2_naive.py:217-218,235): where a slice fits (X
+ * twice and two m x m fp32 matrices in 128 KB of LDS: every convolution kernel) its slices are normalised and
+ * applied by launches of their own, each slice held in registers or LDS by the lanes that own it; larger slices
+ * are units of the tensor-wide launches like whole tensors.  pylo_mi355_plan_finish_supported is 1 for every
+ * tensor that these calls take (all but PYLO_F_ADAM ones).
  * Three launches: sum of squares per 8192-element block, per-tensor scale (fixed-order fp64 sum),
  * update.  16 bytes per element.
  */
@@ -242,10 +243,12 @@ int pylo_mi355_plan_finish_supported(const PyloPlan* plan, int tensor);
  * flag from `step_out` as it stands).  `step_out` of a flagged tensor is overwritten (with the orthogonalised
  * step).  A tensor can carry the flag when pylo_mi355_plan_orthogonalize_supported says so: two dims (any two;
  * the fp32 instructions: the last and the smaller dim multiples of 4) and no PYLO_F_NO_ORTHOGONALIZE in its
- * shape flags; a tensor with more than two dims whose slices fit (pylo_mi355_plan_finish_supported) is
- * orthogonalised slice by slice in the launch that normalises and applies it (fp32 FMA in LDS, `ns_iters`
- * may be 0 there: division by the norm only; `step_out` is left as it was); others are orthogonalised by
- * the caller and passed without the flag.  The plan's workspace holds the operand planes:
+ * shape flags.  The function returns 1 for a tensor whose matrices go through these products (a tensor with
+ * more than two dims: one matrix per slice of the last two dims, each with its own norm; the fp32 instructions
+ * take 2-D tensors only) -- `ns_iters` = 0 with the flag is refused for those, the division by the norm alone
+ * being the caller's -- and 2 for a tensor with more than two dims whose slices are small enough to be
+ * orthogonalised in the launch that normalises and applies them (fp32 FMA in registers or LDS; `ns_iters` may
+ * be 0 there; `step_out` is left as it was).  0: orthogonalised by the caller and passed without the flag.  The plan's workspace holds the operand planes:
  * 18 bytes per element of every such tensor (X as three bf16 planes in both orientations, the orientation
  * that the update product writes twice) plus 28 bytes per element of its m x m matrices -- 2.3 GB for a
  * GPT-2-small set, all tensors resident at once; pylo_mi355_plan_workspace_bytes reports the total.  The

@@ -235,8 +235,9 @@ class Plan:
         """VeLO: 0, or 1 + the index of a tensor whose carried sum of p^2 did not match the tensor (no wait)."""
         return load().pylo_mi355_plan_statistics_stale(self._h)
 
-    def orthogonalize_supported(self, i: int) -> bool:
-        return load().pylo_mi355_plan_orthogonalize_supported(self._h, i) == 1
+    def orthogonalize_supported(self, i: int) -> int:
+        """0: not by the library; 1: by the tiled products (ns_iters > 0); 2: by the per-slice launches (any ns_iters)."""
+        return load().pylo_mi355_plan_orthogonalize_supported(self._h, i)
 
     def finish_supported(self, i: int) -> bool:
         return load().pylo_mi355_plan_finish_supported(self._h, i) == 1

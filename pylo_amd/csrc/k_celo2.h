@@ -905,7 +905,7 @@ __device__ __forceinline__ const float* fin_source(const PyloTensorArgs& a, int 
   return a.step_out;
 }
 
-__global__ __launch_bounds__(kThreads) void k_celo2_sumsq(const TDesc* __restrict__ descs,
+__global__ __launch_bounds__(kThreads) void k_celo2_sumsq(const FinUnit* __restrict__ units,
                                                           const PyloTensorArgs* __restrict__ dyn,
                                                           const Item* __restrict__ items,
                                                           double* __restrict__ fin_part,
@@ -913,15 +913,15 @@ __global__ __launch_bounds__(kThreads) void k_celo2_sumsq(const TDesc* __restric
                                                           const float* __restrict__ ws) {
   __shared__ float red[kWaves];
   const Item it = items[blockIdx.x];
-  const TDesc d = descs[it.tensor];
-  const PyloTensorArgs a = dyn[it.tensor];
+  const FinUnit u = units[it.tensor];
+  const PyloTensorArgs a = dyn[u.tensor];
   if (a.grad == nullptr) return;
   const long long base = (long long)it.a * kFinElems;
-  const long long left = d.n - base;
+  const long long left = u.n - base;
   const unsigned lim = left < (long long)kFinElems ? (unsigned)left : (unsigned)kFinElems;
-  const float* x = fin_source(a, it.tensor, x_alt, ws) + base;
+  const float* x = fin_source(a, u.tensor, x_alt, ws) + u.off + base;
   float s = 0.0f;
-  if (d.n % 4 == 0) {
+  if (u.vec) {
 #pragma unroll
     for (int i = 0; i < kElemIters; ++i) {
       const unsigned off = (i * kThreads + threadIdx.x) * 4u;
@@ -944,17 +944,17 @@ __global__ __launch_bounds__(kThreads) void k_celo2_sumsq(const TDesc* __restric
     fin_part[blockIdx.x] = ((double)red[0] + (double)red[1]) + ((double)red[2] + (double)red[3]);
 }
 
-__global__ __launch_bounds__(kThreads) void k_celo2_finscale(const TDesc* __restrict__ descs,
+__global__ __launch_bounds__(kThreads) void k_celo2_finscale(const FinUnit* __restrict__ units,
                                                              const PyloTensorArgs* __restrict__ dyn,
                                                              const double* __restrict__ fin_part,
                                                              float* __restrict__ fin_scale) {
   __shared__ double red[kWaves];
-  const int t = blockIdx.x;  // one block per tensor of the plan; AdamW tensors have no finishing blocks
-  const TDesc d = descs[t];
-  if (dyn[t].grad == nullptr || d.fin_nblk == 0) return;
+  const int t = blockIdx.x;  // one block per unit: a tensor, or a slice of the last two dims of one with more
+  const FinUnit d = units[t];
+  if (dyn[d.tensor].grad == nullptr || d.nblk == 0) return;
   double s = 0.0;
 #pragma unroll 8
-  for (int b = threadIdx.x; b < d.fin_nblk; b += kThreads) s += fin_part[d.fin_blk0 + b];
+  for (int b = threadIdx.x; b < d.nblk; b += kThreads) s += fin_part[d.blk0 + b];
   s = wave_sum(s);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
   __syncthreads();
@@ -964,31 +964,33 @@ __global__ __launch_bounds__(kThreads) void k_celo2_finscale(const TDesc* __rest
   }
 }
 
-__global__ __launch_bounds__(kThreads) void k_celo2_update(const TDesc* __restrict__ descs,
+__global__ __launch_bounds__(kThreads) void k_celo2_update(const FinUnit* __restrict__ units,
+                                                           const TDesc* __restrict__ descs,
                                                            const PyloTensorArgs* __restrict__ dyn,
                                                            const Item* __restrict__ items,
                                                            const float* __restrict__ fin_scale,
                                                            const long long* __restrict__ x_alt,
                                                            const float* __restrict__ ws) {
   const Item it = items[blockIdx.x];
-  const TDesc d = descs[it.tensor];
-  const PyloTensorArgs a = dyn[it.tensor];
+  const FinUnit u = units[it.tensor];
+  const PyloTensorArgs a = dyn[u.tensor];
   if (a.grad == nullptr) return;
-  const long long base = (long long)it.a * kFinElems;
-  const long long left = d.n - base;
+  const int store = descs[u.tensor].store;
+  const long long base = u.off + (long long)it.a * kFinElems;
+  const long long left = u.n - (long long)it.a * kFinElems;
   const unsigned lim = left < (long long)kFinElems ? (unsigned)left : (unsigned)kFinElems;
-  const float* x = fin_source(a, it.tensor, x_alt, ws) + base;
+  const float* x = fin_source(a, u.tensor, x_alt, ws) + base;
   float* p = a.param + base;
   const float sc = fin_scale[it.tensor], rm = a.step_mult, wd = a.weight_decay, nlr = -a.lr;
-  if (d.store != 0) {
+  if (store != 0) {
     // the parameter in its storage type (fp16, bf16, fp64): widened, updated in fp32, rounded to nearest-even
     for (unsigned off = threadIdx.x; off < lim; off += kThreads) {
-      const float v = *(const gfloat*)(x + off), q = load_stored(a.param, base + off, d.store);
-      store_stored(a.param, base + off, d.store, fmaf(nlr, (v * sc) * rm + wd * q, q));
+      const float v = *(const gfloat*)(x + off), q = load_stored(a.param, base + off, store);
+      store_stored(a.param, base + off, store, fmaf(nlr, (v * sc) * rm + wd * q, q));
     }
     return;
   }
-  if (d.n % 4 == 0) {
+  if (u.vec) {
 #pragma unroll
     for (int i = 0; i < kElemIters; ++i) {
       const unsigned off = (i * kThreads + threadIdx.x) * 4u;

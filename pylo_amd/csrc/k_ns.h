@@ -32,12 +32,14 @@ enum : int { kNsGram = 0, kNsPoly = 1, kNsUpdate = 2 };
 
 struct NsMat {
   int tensor;          // index into the argument table (raw step pointer, flags)
+  int unit;            // the finishing pass's unit whose sum of squares is this matrix's (FinUnit)
   int R, C, m, tall;   // X is R x C row-major; m = min(R, C); tall: R > C
   int n_slabs;         // > 1: the Gram product is split along its reduction
   long long off_x1;    // floats into the workspace: the second X buffer (R x C)
   long long off_a;     // A (m x m)
   long long off_b;     // B' (m x m)
   long long off_part;  // split Gram product: n_slabs partial matrices (m x m each), else unused
+  long long elem_off;  // elements from the tensor's raw step to this matrix (split-bf16 kernels: a slice of a tensor with more dims)
 };
 
 struct NsItem {
@@ -262,14 +264,14 @@ __global__ __launch_bounds__(256) void k_ns_gram_reduce(const NsMat* __restrict_
 
 // s = 1 / (||raw|| + eps) per matrix from the per-block sums of squares of the finishing pass's first kernel.
 __global__ __launch_bounds__(256) void k_ns_scale(const NsMat* __restrict__ mats, int n_mats,
-                                                  const TDesc* __restrict__ descs, const double* __restrict__ fin_part,
+                                                  const FinUnit* __restrict__ units, const double* __restrict__ fin_part,
                                                   float eps, float* __restrict__ scale) {
   __shared__ double red[4];
   const int q = blockIdx.x;
   if (q >= n_mats) return;
-  const TDesc d = descs[mats[q].tensor];
+  const FinUnit d = units[mats[q].unit];
   double s = 0.0;
-  for (int b = threadIdx.x; b < d.fin_nblk; b += 256) s += fin_part[d.fin_blk0 + b];
+  for (int b = threadIdx.x; b < d.nblk; b += 256) s += fin_part[d.blk0 + b];
   s = wave_sum(s);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
   __syncthreads();

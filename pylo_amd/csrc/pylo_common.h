@@ -106,7 +106,7 @@ struct TDesc {
   // the matrix view.
   int aper, aper_col;
   int adam_indep;          // kModeFlat: AdamW on the tensor's own two moments instead of mom[0] / rms
-  int fin_blk0, fin_nblk;  // ELO-CELO2 finishing pass: range of 8192-element blocks (rows of its partials)
+  int fin_unit0, fin_units;  // ELO-CELO2 finishing pass: the tensor's units (FinUnit)
   int slice_len;           // CELO2, N-D or fewer than two dims: elements per slice of the last two dims (or n)
   int nan0;                // gradients pass through torch.nan_to_num (PYLO_F_NAN_TO_NUM)
   int wd_prestep;          // p -= lr * (step + wd * p) against the pre-step parameter (PYLO_F_WD_PRESTEP)
@@ -120,6 +120,16 @@ struct TDesc {
 // index would force the whole struct into scratch memory; a select keeps it in registers.
 template <class T>
 __device__ __forceinline__ T pick(const T (&a)[2], int w) { return w ? a[1] : a[0]; }
+
+// ELO-CELO2 finishing pass: what one normaliser runs over -- a whole tensor, or one slice of the last two dims of a
+// tensor with more dims.
+struct FinUnit {
+  int tensor;
+  int blk0, nblk;   // range of 8192-element blocks (rows of the pass's partial sums)
+  int vec;          // 16-byte accesses: off and n multiples of 4
+  long long off;    // elements from the tensor's start
+  long long n;
+};
 
 struct Item {
   int tensor;

@@ -98,6 +98,8 @@ struct Layout {
   // of the wave-owned and of the block-owned ones
   std::vector<Item> slice_items_l[kSliceLaneSets], slice_items_w, slice_items_b;
   std::vector<int> slice_of_tensor;   // per tensor: index into slice_mats, -1
+  std::vector<FinUnit> fin_units;     // ELO-CELO2 finishing pass: what each normaliser runs over
+  size_t off_fin_units = 0;
   int slice_lds_l[kSliceLaneSets] = {}, slice_lds_w = 0, slice_lds_b = 0;
   size_t off_slice_mats = 0, off_slice_items_l[kSliceLaneSets] = {}, off_slice_items_w = 0, off_slice_items_b = 0;
   int ns_max_m = 0;
@@ -299,30 +301,41 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
   auto take = [&](long long n) { const long long o = ws_floats; ws_floats += (n + 63) / 64 * 64; return o; };
   for (int t = 0; t < T; ++t) {
     const TDesc& d = L.descs[t];
-    if (d.mode != kModeFac2D || d.n == 0 || (shapes[t].flags & PYLO_F_NO_ORTHOGONALIZE)) continue;
+    if (d.n == 0 || (shapes[t].flags & PYLO_F_NO_ORTHOGONALIZE)) continue;
+    // two dims; or more, as one matrix per slice of the last two, where the per-slice launches do not take the
+    // slices (k_slice_finish.h) -- the split-bf16 kernels only, whose tables carry a matrix's place in its tensor
+    const bool slices = d.mode == kModeFacND && L.ns_bf && L.slice_of_tensor[t] < 0 && d.fin_units > 0;
+    if (d.mode != kModeFac2D && !slices) continue;
+    const int R = slices ? (int)shapes[t].shape[shapes[t].ndim - 2] : d.R0;
+    const int C = slices ? (int)shapes[t].shape[shapes[t].ndim - 1] : d.C0;
     // the fp32 kernels load 16 bytes at a time along the contiguous dim of X, A and B'
-    if (!L.ns_bf && (d.C0 % 4 != 0 || std::min(d.R0, d.C0) % 4 != 0)) continue;
+    if (!L.ns_bf && (C % 4 != 0 || std::min(R, C) % 4 != 0)) continue;
+    for (int sl = 0; sl < d.fin_units; ++sl) {
     NsMat mt{};
     mt.tensor = t;
-    mt.R = d.R0; mt.C = d.C0;
-    mt.tall = d.R0 > d.C0;
-    mt.m = std::min(d.R0, d.C0);
+    mt.unit = d.fin_unit0 + sl;
+    mt.elem_off = (long long)sl * R * C;
+    mt.R = R; mt.C = C;
+    mt.tall = R > C;
+    mt.m = std::min(R, C);
     const int K = mt.tall ? mt.R : mt.C;
     mt.n_slabs = K >= kNsSplitMin ? (K + kNsSlabK - 1) / kNsSlabK : 1;
-    mt.off_x1 = take(d.n);
+    mt.off_x1 = take((long long)R * C);
     mt.off_a = take((long long)mt.m * mt.m);
     mt.off_b = take((long long)mt.m * mt.m);
     mt.off_part = mt.n_slabs > 1 ? take((long long)mt.n_slabs * mt.m * mt.m) : 0;
     const int q = (int)L.ns_mats.size();
-    L.ns_of_tensor[t] = q;
-    L.ns_xalt[t] = mt.off_x1;
+    if (sl == 0) {
+      L.ns_of_tensor[t] = q;
+      L.ns_xalt[t] = mt.off_x1;
+    }
     L.ns_max_m = std::max(L.ns_max_m, mt.m);
     const int nt = (mt.m + kNsTile - 1) / kNsTile;
     for (int tm = 0; tm < nt; ++tm)
       for (int tn = tm; tn < nt; ++tn) {
         if (mt.n_slabs > 1) {
-          for (int sl = 0; sl < mt.n_slabs; ++sl)
-            L.ns_gram.push_back(NsItem{q, tm, tn, sl * kNsSlabK, std::min(K, (sl + 1) * kNsSlabK), sl});
+          for (int sb = 0; sb < mt.n_slabs; ++sb)
+            L.ns_gram.push_back(NsItem{q, tm, tn, sb * kNsSlabK, std::min(K, (sb + 1) * kNsSlabK), sb});
         } else {
           L.ns_gram.push_back(NsItem{q, tm, tn, 0, K, -1});
         }
@@ -333,6 +346,7 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       for (int tn = 0; tn < nj; ++tn) L.ns_upd.push_back(NsItem{q, tm, tn, 0, mt.m, -1});
     if (mt.n_slabs > 1) L.ns_split.push_back(q);
     L.ns_mats.push_back(mt);
+    }
   }
   if (L.ns_bf) {
     // same matrices, operands as bf16 planes; the item tables are rebuilt for the uniform (n x m) orientation
@@ -381,7 +395,7 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       b.off_p = take_p(kNsBufs * b.p_stride);
       b.off_a = take((long long)b.m * b.lda);
       b.off_part = b.n_slabs > 1 ? take((long long)b.n_slabs * b.m * b.lda) : 0;
-      b.elem_off = 0;
+      b.elem_off = f.elem_off;
       L.ns_mats[q].off_a = b.off_a;   // the fp32 tables stay consistent for k_ns_scale (tensor index only)
       for (int tr = 0; tr < (b.R + 63) / 64; ++tr)
         for (int tc = 0; tc < (b.C + 63) / 64; ++tc) L.nsb_split_items.push_back(NsTileItem{(int)q, tr, tc});
@@ -529,6 +543,40 @@ void build_slice_tables(Layout& L, const PyloTensorShape* shapes, int T) {
     for (long long b = 0; b < blocks; ++b) items.push_back(Item{q, (int)b, 0, 0});
     L.slice_mats.push_back(sm);
   }
+}
+
+// Units and blocks of ELO-CELO2's finishing pass (after Newton-Schulz): a unit is what one normaliser runs over, cut
+// into linear 8192-element blocks.  MLP tensors of up to two dims are one unit; a tensor with more dims whose slices
+// the per-slice launches do not take (k_slice_finish.h) is one unit per slice of its last two dims.
+int build_fin_tables(Layout& L, const PyloTensorShape* shapes, int T) {
+  L.fin_units.clear(); L.fin_items.clear();
+  for (int t = 0; t < T; ++t) {
+    TDesc& d = L.descs[t];
+    d.fin_unit0 = (int)L.fin_units.size();
+    d.fin_units = 0;
+    if (d.mode == kModeFlat || d.n == 0) continue;
+    long long slices = 1, len = d.n;
+    if (d.mode == kModeFacND) {
+      if (L.slice_of_tensor[t] >= 0) continue;
+      len = shapes[t].shape[shapes[t].ndim - 2] * shapes[t].shape[shapes[t].ndim - 1];
+      slices = d.n / len;
+    }
+    for (long long sl = 0; sl < slices; ++sl) {
+      FinUnit u{};
+      u.tensor = t;
+      u.off = sl * len;
+      u.n = len;
+      u.vec = len % 4 == 0;
+      u.blk0 = (int)L.fin_items.size();
+      const int unit = (int)L.fin_units.size();
+      for (long long c = 0; c * kFinElems < len; ++c) L.fin_items.push_back(Item{unit, (int)c, 0, 0});
+      u.nblk = (int)L.fin_items.size() - u.blk0;
+      L.fin_units.push_back(u);
+    }
+    d.fin_units = (int)slices;
+    if (L.fin_items.size() >= (1u << 30)) return fail("plan: too many blocks in the finishing pass");
+  }
+  return 0;
 }
 
 int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int velo_hidden) {
@@ -701,13 +749,6 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       for (int r = 0; r < d.nblk; r += kSegRows) L.seg_items.push_back(Item{t, r, std::min(kSegRows, d.nblk - r), 0});
       d.nseg = (int)L.seg_items.size() - d.seg0;
     }
-    // blocks of ELO-CELO2's finishing pass (after Newton-Schulz): linear 8192-element pieces of the MLP tensors
-    // (tensors with more dims are finished per slice, k_slice_finish.h)
-    if (kind == PYLO_KIND_CELO2 && d.mode != kModeFlat && d.mode != kModeFacND) {
-      d.fin_blk0 = (int)L.fin_items.size();
-      for (long long c = 0; c * kFinElems < n; ++c) L.fin_items.push_back(Item{t, (int)c, 0, 0});
-      d.fin_nblk = (int)L.fin_items.size() - d.fin_blk0;
-    }
     // blocks of AdafacLO's apply pass: one column per lane where the tensor allows it (ap_items,
     // k_adafac_apply_tile), linear chunks otherwise (ga_items, k_adafac_apply)
     if (kind == PYLO_KIND_ADAFAC) {
@@ -737,6 +778,13 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     }
   }
   if (kind == PYLO_KIND_CELO2 || kind == PYLO_KIND_VELO) build_elem_items(L, T, kind);
+  long long ns_floats = 0;
+  if (kind == PYLO_KIND_CELO2) {
+    L.ns_bf = env_ns_bf();
+    build_slice_tables(L, shapes, T);
+    if (int rc = build_fin_tables(L, shapes, T)) return rc;
+    build_ns_tables(L, shapes, T, ns_floats);
+  }
   size_t off = 0;
   auto take = [&](size_t bytes) {
     size_t o = off;
@@ -761,7 +809,8 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_ga_items = take(sizeof(Item) * L.ga_items.size());
   L.off_fin_items = take(sizeof(Item) * L.fin_items.size());
   L.off_finpart = take(sizeof(double) * L.fin_items.size());
-  L.off_finscale = take(sizeof(float) * T);
+  L.off_finscale = take(sizeof(float) * L.fin_units.size());
+  L.off_fin_units = take(sizeof(FinUnit) * L.fin_units.size());
   L.off_v0a_items = take(sizeof(Item) * L.v0a_items.size());
   L.off_v0b_items = take(sizeof(Item) * L.v0b_items.size());
   L.off_fac_list = take(sizeof(int) * nfac);
@@ -794,9 +843,6 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_piv = take(kind == PYLO_KIND_VELO ? sizeof(float) * 4 * (size_t)T : 0);
   L.off_wmix = take(kind == PYLO_KIND_VELO ? sizeof(float) * 160 * (size_t)T : 0);
   if (kind == PYLO_KIND_CELO2) {
-    long long ns_floats = 0;
-    L.ns_bf = env_ns_bf();
-    build_ns_tables(L, shapes, T, ns_floats);
     L.off_ns_mats = take(sizeof(NsMat) * L.ns_mats.size());
     L.off_ns_gram = take(sizeof(NsItem) * L.ns_gram.size());
     L.off_ns_poly = take(sizeof(NsItem) * L.ns_poly.size());
@@ -809,7 +855,6 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     L.off_nsb_mats = take(sizeof(NsBfMat) * L.nsb_mats.size());
     L.off_nsb_split_items = take(sizeof(NsTileItem) * L.nsb_split_items.size());
     L.off_ns_pw = take(sizeof(bfbits) * (size_t)L.nsb_plane_elems);
-    build_slice_tables(L, shapes, T);
     L.off_slice_mats = take(sizeof(SliceMat) * L.slice_mats.size());
     for (int k = 0; k < kSliceLaneSets; ++k) L.off_slice_items_l[k] = take(sizeof(Item) * L.slice_items_l[k].size());
     L.off_slice_items_w = take(sizeof(Item) * L.slice_items_w.size());
@@ -907,6 +952,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_pp_items, L.pp_items.data(), sizeof(Item) * L.pp_items.size());
   if (e == hipSuccess) e = up(L.off_ga_items, L.ga_items.data(), sizeof(Item) * L.ga_items.size());
   if (e == hipSuccess) e = up(L.off_fin_items, L.fin_items.data(), sizeof(Item) * L.fin_items.size());
+  if (e == hipSuccess) e = up(L.off_fin_units, L.fin_units.data(), sizeof(FinUnit) * L.fin_units.size());
   if (e == hipSuccess) e = up(L.off_fac_list, L.fac_list.data(), sizeof(int) * L.fac_list.size());
   if (e == hipSuccess) e = up(L.off_v0a_items, L.v0a_items.data(), sizeof(Item) * L.v0a_items.size());
   if (e == hipSuccess) e = up(L.off_v0b_items, L.v0b_items.data(), sizeof(Item) * L.v0b_items.size());
@@ -1401,10 +1447,7 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
     const std::string at = " (tensor " + std::to_string(t) + ")";
     if (!a.param || !a.step_out) return fail(w + ": null param/step_out pointer" + at);
     const uintptr_t m = reinterpret_cast<uintptr_t>(a.param) | reinterpret_cast<uintptr_t>(a.step_out);
-    if (d.mode == kModeFacND) {
-      if (L.slice_of_tensor[t] < 0)
-        return fail(w + ": a tensor with more than two dims whose slices of the last two dims do not fit the "
-                    "per-slice pass (pylo_mi355_plan_finish_supported)" + at);
+    if (d.mode == kModeFacND && L.slice_of_tensor[t] >= 0) {
       if (reinterpret_cast<uintptr_t>(a.step_out) % 4 != 0 || reinterpret_cast<uintptr_t>(a.param) % (d.store != 0 ? 2 : 4) != 0)
         return fail(w + ": misaligned pointer" + at);
       if (coeffs && (a.flags & PYLO_ARG_ORTHOGONALIZE) && L.slice_mats[L.slice_of_tensor[t]].no_orth)
@@ -1412,7 +1455,11 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
       any_slices = true;
       continue;
     }
-    if (m % (d.n % 4 == 0 ? 16 : 4) != 0) return fail(w + ": misaligned pointer" + at);
+    const bool vec = d.fin_units > 0 && L.fin_units[d.fin_unit0].vec;
+    if (m % (vec ? 16 : 4) != 0) return fail(w + ": misaligned pointer" + at);
+    if (coeffs && ns_iters == 0 && (a.flags & PYLO_ARG_ORTHOGONALIZE))
+      return fail(w + ": PYLO_ARG_ORTHOGONALIZE with ns_iters = 0 on a tensor that the tiled products orthogonalise "
+                  "(the division by the norm alone is the caller's)" + at);
     if (ns_iters > 0 && (a.flags & PYLO_ARG_ORTHOGONALIZE)) {
       if (L.ns_of_tensor[t] < 0) return fail(w + ": PYLO_ARG_ORTHOGONALIZE on a tensor the library cannot orthogonalise" + at);
       any_ns = true;
@@ -1424,6 +1471,7 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
   const TDesc* descs = P->at<TDesc>(L.off_descs);
   const PyloTensorArgs* dyn = P->at<PyloTensorArgs>(L.off_dyn);
   const Item* fin_items = P->at<Item>(L.off_fin_items);
+  const FinUnit* units = P->at<FinUnit>(L.off_fin_units);
   double* fin_part = P->at<double>(L.off_finpart);
   float* fin_scale = P->at<float>(L.off_finscale);
   const int n_fin = (int)L.fin_items.size();
@@ -1467,9 +1515,9 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
     const int n_mats = (int)L.ns_mats.size(), n_gram = (int)L.ns_gram.size(), n_poly = (int)L.ns_poly.size(),
               n_upd = (int)L.ns_upd.size(), n_split = (int)L.ns_split.size();
     // ||raw||: the finishing pass's sums of squares, taken on the raw steps
-    hipLaunchKernelGGL(k_celo2_sumsq, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_part,
+    hipLaunchKernelGGL(k_celo2_sumsq, dim3(n_fin), dim3(kThreads), 0, s, units, dyn, fin_items, fin_part,
                        (const long long*)nullptr, (const float*)nullptr);
-    hipLaunchKernelGGL(k_ns_scale, dim3(n_mats), dim3(256), 0, s, mats, n_mats, descs, fin_part, ns_eps, scale);
+    hipLaunchKernelGGL(k_ns_scale, dim3(n_mats), dim3(256), 0, s, mats, n_mats, units, fin_part, ns_eps, scale);
     if (L.ns_bf) {
       const NsBfMat* bmats = P->at<NsBfMat>(L.off_nsb_mats);
       const NsTileItem* sitems = P->at<NsTileItem>(L.off_nsb_split_items);
@@ -1554,10 +1602,10 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
     // fp32 kernels: an odd number of iterations leaves the result in the second buffer
     if (!L.ns_bf && (ns_iters & 1)) x_alt = P->at<long long>(L.off_ns_xalt);
   }
-  hipLaunchKernelGGL(k_celo2_sumsq, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_part, x_alt,
+  hipLaunchKernelGGL(k_celo2_sumsq, dim3(n_fin), dim3(kThreads), 0, s, units, dyn, fin_items, fin_part, x_alt,
                      (const float*)ns_ws);
-  hipLaunchKernelGGL(k_celo2_finscale, dim3(P->T), dim3(kThreads), 0, s, descs, dyn, fin_part, fin_scale);
-  hipLaunchKernelGGL(k_celo2_update, dim3(n_fin), dim3(kThreads), 0, s, descs, dyn, fin_items, fin_scale, x_alt,
+  hipLaunchKernelGGL(k_celo2_finscale, dim3((unsigned)L.fin_units.size()), dim3(kThreads), 0, s, units, dyn, fin_part, fin_scale);
+  hipLaunchKernelGGL(k_celo2_update, dim3(n_fin), dim3(kThreads), 0, s, units, descs, dyn, fin_items, fin_scale, x_alt,
                      (const float*)ns_ws);
   HIP_TRY(hipGetLastError());
   return 0;
@@ -1577,15 +1625,12 @@ extern "C" int pylo_mi355_celo2_orthogonalize_finish(PyloPlan* P, const PyloTens
 
 extern "C" int pylo_mi355_plan_finish_supported(const PyloPlan* P, int tensor) {
   if (!P || tensor < 0 || tensor >= P->T || P->kind != PYLO_KIND_CELO2) return 0;
-  const TDesc& d = P->L.descs[tensor];
-  if (d.mode == kModeFlat) return 0;
-  return d.mode != kModeFacND || P->L.slice_of_tensor[tensor] >= 0 ? 1 : 0;
+  return P->L.descs[tensor].mode == kModeFlat ? 0 : 1;
 }
 
 extern "C" int pylo_mi355_plan_orthogonalize_supported(const PyloPlan* P, int tensor) {
   if (!P || tensor < 0 || tensor >= P->T || P->kind != PYLO_KIND_CELO2) return 0;
-  if (P->L.descs[tensor].mode == kModeFacND)
-    return P->L.slice_of_tensor[tensor] >= 0 && !P->L.slice_mats[P->L.slice_of_tensor[tensor]].no_orth ? 1 : 0;
+  if (P->L.slice_of_tensor[tensor] >= 0) return P->L.slice_mats[P->L.slice_of_tensor[tensor]].no_orth ? 0 : 2;
   return P->L.ns_of_tensor[tensor] >= 0 ? 1 : 0;
 }
 

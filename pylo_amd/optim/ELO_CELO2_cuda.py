@@ -263,8 +263,8 @@ class ELO_CELO2_CUDA(Optimizer):
             self._raw_groups.append((buf, idx))
         self._fin_args = np.zeros(len(tensors), dtype=_lib.ARGS_DTYPE)
         self._fin_fast = None
+        # 0: torch products; 1: the library's tiled products (ns_iters > 0); 2: its per-slice launches (any ns_iters)
         self._ns_ok = [self._plan.orthogonalize_supported(i) for i in range(len(tensors))]
-        self._fin_ok = [self._plan.finish_supported(i) for i in range(len(tensors))]
         if self.capturable:
             self._reset_device_steps(tensors)
 
@@ -510,12 +510,9 @@ class ELO_CELO2_CUDA(Optimizer):
             if adam:
                 continue
             orth = bool(group["orthogonalize"]) and p.dim() >= 2
-            if p.dim() > 2:
-                # per slice of the last two dims, all of it in one launch of the library's (any ns_iters)
-                if not self._fin_ok[i] or (orth and not (self._lib_ns and self._ns_ok[i])):
-                    return None
-            # (zero iterations still divide by the Frobenius norm, which the normaliser's epsilon sees: torch path)
-            elif orth and not (self._lib_ns and self._ns_ok[i] and self.ns_iters > 0):
+            # (zero iterations still divide by the Frobenius norm, which the normaliser's epsilon sees: the
+            # per-slice launches do that, the tiled products leave it to torch)
+            if orth and not (self._lib_ns and (self._ns_ok[i] == 2 or (self._ns_ok[i] == 1 and self.ns_iters > 0))):
                 return None
             idx.append(i)
             flags.append(_lib.ARG_ORTHOGONALIZE if orth else 0)
@@ -584,21 +581,14 @@ class ELO_CELO2_CUDA(Optimizer):
                 step = step.mul_(torch.sqrt(sq + 1e-9).view([-1] + [1] * nd))   # the raw steps are scratch
             flag = 0
             # more than two dims: Newton-Schulz and the normaliser are per slice of the last two dims
-            # (ELO_CELO2_naive.py:217-218,235); the library does both where a slice fits its per-slice launch
-            nd_lib = nd > 2 and all(self._fin_ok[i] for i in idx) and (
-                not group["orthogonalize"] or (lib_ns and all(self._ns_ok[i] for i in idx)))
+            # (ELO_CELO2_naive.py:217-218,235), in the library too
             if group["orthogonalize"] and nd >= 2:
-                if nd_lib or (lib_ns and nd == 2 and self.ns_iters > 0 and all(self._ns_ok[i] for i in idx)):
+                ok = min(self._ns_ok[i] for i in idx)
+                if lib_ns and (ok == 2 or (ok == 1 and self.ns_iters > 0)):
                     flag = _lib.ARG_ORTHOGONALIZE
                 else:
                     with _ns_blas():
                         step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
-            if nd > 2 and not nd_lib:
-                # slices too large for the library's per-slice launch
-                step = rms_normalize(step, [-2, -1]) * group["rmsmult"]
-                for j, p in enumerate(ps):
-                    _apply(p, step[j], group["weight_decay"], group["lr"])
-                continue
             step = step.contiguous()
             keep.append(step)
             base, stride = step.data_ptr(), step[0].numel() * 4

@@ -1,8 +1,10 @@
 """Tensors with more than two dims in ``pylo_mi355_celo2_orthogonalize_finish`` / ``pylo_mi355_celo2_finish``:
 Newton-Schulz, the normaliser and the parameter update per slice of the last two dims
-(pylo/optim/CELO2_naive.py:59-73 "over the last two dims"; pylo/optim/ELO_CELO2_naive.py:231-235), each slice
-held in LDS by one lane, a wave or a block.  Against the literal formula in fp64 slice by slice through the
-C-ABI, and through whole optimizer steps against the oracle (parameters at rel 1e-5 / abs 1e-6).
+(pylo/optim/CELO2_naive.py:59-73 "over the last two dims"; pylo/optim/ELO_CELO2_naive.py:231-235).  Small slices
+are held in LDS or registers by one lane, a wave or a block from the raw step to the parameter; larger ones are
+matrices of the tiled products like any 2-D tensor, each with its own norm and normaliser.  Against the literal
+formula in fp64 slice by slice through the C-ABI, and through whole optimizer steps against the oracle
+(parameters at rel 1e-5 / abs 1e-6).
 """
 
 import numpy as np
@@ -20,6 +22,8 @@ SHAPES = [((32, 16, 3, 3), 1), ((6, 4, 1, 1), 1), ((5, 4, 8), 1), ((3, 8, 4), 1)
           ((4, 6, 6), 1), ((70, 7, 7), 1), ((3, 2, 100), 1), ((130, 3, 3), 1),
           ((7, 16, 16), 64), ((2, 3, 4, 70), 64), ((3, 70, 4), 64), ((5, 8, 8), 64),
           ((3, 40, 33), 256), ((2, 64, 128), 256), ((2, 128, 64), 256), ((1, 2, 33, 200), 256)]
+# slices for the tiled products
+LARGE = [(2, 128, 128), (3, 64, 300), (2, 300, 64), (2, 2, 130, 201), (1, 8300, 40)]
 
 
 def _formula(x, iters, dtype=torch.float64, orthogonalise=True):
@@ -45,6 +49,7 @@ def _finish_direct(mats, iters, flag=True, entry="orthogonalize_finish"):
     shapes = [tuple(x.shape) for x in mats]
     plan = _lib.Plan(_lib.KIND_CELO2, shapes, [0] * len(shapes), torch.device("cuda:0"))
     assert all(plan.finish_supported(i) and plan.orthogonalize_supported(i) for i in range(len(mats)))
+    per_slice = [plan.orthogonalize_supported(i) == 2 for i in range(len(mats))]
     steps = [x.clone().contiguous() for x in mats]
     params = [torch.zeros_like(x) for x in mats]
     fin = np.zeros(len(mats), dtype=_lib.ARGS_DTYPE)
@@ -59,8 +64,9 @@ def _finish_direct(mats, iters, flag=True, entry="orthogonalize_finish"):
         plan.celo2_orthogonalize_finish(fin, COEFFS, iters, 1e-8, stream)
     torch.cuda.synchronize()
     plan.close()
-    for x, s in zip(mats, steps):
-        assert torch.equal(x, s)      # the raw step is left as it was
+    for x, s, small in zip(mats, steps, per_slice):
+        if small:
+            assert torch.equal(x, s)      # the per-slice launches leave the raw step as it was
     return params
 
 
@@ -70,7 +76,8 @@ def test_slices_against_the_formula_in_fp64(iters):
     few elements can be nearly singular, where five iterations amplify rounding by up to 3.4445^5: the bar is the
     error of the same formula in fp32 torch products times 1.5, plus 5e-5."""
     gen = torch.Generator(device="cuda").manual_seed(11 + iters)
-    mats = [torch.randn(s, generator=gen, device="cuda") * 10.0 ** (-(i % 4)) for i, (s, _l) in enumerate(SHAPES)]
+    shapes = [s for s, _l in SHAPES] + (LARGE if iters > 0 else [])
+    mats = [torch.randn(s, generator=gen, device="cuda") * 10.0 ** (-(i % 4)) for i, s in enumerate(shapes)]
     got = _finish_direct(mats, iters)
     prev = torch.backends.cuda.matmul.allow_tf32
     torch.backends.cuda.matmul.allow_tf32 = False
@@ -90,7 +97,7 @@ def test_slices_against_the_formula_in_fp64(iters):
 @pytest.mark.parametrize("entry", ["finish", "orthogonalize_finish"])
 def test_slices_without_the_flag_are_normalised_only(entry):
     gen = torch.Generator(device="cuda").manual_seed(3)
-    mats = [torch.randn(s, generator=gen, device="cuda") * 0.1 for s, _l in SHAPES]
+    mats = [torch.randn(s, generator=gen, device="cuda") * 0.1 for s in [s for s, _l in SHAPES] + LARGE]
     # pylo_mi355_celo2_finish ignores the flag; the other entry point honours its absence
     got = _finish_direct(mats, 5, flag=(entry == "finish"), entry=entry)
     for x, y in zip(mats, got):
@@ -98,41 +105,58 @@ def test_slices_without_the_flag_are_normalised_only(entry):
         assert float((y.double() - want).abs().max()) <= 2e-6, tuple(x.shape)
 
 
-def test_lanes_per_slice_and_slices_that_do_not_fit():
+def test_which_kernels_take_a_tensor_and_what_is_refused():
     from pylo_amd import _lib
 
-    shapes = [s for s, _l in SHAPES] + [(2, 128, 128), (3, 64, 300), (64, 64)]
-    plan = _lib.Plan(_lib.KIND_CELO2, shapes, [0] * len(shapes), torch.device("cuda:0"))
-    n = len(SHAPES)
-    assert all(plan.finish_supported(i) for i in range(n))
-    assert not plan.finish_supported(n) and not plan.finish_supported(n + 1) and plan.finish_supported(n + 2)
-    assert not plan.orthogonalize_supported(n) and plan.orthogonalize_supported(n + 2)
+    shapes = [s for s, _l in SHAPES] + LARGE + [(64, 64), (64,)]
+    flags = [0] * (len(shapes) - 1) + [_lib.F_ADAM]
+    plan = _lib.Plan(_lib.KIND_CELO2, shapes, flags, torch.device("cuda:0"))
+    n, k = len(SHAPES), len(LARGE)
+    assert all(plan.finish_supported(i) for i in range(n + k + 1)) and not plan.finish_supported(n + k + 1)
+    assert [plan.orthogonalize_supported(i) for i in range(n + k + 2)] == [2] * n + [1] * k + [1, 0]
+    # zero iterations: the per-slice launches divide by the norm, the tiled products refuse the flag
     x = torch.zeros(2 * 128 * 128, device="cuda")
     fin = np.zeros(len(shapes), dtype=_lib.ARGS_DTYPE)
     fin["grad"][n], fin["param"][n], fin["step_out"][n] = 1, x.data_ptr(), x.data_ptr()
-    with pytest.raises(RuntimeError, match="do not fit"):
-        plan.celo2_orthogonalize_finish(fin, COEFFS, 5, 1e-8, 0)
+    fin["flags"][n] = _lib.ARG_ORTHOGONALIZE
+    with pytest.raises(RuntimeError, match="ns_iters = 0"):
+        plan.celo2_orthogonalize_finish(fin, COEFFS, 0, 1e-8, 0)
     plan.close()
     # a shape flagged as never orthogonalised: finished per slice, the flag refused
-    flags = [_lib.F_NO_ORTHOGONALIZE, 0]
-    plan = _lib.Plan(_lib.KIND_CELO2, [(4, 3, 3), (4, 3, 3)], flags, torch.device("cuda:0"))
-    assert plan.finish_supported(0) and not plan.orthogonalize_supported(0) and plan.orthogonalize_supported(1)
-    fin = np.zeros(2, dtype=_lib.ARGS_DTYPE)
-    fin["grad"][0], fin["param"][0], fin["step_out"][0] = 1, x.data_ptr(), x.data_ptr()
-    fin["flags"][0] = _lib.ARG_ORTHOGONALIZE
-    with pytest.raises(RuntimeError, match="PYLO_F_NO_ORTHOGONALIZE"):
-        plan.celo2_orthogonalize_finish(fin, COEFFS, 5, 1e-8, 0)
+    flags = [_lib.F_NO_ORTHOGONALIZE, 0, _lib.F_NO_ORTHOGONALIZE]
+    plan = _lib.Plan(_lib.KIND_CELO2, [(4, 3, 3), (4, 3, 3), (2, 128, 128)], flags, torch.device("cuda:0"))
+    assert [plan.orthogonalize_supported(i) for i in range(3)] == [0, 2, 0]
+    assert all(plan.finish_supported(i) for i in range(3))
+    for i, msg in ((0, "PYLO_F_NO_ORTHOGONALIZE"), (2, "cannot orthogonalise")):
+        fin = np.zeros(3, dtype=_lib.ARGS_DTYPE)
+        fin["grad"][i], fin["param"][i], fin["step_out"][i] = 1, x.data_ptr(), x.data_ptr()
+        fin["flags"][i] = _lib.ARG_ORTHOGONALIZE
+        with pytest.raises(RuntimeError, match=msg):
+            plan.celo2_orthogonalize_finish(fin, COEFFS, 5, 1e-8, 0)
     plan.close()
+
+
+def test_fp32_matrix_instructions_leave_large_slices_to_the_caller(monkeypatch):
+    """PYLO_MI355_NS_F32=1: the fp32 product kernels take 2-D tensors only; the class orthogonalises large slices
+    with torch products and the library still normalises and applies them per slice."""
+    from pylo_amd import _lib
+
+    monkeypatch.setenv("PYLO_MI355_NS_F32", "1")
+    plan = _lib.Plan(_lib.KIND_CELO2, [(2, 128, 128), (4, 3, 3), (64, 64)], [0, 0, 0], torch.device("cuda:0"))
+    assert [plan.orthogonalize_supported(i) for i in range(3)] == [0, 2, 1]
+    assert all(plan.finish_supported(i) for i in range(3))
+    plan.close()
+    test_whole_steps_against_the_oracle(dict(), True, False)
 
 
 @pytest.mark.parametrize("kw,with_large_slices,cached_table", [
-    (dict(), False, True), (dict(), True, False), (dict(ns_iters=0), False, False),
-    (dict(orthogonalize=False), False, True), (dict(param_scale_mult=True), False, False)])
+    (dict(), False, True), (dict(), True, True), (dict(ns_iters=0), True, False),
+    (dict(orthogonalize=False), True, True), (dict(param_scale_mult=True), False, False)])
 def test_whole_steps_against_the_oracle(kw, with_large_slices, cached_table):
     """ELO_CELO2_CUDA.step() on convolution-shaped tensors next to matrices and vectors, free-running for four
-    steps against the fp64 oracle.  Slices of 128 x 128 do not fit the per-slice launch and stay on torch
-    products.  When the library finishes every tensor itself the finishing table is the cached one (no per-step
-    Python over the tensors); a matrix with zero iterations, large slices or param_scale_mult take the general path.
+    steps against the fp64 oracle, with and without a tensor whose slices go to the tiled products.  When the
+    library finishes every tensor itself the finishing table is the cached one (no per-step Python over the
+    tensors); zero iterations on a matrix or param_scale_mult take the general path.
     lr = 1e-3: among 512 random 3 x 3 slices some are nearly singular, where five iterations amplify the fp32
     rounding of the raw step by up to 3.4445^5 in any fp32 evaluation (the accuracy of the orthogonalised step
     itself is held by test_slices_against_the_formula_in_fp64)."""
@@ -144,7 +168,7 @@ def test_whole_steps_against_the_oracle(kw, with_large_slices, cached_table):
     net = CELO2MLP()
     shapes = [(32, 16, 3, 3), (7, 16, 16), (256, 384), (64,), (3, 40, 33), (2, 64, 128), (6, 4, 1, 1), (5, 4, 8)]
     if with_large_slices:
-        shapes.append((2, 128, 128))
+        shapes += [(2, 128, 128), (3, 64, 300)]
     gen = torch.Generator(device="cuda").manual_seed(21)
     init = [torch.randn(s, generator=gen, device="cuda") * 0.05 for s in shapes]
     ref = [v.double() for v in init]

@@ -106,22 +106,7 @@ def _gram_split(k: int, small: int, batch: int) -> int:
     return 1
 
 
-def rms_normalize(x: torch.Tensor, dims, eps: float = 1e-9) -> torch.Tensor:
-    """x * rsqrt(eps + mean(x^2) over dims) (pylo/optim/CELO2_naive.py:54-56)."""
-    return x * torch.rsqrt(eps + torch.mean(x * x, dim=dims, keepdim=True))
-
-
 _WATCH_ALL = 512   # parameter lists up to this length have every state tensor checked for replacement each step
-
-
-def _apply(p, step, weight_decay, lr):
-    """p <- p - lr (step + wd p) in fp32 on the widened parameter, rounded into p's own dtype
-    (what the library's update kernel does for the tensors it finishes itself)."""
-    if p.dtype == torch.float32:
-        p.add_(step + weight_decay * p, alpha=-lr)
-    else:
-        pf = p.float()
-        p.copy_(pf.add_(step + weight_decay * pf, alpha=-lr))
 
 
 class ELO_CELO2_CUDA(Optimizer):
@@ -557,21 +542,10 @@ class ELO_CELO2_CUDA(Optimizer):
         for buf, idx in self._raw_groups:
             group = tensors[idx[0]][0]
             ps = [tensors[i][1] for i in idx]
-            if any(p.grad is None for p in ps):
-                # a tensor of the bucket sat this step out: one by one
-                for i in idx:
-                    p = tensors[i][1]
-                    if p.grad is None:
-                        continue
-                    step = self._raw[i]
-                    if group["param_scale_mult"]:
-                        pf = p.float()
-                        step = step * torch.sqrt(torch.mean(pf * pf) + 1e-9)
-                    if group["orthogonalize"] and step.dim() >= 2:
-                        with _ns_blas():
-                            step = newton_schulz(step, self.ns_coeffs, self.ns_iters, self.ns_eps)
-                    step = rms_normalize(step, list(range(step.dim()))[-2:]) * group["rmsmult"]
-                    _apply(p, step, group["weight_decay"], group["lr"])
+            # a tensor that sits this step out keeps its row out of the table (its raw step is stale or unset; the
+            # bucket-wide torch operations below run over it and nobody reads the result)
+            present = [p.grad is not None for p in ps]
+            if not any(present):
                 continue
             step = buf
             nd = buf.dim() - 1
@@ -593,6 +567,8 @@ class ELO_CELO2_CUDA(Optimizer):
             keep.append(step)
             base, stride = step.data_ptr(), step[0].numel() * 4
             for j, i in enumerate(idx):
+                if not present[j]:
+                    continue
                 fin["grad"][i] = 1          # "takes part"; the gradient itself is not read
                 fin["param"][i] = ps[j].data_ptr()
                 fin["step_out"][i] = base + j * stride

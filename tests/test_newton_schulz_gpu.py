@@ -204,7 +204,7 @@ def test_groups_without_orthogonalisation_and_with_param_scale():
     _run([(256, 384), (132, 260), (64,)], orthogonalize=False)
     _run([(256, 384), (132, 260), (64,)], param_scale_mult=True)
     _run([(256, 384), (132, 260), (64,)], ns_coeffs=(3.0, -3.2, 1.2), ns_eps=1e-6)
-    # a tensor of a bucket sits a step out: that bucket takes the torch path, the others the library's
+    # a tensor of a bucket sits a step out: its row stays out of the finishing table, the bucket's others go through
     torch.manual_seed(1)
     net = CELO2MLP()
     shapes = [(256, 128), (256, 128), (128, 256)]

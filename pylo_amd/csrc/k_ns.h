@@ -263,12 +263,13 @@ __global__ __launch_bounds__(256) void k_ns_gram_reduce(const NsMat* __restrict_
 }
 
 // s = 1 / (||raw|| + eps) per matrix from the per-block sums of squares of the finishing pass's first kernel.
-__global__ __launch_bounds__(256) void k_ns_scale(const NsMat* __restrict__ mats, int n_mats,
+// (`list`: the matrices of the launch, one block each; nullptr: matrices 0 .. n_mats - 1)
+__global__ __launch_bounds__(256) void k_ns_scale(const NsMat* __restrict__ mats, const int* __restrict__ list, int n_mats,
                                                   const FinUnit* __restrict__ units, const double* __restrict__ fin_part,
                                                   float eps, float* __restrict__ scale) {
   __shared__ double red[4];
-  const int q = blockIdx.x;
-  if (q >= n_mats) return;
+  if ((int)blockIdx.x >= n_mats) return;
+  const int q = list ? list[blockIdx.x] : (int)blockIdx.x;
   const FinUnit d = units[mats[q].unit];
   double s = 0.0;
   for (int b = threadIdx.x; b < d.nblk; b += 256) s += fin_part[d.blk0 + b];

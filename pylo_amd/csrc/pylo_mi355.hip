@@ -75,9 +75,15 @@ bool factored_dims(int kind, const PyloTensorShape& s, int* dc, int* dr) {
 }
 
 // One group of matrices of the split-bf16 Newton-Schulz kernels: its ranges in the job tables.
-struct NsGroup { int gram0, n_gram, poly0, n_poly, upd0, n_upd, upd40, n_upd4, split0, n_split, split_max_m; };
+struct NsGroup {
+  int gram0, n_gram, poly0, n_poly, upd0, n_upd, upd40, n_upd4, split0, n_split, split_max_m;
+  int list0, n_list;       // its matrices (ns_list)
+  int sitem0, n_sitems;    // its tiles of the pass that splits the raw steps into planes
+  int fin0, n_fin;         // its blocks of the finishing pass
+  int unit0, n_units;      // ... and their units
+};
 // One batch of matrices: those whose operand planes share the plane workspace at one time.
-struct NsBatch { int mat0, n_mats, split_item0, n_split_items, group0, n_groups; long long plane_elems; };
+struct NsBatch { int mat0, n_mats, group0, n_groups; long long plane_elems; };
 
 struct Layout {
   std::vector<Item> mx_items;   // ELO-CELO2: statistics and apply items in slab order (k_celo2_elem)
@@ -92,6 +98,10 @@ struct Layout {
   std::vector<int> ns_split;          // matrices whose Gram product is split (k_ns_gram_reduce)
   std::vector<long long> ns_xalt;     // per tensor: offset of its second X buffer, -1 without one
   std::vector<int> ns_of_tensor;      // per tensor: index into ns_mats, -1
+  std::vector<int> ns_group_of_tensor;  // split-bf16 kernels, per tensor: its group (index into ns_groups), -1
+  std::vector<int> ns_list;           // the groups' matrices, group after group
+  int fin_rest0 = 0, n_fin_rest = 0, unit_rest0 = 0, n_unit_rest = 0;   // finishing pass: what belongs to no group
+  size_t off_ns_list = 0;
   // ELO-CELO2: tensors with more than two dims, finished per slice of the last two dims (k_slice_finish.h)
   std::vector<SliceMat> slice_mats;
   // blocks of the lane-owned slices (in registers: 1 x 1, 3 x 3, 5 x 5, 7 x 7; in LDS: up to 12, 28, 64 KB a wave),
@@ -298,22 +308,24 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
   ws_floats = 0;
   L.ns_xalt.assign(T, -1);
   L.ns_of_tensor.assign(T, -1);
+  L.ns_group_of_tensor.assign(T, -1);
   auto take = [&](long long n) { const long long o = ws_floats; ws_floats += (n + 63) / 64 * 64; return o; };
   for (int t = 0; t < T; ++t) {
     const TDesc& d = L.descs[t];
     if (d.n == 0 || (shapes[t].flags & PYLO_F_NO_ORTHOGONALIZE)) continue;
     // two dims; or more, as one matrix per slice of the last two, where the per-slice launches do not take the
     // slices (k_slice_finish.h) -- the split-bf16 kernels only, whose tables carry a matrix's place in its tensor
-    const bool slices = d.mode == kModeFacND && L.ns_bf && L.slice_of_tensor[t] < 0 && d.fin_units > 0;
+    const bool slices = d.mode == kModeFacND && L.ns_bf && L.slice_of_tensor[t] < 0;
     if (d.mode != kModeFac2D && !slices) continue;
     const int R = slices ? (int)shapes[t].shape[shapes[t].ndim - 2] : d.R0;
     const int C = slices ? (int)shapes[t].shape[shapes[t].ndim - 1] : d.C0;
     // the fp32 kernels load 16 bytes at a time along the contiguous dim of X, A and B'
     if (!L.ns_bf && (C % 4 != 0 || std::min(R, C) % 4 != 0)) continue;
-    for (int sl = 0; sl < d.fin_units; ++sl) {
+    const int n_sl = slices ? (int)(d.n / ((long long)R * C)) : 1;
+    for (int sl = 0; sl < n_sl; ++sl) {
     NsMat mt{};
     mt.tensor = t;
-    mt.unit = d.fin_unit0 + sl;
+    mt.unit = sl;        // the finishing pass's tables come later: build_fin_tables adds the tensor's first unit
     mt.elem_off = (long long)sl * R * C;
     mt.R = R; mt.C = C;
     mt.tall = R > C;
@@ -366,6 +378,11 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
     std::vector<int> batch_of;
     L.ns_batches.clear();
     NsBatch batch{};
+    auto mats_of_tensor = [&](size_t q) {
+      size_t e = q;
+      while (e < L.ns_mats.size() && L.ns_mats[e].tensor == L.ns_mats[q].tensor) ++e;
+      return (long long)(e - q);
+    };
     for (size_t q = 0; q < L.ns_mats.size(); ++q) {
       const NsMat& f = L.ns_mats[q];
       NsBfMat b{};
@@ -379,13 +396,15 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       b.lda = up(b.m, 4);
       b.n_slabs = f.n_slabs;
       b.p_stride = (3ll * b.rows_m * b.pad_m + 63) / 64 * 64;
-      const long long need = 3ll * b.rows_m * b.pad_n + 6ll * b.rows_n * b.pad_m + kNsBufs * b.p_stride + 4 * 64;
-      if (pw > 0 && pw + need > budget) {   // this matrix opens the next batch
+      // (the matrices of one tensor -- the slices of one with more than two dims -- stay in one batch)
+      const bool first_of_tensor = q == 0 || L.ns_mats[q - 1].tensor != f.tensor;
+      const long long need = (3ll * b.rows_m * b.pad_n + 6ll * b.rows_n * b.pad_m + kNsBufs * b.p_stride + 4 * 64) *
+                             (first_of_tensor ? mats_of_tensor(q) : 1);
+      if (pw > 0 && first_of_tensor && pw + need > budget) {   // this tensor opens the next batch
         batch.plane_elems = pw;
         L.ns_batches.push_back(batch);
         batch = NsBatch{};
         batch.mat0 = (int)q;
-        batch.split_item0 = (int)L.nsb_split_items.size();
         pw = 0;
         ws_floats = 0;
       }
@@ -397,12 +416,9 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       b.off_part = b.n_slabs > 1 ? take((long long)b.n_slabs * b.m * b.lda) : 0;
       b.elem_off = f.elem_off;
       L.ns_mats[q].off_a = b.off_a;   // the fp32 tables stay consistent for k_ns_scale (tensor index only)
-      for (int tr = 0; tr < (b.R + 63) / 64; ++tr)
-        for (int tc = 0; tc < (b.C + 63) / 64; ++tc) L.nsb_split_items.push_back(NsTileItem{(int)q, tr, tc});
       L.nsb_mats.push_back(b);
       batch_of.push_back((int)L.ns_batches.size());
       batch.n_mats = (int)q + 1 - batch.mat0;
-      batch.n_split_items = (int)L.nsb_split_items.size() - batch.split_item0;
       pw_max = std::max(pw_max, pw);
       ws_max = std::max(ws_max, ws_floats);
     }
@@ -419,19 +435,27 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
     // fill the CUs that the tail of the other's leaves idle.  Matrices are dealt to the groups heaviest first.
     L.ns_groups.clear();
     L.ns_split.clear();
+    L.ns_list.clear();
+    L.nsb_split_items.clear();
     for (NsBatch& bt : L.ns_batches) {
     const int n_groups = std::min<int>(env_ns_groups(), std::max(bt.n_mats / 8, 1));
     std::vector<std::vector<int>> members(n_groups);
     {
-      std::vector<int> order(bt.n_mats);
-      for (int q = 0; q < bt.n_mats; ++q) order[q] = bt.mat0 + q;
-      auto work = [&](int q) { const NsBfMat& b = L.nsb_mats[q]; return (double)b.m * b.m * b.n; };
-      std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return work(x) > work(y); });
+      // (tensor by tensor: the slices of a tensor with more than two dims share a group, which also finishes it)
+      struct Run { int q0, q1; double work; };
+      std::vector<Run> runs;
+      for (int q = bt.mat0; q < bt.mat0 + bt.n_mats; ++q) {
+        const NsBfMat& b = L.nsb_mats[q];
+        const double w = (double)b.m * b.m * b.n;
+        if (!runs.empty() && L.nsb_mats[runs.back().q0].tensor == b.tensor) { runs.back().q1 = q + 1; runs.back().work += w; }
+        else runs.push_back(Run{q, q + 1, w});
+      }
+      std::stable_sort(runs.begin(), runs.end(), [](const Run& x, const Run& y) { return x.work > y.work; });
       std::vector<double> load(n_groups, 0.0);
-      for (int q : order) {
+      for (const Run& r : runs) {
         const int g = (int)(std::min_element(load.begin(), load.end()) - load.begin());
-        members[g].push_back(q);
-        load[g] += work(q);
+        for (int q = r.q0; q < r.q1; ++q) members[g].push_back(q);
+        load[g] += r.work;
       }
       for (auto& mm : members) std::sort(mm.begin(), mm.end());   // neighbours in memory stay neighbours in the tables
     }
@@ -443,8 +467,14 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       std::vector<NsItem> gram, poly, upd, upd4;
       NsGroup grp{};
       grp.split0 = (int)L.ns_split.size();
+      grp.list0 = (int)L.ns_list.size();
+      grp.sitem0 = (int)L.nsb_split_items.size();
       for (int q : members[g]) {
         const NsBfMat& b = L.nsb_mats[q];
+        L.ns_list.push_back(q);
+        L.ns_group_of_tensor[b.tensor] = (int)L.ns_groups.size();
+        for (int tr = 0; tr < (b.R + 63) / 64; ++tr)
+          for (int tc = 0; tc < (b.C + 63) / 64; ++tc) L.nsb_split_items.push_back(NsTileItem{q, tr, tc});
         const bool wide_tiles = b.rows_m % 256 == 0 && up(b.m, 256) <= 1.06 * up(b.m, 128);
         const int nt = (b.m + kNsTile - 1) / kNsTile, n_upper = nt * (nt + 1) / 2;
         // Gram: the tiles of one matrix (of one slab of it) read the same rows of Xs; Poly: the same A
@@ -495,6 +525,8 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       append(L.ns_upd, upd, grp.upd0, grp.n_upd);
       append(L.ns_upd4, upd4, grp.upd40, grp.n_upd4);
       grp.n_split = (int)L.ns_split.size() - grp.split0;
+      grp.n_list = (int)L.ns_list.size() - grp.list0;
+      grp.n_sitems = (int)L.nsb_split_items.size() - grp.sitem0;
       L.ns_groups.push_back(grp);
     }
     }
@@ -547,17 +579,19 @@ void build_slice_tables(Layout& L, const PyloTensorShape* shapes, int T) {
 
 // Units and blocks of ELO-CELO2's finishing pass (after Newton-Schulz): a unit is what one normaliser runs over, cut
 // into linear 8192-element blocks.  MLP tensors of up to two dims are one unit; a tensor with more dims whose slices
-// the per-slice launches do not take (k_slice_finish.h) is one unit per slice of its last two dims.
+// the per-slice launches do not take (k_slice_finish.h) is one unit per slice of its last two dims.  The tables
+// hold the tensors of each group of Newton-Schulz matrices together (a group finishes its own tensors on its own
+// stream), then the tensors of no group.
 int build_fin_tables(Layout& L, const PyloTensorShape* shapes, int T) {
   L.fin_units.clear(); L.fin_items.clear();
-  for (int t = 0; t < T; ++t) {
+  auto add = [&](int t) {
     TDesc& d = L.descs[t];
     d.fin_unit0 = (int)L.fin_units.size();
     d.fin_units = 0;
-    if (d.mode == kModeFlat || d.n == 0) continue;
+    if (d.mode == kModeFlat || d.n == 0) return;
     long long slices = 1, len = d.n;
     if (d.mode == kModeFacND) {
-      if (L.slice_of_tensor[t] >= 0) continue;
+      if (L.slice_of_tensor[t] >= 0) return;
       len = shapes[t].shape[shapes[t].ndim - 2] * shapes[t].shape[shapes[t].ndim - 1];
       slices = d.n / len;
     }
@@ -574,8 +608,25 @@ int build_fin_tables(Layout& L, const PyloTensorShape* shapes, int T) {
       L.fin_units.push_back(u);
     }
     d.fin_units = (int)slices;
+  };
+  for (size_t g = 0; g < L.ns_groups.size(); ++g) {
+    NsGroup& grp = L.ns_groups[g];
+    grp.fin0 = (int)L.fin_items.size();
+    grp.unit0 = (int)L.fin_units.size();
+    for (int t = 0; t < T; ++t)
+      if (L.ns_group_of_tensor[t] == (int)g) add(t);
+    grp.n_fin = (int)L.fin_items.size() - grp.fin0;
+    grp.n_units = (int)L.fin_units.size() - grp.unit0;
     if (L.fin_items.size() >= (1u << 30)) return fail("plan: too many blocks in the finishing pass");
   }
+  L.fin_rest0 = (int)L.fin_items.size();
+  L.unit_rest0 = (int)L.fin_units.size();
+  for (int t = 0; t < T; ++t)
+    if (L.ns_group_of_tensor[t] < 0) add(t);
+  L.n_fin_rest = (int)L.fin_items.size() - L.fin_rest0;
+  L.n_unit_rest = (int)L.fin_units.size() - L.unit_rest0;
+  if (L.fin_items.size() >= (1u << 30)) return fail("plan: too many blocks in the finishing pass");
+  for (NsMat& m : L.ns_mats) m.unit += L.descs[m.tensor].fin_unit0;
   return 0;
 }
 
@@ -782,8 +833,8 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   if (kind == PYLO_KIND_CELO2) {
     L.ns_bf = env_ns_bf();
     build_slice_tables(L, shapes, T);
-    if (int rc = build_fin_tables(L, shapes, T)) return rc;
     build_ns_tables(L, shapes, T, ns_floats);
+    if (int rc = build_fin_tables(L, shapes, T)) return rc;
   }
   size_t off = 0;
   auto take = [&](size_t bytes) {
@@ -854,6 +905,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     L.off_ns_ws = take(sizeof(float) * (size_t)ns_floats);
     L.off_nsb_mats = take(sizeof(NsBfMat) * L.nsb_mats.size());
     L.off_nsb_split_items = take(sizeof(NsTileItem) * L.nsb_split_items.size());
+    L.off_ns_list = take(sizeof(int) * L.ns_list.size());
     L.off_ns_pw = take(sizeof(bfbits) * (size_t)L.nsb_plane_elems);
     L.off_slice_mats = take(sizeof(SliceMat) * L.slice_mats.size());
     for (int k = 0; k < kSliceLaneSets; ++k) L.off_slice_items_l[k] = take(sizeof(Item) * L.slice_items_l[k].size());
@@ -966,6 +1018,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess && kind == PYLO_KIND_CELO2) e = up(L.off_ns_xalt, L.ns_xalt.data(), sizeof(long long) * L.ns_xalt.size());
   if (e == hipSuccess) e = up(L.off_nsb_mats, L.nsb_mats.data(), sizeof(NsBfMat) * L.nsb_mats.size());
   if (e == hipSuccess) e = up(L.off_nsb_split_items, L.nsb_split_items.data(), sizeof(NsTileItem) * L.nsb_split_items.size());
+  if (e == hipSuccess) e = up(L.off_ns_list, L.ns_list.data(), sizeof(int) * L.ns_list.size());
   if (e == hipSuccess) e = up(L.off_slice_mats, L.slice_mats.data(), sizeof(SliceMat) * L.slice_mats.size());
   for (int k = 0; k < kSliceLaneSets; ++k)
     if (e == hipSuccess) e = up(L.off_slice_items_l[k], L.slice_items_l[k].data(), sizeof(Item) * L.slice_items_l[k].size());
@@ -1502,91 +1555,126 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
     HIP_TRY(hipGetLastError());
     return 0;
   }
-  const long long* x_alt = nullptr;
-  float* ns_ws = nullptr;
-  if (any_ns) {
+  // sum of squares, per-unit scale and update over a range of the finishing pass's blocks and units
+  auto finish_range = [&](hipStream_t st, int fin0, int nf, int unit0, int nu, const long long* x_alt, const float* ws) {
+    if (nf == 0) return;
+    hipLaunchKernelGGL(k_celo2_sumsq, dim3(nf), dim3(kThreads), 0, st, units, dyn, fin_items + fin0, fin_part + fin0, x_alt, ws);
+    hipLaunchKernelGGL(k_celo2_finscale, dim3(nu), dim3(kThreads), 0, st, units + unit0, dyn, fin_part, fin_scale + unit0);
+    hipLaunchKernelGGL(k_celo2_update, dim3(nf), dim3(kThreads), 0, st, units, descs, dyn, fin_items + fin0, fin_scale, x_alt, ws);
+  };
+  if (!any_ns) {
+    finish_range(s, 0, n_fin, 0, (int)L.fin_units.size(), nullptr, nullptr);
+  } else if (L.ns_bf) {
+    // The split-bf16 kernels.  Every group of matrices is a chain of its own from the norms of its raw steps to the
+    // update of its parameters, on a stream of its own (the first group on the caller's): the memory-bound ends of
+    // one chain run under the matrix products of the others.
+    const NsMat* mats = P->at<NsMat>(L.off_ns_mats);
+    const NsItem* gram = P->at<NsItem>(L.off_ns_gram);
+    const NsItem* poly = P->at<NsItem>(L.off_ns_poly);
+    const NsItem* upd = P->at<NsItem>(L.off_ns_upd);
+    const NsItem* upd4 = P->at<NsItem>(L.off_ns_upd4);
+    const int* split = P->at<int>(L.off_ns_split);
+    const int* list = P->at<int>(L.off_ns_list);
+    float* scale = P->at<float>(L.off_ns_scale);
+    float* ns_ws = P->at<float>(L.off_ns_ws);
+    const NsBfMat* bmats = P->at<NsBfMat>(L.off_nsb_mats);
+    const NsTileItem* sitems = P->at<NsTileItem>(L.off_nsb_split_items);
+    bfbits* pw = P->at<bfbits>(L.off_ns_pw);
+    if (int rc = ns_bf_lds_once()) return rc;
+    finish_range(s, L.fin_rest0, L.n_fin_rest, L.unit_rest0, L.n_unit_rest, nullptr, nullptr);   // tensors of no group
+    const bool several = L.ns_batches.size() > 1;
+    const float c0 = coeffs[0], c1 = coeffs[1], c2 = coeffs[2];
+    const bool pairs = env_ns_pairs();
+    for (const NsBatch& bt : L.ns_batches) {
+      // the planes' padding: zero from plan creation on when one batch has the memory to itself
+      if (several) {
+        const size_t n16 = (size_t)bt.plane_elems * sizeof(bfbits) / 16;
+        hipLaunchKernelGGL(k_ns_zero, dim3((unsigned)std::min<size_t>((n16 + 255) / 256, 1u << 16)), dim3(256), 0, s,
+                           reinterpret_cast<u32x4*>(pw), n16);
+      }
+      const int n_groups = bt.n_groups;
+      auto stream_of = [&](int g) { return g == 0 ? s : P->ns_side[g - 1]; };
+      if (n_groups > 1) {
+        HIP_TRY(hipEventRecord(P->ns_fork, s));
+        for (int g = 1; g < n_groups; ++g) HIP_TRY(hipStreamWaitEvent(P->ns_side[g - 1], P->ns_fork, 0));
+      }
+      for (int g = 0; g < n_groups; ++g) {
+        // ||raw|| per matrix (the finishing pass's sums of squares, taken on the raw steps), then the planes
+        const NsGroup& G = L.ns_groups[bt.group0 + g];
+        hipStream_t sg = stream_of(g);
+        if (G.n_fin > 0)
+          hipLaunchKernelGGL(k_celo2_sumsq, dim3(G.n_fin), dim3(kThreads), 0, sg, units, dyn, fin_items + G.fin0,
+                             fin_part + G.fin0, (const long long*)nullptr, (const float*)nullptr);
+        if (G.n_list > 0)
+          hipLaunchKernelGGL(k_ns_scale, dim3(G.n_list), dim3(256), 0, sg, mats, list + G.list0, G.n_list, units, fin_part,
+                             ns_eps, scale);
+        if (G.n_sitems > 0)
+          hipLaunchKernelGGL(k_ns_bf_split, dim3((unsigned)G.n_sitems), dim3(256), 0, sg, bmats, sitems + G.sitem0, dyn,
+                             (const float*)scale, pw);
+      }
+      int par = 0;   // which Xl buffer the next update reads
+      for (int it = 0; it < ns_iters;) {
+        // two iterations as one Gram product, four m x m products and one update (k_ns_bf.h), or one iteration
+        const bool pair = pairs && it + 1 < ns_iters;
+        const int last = (it + (pair ? 2 : 1)) == ns_iters;
+        for (int g = 0; g < n_groups; ++g) {
+          const NsGroup& G = L.ns_groups[bt.group0 + g];
+          hipStream_t sg = stream_of(g);
+          auto small = [&](auto kern, NsBufs b) {
+            if (G.n_poly > 0)
+              hipLaunchKernelGGL(kern, dim3(G.n_poly), dim3(256), bf_gemm_lds(2), sg, bmats, poly + G.poly0, dyn, ns_ws, pw,
+                                 par, last, b, c0, c1, c2);
+          };
+          if (G.n_gram > 0)
+            hipLaunchKernelGGL((k_ns_bf_gemm<kNsGram, 2>), dim3(G.n_gram), dim3(256), bf_gemm_lds(2), sg, bmats,
+                               gram + G.gram0, dyn, ns_ws, pw, par, last, NsBufs{0, 0, kNsBufA}, c0, c1, c2);
+          if (G.n_split > 0)
+            hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)G.split_max_m * G.split_max_m + 255) / 256, G.n_split),
+                               dim3(256), 0, sg, bmats, split + G.split0, dyn, ns_ws, pw);
+          small(k_ns_bf_gemm<kNsPoly, 2>, NsBufs{kNsBufA, kNsBufA, kNsBufB});            // B'_t
+          int bq = kNsBufB;
+          if (pair) {
+            small(k_ns_bf_gemm<kNsProd, 2>, NsBufs{kNsBufA, kNsBufB, kNsBufT});          // T = A_t B'_t
+            small(k_ns_bf_gemm<kNsProdA, 2>, NsBufs{kNsBufB, kNsBufT, kNsBufA});         // A_{t+1} = B'_t T
+            small(k_ns_bf_gemm<kNsPoly, 2>, NsBufs{kNsBufA, kNsBufA, kNsBufC});          // B'_{t+1}
+            small(k_ns_bf_gemm<kNsProd, 2>, NsBufs{kNsBufC, kNsBufB, kNsBufT});          // Q = B'_{t+1} B'_t
+            bq = kNsBufT;
+          }
+          if (G.n_upd4 > 0)
+            hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 4>), dim3(G.n_upd4), dim3(256), bf_gemm_lds(4), sg, bmats,
+                               upd4 + G.upd40, dyn, ns_ws, pw, par, last, NsBufs{bq, 0, 0}, c0, c1, c2);
+          if (G.n_upd > 0)
+            hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 2>), dim3(G.n_upd), dim3(256), bf_gemm_lds(2), sg, bmats,
+                               upd + G.upd0, dyn, ns_ws, pw, par, last, NsBufs{bq, 0, 0}, c0, c1, c2);
+        }
+        par ^= 1;
+        it += pair ? 2 : 1;
+      }
+      for (int g = 0; g < n_groups; ++g) {
+        const NsGroup& G = L.ns_groups[bt.group0 + g];
+        finish_range(stream_of(g), G.fin0, G.n_fin, G.unit0, G.n_units, nullptr, nullptr);
+      }
+      for (int g = 1; g < n_groups; ++g) {
+        HIP_TRY(hipEventRecord(P->ns_join[g - 1], P->ns_side[g - 1]));
+        HIP_TRY(hipStreamWaitEvent(s, P->ns_join[g - 1], 0));
+      }
+    }
+  } else {
+    // The fp32 matrix instructions: one chain for all matrices.
     const NsMat* mats = P->at<NsMat>(L.off_ns_mats);
     const NsItem* gram = P->at<NsItem>(L.off_ns_gram);
     const NsItem* poly = P->at<NsItem>(L.off_ns_poly);
     const NsItem* upd = P->at<NsItem>(L.off_ns_upd);
     const int* split = P->at<int>(L.off_ns_split);
     float* scale = P->at<float>(L.off_ns_scale);
-    ns_ws = P->at<float>(L.off_ns_ws);
+    float* ns_ws = P->at<float>(L.off_ns_ws);
     const int n_mats = (int)L.ns_mats.size(), n_gram = (int)L.ns_gram.size(), n_poly = (int)L.ns_poly.size(),
               n_upd = (int)L.ns_upd.size(), n_split = (int)L.ns_split.size();
     // ||raw||: the finishing pass's sums of squares, taken on the raw steps
     hipLaunchKernelGGL(k_celo2_sumsq, dim3(n_fin), dim3(kThreads), 0, s, units, dyn, fin_items, fin_part,
                        (const long long*)nullptr, (const float*)nullptr);
-    hipLaunchKernelGGL(k_ns_scale, dim3(n_mats), dim3(256), 0, s, mats, n_mats, units, fin_part, ns_eps, scale);
-    if (L.ns_bf) {
-      const NsBfMat* bmats = P->at<NsBfMat>(L.off_nsb_mats);
-      const NsTileItem* sitems = P->at<NsTileItem>(L.off_nsb_split_items);
-      bfbits* pw = P->at<bfbits>(L.off_ns_pw);
-      const NsItem* upd4 = P->at<NsItem>(L.off_ns_upd4);
-      if (int rc = ns_bf_lds_once()) return rc;
-      const bool several = L.ns_batches.size() > 1;
-      for (const NsBatch& bt : L.ns_batches) {
-        // the planes' padding: zero from plan creation on when one batch has the memory to itself
-        if (several) {
-          const size_t n16 = (size_t)bt.plane_elems * sizeof(bfbits) / 16;
-          hipLaunchKernelGGL(k_ns_zero, dim3((unsigned)std::min<size_t>((n16 + 255) / 256, 1u << 16)), dim3(256), 0, s,
-                             reinterpret_cast<u32x4*>(pw), n16);
-        }
-        hipLaunchKernelGGL(k_ns_bf_split, dim3((unsigned)bt.n_split_items), dim3(256), 0, s, bmats, sitems + bt.split_item0,
-                           dyn, (const float*)scale, pw);
-        // every group of matrices on a stream of its own, the first on the caller's
-        const int n_groups = bt.n_groups;
-        if (n_groups > 1 && ns_iters > 0) {
-          HIP_TRY(hipEventRecord(P->ns_fork, s));
-          for (int g = 1; g < n_groups; ++g) HIP_TRY(hipStreamWaitEvent(P->ns_side[g - 1], P->ns_fork, 0));
-        }
-        const float c0 = coeffs[0], c1 = coeffs[1], c2 = coeffs[2];
-        const bool pairs = env_ns_pairs();
-        int par = 0;   // which Xl buffer the next update reads
-        for (int it = 0; it < ns_iters;) {
-          // two iterations as one Gram product, four m x m products and one update (k_ns_bf.h), or one iteration
-          const bool pair = pairs && it + 1 < ns_iters;
-          const int last = (it + (pair ? 2 : 1)) == ns_iters;
-          for (int g = 0; g < n_groups; ++g) {
-            const NsGroup& G = L.ns_groups[bt.group0 + g];
-            hipStream_t sg = g == 0 ? s : P->ns_side[g - 1];
-            auto small = [&](auto kern, NsBufs b) {
-              if (G.n_poly > 0)
-                hipLaunchKernelGGL(kern, dim3(G.n_poly), dim3(256), bf_gemm_lds(2), sg, bmats, poly + G.poly0, dyn, ns_ws, pw,
-                                   par, last, b, c0, c1, c2);
-            };
-            if (G.n_gram > 0)
-              hipLaunchKernelGGL((k_ns_bf_gemm<kNsGram, 2>), dim3(G.n_gram), dim3(256), bf_gemm_lds(2), sg, bmats,
-                                 gram + G.gram0, dyn, ns_ws, pw, par, last, NsBufs{0, 0, kNsBufA}, c0, c1, c2);
-            if (G.n_split > 0)
-              hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)G.split_max_m * G.split_max_m + 255) / 256, G.n_split),
-                                 dim3(256), 0, sg, bmats, split + G.split0, dyn, ns_ws, pw);
-            small(k_ns_bf_gemm<kNsPoly, 2>, NsBufs{kNsBufA, kNsBufA, kNsBufB});            // B'_t
-            int bq = kNsBufB;
-            if (pair) {
-              small(k_ns_bf_gemm<kNsProd, 2>, NsBufs{kNsBufA, kNsBufB, kNsBufT});          // T = A_t B'_t
-              small(k_ns_bf_gemm<kNsProdA, 2>, NsBufs{kNsBufB, kNsBufT, kNsBufA});         // A_{t+1} = B'_t T
-              small(k_ns_bf_gemm<kNsPoly, 2>, NsBufs{kNsBufA, kNsBufA, kNsBufC});          // B'_{t+1}
-              small(k_ns_bf_gemm<kNsProd, 2>, NsBufs{kNsBufC, kNsBufB, kNsBufT});          // Q = B'_{t+1} B'_t
-              bq = kNsBufT;
-            }
-            if (G.n_upd4 > 0)
-              hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 4>), dim3(G.n_upd4), dim3(256), bf_gemm_lds(4), sg, bmats,
-                                 upd4 + G.upd40, dyn, ns_ws, pw, par, last, NsBufs{bq, 0, 0}, c0, c1, c2);
-            if (G.n_upd > 0)
-              hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 2>), dim3(G.n_upd), dim3(256), bf_gemm_lds(2), sg, bmats,
-                                 upd + G.upd0, dyn, ns_ws, pw, par, last, NsBufs{bq, 0, 0}, c0, c1, c2);
-          }
-          par ^= 1;
-          it += pair ? 2 : 1;
-        }
-        if (n_groups > 1 && ns_iters > 0)
-          for (int g = 1; g < n_groups; ++g) {
-            HIP_TRY(hipEventRecord(P->ns_join[g - 1], P->ns_side[g - 1]));
-            HIP_TRY(hipStreamWaitEvent(s, P->ns_join[g - 1], 0));
-          }
-      }
-    } else
+    hipLaunchKernelGGL(k_ns_scale, dim3(n_mats), dim3(256), 0, s, mats, (const int*)nullptr, n_mats, units, fin_part, ns_eps,
+                       scale);
     for (int it = 0; it < ns_iters; ++it) {
       const int first = it == 0, par = it & 1;
       hipLaunchKernelGGL(k_ns_gemm<kNsGram>, dim3(n_gram), dim3(256), 0, s, mats, gram, dyn, ns_ws, scale, first, par,
@@ -1599,14 +1687,10 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
       hipLaunchKernelGGL(k_ns_gemm<kNsUpdate>, dim3(n_upd), dim3(256), 0, s, mats, upd, dyn, ns_ws, scale, first, par,
                          coeffs[0], coeffs[1], coeffs[2]);
     }
-    // fp32 kernels: an odd number of iterations leaves the result in the second buffer
-    if (!L.ns_bf && (ns_iters & 1)) x_alt = P->at<long long>(L.off_ns_xalt);
+    // an odd number of iterations leaves the result in the second buffer
+    const long long* x_alt = (ns_iters & 1) ? P->at<long long>(L.off_ns_xalt) : nullptr;
+    finish_range(s, 0, n_fin, 0, (int)L.fin_units.size(), x_alt, ns_ws);
   }
-  hipLaunchKernelGGL(k_celo2_sumsq, dim3(n_fin), dim3(kThreads), 0, s, units, dyn, fin_items, fin_part, x_alt,
-                     (const float*)ns_ws);
-  hipLaunchKernelGGL(k_celo2_finscale, dim3((unsigned)L.fin_units.size()), dim3(kThreads), 0, s, units, dyn, fin_part, fin_scale);
-  hipLaunchKernelGGL(k_celo2_update, dim3(n_fin), dim3(kThreads), 0, s, units, descs, dyn, fin_items, fin_scale, x_alt,
-                     (const float*)ns_ws);
   HIP_TRY(hipGetLastError());
   return 0;
 }

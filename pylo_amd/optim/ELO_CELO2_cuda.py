@@ -234,7 +234,7 @@ class ELO_CELO2_CUDA(Optimizer):
         self._plan = _lib.Plan(_lib.KIND_CELO2, shapes, flags, self.device)
         self._plan_key = key
         # Raw steps of the MLP tensors: tensors of one parameter group and one shape share a
-        # contiguous (count, *shape) buffer, so Newton-Schulz and the normalisation run batched.
+        # contiguous (count, *shape) buffer (what the torch products of Newton-Schulz run batched over).
         buckets = {}
         for i, (group, p, adam) in enumerate(tensors):
             if not adam:
@@ -474,14 +474,15 @@ class ELO_CELO2_CUDA(Optimizer):
         (pylo/optim/ELO_CELO2_cuda.py:288-296).  Matrices are orthogonalised by the library's own matrix-pipe
         kernels inside the finishing call (fp32 accuracy on the bf16 matrix instructions, any two dims; with
         ``PYLO_MI355_NS_F32=1`` the fp32 matrix instructions, dims that are multiples of 4); tensors with more
-        than two dims and buckets in which a tensor sat the step out go through the batched torch products
-        (also everything with ``PYLO_MI355_NS=torch`` in the environment, for comparisons)."""
+        than two dims slice by slice of their last two dims, small slices in launches that hold a slice in
+        registers or LDS, large ones as matrices of the same products.  Batched torch products remain for what the
+        library leaves to the caller (zero iterations on a matrix, the fp32 instructions' other shapes) and for
+        everything with ``PYLO_MI355_NS=torch`` in the environment, for comparisons."""
         self._finish_step(tensors)
 
     # The finishing call's table has one row per tensor as well.  When the step went through the cached rows of
-    # the fused call (every tensor has a gradient) and the library finishes every MLP tensor itself (no tensor
-    # with slices too large for the per-slice launch, no param_scale_mult, no torch products), its static columns are kept too and a
-    # step refreshes parameter pointers and the groups' scalars with a few array operations, whatever the
+    # the fused call (every tensor has a gradient) and the library finishes every MLP tensor itself (no
+    # param_scale_mult, no torch products), its static columns are kept too and a step refreshes parameter pointers and the groups' scalars with a few array operations, whatever the
     # number of tensors.
     def _fin_fast_key(self):
         return (self.ns_iters, self._lib_ns,

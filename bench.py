@@ -144,20 +144,33 @@ def ns_flops(shapes, iters=5):
     return total
 
 
+def ns_chains(iters):
+    """The chain lengths the library uses for `iters` iterations (pylo_mi355.hip, ns_chains): pairs by default,
+    PYLO_MI355_NS_CHAINS / PYLO_MI355_NS_PAIRS=0 in the environment, chains of one on the fp32 kernels."""
+    if os.environ.get("PYLO_MI355_NS_PAIRS", "1") == "0" or os.environ.get("PYLO_MI355_NS_F32") == "1":
+        return [1] * iters
+    try:
+        given = [int(v) for v in os.environ.get("PYLO_MI355_NS_CHAINS", "").split(",") if v]
+    except ValueError:
+        given = []
+    if given and min(given) >= 1 and sum(given) == iters:
+        return given
+    return [2] * (iters // 2) + [1] * (iters % 2)
+
+
 def ns_flops_executed(shapes, iters=5, tile=128):
     """FLOPs (fp32 multiply-adds x 2) that the library's kernels execute: symmetric m x m results on the tiles on
-    and above the diagonal only, and, unless PYLO_MI355_NS_PAIRS=0 (or the fp32 kernels are selected), two
-    iterations sharing one Gram product and one update: per pair one Gram product, five m x m products
-    (2 x Poly, 2 x Prod, ProdA) and one update; an unpaired iteration one Gram product, Poly and one update."""
-    pairs = os.environ.get("PYLO_MI355_NS_PAIRS", "1") != "0" and os.environ.get("PYLO_MI355_NS_F32") != "1"
-    n_pairs, singles = (iters // 2, iters % 2) if pairs else (0, iters)
+    and above the diagonal only, and iterations in chains that share one Gram product and one update: a chain of L
+    iterations is one Gram product, 4 L - 3 products of m x m matrices (L x Poly, 2 (L - 1) x Prod, (L - 1) x
+    ProdA) and one update."""
+    chains = ns_chains(iters)
     total = 0.0
     for s in shapes:
         if len(s) == 2:
             m, n = min(s), max(s)
             nt = -(-m // tile)
             upper = nt * (nt + 1) / 2 * tile * tile
-            total += (n_pairs + singles) * (2.0 * upper * n + 2.0 * m * m * n) + (5 * n_pairs + singles) * 2.0 * upper * m
+            total += len(chains) * (2.0 * upper * n + 2.0 * m * m * n) + sum(4 * L - 3 for L in chains) * 2.0 * upper * m
     return total
 
 

@@ -238,7 +238,8 @@ int pylo_mi355_plan_finish_supported(const PyloPlan* plan, int tensor);
  * sum of three bf16 numbers, six bf16 products per fp32 product, fp32 accumulation; what is dropped is below
  * 2^-24 of a product; two iterations share one Gram product and one update, A' = B' A B' and
  * X'' = (B'' B') X, which costs about 1e-6 of B' in accuracy whatever the spectrum of X -- PYLO_MI355_NS_PAIRS=0
- * in the environment keeps one of each per iteration), with PYLO_MI355_NS_F32=1 in the environment at plan
+ * in the environment keeps one of each per iteration, PYLO_MI355_NS_CHAINS="3,2" lets three and then two
+ * iterations share them, faster and up to ten times less accurate), with PYLO_MI355_NS_F32=1 in the environment at plan
  * creation on the fp32 matrix instructions; then every tensor is normalised and applied as by pylo_mi355_celo2_finish (tensors without the
  * flag from `step_out` as it stands).  `step_out` of a flagged tensor is overwritten (with the orthogonalised
  * step).  A tensor can carry the flag when pylo_mi355_plan_orthogonalize_supported says so: two dims (any two;

@@ -24,10 +24,12 @@
 // What it costs in accuracy is bounded whatever the spectrum of X: A_t as computed is off by eps ||A_t|| in
 // absolute terms, which A_{t+1} = B'_t A_t B'_t inherits relative to its small eigenvalues -- they grow by
 // p(0)^2 = c0^2 in the step, so the error of p(A_{t+1}) in those directions is c1 c0^2 eps sigma_max^2, about
-// 12 times that of p of a freshly formed Gram matrix and about 1e-6 of B' itself; a second chained step would
-// multiply it by c0^2 again, which is why only pairs are merged and the next pair starts from a Gram product
-// of the X it was handed.  PYLO_MI355_NS_PAIRS=0 in the environment keeps one Gram product and one update
-// per iteration.
+// 12 times that of p of a freshly formed Gram matrix and about 1e-6 of B' itself; a second chained step
+// multiplies it by c0^2 again, which is why pairs are the default and the next pair starts from a Gram product
+// of the X it was handed.  The host enqueues chains of any length L (one Gram product, 4 L - 3 products of
+// m x m matrices rotating through four plane buffers, one update): PYLO_MI355_NS_CHAINS="3,2" in the environment
+// trades accuracy for time (1.3e-4 of the result's RMS on a dominant direction over a flat rest, where pairs
+// are at 1e-5), PYLO_MI355_NS_PAIRS=0 keeps one Gram product and one update per iteration.
 //
 // Tile job: 128 x 128 (Gram, Poly, narrow updates) or 128 x 256 outputs (updates with m > 128) by 256 threads =
 // 2 x 2 waves of 64 x 64 / 64 x 128 = 2 x 2 / 2 x 4 accumulators of 32 x 32; 16 reduction steps per stage,

@@ -261,11 +261,40 @@ long long env_ns_budget_elems() {
   return std::max(1ll, mb) * (1ll << 20) / 2;
 }
 
-// PYLO_MI355_NS_PAIRS=0: one Gram product and one update per Newton-Schulz iteration, as the formula is written,
-// instead of one of each per pair of iterations (k_ns_bf.h); read when the products are enqueued.
-bool env_ns_pairs() {
-  const char* e = getenv("PYLO_MI355_NS_PAIRS");
-  return !(e && e[0] == '0');
+// How the Newton-Schulz iterations share their products over the long dim (k_ns_bf.h): a chain of L iterations takes
+// one Gram product, one update and 4 L - 3 products of m x m matrices.  PYLO_MI355_NS_CHAINS="2,3" gives the chain
+// lengths in order (they must add up to the iteration count, else the default applies); PYLO_MI355_NS_PAIRS=0 means
+// chains of one: one Gram product and one update per iteration, as the formula is written.  Read when the products
+// are enqueued.
+std::vector<int> ns_chains(int iters) {
+  std::vector<int> out;
+  const char* p = getenv("PYLO_MI355_NS_PAIRS");
+  if (p && p[0] == '0') {
+    out.assign(iters, 1);
+    return out;
+  }
+  if (const char* e = getenv("PYLO_MI355_NS_CHAINS")) {
+    int sum = 0;
+    for (const char* c = e; *c;) {
+      const int v = atoi(c);
+      if (v < 1) break;
+      out.push_back(v);
+      sum += v;
+      while (*c && *c != ',') ++c;
+      if (*c == ',') ++c;
+    }
+    if (sum == iters) return out;
+    out.clear();
+  }
+  // default: pairs (five iterations: 2, 2, 1).  Longer chains are faster and less accurate: "3,2" takes the
+  // GPT-2-small step from 9.45 to 8.2 ms and stays at the formula's own fp32 error on most inputs, but reaches 1.3e-4
+  // of the result's RMS (against 1e-5 for pairs) on matrices with a dominant direction over a flat rest.
+  for (int left = iters; left > 0;) {
+    const int l = std::min(left, 2);
+    out.push_back(l);
+    left -= l;
+  }
+  return out;
 }
 
 bool env_ns_bf() {
@@ -1584,7 +1613,7 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
     finish_range(s, L.fin_rest0, L.n_fin_rest, L.unit_rest0, L.n_unit_rest, nullptr, nullptr);   // tensors of no group
     const bool several = L.ns_batches.size() > 1;
     const float c0 = coeffs[0], c1 = coeffs[1], c2 = coeffs[2];
-    const bool pairs = env_ns_pairs();
+    const std::vector<int> chains = ns_chains(ns_iters);
     for (const NsBatch& bt : L.ns_batches) {
       // the planes' padding: zero from plan creation on when one batch has the memory to itself
       if (several) {
@@ -1613,10 +1642,12 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
                              (const float*)scale, pw);
       }
       int par = 0;   // which Xl buffer the next update reads
-      for (int it = 0; it < ns_iters;) {
-        // two iterations as one Gram product, four m x m products and one update (k_ns_bf.h), or one iteration
-        const bool pair = pairs && it + 1 < ns_iters;
-        const int last = (it + (pair ? 2 : 1)) == ns_iters;
+      int done = 0;
+      for (size_t ch = 0; ch < chains.size(); ++ch) {
+        // a chain of iterations: one Gram product, 4 len - 3 products of m x m matrices and one update (k_ns_bf.h)
+        const int len = chains[ch];
+        done += len;
+        const int last = done == ns_iters;
         for (int g = 0; g < n_groups; ++g) {
           const NsGroup& G = L.ns_groups[bt.group0 + g];
           hipStream_t sg = stream_of(g);
@@ -1631,24 +1662,30 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
           if (G.n_split > 0)
             hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)G.split_max_m * G.split_max_m + 255) / 256, G.n_split),
                                dim3(256), 0, sg, bmats, split + G.split0, dyn, ns_ws, pw);
+          // A lives in buffer A throughout; B' of the latest iteration in `bprev`, the product of all B' so far in `q`
           small(k_ns_bf_gemm<kNsPoly, 2>, NsBufs{kNsBufA, kNsBufA, kNsBufB});            // B'_t
-          int bq = kNsBufB;
-          if (pair) {
-            small(k_ns_bf_gemm<kNsProd, 2>, NsBufs{kNsBufA, kNsBufB, kNsBufT});          // T = A_t B'_t
-            small(k_ns_bf_gemm<kNsProdA, 2>, NsBufs{kNsBufB, kNsBufT, kNsBufA});         // A_{t+1} = B'_t T
-            small(k_ns_bf_gemm<kNsPoly, 2>, NsBufs{kNsBufA, kNsBufA, kNsBufC});          // B'_{t+1}
-            small(k_ns_bf_gemm<kNsProd, 2>, NsBufs{kNsBufC, kNsBufB, kNsBufT});          // Q = B'_{t+1} B'_t
-            bq = kNsBufT;
+          int bprev = kNsBufB, q = kNsBufB;
+          for (int j = 1; j < len; ++j) {
+            int free_buf[2], nf = 0;
+            for (int b : {kNsBufB, kNsBufT, kNsBufC})
+              if (b != bprev && b != q && nf < 2) free_buf[nf++] = b;
+            const int t = free_buf[0];
+            small(k_ns_bf_gemm<kNsProd, 2>, NsBufs{kNsBufA, bprev, t});                  // T = A B'
+            small(k_ns_bf_gemm<kNsProdA, 2>, NsBufs{bprev, t, kNsBufA});                 // A <- B' T = B' A B'
+            small(k_ns_bf_gemm<kNsPoly, 2>, NsBufs{kNsBufA, kNsBufA, t});                // the next B'
+            const int qn = q == bprev ? free_buf[1] : bprev;                           // (the old B' is done with)
+            small(k_ns_bf_gemm<kNsProd, 2>, NsBufs{t, q, qn});                           // Q <- B' Q
+            bprev = t;
+            q = qn;
           }
           if (G.n_upd4 > 0)
             hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 4>), dim3(G.n_upd4), dim3(256), bf_gemm_lds(4), sg, bmats,
-                               upd4 + G.upd40, dyn, ns_ws, pw, par, last, NsBufs{bq, 0, 0}, c0, c1, c2);
+                               upd4 + G.upd40, dyn, ns_ws, pw, par, last, NsBufs{q, 0, 0}, c0, c1, c2);
           if (G.n_upd > 0)
             hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 2>), dim3(G.n_upd), dim3(256), bf_gemm_lds(2), sg, bmats,
-                               upd + G.upd0, dyn, ns_ws, pw, par, last, NsBufs{bq, 0, 0}, c0, c1, c2);
+                               upd + G.upd0, dyn, ns_ws, pw, par, last, NsBufs{q, 0, 0}, c0, c1, c2);
         }
         par ^= 1;
-        it += pair ? 2 : 1;
       }
       for (int g = 0; g < n_groups; ++g) {
         const NsGroup& G = L.ns_groups[bt.group0 + g];

@@ -159,8 +159,8 @@ def ns_chains(iters):
 
 
 def ns_flops_executed(shapes, iters=5, tile=128):
-    """FLOPs (fp32 multiply-adds x 2) that the library's kernels execute: symmetric m x m results on the tiles on
-    and above the diagonal only, and iterations in chains that share one Gram product and one update: a chain of L
+    """FLOPs (fp32 multiply-adds x 2) that the library's kernels execute: symmetric m x m results on the 64 x 64
+    blocks on and above the diagonal only (whole 128 x 128 tiles above it, three quadrants of those on it), and iterations in chains that share one Gram product and one update: a chain of L
     iterations is one Gram product, 4 L - 3 products of m x m matrices (L x Poly, 2 (L - 1) x Prod, (L - 1) x
     ProdA) and one update."""
     chains = ns_chains(iters)
@@ -169,7 +169,8 @@ def ns_flops_executed(shapes, iters=5, tile=128):
         if len(s) == 2:
             m, n = min(s), max(s)
             nt = -(-m // tile)
-            upper = nt * (nt + 1) / 2 * tile * tile
+            # tiles on and above the diagonal; on a diagonal tile the quadrant below the diagonal is not computed
+            upper = (nt * (nt + 1) / 2 - nt / 4) * tile * tile
             total += len(chains) * (2.0 * upper * n + 2.0 * m * m * n) + sum(4 * L - 3 for L in chains) * 2.0 * upper * m
     return total
 

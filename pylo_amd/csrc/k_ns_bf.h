@@ -129,9 +129,11 @@ __device__ __forceinline__ void bf_stage_issue(const char* g, const int (&off)[R
 
 // acc[hi][hj] += (rows i0.. of P1) x (rows j0.. of P2)^T over the reduction range [k0, k1) (multiples of 16);
 // 128 rows of P1, 64 WN rows of P2.  LDS: two stages of (128 + 64 WN) x 96 bytes.
+// `compute` (the same for all lanes of a wave): false for a wave whose values nobody needs -- it stages and meets the
+// barriers, and leaves the matrix pipe to the other waves of its SIMD.
 template <int WN>
 __device__ __forceinline__ void bf_tile_product(const BfPlanes& P1, int i0, const BfPlanes& P2, int j0, int k0, int k1,
-                                                PYLO_LDS char* lds, v16f (&acc)[2][WN]) {
+                                                PYLO_LDS char* lds, v16f (&acc)[2][WN], bool compute = true) {
   constexpr int RB = 64 * WN, SA = 128 * 96, STAGE = SA + RB * 96;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wi = (wave >> 1) * 64, wj = (wave & 1) * 32 * WN;
@@ -156,23 +158,25 @@ __device__ __forceinline__ void bf_tile_product(const BfPlanes& P1, int i0, cons
       bf_stage_issue<128>(ga, offa, lds + (STAGE - cur), wave);
       bf_stage_issue<RB>(gb, offb, lds + (STAGE - cur) + SA, wave);
     }
-    bf16x8 a[2][3], b[WN][3];
+    if (compute) {
+      bf16x8 a[2][3], b[WN][3];
 #pragma unroll
-    for (int q = 0; q < 3; ++q) {
+      for (int q = 0; q < 3; ++q) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) a[i][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + oa + i * 32 * 96 + q * 32));
+        for (int i = 0; i < 2; ++i) a[i][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + oa + i * 32 * 96 + q * 32));
 #pragma unroll
-      for (int j = 0; j < WN; ++j) b[j][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + ob + j * 32 * 96 + q * 32));
-    }
-    // smallest terms first: l h, h l, m m, m h, h m, h h
+        for (int j = 0; j < WN; ++j) b[j][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + ob + j * 32 * 96 + q * 32));
+      }
+      // smallest terms first: l h, h l, m m, m h, h m, h h
 #pragma unroll
-    for (int term = 0; term < 6; ++term) {
-      constexpr int pa[6] = {2, 0, 1, 1, 0, 0}, pb[6] = {0, 2, 1, 0, 1, 0};
+      for (int term = 0; term < 6; ++term) {
+        constexpr int pa[6] = {2, 0, 1, 1, 0, 0}, pb[6] = {0, 2, 1, 0, 1, 0};
 #pragma unroll
-      for (int hi = 0; hi < 2; ++hi)
+        for (int hi = 0; hi < 2; ++hi)
 #pragma unroll
-        for (int hj = 0; hj < WN; ++hj)
-          acc[hi][hj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[hi][pa[term]], b[hj][pb[term]], acc[hi][hj], 0, 0, 0);
+          for (int hj = 0; hj < WN; ++hj)
+            acc[hi][hj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[hi][pa[term]], b[hj][pb[term]], acc[hi][hj], 0, 0, 0);
+      }
     }
     // the loads into the other stage have landed (they are counted like any other vector-memory load) and
     // every wave has read this one
@@ -301,12 +305,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
   const int i0 = it.tm * kNsTile, j0 = it.tn * 64 * WN;
+  // A tile on the diagonal of a symmetric product: the 64 x 64 quadrant below the diagonal is the mirror image of the
+  // one above it, which its own wave (wave 1) writes to both places; wave 2 computes and stores nothing.
+  const int wave_u = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const bool diag = OP != kNsUpdate && WN == 2 && it.tm == it.tn;
+  const bool idle = diag && wave_u == 2;
   if (OP == kNsGram) {
     const BfPlanes X{pw + mt.off_xs, mt.rows_m};
-    bf_tile_product<WN>(X, i0, X, j0, it.k0, it.k1, lds, acc);
+    bf_tile_product<WN>(X, i0, X, j0, it.k0, it.k1, lds, acc, !idle);
   } else if (OP == kNsPoly) {
     const BfPlanes A{pw + mt.off_p, mt.rows_m};
-    bf_tile_product<WN>(A, i0, A, j0, it.k0, it.k1, lds, acc);
+    bf_tile_product<WN>(A, i0, A, j0, it.k0, it.k1, lds, acc, !idle);
   } else if (OP == kNsUpdate) {
     const BfPlanes X{pw + (par ? mt.off_xl[1] : mt.off_xl[0]), mt.rows_n};   // no run-time index: the struct stays in registers
     const BfPlanes B{pw + mt.off_p + bufs.s1 * mt.p_stride, mt.rows_m};
@@ -314,12 +323,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
   } else {
     const BfPlanes P1{pw + mt.off_p + bufs.s1 * mt.p_stride, mt.rows_m};
     const BfPlanes P2{pw + mt.off_p + bufs.s2 * mt.p_stride, mt.rows_m};
-    bf_tile_product<WN>(P1, i0, P2, j0, it.k0, it.k1, lds, acc);
+    bf_tile_product<WN>(P1, i0, P2, j0, it.k0, it.k1, lds, acc, !idle);
   }
+  if (idle) return;
   float* A32 = ws + mt.off_a;
   const int n_i = OP == kNsUpdate ? n : m;   // rows of the output; its columns are always m
   const bool partial = OP == kNsGram && it.slab >= 0;
-  const bool mirror = OP != kNsUpdate && !partial && it.tm != it.tn;
+  const bool mirror = OP != kNsUpdate && !partial && (it.tm != it.tn || wave_u == 1);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float* xout = a.step_out + mt.elem_off;
   const bool vec_out = (mt.C & 3) == 0;   // rows of the tensor are 16-byte aligned
@@ -390,7 +400,7 @@ __global__ __launch_bounds__(256) void k_ns_bf_gram_reduce(const NsBfMat* __rest
   const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
   if (e >= (long long)m * m) return;
   const int i = (int)(e / m), j = (int)(e - (long long)i * m);
-  if (i / kNsTile > j / kNsTile) return;
+  if (i / 64 > j / 64) return;   // the Gram jobs compute the 64 x 64 blocks on and above the diagonal
   const size_t mm = (size_t)m * lda;
   const float* p = ws + mt.off_part + (size_t)i * lda + j;
   float s = 0.0f;
@@ -405,7 +415,7 @@ __global__ __launch_bounds__(256) void k_ns_bf_gram_reduce(const NsBfMat* __rest
   bfbits* P = pw + mt.off_p;   // buffer A
   A[(size_t)i * lda + j] = s;
   bf_store1(P, mt.rows_m, i, j, s);
-  if (i / kNsTile != j / kNsTile) {
+  if (i / 64 != j / 64) {
     A[(size_t)j * lda + i] = s;
     bf_store1(P, mt.rows_m, j, i, s);
   }

@@ -144,19 +144,21 @@ __device__ __forceinline__ void bf_tile_product(const BfPlanes& P1, int i0, cons
   const char* ga = (const char*)P1.base + ((size_t)(k0 >> 4) * P1.rows + i0) * 96;
   const char* gb = (const char*)P2.base + ((size_t)(k0 >> 4) * P2.rows + j0) * 96;
   const size_t sa = (size_t)P1.rows * 96, sb = (size_t)P2.rows * 96;
+  // a diagonal tile of X X^T or A A: both operands are the same 128 rows, staged once
+  const bool same = WN == 2 && P1.base == P2.base && i0 == j0;
   bf_stage_issue<128>(ga, offa, lds, wave);
-  bf_stage_issue<RB>(gb, offb, lds + SA, wave);
+  if (!same) bf_stage_issue<RB>(gb, offb, lds + SA, wave);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   const int sw = 16 * (kg ^ ((lo >> 3) & 1));
-  const int oa = (wi + lo) * 96 + sw, ob = SA + (wj + lo) * 96 + sw;
+  const int oa = (wi + lo) * 96 + sw, ob = (same ? 0 : SA) + (wj + lo) * 96 + sw;
   int cur = 0;
   for (int k = k0; k < k1; k += kBfBK) {
     if (k + kBfBK < k1) {
       ga += sa;
       gb += sb;
       bf_stage_issue<128>(ga, offa, lds + (STAGE - cur), wave);
-      bf_stage_issue<RB>(gb, offb, lds + (STAGE - cur) + SA, wave);
+      if (!same) bf_stage_issue<RB>(gb, offb, lds + (STAGE - cur) + SA, wave);
     }
     if (compute) {
       bf16x8 a[2][3], b[WN][3];

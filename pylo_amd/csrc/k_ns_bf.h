@@ -80,6 +80,7 @@ struct NsBfMat {
   long long off_a;           // floats into the fp32 workspace: A (m x m)
   long long off_part;        // floats: partial matrices of a split Gram product
   long long elem_off;        // elements from the tensor's raw step to this matrix (a slice of a tensor with more dims)
+  int fpart0, n_fpart;       // its partial sums of squares of A (k_ns_bf_chain_sumsq): first, count
 };
 
 // the m x m plane buffers, and the two products on planes in and planes out (k_ns_bf_gemm's OP, after
@@ -286,15 +287,31 @@ __device__ __forceinline__ void bf_store_planes(PYLO_LDS char* lds, const v16f (
 // WN: the tile has 64 WN columns (Gram and Poly: 2; updates: 2 or 4, a table of jobs each).
 // Registers: 64 / 128 accumulator registers plus what the epilogues need; tiles of 256 columns are held to two
 // waves per SIMD (256 registers: left alone the epilogue takes 296 and a CU runs one job at a time).
+// Which matrices a launch is for, when the chain length is chosen per matrix (k_ns_bf_chain_flag): all of them; those
+// whose first chain is the longer one; the others; or all, the others with another first operand buffer and `last`.
+enum : int { kNsAll = 0, kNsLongOnly = 1, kNsShortOnly = 2, kNsBoth = 3 };
+struct NsPick {
+  const int* flags;
+  int sel, s1_short, last_short;
+};
+
 template <int OP, int WN>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2 : 3))) void k_ns_bf_gemm(const NsBfMat* __restrict__ mats, const NsItem* __restrict__ items,
                                                     const PyloTensorArgs* __restrict__ dyn, float* __restrict__ ws,
                                                     bfbits* __restrict__ pw, int par, int last, NsBufs bufs, float c0,
-                                                    float c1, float c2) {
+                                                    float c1, float c2, NsPick pick) {
   extern __shared__ __attribute__((aligned(16))) char lds_[];
   PYLO_LDS char* lds = (PYLO_LDS char*)lds_;
   const NsItem it = items[blockIdx.x];
   if (it.mat < 0) return;   // a filler job
+  if (pick.sel != kNsAll) {
+    const bool longer = pick.flags[it.mat] != 0;
+    if ((pick.sel == kNsLongOnly && !longer) || (pick.sel == kNsShortOnly && longer)) return;
+    if (pick.sel == kNsBoth && !longer) {
+      bufs.s1 = pick.s1_short;
+      last = pick.last_short;
+    }
+  }
   const NsBfMat mt = mats[it.mat];
   const PyloTensorArgs a = dyn[mt.tensor];
   if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
@@ -394,7 +411,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
 // A = sum over the slabs' partial matrices, in slab order, as fp32 and as planes (both halves).
 __global__ __launch_bounds__(256) void k_ns_bf_gram_reduce(const NsBfMat* __restrict__ mats, const int* __restrict__ split_mats,
                                                            const PyloTensorArgs* __restrict__ dyn, float* __restrict__ ws,
-                                                           bfbits* __restrict__ pw) {
+                                                           bfbits* __restrict__ pw, NsPick pick) {
+  if (pick.sel == kNsShortOnly && pick.flags[split_mats[blockIdx.y]] != 0) return;
   const NsBfMat mt = mats[split_mats[blockIdx.y]];
   const PyloTensorArgs a = dyn[mt.tensor];
   if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
@@ -426,6 +444,51 @@ __global__ __launch_bounds__(256) void k_ns_bf_gram_reduce(const NsBfMat* __rest
 // X0 = raw * s (s = 1 / (||raw|| + eps), scale[mat]) as planes in both layouts.  One block = one 64 x 64
 // tile of the raw step (R x C): the planes in which the tensor's rows stay rows are written straight from
 // the loaded values, the transposed planes through LDS.
+// The length of a matrix's first chain.  With X scaled to unit Frobenius norm, ||A||_F (A = X X^T as computed) bounds
+// the largest eigenvalue of A from above; what a chain of three iterations adds to the error of the result is
+// proportional to it, 196 eps_A lambda_max against 16 eps_A lambda_max for a pair (head of this file), so three
+// iterations are taken where ||A||_F^2 <= tau^2, with tau = 16 / 196: no worse there than a pair is on any matrix.
+// Two launches, sums in a fixed order: 4096 elements of A per block, then one block per matrix.
+constexpr int kNsFlagChunk = 4096;
+// items[b] = {matrix, chunk of 4096 elements of its A}
+__global__ __launch_bounds__(256) void k_ns_bf_chain_sumsq(const NsBfMat* __restrict__ mats, const Item* __restrict__ items,
+                                                           const PyloTensorArgs* __restrict__ dyn, const float* __restrict__ ws,
+                                                           float* __restrict__ part) {
+  __shared__ float red[4];
+  const Item it = items[blockIdx.x];
+  const NsBfMat mt = mats[it.tensor];
+  const PyloTensorArgs a = dyn[mt.tensor];
+  if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
+  const long long mm = (long long)mt.m * mt.m, e0 = (long long)it.a * kNsFlagChunk;
+  const float* A = ws + mt.off_a;
+  float s = 0.0f;
+  for (int i = 0; i < kNsFlagChunk / 256; ++i) {
+    const long long e = e0 + threadIdx.x + 256 * i;
+    if (e < mm) {
+      const int r = (int)(e / mt.m), c = (int)(e - (long long)r * mt.m);
+      const float v = *(const gfloat*)(A + (size_t)r * mt.lda + c);
+      s = fmaf(v, v, s);
+    }
+  }
+  s = wave_sum(s);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) part[mt.fpart0 + it.a] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+__global__ __launch_bounds__(64) void k_ns_bf_chain_flag(const NsBfMat* __restrict__ mats, const int* __restrict__ list,
+                                                         const PyloTensorArgs* __restrict__ dyn, const float* __restrict__ part,
+                                                         float tau2, int* __restrict__ flags) {
+  const int q = list[blockIdx.x];
+  const NsBfMat mt = mats[q];
+  const PyloTensorArgs a = dyn[mt.tensor];
+  if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
+  float s = 0.0f;
+  for (int b = threadIdx.x; b < mt.n_fpart; b += 64) s += part[mt.fpart0 + b];
+  s = wave_sum(s);
+  if (threadIdx.x == 0) flags[q] = s <= tau2 ? 1 : 0;
+}
+
 struct NsTileItem { int mat, tr, tc; };
 
 __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__ mats, const NsTileItem* __restrict__ items,

@@ -79,6 +79,7 @@ struct NsGroup {
   int gram0, n_gram, poly0, n_poly, upd0, n_upd, upd40, n_upd4, split0, n_split, split_max_m;
   int list0, n_list;       // its matrices (ns_list)
   int sitem0, n_sitems;    // its tiles of the pass that splits the raw steps into planes
+  int fitem0, n_fitems;    // its blocks of the pass that sums the squares of A (chain length per matrix)
   int fin0, n_fin;         // its blocks of the finishing pass
   int unit0, n_units;      // ... and their units
 };
@@ -113,6 +114,9 @@ struct Layout {
   int slice_lds_l[kSliceLaneSets] = {}, slice_lds_w = 0, slice_lds_b = 0;
   size_t off_slice_mats = 0, off_slice_items_l[kSliceLaneSets] = {}, off_slice_items_w = 0, off_slice_items_b = 0;
   int ns_max_m = 0;
+  std::vector<Item> ns_flag_items;    // split-bf16 kernels: {matrix, chunk of its A} of k_ns_bf_chain_sumsq, group after group
+  int ns_fpart_total = 0;
+  size_t off_ns_flags = 0, off_ns_fpart = 0, off_ns_flag_items = 0;
   // Newton-Schulz on the bf16 matrix pipe (three-way split operands): tables of their own
   bool ns_bf = false;
   std::vector<NsBfMat> nsb_mats;
@@ -297,6 +301,20 @@ std::vector<int> ns_chains(int iters) {
   return out;
 }
 
+// PYLO_MI355_NS_ADAPTIVE=1: a first chain of three iterations for the matrices whose spectrum allows it
+// (k_ns_bf_chain_flag), pairs for the others -- unless the environment fixes the chains (PYLO_MI355_NS_CHAINS,
+// PYLO_MI355_NS_PAIRS=0).  Off by default: raw steps with a direction that holds more than 8 % of their squared norm
+// never qualify (an untrained MLP's steps, with their common offset, are such), and the test costs 0.04 ms a step.
+// Read when the products are enqueued.
+bool ns_adaptive() {
+  const char* a = getenv("PYLO_MI355_NS_ADAPTIVE");
+  if (!(a && a[0] == '1')) return false;
+  const char* p = getenv("PYLO_MI355_NS_PAIRS");
+  if (p && p[0] == '0') return false;
+  const char* c = getenv("PYLO_MI355_NS_CHAINS");
+  return !(c && c[0]);
+}
+
 bool env_ns_bf() {
   const char* e = getenv("PYLO_MI355_NS_F32");
   return !(e && e[0] == '1');
@@ -466,6 +484,8 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
     L.ns_split.clear();
     L.ns_list.clear();
     L.nsb_split_items.clear();
+    L.ns_flag_items.clear();
+    L.ns_fpart_total = 0;
     for (NsBatch& bt : L.ns_batches) {
     const int n_groups = std::min<int>(env_ns_groups(), std::max(bt.n_mats / 8, 1));
     std::vector<std::vector<int>> members(n_groups);
@@ -498,7 +518,15 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       grp.split0 = (int)L.ns_split.size();
       grp.list0 = (int)L.ns_list.size();
       grp.sitem0 = (int)L.nsb_split_items.size();
+      grp.fitem0 = (int)L.ns_flag_items.size();
       for (int q : members[g]) {
+        {
+          NsBfMat& bw = L.nsb_mats[q];
+          bw.fpart0 = L.ns_fpart_total;
+          bw.n_fpart = (int)(((long long)bw.m * bw.m + kNsFlagChunk - 1) / kNsFlagChunk);
+          L.ns_fpart_total += bw.n_fpart;
+          for (int c = 0; c < bw.n_fpart; ++c) L.ns_flag_items.push_back(Item{q, c, 0, 0});
+        }
         const NsBfMat& b = L.nsb_mats[q];
         L.ns_list.push_back(q);
         L.ns_group_of_tensor[b.tensor] = (int)L.ns_groups.size();
@@ -556,6 +584,7 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       grp.n_split = (int)L.ns_split.size() - grp.split0;
       grp.n_list = (int)L.ns_list.size() - grp.list0;
       grp.n_sitems = (int)L.nsb_split_items.size() - grp.sitem0;
+      grp.n_fitems = (int)L.ns_flag_items.size() - grp.fitem0;
       L.ns_groups.push_back(grp);
     }
     }
@@ -931,6 +960,9 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     L.off_ns_split = take(sizeof(int) * L.ns_split.size());
     L.off_ns_xalt = take(sizeof(long long) * (size_t)T);
     L.off_ns_scale = take(sizeof(float) * L.ns_mats.size());
+    L.off_ns_flags = take(sizeof(int) * L.ns_mats.size());
+    L.off_ns_fpart = take(sizeof(float) * (size_t)L.ns_fpart_total);
+    L.off_ns_flag_items = take(sizeof(Item) * L.ns_flag_items.size());
     L.off_ns_ws = take(sizeof(float) * (size_t)ns_floats);
     L.off_nsb_mats = take(sizeof(NsBfMat) * L.nsb_mats.size());
     L.off_nsb_split_items = take(sizeof(NsTileItem) * L.nsb_split_items.size());
@@ -1048,6 +1080,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_nsb_mats, L.nsb_mats.data(), sizeof(NsBfMat) * L.nsb_mats.size());
   if (e == hipSuccess) e = up(L.off_nsb_split_items, L.nsb_split_items.data(), sizeof(NsTileItem) * L.nsb_split_items.size());
   if (e == hipSuccess) e = up(L.off_ns_list, L.ns_list.data(), sizeof(int) * L.ns_list.size());
+  if (e == hipSuccess) e = up(L.off_ns_flag_items, L.ns_flag_items.data(), sizeof(Item) * L.ns_flag_items.size());
   if (e == hipSuccess) e = up(L.off_slice_mats, L.slice_mats.data(), sizeof(SliceMat) * L.slice_mats.size());
   for (int k = 0; k < kSliceLaneSets; ++k)
     if (e == hipSuccess) e = up(L.off_slice_items_l[k], L.slice_items_l[k].data(), sizeof(Item) * L.slice_items_l[k].size());
@@ -1614,6 +1647,12 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
     const bool several = L.ns_batches.size() > 1;
     const float c0 = coeffs[0], c1 = coeffs[1], c2 = coeffs[2];
     const std::vector<int> chains = ns_chains(ns_iters);
+    // chain lengths chosen per matrix on the device: an odd iteration count of three or more, nothing given in the environment
+    const bool adaptive = ns_adaptive() && ns_iters >= 3 && (ns_iters & 1);
+    int* chain_flags = P->at<int>(L.off_ns_flags);
+    float* chain_part = P->at<float>(L.off_ns_fpart);
+    const Item* flag_items = P->at<Item>(L.off_ns_flag_items);
+    const float chain_tau2 = (16.0f / 196.0f) * (16.0f / 196.0f);
     for (const NsBatch& bt : L.ns_batches) {
       // the planes' padding: zero from plan creation on when one batch has the memory to itself
       if (several) {
@@ -1641,52 +1680,103 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
           hipLaunchKernelGGL(k_ns_bf_split, dim3((unsigned)G.n_sitems), dim3(256), 0, sg, bmats, sitems + G.sitem0, dyn,
                              (const float*)scale, pw);
       }
+      // The launch sequence of one group (every group runs the same one on its own tables), then its launches,
+      // interleaved over the groups so that every stream is fed in turn.
+      enum OpKind { kOpGram, kOpFlag, kOpPoly, kOpProd, kOpProdA, kOpUpdate };
+      struct Op { OpKind kind; NsBufs b; int par, last; NsPick pick; };
+      std::vector<Op> ops;
+      const NsPick all{nullptr, kNsAll, 0, 0};
       int par = 0;   // which Xl buffer the next update reads
-      int done = 0;
-      for (size_t ch = 0; ch < chains.size(); ++ch) {
-        // a chain of iterations: one Gram product, 4 len - 3 products of m x m matrices and one update (k_ns_bf.h)
-        const int len = chains[ch];
-        done += len;
-        const int last = done == ns_iters;
+      // A is buffer A throughout; B' of the latest iteration in `bprev`, the product of all B' so far in `q`
+      int bprev = kNsBufB, q = kNsBufB;
+      auto extend = [&](NsPick pk) {   // one more iteration into the chain: A <- B' A B', the next B', Q <- B' Q
+        int free_buf[2], nf = 0;
+        for (int b : {kNsBufB, kNsBufT, kNsBufC})
+          if (b != bprev && b != q && nf < 2) free_buf[nf++] = b;
+        const int t = free_buf[0];
+        ops.push_back(Op{kOpProd, NsBufs{kNsBufA, bprev, t}, par, 0, pk});
+        ops.push_back(Op{kOpProdA, NsBufs{bprev, t, kNsBufA}, par, 0, pk});
+        ops.push_back(Op{kOpPoly, NsBufs{kNsBufA, kNsBufA, t}, par, 0, pk});
+        const int qn = q == bprev ? free_buf[1] : bprev;   // (the old B' is done with)
+        ops.push_back(Op{kOpProd, NsBufs{t, q, qn}, par, 0, pk});
+        bprev = t;
+        q = qn;
+      };
+      auto open_chain = [&](NsPick pk) {   // Gram product and the first B'
+        ops.push_back(Op{kOpGram, NsBufs{0, 0, kNsBufA}, par, 0, pk});
+        ops.push_back(Op{kOpPoly, NsBufs{kNsBufA, kNsBufA, kNsBufB}, par, 0, pk});
+        bprev = q = kNsBufB;
+      };
+      if (adaptive) {
+        // First chain: two iterations for every matrix, a third for those whose flag says so (k_ns_bf_chain_flag),
+        // then pairs for all -- the last of them is the end for the flagged ones -- and one iteration more for the others.
+        const NsPick longer{chain_flags, kNsLongOnly, 0, 0}, shorter{chain_flags, kNsShortOnly, 0, 0};
+        const int n_pairs = (ns_iters - 3) / 2;
+        open_chain(all);
+        ops.push_back(Op{kOpFlag, NsBufs{0, 0, 0}, par, 0, all});
+        extend(all);
+        const int q_short = q;
+        extend(longer);
+        ops.push_back(Op{kOpUpdate, NsBufs{q, 0, 0}, par, n_pairs == 0, NsPick{chain_flags, kNsBoth, q_short, 0}});
+        par ^= 1;
+        for (int p = 0; p < n_pairs; ++p) {
+          open_chain(all);
+          extend(all);
+          ops.push_back(Op{kOpUpdate, NsBufs{q, 0, 0}, par, p == n_pairs - 1, NsPick{chain_flags, kNsBoth, q, 0}});
+          par ^= 1;
+        }
+        open_chain(shorter);
+        ops.push_back(Op{kOpUpdate, NsBufs{q, 0, 0}, par, 1, shorter});
+      } else {
+        int done = 0;
+        for (size_t ch = 0; ch < chains.size(); ++ch) {
+          // a chain of iterations: one Gram product, 4 len - 3 products of m x m matrices and one update (k_ns_bf.h)
+          done += chains[ch];
+          open_chain(all);
+          for (int j = 1; j < chains[ch]; ++j) extend(all);
+          ops.push_back(Op{kOpUpdate, NsBufs{q, 0, 0}, par, done == ns_iters, all});
+          par ^= 1;
+        }
+      }
+      for (const Op& op : ops)
         for (int g = 0; g < n_groups; ++g) {
           const NsGroup& G = L.ns_groups[bt.group0 + g];
           hipStream_t sg = stream_of(g);
-          auto small = [&](auto kern, NsBufs b) {
+          auto small = [&](auto kern) {
             if (G.n_poly > 0)
               hipLaunchKernelGGL(kern, dim3(G.n_poly), dim3(256), bf_gemm_lds(2), sg, bmats, poly + G.poly0, dyn, ns_ws, pw,
-                                 par, last, b, c0, c1, c2);
+                                 op.par, op.last, op.b, c0, c1, c2, op.pick);
           };
-          if (G.n_gram > 0)
-            hipLaunchKernelGGL((k_ns_bf_gemm<kNsGram, 2>), dim3(G.n_gram), dim3(256), bf_gemm_lds(2), sg, bmats,
-                               gram + G.gram0, dyn, ns_ws, pw, par, last, NsBufs{0, 0, kNsBufA}, c0, c1, c2);
-          if (G.n_split > 0)
-            hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)G.split_max_m * G.split_max_m + 255) / 256, G.n_split),
-                               dim3(256), 0, sg, bmats, split + G.split0, dyn, ns_ws, pw);
-          // A lives in buffer A throughout; B' of the latest iteration in `bprev`, the product of all B' so far in `q`
-          small(k_ns_bf_gemm<kNsPoly, 2>, NsBufs{kNsBufA, kNsBufA, kNsBufB});            // B'_t
-          int bprev = kNsBufB, q = kNsBufB;
-          for (int j = 1; j < len; ++j) {
-            int free_buf[2], nf = 0;
-            for (int b : {kNsBufB, kNsBufT, kNsBufC})
-              if (b != bprev && b != q && nf < 2) free_buf[nf++] = b;
-            const int t = free_buf[0];
-            small(k_ns_bf_gemm<kNsProd, 2>, NsBufs{kNsBufA, bprev, t});                  // T = A B'
-            small(k_ns_bf_gemm<kNsProdA, 2>, NsBufs{bprev, t, kNsBufA});                 // A <- B' T = B' A B'
-            small(k_ns_bf_gemm<kNsPoly, 2>, NsBufs{kNsBufA, kNsBufA, t});                // the next B'
-            const int qn = q == bprev ? free_buf[1] : bprev;                           // (the old B' is done with)
-            small(k_ns_bf_gemm<kNsProd, 2>, NsBufs{t, q, qn});                           // Q <- B' Q
-            bprev = t;
-            q = qn;
+          switch (op.kind) {
+            case kOpGram:
+              if (G.n_gram > 0)
+                hipLaunchKernelGGL((k_ns_bf_gemm<kNsGram, 2>), dim3(G.n_gram), dim3(256), bf_gemm_lds(2), sg, bmats,
+                                   gram + G.gram0, dyn, ns_ws, pw, op.par, op.last, op.b, c0, c1, c2, op.pick);
+              if (G.n_split > 0)
+                hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)G.split_max_m * G.split_max_m + 255) / 256, G.n_split),
+                                   dim3(256), 0, sg, bmats, split + G.split0, dyn, ns_ws, pw, op.pick);
+              break;
+            case kOpFlag:
+              if (G.n_list > 0) {
+                hipLaunchKernelGGL(k_ns_bf_chain_sumsq, dim3(G.n_fitems), dim3(256), 0, sg, bmats, flag_items + G.fitem0, dyn,
+                                   (const float*)ns_ws, chain_part);
+                hipLaunchKernelGGL(k_ns_bf_chain_flag, dim3(G.n_list), dim3(64), 0, sg, bmats, list + G.list0, dyn,
+                                   (const float*)chain_part, chain_tau2, chain_flags);
+              }
+              break;
+            case kOpPoly: small(k_ns_bf_gemm<kNsPoly, 2>); break;
+            case kOpProd: small(k_ns_bf_gemm<kNsProd, 2>); break;
+            case kOpProdA: small(k_ns_bf_gemm<kNsProdA, 2>); break;
+            case kOpUpdate:
+              if (G.n_upd4 > 0)
+                hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 4>), dim3(G.n_upd4), dim3(256), bf_gemm_lds(4), sg, bmats,
+                                   upd4 + G.upd40, dyn, ns_ws, pw, op.par, op.last, op.b, c0, c1, c2, op.pick);
+              if (G.n_upd > 0)
+                hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 2>), dim3(G.n_upd), dim3(256), bf_gemm_lds(2), sg, bmats,
+                                   upd + G.upd0, dyn, ns_ws, pw, op.par, op.last, op.b, c0, c1, c2, op.pick);
+              break;
           }
-          if (G.n_upd4 > 0)
-            hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 4>), dim3(G.n_upd4), dim3(256), bf_gemm_lds(4), sg, bmats,
-                               upd4 + G.upd40, dyn, ns_ws, pw, par, last, NsBufs{q, 0, 0}, c0, c1, c2);
-          if (G.n_upd > 0)
-            hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 2>), dim3(G.n_upd), dim3(256), bf_gemm_lds(2), sg, bmats,
-                               upd + G.upd0, dyn, ns_ws, pw, par, last, NsBufs{q, 0, 0}, c0, c1, c2);
         }
-        par ^= 1;
-      }
       for (int g = 0; g < n_groups; ++g) {
         const NsGroup& G = L.ns_groups[bt.group0 + g];
         finish_range(stream_of(g), G.fin0, G.n_fin, G.unit0, G.n_units, nullptr, nullptr);

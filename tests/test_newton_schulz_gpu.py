@@ -184,6 +184,50 @@ def test_spectra_with_a_dominant_direction(chains, floor, monkeypatch):
     print("chains", pairs, "(shape, library error / rms, fp32 torch formula error / rms):", rows)
 
 
+def test_chain_length_chosen_per_matrix(monkeypatch):
+    """PYLO_MI355_NS_ADAPTIVE=1: the first chain takes three iterations for the matrices whose A = X X^T has
+    ||A||_F^2 <= (16 / 196)^2 (no direction holds more than 8 % of the step's squared norm: what three chained
+    iterations add to the error is then no more than what a pair adds on any matrix) and two for the others.  The
+    choice is made on the device, matrix by matrix; each result is bit-identical to that of the fixed schedule
+    it amounts to, "3,2" or "2,2,1"."""
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    rnd = lambda *s: torch.randn(*s, generator=gen, device="cuda")
+
+    def dominant(r, c, rest):
+        u, v = rnd(r, 1), rnd(1, c)
+        return u @ v / (u.norm() * v.norm()) + rest * rnd(r, c) / (r * c) ** 0.5
+
+    mats = [rnd(768, 3072), dominant(256, 384, 1.0), rnd(768, 768), dominant(130, 1000, 1.0), rnd(64, 64), rnd(8300, 160),
+            dominant(8300, 160, 0.3), rnd(200, 150), rnd(12, 160)]
+    longer = [True, False, True, False, False, True, False, False, False]
+    for x, want in zip(mats, longer):
+        a = (x / x.norm()).double()
+        a = a @ a.T if x.shape[0] <= x.shape[1] else a.T @ a
+        assert (float((a * a).sum()) <= (16 / 196) ** 2) == want, tuple(x.shape)
+    monkeypatch.setenv("PYLO_MI355_NS_ADAPTIVE", "1")
+    chosen = _orthogonalise_direct(mats)
+    monkeypatch.delenv("PYLO_MI355_NS_ADAPTIVE")
+    monkeypatch.setenv("PYLO_MI355_NS_CHAINS", "2,2,1")
+    pairs = _orthogonalise_direct(mats)
+    monkeypatch.setenv("PYLO_MI355_NS_CHAINS", "3,2")
+    three = _orthogonalise_direct(mats)
+    monkeypatch.delenv("PYLO_MI355_NS_CHAINS")
+    default = _orthogonalise_direct(mats)
+    for x, c, p, t, d, want in zip(mats, chosen, pairs, three, default, longer):
+        assert torch.equal(c, t if want else p), tuple(x.shape)
+        assert torch.equal(d, p), tuple(x.shape)            # the default: pairs
+    # other odd counts: a chain of three alone, and three followed by pairs
+    for iters in (3, 7):
+        monkeypatch.setenv("PYLO_MI355_NS_ADAPTIVE", "1")
+        got = _orthogonalise_direct(mats, iters)
+        monkeypatch.delenv("PYLO_MI355_NS_ADAPTIVE")
+        ref = _orthogonalise_direct(mats, iters)
+        for x, y, z, want in zip(mats, got, ref, longer):
+            e = float((y.double() - _reference_direct(x, iters)).abs().max())
+            assert e <= 1e-4, (iters, tuple(x.shape), e)
+            assert torch.equal(y, z) == (not want), (iters, tuple(x.shape))
+
+
 def test_workspace_budget_and_unflagged_tensors(monkeypatch):
     """The operand planes live only during a matrix's own products: under a small PYLO_MI355_NS_WORKSPACE_MB the
     matrices run in batches that share the memory (same arithmetic, bit-identical parameters, smaller workspace);

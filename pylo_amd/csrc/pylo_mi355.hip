@@ -495,7 +495,8 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       std::vector<Run> runs;
       for (int q = bt.mat0; q < bt.mat0 + bt.n_mats; ++q) {
         const NsBfMat& b = L.nsb_mats[q];
-        const double w = (double)b.m * b.m * b.n;
+        // (five iterations in pairs: three Gram products on the upper blocks and three updates, eleven m x m products)
+        const double w = (double)b.m * b.m * (4.6 * b.n + 5.9 * b.m);
         if (!runs.empty() && L.nsb_mats[runs.back().q0].tensor == b.tensor) { runs.back().q1 = q + 1; runs.back().work += w; }
         else runs.push_back(Run{q, q + 1, w});
       }

@@ -1,6 +1,6 @@
 """Benchmark of the fused learned-optimizer step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gpt2s|cfg1|vit_velo|llama_adafac|stress_velo|stress_celo2|stream_ceiling|matrix_ceiling] [--fused-only]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gpt2s|cfg1|vit_velo|llama_adafac|stress_velo|stress_celo2|conv_celo2|stream_ceiling|matrix_ceiling] [--fused-only]
 
 Workload (default): BASELINE config 2 -- ELO-CELO2 on a GPT-2-small-shaped fp32 parameter set
 (98 tensors, 124 355 328 parameters), synthetic per-tensor Gaussian gradients with log-uniform
@@ -51,6 +51,21 @@ def vit_b16_shapes():
     for _ in range(12):
         shapes += [(768,), (768,), (768, 2304), (768, 768), (768,), (768,), (768, 3072), (3072, 768)]
     return shapes + [(768, 1000)]
+
+
+def resnet50_shapes():
+    """Not a BASELINE configuration: ResNet-50, 161 tensors, 25 557 032 elements, 11.3 M of them in 3 x 3 kernels --
+    the tensors with more than two dims that ELO-CELO2 orthogonalises, normalises and applies per slice."""
+    shapes = [(64, 3, 7, 7), (64,), (64,)]
+    inplanes = 64
+    for planes, blocks in ((64, 3), (128, 4), (256, 6), (512, 3)):
+        for b in range(blocks):
+            shapes += [(planes, inplanes, 1, 1), (planes,), (planes,), (planes, planes, 3, 3), (planes,), (planes,),
+                       (planes * 4, planes, 1, 1), (planes * 4,), (planes * 4,)]
+            if b == 0:
+                shapes += [(planes * 4, inplanes, 1, 1), (planes * 4,), (planes * 4,)]
+            inplanes = planes * 4
+    return shapes + [(1000, 2048), (1000,)]
 
 
 def llama_1b_shapes(layers=22):
@@ -217,7 +232,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gpt2s", choices=["gpt2s", "cfg1", "vit_velo", "llama_adafac", "stress_velo", "stress_celo2", "stream_ceiling", "matrix_ceiling"])
+    ap.add_argument("--workload", default="gpt2s", choices=["gpt2s", "cfg1", "vit_velo", "llama_adafac", "stress_velo", "stress_celo2", "conv_celo2", "stream_ceiling", "matrix_ceiling"])
     ap.add_argument("--fused-only", action="store_true",
                     help="loop the C-ABI call alone (no Newton-Schulz / apply), e.g. under rocprofv3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -236,6 +251,9 @@ def main():
     from pylo_amd import ELO_CELO2_CUDA
     from pylo_amd.models import CELO2MLP
 
+    if a.workload == "conv_celo2":
+        print(json.dumps(conv_workload(a.steps, a.warmup)))
+        return
     if a.workload in ("stress_velo", "stress_celo2"):
         print(json.dumps(stress_workload(a.workload, a.steps, a.warmup)))
         return
@@ -454,6 +472,50 @@ def matrix_ceiling(a):
     print(json.dumps({"metric": "attainable_bf16_matrix_rate", "unit": "PFLOP/s", "n_gpus": 1, "steps": a.steps,
                       "warmup": a.warmup, "tile": "128x256, 6 x v_mfma_f32_32x32x16_bf16 per fp32 tile product",
                       "peak_PFLOPs": 2.5, "cases": res}))
+
+
+def conv_workload(steps, warmup):
+    """Whole ELO_CELO2 optimizer.step() on the ResNet-50 parameter set: the fused element call (per-slice feature
+    normalisers for the convolution kernels), then one finishing call in which every kernel's k x k slices are
+    orthogonalised, normalised and applied by the per-slice launches and the one matrix by the tiled products."""
+    import numpy as np
+    import torch
+
+    from pylo_amd import ELO_CELO2_CUDA
+    from pylo_amd.models import CELO2MLP
+
+    dev = torch.device("cuda:0")
+    shapes = resnet50_shapes()
+    gen = torch.Generator(device=dev).manual_seed(1)
+    params = [torch.nn.Parameter(torch.randn(s, generator=gen, device=dev) * 0.02) for s in shapes]
+    for p in params:
+        p.grad = torch.randn(p.shape, generator=gen, device=dev) * 1e-2
+    torch.manual_seed(1)
+    opt = ELO_CELO2_CUDA(params, lr=3e-4, weight_decay=0.1, network=CELO2MLP(), hf_key=None)
+    for _ in range(max(warmup, 4)):
+        opt.step()
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        marks[k][0].record()
+        tensors = opt.fused_step()
+        marks[k][1].record()
+        opt.finish_step(tensors)
+        marks[k][2].record()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    n = sum(p.numel() for p in params)
+    n_nd = sum(p.numel() for p in params if p.dim() > 2)
+    return {"metric": "params_updated_per_sec (whole optimizer.step())", "value": n / (ms * 1e-3), "unit": "params/s",
+            "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "ELO_CELO2 whole optimizer.step(), ResNet-50 parameter set", "params": n,
+                       "tensors": len(shapes), "params_in_tensors_with_more_than_two_dims": n_nd},
+            "fused_call_ms": float(np.mean([m[0].elapsed_time(m[1]) for m in marks])),
+            "finishing_call_ms": float(np.mean([m[1].elapsed_time(m[2]) for m in marks])),
+            "tensors_left_to_torch_products": sum(1 for i, (g, p, adam) in enumerate(opt._tensors())
+                                                  if not adam and p.dim() >= 2 and not opt._ns_ok[i])}
 
 
 def stress_workload(workload, steps, warmup):

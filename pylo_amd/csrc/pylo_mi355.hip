@@ -132,6 +132,10 @@ struct Layout {
   long long stage_floats = 0;
   size_t off_dyn_user = 0, off_stage_ofs = 0, off_cast_items = 0, off_stage = 0;
   std::vector<TDesc> descs;
+  std::vector<Item> sl_lane_items;    // ELO-CELO2: blocks of k_celo2_slices_lane, the classes of slice length one after another
+  std::vector<Item> sl_lane_cls[kSliceLaneClasses];
+  int sl_lane_n[kSliceLaneClasses] = {}, sl_lane_lds[kSliceLaneClasses] = {};   // a launch per class: LDS sized for its longest slice
+  size_t off_sl_lane_items = 0;
   std::vector<Item> p0_items, nd_items, sl_items, seg_items, el_items, ap_items, pp_items, ga_items, fin_items, v0a_items, v0b_items;
   std::vector<int> fac_list;
   std::vector<int> dc, dr;
@@ -313,6 +317,13 @@ bool ns_adaptive() {
   if (p && p[0] == '0') return false;
   const char* c = getenv("PYLO_MI355_NS_CHAINS");
   return !(c && c[0]);
+}
+
+// PYLO_MI355_SLICES_LDS=0: the short slices of ELO-CELO2 tensors with more than two dims stay on the kernel that reads
+// them straight from memory, twice (k_celo2_slices); read at plan creation.
+bool env_slices_lds() {
+  const char* e = getenv("PYLO_MI355_SLICES_LDS");
+  return !(e && e[0] == '0');
 }
 
 bool env_ns_bf() {
@@ -844,6 +855,14 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       // one pass per slice of the last two dims (k_celo2_slices): 256 slices a block, or 4
       const long long n_slices = n / d.slice_len, per = d.slice_len <= kSliceLaneMax ? kThreads : kWaves;
       if (n_slices >= (1ll << 31)) return fail("plan: too many slices");
+      if (d.mode == kModeFacND && d.slice_len <= kSliceLaneMax && env_slices_lds()) {
+        // short slices of a tensor with more than two dims: 64 a block, staged through LDS (k_celo2_slices_lane)
+        int cls = 0;
+        while (d.slice_len > kSliceLaneClassMax[cls]) ++cls;
+        for (long long s0 = 0; s0 < n_slices && n > 0; s0 += 64 * slice_lane_groups(d.slice_len))
+          L.sl_lane_cls[cls].push_back(Item{t, (int)s0, 0, 0});
+        L.sl_lane_lds[cls] = std::max(L.sl_lane_lds[cls], (int)sizeof(float) * 6 * d.slice_len * kSlicePitchF);
+      } else
       for (long long s0 = 0; s0 < n_slices && n > 0; s0 += per) L.sl_items.push_back(Item{t, (int)s0, 0, 0});
     } else if (wide && d.C0 % kTileCols == 0) {
       d.tile_nct = d.C0 / kTileCols;
@@ -911,6 +930,12 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   L.off_p0_items = take(sizeof(Item) * L.p0_items.size());
   L.off_nd_items = take(sizeof(Item) * L.nd_items.size());
   L.off_sl_items = take(sizeof(Item) * L.sl_items.size());
+  for (int c = 0; c < kSliceLaneClasses; ++c) {
+    L.sl_lane_n[c] = (int)L.sl_lane_cls[c].size();
+    L.sl_lane_items.insert(L.sl_lane_items.end(), L.sl_lane_cls[c].begin(), L.sl_lane_cls[c].end());
+    L.sl_lane_cls[c] = std::vector<Item>();
+  }
+  L.off_sl_lane_items = take(sizeof(Item) * L.sl_lane_items.size());
   L.off_seg_items = take(sizeof(Item) * L.seg_items.size());
   L.off_segtot = take(sizeof(double) * kStatW * L.seg_items.size());
   L.off_el_items = take(sizeof(Item) * L.el_items.size());
@@ -1060,6 +1085,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_cast_items, L.cast_items.data(), sizeof(Item) * L.cast_items.size());
   if (e == hipSuccess) e = up(L.off_nd_items, L.nd_items.data(), sizeof(Item) * L.nd_items.size());
   if (e == hipSuccess) e = up(L.off_sl_items, L.sl_items.data(), sizeof(Item) * L.sl_items.size());
+  if (e == hipSuccess) e = up(L.off_sl_lane_items, L.sl_lane_items.data(), sizeof(Item) * L.sl_lane_items.size());
   if (e == hipSuccess) e = up(L.off_seg_items, L.seg_items.data(), sizeof(Item) * L.seg_items.size());
   if (e == hipSuccess) e = up(L.off_el_items, L.el_items.data(), sizeof(Item) * L.el_items.size());
   if (e == hipSuccess) e = up(L.off_ap_items, L.ap_items.data(), sizeof(Item) * L.ap_items.size());
@@ -1502,6 +1528,10 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
   }
   if (n_sl > 0)
     hipLaunchKernelGGL(k_celo2_slices, dim3(n_sl), dim3(kThreads), 0, s, descs, dyn, sl_items, fac_tab, gl, dec, mlp);
+  for (int c = 0, at = 0; c < kSliceLaneClasses; at += L.sl_lane_n[c], ++c)
+    if (L.sl_lane_n[c] > 0)
+      hipLaunchKernelGGL(k_celo2_slices_lane, dim3((unsigned)L.sl_lane_n[c]), dim3(64), L.sl_lane_lds[c], s, descs, dyn,
+                         P->at<Item>(L.off_sl_lane_items) + at, fac_tab, gl, dec, mlp);
   HIP_TRY(mark());
   mark.done();
   stage_out(P, s, 1);   // only the AdamW tensors were updated

@@ -192,20 +192,21 @@ def ns_flops_executed(shapes, iters=5, tile=128):
 
 def whole_step_object(whole_ms, finish_ms, n_params, flops, flops_exec):
     """The matrix-pipe part of the step against the peak of the pipe it runs on.  By default the products run
-    on the bf16 matrix instructions with every fp32 operand split into three bf16 planes: six bf16 products
-    per fp32 product, so the executed work is 6 x the fp32 FLOPs against the 2.5 PFLOP/s of dense bf16;
+    on the fp16 matrix instructions with every fp32 operand split into two fp16 planes (scaled by a power of
+    two): three fp16 products per fp32 product, so the executed work is 3 x the fp32 FLOPs against the
+    2.5 PFLOP/s of dense fp16;
     PYLO_MI355_NS_F32=1 runs them on the fp32 matrix instructions (157.3 TFLOP/s).  `achieved` counts the FLOPs
     the kernels execute (the symmetric halves they skip earn nothing); by the reference's full fp32 products the
     same time is `nominal_fp32_TFLOPs`."""
     f32 = os.environ.get("PYLO_MI355_NS_F32") == "1"
     t = finish_ms * 1e-3
-    mult, peak = (1.0, 157.3) if f32 else (6.0, 2500.0)
+    mult, peak = (1.0, 157.3) if f32 else (3.0, 2500.0)
     return {
         "ms": whole_ms, "params_per_sec": n_params / (whole_ms * 1e-3), "finish_ms": finish_ms,
         "newton_schulz_TFLOP": flops / 1e12, "newton_schulz_TFLOP_executed": flops_exec / 1e12,
         "roofline": {"bound": "mfma",
                      "kernel": ("k_ns_gemm (fp32 matrix instructions)" if f32 else
-                                "k_ns_bf_gemm (bf16 matrix instructions, 6 products per fp32 product)")
+                                "k_ns_bf_gemm (fp16 matrix instructions, 3 products per fp32 product)")
                                + " + finishing pass",
                      "achieved": mult * flops_exec / t / 1e12, "peak": peak, "unit": "TFLOP/s",
                      "frac": mult * flops_exec / t / 1e12 / peak,
@@ -426,7 +427,7 @@ def stream_ceiling(a):
 
 
 def matrix_ceiling(a):
-    """What the bf16 matrix pipe delivers for the instruction mix of the Newton-Schulz products: the library's
+    """What the fp16 matrix pipe delivers for the instruction mix of the Newton-Schulz products: the library's
     bare matrix-pipe kernel (the update product's main loop, 128 x 256 tiles, reduction length 768) on planes of
     the GPT-2-small set's size, with the data path taken away in steps, on random data and on zeros (the pipe's
     power, and with it the clock, depends on the operands).  The yardstick next to the data sheet's 2.5 PFLOP/s."""
@@ -444,16 +445,13 @@ def matrix_ceiling(a):
     res = {}
     for data in ("random", "zeros"):
         gen = torch.Generator(device=dev).manual_seed(0)
-        mk = (lambda n: torch.randint(-32768, 32767, (n,), generator=gen, device=dev, dtype=torch.int16)) if data == "random" \
-            else (lambda n: torch.zeros(n, device=dev, dtype=torch.int16))
-        # random bit patterns with the exponents of numbers around 1 (no NaN or infinity): sign, exponent 120..127, 7 mantissa bits
+        # random numbers around 1 (no NaN or infinity), as fp16 bit patterns
         def planes(n):
-            t = mk(n)
-            if data == "random":
-                t = (t & -32641) | (((t.to(torch.int32) >> 7) & 7) + 120).to(torch.int16) << 7
-            return t
-        x = planes(rows_x * k * 3)
-        b = planes(rows_b * k * 3)
+            if data == "zeros":
+                return torch.zeros(n, device=dev, dtype=torch.float16)
+            return (torch.randn(n, generator=gen, device=dev) * 0.5).to(torch.float16)
+        x = planes(rows_x * k * 2)
+        b = planes(rows_b * k * 2)
         out = torch.zeros((rows_x // 128) * (rows_b // 256) * 256, device=dev)
         for mode, name in ((0, "product loop"), (1, "LDS reads + matrix instructions"), (2, "matrix instructions only")):
             call = lambda: _lib.check(lib.pylo_mi355_matrix_probe(x.data_ptr(), rows_x, b.data_ptr(), rows_b, k, mode,
@@ -467,10 +465,10 @@ def matrix_ceiling(a):
             e1.record()
             torch.cuda.synchronize()
             ms = e0.elapsed_time(e1) / a.steps
-            res[f"{name}, {data}"] = {"ms": ms, "PFLOPs": 12.0 * rows_x * rows_b * k / ms / 1e12}
+            res[f"{name}, {data}"] = {"ms": ms, "PFLOPs": 6.0 * rows_x * rows_b * k / ms / 1e12}
         del x, b, out
-    print(json.dumps({"metric": "attainable_bf16_matrix_rate", "unit": "PFLOP/s", "n_gpus": 1, "steps": a.steps,
-                      "warmup": a.warmup, "tile": "128x256, 6 x v_mfma_f32_32x32x16_bf16 per fp32 tile product",
+    print(json.dumps({"metric": "attainable_fp16_matrix_rate", "unit": "PFLOP/s", "n_gpus": 1, "steps": a.steps,
+                      "warmup": a.warmup, "tile": "128x256, 3 x v_mfma_f32_32x32x16_f16 per fp32 tile product",
                       "peak_PFLOPs": 2.5, "cases": res}))
 
 

@@ -44,14 +44,17 @@
 
 namespace pylo {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef unsigned short bfbits;   // a bf16 in memory
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned short bfbits;   // one number of a plane in memory (an fp16)
+constexpr int kNsPl = 2;                      // planes per matrix
+constexpr int kNsRowB = 32 * kNsPl;           // bytes of one row in a block of 16 reduction steps
+constexpr int kNsRowPc = 2 * kNsPl;           // the same in 16-byte pieces
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) u32x4 luint4;
 
 constexpr int kBfBK = 16;                     // reduction steps per stage
-// LDS of a tile job with 64 WN columns: two stages of (128 + 64 WN) rows x 3 planes x 32 bytes
-constexpr int bf_gemm_lds(int wn) { return 2 * (128 + 64 * wn) * 96; }
+// LDS of a tile job with 64 WN columns: two stages of (128 + 64 WN) rows x 2 planes x 32 bytes
+constexpr int bf_gemm_lds(int wn) { return 2 * (128 + 64 * wn) * kNsRowB; }
 
 // Planes of one matrix with `rows` rows and a (padded) reduction length: stored in blocks of 16 reduction
 // steps, [k / 16][row][plane][k % 16], so that the 128 rows x 3 planes x 16 steps a tile job stages at a
@@ -62,9 +65,9 @@ struct BfPlanes {
   int rows;   // rows allocated (a multiple of the tiles' rows; rows past the matrix hold zeros)
 };
 
-// element offset of (row, k) in plane 0; planes 1 and 2 are 16 and 32 elements further
+// element offset of (row, k) in plane 0; plane 1 is 16 elements further
 __device__ __forceinline__ size_t bf_off(int rows, int row, int k) {
-  return ((size_t)(k >> 4) * rows + row) * 48 + (k & 15);
+  return ((size_t)(k >> 4) * rows + row) * (16 * kNsPl) + (k & 15);
 }
 
 struct NsBfMat {
@@ -87,72 +90,73 @@ struct NsBfMat {
 // kNsGram / kNsPoly / kNsUpdate)
 enum : int { kNsBufA = 0, kNsBufB = 1, kNsBufT = 2, kNsBufC = 3, kNsBufs = 4 };
 enum : int { kNsProd = 3, kNsProdA = 4 };
-struct NsBufs { int s1, s2, d; };   // operand and result buffers of an m x m product; the update's B' is s1
+// operand and result buffers of an m x m product (the update's B' is s1); what turns the accumulators into the
+// product's values (the reciprocal of the operands' plane scales) and the scale of the planes written
+struct NsBufs { int s1, s2, d; float acc_scale, out_scale; };
 
-__device__ __forceinline__ float bf_to_float(bfbits b) { return __uint_as_float((unsigned)b << 16); }
-
-// x = h + m + l
-__device__ __forceinline__ void bf_split(float x, bfbits& h, bfbits& m, bfbits& l) {
-  const __bf16 hb = (__bf16)x;
-  const float r1 = x - (float)hb;
-  const __bf16 mb = (__bf16)r1;
-  const float r2 = r1 - (float)mb;
-  const __bf16 lb = (__bf16)r2;
+// x (already times its plane scale) = h + l + what is left below 2^-22 |x|.  The clamp never acts on a matrix
+// within the bounds the scales were chosen for; it keeps a stray value from becoming an infinity.
+__device__ __forceinline__ void hf_split(float x, bfbits& h, bfbits& l) {
+  x = __builtin_amdgcn_fmed3f(x, -65000.0f, 65000.0f);
+  const _Float16 hb = (_Float16)x;
+  const _Float16 lb = (_Float16)(x - (float)hb);
   h = __builtin_bit_cast(bfbits, hb);
-  m = __builtin_bit_cast(bfbits, mb);
   l = __builtin_bit_cast(bfbits, lb);
 }
 
-// A stage of one operand in LDS: [row][plane][half], 96 bytes a row, as in memory, except that the two
-// 16-byte halves are swapped for every other group of eight rows (rows 8 apart would share banks).
+// A stage of one operand in LDS: [row][plane][half], 64 bytes a row, as in memory, except that the four
+// 16-byte pieces of a row are permuted: piece s of row r sits in slot s ^ ((r / 4) % 4), so that sixteen
+// consecutive rows, read one piece each by sixteen lanes, touch sixteen different 16-byte bank groups (rows 4
+// apart would share them).
 // A wave-wide load instruction moves 64 consecutive 16-byte pieces of the stage from global memory into LDS
-// (the hardware puts lane l's piece at the instruction's LDS base + 16 l); the swap is done on the global
-// side: lane l fetches the piece whose place in LDS it fills.  ROWS x 6 pieces = ROWS x 6 / 256 instructions
+// (the hardware puts lane l's piece at the instruction's LDS base + 16 l); the permutation is done on the global
+// side: lane l fetches the piece whose place in LDS it fills.  ROWS x 4 pieces = ROWS x 4 / 256 instructions
 // per thread; `off[]` holds the lane's byte offsets into the stage in memory (they do not change with k).
 #define PYLO_LDS __attribute__((address_space(3)))
 #define PYLO_GLB __attribute__((address_space(1)))
 
 template <int ROWS>
-__device__ __forceinline__ void bf_stage_offsets(int wave, int lane, int (&off)[ROWS * 6 / 256]) {
+__device__ __forceinline__ void bf_stage_offsets(int wave, int lane, int (&off)[ROWS * kNsRowPc / 256]) {
 #pragma unroll
-  for (int j = 0; j < ROWS * 6 / 256; ++j) {
+  for (int j = 0; j < ROWS * kNsRowPc / 256; ++j) {
     const int p = (j * 4 + wave) * 64 + lane;
-    off[j] = (p ^ (((p / 6) >> 3) & 1)) * 16;
+    off[j] = (p ^ ((p >> 4) & 3)) * 16;   // row p / 4: its four pieces permuted by (row / 4) % 4
   }
 }
 
 template <int ROWS>
-__device__ __forceinline__ void bf_stage_issue(const char* g, const int (&off)[ROWS * 6 / 256], PYLO_LDS char* lds, int wave) {
+__device__ __forceinline__ void bf_stage_issue(const char* g, const int (&off)[ROWS * kNsRowPc / 256], PYLO_LDS char* lds, int wave) {
 #pragma unroll
-  for (int j = 0; j < ROWS * 6 / 256; ++j)
+  for (int j = 0; j < ROWS * kNsRowPc / 256; ++j)
     __builtin_amdgcn_global_load_lds((const PYLO_GLB void*)(g + off[j]), (PYLO_LDS void*)(lds + (j * 4 + wave) * 1024), 16, 0, 0);
 }
 
 // acc[hi][hj] += (rows i0.. of P1) x (rows j0.. of P2)^T over the reduction range [k0, k1) (multiples of 16);
-// 128 rows of P1, 64 WN rows of P2.  LDS: two stages of (128 + 64 WN) x 96 bytes.
+// 128 rows of P1, 64 WN rows of P2.  LDS: two stages of (128 + 64 WN) x 64 bytes.
 // `compute` (the same for all lanes of a wave): false for a wave whose values nobody needs -- it stages and meets the
 // barriers, and leaves the matrix pipe to the other waves of its SIMD.
 template <int WN>
 __device__ __forceinline__ void bf_tile_product(const BfPlanes& P1, int i0, const BfPlanes& P2, int j0, int k0, int k1,
                                                 PYLO_LDS char* lds, v16f (&acc)[2][WN], bool compute = true) {
-  constexpr int RB = 64 * WN, SA = 128 * 96, STAGE = SA + RB * 96;
+  constexpr int RB = 64 * WN, SA = 128 * kNsRowB, STAGE = SA + RB * kNsRowB;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wi = (wave >> 1) * 64, wj = (wave & 1) * 32 * WN;
   const int kg = lane >> 5, lo = lane & 31;
-  int offa[3], offb[RB * 6 / 256];
+  int offa[128 * kNsRowPc / 256], offb[RB * kNsRowPc / 256];
   bf_stage_offsets<128>(wave, lane, offa);
   bf_stage_offsets<RB>(wave, lane, offb);
-  const char* ga = (const char*)P1.base + ((size_t)(k0 >> 4) * P1.rows + i0) * 96;
-  const char* gb = (const char*)P2.base + ((size_t)(k0 >> 4) * P2.rows + j0) * 96;
-  const size_t sa = (size_t)P1.rows * 96, sb = (size_t)P2.rows * 96;
+  const char* ga = (const char*)P1.base + ((size_t)(k0 >> 4) * P1.rows + i0) * kNsRowB;
+  const char* gb = (const char*)P2.base + ((size_t)(k0 >> 4) * P2.rows + j0) * kNsRowB;
+  const size_t sa = (size_t)P1.rows * kNsRowB, sb = (size_t)P2.rows * kNsRowB;
   // a diagonal tile of X X^T or A A: both operands are the same 128 rows, staged once
   const bool same = WN == 2 && P1.base == P2.base && i0 == j0;
   bf_stage_issue<128>(ga, offa, lds, wave);
   if (!same) bf_stage_issue<RB>(gb, offb, lds + SA, wave);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
-  const int sw = 16 * (kg ^ ((lo >> 3) & 1));
-  const int oa = (wi + lo) * 96 + sw, ob = (same ? 0 : SA) + (wj + lo) * 96 + sw;
+  // the lane's rows are lo, lo + 32, ..: all with the same (row / 4) % 4; plane q, half kg is piece 2 q + kg
+  const int sw = 16 * (kg ^ ((lo >> 2) & 3));
+  const int oa = (wi + lo) * kNsRowB + sw, ob = (same ? 0 : SA) + (wj + lo) * kNsRowB + sw;
   int cur = 0;
   for (int k = k0; k < k1; k += kBfBK) {
     if (k + kBfBK < k1) {
@@ -162,23 +166,25 @@ __device__ __forceinline__ void bf_tile_product(const BfPlanes& P1, int i0, cons
       if (!same) bf_stage_issue<RB>(gb, offb, lds + (STAGE - cur) + SA, wave);
     }
     if (compute) {
-      bf16x8 a[2][3], b[WN][3];
+      f16x8 a[2][kNsPl], b[WN][kNsPl];
 #pragma unroll
-      for (int q = 0; q < 3; ++q) {
+      for (int q = 0; q < kNsPl; ++q) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) a[i][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + oa + i * 32 * 96 + q * 32));
+        for (int i = 0; i < 2; ++i)
+          a[i][q] = __builtin_bit_cast(f16x8, *(const luint4*)(lds + cur + ((oa + i * 32 * kNsRowB) ^ (q * 32))));
 #pragma unroll
-        for (int j = 0; j < WN; ++j) b[j][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + cur + ob + j * 32 * 96 + q * 32));
+        for (int j = 0; j < WN; ++j)
+          b[j][q] = __builtin_bit_cast(f16x8, *(const luint4*)(lds + cur + ((ob + j * 32 * kNsRowB) ^ (q * 32))));
       }
-      // smallest terms first: l h, h l, m m, m h, h m, h h
+      // smallest terms first: l h, h l, h h
 #pragma unroll
-      for (int term = 0; term < 6; ++term) {
-        constexpr int pa[6] = {2, 0, 1, 1, 0, 0}, pb[6] = {0, 2, 1, 0, 1, 0};
+      for (int term = 0; term < 3; ++term) {
+        constexpr int pa[3] = {1, 0, 0}, pb[3] = {0, 1, 0};
 #pragma unroll
         for (int hi = 0; hi < 2; ++hi)
 #pragma unroll
           for (int hj = 0; hj < WN; ++hj)
-            acc[hi][hj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[hi][pa[term]], b[hj][pb[term]], acc[hi][hj], 0, 0, 0);
+            acc[hi][hj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[hi][pa[term]], b[hj][pb[term]], acc[hi][hj], 0, 0, 0);
       }
     }
     // the loads into the other stage have landed (they are counted like any other vector-memory load) and
@@ -189,32 +195,21 @@ __device__ __forceinline__ void bf_tile_product(const BfPlanes& P1, int i0, cons
   }
 }
 
-// Four values at consecutive reduction indices k .. k + 3 (k a multiple of 4) of one row: one 8-byte store per plane.
-__device__ __forceinline__ void bf_store4(bfbits* base, int rows, int row, int k, const float (&v)[4]) {
-  bfbits h[4], m[4], l[4];
-#pragma unroll
-  for (int r = 0; r < 4; ++r) bf_split(v[r], h[r], m[r], l[r]);
-  typedef unsigned long long u64;
-  bfbits* p = base + bf_off(rows, row, k);
-  *(u64*)p = (u64)h[0] | (u64)h[1] << 16 | (u64)h[2] << 32 | (u64)h[3] << 48;
-  *(u64*)(p + 16) = (u64)m[0] | (u64)m[1] << 16 | (u64)m[2] << 32 | (u64)m[3] << 48;
-  *(u64*)(p + 32) = (u64)l[0] | (u64)l[1] << 16 | (u64)l[2] << 32 | (u64)l[3] << 48;
-}
-
+// one value (times its plane scale already) into both planes
 __device__ __forceinline__ void bf_store1(bfbits* base, int rows, int row, int k, float v) {
-  bfbits h, m, l;
-  bf_split(v, h, m, l);
+  bfbits h, l;
+  hf_split(v, h, l);
   bfbits* p = base + bf_off(rows, row, k);
   p[0] = h;
-  p[16] = m;
-  p[32] = l;
+  p[16] = l;
 }
 
-// The block's 128 x 64 WN values (accumulator layout) into planes, in one or both orientations, every value
-// split once.
+// The block's 128 x 64 WN values (accumulator layout) times `scale` into planes, in one or both orientations, every
+// value split once.
 //   D   planes whose reduction index is the tile's column index: through the wave's own LDS patch
 //       ([row][plane][32 WN columns], 2 bytes each), 16 rows at a time; the wave reads the patch back as
-//       16-byte pieces in the order the planes have in memory ([16 columns][row][plane][half]).
+//       16-byte pieces in the order the planes have in memory ([16 columns][row][plane][half]: 64 pieces for the
+//       patch's 16 rows, one a lane).
 //   D4  (when not null) planes whose reduction index is the tile's row index: four consecutive rows of a
 //       lane are four consecutive reduction indices, one 8-byte store per plane straight from the registers.
 // Only the lanes of one wave meet in a patch and a wave's LDS instructions execute in order, so the passes
@@ -222,9 +217,9 @@ __device__ __forceinline__ void bf_store1(bfbits* base, int rows, int row, int k
 template <int WN>
 __device__ __forceinline__ void bf_store_planes(PYLO_LDS char* lds, const v16f (&acc)[2][WN], bfbits* __restrict__ D,
                                                 int rows_total, int i0, int j0, int n_rows, int n_cols,
-                                                bfbits* __restrict__ D4, int rows4) {
+                                                bfbits* __restrict__ D4, int rows4, float scale) {
   constexpr int kPlane = 64 * WN + 16;        // bytes: 32 WN columns x 2 + 16 (bank spread)
-  constexpr int kRow = 3 * kPlane, kWave = 16 * kRow;
+  constexpr int kRow = kNsPl * kPlane, kWave = 16 * kRow;
   typedef PYLO_LDS bfbits lbf;
   typedef unsigned long long u64;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -238,23 +233,21 @@ __device__ __forceinline__ void bf_store_planes(PYLO_LDS char* lds, const v16f (
     for (int hj = 0; hj < WN; ++hj)
 #pragma unroll
       for (int g4 = 0; g4 < 2; ++g4) {
-        bfbits h[4], m[4], l[4];
+        bfbits h[4], l[4];
         const int col_l = 32 * hj + (lane & 31);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          bf_split(acc[hi][hj][8 * half + 4 * g4 + r], h[r], m[r], l[r]);
+          hf_split(acc[hi][hj][8 * half + 4 * g4 + r] * scale, h[r], l[r]);
           lbf* q = (lbf*)(patch + (8 * g4 + 4 * (lane >> 5) + r) * kRow + col_l * 2);
           q[0] = h[r];
-          q[kPlane / 2] = m[r];
-          q[kPlane] = l[r];
+          q[kPlane / 2] = l[r];
         }
         if (D4 != nullptr) {
           const int row = wi + 32 * hi + 16 * half + 8 * g4 + 4 * (lane >> 5), col = wj + col_l;
           if (col < n_cols && row < n_rows) {   // values past n_rows are zeros, into the padding
             bfbits* p = D4 + bf_off(rows4, col, row);
             *(u64*)p = (u64)h[0] | (u64)h[1] << 16 | (u64)h[2] << 32 | (u64)h[3] << 48;
-            *(u64*)(p + 16) = (u64)m[0] | (u64)m[1] << 16 | (u64)m[2] << 32 | (u64)m[3] << 48;
-            *(u64*)(p + 32) = (u64)l[0] | (u64)l[1] << 16 | (u64)l[2] << 32 | (u64)l[3] << 48;
+            *(u64*)(p + 16) = (u64)l[0] | (u64)l[1] << 16 | (u64)l[2] << 32 | (u64)l[3] << 48;
           }
         }
       }
@@ -265,15 +258,10 @@ __device__ __forceinline__ void bf_store_planes(PYLO_LDS char* lds, const v16f (
       const int col = wj + 16 * c;
       if (col >= n_cols) continue;
       bfbits* dst = D + bf_off(rows_total, row_w0, col);
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {        // 96 pieces: [row][plane][half]
-        const int pc = lane + 64 * j;
-        if (pc >= 96) continue;
-        const int row_l = pc / 6, rem = pc - 6 * row_l, plane = rem >> 1, hf = rem & 1;
-        if (row_w0 + row_l >= n_rows) continue;
-        const u32x4 w = *(const luint4*)(patch + row_l * kRow + plane * kPlane + (16 * c + 8 * hf) * 2);
-        *(u32x4*)(dst + (size_t)pc * 8) = w;
-      }
+      const int row_l = lane >> 2, plane = (lane >> 1) & 1, hf = lane & 1;   // piece `lane` of [row][plane][half]
+      if (row_w0 + row_l >= n_rows) continue;
+      const u32x4 w = *(const luint4*)(patch + row_l * kRow + plane * kPlane + (16 * c + 8 * hf) * 2);
+      *(u32x4*)(dst + (size_t)lane * 8) = w;
     }
   }
 }
@@ -293,6 +281,7 @@ enum : int { kNsAll = 0, kNsLongOnly = 1, kNsShortOnly = 2, kNsBoth = 3 };
 struct NsPick {
   const int* flags;
   int sel, s1_short, last_short;
+  float acc_scale_short;   // with s1_short: that buffer's planes have a scale of their own
 };
 
 template <int OP, int WN>
@@ -309,6 +298,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
     if ((pick.sel == kNsLongOnly && !longer) || (pick.sel == kNsShortOnly && longer)) return;
     if (pick.sel == kNsBoth && !longer) {
       bufs.s1 = pick.s1_short;
+      bufs.acc_scale = pick.acc_scale_short;
       last = pick.last_short;
     }
   }
@@ -345,6 +335,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
     bf_tile_product<WN>(P1, i0, P2, j0, it.k0, it.k1, lds, acc, !idle);
   }
   if (idle) return;
+  // the operands' planes hold their matrices times a power of two each
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] *= bufs.acc_scale;
   float* A32 = ws + mt.off_a;
   const int n_i = OP == kNsUpdate ? n : m;   // rows of the output; its columns are always m
   const bool partial = OP == kNsGram && it.slab >= 0;
@@ -401,17 +398,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
   // (through LDS) and Xs' (registers)
   if (partial || (OP == kNsUpdate && last)) return;
   if (OP == kNsUpdate) {
-    bf_store_planes<WN>(lds, acc, pw + (par ? mt.off_xl[0] : mt.off_xl[1]), mt.rows_n, i0, j0, n, m, pw + mt.off_xs, mt.rows_m);
+    bf_store_planes<WN>(lds, acc, pw + (par ? mt.off_xl[0] : mt.off_xl[1]), mt.rows_n, i0, j0, n, m, pw + mt.off_xs, mt.rows_m,
+                        bufs.out_scale);
   } else {
     bfbits* D = pw + mt.off_p + (OP == kNsGram ? (int)kNsBufA : bufs.d) * mt.p_stride;
-    bf_store_planes<WN>(lds, acc, D, mt.rows_m, i0, j0, m, m, mirror ? D : nullptr, mt.rows_m);
+    bf_store_planes<WN>(lds, acc, D, mt.rows_m, i0, j0, m, m, mirror ? D : nullptr, mt.rows_m, bufs.out_scale);
   }
 }
 
 // A = sum over the slabs' partial matrices, in slab order, as fp32 and as planes (both halves).
 __global__ __launch_bounds__(256) void k_ns_bf_gram_reduce(const NsBfMat* __restrict__ mats, const int* __restrict__ split_mats,
                                                            const PyloTensorArgs* __restrict__ dyn, float* __restrict__ ws,
-                                                           bfbits* __restrict__ pw, NsPick pick) {
+                                                           bfbits* __restrict__ pw, NsPick pick, float out_scale) {
   if (pick.sel == kNsShortOnly && pick.flags[split_mats[blockIdx.y]] != 0) return;
   const NsBfMat mt = mats[split_mats[blockIdx.y]];
   const PyloTensorArgs a = dyn[mt.tensor];
@@ -434,10 +432,10 @@ __global__ __launch_bounds__(256) void k_ns_bf_gram_reduce(const NsBfMat* __rest
   float* A = ws + mt.off_a;
   bfbits* P = pw + mt.off_p;   // buffer A
   A[(size_t)i * lda + j] = s;
-  bf_store1(P, mt.rows_m, i, j, s);
+  bf_store1(P, mt.rows_m, i, j, s * out_scale);
   if (i / 64 != j / 64) {
     A[(size_t)j * lda + i] = s;
-    bf_store1(P, mt.rows_m, j, i, s);
+    bf_store1(P, mt.rows_m, j, i, s * out_scale);
   }
 }
 
@@ -493,14 +491,14 @@ struct NsTileItem { int mat, tr, tc; };
 
 __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__ mats, const NsTileItem* __restrict__ items,
                                                      const PyloTensorArgs* __restrict__ dyn, const float* __restrict__ scale,
-                                                     bfbits* __restrict__ pw) {
-  constexpr int RP = 72;   // bf16 per row of the tile in LDS: 64 + 8, rows stay 16-byte aligned
-  __shared__ __attribute__((aligned(16))) bfbits tile[3][64][RP];
+                                                     bfbits* __restrict__ pw, float plane_scale) {
+  constexpr int RP = 72;   // numbers per row of the tile in LDS: 64 + 8, rows stay 16-byte aligned
+  __shared__ __attribute__((aligned(16))) bfbits tile[kNsPl][64][RP];
   const NsTileItem it = items[blockIdx.x];
   const NsBfMat mt = mats[it.mat];
   const PyloTensorArgs a = dyn[mt.tensor];
   if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
-  const float s = scale[it.mat];
+  const float s = scale[it.mat] * plane_scale;
   const int R = mt.R, C = mt.C;
   const float* raw = a.step_out + mt.elem_off;
   const bool vec_in = (C & 3) == 0;
@@ -511,7 +509,7 @@ __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__
   const int r0 = it.tr * 64, c0 = it.tc * 64;
   const int t = threadIdx.x;
   // Eight consecutive columns of one row a lane and pass: 32 bytes read, one 16-byte piece per plane written
-  // to the direct planes (the two lanes of a 16-column block fill its 96 bytes) and to the tile in LDS.
+  // to the direct planes (the two lanes of a 16-column block fill its 64 bytes) and to the tile in LDS.
   // Columns and rows past the matrix read as zero; where a piece straddles the edge the zeros land in the
   // planes' padding, which holds zeros anyway.
 #pragma unroll
@@ -535,34 +533,33 @@ __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__
           if (c + e < C) v[e] = *(const gfloat*)(src + e) * s;
       }
     }
-    u32x4 pl[3];
+    u32x4 pl[kNsPl];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      bfbits h0, m0, l0, h1, m1, l1;
-      bf_split(v[2 * q], h0, m0, l0);
-      bf_split(v[2 * q + 1], h1, m1, l1);
+      bfbits h0, l0, h1, l1;
+      hf_split(v[2 * q], h0, l0);
+      hf_split(v[2 * q + 1], h1, l1);
       pl[0][q] = (unsigned)h0 | (unsigned)h1 << 16;
-      pl[1][q] = (unsigned)m0 | (unsigned)m1 << 16;
-      pl[2][q] = (unsigned)l0 | (unsigned)l1 << 16;
+      pl[1][q] = (unsigned)l0 | (unsigned)l1 << 16;
     }
 #pragma unroll
-    for (int q = 0; q < 3; ++q) *(luint4*)&tile[q][lr][lc] = pl[q];
+    for (int q = 0; q < kNsPl; ++q) *(luint4*)&tile[q][lr][lc] = pl[q];
     if (in) {
       bfbits* p = direct + bf_off(rows_d, r, c);
 #pragma unroll
-      for (int q = 0; q < 3; ++q) *(u32x4*)(p + 16 * q) = pl[q];
+      for (int q = 0; q < kNsPl; ++q) *(u32x4*)(p + 16 * q) = pl[q];
     }
   }
   __syncthreads();
   // transposed: a lane takes one column and sixteen rows of the tile, i.e. one row and one 16-step block of
-  // the transposed planes: 96 consecutive bytes, and the lanes of a wave (consecutive columns) the next 96
+  // the transposed planes: 64 consecutive bytes, and the lanes of a wave (consecutive columns) the next 64
   {
     const int lc = t & 63, rb = t >> 6;
     const int c = c0 + lc, r = r0 + 16 * rb;
     if (c < C && r < R) {
       bfbits* p = transp + bf_off(rows_t, c, r);
 #pragma unroll
-      for (int q = 0; q < 3; ++q)
+      for (int q = 0; q < kNsPl; ++q)
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
           u32x4 w;

@@ -319,6 +319,54 @@ bool ns_adaptive() {
   return !(c && c[0]);
 }
 
+// The planes of the Newton-Schulz products are fp16 numbers: every matrix is stored times a power of two that puts its
+// largest possible entry at 12 000 .. 24 000 (the format ends at 65 504), so that the second plane keeps its bits on
+// entries five decades smaller.  No entry exceeds the matrix's largest singular value, and those follow from the
+// coefficients alone: X0 has unit Frobenius norm, so its singular values lie in [0, 1], and every iteration maps
+// sigma to sigma p(sigma^2), p(l) = c2 l^2 + c1 l + c0.  Bounds over all iterations, from a grid of starting values:
+// X (sigma), A = X X^T (sigma^2), B' = p(A), T = A B', and the products of k consecutive B' (q[k], k >= 1).
+struct NsExps {
+  int x, a, b, t;
+  std::vector<int> q;
+};
+inline float pow2(int e) { return std::ldexp(1.0f, e); }
+NsExps ns_plane_exps(float c0, float c1, float c2, int iters) {
+  constexpr int kGrid = 2048;
+  const int n = std::max(iters, 1);
+  double bx = 1.0, ba = 1.0, bb = std::fabs((double)c0), bt = 0.0;
+  std::vector<double> bq(n + 1, 0.0), pv(n);
+  for (int g = 0; g <= kGrid; ++g) {
+    double sig = (double)g / kGrid;
+    for (int t = 0; t < n; ++t) {
+      const double l = sig * sig, pl = (double)c2 * l * l + (double)c1 * l + (double)c0;
+      pv[t] = std::fabs(pl);
+      ba = std::max(ba, l);
+      bb = std::max(bb, pv[t]);
+      bt = std::max(bt, l * pv[t]);
+      sig *= pl;
+      bx = std::max(bx, std::fabs(sig));
+    }
+    for (int t0 = 0; t0 < n; ++t0) {
+      double prod = 1.0;
+      for (int k = 1; t0 + k <= n; ++k) {
+        prod *= pv[t0 + k - 1];
+        bq[k] = std::max(bq[k], prod);
+      }
+    }
+  }
+  auto exp_of = [](double bound) {
+    if (!(bound > 0.0) || !std::isfinite(bound)) return -60;   // (coefficients that diverge: nothing to keep)
+    const int e = (int)std::floor(std::log2(30000.0 / (1.25 * bound)));
+    return std::max(-60, std::min(e, 14));
+  };
+  NsExps ex;
+  ex.x = exp_of(bx); ex.a = exp_of(ba); ex.b = exp_of(bb); ex.t = exp_of(bt);
+  ex.q.resize(n + 1);
+  for (int k = 1; k <= n; ++k) ex.q[k] = exp_of(bq[k]);
+  ex.q[0] = ex.b;
+  return ex;
+}
+
 // PYLO_MI355_SLICES_LDS=0: the short slices of ELO-CELO2 tensors with more than two dims stay on the kernel that reads
 // them straight from memory, twice (k_celo2_slices); read at plan creation.
 bool env_slices_lds() {
@@ -453,10 +501,10 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       b.rows_n = up(b.n, kNsTile);
       b.lda = up(b.m, 4);
       b.n_slabs = f.n_slabs;
-      b.p_stride = (3ll * b.rows_m * b.pad_m + 63) / 64 * 64;
+      b.p_stride = ((long long)kNsPl * b.rows_m * b.pad_m + 63) / 64 * 64;
       // (the matrices of one tensor -- the slices of one with more than two dims -- stay in one batch)
       const bool first_of_tensor = q == 0 || L.ns_mats[q - 1].tensor != f.tensor;
-      const long long need = (3ll * b.rows_m * b.pad_n + 6ll * b.rows_n * b.pad_m + kNsBufs * b.p_stride + 4 * 64) *
+      const long long need = ((long long)kNsPl * b.rows_m * b.pad_n + 2ll * kNsPl * b.rows_n * b.pad_m + kNsBufs * b.p_stride + 4 * 64) *
                              (first_of_tensor ? mats_of_tensor(q) : 1);
       if (pw > 0 && first_of_tensor && pw + need > budget) {   // this tensor opens the next batch
         batch.plane_elems = pw;
@@ -466,9 +514,9 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
         pw = 0;
         ws_floats = 0;
       }
-      b.off_xs = take_p(3ll * b.rows_m * b.pad_n);
-      b.off_xl[0] = take_p(3ll * b.rows_n * b.pad_m);
-      b.off_xl[1] = take_p(3ll * b.rows_n * b.pad_m);
+      b.off_xs = take_p((long long)kNsPl * b.rows_m * b.pad_n);
+      b.off_xl[0] = take_p((long long)kNsPl * b.rows_n * b.pad_m);
+      b.off_xl[1] = take_p((long long)kNsPl * b.rows_n * b.pad_m);
       b.off_p = take_p(kNsBufs * b.p_stride);
       b.off_a = take((long long)b.m * b.lda);
       b.off_part = b.n_slabs > 1 ? take((long long)b.n_slabs * b.m * b.lda) : 0;
@@ -1678,6 +1726,7 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
     const bool several = L.ns_batches.size() > 1;
     const float c0 = coeffs[0], c1 = coeffs[1], c2 = coeffs[2];
     const std::vector<int> chains = ns_chains(ns_iters);
+    const NsExps ex = ns_plane_exps(c0, c1, c2, ns_iters);
     // chain lengths chosen per matrix on the device: an odd iteration count of three or more, nothing given in the environment
     const bool adaptive = ns_adaptive() && ns_iters >= 3 && (ns_iters & 1);
     int* chain_flags = P->at<int>(L.off_ns_flags);
@@ -1709,55 +1758,66 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
                              ns_eps, scale);
         if (G.n_sitems > 0)
           hipLaunchKernelGGL(k_ns_bf_split, dim3((unsigned)G.n_sitems), dim3(256), 0, sg, bmats, sitems + G.sitem0, dyn,
-                             (const float*)scale, pw);
+                             (const float*)scale, pw, pow2(ex.x));
       }
       // The launch sequence of one group (every group runs the same one on its own tables), then its launches,
       // interleaved over the groups so that every stream is fed in turn.
       enum OpKind { kOpGram, kOpFlag, kOpPoly, kOpProd, kOpProdA, kOpUpdate };
       struct Op { OpKind kind; NsBufs b; int par, last; NsPick pick; };
       std::vector<Op> ops;
-      const NsPick all{nullptr, kNsAll, 0, 0};
+      const NsPick all{nullptr, kNsAll, 0, 0, 0.0f};
       int par = 0;   // which Xl buffer the next update reads
       // A is buffer A throughout; B' of the latest iteration in `bprev`, the product of all B' so far in `q`
-      int bprev = kNsBufB, q = kNsBufB;
+      // (`nq` of them); eb[]: the exponent of the scale of the planes in each buffer
+      int bprev = kNsBufB, q = kNsBufB, nq = 1;
+      int eb[kNsBufs] = {};
+      // the accumulators of a product of planes with exponents e1 and e2, and planes out with exponent ed
+      auto bufs = [&](int s1, int s2, int d, int e1, int e2, int ed) {
+        if (d >= 0) eb[d] = ed;
+        return NsBufs{s1, s2, d < 0 ? 0 : d, pow2(-(e1 + e2)), pow2(ed)};
+      };
       auto extend = [&](NsPick pk) {   // one more iteration into the chain: A <- B' A B', the next B', Q <- B' Q
         int free_buf[2], nf = 0;
         for (int b : {kNsBufB, kNsBufT, kNsBufC})
           if (b != bprev && b != q && nf < 2) free_buf[nf++] = b;
         const int t = free_buf[0];
-        ops.push_back(Op{kOpProd, NsBufs{kNsBufA, bprev, t}, par, 0, pk});
-        ops.push_back(Op{kOpProdA, NsBufs{bprev, t, kNsBufA}, par, 0, pk});
-        ops.push_back(Op{kOpPoly, NsBufs{kNsBufA, kNsBufA, t}, par, 0, pk});
+        ops.push_back(Op{kOpProd, bufs(kNsBufA, bprev, t, ex.a, eb[bprev], ex.t), par, 0, pk});
+        ops.push_back(Op{kOpProdA, bufs(bprev, t, kNsBufA, eb[bprev], ex.t, ex.a), par, 0, pk});
+        ops.push_back(Op{kOpPoly, bufs(kNsBufA, kNsBufA, t, ex.a, ex.a, ex.b), par, 0, pk});
         const int qn = q == bprev ? free_buf[1] : bprev;   // (the old B' is done with)
-        ops.push_back(Op{kOpProd, NsBufs{t, q, qn}, par, 0, pk});
+        ++nq;
+        ops.push_back(Op{kOpProd, bufs(t, q, qn, ex.b, eb[q], ex.q[std::min<size_t>(nq, ex.q.size() - 1)]), par, 0, pk});
         bprev = t;
         q = qn;
       };
       auto open_chain = [&](NsPick pk) {   // Gram product and the first B'
-        ops.push_back(Op{kOpGram, NsBufs{0, 0, kNsBufA}, par, 0, pk});
-        ops.push_back(Op{kOpPoly, NsBufs{kNsBufA, kNsBufA, kNsBufB}, par, 0, pk});
+        ops.push_back(Op{kOpGram, bufs(0, 0, kNsBufA, ex.x, ex.x, ex.a), par, 0, pk});
+        ops.push_back(Op{kOpPoly, bufs(kNsBufA, kNsBufA, kNsBufB, ex.a, ex.a, ex.b), par, 0, pk});
         bprev = q = kNsBufB;
+        nq = 1;
+      };
+      auto update = [&](int last, NsPick pk) {   // X <- Q X
+        ops.push_back(Op{kOpUpdate, bufs(q, 0, -1, ex.x, eb[q], ex.x), par, last, pk});
+        par ^= 1;
       };
       if (adaptive) {
         // First chain: two iterations for every matrix, a third for those whose flag says so (k_ns_bf_chain_flag),
         // then pairs for all -- the last of them is the end for the flagged ones -- and one iteration more for the others.
-        const NsPick longer{chain_flags, kNsLongOnly, 0, 0}, shorter{chain_flags, kNsShortOnly, 0, 0};
+        const NsPick longer{chain_flags, kNsLongOnly, 0, 0, 0.0f}, shorter{chain_flags, kNsShortOnly, 0, 0, 0.0f};
         const int n_pairs = (ns_iters - 3) / 2;
         open_chain(all);
-        ops.push_back(Op{kOpFlag, NsBufs{0, 0, 0}, par, 0, all});
+        ops.push_back(Op{kOpFlag, NsBufs{0, 0, 0, 0.0f, 0.0f}, par, 0, all});
         extend(all);
-        const int q_short = q;
+        const int q_short = q, e_short = eb[q];
         extend(longer);
-        ops.push_back(Op{kOpUpdate, NsBufs{q, 0, 0}, par, n_pairs == 0, NsPick{chain_flags, kNsBoth, q_short, 0}});
-        par ^= 1;
+        update(n_pairs == 0, NsPick{chain_flags, kNsBoth, q_short, 0, pow2(-(ex.x + e_short))});
         for (int p = 0; p < n_pairs; ++p) {
           open_chain(all);
           extend(all);
-          ops.push_back(Op{kOpUpdate, NsBufs{q, 0, 0}, par, p == n_pairs - 1, NsPick{chain_flags, kNsBoth, q, 0}});
-          par ^= 1;
+          update(p == n_pairs - 1, NsPick{chain_flags, kNsBoth, q, 0, pow2(-(ex.x + eb[q]))});
         }
         open_chain(shorter);
-        ops.push_back(Op{kOpUpdate, NsBufs{q, 0, 0}, par, 1, shorter});
+        update(1, shorter);
       } else {
         int done = 0;
         for (size_t ch = 0; ch < chains.size(); ++ch) {
@@ -1765,8 +1825,7 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
           done += chains[ch];
           open_chain(all);
           for (int j = 1; j < chains[ch]; ++j) extend(all);
-          ops.push_back(Op{kOpUpdate, NsBufs{q, 0, 0}, par, done == ns_iters, all});
-          par ^= 1;
+          update(done == ns_iters, all);
         }
       }
       for (const Op& op : ops)
@@ -1785,7 +1844,7 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
                                    gram + G.gram0, dyn, ns_ws, pw, op.par, op.last, op.b, c0, c1, c2, op.pick);
               if (G.n_split > 0)
                 hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)G.split_max_m * G.split_max_m + 255) / 256, G.n_split),
-                                   dim3(256), 0, sg, bmats, split + G.split0, dyn, ns_ws, pw, op.pick);
+                                   dim3(256), 0, sg, bmats, split + G.split0, dyn, ns_ws, pw, op.pick, op.b.out_scale);
               break;
             case kOpFlag:
               if (G.n_list > 0) {
@@ -2458,12 +2517,12 @@ extern "C" int pylo_mi355_stream_probe(const float* in, float* out, size_t n, in
 }
 
 // ---------------------------------------------------------------------------------------------
-// Bare matrix-pipe kernel (benchmark instrumentation): what the bf16 matrix instructions deliver for the
+// Bare matrix-pipe kernel (benchmark instrumentation): what the fp16 matrix instructions deliver for the
 // instruction mix of the Newton-Schulz update product, with parts of its data path taken away
 // ---------------------------------------------------------------------------------------------
 namespace {
 
-// The main loop of k_ns_bf_gemm<kNsUpdate, 4> (128 x 256 outputs, six v_mfma_f32_32x32x16_bf16 per pair of
+// The main loop of k_ns_bf_gemm<kNsUpdate, 4> (128 x 256 outputs, three v_mfma_f32_32x32x16_f16 per pair of
 // 32 x 32 blocks and 16 reduction steps) over synthetic planes.  MODE 0: as in the product (operands staged
 // from memory into LDS every 16 steps); 1: the first stage is staged once and read from LDS in every step (no
 // global loads, no barriers); 2: the first stage's fragments stay in registers (matrix instructions only).
@@ -2472,7 +2531,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
     const bfbits* __restrict__ X, int rows_x, const bfbits* __restrict__ B, int rows_b, int K, float* __restrict__ out) {
   extern __shared__ __attribute__((aligned(16))) char lds_[];
   PYLO_LDS char* lds = (PYLO_LDS char*)lds_;
-  constexpr int WN = 4, RB = 64 * WN, SA = 128 * 96;
+  constexpr int WN = 4, RB = 64 * WN, SA = 128 * kNsRowB;
   const int nj = rows_b / RB, i0 = (blockIdx.x / nj) * 128, j0 = (blockIdx.x % nj) * RB;
   v16f acc[2][WN];
 #pragma unroll
@@ -2488,34 +2547,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wi = (wave >> 1) * 64, wj = (wave & 1) * 32 * WN;
     const int kg = lane >> 5, lo = lane & 31;
-    int offa[3], offb[RB * 6 / 256];
+    int offa[128 * kNsRowPc / 256], offb[RB * kNsRowPc / 256];
     bf_stage_offsets<128>(wave, lane, offa);
     bf_stage_offsets<RB>(wave, lane, offb);
-    bf_stage_issue<128>((const char*)X + (size_t)i0 * 96, offa, lds, wave);
-    bf_stage_issue<RB>((const char*)B + (size_t)j0 * 96, offb, lds + SA, wave);
+    bf_stage_issue<128>((const char*)X + (size_t)i0 * kNsRowB, offa, lds, wave);
+    bf_stage_issue<RB>((const char*)B + (size_t)j0 * kNsRowB, offb, lds + SA, wave);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    const int sw = 16 * (kg ^ ((lo >> 3) & 1));
-    const int oa = (wi + lo) * 96 + sw, ob = SA + (wj + lo) * 96 + sw;
-    bf16x8 a[2][3], b[WN][3];
+    const int sw = 16 * (kg ^ ((lo >> 2) & 3));
+    const int oa = (wi + lo) * kNsRowB + sw, ob = SA + (wj + lo) * kNsRowB + sw;
+    f16x8 a[2][kNsPl], b[WN][kNsPl];
     for (int k = 0; k < K; k += kBfBK) {
       if (MODE == 1 || k == 0) {
 #pragma unroll
-        for (int q = 0; q < 3; ++q) {
+        for (int q = 0; q < kNsPl; ++q) {
 #pragma unroll
-          for (int i = 0; i < 2; ++i) a[i][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + oa + i * 32 * 96 + q * 32));
+          for (int i = 0; i < 2; ++i) a[i][q] = __builtin_bit_cast(f16x8, *(const luint4*)(lds + ((oa + i * 32 * kNsRowB) ^ (q * 32))));
 #pragma unroll
-          for (int j = 0; j < WN; ++j) b[j][q] = __builtin_bit_cast(bf16x8, *(const luint4*)(lds + ob + j * 32 * 96 + q * 32));
+          for (int j = 0; j < WN; ++j) b[j][q] = __builtin_bit_cast(f16x8, *(const luint4*)(lds + ((ob + j * 32 * kNsRowB) ^ (q * 32))));
         }
       }
 #pragma unroll
-      for (int term = 0; term < 6; ++term) {
-        constexpr int pa[6] = {2, 0, 1, 1, 0, 0}, pb[6] = {0, 2, 1, 0, 1, 0};
+      for (int term = 0; term < 3; ++term) {
+        constexpr int pa[3] = {1, 0, 0}, pb[3] = {0, 1, 0};
 #pragma unroll
         for (int hi = 0; hi < 2; ++hi)
 #pragma unroll
           for (int hj = 0; hj < WN; ++hj)
-            acc[hi][hj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[hi][pa[term]], b[hj][pb[term]], acc[hi][hj], 0, 0, 0);
+            acc[hi][hj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[hi][pa[term]], b[hj][pb[term]], acc[hi][hj], 0, 0, 0);
       }
       if (MODE == 1) asm volatile("" ::: "memory");   // the fragments are read again in the next step
     }

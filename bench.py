@@ -206,7 +206,7 @@ def whole_step_object(whole_ms, finish_ms, n_params, flops, flops_exec):
         "newton_schulz_TFLOP": flops / 1e12, "newton_schulz_TFLOP_executed": flops_exec / 1e12,
         "roofline": {"bound": "mfma",
                      "kernel": ("k_ns_gemm (fp32 matrix instructions)" if f32 else
-                                "k_ns_bf_gemm (fp16 matrix instructions, 3 products per fp32 product)")
+                                "k_ns_hf_gemm (fp16 matrix instructions, 3 products per fp32 product)")
                                + " + finishing pass",
                      "achieved": mult * flops_exec / t / 1e12, "peak": peak, "unit": "TFLOP/s",
                      "frac": mult * flops_exec / t / 1e12 / peak,

@@ -67,9 +67,9 @@ extern "C" {
 #define PYLO_F_NO_ORTHOGONALIZE 64 /* CELO2 kind: the tensor is never passed to
                                  pylo_mi355_celo2_orthogonalize_finish with PYLO_ARG_ORTHOGONALIZE (its group does not
                                  orthogonalise, or the caller does that itself): no Newton-Schulz workspace is
-                                 reserved for it.  That workspace is 18 bytes per element of every other 2-D
-                                 MLP tensor (three bf16 planes of X in both orientations, twice for the one the
-                                 update product writes), about 4.5 times the tensor's fp32 size, and makes up most
+                                 reserved for it.  That workspace is 12 bytes per element of every other 2-D
+                                 MLP tensor (two fp16 planes of X in both orientations, twice for the one the
+                                 update product writes), three times the tensor's fp32 size, and makes up most
                                  of what pylo_mi355_plan_workspace_bytes reports for an ELO-CELO2 plan */
 
 /* Storage type of the tensor's `grad` and `param` buffers (bits 8-9 of PyloTensorShape.flags).  The reference's
@@ -234,9 +234,10 @@ int pylo_mi355_plan_finish_supported(const PyloPlan* plan, int tensor);
  * X = step_out / (||step_out||_F + ns_eps) and (c0, c1, c2) = ns_coeffs, `ns_iters` times
  *     A = X X^T (the Gram matrix over the smaller dim);  X <- c0 X + (c1 A + c2 A A) X
  * as matrix-pipe products of the library's own that compute the symmetric A and c0 I + c1 A + c2 A A once per
- * pair of tiles -- by default on the bf16 matrix instructions at fp32 accuracy (every fp32 operand is the exact
- * sum of three bf16 numbers, six bf16 products per fp32 product, fp32 accumulation; what is dropped is below
- * 2^-24 of a product; two iterations share one Gram product and one update, A' = B' A B' and
+ * pair of tiles -- by default on the fp16 matrix instructions at fp32 accuracy (every matrix is held as two fp16
+ * planes of its entries times a power of two chosen from bounds that follow from `ns_coeffs`, three fp16 products
+ * per fp32 product, fp32 accumulation; what is dropped is below 2^-22 of a term, under the rounding that the fp32
+ * accumulation adds; two iterations share one Gram product and one update, A' = B' A B' and
  * X'' = (B'' B') X, which costs about 1e-6 of B' in accuracy whatever the spectrum of X -- PYLO_MI355_NS_PAIRS=0
  * in the environment keeps one of each per iteration, PYLO_MI355_NS_CHAINS="3,2" lets three and then two
  * iterations share them, faster and up to ten times less accurate), with PYLO_MI355_NS_F32=1 in the environment at plan
@@ -250,8 +251,8 @@ int pylo_mi355_plan_finish_supported(const PyloPlan* plan, int tensor);
  * being the caller's -- and 2 for a tensor with more than two dims whose slices are small enough to be
  * orthogonalised in the launch that normalises and applies them (fp32 FMA in registers or LDS; `ns_iters` may
  * be 0 there; `step_out` is left as it was).  0: orthogonalised by the caller and passed without the flag.  The plan's workspace holds the operand planes:
- * 18 bytes per element of every such tensor (X as three bf16 planes in both orientations, the orientation
- * that the update product writes twice) plus 28 bytes per element of its m x m matrices -- 2.3 GB for a
+ * 12 bytes per element of every such tensor (X as two fp16 planes in both orientations, the orientation
+ * that the update product writes twice) plus 20 bytes per element of its m x m matrices -- 2.1 GB for a
  * GPT-2-small set, all tensors resident at once; pylo_mi355_plan_workspace_bytes reports the total.  The
  * products of groups of tensors run on streams of the plan's own next to the caller's (forked and joined
  * with events, default priority); the call returns with the caller's stream waiting for them.

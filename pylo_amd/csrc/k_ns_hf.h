@@ -1,13 +1,23 @@
-// Newton-Schulz products at fp32 accuracy on the bf16 matrix pipe.
+// Newton-Schulz products at fp32 accuracy on the fp16 matrix pipe.
 //
-// An fp32 number is the exact sum of three bf16 numbers, x = h + m + l (h = bf16(x), m = bf16(x - h),
-// l = x - h - m: 8 + 8 + 8 significand bits).  A product of two such numbers is nine bf16 products; the
-// three smallest (m l, l m, l l) are below 2^-25 |x y| together, less than the rounding of an fp32
-// multiply-add, and are dropped.  The other six are exact in fp32 and are accumulated in fp32 by
-// v_mfma_f32_32x32x16_bf16, which does sixteen times the multiply-adds of v_mfma_f32_32x32x2_f32 per
-// instruction slot: six of them replace eight fp32 instructions' worth of work at 2.7 times the rate.
+// An fp32 number times a power of two is, to 2^-22 of its size, the sum of two fp16 numbers: x s = h + l with
+// h = fp16(x s), l = fp16(x s - h) (11 + 11 significand bits), as long as h does not overflow (|x s| < 65 504) and l
+// does not fall off the format's lower end (fp16 keeps subnormals down to 2^-24 and the matrix instructions take
+// them as they are: l is exact to 2^-25 absolutely, i.e. entries below 1/8 lose relative, not absolute, accuracy).
+// A product of two such numbers is four fp16 products; the smallest (l l, 2^-22 |x y|) is dropped with the
+// remainders.  The other three are exact in fp32 and are accumulated in fp32 by v_mfma_f32_32x32x16_f16, which does
+// sixteen times the multiply-adds of v_mfma_f32_32x32x2_f32 per instruction slot: three of them replace eight fp32
+// instructions' worth of work.  A product of the iteration is then off by about 6e-8 of its entries' RMS, a quarter
+// of what the fp32 accumulation of a reduction over 256 .. 4096 terms adds anyway (a plain fp32 GEMM: 2.5e-7).
+// The scales: no entry of a matrix exceeds its largest singular value, and the singular values of everything the
+// iteration forms follow from the coefficients alone once X0 has unit Frobenius norm (the host walks a grid of
+// starting values through sigma -> sigma p(sigma^2), ns_plane_exps): X and A = X X^T stay below 1.5, B' = p(A)
+// below c0, products of k such B' below c0^k.  Every kind of matrix gets the power of two that puts its bound at
+// 12 000 .. 24 000; a product's accumulators are scaled back by the reciprocal of its operands' scales (exact) and
+// what it writes is scaled by its own.  A value outside its bound -- there should be none -- is clamped, not made
+// an infinity.
 //
-// Operands therefore live as *planes*: three bf16 matrices (h, m, l) with the reduction index contiguous,
+// Operands therefore live as *planes*: two fp16 matrices (h, l) with the reduction index contiguous,
 // written by the kernel that produces the matrix (never converted inside a product's main loop).
 // With X of m x n or n x m (m the smaller dim), Xs = X as [m][n] and Xl = X as [n][m]:
 //     A   = Xs Xs^T                      (reduction over n; symmetric, tiles on and above the diagonal)
@@ -28,12 +38,12 @@
 // multiplies it by c0^2 again, which is why pairs are the default and the next pair starts from a Gram product
 // of the X it was handed.  The host enqueues chains of any length L (one Gram product, 4 L - 3 products of
 // m x m matrices rotating through four plane buffers, one update): PYLO_MI355_NS_CHAINS="3,2" in the environment
-// trades accuracy for time (1.3e-4 of the result's RMS on a dominant direction over a flat rest, where pairs
-// are at 1e-5), PYLO_MI355_NS_PAIRS=0 keeps one Gram product and one update per iteration.
+// trades accuracy for time (up to 1e-4 of the result's RMS on a dominant direction over a flat rest, where pairs
+// are at 1.3e-5), PYLO_MI355_NS_PAIRS=0 keeps one Gram product and one update per iteration.
 //
 // Tile job: 128 x 128 (Gram, Poly, narrow updates) or 128 x 256 outputs (updates with m > 128) by 256 threads =
 // 2 x 2 waves of 64 x 64 / 64 x 128 = 2 x 2 / 2 x 4 accumulators of 32 x 32; 16 reduction steps per stage,
-// double buffered in LDS (48 / 72 KB), staged from global memory straight into LDS (global_load_lds_dwordx4: no
+// double buffered in LDS (32 / 48 KB), staged from global memory straight into LDS (global_load_lds_dwordx4: no
 // staging registers, no LDS store instructions), one 16-byte read per lane, plane and 32-row block per stage.
 // The planes are allocated with their rows rounded up to whole tiles and the padding holds zeros, so the main
 // loop has no bounds checks; any two dims are taken (the raw step is read and the result written per element
@@ -45,48 +55,48 @@
 namespace pylo {
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef unsigned short bfbits;   // one number of a plane in memory (an fp16)
+typedef unsigned short hbits;   // one number of a plane in memory (an fp16)
 constexpr int kNsPl = 2;                      // planes per matrix
 constexpr int kNsRowB = 32 * kNsPl;           // bytes of one row in a block of 16 reduction steps
 constexpr int kNsRowPc = 2 * kNsPl;           // the same in 16-byte pieces
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) u32x4 luint4;
 
-constexpr int kBfBK = 16;                     // reduction steps per stage
+constexpr int kHfBK = 16;                     // reduction steps per stage
 // LDS of a tile job with 64 WN columns: two stages of (128 + 64 WN) rows x 2 planes x 32 bytes
-constexpr int bf_gemm_lds(int wn) { return 2 * (128 + 64 * wn) * kNsRowB; }
+constexpr int hf_gemm_lds(int wn) { return 2 * (128 + 64 * wn) * kNsRowB; }
 
 // Planes of one matrix with `rows` rows and a (padded) reduction length: stored in blocks of 16 reduction
 // steps, [k / 16][row][plane][k % 16], so that the 128 rows x 3 planes x 16 steps a tile job stages at a
 // time are 12 KB of consecutive memory (whole cache lines; with row-major planes a stage was 32 bytes
 // out of every row and each 128-byte line was fetched from L2 four times).
-struct BfPlanes {
-  const bfbits* base;
+struct HfPlanes {
+  const hbits* base;
   int rows;   // rows allocated (a multiple of the tiles' rows; rows past the matrix hold zeros)
 };
 
 // element offset of (row, k) in plane 0; plane 1 is 16 elements further
-__device__ __forceinline__ size_t bf_off(int rows, int row, int k) {
+__device__ __forceinline__ size_t hf_off(int rows, int row, int k) {
   return ((size_t)(k >> 4) * rows + row) * (16 * kNsPl) + (k & 15);
 }
 
-struct NsBfMat {
+struct NsHfMat {
   int tensor;
   int R, C, m, n, tall;      // X is R x C row-major; m = min, n = max; tall: R > C
   int pad_m, pad_n;          // m and n rounded up to the 16 reduction steps of a stage (the padding holds zeros)
   int rows_m, rows_n;        // rows allocated for the planes whose rows are the m / n index (whole tiles)
   int lda;                   // row pitch of the fp32 A and of the partial matrices: m rounded up to 4
   int n_slabs;
-  long long off_xs;          // elements (bfbits) into the plane workspace: planes of Xs (m rows, reduction n)
+  long long off_xs;          // elements (hbits) into the plane workspace: planes of Xs (m rows, reduction n)
   long long off_xl[2];       // planes of Xl (n rows, reduction m), two buffers (a product reads one and writes the other)
   long long off_p, p_stride; // planes of the m x m matrices (m rows, reduction m): buffer b at off_p + b p_stride
   long long off_a;           // floats into the fp32 workspace: A (m x m)
   long long off_part;        // floats: partial matrices of a split Gram product
   long long elem_off;        // elements from the tensor's raw step to this matrix (a slice of a tensor with more dims)
-  int fpart0, n_fpart;       // its partial sums of squares of A (k_ns_bf_chain_sumsq): first, count
+  int fpart0, n_fpart;       // its partial sums of squares of A (k_ns_hf_chain_sumsq): first, count
 };
 
-// the m x m plane buffers, and the two products on planes in and planes out (k_ns_bf_gemm's OP, after
+// the m x m plane buffers, and the two products on planes in and planes out (k_ns_hf_gemm's OP, after
 // kNsGram / kNsPoly / kNsUpdate)
 enum : int { kNsBufA = 0, kNsBufB = 1, kNsBufT = 2, kNsBufC = 3, kNsBufs = 4 };
 enum : int { kNsProd = 3, kNsProdA = 4 };
@@ -96,12 +106,12 @@ struct NsBufs { int s1, s2, d; float acc_scale, out_scale; };
 
 // x (already times its plane scale) = h + l + what is left below 2^-22 |x|.  The clamp never acts on a matrix
 // within the bounds the scales were chosen for; it keeps a stray value from becoming an infinity.
-__device__ __forceinline__ void hf_split(float x, bfbits& h, bfbits& l) {
+__device__ __forceinline__ void hf_split(float x, hbits& h, hbits& l) {
   x = __builtin_amdgcn_fmed3f(x, -65000.0f, 65000.0f);
   const _Float16 hb = (_Float16)x;
   const _Float16 lb = (_Float16)(x - (float)hb);
-  h = __builtin_bit_cast(bfbits, hb);
-  l = __builtin_bit_cast(bfbits, lb);
+  h = __builtin_bit_cast(hbits, hb);
+  l = __builtin_bit_cast(hbits, lb);
 }
 
 // A stage of one operand in LDS: [row][plane][half], 64 bytes a row, as in memory, except that the four
@@ -116,7 +126,7 @@ __device__ __forceinline__ void hf_split(float x, bfbits& h, bfbits& l) {
 #define PYLO_GLB __attribute__((address_space(1)))
 
 template <int ROWS>
-__device__ __forceinline__ void bf_stage_offsets(int wave, int lane, int (&off)[ROWS * kNsRowPc / 256]) {
+__device__ __forceinline__ void hf_stage_offsets(int wave, int lane, int (&off)[ROWS * kNsRowPc / 256]) {
 #pragma unroll
   for (int j = 0; j < ROWS * kNsRowPc / 256; ++j) {
     const int p = (j * 4 + wave) * 64 + lane;
@@ -125,7 +135,7 @@ __device__ __forceinline__ void bf_stage_offsets(int wave, int lane, int (&off)[
 }
 
 template <int ROWS>
-__device__ __forceinline__ void bf_stage_issue(const char* g, const int (&off)[ROWS * kNsRowPc / 256], PYLO_LDS char* lds, int wave) {
+__device__ __forceinline__ void hf_stage_issue(const char* g, const int (&off)[ROWS * kNsRowPc / 256], PYLO_LDS char* lds, int wave) {
 #pragma unroll
   for (int j = 0; j < ROWS * kNsRowPc / 256; ++j)
     __builtin_amdgcn_global_load_lds((const PYLO_GLB void*)(g + off[j]), (PYLO_LDS void*)(lds + (j * 4 + wave) * 1024), 16, 0, 0);
@@ -136,34 +146,34 @@ __device__ __forceinline__ void bf_stage_issue(const char* g, const int (&off)[R
 // `compute` (the same for all lanes of a wave): false for a wave whose values nobody needs -- it stages and meets the
 // barriers, and leaves the matrix pipe to the other waves of its SIMD.
 template <int WN>
-__device__ __forceinline__ void bf_tile_product(const BfPlanes& P1, int i0, const BfPlanes& P2, int j0, int k0, int k1,
+__device__ __forceinline__ void hf_tile_product(const HfPlanes& P1, int i0, const HfPlanes& P2, int j0, int k0, int k1,
                                                 PYLO_LDS char* lds, v16f (&acc)[2][WN], bool compute = true) {
   constexpr int RB = 64 * WN, SA = 128 * kNsRowB, STAGE = SA + RB * kNsRowB;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wi = (wave >> 1) * 64, wj = (wave & 1) * 32 * WN;
   const int kg = lane >> 5, lo = lane & 31;
   int offa[128 * kNsRowPc / 256], offb[RB * kNsRowPc / 256];
-  bf_stage_offsets<128>(wave, lane, offa);
-  bf_stage_offsets<RB>(wave, lane, offb);
+  hf_stage_offsets<128>(wave, lane, offa);
+  hf_stage_offsets<RB>(wave, lane, offb);
   const char* ga = (const char*)P1.base + ((size_t)(k0 >> 4) * P1.rows + i0) * kNsRowB;
   const char* gb = (const char*)P2.base + ((size_t)(k0 >> 4) * P2.rows + j0) * kNsRowB;
   const size_t sa = (size_t)P1.rows * kNsRowB, sb = (size_t)P2.rows * kNsRowB;
   // a diagonal tile of X X^T or A A: both operands are the same 128 rows, staged once
   const bool same = WN == 2 && P1.base == P2.base && i0 == j0;
-  bf_stage_issue<128>(ga, offa, lds, wave);
-  if (!same) bf_stage_issue<RB>(gb, offb, lds + SA, wave);
+  hf_stage_issue<128>(ga, offa, lds, wave);
+  if (!same) hf_stage_issue<RB>(gb, offb, lds + SA, wave);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   // the lane's rows are lo, lo + 32, ..: all with the same (row / 4) % 4; plane q, half kg is piece 2 q + kg
   const int sw = 16 * (kg ^ ((lo >> 2) & 3));
   const int oa = (wi + lo) * kNsRowB + sw, ob = (same ? 0 : SA) + (wj + lo) * kNsRowB + sw;
   int cur = 0;
-  for (int k = k0; k < k1; k += kBfBK) {
-    if (k + kBfBK < k1) {
+  for (int k = k0; k < k1; k += kHfBK) {
+    if (k + kHfBK < k1) {
       ga += sa;
       gb += sb;
-      bf_stage_issue<128>(ga, offa, lds + (STAGE - cur), wave);
-      if (!same) bf_stage_issue<RB>(gb, offb, lds + (STAGE - cur) + SA, wave);
+      hf_stage_issue<128>(ga, offa, lds + (STAGE - cur), wave);
+      if (!same) hf_stage_issue<RB>(gb, offb, lds + (STAGE - cur) + SA, wave);
     }
     if (compute) {
       f16x8 a[2][kNsPl], b[WN][kNsPl];
@@ -196,10 +206,10 @@ __device__ __forceinline__ void bf_tile_product(const BfPlanes& P1, int i0, cons
 }
 
 // one value (times its plane scale already) into both planes
-__device__ __forceinline__ void bf_store1(bfbits* base, int rows, int row, int k, float v) {
-  bfbits h, l;
+__device__ __forceinline__ void hf_store1(hbits* base, int rows, int row, int k, float v) {
+  hbits h, l;
   hf_split(v, h, l);
-  bfbits* p = base + bf_off(rows, row, k);
+  hbits* p = base + hf_off(rows, row, k);
   p[0] = h;
   p[16] = l;
 }
@@ -215,12 +225,12 @@ __device__ __forceinline__ void bf_store1(bfbits* base, int rows, int row, int k
 // Only the lanes of one wave meet in a patch and a wave's LDS instructions execute in order, so the passes
 // need no barrier, just the compiler kept from moving the reads over the writes.
 template <int WN>
-__device__ __forceinline__ void bf_store_planes(PYLO_LDS char* lds, const v16f (&acc)[2][WN], bfbits* __restrict__ D,
+__device__ __forceinline__ void hf_store_planes(PYLO_LDS char* lds, const v16f (&acc)[2][WN], hbits* __restrict__ D,
                                                 int rows_total, int i0, int j0, int n_rows, int n_cols,
-                                                bfbits* __restrict__ D4, int rows4, float scale) {
+                                                hbits* __restrict__ D4, int rows4, float scale) {
   constexpr int kPlane = 64 * WN + 16;        // bytes: 32 WN columns x 2 + 16 (bank spread)
   constexpr int kRow = kNsPl * kPlane, kWave = 16 * kRow;
-  typedef PYLO_LDS bfbits lbf;
+  typedef PYLO_LDS hbits lbf;
   typedef unsigned long long u64;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   PYLO_LDS char* patch = lds + wave * kWave;
@@ -233,7 +243,7 @@ __device__ __forceinline__ void bf_store_planes(PYLO_LDS char* lds, const v16f (
     for (int hj = 0; hj < WN; ++hj)
 #pragma unroll
       for (int g4 = 0; g4 < 2; ++g4) {
-        bfbits h[4], l[4];
+        hbits h[4], l[4];
         const int col_l = 32 * hj + (lane & 31);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -245,7 +255,7 @@ __device__ __forceinline__ void bf_store_planes(PYLO_LDS char* lds, const v16f (
         if (D4 != nullptr) {
           const int row = wi + 32 * hi + 16 * half + 8 * g4 + 4 * (lane >> 5), col = wj + col_l;
           if (col < n_cols && row < n_rows) {   // values past n_rows are zeros, into the padding
-            bfbits* p = D4 + bf_off(rows4, col, row);
+            hbits* p = D4 + hf_off(rows4, col, row);
             *(u64*)p = (u64)h[0] | (u64)h[1] << 16 | (u64)h[2] << 32 | (u64)h[3] << 48;
             *(u64*)(p + 16) = (u64)l[0] | (u64)l[1] << 16 | (u64)l[2] << 32 | (u64)l[3] << 48;
           }
@@ -257,7 +267,7 @@ __device__ __forceinline__ void bf_store_planes(PYLO_LDS char* lds, const v16f (
     for (int c = 0; c < 2 * WN; ++c) {     // 16 columns = one block of the planes' layout
       const int col = wj + 16 * c;
       if (col >= n_cols) continue;
-      bfbits* dst = D + bf_off(rows_total, row_w0, col);
+      hbits* dst = D + hf_off(rows_total, row_w0, col);
       const int row_l = lane >> 2, plane = (lane >> 1) & 1, hf = lane & 1;   // piece `lane` of [row][plane][half]
       if (row_w0 + row_l >= n_rows) continue;
       const u32x4 w = *(const luint4*)(patch + row_l * kRow + plane * kPlane + (16 * c + 8 * hf) * 2);
@@ -275,7 +285,7 @@ __device__ __forceinline__ void bf_store_planes(PYLO_LDS char* lds, const v16f (
 // WN: the tile has 64 WN columns (Gram and Poly: 2; updates: 2 or 4, a table of jobs each).
 // Registers: 64 / 128 accumulator registers plus what the epilogues need; tiles of 256 columns are held to two
 // waves per SIMD (256 registers: left alone the epilogue takes 296 and a CU runs one job at a time).
-// Which matrices a launch is for, when the chain length is chosen per matrix (k_ns_bf_chain_flag): all of them; those
+// Which matrices a launch is for, when the chain length is chosen per matrix (k_ns_hf_chain_flag): all of them; those
 // whose first chain is the longer one; the others; or all, the others with another first operand buffer and `last`.
 enum : int { kNsAll = 0, kNsLongOnly = 1, kNsShortOnly = 2, kNsBoth = 3 };
 struct NsPick {
@@ -285,9 +295,9 @@ struct NsPick {
 };
 
 template <int OP, int WN>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2 : 3))) void k_ns_bf_gemm(const NsBfMat* __restrict__ mats, const NsItem* __restrict__ items,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2 : 3))) void k_ns_hf_gemm(const NsHfMat* __restrict__ mats, const NsItem* __restrict__ items,
                                                     const PyloTensorArgs* __restrict__ dyn, float* __restrict__ ws,
-                                                    bfbits* __restrict__ pw, int par, int last, NsBufs bufs, float c0,
+                                                    hbits* __restrict__ pw, int par, int last, NsBufs bufs, float c0,
                                                     float c1, float c2, NsPick pick) {
   extern __shared__ __attribute__((aligned(16))) char lds_[];
   PYLO_LDS char* lds = (PYLO_LDS char*)lds_;
@@ -302,7 +312,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
       last = pick.last_short;
     }
   }
-  const NsBfMat mt = mats[it.mat];
+  const NsHfMat mt = mats[it.mat];
   const PyloTensorArgs a = dyn[mt.tensor];
   if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
   const int m = mt.m, n = mt.n, lda = mt.lda;
@@ -320,19 +330,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
   const bool diag = OP != kNsUpdate && WN == 2 && it.tm == it.tn;
   const bool idle = diag && wave_u == 2;
   if (OP == kNsGram) {
-    const BfPlanes X{pw + mt.off_xs, mt.rows_m};
-    bf_tile_product<WN>(X, i0, X, j0, it.k0, it.k1, lds, acc, !idle);
+    const HfPlanes X{pw + mt.off_xs, mt.rows_m};
+    hf_tile_product<WN>(X, i0, X, j0, it.k0, it.k1, lds, acc, !idle);
   } else if (OP == kNsPoly) {
-    const BfPlanes A{pw + mt.off_p, mt.rows_m};
-    bf_tile_product<WN>(A, i0, A, j0, it.k0, it.k1, lds, acc, !idle);
+    const HfPlanes A{pw + mt.off_p, mt.rows_m};
+    hf_tile_product<WN>(A, i0, A, j0, it.k0, it.k1, lds, acc, !idle);
   } else if (OP == kNsUpdate) {
-    const BfPlanes X{pw + (par ? mt.off_xl[1] : mt.off_xl[0]), mt.rows_n};   // no run-time index: the struct stays in registers
-    const BfPlanes B{pw + mt.off_p + bufs.s1 * mt.p_stride, mt.rows_m};
-    bf_tile_product<WN>(X, i0, B, j0, it.k0, it.k1, lds, acc);
+    const HfPlanes X{pw + (par ? mt.off_xl[1] : mt.off_xl[0]), mt.rows_n};   // no run-time index: the struct stays in registers
+    const HfPlanes B{pw + mt.off_p + bufs.s1 * mt.p_stride, mt.rows_m};
+    hf_tile_product<WN>(X, i0, B, j0, it.k0, it.k1, lds, acc);
   } else {
-    const BfPlanes P1{pw + mt.off_p + bufs.s1 * mt.p_stride, mt.rows_m};
-    const BfPlanes P2{pw + mt.off_p + bufs.s2 * mt.p_stride, mt.rows_m};
-    bf_tile_product<WN>(P1, i0, P2, j0, it.k0, it.k1, lds, acc, !idle);
+    const HfPlanes P1{pw + mt.off_p + bufs.s1 * mt.p_stride, mt.rows_m};
+    const HfPlanes P2{pw + mt.off_p + bufs.s2 * mt.p_stride, mt.rows_m};
+    hf_tile_product<WN>(P1, i0, P2, j0, it.k0, it.k1, lds, acc, !idle);
   }
   if (idle) return;
   // the operands' planes hold their matrices times a power of two each
@@ -398,20 +408,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WN == 4 ? 2
   // (through LDS) and Xs' (registers)
   if (partial || (OP == kNsUpdate && last)) return;
   if (OP == kNsUpdate) {
-    bf_store_planes<WN>(lds, acc, pw + (par ? mt.off_xl[0] : mt.off_xl[1]), mt.rows_n, i0, j0, n, m, pw + mt.off_xs, mt.rows_m,
+    hf_store_planes<WN>(lds, acc, pw + (par ? mt.off_xl[0] : mt.off_xl[1]), mt.rows_n, i0, j0, n, m, pw + mt.off_xs, mt.rows_m,
                         bufs.out_scale);
   } else {
-    bfbits* D = pw + mt.off_p + (OP == kNsGram ? (int)kNsBufA : bufs.d) * mt.p_stride;
-    bf_store_planes<WN>(lds, acc, D, mt.rows_m, i0, j0, m, m, mirror ? D : nullptr, mt.rows_m, bufs.out_scale);
+    hbits* D = pw + mt.off_p + (OP == kNsGram ? (int)kNsBufA : bufs.d) * mt.p_stride;
+    hf_store_planes<WN>(lds, acc, D, mt.rows_m, i0, j0, m, m, mirror ? D : nullptr, mt.rows_m, bufs.out_scale);
   }
 }
 
 // A = sum over the slabs' partial matrices, in slab order, as fp32 and as planes (both halves).
-__global__ __launch_bounds__(256) void k_ns_bf_gram_reduce(const NsBfMat* __restrict__ mats, const int* __restrict__ split_mats,
+__global__ __launch_bounds__(256) void k_ns_hf_gram_reduce(const NsHfMat* __restrict__ mats, const int* __restrict__ split_mats,
                                                            const PyloTensorArgs* __restrict__ dyn, float* __restrict__ ws,
-                                                           bfbits* __restrict__ pw, NsPick pick, float out_scale) {
+                                                           hbits* __restrict__ pw, NsPick pick, float out_scale) {
   if (pick.sel == kNsShortOnly && pick.flags[split_mats[blockIdx.y]] != 0) return;
-  const NsBfMat mt = mats[split_mats[blockIdx.y]];
+  const NsHfMat mt = mats[split_mats[blockIdx.y]];
   const PyloTensorArgs a = dyn[mt.tensor];
   if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
   const int m = mt.m, lda = mt.lda;
@@ -430,12 +440,12 @@ __global__ __launch_bounds__(256) void k_ns_bf_gram_reduce(const NsBfMat* __rest
     for (int q = 0; q < 8; ++q) s += v[q];
   }
   float* A = ws + mt.off_a;
-  bfbits* P = pw + mt.off_p;   // buffer A
+  hbits* P = pw + mt.off_p;   // buffer A
   A[(size_t)i * lda + j] = s;
-  bf_store1(P, mt.rows_m, i, j, s * out_scale);
+  hf_store1(P, mt.rows_m, i, j, s * out_scale);
   if (i / 64 != j / 64) {
     A[(size_t)j * lda + i] = s;
-    bf_store1(P, mt.rows_m, j, i, s * out_scale);
+    hf_store1(P, mt.rows_m, j, i, s * out_scale);
   }
 }
 
@@ -449,12 +459,12 @@ __global__ __launch_bounds__(256) void k_ns_bf_gram_reduce(const NsBfMat* __rest
 // Two launches, sums in a fixed order: 4096 elements of A per block, then one block per matrix.
 constexpr int kNsFlagChunk = 4096;
 // items[b] = {matrix, chunk of 4096 elements of its A}
-__global__ __launch_bounds__(256) void k_ns_bf_chain_sumsq(const NsBfMat* __restrict__ mats, const Item* __restrict__ items,
+__global__ __launch_bounds__(256) void k_ns_hf_chain_sumsq(const NsHfMat* __restrict__ mats, const Item* __restrict__ items,
                                                            const PyloTensorArgs* __restrict__ dyn, const float* __restrict__ ws,
                                                            float* __restrict__ part) {
   __shared__ float red[4];
   const Item it = items[blockIdx.x];
-  const NsBfMat mt = mats[it.tensor];
+  const NsHfMat mt = mats[it.tensor];
   const PyloTensorArgs a = dyn[mt.tensor];
   if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
   const long long mm = (long long)mt.m * mt.m, e0 = (long long)it.a * kNsFlagChunk;
@@ -474,11 +484,11 @@ __global__ __launch_bounds__(256) void k_ns_bf_chain_sumsq(const NsBfMat* __rest
   if (threadIdx.x == 0) part[mt.fpart0 + it.a] = (red[0] + red[1]) + (red[2] + red[3]);
 }
 
-__global__ __launch_bounds__(64) void k_ns_bf_chain_flag(const NsBfMat* __restrict__ mats, const int* __restrict__ list,
+__global__ __launch_bounds__(64) void k_ns_hf_chain_flag(const NsHfMat* __restrict__ mats, const int* __restrict__ list,
                                                          const PyloTensorArgs* __restrict__ dyn, const float* __restrict__ part,
                                                          float tau2, int* __restrict__ flags) {
   const int q = list[blockIdx.x];
-  const NsBfMat mt = mats[q];
+  const NsHfMat mt = mats[q];
   const PyloTensorArgs a = dyn[mt.tensor];
   if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
   float s = 0.0f;
@@ -489,13 +499,13 @@ __global__ __launch_bounds__(64) void k_ns_bf_chain_flag(const NsBfMat* __restri
 
 struct NsTileItem { int mat, tr, tc; };
 
-__global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__ mats, const NsTileItem* __restrict__ items,
+__global__ __launch_bounds__(256) void k_ns_hf_split(const NsHfMat* __restrict__ mats, const NsTileItem* __restrict__ items,
                                                      const PyloTensorArgs* __restrict__ dyn, const float* __restrict__ scale,
-                                                     bfbits* __restrict__ pw, float plane_scale) {
+                                                     hbits* __restrict__ pw, float plane_scale) {
   constexpr int RP = 72;   // numbers per row of the tile in LDS: 64 + 8, rows stay 16-byte aligned
-  __shared__ __attribute__((aligned(16))) bfbits tile[kNsPl][64][RP];
+  __shared__ __attribute__((aligned(16))) hbits tile[kNsPl][64][RP];
   const NsTileItem it = items[blockIdx.x];
-  const NsBfMat mt = mats[it.mat];
+  const NsHfMat mt = mats[it.mat];
   const PyloTensorArgs a = dyn[mt.tensor];
   if (a.grad == nullptr || !(a.flags & kArgOrthogonalize)) return;
   const float s = scale[it.mat] * plane_scale;
@@ -503,8 +513,8 @@ __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__
   const float* raw = a.step_out + mt.elem_off;
   const bool vec_in = (C & 3) == 0;
   // direct planes: the tensor's rows are the planes' rows; transposed planes: its columns are
-  bfbits* direct = pw + (mt.tall ? mt.off_xl[0] : mt.off_xs);
-  bfbits* transp = pw + (mt.tall ? mt.off_xs : mt.off_xl[0]);
+  hbits* direct = pw + (mt.tall ? mt.off_xl[0] : mt.off_xs);
+  hbits* transp = pw + (mt.tall ? mt.off_xs : mt.off_xl[0]);
   const int rows_d = mt.tall ? mt.rows_n : mt.rows_m, rows_t = mt.tall ? mt.rows_m : mt.rows_n;
   const int r0 = it.tr * 64, c0 = it.tc * 64;
   const int t = threadIdx.x;
@@ -536,7 +546,7 @@ __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__
     u32x4 pl[kNsPl];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      bfbits h0, l0, h1, l1;
+      hbits h0, l0, h1, l1;
       hf_split(v[2 * q], h0, l0);
       hf_split(v[2 * q + 1], h1, l1);
       pl[0][q] = (unsigned)h0 | (unsigned)h1 << 16;
@@ -545,7 +555,7 @@ __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__
 #pragma unroll
     for (int q = 0; q < kNsPl; ++q) *(luint4*)&tile[q][lr][lc] = pl[q];
     if (in) {
-      bfbits* p = direct + bf_off(rows_d, r, c);
+      hbits* p = direct + hf_off(rows_d, r, c);
 #pragma unroll
       for (int q = 0; q < kNsPl; ++q) *(u32x4*)(p + 16 * q) = pl[q];
     }
@@ -557,7 +567,7 @@ __global__ __launch_bounds__(256) void k_ns_bf_split(const NsBfMat* __restrict__
     const int lc = t & 63, rb = t >> 6;
     const int c = c0 + lc, r = r0 + 16 * rb;
     if (c < C && r < R) {
-      bfbits* p = transp + bf_off(rows_t, c, r);
+      hbits* p = transp + hf_off(rows_t, c, r);
 #pragma unroll
       for (int q = 0; q < kNsPl; ++q)
 #pragma unroll

@@ -30,7 +30,7 @@
 #include "k_velo.h"
 #include "k_celo2_slices.h"
 #include "k_ns.h"
-#include "k_ns_bf.h"
+#include "k_ns_hf.h"
 #include "k_slice_finish.h"
 #include "k_cast.h"
 #include "pylo_common.h"
@@ -74,7 +74,7 @@ bool factored_dims(int kind, const PyloTensorShape& s, int* dc, int* dr) {
   return true;
 }
 
-// One group of matrices of the split-bf16 Newton-Schulz kernels: its ranges in the job tables.
+// One group of matrices of the split-fp16 Newton-Schulz kernels: its ranges in the job tables.
 struct NsGroup {
   int gram0, n_gram, poly0, n_poly, upd0, n_upd, upd40, n_upd4, split0, n_split, split_max_m;
   int list0, n_list;       // its matrices (ns_list)
@@ -93,13 +93,13 @@ struct Layout {
   // ELO-CELO2: Newton-Schulz on the 2-D tensors (k_ns.h)
   std::vector<NsMat> ns_mats;
   std::vector<NsItem> ns_gram, ns_poly, ns_upd;
-  std::vector<NsItem> ns_upd4;        // split-bf16 kernels: update jobs with 256-column tiles
-  std::vector<NsGroup> ns_groups;     // split-bf16 kernels: ranges of the job tables, one per group of matrices
-  std::vector<NsBatch> ns_batches;    // split-bf16 kernels: batches of matrices that run one after another
+  std::vector<NsItem> ns_upd4;        // split-fp16 kernels: update jobs with 256-column tiles
+  std::vector<NsGroup> ns_groups;     // split-fp16 kernels: ranges of the job tables, one per group of matrices
+  std::vector<NsBatch> ns_batches;    // split-fp16 kernels: batches of matrices that run one after another
   std::vector<int> ns_split;          // matrices whose Gram product is split (k_ns_gram_reduce)
   std::vector<long long> ns_xalt;     // per tensor: offset of its second X buffer, -1 without one
   std::vector<int> ns_of_tensor;      // per tensor: index into ns_mats, -1
-  std::vector<int> ns_group_of_tensor;  // split-bf16 kernels, per tensor: its group (index into ns_groups), -1
+  std::vector<int> ns_group_of_tensor;  // split-fp16 kernels, per tensor: its group (index into ns_groups), -1
   std::vector<int> ns_list;           // the groups' matrices, group after group
   int fin_rest0 = 0, n_fin_rest = 0, unit_rest0 = 0, n_unit_rest = 0;   // finishing pass: what belongs to no group
   size_t off_ns_list = 0;
@@ -114,12 +114,12 @@ struct Layout {
   int slice_lds_l[kSliceLaneSets] = {}, slice_lds_w = 0, slice_lds_b = 0;
   size_t off_slice_mats = 0, off_slice_items_l[kSliceLaneSets] = {}, off_slice_items_w = 0, off_slice_items_b = 0;
   int ns_max_m = 0;
-  std::vector<Item> ns_flag_items;    // split-bf16 kernels: {matrix, chunk of its A} of k_ns_bf_chain_sumsq, group after group
+  std::vector<Item> ns_flag_items;    // split-fp16 kernels: {matrix, chunk of its A} of k_ns_hf_chain_sumsq, group after group
   int ns_fpart_total = 0;
   size_t off_ns_flags = 0, off_ns_fpart = 0, off_ns_flag_items = 0;
-  // Newton-Schulz on the bf16 matrix pipe (three-way split operands): tables of their own
-  bool ns_bf = false;
-  std::vector<NsBfMat> nsb_mats;
+  // Newton-Schulz on the fp16 matrix pipe (two-way split operands): tables of their own
+  bool ns_hf = false;
+  std::vector<NsHfMat> nsb_mats;
   std::vector<NsTileItem> nsb_split_items;
   size_t off_nsb_mats = 0, off_nsb_split_items = 0, off_ns_pw = 0, off_ns_upd4 = 0;
   long long nsb_plane_elems = 0;
@@ -248,7 +248,7 @@ void build_elem_items(Layout& L, int T, int kind) {
 }
 
 // PYLO_MI355_NS_F32=1 keeps the Newton-Schulz products on the fp32 matrix instructions (k_ns.h) instead of
-// the split-bf16 ones (k_ns_bf.h); read at plan creation.
+// the split-fp16 ones (k_ns_hf.h); read at plan creation.
 bool env_ns_xcd() {
   const char* e = getenv("PYLO_MI355_NS_XCD");
   return !(e && e[0] == '0');
@@ -262,14 +262,14 @@ int env_ns_groups() {
 }
 
 // PYLO_MI355_NS_WORKSPACE_MB: what the operand planes of the matrices that are orthogonalised at one time may take
-// (in bf16 elements here); read at plan creation.
+// (in fp16 elements here); read at plan creation.
 long long env_ns_budget_elems() {
   const char* e = getenv("PYLO_MI355_NS_WORKSPACE_MB");
   const long long mb = e ? atoll(e) : 8192;
   return std::max(1ll, mb) * (1ll << 20) / 2;
 }
 
-// How the Newton-Schulz iterations share their products over the long dim (k_ns_bf.h): a chain of L iterations takes
+// How the Newton-Schulz iterations share their products over the long dim (k_ns_hf.h): a chain of L iterations takes
 // one Gram product, one update and 4 L - 3 products of m x m matrices.  PYLO_MI355_NS_CHAINS="2,3" gives the chain
 // lengths in order (they must add up to the iteration count, else the default applies); PYLO_MI355_NS_PAIRS=0 means
 // chains of one: one Gram product and one update per iteration, as the formula is written.  Read when the products
@@ -295,8 +295,8 @@ std::vector<int> ns_chains(int iters) {
     out.clear();
   }
   // default: pairs (five iterations: 2, 2, 1).  Longer chains are faster and less accurate: "3,2" takes the
-  // GPT-2-small step from 9.45 to 8.2 ms and stays at the formula's own fp32 error on most inputs, but reaches 1.3e-4
-  // of the result's RMS (against 1e-5 for pairs) on matrices with a dominant direction over a flat rest.
+  // GPT-2-small step from 6.4 to 5.7 ms and stays at the formula's own fp32 error on most inputs, but reaches 1e-4
+  // of the result's RMS (against 1.3e-5 for pairs) on matrices with a dominant direction over a flat rest.
   for (int left = iters; left > 0;) {
     const int l = std::min(left, 2);
     out.push_back(l);
@@ -306,7 +306,7 @@ std::vector<int> ns_chains(int iters) {
 }
 
 // PYLO_MI355_NS_ADAPTIVE=1: a first chain of three iterations for the matrices whose spectrum allows it
-// (k_ns_bf_chain_flag), pairs for the others -- unless the environment fixes the chains (PYLO_MI355_NS_CHAINS,
+// (k_ns_hf_chain_flag), pairs for the others -- unless the environment fixes the chains (PYLO_MI355_NS_CHAINS,
 // PYLO_MI355_NS_PAIRS=0).  Off by default: raw steps with a direction that holds more than 8 % of their squared norm
 // never qualify (an untrained MLP's steps, with their common offset, are such), and the test costs 0.04 ms a step.
 // Read when the products are enqueued.
@@ -374,7 +374,7 @@ bool env_slices_lds() {
   return !(e && e[0] == '0');
 }
 
-bool env_ns_bf() {
+bool env_ns_hf() {
   const char* e = getenv("PYLO_MI355_NS_F32");
   return !(e && e[0] == '1');
 }
@@ -420,13 +420,13 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
     const TDesc& d = L.descs[t];
     if (d.n == 0 || (shapes[t].flags & PYLO_F_NO_ORTHOGONALIZE)) continue;
     // two dims; or more, as one matrix per slice of the last two, where the per-slice launches do not take the
-    // slices (k_slice_finish.h) -- the split-bf16 kernels only, whose tables carry a matrix's place in its tensor
-    const bool slices = d.mode == kModeFacND && L.ns_bf && L.slice_of_tensor[t] < 0;
+    // slices (k_slice_finish.h) -- the split-fp16 kernels only, whose tables carry a matrix's place in its tensor
+    const bool slices = d.mode == kModeFacND && L.ns_hf && L.slice_of_tensor[t] < 0;
     if (d.mode != kModeFac2D && !slices) continue;
     const int R = slices ? (int)shapes[t].shape[shapes[t].ndim - 2] : d.R0;
     const int C = slices ? (int)shapes[t].shape[shapes[t].ndim - 1] : d.C0;
     // the fp32 kernels load 16 bytes at a time along the contiguous dim of X, A and B'
-    if (!L.ns_bf && (C % 4 != 0 || std::min(R, C) % 4 != 0)) continue;
+    if (!L.ns_hf && (C % 4 != 0 || std::min(R, C) % 4 != 0)) continue;
     const int n_sl = slices ? (int)(d.n / ((long long)R * C)) : 1;
     for (int sl = 0; sl < n_sl; ++sl) {
     NsMat mt{};
@@ -466,14 +466,14 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
     L.ns_mats.push_back(mt);
     }
   }
-  if (L.ns_bf) {
-    // same matrices, operands as bf16 planes; the item tables are rebuilt for the uniform (n x m) orientation
+  if (L.ns_hf) {
+    // same matrices, operands as fp16 planes; the item tables are rebuilt for the uniform (n x m) orientation
     L.ns_gram.clear(); L.ns_poly.clear(); L.ns_upd.clear(); L.ns_upd4.clear();
     ws_floats = 0;
     long long pw = 0;
     auto take_p = [&](long long n) { const long long o = pw; pw += (n + 63) / 64 * 64; return o; };
     auto up = [](int x, int q) { return (x + q - 1) / q * q; };
-    auto up16 = [&](int x) { return up(x, kBfBK); };
+    auto up16 = [&](int x) { return up(x, kHfBK); };
     // Planes and fp32 matrices of every matrix.  The planes are only live during a matrix's own products, so
     // the matrices are cut into batches (in tensor order) whose planes fit PYLO_MI355_NS_WORKSPACE_MB (8192 by
     // default); the batches run one after another in the same memory.  A plan whose matrices fit in one batch
@@ -491,7 +491,7 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
     };
     for (size_t q = 0; q < L.ns_mats.size(); ++q) {
       const NsMat& f = L.ns_mats[q];
-      NsBfMat b{};
+      NsHfMat b{};
       b.tensor = f.tensor; b.R = f.R; b.C = f.C; b.m = f.m; b.n = std::max(f.R, f.C); b.tall = f.tall;
       b.pad_m = up16(b.m);
       b.pad_n = up16(b.n);
@@ -553,7 +553,7 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       struct Run { int q0, q1; double work; };
       std::vector<Run> runs;
       for (int q = bt.mat0; q < bt.mat0 + bt.n_mats; ++q) {
-        const NsBfMat& b = L.nsb_mats[q];
+        const NsHfMat& b = L.nsb_mats[q];
         // (five iterations in pairs: three Gram products on the upper blocks and three updates, eleven m x m products)
         const double w = (double)b.m * b.m * (4.6 * b.n + 5.9 * b.m);
         if (!runs.empty() && L.nsb_mats[runs.back().q0].tensor == b.tensor) { runs.back().q1 = q + 1; runs.back().work += w; }
@@ -581,13 +581,13 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
       grp.fitem0 = (int)L.ns_flag_items.size();
       for (int q : members[g]) {
         {
-          NsBfMat& bw = L.nsb_mats[q];
+          NsHfMat& bw = L.nsb_mats[q];
           bw.fpart0 = L.ns_fpart_total;
           bw.n_fpart = (int)(((long long)bw.m * bw.m + kNsFlagChunk - 1) / kNsFlagChunk);
           L.ns_fpart_total += bw.n_fpart;
           for (int c = 0; c < bw.n_fpart; ++c) L.ns_flag_items.push_back(Item{q, c, 0, 0});
         }
-        const NsBfMat& b = L.nsb_mats[q];
+        const NsHfMat& b = L.nsb_mats[q];
         L.ns_list.push_back(q);
         L.ns_group_of_tensor[b.tensor] = (int)L.ns_groups.size();
         for (int tr = 0; tr < (b.R + 63) / 64; ++tr)
@@ -957,7 +957,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
   if (kind == PYLO_KIND_CELO2 || kind == PYLO_KIND_VELO) build_elem_items(L, T, kind);
   long long ns_floats = 0;
   if (kind == PYLO_KIND_CELO2) {
-    L.ns_bf = env_ns_bf();
+    L.ns_hf = env_ns_hf();
     build_slice_tables(L, shapes, T);
     build_ns_tables(L, shapes, T, ns_floats);
     if (int rc = build_fin_tables(L, shapes, T)) return rc;
@@ -1038,10 +1038,10 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
     L.off_ns_fpart = take(sizeof(float) * (size_t)L.ns_fpart_total);
     L.off_ns_flag_items = take(sizeof(Item) * L.ns_flag_items.size());
     L.off_ns_ws = take(sizeof(float) * (size_t)ns_floats);
-    L.off_nsb_mats = take(sizeof(NsBfMat) * L.nsb_mats.size());
+    L.off_nsb_mats = take(sizeof(NsHfMat) * L.nsb_mats.size());
     L.off_nsb_split_items = take(sizeof(NsTileItem) * L.nsb_split_items.size());
     L.off_ns_list = take(sizeof(int) * L.ns_list.size());
-    L.off_ns_pw = take(sizeof(bfbits) * (size_t)L.nsb_plane_elems);
+    L.off_ns_pw = take(sizeof(hbits) * (size_t)L.nsb_plane_elems);
     L.off_slice_mats = take(sizeof(SliceMat) * L.slice_mats.size());
     for (int k = 0; k < kSliceLaneSets; ++k) L.off_slice_items_l[k] = take(sizeof(Item) * L.slice_items_l[k].size());
     L.off_slice_items_w = take(sizeof(Item) * L.slice_items_w.size());
@@ -1152,7 +1152,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_ns_upd4, L.ns_upd4.data(), sizeof(NsItem) * L.ns_upd4.size());
   if (e == hipSuccess) e = up(L.off_ns_split, L.ns_split.data(), sizeof(int) * L.ns_split.size());
   if (e == hipSuccess && kind == PYLO_KIND_CELO2) e = up(L.off_ns_xalt, L.ns_xalt.data(), sizeof(long long) * L.ns_xalt.size());
-  if (e == hipSuccess) e = up(L.off_nsb_mats, L.nsb_mats.data(), sizeof(NsBfMat) * L.nsb_mats.size());
+  if (e == hipSuccess) e = up(L.off_nsb_mats, L.nsb_mats.data(), sizeof(NsHfMat) * L.nsb_mats.size());
   if (e == hipSuccess) e = up(L.off_nsb_split_items, L.nsb_split_items.data(), sizeof(NsTileItem) * L.nsb_split_items.size());
   if (e == hipSuccess) e = up(L.off_ns_list, L.ns_list.data(), sizeof(int) * L.ns_list.size());
   if (e == hipSuccess) e = up(L.off_ns_flag_items, L.ns_flag_items.data(), sizeof(Item) * L.ns_flag_items.size());
@@ -1163,7 +1163,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   if (e == hipSuccess) e = up(L.off_slice_items_b, L.slice_items_b.data(), sizeof(Item) * L.slice_items_b.size());
   // the padding of the operand planes is read by the products and written by nobody: zero, once
   if (e == hipSuccess && L.nsb_plane_elems > 0)
-    e = hipMemsetAsync(P->ws + L.off_ns_pw, 0, sizeof(bfbits) * (size_t)L.nsb_plane_elems, s);
+    e = hipMemsetAsync(P->ws + L.off_ns_pw, 0, sizeof(hbits) * (size_t)L.nsb_plane_elems, s);
   if (e == hipSuccess) e = hipStreamSynchronize(s);
   for (int i = 0; i < kStageSlots && e == hipSuccess; ++i) {
     e = hipHostMalloc(reinterpret_cast<void**>(&P->stage[i]), (sizeof(PyloTensorArgs) * n_tensors + 15) / 16 * 16,
@@ -1589,9 +1589,9 @@ extern "C" int pylo_mi355_celo2_step(PyloPlan* P, const PyloTensorArgs* args, co
 
 namespace {
 
-// The split-bf16 product kernels take their LDS as dynamic shared memory; tiles of 256 columns need more than
+// The split-fp16 product kernels take their LDS as dynamic shared memory; tiles of 256 columns need more than
 // the 64 KB a kernel may have without asking.
-int ns_bf_lds_once() {
+int ns_hf_lds_once() {
   static std::mutex mu;
   static std::vector<int> done;   // devices on which the attribute has been set
   int dev = 0;
@@ -1599,12 +1599,12 @@ int ns_bf_lds_once() {
   std::lock_guard<std::mutex> lock(mu);
   for (int d : done)
     if (d == dev) return 0;
-  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsGram, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(2)));
-  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsPoly, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(2)));
-  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsProd, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(2)));
-  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsProdA, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(2)));
-  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsUpdate, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(2)));
-  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_bf_gemm<kNsUpdate, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(4)));
+  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_hf_gemm<kNsGram, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(2)));
+  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_hf_gemm<kNsPoly, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(2)));
+  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_hf_gemm<kNsProd, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(2)));
+  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_hf_gemm<kNsProdA, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(2)));
+  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_hf_gemm<kNsUpdate, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(2)));
+  HIP_TRY(hipFuncSetAttribute((const void*)k_ns_hf_gemm<kNsUpdate, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(4)));
   done.push_back(dev);
   return 0;
 }
@@ -1705,8 +1705,8 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
   };
   if (!any_ns) {
     finish_range(s, 0, n_fin, 0, (int)L.fin_units.size(), nullptr, nullptr);
-  } else if (L.ns_bf) {
-    // The split-bf16 kernels.  Every group of matrices is a chain of its own from the norms of its raw steps to the
+  } else if (L.ns_hf) {
+    // The split-fp16 kernels.  Every group of matrices is a chain of its own from the norms of its raw steps to the
     // update of its parameters, on a stream of its own (the first group on the caller's): the memory-bound ends of
     // one chain run under the matrix products of the others.
     const NsMat* mats = P->at<NsMat>(L.off_ns_mats);
@@ -1718,10 +1718,10 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
     const int* list = P->at<int>(L.off_ns_list);
     float* scale = P->at<float>(L.off_ns_scale);
     float* ns_ws = P->at<float>(L.off_ns_ws);
-    const NsBfMat* bmats = P->at<NsBfMat>(L.off_nsb_mats);
+    const NsHfMat* bmats = P->at<NsHfMat>(L.off_nsb_mats);
     const NsTileItem* sitems = P->at<NsTileItem>(L.off_nsb_split_items);
-    bfbits* pw = P->at<bfbits>(L.off_ns_pw);
-    if (int rc = ns_bf_lds_once()) return rc;
+    hbits* pw = P->at<hbits>(L.off_ns_pw);
+    if (int rc = ns_hf_lds_once()) return rc;
     finish_range(s, L.fin_rest0, L.n_fin_rest, L.unit_rest0, L.n_unit_rest, nullptr, nullptr);   // tensors of no group
     const bool several = L.ns_batches.size() > 1;
     const float c0 = coeffs[0], c1 = coeffs[1], c2 = coeffs[2];
@@ -1736,7 +1736,7 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
     for (const NsBatch& bt : L.ns_batches) {
       // the planes' padding: zero from plan creation on when one batch has the memory to itself
       if (several) {
-        const size_t n16 = (size_t)bt.plane_elems * sizeof(bfbits) / 16;
+        const size_t n16 = (size_t)bt.plane_elems * sizeof(hbits) / 16;
         hipLaunchKernelGGL(k_ns_zero, dim3((unsigned)std::min<size_t>((n16 + 255) / 256, 1u << 16)), dim3(256), 0, s,
                            reinterpret_cast<u32x4*>(pw), n16);
       }
@@ -1757,7 +1757,7 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
           hipLaunchKernelGGL(k_ns_scale, dim3(G.n_list), dim3(256), 0, sg, mats, list + G.list0, G.n_list, units, fin_part,
                              ns_eps, scale);
         if (G.n_sitems > 0)
-          hipLaunchKernelGGL(k_ns_bf_split, dim3((unsigned)G.n_sitems), dim3(256), 0, sg, bmats, sitems + G.sitem0, dyn,
+          hipLaunchKernelGGL(k_ns_hf_split, dim3((unsigned)G.n_sitems), dim3(256), 0, sg, bmats, sitems + G.sitem0, dyn,
                              (const float*)scale, pw, pow2(ex.x));
       }
       // The launch sequence of one group (every group runs the same one on its own tables), then its launches,
@@ -1801,7 +1801,7 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
         par ^= 1;
       };
       if (adaptive) {
-        // First chain: two iterations for every matrix, a third for those whose flag says so (k_ns_bf_chain_flag),
+        // First chain: two iterations for every matrix, a third for those whose flag says so (k_ns_hf_chain_flag),
         // then pairs for all -- the last of them is the end for the flagged ones -- and one iteration more for the others.
         const NsPick longer{chain_flags, kNsLongOnly, 0, 0, 0.0f}, shorter{chain_flags, kNsShortOnly, 0, 0, 0.0f};
         const int n_pairs = (ns_iters - 3) / 2;
@@ -1821,7 +1821,7 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
       } else {
         int done = 0;
         for (size_t ch = 0; ch < chains.size(); ++ch) {
-          // a chain of iterations: one Gram product, 4 len - 3 products of m x m matrices and one update (k_ns_bf.h)
+          // a chain of iterations: one Gram product, 4 len - 3 products of m x m matrices and one update (k_ns_hf.h)
           done += chains[ch];
           open_chain(all);
           for (int j = 1; j < chains[ch]; ++j) extend(all);
@@ -1834,35 +1834,35 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
           hipStream_t sg = stream_of(g);
           auto small = [&](auto kern) {
             if (G.n_poly > 0)
-              hipLaunchKernelGGL(kern, dim3(G.n_poly), dim3(256), bf_gemm_lds(2), sg, bmats, poly + G.poly0, dyn, ns_ws, pw,
+              hipLaunchKernelGGL(kern, dim3(G.n_poly), dim3(256), hf_gemm_lds(2), sg, bmats, poly + G.poly0, dyn, ns_ws, pw,
                                  op.par, op.last, op.b, c0, c1, c2, op.pick);
           };
           switch (op.kind) {
             case kOpGram:
               if (G.n_gram > 0)
-                hipLaunchKernelGGL((k_ns_bf_gemm<kNsGram, 2>), dim3(G.n_gram), dim3(256), bf_gemm_lds(2), sg, bmats,
+                hipLaunchKernelGGL((k_ns_hf_gemm<kNsGram, 2>), dim3(G.n_gram), dim3(256), hf_gemm_lds(2), sg, bmats,
                                    gram + G.gram0, dyn, ns_ws, pw, op.par, op.last, op.b, c0, c1, c2, op.pick);
               if (G.n_split > 0)
-                hipLaunchKernelGGL(k_ns_bf_gram_reduce, dim3(((size_t)G.split_max_m * G.split_max_m + 255) / 256, G.n_split),
+                hipLaunchKernelGGL(k_ns_hf_gram_reduce, dim3(((size_t)G.split_max_m * G.split_max_m + 255) / 256, G.n_split),
                                    dim3(256), 0, sg, bmats, split + G.split0, dyn, ns_ws, pw, op.pick, op.b.out_scale);
               break;
             case kOpFlag:
               if (G.n_list > 0) {
-                hipLaunchKernelGGL(k_ns_bf_chain_sumsq, dim3(G.n_fitems), dim3(256), 0, sg, bmats, flag_items + G.fitem0, dyn,
+                hipLaunchKernelGGL(k_ns_hf_chain_sumsq, dim3(G.n_fitems), dim3(256), 0, sg, bmats, flag_items + G.fitem0, dyn,
                                    (const float*)ns_ws, chain_part);
-                hipLaunchKernelGGL(k_ns_bf_chain_flag, dim3(G.n_list), dim3(64), 0, sg, bmats, list + G.list0, dyn,
+                hipLaunchKernelGGL(k_ns_hf_chain_flag, dim3(G.n_list), dim3(64), 0, sg, bmats, list + G.list0, dyn,
                                    (const float*)chain_part, chain_tau2, chain_flags);
               }
               break;
-            case kOpPoly: small(k_ns_bf_gemm<kNsPoly, 2>); break;
-            case kOpProd: small(k_ns_bf_gemm<kNsProd, 2>); break;
-            case kOpProdA: small(k_ns_bf_gemm<kNsProdA, 2>); break;
+            case kOpPoly: small(k_ns_hf_gemm<kNsPoly, 2>); break;
+            case kOpProd: small(k_ns_hf_gemm<kNsProd, 2>); break;
+            case kOpProdA: small(k_ns_hf_gemm<kNsProdA, 2>); break;
             case kOpUpdate:
               if (G.n_upd4 > 0)
-                hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 4>), dim3(G.n_upd4), dim3(256), bf_gemm_lds(4), sg, bmats,
+                hipLaunchKernelGGL((k_ns_hf_gemm<kNsUpdate, 4>), dim3(G.n_upd4), dim3(256), hf_gemm_lds(4), sg, bmats,
                                    upd4 + G.upd40, dyn, ns_ws, pw, op.par, op.last, op.b, c0, c1, c2, op.pick);
               if (G.n_upd > 0)
-                hipLaunchKernelGGL((k_ns_bf_gemm<kNsUpdate, 2>), dim3(G.n_upd), dim3(256), bf_gemm_lds(2), sg, bmats,
+                hipLaunchKernelGGL((k_ns_hf_gemm<kNsUpdate, 2>), dim3(G.n_upd), dim3(256), hf_gemm_lds(2), sg, bmats,
                                    upd + G.upd0, dyn, ns_ws, pw, op.par, op.last, op.b, c0, c1, c2, op.pick);
               break;
           }
@@ -2522,13 +2522,13 @@ extern "C" int pylo_mi355_stream_probe(const float* in, float* out, size_t n, in
 // ---------------------------------------------------------------------------------------------
 namespace {
 
-// The main loop of k_ns_bf_gemm<kNsUpdate, 4> (128 x 256 outputs, three v_mfma_f32_32x32x16_f16 per pair of
+// The main loop of k_ns_hf_gemm<kNsUpdate, 4> (128 x 256 outputs, three v_mfma_f32_32x32x16_f16 per pair of
 // 32 x 32 blocks and 16 reduction steps) over synthetic planes.  MODE 0: as in the product (operands staged
 // from memory into LDS every 16 steps); 1: the first stage is staged once and read from LDS in every step (no
 // global loads, no barriers); 2: the first stage's fragments stay in registers (matrix instructions only).
 template <int MODE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k_matrix_probe(
-    const bfbits* __restrict__ X, int rows_x, const bfbits* __restrict__ B, int rows_b, int K, float* __restrict__ out) {
+    const hbits* __restrict__ X, int rows_x, const hbits* __restrict__ B, int rows_b, int K, float* __restrict__ out) {
   extern __shared__ __attribute__((aligned(16))) char lds_[];
   PYLO_LDS char* lds = (PYLO_LDS char*)lds_;
   constexpr int WN = 4, RB = 64 * WN, SA = 128 * kNsRowB;
@@ -2540,24 +2540,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
     for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-  const BfPlanes PX{X, rows_x}, PB{B, rows_b};
+  const HfPlanes PX{X, rows_x}, PB{B, rows_b};
   if (MODE == 0) {
-    bf_tile_product<WN>(PX, i0, PB, j0, 0, K, lds, acc);
+    hf_tile_product<WN>(PX, i0, PB, j0, 0, K, lds, acc);
   } else {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wi = (wave >> 1) * 64, wj = (wave & 1) * 32 * WN;
     const int kg = lane >> 5, lo = lane & 31;
     int offa[128 * kNsRowPc / 256], offb[RB * kNsRowPc / 256];
-    bf_stage_offsets<128>(wave, lane, offa);
-    bf_stage_offsets<RB>(wave, lane, offb);
-    bf_stage_issue<128>((const char*)X + (size_t)i0 * kNsRowB, offa, lds, wave);
-    bf_stage_issue<RB>((const char*)B + (size_t)j0 * kNsRowB, offb, lds + SA, wave);
+    hf_stage_offsets<128>(wave, lane, offa);
+    hf_stage_offsets<RB>(wave, lane, offb);
+    hf_stage_issue<128>((const char*)X + (size_t)i0 * kNsRowB, offa, lds, wave);
+    hf_stage_issue<RB>((const char*)B + (size_t)j0 * kNsRowB, offb, lds + SA, wave);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     const int sw = 16 * (kg ^ ((lo >> 2) & 3));
     const int oa = (wi + lo) * kNsRowB + sw, ob = SA + (wj + lo) * kNsRowB + sw;
     f16x8 a[2][kNsPl], b[WN][kNsPl];
-    for (int k = 0; k < K; k += kBfBK) {
+    for (int k = 0; k < K; k += kHfBK) {
       if (MODE == 1 || k == 0) {
 #pragma unroll
         for (int q = 0; q < kNsPl; ++q) {
@@ -2602,15 +2602,15 @@ extern "C" int pylo_mi355_matrix_probe(const void* x_planes, int rows_x, const v
   static std::mutex mu;
   {
     std::lock_guard<std::mutex> lock(mu);
-    HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<0>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(4)));
-    HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<1>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(4)));
-    HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<2>, hipFuncAttributeMaxDynamicSharedMemorySize, bf_gemm_lds(4)));
+    HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<0>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(4)));
+    HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<1>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(4)));
+    HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<2>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(4)));
   }
-  const bfbits* X = static_cast<const bfbits*>(x_planes);
-  const bfbits* B = static_cast<const bfbits*>(b_planes);
-  if (mode == 0) hipLaunchKernelGGL(k_matrix_probe<0>, dim3(grid), dim3(256), bf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
-  else if (mode == 1) hipLaunchKernelGGL(k_matrix_probe<1>, dim3(grid), dim3(256), bf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
-  else hipLaunchKernelGGL(k_matrix_probe<2>, dim3(grid), dim3(256), bf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
+  const hbits* X = static_cast<const hbits*>(x_planes);
+  const hbits* B = static_cast<const hbits*>(b_planes);
+  if (mode == 0) hipLaunchKernelGGL(k_matrix_probe<0>, dim3(grid), dim3(256), hf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
+  else if (mode == 1) hipLaunchKernelGGL(k_matrix_probe<1>, dim3(grid), dim3(256), hf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
+  else hipLaunchKernelGGL(k_matrix_probe<2>, dim3(grid), dim3(256), hf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
   HIP_TRY(hipGetLastError());
   return 0;
 }

@@ -213,7 +213,7 @@ class ELO_CELO2_CUDA(Optimizer):
         return out
 
     def _ensure_plan(self, tensors):
-        # the plan reserves Newton-Schulz workspace (18 bytes per element) only for the tensors whose group
+        # the plan reserves Newton-Schulz workspace (12 bytes per element) only for the tensors whose group
         # orthogonalises through the library
         no_ns = [not (group["orthogonalize"] and self._lib_ns and self.ns_iters > 0) for group, _p, _a in tensors]
         key = tuple((tuple(p.shape), adam, p.dtype, skip) for (_, p, adam), skip in zip(tensors, no_ns))
@@ -472,7 +472,7 @@ class ELO_CELO2_CUDA(Optimizer):
     def finish_step(self, tensors):
         """Newton-Schulz, RMS normalisation and the parameter update of the MLP tensors
         (pylo/optim/ELO_CELO2_cuda.py:288-296).  Matrices are orthogonalised by the library's own matrix-pipe
-        kernels inside the finishing call (fp32 accuracy on the bf16 matrix instructions, any two dims; with
+        kernels inside the finishing call (fp32 accuracy on the fp16 matrix instructions, any two dims; with
         ``PYLO_MI355_NS_F32=1`` the fp32 matrix instructions, dims that are multiples of 4); tensors with more
         than two dims slice by slice of their last two dims, small slices in launches that hold a slice in
         registers or LDS, large ones as matrices of the same products.  Batched torch products remain for what the

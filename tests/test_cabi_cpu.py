@@ -46,10 +46,10 @@ def test_workspace_sizing_and_error_paths_without_gpu():
     n = C.c_size_t(0)
     shapes = _lib.make_shapes([(50257, 768), (768,), (768, 2304)], [0, _lib.F_ADAM, 0])
     assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, shapes, 3, C.byref(n)) == 0
-    # partial sums and tables are a few % of the 154 MB tensor; the Newton-Schulz operand planes (three bf16
-    # planes of X in both orientations, the second of them twice) add 18 bytes per matrix element
+    # partial sums and tables are a few % of the 154 MB tensor; the Newton-Schulz operand planes (two fp16
+    # planes of X in both orientations, the second of them twice) add 12 bytes per matrix element
     n_mat = 50257 * 768 + 768 * 2304
-    assert 18 * n_mat < n.value < 24 * n_mat
+    assert 12 * n_mat < n.value < 16 * n_mat
     # a CELO2 tensor with fewer than two dims and no AdamW flag takes the MLP (use_adamw_for_1d=False)
     mlp1d = _lib.make_shapes([(768,)], [0])
     assert lib.pylo_mi355_plan_workspace_bytes(_lib.KIND_CELO2, mlp1d, 1, C.byref(n)) == 0

@@ -656,9 +656,9 @@ def other_workload(workload, steps, warmup):
             "algorithmic_bytes_per_launch": n2d * b_elem + n1d * b_vec, "avg_launch_ms": float(mean[k])}
     if workload == "llama_adafac":
         # The 16 -> 32 -> 32 -> 2 element MLP: 1 600 FMAs per element of a >= 2-D tensor.  By default its two
-        # wide layers (1 536 FMAs) run on the bf16 matrix instructions with three-plane operands, six bf16
+        # wide layers (1 536 FMAs) run on the fp16 matrix instructions with two-plane operands, three fp16
         # products per fp32 product, and the kernel is bound by its vector instructions (the splitting of the
-        # activations is vector work; the bf16 matrix instructions run under it about half of the time);
+        # activations is vector work; the matrix instructions run under it);
         # PYLO_MI355_ADAFAC_F32=1 runs the layers on the fp32 matrix instructions.
         t = float(mean[k]) * 1e-3
         f32 = os.environ.get("PYLO_MI355_ADAFAC_F32") == "1"
@@ -667,8 +667,8 @@ def other_workload(workload, steps, warmup):
             roof = {"bound": "mfma", "kernel": "k_adafac_apply_tile (fp32 matrix instructions)", "achieved": fp32_tflops,
                     "peak": 157.3, "unit": "TFLOP/s", "frac": fp32_tflops / 157.3}
         else:
-            bf = n2d * 6 * 1536 * 2.0 / t / 1e12
-            roof = {"bound": "mfma", "kernel": "k_adafac_apply_tile (bf16 matrix instructions, 6 products per fp32 product)",
+            bf = n2d * 3 * 1536 * 2.0 / t / 1e12
+            roof = {"bound": "mfma", "kernel": "k_adafac_apply_tile (fp16 matrix instructions, 3 products per fp32 product)",
                     "achieved": bf, "peak": 2500.0, "unit": "TFLOP/s", "frac": bf / 2500.0,
                     "fp32_equivalent_TFLOPs": fp32_tflops, "fp32_matrix_peak_TFLOPs": 157.3}
         roof.update({"traffic": None, "avg_launch_ms": float(mean[k]), "hbm_GBps": apply_gbs})

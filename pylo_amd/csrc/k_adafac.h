@@ -18,7 +18,7 @@ namespace pylo {
 #endif
 constexpr int kAH = 32;
 constexpr int kAW1 = 0, kAB1 = 960, kAWT = 992, kAWH = 1344, kABH = 2368, kAWO = 2400, kABO = 2464, kANet = 2466;
-constexpr int kAFold = 960;  // per-tensor first-layer rows scaled by the channel normalisers
+constexpr int kAFold = 992;  // per-tensor first-layer rows scaled by the channel normalisers, then the 30 normalisers themselves
 
 __host__ __device__ constexpr bool adafac_channel(int c) { return c != 1 && c != 14; }
 
@@ -182,6 +182,7 @@ __global__ __launch_bounds__(kThreads) void k_adafac_fold(const TDesc* __restric
   __syncthreads();
   float* w = wfold + (size_t)t * kAFold;
   for (int i = threadIdx.x; i < 30 * kAH; i += kThreads) w[i] = net[kAW1 + i] * sc[i / kAH];
+  if (threadIdx.x < 32) w[30 * kAH + threadIdx.x] = threadIdx.x < 30 ? sc[threadIdx.x] : 0.0f;
 }
 
 // Parameter update from the unit step direction * exp(magnitude * exp_mult).  AdafacLO
@@ -467,22 +468,24 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
   }
 }
 
-// ---- the same pass with the element MLP on the bf16 matrix instructions at fp32 accuracy ----------------
-// An fp32 number is the exact sum of three bf16 numbers (8 + 8 + 8 significand bits; taken by truncation:
-// h = x & 0xffff0000, m = (x - h) & 0xffff0000, l = x - h - m, every step exact), and a product of two such
-// sums is the six products h h, h m, m h, m m, h l, l h, each exact in fp32, plus m l + l m + l l, which are
-// dropped.  With truncation |m| < 2^-7 |x| and |l| < 2^-14 |x|, and the three planes have the sign of x: what is
-// dropped is below 2^-20 of |x y| in the worst case (2^-22 on average over the mantissas) and one-signed, a bias
-// towards zero per product; in a dot product of the MLP's width it stays below the rounding of the fp32
-// accumulation, which is what the comparisons with the fp64 evaluation show (the steps of this kernel and of the
-// fp32-instruction one sit at the same distance from it).  The split by rounding that the Newton-Schulz planes
-// use (|m| <= 2^-8, |l| <= 2^-16, signs mixed: 2^-23, unbiased) costs 7 vector instructions a value against
-// 5.5 here, in a kernel that is bound by exactly these instructions.  One
-// v_mfma_f32_32x32x16_bf16 does sixteen times the multiply-adds of v_mfma_f32_16x16x4_f32 in the same 32
-// cycles, so six of them per fp32 product leave 36 matrix instructions per row of 64 elements where the
-// fp32 instructions need 96; the price is vector work (bf16 matrix instructions run under vector instructions of
-// the SIMD's waves about half of the time, fp32 ones never did, but the vector pipe is what fills up):
-// splitting the 16 features and the 2 x 16 hidden values a lane holds costs 5.5 instructions a value.
+// ---- the same pass with the element MLP on the fp16 matrix instructions at fp32 accuracy ----------------
+// An fp32 number within fp16's range is, to 2^-23 of its size, the sum of two fp16 numbers taken by rounding
+// (h = fp16(x), l = fp16(x - h): v_cvt_pk_f16_f32 converts and packs two values in one instruction), and a product
+// of two such sums is the three products h h, h l, l h, each exact in fp32, plus l l (2^-24 of |x y|), which is
+// dropped with the remainders: about 2^-22 of a product, unbiased -- below the rounding of the fp32 accumulation.
+// Range: fp16 ends at 65 504 and resolves 6e-8 absolutely at its lower end, so the operands must be of order one.
+// The hidden values and the weights are; the raw features are not (a second moment of 1e-12 next to its
+// reciprocal root of 1e6), which is why this variant does not use the first-layer rows folded with the channel
+// normalisers: it multiplies each feature by its normaliser (unit second moment over the tensor afterwards, so
+// no feature exceeds sqrt(n) < 46 341 in a tensor of n < 2^31 elements; sixteen multiplications an element) and
+// takes the first layer's rows as they are.  The hidden values are clamped at 65 000 by the instruction that is
+// their ReLU anyway (one as large takes normalised features of 1e4 and more, i.e. a single outlier in a tensor
+// of 1e8 elements).
+// Three v_mfma_f32_32x32x16_f16 per fp32 product leave 18 matrix instructions per row of 64 elements where the
+// fp32 instructions need 96 and three bf16 planes needed 36; the split costs 3.25 vector instructions a value
+// (two conversions and a subtraction per value, a packing conversion per pair and plane) where three bf16
+// planes cost 5.5, in a kernel that is bound by exactly these instructions: splitting the 16 features and the
+// 2 x 16 hidden values a lane holds.
 //
 // Layouts (lane = 32 half + e): units are the M dimension, elements the N dimension, inputs the K
 // dimension.  A operand: lane holds reduction slots 8 half .. 8 half + 7 of unit e.  B operand: lane holds
@@ -496,31 +499,28 @@ __device__ __forceinline__ void adafac_apply_tile(const TDesc& d, const PyloTens
 // Hidden layer: which hidden unit a reduction slot stands for is free as long as both operands agree, so slot
 // 8 half + 4 q + i of step s is unit 8 (2 s + q) + 4 half + i: exactly the sixteen units the lane holds in D
 // after the first layer.  The hidden values never leave their lane; nothing goes through LDS.
-typedef __bf16 abf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 ah16x8 __attribute__((ext_vector_type(8)));
 typedef float av16f __attribute__((ext_vector_type(16)));
 typedef unsigned int au32x4 __attribute__((ext_vector_type(4)));
 
-struct Bf3 { unsigned h, m, l; };   // fp32 bit patterns whose upper halves are the three bf16 planes
-
-__device__ __forceinline__ Bf3 bf3_split(float x) {
-  Bf3 r;
-  r.h = __float_as_uint(x) & 0xffff0000u;
-  const float r1 = x - __uint_as_float(r.h);
-  r.m = __float_as_uint(r1) & 0xffff0000u;
-  r.l = __float_as_uint(r1 - __uint_as_float(r.m));   // at most 8 significant bits left: its lower half is zero
-  return r;
+// two values -> one dword of each plane (`a` in the lower halves), by rounding (v_cvt_pk_f16_f32)
+typedef float af32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 ah16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void hf2_split2(float a, float b, unsigned& h, unsigned& l) {
+  const ah16x2 hh = __builtin_convertvector(af32x2{a, b}, ah16x2);
+  const ah16x2 ll = __builtin_convertvector(af32x2{a - (float)hh[0], b - (float)hh[1]}, ah16x2);
+  h = __builtin_bit_cast(unsigned, hh);
+  l = __builtin_bit_cast(unsigned, ll);
 }
-// upper halves of two fp32 patterns as one dword, `lo` in the lower half
-__device__ __forceinline__ unsigned bf_pack(unsigned lo, unsigned hi) { return __builtin_amdgcn_perm(hi, lo, 0x07060302u); }
 
-// eight values (consecutive inputs of a matrix operand) as three planes of eight bf16
-__device__ __forceinline__ void bf3_pack8(const float (&x)[8], au32x4 (&pl)[3]) {
+// eight values (consecutive inputs of a matrix operand) as two planes of eight fp16
+__device__ __forceinline__ void hf2_pack8(const float (&x)[8], au32x4 (&pl)[2]) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const Bf3 a = bf3_split(x[2 * i]), b = bf3_split(x[2 * i + 1]);
-    pl[0][i] = bf_pack(a.h, b.h);
-    pl[1][i] = bf_pack(a.m, b.m);
-    pl[2][i] = bf_pack(a.l, b.l);
+    unsigned h, l;
+    hf2_split2(x[2 * i], x[2 * i + 1], h, l);
+    pl[0][i] = h;
+    pl[1][i] = l;
   }
 }
 
@@ -531,13 +531,13 @@ __device__ __forceinline__ void half_swap(unsigned& a, unsigned& b) {
   b = r[1];
 }
 
-// acc += W (three planes) x act (three planes), smallest terms first
-__device__ __forceinline__ av16f bf3_mfma(const au32x4 (&w)[3], const au32x4 (&x)[3], av16f acc) {
-  constexpr int pw[6] = {2, 0, 1, 1, 0, 0}, px[6] = {0, 2, 1, 0, 1, 0};
+// acc += W (two planes) x act (two planes), smallest terms first
+__device__ __forceinline__ av16f hf2_mfma(const au32x4 (&w)[2], const au32x4 (&x)[2], av16f acc) {
+  constexpr int pw[3] = {1, 0, 0}, px[3] = {0, 1, 0};
 #pragma unroll
-  for (int t = 0; t < 6; ++t)
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(abf16x8, w[pw[t]]), __builtin_bit_cast(abf16x8, x[px[t]]),
-                                                  acc, 0, 0, 0);
+  for (int t = 0; t < 3; ++t)
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(ah16x8, w[pw[t]]), __builtin_bit_cast(ah16x8, x[px[t]]),
+                                                 acc, 0, 0, 0);
   return acc;
 }
 
@@ -545,7 +545,7 @@ __device__ __forceinline__ av16f bf3_mfma(const au32x4 (&w)[3], const au32x4 (&x
 // indexed by the column has an entry per (row, column mod P), so a lane fetches the row's factor and first-layer
 // terms for its own columns (one per element group) instead of sharing one entry with the wave.
 template <bool PER>
-__device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloTensorArgs& a, int task,
+__device__ __forceinline__ void adafac_apply_tile_hf(const TDesc& d, const PyloTensorArgs& a, int task,
                                                      const EmaConsts& e, const float* __restrict__ fac_tab,
                                                      const float* __restrict__ term_tab, const float* wfold_t,
                                                      const float* net) {
@@ -553,19 +553,26 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
   const int lane = threadIdx.x & 63, half = lane >> 5, el = lane & 31;
   // A operands: first layer (unit el, inputs 8 half ..), hidden layer per reduction step s (slot 8 half + 4 q + i:
   // hidden unit 8 (2 s + q) + 4 half + i)
-  au32x4 w1[3], w2[2][3];
+  au32x4 w1[2], w2[2][2];
   {
     float x[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) x[i] = *(const gfloat*)(wfold_t + adafac_elem_row(8 * half + i) * kAH + el);
-    bf3_pack8(x, w1);
+    for (int i = 0; i < 8; ++i) x[i] = *(const gfloat*)(net + kAW1 + adafac_elem_row(8 * half + i) * kAH + el);
+    hf2_pack8(x, w1);
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
 #pragma unroll
       for (int i = 0; i < 8; ++i)
         x[i] = *(const gfloat*)(net + kAWH + (8 * (2 * s + (i >> 2)) + 4 * half + (i & 3)) * kAH + el);
-      bf3_pack8(x, w2[s]);
+      hf2_pack8(x, w2[s]);
     }
+  }
+  // the normalisers of the sixteen features an element brings itself (the first layer's rows are not folded here)
+  float fsc[16];
+  {
+    const cfloat* sc = launder(wfold_t + 30 * kAH);
+#pragma unroll
+    for (int c = 0; c < 16; ++c) fsc[c] = sc[adafac_elem_row(c)];
   }
   // what belongs to the units this lane holds in D: hidden bias, output weights
   av16f bh;
@@ -644,6 +651,11 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
     lo_features(gg, xp[0], m, xr_[0], rfcf, 1e-6f, f18);
     float flo[8] = {f18[0], f18[2], f18[3], f18[4], f18[5], f18[6], f18[7], f18[8]};
     float fhi[8] = {f18[9], f18[10], f18[11], f18[12], f18[13], f18[15], f18[16], f18[17]};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      flo[i] *= fsc[i];
+      fhi[i] *= fsc[8 + i];
+    }
     // B operands of the first layer: after the swap flo serves group 0 (lanes 0..31: their own inputs 0..7,
     // lanes 32..63: inputs 8..15 of the element 32 lanes below), fhi group 1
 #pragma unroll
@@ -653,9 +665,9 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
       flo[i] = __uint_as_float(u);
       fhi[i] = __uint_as_float(v);
     }
-    au32x4 xb[2][3];
-    bf3_pack8(flo, xb[0]);
-    bf3_pack8(fhi, xb[1]);
+    au32x4 xb[2][2];
+    hf2_pack8(flo, xb[0]);
+    hf2_pack8(fhi, xb[1]);
     // The two groups of 32 elements go through the layers a phase apart, so that the matrix instructions of one
     // have the vector work of the other to run under: first layer of both, then per group split -> hidden layer,
     // then the output layer (on the vector pipe) of both.
@@ -669,31 +681,28 @@ __device__ __forceinline__ void adafac_apply_tile_bf(const TDesc& d, const PyloT
 #pragma unroll
         for (int i = 0; i < 4; ++i) h[gq][4 * j + i] = ta[PER ? gq : 0][j][i] + tb[i];
       }
-      h[gq] = bf3_mfma(w1, xb[gq], h[gq]);
+      h[gq] = hf2_mfma(w1, xb[gq], h[gq]);
     }
     av16f g2[2];
 #pragma unroll
     for (int gq = 0; gq < 2; ++gq) {
       // hidden values of the units this lane holds -> planes, four units (two dwords) per block j
-      unsigned hp[3][4][2];
+      unsigned hp[2][4][2];
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          const Bf3 u0 = bf3_split(relu(h[gq][4 * j + 2 * i])), u1 = bf3_split(relu(h[gq][4 * j + 2 * i + 1]));
-          hp[0][j][i] = bf_pack(u0.h, u1.h);
-          hp[1][j][i] = bf_pack(u0.m, u1.m);
-          hp[2][j][i] = bf_pack(u0.l, u1.l);
-        }
+        for (int i = 0; i < 2; ++i)
+          hf2_split2(__builtin_amdgcn_fmed3f(h[gq][4 * j + 2 * i], 0.0f, 65000.0f),
+                     __builtin_amdgcn_fmed3f(h[gq][4 * j + 2 * i + 1], 0.0f, 65000.0f), hp[0][j][i], hp[1][j][i]);
       // blocks 2 s and 2 s + 1 are the lane's eight slots of reduction step s as they stand
       g2[gq] = bh;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
-        au32x4 hb[3];
+        au32x4 hb[2];
 #pragma unroll
-        for (int q = 0; q < 3; ++q)
+        for (int q = 0; q < 2; ++q)
           hb[q] = au32x4{hp[q][2 * s2][0], hp[q][2 * s2][1], hp[q][2 * s2 + 1][0], hp[q][2 * s2 + 1][1]};
-        g2[gq] = bf3_mfma(w2[s2], hb, g2[gq]);
+        g2[gq] = hf2_mfma(w2[s2], hb, g2[gq]);
       }
     }
     float part[2][2];
@@ -749,7 +758,7 @@ __global__ __launch_bounds__(kThreads) void k_adafac_apply(const TDesc* __restri
 }
 
 // The apply pass for tensors walked column-resident (items hold four wave tasks each).  BF: the element MLP on
-// the bf16 matrix instructions (three-plane operands), else on the fp32 ones.
+// the fp16 matrix instructions (two-plane operands), else on the fp32 ones.
 template <bool BF, bool PER = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(BF ? 2 : PYLO_ADAFAC_WAVES)))
 void k_adafac_apply_tile(const TDesc* __restrict__ descs, const PyloTensorArgs* __restrict__ dyn,
@@ -765,9 +774,9 @@ void k_adafac_apply_tile(const TDesc* __restrict__ descs, const PyloTensorArgs* 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int task = it.a * 4 + wave;
   if (task >= d.atile_ntask) return;
-  static_assert(BF || !PER, "tensors with more than two dims are walked by the bf16 variant only");
+  static_assert(BF || !PER, "tensors with more than two dims are walked by the fp16 variant only");
   if constexpr (BF)
-    adafac_apply_tile_bf<PER>(d, a, task, make_ema(dec), fac_tab, term_tab, wfold + (size_t)it.tensor * kAFold, net);
+    adafac_apply_tile_hf<PER>(d, a, task, make_ema(dec), fac_tab, term_tab, wfold + (size_t)it.tensor * kAFold, net);
   else
     adafac_apply_tile(d, a, task, make_ema(dec), fac_tab, term_tab, wfold + (size_t)it.tensor * kAFold, net, xch[wave]);
 }

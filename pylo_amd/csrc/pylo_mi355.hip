@@ -158,9 +158,9 @@ bool env_matrix_pipe() {
   return !(v && v[0] == '1');
 }
 
-// AdafacLO's element MLP on the bf16 matrix instructions (three-plane operands); PYLO_MI355_ADAFAC_F32=1 keeps
+// AdafacLO's element MLP on the fp16 matrix instructions (two-plane operands); PYLO_MI355_ADAFAC_F32=1 keeps
 // the fp32 matrix instructions.
-bool env_adafac_bf() {
+bool env_adafac_hf() {
   const char* v = std::getenv("PYLO_MI355_ADAFAC_F32");
   return !(v && v[0] == '1');
 }
@@ -932,7 +932,7 @@ int build_layout(int kind, const PyloTensorShape* shapes, int T, Layout& L, int 
       // an (O, I, k, ..) tensor factored over its two leading dims (convolution kernels) is the matrix (O, I * P)
       // for this pass, P = product of the trailing dims (pp_items)
       bool periodic = false;
-      if (d.mode == kModeFacND && n > 0 && env_matrix_pipe() && env_adafac_bf() && e.ndim >= 3 &&
+      if (d.mode == kModeFacND && n > 0 && env_matrix_pipe() && env_adafac_hf() && e.ndim >= 3 &&
           ((edr == 0 && edc == 1) || (edr == 1 && edc == 0))) {
         long long P = 1;
         for (int i = 2; i < e.ndim; ++i) P *= e.shape[i];
@@ -1070,7 +1070,7 @@ struct PyloPlan {
   size_t last_dst = 0;   // where `last` was copied to
   bool have_last = false;
   bool mlp_on_matrix_pipe = true;  // env_matrix_pipe() when the plan was created
-  bool adafac_bf = true;           // AdafacLO's element MLP on the bf16 matrix instructions (PYLO_MI355_ADAFAC_F32=1: fp32 ones)
+  bool adafac_hf = true;           // AdafacLO's element MLP on the fp16 matrix instructions (PYLO_MI355_ADAFAC_F32=1: fp32 ones)
   // optional per-launch timing (pylo_mi355_plan_timing_begin/end)
   std::vector<hipEvent_t> tev;
   int t_steps_max = 0, t_steps = 0, t_per_step = 0;
@@ -1115,7 +1115,7 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
   P->kind = kind;
   P->T = n_tensors;
   P->mlp_on_matrix_pipe = env_matrix_pipe();
-  P->adafac_bf = env_adafac_bf();
+  P->adafac_hf = env_adafac_hf();
   if (int rc = build_layout(kind, shapes, n_tensors, P->L, kVeloHiddenMax)) { delete P; return rc; }
   if (workspace == nullptr || workspace_bytes < P->L.total) { delete P; return fail("plan_create: workspace too small"); }
   if (reinterpret_cast<uintptr_t>(workspace) % 256 != 0) { delete P; return fail("plan_create: workspace must be 256-byte aligned"); }
@@ -2191,7 +2191,7 @@ extern "C" int pylo_mi355_adafac_step(PyloPlan* P, const PyloTensorArgs* args, c
     hipLaunchKernelGGL((k_adafac_apply_tile<true, true>), dim3(n_pp), dim3(kThreads), 0, s, descs, dyn, pp_items, fac_tab,
                        term_tab, dec, wfold, net, gl);
   if (n_ap > 0) {
-    if (P->adafac_bf)
+    if (P->adafac_hf)
       hipLaunchKernelGGL(k_adafac_apply_tile<true>, dim3(n_ap), dim3(kThreads), 0, s, descs, dyn, ap_items, fac_tab,
                          term_tab, dec, wfold, net, gl);
     else

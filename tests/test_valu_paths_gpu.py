@@ -75,8 +75,8 @@ def test_velo_valu(monkeypatch):
 
 @pytest.mark.parametrize("switch", ["PYLO_MI355_VALU_MLP", "PYLO_MI355_ADAFAC_F32"])
 def test_adafac_valu(monkeypatch, switch):
-    """AdafacLO's element MLP runs on the bf16 matrix instructions by default (operands split into three
-    bf16 planes, six products per fp32 product); PYLO_MI355_ADAFAC_F32=1 keeps it on the fp32 matrix
+    """AdafacLO's element MLP runs on the fp16 matrix instructions by default (operands split into two
+    fp16 planes, three products per fp32 product); PYLO_MI355_ADAFAC_F32=1 keeps it on the fp32 matrix
     instructions, PYLO_MI355_VALU_MLP=1 on the vector pipe."""
     from oracle import pylo_oracle as O
     from pylo_amd import AdafacLO_CUDA
@@ -102,7 +102,7 @@ def test_adafac_valu(monkeypatch, switch):
 
 
 def test_adafac_matrix_pipes_against_fp64(monkeypatch):
-    """The split-bf16 MLP gives up no accuracy: the parameter steps of both matrix-pipe variants against the
+    """The split-fp16 MLP gives up no accuracy: the parameter steps of both matrix-pipe variants against the
     oracle evaluated in fp64, relative to the error the fp32 oracle itself makes (both stay below it)."""
     from oracle import pylo_oracle as O
     from pylo_amd import AdafacLO_CUDA

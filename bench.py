@@ -211,7 +211,12 @@ def whole_step_object(whole_ms, finish_ms, n_params, flops, flops_exec):
                      "achieved": mult * flops_exec / t / 1e12, "peak": peak, "unit": "TFLOP/s",
                      "frac": mult * flops_exec / t / 1e12 / peak,
                      "fp32_equivalent_TFLOPs": flops_exec / t / 1e12,
-                     "nominal_fp32_TFLOPs": flops / t / 1e12, "traffic": None},
+                     "nominal_fp32_TFLOPs": flops / t / 1e12,
+                     # the same fp32 products in the work units of the three-plane bf16 scheme these kernels ran
+                     # on before (six 16-bit products per fp32 product): comparable with earlier lines, not a
+                     # rate the pipe executes
+                     "frac_in_six_product_units": None if f32 else 6.0 * flops_exec / t / 1e12 / peak,
+                     "traffic": None},
     }
 
 

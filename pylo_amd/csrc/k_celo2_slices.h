@@ -262,6 +262,48 @@ __global__ __launch_bounds__(64) void k_celo2_slices_lane(const TDesc* __restric
   const float inv_s = 1.0f / (float)S;
   float wreg[6];
   slice_mlp_weights(mlp, wreg);
+  if (S == 1) {
+    // A slice is an element (1 x 1 kernels): nothing to stage, every lane takes its own element, and the next
+    // group's loads are in flight under this group's arithmetic.  Lanes past the end work on the block's first element
+    // and store nothing.
+    struct In { float g, p, m[3], r; SliceFac fac; };
+    auto fetch = [&](long long idx) {
+      In x;
+      x.g = *(const gfloat*)(a.grad + idx);
+      x.p = *(const gfloat*)(a.param + idx);
+      x.m[0] = *(const gfloat*)(a.mom + idx);
+      x.m[1] = *(const gfloat*)(a.mom + n + idx);
+      x.m[2] = *(const gfloat*)(a.mom + 2 * n + idx);
+      x.r = *(const gfloat*)(a.rms + idx);
+      x.fac = slice_gather_nd(d, a, idx, fac_tab);
+      return x;
+    };
+    const long long b0 = it.a;
+    In cur = fetch(b0 + lane < n ? b0 + lane : b0);
+    for (int grp = 0; grp < slice_lane_groups(1); ++grp) {
+      const long long idx = b0 + 64 * grp + lane;
+      if (b0 + 64 * grp >= n) break;
+      const bool mine = idx < n;
+      const long long nidx = idx + 64;
+      const In nxt = fetch(grp + 1 < slice_lane_groups(1) && nidx < n ? nidx : b0);
+      const float g = cond_grad(cur.g, d.gscale, a.clip_val, d.nan0);
+      float m[3] = {cur.m[0], cur.m[1], cur.m[2]}, rms = cur.r, f[30], sc[30];
+      ema_update(e, g, m, rms);
+      slice_features_nd(cur.fac, g, cur.p, m, rms, f);
+#pragma unroll
+      for (int c = 0; c < 30; ++c) sc[c] = rsq(1e-9f + f[c] * f[c]);
+      const float step = slice_mlp_mfma(f, sc, wreg, a.exp_mult);
+      if (mine) {
+        *(gfloat*)(a.mom + idx) = m[0];
+        *(gfloat*)(a.mom + n + idx) = m[1];
+        *(gfloat*)(a.mom + 2 * n + idx) = m[2];
+        *(gfloat*)(a.rms + idx) = rms;
+        *(gfloat*)(a.step_out + idx) = step;
+      }
+      cur = nxt;
+    }
+    return;
+  }
   for (int grp = 0; grp < slice_lane_groups(S); ++grp) {
     const long long s0 = (long long)it.a + 64 * grp, left = n_slices - s0;
     if (left <= 0) break;

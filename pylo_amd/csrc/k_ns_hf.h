@@ -7,8 +7,12 @@
 // A product of two such numbers is four fp16 products; the smallest (l l, 2^-22 |x y|) is dropped with the
 // remainders.  The other three are exact in fp32 and are accumulated in fp32 by v_mfma_f32_32x32x16_f16, which does
 // sixteen times the multiply-adds of v_mfma_f32_32x32x2_f32 per instruction slot: three of them replace eight fp32
-// instructions' worth of work.  A product of the iteration is then off by about 6e-8 of its entries' RMS, a quarter
-// of what the fp32 accumulation of a reduction over 256 .. 4096 terms adds anyway (a plain fp32 GEMM: 2.5e-7).
+// instructions' worth of work.  An operand carries 23 significant bits where fp32 has 24: a product of the iteration
+// is off by about 6e-8 of its entries' RMS, a quarter of what the fp32 accumulation of a reduction over 256 .. 4096
+// terms adds anyway (a plain fp32 GEMM: 2.5e-7), but each entry of the result carries 1 .. 3e-7 of its own size where
+// an fp32 product carries 6e-8.  With the reference's coefficients, which multiply rounding by up to 3.44 an
+// iteration, the result is as far from the fp64 formula as the fp32 torch products are (0.4 .. 0.9 times, tests); with
+// polynomials that do not amplify (1.5 x - 0.5 x^3, 2 x - x^3) it is 3 .. 12 times further, 1e-5 of its RMS at most.
 // The scales: no entry of a matrix exceeds its largest singular value, and the singular values of everything the
 // iteration forms follow from the coefficients alone once X0 has unit Frobenius norm (the host walks a grid of
 // starting values through sigma -> sigma p(sigma^2), ns_plane_exps): X and A = X X^T stay below 1.5, B' = p(A)

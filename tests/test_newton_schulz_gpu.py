@@ -106,7 +106,7 @@ def test_iteration_counts_and_result_buffer(iters, pipe, monkeypatch):
     _run([(256, 384), (384, 256), (132, 260)], steps=2, ns_iters=iters)
 
 
-def _orthogonalise_direct(mats, iters=5):
+def _orthogonalise_direct(mats, iters=5, coeffs=(3.4445, -4.775, 2.0315)):
     """rms_normalize(newton_schulz(x)) of every matrix through the finishing call alone: p = 0, lr = -1."""
     import numpy as np
 
@@ -121,16 +121,16 @@ def _orthogonalise_direct(mats, iters=5):
         fin["grad"][i], fin["param"][i], fin["step_out"][i] = 1, params[i].data_ptr(), steps[i].data_ptr()
         fin["lr"][i], fin["weight_decay"][i], fin["step_mult"][i] = -1.0, 0.0, 1.0
         fin["flags"][i] = _lib.ARG_ORTHOGONALIZE
-    plan.celo2_orthogonalize_finish(fin, (3.4445, -4.775, 2.0315), iters, 1e-8, torch.cuda.current_stream().cuda_stream)
+    plan.celo2_orthogonalize_finish(fin, coeffs, iters, 1e-8, torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     plan.close()
     return params
 
 
-def _reference_direct(x, iters=5, dtype=torch.float64):
+def _reference_direct(x, iters=5, dtype=torch.float64, coeffs=(3.4445, -4.775, 2.0315)):
     """The literal formula (pylo/optim/CELO2_naive.py:59-73) and the RMS normaliser, in fp64 or, as the reference
     runs it, in fp32 torch products."""
-    c0, c1, c2 = 3.4445, -4.775, 2.0315
+    c0, c1, c2 = coeffs
     x = x.to(dtype)
     t = x.shape[0] > x.shape[1]
     if t:
@@ -182,6 +182,38 @@ def test_spectra_with_a_dominant_direction(chains, floor, monkeypatch):
     finally:
         torch.backends.cuda.matmul.allow_tf32 = prev
     print("chains", pairs, "(shape, library error / rms, fp32 torch formula error / rms):", rows)
+
+
+@pytest.mark.parametrize("coeffs,iters", [((1.5, -0.5, 0.0), 8), ((1.875, -1.25, 0.375), 6), ((3.0, -3.2, 1.2), 5),
+                                          ((3.4445, -4.775, 2.0315), 9), ((2.0, -1.0, 0.0), 3), ((0.5, 0.0, 0.0), 4)])
+def test_other_coefficients_and_iteration_counts(coeffs, iters):
+    """The operand planes are fp16 numbers scaled by powers of two that the library derives from the coefficients
+    (bounds on the singular values of everything the iteration forms): other polynomials than the reference's
+    default -- the cubic and quintic Newton-Schulz iterations, one that overshoots (sigma up to 1.09 for 2 - x),
+    one that only shrinks -- and other iteration counts must come out as close to the fp64 formula as the
+    reference's fp32 torch products do (1.5 times their error plus the level of well-conditioned inputs).  Where
+    the polynomial does not amplify rounding the library's 23-bit operands show: 3 .. 12 times the fp32 formula's
+    error, 1e-5 of the result's RMS at most."""
+    gen = torch.Generator(device="cuda").manual_seed(17)
+    rnd = lambda *s: torch.randn(*s, generator=gen, device="cuda")
+    u, v = rnd(300, 1), rnd(1, 520)
+    mats = [rnd(256, 384), rnd(384, 256), rnd(130, 1000), rnd(768, 768), rnd(1, 700), rnd(64, 64),
+            u @ v / (u.norm() * v.norm()) + 0.05 * rnd(300, 520) / (300 * 520) ** 0.5]
+    got = _orthogonalise_direct(mats, iters=iters, coeffs=coeffs)
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    rows = []
+    try:
+        for x, y in zip(mats, got):
+            want = _reference_direct(x, iters=iters, coeffs=coeffs)
+            assert torch.isfinite(y).all(), tuple(x.shape)
+            e = float((y.double() - want).abs().max())
+            e32 = float((_reference_direct(x, iters=iters, dtype=torch.float32, coeffs=coeffs).double() - want).abs().max())
+            rows.append((tuple(x.shape), e, e32))
+            assert e <= 1.5 * e32 + 5e-5, rows[-1]
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+    print("coefficients", coeffs, "iterations", iters, "(shape, library error / rms, fp32 torch formula error / rms):", rows)
 
 
 def test_chain_length_chosen_per_matrix(monkeypatch):

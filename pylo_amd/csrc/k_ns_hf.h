@@ -111,7 +111,8 @@ struct NsBufs { int s1, s2, d; float acc_scale, out_scale; };
 // x (already times its plane scale) = h + l + what is left below 2^-22 |x|.  The clamp never acts on a matrix
 // within the bounds the scales were chosen for; it keeps a stray value from becoming an infinity.
 __device__ __forceinline__ void hf_split(float x, hbits& h, hbits& l) {
-  x = __builtin_amdgcn_fmed3f(x, -65000.0f, 65000.0f);
+  const float c = __builtin_amdgcn_fmed3f(x, -65000.0f, 65000.0f);
+  x = x == x ? c : x;   // (the median of three takes a NaN for the smallest: keep it a NaN)
   const _Float16 hb = (_Float16)x;
   const _Float16 lb = (_Float16)(x - (float)hb);
   h = __builtin_bit_cast(hbits, hb);

@@ -216,6 +216,20 @@ def test_other_coefficients_and_iteration_counts(coeffs, iters):
     print("coefficients", coeffs, "iterations", iters, "(shape, library error / rms, fp32 torch formula error / rms):", rows)
 
 
+def test_a_nan_stays_a_nan_and_stays_in_its_matrix():
+    """A NaN in one raw step makes that matrix's result NaN, as the formula does (its norm is NaN), instead of being
+    clamped into the fp16 planes' range as a finite number; the other matrices of the call are what they are
+    without it."""
+    gen = torch.Generator(device="cuda").manual_seed(23)
+    mats = [torch.randn(s, generator=gen, device="cuda") for s in ((256, 384), (130, 260), (384, 128))]
+    clean = _orthogonalise_direct(mats)
+    mats[1][3, 5] = float("nan")
+    got = _orthogonalise_direct(mats)
+    assert torch.isnan(got[1]).all()
+    assert torch.equal(got[0], clean[0]) and torch.equal(got[2], clean[2])
+    assert torch.isfinite(clean[1]).all()
+
+
 def test_chain_length_chosen_per_matrix(monkeypatch):
     """PYLO_MI355_NS_ADAPTIVE=1: the first chain takes three iterations for the matrices whose A = X X^T has
     ||A||_F^2 <= (16 / 196)^2 (no direction holds more than 8 % of the step's squared norm: what three chained

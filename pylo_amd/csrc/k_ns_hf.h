@@ -130,43 +130,44 @@ __device__ __forceinline__ void hf_split(float x, hbits& h, hbits& l) {
 #define PYLO_LDS __attribute__((address_space(3)))
 #define PYLO_GLB __attribute__((address_space(1)))
 
-template <int ROWS>
-__device__ __forceinline__ void hf_stage_offsets(int wave, int lane, int (&off)[ROWS * kNsRowPc / 256]) {
+// (NW: waves of the block)
+template <int ROWS, int NW = 4>
+__device__ __forceinline__ void hf_stage_offsets(int wave, int lane, int (&off)[ROWS * kNsRowPc / (64 * NW)]) {
 #pragma unroll
-  for (int j = 0; j < ROWS * kNsRowPc / 256; ++j) {
-    const int p = (j * 4 + wave) * 64 + lane;
+  for (int j = 0; j < ROWS * kNsRowPc / (64 * NW); ++j) {
+    const int p = (j * NW + wave) * 64 + lane;
     off[j] = (p ^ ((p >> 4) & 3)) * 16;   // row p / 4: its four pieces permuted by (row / 4) % 4
   }
 }
 
-template <int ROWS>
-__device__ __forceinline__ void hf_stage_issue(const char* g, const int (&off)[ROWS * kNsRowPc / 256], PYLO_LDS char* lds, int wave) {
+template <int ROWS, int NW = 4>
+__device__ __forceinline__ void hf_stage_issue(const char* g, const int (&off)[ROWS * kNsRowPc / (64 * NW)], PYLO_LDS char* lds, int wave) {
 #pragma unroll
-  for (int j = 0; j < ROWS * kNsRowPc / 256; ++j)
-    __builtin_amdgcn_global_load_lds((const PYLO_GLB void*)(g + off[j]), (PYLO_LDS void*)(lds + (j * 4 + wave) * 1024), 16, 0, 0);
+  for (int j = 0; j < ROWS * kNsRowPc / (64 * NW); ++j)
+    __builtin_amdgcn_global_load_lds((const PYLO_GLB void*)(g + off[j]), (PYLO_LDS void*)(lds + (j * NW + wave) * 1024), 16, 0, 0);
 }
 
 // acc[hi][hj] += (rows i0.. of P1) x (rows j0.. of P2)^T over the reduction range [k0, k1) (multiples of 16);
 // 128 rows of P1, 64 WN rows of P2.  LDS: two stages of (128 + 64 WN) x 64 bytes.
 // `compute` (the same for all lanes of a wave): false for a wave whose values nobody needs -- it stages and meets the
 // barriers, and leaves the matrix pipe to the other waves of its SIMD.
-template <int WN>
+template <int WN, int NW = 4>
 __device__ __forceinline__ void hf_tile_product(const HfPlanes& P1, int i0, const HfPlanes& P2, int j0, int k0, int k1,
                                                 PYLO_LDS char* lds, v16f (&acc)[2][WN], bool compute = true) {
-  constexpr int RB = 64 * WN, SA = 128 * kNsRowB, STAGE = SA + RB * kNsRowB;
+  constexpr int RA = 32 * NW, RB = 64 * WN, SA = RA * kNsRowB, STAGE = SA + RB * kNsRowB;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wi = (wave >> 1) * 64, wj = (wave & 1) * 32 * WN;
   const int kg = lane >> 5, lo = lane & 31;
-  int offa[128 * kNsRowPc / 256], offb[RB * kNsRowPc / 256];
-  hf_stage_offsets<128>(wave, lane, offa);
-  hf_stage_offsets<RB>(wave, lane, offb);
+  int offa[RA * kNsRowPc / (64 * NW)], offb[RB * kNsRowPc / (64 * NW)];
+  hf_stage_offsets<RA, NW>(wave, lane, offa);
+  hf_stage_offsets<RB, NW>(wave, lane, offb);
   const char* ga = (const char*)P1.base + ((size_t)(k0 >> 4) * P1.rows + i0) * kNsRowB;
   const char* gb = (const char*)P2.base + ((size_t)(k0 >> 4) * P2.rows + j0) * kNsRowB;
   const size_t sa = (size_t)P1.rows * kNsRowB, sb = (size_t)P2.rows * kNsRowB;
   // a diagonal tile of X X^T or A A: both operands are the same 128 rows, staged once
   const bool same = WN == 2 && P1.base == P2.base && i0 == j0;
-  hf_stage_issue<128>(ga, offa, lds, wave);
-  if (!same) hf_stage_issue<RB>(gb, offb, lds + SA, wave);
+  hf_stage_issue<RA, NW>(ga, offa, lds, wave);
+  if (!same) hf_stage_issue<RB, NW>(gb, offb, lds + SA, wave);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   // the lane's rows are lo, lo + 32, ..: all with the same (row / 4) % 4; plane q, half kg is piece 2 q + kg
@@ -177,8 +178,8 @@ __device__ __forceinline__ void hf_tile_product(const HfPlanes& P1, int i0, cons
     if (k + kHfBK < k1) {
       ga += sa;
       gb += sb;
-      hf_stage_issue<128>(ga, offa, lds + (STAGE - cur), wave);
-      if (!same) hf_stage_issue<RB>(gb, offb, lds + (STAGE - cur) + SA, wave);
+      hf_stage_issue<RA, NW>(ga, offa, lds + (STAGE - cur), wave);
+      if (!same) hf_stage_issue<RB, NW>(gb, offb, lds + (STAGE - cur) + SA, wave);
     }
     if (compute) {
       f16x8 a[2][kNsPl], b[WN][kNsPl];

@@ -2589,6 +2589,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
   out[(size_t)blockIdx.x * 256 + threadIdx.x] = sum;
 }
 
+// MODE 3: the same loop with tiles of 256 x 256 outputs by 512 threads (4 x 2 waves of 64 x 128): two thirds of the
+// bytes staged per product.
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k_matrix_probe_wide(
+    const hbits* __restrict__ X, int rows_x, const hbits* __restrict__ B, int rows_b, int K, float* __restrict__ out) {
+  extern __shared__ __attribute__((aligned(16))) char lds_[];
+  PYLO_LDS char* lds = (PYLO_LDS char*)lds_;
+  constexpr int WN = 4;
+  const int nj = rows_b / 256, i0 = (blockIdx.x / nj) * 256, j0 = (blockIdx.x % nj) * 256;
+  v16f acc[2][WN];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  const HfPlanes PX{X, rows_x}, PB{B, rows_b};
+  hf_tile_product<WN, 8>(PX, i0, PB, j0, 0, K, lds, acc);
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sum += acc[i][j][r];
+  out[(size_t)blockIdx.x * 512 + threadIdx.x] = sum;
+}
+
 }  // namespace
 
 extern "C" int pylo_mi355_matrix_probe(const void* x_planes, int rows_x, const void* b_planes, int rows_b, int k_steps,
@@ -2596,7 +2623,8 @@ extern "C" int pylo_mi355_matrix_probe(const void* x_planes, int rows_x, const v
   if (!x_planes || !b_planes || !out) return fail("matrix_probe: null pointer");
   if (rows_x <= 0 || rows_x % 128 != 0 || rows_b <= 0 || rows_b % 256 != 0 || k_steps <= 0 || k_steps % 16 != 0)
     return fail("matrix_probe: rows_x must be a multiple of 128, rows_b of 256, k_steps of 16");
-  if (mode < 0 || mode > 2) return fail("matrix_probe: mode must be 0, 1 or 2");
+  if (mode < 0 || mode > 3) return fail("matrix_probe: mode must be 0 .. 3");
+  if (mode == 3 && rows_x % 256 != 0) return fail("matrix_probe: mode 3 takes rows_x in multiples of 256");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const unsigned grid = (unsigned)(rows_x / 128) * (unsigned)(rows_b / 256);
   static std::mutex mu;
@@ -2605,12 +2633,14 @@ extern "C" int pylo_mi355_matrix_probe(const void* x_planes, int rows_x, const v
     HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<0>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(4)));
     HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<1>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(4)));
     HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<2>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(4)));
+    HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe_wide, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 512 * kNsRowB));
   }
   const hbits* X = static_cast<const hbits*>(x_planes);
   const hbits* B = static_cast<const hbits*>(b_planes);
   if (mode == 0) hipLaunchKernelGGL(k_matrix_probe<0>, dim3(grid), dim3(256), hf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
   else if (mode == 1) hipLaunchKernelGGL(k_matrix_probe<1>, dim3(grid), dim3(256), hf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
-  else hipLaunchKernelGGL(k_matrix_probe<2>, dim3(grid), dim3(256), hf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
+  else if (mode == 2) hipLaunchKernelGGL(k_matrix_probe<2>, dim3(grid), dim3(256), hf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
+  else hipLaunchKernelGGL(k_matrix_probe_wide, dim3(grid / 2), dim3(512), 2 * 512 * kNsRowB, s, X, rows_x, B, rows_b, k_steps, out);
   HIP_TRY(hipGetLastError());
   return 0;
 }

@@ -149,6 +149,42 @@ def test_fp32_matrix_instructions_leave_large_slices_to_the_caller(monkeypatch):
     test_whole_steps_against_the_oracle(dict(), True, False)
 
 
+def test_short_slices_of_every_length_class_against_the_oracle():
+    """The feature pass of short slices (one lane per slice, staged through LDS in blocks of several groups of 64
+    slices; slices of one element straight from memory) over every class of slice length, with slice counts that
+    leave the last group and the last block ragged: accumulators, raw steps and parameters through whole
+    free-running steps against the fp64 oracle."""
+    from oracle import pylo_oracle as O
+    from pylo_amd import ELO_CELO2_CUDA
+    from pylo_amd.models import CELO2MLP
+
+    torch.manual_seed(2)
+    net = CELO2MLP()
+    # slices x length: 1480 x 1, 63 x 1, 577 x 2, 450 x 4, 300 x 6, 200 x 9, 273 x 16, 77 x 25, 70 x 32
+    shapes = [(40, 37, 1, 1), (9, 7, 1, 1), (577, 1, 2), (9, 50, 2, 2), (20, 15, 2, 3), (8, 25, 3, 3), (21, 13, 4, 4),
+              (7, 11, 5, 5), (10, 7, 4, 8), (48, 64)]
+    gen = torch.Generator(device="cuda").manual_seed(31)
+    init = [torch.randn(s, generator=gen, device="cuda") * 0.05 for s in shapes]
+    ref = [v.double() for v in init]
+    gpu = [torch.nn.Parameter(v.clone()) for v in init]
+    cfg = dict(lr=1e-3, weight_decay=0.1, adam_lr_mult=20.0)
+    orc = O.EloCelo2Oracle(ref, net.state_dict(), device="cuda", **cfg).double_()
+    opt = ELO_CELO2_CUDA(gpu, network=net, hf_key=None, **cfg)
+    for t in range(3):
+        grads = [torch.randn(s, generator=gen, device="cuda") * 10.0 ** (-1 - i % 3) for i, s in enumerate(shapes)]
+        for p, g in zip(gpu, grads):
+            p.grad = g
+        orc.step([g.double() for g in grads])
+        opt.step()
+        torch.cuda.synchronize()
+        for i, p in enumerate(gpu):
+            assert max_err(p, ref[i], 1e-5, 1e-6) <= 1.0, (t, i, shapes[i])
+            st = opt.state[p]
+            for key in ("mom", "rms"):
+                if key in st and key in orc.state[i]:
+                    assert max_err(st[key], orc.state[i][key], 1e-5, 1e-6) <= 1.0, (t, i, shapes[i], key)
+
+
 @pytest.mark.parametrize("kw,with_large_slices,cached_table", [
     (dict(), False, True), (dict(), True, True), (dict(ns_iters=0), True, False),
     (dict(orthogonalize=False), True, True), (dict(param_scale_mult=True), False, False)])

@@ -459,7 +459,8 @@ def matrix_ceiling(a):
         b = planes(rows_b * k * 2)
         out = torch.zeros((rows_x // 128) * (rows_b // 256) * 256, device=dev)
         for mode, name in ((0, "product loop"), (1, "LDS reads + matrix instructions"), (2, "matrix instructions only"),
-                           (3, "product loop, 256 x 256 tiles by 512 threads")):
+                           (3, "product loop, 256 x 256 tiles by 512 threads"),
+                           (4, "product loop, first operand straight into registers")):
             call = lambda: _lib.check(lib.pylo_mi355_matrix_probe(x.data_ptr(), rows_x, b.data_ptr(), rows_b, k, mode,
                                                                   out.data_ptr(), stream), "matrix_probe")
             for _ in range(max(a.warmup, 3)):

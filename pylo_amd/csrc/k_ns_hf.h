@@ -54,6 +54,8 @@
 // where the tensor's rows are not 16-byte aligned).
 #pragma once
 
+#include <type_traits>
+
 #include "k_ns.h"
 
 namespace pylo {
@@ -208,6 +210,87 @@ __device__ __forceinline__ void hf_tile_product(const HfPlanes& P1, int i0, cons
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     cur = STAGE - cur;
+  }
+}
+
+// The same product with the first operand's fragments loaded straight from memory into registers, two steps ahead (a
+// lane's fragment of a row is 16 consecutive bytes of the planes): only the second operand goes through LDS, 48 KB
+// of LDS traffic a step and block instead of 73.  128 rows of P1 (by 256 threads), 64 WN rows of P2; LDS: two
+// stages of 64 WN x 64 bytes.  Benchmark instrumentation only (pylo_mi355_matrix_probe, mode 4): the bare loop is
+// 8 - 12 % faster this way on one large operand, the update product inside whole steps (four groups of matrices on
+// four streams) 2.5 % slower.
+template <int WN>
+__device__ __forceinline__ void hf_tile_product_direct(const HfPlanes& P1, int i0, const HfPlanes& P2, int j0, int k0, int k1,
+                                                       PYLO_LDS char* lds, v16f (&acc)[2][WN]) {
+  constexpr int RB = 64 * WN, STAGE = RB * kNsRowB;
+  typedef PYLO_GLB u32x4 gu32x4;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wi = (wave >> 1) * 64, wj = (wave & 1) * 32 * WN;
+  const int kg = lane >> 5, lo = lane & 31;
+  int offb[RB * kNsRowPc / 256];
+  hf_stage_offsets<RB>(wave, lane, offb);
+  const char* ga = (const char*)P1.base + ((size_t)(k0 >> 4) * P1.rows + i0 + wi + lo) * kNsRowB + 16 * kg;
+  const char* gb = (const char*)P2.base + ((size_t)(k0 >> 4) * P2.rows + j0) * kNsRowB;
+  const size_t sa = (size_t)P1.rows * kNsRowB, sb = (size_t)P2.rows * kNsRowB;
+  u32x4 an[2][2][kNsPl];   // the fragments of this step and the next (slot = step % 2), refilled for two steps on
+  auto fetch_a = [&](auto slot, const char* g) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int q = 0; q < kNsPl; ++q) an[slot.value][i][q] = *(const gu32x4*)(g + i * 32 * kNsRowB + q * 32);
+  };
+  typedef std::integral_constant<int, 0> S0;
+  typedef std::integral_constant<int, 1> S1;
+  hf_stage_issue<RB>(gb, offb, lds, wave);
+  fetch_a(S0(), ga);
+  if (k0 + kHfBK < k1) fetch_a(S1(), ga + sa);
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  const int ob = (wj + lo) * kNsRowB + 16 * (kg ^ ((lo >> 2) & 3));
+  int cur = 0;
+  ga += sa;
+  auto step = [&](auto slot, int k) {
+    f16x8 a[2][kNsPl], b[WN][kNsPl];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int q = 0; q < kNsPl; ++q) a[i][q] = __builtin_bit_cast(f16x8, an[slot.value][i][q]);
+    const bool more_b = k + kHfBK < k1, more_a = k + 2 * kHfBK < k1;
+    if (more_b) {
+      gb += sb;
+      hf_stage_issue<RB>(gb, offb, lds + (STAGE - cur), wave);
+    }
+    if (more_a) {
+      ga += sa;
+      fetch_a(slot, ga);
+    }
+#pragma unroll
+    for (int q = 0; q < kNsPl; ++q)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+        b[j][q] = __builtin_bit_cast(f16x8, *(const luint4*)(lds + cur + ((ob + j * 32 * kNsRowB) ^ (q * 32))));
+#pragma unroll
+    for (int term = 0; term < 3; ++term) {
+      constexpr int pa[3] = {1, 0, 0}, pb[3] = {0, 1, 0};
+#pragma unroll
+      for (int hi = 0; hi < 2; ++hi)
+#pragma unroll
+        for (int hj = 0; hj < WN; ++hj)
+          acc[hi][hj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[hi][pa[term]], b[hj][pb[term]], acc[hi][hj], 0, 0, 0);
+    }
+    // the second operand's next stage has landed and every wave has read this one; the fragments just asked for
+    // (the newest loads: loads complete in order) may still be on their way.  The bare barrier: a __syncthreads()
+    // would wait for them too.
+    if (more_a) __builtin_amdgcn_s_waitcnt((2 * kNsPl) | (7 << 4));   // vmcnt <= 4, lgkmcnt 0
+    else __builtin_amdgcn_s_waitcnt(7 << 4);                            // vmcnt 0, lgkmcnt 0
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    cur = STAGE - cur;
+  };
+  for (int k = k0; k < k1; k += 2 * kHfBK) {
+    step(S0(), k);
+    if (k + kHfBK < k1) step(S1(), k + kHfBK);
   }
 }
 

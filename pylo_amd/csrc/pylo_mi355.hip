@@ -2543,6 +2543,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
   const HfPlanes PX{X, rows_x}, PB{B, rows_b};
   if (MODE == 0) {
     hf_tile_product<WN>(PX, i0, PB, j0, 0, K, lds, acc);
+  } else if (MODE == 4) {
+    hf_tile_product_direct<WN>(PX, i0, PB, j0, 0, K, lds, acc);
   } else {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wi = (wave >> 1) * 64, wj = (wave & 1) * 32 * WN;
@@ -2623,7 +2625,7 @@ extern "C" int pylo_mi355_matrix_probe(const void* x_planes, int rows_x, const v
   if (!x_planes || !b_planes || !out) return fail("matrix_probe: null pointer");
   if (rows_x <= 0 || rows_x % 128 != 0 || rows_b <= 0 || rows_b % 256 != 0 || k_steps <= 0 || k_steps % 16 != 0)
     return fail("matrix_probe: rows_x must be a multiple of 128, rows_b of 256, k_steps of 16");
-  if (mode < 0 || mode > 3) return fail("matrix_probe: mode must be 0 .. 3");
+  if (mode < 0 || mode > 4) return fail("matrix_probe: mode must be 0 .. 4");
   if (mode == 3 && rows_x % 256 != 0) return fail("matrix_probe: mode 3 takes rows_x in multiples of 256");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const unsigned grid = (unsigned)(rows_x / 128) * (unsigned)(rows_b / 256);
@@ -2634,13 +2636,15 @@ extern "C" int pylo_mi355_matrix_probe(const void* x_planes, int rows_x, const v
     HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<1>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(4)));
     HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<2>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(4)));
     HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe_wide, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 512 * kNsRowB));
+    HIP_TRY(hipFuncSetAttribute((const void*)k_matrix_probe<4>, hipFuncAttributeMaxDynamicSharedMemorySize, hf_gemm_lds(4)));
   }
   const hbits* X = static_cast<const hbits*>(x_planes);
   const hbits* B = static_cast<const hbits*>(b_planes);
   if (mode == 0) hipLaunchKernelGGL(k_matrix_probe<0>, dim3(grid), dim3(256), hf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
   else if (mode == 1) hipLaunchKernelGGL(k_matrix_probe<1>, dim3(grid), dim3(256), hf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
   else if (mode == 2) hipLaunchKernelGGL(k_matrix_probe<2>, dim3(grid), dim3(256), hf_gemm_lds(4), s, X, rows_x, B, rows_b, k_steps, out);
-  else hipLaunchKernelGGL(k_matrix_probe_wide, dim3(grid / 2), dim3(512), 2 * 512 * kNsRowB, s, X, rows_x, B, rows_b, k_steps, out);
+  else if (mode == 3) hipLaunchKernelGGL(k_matrix_probe_wide, dim3(grid / 2), dim3(512), 2 * 512 * kNsRowB, s, X, rows_x, B, rows_b, k_steps, out);
+  else hipLaunchKernelGGL(k_matrix_probe<4>, dim3(grid), dim3(256), 2 * 256 * kNsRowB, s, X, rows_x, B, rows_b, k_steps, out);
   HIP_TRY(hipGetLastError());
   return 0;
 }

@@ -27,6 +27,7 @@ constexpr int kNsBK = 16;        // reduction steps per stage
 constexpr int kNsLd = kNsTile + 4;   // LDS row pitch in floats (16-byte aligned rows)
 constexpr int kNsSlabK = 2048;   // reduction length of one slab of a split Gram product
 constexpr int kNsSplitMin = 8192;   // Gram products with a reduction at least this long are split
+constexpr int kNsFewJobs = 512;     // a plan with fewer Gram tile jobs than this splits them further (two per CU)
 
 enum : int { kNsGram = 0, kNsPoly = 1, kNsUpdate = 2 };
 
@@ -35,6 +36,7 @@ struct NsMat {
   int unit;            // the finishing pass's unit whose sum of squares is this matrix's (FinUnit)
   int R, C, m, tall;   // X is R x C row-major; m = min(R, C); tall: R > C
   int n_slabs;         // > 1: the Gram product is split along its reduction
+  int slab_k;          // reduction length of one slab
   long long off_x1;    // floats into the workspace: the second X buffer (R x C)
   long long off_a;     // A (m x m)
   long long off_b;     // B' (m x m)

@@ -438,6 +438,7 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
     mt.m = std::min(R, C);
     const int K = mt.tall ? mt.R : mt.C;
     mt.n_slabs = K >= kNsSplitMin ? (K + kNsSlabK - 1) / kNsSlabK : 1;
+    mt.slab_k = kNsSlabK;
     mt.off_x1 = take((long long)R * C);
     mt.off_a = take((long long)mt.m * mt.m);
     mt.off_b = take((long long)mt.m * mt.m);
@@ -467,6 +468,27 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
     }
   }
   if (L.ns_hf) {
+    // A plan with few matrices (a convolutional net's one classifier, a small MLP) has fewer Gram tile jobs than the
+    // part has CUs, each a long reduction: split them along it, up to eight ways, until there are two jobs a CU.
+    {
+      long long jobs = 0;
+      for (const NsMat& f : L.ns_mats) {
+        const long long nt = (f.m + kNsTile - 1) / kNsTile;
+        jobs += nt * (nt + 1) / 2 * f.n_slabs;
+      }
+      if (jobs > 0 && jobs < kNsFewJobs) {
+        const int ways = (int)std::min<long long>(8, (kNsFewJobs + jobs - 1) / jobs);
+        for (NsMat& f : L.ns_mats) {
+          if (f.n_slabs > 1) continue;
+          const int K = f.tall ? f.R : f.C;
+          const int sk = std::max(256, ((K + ways - 1) / ways + 15) / 16 * 16);
+          if ((K + sk - 1) / sk > 1) {
+            f.slab_k = sk;
+            f.n_slabs = (K + sk - 1) / sk;
+          }
+        }
+      }
+    }
     // same matrices, operands as fp16 planes; the item tables are rebuilt for the uniform (n x m) orientation
     L.ns_gram.clear(); L.ns_poly.clear(); L.ns_upd.clear(); L.ns_upd4.clear();
     ws_floats = 0;
@@ -596,8 +618,9 @@ void build_ns_tables(Layout& L, const PyloTensorShape* shapes, int T, long long&
         const int nt = (b.m + kNsTile - 1) / kNsTile, n_upper = nt * (nt + 1) / 2;
         // Gram: the tiles of one matrix (of one slab of it) read the same rows of Xs; Poly: the same A
         for (int sl = 0; sl < b.n_slabs; ++sl) {
-          const int k0 = b.n_slabs > 1 ? sl * kNsSlabK : 0;
-          const int k1 = b.n_slabs > 1 ? up16(std::min(b.n, (sl + 1) * kNsSlabK)) : up16(b.n);
+          const int slab_k = L.ns_mats[q].slab_k;
+          const int k0 = b.n_slabs > 1 ? sl * slab_k : 0;
+          const int k1 = b.n_slabs > 1 ? up16(std::min(b.n, (sl + 1) * slab_k)) : up16(b.n);
           for (int tm = 0; tm < nt; ++tm)
             for (int tn = tm; tn < nt; ++tn) gram.push_back(NsItem{q, tm, tn, k0, k1, b.n_slabs > 1 ? sl : -1});
           gram_units.push_back({n_upper, (long long)(k1 - k0)});

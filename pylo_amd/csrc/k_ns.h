@@ -41,7 +41,7 @@ struct NsMat {
   long long off_a;     // A (m x m)
   long long off_b;     // B' (m x m)
   long long off_part;  // split Gram product: n_slabs partial matrices (m x m each), else unused
-  long long elem_off;  // elements from the tensor's raw step to this matrix (split-bf16 kernels: a slice of a tensor with more dims)
+  long long elem_off;  // elements from the tensor's raw step to this matrix (split-fp16 kernels: a slice of a tensor with more dims)
 };
 
 struct NsItem {

@@ -1,6 +1,6 @@
 """Benchmark of the fused learned-optimizer step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gpt2s|cfg1|vit_velo|llama_adafac|stress_velo|stress_celo2|conv_celo2|stream_ceiling|matrix_ceiling] [--fused-only]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gpt2s|cfg1|vit_velo|llama_adafac|stress_velo|stress_celo2|conv_celo2|llama_celo2|stream_ceiling|matrix_ceiling] [--fused-only]
 
 Workload (default): BASELINE config 2 -- ELO-CELO2 on a GPT-2-small-shaped fp32 parameter set
 (98 tensors, 124 355 328 parameters), synthetic per-tensor Gaussian gradients with log-uniform
@@ -238,7 +238,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gpt2s", choices=["gpt2s", "cfg1", "vit_velo", "llama_adafac", "stress_velo", "stress_celo2", "conv_celo2", "stream_ceiling", "matrix_ceiling"])
+    ap.add_argument("--workload", default="gpt2s", choices=["gpt2s", "cfg1", "vit_velo", "llama_adafac", "stress_velo", "stress_celo2", "conv_celo2", "llama_celo2", "stream_ceiling", "matrix_ceiling"])
     ap.add_argument("--fused-only", action="store_true",
                     help="loop the C-ABI call alone (no Newton-Schulz / apply), e.g. under rocprofv3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -257,8 +257,8 @@ def main():
     from pylo_amd import ELO_CELO2_CUDA
     from pylo_amd.models import CELO2MLP
 
-    if a.workload == "conv_celo2":
-        print(json.dumps(conv_workload(a.steps, a.warmup)))
+    if a.workload in ("conv_celo2", "llama_celo2"):
+        print(json.dumps(conv_workload(a.steps, a.warmup, a.workload)))
         return
     if a.workload in ("stress_velo", "stress_celo2"):
         print(json.dumps(stress_workload(a.workload, a.steps, a.warmup)))
@@ -479,10 +479,13 @@ def matrix_ceiling(a):
                       "peak_PFLOPs": 2.5, "cases": res}))
 
 
-def conv_workload(steps, warmup):
-    """Whole ELO_CELO2 optimizer.step() on the ResNet-50 parameter set: the fused element call (per-slice feature
-    normalisers for the convolution kernels), then one finishing call in which every kernel's k x k slices are
-    orthogonalised, normalised and applied by the per-slice launches and the one matrix by the tiled products."""
+def conv_workload(steps, warmup, which="conv_celo2"):
+    """Whole ELO_CELO2 optimizer.step() on a parameter set that is not a BASELINE configuration.
+    conv_celo2: ResNet-50 -- the fused element call (per-slice feature normalisers for the convolution kernels), then
+    one finishing call in which every kernel's k x k slices are orthogonalised, normalised and applied by the
+    per-slice launches and the one matrix by the tiled products.
+    llama_celo2: the Llama-1.1B set of config 4 under ELO-CELO2 (matrices with a smaller dim of 2048, the two
+    32000 x 2048 embeddings orthogonalised like the rest): how the products do on larger m."""
     import numpy as np
     import torch
 
@@ -490,7 +493,8 @@ def conv_workload(steps, warmup):
     from pylo_amd.models import CELO2MLP
 
     dev = torch.device("cuda:0")
-    shapes = resnet50_shapes()
+    shapes = resnet50_shapes() if which == "conv_celo2" else llama_1b_shapes()
+    label = "ResNet-50 parameter set" if which == "conv_celo2" else "Llama-1.1B parameter set"
     gen = torch.Generator(device=dev).manual_seed(1)
     params = [torch.nn.Parameter(torch.randn(s, generator=gen, device=dev) * 0.02) for s in shapes]
     for p in params:
@@ -515,7 +519,8 @@ def conv_workload(steps, warmup):
     return {"metric": "params_updated_per_sec (whole optimizer.step())", "value": n / (ms * 1e-3), "unit": "params/s",
             "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-            "config": {"workload": "ELO_CELO2 whole optimizer.step(), ResNet-50 parameter set", "params": n,
+            "newton_schulz_TFLOP": ns_flops(shapes) / 1e12, "newton_schulz_TFLOP_executed": ns_flops_executed(shapes) / 1e12,
+            "config": {"workload": "ELO_CELO2 whole optimizer.step(), " + label, "params": n,
                        "tensors": len(shapes), "params_in_tensors_with_more_than_two_dims": n_nd},
             "fused_call_ms": float(np.mean([m[0].elapsed_time(m[1]) for m in marks])),
             "finishing_call_ms": float(np.mean([m[1].elapsed_time(m[2]) for m in marks])),

@@ -1111,6 +1111,9 @@ struct PyloPlan {
   // ELO-CELO2: the Newton-Schulz chains of the groups of matrices after the first run on streams of the plan's own
   hipStream_t ns_side[3] = {nullptr, nullptr, nullptr};
   hipEvent_t ns_fork = nullptr, ns_join[3] = {nullptr, nullptr, nullptr};
+  // the per-slice finishing launches next to the matrices' products, where the groups leave a hardware queue free
+  hipStream_t slice_side = nullptr;
+  hipEvent_t slice_fork = nullptr, slice_join = nullptr;
 
   template <class Tp>
   Tp* at(size_t off) const { return reinterpret_cast<Tp*>(ws + off); }
@@ -1216,6 +1219,13 @@ int pylo_mi355_plan_create(int kind, const PyloTensorShape* shapes, int n_tensor
     if (e == hipSuccess) e = hipStreamCreateWithFlags(&P->ns_side[g - 1], hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreateWithFlags(&P->ns_join[g - 1], hipEventDisableTiming);
   }
+  bool plan_has_slices = !L.slice_items_w.empty() || !L.slice_items_b.empty();
+  for (const auto& v : L.slice_items_l) plan_has_slices = plan_has_slices || !v.empty();
+  if (e == hipSuccess && plan_has_slices && ns_streams >= 1 && ns_streams <= 3) {   // main + groups + this one <= 4 queues
+    e = hipStreamCreateWithFlags(&P->slice_side, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&P->slice_fork, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&P->slice_join, hipEventDisableTiming);
+  }
   if (e != hipSuccess) {
     pylo_mi355_plan_destroy(P);
     return fail(std::string("plan_create: ") + hipGetErrorString(e));
@@ -1232,6 +1242,9 @@ int pylo_mi355_plan_destroy(PyloPlan* P) {
   if (P->side) (void)hipStreamDestroy(P->side);
   if (P->stale_host) (void)hipHostFree(P->stale_host);
   if (P->ns_fork) (void)hipEventDestroy(P->ns_fork);
+  if (P->slice_fork) (void)hipEventDestroy(P->slice_fork);
+  if (P->slice_join) (void)hipEventDestroy(P->slice_join);
+  if (P->slice_side) (void)hipStreamDestroy(P->slice_side);
   for (int g = 0; g < 3; ++g) {
     if (P->ns_join[g]) (void)hipEventDestroy(P->ns_join[g]);
     if (P->ns_side[g]) (void)hipStreamDestroy(P->ns_side[g]);
@@ -1692,9 +1705,18 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
   double* fin_part = P->at<double>(L.off_finpart);
   float* fin_scale = P->at<float>(L.off_finscale);
   const int n_fin = (int)L.fin_items.size();
+  // The per-slice launches touch only their own tensors: next to the matrices' chains of products they run on a stream
+  // of their own (forked from and joined into the caller's like the groups').
+  const bool slices_aside = any_slices && any_ns && L.ns_hf && P->slice_side != nullptr;
   if (any_slices) {
     // tensors with more than two dims: everything per slice, in LDS (k_slice_finish.h)
     if (int rc = slice_lds_once()) return rc;
+    hipStream_t caller = s;
+    if (slices_aside) {
+      HIP_TRY(hipEventRecord(P->slice_fork, caller));
+      HIP_TRY(hipStreamWaitEvent(P->slice_side, P->slice_fork, 0));
+    }
+    hipStream_t s = slices_aside ? P->slice_side : caller;
     const SliceMat* smats = P->at<SliceMat>(L.off_slice_mats);
     const float c0 = coeffs ? coeffs[0] : 0.0f, c1 = coeffs ? coeffs[1] : 0.0f, c2 = coeffs ? coeffs[2] : 0.0f;
     const int orth_call = coeffs != nullptr;
@@ -1714,6 +1736,7 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
     if (!L.slice_items_b.empty())
       hipLaunchKernelGGL(k_celo2_slice_finish<true>, dim3((unsigned)L.slice_items_b.size()), dim3(256), L.slice_lds_b, s,
                          smats, P->at<Item>(L.off_slice_items_b), descs, dyn, orth_call, ns_iters, ns_eps, c0, c1, c2);
+    if (slices_aside) HIP_TRY(hipEventRecord(P->slice_join, P->slice_side));
   }
   if (n_fin == 0) {
     HIP_TRY(hipGetLastError());
@@ -1931,6 +1954,7 @@ int finish_impl(PyloPlan* P, const PyloTensorArgs* args, const float* coeffs, in
     const long long* x_alt = (ns_iters & 1) ? P->at<long long>(L.off_ns_xalt) : nullptr;
     finish_range(s, 0, n_fin, 0, (int)L.fin_units.size(), x_alt, ns_ws);
   }
+  if (slices_aside) HIP_TRY(hipStreamWaitEvent(s, P->slice_join, 0));
   HIP_TRY(hipGetLastError());
   return 0;
 }

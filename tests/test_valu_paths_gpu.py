@@ -132,3 +132,51 @@ def test_adafac_matrix_pipes_against_fp64(monkeypatch):
         errs[name] = max(float((p.detach().double() - b).abs().max()) for p, b in zip(gpu, ref64))
     print("max |p - fp64 oracle|: fp32 oracle", own, " HIP", errs)
     assert errs["fp16x2"] <= 1.5 * max(own, errs["fp32"]), (errs, own)
+
+
+def test_adafac_fp16_planes_keep_their_range():
+    """The default element MLP splits its operands into fp16 planes, which want numbers of order one: gradients of
+    1e-12 next to a single outlier ten thousand times the rest (raw features from 1e-24 to 1e12, normalised features up
+    to the square root of the element count, hidden values in the thousands) must come out finite and as close to the
+    fp64 evaluation as the fp32 matrix instructions and the fp32 oracle bring them (lr = step_mult = 1: the step
+    itself is what is compared)."""
+    from oracle import pylo_oracle as O
+    from pylo_amd import AdafacLO_CUDA
+    from pylo_amd.models import MetaMLP
+
+    torch.manual_seed(4)
+    net = MetaMLP(39, 32, 1)
+    shapes = [(256, 512), (128, 1024), (64, 2048)]
+    gen = torch.Generator().manual_seed(9)
+    init = [torch.randn(s, generator=gen) * 0.01 for s in shapes]
+    grads = [torch.randn(shapes[0], generator=gen) * 1e-12, torch.randn(shapes[1], generator=gen) * 1e-3,
+             torch.randn(shapes[2], generator=gen) * 10.0]
+    grads[0][7, 11] = 1e-8           # ten thousand times its neighbours
+    grads[1][100, 5] = 50.0
+    grads[2][3, 2000] = 2e5
+    kw = dict(lr=1.0, step_mult=1.0, exp_mult=0.1)
+    ref64 = [v.double().cuda() for v in init]
+    ref32 = [v.clone().cuda() for v in init]
+    O.AdafacOracle(ref64, net.state_dict(), device="cuda", **kw).double_().step([g.double().cuda() for g in grads])
+    O.AdafacOracle(ref32, net.state_dict(), device="cuda", **kw).step([g.cuda() for g in grads])
+    outs = {}
+    for name, env in (("fp16x2", "0"), ("fp32", "1")):
+        mp = pytest.MonkeyPatch()
+        mp.setenv("PYLO_MI355_ADAFAC_F32", env)
+        try:
+            gpu = [torch.nn.Parameter(v.clone().cuda()) for v in init]
+            opt = AdafacLO_CUDA(gpu, network=copy.deepcopy(net), **kw)
+            for p, g in zip(gpu, grads):
+                p.grad = g.cuda()
+            opt.step()
+            torch.cuda.synchronize()
+            outs[name] = [p.detach().clone() for p in gpu]
+        finally:
+            mp.undo()
+    for i in range(len(shapes)):
+        own = float((ref32[i].double() - ref64[i]).abs().max())
+        e = {name: float((outs[name][i].double() - ref64[i]).abs().max()) for name in outs}
+        size = float((ref64[i] - init[i].double().cuda()).abs().max())
+        print(shapes[i], "largest step", size, "max |p - fp64 oracle|: fp32 oracle", own, " HIP", e)
+        assert torch.isfinite(outs["fp16x2"][i]).all(), i
+        assert e["fp16x2"] <= 2.0 * max(own, e["fp32"]) + 1e-7 * size, (i, e, own)
